@@ -1,0 +1,159 @@
+/* nl_hecate_rocm — C ABI of the MI355X (gfx950) memory-rule kernel library.
+ *
+ * Drop-in boundary: every function whose name ends in `_cuda` has exactly the
+ * name, argument order, argument types and buffer layout of the `extern "C"`
+ * declaration in the reference's core/src/cuda_ffi.rs (line cited per
+ * function), so a `rocm` cargo feature can bind this library with the same
+ * Rust declarations.  Functions ending in `_rocm` and `nlh_*` are additions
+ * with no reference symbol.
+ *
+ * Conventions (core/src/cuda_ffi.rs, the .cu files under core/kernels):
+ *   - all pointers are device memory owned by the caller; row-major; f32 unless
+ *     stated; bf16 travels as uint16_t; sizes are int.
+ *   - no stream argument: work is enqueued on the null stream (or the stream
+ *     given to nlh_set_stream) and is asynchronous; the caller synchronises.
+ *   - void functions report a bad argument or a failed launch by printing a
+ *     message and abort()ing, like the reference; nlh_set_error_mode(1) turns
+ *     that into a recorded error (nlh_last_error) and an early return.
+ *   - chain = one (batch, head) pair; `batch_size` counts chains.
+ */
+#ifndef NL_HECATE_FFI_H
+#define NL_HECATE_FFI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ── library control (no reference counterpart) ─────────────────────────── */
+const char *nlh_version(void);
+void nlh_set_error_mode(int mode);     /* 0 = abort (reference behaviour), 1 = record */
+const char *nlh_last_error(void);      /* "" when no error is recorded */
+void nlh_clear_error(void);
+void nlh_set_stream(void *hip_stream); /* hipStream_t; NULL = null stream */
+void nlh_release_workspace(void);      /* frees the library's device scratch */
+/* Runs the cross-lane primitives on known data; returns 0 when all agree. */
+int nlh_selftest_lane_ops(void);
+
+/* ── Titans LMM, exact per-token rule ───────────────────────────────────────
+ * Per token: e = clip(M k - v); S = eta S - theta e k^T; M = (1-alpha) M + S;
+ * M projected to |M|_F <= m_norm_max; y = M q.
+ * k,v,q [batch, seq_len, d]; gates [batch, seq_len]; chain b reads tokens at
+ * b*input_stride*d (gates at b*input_stride) and initial states at b*m_stride;
+ * outputs use the local seq_len: y [batch, seq_len, d],
+ * m_states / s_states [batch, seq_len+1, d*d].
+ * error_clip <= 0 and m_norm_max <= 0 or >= 1e30 disable clip / projection. */
+/* core/src/cuda_ffi.rs:134 */
+void titans_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                             const float *alpha, const float *theta, const float *eta,
+                             const float *m_initial, const float *s_initial,
+                             float *m_states, float *s_states, float *y,
+                             int seq_len, int d, int batch_size, int input_stride, int m_stride,
+                             float error_clip, float m_norm_max);
+/* core/src/cuda_ffi.rs:156.  d_m_initial / d_s_initial [d*d] are ACCUMULATED
+ * (+=) with the sum over the batch; the caller zeroes them. */
+void titans_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                              const float *alpha, const float *theta, const float *eta,
+                              const float *m_states, const float *s_states, const float *d_y,
+                              float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                              float *d_alpha, float *d_theta, float *d_eta,
+                              float *d_m_initial, float *d_s_initial,
+                              int seq_len, int d, int batch_size, float error_clip);
+/* core/src/cuda_ffi.rs:230.  One chain; stores M/S at slot 0 and after every
+ * token with (t+1)%C==0 or t+1==seq_len. */
+void titans_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                  const float *alpha, const float *theta, const float *eta,
+                                  const float *m_initial, const float *s_initial,
+                                  float *m_states, float *s_states, float *y,
+                                  int seq_len, int d, int checkpoint_interval, float error_clip,
+                                  float m_norm_max);
+/* core/src/cuda_ffi.rs:262.  Tokens [t_start, t_end); token tensors are
+ * indexed by absolute t with stride seq_len; m_states / s_states are the
+ * segment-local trajectory [batch, t_end-t_start+1, d*d]; seeds and outs are
+ * [batch, d*d] (not summed over the batch). */
+void titans_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                      const float *alpha, const float *theta, const float *eta,
+                                      const float *m_states, const float *s_states, const float *d_y,
+                                      const float *d_m_seed, const float *d_s_seed,
+                                      float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                      float *d_alpha, float *d_theta, float *d_eta,
+                                      float *d_m_out, float *d_s_out,
+                                      int t_start, int t_end, int d, int batch_size, int seq_len,
+                                      float error_clip);
+
+/* ── Delta rule (Titans without momentum) ────────────────────────────────── */
+/* core/src/cuda_ffi.rs:86 */
+void delta_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                            const float *alpha, const float *theta, const float *m_initial,
+                            float *m_states, float *y, int seq_len, int d, int batch_size,
+                            int input_stride, int m_stride, float error_clip, float m_norm_max);
+/* core/src/cuda_ffi.rs:109 */
+void delta_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                             const float *alpha, const float *theta,
+                             const float *m_states, const float *d_y,
+                             float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                             float *d_alpha, float *d_theta, float *d_m_initial,
+                             int seq_len, int d, int batch_size, float error_clip);
+/* core/src/cuda_ffi.rs:221 */
+void delta_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                 const float *alpha, const float *theta, const float *m_initial,
+                                 float *m_states, float *y, int seq_len, int d,
+                                 int checkpoint_interval, float error_clip, float m_norm_max);
+/* core/src/cuda_ffi.rs:250 */
+void delta_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                     const float *alpha, const float *theta,
+                                     const float *m_states, const float *d_y, const float *d_m_seed,
+                                     float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                     float *d_alpha, float *d_theta, float *d_m_out,
+                                     int t_start, int t_end, int d, int batch_size, int seq_len,
+                                     float error_clip);
+
+/* ── DGD: same update as Delta, no projection (core/kernels/dgd_forward.cu:6-11) */
+/* core/src/cuda_ffi.rs:291 */
+void dgd_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                          const float *alpha, const float *theta, const float *m_initial,
+                          float *m_states, float *y, int seq_len, int d, int batch_size,
+                          int input_stride, int m_stride, float error_clip);
+/* core/src/cuda_ffi.rs:309 (single chain: no batch argument) */
+void dgd_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                           const float *alpha, const float *theta,
+                           const float *m_states, const float *d_y,
+                           float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                           float *d_alpha, float *d_theta, float *d_m_initial,
+                           int seq_len, int d, float error_clip);
+/* core/src/cuda_ffi.rs:329 */
+void dgd_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                               const float *alpha, const float *theta, const float *m_initial,
+                               float *m_states, float *y, int seq_len, int d,
+                               int checkpoint_interval, float error_clip);
+/* core/src/cuda_ffi.rs:337 */
+void dgd_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                   const float *alpha, const float *theta,
+                                   const float *m_states, const float *d_y, const float *d_m_seed,
+                                   float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                   float *d_alpha, float *d_theta, float *d_m_out,
+                                   int t_start, int t_end, int d, int batch_size, int seq_len,
+                                   float error_clip);
+
+/* ── Batched checkpointed forward (addition) ────────────────────────────────
+ * The reference loops the single-chain *_forward_ckpt over heads
+ * (core/src/gpu_forward.rs:1611-1662); these take all chains in one launch.
+ * m_ckpt / s_ckpt [batch, n_ckpt, d*d], n_ckpt = checkpoint_count(seq_len, C)
+ * (core/src/gpu_forward.rs:2885-2897); inputs are dense [batch, seq_len, ...]. */
+void titans_forward_ckpt_batched_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                          const float *alpha, const float *theta, const float *eta,
+                                          const float *m_initial, const float *s_initial,
+                                          float *m_ckpt, float *s_ckpt, float *y,
+                                          int seq_len, int d, int batch_size, int checkpoint_interval,
+                                          float error_clip, float m_norm_max);
+void delta_forward_ckpt_batched_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                         const float *alpha, const float *theta,
+                                         const float *m_initial, float *m_ckpt, float *y,
+                                         int seq_len, int d, int batch_size, int checkpoint_interval,
+                                         float error_clip, float m_norm_max);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NL_HECATE_FFI_H */

@@ -1,0 +1,847 @@
+// Exact per-token memory rules (Delta / DGD / Titans LMM), forward and backward,
+// for gfx950.
+//
+// Layout of the work.  One (batch, head) chain carries a d x d matrix M (and the
+// momentum S).  Without error clipping and M-norm projection the rows of M are
+// independent recurrences: row i needs only e_i = M[i,:].k - v_i.  The kernels
+// exploit that: a lane owns RPL rows x 4 columns of every state matrix in
+// registers, the D/4 lanes that share a row sit inside one DPP row (row sums are
+// DPP adds, no LDS, no barrier), a wave owns 64/(D/4) row groups and a workgroup
+// of 4 waves owns a slab of rows.  A chain is split over `parts` workgroups so
+// that 64-128 chains still fill 256 CUs; workgroups of one chain never
+// communicate during the recurrence.  Only the column sums (d_q, d_k) and the
+// gate gradients cross rows, and those are outputs, not feedback: they are
+// reduced per tile through LDS and, across the workgroups of a chain, through a
+// small partial-sum buffer and a finalize kernel (deterministic summation order).
+//
+// State never round-trips through HBM inside the recurrence; k/v/q/dY are
+// streamed through double-buffered LDS tiles with 16-byte coalesced loads.
+//
+// When clipping or projection is active the rows couple through one scalar per
+// token; the COUPLED instantiation keeps a whole chain in one workgroup and
+// pays two barriers per coupled reduction.
+#include <hip/hip_runtime.h>
+#include <math.h>
+
+#include "../../include/nl_hecate_ffi.h"
+#include "lane_ops.h"
+#include "rule_tiles.h"
+#include "runtime.h"
+
+namespace nlh {
+
+constexpr int TB = 16;  // tokens per LDS tile
+
+// blockIdx -> (chain, part).  Workgroups are dealt round-robin to the 8 XCDs, so
+// consecutive block ids land on different L2s; remap so that the parts of one
+// chain (which read the same k/q rows) share an XCD.
+__device__ __forceinline__ void map_block(int parts, int &chain, int &part) {
+    int n = blockIdx.x, nb = gridDim.x, L = n;
+    if (nb % 8 == 0) L = (n % 8) * (nb / 8) + n / 8;
+    chain = L / parts;
+    part = L % parts;
+}
+
+__device__ __forceinline__ bool mnorm_active(float m_norm_max) {
+    return m_norm_max > 0.f && m_norm_max < 1e30f;  // core/kernels/m_norm_project.cuh:27
+}
+
+__device__ __forceinline__ float4 f4_zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ float4 f4_scale(float a, const float4 &x) {
+    return make_float4(a * x.x, a * x.y, a * x.z, a * x.w);
+}
+// a*x + b*y
+__device__ __forceinline__ float4 f4_axpby(float a, const float4 &x, float b, const float4 &y) {
+    return make_float4(a * x.x + b * y.x, a * x.y + b * y.y, a * x.z + b * y.z, a * x.w + b * y.w);
+}
+__device__ __forceinline__ void f4_fma(float4 &acc, float a, const float4 &x) {
+    acc.x += a * x.x; acc.y += a * x.y; acc.z += a * x.z; acc.w += a * x.w;
+}
+__device__ __forceinline__ void f4_add(float4 &acc, const float4 &x) {
+    acc.x += x.x; acc.y += x.y; acc.z += x.z; acc.w += x.w;
+}
+
+// Workgroup-wide sum of one float per lane (COUPLED kernels only: every wave of
+// the workgroup must call it).  `slot` points at kWaves floats of LDS that no
+// other reduction uses until the next barrier after this one.
+__device__ __forceinline__ float block_allreduce(float x, float *slot, int tid) {
+    x = wave_allreduce(x);
+    if ((tid & 63) == 0) slot[tid >> 6] = x;
+    __syncthreads();
+    return slot[0] + slot[1] + slot[2] + slot[3];
+}
+
+// ───────────────────────────── forward ─────────────────────────────────────
+struct FwdArgs {
+    const float *k, *v, *q, *alpha, *theta, *eta, *m_initial, *s_initial;
+    float *m_out, *s_out, *y;
+    int seq_len, input_stride, ckpt_interval, parts;
+    long long m_stride;      // elements between chains in m_initial / s_initial
+    long long state_stride;  // elements between chains in m_out / s_out
+    float error_clip, m_norm_max;
+};
+
+enum { STORE_NONE = 0, STORE_TRAJ = 1, STORE_CKPT = 2 };
+
+template <int D, int RPL, bool HAS_S, int STORE, bool COUPLED>
+__global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
+    constexpr int LPR = D / 4;          // lanes per row
+    constexpr int RG = 64 / LPR;        // row groups per wave
+    constexpr int ROWS_WG = kWaves * RG * RPL;
+    constexpr int DD = D * D;
+
+    __shared__ __align__(16) float sk[2][TB * D];
+    __shared__ __align__(16) float sq[2][TB * D];
+    __shared__ __align__(16) float sv[2][TB * D];
+    __shared__ float sg[2][3 * TB];
+    __shared__ float sy[2][TB * ROWS_WG];
+    __shared__ float sred[4][kWaves];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cb = lane % LPR, g = lane / LPR;
+    int chain, part;
+    map_block(a.parts, chain, part);
+    const int row_local = (wave * RG + g) * RPL;
+    const int row0 = part * ROWS_WG + row_local;
+
+    const float *kb = a.k + (size_t)chain * a.input_stride * D;
+    const float *vb = a.v + (size_t)chain * a.input_stride * D;
+    const float *qb = a.q + (size_t)chain * a.input_stride * D;
+    const float *ab = a.alpha + (size_t)chain * a.input_stride;
+    const float *tb = a.theta + (size_t)chain * a.input_stride;
+    const float *eb = HAS_S ? a.eta + (size_t)chain * a.input_stride : nullptr;
+    float *yb = a.y + (size_t)chain * a.seq_len * D;
+    float *mo = a.m_out + (size_t)chain * a.state_stride;
+    float *so = HAS_S ? a.s_out + (size_t)chain * a.state_stride : nullptr;
+
+    float4 M[RPL], S[RPL];
+    bool valid[RPL];
+#pragma unroll
+    for (int r = 0; r < RPL; r++) {
+        valid[r] = (row0 + r) < D;
+        M[r] = f4_zero();
+        S[r] = f4_zero();
+        if (valid[r]) {
+            size_t off = (size_t)(row0 + r) * D + cb * 4;
+            M[r] = *reinterpret_cast<const float4 *>(a.m_initial + (size_t)chain * a.m_stride + off);
+            if (HAS_S)
+                S[r] = *reinterpret_cast<const float4 *>(a.s_initial + (size_t)chain * a.m_stride + off);
+            if (STORE != STORE_NONE) {
+                *reinterpret_cast<float4 *>(mo + off) = M[r];
+                if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
+            }
+        }
+    }
+    int ckpt_slot = 1;
+
+    const int seq_len = a.seq_len;
+    const int ntiles = (seq_len + TB - 1) / TB;
+    const bool clip_on = COUPLED && a.error_clip > 0.f;
+    const bool mn_on = COUPLED && mnorm_active(a.m_norm_max);
+
+    TileRegs<D, TB> rk, rq, rv;
+    GateRegs<TB> rg;
+    rk.load(kb, 0, 0, seq_len, tid);
+    rq.load(qb, 0, 0, seq_len, tid);
+    rv.load(vb, 0, 0, seq_len, tid);
+    rg.load(ab, tb, eb, 0, 0, seq_len, tid);
+
+    auto flush_y = [&](int ti) {
+        const float *src = sy[ti & 1];
+        int t0 = ti * TB;
+        for (int idx = tid; idx < TB * ROWS_WG; idx += kThreads) {
+            int tt = idx / ROWS_WG, r = idx % ROWS_WG;
+            int row = part * ROWS_WG + r, t = t0 + tt;
+            if (row < D && t < seq_len) yb[(size_t)t * D + row] = src[idx];
+        }
+    };
+
+    for (int ti = 0; ti < ntiles; ti++) {
+        const int buf = ti & 1, t0 = ti * TB;
+        rk.store_lds(sk[buf], tid);
+        rq.store_lds(sq[buf], tid);
+        rv.store_lds(sv[buf], tid);
+        rg.store_lds(sg[buf], tid);
+        __syncthreads();
+        if (ti > 0) flush_y(ti - 1);
+        if (ti + 1 < ntiles) {
+            rk.load(kb, t0 + TB, 0, seq_len, tid);
+            rq.load(qb, t0 + TB, 0, seq_len, tid);
+            rv.load(vb, t0 + TB, 0, seq_len, tid);
+            rg.load(ab, tb, eb, t0 + TB, 0, seq_len, tid);
+        }
+        const int tn = min(TB, seq_len - t0);
+        for (int tl = 0; tl < tn; tl++) {
+            const int t = t0 + tl;
+            const float4 kk = *reinterpret_cast<const float4 *>(&sk[buf][tl * D + cb * 4]);
+            const float4 qq = *reinterpret_cast<const float4 *>(&sq[buf][tl * D + cb * 4]);
+            const float al = sg[buf][tl], th = sg[buf][TB + tl], et = sg[buf][2 * TB + tl];
+            const float ret = 1.f - al;
+            float e[RPL];
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                float p = group_allreduce<LPR>(dot4(M[r], kk));
+                float vv = sv[buf][tl * D + (valid[r] ? row0 + r : 0)];
+                e[r] = valid[r] ? p - vv : 0.f;
+            }
+            if (COUPLED && clip_on) {
+                float sq_sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < RPL; r++) sq_sum += e[r] * e[r];
+                if (cb != 0) sq_sum = 0.f;
+                float nrm = sqrtf(block_allreduce(sq_sum, sred[(t & 1) * 2], tid));
+                if (nrm > a.error_clip) {
+                    float sc = a.error_clip / nrm;
+#pragma unroll
+                    for (int r = 0; r < RPL; r++) e[r] *= sc;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                float te = th * e[r];
+                if (HAS_S) {
+                    S[r] = f4_axpby(et, S[r], -te, kk);
+                    M[r] = f4_axpby(ret, M[r], 1.f, S[r]);
+                } else {
+                    M[r] = f4_axpby(ret, M[r], -te, kk);
+                }
+            }
+            if (COUPLED && mn_on) {
+                float sq_sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < RPL; r++) sq_sum += dot4(M[r], M[r]);
+                float fn = sqrtf(block_allreduce(sq_sum, sred[(t & 1) * 2 + 1], tid));
+                if (fn > a.m_norm_max) {
+                    float sc = a.m_norm_max / fn;
+#pragma unroll
+                    for (int r = 0; r < RPL; r++) M[r] = f4_scale(sc, M[r]);
+                }
+            }
+            if (STORE == STORE_TRAJ) {
+#pragma unroll
+                for (int r = 0; r < RPL; r++)
+                    if (valid[r]) {
+                        size_t off = (size_t)(t + 1) * DD + (size_t)(row0 + r) * D + cb * 4;
+                        *reinterpret_cast<float4 *>(mo + off) = M[r];
+                        if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
+                    }
+            } else if (STORE == STORE_CKPT) {
+                if (((t + 1) % a.ckpt_interval == 0) || (t + 1 == seq_len)) {
+#pragma unroll
+                    for (int r = 0; r < RPL; r++)
+                        if (valid[r]) {
+                            size_t off = (size_t)ckpt_slot * DD + (size_t)(row0 + r) * D + cb * 4;
+                            *reinterpret_cast<float4 *>(mo + off) = M[r];
+                            if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
+                        }
+                    ckpt_slot++;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                float yy = group_allreduce<LPR>(dot4(M[r], qq));
+                if (cb == 0) sy[buf][tl * ROWS_WG + row_local + r] = yy;
+            }
+        }
+    }
+    __syncthreads();
+    if (ntiles > 0) flush_y(ntiles - 1);
+}
+
+// ───────────────────────────── backward ────────────────────────────────────
+// Reverse sweep over [t_start, t_end) of every chain, reading the trajectory
+// M_{t_start..t_end}, S_{t_start..t_end-1} from memory (the reference's
+// *_backward and *_backward_segment contract).
+struct BwdArgs {
+    const float *k, *v, *q, *alpha, *theta, *eta, *m_states, *s_states, *d_y;
+    const float *d_m_seed, *d_s_seed;      // [B, dd] or null (zero)
+    float *d_k, *d_v, *d_q, *d_alpha, *d_theta, *d_eta;
+    float *ws_dq, *ws_dk, *ws_gate;        // partial sums when parts > 1
+    float *d_m_out, *d_s_out;              // [B, dd]
+    int seq_len, t_start, t_end, parts, batch;
+    long long traj_stride;                 // elements between chains in m_states
+    float error_clip;
+};
+
+template <int D, int RPL, bool HAS_S, bool COUPLED>
+__global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
+    // smaller token tile than forward: the per-wave output partials share LDS
+    constexpr int TB = D >= 128 ? 4 : (D >= 64 ? 8 : 16);
+    constexpr int LPR = D / 4;
+    constexpr int RG = 64 / LPR;
+    constexpr int ROWS_WG = kWaves * RG * RPL;
+    constexpr int DD = D * D;
+
+    __shared__ __align__(16) float sk[2][TB * D];
+    __shared__ __align__(16) float sq[2][TB * D];
+    __shared__ __align__(16) float sv[2][TB * D];
+    __shared__ __align__(16) float sdy[2][TB * D];
+    __shared__ float sg[2][3 * TB];
+    __shared__ __align__(16) float sdq[2][TB * kWaves * D];
+    __shared__ __align__(16) float sdk[2][TB * kWaves * D];
+    __shared__ float sdv[2][TB * ROWS_WG];
+    __shared__ float sgate[2][TB * kWaves * 4];
+    __shared__ float sred[2][kWaves];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cb = lane % LPR, g = lane / LPR;
+    int chain, part;
+    map_block(a.parts, chain, part);
+    const int row_local = (wave * RG + g) * RPL;
+    const int row0 = part * ROWS_WG + row_local;
+    const int seq_len = a.seq_len, t_start = a.t_start, t_end = a.t_end;
+
+    const size_t tok = (size_t)chain * seq_len;
+    const float *kb = a.k + tok * D, *vb = a.v + tok * D, *qb = a.q + tok * D;
+    const float *dyb = a.d_y + tok * D;
+    const float *ab = a.alpha + tok, *tb = a.theta + tok;
+    const float *eb = HAS_S ? a.eta + tok : nullptr;
+    const float *ms = a.m_states + (size_t)chain * a.traj_stride;
+    const float *ss = HAS_S ? a.s_states + (size_t)chain * a.traj_stride : nullptr;
+
+    float4 dM[RPL], dS[RPL], Mn[RPL], Mt[RPL], St[RPL];
+    bool valid[RPL];
+    size_t roff[RPL];
+    const int seg_len = t_end - t_start;
+#pragma unroll
+    for (int r = 0; r < RPL; r++) {
+        valid[r] = (row0 + r) < D;
+        roff[r] = (size_t)(valid[r] ? row0 + r : 0) * D + cb * 4;
+        dM[r] = dS[r] = Mn[r] = Mt[r] = St[r] = f4_zero();
+        if (valid[r]) {
+            if (a.d_m_seed) dM[r] = *reinterpret_cast<const float4 *>(a.d_m_seed + (size_t)chain * DD + roff[r]);
+            if (HAS_S && a.d_s_seed)
+                dS[r] = *reinterpret_cast<const float4 *>(a.d_s_seed + (size_t)chain * DD + roff[r]);
+            if (seg_len > 0) {
+                Mn[r] = *reinterpret_cast<const float4 *>(ms + (size_t)seg_len * DD + roff[r]);
+                Mt[r] = *reinterpret_cast<const float4 *>(ms + (size_t)(seg_len - 1) * DD + roff[r]);
+                if (HAS_S) St[r] = *reinterpret_cast<const float4 *>(ss + (size_t)(seg_len - 1) * DD + roff[r]);
+            }
+        }
+    }
+
+    const int ntiles = (seg_len + TB - 1) / TB;
+    const bool clip_on = COUPLED && a.error_clip > 0.f;
+
+    TileRegs<D, TB> rk, rq, rv, rdy;
+    GateRegs<TB> rg;
+    auto load_tile = [&](int ti) {
+        int t0 = t_start + ti * TB;
+        rk.load(kb, t0, t_start, t_end, tid);
+        rq.load(qb, t0, t_start, t_end, tid);
+        rv.load(vb, t0, t_start, t_end, tid);
+        rdy.load(dyb, t0, t_start, t_end, tid);
+        rg.load(ab, tb, eb, t0, t_start, t_end, tid);
+    };
+    // Reduce the per-wave partial outputs of tile ti and write them out.
+    auto flush = [&](int ti, int ob) {
+        const int t0 = t_start + ti * TB;
+        const size_t pbase = ((size_t)part * a.batch + chain) * seq_len;
+        for (int idx = tid; idx < TB * D; idx += kThreads) {
+            int tt = idx / D, col = idx % D, t = t0 + tt;
+            if (t >= t_end) continue;
+            float sq_ = 0.f, sk_ = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) {
+                sq_ += sdq[ob][(tt * kWaves + w) * D + col];
+                sk_ += sdk[ob][(tt * kWaves + w) * D + col];
+            }
+            if (a.parts == 1) {
+                a.d_q[(tok + t) * D + col] = sq_;
+                a.d_k[(tok + t) * D + col] = sk_;
+            } else {
+                a.ws_dq[(pbase + t) * D + col] = sq_;
+                a.ws_dk[(pbase + t) * D + col] = sk_;
+            }
+        }
+        for (int idx = tid; idx < TB * ROWS_WG; idx += kThreads) {
+            int tt = idx / ROWS_WG, r = idx % ROWS_WG, t = t0 + tt;
+            int row = part * ROWS_WG + r;
+            if (t < t_end && row < D) a.d_v[(tok + t) * D + row] = sdv[ob][idx];
+        }
+        if (tid < TB && t0 + tid < t_end) {
+            float ga = 0.f, ge = 0.f, gt = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) {
+                ga += sgate[ob][(tid * kWaves + w) * 4 + 0];
+                ge += sgate[ob][(tid * kWaves + w) * 4 + 1];
+                gt += sgate[ob][(tid * kWaves + w) * 4 + 2];
+            }
+            int t = t0 + tid;
+            if (a.parts == 1) {
+                a.d_alpha[tok + t] = -ga;
+                if (HAS_S) a.d_eta[tok + t] = ge;
+                a.d_theta[tok + t] = -gt;
+            } else {
+                float *wg = a.ws_gate + (pbase + t) * 4;
+                wg[0] = -ga; wg[1] = ge; wg[2] = -gt;
+            }
+        }
+    };
+
+    if (ntiles > 0) load_tile(ntiles - 1);
+    for (int ti = ntiles - 1; ti >= 0; ti--) {
+        const int buf = ti & 1, t0 = t_start + ti * TB;
+        rk.store_lds(sk[buf], tid);
+        rq.store_lds(sq[buf], tid);
+        rv.store_lds(sv[buf], tid);
+        rdy.store_lds(sdy[buf], tid);
+        rg.store_lds(sg[buf], tid);
+        __syncthreads();
+        if (ti + 1 < ntiles) flush(ti + 1, buf ^ 1);
+        if (ti > 0) load_tile(ti - 1);
+        const int tn = min(TB, t_end - t0);
+        for (int tl = tn - 1; tl >= 0; tl--) {
+            const int t = t0 + tl;
+            const int lt = t - t_start;  // index into the local trajectory
+            // prefetch the states of token t-1
+            float4 Mp[RPL], Sp[RPL];
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                Mp[r] = Sp[r] = f4_zero();
+                if (valid[r] && lt > 0) {
+                    Mp[r] = *reinterpret_cast<const float4 *>(ms + (size_t)(lt - 1) * DD + roff[r]);
+                    if (HAS_S) Sp[r] = *reinterpret_cast<const float4 *>(ss + (size_t)(lt - 1) * DD + roff[r]);
+                }
+            }
+            const float4 kk = *reinterpret_cast<const float4 *>(&sk[buf][tl * D + cb * 4]);
+            const float4 qq = *reinterpret_cast<const float4 *>(&sq[buf][tl * D + cb * 4]);
+            const float al = sg[buf][tl], th = sg[buf][TB + tl], et = sg[buf][2 * TB + tl];
+            const float ret = 1.f - al;
+            float4 cq = f4_zero(), ck = f4_zero();
+            float pa = 0.f, pe = 0.f, pt = 0.f;
+            float e[RPL], gk[RPL];
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                const int rr = valid[r] ? row0 + r : 0;
+                const float dy = valid[r] ? sdy[buf][tl * D + rr] : 0.f;
+                f4_fma(dM[r], dy, qq);          // d_M += dy q^T
+                f4_fma(cq, dy, Mn[r]);          // d_q = M_{t+1}^T dy
+                if (HAS_S) f4_add(dS[r], dM[r]);
+                pa += dot4(Mt[r], dM[r]);
+                if (HAS_S) pe += dot4(St[r], dS[r]);
+                const float4 &G = HAS_S ? dS[r] : dM[r];
+                float p = group_allreduce<LPR>(dot4(Mt[r], kk));
+                e[r] = valid[r] ? p - sv[buf][tl * D + rr] : 0.f;
+                gk[r] = group_allreduce<LPR>(dot4(G, kk));
+            }
+            if (COUPLED && clip_on) {
+                float sq_sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < RPL; r++) sq_sum += e[r] * e[r];
+                if (cb != 0) sq_sum = 0.f;
+                float nrm = sqrtf(block_allreduce(sq_sum, sred[t & 1], tid));
+                if (nrm > a.error_clip) {
+                    float sc = a.error_clip / nrm;
+#pragma unroll
+                    for (int r = 0; r < RPL; r++) e[r] *= sc;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                float4 &G = HAS_S ? dS[r] : dM[r];
+                const float derr = -th * gk[r];
+                if (cb == 0) {
+                    pt += e[r] * gk[r];
+                    sdv[buf][tl * ROWS_WG + row_local + r] = -derr;
+                }
+                f4_fma(ck, -th * e[r], G);      // -theta dS^T e
+                f4_fma(ck, derr, Mt[r]);        // + M_t^T d_err
+                if (HAS_S) {
+                    dS[r] = f4_scale(et, dS[r]);
+                    dM[r] = f4_axpby(ret, dM[r], derr, kk);
+                } else {
+                    dM[r] = f4_axpby(ret, dM[r], derr, kk);
+                }
+                Mn[r] = Mt[r];
+                Mt[r] = Mp[r];
+                St[r] = Sp[r];
+            }
+            // column sums over the row groups of this wave, scalars over the wave
+            cq.x = stride_allreduce<LPR>(cq.x); cq.y = stride_allreduce<LPR>(cq.y);
+            cq.z = stride_allreduce<LPR>(cq.z); cq.w = stride_allreduce<LPR>(cq.w);
+            ck.x = stride_allreduce<LPR>(ck.x); ck.y = stride_allreduce<LPR>(ck.y);
+            ck.z = stride_allreduce<LPR>(ck.z); ck.w = stride_allreduce<LPR>(ck.w);
+            pa = wave_allreduce(pa);
+            pt = wave_allreduce(pt);
+            if (HAS_S) pe = wave_allreduce(pe);
+            if (g == 0) {
+                *reinterpret_cast<float4 *>(&sdq[buf][(tl * kWaves + wave) * D + cb * 4]) = cq;
+                *reinterpret_cast<float4 *>(&sdk[buf][(tl * kWaves + wave) * D + cb * 4]) = ck;
+            }
+            if (lane == 0) {
+                float *gp = &sgate[buf][(tl * kWaves + wave) * 4];
+                gp[0] = pa; gp[1] = pe; gp[2] = pt;
+            }
+        }
+    }
+    __syncthreads();
+    if (ntiles > 0) flush(0, 0);
+#pragma unroll
+    for (int r = 0; r < RPL; r++)
+        if (valid[r]) {
+            *reinterpret_cast<float4 *>(a.d_m_out + (size_t)chain * DD + roff[r]) = dM[r];
+            if (HAS_S) *reinterpret_cast<float4 *>(a.d_s_out + (size_t)chain * DD + roff[r]) = dS[r];
+        }
+}
+
+// Sum the per-part partial d_q / d_k / gate gradients of a split chain.
+__global__ void finalize_parts_kernel(const float *ws_dq, const float *ws_dk, const float *ws_gate,
+                                      float *d_q, float *d_k, float *d_alpha, float *d_theta,
+                                      float *d_eta, int parts, int batch, int seq_len, int d,
+                                      int t_start, int t_end) {
+    const int chain = blockIdx.y;
+    const size_t n_tok = (size_t)batch * seq_len;
+    const int seg = t_end - t_start;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < seg * d; idx += gridDim.x * blockDim.x) {
+        int t = t_start + idx / d, col = idx % d;
+        size_t o = ((size_t)chain * seq_len + t) * d + col;
+        float sq_ = 0.f, sk_ = 0.f;
+        for (int p = 0; p < parts; p++) {
+            sq_ += ws_dq[(size_t)p * n_tok * d + o];
+            sk_ += ws_dk[(size_t)p * n_tok * d + o];
+        }
+        d_q[o] = sq_;
+        d_k[o] = sk_;
+    }
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < seg; idx += gridDim.x * blockDim.x) {
+        size_t o = (size_t)chain * seq_len + t_start + idx;
+        float ga = 0.f, ge = 0.f, gt = 0.f;
+        for (int p = 0; p < parts; p++) {
+            const float *wg = ws_gate + ((size_t)p * n_tok + o) * 4;
+            ga += wg[0]; ge += wg[1]; gt += wg[2];
+        }
+        d_alpha[o] = ga;
+        d_theta[o] = gt;
+        if (d_eta) d_eta[o] = ge;
+    }
+}
+
+// dst[i] += sum_b src[b, i] — the initial-state gradients are summed over the
+// batch into a caller-zeroed [dd] buffer (core/kernels/titans_backward.cu:337-341);
+// a fixed summation order keeps the result reproducible.
+__global__ void accumulate_over_batch_kernel(const float *src, float *dst, int batch, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    for (int b = 0; b < batch; b++) s += src[(size_t)b * n + i];
+    dst[i] += s;
+}
+
+// ───────────────────────────── host dispatch ───────────────────────────────
+static bool coupled_needed(float error_clip, float m_norm_max) {
+    return error_clip > 0.f || (m_norm_max > 0.f && m_norm_max < 1e30f);
+}
+
+// rows of a chain that one workgroup owns, for a given D and RPL
+static int rows_per_wg(int d, int rpl) { return kWaves * (64 / (d / 4)) * rpl; }
+
+// Pick rows-per-lane: whole chain in one workgroup when coupled; otherwise split
+// chains until roughly one workgroup per CU is reached.
+static int pick_rpl(int d, int batch, bool coupled) {
+    if (d != 64) return d == 128 ? 4 : 1;
+    if (coupled) return 4;
+    if (batch >= 256) return 4;
+    if (batch >= 128) return 2;
+    return 1;
+}
+
+template <int D, int RPL, bool HAS_S, int STORE>
+static void launch_fwd_c(const FwdArgs &a, int batch, bool coupled) {
+    dim3 grid(batch * a.parts), block(kThreads);
+    if (coupled)
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, true>), grid, block, 0, stream(), a);
+    else
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, false>), grid, block, 0, stream(), a);
+    check_launch("rule_fwd_kernel");
+}
+
+template <bool HAS_S, int STORE>
+static bool launch_fwd(FwdArgs a, int d, int batch) {
+    const bool coupled = coupled_needed(a.error_clip, a.m_norm_max);
+    const int rpl = pick_rpl(d, batch, coupled);
+    a.parts = ceil_div(d, rows_per_wg(d, rpl));
+    if (coupled && a.parts != 1) return false;
+    switch (d) {
+        case 8: launch_fwd_c<8, 1, HAS_S, STORE>(a, batch, coupled); return true;
+        case 16: launch_fwd_c<16, 1, HAS_S, STORE>(a, batch, coupled); return true;
+        case 32: launch_fwd_c<32, 1, HAS_S, STORE>(a, batch, coupled); return true;
+        case 64:
+            if (rpl == 1) launch_fwd_c<64, 1, HAS_S, STORE>(a, batch, false);
+            else if (rpl == 2) launch_fwd_c<64, 2, HAS_S, STORE>(a, batch, false);
+            else launch_fwd_c<64, 4, HAS_S, STORE>(a, batch, coupled);
+            return true;
+        case 128: launch_fwd_c<128, 4, HAS_S, STORE>(a, batch, false); return true;
+        default: return false;
+    }
+}
+
+template <int D, int RPL, bool HAS_S>
+static void launch_bwd_c(const BwdArgs &a, bool coupled) {
+    dim3 grid(a.batch * a.parts), block(kThreads);
+    if (coupled)
+        hipLaunchKernelGGL((rule_bwd_traj_kernel<D, RPL, HAS_S, true>), grid, block, 0, stream(), a);
+    else
+        hipLaunchKernelGGL((rule_bwd_traj_kernel<D, RPL, HAS_S, false>), grid, block, 0, stream(), a);
+    check_launch("rule_bwd_traj_kernel");
+}
+
+template <bool HAS_S>
+static bool launch_bwd(BwdArgs a, int d) {
+    const bool coupled = a.error_clip > 0.f;
+    const int rpl = pick_rpl(d, a.batch, coupled);
+    a.parts = ceil_div(d, rows_per_wg(d, rpl));
+    if (coupled && a.parts != 1) return false;
+    if (a.parts > 1) {
+        size_t n = (size_t)a.parts * a.batch * a.seq_len;
+        a.ws_dq = scratch(2, n * d * sizeof(float));
+        a.ws_dk = scratch(3, n * d * sizeof(float));
+        a.ws_gate = scratch(4, n * 4 * sizeof(float));
+        if (failed()) return true;
+    }
+    switch (d) {
+        case 8: launch_bwd_c<8, 1, HAS_S>(a, coupled); break;
+        case 16: launch_bwd_c<16, 1, HAS_S>(a, coupled); break;
+        case 32: launch_bwd_c<32, 1, HAS_S>(a, coupled); break;
+        case 64:
+            if (rpl == 1) launch_bwd_c<64, 1, HAS_S>(a, false);
+            else if (rpl == 2) launch_bwd_c<64, 2, HAS_S>(a, false);
+            else launch_bwd_c<64, 4, HAS_S>(a, coupled);
+            break;
+        case 128: launch_bwd_c<128, 4, HAS_S>(a, false); break;
+        default: return false;
+    }
+    if (a.parts > 1 && a.t_end > a.t_start) {
+        dim3 grid(ceil_div((long long)(a.t_end - a.t_start) * d, 256), a.batch);
+        hipLaunchKernelGGL(finalize_parts_kernel, grid, dim3(256), 0, stream(), a.ws_dq, a.ws_dk,
+                           a.ws_gate, a.d_q, a.d_k, a.d_alpha, a.d_theta, HAS_S ? a.d_eta : nullptr,
+                           a.parts, a.batch, a.seq_len, d, a.t_start, a.t_end);
+        check_launch("finalize_parts_kernel");
+    }
+    return true;
+}
+
+static void accumulate_over_batch(const float *src, float *dst, int batch, int n) {
+    hipLaunchKernelGGL(accumulate_over_batch_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream(),
+                       src, dst, batch, n);
+    check_launch("accumulate_over_batch_kernel");
+}
+
+static bool check_dims(const char *fn, int seq_len, int d, int batch) {
+    if (d <= 0) { fail("%s: d=%d must be > 0.", fn, d); return false; }
+    if (seq_len < 0 || batch < 0) { fail("%s: seq_len=%d batch=%d must be >= 0.", fn, seq_len, batch); return false; }
+    return true;
+}
+
+static void unsupported(const char *fn, int d, bool coupled) {
+    fail("%s: d=%d%s is not supported by the gfx950 kernels (d in {8,16,32,64,128}; "
+         "clip / M-norm projection need d <= 64).", fn, d, coupled ? " with clip/projection" : "");
+}
+
+}  // namespace nlh
+
+using namespace nlh;
+
+// ───────────────────────────── C ABI ───────────────────────────────────────
+extern "C" {
+
+void titans_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                             const float *alpha, const float *theta, const float *eta,
+                             const float *m_initial, const float *s_initial,
+                             float *m_states, float *s_states, float *y,
+                             int seq_len, int d, int batch_size, int input_stride, int m_stride,
+                             float error_clip, float m_norm_max) {
+    if (!check_dims("titans_forward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
+    FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial, m_states, s_states, y,
+              seq_len, input_stride, 1, 1, m_stride, (long long)(seq_len + 1) * d * d,
+              error_clip, m_norm_max};
+    if (!launch_fwd<true, STORE_TRAJ>(a, d, batch_size))
+        unsupported("titans_forward_f32_cuda", d, coupled_needed(error_clip, m_norm_max));
+}
+
+void delta_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                            const float *alpha, const float *theta, const float *m_initial,
+                            float *m_states, float *y, int seq_len, int d, int batch_size,
+                            int input_stride, int m_stride, float error_clip, float m_norm_max) {
+    if (!check_dims("delta_forward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
+    FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial, nullptr, m_states, nullptr, y,
+              seq_len, input_stride, 1, 1, m_stride, (long long)(seq_len + 1) * d * d,
+              error_clip, m_norm_max};
+    if (!launch_fwd<false, STORE_TRAJ>(a, d, batch_size))
+        unsupported("delta_forward_f32_cuda", d, coupled_needed(error_clip, m_norm_max));
+}
+
+void dgd_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                          const float *alpha, const float *theta, const float *m_initial,
+                          float *m_states, float *y, int seq_len, int d, int batch_size,
+                          int input_stride, int m_stride, float error_clip) {
+    // Same update as the Delta rule without the M-norm projection
+    // (core/kernels/dgd_forward.cu:6-11).
+    delta_forward_f32_cuda(k_mem, v_mem, q_mem, alpha, theta, m_initial, m_states, y, seq_len, d,
+                           batch_size, input_stride, m_stride, error_clip, 0.0f);
+}
+
+static int n_ckpt(int seq_len, int c) {  // core/src/gpu_forward.rs:2885-2897
+    int n = 1;
+    for (int t = 0; t < seq_len; t++) n += (((t + 1) % c == 0) || (t + 1 == seq_len));
+    return n;
+}
+
+void titans_forward_ckpt_batched_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                          const float *alpha, const float *theta, const float *eta,
+                                          const float *m_initial, const float *s_initial,
+                                          float *m_ckpt, float *s_ckpt, float *y,
+                                          int seq_len, int d, int batch_size, int checkpoint_interval,
+                                          float error_clip, float m_norm_max) {
+    if (!check_dims("titans_forward_ckpt", seq_len, d, batch_size) || batch_size == 0) return;
+    if (checkpoint_interval <= 0) { fail("titans_forward_ckpt: checkpoint_interval=%d must be > 0.", checkpoint_interval); return; }
+    FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial, m_ckpt, s_ckpt, y,
+              seq_len, seq_len, checkpoint_interval, 1, (long long)d * d,
+              (long long)n_ckpt(seq_len, checkpoint_interval) * d * d, error_clip, m_norm_max};
+    if (!launch_fwd<true, STORE_CKPT>(a, d, batch_size))
+        unsupported("titans_forward_ckpt", d, coupled_needed(error_clip, m_norm_max));
+}
+
+void delta_forward_ckpt_batched_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                         const float *alpha, const float *theta,
+                                         const float *m_initial, float *m_ckpt, float *y,
+                                         int seq_len, int d, int batch_size, int checkpoint_interval,
+                                         float error_clip, float m_norm_max) {
+    if (!check_dims("delta_forward_ckpt", seq_len, d, batch_size) || batch_size == 0) return;
+    if (checkpoint_interval <= 0) { fail("delta_forward_ckpt: checkpoint_interval=%d must be > 0.", checkpoint_interval); return; }
+    FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial, nullptr, m_ckpt, nullptr, y,
+              seq_len, seq_len, checkpoint_interval, 1, (long long)d * d,
+              (long long)n_ckpt(seq_len, checkpoint_interval) * d * d, error_clip, m_norm_max};
+    if (!launch_fwd<false, STORE_CKPT>(a, d, batch_size))
+        unsupported("delta_forward_ckpt", d, coupled_needed(error_clip, m_norm_max));
+}
+
+void titans_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                  const float *alpha, const float *theta, const float *eta,
+                                  const float *m_initial, const float *s_initial,
+                                  float *m_states, float *s_states, float *y,
+                                  int seq_len, int d, int checkpoint_interval, float error_clip,
+                                  float m_norm_max) {
+    titans_forward_ckpt_batched_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial,
+                                         m_states, s_states, y, seq_len, d, 1, checkpoint_interval,
+                                         error_clip, m_norm_max);
+}
+
+void delta_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                 const float *alpha, const float *theta, const float *m_initial,
+                                 float *m_states, float *y, int seq_len, int d,
+                                 int checkpoint_interval, float error_clip, float m_norm_max) {
+    delta_forward_ckpt_batched_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, m_initial, m_states, y,
+                                        seq_len, d, 1, checkpoint_interval, error_clip, m_norm_max);
+}
+
+void dgd_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                               const float *alpha, const float *theta, const float *m_initial,
+                               float *m_states, float *y, int seq_len, int d,
+                               int checkpoint_interval, float error_clip) {
+    delta_forward_ckpt_batched_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, m_initial, m_states, y,
+                                        seq_len, d, 1, checkpoint_interval, error_clip, 0.0f);
+}
+
+void titans_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                      const float *alpha, const float *theta, const float *eta,
+                                      const float *m_states, const float *s_states, const float *d_y,
+                                      const float *d_m_seed, const float *d_s_seed,
+                                      float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                      float *d_alpha, float *d_theta, float *d_eta,
+                                      float *d_m_out, float *d_s_out,
+                                      int t_start, int t_end, int d, int batch_size, int seq_len,
+                                      float error_clip) {
+    if (!check_dims("titans_backward_segment_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
+    if (t_start < 0 || t_end < t_start || t_end > seq_len) {
+        fail("titans_backward_segment_f32_cuda: bad range [%d,%d) for seq_len=%d.", t_start, t_end, seq_len);
+        return;
+    }
+    BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_states, s_states, d_y, d_m_seed, d_s_seed,
+              d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
+              d_m_out, d_s_out, seq_len, t_start, t_end, 1, batch_size,
+              (long long)(t_end - t_start + 1) * d * d, error_clip};
+    if (!launch_bwd<true>(a, d)) unsupported("titans_backward_segment_f32_cuda", d, error_clip > 0.f);
+}
+
+void delta_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                     const float *alpha, const float *theta,
+                                     const float *m_states, const float *d_y, const float *d_m_seed,
+                                     float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                     float *d_alpha, float *d_theta, float *d_m_out,
+                                     int t_start, int t_end, int d, int batch_size, int seq_len,
+                                     float error_clip) {
+    if (!check_dims("delta_backward_segment_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
+    if (t_start < 0 || t_end < t_start || t_end > seq_len) {
+        fail("delta_backward_segment_f32_cuda: bad range [%d,%d) for seq_len=%d.", t_start, t_end, seq_len);
+        return;
+    }
+    BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_states, nullptr, d_y, d_m_seed, nullptr,
+              d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr, nullptr, nullptr, nullptr,
+              d_m_out, nullptr, seq_len, t_start, t_end, 1, batch_size,
+              (long long)(t_end - t_start + 1) * d * d, error_clip};
+    if (!launch_bwd<false>(a, d)) unsupported("delta_backward_segment_f32_cuda", d, error_clip > 0.f);
+}
+
+void dgd_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                   const float *alpha, const float *theta,
+                                   const float *m_states, const float *d_y, const float *d_m_seed,
+                                   float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                   float *d_alpha, float *d_theta, float *d_m_out,
+                                   int t_start, int t_end, int d, int batch_size, int seq_len,
+                                   float error_clip) {
+    delta_backward_segment_f32_cuda(k_mem, v_mem, q_mem, alpha, theta, m_states, d_y, d_m_seed,
+                                    d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_m_out,
+                                    t_start, t_end, d, batch_size, seq_len, error_clip);
+}
+
+void titans_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                              const float *alpha, const float *theta, const float *eta,
+                              const float *m_states, const float *s_states, const float *d_y,
+                              float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                              float *d_alpha, float *d_theta, float *d_eta,
+                              float *d_m_initial, float *d_s_initial,
+                              int seq_len, int d, int batch_size, float error_clip) {
+    if (!check_dims("titans_backward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
+    const size_t dd = (size_t)d * d;
+    float *dm = scratch(0, (size_t)batch_size * dd * sizeof(float));
+    float *ds = scratch(1, (size_t)batch_size * dd * sizeof(float));
+    if (failed()) return;
+    BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_states, s_states, d_y, nullptr, nullptr,
+              d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
+              dm, ds, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
+    if (!launch_bwd<true>(a, d)) { unsupported("titans_backward_f32_cuda", d, error_clip > 0.f); return; }
+    accumulate_over_batch(dm, d_m_initial, batch_size, (int)dd);
+    accumulate_over_batch(ds, d_s_initial, batch_size, (int)dd);
+}
+
+void delta_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                             const float *alpha, const float *theta,
+                             const float *m_states, const float *d_y,
+                             float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                             float *d_alpha, float *d_theta, float *d_m_initial,
+                             int seq_len, int d, int batch_size, float error_clip) {
+    if (!check_dims("delta_backward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
+    const size_t dd = (size_t)d * d;
+    float *dm = scratch(0, (size_t)batch_size * dd * sizeof(float));
+    if (failed()) return;
+    BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_states, nullptr, d_y, nullptr, nullptr,
+              d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr, nullptr, nullptr, nullptr,
+              dm, nullptr, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
+    if (!launch_bwd<false>(a, d)) { unsupported("delta_backward_f32_cuda", d, error_clip > 0.f); return; }
+    accumulate_over_batch(dm, d_m_initial, batch_size, (int)dd);
+}
+
+void dgd_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                           const float *alpha, const float *theta,
+                           const float *m_states, const float *d_y,
+                           float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                           float *d_alpha, float *d_theta, float *d_m_initial,
+                           int seq_len, int d, float error_clip) {
+    // Single chain: the reference entry point has no batch argument
+    // (core/src/cuda_ffi.rs:309-326).
+    delta_backward_f32_cuda(k_mem, v_mem, q_mem, alpha, theta, m_states, d_y, d_k_mem, d_v_mem,
+                            d_q_mem, d_alpha, d_theta, d_m_initial, seq_len, d, 1, error_clip);
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+#include "runtime.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../../include/nl_hecate_ffi.h"
+
+namespace nlh {
+
+static int g_error_mode = 0;
+static bool g_failed = false;
+static char g_error[512] = "";
+static hipStream_t g_stream = nullptr;
+
+struct Slot {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+    int device = -1;
+};
+static Slot g_slots[kScratchSlots];
+
+void fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    g_failed = true;
+    if (g_error_mode == 0) {
+        fprintf(stderr, "[nl_hecate_rocm FATAL] %s\n", g_error);
+        abort();
+    }
+}
+
+bool failed() { return g_failed; }
+
+void check_hip(hipError_t e, const char *what) {
+    if (e != hipSuccess) fail("%s: %s", what, hipGetErrorString(e));
+}
+
+void check_launch(const char *kernel) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) fail("%s launch failed: %s", kernel, hipGetErrorString(e));
+}
+
+hipStream_t stream() { return g_stream; }
+
+float *scratch(int slot, size_t bytes) {
+    if (slot < 0 || slot >= kScratchSlots) {
+        fail("scratch slot %d out of range", slot);
+        return nullptr;
+    }
+    int dev = 0;
+    check_hip(hipGetDevice(&dev), "hipGetDevice");
+    Slot &s = g_slots[slot];
+    if (s.ptr && (s.device != dev || s.bytes < bytes)) {
+        // Earlier launches may still read the old buffer.
+        check_hip(hipDeviceSynchronize(), "scratch: hipDeviceSynchronize");
+        check_hip(hipFree(s.ptr), "scratch: hipFree");
+        s = Slot();
+    }
+    if (!s.ptr) {
+        size_t want = bytes < 256 ? 256 : bytes;
+        check_hip(hipMalloc(&s.ptr, want), "scratch: hipMalloc");
+        s.bytes = want;
+        s.device = dev;
+    }
+    return (float *)s.ptr;
+}
+
+}  // namespace nlh
+
+extern "C" {
+
+void nlh_set_error_mode(int mode) { nlh::g_error_mode = mode ? 1 : 0; }
+
+const char *nlh_last_error(void) { return nlh::g_failed ? nlh::g_error : ""; }
+
+void nlh_clear_error(void) {
+    nlh::g_failed = false;
+    nlh::g_error[0] = 0;
+}
+
+void nlh_set_stream(void *hip_stream) { nlh::g_stream = (hipStream_t)hip_stream; }
+
+void nlh_release_workspace(void) {
+    for (auto &s : nlh::g_slots) {
+        if (s.ptr) {
+            (void)hipDeviceSynchronize();
+            (void)hipFree(s.ptr);
+        }
+        s = nlh::Slot();
+    }
+}
+
+const char *nlh_version(void) { return "nl_hecate_rocm 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,76 @@
+// On-device check of the cross-lane primitives against host arithmetic.
+#include <hip/hip_runtime.h>
+
+#include <stdio.h>
+
+#include <vector>
+
+#include "../../include/nl_hecate_ffi.h"
+#include "lane_ops.h"
+#include "runtime.h"
+
+namespace nlh {
+
+// out[0..5][64]: group sums for G=4,16,64; stride sums for LPR=16, 2; swapadd32(a,b)
+__global__ void lane_ops_kernel(const float *in, const float *in2, float *out) {
+    int l = threadIdx.x;
+    float x = in[l], y = in2[l];
+    out[0 * 64 + l] = group_allreduce<4>(x);
+    out[1 * 64 + l] = group_allreduce<16>(x);
+    out[2 * 64 + l] = group_allreduce<64>(x);
+    out[3 * 64 + l] = stride_allreduce<16>(x);
+    out[4 * 64 + l] = stride_allreduce<2>(x);
+    out[5 * 64 + l] = swapadd32(x, y);
+    out[6 * 64 + l] = swapadd16(x, y);
+    out[7 * 64 + l] = stride_allreduce<8>(x);
+    out[8 * 64 + l] = group_allreduce<8>(x);
+    out[9 * 64 + l] = group_allreduce<32>(x);
+}
+
+}  // namespace nlh
+
+extern "C" int nlh_selftest_lane_ops(void) {
+    using namespace nlh;
+    const int NT = 10;
+    std::vector<float> a(64), b(64), o(NT * 64);
+    // small integers: every sum is exact, so results compare with ==
+    for (int i = 0; i < 64; i++) { a[i] = (float)((i * 37 + 11) % 23 - 9); b[i] = (float)((i * 53 + 5) % 31 - 13); }
+    float *din, *din2, *dout;
+    if (hipMalloc(&din, 256) != hipSuccess || hipMalloc(&din2, 256) != hipSuccess ||
+        hipMalloc(&dout, NT * 256) != hipSuccess) return -1;
+    (void)hipMemcpy(din, a.data(), 256, hipMemcpyHostToDevice);
+    (void)hipMemcpy(din2, b.data(), 256, hipMemcpyHostToDevice);
+    hipLaunchKernelGGL(lane_ops_kernel, dim3(1), dim3(64), 0, stream(), din, din2, dout);
+    if (hipDeviceSynchronize() != hipSuccess) return -2;
+    (void)hipMemcpy(o.data(), dout, NT * 256, hipMemcpyDeviceToHost);
+    (void)hipFree(din); (void)hipFree(din2); (void)hipFree(dout);
+    int bad = 0;
+    std::vector<float> want(NT * 64);
+    auto gsum = [&](int l, int G) { float s = 0; for (int j = (l / G) * G; j < (l / G + 1) * G; j++) s += a[j]; return s; };
+    auto ssum = [&](int l, int LPR) { float s = 0; for (int j = l % LPR; j < 64; j += LPR) s += a[j]; return s; };
+    for (int l = 0; l < 64; l++) {
+        want[0 * 64 + l] = gsum(l, 4);
+        want[1 * 64 + l] = gsum(l, 16);
+        want[2 * 64 + l] = gsum(l, 64);
+        want[3 * 64 + l] = ssum(l, 16);
+        want[4 * 64 + l] = ssum(l, 2);
+        want[5 * 64 + l] = l < 32 ? a[l] + a[l + 32] : b[l - 32] + b[l];
+        int row = l / 16, c = l % 16;
+        want[6 * 64 + l] = (row % 2 == 0) ? a[row * 16 + c] + a[(row + 1) * 16 + c]
+                                          : b[(row - 1) * 16 + c] + b[row * 16 + c];
+        want[7 * 64 + l] = ssum(l, 8);
+        want[8 * 64 + l] = gsum(l, 8);
+        want[9 * 64 + l] = gsum(l, 32);
+    }
+    for (int t = 0; t < NT; t++) {
+        int nb = 0;
+        for (int l = 0; l < 64; l++) nb += o[t * 64 + l] != want[t * 64 + l];
+        if (nb) {
+            fprintf(stderr, "lane-op selftest %d: %d lanes differ; got/want:", t, nb);
+            for (int l = 0; l < 64; l++) fprintf(stderr, " %g/%g", o[t * 64 + l], want[t * 64 + l]);
+            fprintf(stderr, "\n");
+        }
+        bad += nb;
+    }
+    return bad;
+}
