@@ -153,6 +153,50 @@ void delta_forward_ckpt_batched_f32_rocm(const float *k_mem, const float *v_mem,
                                          int seq_len, int d, int batch_size, int checkpoint_interval,
                                          float error_clip, float m_norm_max);
 
+
+/* ── Checkpointed backward (addition) ───────────────────────────────────────
+ * Replaces the host loop titans_backward_checkpointed /
+ * delta_backward_checkpointed (core/src/gpu_backward.rs:1770-1962): one call
+ * walks the C-token segments in reverse.  m_ckpt / s_ckpt are the output of
+ * the batched checkpointed forward; gradients have the layout of
+ * *_backward_f32_cuda, including the accumulate-over-batch contract of
+ * d_m_initial / d_s_initial.
+ * `_replay_`: replays every segment through a scratch trajectory in device
+ * memory, the reference's schedule without its host synchronisations. */
+void titans_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                          const float *alpha, const float *theta, const float *eta,
+                                          const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                                          float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                          float *d_alpha, float *d_theta, float *d_eta,
+                                          float *d_m_initial, float *d_s_initial,
+                                          int seq_len, int d, int batch_size, int checkpoint_interval,
+                                          float error_clip, float m_norm_max);
+void delta_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                         const float *alpha, const float *theta,
+                                         const float *m_ckpt, const float *d_y,
+                                         float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                         float *d_alpha, float *d_theta, float *d_m_initial,
+                                         int seq_len, int d, int batch_size, int checkpoint_interval,
+                                         float error_clip, float m_norm_max);
+/* Fused form: the replayed trajectory stays in LDS and registers (two-level
+ * recomputation inside one kernel); takes the `_replay_` schedule instead when
+ * clip / projection is active or checkpoint_interval > 64. */
+void titans_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                   const float *alpha, const float *theta, const float *eta,
+                                   const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                                   float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                   float *d_alpha, float *d_theta, float *d_eta,
+                                   float *d_m_initial, float *d_s_initial,
+                                   int seq_len, int d, int batch_size, int checkpoint_interval,
+                                   float error_clip, float m_norm_max);
+void delta_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                  const float *alpha, const float *theta,
+                                  const float *m_ckpt, const float *d_y,
+                                  float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                  float *d_alpha, float *d_theta, float *d_m_initial,
+                                  int seq_len, int d, int batch_size, int checkpoint_interval,
+                                  float error_clip, float m_norm_max);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,52 +24,9 @@
 #include <math.h>
 
 #include "../../include/nl_hecate_ffi.h"
-#include "lane_ops.h"
-#include "rule_tiles.h"
-#include "runtime.h"
+#include "rule_common.h"
 
 namespace nlh {
-
-constexpr int TB = 16;  // tokens per LDS tile
-
-// blockIdx -> (chain, part).  Workgroups are dealt round-robin to the 8 XCDs, so
-// consecutive block ids land on different L2s; remap so that the parts of one
-// chain (which read the same k/q rows) share an XCD.
-__device__ __forceinline__ void map_block(int parts, int &chain, int &part) {
-    int n = blockIdx.x, nb = gridDim.x, L = n;
-    if (nb % 8 == 0) L = (n % 8) * (nb / 8) + n / 8;
-    chain = L / parts;
-    part = L % parts;
-}
-
-__device__ __forceinline__ bool mnorm_active(float m_norm_max) {
-    return m_norm_max > 0.f && m_norm_max < 1e30f;  // core/kernels/m_norm_project.cuh:27
-}
-
-__device__ __forceinline__ float4 f4_zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
-__device__ __forceinline__ float4 f4_scale(float a, const float4 &x) {
-    return make_float4(a * x.x, a * x.y, a * x.z, a * x.w);
-}
-// a*x + b*y
-__device__ __forceinline__ float4 f4_axpby(float a, const float4 &x, float b, const float4 &y) {
-    return make_float4(a * x.x + b * y.x, a * x.y + b * y.y, a * x.z + b * y.z, a * x.w + b * y.w);
-}
-__device__ __forceinline__ void f4_fma(float4 &acc, float a, const float4 &x) {
-    acc.x += a * x.x; acc.y += a * x.y; acc.z += a * x.z; acc.w += a * x.w;
-}
-__device__ __forceinline__ void f4_add(float4 &acc, const float4 &x) {
-    acc.x += x.x; acc.y += x.y; acc.z += x.z; acc.w += x.w;
-}
-
-// Workgroup-wide sum of one float per lane (COUPLED kernels only: every wave of
-// the workgroup must call it).  `slot` points at kWaves floats of LDS that no
-// other reduction uses until the next barrier after this one.
-__device__ __forceinline__ float block_allreduce(float x, float *slot, int tid) {
-    x = wave_allreduce(x);
-    if ((tid & 63) == 0) slot[tid >> 6] = x;
-    __syncthreads();
-    return slot[0] + slot[1] + slot[2] + slot[3];
-}
 
 // ───────────────────────────── forward ─────────────────────────────────────
 struct FwdArgs {
@@ -529,7 +486,16 @@ __global__ void accumulate_over_batch_kernel(const float *src, float *dst, int b
 }
 
 // ───────────────────────────── host dispatch ───────────────────────────────
-static bool coupled_needed(float error_clip, float m_norm_max) {
+void finalize_parts(const float *ws_dq, const float *ws_dk, const float *ws_gate,
+                    float *d_q, float *d_k, float *d_alpha, float *d_theta, float *d_eta,
+                    int parts, int batch, int seq_len, int d, int t_start, int t_end) {
+    dim3 grid(ceil_div((long long)(t_end - t_start) * d, 256), batch);
+    hipLaunchKernelGGL(finalize_parts_kernel, grid, dim3(256), 0, stream(), ws_dq, ws_dk, ws_gate,
+                       d_q, d_k, d_alpha, d_theta, d_eta, parts, batch, seq_len, d, t_start, t_end);
+    check_launch("finalize_parts_kernel");
+}
+
+bool coupled_needed(float error_clip, float m_norm_max) {
     return error_clip > 0.f || (m_norm_max > 0.f && m_norm_max < 1e30f);
 }
 
@@ -611,31 +577,87 @@ static bool launch_bwd(BwdArgs a, int d) {
         case 128: launch_bwd_c<128, 4, HAS_S>(a, false); break;
         default: return false;
     }
-    if (a.parts > 1 && a.t_end > a.t_start) {
-        dim3 grid(ceil_div((long long)(a.t_end - a.t_start) * d, 256), a.batch);
-        hipLaunchKernelGGL(finalize_parts_kernel, grid, dim3(256), 0, stream(), a.ws_dq, a.ws_dk,
-                           a.ws_gate, a.d_q, a.d_k, a.d_alpha, a.d_theta, HAS_S ? a.d_eta : nullptr,
-                           a.parts, a.batch, a.seq_len, d, a.t_start, a.t_end);
-        check_launch("finalize_parts_kernel");
-    }
+    if (a.parts > 1 && a.t_end > a.t_start)
+        finalize_parts(a.ws_dq, a.ws_dk, a.ws_gate, a.d_q, a.d_k, a.d_alpha, a.d_theta,
+                       HAS_S ? a.d_eta : nullptr, a.parts, a.batch, a.seq_len, d, a.t_start, a.t_end);
     return true;
 }
 
-static void accumulate_over_batch(const float *src, float *dst, int batch, int n) {
+void accumulate_over_batch(const float *src, float *dst, int batch, int n) {
     hipLaunchKernelGGL(accumulate_over_batch_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream(),
                        src, dst, batch, n);
     check_launch("accumulate_over_batch_kernel");
 }
 
-static bool check_dims(const char *fn, int seq_len, int d, int batch) {
+int n_ckpt_count(int seq_len, int c) {  // core/src/gpu_forward.rs:2885-2897
+    int n = 1;
+    for (int t = 0; t < seq_len; t++) n += (((t + 1) % c == 0) || (t + 1 == seq_len));
+    return n;
+}
+
+bool check_dims(const char *fn, int seq_len, int d, int batch) {
     if (d <= 0) { fail("%s: d=%d must be > 0.", fn, d); return false; }
     if (seq_len < 0 || batch < 0) { fail("%s: seq_len=%d batch=%d must be >= 0.", fn, seq_len, batch); return false; }
     return true;
 }
 
-static void unsupported(const char *fn, int d, bool coupled) {
+void unsupported(const char *fn, int d, bool coupled) {
     fail("%s: d=%d%s is not supported by the gfx950 kernels (d in {8,16,32,64,128}; "
          "clip / M-norm projection need d <= 64).", fn, d, coupled ? " with clip/projection" : "");
+}
+
+
+// ── Checkpointed backward, replay-through-memory schedule ───────────────────
+// The schedule of titans_backward_checkpointed / delta_backward_checkpointed
+// (core/src/gpu_backward.rs:1770-1962) run inside the library: for each
+// C-token segment in reverse, replay the forward from the segment's checkpoint
+// into a scratch trajectory, then run the segment backward seeded by the later
+// segment.  No host synchronisation between segments: stream order suffices.
+template <bool HAS_S>
+static void backward_ckpt_replay(const float *k, const float *v, const float *q,
+                                 const float *alpha, const float *theta, const float *eta,
+                                 const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                                 float *d_k, float *d_v, float *d_q,
+                                 float *d_alpha, float *d_theta, float *d_eta,
+                                 float *d_m_initial, float *d_s_initial,
+                                 int seq_len, int d, int batch, int C,
+                                 float error_clip, float m_norm_max, const char *fn) {
+    const size_t dd = (size_t)d * d;
+    const int nck = n_ckpt_count(seq_len, C);
+    const int max_seg = C < seq_len ? C : seq_len;
+    const size_t traj = (size_t)batch * (max_seg + 1) * dd * sizeof(float);
+    float *lm = scratch(5, traj);
+    float *ls = HAS_S ? scratch(6, traj) : nullptr;
+    float *ly = scratch(7, (size_t)batch * max_seg * d * sizeof(float));
+    float *seed_m = scratch(8, 2 * batch * dd * sizeof(float));
+    float *seed_s = HAS_S ? scratch(9, 2 * batch * dd * sizeof(float)) : nullptr;
+    if (failed()) return;
+    check_hip(hipMemsetAsync(seed_m, 0, batch * dd * sizeof(float), stream()), "memset seed");
+    if (HAS_S) check_hip(hipMemsetAsync(seed_s, 0, batch * dd * sizeof(float), stream()), "memset seed");
+    const int nseg = ceil_div(seq_len, C);
+    int cur = 0;
+    for (int g = nseg - 1; g >= 0; g--) {
+        const int t0 = g * C, t1 = (t0 + C < seq_len) ? t0 + C : seq_len, seg = t1 - t0;
+        FwdArgs fa{k + (size_t)t0 * d, v + (size_t)t0 * d, q + (size_t)t0 * d, alpha + t0, theta + t0,
+                   HAS_S ? eta + t0 : nullptr, m_ckpt + (size_t)g * dd,
+                   HAS_S ? s_ckpt + (size_t)g * dd : nullptr, lm, ls, ly,
+                   seg, seq_len, 1, 1, (long long)(nck * dd), (long long)((seg + 1) * dd),
+                   error_clip, m_norm_max};
+        if (!launch_fwd<HAS_S, STORE_TRAJ>(fa, d, batch)) {
+            unsupported(fn, d, coupled_needed(error_clip, m_norm_max));
+            return;
+        }
+        float *out_m = seed_m + (size_t)(cur ^ 1) * batch * dd;
+        float *out_s = HAS_S ? seed_s + (size_t)(cur ^ 1) * batch * dd : nullptr;
+        BwdArgs ba{k, v, q, alpha, theta, eta, lm, ls, d_y,
+                   seed_m + (size_t)cur * batch * dd, HAS_S ? seed_s + (size_t)cur * batch * dd : nullptr,
+                   d_k, d_v, d_q, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
+                   out_m, out_s, seq_len, t0, t1, 1, batch, (long long)((seg + 1) * dd), error_clip};
+        if (!launch_bwd<HAS_S>(ba, d)) { unsupported(fn, d, error_clip > 0.f); return; }
+        cur ^= 1;
+    }
+    accumulate_over_batch(seed_m + (size_t)cur * batch * dd, d_m_initial, batch, (int)dd);
+    if (HAS_S) accumulate_over_batch(seed_s + (size_t)cur * batch * dd, d_s_initial, batch, (int)dd);
 }
 
 }  // namespace nlh
@@ -681,11 +703,7 @@ void dgd_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q
                            batch_size, input_stride, m_stride, error_clip, 0.0f);
 }
 
-static int n_ckpt(int seq_len, int c) {  // core/src/gpu_forward.rs:2885-2897
-    int n = 1;
-    for (int t = 0; t < seq_len; t++) n += (((t + 1) % c == 0) || (t + 1 == seq_len));
-    return n;
-}
+static int n_ckpt(int seq_len, int c) { return n_ckpt_count(seq_len, c); }
 
 void titans_forward_ckpt_batched_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
                                           const float *alpha, const float *theta, const float *eta,
@@ -842,6 +860,39 @@ void dgd_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *
     // (core/src/cuda_ffi.rs:309-326).
     delta_backward_f32_cuda(k_mem, v_mem, q_mem, alpha, theta, m_states, d_y, d_k_mem, d_v_mem,
                             d_q_mem, d_alpha, d_theta, d_m_initial, seq_len, d, 1, error_clip);
+}
+
+void titans_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                          const float *alpha, const float *theta, const float *eta,
+                                          const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                                          float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                          float *d_alpha, float *d_theta, float *d_eta,
+                                          float *d_m_initial, float *d_s_initial,
+                                          int seq_len, int d, int batch_size, int checkpoint_interval,
+                                          float error_clip, float m_norm_max) {
+    const char *fn = "titans_backward_ckpt_replay_f32_rocm";
+    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0 || seq_len == 0) return;
+    if (checkpoint_interval <= 0) { fail("%s: checkpoint_interval=%d must be > 0.", fn, checkpoint_interval); return; }
+    backward_ckpt_replay<true>(k_mem, v_mem, q_mem, alpha, theta, eta, m_ckpt, s_ckpt, d_y,
+                               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
+                               d_m_initial, d_s_initial, seq_len, d, batch_size,
+                               checkpoint_interval, error_clip, m_norm_max, fn);
+}
+
+void delta_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                         const float *alpha, const float *theta,
+                                         const float *m_ckpt, const float *d_y,
+                                         float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                         float *d_alpha, float *d_theta, float *d_m_initial,
+                                         int seq_len, int d, int batch_size, int checkpoint_interval,
+                                         float error_clip, float m_norm_max) {
+    const char *fn = "delta_backward_ckpt_replay_f32_rocm";
+    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0 || seq_len == 0) return;
+    if (checkpoint_interval <= 0) { fail("%s: checkpoint_interval=%d must be > 0.", fn, checkpoint_interval); return; }
+    backward_ckpt_replay<false>(k_mem, v_mem, q_mem, alpha, theta, nullptr, m_ckpt, nullptr, d_y,
+                                d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr,
+                                d_m_initial, nullptr, seq_len, d, batch_size,
+                                checkpoint_interval, error_clip, m_norm_max, fn);
 }
 
 }  // extern "C"

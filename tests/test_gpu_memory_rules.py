@@ -321,3 +321,73 @@ def test_argument_errors_are_reported():
     finally:
         lib.nlh_clear_error()
         lib.nlh_set_error_mode(0)
+
+
+# ── one-call checkpointed backward: fused (on-chip replay) and replay schedule ──
+def _oracle_ckpt_grads(x, C, has_s, clip=0.0, mx=F32_MAX):
+    B, s, d = x["k"].shape
+    outs = []
+    for b in range(B):
+        y, mc, sc = orc.forward_ckpt(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b],
+                                     x["eta"][b], x["m0"][b], x["s0"][b], C, has_s, clip, mx)
+        outs.append(orc.backward_ckpt(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b],
+                                      x["eta"][b], mc, sc, x["dy"][b], C, has_s, clip, mx))
+    g = {n: np.stack([o[n] for o in outs]) for n in outs[0] if n not in ("d_m", "d_s")}
+    g["d_m_initial"] = sum(o["d_m"] for o in outs)
+    g["d_s_initial"] = sum(o["d_s"] for o in outs)
+    return g
+
+
+def _gpu_ckpt_fwd_bwd(x, C, has_s, entry, clip=0.0, mx=F32_MAX):
+    B, s, d = x["k"].shape
+    n = orc.checkpoint_count(s, C)
+    k, v, q, dy = dev(x["k"]), dev(x["v"]), dev(x["q"]), dev(x["dy"])
+    al, th, et = dev(x["alpha"]), dev(x["theta"]), dev(x["eta"])
+    mc, sc, y = zeros(B, n, d, d), zeros(B, n, d, d), zeros(B, s, d)
+    g = dict(d_k=zeros(B, s, d), d_v=zeros(B, s, d), d_q=zeros(B, s, d), d_alpha=zeros(B, s),
+             d_theta=zeros(B, s), d_m_initial=zeros(d, d))
+    if has_s:
+        g.update(d_eta=zeros(B, s), d_s_initial=zeros(d, d))
+        D.call("titans_forward_ckpt_batched_f32_rocm", k, v, q, al, th, et, dev(x["m0"]), dev(x["s0"]),
+               mc, sc, y, s, d, B, C, clip, mx)
+        D.call("titans_backward_ckpt" + entry + "_f32_rocm", k, v, q, al, th, et, mc, sc, dy,
+               g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"],
+               g["d_m_initial"], g["d_s_initial"], s, d, B, C, clip, mx)
+    else:
+        D.call("delta_forward_ckpt_batched_f32_rocm", k, v, q, al, th, dev(x["m0"]), mc, y,
+               s, d, B, C, clip, mx)
+        D.call("delta_backward_ckpt" + entry + "_f32_rocm", k, v, q, al, th, mc, dy,
+               g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_m_initial"],
+               s, d, B, C, clip, mx)
+    torch.cuda.synchronize()
+    return {n_: host(t) for n_, t in g.items()}
+
+
+@pytest.mark.parametrize("entry", ["", "_replay"])
+@pytest.mark.parametrize("B,s,d,C", [(3, 200, 64, 64), (2, 19, 64, 5), (2, 77, 64, 64), (3, 50, 16, 8),
+                                     (2, 40, 32, 16), (2, 30, 128, 64), (1, 130, 8, 64),
+                                     (2, 150, 64, 100), (2, 9, 64, 1), (5, 64, 64, 64)])
+def test_checkpointed_backward_one_call(entry, B, s, d, C):
+    x = rule_inputs(B, s, d, 7000 + s + d + C, m0_scale=0.2)
+    for has_s in (True, False):
+        g = _gpu_ckpt_fwd_bwd(x, C, has_s, entry)
+        go = _oracle_ckpt_grads(x, C, has_s)
+        for n in g:
+            assert_close(f"{n} has_s={has_s}", g[n], go[n])
+
+
+def test_checkpointed_backward_with_clip_takes_replay_schedule():
+    x = rule_inputs(2, 40, 64, 7100, m0_scale=0.3)
+    x["v"] *= 2.0
+    g = _gpu_ckpt_fwd_bwd(x, 16, True, "", clip=0.7, mx=1.5)
+    go = _oracle_ckpt_grads(x, 16, True, 0.7, 1.5)
+    for n in g:
+        assert_close(n, g[n], go[n])
+
+
+def test_checkpointed_backward_is_deterministic():
+    x = rule_inputs(4, 130, 64, 7200, m0_scale=0.2)
+    g1 = _gpu_ckpt_fwd_bwd(x, 64, True, "")
+    g2 = _gpu_ckpt_fwd_bwd(x, 64, True, "")
+    for n in g1:
+        assert np.array_equal(g1[n], g2[n]), n
