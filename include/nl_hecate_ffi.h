@@ -33,6 +33,10 @@ const char *nlh_last_error(void);      /* "" when no error is recorded */
 void nlh_clear_error(void);
 void nlh_set_stream(void *hip_stream); /* hipStream_t; NULL = null stream */
 void nlh_release_workspace(void);      /* frees the library's device scratch */
+/* hipEvent pair on the launch stream: start, then stop returns elapsed ms
+ * (blocks until the stop event completes); negative on failure. */
+int nlh_timer_start(void);
+float nlh_timer_stop_ms(void);
 /* Runs the cross-lane primitives on known data; returns 0 when all agree. */
 int nlh_selftest_lane_ops(void);
 

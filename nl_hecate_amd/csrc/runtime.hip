@@ -94,6 +94,23 @@ void nlh_release_workspace(void) {
     }
 }
 
+// Event timer on the launch stream (one outstanding interval at a time).
+static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+
+int nlh_timer_start(void) {
+    if (!g_ev0 && (hipEventCreate(&g_ev0) != hipSuccess || hipEventCreate(&g_ev1) != hipSuccess)) return -1;
+    return hipEventRecord(g_ev0, nlh::stream()) == hipSuccess ? 0 : -1;
+}
+
+float nlh_timer_stop_ms(void) {
+    float ms = -1.f;
+    if (!g_ev0) return ms;
+    if (hipEventRecord(g_ev1, nlh::stream()) != hipSuccess) return ms;
+    if (hipEventSynchronize(g_ev1) != hipSuccess) return ms;
+    if (hipEventElapsedTime(&ms, g_ev0, g_ev1) != hipSuccess) return -1.f;
+    return ms;
+}
+
 const char *nlh_version(void) { return "nl_hecate_rocm 0.1 (gfx950)"; }
 
 }  // extern "C"
