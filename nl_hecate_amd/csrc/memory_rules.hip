@@ -23,6 +23,8 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 
+#include <type_traits>
+
 #include "../../include/nl_hecate_ffi.h"
 #include "rule_common.h"
 
@@ -46,6 +48,7 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
     constexpr int RG = 64 / LPR;        // row groups per wave
     constexpr int ROWS_WG = kWaves * RG * RPL;
     constexpr int DD = D * D;
+    constexpr bool ALL_VALID = (D % ROWS_WG) == 0;  // every lane owns real rows
 
     __shared__ __align__(16) float sk[2][TB * D];
     __shared__ __align__(16) float sq[2][TB * D];
@@ -75,7 +78,7 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
     bool valid[RPL];
 #pragma unroll
     for (int r = 0; r < RPL; r++) {
-        valid[r] = (row0 + r) < D;
+        valid[r] = ALL_VALID || (row0 + r) < D;
         M[r] = f4_zero();
         S[r] = f4_zero();
         if (valid[r]) {
@@ -128,78 +131,93 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
             rg.load(ab, tb, eb, t0 + TB, 0, seq_len, tid);
         }
         const int tn = min(TB, seq_len - t0);
-        for (int tl = 0; tl < tn; tl++) {
-            const int t = t0 + tl;
-            const float4 kk = *reinterpret_cast<const float4 *>(&sk[buf][tl * D + cb * 4]);
-            const float4 qq = *reinterpret_cast<const float4 *>(&sq[buf][tl * D + cb * 4]);
-            const float al = sg[buf][tl], th = sg[buf][TB + tl], et = sg[buf][2 * TB + tl];
-            const float ret = 1.f - al;
-            float e[RPL];
+        // FAST: a full tile with no checkpoint boundary strictly inside it and no
+        // coupled reduction; the 16 tokens are straight-line code, so LDS reads
+        // of later tokens overlap the dependent chain of earlier ones.
+        auto run_tile = [&](auto fast_c) {
+            constexpr bool FAST = decltype(fast_c)::value;
 #pragma unroll
-            for (int r = 0; r < RPL; r++) {
-                float p = group_allreduce<LPR>(dot4(M[r], kk));
-                float vv = sv[buf][tl * D + (valid[r] ? row0 + r : 0)];
-                e[r] = valid[r] ? p - vv : 0.f;
-            }
-            if (COUPLED && clip_on) {
-                float sq_sum = 0.f;
+            for (int tl = 0; tl < TB; tl++) {
+                if (!FAST && tl >= tn) break;
+                const int t = t0 + tl;
+                const float4 kk = *reinterpret_cast<const float4 *>(&sk[buf][tl * D + cb * 4]);
+                const float4 qq = *reinterpret_cast<const float4 *>(&sq[buf][tl * D + cb * 4]);
+                const float al = sg[buf][tl], th = sg[buf][TB + tl], et = sg[buf][2 * TB + tl];
+                const float ret = 1.f - al;
+                float e[RPL];
 #pragma unroll
-                for (int r = 0; r < RPL; r++) sq_sum += e[r] * e[r];
-                if (cb != 0) sq_sum = 0.f;
-                float nrm = sqrtf(block_allreduce(sq_sum, sred[(t & 1) * 2], tid));
-                if (nrm > a.error_clip) {
-                    float sc = a.error_clip / nrm;
-#pragma unroll
-                    for (int r = 0; r < RPL; r++) e[r] *= sc;
+                for (int r = 0; r < RPL; r++) {
+                    float p = group_allreduce<LPR>(dot4(M[r], kk));
+                    float vv = sv[buf][tl * D + (valid[r] ? row0 + r : 0)];
+                    e[r] = valid[r] ? p - vv : 0.f;
                 }
-            }
+                if (COUPLED && clip_on) {
+                    float sq_sum = 0.f;
 #pragma unroll
-            for (int r = 0; r < RPL; r++) {
-                float te = th * e[r];
-                if (HAS_S) {
-                    S[r] = f4_axpby(et, S[r], -te, kk);
-                    M[r] = f4_axpby(ret, M[r], 1.f, S[r]);
-                } else {
-                    M[r] = f4_axpby(ret, M[r], -te, kk);
-                }
-            }
-            if (COUPLED && mn_on) {
-                float sq_sum = 0.f;
+                    for (int r = 0; r < RPL; r++) sq_sum += e[r] * e[r];
+                    if (cb != 0) sq_sum = 0.f;
+                    float nrm = sqrtf(block_allreduce(sq_sum, sred[(t & 1) * 2], tid));
+                    if (nrm > a.error_clip) {
+                        float sc = a.error_clip / nrm;
 #pragma unroll
-                for (int r = 0; r < RPL; r++) sq_sum += dot4(M[r], M[r]);
-                float fn = sqrtf(block_allreduce(sq_sum, sred[(t & 1) * 2 + 1], tid));
-                if (fn > a.m_norm_max) {
-                    float sc = a.m_norm_max / fn;
-#pragma unroll
-                    for (int r = 0; r < RPL; r++) M[r] = f4_scale(sc, M[r]);
-                }
-            }
-            if (STORE == STORE_TRAJ) {
-#pragma unroll
-                for (int r = 0; r < RPL; r++)
-                    if (valid[r]) {
-                        size_t off = (size_t)(t + 1) * DD + (size_t)(row0 + r) * D + cb * 4;
-                        *reinterpret_cast<float4 *>(mo + off) = M[r];
-                        if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
+                        for (int r = 0; r < RPL; r++) e[r] *= sc;
                     }
-            } else if (STORE == STORE_CKPT) {
-                if (((t + 1) % a.ckpt_interval == 0) || (t + 1 == seq_len)) {
+                }
+#pragma unroll
+                for (int r = 0; r < RPL; r++) {
+                    float te = th * e[r];
+                    if (HAS_S) {
+                        S[r] = f4_axpby(et, S[r], -te, kk);
+                        M[r] = f4_axpby(ret, M[r], 1.f, S[r]);
+                    } else {
+                        M[r] = f4_axpby(ret, M[r], -te, kk);
+                    }
+                }
+                if (COUPLED && mn_on) {
+                    float sq_sum = 0.f;
+#pragma unroll
+                    for (int r = 0; r < RPL; r++) sq_sum += dot4(M[r], M[r]);
+                    float fn = sqrtf(block_allreduce(sq_sum, sred[(t & 1) * 2 + 1], tid));
+                    if (fn > a.m_norm_max) {
+                        float sc = a.m_norm_max / fn;
+#pragma unroll
+                        for (int r = 0; r < RPL; r++) M[r] = f4_scale(sc, M[r]);
+                    }
+                }
+                if (STORE == STORE_TRAJ) {
 #pragma unroll
                     for (int r = 0; r < RPL; r++)
-                        if (valid[r]) {
-                            size_t off = (size_t)ckpt_slot * DD + (size_t)(row0 + r) * D + cb * 4;
+                        if (ALL_VALID || valid[r]) {
+                            size_t off = (size_t)(t + 1) * DD + (size_t)(row0 + r) * D + cb * 4;
                             *reinterpret_cast<float4 *>(mo + off) = M[r];
                             if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
                         }
-                    ckpt_slot++;
+                } else if (STORE == STORE_CKPT) {
+                    // in FAST tiles a boundary can only be the tile's last token
+                    if ((!FAST || tl == TB - 1) &&
+                        (((t + 1) % a.ckpt_interval == 0) || (t + 1 == seq_len))) {
+#pragma unroll
+                        for (int r = 0; r < RPL; r++)
+                            if (ALL_VALID || valid[r]) {
+                                size_t off = (size_t)ckpt_slot * DD + (size_t)(row0 + r) * D + cb * 4;
+                                *reinterpret_cast<float4 *>(mo + off) = M[r];
+                                if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
+                            }
+                        ckpt_slot++;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < RPL; r++) {
+                    float yy = group_allreduce<LPR>(dot4(M[r], qq));
+                    // all LPR lanes of the row hold yy: same-value store, no divergence
+                    sy[buf][tl * ROWS_WG + row_local + r] = yy;
                 }
             }
-#pragma unroll
-            for (int r = 0; r < RPL; r++) {
-                float yy = group_allreduce<LPR>(dot4(M[r], qq));
-                if (cb == 0) sy[buf][tl * ROWS_WG + row_local + r] = yy;
-            }
-        }
+        };
+        const bool fast = !COUPLED && tn == TB &&
+                          (STORE != STORE_CKPT || a.ckpt_interval % TB == 0);
+        if (fast) run_tile(std::true_type{});
+        else run_tile(std::false_type{});
     }
     __syncthreads();
     if (ntiles > 0) flush_y(ntiles - 1);

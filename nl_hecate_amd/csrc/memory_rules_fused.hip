@@ -24,6 +24,8 @@
 // replay-through-memory schedule instead.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../../include/nl_hecate_ffi.h"
 #include "rule_common.h"
 
@@ -47,6 +49,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
     constexpr int RG = 64 / LPR;
     constexpr int ROWS_WG = kWaves * RG;
     constexpr int DD = D * D;
+    constexpr bool ALL_VALID = (D % ROWS_WG) == 0;  // every lane owns a real row
 
     __shared__ __align__(16) float4 subck[NSUB_MAX][HAS_S ? 2 : 1][kThreads];
     __shared__ float ebuf[C_MAX * ROWS_WG];
@@ -57,15 +60,17 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
     __shared__ __align__(16) float sdq[2][SUB * kWaves * D];
     __shared__ __align__(16) float sdk[2][SUB * kWaves * D];
     __shared__ float sdv[2][SUB * ROWS_WG];
-    __shared__ float sgate[2][SUB * kWaves * 4];
+    constexpr int NG = HAS_S ? 3 : 2;  // gate gradients per token: alpha, theta(, eta)
+    __shared__ float sgate[2][kWaves * NG * SUB];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cb = lane % LPR, g = lane / LPR;
+    const int g16 = lane >> 4;  // DPP row of the lane
     int chain, part;
     map_block(a.parts, chain, part);
     const int row_local = wave * RG + g;
     const int row = part * ROWS_WG + row_local;
-    const bool valid = row < D;
+    const bool valid = ALL_VALID || row < D;
     const int rr = valid ? row : 0;
     const size_t roff = (size_t)rr * D + cb * 4;
     const int seq_len = a.seq_len, C = a.C;
@@ -132,9 +137,9 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
             float ga = 0.f, ge = 0.f, gt = 0.f;
 #pragma unroll
             for (int w = 0; w < kWaves; w++) {
-                ga += sgate[fob][(tid * kWaves + w) * 4 + 0];
-                ge += sgate[fob][(tid * kWaves + w) * 4 + 1];
-                gt += sgate[fob][(tid * kWaves + w) * 4 + 2];
+                ga += sgate[fob][w * (NG * SUB) + tid * NG + 0];
+                gt += sgate[fob][w * (NG * SUB) + tid * NG + 1];
+                if (HAS_S) ge += sgate[fob][w * (NG * SUB) + tid * NG + 2];
             }
             const int t = ft0 + tid;
             if (a.parts == 1) {
@@ -176,49 +181,44 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
 
         const int t0s = seg_t0(sg), t1 = seg_t1(sg);
         const int tb0 = t0s + j * SUB;
-        if (phase == 0) {
-            // ── level 1: forward replay, park sub-checkpoint and errors ──
-            if (j == 0) {
-                M = S = f4_zero();
-                if (valid) {
-                    M = *reinterpret_cast<const float4 *>(mck + (size_t)sg * DD + roff);
-                    if (HAS_S) S = *reinterpret_cast<const float4 *>(sck + (size_t)sg * DD + roff);
-                }
-            }
-            subck[j][0][tid] = M;
-            if (HAS_S) subck[j][HAS_S ? 1 : 0][tid] = S;
+        // FULL blocks (all SUB tokens inside the segment) run as straight-line
+        // code: no per-token branch, so LDS reads and the independent parts of
+        // neighbouring tokens overlap the dependent chain.
+        auto level1 = [&](auto full_c) {
+            constexpr bool FULL = decltype(full_c)::value;
 #pragma unroll
             for (int i = 0; i < SUB; i++) {
                 const int t = tb0 + i;
-                if (t < t1) {
-                    const float4 kk = *reinterpret_cast<const float4 *>(&tA[buf][i * D + cb * 4]);
-                    const float vv = tB[buf][i * D + rr];
-                    const float al = tg[buf][i], th = tg[buf][SUB + i], et = tg[buf][2 * SUB + i];
-                    float p = group_allreduce<LPR>(dot4(M, kk));
-                    float e = valid ? p - vv : 0.f;
-                    if (cb == 0) ebuf[(t - t0s) * ROWS_WG + row_local] = e;
-                    const float te = th * e;
-                    if (HAS_S) {
-                        S = f4_axpby(et, S, -te, kk);
-                        M = f4_axpby(1.f - al, M, 1.f, S);
-                    } else {
-                        M = f4_axpby(1.f - al, M, -te, kk);
-                    }
+                if (!FULL && t >= t1) break;
+                const float4 kk = *reinterpret_cast<const float4 *>(&tA[buf][i * D + cb * 4]);
+                const float vv = tB[buf][i * D + rr];
+                const float al = tg[buf][i], th = tg[buf][SUB + i], et = tg[buf][2 * SUB + i];
+                float p = group_allreduce<LPR>(dot4(M, kk));
+                float e = valid ? p - vv : 0.f;
+                ebuf[(t - t0s) * ROWS_WG + row_local] = e;  // same value from all lanes of the row
+                const float te = th * e;
+                if (HAS_S) {
+                    S = f4_axpby(et, S, -te, kk);
+                    M = f4_axpby(1.f - al, M, 1.f, S);
+                } else {
+                    M = f4_axpby(1.f - al, M, -te, kk);
                 }
             }
-        } else {
-            // ── level 2: replay the block into registers, then reverse it ──
+        };
+        auto level2 = [&](auto full_c) {
+            constexpr bool FULL = decltype(full_c)::value;
             float4 Mtr[SUB + 1], Str[SUB];
             float ev[SUB];
-            M = subck[j][0][tid];
-            if (HAS_S) S = subck[j][HAS_S ? 1 : 0][tid];
+            float gsum[NG * SUB];  // per-lane gate-gradient partials, [token][component]
+#pragma unroll
+            for (int i = 0; i < NG * SUB; i++) gsum[i] = 0.f;
 #pragma unroll
             for (int i = 0; i < SUB; i++) {
                 const int t = tb0 + i;
                 Mtr[i] = M;
                 Str[i] = S;
                 ev[i] = 0.f;
-                if (t < t1) {
+                if (FULL || t < t1) {
                     const float4 kk = *reinterpret_cast<const float4 *>(&tA[buf][i * D + cb * 4]);
                     const float al = tg[buf][i], th = tg[buf][SUB + i], et = tg[buf][2 * SUB + i];
                     const float e = ebuf[(t - t0s) * ROWS_WG + row_local];
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
 #pragma unroll
             for (int i = SUB - 1; i >= 0; i--) {
                 const int t = tb0 + i;
-                if (t < t1) {
+                if (FULL || t < t1) {
                     const float4 kk = *reinterpret_cast<const float4 *>(&tA[buf][i * D + cb * 4]);
                     const float4 qq = *reinterpret_cast<const float4 *>(&tB[buf][i * D + cb * 4]);
                     const float dy = valid ? tC[buf][i * D + rr] : 0.f;
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                     const float gk = group_allreduce<LPR>(dot4(G, kk));
                     const float derr = -th * gk;
                     float pt = (cb == 0) ? e * gk : 0.f;
-                    if (cb == 0) sdv[ob][i * ROWS_WG + row_local] = -derr;
+                    sdv[ob][i * ROWS_WG + row_local] = -derr;  // same value from all lanes of the row
                     float4 ck = f4_scale(-th * e, G);
                     f4_fma(ck, derr, Mt);
                     if (HAS_S) dS = f4_scale(et, dS);
@@ -260,9 +260,8 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                     // column sums over the row groups of the wave
                     if constexpr (D == 64) {
                         // reduce-scatter: lane (g, cb) ends with column 4*cb + g
-                        float uq = swapadd32(cq.x, cq.z), wq = swapadd32(cq.y, cq.w);
-                        float uk = swapadd32(ck.x, ck.z), wk = swapadd32(ck.y, ck.w);
-                        float fq = swapadd16(uq, wq), fk = swapadd16(uk, wk);
+                        float fq, fk;
+                        colreduce4x2(cq, ck, fq, fk);
                         sdq[ob][(i * kWaves + wave) * D + cb * 4 + g] = fq;
                         sdk[ob][(i * kWaves + wave) * D + cb * 4 + g] = fk;
                     } else {
@@ -275,15 +274,38 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                             *reinterpret_cast<float4 *>(&sdk[ob][(i * kWaves + wave) * D + cb * 4]) = ck;
                         }
                     }
-                    pa = wave_allreduce(pa);
-                    pt = wave_allreduce(pt);
-                    if (HAS_S) pe = wave_allreduce(pe);
-                    if (lane == 0) {
-                        float *gp = &sgate[ob][(i * kWaves + wave) * 4];
-                        gp[0] = pa; gp[1] = pe; gp[2] = pt;
-                    }
+                    gsum[i * NG + 0] = pa;
+                    gsum[i * NG + 1] = pt;
+                    if (HAS_S) gsum[i * NG + 2] = pe;
                 }
             }
+            // one batched wave reduction for the block's gate gradients
+            float gtot[NG * SUB / 4];
+            wave_reduce_scatter<NG * SUB>(gsum, gtot);
+#pragma unroll
+            for (int n = 0; n < NG * SUB / 4; n++)  // same value from the 16 lanes of a DPP row
+                sgate[ob][wave * (NG * SUB) + 4 * n + 2 * (g16 & 1) + (g16 >> 1)] = gtot[n];
+        };
+        const bool full = tb0 + SUB <= t1;
+        if (phase == 0) {
+            // ── level 1: forward replay, park sub-checkpoint and errors ──
+            if (j == 0) {
+                M = S = f4_zero();
+                if (valid) {
+                    M = *reinterpret_cast<const float4 *>(mck + (size_t)sg * DD + roff);
+                    if (HAS_S) S = *reinterpret_cast<const float4 *>(sck + (size_t)sg * DD + roff);
+                }
+            }
+            subck[j][0][tid] = M;
+            if (HAS_S) subck[j][HAS_S ? 1 : 0][tid] = S;
+            if (full) level1(std::true_type{});
+            else level1(std::false_type{});
+        } else {
+            // ── level 2: replay the block into registers, then reverse it ──
+            M = subck[j][0][tid];
+            if (HAS_S) S = subck[j][HAS_S ? 1 : 0][tid];
+            if (full) level2(std::true_type{});
+            else level2(std::false_type{});
             ft0 = tb0;
             ft1 = min(tb0 + SUB, t1);
             fob = ob;

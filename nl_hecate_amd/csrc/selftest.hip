@@ -25,13 +25,40 @@ __global__ void lane_ops_kernel(const float *in, const float *in2, float *out) {
     out[7 * 64 + l] = stride_allreduce<8>(x);
     out[8 * 64 + l] = group_allreduce<8>(x);
     out[9 * 64 + l] = group_allreduce<32>(x);
+    {
+        // column reduce-scatter and batched wave reduction
+        float4 q4 = make_float4(x, y, x + y, x - y), k4 = make_float4(2.f * x, 3.f * y, y, x);
+        float fq, fk;
+        colreduce4x2(q4, k4, fq, fk);
+        out[12 * 64 + l] = fq;
+        out[13 * 64 + l] = fk;
+        float v[8], r[2];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = x * (float)(i + 1) + (float)i;
+        wave_reduce_scatter<8>(v, r);
+        out[14 * 64 + l] = r[0];
+        out[15 * 64 + l] = r[1];
+    }
+    // The row-exchange results are read by the very next VALU instruction in
+    // lane_ops.h (no padding after the swap); these two probes pin that this
+    // is safe.  (A VALU write right BEFORE a swap does need 2 wait states.)
+    {
+        float a = x, b = y;
+        asm volatile("s_nop 4\n\tv_permlane32_swap_b32 %0, %1\n\tv_add_f32 %0, %0, %1"
+                     : "+v"(a), "+v"(b));
+        out[10 * 64 + l] = a;
+        a = x; b = y;
+        asm volatile("s_nop 4\n\tv_permlane16_swap_b32 %0, %1\n\tv_add_f32 %0, %0, %1"
+                     : "+v"(a), "+v"(b));
+        out[11 * 64 + l] = a;
+    }
 }
 
 }  // namespace nlh
 
 extern "C" int nlh_selftest_lane_ops(void) {
     using namespace nlh;
-    const int NT = 10;
+    const int NT = 16;
     std::vector<float> a(64), b(64), o(NT * 64);
     // small integers: every sum is exact, so results compare with ==
     for (int i = 0; i < 64; i++) { a[i] = (float)((i * 37 + 11) % 23 - 9); b[i] = (float)((i * 53 + 5) % 31 - 13); }
@@ -61,6 +88,26 @@ extern "C" int nlh_selftest_lane_ops(void) {
         want[7 * 64 + l] = ssum(l, 8);
         want[8 * 64 + l] = gsum(l, 8);
         want[9 * 64 + l] = gsum(l, 32);
+        {
+            int g = l / 16, cb = l % 16;
+            float sq = 0, sk = 0;
+            for (int gg = 0; gg < 4; gg++) {
+                float xa = a[gg * 16 + cb], yb = b[gg * 16 + cb];
+                float qv[4] = {xa, yb, xa + yb, xa - yb}, kv[4] = {2.f * xa, 3.f * yb, yb, xa};
+                sq += qv[g];
+                sk += kv[g];
+            }
+            want[12 * 64 + l] = sq;
+            want[13 * 64 + l] = sk;
+            float suma = 0;
+            for (int j = 0; j < 64; j++) suma += a[j];
+            for (int n = 0; n < 2; n++) {
+                int i = 4 * n + 2 * (g & 1) + (g >> 1);
+                want[(14 + n) * 64 + l] = suma * (float)(i + 1) + 64.f * (float)i;
+            }
+        }
+        want[10 * 64 + l] = want[5 * 64 + l];
+        want[11 * 64 + l] = want[6 * 64 + l];
     }
     for (int t = 0; t < NT; t++) {
         int nb = 0;
