@@ -140,6 +140,44 @@ void dgd_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const
                                    int t_start, int t_end, int d, int batch_size, int seq_len,
                                    float error_clip);
 
+/* ── Frozen-M0 chunkwise rule ────────────────────────────────────────────────
+ * Errors of a chunk are taken against the chunk-start M; S/M then evolve per
+ * token and y reads the evolving M.  m_chunk_states / s_chunk_states
+ * [batch, num_chunks+1, d*d]: slot 0 = initial, slot c+1 = end of chunk c.
+ * Backward: d_M propagates by retention only, the error path goes to the
+ * chunk-start M (core/kernels/titans_chunkwise_backward.cu). */
+/* core/src/cuda_ffi.rs:376 */
+void titans_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                       const float *alpha, const float *theta, const float *eta,
+                                       const float *m_initial, const float *s_initial,
+                                       float *m_chunk_states, float *s_chunk_states, float *y,
+                                       int seq_len, int d, int batch_size, int chunk_size,
+                                       float error_clip, float m_norm_max);
+/* core/src/cuda_ffi.rs:386 */
+void titans_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                        const float *alpha, const float *theta, const float *eta,
+                                        const float *m_chunk_states, const float *s_chunk_states,
+                                        const float *d_y,
+                                        float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                        float *d_alpha, float *d_theta, float *d_eta,
+                                        float *d_m_initial, float *d_s_initial,
+                                        int seq_len, int d, int batch_size, int chunk_size,
+                                        float error_clip, float m_norm_max);
+/* core/src/cuda_ffi.rs:356 */
+void delta_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                      const float *alpha, const float *theta, const float *m_initial,
+                                      float *m_chunk_states, float *y,
+                                      int seq_len, int d, int batch_size, int chunk_size,
+                                      float error_clip, float m_norm_max);
+/* core/src/cuda_ffi.rs:365 */
+void delta_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                       const float *alpha, const float *theta,
+                                       const float *m_chunk_states, const float *d_y,
+                                       float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                       float *d_alpha, float *d_theta, float *d_m_initial,
+                                       int seq_len, int d, int batch_size, int chunk_size,
+                                       float error_clip, float m_norm_max);
+
 /* ── Batched checkpointed forward (addition) ────────────────────────────────
  * The reference loops the single-chain *_forward_ckpt over heads
  * (core/src/gpu_forward.rs:1611-1662); these take all chains in one launch.

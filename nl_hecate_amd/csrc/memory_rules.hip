@@ -42,7 +42,10 @@ struct FwdArgs {
 
 enum { STORE_NONE = 0, STORE_TRAJ = 1, STORE_CKPT = 2 };
 
-template <int D, int RPL, bool HAS_S, int STORE, bool COUPLED>
+// FROZEN: the frozen-M0 chunkwise rule (core/kernels/titans_chunkwise_forward.cu):
+// errors of a chunk are taken against the chunk-start M; ckpt_interval is the
+// chunk size and the stored checkpoints are the chunk-boundary states.
+template <int D, int RPL, bool HAS_S, int STORE, bool COUPLED, bool FROZEN>
 __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
     constexpr int LPR = D / 4;          // lanes per row
     constexpr int RG = 64 / LPR;        // row groups per wave
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
     float *mo = a.m_out + (size_t)chain * a.state_stride;
     float *so = HAS_S ? a.s_out + (size_t)chain * a.state_stride : nullptr;
 
-    float4 M[RPL], S[RPL];
+    float4 M[RPL], S[RPL], M0[FROZEN ? RPL : 1];
     bool valid[RPL];
 #pragma unroll
     for (int r = 0; r < RPL; r++) {
@@ -93,6 +96,10 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
         }
     }
     int ckpt_slot = 1;
+    if (FROZEN) {
+#pragma unroll
+        for (int r = 0; r < RPL; r++) M0[r] = M[r];
+    }
 
     const int seq_len = a.seq_len;
     const int ntiles = (seq_len + TB - 1) / TB;
@@ -147,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
                 float e[RPL];
 #pragma unroll
                 for (int r = 0; r < RPL; r++) {
-                    float p = group_allreduce<LPR>(dot4(M[r], kk));
+                    float p = group_allreduce<LPR>(dot4(FROZEN ? M0[r] : M[r], kk));
                     float vv = sv[buf][tl * D + (valid[r] ? row0 + r : 0)];
                     e[r] = valid[r] ? p - vv : 0.f;
                 }
@@ -192,18 +199,25 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
                             *reinterpret_cast<float4 *>(mo + off) = M[r];
                             if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
                         }
-                } else if (STORE == STORE_CKPT) {
+                }
+                if (STORE == STORE_CKPT || FROZEN) {
                     // in FAST tiles a boundary can only be the tile's last token
                     if ((!FAST || tl == TB - 1) &&
                         (((t + 1) % a.ckpt_interval == 0) || (t + 1 == seq_len))) {
+                        if (STORE == STORE_CKPT) {
 #pragma unroll
-                        for (int r = 0; r < RPL; r++)
-                            if (ALL_VALID || valid[r]) {
-                                size_t off = (size_t)ckpt_slot * DD + (size_t)(row0 + r) * D + cb * 4;
-                                *reinterpret_cast<float4 *>(mo + off) = M[r];
-                                if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
-                            }
-                        ckpt_slot++;
+                            for (int r = 0; r < RPL; r++)
+                                if (ALL_VALID || valid[r]) {
+                                    size_t off = (size_t)ckpt_slot * DD + (size_t)(row0 + r) * D + cb * 4;
+                                    *reinterpret_cast<float4 *>(mo + off) = M[r];
+                                    if (HAS_S) *reinterpret_cast<float4 *>(so + off) = S[r];
+                                }
+                            ckpt_slot++;
+                        }
+                        if (FROZEN) {
+#pragma unroll
+                            for (int r = 0; r < RPL; r++) M0[r] = M[r];
+                        }
                     }
                 }
 #pragma unroll
@@ -215,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
             }
         };
         const bool fast = !COUPLED && tn == TB &&
-                          (STORE != STORE_CKPT || a.ckpt_interval % TB == 0);
+                          ((STORE != STORE_CKPT && !FROZEN) || a.ckpt_interval % TB == 0);
         if (fast) run_tile(std::true_type{});
         else run_tile(std::false_type{});
     }
@@ -238,7 +252,11 @@ struct BwdArgs {
     float error_clip;
 };
 
-template <int D, int RPL, bool HAS_S, bool COUPLED>
+// FROZEN: the range is one chunk of the frozen-M0 rule
+// (core/kernels/titans_chunkwise_backward.cu): errors and M^T d_err use the
+// chunk-start M (m_states slot 0), d_M propagates by retention only, and the
+// error path is collected in d_M0, added to d_M at the chunk start.
+template <int D, int RPL, bool HAS_S, bool COUPLED, bool FROZEN>
 __global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
     // smaller token tile than forward: the per-wave output partials share LDS
     constexpr int TB = D >= 128 ? 4 : (D >= 64 ? 8 : 16);
@@ -274,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
     const float *ms = a.m_states + (size_t)chain * a.traj_stride;
     const float *ss = HAS_S ? a.s_states + (size_t)chain * a.traj_stride : nullptr;
 
-    float4 dM[RPL], dS[RPL], Mn[RPL], Mt[RPL], St[RPL];
+    float4 dM[RPL], dS[RPL], Mn[RPL], Mt[RPL], St[RPL], M0[FROZEN ? RPL : 1], dM0[FROZEN ? RPL : 1];
     bool valid[RPL];
     size_t roff[RPL];
     const int seg_len = t_end - t_start;
@@ -283,6 +301,10 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
         valid[r] = (row0 + r) < D;
         roff[r] = (size_t)(valid[r] ? row0 + r : 0) * D + cb * 4;
         dM[r] = dS[r] = Mn[r] = Mt[r] = St[r] = f4_zero();
+        if (FROZEN) {
+            dM0[r] = f4_zero();
+            M0[r] = valid[r] ? *reinterpret_cast<const float4 *>(ms + roff[r]) : f4_zero();
+        }
         if (valid[r]) {
             if (a.d_m_seed) dM[r] = *reinterpret_cast<const float4 *>(a.d_m_seed + (size_t)chain * DD + roff[r]);
             if (HAS_S && a.d_s_seed)
@@ -396,7 +418,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
                 pa += dot4(Mt[r], dM[r]);
                 if (HAS_S) pe += dot4(St[r], dS[r]);
                 const float4 &G = HAS_S ? dS[r] : dM[r];
-                float p = group_allreduce<LPR>(dot4(Mt[r], kk));
+                float p = group_allreduce<LPR>(dot4(FROZEN ? M0[r] : Mt[r], kk));
                 e[r] = valid[r] ? p - sv[buf][tl * D + rr] : 0.f;
                 gk[r] = group_allreduce<LPR>(dot4(G, kk));
             }
@@ -420,11 +442,12 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
                     pt += e[r] * gk[r];
                     sdv[buf][tl * ROWS_WG + row_local + r] = -derr;
                 }
-                f4_fma(ck, -th * e[r], G);      // -theta dS^T e
-                f4_fma(ck, derr, Mt[r]);        // + M_t^T d_err
-                if (HAS_S) {
-                    dS[r] = f4_scale(et, dS[r]);
-                    dM[r] = f4_axpby(ret, dM[r], derr, kk);
+                f4_fma(ck, -th * e[r], G);                     // -theta dS^T e
+                f4_fma(ck, derr, FROZEN ? M0[r] : Mt[r]);      // + M^T d_err
+                if (HAS_S) dS[r] = f4_scale(et, dS[r]);
+                if (FROZEN) {
+                    dM[r] = f4_scale(ret, dM[r]);
+                    f4_fma(dM0[r], derr, kk);
                 } else {
                     dM[r] = f4_axpby(ret, dM[r], derr, kk);
                 }
@@ -455,6 +478,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_traj_kernel(BwdArgs a) {
 #pragma unroll
     for (int r = 0; r < RPL; r++)
         if (valid[r]) {
+            if (FROZEN) f4_add(dM[r], dM0[r]);
             *reinterpret_cast<float4 *>(a.d_m_out + (size_t)chain * DD + roff[r]) = dM[r];
             if (HAS_S) *reinterpret_cast<float4 *>(a.d_s_out + (size_t)chain * DD + roff[r]) = dS[r];
         }
@@ -530,47 +554,47 @@ static int pick_rpl(int d, int batch, bool coupled) {
     return 1;
 }
 
-template <int D, int RPL, bool HAS_S, int STORE>
+template <int D, int RPL, bool HAS_S, int STORE, bool FROZEN>
 static void launch_fwd_c(const FwdArgs &a, int batch, bool coupled) {
     dim3 grid(batch * a.parts), block(kThreads);
     if (coupled)
-        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, true>), grid, block, 0, stream(), a);
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, true, FROZEN>), grid, block, 0, stream(), a);
     else
-        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, false>), grid, block, 0, stream(), a);
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, false, FROZEN>), grid, block, 0, stream(), a);
     check_launch("rule_fwd_kernel");
 }
 
-template <bool HAS_S, int STORE>
+template <bool HAS_S, int STORE, bool FROZEN = false>
 static bool launch_fwd(FwdArgs a, int d, int batch) {
     const bool coupled = coupled_needed(a.error_clip, a.m_norm_max);
     const int rpl = pick_rpl(d, batch, coupled);
     a.parts = ceil_div(d, rows_per_wg(d, rpl));
     if (coupled && a.parts != 1) return false;
     switch (d) {
-        case 8: launch_fwd_c<8, 1, HAS_S, STORE>(a, batch, coupled); return true;
-        case 16: launch_fwd_c<16, 1, HAS_S, STORE>(a, batch, coupled); return true;
-        case 32: launch_fwd_c<32, 1, HAS_S, STORE>(a, batch, coupled); return true;
+        case 8: launch_fwd_c<8, 1, HAS_S, STORE, FROZEN>(a, batch, coupled); return true;
+        case 16: launch_fwd_c<16, 1, HAS_S, STORE, FROZEN>(a, batch, coupled); return true;
+        case 32: launch_fwd_c<32, 1, HAS_S, STORE, FROZEN>(a, batch, coupled); return true;
         case 64:
-            if (rpl == 1) launch_fwd_c<64, 1, HAS_S, STORE>(a, batch, false);
-            else if (rpl == 2) launch_fwd_c<64, 2, HAS_S, STORE>(a, batch, false);
-            else launch_fwd_c<64, 4, HAS_S, STORE>(a, batch, coupled);
+            if (rpl == 1) launch_fwd_c<64, 1, HAS_S, STORE, FROZEN>(a, batch, false);
+            else if (rpl == 2) launch_fwd_c<64, 2, HAS_S, STORE, FROZEN>(a, batch, false);
+            else launch_fwd_c<64, 4, HAS_S, STORE, FROZEN>(a, batch, coupled);
             return true;
-        case 128: launch_fwd_c<128, 4, HAS_S, STORE>(a, batch, false); return true;
+        case 128: launch_fwd_c<128, 4, HAS_S, STORE, FROZEN>(a, batch, false); return true;
         default: return false;
     }
 }
 
-template <int D, int RPL, bool HAS_S>
+template <int D, int RPL, bool HAS_S, bool FROZEN>
 static void launch_bwd_c(const BwdArgs &a, bool coupled) {
     dim3 grid(a.batch * a.parts), block(kThreads);
     if (coupled)
-        hipLaunchKernelGGL((rule_bwd_traj_kernel<D, RPL, HAS_S, true>), grid, block, 0, stream(), a);
+        hipLaunchKernelGGL((rule_bwd_traj_kernel<D, RPL, HAS_S, true, FROZEN>), grid, block, 0, stream(), a);
     else
-        hipLaunchKernelGGL((rule_bwd_traj_kernel<D, RPL, HAS_S, false>), grid, block, 0, stream(), a);
+        hipLaunchKernelGGL((rule_bwd_traj_kernel<D, RPL, HAS_S, false, FROZEN>), grid, block, 0, stream(), a);
     check_launch("rule_bwd_traj_kernel");
 }
 
-template <bool HAS_S>
+template <bool HAS_S, bool FROZEN = false>
 static bool launch_bwd(BwdArgs a, int d) {
     const bool coupled = a.error_clip > 0.f;
     const int rpl = pick_rpl(d, a.batch, coupled);
@@ -584,15 +608,15 @@ static bool launch_bwd(BwdArgs a, int d) {
         if (failed()) return true;
     }
     switch (d) {
-        case 8: launch_bwd_c<8, 1, HAS_S>(a, coupled); break;
-        case 16: launch_bwd_c<16, 1, HAS_S>(a, coupled); break;
-        case 32: launch_bwd_c<32, 1, HAS_S>(a, coupled); break;
+        case 8: launch_bwd_c<8, 1, HAS_S, FROZEN>(a, coupled); break;
+        case 16: launch_bwd_c<16, 1, HAS_S, FROZEN>(a, coupled); break;
+        case 32: launch_bwd_c<32, 1, HAS_S, FROZEN>(a, coupled); break;
         case 64:
-            if (rpl == 1) launch_bwd_c<64, 1, HAS_S>(a, false);
-            else if (rpl == 2) launch_bwd_c<64, 2, HAS_S>(a, false);
-            else launch_bwd_c<64, 4, HAS_S>(a, coupled);
+            if (rpl == 1) launch_bwd_c<64, 1, HAS_S, FROZEN>(a, false);
+            else if (rpl == 2) launch_bwd_c<64, 2, HAS_S, FROZEN>(a, false);
+            else launch_bwd_c<64, 4, HAS_S, FROZEN>(a, coupled);
             break;
-        case 128: launch_bwd_c<128, 4, HAS_S>(a, false); break;
+        case 128: launch_bwd_c<128, 4, HAS_S, FROZEN>(a, false); break;
         default: return false;
     }
     if (a.parts > 1 && a.t_end > a.t_start)
@@ -631,7 +655,7 @@ void unsupported(const char *fn, int d, bool coupled) {
 // C-token segment in reverse, replay the forward from the segment's checkpoint
 // into a scratch trajectory, then run the segment backward seeded by the later
 // segment.  No host synchronisation between segments: stream order suffices.
-template <bool HAS_S>
+template <bool HAS_S, bool FROZEN = false>
 static void backward_ckpt_replay(const float *k, const float *v, const float *q,
                                  const float *alpha, const float *theta, const float *eta,
                                  const float *m_ckpt, const float *s_ckpt, const float *d_y,
@@ -659,9 +683,9 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
         FwdArgs fa{k + (size_t)t0 * d, v + (size_t)t0 * d, q + (size_t)t0 * d, alpha + t0, theta + t0,
                    HAS_S ? eta + t0 : nullptr, m_ckpt + (size_t)g * dd,
                    HAS_S ? s_ckpt + (size_t)g * dd : nullptr, lm, ls, ly,
-                   seg, seq_len, 1, 1, (long long)(nck * dd), (long long)((seg + 1) * dd),
+                   seg, seq_len, C, 1, (long long)(nck * dd), (long long)((seg + 1) * dd),
                    error_clip, m_norm_max};
-        if (!launch_fwd<HAS_S, STORE_TRAJ>(fa, d, batch)) {
+        if (!launch_fwd<HAS_S, STORE_TRAJ, FROZEN>(fa, d, batch)) {
             unsupported(fn, d, coupled_needed(error_clip, m_norm_max));
             return;
         }
@@ -671,11 +695,38 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
                    seed_m + (size_t)cur * batch * dd, HAS_S ? seed_s + (size_t)cur * batch * dd : nullptr,
                    d_k, d_v, d_q, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
                    out_m, out_s, seq_len, t0, t1, 1, batch, (long long)((seg + 1) * dd), error_clip};
-        if (!launch_bwd<HAS_S>(ba, d)) { unsupported(fn, d, error_clip > 0.f); return; }
+        if (!launch_bwd<HAS_S, FROZEN>(ba, d)) { unsupported(fn, d, error_clip > 0.f); return; }
         cur ^= 1;
     }
     accumulate_over_batch(seed_m + (size_t)cur * batch * dd, d_m_initial, batch, (int)dd);
     if (HAS_S) accumulate_over_batch(seed_s + (size_t)cur * batch * dd, d_s_initial, batch, (int)dd);
+}
+
+
+// One-call checkpointed / chunkwise backward: fused on-chip replay when it
+// covers the case, the replay-through-memory schedule otherwise.
+static void backward_ckpt_any(bool has_s, bool frozen, bool allow_fused,
+                              const float *k, const float *v, const float *q,
+                              const float *alpha, const float *theta, const float *eta,
+                              const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                              float *d_k, float *d_v, float *d_q,
+                              float *d_alpha, float *d_theta, float *d_eta,
+                              float *d_m_initial, float *d_s_initial,
+                              int seq_len, int d, int batch, int C,
+                              float error_clip, float m_norm_max, const char *fn) {
+    if (!check_dims(fn, seq_len, d, batch) || batch == 0 || seq_len == 0) return;
+    if (C <= 0) { fail("%s: interval/chunk size %d must be > 0.", fn, C); return; }
+    if (allow_fused && !coupled_needed(error_clip, m_norm_max) &&
+        backward_ckpt_fused(has_s, frozen, k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v,
+                            d_q, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d, batch, C))
+        return;
+#define NLH_REPLAY(HS, FZ)                                                                         \
+    backward_ckpt_replay<HS, FZ>(k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v, d_q,  \
+                                 d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d,   \
+                                 batch, C, error_clip, m_norm_max, fn)
+    if (has_s) { if (frozen) NLH_REPLAY(true, true); else NLH_REPLAY(true, false); }
+    else { if (frozen) NLH_REPLAY(false, true); else NLH_REPLAY(false, false); }
+#undef NLH_REPLAY
 }
 
 }  // namespace nlh
@@ -888,13 +939,10 @@ void titans_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem
                                           float *d_m_initial, float *d_s_initial,
                                           int seq_len, int d, int batch_size, int checkpoint_interval,
                                           float error_clip, float m_norm_max) {
-    const char *fn = "titans_backward_ckpt_replay_f32_rocm";
-    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0 || seq_len == 0) return;
-    if (checkpoint_interval <= 0) { fail("%s: checkpoint_interval=%d must be > 0.", fn, checkpoint_interval); return; }
-    backward_ckpt_replay<true>(k_mem, v_mem, q_mem, alpha, theta, eta, m_ckpt, s_ckpt, d_y,
-                               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
-                               d_m_initial, d_s_initial, seq_len, d, batch_size,
-                               checkpoint_interval, error_clip, m_norm_max, fn);
+    backward_ckpt_any(true, false, false, k_mem, v_mem, q_mem, alpha, theta, eta, m_ckpt, s_ckpt, d_y,
+                      d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial,
+                      seq_len, d, batch_size, checkpoint_interval, error_clip, m_norm_max,
+                      "titans_backward_ckpt_replay_f32_rocm");
 }
 
 void delta_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
@@ -904,13 +952,97 @@ void delta_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem,
                                          float *d_alpha, float *d_theta, float *d_m_initial,
                                          int seq_len, int d, int batch_size, int checkpoint_interval,
                                          float error_clip, float m_norm_max) {
-    const char *fn = "delta_backward_ckpt_replay_f32_rocm";
-    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0 || seq_len == 0) return;
-    if (checkpoint_interval <= 0) { fail("%s: checkpoint_interval=%d must be > 0.", fn, checkpoint_interval); return; }
-    backward_ckpt_replay<false>(k_mem, v_mem, q_mem, alpha, theta, nullptr, m_ckpt, nullptr, d_y,
-                                d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr,
-                                d_m_initial, nullptr, seq_len, d, batch_size,
-                                checkpoint_interval, error_clip, m_norm_max, fn);
+    backward_ckpt_any(false, false, false, k_mem, v_mem, q_mem, alpha, theta, nullptr, m_ckpt, nullptr,
+                      d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr, d_m_initial, nullptr,
+                      seq_len, d, batch_size, checkpoint_interval, error_clip, m_norm_max,
+                      "delta_backward_ckpt_replay_f32_rocm");
+}
+
+void titans_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                   const float *alpha, const float *theta, const float *eta,
+                                   const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                                   float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                   float *d_alpha, float *d_theta, float *d_eta,
+                                   float *d_m_initial, float *d_s_initial,
+                                   int seq_len, int d, int batch_size, int checkpoint_interval,
+                                   float error_clip, float m_norm_max) {
+    backward_ckpt_any(true, false, true, k_mem, v_mem, q_mem, alpha, theta, eta, m_ckpt, s_ckpt, d_y,
+                      d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial,
+                      seq_len, d, batch_size, checkpoint_interval, error_clip, m_norm_max,
+                      "titans_backward_ckpt_f32_rocm");
+}
+
+void delta_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                  const float *alpha, const float *theta,
+                                  const float *m_ckpt, const float *d_y,
+                                  float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                  float *d_alpha, float *d_theta, float *d_m_initial,
+                                  int seq_len, int d, int batch_size, int checkpoint_interval,
+                                  float error_clip, float m_norm_max) {
+    backward_ckpt_any(false, false, true, k_mem, v_mem, q_mem, alpha, theta, nullptr, m_ckpt, nullptr,
+                      d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr, d_m_initial, nullptr,
+                      seq_len, d, batch_size, checkpoint_interval, error_clip, m_norm_max,
+                      "delta_backward_ckpt_f32_rocm");
+}
+
+// ── frozen-M0 chunkwise rule ────────────────────────────────────────────────
+void titans_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                       const float *alpha, const float *theta, const float *eta,
+                                       const float *m_initial, const float *s_initial,
+                                       float *m_chunk_states, float *s_chunk_states, float *y,
+                                       int seq_len, int d, int batch_size, int chunk_size,
+                                       float error_clip, float m_norm_max) {
+    const char *fn = "titans_chunkwise_forward_f32_cuda";
+    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0) return;
+    if (chunk_size <= 0) { fail("%s: chunk_size=%d must be > 0.", fn, chunk_size); return; }
+    FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial,
+              m_chunk_states, s_chunk_states, y, seq_len, seq_len, chunk_size, 1, (long long)d * d,
+              (long long)n_ckpt_count(seq_len, chunk_size) * d * d, error_clip, m_norm_max};
+    if (!launch_fwd<true, STORE_CKPT, true>(a, d, batch_size))
+        unsupported(fn, d, coupled_needed(error_clip, m_norm_max));
+}
+
+void delta_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                      const float *alpha, const float *theta, const float *m_initial,
+                                      float *m_chunk_states, float *y,
+                                      int seq_len, int d, int batch_size, int chunk_size,
+                                      float error_clip, float m_norm_max) {
+    const char *fn = "delta_chunkwise_forward_f32_cuda";
+    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0) return;
+    if (chunk_size <= 0) { fail("%s: chunk_size=%d must be > 0.", fn, chunk_size); return; }
+    FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial, nullptr,
+              m_chunk_states, nullptr, y, seq_len, seq_len, chunk_size, 1, (long long)d * d,
+              (long long)n_ckpt_count(seq_len, chunk_size) * d * d, error_clip, m_norm_max};
+    if (!launch_fwd<false, STORE_CKPT, true>(a, d, batch_size))
+        unsupported(fn, d, coupled_needed(error_clip, m_norm_max));
+}
+
+void titans_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                        const float *alpha, const float *theta, const float *eta,
+                                        const float *m_chunk_states, const float *s_chunk_states,
+                                        const float *d_y,
+                                        float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                        float *d_alpha, float *d_theta, float *d_eta,
+                                        float *d_m_initial, float *d_s_initial,
+                                        int seq_len, int d, int batch_size, int chunk_size,
+                                        float error_clip, float m_norm_max) {
+    backward_ckpt_any(true, true, true, k_mem, v_mem, q_mem, alpha, theta, eta, m_chunk_states,
+                      s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
+                      d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, error_clip,
+                      m_norm_max, "titans_chunkwise_backward_f32_cuda");
+}
+
+void delta_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                       const float *alpha, const float *theta,
+                                       const float *m_chunk_states, const float *d_y,
+                                       float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                       float *d_alpha, float *d_theta, float *d_m_initial,
+                                       int seq_len, int d, int batch_size, int chunk_size,
+                                       float error_clip, float m_norm_max) {
+    backward_ckpt_any(false, true, true, k_mem, v_mem, q_mem, alpha, theta, nullptr, m_chunk_states,
+                      nullptr, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr,
+                      d_m_initial, nullptr, seq_len, d, batch_size, chunk_size, error_clip,
+                      m_norm_max, "delta_chunkwise_backward_f32_cuda");
 }
 
 }  // extern "C"

@@ -43,7 +43,9 @@ struct FusedArgs {
     int seq_len, C, n_ckpt, parts, batch;
 };
 
-template <int D, bool HAS_S>
+// FROZEN: frozen-M0 chunkwise rule, segment = chunk
+// (core/kernels/titans_chunkwise_backward.cu:118-358).
+template <int D, bool HAS_S, bool FROZEN>
 __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
     constexpr int LPR = D / 4;
     constexpr int RG = 64 / LPR;
@@ -85,6 +87,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
 
     float4 dM = f4_zero(), dS = f4_zero();
     float4 M = f4_zero(), S = f4_zero();
+    float4 M0f = f4_zero(), dM0 = f4_zero();  // FROZEN: chunk-start M and its gradient
 
     // ── work items: (segment, phase, block) in processing order ──
     const int nseg = (seq_len + C - 1) / C;
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                 const float4 kk = *reinterpret_cast<const float4 *>(&tA[buf][i * D + cb * 4]);
                 const float vv = tB[buf][i * D + rr];
                 const float al = tg[buf][i], th = tg[buf][SUB + i], et = tg[buf][2 * SUB + i];
-                float p = group_allreduce<LPR>(dot4(M, kk));
+                float p = group_allreduce<LPR>(dot4(FROZEN ? M0f : M, kk));
                 float e = valid ? p - vv : 0.f;
                 ebuf[(t - t0s) * ROWS_WG + row_local] = e;  // same value from all lanes of the row
                 const float te = th * e;
@@ -254,9 +257,14 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                     float pt = (cb == 0) ? e * gk : 0.f;
                     sdv[ob][i * ROWS_WG + row_local] = -derr;  // same value from all lanes of the row
                     float4 ck = f4_scale(-th * e, G);
-                    f4_fma(ck, derr, Mt);
+                    f4_fma(ck, derr, FROZEN ? M0f : Mt);
                     if (HAS_S) dS = f4_scale(et, dS);
-                    dM = f4_axpby(1.f - al, dM, derr, kk);
+                    if (FROZEN) {
+                        dM = f4_scale(1.f - al, dM);
+                        f4_fma(dM0, derr, kk);
+                    } else {
+                        dM = f4_axpby(1.f - al, dM, derr, kk);
+                    }
                     // column sums over the row groups of the wave
                     if constexpr (D == 64) {
                         // reduce-scatter: lane (g, cb) ends with column 4*cb + g
@@ -295,6 +303,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                     M = *reinterpret_cast<const float4 *>(mck + (size_t)sg * DD + roff);
                     if (HAS_S) S = *reinterpret_cast<const float4 *>(sck + (size_t)sg * DD + roff);
                 }
+                if (FROZEN) M0f = M;
             }
             subck[j][0][tid] = M;
             if (HAS_S) subck[j][HAS_S ? 1 : 0][tid] = S;
@@ -306,6 +315,10 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
             if (HAS_S) S = subck[j][HAS_S ? 1 : 0][tid];
             if (full) level2(std::true_type{});
             else level2(std::false_type{});
+            if (FROZEN && j == 0) {  // chunk start: the error path joins d_M
+                f4_add(dM, dM0);
+                dM0 = f4_zero();
+            }
             ft0 = tb0;
             ft1 = min(tb0 + SUB, t1);
             fob = ob;
@@ -322,22 +335,21 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
     }
 }
 
-template <int D, bool HAS_S>
+template <int D, bool HAS_S, bool FROZEN>
 static void launch_fused_d(const FusedArgs &a) {
-    hipLaunchKernelGGL((rule_bwd_fused_kernel<D, HAS_S>), dim3(a.batch * a.parts), dim3(kThreads), 0,
-                       stream(), a);
+    hipLaunchKernelGGL((rule_bwd_fused_kernel<D, HAS_S, FROZEN>), dim3(a.batch * a.parts),
+                       dim3(kThreads), 0, stream(), a);
     check_launch("rule_bwd_fused_kernel");
 }
 
-// Returns false when the fused kernel does not cover (d, C).
-template <bool HAS_S>
-static bool backward_ckpt_fused(const float *k, const float *v, const float *q,
-                                const float *alpha, const float *theta, const float *eta,
-                                const float *m_ckpt, const float *s_ckpt, const float *d_y,
-                                float *d_k, float *d_v, float *d_q,
-                                float *d_alpha, float *d_theta, float *d_eta,
-                                float *d_m_initial, float *d_s_initial,
-                                int seq_len, int d, int batch, int C) {
+template <bool HAS_S, bool FROZEN>
+static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q,
+                                  const float *alpha, const float *theta, const float *eta,
+                                  const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                                  float *d_k, float *d_v, float *d_q,
+                                  float *d_alpha, float *d_theta, float *d_eta,
+                                  float *d_m_initial, float *d_s_initial,
+                                  int seq_len, int d, int batch, int C) {
     if (C > C_MAX) return false;
     if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) return false;
     const size_t dd = (size_t)d * d;
@@ -355,11 +367,11 @@ static bool backward_ckpt_fused(const float *k, const float *v, const float *q,
     }
     if (failed()) return true;
     switch (d) {
-        case 8: launch_fused_d<8, HAS_S>(a); break;
-        case 16: launch_fused_d<16, HAS_S>(a); break;
-        case 32: launch_fused_d<32, HAS_S>(a); break;
-        case 64: launch_fused_d<64, HAS_S>(a); break;
-        case 128: launch_fused_d<128, HAS_S>(a); break;
+        case 8: launch_fused_d<8, HAS_S, FROZEN>(a); break;
+        case 16: launch_fused_d<16, HAS_S, FROZEN>(a); break;
+        case 32: launch_fused_d<32, HAS_S, FROZEN>(a); break;
+        case 64: launch_fused_d<64, HAS_S, FROZEN>(a); break;
+        case 128: launch_fused_d<128, HAS_S, FROZEN>(a); break;
     }
     if (a.parts > 1)
         finalize_parts(a.ws_dq, a.ws_dk, a.ws_gate, d_q, d_k, d_alpha, d_theta,
@@ -369,53 +381,21 @@ static bool backward_ckpt_fused(const float *k, const float *v, const float *q,
     return true;
 }
 
+bool backward_ckpt_fused(bool has_s, bool frozen, const float *k, const float *v, const float *q,
+                         const float *alpha, const float *theta, const float *eta,
+                         const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                         float *d_k, float *d_v, float *d_q,
+                         float *d_alpha, float *d_theta, float *d_eta,
+                         float *d_m_initial, float *d_s_initial,
+                         int seq_len, int d, int batch, int C) {
+#define NLH_FUSED(HS, FZ)                                                                        \
+    return backward_ckpt_fused_t<HS, FZ>(k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k,  \
+                                         d_v, d_q, d_alpha, d_theta, d_eta, d_m_initial,        \
+                                         d_s_initial, seq_len, d, batch, C)
+    if (has_s) { if (frozen) NLH_FUSED(true, true); else NLH_FUSED(true, false); }
+    if (frozen) NLH_FUSED(false, true);
+    NLH_FUSED(false, false);
+#undef NLH_FUSED
+}
+
 }  // namespace nlh
-
-using namespace nlh;
-
-extern "C" {
-
-void titans_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
-                                   const float *alpha, const float *theta, const float *eta,
-                                   const float *m_ckpt, const float *s_ckpt, const float *d_y,
-                                   float *d_k_mem, float *d_v_mem, float *d_q_mem,
-                                   float *d_alpha, float *d_theta, float *d_eta,
-                                   float *d_m_initial, float *d_s_initial,
-                                   int seq_len, int d, int batch_size, int checkpoint_interval,
-                                   float error_clip, float m_norm_max) {
-    const char *fn = "titans_backward_ckpt_f32_rocm";
-    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0 || seq_len == 0) return;
-    if (checkpoint_interval <= 0) { fail("%s: checkpoint_interval=%d must be > 0.", fn, checkpoint_interval); return; }
-    if (!coupled_needed(error_clip, m_norm_max) &&
-        backward_ckpt_fused<true>(k_mem, v_mem, q_mem, alpha, theta, eta, m_ckpt, s_ckpt, d_y,
-                                  d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
-                                  d_m_initial, d_s_initial, seq_len, d, batch_size, checkpoint_interval))
-        return;
-    titans_backward_ckpt_replay_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_ckpt, s_ckpt, d_y,
-                                         d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
-                                         d_m_initial, d_s_initial, seq_len, d, batch_size,
-                                         checkpoint_interval, error_clip, m_norm_max);
-}
-
-void delta_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
-                                  const float *alpha, const float *theta,
-                                  const float *m_ckpt, const float *d_y,
-                                  float *d_k_mem, float *d_v_mem, float *d_q_mem,
-                                  float *d_alpha, float *d_theta, float *d_m_initial,
-                                  int seq_len, int d, int batch_size, int checkpoint_interval,
-                                  float error_clip, float m_norm_max) {
-    const char *fn = "delta_backward_ckpt_f32_rocm";
-    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0 || seq_len == 0) return;
-    if (checkpoint_interval <= 0) { fail("%s: checkpoint_interval=%d must be > 0.", fn, checkpoint_interval); return; }
-    if (!coupled_needed(error_clip, m_norm_max) &&
-        backward_ckpt_fused<false>(k_mem, v_mem, q_mem, alpha, theta, nullptr, m_ckpt, nullptr, d_y,
-                                   d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr,
-                                   d_m_initial, nullptr, seq_len, d, batch_size, checkpoint_interval))
-        return;
-    delta_backward_ckpt_replay_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, m_ckpt, d_y,
-                                        d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_m_initial,
-                                        seq_len, d, batch_size, checkpoint_interval, error_clip,
-                                        m_norm_max);
-}
-
-}  // extern "C"
