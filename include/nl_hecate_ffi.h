@@ -239,6 +239,81 @@ void delta_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const 
                                   int seq_len, int d, int batch_size, int checkpoint_interval,
                                   float error_clip, float m_norm_max);
 
+/* ── Glue either side of the memory rules ───────────────────────────────────
+ * Elementwise kernels take n elements; all are asynchronous. */
+/* core/src/cuda_ffi.rs:552 */
+void sigmoid_cuda(const float *x, float *out, int n);
+/* core/kernels/elementwise.cu:47 (softplus, identity above 20; not in cuda_ffi.rs) */
+void softplus_cuda(const float *x, float *out, int n);
+/* core/src/cuda_ffi.rs:555 */
+void elemwise_mul_cuda(const float *a, const float *b, float *out, int n);
+/* core/src/cuda_ffi.rs:558: d_a = d_out*b, d_b = d_out*a */
+void gating_backward_cuda(const float *d_out, const float *a, const float *b, float *d_a, float *d_b, int n);
+/* core/src/cuda_ffi.rs:564: d_x = d_gate*gate*(1-gate) */
+void sigmoid_backward_cuda(const float *d_gate, const float *gate, float *d_x, int n);
+/* core/src/cuda_ffi.rs:569 / 572: round-to-nearest-even */
+void f32_to_bf16_cuda(const float *src, uint16_t *dst, int n);
+void bf16_to_f32_cuda(const uint16_t *src, float *dst, int n);
+/* core/src/cuda_ffi.rs:579: gate[t] = act(k_t.w[:d] + v_t.w[d:] + *bias_ptr);
+ * activation 0 = sigmoid, 1 = softplus (identity above 20) */
+void gate_compute_cuda(const float *k_mem, const float *v_mem, const float *w_gate,
+                       const float *bias_ptr, float *gate_out, int seq_len, int d, int activation);
+/* core/src/cuda_ffi.rs:587 / 591 */
+void clamp_f32_cuda(float *inout, int n, float lo, float hi);
+void theta_clamp_mask_cuda(const float *theta, float *d_theta, int n, float lo, float hi);
+/* core/src/cuda_ffi.rs:599: d_w / d_b of the gate projections from the cached
+ * gate OUTPUTS (sigmoid' = a(1-a), softplus' = 1-exp(-theta)); outputs are
+ * overwritten. */
+void gate_backward_cuda(const float *d_alpha, const float *alpha, const float *d_theta,
+                        const float *theta, const float *d_eta, const float *eta,
+                        const float *k_mem, const float *v_mem,
+                        float *d_w_alpha, float *d_b_alpha, float *d_w_theta, float *d_b_theta,
+                        float *d_w_eta, float *d_b_eta, int T, int D, int has_theta, int has_eta);
+/* core/src/cuda_ffi.rs:611: y += alpha*x */
+void saxpy_cuda(float alpha, const float *x, float *y, int n);
+/* core/src/cuda_ffi.rs:507 / 514: rows normalised in place, norms = pre-normalisation L2 norms */
+void l2_normalize_rows_f32_cuda(float *x, float *norms, int n_rows, int d, float eps);
+void l2_normalize_backward_f32_cuda(const float *d_out, const float *x_norm, const float *norms,
+                                    float *d_in, int n_rows, int d, float eps);
+/* core/src/cuda_ffi.rs:1035: [bs,s,nh*hd] -> [bs*nh,s,hd] (forward=1) or back (0) */
+void transpose_heads_f32_cuda(const float *input, float *output, int bs, int s, int nh, int hd, int forward);
+/* core/src/cuda_ffi.rs:1043 / 1051: [bs,s] -> [bs*nh,s] and its adjoint */
+void broadcast_heads_f32_cuda(const float *input, float *output, int bs, int s, int nh);
+void sum_heads_f32_cuda(const float *input, float *output, int bs, int s, int nh);
+/* core/src/cuda_ffi.rs:458: dst[b, t, :] = src[b, :]; returns 0 / 1 (overflow) / 2 (launch) */
+int broadcast_fill_f32_cuda(float *dst, const float *src, int dd, int n_slots, int n_batch);
+/* core/src/cuda_ffi.rs:467 / 471: Frobenius clamp, no-op for max <= 0 or >= 1e30 */
+void m_norm_clamp_f32_cuda(float *m, int d, float m_norm_max);
+void m_norm_clamp_batch_f32_cuda(float *m, int d, int batch_size, float m_norm_max);
+/* core/src/cuda_ffi.rs:478: norm_out[0] = |M k - v|_2 */
+void dgd_delta_norm_cuda(const float *m, const float *k, const float *v, float *norm_out, int d);
+
+/* ── AdamW and gradient clipping; return hipError_t as unsigned, 0 = success ─ */
+/* core/src/cuda_ffi.rs:674 */
+unsigned adamw_update_cuda(float *w, const float *g, float *m, float *v, int n, float lr, float beta1,
+                           float beta2, float eps, float bc1_inv, float bc2_inv, float weight_decay);
+/* core/src/cuda_ffi.rs:686 / 693: ceil(n/256) partial sums, one per 256
+ * elements; *out_num_blocks (host) receives that count */
+unsigned grad_norm_sq_cuda(const float *g, float *partial_sums, int n, int *out_num_blocks);
+unsigned dot_product_partial_f32_cuda(const float *a, const float *b, float *partial_sums, int n,
+                                      int *out_num_blocks);
+/* core/src/cuda_ffi.rs:700 */
+unsigned grad_scale_cuda(float *g, float scale, int n);
+/* core/src/cuda_ffi.rs:706: out_norm = sqrt(sum), out_scale = min(1, max/norm) on device */
+unsigned reduce_partials_clip_cuda(const float *partial_sums, int total_partials, float max_grad_norm,
+                                   float *out_norm, float *out_scale);
+/* core/src/cuda_ffi.rs:714: g *= *scale_ptr unless it is >= 1 */
+unsigned grad_scale_conditional_cuda(float *g, const float *scale_ptr, int n);
+/* Additions: every tensor of a step in one launch.  The pointer / size /
+ * bias-correction arrays are HOST arrays of `count` entries (device pointers
+ * inside); replaces the per-tensor loop of core/src/gpu_optimizer.rs:403-515
+ * and the partial-sum pipeline of core/src/gpu_stacked_optimizer.rs:193. */
+unsigned adamw_update_multi_rocm(float *const *w, const float *const *g, float *const *m, float *const *v,
+                                 const int *n, const float *bc1_inv, const float *bc2_inv, int count,
+                                 float lr, float beta1, float beta2, float eps, float weight_decay);
+unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, float max_grad_norm,
+                                   float *out_norm, float *out_scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -254,3 +254,115 @@ def backward_ckpt(k, v, q, alpha, theta, eta, mc, sc, d_y, C, has_s=True, error_
           g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], g["d_m"], g["d_s"],
           s, d, C, int(has_s), float(error_clip), float(m_norm_max))
     return g
+
+
+# ── pieces around the memory rules (nlh_oracle_layer.c) ────────────────────
+def adamw_step(params, grads, m, v, lr, beta1, beta2, eps, bc1_inv, bc2_inv, weight_decay):
+    """In place on float32 arrays (core/src/adamw.rs:102-126)."""
+    f = lib().orc_adamw_step
+    f.restype = None
+    for a in (params, grads, m, v):
+        assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    f(p(params), p(grads), p(m), p(v), ctypes.c_int64(params.size), *[ctypes.c_float(x) for x in
+      (lr, beta1, beta2, eps, bc1_inv, bc2_inv, weight_decay)])
+
+
+def grad_norm_clip(grads, max_grad_norm):
+    """-> (norm, scale) over a list of float32 arrays (core/src/adamw.rs:203-262)."""
+    n = len(grads)
+    ptrs = (ctypes.c_void_p * n)(*[g.ctypes.data for g in grads])
+    sizes = (ctypes.c_int64 * n)(*[g.size for g in grads])
+    scale = ctypes.c_float(0)
+    f = lib().orc_grad_norm_clip
+    f.restype = ctypes.c_float
+    norm = f(ptrs, sizes, ctypes.c_int(n), ctypes.c_float(max_grad_norm), ctypes.byref(scale))
+    return float(norm), float(scale.value)
+
+
+def pulse(step, chunk_sizes, seq_len=0):
+    k = len(chunk_sizes)
+    cs = (ctypes.c_int64 * k)(*chunk_sizes)
+    out = (ctypes.c_int * k)()
+    f = lib().orc_pulse
+    f.restype = None
+    f(ctypes.c_int64(step), cs, ctypes.c_int(k), ctypes.c_int64(seq_len), out)
+    return [bool(x) for x in out]
+
+
+def gate_compute(k, v, w, bias, activation):
+    f = np.float32
+    n, d = k.shape
+    out = np.zeros(n, f)
+    _call("orc_gate_compute", _c(k, f), _c(v, f), _c(w, f), float(bias), out, n, d, int(activation))
+    return out
+
+
+def gate_backward(d_alpha, alpha, d_theta, theta, d_eta, eta, k, v, has_theta=True, has_eta=True):
+    f = np.float32
+    T, D = k.shape
+    o = {n: np.zeros(2 * D, f) for n in ("d_w_alpha", "d_w_theta", "d_w_eta")}
+    o.update({n: np.zeros(1, f) for n in ("d_b_alpha", "d_b_theta", "d_b_eta")})
+    z = np.zeros(T, f)
+    _call("orc_gate_backward", _c(d_alpha, f), _c(alpha, f),
+          _c(d_theta if has_theta else z, f), _c(theta if has_theta else z, f),
+          _c(d_eta if has_eta else z, f), _c(eta if has_eta else z, f), _c(k, f), _c(v, f),
+          o["d_w_alpha"], o["d_b_alpha"], o["d_w_theta"], o["d_b_theta"], o["d_w_eta"], o["d_b_eta"],
+          T, D, int(has_theta), int(has_eta))
+    return o
+
+
+def l2_normalize_rows(x, eps=1e-8):
+    f = np.float32
+    x = _c(x, f).copy()
+    n, d = x.shape
+    norms = np.zeros(n, f)
+    _call("orc_l2_normalize_rows", x, norms, n, d, float(eps))
+    return x, norms
+
+
+def l2_normalize_backward(d_out, x_norm, norms, eps=1e-8):
+    f = np.float32
+    n, d = d_out.shape
+    d_in = np.zeros((n, d), f)
+    _call("orc_l2_normalize_backward", _c(d_out, f), _c(x_norm, f), _c(norms, f), d_in, n, d, float(eps))
+    return d_in
+
+
+def f32_to_bf16(x):
+    x = _c(x, np.float32)
+    out = np.zeros(x.shape, np.uint16)
+    fn = lib().orc_f32_to_bf16
+    fn.restype = None
+    fn(x.ctypes.data_as(ctypes.c_void_p), out.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(x.size))
+    return out
+
+
+def bf16_to_f32(x):
+    x = _c(x, np.uint16)
+    out = np.zeros(x.shape, np.float32)
+    fn = lib().orc_bf16_to_f32
+    fn.restype = None
+    fn(x.ctypes.data_as(ctypes.c_void_p), out.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(x.size))
+    return out
+
+
+def swa_forward(q, k, v, window, num_heads, n_persistent=0):
+    """q,k,v uint16 (bf16 bits) [B, s, H*hd] -> out uint16, attn_weights uint16 [B,H,s,np+window]."""
+    B, s, td = q.shape
+    hd = td // num_heads
+    out = np.zeros((B, s, td), np.uint16)
+    aw = np.zeros((B, num_heads, s, n_persistent + window), np.uint16)
+    _call("orc_swa_forward", _c(q, np.uint16), _c(k, np.uint16), _c(v, np.uint16), out, aw,
+          s, num_heads, hd, window, B, n_persistent)
+    return out, aw
+
+
+def swa_backward(q, k, v, aw, d_out, window, num_heads, n_persistent=0):
+    B, s, td = q.shape
+    hd = td // num_heads
+    f = np.float32
+    dq, dk, dv = np.zeros((B, s, td), f), np.zeros((B, s, td), f), np.zeros((B, s, td), f)
+    _call("orc_swa_backward", _c(q, np.uint16), _c(k, np.uint16), _c(v, np.uint16), _c(aw, np.uint16),
+          _c(d_out, f), dq, dk, dv, s, num_heads, hd, window, B, n_persistent)
+    return dq, dk, dv
