@@ -288,6 +288,22 @@ void m_norm_clamp_batch_f32_cuda(float *m, int d, int batch_size, float m_norm_m
 /* core/src/cuda_ffi.rs:478: norm_out[0] = |M k - v|_2 */
 void dgd_delta_norm_cuda(const float *m, const float *k, const float *v, float *norm_out, int d);
 
+/* ── Sliding-window attention (bf16 storage as uint16_t, f32 math) ──────────
+ * q,k,v,out [batch, seq, heads*hd]; attn_weights [batch, heads, seq,
+ * n_persistent + window].  Query t sees prefix keys [0, min(t+1, n_persistent))
+ * (slot = key) and local keys [ls, t], ls = max(t+1-window, n_persistent)
+ * (slot = n_persistent + key - ls); unused slots are written as 0. */
+/* core/src/cuda_ffi.rs:26 */
+void swa_forward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out,
+                          uint16_t *attn_weights, int seq_len, int num_heads, int head_dim,
+                          int window_size, int batch_size, int n_persistent);
+/* core/src/cuda_ffi.rs:62.  d_q is overwritten; d_k and d_v are ACCUMULATED
+ * (+=) into caller-zeroed buffers.  Differentiates through the stored weights. */
+void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                           const uint16_t *attn_weights, const float *d_attn_out,
+                           float *d_q, float *d_k, float *d_v, int seq_len, int num_heads, int head_dim,
+                           int window_size, int batch_size, int n_persistent);
+
 /* ── AdamW and gradient clipping; return hipError_t as unsigned, 0 = success ─ */
 /* core/src/cuda_ffi.rs:674 */
 unsigned adamw_update_cuda(float *w, const float *g, float *m, float *v, int n, float lr, float beta1,

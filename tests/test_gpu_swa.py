@@ -1,0 +1,94 @@
+"""GPU parity of sliding-window attention (bf16 storage, f32 math) against the
+CPU oracle.  bf16 path: relative 2e-2; with identical stored weights the
+backward agrees to fp32 round-off (1e-4).  The reference's own bounds are
+absolute 1e-2 forward / 5e-2 backward (core/tests/test_cuda_swa.rs:100,325)."""
+import numpy as np
+import pytest
+import torch
+
+from nl_hecate_amd import dispatch as D
+from oracle import pyoracle as orc
+from tests.gpu_util import assert_close, dev, host, zeros, REL_TOL_BF16
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(B, s, H, hd, seed):
+    r = np.random.default_rng(seed)
+    q, k, v = (orc.f32_to_bf16(r.standard_normal((B, s, H * hd)).astype(np.float32)) for _ in range(3))
+    go = r.standard_normal((B, s, H * hd)).astype(np.float32)
+    return q, k, v, go
+
+
+def _u16(a):
+    return torch.from_numpy(a.view(np.int16)).cuda().view(torch.uint16)
+
+
+def gpu_forward(q, k, v, ws, H, npers):
+    B, s, td = q.shape
+    out = torch.zeros(B, s, td, dtype=torch.uint16, device="cuda")
+    aw = torch.full((B, H, s, npers + ws), 0x7fc0, dtype=torch.uint16, device="cuda")  # NaN canary
+    D.call("swa_forward_f32_cuda", _u16(q), _u16(k), _u16(v), out, aw, s, H, td // H, ws, B, npers)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), aw.cpu().numpy()
+
+
+def gpu_backward(q, k, v, aw, go, ws, H, npers):
+    B, s, td = q.shape
+    dq, dk, dv = zeros(B, s, td), zeros(B, s, td), zeros(B, s, td)
+    D.call("swa_backward_f32_cuda", _u16(q), _u16(k), _u16(v), _u16(aw), dev(go), dq, dk, dv,
+           s, H, td // H, ws, B, npers)
+    torch.cuda.synchronize()
+    return host(dq), host(dk), host(dv)
+
+
+@pytest.mark.parametrize("B,s,H,hd,ws,npers", [(2, 40, 2, 64, 16, 0), (1, 70, 3, 32, 64, 0),
+                                               (2, 33, 2, 64, 8, 5), (1, 20, 1, 8, 32, 0),
+                                               (1, 600, 2, 64, 512, 0), (1, 50, 2, 24, 7, 3)])
+def test_swa_forward_backward_parity(B, s, H, hd, ws, npers):
+    q, k, v, go = _case(B, s, H, hd, 100 + s + ws)
+    out, aw = gpu_forward(q, k, v, ws, H, npers)
+    oo, awo = orc.swa_forward(q, k, v, ws, H, npers)
+    assert_close("out", orc.bf16_to_f32(out), orc.bf16_to_f32(oo), REL_TOL_BF16)
+    w, wo = orc.bf16_to_f32(aw), orc.bf16_to_f32(awo)
+    assert np.abs(w - wo).max() < 1e-2, "test_cuda_swa.rs:100 bound"
+    assert np.all(w[wo == 0] == 0), "unused slots are written as zero"
+    assert np.allclose(w.sum(-1), 1.0, atol=2e-2)
+    # backward on identical stored weights: fp32 round-off only
+    dq, dk, dv = gpu_backward(q, k, v, awo, go, ws, H, npers)
+    oq, ok, ov = orc.swa_backward(q, k, v, awo, go, ws, H, npers)
+    assert_close("d_q", dq, oq, 1e-4)
+    assert_close("d_k", dk, ok, 1e-4)
+    assert_close("d_v", dv, ov, 1e-4)
+    # end to end (GPU weights): bf16 tolerance
+    dq2, dk2, dv2 = gpu_backward(q, k, v, aw, go, ws, H, npers)
+    assert_close("d_q e2e", dq2, oq, REL_TOL_BF16)
+    assert_close("d_k e2e", dk2, ok, REL_TOL_BF16)
+    assert_close("d_v e2e", dv2, ov, REL_TOL_BF16)
+
+
+def test_swa_known_answers_on_gpu():
+    """core/src/swa.rs:286-344: window 1 copies V; identical keys average V."""
+    bf = lambda x: orc.f32_to_bf16(np.asarray(x, np.float32))
+    q = bf(np.tile([1.0, 0, 0, 0, 0, 0, 0, 0], (1, 4, 1)))
+    vals = np.zeros((1, 4, 8), np.float32)
+    vals[0, :, 0] = [10, 20, 30, 40]
+    out, aw = gpu_forward(q, q, bf(vals), 1, 1, 0)
+    assert np.array_equal(orc.bf16_to_f32(out), vals)
+    out, aw = gpu_forward(q, q, bf(vals), 2, 1, 0)
+    assert abs(orc.bf16_to_f32(out)[0, 3, 0] - 35.0) < 0.2
+
+
+def test_swa_backward_accumulates_dk_dv_and_overwrites_dq():
+    q, k, v, go = _case(1, 30, 2, 16, 7)
+    out, aw = gpu_forward(q, k, v, 8, 2, 0)
+    B, s, td = q.shape
+    dq = torch.full((B, s, td), 5.0, device="cuda")
+    dk = torch.full((B, s, td), 1.0, device="cuda")
+    dv = torch.full((B, s, td), 2.0, device="cuda")
+    D.call("swa_backward_f32_cuda", _u16(q), _u16(k), _u16(v), _u16(aw), dev(go), dq, dk, dv, s, 2, 16, 8, B, 0)
+    torch.cuda.synchronize()
+    oq, ok, ov = orc.swa_backward(q, k, v, aw, go, 8, 2, 0)
+    assert_close("d_q", host(dq), oq, 1e-4)
+    assert_close("d_k", host(dk) - 1.0, ok, 1e-4)
+    assert_close("d_v", host(dv) - 2.0, ov, 1e-4)
