@@ -330,6 +330,57 @@ unsigned adamw_update_multi_rocm(float *const *w, const float *const *g, float *
 unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, float max_grad_norm,
                                    float *out_norm, float *out_scale);
 
+/* ── CMS Conductor / Pulse and level dispatch (additions) ───────────────────
+ * Host-side state machines that the reference keeps in Rust; here behind the
+ * C ABI so that the level loop, the optimizer gating and the MAG combine are
+ * one library. */
+typedef struct nlh_conductor nlh_conductor;
+typedef struct nlh_adamw nlh_adamw;
+
+/* core/src/conductor.rs:47-55 Conductor::new (k levels, 1 <= k <= 8) */
+nlh_conductor *nlh_conductor_new(int k, const long long *chunk_sizes);
+void nlh_conductor_free(nlh_conductor *c);
+/* core/src/conductor.rs:61 set_seq_len */
+void nlh_conductor_set_seq_len(nlh_conductor *c, long long seq_len);
+/* core/src/conductor.rs:136-144 pulse: level l is active iff step % chunk_sizes[l] == 0
+ * or seq_len >= chunk_sizes[l] > 0.  active[k] receives 0/1; returns the
+ * bitmask of core/src/gpu_forward.rs:2449 pulse_to_bitmask. */
+unsigned nlh_conductor_pulse(const nlh_conductor *c, int *active);
+/* core/src/conductor.rs:147 advance, :152 step */
+void nlh_conductor_advance(nlh_conductor *c);
+long long nlh_conductor_step(const nlh_conductor *c);
+unsigned nlh_pulse_to_bitmask(const int *active, int k);
+/* core/src/conductor.rs:105-128 restore: 0 ok, 1 config mismatch, 2 pulse mismatch */
+int nlh_conductor_restore(nlh_conductor *c, int k, const long long *chunk_sizes, long long step,
+                          long long stream_pulse_id);
+
+/* Frequency-aware AdamW (core/src/adamw.rs, core/src/gpu_optimizer.rs:403-515):
+ * group -1 tensors update every step with the global step's bias correction;
+ * group l tensors update only when level l's pulse is on, with that level's
+ * own step counter.  w/g/m/v are device buffers owned by the caller. */
+nlh_adamw *nlh_adamw_new(int k, float beta1, float beta2, float eps, float weight_decay);
+void nlh_adamw_free(nlh_adamw *o);
+int nlh_adamw_add_tensor(nlh_adamw *o, int group, float *w, float *g, float *m, float *v, int n);
+void nlh_adamw_set_clamp(nlh_adamw *o, int tensor, float lo, float hi);
+/* norm_scale: device buffer of 2 floats {pre-clip norm, applied scale}; may be
+ * NULL when max_grad_norm <= 0.  Returns 0 on success. */
+unsigned nlh_adamw_step(nlh_adamw *o, const int *active_levels, float lr, float max_grad_norm,
+                        float *norm_scale);
+unsigned nlh_adamw_swa_step(const nlh_adamw *o);
+unsigned nlh_adamw_level_step(const nlh_adamw *o, int level);
+
+/* Level combine + MAG sigmoid gate (core/src/gpu_forward.rs:1027-1070):
+ * gate = sigmoid(c * sum_l y_l), gated = attn_out * gate, c = 1/sqrt(k) if k > 2.
+ * y_levels: HOST array of k device pointers; y_combined may be NULL. */
+void cms_combine_gate_rocm(const float *const *y_levels, int k, const float *attn_out,
+                           float *y_combined, float *gate, float *gated, long long n);
+/* core/src/gpu_backward.rs:263-283 */
+void cms_gate_backward_rocm(const float *d_gated, const float *attn_out, const float *gate, int k,
+                            float *d_attn, float *d_y_combined, long long n);
+/* Frozen level (core/src/gpu_forward.rs:2906-2950): y = M_h q per head, token-major */
+void memory_read_only_f32_rocm(const float *q_mem, const float *m, float *y, long long n_tokens, int nh,
+                               int hd);
+
 #ifdef __cplusplus
 }
 #endif

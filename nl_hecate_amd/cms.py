@@ -1,0 +1,107 @@
+"""Host-side mirror of the reference's CMS timing and optimizer types
+(core/src/conductor.rs, core/src/adamw.rs, core/src/gpu_optimizer.rs) over the
+C ABI.  Same names and semantics: `Conductor.pulse()` does not advance;
+`advance()` is called after every observer has read the pulse."""
+import ctypes
+from dataclasses import dataclass
+from typing import List
+
+from .ffi import lib
+
+
+@dataclass
+class Pulse:
+    """core/src/conductor.rs:12-17."""
+    global_step: int
+    active_levels: List[bool]
+
+    def bitmask(self) -> int:
+        """core/src/gpu_forward.rs:2449 pulse_to_bitmask."""
+        k = len(self.active_levels)
+        arr = (ctypes.c_int * k)(*[int(a) for a in self.active_levels])
+        return lib.nlh_pulse_to_bitmask(arr, k)
+
+
+class RestoreError(Exception):
+    pass
+
+
+class Conductor:
+    """core/src/conductor.rs:36-155."""
+
+    def __init__(self, k, chunk_sizes):
+        assert len(chunk_sizes) == k, "chunk_sizes length must equal k"
+        assert k >= 1, "k must be at least 1"
+        for i, cs in enumerate(chunk_sizes):
+            assert cs >= 1, f"chunk_sizes[{i}] must be >= 1"
+        self.k = k
+        self.chunk_sizes = list(chunk_sizes)
+        arr = (ctypes.c_longlong * k)(*chunk_sizes)
+        self._h = lib.nlh_conductor_new(k, arr)
+        if not self._h:
+            raise ValueError("nlh_conductor_new failed")
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib.nlh_conductor_free(self._h)
+            self._h = None
+
+    def set_seq_len(self, seq_len):
+        lib.nlh_conductor_set_seq_len(self._h, seq_len)
+
+    def pulse(self) -> Pulse:
+        act = (ctypes.c_int * self.k)()
+        lib.nlh_conductor_pulse(self._h, act)
+        return Pulse(self.step(), [bool(a) for a in act])
+
+    def advance(self):
+        lib.nlh_conductor_advance(self._h)
+
+    def step(self) -> int:
+        return lib.nlh_conductor_step(self._h)
+
+    def restore(self, k, chunk_sizes, step, stream_pulse_id):
+        arr = (ctypes.c_longlong * len(chunk_sizes))(*chunk_sizes)
+        rc = lib.nlh_conductor_restore(self._h, k, arr, step, stream_pulse_id)
+        if rc == 1:
+            raise RestoreError("ConfigMismatch")
+        if rc == 2:
+            raise RestoreError("PulseMismatch")
+
+
+class FrequencyAwareAdamW:
+    """core/src/adamw.rs FrequencyAwareAdamW / core/src/gpu_optimizer.rs:403 gpu_adamw_update:
+    always-active tensors (group -1) and per-level tensors gated by the Pulse."""
+
+    def __init__(self, k, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01):
+        self.k = k
+        self._h = lib.nlh_adamw_new(k, beta1, beta2, eps, weight_decay)
+        self._keep = []
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib.nlh_adamw_free(self._h)
+            self._h = None
+
+    def add_tensor(self, group, w, g, m, v):
+        for t in (w, g, m, v):
+            assert t.is_cuda and t.is_contiguous() and t.numel() == w.numel()
+        self._keep.append((w, g, m, v))
+        return lib.nlh_adamw_add_tensor(self._h, group, w.data_ptr(), g.data_ptr(), m.data_ptr(),
+                                        v.data_ptr(), w.numel())
+
+    def set_clamp(self, tensor_id, lo, hi):
+        lib.nlh_adamw_set_clamp(self._h, tensor_id, lo, hi)
+
+    def step(self, pulse: Pulse, lr, max_grad_norm=0.0, norm_scale=None):
+        act = (ctypes.c_int * self.k)(*[int(a) for a in pulse.active_levels[:self.k]])
+        rc = lib.nlh_adamw_step(self._h, act, lr, max_grad_norm,
+                                norm_scale.data_ptr() if norm_scale is not None else None)
+        if rc:
+            raise RuntimeError(f"nlh_adamw_step failed ({rc})")
+
+    def swa_step(self):
+        return lib.nlh_adamw_swa_step(self._h)
+
+    def level_step(self, level):
+        return lib.nlh_adamw_level_step(self._h, level)
