@@ -22,6 +22,10 @@
  *   checkpoint / segment schedule : equality with the full-trajectory result
  *       for C in {1,4,8,>=s,non-divisor}; checkpoint_count table
  *       (core/src/gpu_forward.rs:2885-2897).
+ *   orc_selfref_*   : finite differences of the double-precision forward for the
+ *       input and all six initial memories (as core/src/chunkwise_self_ref.rs:
+ *       810-917 does), an independent numpy implementation, frozen-snapshot
+ *       property of the self-generated targets (:974-1015), remainder chunk.
  *   orc_chunkwise_* : C=1 equals the exact rule; finite differences of the
  *       chunkwise forward in double precision; numpy matrix form.
  */
@@ -34,18 +38,28 @@
 #define REAL float
 #define SFX _f32
 #define SQRT sqrtf
+#define EXP expf
+#define LOG logf
 #include "rules.inc"
+#include "selfref.inc"
 #undef REAL
 #undef SFX
 #undef SQRT
+#undef EXP
+#undef LOG
 
 #define REAL double
 #define SFX _f64
 #define SQRT sqrt
+#define EXP exp
+#define LOG log
 #include "rules.inc"
+#include "selfref.inc"
 #undef REAL
 #undef SFX
 #undef SQRT
+#undef EXP
+#undef LOG
 
 /* ── SimpleRng: xorshift64, core/src/tensor.rs:380-408 ──────────────────── */
 void orc_simple_rng_fill_uniform(uint64_t seed, float scale, float *buf, int64_t n) {

@@ -366,3 +366,37 @@ def swa_backward(q, k, v, aw, d_out, window, num_heads, n_persistent=0):
     _call("orc_swa_backward", _c(q, np.uint16), _c(k, np.uint16), _c(v, np.uint16), _c(aw, np.uint16),
           _c(d_out, f), dq, dk, dv, s, num_heads, hd, window, B, n_persistent)
     return dq, dk, dv
+
+
+# ── HOPE self-referential memory (selfref.inc) ─────────────────────────────
+def selfref_forward(mems, embedded, chunk_size, self_gen=True):
+    """mems [6,d,d] (k,v,q,eta,alpha,mem), embedded [s,d]; float32 or float64.
+    Returns y [s,d], final memories [6,d,d] and the cache dict for the backward."""
+    dt = embedded.dtype
+    sfx, real = _sfx(dt)
+    s, d = embedded.shape
+    nc = (s + chunk_size - 1) // chunk_size
+    m = _c(mems, dt).copy()
+    c = dict(k=np.zeros((s, d), dt), v=np.zeros((s, d), dt), q=np.zeros((s, d), dt),
+             alpha=np.zeros(s, dt), theta=np.zeros(s, dt), alpha_mean=np.zeros(s, dt),
+             eta_mean=np.zeros(s, dt), traj=np.zeros((6, s + 1, d, d), dt),
+             frozen=np.zeros((nc, 6, d, d), dt), v_hat=np.zeros((6, s, d), dt),
+             embedded=_c(embedded, dt), chunk_size=chunk_size, self_gen=self_gen)
+    y = np.zeros((s, d), dt)
+    _call("orc_selfref_forward" + sfx, m, c["embedded"], y, c["k"], c["v"], c["q"], c["alpha"],
+          c["theta"], c["alpha_mean"], c["eta_mean"], c["traj"], c["frozen"], c["v_hat"],
+          s, d, chunk_size, int(self_gen), real=real)
+    return y, m, c
+
+
+def selfref_backward(cache, d_y):
+    dt = d_y.dtype
+    sfx, real = _sfx(dt)
+    s, d = d_y.shape
+    c = cache
+    d_emb = np.zeros((s, d), dt)
+    d_mems = np.zeros((6, d, d), dt)
+    _call("orc_selfref_backward" + sfx, c["embedded"], _c(d_y, dt), c["k"], c["v"], c["q"], c["alpha"],
+          c["theta"], c["alpha_mean"], c["eta_mean"], c["traj"], c["frozen"], c["v_hat"],
+          d_emb, d_mems, s, d, c["chunk_size"], int(c["self_gen"]), real=real)
+    return d_emb, d_mems
