@@ -381,6 +381,29 @@ void cms_gate_backward_rocm(const float *d_gated, const float *attn_out, const f
 void memory_read_only_f32_rocm(const float *q_mem, const float *m, float *y, long long n_tokens, int nh,
                                int hd);
 
+/* HOPE self-referential memory, chunkwise with frozen snapshots.  The reference runs it
+ * on the CPU only (core/src/chunkwise_self_ref.rs:52-222 chunkwise_self_ref_step,
+ * :336-620 chunkwise_self_ref_step_backward); these are the batched GPU forms.
+ * Component order of every [6, d*d] block: m_k, m_v, m_q, m_eta, m_alpha, m_mem (:27-29).
+ *   mems      [batch, 6, d*d]   in: initial memories, out: final memories
+ *   embedded  [batch, seq_len, d]
+ *   y, k/v/q_cache [batch, seq_len, d];  alpha/theta/alpha_mean/eta_mean_cache [batch, seq_len]
+ *   frozen    [batch, num_chunks, 6, d*d], num_chunks = ceil(seq_len / chunk_size)
+ * d in {16, 32, 64}. */
+void selfref_chunkwise_forward_f32_rocm(float *mems, const float *embedded, float *y, float *k_cache,
+                                        float *v_cache, float *q_cache, float *alpha_cache,
+                                        float *theta_cache, float *alpha_mean_cache, float *eta_mean_cache,
+                                        float *frozen, int seq_len, int d, int batch_size, int chunk_size,
+                                        int self_generated_values);
+/* d_embedded [batch, seq_len, d] and d_mems [batch, 6, d*d] (gradient w.r.t. the initial
+ * memories, per chain) are overwritten. */
+void selfref_chunkwise_backward_f32_rocm(const float *embedded, const float *d_y, const float *k_cache,
+                                         const float *v_cache, const float *q_cache,
+                                         const float *alpha_cache, const float *theta_cache,
+                                         const float *alpha_mean_cache, const float *eta_mean_cache,
+                                         const float *frozen, float *d_embedded, float *d_mems, int seq_len,
+                                         int d, int batch_size, int chunk_size, int self_generated_values);
+
 #ifdef __cplusplus
 }
 #endif
