@@ -7,9 +7,12 @@ synthetic input that is already resident in HBM.  Prints ONE JSON line.
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 Workloads (BASELINE.json `configs`):
-  titans_exact_c2   configs[1]: Titans LMM exact recurrence, 8 heads x 64 (d=512),
-                    batch 8, seq 2048, fp32, state checkpoints every 64 tokens
-                    (checkpointed forward + fused checkpointed backward).
+  titans_exact_c2   configs[1] (default): Titans LMM exact recurrence, 8 heads x 64
+                    (d=512), batch 8, seq 2048, fp32, state checkpoints every 64
+                    tokens (checkpointed forward + fused checkpointed backward).
+  hope_selfref_c4   configs[3]: HOPE self-referential memory, 8 heads x 64, batch 8,
+                    seq 2048, fp32, self-generated values, frozen snapshots per
+                    64-token chunk; grads to x and to the six initial memories.
 """
 import argparse
 import ctypes
@@ -52,6 +55,14 @@ def make_inputs(B, s, d, seed):
     return {n: t.contiguous() for n, t in x.items()}
 
 
+# HOPE self-referential memory, per head-token at d=64, counted on the update
+# equations as the reference evaluates them: forward 54 d^2 flop (5 projections,
+# read, and per memory: target, error, update), forward + backward 260 d^2.
+FLOP_HOPE_FWD = 54 * D_HEAD * D_HEAD
+FLOP_HOPE_BWD = 206 * D_HEAD * D_HEAD
+BYTES_HOPE_BWD = 4 * 4 * D_HEAD + 2 * 6 * D_HEAD * D_HEAD * 4 // 64   # x, dy, d_x + caches; snapshots / 64 tokens
+
+
 def cpu_baseline(x, heads, budget_s=12.0):
     """C restatement of the reference's Rust loops (oracle), one thread, on a
     bounded sample of the same inputs: whole batch elements (8 chains each)
@@ -76,28 +87,23 @@ def cpu_baseline(x, heads, budget_s=12.0):
                       f"full-trajectory forward + backward, {el:.1f} s"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="titans_exact_c2")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
+def cpu_baseline_hope(mems, x, dy, C, budget_s=12.0):
+    """Same oracle, HOPE path: whole chains until the time budget is used."""
+    from oracle import pyoracle as orc
+    B, s, d = x.shape
+    done = 0
+    t_start = time.perf_counter()
+    while done < B and time.perf_counter() - t_start < budget_s:
+        _, _, c = orc.selfref_forward(mems[done].numpy(), x[done].numpy(), C, True)
+        orc.selfref_backward(c, dy[done].numpy())
+        done += 1
+    el = time.perf_counter() - t_start
+    return {"value": done * s / 8 / el, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{done} of {B} chains of {s} tokens (8 chains = one sequence of d=512), "
+                      f"forward + backward, {el:.1f} s"}
 
-    import torch
-    from nl_hecate_amd import dispatch as D
-    from nl_hecate_amd.ffi import lib
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback).")
-    torch.cuda.set_device(0)
-    lib.load()
-
-    if args.workload != "titans_exact_c2":
-        sys.exit(f"unknown workload {args.workload}")
+def setup_titans_exact_c2(torch, D, lib):
     bs, heads, d, s, C = 8, 8, 64, 2048, 64
     B = bs * heads
     x = make_inputs(B, s, d, 0x5EED0002)
@@ -118,6 +124,90 @@ def main():
                dv["eta"], mc, sc, dv["dy"], g["dk"], g["dv"], g["dq"], g["da"], g["dt"], g["de"],
                g["dm"], g["ds"], s, d, B, C, 0.0, F32_MAX)
 
+    return dict(
+        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s,
+        flop_fwd=FLOP_FWD, flop_bwd=FLOP_BWD, bytes_bwd=BYTES_BWD,
+        traffic_bwd=int((193.7 + 298.0) * 2**20),   # measured: 193.7 MiB read, 298.0 MiB written
+        kernel="rule_bwd_fused_kernel<64,true> (+ finalize, per launch of the backward entry point)",
+        kernel_names={"forward": "forward_ckpt", "backward": "backward_ckpt_fused"},
+        config={"workload": "BASELINE configs[1]: Titans LMM exact recurrence, 8 heads x 64 (d=512), "
+                            "batch 8, seq 2048, fp32 state, checkpoints every 64 tokens, fwd+bwd",
+                "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "checkpoint_interval": C},
+        cpu=lambda: cpu_baseline(x, heads))
+
+
+def setup_hope_selfref_c4(torch, D, lib):
+    from nl_hecate_amd import selfref as SR
+    bs, heads, d, s, C = 8, 8, 64, 2048, 64
+    B = bs * heads
+    g = torch.Generator(device="cpu").manual_seed(0x5EED0004)
+    lim = (6.0 / (2 * d)) ** 0.5
+    mems = (torch.rand(B, 6, d, d, generator=g) * 2 - 1) * lim
+    mems[:, 5] = 0.0
+    x = torch.randn(B, s, d, generator=g) / (heads * d) ** 0.5
+    dy = torch.randn(B, s, d, generator=g)
+    m0, xd, dyd = mems.cuda(), x.cuda(), dy.cuda()
+    st = {}
+
+    def fwd():
+        m = m0.clone()
+        st["y"], st["cache"] = SR.chunkwise_self_ref_step(m, xd, C, True)
+
+    def bwd():
+        st["g"] = SR.chunkwise_self_ref_step_backward(st["cache"], dyd)
+
+    return dict(
+        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s,
+        flop_fwd=FLOP_HOPE_FWD, flop_bwd=FLOP_HOPE_BWD, bytes_bwd=BYTES_HOPE_BWD,
+        traffic_bwd=int((4041.7 + 2214.0) * 2**20),  # measured: per-token G trajectory through HBM
+        kernel="selfref_bwd_kernel<64,true> (one launch of the backward entry point)",
+        kernel_names={"forward": "selfref_forward", "backward": "selfref_backward"},
+        config={"workload": "BASELINE configs[3]: HOPE self-referential memory, 8 heads x 64 (d=512), "
+                            "batch 8, seq 2048, fp32, self-generated values, frozen snapshots per 64 tokens, fwd+bwd",
+                "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "chunk_size": C},
+        cpu=lambda: cpu_baseline_hope(mems, x, dy, C))
+
+
+WORKLOADS = {"titans_exact_c2": setup_titans_exact_c2, "hope_selfref_c4": setup_hope_selfref_c4}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="titans_exact_c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="launch a plain map kernel (256 MiB read, 256 MiB written) 5 times and exit: "
+                         "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
+
+    import torch
+    from nl_hecate_amd import dispatch as D
+    from nl_hecate_amd.ffi import lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback).")
+    torch.cuda.set_device(0)
+    lib.load()
+
+    if args.calibrate_copy:
+        n = 64 << 20
+        a = torch.randn(n, dtype=torch.float32, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(5):
+            D.call("sigmoid_cuda", a, b, n)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_kernel": "map_kernel (sigmoid_cuda)", "launches": 5,
+                          "read_bytes_per_launch": 4 * n, "written_bytes_per_launch": 4 * n}))
+        return
+
+    w = WORKLOADS[args.workload](torch, D, lib)
+    fwd, bwd = w["fwd"], w["bwd"]
+
     for _ in range(args.warmup):
         fwd(); bwd()
     torch.cuda.synchronize()
@@ -131,8 +221,7 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = wall_ms / args.steps
-    tokens = bs * s
-    value = tokens / (ms_per_step * 1e-3)
+    value = w["tokens"] / (ms_per_step * 1e-3)
 
     # per-kernel durations with events on the launch stream (outside the timed region)
     def avg_ms(fn, n=10):
@@ -141,30 +230,39 @@ def main():
             fn()
         return lib.nlh_timer_stop_ms() / n
     fwd_ms, bwd_ms = avg_ms(fwd), avg_ms(bwd)
-    head_tokens = B * s
-    bwd_tflops = FLOP_BWD * head_tokens / (bwd_ms * 1e-3) / 1e12
-    roofline = {"kernel": "rule_bwd_fused_kernel<64,true> (+ finalize, per launch of the backward entry point)",
+    # the dominant kernel alone: event pairs around its launches inside the entry point
+    lib.nlh_kernel_timer_enable(1)
+    for _ in range(10):
+        bwd()
+    n_launch, name = ctypes.c_int(0), ctypes.create_string_buffer(128)
+    kern_ms = lib.nlh_kernel_timer_read_ms(ctypes.byref(n_launch), name, 128) / max(n_launch.value, 1)
+    lib.nlh_kernel_timer_enable(0)
+    assert n_launch.value == 10 and name.value.decode() in w["kernel"], (n_launch.value, name.value)
+    head_tokens = w["head_tokens"]
+    bwd_tflops = w["flop_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e12
+    roofline = {"kernel": w["kernel"],
                 "bound": "mfma", "achieved": bwd_tflops, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                "frac": bwd_tflops / PEAK_FP32_TFLOPS, "traffic": None,
+                "frac": bwd_tflops / PEAK_FP32_TFLOPS, "traffic": w["traffic_bwd"],
+                "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel; "
+                                "see profiles/" + args.workload + "_kernels_and_hbm_traffic.txt)",
+                "algorithmic_bytes": w["bytes_bwd"] * head_tokens,
                 "note": "fp32 vector/matrix peak (157.3 TFLOP/s); rank-1 and mat-vec work, not a contraction",
-                "avg_launch_ms": bwd_ms,
-                "hbm": {"achieved": BYTES_BWD * head_tokens / (bwd_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                "avg_launch_ms": kern_ms, "entry_point_ms": bwd_ms,
+                "hbm": {"achieved": w["bytes_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                         "unit": "GB/s"}}
     out = {
         "metric": METRIC, "value": value, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "BASELINE configs[1]: Titans LMM exact recurrence, 8 heads x 64 (d=512), "
-                               "batch 8, seq 2048, fp32 state, checkpoints every 64 tokens, fwd+bwd",
-                   "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "checkpoint_interval": C},
+        "config": w["config"],
         "event_ms_per_step": ev_ms / args.steps,
-        "kernels_ms": {"forward_ckpt": fwd_ms, "backward_ckpt_fused": bwd_ms},
-        "fwd_fp32_tflops": FLOP_FWD * head_tokens / (fwd_ms * 1e-3) / 1e12,
+        "kernels_ms": {w["kernel_names"]["forward"]: fwd_ms, w["kernel_names"]["backward"]: bwd_ms},
+        "fwd_fp32_tflops": w["flop_fwd"] * head_tokens / (fwd_ms * 1e-3) / 1e12,
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(x, heads)
+        out["cpu_baseline"] = w["cpu"]()
     print(json.dumps(out))
 
 

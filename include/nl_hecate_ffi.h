@@ -37,6 +37,12 @@ void nlh_release_workspace(void);      /* frees the library's device scratch */
  * (blocks until the stop event completes); negative on failure. */
 int nlh_timer_start(void);
 float nlh_timer_stop_ms(void);
+/* Per-kernel timing of the dominant kernel of an entry point (the fused checkpointed
+ * backward, the self-referential backward): while enabled, each such launch is bracketed
+ * by an event pair on the launch stream (at most 256 between reads).  read_ms waits for
+ * them, returns their summed duration, the launch count and the kernel's name, and resets. */
+int nlh_kernel_timer_enable(int on);
+float nlh_kernel_timer_read_ms(int *launches, char *name, int name_len);
 /* Runs the cross-lane primitives on known data; returns 0 when all agree. */
 int nlh_selftest_lane_ops(void);
 

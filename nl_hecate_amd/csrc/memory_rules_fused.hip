@@ -337,6 +337,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
 
 template <int D, bool HAS_S, bool FROZEN>
 static void launch_fused_d(const FusedArgs &a) {
+    KernelTimer kt("rule_bwd_fused_kernel");
     hipLaunchKernelGGL((rule_bwd_fused_kernel<D, HAS_S, FROZEN>), dim3(a.batch * a.parts),
                        dim3(kThreads), 0, stream(), a);
     check_launch("rule_bwd_fused_kernel");

@@ -23,6 +23,15 @@ hipStream_t stream();   // launch stream (the null stream unless nlh_set_stream 
 float *scratch(int slot, size_t bytes);
 constexpr int kScratchSlots = 12;
 
+// Optional per-kernel timing: while enabled (nlh_kernel_timer_enable), a
+// KernelTimer around a launch records an event pair on the launch stream;
+// nlh_kernel_timer_read_ms sums the pairs.  Off by default: no events, no cost.
+struct KernelTimer {
+    explicit KernelTimer(const char *name);
+    ~KernelTimer();
+    int slot;
+};
+
 inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 }  // namespace nlh

@@ -9,6 +9,15 @@
 
 namespace nlh {
 
+// per-kernel timing state (see runtime.h)
+constexpr int kKtMax = 256;
+static bool g_kt_on = false;
+static int g_kt_used = 0;
+static hipEvent_t g_kt_ev[kKtMax][2];
+static int g_kt_created = 0;
+static char g_kt_name[128] = {0};
+
+
 static int g_error_mode = 0;
 static bool g_failed = false;
 static char g_error[512] = "";
@@ -69,6 +78,22 @@ float *scratch(int slot, size_t bytes) {
     return (float *)s.ptr;
 }
 
+KernelTimer::KernelTimer(const char *name) : slot(-1) {
+    if (!g_kt_on || g_kt_used >= kKtMax) return;
+    if (g_kt_used >= g_kt_created) {
+        if (hipEventCreate(&g_kt_ev[g_kt_created][0]) != hipSuccess ||
+            hipEventCreate(&g_kt_ev[g_kt_created][1]) != hipSuccess)
+            return;
+        g_kt_created++;
+    }
+    slot = g_kt_used++;
+    snprintf(g_kt_name, sizeof(g_kt_name), "%s", name);
+    (void)hipEventRecord(g_kt_ev[slot][0], stream());
+}
+KernelTimer::~KernelTimer() {
+    if (slot >= 0) (void)hipEventRecord(g_kt_ev[slot][1], stream());
+}
+
 }  // namespace nlh
 
 extern "C" {
@@ -109,6 +134,28 @@ float nlh_timer_stop_ms(void) {
     if (hipEventSynchronize(g_ev1) != hipSuccess) return ms;
     if (hipEventElapsedTime(&ms, g_ev0, g_ev1) != hipSuccess) return -1.f;
     return ms;
+}
+
+int nlh_kernel_timer_enable(int on) {
+    nlh::g_kt_on = on != 0;
+    nlh::g_kt_used = 0;
+    nlh::g_kt_name[0] = 0;
+    return 0;
+}
+
+float nlh_kernel_timer_read_ms(int *launches, char *name, int name_len) {
+    float total = 0.f;
+    for (int i = 0; i < nlh::g_kt_used; i++) {
+        float ms = 0.f;
+        if (hipEventSynchronize(nlh::g_kt_ev[i][1]) != hipSuccess ||
+            hipEventElapsedTime(&ms, nlh::g_kt_ev[i][0], nlh::g_kt_ev[i][1]) != hipSuccess)
+            return -1.f;
+        total += ms;
+    }
+    if (launches) *launches = nlh::g_kt_used;
+    if (name && name_len > 0) snprintf(name, name_len, "%s", nlh::g_kt_name);
+    nlh::g_kt_used = 0;
+    return total;
 }
 
 const char *nlh_version(void) { return "nl_hecate_rocm 0.1 (gfx950)"; }

@@ -43,6 +43,14 @@ __device__ __forceinline__ float sr_softplus(float x) {
 
 constexpr int DPP_ROR4 = 0x124;
 
+// Barrier for data exchanged through LDS only.  __syncthreads() also waits for
+// every outstanding global load and store of the wave, which would put the HBM
+// round trip of the per-token cache writes and of the prefetched trajectory
+// reads on the critical path of each token.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ float quad_allreduce(float x) { return group_allreduce<4>(x); }
 
 // Sum over the 16 lanes of a wave that share (lane % 4): the rows a wave owns.
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(4 * D) void selfref_fwd_kernel(
                 float *dst = cq == 0 ? k_cache : cq == 1 ? v_cache : q_cache;
                 dst[(b * s + t) * D + r] = val;
             }
-            __syncthreads();
+            lds_barrier();
             float em = 0.f, am = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; w++) { em += gpart[pb][2 * w]; am += gpart[pb][2 * w + 1]; }
@@ -455,7 +463,7 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                 if (lane == 0) { sp[pb][wave][0] = alp; sp[pb][wave][1] = thp; }
                 if (cq == 0) wv[pb][0][r] = w;
                 if (!SG && cq == 1) wv[pb][1][r] = wh;
-                __syncthreads();
+                lds_barrier();
 
                 float dal = 0.f, dth = 0.f;
 #pragma unroll
@@ -585,6 +593,7 @@ void launch_bwd(bool sg, int batch, const float *emb, const float *dy, const flo
                 const float *qc, const float *al, const float *th, const float *am, const float *em,
                 const float *frozen, float *d_emb, float *d_mems, float *gtraj, float *htraj, float *rp, int s,
                 int C, int nc) {
+    KernelTimer kt("selfref_bwd_kernel");
     if (sg)
         hipLaunchKernelGGL((selfref_bwd_kernel<D, true>), dim3(batch), dim3(4 * D), 0, stream(), emb, dy, kc, vc,
                            qc, al, th, am, em, frozen, d_emb, d_mems, gtraj, htraj, rp, s, C, nc);
