@@ -410,6 +410,23 @@ void selfref_chunkwise_backward_f32_rocm(const float *embedded, const float *d_y
                                          const float *frozen, float *d_embedded, float *d_mems, int seq_len,
                                          int d, int batch_size, int chunk_size, int self_generated_values);
 
+/* Frozen-M0 chunkwise Titans rule in matrix form on the matrix cores (same semantics as
+ * titans_chunkwise_{forward,backward}_f32_cuda, core/src/cuda_ffi.rs:376/386, with
+ * error_clip = 0 and no M-norm projection); no counterpart in the reference.
+ * k/v/q: bf16 bit patterns [batch, seq_len, 64] (..._bf16_rocm) or float (..._mm_f32_rocm);
+ * gates, states, y and all gradients are float.  d = 64, chunk_size in 1..64.
+ * m_initial / s_initial [batch, d*d]; m/s_chunk_states [batch, num_chunks+1, d*d]. */
+void titans_chunkwise_forward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                        const float *alpha, const float *theta, const float *eta,
+                                        const float *m_initial, const float *s_initial,
+                                        float *m_chunk_states, float *s_chunk_states, float *y,
+                                        int seq_len, int d, int batch_size, int chunk_size);
+void titans_chunkwise_forward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                          const float *alpha, const float *theta, const float *eta,
+                                          const float *m_initial, const float *s_initial,
+                                          float *m_chunk_states, float *s_chunk_states, float *y,
+                                          int seq_len, int d, int batch_size, int chunk_size);
+
 #ifdef __cplusplus
 }
 #endif
