@@ -426,6 +426,23 @@ void titans_chunkwise_forward_mm_f32_rocm(const float *k_mem, const float *v_mem
                                           const float *m_initial, const float *s_initial,
                                           float *m_chunk_states, float *s_chunk_states, float *y,
                                           int seq_len, int d, int batch_size, int chunk_size);
+/* d_k/d_v/d_q [batch, seq_len, 64] and d_alpha/d_theta/d_eta [batch, seq_len] are overwritten;
+ * d_m_initial / d_s_initial [d*d] are accumulated (+=) with the sum over the batch, like the
+ * reference's chunkwise backward. */
+void titans_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                         const float *alpha, const float *theta, const float *eta,
+                                         const float *m_chunk_states, const float *s_chunk_states,
+                                         const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                         float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
+                                         float *d_s_initial, int seq_len, int d, int batch_size,
+                                         int chunk_size);
+void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                           const float *alpha, const float *theta, const float *eta,
+                                           const float *m_chunk_states, const float *s_chunk_states,
+                                           const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                           float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
+                                           float *d_s_initial, int seq_len, int d, int batch_size,
+                                           int chunk_size);
 
 #ifdef __cplusplus
 }

@@ -341,6 +341,378 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
     }
 }
 
+// ── backward, chunk-local pass: what the adjoint scan needs ─────────────────
+//   T_a, T_b as in the forward (the chunk map is right-multiplication by symmetric matrices)
+//   C_1 = G0  = (a.dY)^T Q + dE_loc^T K,   dE_loc[j] = -theta_j sum_{t>=j} c[t,j] (q_t.k_j) dy_t
+//   C_2 = GS0 = (beta.dY)^T Q
+template <class TIn>
+__global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restrict__ k, const TIn *__restrict__ q,
+                                                            const float *__restrict__ d_y,
+                                                            const float *__restrict__ alpha,
+                                                            const float *__restrict__ theta,
+                                                            const float *__restrict__ eta, float *__restrict__ loc,
+                                                            float *__restrict__ locs, int s, int C, int nc,
+                                                            int has_s) {
+    extern __shared__ float smem[];
+    float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Cc = Ds + MAT, *El = Cc + MAT;
+    __shared__ Coef cf;
+    __shared__ float wM[CW], wS[CW];
+    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    stage(Ks, k + tok * HD, L);
+    stage(Qs, q + tok * HD, L);
+    stage(Ds, d_y + tok * HD, L);
+    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+    __syncthreads();
+    coefficients(cf, L, Cc, nullptr, nullptr);
+    __syncthreads();
+    if (threadIdx.x < CW) {
+        wM[threadIdx.x] = -cf.th[threadIdx.x] * cf.cl[threadIdx.x];
+        wS[threadIdx.x] = -cf.th[threadIdx.x] * cf.bl[threadIdx.x];
+    }
+    const float aL = cf.a[L - 1], betaL = cf.beta[L - 1], hL = cf.h[L - 1];
+    if (threadIdx.x == 0) {
+        float *sc = locs + ((size_t)chain * nc + ci) * 4;
+        sc[0] = aL; sc[1] = betaL; sc[2] = hL; sc[3] = 0.f;
+    }
+    __syncthreads();
+    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1);
+    float *out = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
+    auto bK = [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; };
+#pragma unroll 1
+    for (int o = 0; o < 2; o++) {
+        const float *wv = o ? wS : wM;
+        f32x16 acc = zero16();
+        mma32(acc, 64, [&](int m, int kk) { return Ks[kk * LDM + m0 + m] * wv[kk]; }, bK);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int row = m0 + c_row(i), col = n0 + c_col();
+            out[(size_t)o * HD * HD + row * HD + col] = acc[i] + ((o == 0 && row == col) ? aL : 0.f);
+        }
+    }
+    {   // Cc <- c[t][j] * (q_t . k_j), in place (own tile only)
+        f32x16 p = zero16();
+        mma32(p, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+#pragma unroll
+        for (int i = 0; i < 16; i++) Cc[(m0 + c_row(i)) * LDM + n0 + c_col()] *= p[i];
+    }
+    __syncthreads();
+    {   // dE_loc[j][i] = -theta_j sum_t Cc[t][j] dY[t][i]
+        f32x16 e = zero16();
+        mma32(e, 64, [&](int m, int kk) { return Cc[kk * LDM + m0 + m]; },
+              [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int row = m0 + c_row(i);
+            El[row * LDM + n0 + c_col()] = -cf.th[row] * e[i];
+        }
+    }
+    __syncthreads();
+    f32x16 g0 = zero16(), gs = zero16();
+    mma32(g0, 64, [&](int m, int kk) { return cf.a[kk] * Ds[kk * LDM + m0 + m]; },
+          [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+    mma32(g0, 64, [&](int m, int kk) { return El[kk * LDM + m0 + m]; }, bK);
+    if (has_s)
+        mma32(gs, 64, [&](int m, int kk) { return cf.beta[kk] * Ds[kk * LDM + m0 + m]; },
+              [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int row = m0 + c_row(i), col = n0 + c_col();
+        out[(size_t)2 * HD * HD + row * HD + col] = g0[i];
+        out[(size_t)3 * HD * HD + row * HD + col] = gs[i];
+    }
+}
+constexpr size_t kLocalBwdLds = 5 * MAT * sizeof(float);
+
+// <M0, dMo>, <S0, dMo>, <S0, dSo> per chunk (dMo, dSo: adjoints of the chunk's end state)
+__global__ __launch_bounds__(kThr) void cw_state_dots_kernel(const float *__restrict__ m_states,
+                                                             const float *__restrict__ s_states,
+                                                             const float *__restrict__ dm_states,
+                                                             const float *__restrict__ ds_states,
+                                                             float *__restrict__ scal, int nc, int has_s) {
+    __shared__ float slot[3][4];
+    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc;
+    const size_t o0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, o1 = o0 + HD * HD;
+    float x0 = 0.f, x1 = 0.f, x2 = 0.f;
+    for (int e = threadIdx.x; e < HD * HD; e += kThr) {
+        const float m = m_states[o0 + e], dm = dm_states[o1 + e];
+        x0 = fmaf(m, dm, x0);
+        if (has_s) {
+            const float sv = s_states[o0 + e];
+            x1 = fmaf(sv, dm, x1);
+            x2 = fmaf(sv, ds_states[o1 + e], x2);
+        }
+    }
+    x0 = wave_allreduce(x0); x1 = wave_allreduce(x1); x2 = wave_allreduce(x2);
+    if ((threadIdx.x & 63) == 0) {
+        slot[0][threadIdx.x >> 6] = x0; slot[1][threadIdx.x >> 6] = x1; slot[2][threadIdx.x >> 6] = x2;
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const float *p = slot[threadIdx.x];
+        scal[((size_t)chain * nc + ci) * 4 + threadIdx.x] = p[0] + p[1] + p[2] + p[3];
+    }
+}
+
+// Row sums of a 32x32 accumulator tile: every lane gets, for each of its 16 rows, the sum
+// over the tile's 32 columns.
+__device__ __forceinline__ void tile_row_sums(f32x16 &x) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) x[i] = group_allreduce<32>(x[i]);
+}
+
+// ── backward, main per-chunk pass: dQ, dK, dV, dtheta; exports for the gate pass ──
+//   pvec [chain][token][4] = p0, ps, g1, g2   xs [chain][chunk][64][64] = X[t][j] = (dy_t.e_j)(q_t.k_j)
+template <class TIn>
+__global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
+    const TIn *__restrict__ k, const TIn *__restrict__ v, const TIn *__restrict__ q, const float *__restrict__ d_y,
+    const float *__restrict__ alpha, const float *__restrict__ theta, const float *__restrict__ eta,
+    const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
+    const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
+    float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, int s, int C, int nc,
+    int has_s) {
+    extern __shared__ float smem[];
+    float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Es = Ds + MAT, *Ms = Es + MAT, *B5 = Ms + MAT,
+          *B6 = B5 + MAT, *B7 = B6 + MAT, *B8 = B7 + MAT;
+    __shared__ Coef cf;
+    __shared__ float part[5][2][CW];   // p0, ps, dtheta, g1, g2: one partial per column half
+    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, st1 = st0 + HD * HD;
+    float *Ss = B5, *Cc = B6;
+    stage(Ks, k + tok * HD, L);
+    stage(Qs, q + tok * HD, L);
+    stage(Ds, d_y + tok * HD, L);
+    stage(Es, v + tok * HD, L);
+    stage(Ms, m_states + st0, 64);
+    if (has_s) stage(Ss, s_states + st0, 64);
+    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+    __syncthreads();
+    coefficients(cf, L, Cc, nullptr, nullptr);
+    __syncthreads();
+    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1;
+    const bool writer = (threadIdx.x & 31) == 0;
+    f32x16 p = zero16(), dq = zero16();
+    {
+        f32x16 e = zero16(), ym = zero16(), ys = zero16();
+        mma32(e, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+        mma32(p, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        mma32(ym, 64, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; });
+        if (has_s)
+            mma32(ys, 64, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
+                  [&](int kk, int n) { return Ss[kk * LDM + n0 + n]; });
+        f32x16 r0, r1;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int row = m0 + c_row(i), col = n0 + c_col();
+            Es[row * LDM + col] = e[i] - Es[row * LDM + col];
+            const float qv = Qs[row * LDM + col];
+            r0[i] = ym[i] * qv; r1[i] = ys[i] * qv;
+            dq[i] = cf.a[row] * ym[i] + cf.beta[row] * ys[i];
+        }
+        tile_row_sums(r0); tile_row_sums(r1);
+        if (writer) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) { part[0][nh][m0 + c_row(i)] = r0[i]; part[1][nh][m0 + c_row(i)] = r1[i]; }
+        }
+    }
+    __syncthreads();   // E complete; S0 no longer needed
+    float *CP = B5, *CR = B7;
+    {
+        f32x16 r = zero16();
+        mma32(r, 64, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return Es[(n0 + n) * LDM + kk]; });
+        float *xo = xs + ((size_t)chain * nc + ci) * CW * CW;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int row = m0 + c_row(i), col = n0 + c_col();
+            const float c = Cc[row * LDM + col];
+            xo[row * CW + col] = r[i] * p[i];
+            CP[row * LDM + col] = c * p[i];
+            CR[row * LDM + col] = c * r[i];
+        }
+    }
+    __syncthreads();   // CP, CR complete; Cc no longer needed
+    mma32(dq, 64, [&](int m, int kk) { return -cf.th[kk] * CR[(m0 + m) * LDM + kk]; },
+          [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int row = m0 + c_row(i), col = n0 + c_col();
+        if (row < L) d_q[(tok + row) * HD + col] = dq[i];
+    }
+    float *dMs = B6, *dSs = B8;
+    stage(dMs, dm_states + st1, 64);
+    if (has_s) stage(dSs, ds_states + st1, 64);
+    __syncthreads();
+    {
+        // Dk[j][i] = sum_t CP[t][j] dY[t][i] + cl_j (K dMo^T)[j][i] + bl_j (K dSo^T)[j][i]
+        f32x16 dk = zero16(), t1 = zero16(), t2 = zero16();
+        mma32(dk, 64, [&](int m, int kk) { return CP[kk * LDM + m0 + m]; },
+              [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
+        mma32(t1, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return dMs[(n0 + n) * LDM + kk]; });
+        if (has_s)
+            mma32(t2, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+                  [&](int kk, int n) { return dSs[(n0 + n) * LDM + kk]; });
+        f32x16 rt;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int row = m0 + c_row(i), col = n0 + c_col();
+            dk[i] += cf.cl[row] * t1[i] + cf.bl[row] * t2[i];
+            rt[i] = Es[row * LDM + col] * dk[i];
+            dk[i] *= -cf.th[row];                                 // dE = -theta_j Dk
+            if (row < L) d_v[(tok + row) * HD + col] = -dk[i];    // dV = -dE
+        }
+        tile_row_sums(rt);
+        if (writer) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) part[2][nh][m0 + c_row(i)] = rt[i];
+        }
+        __syncthreads();   // every wave is done reading CP
+#pragma unroll
+        for (int i = 0; i < 16; i++) CP[(m0 + c_row(i)) * LDM + n0 + c_col()] = dk[i];
+    }
+    __syncthreads();
+    {
+        const float *dE = B5;
+        // DTe[j][n] = sum_t CR[t][j] Q[t][n] + cl_j (E dMo)[j][n] + bl_j (E dSo)[j][n]
+        f32x16 dt = zero16(), t3 = zero16(), t4 = zero16(), em = zero16();
+        mma32(dt, 64, [&](int m, int kk) { return CR[kk * LDM + m0 + m]; },
+              [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+        mma32(t3, 64, [&](int m, int kk) { return Es[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return dMs[kk * LDM + n0 + n]; });
+        if (has_s)
+            mma32(t4, 64, [&](int m, int kk) { return Es[(m0 + m) * LDM + kk]; },
+                  [&](int kk, int n) { return dSs[kk * LDM + n0 + n]; });
+        mma32(em, 64, [&](int m, int kk) { return dE[(m0 + m) * LDM + kk]; },
+              [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; });
+        f32x16 r3, r4;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int row = m0 + c_row(i), col = n0 + c_col();
+            const float kv = Ks[row * LDM + col];
+            r3[i] = t3[i] * kv; r4[i] = t4[i] * kv;
+            const float dte = dt[i] + cf.cl[row] * t3[i] + cf.bl[row] * t4[i];
+            if (row < L) d_k[(tok + row) * HD + col] = -cf.th[row] * dte + em[i];
+        }
+        tile_row_sums(r3); tile_row_sums(r4);
+        if (writer) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) { part[3][nh][m0 + c_row(i)] = r3[i]; part[4][nh][m0 + c_row(i)] = r4[i]; }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < L) {
+        const int t = threadIdx.x;
+        d_theta[tok + t] = -(part[2][0][t] + part[2][1][t]);
+        float *pv = pvec + (tok + t) * 4;
+        pv[0] = part[0][0][t] + part[0][1][t];
+        pv[1] = part[1][0][t] + part[1][1][t];
+        pv[2] = part[3][0][t] + part[3][1][t];
+        pv[3] = part[4][0][t] + part[4][1][t];
+    }
+}
+constexpr size_t kGradsBwdLds = 9 * MAT * sizeof(float);
+
+// ── backward, gate pass: d_alpha, d_eta of one chunk ────────────────────────
+//   d_alpha_t = -<M_{t-1}, A_t>,  d_eta_t = <S_{t-1}, B_t>  with A, B the adjoints of M_t, S_t:
+//   <M_tau, dy_t' q_t'^T> = a_tau p0[t'] + beta_tau ps[t'] + sum_j W[tau][j] X[t'][j]
+//   <S_tau, dy_t' q_t'^T> = h_tau ps[t'] + sum_j Ws[tau][j] X[t'][j],  Ws[tau][j] = -theta_j bb[j][tau]
+//   and the same with dMo / dSo in place of dy q^T (g1, g2 and the three state dots).
+__global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restrict__ alpha,
+                                                            const float *__restrict__ theta,
+                                                            const float *__restrict__ eta,
+                                                            const float *__restrict__ pvec,
+                                                            const float *__restrict__ xs,
+                                                            const float *__restrict__ scal,
+                                                            float *__restrict__ d_alpha, float *__restrict__ d_eta,
+                                                            int s, int C, int nc, int has_s) {
+    extern __shared__ float smem[];
+    float *Xs = smem, *Cc = Xs + MAT, *Bb = Cc + MAT, *Rr = Bb + MAT;
+    __shared__ Coef cf;
+    __shared__ float p0[CW], ps[CW], g1[CW], g2[CW], um[CW], usm[CW], uss[CW];
+    __shared__ float part[2][2][CW];
+    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    stage(Xs, xs + ((size_t)chain * nc + ci) * CW * CW, 64);
+    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+    if (threadIdx.x < CW) {
+        const int t = threadIdx.x;
+        const float4 pv = t < L ? *reinterpret_cast<const float4 *>(pvec + (tok + t) * 4) : make_float4(0, 0, 0, 0);
+        p0[t] = pv.x; ps[t] = pv.y; g1[t] = pv.z; g2[t] = pv.w;
+    }
+    const float m0dm = scal[((size_t)chain * nc + ci) * 4 + 0], s0dm = scal[((size_t)chain * nc + ci) * 4 + 1],
+                s0ds = scal[((size_t)chain * nc + ci) * 4 + 2];
+    __syncthreads();
+    coefficients(cf, L, Cc, Bb, Rr);
+    __syncthreads();
+    if (threadIdx.x < CW) {   // mat-vecs with W and Ws
+        const int tau = threadIdx.x;
+        float x0 = 0.f, x1 = 0.f, x2 = 0.f;
+        for (int j = 0; j <= tau && j < L; j++) {
+            const float wf = -cf.th[j] * Cc[tau * LDM + j], wsv = -cf.th[j] * Bb[j * LDM + tau];
+            x0 = fmaf(wf, g1[j], x0); x1 = fmaf(wsv, g1[j], x1); x2 = fmaf(wsv, g2[j], x2);
+        }
+        um[tau] = cf.a[tau] * m0dm + cf.beta[tau] * s0dm + x0;
+        usm[tau] = cf.h[tau] * s0dm + x1;
+        uss[tau] = cf.h[tau] * s0ds + x2;
+    }
+    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1;
+    f32x16 ua = zero16(), us = zero16();
+    mma32(ua, 64, [&](int m, int kk) { return -cf.th[kk] * Cc[(m0 + m) * LDM + kk]; },
+          [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
+    if (has_s)
+        mma32(us, 64, [&](int m, int kk) { return -cf.th[kk] * Bb[kk * LDM + m0 + m]; },
+              [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
+    // row tau feeds token tau+1: weights r[tau+1][t'] (d_alpha) and c[t'][tau+1] (d_eta), zero for t' <= tau
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int tau = m0 + c_row(i), tp = n0 + c_col();
+        const float uM = cf.a[tau] * p0[tp] + cf.beta[tau] * ps[tp] + ua[i];
+        const float uS = cf.h[tau] * ps[tp] + us[i];
+        const bool ok = tau + 1 < CW;
+        ua[i] = ok ? Rr[(tau + 1) * LDM + tp] * uM : 0.f;
+        us[i] = ok ? Cc[tp * LDM + tau + 1] * uS : 0.f;
+    }
+    tile_row_sums(ua); tile_row_sums(us);
+    if ((threadIdx.x & 31) == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) { part[0][nh][m0 + c_row(i)] = ua[i]; part[1][nh][m0 + c_row(i)] = us[i]; }
+    }
+    __syncthreads();
+    if (threadIdx.x < L) {
+        const int t = threadIdx.x;
+        float da, de;
+        if (t == 0) {
+            da = Rr[L - 1] * m0dm; de = cf.cl[0] * s0dm + cf.bl[0] * s0ds;
+            for (int tp = 0; tp < L; tp++) {
+                da = fmaf(Rr[tp], p0[tp], da);
+                de = fmaf(Cc[tp * LDM], ps[tp], de);
+            }
+        } else {
+            da = part[0][0][t - 1] + part[0][1][t - 1] + Rr[t * LDM + L - 1] * um[t - 1];
+            de = part[1][0][t - 1] + part[1][1][t - 1] + cf.cl[t] * usm[t - 1] + cf.bl[t] * uss[t - 1];
+        }
+        d_alpha[tok + t] = -da;
+        if (has_s) d_eta[tok + t] = de;
+    }
+}
+constexpr size_t kGatesBwdLds = 4 * MAT * sizeof(float);
+
+// dst[e] += sum over chains of st[chain][slot 0][e]
+__global__ void cw_accumulate_slot0_kernel(const float *__restrict__ st, float *__restrict__ dst, int batch,
+                                           size_t chain_stride) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= HD * HD) return;
+    float x = 0.f;
+    for (int b = 0; b < batch; b++) x += st[(size_t)b * chain_stride + e];
+    dst[e] += x;
+}
+
 constexpr size_t kOutFwdLds = 7 * MAT * sizeof(float);
 
 struct Scratch {
@@ -373,10 +745,11 @@ void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const 
     if (failed()) return;
     static bool attr_set = false;
     if (!attr_set) {
+        const size_t lds = kOutFwdLds;
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<float>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kOutFwdLds), "LDS size");
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "dynamic LDS size");
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<uint16_t>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kOutFwdLds), "LDS size");
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "dynamic LDS size");
         attr_set = true;
     }
     hipLaunchKernelGGL((cw_local_fwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), 0, stream(), k, v, alpha, theta,
@@ -388,6 +761,64 @@ void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const 
     hipLaunchKernelGGL((cw_out_fwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kOutFwdLds, stream(), k, v, q, alpha,
                        theta, eta, m_states, s_states, y, seq_len, chunk_size, nc, (int)has_s);
     check_launch("cw_out_fwd_kernel");
+}
+
+template <class K>
+void set_lds(K kernel, size_t bytes) {
+    check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)bytes), "dynamic LDS size");
+}
+
+template <class TIn>
+void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const float *alpha, const float *theta,
+                 const float *eta, const float *m_states, const float *s_states, const float *d_y, float *d_k,
+                 float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
+                 float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s) {
+    if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
+    const int nc = ceil_div(seq_len, chunk_size);
+    Scratch sc = local_scratch(batch, nc);
+    const size_t st_bytes = (size_t)batch * (nc + 1) * HD * HD * sizeof(float);
+    float *dm_states = scratch(5, st_bytes);
+    float *ds_states = scratch(6, st_bytes);
+    float *xs = scratch(7, (size_t)batch * nc * CW * CW * sizeof(float));
+    float *pvec = scratch(8, (size_t)batch * seq_len * 4 * sizeof(float));
+    float *scal = scratch(9, (size_t)batch * nc * 4 * sizeof(float));
+    if (failed()) return;
+    static bool attr_set = false;
+    if (!attr_set) {
+        set_lds(cw_local_bwd_kernel<float>, kLocalBwdLds);
+        set_lds(cw_local_bwd_kernel<uint16_t>, kLocalBwdLds);
+        set_lds(cw_grads_bwd_kernel<float>, kGradsBwdLds);
+        set_lds(cw_grads_bwd_kernel<uint16_t>, kGradsBwdLds);
+        set_lds(cw_gates_bwd_kernel, kGatesBwdLds);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kLocalBwdLds, stream(), k, q, d_y,
+                       alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc, (int)has_s);
+    check_launch("cw_local_bwd_kernel");
+    hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr, sc.loc,
+                       sc.locs, dm_states, ds_states, nc, (int)has_s);
+    check_launch("cw_scan_kernel");
+    hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(kThr), 0, stream(), m_states, s_states,
+                       dm_states, ds_states, scal, nc, (int)has_s);
+    check_launch("cw_state_dots_kernel");
+    {
+        KernelTimer kt("cw_grads_bwd_kernel");
+        hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kGradsBwdLds, stream(), k, v, q,
+                           d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta,
+                           pvec, xs, seq_len, chunk_size, nc, (int)has_s);
+        check_launch("cw_grads_bwd_kernel");
+    }
+    hipLaunchKernelGGL(cw_gates_bwd_kernel, dim3(batch * nc), dim3(kThr), kGatesBwdLds, stream(), alpha, theta, eta,
+                       pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size, nc, (int)has_s);
+    check_launch("cw_gates_bwd_kernel");
+    const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
+    hipLaunchKernelGGL(cw_accumulate_slot0_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), dm_states,
+                       d_m_initial, batch, chain_stride);
+    if (has_s && d_s_initial)
+        hipLaunchKernelGGL(cw_accumulate_slot0_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), ds_states,
+                           d_s_initial, batch, chain_stride);
+    check_launch("cw_accumulate_slot0_kernel");
 }
 
 }  // namespace
@@ -412,4 +843,28 @@ extern "C" void titans_chunkwise_forward_mm_f32_rocm(const float *k_mem, const f
                                                      int seq_len, int d, int batch_size, int chunk_size) {
     forward_mm<float>("titans_chunkwise_forward_mm_f32_rocm", k_mem, v_mem, q_mem, alpha, theta, eta, m_initial,
                       s_initial, m_chunk_states, s_chunk_states, y, seq_len, d, batch_size, chunk_size, true);
+}
+
+extern "C" void titans_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem,
+                                                    const uint16_t *q_mem, const float *alpha, const float *theta,
+                                                    const float *eta, const float *m_chunk_states,
+                                                    const float *s_chunk_states, const float *d_y, float *d_k_mem,
+                                                    float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta,
+                                                    float *d_eta, float *d_m_initial, float *d_s_initial,
+                                                    int seq_len, int d, int batch_size, int chunk_size) {
+    backward_mm<uint16_t>("titans_chunkwise_backward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
+                          m_chunk_states, s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
+                          d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, true);
+}
+
+extern "C" void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                                      const float *alpha, const float *theta, const float *eta,
+                                                      const float *m_chunk_states, const float *s_chunk_states,
+                                                      const float *d_y, float *d_k_mem, float *d_v_mem,
+                                                      float *d_q_mem, float *d_alpha, float *d_theta, float *d_eta,
+                                                      float *d_m_initial, float *d_s_initial, int seq_len, int d,
+                                                      int batch_size, int chunk_size) {
+    backward_mm<float>("titans_chunkwise_backward_mm_f32_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
+                       m_chunk_states, s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
+                       d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, true);
 }

@@ -75,3 +75,64 @@ def test_forward_matches_oracle(B, s, C, bf16):
     assert_close("y", host(got["y"]), want["y"], tol)
     assert_close("m_chunk_states", host(got["mc"]), want["mc"], tol)
     assert_close("s_chunk_states", host(got["sc"]), want["sc"], tol)
+
+
+@pytest.mark.parametrize("B,s,C", CASES)
+@pytest.mark.parametrize("bf16", [True, False])
+def test_backward_matches_oracle(B, s, C, bf16):
+    x = make(B, s, 64, seed=7 + B * 100 + s + C, bf16=bf16)
+    print(f"chunkwise_mm backward B={B} s={s} C={C} bf16={bf16}", flush=True)
+    _, want = oracle_chunkwise(x, C)
+    f = gpu_forward(x, C, bf16)
+    d = 64
+    g = dict(d_k=zeros(B, s, d), d_v=zeros(B, s, d), d_q=zeros(B, s, d), d_alpha=zeros(B, s),
+             d_theta=zeros(B, s), d_eta=zeros(B, s), d_m_initial=zeros(d, d), d_s_initial=zeros(d, d))
+    name = "titans_chunkwise_backward_bf16_rocm" if bf16 else "titans_chunkwise_backward_mm_f32_rocm"
+    D.call(name, f["k"], f["v"], f["q"], f["al"], f["th"], f["et"], f["mc"], f["sc"], dev(x["dy"]),
+           g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], g["d_m_initial"],
+           g["d_s_initial"], s, d, B, C)
+    torch.cuda.synchronize()
+    tol = 1e-3 if bf16 else 2e-4
+    for n in g:
+        assert_close(n, host(g[n]), want[n], tol)
+
+
+def test_initial_state_gradients_accumulate():
+    x = make(2, 64, 64, seed=3, bf16=False)
+    _, want = oracle_chunkwise(x, 32)
+    f = gpu_forward(x, 32, False)
+    B, s, d = 2, 64, 64
+    junk = [zeros(B, s, d) for _ in range(3)] + [zeros(B, s) for _ in range(3)]
+    dm, ds = torch.ones(d, d, device="cuda"), torch.ones(d, d, device="cuda")
+    D.call("titans_chunkwise_backward_mm_f32_rocm", f["k"], f["v"], f["q"], f["al"], f["th"], f["et"],
+           f["mc"], f["sc"], dev(x["dy"]), *junk, dm, ds, s, d, B, 32)
+    torch.cuda.synchronize()
+    assert_close("d_m_initial", host(dm) - 1.0, want["d_m_initial"], 2e-4)
+    assert_close("d_s_initial", host(ds) - 1.0, want["d_s_initial"], 2e-4)
+
+
+def test_matrix_form_agrees_with_sequential_kernels_at_benchmark_shape():
+    """B' = 16 chains of the config-3 shape (seq 4096, C = 64) are too long for the CPU
+    oracle; the sequential frozen-M0 kernels (parity-tested against it) are the yardstick."""
+    B, s, d, C = 16, 4096, 64, 64
+    x = make(B, s, d, seed=99, bf16=True, m0_scale=0.0)
+    f = gpu_forward(x, C, True)
+    k, v, q = (t.to(torch.float32) for t in (f["k"], f["v"], f["q"]))
+    nc = s // C
+    mc, sc, y = zeros(B, nc + 1, d, d), zeros(B, nc + 1, d, d), zeros(B, s, d)
+    F32_MAX = float(np.finfo(np.float32).max)
+    D.call("titans_chunkwise_forward_f32_cuda", k, v, q, f["al"], f["th"], f["et"], dev(x["m0"]),
+           dev(x["s0"]), mc, sc, y, s, d, B, C, 0.0, F32_MAX)
+    mk = lambda: dict(d_k=zeros(B, s, d), d_v=zeros(B, s, d), d_q=zeros(B, s, d), d_alpha=zeros(B, s),
+                      d_theta=zeros(B, s), d_eta=zeros(B, s), d_m_initial=zeros(d, d), d_s_initial=zeros(d, d))
+    g1, g2 = mk(), mk()
+    dy = dev(x["dy"])
+    D.call("titans_chunkwise_backward_f32_cuda", k, v, q, f["al"], f["th"], f["et"], mc, sc, dy,
+           *[g1[n] for n in g1], s, d, B, C, 0.0, F32_MAX)
+    D.call("titans_chunkwise_backward_bf16_rocm", f["k"], f["v"], f["q"], f["al"], f["th"], f["et"],
+           f["mc"], f["sc"], dy, *[g2[n] for n in g2], s, d, B, C)
+    torch.cuda.synchronize()
+    assert_close("y", host(f["y"]), host(y), 1e-3)
+    assert_close("m_chunk_states", host(f["mc"]), host(mc), 1e-3)
+    for n in g1:
+        assert_close(n, host(g2[n]), host(g1[n]), 1e-3)
