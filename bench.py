@@ -7,7 +7,10 @@ synthetic input that is already resident in HBM.  Prints ONE JSON line.
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 Workloads (BASELINE.json `configs`):
-  titans_exact_c2   configs[1] (default): Titans LMM exact recurrence, 8 heads x 64
+  titans_chunkwise_c3  configs[2] (default; the metric's d=512, L=4096): Titans LMM
+                    chunkwise training, chunk 64, 8 heads x 64, batch 16, seq 4096,
+                    bf16 k/v/q, fp32 accumulate and state; matrix-core kernels.
+  titans_exact_c2   configs[1]: Titans LMM exact recurrence, 8 heads x 64
                     (d=512), batch 8, seq 2048, fp32, state checkpoints every 64
                     tokens (checkpointed forward + fused checkpointed backward).
   hope_selfref_c4   configs[3]: HOPE self-referential memory, 8 heads x 64, batch 8,
@@ -87,6 +90,30 @@ def cpu_baseline(x, heads, budget_s=12.0):
                       f"full-trajectory forward + backward, {el:.1f} s"}
 
 
+# Chunkwise (matrix form), per head-token at d=64, C=64: compulsory HBM bytes forward 1164
+# (bf16 k,v,q, gates, fp32 y, chunk states), backward 1944; flops forward 57 344, backward ~143 k.
+BYTES_CW_FWD, BYTES_CW_BWD = 1164, 1944
+FLOP_CW_FWD, FLOP_CW_BWD = 57344, 143360
+
+
+def cpu_baseline_chunkwise(x, C, budget_s=12.0):
+    """Oracle of the frozen-M0 chunkwise rule, one thread, whole chains until the budget is used."""
+    from oracle import pyoracle as orc
+    B, s, d = x["k"].shape
+    npx = {n: t.float().numpy() for n, t in x.items()}
+    done = 0
+    t_start = time.perf_counter()
+    while done < B and time.perf_counter() - t_start < budget_s:
+        a = [npx[n][done] for n in ("k", "v", "q", "alpha", "theta", "eta")]
+        y, mc, sc = orc.chunkwise_forward(*a, npx["m0"][done], npx["s0"][done], C, True)
+        orc.chunkwise_backward(*a, mc, sc, npx["dy"][done], C, True)
+        done += 1
+    el = time.perf_counter() - t_start
+    return {"value": done * s / 8 / el, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{done} of {B} chains of {s} tokens (8 chains = one sequence of d=512), chunkwise "
+                      f"forward + backward, {el:.1f} s"}
+
+
 def cpu_baseline_hope(mems, x, dy, C, budget_s=12.0):
     """Same oracle, HOPE path: whole chains until the time budget is used."""
     from oracle import pyoracle as orc
@@ -136,6 +163,40 @@ def setup_titans_exact_c2(torch, D, lib):
         cpu=lambda: cpu_baseline(x, heads))
 
 
+def setup_titans_chunkwise_c3(torch, D, lib):
+    bs, heads, d, s, C = 16, 8, 64, 4096, 64
+    B = bs * heads
+    x = make_inputs(B, s, d, 0x5EED0003)
+    for n in ("k", "v", "q"):
+        x[n] = x[n].to(torch.bfloat16)
+    dv = {n: t.cuda() for n, t in x.items()}
+    nc = s // C
+    z = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device="cuda")
+    mc, sc, y = z(B, nc + 1, d, d), z(B, nc + 1, d, d), z(B, s, d)
+    g = dict(dk=z(B, s, d), dv=z(B, s, d), dq=z(B, s, d), da=z(B, s), dt=z(B, s), de=z(B, s),
+             dm=z(d, d), ds=z(d, d))
+
+    def fwd():
+        D.call("titans_chunkwise_forward_bf16_rocm", dv["k"], dv["v"], dv["q"], dv["alpha"], dv["theta"],
+               dv["eta"], dv["m0"], dv["s0"], mc, sc, y, s, d, B, C)
+
+    def bwd():
+        D.call("titans_chunkwise_backward_bf16_rocm", dv["k"], dv["v"], dv["q"], dv["alpha"], dv["theta"],
+               dv["eta"], mc, sc, dv["dy"], g["dk"], g["dv"], g["dq"], g["da"], g["dt"], g["de"],
+               g["dm"], g["ds"], s, d, B, C)
+
+    return dict(
+        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16",
+        flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_bwd=BYTES_CW_BWD,
+        traffic_bwd=None,
+        kernel="cw_grads_bwd_kernel<bf16> (the largest of the backward entry point's kernels)",
+        kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
+        config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
+                            "batch 16, seq 4096, bf16 k/v/q with fp32 accumulate and fp32 M/S, fwd+bwd",
+                "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "chunk_size": C},
+        cpu=lambda: cpu_baseline_chunkwise(x, C))
+
+
 def setup_hope_selfref_c4(torch, D, lib):
     from nl_hecate_amd import selfref as SR
     bs, heads, d, s, C = 8, 8, 64, 2048, 64
@@ -168,7 +229,8 @@ def setup_hope_selfref_c4(torch, D, lib):
         cpu=lambda: cpu_baseline_hope(mems, x, dy, C))
 
 
-WORKLOADS = {"titans_exact_c2": setup_titans_exact_c2, "hope_selfref_c4": setup_hope_selfref_c4}
+WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
+             "hope_selfref_c4": setup_hope_selfref_c4}
 
 
 def main():
@@ -176,7 +238,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="titans_exact_c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="titans_chunkwise_c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch a plain map kernel (256 MiB read, 256 MiB written) 5 times and exit: "
@@ -240,21 +302,27 @@ def main():
     assert n_launch.value == 10 and name.value.decode() in w["kernel"], (n_launch.value, name.value)
     head_tokens = w["head_tokens"]
     bwd_tflops = w["flop_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e12
+    bwd_gbs = w["bytes_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e9
+    hbm_bound = w.get("bound") == "hbm"
     roofline = {"kernel": w["kernel"],
-                "bound": "mfma", "achieved": bwd_tflops, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                "frac": bwd_tflops / PEAK_FP32_TFLOPS, "traffic": w["traffic_bwd"],
+                "bound": "hbm" if hbm_bound else "mfma",
+                "achieved": bwd_gbs if hbm_bound else bwd_tflops,
+                "peak": PEAK_HBM_GBS if hbm_bound else PEAK_FP32_TFLOPS,
+                "unit": "GB/s" if hbm_bound else "TFLOP/s",
+                "frac": bwd_gbs / PEAK_HBM_GBS if hbm_bound else bwd_tflops / PEAK_FP32_TFLOPS,
+                "traffic": w["traffic_bwd"],
                 "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel; "
                                 "see profiles/" + args.workload + "_kernels_and_hbm_traffic.txt)",
                 "algorithmic_bytes": w["bytes_bwd"] * head_tokens,
-                "note": "fp32 vector/matrix peak (157.3 TFLOP/s); rank-1 and mat-vec work, not a contraction",
                 "avg_launch_ms": kern_ms, "entry_point_ms": bwd_ms,
-                "hbm": {"achieved": w["bytes_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                        "unit": "GB/s"}}
+                "hbm": {"achieved": bwd_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s"},
+                "fp32_matrix": {"achieved": bwd_tflops, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                                "frac": bwd_tflops / PEAK_FP32_TFLOPS}}
     out = {
         "metric": METRIC, "value": value, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": w.get("dtype", "f32"), "data": "synthetic",
         "config": w["config"],
         "event_ms_per_step": ev_ms / args.steps,
         "kernels_ms": {w["kernel_names"]["forward"]: fwd_ms, w["kernel_names"]["backward"]: bwd_ms},

@@ -46,35 +46,68 @@ constexpr int kThr = 256;       // 4 waves, one 32x32 output tile each
 __device__ __forceinline__ float to_f32(float x) { return x; }
 __device__ __forceinline__ float to_f32(uint16_t u) { return __uint_as_float((uint32_t)u << 16); }
 
-// Stage a row-major [nrows <= 64][64] global tile into LDS; rows >= nrows are zero.
+// Staging of a row-major [nrows <= 64][64] global tile into LDS in two halves, so that the
+// loads of every tile of a phase are in flight together: fetch() issues the global loads
+// into registers (rows >= nrows read as zero), commit() converts and stores to LDS.
+template <class T> struct Tile;
+template <> struct Tile<float> { float4 x[4]; };
+template <> struct Tile<uint16_t> { uint2 x[4]; };
+
+template <class T>
+__device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows) {
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
+        if constexpr (sizeof(T) == 4)
+            r.x[it] = rr < nrows ? *reinterpret_cast<const float4 *>(src + rr * 64 + cc) : make_float4(0, 0, 0, 0);
+        else
+            r.x[it] = rr < nrows ? *reinterpret_cast<const uint2 *>(src + rr * 64 + cc) : make_uint2(0, 0);
+    }
+}
+template <class T>
+__device__ __forceinline__ void commit(float *dst, const Tile<T> &r) {
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
+        float *p = dst + rr * LDM + cc;
+        if constexpr (sizeof(T) == 4) {
+            p[0] = r.x[it].x; p[1] = r.x[it].y; p[2] = r.x[it].z; p[3] = r.x[it].w;
+        } else {
+            p[0] = __uint_as_float(r.x[it].x << 16); p[1] = __uint_as_float(r.x[it].x & 0xffff0000u);
+            p[2] = __uint_as_float(r.x[it].y << 16); p[3] = __uint_as_float(r.x[it].y & 0xffff0000u);
+        }
+    }
+}
 template <class T>
 __device__ __forceinline__ void stage(float *dst, const T *src, int nrows) {
-    for (int e = threadIdx.x * 4; e < 64 * 64; e += kThr * 4) {
-        const int rr = e >> 6, cc = e & 63;
-        float x0 = 0.f, x1 = 0.f, x2 = 0.f, x3 = 0.f;
-        if (rr < nrows) {
-            if constexpr (sizeof(T) == 4) {
-                const float4 t = *reinterpret_cast<const float4 *>(src + rr * 64 + cc);
-                x0 = t.x; x1 = t.y; x2 = t.z; x3 = t.w;
-            } else {
-                const uint2 t = *reinterpret_cast<const uint2 *>(src + rr * 64 + cc);
-                x0 = __uint_as_float(t.x << 16); x1 = __uint_as_float(t.x & 0xffff0000u);
-                x2 = __uint_as_float(t.y << 16); x3 = __uint_as_float(t.y & 0xffff0000u);
-            }
-        }
-        float *p = dst + rr * LDM + cc;
-        p[0] = x0; p[1] = x1; p[2] = x2; p[3] = x3;
-    }
+    Tile<T> r;
+    fetch(r, src, nrows);
+    commit(dst, r);
 }
 
 // One wave: acc (32x32) += sum_k a(m,k) b(k,n), m,n in [0,32), k in [0,K).
 // Operand layout of v_mfma_f32_32x32x2_f32: lane l supplies A[l%32][l/32] and B[l/32][l%32].
+// K = 64: four groups of 8 instructions; the operands of group g+1 are read from LDS while
+// group g runs on the matrix core.
 template <class FA, class FB>
-__device__ __forceinline__ void mma32(f32x16 &acc, int K, FA a, FB b) {
+__device__ __forceinline__ void mma32(f32x16 &acc, int /*K*/, FA a, FB b) {
     const int l = threadIdx.x & 63, mn = l & 31, hf = l >> 5;
-#pragma unroll 8
-    for (int k = 0; k < K; k += 2)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a(mn, k + hf), b(k + hf, mn), acc, 0, 0, 0);
+    float av[2][8], bv[2][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) { av[0][i] = a(mn, 2 * i + hf); bv[0][i] = b(2 * i + hf, mn); }
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        if (g < 3) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                av[(g + 1) & 1][i] = a(mn, 16 * (g + 1) + 2 * i + hf);
+                bv[(g + 1) & 1][i] = b(16 * (g + 1) + 2 * i + hf, mn);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[g & 1][i], bv[g & 1][i], acc, 0, 0, 0);
+    }
 }
 // Accumulator element i of lane l is C[8*(i/4) + 4*(l/32) + i%4][l%32].
 __device__ __forceinline__ int c_row(int i) { return 8 * (i >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (i & 3); }
@@ -103,20 +136,30 @@ __device__ __forceinline__ void load_gates(Coef &cf, const float *alpha, const f
     }
 }
 
-// Column j of r, bb, c (thread j), optionally stored: Cc[t][j], Bb[j][t], Rr[j][t]
-// (stride LDM; entries outside j <= t < L are zero), plus the vectors.
-// Call after load_gates + barrier; needs a barrier afterwards.
-__device__ __forceinline__ void coefficients(Coef &cf, int L, float *Cc, float *Bb, float *Rr) {
-    const int j = threadIdx.x;
-    if (j < CW) {
+__device__ __forceinline__ float lane_bcast(float x, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+
+// Column j of r, bb, c (thread j of wave 0), optionally stored: Cc[t][j], Bb[j][t], Rr[j][t]
+// (stride LDM; entries outside j <= t < L are zero), plus the vectors (wave 1).  The gates
+// are read from global memory into one register per lane and broadcast per step, so the
+// sequential loops carry no memory latency.  Needs a barrier afterwards.
+__device__ __forceinline__ void coefficients(Coef &cf, const float *alpha, const float *eta, int L, bool has_s,
+                                             float *Cc, float *Bb, float *Rr) {
+    const int j = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (w >= 2) return;
+    const float keep_j = j < L ? 1.f - alpha[j] : 1.f;
+    const float eta_j = (j < L && has_s) ? eta[j] : 0.f;
+    if (w == 0) {
         float rr = 1.f, b = 1.f, cc = 1.f;
+#pragma unroll 8
         for (int t = 0; t < CW; t++) {
+            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
             float vr = 0.f, vb = 0.f, vc = 0.f;
             if (t >= j && t < L && j < L) {
                 if (t > j) {
-                    const float keep = 1.f - cf.al[t];
                     rr *= keep;
-                    b *= cf.et[t];
+                    b *= et;
                     cc = keep * cc + b;
                 }
                 vr = rr; vb = b; vc = cc;
@@ -127,19 +170,20 @@ __device__ __forceinline__ void coefficients(Coef &cf, int L, float *Cc, float *
         }
         cf.cl[j] = j < L ? cc : 0.f;
         cf.bl[j] = j < L ? b : 0.f;
-    } else if (j == CW) {
-        float a = 1.f, h = 1.f, beta = 0.f;
+    } else {
+        // a_t, beta_t, h_t: every lane runs the same scalar recurrence, lane t keeps step t
+        float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f, kh = 0.f;
+#pragma unroll 8
         for (int t = 0; t < CW; t++) {
-            if (t < L) {
-                const float keep = 1.f - cf.al[t];
-                a *= keep;
-                h *= cf.et[t];
-                beta = keep * beta + h;
-            }
-            cf.a[t] = t < L ? a : 0.f;
-            cf.beta[t] = t < L ? beta : 0.f;
-            cf.h[t] = t < L ? h : 0.f;
+            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
+            a *= keep;
+            h *= et;
+            beta = keep * beta + h;
+            if (t == j) { ka = a; kb = beta; kh = h; }
         }
+        cf.a[j] = j < L ? ka : 0.f;
+        cf.beta[j] = j < L ? kb : 0.f;
+        cf.h[j] = j < L ? kh : 0.f;
     }
 }
 
@@ -162,11 +206,15 @@ __global__ __launch_bounds__(kThr) void cw_local_fwd_kernel(const TIn *__restric
     __shared__ float wM[CW], wS[CW];
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
-    stage(Ks, k + tok * HD, L);
-    stage(Vs, v + tok * HD, L);
-    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-    __syncthreads();
-    coefficients(cf, L, nullptr, nullptr, nullptr);
+    {
+        Tile<TIn> tk, tv;
+        fetch(tk, k + tok * HD, L);
+        fetch(tv, v + tok * HD, L);
+        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, nullptr, nullptr, nullptr);
+        commit(Ks, tk);
+        commit(Vs, tv);
+    }
     __syncthreads();
     if (threadIdx.x < CW) {
         wM[threadIdx.x] = -cf.th[threadIdx.x] * cf.cl[threadIdx.x];
@@ -225,28 +273,42 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
         s1p[slot * HD * HD + (r0 + rr) * HD + cc] = x1;
         if (s2p) s2p[slot * HD * HD + (r0 + rr) * HD + cc] = x2;
     }
-    for (int step = 0; step < nc; step++) {
+    // Operands of step+1 (two 64x64 matrices, this wave's tile of the additive term, the two
+    // scalars) are fetched into registers while step runs, so a step costs no HBM round trip.
+    Tile<float> ta, tb;
+    float cnext[16], s1n = 0.f, s2n = 0.f;
+    auto prefetch = [&](int step) {
         const int ci = FWD ? step : nc - 1 - step;
         const float *lc = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
         const float *sc = locs + ((size_t)chain * nc + ci) * 4;
+        fetch(ta, lc, 64);
+        fetch(tb, lc + HD * HD, 64);
+        s1n = sc[1]; s2n = sc[2];
+        const float *Cm = lc + (FWD ? 2 + which : (which ? 3 : 2)) * HD * HD;
+#pragma unroll
+        for (int i = 0; i < 16; i++) cnext[i] = Cm[(r0 + c_row(i)) * HD + n0 + c_col()];
+    };
+    prefetch(0);
+    float cadd[16], s1, s2;
+    for (int step = 0; step < nc; step++) {
+        const int ci = FWD ? step : nc - 1 - step;
         __syncthreads();  // previous step's readers of Ta/Tb and writers of X1/X2 are done
-        stage(Ta, lc, 64);
-        stage(Tb, lc + HD * HD, 64);
-        const float s1 = sc[1], s2 = sc[2];
+        commit(Ta, ta);
+        commit(Tb, tb);
+        s1 = s1n; s2 = s2n;
+#pragma unroll
+        for (int i = 0; i < 16; i++) cadd[i] = cnext[i];
         __syncthreads();
+        if (step + 1 < nc) prefetch(step + 1);
         f32x16 acc = zero16();
         float out[16];
         if (FWD) {
             const float *T = which ? Tb : Ta;
             mma32(acc, 64, [&](int m, int kk) { return X1[m * LDM + kk]; },
                   [&](int kk, int n) { return T[kk * LDM + n0 + n]; });
-            const float *Cm = lc + (2 + which) * HD * HD;
             const float sx = which ? s2 : s1;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int row = c_row(i), col = n0 + c_col();
-                out[i] = acc[i] + sx * X2[row * LDM + col] + Cm[(r0 + row) * HD + col];
-            }
+            for (int i = 0; i < 16; i++) out[i] = acc[i] + sx * X2[c_row(i) * LDM + n0 + c_col()] + cadd[i];
         } else {
             const float *Xs = which ? X2 : X1;
             const float *T = which ? Tb : Ta;
@@ -254,23 +316,17 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
                   [&](int kk, int n) { return T[kk * LDM + n0 + n]; });
             if (which) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) part[w & 1][c_row(i) * 33 + c_col()] = acc[i];
-                const float *Cm = lc + 3 * HD * HD;
-#pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int row = c_row(i), col = n0 + c_col();
-                    out[i] = s1 * X1[row * LDM + col] + s2 * X2[row * LDM + col] + Cm[(r0 + row) * HD + col];
+                    part[w & 1][row * 33 + c_col()] = acc[i];
+                    out[i] = s1 * X1[row * LDM + col] + s2 * X2[row * LDM + col] + cadd[i];
                 }
             }
         }
         __syncthreads();  // all reads of the old X1/X2 are done; partial products are in LDS
         if (!FWD && !which) {
-            const float *Cm = lc + 2 * HD * HD;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int row = c_row(i), col = n0 + c_col();
-                out[i] = acc[i] + part[w & 1][row * 33 + c_col()] + Cm[(r0 + row) * HD + col];
-            }
+            for (int i = 0; i < 16; i++) out[i] = acc[i] + part[w & 1][c_row(i) * 33 + c_col()] + cadd[i];
         }
         float *Xd = which ? X2 : X1;
         float *gd = which ? s2p : s1p;
@@ -299,14 +355,22 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
     __shared__ Coef cf;
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
-    stage(Ks, k + tok * HD, L);
-    stage(Qs, q + tok * HD, L);
-    stage(Es, v + tok * HD, L);
-    stage(Ms, m_states + ((size_t)chain * (nc + 1) + ci) * HD * HD, 64);
-    if (has_s) stage(Ss, s_states + ((size_t)chain * (nc + 1) + ci) * HD * HD, 64);
-    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-    __syncthreads();
-    coefficients(cf, L, Cc, nullptr, nullptr);
+    {
+        Tile<TIn> tk, tq, tv;
+        Tile<float> tm, ts;
+        fetch(tk, k + tok * HD, L);
+        fetch(tq, q + tok * HD, L);
+        fetch(tv, v + tok * HD, L);
+        fetch(tm, m_states + ((size_t)chain * (nc + 1) + ci) * HD * HD, 64);
+        if (has_s) fetch(ts, s_states + ((size_t)chain * (nc + 1) + ci) * HD * HD, 64);
+        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, nullptr, nullptr);
+        commit(Ks, tk);
+        commit(Qs, tq);
+        commit(Es, tv);
+        commit(Ms, tm);
+        if (has_s) commit(Ss, ts);
+    }
     __syncthreads();
     const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1);
     {
@@ -359,12 +423,18 @@ __global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restric
     __shared__ float wM[CW], wS[CW];
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
-    stage(Ks, k + tok * HD, L);
-    stage(Qs, q + tok * HD, L);
-    stage(Ds, d_y + tok * HD, L);
-    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-    __syncthreads();
-    coefficients(cf, L, Cc, nullptr, nullptr);
+    {
+        Tile<TIn> tk, tq;
+        Tile<float> td;
+        fetch(tk, k + tok * HD, L);
+        fetch(tq, q + tok * HD, L);
+        fetch(td, d_y + tok * HD, L);
+        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, nullptr, nullptr);
+        commit(Ks, tk);
+        commit(Qs, tq);
+        commit(Ds, td);
+    }
     __syncthreads();
     if (threadIdx.x < CW) {
         wM[threadIdx.x] = -cf.th[threadIdx.x] * cf.cl[threadIdx.x];
@@ -481,15 +551,24 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     const size_t tok = (size_t)chain * s + t0;
     const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, st1 = st0 + HD * HD;
     float *Ss = B5, *Cc = B6;
-    stage(Ks, k + tok * HD, L);
-    stage(Qs, q + tok * HD, L);
-    stage(Ds, d_y + tok * HD, L);
-    stage(Es, v + tok * HD, L);
-    stage(Ms, m_states + st0, 64);
-    if (has_s) stage(Ss, s_states + st0, 64);
-    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-    __syncthreads();
-    coefficients(cf, L, Cc, nullptr, nullptr);
+    {
+        Tile<TIn> tk, tq, tv;
+        Tile<float> td, tm, ts;
+        fetch(tk, k + tok * HD, L);
+        fetch(tq, q + tok * HD, L);
+        fetch(tv, v + tok * HD, L);
+        fetch(td, d_y + tok * HD, L);
+        fetch(tm, m_states + st0, 64);
+        if (has_s) fetch(ts, s_states + st0, 64);
+        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, nullptr, nullptr);
+        commit(Ks, tk);
+        commit(Qs, tq);
+        commit(Es, tv);
+        commit(Ds, td);
+        commit(Ms, tm);
+        if (has_s) commit(Ss, ts);
+    }
     __syncthreads();
     const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1;
     const bool writer = (threadIdx.x & 31) == 0;
@@ -521,6 +600,9 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
         }
     }
     __syncthreads();   // E complete; S0 no longer needed
+    Tile<float> tdm, tds;   // adjoint states: in flight during the next two phases
+    fetch(tdm, dm_states + st1, 64);
+    if (has_s) fetch(tds, ds_states + st1, 64);
     float *CP = B5, *CR = B7;
     {
         f32x16 r = zero16();
@@ -545,8 +627,8 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
         if (row < L) d_q[(tok + row) * HD + col] = dq[i];
     }
     float *dMs = B6, *dSs = B8;
-    stage(dMs, dm_states + st1, 64);
-    if (has_s) stage(dSs, ds_states + st1, 64);
+    commit(dMs, tdm);
+    if (has_s) commit(dSs, tds);
     __syncthreads();
     {
         // Dk[j][i] = sum_t CP[t][j] dY[t][i] + cl_j (K dMo^T)[j][i] + bl_j (K dSo^T)[j][i]
@@ -638,7 +720,8 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     __shared__ float part[2][2][CW];
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
-    stage(Xs, xs + ((size_t)chain * nc + ci) * CW * CW, 64);
+    Tile<float> tx;
+    fetch(tx, xs + ((size_t)chain * nc + ci) * CW * CW, 64);
     load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
     if (threadIdx.x < CW) {
         const int t = threadIdx.x;
@@ -647,8 +730,8 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     }
     const float m0dm = scal[((size_t)chain * nc + ci) * 4 + 0], s0dm = scal[((size_t)chain * nc + ci) * 4 + 1],
                 s0ds = scal[((size_t)chain * nc + ci) * 4 + 2];
-    __syncthreads();
-    coefficients(cf, L, Cc, Bb, Rr);
+    coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, Bb, Rr);
+    commit(Xs, tx);
     __syncthreads();
     if (threadIdx.x < CW) {   // mat-vecs with W and Ws
         const int tau = threadIdx.x;
