@@ -1,5 +1,5 @@
 // Frozen-M0 chunkwise Titans / Delta rule in matrix form on the fp32 matrix
-// cores (v_mfma_f32_32x32x2_f32), head size 64, chunks of up to 64 tokens.
+// cores (v_mfma_f32_16x16x4_f32), head size 64, chunks of up to 64 tokens.
 //
 // Semantics are those of core/kernels/titans_chunkwise_forward.cu and
 // titans_chunkwise_backward.cu (errors of a chunk taken against the chunk-start
@@ -35,13 +35,13 @@
 namespace nlh {
 namespace {
 
-using f32x16 = __attribute__((ext_vector_type(16))) float;
+using f32x4 = __attribute__((ext_vector_type(4))) float;
 
 constexpr int CW = 64;          // tokens per chunk tile
 constexpr int HD = 64;          // head size
 constexpr int LDM = 65;         // LDS row stride in floats (odd: conflict-free rows and columns)
 constexpr int MAT = 64 * LDM;   // floats per 64x64 LDS matrix
-constexpr int kThr = 256;       // 4 waves, one 32x32 output tile each
+constexpr int kThr = 512;       // 8 waves (two per SIMD), one 16x32 output strip each
 
 __device__ __forceinline__ float to_f32(float x) { return x; }
 __device__ __forceinline__ float to_f32(uint16_t u) { return __uint_as_float((uint32_t)u << 16); }
@@ -50,13 +50,13 @@ __device__ __forceinline__ float to_f32(uint16_t u) { return __uint_as_float((ui
 // loads of every tile of a phase are in flight together: fetch() issues the global loads
 // into registers (rows >= nrows read as zero), commit() converts and stores to LDS.
 template <class T> struct Tile;
-template <> struct Tile<float> { float4 x[4]; };
-template <> struct Tile<uint16_t> { uint2 x[4]; };
+template <> struct Tile<float> { float4 x[2]; };
+template <> struct Tile<uint16_t> { uint2 x[2]; };
 
 template <class T>
 __device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows) {
 #pragma unroll
-    for (int it = 0; it < 4; it++) {
+    for (int it = 0; it < 2; it++) {
         const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
         if constexpr (sizeof(T) == 4)
             r.x[it] = rr < nrows ? *reinterpret_cast<const float4 *>(src + rr * 64 + cc) : make_float4(0, 0, 0, 0);
@@ -67,7 +67,7 @@ __device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows) {
 template <class T>
 __device__ __forceinline__ void commit(float *dst, const Tile<T> &r) {
 #pragma unroll
-    for (int it = 0; it < 4; it++) {
+    for (int it = 0; it < 2; it++) {
         const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
         float *p = dst + rr * LDM + cc;
         if constexpr (sizeof(T) == 4) {
@@ -85,39 +85,63 @@ __device__ __forceinline__ void stage(float *dst, const T *src, int nrows) {
     commit(dst, r);
 }
 
-// One wave: acc (32x32) += sum_k a(m,k) b(k,n), m,n in [0,32), k in [0,K).
-// Operand layout of v_mfma_f32_32x32x2_f32: lane l supplies A[l%32][l/32] and B[l/32][l%32].
-// K = 64: four groups of 8 instructions; the operands of group g+1 are read from LDS while
-// group g runs on the matrix core.
-template <class FA, class FB>
-__device__ __forceinline__ void mma32(f32x16 &acc, int /*K*/, FA a, FB b) {
-    const int l = threadIdx.x & 63, mn = l & 31, hf = l >> 5;
-    float av[2][8], bv[2][8];
+// Output strip of one wave: 16 rows x 32 columns = two 16x16 accumulator tiles side by side.
+// With 8 waves a 64x64 product is 8 strips; two waves share a SIMD, so one wave's LDS reads,
+// epilogue arithmetic and stores overlap the other's matrix-core work.
+struct Strip { f32x4 t[2]; };
+__device__ __forceinline__ Strip zero_strip() {
+    Strip z;
 #pragma unroll
-    for (int i = 0; i < 8; i++) { av[0][i] = a(mn, 2 * i + hf); bv[0][i] = b(2 * i + hf, mn); }
+    for (int i = 0; i < 4; i++) { z.t[0][i] = 0.f; z.t[1][i] = 0.f; }
+    return z;
+}
+// acc += sum_{k<64} a(m,k) b(k,n), m in [0,16), n in [0,32).
+// Operand layout of v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][l/16] and B[l/16][l%16].
+// Sixteen k-steps in four groups; the operands of group g+1 are read while group g runs.
+template <class FA, class FB>
+__device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
+    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4;
+    float av[2][4], b0[2][4], b1[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { av[0][i] = a(r, 4 * i + kq); b0[0][i] = b(4 * i + kq, r); b1[0][i] = b(4 * i + kq, 16 + r); }
 #pragma unroll
     for (int g = 0; g < 4; g++) {
         if (g < 3) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                av[(g + 1) & 1][i] = a(mn, 16 * (g + 1) + 2 * i + hf);
-                bv[(g + 1) & 1][i] = b(16 * (g + 1) + 2 * i + hf, mn);
+            for (int i = 0; i < 4; i++) {
+                const int kk = 16 * (g + 1) + 4 * i + kq;
+                av[(g + 1) & 1][i] = a(r, kk); b0[(g + 1) & 1][i] = b(kk, r); b1[(g + 1) & 1][i] = b(kk, 16 + r);
             }
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[g & 1][i], bv[g & 1][i], acc, 0, 0, 0);
+        for (int i = 0; i < 4; i++) {
+            acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g & 1][i], b0[g & 1][i], acc.t[0], 0, 0, 0);
+            acc.t[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g & 1][i], b1[g & 1][i], acc.t[1], 0, 0, 0);
+        }
     }
 }
-// Accumulator element i of lane l is C[8*(i/4) + 4*(l/32) + i%4][l%32].
-__device__ __forceinline__ int c_row(int i) { return 8 * (i >> 2) + 4 * ((threadIdx.x & 63) >> 5) + (i & 3); }
-__device__ __forceinline__ int c_col() { return threadIdx.x & 31; }
-__device__ __forceinline__ f32x16 zero16() {
-    f32x16 z;
+// Element i of tile tl of lane l is C[4*(l/16) + i][16*tl + l%16] of the strip.
+template <class F>
+__device__ __forceinline__ void for_c(Strip &acc, F f) {
+    const int l = threadIdx.x & 63;
 #pragma unroll
-    for (int i = 0; i < 16; i++) z[i] = 0.f;
-    return z;
+    for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float x = acc.t[tl][i];
+            f(4 * (l >> 4) + i, 16 * tl + (l & 15), x);
+            acc.t[tl][i] = x;
+        }
 }
+// Row sums of a strip: afterwards t[0][i] of every lane holds the sum over the 32 columns of
+// strip row 4*(l/16) + i.
+__device__ __forceinline__ void strip_row_sums(Strip &x) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) x.t[0][i] = group_allreduce<16>(x.t[0][i] + 0.f) + group_allreduce<16>(x.t[1][i] + 0.f);
+}
+// lanes that publish the row sums (one per 16-lane group), and the strip rows they hold
+__device__ __forceinline__ bool row_writer() { return (threadIdx.x & 15) == 0; }
+__device__ __forceinline__ int row_of(int i) { return 4 * ((threadIdx.x & 63) >> 4) + i; }
 
 // Gate coefficients of one chunk (L <= 64 tokens), all in LDS.
 struct Coef {
@@ -194,6 +218,10 @@ constexpr size_t kLocMats = 4;
 // ── pass 1 (forward) / shared with the backward: chunk-local matrices ───────
 // T_a = a_L I + K^T diag(wM) K,  T_b = K^T diag(wS) K  (both symmetric);
 // forward also C_1 = -(V.wM)^T K, C_2 = -(V.wS)^T K.
+#define NLH_STRIP_ORIGIN() \
+    const int w = threadIdx.x >> 6, m0 = 16 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1; \
+    (void)nh
+
 template <class TIn>
 __global__ __launch_bounds__(kThr) void cw_local_fwd_kernel(const TIn *__restrict__ k, const TIn *__restrict__ v,
                                                             const float *__restrict__ alpha,
@@ -226,22 +254,21 @@ __global__ __launch_bounds__(kThr) void cw_local_fwd_kernel(const TIn *__restric
         sc[0] = aL; sc[1] = betaL; sc[2] = hL; sc[3] = 0.f;
     }
     __syncthreads();
-    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1);
+    NLH_STRIP_ORIGIN();
     float *out = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
     auto bK = [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; };
 #pragma unroll 1
     for (int o = 0; o < 4; o++) {
         const float *Am = o < 2 ? Ks : Vs;
         const float *wv = (o & 1) ? wS : wM;
-        f32x16 acc = zero16();
-        mma32(acc, 64, [&](int m, int kk) { return Am[kk * LDM + m0 + m] * wv[kk]; }, bK);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            float x = o < 2 ? acc[i] : -acc[i];
-            if (o == 0 && row == col) x += aL;
-            out[(size_t)o * HD * HD + row * HD + col] = x;
-        }
+        Strip acc = zero_strip();
+        mma(acc, [&](int m, int kk) { return Am[kk * LDM + m0 + m] * wv[kk]; }, bK);
+        for_c(acc, [&](int r, int c, float &x) {
+            const int row = m0 + r, col = n0 + c;
+            float y = o < 2 ? x : -x;
+            if (o == 0 && row == col) y += aL;
+            out[(size_t)o * HD * HD + row * HD + col] = y;
+        });
     }
 }
 
@@ -250,17 +277,17 @@ __global__ __launch_bounds__(kThr) void cw_local_fwd_kernel(const TIn *__restric
 //       states[chain][c+1] = f(states[chain][c]), slot 0 = initial state
 // BWD:  X1' = X1 T_a + X2 T_b + C_1, X2' = s1 X1 + s2 X2 + C_2
 //       states[chain][c] = g(states[chain][c+1]), slot nc = 0
+// Eight strips per step: (product 0/1) x (16-row half) x (32-column half).
 template <bool FWD>
 __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__ init1,
                                                        const float *__restrict__ init2,
                                                        const float *__restrict__ loc,
                                                        const float *__restrict__ locs, float *__restrict__ st1,
                                                        float *__restrict__ st2, int nc, int has_s) {
-    __shared__ float X1[32 * LDM], X2[32 * LDM], Ta[MAT], Tb[MAT], part[2][32 * 33];
+    __shared__ float X1[32 * LDM], X2[32 * LDM], Ta[MAT], Tb[MAT], part[4][16 * 33];
     const int chain = blockIdx.x >> 1, r0 = 32 * (blockIdx.x & 1);
-    const int w = threadIdx.x >> 6, n0 = 32 * (w & 1), which = w >> 1;
+    const int w = threadIdx.x >> 6, which = w >> 2, m0 = 16 * ((w >> 1) & 1), n0 = 32 * (w & 1), pidx = w & 3;
     float *s1p = st1 + (size_t)chain * (nc + 1) * HD * HD, *s2p = st2 ? st2 + (size_t)chain * (nc + 1) * HD * HD : nullptr;
-    // initial state of this row block
     for (int e = threadIdx.x; e < 32 * 64; e += kThr) {
         const int rr = e >> 6, cc = e & 63;
         float x1 = 0.f, x2 = 0.f;
@@ -273,10 +300,11 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
         s1p[slot * HD * HD + (r0 + rr) * HD + cc] = x1;
         if (s2p) s2p[slot * HD * HD + (r0 + rr) * HD + cc] = x2;
     }
-    // Operands of step+1 (two 64x64 matrices, this wave's tile of the additive term, the two
+    // Operands of step+1 (two 64x64 matrices, this wave's strip of the additive term, the two
     // scalars) are fetched into registers while step runs, so a step costs no HBM round trip.
     Tile<float> ta, tb;
-    float cnext[16], s1n = 0.f, s2n = 0.f;
+    Strip cnext = zero_strip(), cadd;
+    float s1n = 0.f, s2n = 0.f, s1, s2;
     auto prefetch = [&](int step) {
         const int ci = FWD ? step : nc - 1 - step;
         const float *lc = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
@@ -285,58 +313,48 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
         fetch(tb, lc + HD * HD, 64);
         s1n = sc[1]; s2n = sc[2];
         const float *Cm = lc + (FWD ? 2 + which : (which ? 3 : 2)) * HD * HD;
-#pragma unroll
-        for (int i = 0; i < 16; i++) cnext[i] = Cm[(r0 + c_row(i)) * HD + n0 + c_col()];
+        for_c(cnext, [&](int r, int c, float &x) { x = Cm[(r0 + m0 + r) * HD + n0 + c]; });
     };
     prefetch(0);
-    float cadd[16], s1, s2;
     for (int step = 0; step < nc; step++) {
         const int ci = FWD ? step : nc - 1 - step;
         __syncthreads();  // previous step's readers of Ta/Tb and writers of X1/X2 are done
         commit(Ta, ta);
         commit(Tb, tb);
-        s1 = s1n; s2 = s2n;
-#pragma unroll
-        for (int i = 0; i < 16; i++) cadd[i] = cnext[i];
+        s1 = s1n; s2 = s2n; cadd = cnext;
         __syncthreads();
         if (step + 1 < nc) prefetch(step + 1);
-        f32x16 acc = zero16();
-        float out[16];
+        Strip acc = zero_strip(), out = zero_strip();
+        const float *T = which ? Tb : Ta;
+        const float *Xs = (FWD || !which) ? X1 : X2;
+        mma(acc, [&](int m, int kk) { return Xs[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return T[kk * LDM + n0 + n]; });
         if (FWD) {
-            const float *T = which ? Tb : Ta;
-            mma32(acc, 64, [&](int m, int kk) { return X1[m * LDM + kk]; },
-                  [&](int kk, int n) { return T[kk * LDM + n0 + n]; });
             const float sx = which ? s2 : s1;
+            for_c(out, [&](int r, int c, float &x) { x = sx * X2[(m0 + r) * LDM + n0 + c]; });
 #pragma unroll
-            for (int i = 0; i < 16; i++) out[i] = acc[i] + sx * X2[c_row(i) * LDM + n0 + c_col()] + cadd[i];
-        } else {
-            const float *Xs = which ? X2 : X1;
-            const float *T = which ? Tb : Ta;
-            mma32(acc, 64, [&](int m, int kk) { return Xs[m * LDM + kk]; },
-                  [&](int kk, int n) { return T[kk * LDM + n0 + n]; });
-            if (which) {
+            for (int i = 0; i < 4; i++) { out.t[0][i] += acc.t[0][i] + cadd.t[0][i]; out.t[1][i] += acc.t[1][i] + cadd.t[1][i]; }
+        } else if (which) {
+            for_c(acc, [&](int r, int c, float &x) { part[pidx][r * 33 + c] = x; });
+            for_c(out, [&](int r, int c, float &x) {
+                x = s1 * X1[(m0 + r) * LDM + n0 + c] + s2 * X2[(m0 + r) * LDM + n0 + c];
+            });
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int row = c_row(i), col = n0 + c_col();
-                    part[w & 1][row * 33 + c_col()] = acc[i];
-                    out[i] = s1 * X1[row * LDM + col] + s2 * X2[row * LDM + col] + cadd[i];
-                }
-            }
+            for (int i = 0; i < 4; i++) { out.t[0][i] += cadd.t[0][i]; out.t[1][i] += cadd.t[1][i]; }
         }
         __syncthreads();  // all reads of the old X1/X2 are done; partial products are in LDS
         if (!FWD && !which) {
+            for_c(out, [&](int r, int c, float &x) { x = part[pidx][r * 33 + c]; });
 #pragma unroll
-            for (int i = 0; i < 16; i++) out[i] = acc[i] + part[w & 1][c_row(i) * 33 + c_col()] + cadd[i];
+            for (int i = 0; i < 4; i++) { out.t[0][i] += acc.t[0][i] + cadd.t[0][i]; out.t[1][i] += acc.t[1][i] + cadd.t[1][i]; }
         }
         float *Xd = which ? X2 : X1;
         float *gd = which ? s2p : s1p;
         const size_t slot = FWD ? ci + 1 : ci;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = c_row(i), col = n0 + c_col();
-            Xd[row * LDM + col] = out[i];
-            if (gd) gd[slot * HD * HD + (r0 + row) * HD + col] = out[i];
-        }
+        for_c(out, [&](int r, int c, float &x) {
+            Xd[(m0 + r) * LDM + n0 + c] = x;
+            if (gd) gd[slot * HD * HD + (r0 + m0 + r) * HD + n0 + c] = x;
+        });
     }
 }
 
@@ -351,7 +369,7 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
                                                           const float *__restrict__ s_states,
                                                           float *__restrict__ y, int s, int C, int nc, int has_s) {
     extern __shared__ float smem[];
-    float *Ks = smem, *Qs = Ks + MAT, *Es = Qs + MAT, *Ms = Es + MAT, *Ss = Ms + MAT, *Cc = Ss + MAT, *Pw = Cc + MAT;
+    float *Ks = smem, *Qs = Ks + MAT, *Es = Qs + MAT, *Ms = Es + MAT, *Ss = Ms + MAT, *Cc = Ss + MAT;
     __shared__ Coef cf;
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
@@ -372,37 +390,36 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
         if (has_s) commit(Ss, ts);
     }
     __syncthreads();
-    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1);
+    NLH_STRIP_ORIGIN();
     {
-        // E[t][i] = sum_k K[t][k] M0[i][k] - V[t][i]   (in place over V: tiles are disjoint per wave)
-        f32x16 e = zero16(), p = zero16();
-        mma32(e, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
-        // P[t][j] = sum_k Q[t][k] K[j][k]
-        mma32(p, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            Es[row * LDM + col] = e[i] - Es[row * LDM + col];
-            // W[t][j] = -theta_j c[t][j]; Cc is zero outside j <= t < L
-            Pw[row * LDM + col] = -cf.th[col] * Cc[row * LDM + col] * p[i];
-        }
+        // E[t][i] = sum_k K[t][k] M0[i][k] - V[t][i]   (in place over V: strips are disjoint per wave)
+        Strip e = zero_strip(), p = zero_strip();
+        mma(e, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+        // P[t][j] = sum_k Q[t][k] K[j][k];  Pw = W.P over the coefficient matrix, W[t][j] = -theta_j c[t][j]
+        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        for_c(e, [&](int r, int c, float &x) { float *d = Es + (m0 + r) * LDM + n0 + c; *d = x - *d; });
+        for_c(p, [&](int r, int c, float &x) { float *d = Cc + (m0 + r) * LDM + n0 + c; *d = -cf.th[n0 + c] * *d * x; });
     }
     __syncthreads();
-    f32x16 y0 = zero16(), y1 = zero16(), y2 = zero16();
-    mma32(y0, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
-          [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+    const float *Pw = Cc;
+    Strip y0 = zero_strip(), y1 = zero_strip(), y2 = zero_strip();
+    mma(y0, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+        [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
     if (has_s)
-        mma32(y1, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ss[(n0 + n) * LDM + kk]; });
-    mma32(y2, 64, [&](int m, int kk) { return Pw[(m0 + m) * LDM + kk]; },
-          [&](int kk, int n) { return Es[kk * LDM + n0 + n]; });
+        mma(y1, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ss[(n0 + n) * LDM + kk]; });
+    mma(y2, [&](int m, int kk) { return Pw[(m0 + m) * LDM + kk]; },
+        [&](int kk, int n) { return Es[kk * LDM + n0 + n]; });
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const int row = m0 + c_row(i), col = n0 + c_col();
-        if (row < L) y[(tok + row) * HD + col] = cf.a[row] * y0[i] + cf.beta[row] * y1[i] + y2[i];
-    }
+    for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = m0 + row_of(i), col = n0 + 16 * tl + (threadIdx.x & 15);
+            if (row < L)
+                y[(tok + row) * HD + col] = cf.a[row] * y0.t[tl][i] + cf.beta[row] * y1.t[tl][i] + y2.t[tl][i];
+        }
 }
 
 // ── backward, chunk-local pass: what the adjoint scan needs ─────────────────
@@ -446,66 +463,56 @@ __global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restric
         sc[0] = aL; sc[1] = betaL; sc[2] = hL; sc[3] = 0.f;
     }
     __syncthreads();
-    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1);
+    NLH_STRIP_ORIGIN();
     float *out = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
     auto bK = [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; };
 #pragma unroll 1
     for (int o = 0; o < 2; o++) {
         const float *wv = o ? wS : wM;
-        f32x16 acc = zero16();
-        mma32(acc, 64, [&](int m, int kk) { return Ks[kk * LDM + m0 + m] * wv[kk]; }, bK);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            out[(size_t)o * HD * HD + row * HD + col] = acc[i] + ((o == 0 && row == col) ? aL : 0.f);
-        }
+        Strip acc = zero_strip();
+        mma(acc, [&](int m, int kk) { return Ks[kk * LDM + m0 + m] * wv[kk]; }, bK);
+        for_c(acc, [&](int r, int c, float &x) {
+            const int row = m0 + r, col = n0 + c;
+            out[(size_t)o * HD * HD + row * HD + col] = x + ((o == 0 && row == col) ? aL : 0.f);
+        });
     }
-    {   // Cc <- c[t][j] * (q_t . k_j), in place (own tile only)
-        f32x16 p = zero16();
-        mma32(p, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-#pragma unroll
-        for (int i = 0; i < 16; i++) Cc[(m0 + c_row(i)) * LDM + n0 + c_col()] *= p[i];
+    {   // Cc <- c[t][j] * (q_t . k_j), in place (own strip only)
+        Strip p = zero_strip();
+        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        for_c(p, [&](int r, int c, float &x) { Cc[(m0 + r) * LDM + n0 + c] *= x; });
     }
     __syncthreads();
     {   // dE_loc[j][i] = -theta_j sum_t Cc[t][j] dY[t][i]
-        f32x16 e = zero16();
-        mma32(e, 64, [&](int m, int kk) { return Cc[kk * LDM + m0 + m]; },
-              [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i);
-            El[row * LDM + n0 + c_col()] = -cf.th[row] * e[i];
-        }
+        Strip e = zero_strip();
+        mma(e, [&](int m, int kk) { return Cc[kk * LDM + m0 + m]; },
+            [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
+        for_c(e, [&](int r, int c, float &x) { El[(m0 + r) * LDM + n0 + c] = -cf.th[m0 + r] * x; });
     }
     __syncthreads();
-    f32x16 g0 = zero16(), gs = zero16();
-    mma32(g0, 64, [&](int m, int kk) { return cf.a[kk] * Ds[kk * LDM + m0 + m]; },
-          [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
-    mma32(g0, 64, [&](int m, int kk) { return El[kk * LDM + m0 + m]; }, bK);
+    Strip g0 = zero_strip(), gs = zero_strip();
+    mma(g0, [&](int m, int kk) { return cf.a[kk] * Ds[kk * LDM + m0 + m]; },
+        [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+    mma(g0, [&](int m, int kk) { return El[kk * LDM + m0 + m]; }, bK);
     if (has_s)
-        mma32(gs, 64, [&](int m, int kk) { return cf.beta[kk] * Ds[kk * LDM + m0 + m]; },
-              [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const int row = m0 + c_row(i), col = n0 + c_col();
-        out[(size_t)2 * HD * HD + row * HD + col] = g0[i];
-        out[(size_t)3 * HD * HD + row * HD + col] = gs[i];
-    }
+        mma(gs, [&](int m, int kk) { return cf.beta[kk] * Ds[kk * LDM + m0 + m]; },
+            [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+    for_c(g0, [&](int r, int c, float &x) { out[(size_t)2 * HD * HD + (m0 + r) * HD + n0 + c] = x; });
+    for_c(gs, [&](int r, int c, float &x) { out[(size_t)3 * HD * HD + (m0 + r) * HD + n0 + c] = x; });
 }
 constexpr size_t kLocalBwdLds = 5 * MAT * sizeof(float);
 
 // <M0, dMo>, <S0, dMo>, <S0, dSo> per chunk (dMo, dSo: adjoints of the chunk's end state)
-__global__ __launch_bounds__(kThr) void cw_state_dots_kernel(const float *__restrict__ m_states,
-                                                             const float *__restrict__ s_states,
-                                                             const float *__restrict__ dm_states,
-                                                             const float *__restrict__ ds_states,
-                                                             float *__restrict__ scal, int nc, int has_s) {
+__global__ __launch_bounds__(256) void cw_state_dots_kernel(const float *__restrict__ m_states,
+                                                            const float *__restrict__ s_states,
+                                                            const float *__restrict__ dm_states,
+                                                            const float *__restrict__ ds_states,
+                                                            float *__restrict__ scal, int nc, int has_s) {
     __shared__ float slot[3][4];
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc;
     const size_t o0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, o1 = o0 + HD * HD;
     float x0 = 0.f, x1 = 0.f, x2 = 0.f;
-    for (int e = threadIdx.x; e < HD * HD; e += kThr) {
+    for (int e = threadIdx.x; e < HD * HD; e += 256) {
         const float m = m_states[o0 + e], dm = dm_states[o1 + e];
         x0 = fmaf(m, dm, x0);
         if (has_s) {
@@ -523,13 +530,6 @@ __global__ __launch_bounds__(kThr) void cw_state_dots_kernel(const float *__rest
         const float *p = slot[threadIdx.x];
         scal[((size_t)chain * nc + ci) * 4 + threadIdx.x] = p[0] + p[1] + p[2] + p[3];
     }
-}
-
-// Row sums of a 32x32 accumulator tile: every lane gets, for each of its 16 rows, the sum
-// over the tile's 32 columns.
-__device__ __forceinline__ void tile_row_sums(f32x16 &x) {
-#pragma unroll
-    for (int i = 0; i < 16; i++) x[i] = group_allreduce<32>(x[i]);
 }
 
 // ── backward, main per-chunk pass: dQ, dK, dV, dtheta; exports for the gate pass ──
@@ -570,34 +570,39 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
         if (has_s) commit(Ss, ts);
     }
     __syncthreads();
-    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1;
-    const bool writer = (threadIdx.x & 31) == 0;
-    f32x16 p = zero16(), dq = zero16();
+    NLH_STRIP_ORIGIN();
+    auto publish = [&](int which, Strip &x) {   // row sums of x -> part[which][column half][row]
+        strip_row_sums(x);
+        if (row_writer()) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) part[which][nh][m0 + row_of(i)] = x.t[0][i];
+        }
+    };
+    Strip p = zero_strip(), dq = zero_strip();
     {
-        f32x16 e = zero16(), ym = zero16(), ys = zero16();
-        mma32(e, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
-        mma32(p, 64, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-        mma32(ym, 64, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; });
+        Strip e = zero_strip(), ym = zero_strip(), ys = zero_strip(), r0 = zero_strip(), r1 = zero_strip();
+        mma(e, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        mma(ym, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; });
         if (has_s)
-            mma32(ys, 64, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
-                  [&](int kk, int n) { return Ss[kk * LDM + n0 + n]; });
-        f32x16 r0, r1;
+            mma(ys, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
+                [&](int kk, int n) { return Ss[kk * LDM + n0 + n]; });
+        for_c(e, [&](int r, int c, float &x) { float *d = Es + (m0 + r) * LDM + n0 + c; *d = x - *d; });
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            Es[row * LDM + col] = e[i] - Es[row * LDM + col];
-            const float qv = Qs[row * LDM + col];
-            r0[i] = ym[i] * qv; r1[i] = ys[i] * qv;
-            dq[i] = cf.a[row] * ym[i] + cf.beta[row] * ys[i];
-        }
-        tile_row_sums(r0); tile_row_sums(r1);
-        if (writer) {
+        for (int tl = 0; tl < 2; tl++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) { part[0][nh][m0 + c_row(i)] = r0[i]; part[1][nh][m0 + c_row(i)] = r1[i]; }
-        }
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (threadIdx.x & 15);
+                const float qv = Qs[row * LDM + col];
+                r0.t[tl][i] = ym.t[tl][i] * qv;
+                r1.t[tl][i] = ys.t[tl][i] * qv;
+                dq.t[tl][i] = cf.a[row] * ym.t[tl][i] + cf.beta[row] * ys.t[tl][i];
+            }
+        publish(0, r0);
+        publish(1, r1);
     }
     __syncthreads();   // E complete; S0 no longer needed
     Tile<float> tdm, tds;   // adjoint states: in flight during the next two phases
@@ -605,87 +610,84 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     if (has_s) fetch(tds, ds_states + st1, 64);
     float *CP = B5, *CR = B7;
     {
-        f32x16 r = zero16();
-        mma32(r, 64, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Es[(n0 + n) * LDM + kk]; });
+        Strip r = zero_strip();
+        mma(r, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Es[(n0 + n) * LDM + kk]; });
         float *xo = xs + ((size_t)chain * nc + ci) * CW * CW;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            const float c = Cc[row * LDM + col];
-            xo[row * CW + col] = r[i] * p[i];
-            CP[row * LDM + col] = c * p[i];
-            CR[row * LDM + col] = c * r[i];
-        }
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (threadIdx.x & 15);
+                const float c = Cc[row * LDM + col], pv = p.t[tl][i], rv = r.t[tl][i];
+                xo[row * CW + col] = rv * pv;
+                CP[row * LDM + col] = c * pv;
+                CR[row * LDM + col] = c * rv;
+            }
     }
     __syncthreads();   // CP, CR complete; Cc no longer needed
-    mma32(dq, 64, [&](int m, int kk) { return -cf.th[kk] * CR[(m0 + m) * LDM + kk]; },
-          [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const int row = m0 + c_row(i), col = n0 + c_col();
-        if (row < L) d_q[(tok + row) * HD + col] = dq[i];
-    }
+    mma(dq, [&](int m, int kk) { return -cf.th[kk] * CR[(m0 + m) * LDM + kk]; },
+        [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
+    for_c(dq, [&](int r, int c, float &x) {
+        if (m0 + r < L) d_q[(tok + m0 + r) * HD + n0 + c] = x;
+    });
     float *dMs = B6, *dSs = B8;
     commit(dMs, tdm);
     if (has_s) commit(dSs, tds);
     __syncthreads();
     {
         // Dk[j][i] = sum_t CP[t][j] dY[t][i] + cl_j (K dMo^T)[j][i] + bl_j (K dSo^T)[j][i]
-        f32x16 dk = zero16(), t1 = zero16(), t2 = zero16();
-        mma32(dk, 64, [&](int m, int kk) { return CP[kk * LDM + m0 + m]; },
-              [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
-        mma32(t1, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return dMs[(n0 + n) * LDM + kk]; });
+        Strip dk = zero_strip(), t1 = zero_strip(), t2 = zero_strip(), rt = zero_strip();
+        mma(dk, [&](int m, int kk) { return CP[kk * LDM + m0 + m]; },
+            [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
+        mma(t1, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return dMs[(n0 + n) * LDM + kk]; });
         if (has_s)
-            mma32(t2, 64, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
-                  [&](int kk, int n) { return dSs[(n0 + n) * LDM + kk]; });
-        f32x16 rt;
+            mma(t2, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; },
+                [&](int kk, int n) { return dSs[(n0 + n) * LDM + kk]; });
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            dk[i] += cf.cl[row] * t1[i] + cf.bl[row] * t2[i];
-            rt[i] = Es[row * LDM + col] * dk[i];
-            dk[i] *= -cf.th[row];                                 // dE = -theta_j Dk
-            if (row < L) d_v[(tok + row) * HD + col] = -dk[i];    // dV = -dE
-        }
-        tile_row_sums(rt);
-        if (writer) {
+        for (int tl = 0; tl < 2; tl++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) part[2][nh][m0 + c_row(i)] = rt[i];
-        }
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (threadIdx.x & 15);
+                float x = dk.t[tl][i] + cf.cl[row] * t1.t[tl][i] + cf.bl[row] * t2.t[tl][i];
+                rt.t[tl][i] = Es[row * LDM + col] * x;
+                x *= -cf.th[row];                                 // dE = -theta_j Dk
+                dk.t[tl][i] = x;
+                if (row < L) d_v[(tok + row) * HD + col] = -x;    // dV = -dE
+            }
+        publish(2, rt);
         __syncthreads();   // every wave is done reading CP
-#pragma unroll
-        for (int i = 0; i < 16; i++) CP[(m0 + c_row(i)) * LDM + n0 + c_col()] = dk[i];
+        for_c(dk, [&](int r, int c, float &x) { CP[(m0 + r) * LDM + n0 + c] = x; });
     }
     __syncthreads();
     {
         const float *dE = B5;
         // DTe[j][n] = sum_t CR[t][j] Q[t][n] + cl_j (E dMo)[j][n] + bl_j (E dSo)[j][n]
-        f32x16 dt = zero16(), t3 = zero16(), t4 = zero16(), em = zero16();
-        mma32(dt, 64, [&](int m, int kk) { return CR[kk * LDM + m0 + m]; },
-              [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
-        mma32(t3, 64, [&](int m, int kk) { return Es[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return dMs[kk * LDM + n0 + n]; });
+        Strip dt = zero_strip(), t3 = zero_strip(), t4 = zero_strip(), em = zero_strip(), r3 = zero_strip(),
+              r4 = zero_strip();
+        mma(dt, [&](int m, int kk) { return CR[kk * LDM + m0 + m]; },
+            [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+        mma(t3, [&](int m, int kk) { return Es[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return dMs[kk * LDM + n0 + n]; });
         if (has_s)
-            mma32(t4, 64, [&](int m, int kk) { return Es[(m0 + m) * LDM + kk]; },
-                  [&](int kk, int n) { return dSs[kk * LDM + n0 + n]; });
-        mma32(em, 64, [&](int m, int kk) { return dE[(m0 + m) * LDM + kk]; },
-              [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; });
-        f32x16 r3, r4;
+            mma(t4, [&](int m, int kk) { return Es[(m0 + m) * LDM + kk]; },
+                [&](int kk, int n) { return dSs[kk * LDM + n0 + n]; });
+        mma(em, [&](int m, int kk) { return dE[(m0 + m) * LDM + kk]; },
+            [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; });
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int row = m0 + c_row(i), col = n0 + c_col();
-            const float kv = Ks[row * LDM + col];
-            r3[i] = t3[i] * kv; r4[i] = t4[i] * kv;
-            const float dte = dt[i] + cf.cl[row] * t3[i] + cf.bl[row] * t4[i];
-            if (row < L) d_k[(tok + row) * HD + col] = -cf.th[row] * dte + em[i];
-        }
-        tile_row_sums(r3); tile_row_sums(r4);
-        if (writer) {
+        for (int tl = 0; tl < 2; tl++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) { part[3][nh][m0 + c_row(i)] = r3[i]; part[4][nh][m0 + c_row(i)] = r4[i]; }
-        }
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (threadIdx.x & 15);
+                const float kv = Ks[row * LDM + col];
+                r3.t[tl][i] = t3.t[tl][i] * kv;
+                r4.t[tl][i] = t4.t[tl][i] * kv;
+                const float dte = dt.t[tl][i] + cf.cl[row] * t3.t[tl][i] + cf.bl[row] * t4.t[tl][i];
+                if (row < L) d_k[(tok + row) * HD + col] = -cf.th[row] * dte + em.t[tl][i];
+            }
+        publish(3, r3);
+        publish(4, r4);
     }
     __syncthreads();
     if (threadIdx.x < L) {
@@ -733,8 +735,8 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, Bb, Rr);
     commit(Xs, tx);
     __syncthreads();
-    if (threadIdx.x < CW) {   // mat-vecs with W and Ws
-        const int tau = threadIdx.x;
+    if (threadIdx.x >= kThr - CW) {   // mat-vecs with W and Ws (last wave; the matrix products start meanwhile)
+        const int tau = threadIdx.x - (kThr - CW);
         float x0 = 0.f, x1 = 0.f, x2 = 0.f;
         for (int j = 0; j <= tau && j < L; j++) {
             const float wf = -cf.th[j] * Cc[tau * LDM + j], wsv = -cf.th[j] * Bb[j * LDM + tau];
@@ -744,27 +746,30 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
         usm[tau] = cf.h[tau] * s0dm + x1;
         uss[tau] = cf.h[tau] * s0ds + x2;
     }
-    const int w = threadIdx.x >> 6, m0 = 32 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1;
-    f32x16 ua = zero16(), us = zero16();
-    mma32(ua, 64, [&](int m, int kk) { return -cf.th[kk] * Cc[(m0 + m) * LDM + kk]; },
-          [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
+    NLH_STRIP_ORIGIN();
+    Strip ua = zero_strip(), us = zero_strip();
+    mma(ua, [&](int m, int kk) { return -cf.th[kk] * Cc[(m0 + m) * LDM + kk]; },
+        [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
     if (has_s)
-        mma32(us, 64, [&](int m, int kk) { return -cf.th[kk] * Bb[kk * LDM + m0 + m]; },
-              [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
+        mma(us, [&](int m, int kk) { return -cf.th[kk] * Bb[kk * LDM + m0 + m]; },
+            [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
     // row tau feeds token tau+1: weights r[tau+1][t'] (d_alpha) and c[t'][tau+1] (d_eta), zero for t' <= tau
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const int tau = m0 + c_row(i), tp = n0 + c_col();
-        const float uM = cf.a[tau] * p0[tp] + cf.beta[tau] * ps[tp] + ua[i];
-        const float uS = cf.h[tau] * ps[tp] + us[i];
-        const bool ok = tau + 1 < CW;
-        ua[i] = ok ? Rr[(tau + 1) * LDM + tp] * uM : 0.f;
-        us[i] = ok ? Cc[tp * LDM + tau + 1] * uS : 0.f;
-    }
-    tile_row_sums(ua); tile_row_sums(us);
-    if ((threadIdx.x & 31) == 0) {
+    for (int tl = 0; tl < 2; tl++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) { part[0][nh][m0 + c_row(i)] = ua[i]; part[1][nh][m0 + c_row(i)] = us[i]; }
+        for (int i = 0; i < 4; i++) {
+            const int tau = m0 + row_of(i), tp = n0 + 16 * tl + (threadIdx.x & 15);
+            const float uM = cf.a[tau] * p0[tp] + cf.beta[tau] * ps[tp] + ua.t[tl][i];
+            const float uS = cf.h[tau] * ps[tp] + us.t[tl][i];
+            const bool ok = tau + 1 < CW;
+            ua.t[tl][i] = ok ? Rr[(tau + 1) * LDM + tp] * uM : 0.f;
+            us.t[tl][i] = ok ? Cc[tp * LDM + tau + 1] * uS : 0.f;
+        }
+    strip_row_sums(ua);
+    strip_row_sums(us);
+    if (row_writer()) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) { part[0][nh][m0 + row_of(i)] = ua.t[0][i]; part[1][nh][m0 + row_of(i)] = us.t[0][i]; }
     }
     __syncthreads();
     if (threadIdx.x < L) {
@@ -786,17 +791,23 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
 }
 constexpr size_t kGatesBwdLds = 4 * MAT * sizeof(float);
 
-// dst[e] += sum over chains of st[chain][slot 0][e]
-__global__ void cw_accumulate_slot0_kernel(const float *__restrict__ st, float *__restrict__ dst, int batch,
-                                           size_t chain_stride) {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= HD * HD) return;
+// Sum over chains of st[chain][slot 0][.]: stage 1 sums `per` chains per block row into
+// tmp[rows][4096]; stage 2 adds the rows to dst (+=).
+__global__ void cw_sum_slot0_kernel(const float *__restrict__ st, float *__restrict__ tmp, int batch, int per,
+                                    size_t chain_stride) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x, b0 = blockIdx.y * per, b1 = min(batch, b0 + per);
     float x = 0.f;
-    for (int b = 0; b < batch; b++) x += st[(size_t)b * chain_stride + e];
+    for (int b = b0; b < b1; b++) x += st[(size_t)b * chain_stride + e];
+    tmp[(size_t)blockIdx.y * HD * HD + e] = x;
+}
+__global__ void cw_add_rows_kernel(const float *__restrict__ tmp, float *__restrict__ dst, int rows) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    float x = 0.f;
+    for (int r = 0; r < rows; r++) x += tmp[(size_t)r * HD * HD + e];
     dst[e] += x;
 }
 
-constexpr size_t kOutFwdLds = 7 * MAT * sizeof(float);
+constexpr size_t kOutFwdLds = 6 * MAT * sizeof(float);
 
 struct Scratch {
     float *loc, *locs;
@@ -882,7 +893,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr, sc.loc,
                        sc.locs, dm_states, ds_states, nc, (int)has_s);
     check_launch("cw_scan_kernel");
-    hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(kThr), 0, stream(), m_states, s_states,
+    hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(256), 0, stream(), m_states, s_states,
                        dm_states, ds_states, scal, nc, (int)has_s);
     check_launch("cw_state_dots_kernel");
     {
@@ -896,12 +907,16 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                        pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size, nc, (int)has_s);
     check_launch("cw_gates_bwd_kernel");
     const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
-    hipLaunchKernelGGL(cw_accumulate_slot0_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), dm_states,
-                       d_m_initial, batch, chain_stride);
-    if (has_s && d_s_initial)
-        hipLaunchKernelGGL(cw_accumulate_slot0_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), ds_states,
-                           d_s_initial, batch, chain_stride);
-    check_launch("cw_accumulate_slot0_kernel");
+    const int per = 8, rows = ceil_div(batch, per);
+    float *tmp = scratch(10, (size_t)rows * HD * HD * sizeof(float));
+    if (failed()) return;
+    for (int which = 0; which < (has_s && d_s_initial ? 2 : 1); which++) {
+        hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows), dim3(256), 0, stream(),
+                           which ? ds_states : dm_states, tmp, batch, per, chain_stride);
+        hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), tmp,
+                           which ? d_s_initial : d_m_initial, rows);
+    }
+    check_launch("cw_sum_slot0_kernel");
 }
 
 }  // namespace
