@@ -150,14 +150,20 @@ struct Coef {
     float cl[CW], bl[CW];           // c[L-1,j], bb[j,L-1]
 };
 
-__device__ __forceinline__ void load_gates(Coef &cf, const float *alpha, const float *theta, const float *eta,
-                                           int L, bool has_s) {
+// Gates of token (lane % 64) of a chunk, one register each; zero beyond L (eta = 0 without S).
+struct Gates { float al, th, et; };
+__device__ __forceinline__ Gates fetch_gates(const float *alpha, const float *theta, const float *eta, int L,
+                                             bool has_s) {
+    const int t = threadIdx.x & 63;
+    Gates g;
+    g.al = t < L ? alpha[t] : 0.f;
+    g.th = t < L ? theta[t] : 0.f;
+    g.et = (t < L && has_s) ? eta[t] : 0.f;
+    return g;
+}
+__device__ __forceinline__ void load_gates(Coef &cf, const Gates &g) {
     const int t = threadIdx.x;
-    if (t < CW) {
-        cf.al[t] = t < L ? alpha[t] : 0.f;
-        cf.th[t] = t < L ? theta[t] : 0.f;
-        cf.et[t] = (t < L && has_s) ? eta[t] : 0.f;
-    }
+    if (t < CW) { cf.al[t] = g.al; cf.th[t] = g.th; cf.et[t] = g.et; }
 }
 
 __device__ __forceinline__ float lane_bcast(float x, int lane) {
@@ -168,32 +174,31 @@ __device__ __forceinline__ float lane_bcast(float x, int lane) {
 // (stride LDM; entries outside j <= t < L are zero), plus the vectors (wave 1).  The gates
 // are read from global memory into one register per lane and broadcast per step, so the
 // sequential loops carry no memory latency.  Needs a barrier afterwards.
-__device__ __forceinline__ void coefficients(Coef &cf, const float *alpha, const float *eta, int L, bool has_s,
-                                             float *Cc, float *Bb, float *Rr) {
+__device__ __forceinline__ void coefficients(Coef &cf, const Gates &g, int L, float *Cc, float *Bb, float *Rr) {
     const int j = threadIdx.x & 63, w = threadIdx.x >> 6;
     if (w >= 2) return;
-    const float keep_j = j < L ? 1.f - alpha[j] : 1.f;
-    const float eta_j = (j < L && has_s) ? eta[j] : 0.f;
+    const float keep_j = 1.f - g.al;   // 1 beyond L
+    const float eta_j = g.et;          // 0 beyond L
     if (w == 0) {
-        float rr = 1.f, b = 1.f, cc = 1.f;
-#pragma unroll 8
+        // branch-free: tokens after j update the running products; lanes t >= L broadcast
+        // keep = 1, eta = 0, which leaves rr and cc unchanged
+        float rr = 1.f, b = 1.f, cc = 1.f, blv = 0.f;
+        const bool jv = j < L;
+#pragma unroll 16
         for (int t = 0; t < CW; t++) {
             const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
-            float vr = 0.f, vb = 0.f, vc = 0.f;
-            if (t >= j && t < L && j < L) {
-                if (t > j) {
-                    rr *= keep;
-                    b *= et;
-                    cc = keep * cc + b;
-                }
-                vr = rr; vb = b; vc = cc;
-            }
-            if (Cc) Cc[t * LDM + j] = vc;
-            if (Bb) Bb[j * LDM + t] = vb;
-            if (Rr) Rr[j * LDM + t] = vr;
+            const bool after = t > j;
+            rr *= after ? keep : 1.f;
+            b *= after ? et : 1.f;
+            cc = after ? fmaf(keep, cc, b) : cc;
+            blv = (t == L - 1) ? b : blv;
+            const bool valid = jv && t >= j && t < L;
+            if (Cc) Cc[t * LDM + j] = valid ? cc : 0.f;
+            if (Bb) Bb[j * LDM + t] = valid ? b : 0.f;
+            if (Rr) Rr[j * LDM + t] = valid ? rr : 0.f;
         }
-        cf.cl[j] = j < L ? cc : 0.f;
-        cf.bl[j] = j < L ? b : 0.f;
+        cf.cl[j] = jv ? cc : 0.f;
+        cf.bl[j] = jv ? blv : 0.f;
     } else {
         // a_t, beta_t, h_t: every lane runs the same scalar recurrence, lane t keeps step t
         float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f, kh = 0.f;
@@ -238,8 +243,9 @@ __global__ __launch_bounds__(kThr) void cw_local_fwd_kernel(const TIn *__restric
         Tile<TIn> tk, tv;
         fetch(tk, k + tok * HD, L);
         fetch(tv, v + tok * HD, L);
-        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, nullptr, nullptr, nullptr);
+        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        load_gates(cf, gt);
+        coefficients(cf, gt, L, nullptr, nullptr, nullptr);
         commit(Ks, tk);
         commit(Vs, tv);
     }
@@ -367,30 +373,43 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
                                                           const float *__restrict__ eta,
                                                           const float *__restrict__ m_states,
                                                           const float *__restrict__ s_states,
-                                                          float *__restrict__ y, int s, int C, int nc, int has_s) {
+                                                          float *__restrict__ y, int s, int C, int nc, int has_s,
+                                                          int ntask) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Es = Qs + MAT, *Ms = Es + MAT, *Ss = Ms + MAT, *Cc = Ss + MAT;
     __shared__ Coef cf;
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0;
-    {
-        Tile<TIn> tk, tq, tv;
-        Tile<float> tm, ts;
+    NLH_STRIP_ORIGIN();
+    // Persistent over chunk tasks: the tiles and gates of the next task are fetched into
+    // registers while the current one computes, so no task waits for HBM.
+    Tile<TIn> tk, tq, tv;
+    Tile<float> tm, ts;
+    Gates gt;
+    auto fetch_task = [&](int task) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
         fetch(tk, k + tok * HD, L);
         fetch(tq, q + tok * HD, L);
         fetch(tv, v + tok * HD, L);
         fetch(tm, m_states + ((size_t)chain * (nc + 1) + ci) * HD * HD, 64);
         if (has_s) fetch(ts, s_states + ((size_t)chain * (nc + 1) + ci) * HD * HD, 64);
-        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, nullptr, nullptr);
-        commit(Ks, tk);
-        commit(Qs, tq);
-        commit(Es, tv);
-        commit(Ms, tm);
-        if (has_s) commit(Ss, ts);
-    }
+    };
+    // contiguous task range per workgroup: consecutive chunks of a chain share pages and cache lines
+    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per,
+              task_hi = min(ntask, task_lo + per);
+    if (task_lo < task_hi) fetch_task(task_lo);
+    for (int task = task_lo; task < task_hi; task++) {
+    const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    load_gates(cf, gt);
+    coefficients(cf, gt, L, Cc, nullptr, nullptr);
+    commit(Ks, tk);
+    commit(Qs, tq);
+    commit(Es, tv);
+    commit(Ms, tm);
+    if (has_s) commit(Ss, ts);
     __syncthreads();
-    NLH_STRIP_ORIGIN();
+    if (task + 1 < task_hi) fetch_task(task + 1);
     {
         // E[t][i] = sum_k K[t][k] M0[i][k] - V[t][i]   (in place over V: strips are disjoint per wave)
         Strip e = zero_strip(), p = zero_strip();
@@ -420,6 +439,8 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
             if (row < L)
                 y[(tok + row) * HD + col] = cf.a[row] * y0.t[tl][i] + cf.beta[row] * y1.t[tl][i] + y2.t[tl][i];
         }
+    __syncthreads();   // LDS is rewritten by the next task
+    }
 }
 
 // ── backward, chunk-local pass: what the adjoint scan needs ─────────────────
@@ -433,26 +454,36 @@ __global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restric
                                                             const float *__restrict__ theta,
                                                             const float *__restrict__ eta, float *__restrict__ loc,
                                                             float *__restrict__ locs, int s, int C, int nc,
-                                                            int has_s) {
+                                                            int has_s, int ntask) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Cc = Ds + MAT, *El = Cc + MAT;
     __shared__ Coef cf;
     __shared__ float wM[CW], wS[CW];
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0;
-    {
-        Tile<TIn> tk, tq;
-        Tile<float> td;
+    NLH_STRIP_ORIGIN();
+    Tile<TIn> tk, tq;
+    Tile<float> td;
+    Gates gt;
+    auto fetch_task = [&](int task) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
         fetch(tk, k + tok * HD, L);
         fetch(tq, q + tok * HD, L);
         fetch(td, d_y + tok * HD, L);
-        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, nullptr, nullptr);
-        commit(Ks, tk);
-        commit(Qs, tq);
-        commit(Ds, td);
-    }
+    };
+    // contiguous task range per workgroup: consecutive chunks of a chain share pages and cache lines
+    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per,
+              task_hi = min(ntask, task_lo + per);
+    if (task_lo < task_hi) fetch_task(task_lo);
+    for (int task = task_lo; task < task_hi; task++) {
+    const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+    load_gates(cf, gt);
+    coefficients(cf, gt, L, Cc, nullptr, nullptr);
+    commit(Ks, tk);
+    commit(Qs, tq);
+    commit(Ds, td);
     __syncthreads();
+    if (task + 1 < task_hi) fetch_task(task + 1);
     if (threadIdx.x < CW) {
         wM[threadIdx.x] = -cf.th[threadIdx.x] * cf.cl[threadIdx.x];
         wS[threadIdx.x] = -cf.th[threadIdx.x] * cf.bl[threadIdx.x];
@@ -463,7 +494,6 @@ __global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restric
         sc[0] = aL; sc[1] = betaL; sc[2] = hL; sc[3] = 0.f;
     }
     __syncthreads();
-    NLH_STRIP_ORIGIN();
     float *out = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
     auto bK = [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; };
 #pragma unroll 1
@@ -499,6 +529,8 @@ __global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restric
             [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
     for_c(g0, [&](int r, int c, float &x) { out[(size_t)2 * HD * HD + (m0 + r) * HD + n0 + c] = x; });
     for_c(gs, [&](int r, int c, float &x) { out[(size_t)3 * HD * HD + (m0 + r) * HD + n0 + c] = x; });
+    __syncthreads();   // LDS is rewritten by the next task
+    }
 }
 constexpr size_t kLocalBwdLds = 5 * MAT * sizeof(float);
 
@@ -541,36 +573,47 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
     const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, int s, int C, int nc,
-    int has_s) {
+    int has_s, int ntask) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Es = Ds + MAT, *Ms = Es + MAT, *B5 = Ms + MAT,
           *B6 = B5 + MAT, *B7 = B6 + MAT, *B8 = B7 + MAT;
     __shared__ Coef cf;
     __shared__ float part[5][2][CW];   // p0, ps, dtheta, g1, g2: one partial per column half
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0;
-    const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, st1 = st0 + HD * HD;
     float *Ss = B5, *Cc = B6;
-    {
-        Tile<TIn> tk, tq, tv;
-        Tile<float> td, tm, ts;
+    NLH_STRIP_ORIGIN();
+    Tile<TIn> tk, tq, tv;
+    Tile<float> td, tm, ts;
+    Gates gt;
+    auto fetch_task = [&](int task) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD;
+        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
         fetch(tk, k + tok * HD, L);
         fetch(tq, q + tok * HD, L);
         fetch(tv, v + tok * HD, L);
         fetch(td, d_y + tok * HD, L);
         fetch(tm, m_states + st0, 64);
         if (has_s) fetch(ts, s_states + st0, 64);
-        load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, nullptr, nullptr);
-        commit(Ks, tk);
-        commit(Qs, tq);
-        commit(Es, tv);
-        commit(Ds, td);
-        commit(Ms, tm);
-        if (has_s) commit(Ss, ts);
-    }
+    };
+    // one task per workgroup: with the task loop the compiler keeps the LDS addresses of every
+    // phase live across the loop and spills
+    {
+    const int task = blockIdx.x;
+    (void)ntask;
+    const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    const size_t st1 = ((size_t)chain * (nc + 1) + ci + 1) * HD * HD;
+    fetch_task(task);
+    load_gates(cf, gt);
+    coefficients(cf, gt, L, Cc, nullptr, nullptr);
+    commit(Ks, tk);
+    commit(Qs, tq);
+    commit(Es, tv);
+    commit(Ds, td);
+    commit(Ms, tm);
+    if (has_s) commit(Ss, ts);
     __syncthreads();
-    NLH_STRIP_ORIGIN();
     auto publish = [&](int which, Strip &x) {   // row sums of x -> part[which][column half][row]
         strip_row_sums(x);
         if (row_writer()) {
@@ -699,6 +742,7 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
         pv[2] = part[3][0][t] + part[3][1][t];
         pv[3] = part[4][0][t] + part[4][1][t];
     }
+    }
 }
 constexpr size_t kGradsBwdLds = 9 * MAT * sizeof(float);
 
@@ -724,7 +768,8 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     const size_t tok = (size_t)chain * s + t0;
     Tile<float> tx;
     fetch(tx, xs + ((size_t)chain * nc + ci) * CW * CW, 64);
-    load_gates(cf, alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+    const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        load_gates(cf, gt);
     if (threadIdx.x < CW) {
         const int t = threadIdx.x;
         const float4 pv = t < L ? *reinterpret_cast<const float4 *>(pvec + (tok + t) * 4) : make_float4(0, 0, 0, 0);
@@ -732,7 +777,7 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     }
     const float m0dm = scal[((size_t)chain * nc + ci) * 4 + 0], s0dm = scal[((size_t)chain * nc + ci) * 4 + 1],
                 s0ds = scal[((size_t)chain * nc + ci) * 4 + 2];
-    coefficients(cf, alpha + tok, eta + tok, L, has_s != 0, Cc, Bb, Rr);
+    coefficients(cf, gt, L, Cc, Bb, Rr);
     commit(Xs, tx);
     __syncthreads();
     if (threadIdx.x >= kThr - CW) {   // mat-vecs with W and Ws (last wave; the matrix products start meanwhile)
@@ -809,6 +854,19 @@ __global__ void cw_add_rows_kernel(const float *__restrict__ tmp, float *__restr
 
 constexpr size_t kOutFwdLds = 6 * MAT * sizeof(float);
 
+// One workgroup per compute unit for the kernels whose LDS footprint allows no more.
+int persistent_grid(int ntask) {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        check_hip(hipGetDevice(&dev), "hipGetDevice");
+        check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
+        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    return ntask < cus ? ntask : cus;
+}
+
 struct Scratch {
     float *loc, *locs;
 };
@@ -852,8 +910,9 @@ void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const 
     hipLaunchKernelGGL((cw_scan_kernel<true>), dim3(batch * 2), dim3(kThr), 0, stream(), m_initial, s_initial,
                        sc.loc, sc.locs, m_states, has_s ? s_states : nullptr, nc, (int)has_s);
     check_launch("cw_scan_kernel");
-    hipLaunchKernelGGL((cw_out_fwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kOutFwdLds, stream(), k, v, q, alpha,
-                       theta, eta, m_states, s_states, y, seq_len, chunk_size, nc, (int)has_s);
+    hipLaunchKernelGGL((cw_out_fwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kOutFwdLds,
+                       stream(), k, v, q, alpha, theta, eta, m_states, s_states, y, seq_len, chunk_size, nc,
+                       (int)has_s, batch * nc);
     check_launch("cw_out_fwd_kernel");
 }
 
@@ -887,8 +946,9 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         set_lds(cw_gates_bwd_kernel, kGatesBwdLds);
         attr_set = true;
     }
-    hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kLocalBwdLds, stream(), k, q, d_y,
-                       alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc, (int)has_s);
+    hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
+                       stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc, (int)has_s,
+                       batch * nc);
     check_launch("cw_local_bwd_kernel");
     hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr, sc.loc,
                        sc.locs, dm_states, ds_states, nc, (int)has_s);
@@ -898,9 +958,9 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     check_launch("cw_state_dots_kernel");
     {
         KernelTimer kt("cw_grads_bwd_kernel");
-        hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kGradsBwdLds, stream(), k, v, q,
-                           d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta,
-                           pvec, xs, seq_len, chunk_size, nc, (int)has_s);
+        hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kGradsBwdLds,
+                           stream(), k, v, q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k,
+                           d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc);
         check_launch("cw_grads_bwd_kernel");
     }
     hipLaunchKernelGGL(cw_gates_bwd_kernel, dim3(batch * nc), dim3(kThr), kGatesBwdLds, stream(), alpha, theta, eta,
