@@ -443,6 +443,31 @@ void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_me
                                            float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                                            float *d_s_initial, int seq_len, int d, int batch_size,
                                            int chunk_size);
+/* core/src/cuda_ffi.rs:401: predictions[r] -= v[r], then rows with |.|_2 > error_clip are scaled to
+ * error_clip (no clip for error_clip <= 0). */
+void error_subtract_clip_f32_cuda(float *predictions, const float *v, int total_rows, int d, float error_clip);
+/* core/src/cuda_ffi.rs:1000 / 973: k_mem and q_mem are L2-normalised IN PLACE (norm floor 1e-8),
+ * the gates come from the normalised k and raw v (alpha = clamp(sigmoid), theta = clamp(softplus),
+ * eta = sigmoid), then the full-trajectory recurrence runs; alpha/theta/eta/k_norms/q_norms
+ * [batch*seq_len] are written for the backward. */
+void titans_fused_forward_f32_cuda(float *k_mem, const float *v_mem, float *q_mem, const float *w_alpha,
+                                   const float *b_alpha_ptr, const float *w_theta, const float *b_theta_ptr,
+                                   const float *w_eta, const float *b_eta_ptr, float alpha_floor,
+                                   float alpha_ceil, float theta_floor, float theta_ceil,
+                                   const float *m_initial, const float *s_initial, float *m_states,
+                                   float *s_states, float *y, float *alpha_out, float *theta_out,
+                                   float *eta_out, float *k_norms_out, float *q_norms_out, int seq_len, int d,
+                                   int batch_size, float error_clip, float m_norm_max);
+void dgd_fused_forward_f32_cuda(float *k_mem, const float *v_mem, float *q_mem, const float *w_alpha,
+                                const float *b_alpha_ptr, const float *w_theta, const float *b_theta_ptr,
+                                float alpha_floor, float alpha_ceil, float theta_floor, float theta_ceil,
+                                const float *m_initial, float *m_states, float *y, float *alpha_out,
+                                float *theta_out, float *k_norms_out, float *q_norms_out, int seq_len, int d,
+                                int batch_size, float error_clip);
+/* core/src/cuda_ffi.rs:50: attention of the newest token (position cache_len-1) over a bf16 KV
+ * cache [cache_len, heads*hd]; q, out [1, heads*hd]; no weights are kept. */
+void swa_single_token_cuda(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
+                           int cache_len, int num_heads, int head_dim, int window_size, int n_persistent);
 
 #ifdef __cplusplus
 }

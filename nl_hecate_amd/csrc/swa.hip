@@ -14,6 +14,7 @@
 // has no atomics: pass 1 writes d_q and the per-slot score gradients, pass 2
 // gathers d_k / d_v per key in a fixed order, so results are reproducible.
 #include <hip/hip_runtime.h>
+#include <float.h>
 #include <math.h>
 
 #include "../../include/nl_hecate_ffi.h"
@@ -235,6 +236,75 @@ __global__ __launch_bounds__(kSwaWaves * 64) void swa_backward_key_kernel(
     }
 }
 
+// Decode-time attention of the newest token against a KV cache
+// (core/kernels/swa_forward.cu:187-291): same two-range mask as the full kernel
+// for query position cache_len-1, no attention weights kept.  One workgroup per
+// head; a thread scores whole keys (no per-key reduction), then the block
+// normalises and gathers.
+constexpr int kDecThreads = 256;
+__global__ __launch_bounds__(kDecThreads) void swa_single_token_kernel(
+    const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_cache,
+    const unsigned short *__restrict__ v_cache, unsigned short *__restrict__ out, int cache_len, int num_heads,
+    int head_dim, int window, int n_persistent) {
+    extern __shared__ float dsm[];
+    float *qf = dsm, *sc = dsm + head_dim, *red = sc + n_persistent + window;  // red [kDecThreads]
+    __shared__ float wred[kDecThreads / 64];
+    const int h = blockIdx.x, tid = threadIdx.x, total = num_heads * head_dim, hoff = h * head_dim;
+    const int aw = n_persistent + window;
+    const SwaGeom g = swa_geom(cache_len - 1, window, n_persistent);
+    for (int d = tid; d < head_dim; d += kDecThreads) qf[d] = bf2f(q[hoff + d]);
+    __syncthreads();
+    const float scale = rsqrtf((float)head_dim);
+    auto key_of = [&](int w) -> int {   // cache row of score slot w, or -1 when masked
+        if (w < n_persistent) return w < g.n_p ? w : -1;
+        const int l = w - n_persistent;
+        return l < g.ll ? g.ls + l : -1;
+    };
+    float mx = -FLT_MAX;
+    for (int w = tid; w < aw; w += kDecThreads) {
+        const int kp = key_of(w);
+        float sv = -FLT_MAX;
+        if (kp >= 0) {
+            const unsigned short *kr = k_cache + (size_t)kp * total + hoff;
+            float acc = 0.f;
+            for (int d = 0; d < head_dim; d++) acc = fmaf(qf[d], bf2f(kr[d]), acc);
+            sv = acc * scale;
+        }
+        sc[w] = sv;
+        mx = fmaxf(mx, sv);
+    }
+    // block max
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if ((tid & 63) == 0) wred[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(wred[0], wred[1]), fmaxf(wred[2], wred[3]));
+    __syncthreads();
+    float sum = 0.f;
+    for (int w = tid; w < aw; w += kDecThreads) {
+        const float e = expf(sc[w] - mx);
+        sc[w] = e;
+        sum += e;
+    }
+    sum = wave_allreduce(sum);
+    if ((tid & 63) == 0) wred[tid >> 6] = sum;
+    __syncthreads();
+    const float inv = 1.f / (wred[0] + wred[1] + wred[2] + wred[3]);
+    // weighted sum of V: thread (grp, d) walks the slots congruent to grp
+    const int ngrp = kDecThreads / head_dim;   // head_dim <= 256 and divides 256 (checked on the host)
+    const int d = tid % head_dim, grp = tid / head_dim;
+    float acc = 0.f;
+    for (int w = grp; w < aw; w += ngrp) {
+        const int kp = key_of(w);
+        if (kp >= 0) acc = fmaf(sc[w] * inv, bf2f(v_cache[(size_t)kp * total + hoff + d]), acc);
+    }
+    red[tid] = acc;
+    __syncthreads();
+    if (grp == 0) {
+        for (int gg = 1; gg < ngrp; gg++) acc += red[gg * head_dim + d];
+        out[hoff + d] = f2bf(acc);
+    }
+}
+
 static bool swa_check(const char *fn, int seq_len, int num_heads, int head_dim, int window, int batch,
                       int n_persistent) {
     if (seq_len <= 0 || num_heads <= 0 || head_dim <= 0 || window <= 0 || batch <= 0 || n_persistent < 0) {
@@ -288,6 +358,29 @@ void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t 
     hipLaunchKernelGGL(swa_backward_key_kernel, grid, blk, 0, stream(), q, attn_weights, d_attn_out, ds, d_k,
                        d_v, seq_len, num_heads, head_dim, window_size, n_persistent, nq);
     check_launch("swa_backward_key_kernel");
+}
+
+void swa_single_token_cuda(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
+                           int cache_len, int num_heads, int head_dim, int window_size, int n_persistent) {
+    const char *fn = "swa_single_token_cuda";
+    if (cache_len <= 0 || num_heads <= 0 || head_dim <= 0 || window_size <= 0 || n_persistent < 0) {
+        fail("%s: bad shape (cache_len=%d heads=%d head_dim=%d window=%d n_persistent=%d).", fn, cache_len,
+             num_heads, head_dim, window_size, n_persistent);
+        return;
+    }
+    if (head_dim > kDecThreads || kDecThreads % head_dim != 0) {
+        fail("%s: head_dim=%d unsupported (must divide %d).", fn, head_dim, kDecThreads);
+        return;
+    }
+    const size_t lds = ((size_t)head_dim + n_persistent + window_size + kDecThreads) * sizeof(float);
+    if (lds > 64 * 1024) {
+        fail("%s: window + n_persistent = %d needs %zu bytes of LDS (limit 65536).", fn,
+             window_size + n_persistent, lds);
+        return;
+    }
+    hipLaunchKernelGGL(swa_single_token_kernel, dim3(num_heads), dim3(kDecThreads), lds, stream(), q, k_cache,
+                       v_cache, out, cache_len, num_heads, head_dim, window_size, n_persistent);
+    check_launch("swa_single_token_kernel");
 }
 
 }  // extern "C"

@@ -400,3 +400,48 @@ def selfref_backward(cache, d_y):
           c["theta"], c["alpha_mean"], c["eta_mean"], c["traj"], c["frozen"], c["v_hat"],
           d_emb, d_mems, s, d, c["chunk_size"], int(c["self_gen"]), real=real)
     return d_emb, d_mems
+
+
+# ── compositions the reference ships as single kernels ─────────────────────
+def error_subtract_clip(pred, v, error_clip):
+    """core/kernels/error_subtract_clip.cu:18-70: e = pred - v per row; rows with |e|_2 > clip
+    are scaled to clip (float32 arithmetic, clip <= 0: off)."""
+    f = np.float32
+    e = (_c(pred, f) - _c(v, f)).astype(f)
+    if error_clip > 0:
+        for r in range(e.shape[0]):
+            n = np.sqrt(np.sum(e[r] * e[r], dtype=f), dtype=f)
+            if n > f(error_clip):
+                e[r] = e[r] * (f(error_clip) / n)
+    return e
+
+
+def fused_forward(k, v, q, w_alpha, b_alpha, w_theta, b_theta, w_eta, b_eta, alpha_lim, theta_lim, m0, s0,
+                  error_clip=0.0, m_norm_max=F32_MAX):
+    """One chain of core/kernels/titans_forward.cu:569-760 (w_eta None: dgd_forward.cu's fused form):
+    normalise k, q rows (norm floor 1e-8), gates from normalised k and raw v, clamp alpha / theta,
+    then the exact recurrence.  Returns a dict of everything the kernel writes."""
+    f = np.float32
+    kn, knorm = l2_normalize_rows(k)
+    qn, qnorm = l2_normalize_rows(q)
+    alpha = np.clip(gate_compute(kn, v, w_alpha, b_alpha, 0), f(alpha_lim[0]), f(alpha_lim[1])).astype(f)
+    theta = np.clip(gate_compute(kn, v, w_theta, b_theta, 1), f(theta_lim[0]), f(theta_lim[1])).astype(f)
+    out = dict(k=kn, q=qn, k_norms=knorm, q_norms=qnorm, alpha=alpha, theta=theta)
+    if w_eta is not None:
+        eta = gate_compute(kn, v, w_eta, b_eta, 0)
+        y, ms, ss = titans_forward(kn, _c(v, f), qn, alpha, theta, eta, m0, s0, error_clip, m_norm_max)
+        out.update(eta=eta, y=y, m_states=ms, s_states=ss)
+    else:
+        y, ms = delta_forward(kn, _c(v, f), qn, alpha, theta, m0, error_clip, F32_MAX)  # DGD: no projection
+        out.update(y=y, m_states=ms)
+    return out
+
+
+def swa_single_token(q, k_cache, v_cache, window, num_heads, n_persistent=0):
+    """core/kernels/swa_forward.cu:187-291: the full kernel's output row for query position
+    cache_len-1 (q uint16 [H*hd], caches uint16 [cache_len, H*hd])."""
+    cache_len, td = k_cache.shape
+    qf = np.zeros((1, cache_len, td), np.uint16)
+    qf[0, -1] = q
+    out, _ = swa_forward(qf, k_cache[None], v_cache[None], window, num_heads, n_persistent)
+    return out[0, -1]
