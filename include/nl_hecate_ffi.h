@@ -468,6 +468,35 @@ void dgd_fused_forward_f32_cuda(float *k_mem, const float *v_mem, float *q_mem, 
  * cache [cache_len, heads*hd]; q, out [1, heads*hd]; no weights are kept. */
 void swa_single_token_cuda(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
                            int cache_len, int num_heads, int head_dim, int window_size, int n_persistent);
+/* Phase-2 kernels of the split chunkwise path (core/src/cuda_ffi.rs:407-453): the recurrence /
+ * reverse sweep of chunk `chunk_idx` with the chunk's errors [batch, chunk_size, d] supplied by
+ * the caller.  Forward: m_work / s_work [batch, d*d] are the running state (in/out); slot
+ * chunk_idx of m/s_chunk_states [batch, num_chunks+1, d*d] receives the state at the chunk start
+ * (and slot num_chunks the final state after the last chunk).  Backward: d_M / d_S [batch, d*d]
+ * persist across chunks (in/out, per chain), d_M0 [batch, d*d] is written, m/s_recompute
+ * [batch, chunk_size+1, d*d] are caller scratch for the replayed states.  d in {16, 32, 64}. */
+void delta_phase2_forward_f32_cuda(const float *k_mem, const float *q_mem, const float *alpha,
+                                   const float *theta, const float *errors, float *m_work,
+                                   float *m_chunk_states, float *y, int seq_len, int d, int batch_size,
+                                   int chunk_size, int chunk_idx, float m_norm_max);
+void titans_phase2_forward_f32_cuda(const float *k_mem, const float *q_mem, const float *alpha,
+                                    const float *theta, const float *eta, const float *errors,
+                                    float *m_work, float *s_work, float *m_chunk_states,
+                                    float *s_chunk_states, float *y, int seq_len, int d, int batch_size,
+                                    int chunk_size, int chunk_idx, float m_norm_max);
+void delta_phase2_backward_f32_cuda(const float *k_mem, const float *q_mem, const float *alpha,
+                                    const float *theta, const float *errors, const float *m_chunk_states,
+                                    const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                    float *d_alpha, float *d_theta, float *d_M, float *d_M0,
+                                    float *m_recompute, int seq_len, int d, int batch_size, int chunk_size,
+                                    int chunk_idx, float m_norm_max);
+void titans_phase2_backward_f32_cuda(const float *k_mem, const float *q_mem, const float *alpha,
+                                     const float *theta, const float *eta, const float *errors,
+                                     const float *m_chunk_states, const float *s_chunk_states,
+                                     const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                     float *d_alpha, float *d_theta, float *d_eta, float *d_M, float *d_S,
+                                     float *d_M0, float *m_recompute, float *s_recompute, int seq_len, int d,
+                                     int batch_size, int chunk_size, int chunk_idx, float m_norm_max);
 
 #ifdef __cplusplus
 }

@@ -445,3 +445,79 @@ def swa_single_token(q, k_cache, v_cache, window, num_heads, n_persistent=0):
     qf[0, -1] = q
     out, _ = swa_forward(qf, k_cache[None], v_cache[None], window, num_heads, n_persistent)
     return out[0, -1]
+
+
+# ── phase-2 kernels of the split chunkwise path (errors supplied) ───────────
+def _project(m, m_norm_max):
+    f = np.float32
+    if 0 < m_norm_max < 1e30:
+        n = np.sqrt(np.sum(m * m, dtype=f), dtype=f)
+        if n > f(m_norm_max):
+            m = (m * (f(m_norm_max) / n)).astype(f)
+    return m
+
+
+def phase2_forward(k, q, alpha, theta, eta, errors, m, s, m_norm_max=F32_MAX):
+    """One chain, one chunk (core/kernels/titans_phase2_forward.cu:107-139; eta None: the Delta
+    kernel): S' = eta S - theta e k^T, M' = (1-alpha) M + S', project, y = M' q.
+    Returns y [C,d], final M, final S."""
+    f = np.float32
+    m, s = _c(m, f).copy(), (None if eta is None else _c(s, f).copy())
+    ys = []
+    for t in range(k.shape[0]):
+        upd = (-f(theta[t]) * np.outer(errors[t], k[t])).astype(f)
+        if eta is None:
+            m = ((f(1) - f(alpha[t])) * m + upd).astype(f)
+        else:
+            s = (f(eta[t]) * s + upd).astype(f)
+            m = ((f(1) - f(alpha[t])) * m + s).astype(f)
+        m = _project(m, m_norm_max)
+        ys.append((m @ q[t]).astype(f))
+    return np.array(ys, f), m, s
+
+
+def phase2_backward(k, q, alpha, theta, eta, errors, m0, s0, d_y, d_m, d_s, m_norm_max=F32_MAX):
+    """One chain, one chunk (core/kernels/titans_phase2_backward.cu:88-285; eta None: Delta).
+    d_m / d_s: adjoints carried in from later chunks.  Returns the per-token gradients, the
+    updated d_m / d_s and d_m0 (the error path onto the chunk-start matrix)."""
+    f = np.float64   # float64 yardstick: the kernel's float32 sums are compared at 1e-4
+    C, d = k.shape
+    has_s = eta is not None
+    ms, ss = [np.asarray(m0, f)], [np.asarray(s0, f) if has_s else None]
+    for t in range(C):
+        upd = -theta[t] * np.outer(errors[t], k[t])
+        if has_s:
+            ss.append(eta[t] * ss[-1] + upd)
+            mn = (1 - alpha[t]) * ms[-1] + ss[-1]
+        else:
+            mn = (1 - alpha[t]) * ms[-1] + upd
+        if 0 < m_norm_max < 1e30:
+            n = np.linalg.norm(mn)
+            if n > m_norm_max:
+                mn = mn * (m_norm_max / n)
+        ms.append(mn)
+    dm, ds = np.asarray(d_m, f).copy(), (np.asarray(d_s, f).copy() if has_s else None)
+    dm0 = np.zeros((d, d), f)
+    g = {n: np.zeros((C, d), f) for n in ("d_k", "d_v", "d_q")}
+    g.update({n: np.zeros(C, f) for n in ("d_alpha", "d_theta", "d_eta")})
+    for t in range(C - 1, -1, -1):
+        dm += np.outer(d_y[t], q[t])
+        g["d_q"][t] = ms[t + 1].T @ d_y[t]
+        if has_s:
+            ds += dm
+            G = ds
+        else:
+            G = dm
+        g["d_alpha"][t] = -(ms[t] * dm).sum()
+        if has_s:
+            g["d_eta"][t] = (ss[t] * ds).sum()
+        g["d_theta"][t] = -(np.outer(errors[t], k[t]) * G).sum()
+        d_err = -theta[t] * (G @ k[t])
+        g["d_k"][t] = -theta[t] * (G.T @ errors[t]) + ms[0].T @ d_err
+        g["d_v"][t] = -d_err
+        dm0 += np.outer(d_err, k[t])
+        dm = (1 - alpha[t]) * dm
+        if has_s:
+            ds = eta[t] * ds
+    g.update(d_m=dm + dm0, d_s=ds, d_m0=dm0)
+    return g

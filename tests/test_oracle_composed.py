@@ -55,3 +55,39 @@ def test_single_token_decode_matches_sdpa():
     vf = torch.from_numpy(orc.bf16_to_f32(vc)).view(L, H, hd).permute(1, 0, 2)[None, :, L - window:]
     want = torch.nn.functional.scaled_dot_product_attention(qf, kf, vf).reshape(td).numpy()
     assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()
+
+
+def _close(a, b, tol):
+    return np.abs(np.asarray(a, np.float64) - b).max() <= tol * max(np.abs(b).max(), 1e-30)
+
+
+def test_phase2_oracle_chained_equals_chunkwise_oracle():
+    """The numpy phase-2 restatement, fed errors = M0 k - v chunk by chunk, is the chunkwise rule."""
+    r = np.random.default_rng(3)
+    f = np.float32
+    s, d, C = 22, 6, 8
+    k, v, q, dy = (r.standard_normal((s, d)).astype(f) for _ in range(4))
+    sg = lambda x: (1 / (1 + np.exp(-x))).astype(f)
+    al, th, et = (sg(r.standard_normal(s)) for _ in range(3))
+    m0, s0 = (0.2 * r.standard_normal((d, d)).astype(f) for _ in range(2))
+    for has_s in (True, False):
+        y, mc, sc = orc.chunkwise_forward(k, v, q, al, th, et, m0, s0 if has_s else 0 * s0, 8, has_s)
+        g = orc.chunkwise_backward(k, v, q, al, th, et, mc, sc, dy, 8, has_s)
+        nc = (s + C - 1) // C
+        m, sm = m0.copy(), (s0.copy() if has_s else None)
+        errs = []
+        for ci in range(nc):
+            sl = slice(ci * C, min(s, ci * C + C))
+            e = orc.error_subtract_clip(k[sl] @ m.T, v[sl], 0.0)
+            errs.append(e)
+            yy, m, sm = orc.phase2_forward(k[sl], q[sl], al[sl], th[sl], et[sl] if has_s else None, e, m, sm)
+            assert _close(yy, y[sl], 1e-5) and _close(m, mc[ci + 1], 1e-5)
+        dm, ds = np.zeros((d, d)), np.zeros((d, d))
+        for ci in range(nc - 1, -1, -1):
+            sl = slice(ci * C, min(s, ci * C + C))
+            o = orc.phase2_backward(k[sl], q[sl], al[sl], th[sl], et[sl] if has_s else None, errs[ci], mc[ci],
+                                    sc[ci], dy[sl], dm, ds)
+            dm, ds = o["d_m"], o["d_s"]
+            for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta") + (("d_eta",) if has_s else ()):
+                assert _close(o[n], g[n][sl], 1e-4), n
+        assert _close(dm, g["d_m"], 1e-4)
