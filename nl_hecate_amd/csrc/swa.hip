@@ -20,6 +20,7 @@
 #include "../../include/nl_hecate_ffi.h"
 #include "lane_ops.h"
 #include "runtime.h"
+#include "swa_mfma.h"
 
 namespace nlh {
 
@@ -331,6 +332,9 @@ void swa_forward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t *
                           uint16_t *attn_weights, int seq_len, int num_heads, int head_dim,
                           int window_size, int batch_size, int n_persistent) {
     if (!swa_check("swa_forward_f32_cuda", seq_len, num_heads, head_dim, window_size, batch_size, n_persistent))
+        return;
+    if (swa_forward_mfma(q, k, v, out, attn_weights, seq_len, num_heads, head_dim, window_size, batch_size,
+                         n_persistent))
         return;
     const long long nq = (long long)batch_size * num_heads * seq_len;
     const size_t lds = (size_t)kSwaWaves * (((head_dim + 3) & ~3) + n_persistent + window_size) * sizeof(float);

@@ -1,0 +1,11 @@
+// Matrix-core sliding-window attention paths (head size 64, no persistent prefix,
+// window <= 512).  Each returns false without launching when the shape is not covered.
+#pragma once
+#include <stdint.h>
+
+namespace nlh {
+
+bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
+                      int seq_len, int num_heads, int head_dim, int window, int batch, int n_persistent);
+
+}  // namespace nlh
