@@ -350,6 +350,9 @@ void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t 
                            int window_size, int batch_size, int n_persistent) {
     if (!swa_check("swa_backward_f32_cuda", seq_len, num_heads, head_dim, window_size, batch_size, n_persistent))
         return;
+    if (swa_backward_mfma(q, k, v, attn_weights, d_attn_out, d_q, d_k, d_v, seq_len, num_heads, head_dim,
+                          window_size, batch_size, n_persistent))
+        return;
     const long long nq = (long long)batch_size * num_heads * seq_len;
     const int aw = n_persistent + window_size;
     float *ds = scratch(0, (size_t)nq * aw * sizeof(float));

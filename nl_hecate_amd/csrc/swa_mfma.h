@@ -8,4 +8,8 @@ namespace nlh {
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
                       int seq_len, int num_heads, int head_dim, int window, int batch, int n_persistent);
 
+bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *attn_weights,
+                       const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
+                       int head_dim, int window, int batch, int n_persistent);
+
 }  // namespace nlh

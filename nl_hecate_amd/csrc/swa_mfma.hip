@@ -203,6 +203,279 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     }
 }
 
+__device__ __forceinline__ float bf2f(unsigned short h) { return __uint_as_float(((unsigned)h) << 16); }
+// x = hi + lo with hi, lo bf16: the pair carries 16 mantissa bits through a bf16 product
+__device__ __forceinline__ void split4(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const unsigned short h = f2bf(x[i]);
+        hi[i] = (short)h;
+        lo[i] = (short)f2bf(x[i] - bf2f(h));
+    }
+}
+
+// Backward, query pass (one workgroup per 64 queries): D_t = sum_j w dW and
+//   d_q[t] = sum_j dS[t,j] k_j,  dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd)
+// on the stored (bf16) weights.  Same tiling as the forward; dO and dS enter the bf16
+// products as hi + lo pairs.  D_t goes to dvec for the key pass.
+__global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
+                                                             const unsigned short *__restrict__ v,
+                                                             const unsigned short *__restrict__ attn_w,
+                                                             const float *__restrict__ d_out,
+                                                             float *__restrict__ d_q, float *__restrict__ dvec,
+                                                             int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short St[2][KS][LDH];
+    __shared__ __align__(16) unsigned short Pw[4][16][KS];
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const int t0 = blockIdx.x * QB, h = blockIdx.y, b = blockIdx.z;
+    const int total = H * HD, hoff = h * HD;
+    const int base = t0 + QB - NS * KS;
+    const int tq = t0 + 16 * wave + r;
+    const size_t row0 = (size_t)b * s;
+    const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
+    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+
+    bf16x4 doh[4], dol[4];
+#pragma unroll
+    for (int sp = 0; sp < 4; sp++) {
+        f32x4 x = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (tq < s) x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * sp + 4 * g);
+        split4(x, doh[sp], dol[sp]);
+    }
+    f32x4 acc[NT];
+#pragma unroll
+    for (int i = 0; i < NT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto load_rows = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c, key = base + KS * stage + (chunk >> 3);
+            regs[c] = make_uint4(0, 0, 0, 0);
+            if (key >= 0 && key < s)
+                regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + 8 * (chunk & 7));
+        }
+    };
+    // this wave's 16 weight rows for the 64 keys of a stage, zero outside the slot range
+    auto stage_weights = [&](int stage) {
+#pragma unroll 4
+        for (int qi = 0; qi < 16; qi++) {
+            const int tt = t0 + 16 * wave + qi, key = base + KS * stage + l;
+            const int slot = key - max(tt + 1 - ws, 0);
+            unsigned short w = 0;
+            if (tt < s && key <= tt && slot >= 0 && slot < ws) w = awb[(size_t)tt * ws + slot];
+            Pw[wave][qi][l] = w;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    uint4 stg[2];
+
+    // ---- sweep 1: dW^T tiles and D ----
+    float dsum = 0.f;
+    load_rows(v, st_lo, stg);
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        if (st < st_lo) continue;
+        const int buf = st & 1;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&St[buf][chunk >> 3][8 * (chunk & 7)]) = stg[c];
+        }
+        stage_weights(st);
+        __syncthreads();
+        if (st + 1 < NS) load_rows(v, st + 1, stg);
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+#pragma unroll
+            for (int sp = 0; sp < 4; sp++) {
+                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&St[buf][16 * kt + r][16 * sp + 4 * g]);
+                acc[4 * st + kt] = mfma16(a, doh[sp], acc[4 * st + kt]);
+                acc[4 * st + kt] = mfma16(a, dol[sp], acc[4 * st + kt]);
+            }
+            const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dsum = fmaf(bf2f((unsigned short)pb[i]), acc[4 * st + kt][i], dsum);
+        }
+        asm volatile("" ::: "memory");
+    }
+    dsum += __shfl_xor(dsum, 16, 64);
+    dsum += __shfl_xor(dsum, 32, 64);
+    if (g == 0 && tq < s) dvec[(size_t)(b * H + h) * s + tq] = dsum;
+
+    // ---- sweep 2: d_q^T = K^T dS^T ----
+    f32x4 dq[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) dq[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float scale = 0.125f;
+    __syncthreads();
+    load_rows(k, st_lo, stg);
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        if (st < st_lo) continue;
+        const int buf = st & 1;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c, key = chunk >> 3, d0 = 8 * (chunk & 7);
+            const unsigned w[4] = {stg[c].x, stg[c].y, stg[c].z, stg[c].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                St[buf][d0 + 2 * j][key] = (unsigned short)(w[j] & 0xffffu);
+                St[buf][d0 + 2 * j + 1][key] = (unsigned short)(w[j] >> 16);
+            }
+        }
+        stage_weights(st);
+        __syncthreads();
+        if (st + 1 < NS) load_rows(k, st + 1, stg);
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+            const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
+            f32x4 ds;
+#pragma unroll
+            for (int i = 0; i < 4; i++) ds[i] = bf2f((unsigned short)pb[i]) * (acc[4 * st + kt][i] - dsum) * scale;
+            bf16x4 dsh, dsl;
+            split4(ds, dsh, dsl);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&St[buf][16 * dt + r][16 * kt + 4 * g]);
+                dq[dt] = mfma16(a, dsh, dq[dt]);
+                dq[dt] = mfma16(a, dsl, dq[dt]);
+            }
+        }
+        asm volatile("" ::: "memory");
+    }
+    if (tq < s) {
+        float *ob = d_q + (row0 + tq) * total + hoff;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = dq[dt];
+    }
+}
+
+// Backward, key pass (one workgroup per 64 keys, one wave per 16 keys): over the up to 575
+// queries t in [j, j + window) that see key j,
+//   d_v[j] += sum_t w[t,j] dO_t,   d_k[j] += sum_t dS[t,j] q_t,   dS recomputed from w, dO.v_j, D_t.
+// A tile of dS / w in accumulator layout (rows = queries, column = the lane's key) is exactly
+// the A operand of the products with Q^T / dO^T, which are staged transposed in LDS.
+__global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned short *__restrict__ q,
+                                                             const unsigned short *__restrict__ v,
+                                                             const unsigned short *__restrict__ attn_w,
+                                                             const float *__restrict__ d_out,
+                                                             const float *__restrict__ dvec,
+                                                             float *__restrict__ d_k, float *__restrict__ d_v,
+                                                             int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Dh[KS][LDH], Dl[KS][LDH];      // dO hi / lo, [query][dim]
+    __shared__ __align__(16) unsigned short DhT[HD][LDH], DlT[HD][LDH];    // transposed, [dim][query]
+    __shared__ __align__(16) unsigned short QT[HD][LDH];                   // Q^T, [dim][query]
+    __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
+    __shared__ float Dv[KS];
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const int j0 = blockIdx.x * QB, h = blockIdx.y, b = blockIdx.z;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
+    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+    const float *dvb = dvec + (size_t)(b * H + h) * s;
+
+    bf16x4 vf[4];
+#pragma unroll
+    for (int sp = 0; sp < 4; sp++) {
+        vf[sp] = bf16x4{0, 0, 0, 0};
+        if (kj < s) vf[sp] = *reinterpret_cast<const bf16x4 *>(v + (row0 + kj) * total + hoff + 16 * sp + 4 * g);
+    }
+    f32x4 dk[4], dv[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { dk[i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+    const float scale = 0.125f;
+    const int t_last = min(s - 1, j0 + QB - 1 + ws - 1);
+
+    for (int st = 0; st < NS; st++) {
+        const int qs0 = j0 + KS * st;
+        if (qs0 > t_last) break;
+        __syncthreads();   // previous stage's readers are done
+        // dO: 64 rows x 16 chunks of 4 floats
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int chunk = tid + 256 * c, qi = chunk >> 4, d0 = 4 * (chunk & 15), t = qs0 + qi;
+            f32x4 x = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (t < s) x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + d0);
+            bf16x4 hi, lo;
+            split4(x, hi, lo);
+            *reinterpret_cast<bf16x4 *>(&Dh[qi][d0]) = hi;
+            *reinterpret_cast<bf16x4 *>(&Dl[qi][d0]) = lo;
+#pragma unroll
+            for (int j = 0; j < 4; j++) { DhT[d0 + j][qi] = (unsigned short)hi[j]; DlT[d0 + j][qi] = (unsigned short)lo[j]; }
+        }
+        // Q^T: 64 rows x 8 chunks of 8 bf16
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c, qi = chunk >> 3, d0 = 8 * (chunk & 7), t = qs0 + qi;
+            uint4 x = make_uint4(0, 0, 0, 0);
+            if (t < s) x = *reinterpret_cast<const uint4 *>(q + (row0 + t) * total + hoff + d0);
+            const unsigned w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                QT[d0 + 2 * j][qi] = (unsigned short)(w[j] & 0xffffu);
+                QT[d0 + 2 * j + 1][qi] = (unsigned short)(w[j] >> 16);
+            }
+        }
+        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t)
+#pragma unroll
+        for (int c = 0; c < 16; c++) {
+            const int qi = 4 * c + wave, t = qs0 + qi, key = j0 + l;
+            const int slot = key - max(t + 1 - ws, 0);
+            unsigned short w = 0;
+            if (t < s && key <= t && slot >= 0 && slot < ws) w = awb[(size_t)t * ws + slot];
+            Pt[qi][l] = w;
+        }
+        if (tid < KS) Dv[tid] = (qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
+        __syncthreads();
+#pragma unroll
+        for (int qt = 0; qt < 4; qt++) {
+            f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int sp = 0; sp < 4; sp++) {
+                const bf16x4 ah = *reinterpret_cast<const bf16x4 *>(&Dh[16 * qt + r][16 * sp + 4 * g]);
+                const bf16x4 al = *reinterpret_cast<const bf16x4 *>(&Dl[16 * qt + r][16 * sp + 4 * g]);
+                dw = mfma16(ah, vf[sp], dw);
+                dw = mfma16(al, vf[sp], dw);
+            }
+            // accumulator layout: rows = queries 16 qt + 4g + i, column = key r of this wave
+            bf16x4 pa;
+            f32x4 ds;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int qi = 16 * qt + 4 * g + i;
+                const unsigned short pw = Pt[qi][16 * wave + r];
+                pa[i] = (short)pw;
+                ds[i] = bf2f(pw) * (dw[i] - Dv[qi]) * scale;
+            }
+            bf16x4 dsh, dsl;
+            split4(ds, dsh, dsl);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const bf16x4 bh = *reinterpret_cast<const bf16x4 *>(&DhT[16 * dt + r][16 * qt + 4 * g]);
+                const bf16x4 bl = *reinterpret_cast<const bf16x4 *>(&DlT[16 * dt + r][16 * qt + 4 * g]);
+                const bf16x4 bq = *reinterpret_cast<const bf16x4 *>(&QT[16 * dt + r][16 * qt + 4 * g]);
+                dv[dt] = mfma16(pa, bh, dv[dt]);
+                dv[dt] = mfma16(pa, bl, dv[dt]);
+                dk[dt] = mfma16(dsh, bq, dk[dt]);
+                dk[dt] = mfma16(dsl, bq, dk[dt]);
+            }
+        }
+    }
+    // accumulate: rows = keys 16 wave + 4g + i, column = dim 16 dt + r
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int key = j0 + 16 * wave + 4 * g + i;
+        if (key >= s) continue;
+        float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            pk[16 * dt + r] += dk[dt][i];
+            pv[16 * dt + r] += dv[dt][i];
+        }
+    }
+}
+
 }  // namespace
 
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
@@ -215,4 +488,22 @@ bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, u
     return true;
 }
 
+}  // namespace nlh
+
+namespace nlh {
+bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *attn_weights,
+                       const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
+                       int head_dim, int window, int batch, int n_persistent) {
+    if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
+    float *dvec = scratch(1, (size_t)batch * num_heads * seq_len * sizeof(float));
+    if (failed()) return true;
+    const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
+    hipLaunchKernelGGL(swa_bwd_q_mfma_kernel, grid, dim3(256), 0, stream(), k, v, attn_weights, d_attn_out, d_q, dvec,
+                       seq_len, num_heads, window);
+    check_launch("swa_bwd_q_mfma_kernel");
+    hipLaunchKernelGGL(swa_bwd_k_mfma_kernel, grid, dim3(256), 0, stream(), q, v, attn_weights, d_attn_out, dvec, d_k,
+                       d_v, seq_len, num_heads, window);
+    check_launch("swa_bwd_k_mfma_kernel");
+    return true;
+}
 }  // namespace nlh
