@@ -242,7 +242,8 @@ def setup_swa_c5(torch, D, lib):
 
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * heads * s, bound="hbm", dtype="bf16",
-        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_bwd=BYTES_SWA_BWD, traffic_bwd=None,
+        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_bwd=BYTES_SWA_BWD,
+        traffic_bwd=int((1441.1 + 128.0 + 1057.9 + 65.0) * 2**20),   # measured: key pass + query pass
         kernel=None,
         kernel_names={"forward": "swa_forward", "backward": "swa_backward"},
         config={"workload": "BASELINE configs[4], attention branch: sliding-window attention, window 512, 8 heads x 64, "

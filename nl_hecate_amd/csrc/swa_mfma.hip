@@ -255,16 +255,21 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
                 regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + 8 * (chunk & 7));
         }
     };
-    // this wave's 16 weight rows for the 64 keys of a stage, zero outside the slot range
-    auto stage_weights = [&](int stage) {
-#pragma unroll 4
+    // this wave's 16 weight rows for the 64 keys of a stage (zero outside the slot range):
+    // fetched into registers one stage ahead, then written to the wave's LDS tile
+    unsigned short wreg[16];
+    auto fetch_weights = [&](int stage) {
+#pragma unroll
         for (int qi = 0; qi < 16; qi++) {
             const int tt = t0 + 16 * wave + qi, key = base + KS * stage + l;
             const int slot = key - max(tt + 1 - ws, 0);
-            unsigned short w = 0;
-            if (tt < s && key <= tt && slot >= 0 && slot < ws) w = awb[(size_t)tt * ws + slot];
-            Pw[wave][qi][l] = w;
+            wreg[qi] = 0;
+            if (tt < s && key <= tt && slot >= 0 && slot < ws) wreg[qi] = awb[(size_t)tt * ws + slot];
         }
+    };
+    auto commit_weights = [&]() {
+#pragma unroll
+        for (int qi = 0; qi < 16; qi++) Pw[wave][qi][l] = wreg[qi];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
     uint4 stg[2];
@@ -272,6 +277,7 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
     // ---- sweep 1: dW^T tiles and D ----
     float dsum = 0.f;
     load_rows(v, st_lo, stg);
+    fetch_weights(st_lo);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
@@ -281,9 +287,9 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
             const int chunk = tid + 256 * c;
             *reinterpret_cast<uint4 *>(&St[buf][chunk >> 3][8 * (chunk & 7)]) = stg[c];
         }
-        stage_weights(st);
+        commit_weights();
         __syncthreads();
-        if (st + 1 < NS) load_rows(v, st + 1, stg);
+        if (st + 1 < NS) { load_rows(v, st + 1, stg); fetch_weights(st + 1); }
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
 #pragma unroll
@@ -309,6 +315,7 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
     const float scale = 0.125f;
     __syncthreads();
     load_rows(k, st_lo, stg);
+    fetch_weights(st_lo);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
@@ -323,9 +330,9 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
                 St[buf][d0 + 2 * j + 1][key] = (unsigned short)(w[j] >> 16);
             }
         }
-        stage_weights(st);
+        commit_weights();
         __syncthreads();
-        if (st + 1 < NS) load_rows(k, st + 1, stg);
+        if (st + 1 < NS) { load_rows(k, st + 1, stg); fetch_weights(st + 1); }
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
             const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
@@ -387,47 +394,65 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     const float scale = 0.125f;
     const int t_last = min(s - 1, j0 + QB - 1 + ws - 1);
 
+    // global -> register fetch of one stage (64 queries), issued one stage ahead of its use
+    f32x4 gdo[4];
+    uint4 gq[2];
+    unsigned short gw[16];
+    float gd = 0.f;
+    auto fetch_stage = [&](int st) {
+        const int qs0 = j0 + KS * st;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int chunk = tid + 256 * c, t = qs0 + (chunk >> 4);
+            gdo[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (t < s) gdo[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + 4 * (chunk & 15));
+        }
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c, t = qs0 + (chunk >> 3);
+            gq[c] = make_uint4(0, 0, 0, 0);
+            if (t < s) gq[c] = *reinterpret_cast<const uint4 *>(q + (row0 + t) * total + hoff + 8 * (chunk & 7));
+        }
+        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t)
+#pragma unroll
+        for (int c = 0; c < 16; c++) {
+            const int t = qs0 + 4 * c + wave, key = j0 + l;
+            const int slot = key - max(t + 1 - ws, 0);
+            gw[c] = 0;
+            if (t < s && key <= t && slot >= 0 && slot < ws) gw[c] = awb[(size_t)t * ws + slot];
+        }
+        gd = (tid < KS && qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
+    };
+    fetch_stage(0);
     for (int st = 0; st < NS; st++) {
         const int qs0 = j0 + KS * st;
         if (qs0 > t_last) break;
         __syncthreads();   // previous stage's readers are done
-        // dO: 64 rows x 16 chunks of 4 floats
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            const int chunk = tid + 256 * c, qi = chunk >> 4, d0 = 4 * (chunk & 15), t = qs0 + qi;
-            f32x4 x = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (t < s) x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + d0);
+            const int chunk = tid + 256 * c, qi = chunk >> 4, d0 = 4 * (chunk & 15);
             bf16x4 hi, lo;
-            split4(x, hi, lo);
+            split4(gdo[c], hi, lo);
             *reinterpret_cast<bf16x4 *>(&Dh[qi][d0]) = hi;
             *reinterpret_cast<bf16x4 *>(&Dl[qi][d0]) = lo;
 #pragma unroll
             for (int j = 0; j < 4; j++) { DhT[d0 + j][qi] = (unsigned short)hi[j]; DlT[d0 + j][qi] = (unsigned short)lo[j]; }
         }
-        // Q^T: 64 rows x 8 chunks of 8 bf16
 #pragma unroll
         for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, qi = chunk >> 3, d0 = 8 * (chunk & 7), t = qs0 + qi;
-            uint4 x = make_uint4(0, 0, 0, 0);
-            if (t < s) x = *reinterpret_cast<const uint4 *>(q + (row0 + t) * total + hoff + d0);
-            const unsigned w[4] = {x.x, x.y, x.z, x.w};
+            const int chunk = tid + 256 * c, qi = chunk >> 3, d0 = 8 * (chunk & 7);
+            const unsigned w[4] = {gq[c].x, gq[c].y, gq[c].z, gq[c].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 QT[d0 + 2 * j][qi] = (unsigned short)(w[j] & 0xffffu);
                 QT[d0 + 2 * j + 1][qi] = (unsigned short)(w[j] >> 16);
             }
         }
-        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t)
 #pragma unroll
-        for (int c = 0; c < 16; c++) {
-            const int qi = 4 * c + wave, t = qs0 + qi, key = j0 + l;
-            const int slot = key - max(t + 1 - ws, 0);
-            unsigned short w = 0;
-            if (t < s && key <= t && slot >= 0 && slot < ws) w = awb[(size_t)t * ws + slot];
-            Pt[qi][l] = w;
-        }
-        if (tid < KS) Dv[tid] = (qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
+        for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
+        if (tid < KS) Dv[tid] = gd;
         __syncthreads();
+        if (qs0 + KS <= t_last) fetch_stage(st + 1);
 #pragma unroll
         for (int qt = 0; qt < 4; qt++) {
             f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};
