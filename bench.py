@@ -15,6 +15,12 @@ Workloads (BASELINE.json `configs`):
                     tokens (checkpointed forward + fused checkpointed backward).
   swa_c5            the attention branch of configs[4]: sliding-window attention, window 512,
                     8 heads x 64, bf16 storage, fp32 softmax, batch 8, seq 4096, fwd+bwd.
+  mag_layer_c5      configs[4]: the full layer — CMS of k=4 Titans levels (periods 1, 8, 64, 512;
+                    chunkwise rule, chunk 64) gating sliding-window attention (window 512), 8 heads
+                    x 64, batch 8, seq 4096: forward + backward + frequency-aware AdamW step.
+  adamw_c5          the optimizer step of configs[4]: frequency-aware AdamW over the layer's
+                    parameter set (d=512, k=4 levels, all levels firing), gradient-norm clip
+                    + update in two launches; here a "token" is a parameter.
   hope_selfref_c4   configs[3]: HOPE self-referential memory, 8 heads x 64, batch 8,
                     seq 2048, fp32, self-generated values, frozen snapshots per
                     64-token chunk; grads to x and to the six initial memories.
@@ -252,6 +258,100 @@ def setup_swa_c5(torch, D, lib):
         cpu=lambda: cpu_baseline_swa(q, k, v, d_out, window, heads))
 
 
+def setup_mag_layer_c5(torch, D, lib):
+    from nl_hecate_amd.mag_layer import MagLayer, MagTrainer
+    bs, heads, d, s, k, window = 8, 8, 512, 4096, 4, 512
+    layer = MagLayer(d, heads, k, window, [1, 8, 64, 512], rule="chunkwise", chunk=64, seed=0x5EED0007)
+    tr = MagTrainer(layer, lr=3e-4, beta1=0.9, beta2=0.95, weight_decay=0.1)
+    g = torch.Generator(device="cpu").manual_seed(0x5EED0008)
+    x = (torch.randn(bs, s, d, generator=g) / d ** 0.5).cuda()
+    d_out = torch.randn(bs, s, d, generator=g).cuda()
+    st = {}
+
+    def fwd():
+        st["out"], st["cache"] = layer.forward(x)
+
+    def bwd():
+        _, gr = layer.backward(st["cache"], d_out)
+        for dst, src in zip(tr.grads.tensors(), gr.tensors()):
+            dst.copy_(src)
+        tr.opt.step(st["cache"]["pulse"], tr.lr, tr.max_grad_norm, tr.scale)
+
+    # per token: 4 levels x 8 heads x chunkwise memory + 8 heads x SWA (algorithmic bytes / flops of the parts)
+    return dict(
+        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * s, bound="hbm", dtype="bf16",
+        flop_fwd=4 * 8 * FLOP_CW_FWD + 8 * FLOP_SWA_FWD, flop_bwd=4 * 8 * FLOP_CW_BWD + 8 * FLOP_SWA_BWD,
+        bytes_bwd=4 * 8 * BYTES_CW_BWD + 8 * BYTES_SWA_BWD, traffic_bwd=None, kernel=None,
+        kernel_names={"forward": "layer_forward", "backward": "layer_backward_and_adamw"},
+        config={"workload": "BASELINE configs[4]: full layer, CMS k=4 Titans levels at periods [1,8,64,512] (chunkwise "
+                            "rule, chunk 64, bf16 k/v/q) with MAG sigmoid gating over sliding-window attention "
+                            "(window 512, bf16, fp32 softmax), 8 heads x 64 (d=512), batch 8, seq 4096, x ~ N(0,1/d), "
+                            "Xavier weights; forward + backward + AdamW (lr 3e-4, betas 0.9/0.95, wd 0.1); the dense "
+                            "projections are library GEMMs",
+                "batch": bs, "heads": heads, "d_model": d, "seq_len": s, "levels": k, "window": window},
+        cpu=lambda: {"value": None, "unit": "tokens/s", "cores": 1, "kind": "port",
+                     "sample": "not timed: the layer has no CPU restatement beyond its parts (see the per-part workloads)"})
+
+
+def cpu_baseline_adamw(tensors, budget_s=12.0):
+    from oracle import pyoracle as orc
+    host = [(w.cpu().numpy().copy(), g.cpu().numpy(), m.cpu().numpy().copy(), v.cpu().numpy().copy())
+            for w, g, m, v in tensors]
+    n = sum(w.size for w, _, _, _ in host)
+    t_start = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t_start < budget_s:
+        orc.grad_norm_clip([g for _, g, _, _ in host], 1.0)
+        for w, g, m, v in host:
+            orc.adamw_step(w, g, m, v, 3e-4, 0.9, 0.95, 1e-8, 10.0, 20.0, 0.1)
+        reps += 1
+    el = time.perf_counter() - t_start
+    return {"value": reps * n / el, "unit": "params/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} optimizer steps over all {n} parameters (clip + update), {el:.1f} s"}
+
+
+def setup_adamw_c5(torch, D, lib):
+    from nl_hecate_amd.cms import FrequencyAwareAdamW, Pulse
+    d, k = 512, 4
+    g = torch.Generator(device="cpu").manual_seed(0x5EED0006)
+    opt = FrequencyAwareAdamW(k, 0.9, 0.95, 1e-8, 0.1)
+    tensors = []
+
+    def add(group, *shape):
+        w = (torch.randn(*shape, generator=g) * 0.02).cuda()
+        gr = torch.randn(*shape, generator=g).cuda()
+        m, v = torch.zeros_like(w), torch.zeros_like(w)
+        opt.add_tensor(group, w, gr, m, v)
+        tensors.append((w, gr, m, v))
+
+    for _ in range(4):                # attention branch: W_q, W_k, W_v, W_o
+        add(-1, d, d)
+    for level in range(k):            # per level: three memory projections, three gate vectors + biases
+        for _ in range(3):
+            add(level, d, d)
+        for _ in range(3):
+            add(level, 2 * d)
+            add(level, 1)
+    n = sum(w.numel() for w, _, _, _ in tensors)
+    pulse = Pulse(0, [True] * k)
+    scale = torch.zeros(2, dtype=torch.float32, device="cuda")
+
+    def fwd():
+        pass
+
+    def bwd():
+        opt.step(pulse, 3e-4, 1.0, scale)
+
+    return dict(
+        fwd=fwd, bwd=bwd, tokens=n, head_tokens=n, bound="hbm", dtype="f32", unit="params/s",
+        flop_fwd=0, flop_bwd=12, bytes_bwd=28, traffic_bwd=None, kernel=None,
+        kernel_names={"forward": "none", "backward": "adamw_step"},
+        config={"workload": "BASELINE configs[4], optimizer step: frequency-aware AdamW (lr 3e-4, betas 0.9/0.95, wd 0.1) "
+                            "with gradient-norm clip over the layer's parameters, d=512, k=4 levels, all firing",
+                "parameters": n, "tensors": len(tensors)},
+        cpu=lambda: cpu_baseline_adamw(tensors))
+
+
 def setup_hope_selfref_c4(torch, D, lib):
     from nl_hecate_amd import selfref as SR
     bs, heads, d, s, C = 8, 8, 64, 2048, 64
@@ -285,7 +385,8 @@ def setup_hope_selfref_c4(torch, D, lib):
 
 
 WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
-             "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5}
+             "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5,
+             "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5}
 
 
 def main():
@@ -377,14 +478,14 @@ def main():
                 "fp32_matrix": {"achieved": bwd_tflops, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                                 "frac": bwd_tflops / PEAK_FP32_TFLOPS}}
     out = {
-        "metric": METRIC, "value": value, "unit": "tokens/s", "n_gpus": 1,
+        "metric": METRIC, "value": value, "unit": w.get("unit", "tokens/s"), "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.get("dtype", "f32"), "data": "synthetic",
         "config": w["config"],
         "event_ms_per_step": ev_ms / args.steps,
         "kernels_ms": {w["kernel_names"]["forward"]: fwd_ms, w["kernel_names"]["backward"]: bwd_ms},
-        "fwd_fp32_tflops": w["flop_fwd"] * head_tokens / (fwd_ms * 1e-3) / 1e12,
+        "fwd_fp32_tflops": w["flop_fwd"] * head_tokens / (max(fwd_ms, 1e-9) * 1e-3) / 1e12,
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:

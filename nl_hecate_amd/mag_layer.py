@@ -1,0 +1,265 @@
+"""Host orchestration of one MAG layer (sliding-window attention gated by a CMS of
+Titans memories) on the GPU library: the recipe of
+core/src/gpu_forward.rs:864-1071 (forward), core/src/gpu_backward.rs:212-435
+(backward) and, per level, gpu_memory_forward (gpu_forward.rs:1197-1540) /
+gpu_memory_backward (gpu_backward.rs:459-640, 2047-2115).
+
+Everything heavy is a call into the C ABI; the dense projections are plain
+GEMMs (torch.matmul, i.e. rocBLAS/hipBLASLt: the reference's cublasSgemm call
+sites).  Tensors are float32 CUDA tensors unless noted.  The gate -> k/v
+gradient term is not propagated, as on the reference's GPU path.
+"""
+import ctypes
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import torch
+
+from . import dispatch as D
+from .cms import Conductor, FrequencyAwareAdamW, Pulse
+from .ffi import lib
+
+F32_MAX = 3.4028234663852886e38
+
+
+@dataclass
+class MemoryLevelParams:
+    """Outer-loop parameters of one CMS level (core/src/model.rs MemoryLevelParams)."""
+    w_k: torch.Tensor          # [d, d]
+    w_v: torch.Tensor
+    w_q: torch.Tensor
+    w_alpha: torch.Tensor      # [2d]
+    b_alpha: torch.Tensor      # [1]
+    w_theta: torch.Tensor
+    b_theta: torch.Tensor
+    w_eta: torch.Tensor
+    b_eta: torch.Tensor
+
+    def tensors(self):
+        return [self.w_k, self.w_v, self.w_q, self.w_alpha, self.b_alpha, self.w_theta, self.b_theta,
+                self.w_eta, self.b_eta]
+
+
+@dataclass
+class MagParams:
+    w_q: torch.Tensor          # attention branch, [d, d] each
+    w_k: torch.Tensor
+    w_v: torch.Tensor
+    w_o: torch.Tensor
+    levels: List[MemoryLevelParams] = field(default_factory=list)
+
+    def tensors(self):
+        return [self.w_q, self.w_k, self.w_v, self.w_o] + [t for l in self.levels for t in l.tensors()]
+
+
+def init_params(d, k, seed=0, device="cuda"):
+    """Xavier-uniform matrices, small gate vectors, biases that start alpha low, theta small, eta high."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    lim = math.sqrt(6.0 / (2 * d))
+    mat = lambda: ((torch.rand(d, d, generator=g) * 2 - 1) * lim).to(device)
+    vec = lambda: ((torch.rand(2 * d, generator=g) * 2 - 1) * 0.05).to(device)
+    one = lambda x: torch.full((1,), x, dtype=torch.float32, device=device)
+    p = MagParams(mat(), mat(), mat(), mat())
+    for _ in range(k):
+        p.levels.append(MemoryLevelParams(mat(), mat(), mat(), vec(), one(-2.0), vec(), one(-3.0), vec(), one(2.0)))
+    return p
+
+
+def _new(*shape, dtype=torch.float32):
+    return torch.empty(*shape, dtype=dtype, device="cuda")
+
+
+def _zeros(*shape, dtype=torch.float32):
+    return torch.zeros(*shape, dtype=dtype, device="cuda")
+
+
+class MagLayer:
+    """k Titans levels + SWA, MAG sigmoid gating.  `rule`: "exact" (checkpointed exact recurrence,
+    fp32) or "chunkwise" (frozen-M0 chunkwise rule in matrix form, bf16 k/v/q)."""
+
+    def __init__(self, d, heads, k, window, periods, rule="exact", chunk=64, params=None, seed=0):
+        assert d % heads == 0
+        self.d, self.nh, self.hd, self.k, self.window = d, heads, d // heads, k, window
+        self.rule, self.chunk = rule, chunk
+        self.p = params if params is not None else init_params(d, k, seed)
+        self.conductor = Conductor(k, list(periods))
+        # per-level context memory, one matrix per (batch element, head); created on first use
+        self.m_state: List[Optional[torch.Tensor]] = [None] * k
+        self.s_state: List[Optional[torch.Tensor]] = [None] * k
+
+    # ── one level ────────────────────────────────────────────────────────────
+    def _level_forward(self, lv, x2, bs, s, active):
+        """gpu_memory_forward: projections, L2 norm, gates, head split, recurrence."""
+        d, nh, hd = self.d, self.nh, self.hd
+        lp = self.p.levels[lv]
+        B = bs * nh
+        n = bs * s
+        if self.m_state[lv] is None:
+            self.m_state[lv], self.s_state[lv] = _zeros(B, hd * hd), _zeros(B, hd * hd)
+        y = _new(bs, s, d)
+        if not active:
+            # frozen level (gpu_memory_read_only, gpu_forward.rs:2906-2950): y = M_h q with the raw
+            # projection q and the context memory of the first batch slot, shared by the batch
+            q_raw = x2 @ lp.w_q.t()
+            m_shared = self.m_state[lv][:nh].contiguous()
+            D.call("memory_read_only_f32_rocm", q_raw, m_shared, y, n, nh, hd)
+            return y, dict(active=False, m_shared=m_shared)
+        k_mem, v_mem, q_mem = x2 @ lp.w_k.t(), x2 @ lp.w_v.t(), x2 @ lp.w_q.t()
+        k_norms, q_norms = _new(n), _new(n)
+        D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
+        D.call("l2_normalize_rows_f32_cuda", q_mem, q_norms, n, d, 1e-8)
+        c = dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, k_norms=k_norms, q_norms=q_norms, active=active)
+        alpha, theta, eta = _new(n), _new(n), _new(n)
+        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_alpha, lp.b_alpha, alpha, n, d, 0)
+        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_theta, lp.b_theta, theta, n, d, 1)
+        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_eta, lp.b_eta, eta, n, d, 0)
+        kh, vh, qh = _new(B, s, hd), _new(B, s, hd), _new(B, s, hd)
+        for src, dst in ((k_mem, kh), (v_mem, vh), (q_mem, qh)):
+            D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 1)
+        ah, th, eh = _new(B, s), _new(B, s), _new(B, s)
+        for src, dst in ((alpha, ah), (theta, th), (eta, eh)):
+            D.call("broadcast_heads_f32_cuda", src, dst, bs, s, nh)
+        yh = _new(B, s, hd)
+        C = self.chunk
+        if self.rule == "exact":
+            n_ck = 1 + sum(1 for t in range(s) if (t + 1) % C == 0 or t + 1 == s)
+            mc, sc = _new(B, n_ck, hd * hd), _new(B, n_ck, hd * hd)
+            D.call("titans_forward_ckpt_batched_f32_rocm", kh, vh, qh, ah, th, eh, self.m_state[lv],
+                   self.s_state[lv], mc, sc, yh, s, hd, B, C, 0.0, F32_MAX)
+        else:
+            nc = (s + C - 1) // C
+            mc, sc = _new(B, nc + 1, hd * hd), _new(B, nc + 1, hd * hd)
+            kh, vh, qh = kh.to(torch.bfloat16), vh.to(torch.bfloat16), qh.to(torch.bfloat16)
+            D.call("titans_chunkwise_forward_bf16_rocm", kh, vh, qh, ah, th, eh, self.m_state[lv],
+                   self.s_state[lv], mc, sc, yh, s, hd, B, C)
+        # context memory carries over to the next step (copy_final_m_batch, gpu_forward.rs:2824)
+        self.m_state[lv], self.s_state[lv] = mc[:, -1].contiguous(), sc[:, -1].contiguous()
+        D.call("transpose_heads_f32_cuda", yh, y, bs, s, nh, hd, 0)
+        c.update(alpha=alpha, theta=theta, eta=eta, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc)
+        return y, c
+
+    def _level_backward(self, lv, c, x2, d_y, bs, s, grads):
+        """gpu_memory_backward + accumulate_projection_grads; returns the level's d_x [bs*s, d]."""
+        d, nh, hd = self.d, self.nh, self.hd
+        lp, g = self.p.levels[lv], grads.levels[lv]
+        B, n = bs * nh, bs * s
+        if not c["active"]:
+            # read-only level: y = M_h q, only the q path carries gradient
+            m = c["m_shared"].view(nh, hd, hd)
+            dq = torch.einsum("hij,bthi->bthj", m, d_y.view(bs, s, nh, hd)).reshape(n, d)
+            g.w_q += dq.t() @ x2
+            return dq @ lp.w_q
+        dyh = _new(B, s, hd)
+        D.call("transpose_heads_f32_cuda", d_y, dyh, bs, s, nh, hd, 1)
+        dkh, dvh, dqh = _new(B, s, hd), _new(B, s, hd), _new(B, s, hd)
+        dah, dth, deh = _new(B, s), _new(B, s), _new(B, s)
+        dm, ds = _zeros(hd, hd), _zeros(hd, hd)
+        C = self.chunk
+        if self.rule == "exact":
+            D.call("titans_backward_ckpt_f32_rocm", c["kh"], c["vh"], c["qh"], c["ah"], c["th"], c["eh"], c["mc"],
+                   c["sc"], dyh, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, B, C, 0.0, F32_MAX)
+        else:
+            D.call("titans_chunkwise_backward_bf16_rocm", c["kh"], c["vh"], c["qh"], c["ah"], c["th"], c["eh"],
+                   c["mc"], c["sc"], dyh, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, B, C)
+        d_alpha, d_theta, d_eta = _new(n), _new(n), _new(n)
+        for src, dst in ((dah, d_alpha), (dth, d_theta), (deh, d_eta)):
+            D.call("sum_heads_f32_cuda", src, dst, bs, s, nh)
+        dk, dv, dq = _new(n, d), _new(n, d), _new(n, d)
+        for src, dst in ((dkh, dk), (dvh, dv), (dqh, dq)):
+            D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 0)
+        # gate projections (d_w, d_b) from the cached gate outputs
+        D.call("gate_backward_cuda", d_alpha, c["alpha"], d_theta, c["theta"], d_eta, c["eta"], c["k_mem"],
+               c["v_mem"], g.w_alpha, g.b_alpha, g.w_theta, g.b_theta, g.w_eta, g.b_eta, n, d, 1, 1)
+        dk_in, dq_in = _new(n, d), _new(n, d)
+        D.call("l2_normalize_backward_f32_cuda", dk, c["k_mem"], c["k_norms"], dk_in, n, d, 1e-8)
+        D.call("l2_normalize_backward_f32_cuda", dq, c["q_mem"], c["q_norms"], dq_in, n, d, 1e-8)
+        g.w_k += dk_in.t() @ x2
+        g.w_v += dv.t() @ x2
+        g.w_q += dq_in.t() @ x2
+        return dk_in @ lp.w_k + dv @ lp.w_v + dq_in @ lp.w_q
+
+    # ── the layer ────────────────────────────────────────────────────────────
+    def forward(self, x):
+        """x [bs, s, d] -> (out [bs, s, d], cache).  Does not advance the Conductor."""
+        bs, s, d = x.shape
+        p, nh, hd = self.p, self.nh, self.hd
+        x2 = x.reshape(bs * s, d)
+        self.conductor.set_seq_len(s)
+        pulse = self.conductor.pulse()
+        q = (x2 @ p.w_q.t()).to(torch.bfloat16).view(bs, s, d)
+        k = (x2 @ p.w_k.t()).to(torch.bfloat16).view(bs, s, d)
+        v = (x2 @ p.w_v.t()).to(torch.bfloat16).view(bs, s, d)
+        attn_bf, aw = _new(bs, s, d, dtype=torch.bfloat16), _new(bs, nh, s, self.window, dtype=torch.bfloat16)
+        D.call("swa_forward_f32_cuda", q, k, v, attn_bf, aw, s, nh, hd, self.window, bs, 0)
+        attn = attn_bf.to(torch.float32)
+        ys, caches = [], []
+        for lv in range(self.k):
+            y, c = self._level_forward(lv, x2, bs, s, pulse.active_levels[lv])
+            ys.append(y)
+            caches.append(c)
+        y_comb, gate, gated = _new(bs, s, d), _new(bs, s, d), _new(bs, s, d)
+        ptrs = (ctypes.c_void_p * self.k)(*[y.data_ptr() for y in ys])
+        lib.cms_combine_gate_rocm(ptrs, self.k, attn.data_ptr(), y_comb.data_ptr(), gate.data_ptr(),
+                                  gated.data_ptr(), bs * s * d)
+        out = (gated.view(bs * s, d) @ p.w_o.t()).view(bs, s, d)
+        cache = dict(x=x, q=q, k=k, v=v, aw=aw, attn=attn, gate=gate, gated=gated, levels=caches, pulse=pulse,
+                     ys=ys)
+        return out, cache
+
+    def backward(self, cache, d_out):
+        """-> (d_x [bs, s, d], grads: MagParams of gradients)."""
+        x = cache["x"]
+        bs, s, d = x.shape
+        p, nh, hd = self.p, self.nh, self.hd
+        n = bs * s
+        x2 = x.reshape(n, d)
+        do2 = d_out.reshape(n, d)
+        grads = MagParams(*[torch.zeros_like(t) for t in (p.w_q, p.w_k, p.w_v, p.w_o)],
+                          levels=[MemoryLevelParams(*[torch.zeros_like(t) for t in l.tensors()]) for l in p.levels])
+        d_gated = do2 @ p.w_o
+        grads.w_o += do2.t() @ cache["gated"].view(n, d)
+        d_attn, d_ycomb = _new(bs, s, d), _new(bs, s, d)
+        D.call("cms_gate_backward_rocm", d_gated, cache["attn"], cache["gate"], self.k, d_attn, d_ycomb, n * d)
+        d_x = _zeros(n, d)
+        for lv in range(self.k):
+            d_x += self._level_backward(lv, cache["levels"][lv], x2, d_ycomb, bs, s, grads)
+        dq, dk, dv = _new(bs, s, d), _zeros(bs, s, d), _zeros(bs, s, d)
+        D.call("swa_backward_f32_cuda", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv, s, nh,
+               hd, self.window, bs, 0)
+        dq2, dk2, dv2 = dq.view(n, d), dk.view(n, d), dv.view(n, d)
+        grads.w_q += dq2.t() @ x2
+        grads.w_k += dk2.t() @ x2
+        grads.w_v += dv2.t() @ x2
+        d_x += dq2 @ p.w_q + dk2 @ p.w_k + dv2 @ p.w_v
+        return d_x.view(bs, s, d), grads
+
+
+class MagTrainer:
+    """forward + backward + frequency-aware AdamW step (core/src/gpu_optimizer.rs:403-515)."""
+
+    def __init__(self, layer: MagLayer, lr=3e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1,
+                 max_grad_norm=1.0):
+        self.layer, self.lr, self.max_grad_norm = layer, lr, max_grad_norm
+        p = layer.p
+        self.grads = MagParams(*[torch.zeros_like(t) for t in (p.w_q, p.w_k, p.w_v, p.w_o)],
+                               levels=[MemoryLevelParams(*[torch.zeros_like(t) for t in l.tensors()])
+                                       for l in p.levels])
+        self.opt = FrequencyAwareAdamW(layer.k, beta1, beta2, eps, weight_decay)
+        self.state = []
+        groups = [-1] * 4 + [lv for lv in range(layer.k) for _ in range(9)]
+        for grp, w, g in zip(groups, p.tensors(), self.grads.tensors()):
+            m, v = torch.zeros_like(w), torch.zeros_like(w)
+            self.state.append((m, v))
+            self.opt.add_tensor(grp, w, g, m, v)
+        self.scale = torch.zeros(2, dtype=torch.float32, device="cuda")
+
+    def step(self, x, d_out_fn):
+        """One training step; d_out_fn(out) gives the upstream gradient.  Returns out."""
+        out, cache = self.layer.forward(x)
+        _, g = self.layer.backward(cache, d_out_fn(out))
+        for dst, src in zip(self.grads.tensors(), g.tensors()):
+            dst.copy_(src)
+        self.opt.step(cache["pulse"], self.lr, self.max_grad_norm, self.scale)
+        self.layer.conductor.advance()
+        return out
