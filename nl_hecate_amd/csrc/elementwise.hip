@@ -214,19 +214,30 @@ __global__ void gate_backward_stage1(const float *__restrict__ d_alpha, const fl
     }
 }
 
-__global__ void gate_backward_stage2(const float *__restrict__ part, int nblk, int twoD,
-                                     float *d_w_alpha, float *d_b_alpha, float *d_w_theta,
-                                     float *d_b_theta, float *d_w_eta, float *d_b_eta,
-                                     int has_theta, int has_eta) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i > twoD) return;
+// 64 columns per workgroup, 4 thread groups each summing a quarter of the partial blocks,
+// combined in a fixed order.
+__global__ __launch_bounds__(256) void gate_backward_stage2(const float *__restrict__ part, int nblk, int twoD,
+                                                            float *d_w_alpha, float *d_b_alpha, float *d_w_theta,
+                                                            float *d_b_theta, float *d_w_eta, float *d_b_eta,
+                                                            int has_theta, int has_eta) {
+    __shared__ float red[4][3][64];
+    const int col = threadIdx.x & 63, seg = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + col;
     float s[3] = {0.f, 0.f, 0.f};
-    for (int b = 0; b < nblk; b++) {
-        const float *pb = part + (size_t)b * 3 * (twoD + 1);
-        s[0] += pb[i];
-        s[1] += pb[(twoD + 1) + i];
-        s[2] += pb[2 * (twoD + 1) + i];
+    if (i <= twoD) {
+        const int per = (nblk + 3) / 4, b0 = seg * per, b1 = min(nblk, b0 + per);
+        for (int b = b0; b < b1; b++) {
+            const float *pb = part + (size_t)b * 3 * (twoD + 1);
+            s[0] += pb[i];
+            s[1] += pb[(twoD + 1) + i];
+            s[2] += pb[2 * (twoD + 1) + i];
+        }
     }
+    red[seg][0][col] = s[0]; red[seg][1][col] = s[1]; red[seg][2][col] = s[2];
+    __syncthreads();
+    if (seg != 0 || i > twoD) return;
+#pragma unroll
+    for (int g = 1; g < 4; g++) { s[0] += red[g][0][col]; s[1] += red[g][1][col]; s[2] += red[g][2][col]; }
     if (i < twoD) {
         d_w_alpha[i] = s[0];
         if (has_theta) d_w_theta[i] = s[1];
@@ -436,7 +447,7 @@ void gate_backward_cuda(const float *d_alpha, const float *alpha, const float *d
                            d_theta, theta, d_eta, eta, k_mem, v_mem, part, T, D, has_theta, has_eta);
         check_launch("gate_backward_stage1");
     }
-    hipLaunchKernelGGL(gate_backward_stage2, dim3(ceil_div(twoD + 1, kEwThreads)), dim3(kEwThreads), 0,
+    hipLaunchKernelGGL(gate_backward_stage2, dim3(ceil_div(twoD + 1, 64)), dim3(256), 0,
                        stream(), part, nblk, twoD, d_w_alpha, d_b_alpha, d_w_theta, d_b_theta, d_w_eta,
                        d_b_eta, has_theta, has_eta);
     check_launch("gate_backward_stage2");
