@@ -443,6 +443,28 @@ void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_me
                                            float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                                            float *d_s_initial, int seq_len, int d, int batch_size,
                                            int chunk_size);
+/* Delta rule (no momentum state) in the same matrix form: semantics of
+ * delta_chunkwise_{forward,backward}_f32_cuda (core/src/cuda_ffi.rs:356/365) with
+ * error_clip = 0 and no M-norm projection.  d_m_initial [d*d] is accumulated (+=). */
+void delta_chunkwise_forward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                       const float *alpha, const float *theta, const float *m_initial,
+                                       float *m_chunk_states, float *y, int seq_len, int d, int batch_size,
+                                       int chunk_size);
+void delta_chunkwise_forward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                         const float *alpha, const float *theta, const float *m_initial,
+                                         float *m_chunk_states, float *y, int seq_len, int d, int batch_size,
+                                         int chunk_size);
+void delta_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                        const float *alpha, const float *theta, const float *m_chunk_states,
+                                        const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                        float *d_alpha, float *d_theta, float *d_m_initial, int seq_len, int d,
+                                        int batch_size, int chunk_size);
+void delta_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                          const float *alpha, const float *theta, const float *m_chunk_states,
+                                          const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                          float *d_alpha, float *d_theta, float *d_m_initial, int seq_len, int d,
+                                          int batch_size, int chunk_size);
+
 /* core/src/cuda_ffi.rs:401: predictions[r] -= v[r], then rows with |.|_2 > error_clip are scaled to
  * error_clip (no clip for error_clip <= 0). */
 void error_subtract_clip_f32_cuda(float *predictions, const float *v, int total_rows, int d, float error_clip);

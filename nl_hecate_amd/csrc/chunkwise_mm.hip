@@ -1026,3 +1026,42 @@ extern "C" void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const 
                        m_chunk_states, s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
                        d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, true);
 }
+
+// Delta rule (no momentum state): the same passes with eta = 0 and no S traffic.
+extern "C" void delta_chunkwise_forward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem,
+                                                  const uint16_t *q_mem, const float *alpha, const float *theta,
+                                                  const float *m_initial, float *m_chunk_states, float *y,
+                                                  int seq_len, int d, int batch_size, int chunk_size) {
+    forward_mm<uint16_t>("delta_chunkwise_forward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial,
+                         nullptr, m_chunk_states, nullptr, y, seq_len, d, batch_size, chunk_size, false);
+}
+
+extern "C" void delta_chunkwise_forward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                                    const float *alpha, const float *theta, const float *m_initial,
+                                                    float *m_chunk_states, float *y, int seq_len, int d,
+                                                    int batch_size, int chunk_size) {
+    forward_mm<float>("delta_chunkwise_forward_mm_f32_rocm", k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial,
+                      nullptr, m_chunk_states, nullptr, y, seq_len, d, batch_size, chunk_size, false);
+}
+
+extern "C" void delta_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const uint16_t *v_mem,
+                                                   const uint16_t *q_mem, const float *alpha, const float *theta,
+                                                   const float *m_chunk_states, const float *d_y, float *d_k_mem,
+                                                   float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta,
+                                                   float *d_m_initial, int seq_len, int d, int batch_size,
+                                                   int chunk_size) {
+    backward_mm<uint16_t>("delta_chunkwise_backward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, nullptr,
+                          m_chunk_states, nullptr, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr,
+                          d_m_initial, nullptr, seq_len, d, batch_size, chunk_size, false);
+}
+
+extern "C" void delta_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                                     const float *alpha, const float *theta,
+                                                     const float *m_chunk_states, const float *d_y, float *d_k_mem,
+                                                     float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta,
+                                                     float *d_m_initial, int seq_len, int d, int batch_size,
+                                                     int chunk_size) {
+    backward_mm<float>("delta_chunkwise_backward_mm_f32_rocm", k_mem, v_mem, q_mem, alpha, theta, nullptr,
+                       m_chunk_states, nullptr, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr,
+                       d_m_initial, nullptr, seq_len, d, batch_size, chunk_size, false);
+}

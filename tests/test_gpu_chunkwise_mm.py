@@ -136,3 +136,34 @@ def test_matrix_form_agrees_with_sequential_kernels_at_benchmark_shape():
     assert_close("m_chunk_states", host(f["mc"]), host(mc), 1e-3)
     for n in g1:
         assert_close(n, host(g2[n]), host(g1[n]), 1e-3)
+
+
+@pytest.mark.parametrize("B,s,C", [(2, 128, 64), (3, 200, 64), (2, 50, 16)])
+@pytest.mark.parametrize("bf16", [True, False])
+def test_delta_matrix_form_matches_oracle(B, s, C, bf16):
+    d = 64
+    x = make(B, s, d, seed=31 + B * 100 + s + C, bf16=bf16)
+    print(f"chunkwise_mm delta B={B} s={s} C={C} bf16={bf16}", flush=True)
+    fw, bw = [], []
+    for b in range(B):
+        a = [x[n][b] for n in ("k", "v", "q", "alpha", "theta")] + [None]
+        y, mc, _ = orc.chunkwise_forward(*a, x["m0"][b], None, C, False)
+        fw.append((y, mc))
+        bw.append(orc.chunkwise_backward(*a, mc, None, x["dy"][b], C, False))
+    nc = (s + C - 1) // C
+    cv = (lambda a: dev(a).to(torch.bfloat16).contiguous()) if bf16 else dev
+    k, v, q = cv(x["k"]), cv(x["v"]), cv(x["q"])
+    al, th = dev(x["alpha"]), dev(x["theta"])
+    mc, y = zeros(B, nc + 1, d, d), zeros(B, s, d)
+    sfx = "bf16_rocm" if bf16 else "mm_f32_rocm"
+    D.call("delta_chunkwise_forward_" + sfx, k, v, q, al, th, dev(x["m0"]), mc, y, s, d, B, C)
+    g = dict(d_k=zeros(B, s, d), d_v=zeros(B, s, d), d_q=zeros(B, s, d), d_alpha=zeros(B, s),
+             d_theta=zeros(B, s), d_m=zeros(d, d))
+    D.call("delta_chunkwise_backward_" + sfx, k, v, q, al, th, mc, dev(x["dy"]), *[g[n] for n in g], s, d, B, C)
+    torch.cuda.synchronize()
+    tol = 1e-3 if bf16 else 2e-4
+    assert_close("y", host(y), np.stack([f[0] for f in fw]), tol)
+    assert_close("m_chunk_states", host(mc), np.stack([f[1] for f in fw]), tol)
+    for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta"):
+        assert_close(n, host(g[n]), np.stack([o[n] for o in bw]), tol)
+    assert_close("d_m_initial", host(g["d_m"]), sum(o["d_m"] for o in bw), tol)
