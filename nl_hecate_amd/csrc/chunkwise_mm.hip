@@ -29,6 +29,7 @@
 #include <stdint.h>
 
 #include "../../include/nl_hecate_ffi.h"
+#include "chunkwise_chain.h"
 #include "rule_common.h"
 #include "runtime.h"
 
@@ -990,6 +991,10 @@ extern "C" void titans_chunkwise_forward_bf16_rocm(const uint16_t *k_mem, const 
                                                    const float *s_initial, float *m_chunk_states,
                                                    float *s_chunk_states, float *y, int seq_len, int d,
                                                    int batch_size, int chunk_size) {
+    if (chunkwise_chain_forward_bf16("titans_chunkwise_forward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
+                                     m_initial, s_initial, m_chunk_states, s_chunk_states, y, seq_len, d, batch_size,
+                                     chunk_size, true))
+        return;
     forward_mm<uint16_t>("titans_chunkwise_forward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, eta, m_initial,
                          s_initial, m_chunk_states, s_chunk_states, y, seq_len, d, batch_size, chunk_size, true);
 }
@@ -1032,6 +1037,10 @@ extern "C" void delta_chunkwise_forward_bf16_rocm(const uint16_t *k_mem, const u
                                                   const uint16_t *q_mem, const float *alpha, const float *theta,
                                                   const float *m_initial, float *m_chunk_states, float *y,
                                                   int seq_len, int d, int batch_size, int chunk_size) {
+    if (chunkwise_chain_forward_bf16("delta_chunkwise_forward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, nullptr,
+                                     m_initial, nullptr, m_chunk_states, nullptr, y, seq_len, d, batch_size,
+                                     chunk_size, false))
+        return;
     forward_mm<uint16_t>("delta_chunkwise_forward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial,
                          nullptr, m_chunk_states, nullptr, y, seq_len, d, batch_size, chunk_size, false);
 }
