@@ -197,7 +197,7 @@ def setup_titans_chunkwise_c3(torch, D, lib):
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16",
         flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_bwd=BYTES_CW_BWD,
         traffic_bwd=int((838.3 + 522.0) * 2**20),   # measured for cw_grads_bwd_kernel: 838.3 MiB read, 522.0 MiB written
-        kernel="cw_grads_bwd_kernel<bf16> (the largest of the backward entry point's kernels)",
+        kernel="cw_grads_bf16_kernel (the per-chunk gradient pass of the backward entry point)",
         kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
         config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
                             "batch 16, seq 4096, bf16 k/v/q with fp32 accumulate and fp32 M/S, fwd+bwd",

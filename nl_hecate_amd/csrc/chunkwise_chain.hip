@@ -22,21 +22,13 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "bf16_tiles.h"
 #include "chunkwise_chain.h"
 #include "runtime.h"
 
 namespace nlh {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned short u16;
-
-constexpr int HD = 64;             // head size
-constexpr int CW = 64;             // tokens per chunk tile
-constexpr int LDB = 72;            // LDS row stride of a bf16 matrix (144 B: 16-byte rows, conflict-free operand reads)
-constexpr int BMAT = 64 * LDB;     // elements per bf16 matrix
 constexpr int kChainThr = 512;     // 8 waves
 
 // Work split of the eight waves: a 64x64 product is four 32x32 blocks (2x2 tiles of 16x16; an
@@ -54,47 +46,6 @@ constexpr int kChainThr = 512;     // 8 waves
 constexpr int kTableFloats = CW * CW;
 constexpr int kVecFloats = 4 * CW + 16;
 __device__ __forceinline__ bool tile_live(int bi, int rt, int ct) { return 2 * (bi & 1) + ct >= 2 * (bi >> 1) + rt; }
-
-__device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
-__device__ __forceinline__ float bf2f(u16 h) { return __uint_as_float(((unsigned)h) << 16); }
-__device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-// Operand of one 16x16x32 step from a bf16 matrix whose rows run along the contraction:
-// lane l supplies row row0 + l%16, contraction indices 32*ks + 8*(l/16) .. +8.  The same
-// loader serves A (rows = output rows) and B (rows = output columns).
-__device__ __forceinline__ bf16x8 ld_op(const u16 *X, int row0, int ks) {
-    const int l = threadIdx.x & 63;
-    return *reinterpret_cast<const bf16x8 *>(X + (row0 + (l & 15)) * LDB + 32 * ks + 8 * (l >> 4));
-}
-// x = hi + lo with hi, lo bf16; both stored as four consecutive elements at off.
-__device__ __forceinline__ void split_store(u16 *H, u16 *Lo, int off, f32x4 x) {
-    bf16x4 h, lo;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const __bf16 hb = (__bf16)x[i];
-        h[i] = hb;
-        lo[i] = (__bf16)(x[i] - (float)hb);
-    }
-    *reinterpret_cast<bf16x4 *>(H + off) = h;
-    *reinterpret_cast<bf16x4 *>(Lo + off) = lo;
-}
-__device__ __forceinline__ float lane_bcast(float x, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
-}
-
-// Gates of token (lane) of a chunk; zero beyond L (eta = 0 without momentum).
-struct Gates { float al, th, et; };
-template <bool HAS_S>
-__device__ __forceinline__ Gates fetch_gates(const float *alpha, const float *theta, const float *eta, size_t tok,
-                                             int L) {
-    const int t = threadIdx.x & 63;
-    Gates g;
-    g.al = t < L ? alpha[tok + t] : 0.f;
-    g.th = t < L ? theta[tok + t] : 0.f;
-    g.et = (HAS_S && t < L) ? eta[tok + t] : 0.f;
-    return g;
-}
 
 // Coefficients of one chunk from its gates: two waves per chunk.  Wave role 0 (lane j): the
 // column recurrences c[t][j], bb[j][t] over t.  Role 1 (lane t): a_t, beta_t, h_t.

@@ -1,0 +1,619 @@
+// Backward of the frozen-M0 chunkwise Titans / Delta rule on bf16 tokens: the per-chunk
+// gradients d_q, d_k, d_v, d_theta and what the gate pass needs, on the bf16 matrix cores.
+//
+// Same mathematics as cw_grads_bwd_kernel of chunkwise_mm.hip (which documents the
+// formulas); inputs are the chunk-start states M0, S0 and the adjoints dMo, dSo of the
+// chunk-end states from the adjoint scan.  With E = K M0^T - V, P = Q K^T, R = dY E^T,
+// c = coefficient table, cl_j = c[L-1][j], bl_j = bb[j][L-1]:
+//   X   = R.P                                   (to the gate pass)
+//   dQ  = a.(dY M0) + beta.(dY S0) + (-theta_j c.R) K
+//   Dk  = (c.P)^T dY + cl.(K dMo^T) + bl.(K dSo^T)        [token j][row i]
+//   dE  = -theta_j Dk,  dV = -dE,  d_theta_j = -sum_i E Dk
+//   DTe = (c.R)^T Q + cl.(E dMo) + bl.(E dSo)             [token j][column c]
+//   dK  = -theta_j DTe + dE M0
+// plus the row sums p0, ps, g1, g2 and the three state dots of the gate pass.
+//
+// Precision: k, v, q are exact in bf16.  E is formed against a hi + lo bf16 pair of M0
+// (its two terms nearly cancel once the memory has learned); every other fp32 operand (dY,
+// states, adjoints, E, c.P, c.R, dE) enters the matrix cores rounded to one bf16, products
+// accumulate in fp32.  That is the bf16-input / fp32-accumulate contract: results agree with
+// the fp32 oracle to a few 1e-3, inside the 2e-2 stated for this path.
+//
+// One workgroup per compute unit walks over chunks.  While one chunk computes, every 128-byte
+// line of the next chunk's inputs is touched by one 4-byte load, so that the real loads at the
+// top of the next step come from the L2 cache; holding the inputs themselves in registers
+// across a step would not fit beside the accumulators.  Every output tile is computed transposed
+// (rows = feature, columns = token) so that a lane ends up with four consecutive features of
+// one token: 16-byte stores.  Waves 0..3 (group A) hold P and produce X, c.P, c.R, Dk; waves
+// 4..7 (group B) hold dQ and produce -theta c.R, dQ, DTe, dK.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "bf16_tiles.h"
+#include "chunkwise_grads.h"
+#include "runtime.h"
+
+namespace nlh {
+namespace {
+
+// Per-chunk coefficients in HBM, written by cw_coef_bwd_kernel:
+//   tab_a [chunk][block bi][rt][ct][lane l][r]: c[t][j] (zero outside j <= t < L) at
+//         j = 32 (bi/2) + 16 rt + 4 (l/16) + r, t = 32 (bi%2) + 16 ct + l%16   (group B: R^T)
+//   tab_b same for t = 32 (bi/2) + 16 rt + 4 (l/16) + r, j = 32 (bi%2) + 16 ct + l%16  (group A: P, R)
+//   vecs  [chunk][kVecB]: a_t, beta_t, cl_j, bl_j, theta_j, then four zeros
+// Tiles entirely above the diagonal are neither written nor read.
+constexpr int kTab = CW * CW;
+constexpr int kVecB = 5 * CW + 16;
+__device__ __forceinline__ bool live_a(int bi, int rt, int ct) { return 2 * (bi & 1) + ct >= 2 * (bi >> 1) + rt; }
+__device__ __forceinline__ bool live_b(int bi, int rt, int ct) { return 2 * (bi >> 1) + rt >= 2 * (bi & 1) + ct; }
+
+template <bool HAS_S>
+__global__ __launch_bounds__(256) void cw_coef_bwd_kernel(const float *__restrict__ alpha,
+                                                          const float *__restrict__ theta,
+                                                          const float *__restrict__ eta, float *__restrict__ tab_a,
+                                                          float *__restrict__ tab_b, float *__restrict__ vecs,
+                                                          int s, int C, int nc, int nchunks) {
+    const int chunk = blockIdx.x * 2 + (threadIdx.x >> 7), role = (threadIdx.x >> 6) & 1, j = threadIdx.x & 63;
+    if (chunk >= nchunks) return;
+    const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
+    const Gates g = fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, L);
+    const float keep_j = 1.f - g.al;   // 1 beyond L
+    const float eta_j = g.et;          // 0 beyond L
+    float *vo = vecs + (size_t)chunk * kVecB;
+    if (role == 0) {
+        float *ta = tab_a + (size_t)chunk * kTab, *tb = tab_b + (size_t)chunk * kTab;
+        float b = 1.f, cc = 1.f, blv = 0.f;
+        const bool jv = j < L;
+        const int ja = (j >> 5) * 2048 + ((j >> 4) & 1) * 512 + ((j & 15) >> 2) * 64 + (j & 3);
+        const int jb = (j >> 5) * 1024 + ((j >> 4) & 1) * 256 + (j & 15) * 4;
+#pragma unroll
+        for (int t = 0; t < CW; t++) {
+            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
+            const bool after = t > j;
+            b *= after ? et : 1.f;
+            cc = after ? fmaf(keep, cc, b) : cc;
+            blv = (t == L - 1) ? b : blv;
+            if ((t >> 4) >= (j >> 4)) {
+                const float x = (jv && t >= j && t < L) ? cc : 0.f;
+                ta[ja + (t >> 5) * 1024 + ((t >> 4) & 1) * 256 + (t & 15) * 4] = x;
+                tb[jb + (t >> 5) * 2048 + ((t >> 4) & 1) * 512 + ((t & 15) >> 2) * 64 + (t & 3)] = x;
+            }
+        }
+        vo[2 * CW + j] = jv ? cc : 0.f;
+        vo[3 * CW + j] = jv ? blv : 0.f;
+        vo[4 * CW + j] = g.th;
+    } else {
+        float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f;
+#pragma unroll
+        for (int t = 0; t < CW; t++) {
+            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
+            a *= keep;
+            h *= et;
+            beta = fmaf(keep, beta, h);
+            if (t == j) { ka = a; kb = beta; }
+        }
+        vo[j] = j < L ? ka : 0.f;
+        vo[CW + j] = j < L ? kb : 0.f;
+        if (j < 4) vo[5 * CW + j] = 0.f;   // what tiles above the diagonal read
+    }
+}
+
+// Sum over the four 16-lane groups of a wave (lanes with equal l%16).
+__device__ __forceinline__ float sum_groups(float x) {
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
+}
+__device__ __forceinline__ float sum_wave(float x) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) x += __shfl_xor(x, m);
+    return x;
+}
+__device__ __forceinline__ f32x4 bf4_to_f32(const u16 *p) {
+    const uint2 b = *reinterpret_cast<const uint2 *>(p);
+    return f32x4{__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u), __uint_as_float(b.y << 16),
+                 __uint_as_float(b.y & 0xffff0000u)};
+}
+
+template <bool HAS_S>
+__global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
+    const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q, const float *__restrict__ d_y,
+    const float *__restrict__ tab_a, const float *__restrict__ tab_b, const float *__restrict__ vecs,
+    const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
+    const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
+    float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
+    int C, int nc, int ntask) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Kt = Kr + BMAT;   // K [t][c], K^T [c][t]
+    u16 *Qr = Kt + BMAT, *Qt = Qr + BMAT;                            // Q, Q^T
+    u16 *Vr = Qt + BMAT;                                             // V [t][i]
+    u16 *dYr = Vr + BMAT, *dYt = dYr + BMAT;                         // dY [t][i], dY^T [i][t]
+    u16 *M0h = dYt + BMAT, *M0l = M0h + BMAT, *M0t = M0l + BMAT;     // M0 [i][c] hi / lo, M0^T [c][i]
+    u16 *S0t = M0t + BMAT;                                           // S0^T [c][i]
+    u16 *dMr = S0t + BMAT, *dMt = dMr + BMAT;                        // dMo [i][c], dMo^T [c][i]
+    u16 *dSr = dMt + BMAT, *dSt = dSr + BMAT;                        // dSo
+    u16 *Er = dSt + BMAT;                                            // E [t][i]
+    u16 *CPt = Vr, *CRt = M0h, *ThCR = M0l, *dEr = S0t;              // reuse once their first tenants are dead
+    float *cvec = reinterpret_cast<float *>(Er + BMAT);              // a, beta, cl, bl, theta [64] each
+    float *part = cvec + 5 * CW;                                     // [5][2][64]: p0, ps, rt, g1, g2 per half
+    float *dots = part + 5 * 2 * CW;                                 // [3][8]
+
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
+    const bool grpA = w < 4;
+    const int bi = w & 3, bm = 32 * (bi >> 1), bn = 32 * (bi & 1);
+    // Staging maps.  A wave instruction reads whole or half 128-byte lines (the rate of line
+    // requests, not bytes, bounds a compute unit), and the 2-byte transposed LDS writes of a
+    // wave land on 16 different banks.
+    //   bf16 tile: row st_t, 8-element block st_cb (16 rows x 64 bytes per wave)
+    //   fp32 tile: row ft, 4-element blocks fg0 and fg0 + 8 (8 rows x 128 bytes per wave and pass)
+    const int st_t = 16 * (w & 3) + (l & 15), st_cb = 4 * (w >> 2) + (l >> 4);
+    const int ft = 8 * w + (l >> 3), fg0 = l & 7;
+
+    // inputs of the current task in registers (only while they are staged)
+    uint4 nK, nQ, nV;
+    f32x4 ndY[2], nM0[2], nS0[2], ndM[2], ndS[2], ntab[2][2];
+    float nvec = 0.f;
+    auto fetch = [&](int task) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0, row = tok + min(st_t, L - 1), frow = tok + min(ft, L - 1);
+        nK = *reinterpret_cast<const uint4 *>(k + row * HD + st_cb * 8);
+        nQ = *reinterpret_cast<const uint4 *>(q + row * HD + st_cb * 8);
+        nV = *reinterpret_cast<const uint4 *>(v + row * HD + st_cb * 8);
+        const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD + ft * HD, st1 = st0 + HD * HD;
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int c4 = (fg0 + 8 * it) * 4;
+            ndY[it] = *reinterpret_cast<const f32x4 *>(d_y + frow * HD + c4);
+            nM0[it] = *reinterpret_cast<const f32x4 *>(m_states + st0 + c4);
+            ndM[it] = *reinterpret_cast<const f32x4 *>(dm_states + st1 + c4);
+            if (HAS_S) {
+                nS0[it] = *reinterpret_cast<const f32x4 *>(s_states + st0 + c4);
+                ndS[it] = *reinterpret_cast<const f32x4 *>(ds_states + st1 + c4);
+            }
+        }
+        nvec = vecs[(size_t)task * kVecB + min(tid, 5 * CW - 1)];
+    };
+    // the coefficient table of a task is requested separately, once the previous one has been used
+    auto fetch_tab = [&](int task) {
+        const float *zero = vecs + (size_t)task * kVecB + 5 * CW;
+        const float *tb = (grpA ? tab_b : tab_a) + (size_t)task * kTab;
+#pragma unroll
+        for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                const bool live = grpA ? live_b(bi, rt, ct) : live_a(bi, rt, ct);
+                ntab[rt][ct] =
+                    *reinterpret_cast<const f32x4 *>(live ? tb + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4 : zero);
+            }
+    };
+
+    // contiguous task range per workgroup: consecutive chunks of a chain share pages and cache lines
+    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per,
+              task_hi = min(ntask, task_lo + per);
+    if (task_lo >= task_hi) return;
+    // One load per 128-byte line of a task's inputs: 3 bf16 tiles of 64 lines, then 5 fp32 tiles of
+    // 128 lines; thread tid takes lines tid and tid + 512.
+    float touched0 = 0.f, touched1 = 0.f;
+    auto touch = [&](int task) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, st1 = st0 + HD * HD;
+        auto line = [&](int ln) -> const void * {
+            if (ln < 192) {
+                const u16 *base = ln < 64 ? k : (ln < 128 ? q : v);
+                return base + (tok + min(ln & 63, L - 1)) * HD;
+            }
+            const int f = (ln - 192) >> 7, o = (ln - 192) & 127;   // line o of fp32 tile f: row o/2, half o%2
+            if (f == 0) return d_y + (tok + min(o >> 1, L - 1)) * HD + (o & 1) * 32;
+            const float *base = f == 1 ? m_states + st0 : (f == 2 ? (HAS_S ? s_states + st0 : m_states + st0)
+                                : (f == 3 ? dm_states + st1 : (HAS_S ? ds_states + st1 : dm_states + st1)));
+            return base + o * 32;
+        };
+        touched0 = *reinterpret_cast<const float *>(line(tid));
+        touched1 = *reinterpret_cast<const float *>(line(min(tid + 512, 831)));
+    };
+    fetch_tab(task_lo);
+
+    for (int task = task_lo; task < task_hi; task++) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        // ── load and stage everything ──
+        asm volatile("" ::"v"(touched0), "v"(touched1));   // the touches of this task end here
+        fetch(task);
+        {
+            if (st_t >= L) { nK = make_uint4(0, 0, 0, 0); nQ = nK; nV = nK; }
+            if (ft >= L) { ndY[0] = zero4(); ndY[1] = zero4(); }
+            *reinterpret_cast<uint4 *>(Kr + st_t * LDB + st_cb * 8) = nK;
+            *reinterpret_cast<uint4 *>(Qr + st_t * LDB + st_cb * 8) = nQ;
+            *reinterpret_cast<uint4 *>(Vr + st_t * LDB + st_cb * 8) = nV;
+            const unsigned kw[4] = {nK.x, nK.y, nK.z, nK.w}, qw[4] = {nQ.x, nQ.y, nQ.z, nQ.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                Kt[(st_cb * 8 + 2 * i) * LDB + st_t] = (u16)(kw[i] & 0xffffu);
+                Kt[(st_cb * 8 + 2 * i + 1) * LDB + st_t] = (u16)(kw[i] >> 16);
+                Qt[(st_cb * 8 + 2 * i) * LDB + st_t] = (u16)(qw[i] & 0xffffu);
+                Qt[(st_cb * 8 + 2 * i + 1) * LDB + st_t] = (u16)(qw[i] >> 16);
+            }
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f;
+#pragma unroll
+            for (int it = 0; it < 2; it++) {
+                const int c4 = (fg0 + 8 * it) * 4, off = ft * LDB + c4;
+                bf16_store(dYr, off, ndY[it]);
+                split_store(M0h, M0l, off, nM0[it]);
+                bf16_store(dMr, off, ndM[it]);
+                if (HAS_S) bf16_store(dSr, off, ndS[it]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int toff = (c4 + i) * LDB + ft;
+                    reinterpret_cast<__bf16 *>(dYt)[toff] = (__bf16)ndY[it][i];
+                    reinterpret_cast<__bf16 *>(M0t)[toff] = (__bf16)nM0[it][i];
+                    reinterpret_cast<__bf16 *>(dMt)[toff] = (__bf16)ndM[it][i];
+                    if (HAS_S) {
+                        reinterpret_cast<__bf16 *>(S0t)[toff] = (__bf16)nS0[it][i];
+                        reinterpret_cast<__bf16 *>(dSt)[toff] = (__bf16)ndS[it][i];
+                    }
+                    d0 = fmaf(nM0[it][i], ndM[it][i], d0);
+                    if (HAS_S) { d1 = fmaf(nS0[it][i], ndM[it][i], d1); d2 = fmaf(nS0[it][i], ndS[it][i], d2); }
+                }
+            }
+            d0 = sum_wave(d0); d1 = sum_wave(d1); d2 = sum_wave(d2);
+            if (l == 0) { dots[w] = d0; dots[8 + w] = d1; dots[16 + w] = d2; }
+            if (tid < 5 * CW) cvec[tid] = nvec;
+        }
+        __syncthreads();
+        touch(min(task + 1, task_hi - 1));
+
+        // ── P, E^T (group A); dQ^T = a.(M0^T dY^T) + beta.(S0^T dY^T), p0, ps (group B) ──
+        f32x4 keep[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};   // group A: P [t][j]; group B: dQ^T [c][t]
+        if (grpA) {
+            f32x4 e[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                bf16x8 bK[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) bK[ct] = ld_op(Kr, bn + 16 * ct, ks);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const bf16x8 aq = ld_op(Qr, bm + 16 * rt, ks);
+                    const bf16x8 mh = ld_op(M0h, bm + 16 * rt, ks), ml = ld_op(M0l, bm + 16 * rt, ks);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) {
+                        keep[rt][ct] = mfma32(aq, bK[ct], keep[rt][ct]);   // P[t][j]
+                        e[rt][ct] = mfma32(mh, bK[ct], e[rt][ct]);         // E^T[i][t]
+                        e[rt][ct] = mfma32(ml, bK[ct], e[rt][ct]);
+                    }
+                }
+            }
+            // -identity operand of E^T = M0 K^T - V^T: rows i = bm + 16 rt + l%16 meet contraction
+            // indices 32 (bm/32) + 8 (l/16) + e
+            bf16x8 negI[2];
+#pragma unroll
+            for (int rt = 0; rt < 2; rt++) {
+                const int hit = 16 * rt + r16 - 8 * g;
+                uint4 bits;
+                bits.x = (hit == 0 ? 0xBF80u : 0u) | (hit == 1 ? 0xBF800000u : 0u);
+                bits.y = (hit == 2 ? 0xBF80u : 0u) | (hit == 3 ? 0xBF800000u : 0u);
+                bits.z = (hit == 4 ? 0xBF80u : 0u) | (hit == 5 ? 0xBF800000u : 0u);
+                bits.w = (hit == 6 ? 0xBF80u : 0u) | (hit == 7 ? 0xBF800000u : 0u);
+                negI[rt] = __builtin_bit_cast(bf16x8, bits);
+            }
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                const bf16x8 bv = ld_op(Vr, bn + 16 * ct, bm >> 5);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    e[rt][ct] = mfma32(negI[rt], bv, e[rt][ct]);
+                    bf16_store(Er, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g, e[rt][ct]);   // E[t][i .. i+3]
+                }
+            }
+        } else {
+            // one product at a time: its row sums and its share of dQ^T, then the accumulators are free
+            auto half = [&](const u16 *St, int which, int voff) {
+                f32x4 ym[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    bf16x8 bD[2];
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) bD[ct] = ld_op(dYr, bn + 16 * ct, ks);
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++) {
+                        const bf16x8 am = ld_op(St, bm + 16 * rt, ks);
+#pragma unroll
+                        for (int ct = 0; ct < 2; ct++) ym[rt][ct] = mfma32(am, bD[ct], ym[rt][ct]);   // [c][t]
+                    }
+                }
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) {
+                    const int t = bn + 16 * ct + r16;
+                    const float at = cvec[voff + t];
+                    float p0 = 0.f;
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++) {
+                        const f32x4 qv = bf4_to_f32(Qr + t * LDB + bm + 16 * rt + 4 * g);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) p0 = fmaf(ym[rt][ct][r], qv[r], p0);
+                        keep[rt][ct] += at * ym[rt][ct];
+                    }
+                    p0 = sum_groups(p0);
+                    if (g == 0) part[(which * 2 + (bi >> 1)) * CW + t] = p0;
+                }
+            };
+            half(M0t, 0, 0);
+            if (HAS_S) {
+                half(S0t, 1, CW);
+            } else {
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++)
+                    if (g == 0) part[(1 * 2 + (bi >> 1)) * CW + bn + 16 * ct + r16] = 0.f;
+            }
+        }
+        __syncthreads();
+
+        // ── R = dY E^T: X, (c.P)^T, (c.R)^T (group A); R^T: -theta c.R (group B) ──
+        {
+            f32x4 rr[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+            const u16 *Am = grpA ? dYr : Er, *Bm = grpA ? Er : dYr;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                bf16x8 bb[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) bb[ct] = ld_op(Bm, bn + 16 * ct, ks);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const bf16x8 aa = ld_op(Am, bm + 16 * rt, ks);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) rr[rt][ct] = mfma32(aa, bb[ct], rr[rt][ct]);
+                }
+            }
+            if (grpA) {   // rr = R[t][j] at the positions of P
+                float *xo = xs + (size_t)task * kTab;
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) {
+                        *reinterpret_cast<f32x4 *>(xo + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4) = rr[rt][ct] * keep[rt][ct];
+                        const int off = (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g;   // [j][t .. t+3]
+                        bf16_store(CPt, off, ntab[rt][ct] * keep[rt][ct]);
+                        bf16_store(CRt, off, ntab[rt][ct] * rr[rt][ct]);
+                    }
+            } else {      // rr = R^T[j][t]
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const f32x4 th = *reinterpret_cast<const f32x4 *>(cvec + 4 * CW + bm + 16 * rt + 4 * g);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++)   // [t][j .. j+3]
+                        bf16_store(ThCR, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g,
+                                   -(th * ntab[rt][ct] * rr[rt][ct]));
+                }
+            }
+        }
+        __syncthreads();
+
+        f32x4 dte[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};   // group B: DTe^T [c][j] (theta applied later)
+        if (grpA) {
+            // ── Dk^T [i][j] = dY^T (c.P) + cl.(dMo K^T) + bl.(dSo K^T); dE, dV, d_theta ──
+            f32x4 dk[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+            auto state_term = [&](const u16 *Ar, int voff) {   // dk += cvec[voff + j] . (Ar K^T)
+                f32x4 t1[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    bf16x8 bK[2];
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) bK[ct] = ld_op(Kr, bn + 16 * ct, ks);
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++) {
+                        const bf16x8 am = ld_op(Ar, bm + 16 * rt, ks);
+#pragma unroll
+                        for (int ct = 0; ct < 2; ct++) t1[rt][ct] = mfma32(am, bK[ct], t1[rt][ct]);
+                    }
+                }
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) {
+                    const float cj = cvec[voff + bn + 16 * ct + r16];
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++) dk[rt][ct] += cj * t1[rt][ct];
+                }
+            };
+            state_term(dMr, 2 * CW);
+            if (HAS_S) state_term(dSr, 3 * CW);
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                bf16x8 bP[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) bP[ct] = ld_op(CPt, bn + 16 * ct, ks);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const bf16x8 ay = ld_op(dYt, bm + 16 * rt, ks);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) dk[rt][ct] = mfma32(ay, bP[ct], dk[rt][ct]);
+                }
+            }
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                const int j = bn + 16 * ct + r16;
+                const float thj = cvec[4 * CW + j];
+                float rs = 0.f;
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const f32x4 x = dk[rt][ct];                                              // Dk[j][i .. i+3]
+                    const f32x4 ev = bf4_to_f32(Er + j * LDB + bm + 16 * rt + 4 * g);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) rs = fmaf(ev[r], x[r], rs);
+                    dk[rt][ct] = thj * x;                                                    // dV = theta_j Dk = -dE
+                }
+                rs = sum_groups(rs);
+                if (g == 0) part[(2 * 2 + (bi >> 1)) * CW + j] = rs;
+            }
+            // S0^T was last read two barriers ago: dE may take its place now
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                const int j = bn + 16 * ct + r16;
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    bf16_store(dEr, j * LDB + bm + 16 * rt + 4 * g, -dk[rt][ct]);
+                    if (j < L) *reinterpret_cast<f32x4 *>(d_v + (tok + j) * HD + bm + 16 * rt + 4 * g) = dk[rt][ct];
+                }
+            }
+        } else {
+            // ── dQ^T += K^T (-theta c.R)^T; DTe^T [c][j] = Q^T (c.R) + cl.(dMo^T E^T) + bl.(dSo^T E^T); g1, g2 ──
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                bf16x8 bT[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) bT[ct] = ld_op(ThCR, bn + 16 * ct, ks);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const bf16x8 ak = ld_op(Kt, bm + 16 * rt, ks);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) keep[rt][ct] = mfma32(ak, bT[ct], keep[rt][ct]);
+                }
+            }
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                const int t = bn + 16 * ct + r16;
+                if (t < L) {
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++)
+                        *reinterpret_cast<f32x4 *>(d_q + (tok + t) * HD + bm + 16 * rt + 4 * g) = keep[rt][ct];
+                }
+            }
+            auto state_term = [&](const u16 *At, int which, int voff) {   // dte += cvec[voff + j] . (At E^T); g sums
+                f32x4 t3[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    bf16x8 bE[2];
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) bE[ct] = ld_op(Er, bn + 16 * ct, ks);
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++) {
+                        const bf16x8 am = ld_op(At, bm + 16 * rt, ks);
+#pragma unroll
+                        for (int ct = 0; ct < 2; ct++) t3[rt][ct] = mfma32(am, bE[ct], t3[rt][ct]);
+                    }
+                }
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) {
+                    const int j = bn + 16 * ct + r16;
+                    const float cj = cvec[voff + j];
+                    float g1 = 0.f;
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++) {
+                        const f32x4 kv = bf4_to_f32(Kr + j * LDB + bm + 16 * rt + 4 * g);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) g1 = fmaf(t3[rt][ct][r], kv[r], g1);
+                        dte[rt][ct] += cj * t3[rt][ct];
+                    }
+                    g1 = sum_groups(g1);
+                    if (g == 0) part[(which * 2 + (bi >> 1)) * CW + j] = g1;
+                }
+            };
+            state_term(dMt, 3, 2 * CW);
+            if (HAS_S) {
+                state_term(dSt, 4, 3 * CW);
+            } else {
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++)
+                    if (g == 0) part[(4 * 2 + (bi >> 1)) * CW + bn + 16 * ct + r16] = 0.f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                bf16x8 bC[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) bC[ct] = ld_op(CRt, bn + 16 * ct, ks);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const bf16x8 aq = ld_op(Qt, bm + 16 * rt, ks);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) dte[rt][ct] = mfma32(aq, bC[ct], dte[rt][ct]);
+                }
+            }
+        }
+        fetch_tab(min(task + 1, task_hi - 1));   // the table registers are free since the second phase
+        __syncthreads();       // dE complete
+
+        if (!grpA) {
+            // ── dK^T [c][j] = -theta_j DTe^T + M0^T dE^T ──
+            f32x4 em[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                bf16x8 bE[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) bE[ct] = ld_op(dEr, bn + 16 * ct, ks);
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++) {
+                    const bf16x8 am = ld_op(M0t, bm + 16 * rt, ks);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) em[rt][ct] = mfma32(am, bE[ct], em[rt][ct]);
+                }
+            }
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                const int j = bn + 16 * ct + r16;
+                const float thj = cvec[4 * CW + j];
+                if (j < L) {
+#pragma unroll
+                    for (int rt = 0; rt < 2; rt++)
+                        *reinterpret_cast<f32x4 *>(d_k + (tok + j) * HD + bm + 16 * rt + 4 * g) =
+                            em[rt][ct] - thj * dte[rt][ct];
+                }
+            }
+        } else if (tid < L) {
+            const int t = tid;
+            d_theta[tok + t] = -(part[(2 * 2) * CW + t] + part[(2 * 2 + 1) * CW + t]);
+            *reinterpret_cast<f32x4 *>(pvec + (tok + t) * 4) =
+                f32x4{part[t] + part[CW + t], part[2 * CW + t] + part[3 * CW + t],
+                      part[6 * CW + t] + part[7 * CW + t], part[8 * CW + t] + part[9 * CW + t]};
+        } else if (tid >= 64 && tid < 67) {
+            const float *p = dots + 8 * (tid - 64);
+            scal[(size_t)task * 4 + (tid - 64)] = p[0] + p[1] + p[2] + p[3] + p[4] + p[5] + p[6] + p[7];
+        }
+        __syncthreads();   // LDS is rewritten by the next task
+    }
+}
+
+constexpr size_t kGradsLds = 16 * BMAT * sizeof(u16) + (5 * CW + 10 * CW + 24) * sizeof(float);
+
+}  // namespace
+
+size_t chunkwise_grads_table_floats() { return kTab; }
+size_t chunkwise_grads_vec_floats() { return kVecB; }
+
+bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
+                          const float *alpha, const float *theta, const float *eta, const float *m_states,
+                          const float *s_states, const float *dm_states, const float *ds_states, float *d_k,
+                          float *d_v, float *d_q, float *d_theta, float *pvec, float *xs, float *scal,
+                          float *tab_a, float *tab_b, float *vecs, int seq_len, int batch, int chunk_size,
+                          bool has_s, int grid) {
+    const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
+    static bool attr_set = false;
+    if (!attr_set) {
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_grads_bf16_kernel<true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_grads_bf16_kernel<false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
+        attr_set = true;
+    }
+    if (failed()) return true;
+    if (has_s) {
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
+                           eta, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
+        check_launch("cw_coef_bwd_kernel");
+        KernelTimer kt("cw_grads_bf16_kernel");
+        hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
+                           tab_a, tab_b, vecs, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec,
+                           xs, scal, seq_len, chunk_size, nc, ntask);
+        check_launch("cw_grads_bf16_kernel");
+    } else {
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
+                           nullptr, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
+        check_launch("cw_coef_bwd_kernel");
+        KernelTimer kt("cw_grads_bf16_kernel");
+        hipLaunchKernelGGL(cw_grads_bf16_kernel<false>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
+                           tab_a, tab_b, vecs, m_states, nullptr, dm_states, nullptr, d_k, d_v, d_q, d_theta, pvec,
+                           xs, scal, seq_len, chunk_size, nc, ntask);
+        check_launch("cw_grads_bf16_kernel");
+    }
+    return true;
+}
+
+}  // namespace nlh

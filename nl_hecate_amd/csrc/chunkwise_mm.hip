@@ -30,6 +30,7 @@
 
 #include "../../include/nl_hecate_ffi.h"
 #include "chunkwise_chain.h"
+#include "chunkwise_grads.h"
 #include "rule_common.h"
 #include "runtime.h"
 
@@ -759,7 +760,7 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
                                                             const float *__restrict__ xs,
                                                             const float *__restrict__ scal,
                                                             float *__restrict__ d_alpha, float *__restrict__ d_eta,
-                                                            int s, int C, int nc, int has_s) {
+                                                            int s, int C, int nc, int has_s, int xs_tiled) {
     extern __shared__ float smem[];
     float *Xs = smem, *Cc = Xs + MAT, *Bb = Cc + MAT, *Rr = Bb + MAT;
     __shared__ Coef cf;
@@ -767,6 +768,8 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     __shared__ float part[2][2][CW];
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
+    // xs is row-major [t][j], or (xs_tiled) in the accumulator-tile order of the bf16 pass:
+    // [block bi][rt][ct][lane][r] holds X[32 (bi/2) + 16 rt + 4 (lane/16) + r][32 (bi%2) + 16 ct + lane%16]
     Tile<float> tx;
     fetch(tx, xs + ((size_t)chain * nc + ci) * CW * CW, 64);
     const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
@@ -779,7 +782,17 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
     const float m0dm = scal[((size_t)chain * nc + ci) * 4 + 0], s0dm = scal[((size_t)chain * nc + ci) * 4 + 1],
                 s0ds = scal[((size_t)chain * nc + ci) * 4 + 2];
     coefficients(cf, gt, L, Cc, Bb, Rr);
-    commit(Xs, tx);
+    if (xs_tiled) {
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int qd = it * kThr + threadIdx.x, ln = qd & 63, ct = (qd >> 6) & 1, rt = (qd >> 7) & 1, bi = qd >> 8;
+            const int t = 32 * (bi >> 1) + 16 * rt + 4 * (ln >> 4), j = 32 * (bi & 1) + 16 * ct + (ln & 15);
+            Xs[t * LDM + j] = tx.x[it].x; Xs[(t + 1) * LDM + j] = tx.x[it].y;
+            Xs[(t + 2) * LDM + j] = tx.x[it].z; Xs[(t + 3) * LDM + j] = tx.x[it].w;
+        }
+    } else {
+        commit(Xs, tx);
+    }
     __syncthreads();
     if (threadIdx.x >= kThr - CW) {   // mat-vecs with W and Ws (last wave; the matrix products start meanwhile)
         const int tau = threadIdx.x - (kThr - CW);
@@ -954,10 +967,21 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr, sc.loc,
                        sc.locs, dm_states, ds_states, nc, (int)has_s);
     check_launch("cw_scan_kernel");
-    hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(256), 0, stream(), m_states, s_states,
-                       dm_states, ds_states, scal, nc, (int)has_s);
-    check_launch("cw_state_dots_kernel");
-    {
+    int xs_tiled = 0;
+    if constexpr (sizeof(TIn) == 2) {
+        const size_t nchunks = (size_t)batch * nc;
+        float *tab_a = scratch(12, nchunks * chunkwise_grads_table_floats() * sizeof(float));
+        float *tab_b = scratch(13, nchunks * chunkwise_grads_table_floats() * sizeof(float));
+        float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
+        if (failed()) return;
+        chunkwise_grads_bf16(k, v, q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q,
+                             d_theta, pvec, xs, scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
+                             persistent_grid(batch * nc));
+        xs_tiled = 1;
+    } else {
+        hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(256), 0, stream(), m_states, s_states,
+                           dm_states, ds_states, scal, nc, (int)has_s);
+        check_launch("cw_state_dots_kernel");
         KernelTimer kt("cw_grads_bwd_kernel");
         hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kGradsBwdLds,
                            stream(), k, v, q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k,
@@ -965,7 +989,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         check_launch("cw_grads_bwd_kernel");
     }
     hipLaunchKernelGGL(cw_gates_bwd_kernel, dim3(batch * nc), dim3(kThr), kGatesBwdLds, stream(), alpha, theta, eta,
-                       pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size, nc, (int)has_s);
+                       pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size, nc, (int)has_s, xs_tiled);
     check_launch("cw_gates_bwd_kernel");
     const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
     const int per = 8, rows = ceil_div(batch, per);

@@ -21,7 +21,7 @@ hipStream_t stream();   // launch stream (the null stream unless nlh_set_stream 
 // nlh_release_workspace().  Slots let one entry point hold several buffers.
 // Work on the launch stream is ordered, so reuse across calls is safe.
 float *scratch(int slot, size_t bytes);
-constexpr int kScratchSlots = 12;
+constexpr int kScratchSlots = 16;
 
 // Optional per-kernel timing: while enabled (nlh_kernel_timer_enable), a
 // KernelTimer around a launch records an event pair on the launch stream;

@@ -1,8 +1,10 @@
 """GPU parity of the matrix-form (matrix-core) chunkwise Titans rule against the CPU
 oracle of the frozen-M0 chunkwise rule.  Inputs k, v, q are bf16 (or float); the oracle
 runs in float32 on the same (bf16-rounded) values.  Stated tolerance for bf16-input /
-fp32-accumulate paths is relative 2e-2; the arithmetic here is fp32 throughout, so the
-tests hold the results to 1e-3 (bf16 inputs) and 1e-4 (float inputs)."""
+fp32-accumulate paths is relative 2e-2.  The bf16 forward carries every fp32 operand as a
+hi + lo bf16 pair and is held to 1e-3; the bf16 backward feeds its fp32 operands to the
+matrix cores as single bf16 values (fp32 accumulation) and is held to 1e-2; the float
+entry points compute in fp32 throughout and are held to 1e-4 / 2e-4."""
 import numpy as np
 import pytest
 import torch
@@ -92,7 +94,7 @@ def test_backward_matches_oracle(B, s, C, bf16):
            g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], g["d_m_initial"],
            g["d_s_initial"], s, d, B, C)
     torch.cuda.synchronize()
-    tol = 1e-3 if bf16 else 2e-4
+    tol = 1e-2 if bf16 else 2e-4
     for n in g:
         assert_close(n, host(g[n]), want[n], tol)
 
@@ -135,7 +137,7 @@ def test_matrix_form_agrees_with_sequential_kernels_at_benchmark_shape():
     assert_close("y", host(f["y"]), host(y), 1e-3)
     assert_close("m_chunk_states", host(f["mc"]), host(mc), 1e-3)
     for n in g1:
-        assert_close(n, host(g2[n]), host(g1[n]), 1e-3)
+        assert_close(n, host(g2[n]), host(g1[n]), 1e-2)
 
 
 @pytest.mark.parametrize("B,s,C", [(2, 128, 64), (3, 200, 64), (2, 50, 16)])
@@ -164,6 +166,7 @@ def test_delta_matrix_form_matches_oracle(B, s, C, bf16):
     tol = 1e-3 if bf16 else 2e-4
     assert_close("y", host(y), np.stack([f[0] for f in fw]), tol)
     assert_close("m_chunk_states", host(mc), np.stack([f[1] for f in fw]), tol)
+    tol = 1e-2 if bf16 else 2e-4
     for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta"):
         assert_close(n, host(g[n]), np.stack([o[n] for o in bw]), tol)
     assert_close("d_m_initial", host(g["d_m"]), sum(o["d_m"] for o in bw), tol)
