@@ -1,0 +1,225 @@
+// Backward of the frozen-M0 chunkwise Titans / Delta rule on bf16 tokens: the adjoint scan.
+//
+// dMo, dSo are the adjoints of a chunk's end state; walking the chunks of a chain backwards,
+//   dE  = (W.P)^T dY + wM.(K dMo^T) + wS.(K dSo^T)          [token j][row i]
+//   dM0 = a_L dMo + (a.dY)^T Q + dE^T K
+//   dS0 = beta_L dMo + h_L dSo + (beta.dY)^T Q
+// with P = Q K^T, W[t][j] = -theta_j c[t][j], wM_j = -theta_j c[L-1][j], wS_j = -theta_j bb[j][L-1]
+// (the adjoint of the chunk map of chunkwise_mm.hip, written without its 64x64 transfer
+// matrices).  The rows of dM, dS never mix, so a chain is split over two workgroups of 32 rows
+// each; each walks all chunks with its rows of dM and dS in registers (fp32) and, as bf16
+// hi + lo pairs, in LDS as operands of the next step.  HBM sees k, q, dY and the coefficient
+// table once per step and receives one adjoint snapshot per chunk: dm_states[chain][c] is the
+// adjoint of the state at the start of chunk c (slot num_chunks = 0).
+//
+// Every fp32 operand enters the bf16 matrix cores as a hi + lo pair: this path is recurrent.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "bf16_tiles.h"
+#include "chunkwise_grads.h"
+#include "runtime.h"
+
+namespace nlh {
+namespace {
+
+constexpr int HMAT = 32 * LDB;   // elements of a 32-row bf16 matrix
+
+template <bool HAS_S>
+__global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
+    const u16 *__restrict__ k, const u16 *__restrict__ q, const float *__restrict__ d_y,
+    const float *__restrict__ tab_b, const float *__restrict__ vecs, float *__restrict__ dm_states,
+    float *__restrict__ ds_states, int s, int C, int nc, int batch, int tab_floats, int vec_floats) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Kt = Kr + BMAT;   // K [j][c], K^T [c][j]
+    u16 *Qr = Kt + BMAT, *Qt = Qr + BMAT;                            // Q [t][c], Q^T [c][t]
+    u16 *WPh = Qt + BMAT, *WPl = WPh + BMAT;                         // (W.P)^T [j][t]
+    u16 *dYh = WPl + BMAT, *dYl = dYh + HMAT;                        // dY^T [i][t] (this workgroup's 32 rows i)
+    u16 *dYah = dYl + HMAT, *dYal = dYah + HMAT;                     // (a.dY)^T
+    u16 *dYbh = dYal + HMAT, *dYbl = dYbh + HMAT;                    // (beta.dY)^T
+    u16 *dMh = dYbl + HMAT, *dMl = dMh + HMAT;                       // dMo [i][c]
+    u16 *dSh = dMl + HMAT, *dSl = dSh + HMAT;                        // dSo [i][c]
+    u16 *dEh = dSl + HMAT, *dEl = dEh + HMAT;                        // dE^T [i][j]
+    float *cvec = reinterpret_cast<float *>(dEl + HMAT);             // a, beta, cl, bl, theta [64] each, .., h_L
+
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
+    const int chain = blockIdx.x % batch, half = blockIdx.x / batch, i0 = 32 * half;
+    const size_t chain_tok = (size_t)chain * s, state0 = (size_t)chain * (nc + 1) * HD * HD;
+    const int st_t = 16 * (w & 3) + (l & 15), st_cb = 4 * (w >> 2) + (l >> 4);   // bf16 tile: row, 8-element block
+    const int yt = tid >> 3, yg = tid & 7;                                        // dY tile: row t, 4-element block
+
+    // zero what is never written again: tiles of (W.P)^T above the diagonal
+    for (int e = tid; e < BMAT / 2; e += kTileThr) {
+        reinterpret_cast<unsigned *>(WPh)[e] = 0u;
+        reinterpret_cast<unsigned *>(WPl)[e] = 0u;
+    }
+
+    // registers of the next step (chunk c - 1)
+    uint4 nK, nQ;
+    f32x4 ndY, ntab[2];
+    float na = 0.f, nb = 0.f, nvec = 0.f;
+    const int tt = w >> 1, jt0 = 2 * (w & 1);   // phase A: P tiles (tt, jt0) and (tt, jt0 + 1)
+    auto fetch = [&](int c) {
+        const int L = min(C, s - c * C);
+        const size_t tok = chain_tok + (size_t)c * C;
+        const size_t row = tok + min(st_t, L - 1);
+        nK = *reinterpret_cast<const uint4 *>(k + row * HD + st_cb * 8);
+        nQ = *reinterpret_cast<const uint4 *>(q + row * HD + st_cb * 8);
+        ndY = *reinterpret_cast<const f32x4 *>(d_y + (tok + min(yt, L - 1)) * HD + i0 + yg * 4);
+        const size_t chunk = (size_t)chain * nc + c;
+        const float *vo = vecs + chunk * vec_floats, *tb = tab_b + chunk * tab_floats;
+        na = vo[yt];
+        nb = vo[CW + yt];
+        nvec = vo[min(tid, 5 * CW + 7)];
+#pragma unroll
+        for (int x = 0; x < 2; x++) {
+            const int jt = jt0 + x, bi = 2 * (tt >> 1) + (jt >> 1);
+            ntab[x] = *reinterpret_cast<const f32x4 *>(
+                jt <= tt ? tb + (((bi * 2 + (tt & 1)) * 2 + (jt & 1)) * 64 + l) * 4 : vo + 5 * CW);
+        }
+    };
+    f32x4 ctab[2];
+    auto commit = [&](int c) {
+        const int L = min(C, s - c * C);
+        if (st_t >= L) { nK = make_uint4(0, 0, 0, 0); nQ = nK; }
+        if (yt >= L) ndY = zero4();
+        *reinterpret_cast<uint4 *>(Kr + st_t * LDB + st_cb * 8) = nK;
+        *reinterpret_cast<uint4 *>(Qr + st_t * LDB + st_cb * 8) = nQ;
+        const unsigned kw[4] = {nK.x, nK.y, nK.z, nK.w}, qw[4] = {nQ.x, nQ.y, nQ.z, nQ.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            Kt[(st_cb * 8 + 2 * e) * LDB + st_t] = (u16)(kw[e] & 0xffffu);
+            Kt[(st_cb * 8 + 2 * e + 1) * LDB + st_t] = (u16)(kw[e] >> 16);
+            Qt[(st_cb * 8 + 2 * e) * LDB + st_t] = (u16)(qw[e] & 0xffffu);
+            Qt[(st_cb * 8 + 2 * e + 1) * LDB + st_t] = (u16)(qw[e] >> 16);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int off = (yg * 4 + e) * LDB + yt;
+            auto put = [&](u16 *H, u16 *Lo, float x) {
+                const __bf16 hb = (__bf16)x;
+                reinterpret_cast<__bf16 *>(H)[off] = hb;
+                reinterpret_cast<__bf16 *>(Lo)[off] = (__bf16)(x - (float)hb);
+            };
+            put(dYh, dYl, ndY[e]);
+            put(dYah, dYal, na * ndY[e]);
+            if (HAS_S) put(dYbh, dYbl, nb * ndY[e]);
+        }
+        if (tid < 5 * CW + 8) cvec[tid] = nvec;
+        ctab[0] = ntab[0];
+        ctab[1] = ntab[1];
+    };
+
+    // fp32 master: transposed tile rows c = 16 (w/2) + 4 (l/16) + r, column i = 16 (w%2) + l%16
+    const int rt = w >> 1, ct = w & 1;
+    f32x4 dM = zero4(), dS = zero4();
+    auto publish = [&](int slot) {
+        const size_t o = state0 + (size_t)slot * HD * HD + (i0 + 16 * ct + r16) * HD + 16 * rt + 4 * g;
+        *reinterpret_cast<f32x4 *>(dm_states + o) = dM;
+        if (HAS_S) *reinterpret_cast<f32x4 *>(ds_states + o) = dS;
+        const int off = (16 * ct + r16) * LDB + 16 * rt + 4 * g;
+        split_store(dMh, dMl, off, dM);
+        if (HAS_S) split_store(dSh, dSl, off, dS);
+    };
+
+    fetch(nc - 1);
+    publish(nc);
+    for (int c = nc - 1; c >= 0; c--) {
+        const int L = min(C, s - c * C);
+        commit(c);
+        __syncthreads();
+        fetch(max(c - 1, 0));
+        // ── (W.P)^T: this wave's two tiles of P[t][j] ──
+        {
+            const bf16x8 aq[2] = {ld_op(Qr, 16 * tt, 0), ld_op(Qr, 16 * tt, 1)};
+#pragma unroll
+            for (int x = 0; x < 2; x++) {
+                const int jt = jt0 + x;
+                if (jt <= tt) {
+                    f32x4 p = zero4();
+#pragma unroll
+                    for (int ks = 0; ks < 2; ks++) p = mfma32(aq[ks], ld_op(Kr, 16 * jt, ks), p);
+                    const float nth = -cvec[4 * CW + 16 * jt + r16];
+                    split_store(WPh, WPl, (16 * jt + r16) * LDB + 16 * tt + 4 * g, nth * ctab[x] * p);   // [j][t .. t+3]
+                }
+            }
+        }
+        __syncthreads();
+        // ── dE[j][i]: tile rows j = 16 rt.., columns i = 16 ct.. ──
+        {
+            f32x4 e1 = zero4(), e2 = zero4(), e3 = zero4();
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const bf16x8 wh = ld_op(WPh, 16 * rt, ks), wl = ld_op(WPl, 16 * rt, ks), ak = ld_op(Kr, 16 * rt, ks);
+                const bf16x8 yh = ld_op(dYh, 16 * ct, ks), yl = ld_op(dYl, 16 * ct, ks);
+                e1 = mfma32(wh, yh, e1);
+                e1 = mfma32(wl, yh, e1);
+                e1 = mfma32(wh, yl, e1);
+                e2 = mfma32(ak, ld_op(dMh, 16 * ct, ks), e2);
+                e2 = mfma32(ak, ld_op(dMl, 16 * ct, ks), e2);
+                if (HAS_S) {
+                    e3 = mfma32(ak, ld_op(dSh, 16 * ct, ks), e3);
+                    e3 = mfma32(ak, ld_op(dSl, 16 * ct, ks), e3);
+                }
+            }
+            const int j4 = 16 * rt + 4 * g;
+            const f32x4 th = *reinterpret_cast<const f32x4 *>(cvec + 4 * CW + j4);
+            const f32x4 cl = *reinterpret_cast<const f32x4 *>(cvec + 2 * CW + j4);
+            const f32x4 bl = *reinterpret_cast<const f32x4 *>(cvec + 3 * CW + j4);
+            split_store(dEh, dEl, (16 * ct + r16) * LDB + j4, e1 - th * (cl * e2 + bl * e3));   // [i][j .. j+3]
+        }
+        __syncthreads();
+        // ── dM0^T, dS0^T: tile rows c = 16 rt.., columns i = 16 ct.. ──
+        {
+            f32x4 am = zero4(), as = zero4();
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const bf16x8 aq = ld_op(Qt, 16 * rt, ks), ak = ld_op(Kt, 16 * rt, ks);
+                am = mfma32(aq, ld_op(dYah, 16 * ct, ks), am);
+                am = mfma32(aq, ld_op(dYal, 16 * ct, ks), am);
+                am = mfma32(ak, ld_op(dEh, 16 * ct, ks), am);
+                am = mfma32(ak, ld_op(dEl, 16 * ct, ks), am);
+                if (HAS_S) {
+                    as = mfma32(aq, ld_op(dYbh, 16 * ct, ks), as);
+                    as = mfma32(aq, ld_op(dYbl, 16 * ct, ks), as);
+                }
+            }
+            const float aL = cvec[L - 1], betaL = cvec[CW + L - 1], hL = cvec[5 * CW + 4];
+            const f32x4 dMn = aL * dM + am;
+            if (HAS_S) dS = betaL * dM + hL * dS + as;
+            dM = dMn;
+        }
+        publish(c);
+        __syncthreads();
+    }
+}
+
+constexpr size_t kAdjointLds = (6 * BMAT + 12 * HMAT) * sizeof(u16) + (5 * CW + 8) * sizeof(float);
+
+}  // namespace
+
+bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
+                            const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
+                            int chunk_size, bool has_s) {
+    const int nc = ceil_div(seq_len, chunk_size);
+    static bool attr_set = false;
+    if (!attr_set) {
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_adjoint_chain_kernel<true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAdjointLds), "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_adjoint_chain_kernel<false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAdjointLds), "dynamic LDS size");
+        attr_set = true;
+    }
+    if (failed()) return true;
+    const int tabf = (int)chunkwise_grads_table_floats(), vecf = (int)chunkwise_grads_vec_floats();
+    if (has_s)
+        hipLaunchKernelGGL(cw_adjoint_chain_kernel<true>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
+                           d_y, tab_b, vecs, dm_states, ds_states, seq_len, chunk_size, nc, batch, tabf, vecf);
+    else
+        hipLaunchKernelGGL(cw_adjoint_chain_kernel<false>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
+                           d_y, tab_b, vecs, dm_states, nullptr, seq_len, chunk_size, nc, batch, tabf, vecf);
+    check_launch("cw_adjoint_chain_kernel");
+    return true;
+}
+
+}  // namespace nlh

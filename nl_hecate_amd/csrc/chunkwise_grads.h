@@ -1,7 +1,11 @@
-// Per-chunk gradient pass of the chunkwise rule on bf16 tokens (head size 64, chunks of up
-// to 64 tokens): d_q, d_k, d_v, d_theta, and for the gate pass pvec [token][4], xs
-// [chunk][64*64] in accumulator-tile order, scal [chunk][4].  tab_a, tab_b (table_floats per
-// chunk) and vecs (vec_floats per chunk) are scratch the pass fills itself.
+// Backward of the chunkwise rule on bf16 tokens (head size 64, chunks of up to 64 tokens), three
+// launches on the library's stream:
+//   chunkwise_backward_coefficients: per-chunk coefficient tables tab_a, tab_b (table_floats per
+//     chunk) and vectors vecs (vec_floats per chunk) from the gates
+//   chunkwise_adjoint_bf16: the adjoint scan; dm_states / ds_states [batch][num_chunks + 1][64*64],
+//     slot c = adjoint of the state at the start of chunk c
+//   chunkwise_grads_bf16: d_q, d_k, d_v, d_theta, and for the gate pass pvec [token][4], xs
+//     [chunk][64*64] in accumulator-tile order, scal [chunk][4]
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -11,11 +15,17 @@ namespace nlh {
 size_t chunkwise_grads_table_floats();
 size_t chunkwise_grads_vec_floats();
 
+void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta, float *tab_a,
+                                     float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s);
+
+bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
+                            const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
+                            int chunk_size, bool has_s);
+
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
-                          const float *alpha, const float *theta, const float *eta, const float *m_states,
-                          const float *s_states, const float *dm_states, const float *ds_states, float *d_k,
-                          float *d_v, float *d_q, float *d_theta, float *pvec, float *xs, float *scal,
-                          float *tab_a, float *tab_b, float *vecs, int seq_len, int batch, int chunk_size,
-                          bool has_s, int grid);
+                          const float *m_states, const float *s_states, const float *dm_states,
+                          const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
+                          float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
+                          int seq_len, int batch, int chunk_size, bool has_s, int grid);
 
 }  // namespace nlh

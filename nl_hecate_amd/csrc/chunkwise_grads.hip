@@ -40,7 +40,7 @@ namespace {
 //   tab_a [chunk][block bi][rt][ct][lane l][r]: c[t][j] (zero outside j <= t < L) at
 //         j = 32 (bi/2) + 16 rt + 4 (l/16) + r, t = 32 (bi%2) + 16 ct + l%16   (group B: R^T)
 //   tab_b same for t = 32 (bi/2) + 16 rt + 4 (l/16) + r, j = 32 (bi%2) + 16 ct + l%16  (group A: P, R)
-//   vecs  [chunk][kVecB]: a_t, beta_t, cl_j, bl_j, theta_j, then four zeros
+//   vecs  [chunk][kVecB]: a_t, beta_t, cl_j, bl_j, theta_j, then four zeros and h_L
 // Tiles entirely above the diagonal are neither written nor read.
 constexpr int kTab = CW * CW;
 constexpr int kVecB = 5 * CW + 16;
@@ -83,18 +83,19 @@ __global__ __launch_bounds__(256) void cw_coef_bwd_kernel(const float *__restric
         vo[3 * CW + j] = jv ? blv : 0.f;
         vo[4 * CW + j] = g.th;
     } else {
-        float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f;
+        float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f, kh = 0.f;
 #pragma unroll
         for (int t = 0; t < CW; t++) {
             const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
             a *= keep;
             h *= et;
             beta = fmaf(keep, beta, h);
-            if (t == j) { ka = a; kb = beta; }
+            if (t == j) { ka = a; kb = beta; kh = h; }
         }
         vo[j] = j < L ? ka : 0.f;
         vo[CW + j] = j < L ? kb : 0.f;
         if (j < 4) vo[5 * CW + j] = 0.f;   // what tiles above the diagonal read
+        if (j == L - 1) vo[5 * CW + 4] = kh;
     }
 }
 
@@ -578,12 +579,23 @@ constexpr size_t kGradsLds = 16 * BMAT * sizeof(u16) + (5 * CW + 10 * CW + 24) *
 size_t chunkwise_grads_table_floats() { return kTab; }
 size_t chunkwise_grads_vec_floats() { return kVecB; }
 
+void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta, float *tab_a,
+                                     float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s) {
+    const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
+    if (has_s)
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
+                           eta, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
+    else
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
+                           nullptr, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
+    check_launch("cw_coef_bwd_kernel");
+}
+
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
-                          const float *alpha, const float *theta, const float *eta, const float *m_states,
-                          const float *s_states, const float *dm_states, const float *ds_states, float *d_k,
-                          float *d_v, float *d_q, float *d_theta, float *pvec, float *xs, float *scal,
-                          float *tab_a, float *tab_b, float *vecs, int seq_len, int batch, int chunk_size,
-                          bool has_s, int grid) {
+                          const float *m_states, const float *s_states, const float *dm_states,
+                          const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
+                          float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
+                          int seq_len, int batch, int chunk_size, bool has_s, int grid) {
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     static bool attr_set = false;
     if (!attr_set) {
@@ -594,25 +606,16 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
         attr_set = true;
     }
     if (failed()) return true;
-    if (has_s) {
-        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
-                           eta, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
-        check_launch("cw_coef_bwd_kernel");
-        KernelTimer kt("cw_grads_bf16_kernel");
+    KernelTimer kt("cw_grads_bf16_kernel");
+    if (has_s)
         hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
                            tab_a, tab_b, vecs, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec,
                            xs, scal, seq_len, chunk_size, nc, ntask);
-        check_launch("cw_grads_bf16_kernel");
-    } else {
-        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
-                           nullptr, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
-        check_launch("cw_coef_bwd_kernel");
-        KernelTimer kt("cw_grads_bf16_kernel");
+    else
         hipLaunchKernelGGL(cw_grads_bf16_kernel<false>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
                            tab_a, tab_b, vecs, m_states, nullptr, dm_states, nullptr, d_k, d_v, d_q, d_theta, pvec,
                            xs, scal, seq_len, chunk_size, nc, ntask);
-        check_launch("cw_grads_bf16_kernel");
-    }
+    check_launch("cw_grads_bf16_kernel");
     return true;
 }
 

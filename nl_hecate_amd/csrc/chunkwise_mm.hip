@@ -943,7 +943,8 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                  float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s) {
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
     const int nc = ceil_div(seq_len, chunk_size);
-    Scratch sc = local_scratch(batch, nc);
+    Scratch sc{nullptr, nullptr};
+    if constexpr (sizeof(TIn) == 4) sc = local_scratch(batch, nc);
     const size_t st_bytes = (size_t)batch * (nc + 1) * HD * HD * sizeof(float);
     float *dm_states = scratch(5, st_bytes);
     float *ds_states = scratch(6, st_bytes);
@@ -960,25 +961,28 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         set_lds(cw_gates_bwd_kernel, kGatesBwdLds);
         attr_set = true;
     }
-    hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
-                       stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc, (int)has_s,
-                       batch * nc);
-    check_launch("cw_local_bwd_kernel");
-    hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr, sc.loc,
-                       sc.locs, dm_states, ds_states, nc, (int)has_s);
-    check_launch("cw_scan_kernel");
     int xs_tiled = 0;
     if constexpr (sizeof(TIn) == 2) {
+        // bf16 tokens: coefficient pre-pass, adjoint scan and per-chunk gradients on the bf16 matrix cores
         const size_t nchunks = (size_t)batch * nc;
         float *tab_a = scratch(12, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *tab_b = scratch(13, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
         if (failed()) return;
-        chunkwise_grads_bf16(k, v, q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q,
-                             d_theta, pvec, xs, scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
+        chunkwise_backward_coefficients(alpha, theta, eta, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s);
+        chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_states, ds_states, seq_len, batch, chunk_size, has_s);
+        chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec, xs,
+                             scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
                              persistent_grid(batch * nc));
         xs_tiled = 1;
     } else {
+        hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
+                           stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc,
+                           (int)has_s, batch * nc);
+        check_launch("cw_local_bwd_kernel");
+        hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr,
+                           sc.loc, sc.locs, dm_states, ds_states, nc, (int)has_s);
+        check_launch("cw_scan_kernel");
         hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(256), 0, stream(), m_states, s_states,
                            dm_states, ds_states, scal, nc, (int)has_s);
         check_launch("cw_state_dots_kernel");
