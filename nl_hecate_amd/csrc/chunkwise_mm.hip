@@ -172,36 +172,32 @@ __device__ __forceinline__ float lane_bcast(float x, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
 }
 
-// Column j of r, bb, c (thread j of wave 0), optionally stored: Cc[t][j], Bb[j][t], Rr[j][t]
+// Column j of c, bb, r (thread j of waves 0, 2, 3), optionally stored: Cc[t][j], Bb[j][t], Rr[j][t]
 // (stride LDM; entries outside j <= t < L are zero), plus the vectors (wave 1).  The gates
 // are read from global memory into one register per lane and broadcast per step, so the
 // sequential loops carry no memory latency.  Needs a barrier afterwards.
 __device__ __forceinline__ void coefficients(Coef &cf, const Gates &g, int L, float *Cc, float *Bb, float *Rr) {
     const int j = threadIdx.x & 63, w = threadIdx.x >> 6;
-    if (w >= 2) return;
+    if (w >= 4) return;
     const float keep_j = 1.f - g.al;   // 1 beyond L
     const float eta_j = g.et;          // 0 beyond L
+    const bool jv = j < L;
     if (w == 0) {
         // branch-free: tokens after j update the running products; lanes t >= L broadcast
-        // keep = 1, eta = 0, which leaves rr and cc unchanged
-        float rr = 1.f, b = 1.f, cc = 1.f, blv = 0.f;
-        const bool jv = j < L;
+        // keep = 1, eta = 0, which leaves cc unchanged
+        float b = 1.f, cc = 1.f, blv = 0.f;
 #pragma unroll 16
         for (int t = 0; t < CW; t++) {
             const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
             const bool after = t > j;
-            rr *= after ? keep : 1.f;
             b *= after ? et : 1.f;
             cc = after ? fmaf(keep, cc, b) : cc;
             blv = (t == L - 1) ? b : blv;
-            const bool valid = jv && t >= j && t < L;
-            if (Cc) Cc[t * LDM + j] = valid ? cc : 0.f;
-            if (Bb) Bb[j * LDM + t] = valid ? b : 0.f;
-            if (Rr) Rr[j * LDM + t] = valid ? rr : 0.f;
+            if (Cc) Cc[t * LDM + j] = (jv && t >= j && t < L) ? cc : 0.f;
         }
         cf.cl[j] = jv ? cc : 0.f;
         cf.bl[j] = jv ? blv : 0.f;
-    } else {
+    } else if (w == 1) {
         // a_t, beta_t, h_t: every lane runs the same scalar recurrence, lane t keeps step t
         float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f, kh = 0.f;
 #pragma unroll 8
@@ -215,6 +211,24 @@ __device__ __forceinline__ void coefficients(Coef &cf, const Gates &g, int L, fl
         cf.a[j] = j < L ? ka : 0.f;
         cf.beta[j] = j < L ? kb : 0.f;
         cf.h[j] = j < L ? kh : 0.f;
+    } else if (w == 2) {
+        if (!Bb) return;
+        float b = 1.f;
+#pragma unroll 16
+        for (int t = 0; t < CW; t++) {
+            const float et = lane_bcast(eta_j, t);
+            b *= t > j ? et : 1.f;
+            Bb[j * LDM + t] = (jv && t >= j && t < L) ? b : 0.f;
+        }
+    } else {
+        if (!Rr) return;
+        float rr = 1.f;
+#pragma unroll 16
+        for (int t = 0; t < CW; t++) {
+            const float keep = lane_bcast(keep_j, t);
+            rr *= t > j ? keep : 1.f;
+            Rr[j * LDM + t] = (jv && t >= j && t < L) ? rr : 0.f;
+        }
     }
 }
 
