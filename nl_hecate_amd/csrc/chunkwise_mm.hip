@@ -767,64 +767,94 @@ constexpr size_t kGradsBwdLds = 9 * MAT * sizeof(float);
 //   <M_tau, dy_t' q_t'^T> = a_tau p0[t'] + beta_tau ps[t'] + sum_j W[tau][j] X[t'][j]
 //   <S_tau, dy_t' q_t'^T> = h_tau ps[t'] + sum_j Ws[tau][j] X[t'][j],  Ws[tau][j] = -theta_j bb[j][tau]
 //   and the same with dMo / dSo in place of dy q^T (g1, g2 and the three state dots).
-__global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restrict__ alpha,
+__global__ __launch_bounds__(kThr, 4) void cw_gates_bwd_kernel(const float *__restrict__ alpha,
                                                             const float *__restrict__ theta,
                                                             const float *__restrict__ eta,
                                                             const float *__restrict__ pvec,
                                                             const float *__restrict__ xs,
                                                             const float *__restrict__ scal,
                                                             float *__restrict__ d_alpha, float *__restrict__ d_eta,
-                                                            int s, int C, int nc, int has_s, int xs_tiled) {
+                                                            int s, int C, int nc, int has_s, int xs_tiled, int ntask) {
     extern __shared__ float smem[];
-    float *Xs = smem, *Cc = Xs + MAT, *Bb = Cc + MAT, *Rr = Bb + MAT;
+    float *Xs = smem, *Cc = Xs + MAT, *Bb = Cc + MAT, *Rr = Bb + MAT;   // Xs[t'][j] = -theta_j X[t'][j]
     __shared__ Coef cf;
-    __shared__ float p0[CW], ps[CW], g1[CW], g2[CW], um[CW], usm[CW], uss[CW];
+    __shared__ float p0[CW], ps[CW], g1[CW], g2[CW], um[CW], usm[CW], uss[CW];   // g1, g2 scaled by -theta_j
     __shared__ float part[2][2][CW];
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    // Persistent over chunk tasks; the small inputs of the next task are fetched into registers
+    // while the current one computes.
     // xs is row-major [t][j], or (xs_tiled) in the accumulator-tile order of the bf16 pass:
     // [block bi][rt][ct][lane][r] holds X[32 (bi/2) + 16 rt + 4 (lane/16) + r][32 (bi%2) + 16 ct + lane%16]
     Tile<float> tx;
-    fetch(tx, xs + ((size_t)chain * nc + ci) * CW * CW, 64);
-    const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        load_gates(cf, gt);
-    if (threadIdx.x < CW) {
-        const int t = threadIdx.x;
-        const float4 pv = t < L ? *reinterpret_cast<const float4 *>(pvec + (tok + t) * 4) : make_float4(0, 0, 0, 0);
-        p0[t] = pv.x; ps[t] = pv.y; g1[t] = pv.z; g2[t] = pv.w;
+    Gates gt;
+    float4 pv;
+    float sc0 = 0.f, sc1 = 0.f, sc2 = 0.f;
+    auto fetch_task = [&](int task) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        fetch(tx, xs + (size_t)task * CW * CW, 64);
+        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        pv = *reinterpret_cast<const float4 *>(pvec + (tok + min(lane, L - 1)) * 4);
+        sc0 = scal[(size_t)task * 4 + 0]; sc1 = scal[(size_t)task * 4 + 1]; sc2 = scal[(size_t)task * 4 + 2];
+    };
+    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per,
+              task_hi = min(ntask, task_lo + per);
+    if (task_lo >= task_hi) return;
+    fetch_task(task_lo);
+    for (int task = task_lo; task < task_hi; task++) {
+    const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    const float m0dm = sc0, s0dm = sc1, s0ds = sc2;
+    load_gates(cf, gt);
+    if (wv == 4) {
+        const bool in = lane < L;
+        p0[lane] = in ? pv.x : 0.f; ps[lane] = in ? pv.y : 0.f;
+        g1[lane] = in ? -gt.th * pv.z : 0.f; g2[lane] = in ? -gt.th * pv.w : 0.f;
     }
-    const float m0dm = scal[((size_t)chain * nc + ci) * 4 + 0], s0dm = scal[((size_t)chain * nc + ci) * 4 + 1],
-                s0ds = scal[((size_t)chain * nc + ci) * 4 + 2];
     coefficients(cf, gt, L, Cc, Bb, Rr);
     if (xs_tiled) {
 #pragma unroll
         for (int it = 0; it < 2; it++) {
             const int qd = it * kThr + threadIdx.x, ln = qd & 63, ct = (qd >> 6) & 1, rt = (qd >> 7) & 1, bi = qd >> 8;
             const int t = 32 * (bi >> 1) + 16 * rt + 4 * (ln >> 4), j = 32 * (bi & 1) + 16 * ct + (ln & 15);
-            Xs[t * LDM + j] = tx.x[it].x; Xs[(t + 1) * LDM + j] = tx.x[it].y;
-            Xs[(t + 2) * LDM + j] = tx.x[it].z; Xs[(t + 3) * LDM + j] = tx.x[it].w;
+            const float nth = -__shfl(gt.th, j);
+            Xs[t * LDM + j] = nth * tx.x[it].x; Xs[(t + 1) * LDM + j] = nth * tx.x[it].y;
+            Xs[(t + 2) * LDM + j] = nth * tx.x[it].z; Xs[(t + 3) * LDM + j] = nth * tx.x[it].w;
         }
     } else {
-        commit(Xs, tx);
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
+            float *p = Xs + rr * LDM + cc;
+            p[0] = -__shfl(gt.th, cc) * tx.x[it].x; p[1] = -__shfl(gt.th, cc + 1) * tx.x[it].y;
+            p[2] = -__shfl(gt.th, cc + 2) * tx.x[it].z; p[3] = -__shfl(gt.th, cc + 3) * tx.x[it].w;
+        }
     }
     __syncthreads();
-    if (threadIdx.x >= kThr - CW) {   // mat-vecs with W and Ws (last wave; the matrix products start meanwhile)
-        const int tau = threadIdx.x - (kThr - CW);
+    if (task + 1 < task_hi) fetch_task(task + 1);
+    {   // mat-vecs with c and bb: thread (tau, segment of 8 tokens j), then a sum over the 8 segments
+        const int tau = threadIdx.x >> 3, j0 = (threadIdx.x & 7) * 8;
         float x0 = 0.f, x1 = 0.f, x2 = 0.f;
-        for (int j = 0; j <= tau && j < L; j++) {
-            const float wf = -cf.th[j] * Cc[tau * LDM + j], wsv = -cf.th[j] * Bb[j * LDM + tau];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int j = j0 + i;   // entries beyond the diagonal or beyond L are stored as zero
+            const float wf = Cc[tau * LDM + j], wsv = Bb[j * LDM + tau];
             x0 = fmaf(wf, g1[j], x0); x1 = fmaf(wsv, g1[j], x1); x2 = fmaf(wsv, g2[j], x2);
         }
-        um[tau] = cf.a[tau] * m0dm + cf.beta[tau] * s0dm + x0;
-        usm[tau] = cf.h[tau] * s0dm + x1;
-        uss[tau] = cf.h[tau] * s0ds + x2;
+#pragma unroll
+        for (int m = 1; m < 8; m <<= 1) { x0 += __shfl_xor(x0, m); x1 += __shfl_xor(x1, m); x2 += __shfl_xor(x2, m); }
+        if ((threadIdx.x & 7) == 0) {
+            um[tau] = cf.a[tau] * m0dm + cf.beta[tau] * s0dm + x0;
+            usm[tau] = cf.h[tau] * s0dm + x1;
+            uss[tau] = cf.h[tau] * s0ds + x2;
+        }
     }
     NLH_STRIP_ORIGIN();
     Strip ua = zero_strip(), us = zero_strip();
-    mma(ua, [&](int m, int kk) { return -cf.th[kk] * Cc[(m0 + m) * LDM + kk]; },
+    mma(ua, [&](int m, int kk) { return Cc[(m0 + m) * LDM + kk]; },
         [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
     if (has_s)
-        mma(us, [&](int m, int kk) { return -cf.th[kk] * Bb[kk * LDM + m0 + m]; },
+        mma(us, [&](int m, int kk) { return Bb[kk * LDM + m0 + m]; },
             [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
     // row tau feeds token tau+1: weights r[tau+1][t'] (d_alpha) and c[t'][tau+1] (d_eta), zero for t' <= tau
 #pragma unroll
@@ -844,22 +874,27 @@ __global__ __launch_bounds__(kThr) void cw_gates_bwd_kernel(const float *__restr
 #pragma unroll
         for (int i = 0; i < 4; i++) { part[0][nh][m0 + row_of(i)] = ua.t[0][i]; part[1][nh][m0 + row_of(i)] = us.t[0][i]; }
     }
+    // token 0 has no predecessor row: its sums run over the first column of r and c (one wave)
+    float da0 = 0.f, de0 = 0.f;
+    if (wv == 0) {
+        da0 = wave_allreduce(lane < L ? Rr[lane] * p0[lane] : 0.f);
+        de0 = wave_allreduce(lane < L ? Cc[lane * LDM] * ps[lane] : 0.f);
+    }
     __syncthreads();
     if (threadIdx.x < L) {
         const int t = threadIdx.x;
         float da, de;
         if (t == 0) {
-            da = Rr[L - 1] * m0dm; de = cf.cl[0] * s0dm + cf.bl[0] * s0ds;
-            for (int tp = 0; tp < L; tp++) {
-                da = fmaf(Rr[tp], p0[tp], da);
-                de = fmaf(Cc[tp * LDM], ps[tp], de);
-            }
+            da = Rr[L - 1] * m0dm + da0;
+            de = cf.cl[0] * s0dm + cf.bl[0] * s0ds + de0;
         } else {
             da = part[0][0][t - 1] + part[0][1][t - 1] + Rr[t * LDM + L - 1] * um[t - 1];
             de = part[1][0][t - 1] + part[1][1][t - 1] + cf.cl[t] * usm[t - 1] + cf.bl[t] * uss[t - 1];
         }
         d_alpha[tok + t] = -da;
         if (has_s) d_eta[tok + t] = de;
+    }
+    __syncthreads();   // LDS is rewritten by the next task
     }
 }
 constexpr size_t kGatesBwdLds = 4 * MAT * sizeof(float);
@@ -1006,8 +1041,9 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                            d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc);
         check_launch("cw_grads_bwd_kernel");
     }
-    hipLaunchKernelGGL(cw_gates_bwd_kernel, dim3(batch * nc), dim3(kThr), kGatesBwdLds, stream(), alpha, theta, eta,
-                       pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size, nc, (int)has_s, xs_tiled);
+    hipLaunchKernelGGL(cw_gates_bwd_kernel, dim3(min(batch * nc, 2 * persistent_grid(1 << 30))), dim3(kThr),
+                       kGatesBwdLds, stream(), alpha, theta, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size,
+                       nc, (int)has_s, xs_tiled, batch * nc);
     check_launch("cw_gates_bwd_kernel");
     const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
     const int per = 8, rows = ceil_div(batch, per);
