@@ -42,6 +42,7 @@ METRIC = "Titans LMM fwd+bwd tokens/s (d=512, L=4096, 1 GPU); % of HBM/MFMA roof
 # Published MI355X peaks used as roofline denominators.
 PEAK_HBM_GBS = 8000.0
 PEAK_FP32_TFLOPS = 157.3
+PEAK_BF16_TFLOPS = 2500.0
 
 # Algorithmic work per head-token at d=64 (fp32): forward 9 d^2 flop
 # (M k, S update, M update, M q), backward 30 d^2 flop (one replay + reverse
@@ -196,7 +197,8 @@ def setup_titans_chunkwise_c3(torch, D, lib):
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16",
         flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_bwd=BYTES_CW_BWD,
-        traffic_bwd=int((838.3 + 522.0) * 2**20),   # measured for cw_grads_bwd_kernel: 838.3 MiB read, 522.0 MiB written
+        matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
+        traffic_bwd=int((1707.6 + 522.3) * 2**20),   # measured for cw_grads_bf16_kernel: 1707.6 MiB read, 522.3 MiB written
         kernel="cw_grads_bf16_kernel (the per-chunk gradient pass of the backward entry point)",
         kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
         config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
@@ -249,6 +251,7 @@ def setup_swa_c5(torch, D, lib):
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * heads * s, bound="hbm", dtype="bf16",
         flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_bwd=BYTES_SWA_BWD,
+        matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
         traffic_bwd=int((1441.1 + 128.0 + 1057.9 + 65.0) * 2**20),   # measured: key pass + query pass
         kernel=None,
         kernel_names={"forward": "swa_forward", "backward": "swa_backward"},
@@ -475,8 +478,11 @@ def main():
                 "algorithmic_bytes": w["bytes_bwd"] * head_tokens,
                 "avg_launch_ms": kern_ms, "entry_point_ms": bwd_ms,
                 "hbm": {"achieved": bwd_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s"},
-                "fp32_matrix": {"achieved": bwd_tflops, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                                "frac": bwd_tflops / PEAK_FP32_TFLOPS}}
+                w.get("matrix", "fp32_matrix"): {"achieved": bwd_tflops, "peak": w.get("matrix_peak", PEAK_FP32_TFLOPS),
+                                                 "unit": "TFLOP/s",
+                                                 "frac": bwd_tflops / w.get("matrix_peak", PEAK_FP32_TFLOPS)},
+                "entry_point": {"achieved": w["bytes_bwd"] * head_tokens / (bwd_ms * 1e-3) / 1e9, "unit": "GB/s",
+                                "frac": w["bytes_bwd"] * head_tokens / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}}
     out = {
         "metric": METRIC, "value": value, "unit": w.get("unit", "tokens/s"), "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -485,7 +491,7 @@ def main():
         "config": w["config"],
         "event_ms_per_step": ev_ms / args.steps,
         "kernels_ms": {w["kernel_names"]["forward"]: fwd_ms, w["kernel_names"]["backward"]: bwd_ms},
-        "fwd_fp32_tflops": w["flop_fwd"] * head_tokens / (max(fwd_ms, 1e-9) * 1e-3) / 1e12,
+        "fwd_tflops": w["flop_fwd"] * head_tokens / (max(fwd_ms, 1e-9) * 1e-3) / 1e12,
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
