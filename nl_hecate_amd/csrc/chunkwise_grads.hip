@@ -17,7 +17,7 @@
 // (its two terms nearly cancel once the memory has learned); every other fp32 operand (dY,
 // states, adjoints, E, c.P, c.R, dE) enters the matrix cores rounded to one bf16, products
 // accumulate in fp32.  That is the bf16-input / fp32-accumulate contract: results agree with
-// the fp32 oracle to a few 1e-3, inside the 2e-2 stated for this path.
+// an fp32 evaluation of the same rule to a few 1e-3, inside the 2e-2 stated for this path.
 //
 // One workgroup per compute unit walks over chunks.  While one chunk computes, every 128-byte
 // line of the next chunk's inputs is touched by one 4-byte load, so that the real loads at the
