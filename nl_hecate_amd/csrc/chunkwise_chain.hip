@@ -102,33 +102,42 @@ __global__ __launch_bounds__(256) void cw_coef_kernel(const float *__restrict__ 
 // Pipeline of one chunk step.  Every global load of chunk c+1 (tokens, W, coefficient vectors)
 // is issued at the top of step c and first touched at the bottom of step c, after the matrix
 // work and before the stores of step c, so no wait inside a step ever meets a load in flight
-// or a store just issued.
+// or a store just issued.  The requests and their landing are unconditional (past the end they
+// repeat the last chunk): memory waits are placed per program point, not per path.
+//
+// The rows of M and S never mix, so a chain is split over two workgroups of 32 rows each
+// (workgroup = blockIdx.x / batch picks the half, so both halves of a chain share an XCD's L2
+// for K, Q and W).  Waves 0..3 (group X): E, then Y^T, one 16-token strip each.  Waves 4..7
+// (group Y): one 32x32 block of W.P each, then one 16-column strip of the transposed state
+// update; they hold the fp32 master state.
 template <bool HAS_S>
 __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q,
     const float *__restrict__ table, const float *__restrict__ vecs, const float *__restrict__ m_initial,
     const float *__restrict__ s_initial, float *__restrict__ m_states, float *__restrict__ s_states,
-    float *__restrict__ y, int s, int C, int nc) {
+    float *__restrict__ y, int s, int C, int nc, int batch) {
+    constexpr int HMAT = 32 * LDB;   // a 32-row matrix
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *Kr = reinterpret_cast<u16 *>(smem_raw);   // K [t][c]
     u16 *Kt0 = Kr + BMAT, *Kt1 = Kt0 + BMAT;       // K^T [c][t] of this chunk / V [t][i] until K^T of the next lands
     u16 *Qr0 = Kt1 + BMAT, *Qr1 = Qr0 + BMAT;      // Q [t][c], alternating between chunks
-    u16 *Mh = Qr1 + BMAT, *Ml = Mh + BMAT;         // chunk-start M [i][c], hi / lo
-    u16 *Sh = Ml + BMAT, *Sl = Sh + BMAT;          // chunk-start S
-    u16 *Eh = Sl + BMAT, *El = Eh + BMAT;          // E^T [i][t]
-    u16 *EMh = El + BMAT, *EMl = EMh + BMAT;       // (E.wM)^T
-    u16 *ESh = EMl + BMAT, *ESl = ESh + BMAT;      // (E.wS)^T
-    u16 *WPh = ESl + BMAT, *WPl = WPh + BMAT;      // W.P [t][j]
-    float *cvec = reinterpret_cast<float *>(WPl + BMAT);   // a, beta, wM, wS [64] each, then a_L, beta_L, h_L
+    u16 *WPh = Qr1 + BMAT, *WPl = WPh + BMAT;      // W.P [t][j]
+    u16 *Mh = WPl + BMAT, *Ml = Mh + HMAT;         // chunk-start M [i][c], this workgroup's 32 rows, hi / lo
+    u16 *Sh = Ml + HMAT, *Sl = Sh + HMAT;          // chunk-start S
+    u16 *Eh = Sl + HMAT, *El = Eh + HMAT;          // E^T [i][t]
+    u16 *EMh = El + HMAT, *EMl = EMh + HMAT;       // (E.wM)^T
+    u16 *ESh = EMl + HMAT, *ESl = ESh + HMAT;      // (E.wS)^T
+    float *cvec = reinterpret_cast<float *>(ESl + HMAT);   // a, beta, wM, wS [64] each, then a_L, beta_L, h_L
 
-    const int chain = blockIdx.x, tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
+    const int chain = blockIdx.x % batch, i0 = 32 * (blockIdx.x / batch);
     const bool grpX = w < 4;
-    const int bi = w & 3, bm = 32 * (bi >> 1), bn = 32 * (bi & 1);   // origin of this wave's 32x32 block
+    const int bi = w & 3, bm = 32 * (bi >> 1), bn = 32 * (bi & 1);   // group Y: 32x32 block of P^T; group X: strip bi
     const size_t chain_tok = (size_t)chain * s;
     const size_t state0 = (size_t)chain * (nc + 1) * HD * HD;
 
-    // -V enters E = K M0^T - V as one more step of the product: A = V (rows t), B = -identity.
-    // Output columns bn + 16 ct + l%16 meet contraction indices 32 (bn/32) + 8 (l/16) + e.
+    // -V enters E = K M0^T - V as one more step of the product: A = V (rows t, this half's 32
+    // columns as contraction), B = -identity: column 16 ct + l%16 meets contraction index 8 (l/16) + e.
     bf16x8 negI[2];
 #pragma unroll
     for (int ct = 0; ct < 2; ct++) {
@@ -141,21 +150,21 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
         negI[ct] = __builtin_bit_cast(bf16x8, bits);
     }
 
-    // Registers of the next chunk.  Every wave: 8 consecutive bf16 of one row of K, Q, V
-    // (lane -> row st_t, 8-column block st_cb) and W at the accumulator positions of its P^T
-    // block (used by group Y).  Threads 0..271: one float of the coefficient vectors.
-    const int st_t = 32 * (w & 1) + (l & 31), st_cb = 2 * (w >> 1) + (l >> 5);
+    // Registers of the next chunk.  K, Q: row st_t, 8-element block st_cb (16 rows x 64 bytes per
+    // wave instruction).  V (threads 0..255): row vt, block vcb of this half's 32 columns.  Group Y:
+    // W at the accumulator positions of its P^T block.  Threads 0..259: one float of the vectors.
+    const int st_t = 16 * (w & 3) + (l & 15), st_cb = 4 * (w >> 2) + (l >> 4);
+    const int vt = (tid >> 2) & 63, vcb = tid & 3;
     uint4 sk, sq, sv;
     f32x4 wn[2][2], wc[2][2];
     float vn = 0.f;
-    // All loads are unconditional (rows beyond a short last chunk re-read its last row and are
-    // zeroed when committed; tiles of W above the diagonal read the zero pad of vecs).
     auto fetch = [&](int c) {
         const int L = min(C, s - c * C);
-        const size_t o = (chain_tok + (size_t)c * C + min(st_t, L - 1)) * HD + st_cb * 8;
+        const size_t tok = chain_tok + (size_t)c * C;
+        const size_t o = (tok + min(st_t, L - 1)) * HD + st_cb * 8;
         sk = *reinterpret_cast<const uint4 *>(k + o);
         sq = *reinterpret_cast<const uint4 *>(q + o);
-        sv = *reinterpret_cast<const uint4 *>(v + o);
+        sv = *reinterpret_cast<const uint4 *>(v + (tok + min(vt, L - 1)) * HD + i0 + vcb * 8);
         const size_t chunk = (size_t)chain * nc + c;
         const float *tb = table + chunk * kTableFloats, *vo = vecs + chunk * kVecFloats;
 #pragma unroll
@@ -163,11 +172,13 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
 #pragma unroll
             for (int ct = 0; ct < 2; ct++)
                 wn[rt][ct] = *reinterpret_cast<const f32x4 *>(
-                    tile_live(bi, rt, ct) ? tb + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4 : vo + 4 * CW + 4);
+                    (!grpX && tile_live(bi, rt, ct)) ? tb + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4 : vo + 4 * CW + 4);
         vn = vo[min(tid, 4 * CW + 3)];
     };
     auto land = [&](int c) {   // wait for the loads here; zero the rows beyond a short chunk
-        if (st_t >= min(C, s - c * C)) { sk = make_uint4(0, 0, 0, 0); sq = sk; sv = sk; }
+        const int L = min(C, s - c * C);
+        if (st_t >= L) { sk = make_uint4(0, 0, 0, 0); sq = sk; }
+        if (vt >= L) sv = make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int rt = 0; rt < 2; rt++)
 #pragma unroll
@@ -185,46 +196,42 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
             Kt[(st_cb * 8 + 2 * i + 1) * LDB + st_t] = (u16)(kw[i] >> 16);
         }
     };
+    auto commit_v = [&](u16 *dst) {
+        if (tid < 256) *reinterpret_cast<uint4 *>(dst + vt * LDB + vcb * 8) = sv;
+    };
     auto commit_vecs = [&]() {
         if (tid < 4 * CW + 4) cvec[tid] = vn;
     };
 
-    // fp32 master state (group Y), transposed block:
-    //   Mm[rt][ct][r] = M[i = bn + 16 ct + l%16][c = bm + 16 rt + 4 (l/16) + r]
-    // Group X has no state; it borrows the same registers as accumulators of Q M0^T and Q S0^T.
-    f32x4 Mm[2][2], Sm[2][2];
-    auto state_off = [&](int rt, int ct) { return (bn + 16 * ct + r16) * HD + bm + 16 * rt + 4 * g; };
+    // fp32 master state (group Y), transposed strip:
+    //   Mm[ct][r] = M[i = i0 + 16 ct + l%16][c = 16 bi + 4 (l/16) + r]
+    // Group X has no state; it borrows the same registers as accumulators of M0 Q^T and S0 Q^T.
+    f32x4 Mm[2], Sm[2];
     auto publish_state = [&](int slot) {   // -> HBM snapshot
 #pragma unroll
-        for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-            for (int ct = 0; ct < 2; ct++) {
-                const size_t o = state0 + (size_t)slot * HD * HD + state_off(rt, ct);
-                *reinterpret_cast<f32x4 *>(m_states + o) = Mm[rt][ct];
-                if (HAS_S) *reinterpret_cast<f32x4 *>(s_states + o) = Sm[rt][ct];
-            }
+        for (int ct = 0; ct < 2; ct++) {
+            const size_t o = state0 + (size_t)slot * HD * HD + (i0 + 16 * ct + r16) * HD + 16 * bi + 4 * g;
+            *reinterpret_cast<f32x4 *>(m_states + o) = Mm[ct];
+            if (HAS_S) *reinterpret_cast<f32x4 *>(s_states + o) = Sm[ct];
+        }
     };
     auto stage_state = [&]() {             // -> LDS operands of the next chunk
 #pragma unroll
-        for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-            for (int ct = 0; ct < 2; ct++) {
-                const int off = (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g;
-                split_store(Mh, Ml, off, Mm[rt][ct]);
-                if (HAS_S) split_store(Sh, Sl, off, Sm[rt][ct]);
-            }
+        for (int ct = 0; ct < 2; ct++) {
+            const int off = (16 * ct + r16) * LDB + 16 * bi + 4 * g;
+            split_store(Mh, Ml, off, Mm[ct]);
+            if (HAS_S) split_store(Sh, Sl, off, Sm[ct]);
+        }
     };
 
     fetch(0);
     if (!grpX) {
 #pragma unroll
-        for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-            for (int ct = 0; ct < 2; ct++) {
-                const size_t o = (size_t)chain * HD * HD + state_off(rt, ct);
-                Mm[rt][ct] = *reinterpret_cast<const f32x4 *>(m_initial + o);
-                Sm[rt][ct] = HAS_S ? *reinterpret_cast<const f32x4 *>(s_initial + o) : zero4();
-            }
+        for (int ct = 0; ct < 2; ct++) {
+            const size_t o = (size_t)chain * HD * HD + (i0 + 16 * ct + r16) * HD + 16 * bi + 4 * g;
+            Mm[ct] = *reinterpret_cast<const f32x4 *>(m_initial + o);
+            Sm[ct] = HAS_S ? *reinterpret_cast<const f32x4 *>(s_initial + o) : zero4();
+        }
         publish_state(0);
         stage_state();
     }
@@ -232,188 +239,137 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
     commit_rows(Kr, sk);
     commit_rows(Qr0, sq);
     commit_kt(Kt0);
-    commit_rows(Kt1, sv);
+    commit_v(Kt1);
     commit_vecs();
     __syncthreads();
 
     for (int c = 0; c < nc; c++) {
         const int t0 = c * C, L = min(C, s - t0);
         const size_t tok = chain_tok + t0;
-        const bool more = c + 1 < nc;
         // this chunk: Q in Qc, K^T in Kc, V in Kn (until K^T of the next chunk replaces it)
         u16 *Qc = (c & 1) ? Qr1 : Qr0, *Kc = (c & 1) ? Kt1 : Kt0;
         u16 *Qn = (c & 1) ? Qr0 : Qr1, *Kn = (c & 1) ? Kt0 : Kt1;
-        if (more) fetch(c + 1);
+        fetch(min(c + 1, nc - 1));
         // ── first half: E^T, (E.wM)^T, (E.wS)^T (group X) and W.P (group Y) ──
-        {
+        if (grpX) {
+            // E[t][i]: rows t = 16 bi .., columns i = 16 ct ..
+            const bf16x8 aK[2] = {ld_op(Kr, 16 * bi, 0), ld_op(Kr, 16 * bi, 1)};
+            const bf16x8 aV = ld_op(Kn, 16 * bi, 0);
+            const f32x4 wm = *reinterpret_cast<const f32x4 *>(cvec + 2 * CW + 16 * bi + 4 * g);
+            const f32x4 wsv = *reinterpret_cast<const f32x4 *>(cvec + 3 * CW + 16 * bi + 4 * g);
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++) {
+                f32x4 e = zero4();
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    e = mfma32(aK[ks], ld_op(Mh, 16 * ct, ks), e);
+                    e = mfma32(aK[ks], ld_op(Ml, 16 * ct, ks), e);
+                }
+                e = mfma32(aV, negI[ct], e);
+                const int off = (16 * ct + r16) * LDB + 16 * bi + 4 * g;   // [i][t .. t+3]
+                split_store(Eh, El, off, e);
+                split_store(EMh, EMl, off, e * wm);
+                if (HAS_S) split_store(ESh, ESl, off, e * wsv);
+            }
+        } else {
             bf16x8 aK[2][2];
 #pragma unroll
             for (int rt = 0; rt < 2; rt++)
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++) aK[rt][ks] = ld_op(Kr, bm + 16 * rt, ks);
             f32x4 acc[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
-            if (grpX) {
-                const bf16x8 aV[2] = {ld_op(Kn, bm, bn >> 5), ld_op(Kn, bm + 16, bn >> 5)};
 #pragma unroll
-                for (int ks = 0; ks < 2; ks++)
+            for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                    for (int ct = 0; ct < 2; ct++) {
-                        const bf16x8 bh = ld_op(Mh, bn + 16 * ct, ks), bl = ld_op(Ml, bn + 16 * ct, ks);
+                for (int ct = 0; ct < 2; ct++) {
+                    const bf16x8 bq = ld_op(Qc, bn + 16 * ct, ks);
 #pragma unroll
-                        for (int rt = 0; rt < 2; rt++) {   // E[t][i]: rows t, columns i
-                            acc[rt][ct] = mfma32(aK[rt][ks], bh, acc[rt][ct]);
-                            acc[rt][ct] = mfma32(aK[rt][ks], bl, acc[rt][ct]);
-                        }
-                    }
-#pragma unroll
-                for (int rt = 0; rt < 2; rt++) {
-                    const f32x4 wm = *reinterpret_cast<const f32x4 *>(cvec + 2 * CW + bm + 16 * rt + 4 * g);
-                    const f32x4 wsv = *reinterpret_cast<const f32x4 *>(cvec + 3 * CW + bm + 16 * rt + 4 * g);
-#pragma unroll
-                    for (int ct = 0; ct < 2; ct++) {
-                        const f32x4 ev = mfma32(aV[rt], negI[ct], acc[rt][ct]);
-                        const int off = (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g;   // [i][t .. t+3]
-                        split_store(Eh, El, off, ev);
-                        split_store(EMh, EMl, off, ev * wm);
-                        if (HAS_S) split_store(ESh, ESl, off, ev * wsv);
-                    }
+                    for (int rt = 0; rt < 2; rt++)     // P^T[j][t]: rows j, columns t
+                        acc[rt][ct] = mfma32(aK[rt][ks], bq, acc[rt][ct]);
                 }
-            } else {
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                    for (int ct = 0; ct < 2; ct++) {
-                        const bf16x8 bq = ld_op(Qc, bn + 16 * ct, ks);
-#pragma unroll
-                        for (int rt = 0; rt < 2; rt++)     // P^T[j][t]: rows j, columns t
-                            acc[rt][ct] = mfma32(aK[rt][ks], bq, acc[rt][ct]);
-                    }
-#pragma unroll
-                for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-                    for (int ct = 0; ct < 2; ct++)         // [t][j .. j+3]
-                        split_store(WPh, WPl, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g,
-                                    wc[rt][ct] * acc[rt][ct]);
-            }
-        }
-        __syncthreads();
-        // ── second half: Y (group X) and the state update (group Y) ──
-        f32x4 y2[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};   // group X: (W.P) E; group Y: unused
-        if (grpX) {
-            // rows t in [bm, bm+32), columns i in [bn, bn+32)
-            f32x4(&y0)[2][2] = Mm, (&y1)[2][2] = Sm;
 #pragma unroll
             for (int rt = 0; rt < 2; rt++)
 #pragma unroll
-                for (int ct = 0; ct < 2; ct++) { y0[rt][ct] = zero4(); y1[rt][ct] = zero4(); }
+                for (int ct = 0; ct < 2; ct++)         // [t][j .. j+3]
+                    split_store(WPh, WPl, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g,
+                                wc[rt][ct] * acc[rt][ct]);
+        }
+        __syncthreads();
+        // ── second half: Y^T (group X) and the state update (group Y) ──
+        f32x4 y2[2] = {zero4(), zero4()};   // group X: E^T (W.P)^T, then the finished Y^T; group Y: unused
+        if (grpX) {
+            // Y^T[i][t]: rows i = 16 rt .., columns t = 16 bi ..: a lane ends up with four consecutive
+            // i of one token
+            f32x4(&y0)[2] = Mm, (&y1)[2] = Sm;
+            y0[0] = y0[1] = y1[0] = y1[1] = zero4();
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                bf16x8 aQ[2], aWh[2], aWl[2];
+                const bf16x8 bQ = ld_op(Qc, 16 * bi, ks), bWh = ld_op(WPh, 16 * bi, ks), bWl = ld_op(WPl, 16 * bi, ks);
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
-                    aQ[rt] = ld_op(Qc, bm + 16 * rt, ks);
-                    aWh[rt] = ld_op(WPh, bm + 16 * rt, ks);
-                    aWl[rt] = ld_op(WPl, bm + 16 * rt, ks);
-                }
-#pragma unroll
-                for (int ct = 0; ct < 2; ct++) {
-                    const int i0 = bn + 16 * ct;
-                    const bf16x8 mh = ld_op(Mh, i0, ks), ml = ld_op(Ml, i0, ks);
-                    const bf16x8 eh = ld_op(Eh, i0, ks), el = ld_op(El, i0, ks);
-#pragma unroll
-                    for (int rt = 0; rt < 2; rt++) {
-                        y0[rt][ct] = mfma32(aQ[rt], mh, y0[rt][ct]);
-                        y0[rt][ct] = mfma32(aQ[rt], ml, y0[rt][ct]);
-                        y2[rt][ct] = mfma32(aWh[rt], eh, y2[rt][ct]);
-                        y2[rt][ct] = mfma32(aWl[rt], eh, y2[rt][ct]);
-                        y2[rt][ct] = mfma32(aWh[rt], el, y2[rt][ct]);
-                    }
+                    const bf16x8 eh = ld_op(Eh, 16 * rt, ks);
+                    y0[rt] = mfma32(ld_op(Mh, 16 * rt, ks), bQ, y0[rt]);
+                    y0[rt] = mfma32(ld_op(Ml, 16 * rt, ks), bQ, y0[rt]);
+                    y2[rt] = mfma32(eh, bWh, y2[rt]);
+                    y2[rt] = mfma32(eh, bWl, y2[rt]);
+                    y2[rt] = mfma32(ld_op(El, 16 * rt, ks), bWh, y2[rt]);
                     if (HAS_S) {
-                        const bf16x8 sh = ld_op(Sh, i0, ks), sl = ld_op(Sl, i0, ks);
-#pragma unroll
-                        for (int rt = 0; rt < 2; rt++) {
-                            y1[rt][ct] = mfma32(aQ[rt], sh, y1[rt][ct]);
-                            y1[rt][ct] = mfma32(aQ[rt], sl, y1[rt][ct]);
-                        }
+                        y1[rt] = mfma32(ld_op(Sh, 16 * rt, ks), bQ, y1[rt]);
+                        y1[rt] = mfma32(ld_op(Sl, 16 * rt, ks), bQ, y1[rt]);
                     }
                 }
             }
+            const float at = cvec[16 * bi + r16], bt = cvec[CW + 16 * bi + r16];
 #pragma unroll
-            for (int rt = 0; rt < 2; rt++) {
-                const f32x4 at = *reinterpret_cast<const f32x4 *>(cvec + bm + 16 * rt + 4 * g);
-                const f32x4 bt = *reinterpret_cast<const f32x4 *>(cvec + CW + bm + 16 * rt + 4 * g);
-#pragma unroll
-                for (int ct = 0; ct < 2; ct++) y2[rt][ct] += at * y0[rt][ct] + bt * y1[rt][ct];
-            }
+            for (int rt = 0; rt < 2; rt++) y2[rt] += at * y0[rt] + bt * y1[rt];
         } else {
-            // transposed state block: rows c in [bm, bm+32), columns i in [bn, bn+32)
-            f32x4 am[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}}, as[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+            // transposed state strip: rows c = 16 bi .., columns i = 16 ct ..
+            f32x4 am[2] = {zero4(), zero4()}, as[2] = {zero4(), zero4()};
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                bf16x8 aKt[2];
-#pragma unroll
-                for (int rt = 0; rt < 2; rt++) aKt[rt] = ld_op(Kc, bm + 16 * rt, ks);
+                const bf16x8 aKt = ld_op(Kc, 16 * bi, ks);
 #pragma unroll
                 for (int ct = 0; ct < 2; ct++) {
-                    const int i0 = bn + 16 * ct;
-                    const bf16x8 mh = ld_op(EMh, i0, ks), ml = ld_op(EMl, i0, ks);
-#pragma unroll
-                    for (int rt = 0; rt < 2; rt++) {
-                        am[rt][ct] = mfma32(aKt[rt], mh, am[rt][ct]);
-                        am[rt][ct] = mfma32(aKt[rt], ml, am[rt][ct]);
-                    }
+                    am[ct] = mfma32(aKt, ld_op(EMh, 16 * ct, ks), am[ct]);
+                    am[ct] = mfma32(aKt, ld_op(EMl, 16 * ct, ks), am[ct]);
                     if (HAS_S) {
-                        const bf16x8 sh = ld_op(ESh, i0, ks), sl = ld_op(ESl, i0, ks);
-#pragma unroll
-                        for (int rt = 0; rt < 2; rt++) {
-                            as[rt][ct] = mfma32(aKt[rt], sh, as[rt][ct]);
-                            as[rt][ct] = mfma32(aKt[rt], sl, as[rt][ct]);
-                        }
+                        as[ct] = mfma32(aKt, ld_op(ESh, 16 * ct, ks), as[ct]);
+                        as[ct] = mfma32(aKt, ld_op(ESl, 16 * ct, ks), as[ct]);
                     }
                 }
             }
             const float aL = cvec[4 * CW], betaL = cvec[4 * CW + 1], hL = cvec[4 * CW + 2];
 #pragma unroll
-            for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-                for (int ct = 0; ct < 2; ct++) {
-                    Mm[rt][ct] = aL * Mm[rt][ct] + betaL * Sm[rt][ct] + am[rt][ct];
-                    if (HAS_S) Sm[rt][ct] = hL * Sm[rt][ct] + as[rt][ct];
-                }
+            for (int ct = 0; ct < 2; ct++) {
+                Mm[ct] = aL * Mm[ct] + betaL * Sm[ct] + am[ct];
+                if (HAS_S) Sm[ct] = hL * Sm[ct] + as[ct];
+            }
         }
         // tokens of the next chunk land: K and V of this one are no longer read
-        if (more) {
-            land(c + 1);
-            commit_rows(Kr, sk);
-            commit_rows(Qn, sq);
-            commit_kt(Kn);
-        }
+        land(min(c + 1, nc - 1));
+        commit_rows(Kr, sk);
+        commit_rows(Qn, sq);
+        commit_kt(Kn);
         // results of this chunk leave
         if (grpX) {
+            const int t = 16 * bi + r16;
+            if (t < L) {
 #pragma unroll
-            for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int t = bm + 16 * rt + 4 * g + r;
-                    if (t < L) {
-#pragma unroll
-                        for (int ct = 0; ct < 2; ct++) y[(tok + t) * HD + bn + 16 * ct + r16] = y2[rt][ct][r];
-                    }
-                }
+                for (int rt = 0; rt < 2; rt++)
+                    *reinterpret_cast<f32x4 *>(y + (tok + t) * HD + i0 + 16 * rt + 4 * g) = y2[rt];
+            }
         } else {
             publish_state(c + 1);
         }
         __syncthreads();
-        if (more) {
-            if (!grpX) stage_state();
-            commit_rows(Kc, sv);   // K^T of this chunk is no longer read
-            commit_vecs();
-        }
+        if (!grpX) stage_state();
+        commit_v(Kc);   // K^T of this chunk is no longer read
+        commit_vecs();
         __syncthreads();
     }
 }
 
-constexpr size_t kChainFwdLds = 17 * BMAT * sizeof(u16) + (4 * CW + 4) * sizeof(float);
+constexpr size_t kChainFwdLds = (7 * BMAT + 10 * 32 * LDB) * sizeof(u16) + (4 * CW + 4) * sizeof(float);
 
 template <bool HAS_S>
 void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, const float *alpha, const float *theta,
@@ -433,8 +389,8 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
     hipLaunchKernelGGL(cw_coef_kernel<HAS_S>, dim3(ceil_div(nchunks, 2)), dim3(256), 0, stream(), alpha, theta, eta,
                        table, vecs, seq_len, chunk_size, nc, nchunks);
     check_launch("cw_coef_kernel");
-    hipLaunchKernelGGL(cw_chain_fwd_kernel<HAS_S>, dim3(batch), dim3(kChainThr), kChainFwdLds, stream(), k, v, q,
-                       table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc);
+    hipLaunchKernelGGL(cw_chain_fwd_kernel<HAS_S>, dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k, v, q,
+                       table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch);
     check_launch(fn);
 }
 
