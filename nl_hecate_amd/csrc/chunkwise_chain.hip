@@ -54,15 +54,17 @@ __global__ __launch_bounds__(256) void cw_coef_kernel(const float *__restrict__ 
                                                       const float *__restrict__ theta,
                                                       const float *__restrict__ eta, float *__restrict__ table,
                                                       float *__restrict__ vecs, int s, int C, int nc, int nchunks) {
-    const int chunk = blockIdx.x * 2 + (threadIdx.x >> 7), role = (threadIdx.x >> 6) & 1, j = threadIdx.x & 63;
-    if (chunk >= nchunks) return;
+    // The table is assembled in LDS and leaves as 16-byte stores of consecutive lanes.
+    __shared__ __align__(16) float stage[2][kTableFloats];
+    const int chunk = min(blockIdx.x * 2 + (int)(threadIdx.x >> 7), nchunks - 1);   // an odd tail is done twice
+    const int role = (threadIdx.x >> 6) & 1, j = threadIdx.x & 63;
     const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
     const Gates g = fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, L);
     const float keep_j = 1.f - g.al;   // 1 beyond L
     const float eta_j = g.et;          // 0 beyond L
     float *vo = vecs + (size_t)chunk * kVecFloats;
     if (role == 0) {
-        float *to = table + (size_t)chunk * kTableFloats;
+        float *to = stage[threadIdx.x >> 7];
         float b = 1.f, cc = 1.f, blv = 0.f;
         const bool jv = j < L;
         const float nth = -g.th;
@@ -96,6 +98,14 @@ __global__ __launch_bounds__(256) void cw_coef_kernel(const float *__restrict__ 
         vo[CW + j] = j < L ? kb : 0.f;
         if (j == L - 1) { vo[4 * CW] = ka; vo[4 * CW + 1] = kb; vo[4 * CW + 2] = kh; }
         if (j < 4) vo[4 * CW + 4 + j] = 0.f;   // zero pad: what tiles of W above the diagonal read
+    }
+    __syncthreads();
+    const float *from = stage[threadIdx.x >> 7];
+    float *out = table + (size_t)chunk * kTableFloats;
+    for (int qd = threadIdx.x & 127; qd < kTableFloats / 4; qd += 128) {
+        const int tile = qd >> 6;   // (bi, rt, ct) = (tile / 4, tile / 2 % 2, tile % 2)
+        if (tile_live(tile >> 2, (tile >> 1) & 1, tile & 1))
+            *reinterpret_cast<f32x4 *>(out + qd * 4) = *reinterpret_cast<const f32x4 *>(from + qd * 4);
     }
 }
 

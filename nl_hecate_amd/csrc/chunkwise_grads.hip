@@ -48,20 +48,22 @@ __device__ __forceinline__ bool live_a(int bi, int rt, int ct) { return 2 * (bi 
 __device__ __forceinline__ bool live_b(int bi, int rt, int ct) { return 2 * (bi >> 1) + rt >= 2 * (bi & 1) + ct; }
 
 template <bool HAS_S>
-__global__ __launch_bounds__(256) void cw_coef_bwd_kernel(const float *__restrict__ alpha,
+__global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restrict__ alpha,
                                                           const float *__restrict__ theta,
                                                           const float *__restrict__ eta, float *__restrict__ tab_a,
                                                           float *__restrict__ tab_b, float *__restrict__ vecs,
                                                           int s, int C, int nc, int nchunks) {
-    const int chunk = blockIdx.x * 2 + (threadIdx.x >> 7), role = (threadIdx.x >> 6) & 1, j = threadIdx.x & 63;
-    if (chunk >= nchunks) return;
+    // One chunk per workgroup of two waves; both tables are assembled in LDS and leave as 16-byte
+    // stores of consecutive lanes.
+    __shared__ __align__(16) float stage[2][kTab];
+    const int chunk = blockIdx.x, role = threadIdx.x >> 6, j = threadIdx.x & 63;
     const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
     const Gates g = fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, L);
     const float keep_j = 1.f - g.al;   // 1 beyond L
     const float eta_j = g.et;          // 0 beyond L
     float *vo = vecs + (size_t)chunk * kVecB;
     if (role == 0) {
-        float *ta = tab_a + (size_t)chunk * kTab, *tb = tab_b + (size_t)chunk * kTab;
+        float *ta = stage[0], *tb = stage[1];
         float b = 1.f, cc = 1.f, blv = 0.f;
         const bool jv = j < L;
         const int ja = (j >> 5) * 2048 + ((j >> 4) & 1) * 512 + ((j & 15) >> 2) * 64 + (j & 3);
@@ -96,6 +98,13 @@ __global__ __launch_bounds__(256) void cw_coef_bwd_kernel(const float *__restric
         vo[CW + j] = j < L ? kb : 0.f;
         if (j < 4) vo[5 * CW + j] = 0.f;   // what tiles above the diagonal read
         if (j == L - 1) vo[5 * CW + 4] = kh;
+    }
+    __syncthreads();
+    float *oa = tab_a + (size_t)chunk * kTab, *ob = tab_b + (size_t)chunk * kTab;
+    for (int qd = threadIdx.x; qd < kTab / 4; qd += 128) {
+        const int tile = qd >> 6, bi = tile >> 2, rt = (tile >> 1) & 1, ct = tile & 1;
+        if (live_a(bi, rt, ct)) *reinterpret_cast<f32x4 *>(oa + qd * 4) = *reinterpret_cast<const f32x4 *>(stage[0] + qd * 4);
+        if (live_b(bi, rt, ct)) *reinterpret_cast<f32x4 *>(ob + qd * 4) = *reinterpret_cast<const f32x4 *>(stage[1] + qd * 4);
     }
 }
 
@@ -583,10 +592,10 @@ void chunkwise_backward_coefficients(const float *alpha, const float *theta, con
                                      float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s) {
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     if (has_s)
-        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
                            eta, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
     else
-        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ceil_div(ntask, 2)), dim3(256), 0, stream(), alpha, theta,
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
                            nullptr, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
     check_launch("cw_coef_bwd_kernel");
 }
