@@ -30,6 +30,11 @@
 
 namespace nlh {
 
+static __global__ void zero_fill_kernel(float *__restrict__ p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
 // ───────────────────────────── forward ─────────────────────────────────────
 struct FwdArgs {
     const float *k, *v, *q, *alpha, *theta, *eta, *m_initial, *s_initial;
@@ -674,8 +679,11 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
     float *seed_m = scratch(8, 2 * batch * dd * sizeof(float));
     float *seed_s = HAS_S ? scratch(9, 2 * batch * dd * sizeof(float)) : nullptr;
     if (failed()) return;
-    check_hip(hipMemsetAsync(seed_m, 0, batch * dd * sizeof(float), stream()), "memset seed");
-    if (HAS_S) check_hip(hipMemsetAsync(seed_s, 0, batch * dd * sizeof(float), stream()), "memset seed");
+    // cleared by a kernel, not a memset node: the call stays replayable inside a captured graph
+    const size_t nseed = (size_t)batch * dd;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(ceil_div(nseed, 256)), dim3(256), 0, stream(), seed_m, nseed);
+    if (HAS_S) hipLaunchKernelGGL(zero_fill_kernel, dim3(ceil_div(nseed, 256)), dim3(256), 0, stream(), seed_s, nseed);
+    check_launch("zero_fill_kernel");
     const int nseg = ceil_div(seq_len, C);
     int cur = 0;
     for (int g = nseg - 1; g >= 0; g--) {

@@ -98,6 +98,13 @@ class MagLayer:
         self.m_state: List[Optional[torch.Tensor]] = [None] * k
         self.s_state: List[Optional[torch.Tensor]] = [None] * k
 
+    def ensure_state(self, bs):
+        """Creates the (zero) context memories of every level for batch size bs if they do not exist."""
+        for lv in range(self.k):
+            if self.m_state[lv] is None:
+                self.m_state[lv] = _zeros(bs * self.nh, self.hd * self.hd)
+                self.s_state[lv] = _zeros(bs * self.nh, self.hd * self.hd)
+
     # ── one level ────────────────────────────────────────────────────────────
     def _level_forward(self, lv, x2, bs, s, active):
         """gpu_memory_forward: projections, L2 norm, gates, head split, recurrence."""
@@ -144,7 +151,9 @@ class MagLayer:
             D.call("titans_chunkwise_forward_bf16_rocm", kh, vh, qh, ah, th, eh, self.m_state[lv],
                    self.s_state[lv], mc, sc, yh, s, hd, B, C)
         # context memory carries over to the next step (copy_final_m_batch, gpu_forward.rs:2824)
-        self.m_state[lv], self.s_state[lv] = mc[:, -1].contiguous(), sc[:, -1].contiguous()
+        # (in place: the buffers keep their addresses, so a captured step can be replayed)
+        self.m_state[lv].copy_(mc[:, -1])
+        self.s_state[lv].copy_(sc[:, -1])
         D.call("transpose_heads_f32_cuda", yh, y, bs, s, nh, hd, 0)
         c.update(alpha=alpha, theta=theta, eta=eta, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc)
         return y, c
@@ -263,6 +272,51 @@ class MagTrainer:
             self.state.append((m, v))
             self.opt.add_tensor(grp, w, g, m, v)
         self.scale = torch.zeros(2, dtype=torch.float32, device="cuda")
+
+    def _forward_backward(self, x, d_out):
+        out, cache = self.layer.forward(x)
+        _, g = self.layer.backward(cache, d_out)
+        for dst, src in zip(self.grads.tensors(), g.tensors()):
+            dst.copy_(src)
+        return out
+
+    def step_graphed(self, x, d_out):
+        """One training step with a given upstream gradient.  Forward + backward (some 330 launches,
+        launch-bound on the host) are replayed from a HIP graph captured once per pulse pattern and
+        input shape; the optimizer runs eagerly, its bias corrections change every step.  Returns the
+        layer output (a buffer the next replay overwrites)."""
+        layer = self.layer
+        layer.conductor.set_seq_len(x.shape[1])
+        pulse = layer.conductor.pulse()
+        key = (tuple(bool(a) for a in pulse.active_levels), tuple(x.shape))
+        graphs = self.__dict__.setdefault("_graphs", {})
+        if key not in graphs:
+            xs, ds = x.clone(), d_out.clone()
+            # Warm-up on a side stream sizes every scratch buffer (nothing may allocate while a graph
+            # is captured); it advances the context memories, which are put back afterwards.
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                lib.nlh_set_stream(ctypes.c_void_p(side.cuda_stream))
+                layer.ensure_state(x.shape[0])
+                saved = [(m.clone(), z.clone()) for m, z in zip(layer.m_state, layer.s_state)]
+                self._forward_backward(xs, ds)
+                for (m, z), m0, z0 in zip(saved, layer.m_state, layer.s_state):
+                    m0.copy_(m); z0.copy_(z)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                lib.nlh_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+                out = self._forward_backward(xs, ds)
+            lib.nlh_set_stream(None)
+            graphs[key] = (graph, xs, ds, out)
+        graph, xs, ds, out = graphs[key]
+        xs.copy_(x)
+        ds.copy_(d_out)
+        graph.replay()
+        self.opt.step(pulse, self.lr, self.max_grad_norm, self.scale)
+        layer.conductor.advance()
+        return out
 
     def step(self, x, d_out_fn):
         """One training step; d_out_fn(out) gives the upstream gradient.  Returns out."""
