@@ -260,6 +260,10 @@ void sigmoid_backward_cuda(const float *d_gate, const float *gate, float *d_x, i
 /* core/src/cuda_ffi.rs:569 / 572: round-to-nearest-even */
 void f32_to_bf16_cuda(const float *src, uint16_t *dst, int n);
 void bf16_to_f32_cuda(const uint16_t *src, float *dst, int n);
+/* Operand packing for a split-bf16 GEMM (no counterpart in the reference, whose projections are
+ * fp32 cuBLAS calls): row r of out [n, 3*count*d] = [hi(src0..) | lo(src0..) | hi(src0..)] with
+ * x = hi + lo, hi = bf16(x), lo = bf16(x - hi); srcs: count (1..4) host-side pointers to [n, d] floats. */
+void split_pack_bf16_rocm(const float *const *srcs, int count, uint16_t *out, long long n, int d);
 /* core/src/cuda_ffi.rs:579: gate[t] = act(k_t.w[:d] + v_t.w[d:] + *bias_ptr);
  * activation 0 = sigmoid, 1 = softplus (identity above 20) */
 void gate_compute_cuda(const float *k_mem, const float *v_mem, const float *w_gate,

@@ -414,6 +414,40 @@ void f32_to_bf16_cuda(const float *src, uint16_t *dst, int n) {
 void bf16_to_f32_cuda(const uint16_t *src, float *dst, int n) {
     launch_map(n, aligned16(dst) && ((((uintptr_t)src) & 7) == 0), FromBf16F{src, dst}, "bf16_to_f32");
 }
+// Operand packing of the split-bf16 GEMMs: row r of out is [hi(src0 .. src{count-1}) | lo(..) | hi(..)],
+// 3*count*d bf16 values, where x = hi + lo with hi = bf16(x), lo = bf16(x - hi).
+struct SplitSrcs { const float *p[4]; };
+__global__ void split_pack_bf16_kernel(SplitSrcs src, int count, uint16_t *__restrict__ out, long long n, int d) {
+    const int d4 = d / 4;
+    const long long total = n * count * d4;
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+         e += (long long)gridDim.x * blockDim.x) {
+        const int c4 = (int)(e % d4), sidx = (int)((e / d4) % count);
+        const long long r = e / ((long long)d4 * count);
+        const float4 x = *reinterpret_cast<const float4 *>(src.p[sidx] + r * d + c4 * 4);
+        const __bf16 h0 = (__bf16)x.x, h1 = (__bf16)x.y, h2 = (__bf16)x.z, h3 = (__bf16)x.w;
+        const __bf16 l0 = (__bf16)(x.x - (float)h0), l1 = (__bf16)(x.y - (float)h1), l2 = (__bf16)(x.z - (float)h2),
+                     l3 = (__bf16)(x.w - (float)h3);
+        typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+        uint16_t *o = out + r * (3LL * count * d) + (long long)sidx * d + c4 * 4;
+        const bf4 hv = {h0, h1, h2, h3}, lv = {l0, l1, l2, l3};
+        *reinterpret_cast<bf4 *>(o) = hv;
+        *reinterpret_cast<bf4 *>(o + (long long)count * d) = lv;
+        *reinterpret_cast<bf4 *>(o + 2LL * count * d) = hv;
+    }
+}
+void split_pack_bf16_rocm(const float *const *srcs, int count, uint16_t *out, long long n, int d) {
+    if (n <= 0) return;
+    if (count < 1 || count > 4 || d <= 0 || d % 4) {
+        fail("split_pack_bf16_rocm: count=%d must be 1..4 and d=%d a multiple of 4.", count, d);
+        return;
+    }
+    SplitSrcs s{};
+    for (int i = 0; i < count; i++) s.p[i] = srcs[i];
+    hipLaunchKernelGGL(split_pack_bf16_kernel, dim3(ew_blocks(n * count * (d / 4))), dim3(kEwThreads), 0, stream(), s,
+                       count, out, n, d);
+    check_launch("split_pack_bf16_kernel");
+}
 void saxpy_cuda(float alpha, const float *x, float *y, int n) {
     launch_map(n, aligned16(x) && aligned16(y), SaxpyF{alpha, x, y}, "saxpy");
 }

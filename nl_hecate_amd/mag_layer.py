@@ -111,18 +111,35 @@ class MagLayer:
     # x W^T ~ xh Wh^T + xl Wh^T + xh Wl^T as ONE bf16 GEMM with fp32 accumulation and fp32 output over the
     # tripled contraction [xh | xl | xh] . [Wh | Wh | Wl]^T.  Agrees with the fp32 GEMM to 5e-6 and runs
     # about three times faster on the bf16 matrix cores; the operand copies are made once per step.
+    # The backward's d_x = sum_s d_s W_s of a group of three projections is the same construction with
+    # the three upstream gradients side by side: [H | L | H] (9d wide) against [Wh^T | Wh^T | Wl^T].
+    @staticmethod
+    def _pack_split(srcs):
+        """[n, d] float tensors -> [n, 3*len*d] bf16: [hi(all) | lo(all) | hi(all)] (one pass)."""
+        n, d = srcs[0].shape
+        out = _new(n, 3 * len(srcs) * d, dtype=torch.bfloat16)
+        ptrs = (ctypes.c_void_p * len(srcs))(*[t.data_ptr() for t in srcs])
+        lib.split_pack_bf16_rocm(ptrs, len(srcs), out.data_ptr(), n, d)
+        return out
+
     def _split_operands(self, x2):
-        xh = x2.to(torch.bfloat16)
-        xl = (x2 - xh.float()).to(torch.bfloat16)
+        d, groups = self.d, 1 + self.k
         wh = self._pack.to(torch.bfloat16)
         wl = (self._pack - wh.float()).to(torch.bfloat16)
-        return torch.cat([xh, xl, xh], 1), torch.cat([wh, wh, wl], 1)
+        wht, wlt = (w.view(groups, 3 * d, d).transpose(1, 2) for w in (wh, wl))   # [group, d_in, 3 d_out]
+        return self._pack_split([x2]), torch.cat([wh, wh, wl], 1), torch.cat([wht, wht, wlt], 2).contiguous()
+
+    def _input_grad(self, ops, group, grads3, weights3):
+        """sum_s grads3[s] @ weights3[s] for projection group `group` (0: attention q, k, v; 1 + lv: level k, v, q)."""
+        if ops is None:
+            return grads3[0] @ weights3[0] + grads3[1] @ weights3[1] + grads3[2] @ weights3[2]
+        return torch.mm(self._pack_split(list(grads3)), ops[2][group].t(), out_dtype=torch.float32)
 
     def _project(self, ops, x2, w, index):
         """x2 @ w^T for the packed projection number `index` (w is its fp32 view)."""
         if ops is None:
             return x2 @ w.t()
-        xa, wb = ops
+        xa, wb = ops[0], ops[1]
         d = self.d
         return torch.mm(xa, wb[index * d:(index + 1) * d].t(), out_dtype=torch.float32)
 
@@ -156,7 +173,7 @@ class MagLayer:
         k_norms, q_norms = _new(n), _new(n)
         D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
         D.call("l2_normalize_rows_f32_cuda", q_mem, q_norms, n, d, 1e-8)
-        c = dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, k_norms=k_norms, q_norms=q_norms, active=active)
+        c = dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, k_norms=k_norms, q_norms=q_norms, active=active, ops=ops)
         alpha, theta, eta = _new(n), _new(n), _new(n)
         D.call("gate_compute_cuda", k_mem, v_mem, lp.w_alpha, lp.b_alpha, alpha, n, d, 0)
         D.call("gate_compute_cuda", k_mem, v_mem, lp.w_theta, lp.b_theta, theta, n, d, 1)
@@ -226,7 +243,7 @@ class MagLayer:
         g.w_k += _wgrad(dk_in, x2)
         g.w_v += _wgrad(dv, x2)
         g.w_q += _wgrad(dq_in, x2)
-        return dk_in @ lp.w_k + dv @ lp.w_v + dq_in @ lp.w_q
+        return self._input_grad(c.get("ops"), 1 + lv, (dk_in, dv, dq_in), (lp.w_k, lp.w_v, lp.w_q))
 
     # ── the layer ────────────────────────────────────────────────────────────
     def forward(self, x):
@@ -254,7 +271,7 @@ class MagLayer:
                                   gated.data_ptr(), bs * s * d)
         out = (gated.view(bs * s, d) @ p.w_o.t()).view(bs, s, d)
         cache = dict(x=x, q=q, k=k, v=v, aw=aw, attn=attn, gate=gate, gated=gated, levels=caches, pulse=pulse,
-                     ys=ys)
+                     ys=ys, ops=ops)
         return out, cache
 
     def backward(self, cache, d_out):
@@ -281,7 +298,7 @@ class MagLayer:
         grads.w_q += _wgrad(dq2, x2)
         grads.w_k += _wgrad(dk2, x2)
         grads.w_v += _wgrad(dv2, x2)
-        d_x += dq2 @ p.w_q + dk2 @ p.w_k + dv2 @ p.w_v
+        d_x += self._input_grad(cache["ops"], 0, (dq2, dk2, dv2), (p.w_q, p.w_k, p.w_v))
         return d_x.view(bs, s, d), grads
 
 
