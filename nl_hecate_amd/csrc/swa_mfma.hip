@@ -50,6 +50,22 @@ __device__ __forceinline__ f32x4 mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
 }
 
+// Workgroup -> (block of the sequence, head * batch) with all blocks of one head on one XCD.
+// Workgroups go to the 8 XCDs round robin in linear order, and each XCD has its own L2; blocks
+// of one head share K and V rows, so they are given linear ids that are equal modulo 8.
+struct BlockCoord { int x, h, b; };
+__device__ __forceinline__ BlockCoord xcd_block_coord(int H) {
+    const int gx = gridDim.x, heads = gridDim.y * gridDim.z;
+    const int lin = blockIdx.x + gx * (blockIdx.y + gridDim.y * blockIdx.z);
+    int x = blockIdx.x, bh = blockIdx.y + gridDim.y * blockIdx.z;
+    if ((heads & 7) == 0) {
+        const int xcd = lin & 7, slot = lin >> 3;
+        bh = (slot / gx) * 8 + xcd;
+        x = slot % gx;
+    }
+    return BlockCoord{x, bh % H, bh / H};
+}
+
 __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
                                                            const unsigned short *__restrict__ k,
                                                            const unsigned short *__restrict__ v,
@@ -59,7 +75,8 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage (row-major), then V^T stage [d][key]
     __shared__ __align__(16) unsigned short Pw[4][16][KS];    // per wave: normalised weights of one stage
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const int t0 = blockIdx.x * QB, h = blockIdx.y, b = blockIdx.z;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * QB, h = bc.h, b = bc.b;
     const int total = H * HD, hoff = h * HD;
     const int base = t0 + QB - NS * KS;               // first key of stage 0 (may be negative)
     const int tq = t0 + 16 * wave + r;                // this lane's query (column of S^T)
@@ -85,6 +102,16 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
             regs[c] = make_uint4(0, 0, 0, 0);
             if (key >= 0 && key < s)
                 regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + 8 * (chunk & 7));
+        }
+    };
+    // rows for a transposed stage: the thread takes 8 dims of two neighbouring keys
+    auto load_pairs = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
+        const int kp = tid & 31, d0 = 8 * (tid >> 5);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int key = base + KS * stage + 2 * kp + c;
+            regs[c] = make_uint4(0, 0, 0, 0);
+            if (key >= 0 && key < s) regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + d0);
         }
     };
     uint4 stg[2];
@@ -146,24 +173,24 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     for (int i = 0; i < 4; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
     __syncthreads();   // every wave is done with the last K stage
-    load_rows(v, st_lo, stg);
+    load_pairs(v, st_lo, stg);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
         const int buf = st & 1;
-        // transposed staging: chunk = (key, 8 dims) -> Vt[dim][key]
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, key = chunk >> 3, d0 = 8 * (chunk & 7);
-            const unsigned w[4] = {stg[c].x, stg[c].y, stg[c].z, stg[c].w};
+        // transposed staging as 32-bit key pairs (bank = key pair: no conflicts): Vt[dim][key]
+        {
+            const int kp = tid & 31, d0 = 8 * (tid >> 5);
+            const unsigned e[4] = {stg[0].x, stg[0].y, stg[0].z, stg[0].w};
+            const unsigned o2[4] = {stg[1].x, stg[1].y, stg[1].z, stg[1].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                Ks[buf][d0 + 2 * j][key] = (unsigned short)(w[j] & 0xffffu);
-                Ks[buf][d0 + 2 * j + 1][key] = (unsigned short)(w[j] >> 16);
+                *reinterpret_cast<unsigned *>(&Ks[buf][d0 + 2 * j][2 * kp]) = (e[j] & 0xffffu) | (o2[j] << 16);
+                *reinterpret_cast<unsigned *>(&Ks[buf][d0 + 2 * j + 1][2 * kp]) = (e[j] >> 16) | (o2[j] & 0xffff0000u);
             }
         }
         __syncthreads();
-        if (st + 1 < NS) load_rows(v, st + 1, stg);
+        if (st + 1 < NS) load_pairs(v, st + 1, stg);
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
             f32x4 p = acc[4 * st + kt];
@@ -214,20 +241,25 @@ __device__ __forceinline__ void split4(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
     }
 }
 
-// Backward, query pass (one workgroup per 64 queries): D_t = sum_j w dW and
-//   d_q[t] = sum_j dS[t,j] k_j,  dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd)
-// on the stored (bf16) weights.  Same tiling as the forward; dO and dS enter the bf16
-// products as hi + lo pairs.  D_t goes to dvec for the key pass.
-__global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
-                                                             const unsigned short *__restrict__ v,
-                                                             const unsigned short *__restrict__ attn_w,
-                                                             const float *__restrict__ d_out,
-                                                             float *__restrict__ d_q, float *__restrict__ dvec,
-                                                             int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short St[2][KS][LDH];
-    __shared__ __align__(16) unsigned short Pw[4][16][KS];
+// Backward, query pass (one workgroup per 64 queries, one wave per 16 queries):
+//   D_t = sum_j w dW = dO_t . O_t with O_t = sum_j w[t,j] v_j recomputed from the stored (bf16) weights,
+//   dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd),  d_q[t] = sum_j dS[t,j] k_j.
+// Two sweeps over the window: the first rebuilds O^T (four accumulators) and from it D; the second
+// recomputes each dW tile next to its use, so no score tile outlives a stage and the kernel fits
+// two to three workgroups per compute unit.  dO and dS enter the bf16 products as hi + lo pairs.
+// D_t goes to dvec for the key pass.
+__global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
+                                                                const unsigned short *__restrict__ v,
+                                                                const unsigned short *__restrict__ attn_w,
+                                                                const float *__restrict__ d_out,
+                                                                float *__restrict__ d_q, float *__restrict__ dvec,
+                                                                int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [key][dim]
+    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][key]: V (sweep 1), K (sweep 2)
+    __shared__ __align__(16) unsigned short Pw[4][16][KS];    // per wave: weights of one stage, [query][key]
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const int t0 = blockIdx.x * QB, h = blockIdx.y, b = blockIdx.z;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * QB, h = bc.h, b = bc.b;
     const int total = H * HD, hoff = h * HD;
     const int base = t0 + QB - NS * KS;
     const int tq = t0 + 16 * wave + r;
@@ -235,16 +267,14 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
     const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
     const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
 
+    f32x4 dof[4];     // dO_t at dims 16 sp + 4 g .. +3: the positions of this lane in an O^T tile
     bf16x4 doh[4], dol[4];
 #pragma unroll
     for (int sp = 0; sp < 4; sp++) {
-        f32x4 x = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (tq < s) x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * sp + 4 * g);
-        split4(x, doh[sp], dol[sp]);
+        dof[sp] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (tq < s) dof[sp] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * sp + 4 * g);
+        split4(dof[sp], doh[sp], dol[sp]);
     }
-    f32x4 acc[NT];
-#pragma unroll
-    for (int i = 0; i < NT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     auto load_rows = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
 #pragma unroll
@@ -253,6 +283,34 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
             regs[c] = make_uint4(0, 0, 0, 0);
             if (key >= 0 && key < s)
                 regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + 8 * (chunk & 7));
+        }
+    };
+    auto commit_rows = [&](int buf, const uint4 (&regs)[2]) {
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Vr[buf][chunk >> 3][8 * (chunk & 7)]) = regs[c];
+        }
+    };
+    // rows for a transposed stage: the thread takes 8 dims of two neighbouring keys, so that the
+    // transposed tile is written as 32-bit key pairs (bank = key pair: no conflicts)
+    auto load_pairs = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
+        const int kp = tid & 31, d0 = 8 * (tid >> 5);
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int key = base + KS * stage + 2 * kp + c;
+            regs[c] = make_uint4(0, 0, 0, 0);
+            if (key >= 0 && key < s) regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + d0);
+        }
+    };
+    auto commit_transposed = [&](int buf, const uint4 (&regs)[2]) {
+        const int kp = tid & 31, d0 = 8 * (tid >> 5);
+        const unsigned e[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
+        const unsigned o[4] = {regs[1].x, regs[1].y, regs[1].z, regs[1].w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j][2 * kp]) = (e[j] & 0xffffu) | (o[j] << 16);
+            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j + 1][2 * kp]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
         }
     };
     // this wave's 16 weight rows for the 64 keys of a stage (zero outside the slot range):
@@ -272,78 +330,76 @@ __global__ __launch_bounds__(256) void swa_bwd_q_mfma_kernel(const unsigned shor
         for (int qi = 0; qi < 16; qi++) Pw[wave][qi][l] = wreg[qi];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
-    uint4 stg[2];
+    uint4 sv[2], sk[2];
 
-    // ---- sweep 1: dW^T tiles and D ----
-    float dsum = 0.f;
-    load_rows(v, st_lo, stg);
+    // ---- sweep 1: O^T = V^T P^T, then D = dO . O ----
+    f32x4 ot[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    load_pairs(v, st_lo, sv);
     fetch_weights(st_lo);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
+#pragma unroll 1
+    for (int st = st_lo; st < NS; st++) {
         const int buf = st & 1;
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c;
-            *reinterpret_cast<uint4 *>(&St[buf][chunk >> 3][8 * (chunk & 7)]) = stg[c];
-        }
+        commit_transposed(buf, sv);
         commit_weights();
         __syncthreads();
-        if (st + 1 < NS) { load_rows(v, st + 1, stg); fetch_weights(st + 1); }
+        if (st + 1 < NS) { load_pairs(v, st + 1, sv); fetch_weights(st + 1); }
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
-#pragma unroll
-            for (int sp = 0; sp < 4; sp++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&St[buf][16 * kt + r][16 * sp + 4 * g]);
-                acc[4 * st + kt] = mfma16(a, doh[sp], acc[4 * st + kt]);
-                acc[4 * st + kt] = mfma16(a, dol[sp], acc[4 * st + kt]);
-            }
             const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
 #pragma unroll
-            for (int i = 0; i < 4; i++) dsum = fmaf(bf2f((unsigned short)pb[i]), acc[4 * st + kt][i], dsum);
+            for (int dt = 0; dt < 4; dt++) {
+                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Tt[buf][16 * dt + r][16 * kt + 4 * g]);
+                ot[dt] = mfma16(a, pb, ot[dt]);
+            }
         }
         asm volatile("" ::: "memory");
     }
+    float dsum = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) dsum = fmaf(dof[dt][i], ot[dt][i], dsum);
     dsum += __shfl_xor(dsum, 16, 64);
     dsum += __shfl_xor(dsum, 32, 64);
     if (g == 0 && tq < s) dvec[(size_t)(b * H + h) * s + tq] = dsum;
 
-    // ---- sweep 2: d_q^T = K^T dS^T ----
+    // ---- sweep 2: dW^T tiles recomputed, dS, d_q^T = K^T dS^T ----
     f32x4 dq[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) dq[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     const float scale = 0.125f;
     __syncthreads();
-    load_rows(k, st_lo, stg);
+    load_rows(v, st_lo, sv);
+    load_pairs(k, st_lo, sk);
     fetch_weights(st_lo);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
+#pragma unroll 1
+    for (int st = st_lo; st < NS; st++) {
         const int buf = st & 1;
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, key = chunk >> 3, d0 = 8 * (chunk & 7);
-            const unsigned w[4] = {stg[c].x, stg[c].y, stg[c].z, stg[c].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                St[buf][d0 + 2 * j][key] = (unsigned short)(w[j] & 0xffffu);
-                St[buf][d0 + 2 * j + 1][key] = (unsigned short)(w[j] >> 16);
-            }
-        }
+        commit_rows(buf, sv);
+        commit_transposed(buf, sk);
         commit_weights();
         __syncthreads();
-        if (st + 1 < NS) { load_rows(k, st + 1, stg); fetch_weights(st + 1); }
+        if (st + 1 < NS) { load_rows(v, st + 1, sv); load_pairs(k, st + 1, sk); fetch_weights(st + 1); }
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
+            f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key 16 kt + 4 g + i][query r]
+#pragma unroll
+            for (int sp = 0; sp < 4; sp++) {
+                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Vr[buf][16 * kt + r][16 * sp + 4 * g]);
+                dw = mfma16(a, doh[sp], dw);
+                dw = mfma16(a, dol[sp], dw);
+            }
             const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
             f32x4 ds;
 #pragma unroll
-            for (int i = 0; i < 4; i++) ds[i] = bf2f((unsigned short)pb[i]) * (acc[4 * st + kt][i] - dsum) * scale;
+            for (int i = 0; i < 4; i++) ds[i] = bf2f((unsigned short)pb[i]) * (dw[i] - dsum) * scale;
             bf16x4 dsh, dsl;
             split4(ds, dsh, dsl);
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&St[buf][16 * dt + r][16 * kt + 4 * g]);
+                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Tt[buf][16 * dt + r][16 * kt + 4 * g]);
                 dq[dt] = mfma16(a, dsh, dq[dt]);
                 dq[dt] = mfma16(a, dsl, dq[dt]);
             }
@@ -375,7 +431,8 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
     __shared__ float Dv[KS];
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const int j0 = blockIdx.x * QB, h = blockIdx.y, b = blockIdx.z;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int j0 = bc.x * QB, h = bc.h, b = bc.b;
     const int total = H * HD, hoff = h * HD;
     const size_t row0 = (size_t)b * s;
     const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
@@ -399,19 +456,25 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     uint4 gq[2];
     unsigned short gw[16];
     float gd = 0.f;
+    const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // dO: query pair, first dim (+32 for the second half)
+    const int qpair = tid & 31, qd0 = 8 * (tid >> 5);                        // Q: query pair, first dim
     auto fetch_stage = [&](int st) {
         const int qs0 = j0 + KS * st;
+        // dO: query pair (2 rows) x 4 dims per load, Q: query pair x 8 dims; pairs so that the
+        // transposed tiles are written as 32-bit words without bank conflicts
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int chunk = tid + 256 * c, t = qs0 + (chunk >> 4);
-            gdo[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (t < s) gdo[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + 4 * (chunk & 15));
-        }
+        for (int cc = 0; cc < 2; cc++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int t = qs0 + 2 * dpair + c;
+                gdo[2 * cc + c] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (t < s) gdo[2 * cc + c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dd0 + 32 * cc);
+            }
 #pragma unroll
         for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, t = qs0 + (chunk >> 3);
+            const int t = qs0 + 2 * qpair + c;
             gq[c] = make_uint4(0, 0, 0, 0);
-            if (t < s) gq[c] = *reinterpret_cast<const uint4 *>(q + (row0 + t) * total + hoff + 8 * (chunk & 7));
+            if (t < s) gq[c] = *reinterpret_cast<const uint4 *>(q + (row0 + t) * total + hoff + qd0);
         }
         // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t)
 #pragma unroll
@@ -429,23 +492,29 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
         if (qs0 > t_last) break;
         __syncthreads();   // previous stage's readers are done
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int chunk = tid + 256 * c, qi = chunk >> 4, d0 = 4 * (chunk & 15);
-            bf16x4 hi, lo;
-            split4(gdo[c], hi, lo);
-            *reinterpret_cast<bf16x4 *>(&Dh[qi][d0]) = hi;
-            *reinterpret_cast<bf16x4 *>(&Dl[qi][d0]) = lo;
+        for (int cc = 0; cc < 2; cc++) {
+            bf16x4 hi[2], lo[2];
 #pragma unroll
-            for (int j = 0; j < 4; j++) { DhT[d0 + j][qi] = (unsigned short)hi[j]; DlT[d0 + j][qi] = (unsigned short)lo[j]; }
-        }
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, qi = chunk >> 3, d0 = 8 * (chunk & 7);
-            const unsigned w[4] = {gq[c].x, gq[c].y, gq[c].z, gq[c].w};
+            for (int c = 0; c < 2; c++) {
+                split4(gdo[2 * cc + c], hi[c], lo[c]);
+                *reinterpret_cast<bf16x4 *>(&Dh[2 * dpair + c][dd0 + 32 * cc]) = hi[c];
+                *reinterpret_cast<bf16x4 *>(&Dl[2 * dpair + c][dd0 + 32 * cc]) = lo[c];
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                QT[d0 + 2 * j][qi] = (unsigned short)(w[j] & 0xffffu);
-                QT[d0 + 2 * j + 1][qi] = (unsigned short)(w[j] >> 16);
+                *reinterpret_cast<unsigned *>(&DhT[dd0 + 32 * cc + j][2 * dpair]) =
+                    (unsigned)(unsigned short)hi[0][j] | ((unsigned)(unsigned short)hi[1][j] << 16);
+                *reinterpret_cast<unsigned *>(&DlT[dd0 + 32 * cc + j][2 * dpair]) =
+                    (unsigned)(unsigned short)lo[0][j] | ((unsigned)(unsigned short)lo[1][j] << 16);
+            }
+        }
+        {
+            const unsigned e[4] = {gq[0].x, gq[0].y, gq[0].z, gq[0].w};
+            const unsigned o[4] = {gq[1].x, gq[1].y, gq[1].z, gq[1].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                *reinterpret_cast<unsigned *>(&QT[qd0 + 2 * j][2 * qpair]) = (e[j] & 0xffffu) | (o[j] << 16);
+                *reinterpret_cast<unsigned *>(&QT[qd0 + 2 * j + 1][2 * qpair]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
             }
         }
 #pragma unroll
