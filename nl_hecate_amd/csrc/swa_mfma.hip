@@ -245,27 +245,38 @@ __device__ __forceinline__ void split4(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
 //   D_t = sum_j w dW = dO_t . O_t with O_t = sum_j w[t,j] v_j recomputed from the stored (bf16) weights,
 //   dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd),  d_q[t] = sum_j dS[t,j] k_j.
 // Two sweeps over the window: the first rebuilds O^T (four accumulators) and from it D; the second
-// recomputes each dW tile next to its use, so no score tile outlives a stage and the kernel fits
-// two to three workgroups per compute unit.  dO and dS enter the bf16 products as hi + lo pairs.
-// D_t goes to dvec for the key pass.
+// recomputes each dW tile next to its use, so no score tile outlives a stage.  dO and dS enter the
+// bf16 products as hi + lo pairs.  D_t goes to dvec for the key pass.
+//
+// The weights never pass through LDS.  Within a stage of 64 keys, element i of lane group g in
+// 16-key tile kt stands for key 32 (kt / 2) + 8 g + 4 (kt % 2) + i, so that the B operands of one
+// query for two tiles are 8 consecutive slots of its weight row: one 16-byte load (2-byte aligned)
+// per lane, kept in registers for the second sweep.  The LDS tiles of V and K are stored in that key
+// order (stage_pos).  Only the last stage, the one that holds the queries themselves, is read slot
+// by slot: its groups can end inside the 16 bytes, and a load that runs past the query's row would
+// leave the array at its last row.
+__device__ __forceinline__ int stage_pos(int key) {   // key 32 a + 8 g + 4 c + i -> 16 (2 a + c) + 4 g + i
+    return (key & 0x23) | ((key & 0x18) >> 1) | ((key & 0x04) << 2);
+}
+
 __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
                                                                 const unsigned short *__restrict__ v,
                                                                 const unsigned short *__restrict__ attn_w,
                                                                 const float *__restrict__ d_out,
                                                                 float *__restrict__ d_q, float *__restrict__ dvec,
                                                                 int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [key][dim]
-    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][key]: V (sweep 1), K (sweep 2)
-    __shared__ __align__(16) unsigned short Pw[4][16][KS];    // per wave: weights of one stage, [query][key]
+    __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [stage_pos(key)][dim]
+    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][stage_pos(key)]: V (sweep 1), K (sweep 2)
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * QB, h = bc.h, b = bc.b;
     const int total = H * HD, hoff = h * HD;
     const int base = t0 + QB - NS * KS;
     const int tq = t0 + 16 * wave + r;
+    const int lsq = max(tq + 1 - ws, 0);
     const size_t row0 = (size_t)b * s;
     const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
-    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+    const unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
 
     f32x4 dof[4];     // dO_t at dims 16 sp + 4 g .. +3: the positions of this lane in an O^T tile
     bf16x4 doh[4], dol[4];
@@ -289,7 +300,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
 #pragma unroll
         for (int c = 0; c < 2; c++) {
             const int chunk = tid + 256 * c;
-            *reinterpret_cast<uint4 *>(&Vr[buf][chunk >> 3][8 * (chunk & 7)]) = regs[c];
+            *reinterpret_cast<uint4 *>(&Vr[buf][stage_pos(chunk >> 3)][8 * (chunk & 7)]) = regs[c];
         }
     };
     // rows for a transposed stage: the thread takes 8 dims of two neighbouring keys, so that the
@@ -304,31 +315,53 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
         }
     };
     auto commit_transposed = [&](int buf, const uint4 (&regs)[2]) {
-        const int kp = tid & 31, d0 = 8 * (tid >> 5);
+        const int col = stage_pos(2 * (tid & 31)), d0 = 8 * (tid >> 5);
         const unsigned e[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
         const unsigned o[4] = {regs[1].x, regs[1].y, regs[1].z, regs[1].w};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j][2 * kp]) = (e[j] & 0xffffu) | (o[j] << 16);
-            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j + 1][2 * kp]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
+            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j][col]) = (e[j] & 0xffffu) | (o[j] << 16);
+            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j + 1][col]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
         }
     };
-    // this wave's 16 weight rows for the 64 keys of a stage (zero outside the slot range):
-    // fetched into registers one stage ahead, then written to the wave's LDS tile
-    unsigned short wreg[16];
-    auto fetch_weights = [&](int stage) {
+    // weights of this lane's query for the keys of its group in a stage: wv[stage][half] holds the
+    // 8 keys 32 half + 8 g .. + 7 (B operands of tiles 2 half and 2 half + 1), zero outside the window
+    uint4 wv[NS][2];
+    auto fetch_weights = [&](int stage, uint4 (&w)[2]) {
 #pragma unroll
-        for (int qi = 0; qi < 16; qi++) {
-            const int tt = t0 + 16 * wave + qi, key = base + KS * stage + l;
-            const int slot = key - max(tt + 1 - ws, 0);
-            wreg[qi] = 0;
-            if (tt < s && key <= tt && slot >= 0 && slot < ws) wreg[qi] = awb[(size_t)tt * ws + slot];
+        for (int hf = 0; hf < 2; hf++) {
+            const int key0 = base + KS * stage + 32 * hf + 8 * g;
+            w[hf] = make_uint4(0, 0, 0, 0);
+            if (stage < NS - 1) {
+                // keys below t0: the group never runs past the query; it may start before the window
+                if (tq < s && key0 + 7 >= lsq) {
+                    uint4 x;
+                    __builtin_memcpy(&x, wrow + (key0 - lsq), 16);
+                    const int cut = lsq - key0;   // elements below cut are outside the window
+                    x.x &= (cut > 0 ? 0u : 0xffffu) | (cut > 1 ? 0u : 0xffff0000u);
+                    x.y &= (cut > 2 ? 0u : 0xffffu) | (cut > 3 ? 0u : 0xffff0000u);
+                    x.z &= (cut > 4 ? 0u : 0xffffu) | (cut > 5 ? 0u : 0xffff0000u);
+                    x.w &= (cut > 6 ? 0u : 0xffffu) | (cut > 7 ? 0u : 0xffff0000u);
+                    w[hf] = x;
+                }
+            } else {
+                unsigned d[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int key = key0 + e;
+                    unsigned x = 0;
+                    if (tq < s && key >= lsq && key <= tq) x = wrow[key - lsq];
+                    d[e >> 1] |= x << (16 * (e & 1));
+                }
+                w[hf] = make_uint4(d[0], d[1], d[2], d[3]);
+            }
         }
     };
-    auto commit_weights = [&]() {
-#pragma unroll
-        for (int qi = 0; qi < 16; qi++) Pw[wave][qi][l] = wreg[qi];
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    auto b_operand = [&](const uint4 &w, int odd) {
+        const unsigned lo = odd ? w.z : w.x, hi = odd ? w.w : w.y;
+        bf16x4 pb;
+        pb[0] = (short)(lo & 0xffffu); pb[1] = (short)(lo >> 16); pb[2] = (short)(hi & 0xffffu); pb[3] = (short)(hi >> 16);
+        return pb;
     };
     uint4 sv[2], sk[2];
 
@@ -336,25 +369,26 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
     f32x4 ot[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < NS; st++) { wv[st][0] = make_uint4(0, 0, 0, 0); wv[st][1] = make_uint4(0, 0, 0, 0); }
     load_pairs(v, st_lo, sv);
-    fetch_weights(st_lo);
-#pragma unroll 1
-    for (int st = st_lo; st < NS; st++) {
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        if (st < st_lo) continue;
         const int buf = st & 1;
+        fetch_weights(st, wv[st]);
         commit_transposed(buf, sv);
-        commit_weights();
         __syncthreads();
-        if (st + 1 < NS) { load_pairs(v, st + 1, sv); fetch_weights(st + 1); }
+        if (st + 1 < NS) load_pairs(v, st + 1, sv);
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
-            const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
+            const bf16x4 pb = b_operand(wv[st][kt >> 1], kt & 1);
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
                 const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Tt[buf][16 * dt + r][16 * kt + 4 * g]);
                 ot[dt] = mfma16(a, pb, ot[dt]);
             }
         }
-        asm volatile("" ::: "memory");
     }
     float dsum = 0.f;
 #pragma unroll
@@ -373,25 +407,24 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
     __syncthreads();
     load_rows(v, st_lo, sv);
     load_pairs(k, st_lo, sk);
-    fetch_weights(st_lo);
-#pragma unroll 1
-    for (int st = st_lo; st < NS; st++) {
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        if (st < st_lo) continue;
         const int buf = st & 1;
         commit_rows(buf, sv);
         commit_transposed(buf, sk);
-        commit_weights();
         __syncthreads();
-        if (st + 1 < NS) { load_rows(v, st + 1, sv); load_pairs(k, st + 1, sk); fetch_weights(st + 1); }
+        if (st + 1 < NS) { load_rows(v, st + 1, sv); load_pairs(k, st + 1, sk); }
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
-            f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key 16 kt + 4 g + i][query r]
+            f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key of (kt, g, i)][query r]
 #pragma unroll
             for (int sp = 0; sp < 4; sp++) {
                 const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Vr[buf][16 * kt + r][16 * sp + 4 * g]);
                 dw = mfma16(a, doh[sp], dw);
                 dw = mfma16(a, dol[sp], dw);
             }
-            const bf16x4 pb = *reinterpret_cast<const bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]);
+            const bf16x4 pb = b_operand(wv[st][kt >> 1], kt & 1);
             f32x4 ds;
 #pragma unroll
             for (int i = 0; i < 4; i++) ds[i] = bf2f((unsigned short)pb[i]) * (dw[i] - dsum) * scale;
@@ -404,7 +437,6 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
                 dq[dt] = mfma16(a, dsl, dq[dt]);
             }
         }
-        asm volatile("" ::: "memory");
     }
     if (tq < s) {
         float *ob = d_q + (row0 + tq) * total + hoff;

@@ -44,7 +44,8 @@ def gpu_backward(q, k, v, aw, go, ws, H, npers):
 
 @pytest.mark.parametrize("B,s,H,hd,ws,npers", [(2, 40, 2, 64, 16, 0), (1, 70, 3, 32, 64, 0),
                                                (2, 33, 2, 64, 8, 5), (1, 20, 1, 8, 32, 0),
-                                               (1, 600, 2, 64, 512, 0), (1, 50, 2, 24, 7, 3)])
+                                               (1, 600, 2, 64, 512, 0), (1, 50, 2, 24, 7, 3),
+                                               (2, 200, 2, 64, 101, 0), (1, 1100, 1, 64, 300, 0)])
 def test_swa_forward_backward_parity(B, s, H, hd, ws, npers):
     q, k, v, go = _case(B, s, H, hd, 100 + s + ws)
     out, aw = gpu_forward(q, k, v, ws, H, npers)
