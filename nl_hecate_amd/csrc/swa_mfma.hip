@@ -3,17 +3,29 @@
 // are those of core/kernels/swa_forward.cu / swa_backward.cu; other shapes stay
 // on the wave-per-query kernels of swa.hip.
 //
+// All products are v_mfma_f32_16x16x32_bf16 steps (a 16x16x16 step costs the same
+// cycles for half the work), so every operand is 8 consecutive contraction
+// elements per lane: lane (r = l % 16, g = l / 16) supplies row r, contraction
+// elements 8 g .. 8 g + 7 of a 32-wide step.
+//
+// Key order.  A 16x16 result tile leaves four rows 4 g + i in a lane.  Where such
+// tiles become an operand again with the keys as contraction index (the weights in
+// O^T = V^T P^T, dS in d_q^T = K^T dS^T), two tiles (c = 0, 1) of a 32-key half hf
+// give the lane its 8 elements; row 4 g + i of tile (hf, c) therefore stands for key
+// 32 hf + 8 g + 4 c + i of the stage, so that those 8 elements are 8 CONSECUTIVE
+// keys: the matching operand is a plain 16-byte LDS read, and in the weight array
+// they are 16 consecutive bytes of the query's slot row (a 2-byte aligned 16-byte
+// access).  A tile's rows come from an LDS matrix whose rows are stored in that
+// order (stage_pos).
+//
 // Forward.  One workgroup per (64 queries, head, batch), one wave per 16 queries.
 // The wave computes S^T = K Q^T for its 16 queries against the 576 keys
-// [t0-512, t0+64) that the block can see, 36 tiles of 16x16 kept in registers
-// (v_mfma_f32_16x16x16_bf16: A = 16 keys x 16 dims from an LDS-staged K tile,
-// B = the wave's Q fragment).  In this orientation a lane owns ONE query column
-// and 144 of its keys, so the softmax is a per-lane reduction plus two
-// exchanges, and the normalised tile is already laid out as the B operand of
+// [t0-512, t0+64) that the block can see, 36 tiles kept in registers.  A lane owns
+// ONE query column and 144 of its keys, so the softmax is a per-lane reduction plus
+// two exchanges, and the normalised tiles are already the B operand of
 // O^T = V^T P^T: no shuffles between the two products.  V tiles are staged
-// transposed in LDS.  The normalised weights (part of the contract) leave
-// through a per-wave LDS tile so that each store instruction writes 128
-// contiguous bytes of one query's slot row.
+// transposed in LDS.  The normalised weights (part of the contract) leave straight
+// from the operand registers.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -25,7 +37,8 @@
 namespace nlh {
 namespace {
 
-typedef short bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bh8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bh2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int HD = 64;        // head size
@@ -33,21 +46,42 @@ constexpr int QB = 64;        // queries per workgroup
 constexpr int KS = 64;        // keys per LDS stage
 constexpr int NS = 9;         // stages: 576 keys
 constexpr int NT = 36;        // 16-key tiles
-constexpr int LDH = 72;       // LDS row stride in bf16 elements (144 B: 16-byte aligned rows)
+constexpr int LDH = 72;       // LDS row stride in bf16 elements (144 B: 16-byte rows, conflict-free operand reads)
 
-__device__ __forceinline__ unsigned short f2bf(float f) {
-    unsigned u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (unsigned short)(u >> 16);
+__device__ __forceinline__ f32x4 mfma32(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bh8, a), __builtin_bit_cast(bh8, b), c, 0, 0, 0);
 }
-__device__ __forceinline__ bf16x4 pack4(f32x4 x) {
-    bf16x4 r;
-    r[0] = (short)f2bf(x[0]); r[1] = (short)f2bf(x[1]); r[2] = (short)f2bf(x[2]); r[3] = (short)f2bf(x[3]);
-    return r;
+// two floats -> two bf16 (round to nearest even) in one dword, x in the low half
+__device__ __forceinline__ unsigned pack2(float x, float y) {
+    const bh2 p = {(__bf16)x, (__bf16)y};
+    return __builtin_bit_cast(unsigned, p);
 }
-__device__ __forceinline__ f32x4 mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+__device__ __forceinline__ float bf_lo(unsigned w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf_hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
+// x, y = hi + lo with hi, lo bf16: the pair carries 16 mantissa bits through a bf16 product
+__device__ __forceinline__ void split2(float x, float y, unsigned &hi, unsigned &lo) {
+    hi = pack2(x, y);
+    lo = pack2(x - bf_lo(hi), y - bf_hi(hi));
+}
+__device__ __forceinline__ void split8(f32x4 a, f32x4 b, uint4 &hi, uint4 &lo) {
+    split2(a[0], a[1], hi.x, lo.x);
+    split2(a[2], a[3], hi.y, lo.y);
+    split2(b[0], b[1], hi.z, lo.z);
+    split2(b[2], b[3], hi.w, lo.w);
+}
+// position of a stage's key 32 a + 8 g + 4 c + i in tile order: 16 (2 a + c) + 4 g + i
+__device__ __forceinline__ int stage_pos(int key) {
+    return (key & 0x23) | ((key & 0x18) >> 1) | ((key & 0x04) << 2);
+}
+// key (relative to the stage) of element i of lane group g in tile kt
+__device__ __forceinline__ int tile_key(int kt, int g, int i) { return 32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i; }
+// clears the elements below cut of 8 packed bf16
+__device__ __forceinline__ uint4 mask_below(uint4 x, int cut) {
+    x.x &= (cut > 0 ? 0u : 0xffffu) | (cut > 1 ? 0u : 0xffff0000u);
+    x.y &= (cut > 2 ? 0u : 0xffffu) | (cut > 3 ? 0u : 0xffff0000u);
+    x.z &= (cut > 4 ? 0u : 0xffffu) | (cut > 5 ? 0u : 0xffff0000u);
+    x.w &= (cut > 6 ? 0u : 0xffffu) | (cut > 7 ? 0u : 0xffff0000u);
+    return x;
 }
 
 // Workgroup -> (block of the sequence, head * batch) with all blocks of one head on one XCD.
@@ -66,14 +100,62 @@ __device__ __forceinline__ BlockCoord xcd_block_coord(int H) {
     return BlockCoord{x, bh % H, bh / H};
 }
 
+// Cooperative loads of one stage (64 rows of 64 bf16 = 512 chunks of 16 B, two per thread of a
+// 256-thread block).  rows: chunk = (row, 8 dims), consecutive lanes along a row.  pairs: the thread
+// takes 8 dims of two neighbouring rows, for a transposed tile written as 32-bit row pairs.
+struct StageSrc { const unsigned short *p; size_t row0; int total, hoff, s; };
+__device__ __forceinline__ void load_rows(const StageSrc &m, int first, uint4 (&regs)[2]) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int chunk = tid + 256 * c, row = first + (chunk >> 3);
+        regs[c] = make_uint4(0, 0, 0, 0);
+        if (row >= 0 && row < m.s)
+            regs[c] = *reinterpret_cast<const uint4 *>(m.p + (m.row0 + row) * m.total + m.hoff + 8 * (chunk & 7));
+    }
+}
+__device__ __forceinline__ void load_pairs(const StageSrc &m, int first, uint4 (&regs)[2]) {
+    const int tid = threadIdx.x, kp = tid & 31, d0 = 8 * (tid >> 5);
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int row = first + 2 * kp + c;
+        regs[c] = make_uint4(0, 0, 0, 0);
+        if (row >= 0 && row < m.s) regs[c] = *reinterpret_cast<const uint4 *>(m.p + (m.row0 + row) * m.total + m.hoff + d0);
+    }
+}
+// rows in tile order: row -> T[stage_pos(row)][dim]
+__device__ __forceinline__ void commit_rows_tiled(unsigned short (*T)[LDH], const uint4 (&regs)[2]) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int chunk = tid + 256 * c;
+        *reinterpret_cast<uint4 *>(&T[stage_pos(chunk >> 3)][8 * (chunk & 7)]) = regs[c];
+    }
+}
+// transposed: T[dim][row], rows in natural order (bank = row pair: no conflicts)
+__device__ __forceinline__ void commit_transposed(unsigned short (*T)[LDH], const uint4 (&regs)[2]) {
+    const int tid = threadIdx.x, col = 2 * (tid & 31), d0 = 8 * (tid >> 5);
+    const unsigned e[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
+    const unsigned o[4] = {regs[1].x, regs[1].y, regs[1].z, regs[1].w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        *reinterpret_cast<unsigned *>(&T[d0 + 2 * j][col]) = (e[j] & 0xffffu) | (o[j] << 16);
+        *reinterpret_cast<unsigned *>(&T[d0 + 2 * j + 1][col]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
+    }
+}
+// operand of a 32-wide step: row r of the tile at row0, contraction elements 32 ks + 8 g .. + 7
+__device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int ks) {
+    const int l = threadIdx.x & 63;
+    return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
+}
+
 __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
                                                            const unsigned short *__restrict__ k,
                                                            const unsigned short *__restrict__ v,
                                                            unsigned short *__restrict__ out,
                                                            unsigned short *__restrict__ attn_w, int s, int H,
                                                            int ws) {
-    __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage (row-major), then V^T stage [d][key]
-    __shared__ __align__(16) unsigned short Pw[4][16][KS];    // per wave: normalised weights of one stage
+    __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage [stage_pos(key)][dim], then V^T stage [dim][key]
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * QB, h = bc.h, b = bc.b;
@@ -83,59 +165,32 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     const size_t row0 = (size_t)b * s;
     const int first_key = max(t0 + 1 - ws, 0);        // smallest key any query of the block sees
     const int st_lo = max(0, (first_key - base) / KS);   // stages before it hold masked keys only
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
 
-    bf16x4 qf[4];
+    uint4 qf[2];
 #pragma unroll
-    for (int st = 0; st < 4; st++) {
-        qf[st] = bf16x4{0, 0, 0, 0};
-        if (tq < s) qf[st] = *reinterpret_cast<const bf16x4 *>(q + (row0 + tq) * total + hoff + 16 * st + 4 * g);
+    for (int ks = 0; ks < 2; ks++) {
+        qf[ks] = make_uint4(0, 0, 0, 0);
+        if (tq < s) qf[ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
     }
     f32x4 acc[NT];
 #pragma unroll
     for (int i = 0; i < NT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // cooperative stage loads: 64 rows x 128 B = 512 chunks of 16 B, two per thread
-    auto load_rows = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, key = base + KS * stage + (chunk >> 3);
-            regs[c] = make_uint4(0, 0, 0, 0);
-            if (key >= 0 && key < s)
-                regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + 8 * (chunk & 7));
-        }
-    };
-    // rows for a transposed stage: the thread takes 8 dims of two neighbouring keys
-    auto load_pairs = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
-        const int kp = tid & 31, d0 = 8 * (tid >> 5);
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int key = base + KS * stage + 2 * kp + c;
-            regs[c] = make_uint4(0, 0, 0, 0);
-            if (key >= 0 && key < s) regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + d0);
-        }
-    };
     uint4 stg[2];
 
     // ---- pass A: S^T tiles ----
-    load_rows(k, st_lo, stg);
+    load_rows(km, base + KS * st_lo, stg);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
         const int buf = st & 1;
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c;
-            *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = stg[c];
-        }
+        commit_rows_tiled(Ks[buf], stg);
         __syncthreads();
-        if (st + 1 < NS) load_rows(k, st + 1, stg);
+        if (st + 1 < NS) load_rows(km, base + KS * (st + 1), stg);
 #pragma unroll
         for (int kt = 0; kt < 4; kt++)
 #pragma unroll
-            for (int sp = 0; sp < 4; sp++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Ks[buf][16 * kt + r][16 * sp + 4 * g]);
-                acc[4 * st + kt] = mfma16(a, qf[sp], acc[4 * st + kt]);
-            }
+            for (int ks = 0; ks < 2; ks++) acc[4 * st + kt] = mfma32(ld_op(Ks[buf], 16 * kt, ks), qf[ks], acc[4 * st + kt]);
     }
 
     // ---- mask, scale, softmax over this lane's query column ----
@@ -146,7 +201,7 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     for (int T = 0; T < NT; T++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int key = base + 16 * T + 4 * g + i;
+            const int key = base + KS * (T >> 2) + tile_key(T & 3, g, i);
             const bool ok = key >= lsq && key <= tq && tq < s;
             const float x = ok ? acc[T][i] * scale : -INFINITY;
             acc[T][i] = x;
@@ -171,52 +226,41 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     f32x4 o[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+    unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
     __syncthreads();   // every wave is done with the last K stage
-    load_pairs(v, st_lo, stg);
+    load_pairs(vm, base + KS * st_lo, stg);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
         const int buf = st & 1;
-        // transposed staging as 32-bit key pairs (bank = key pair: no conflicts): Vt[dim][key]
-        {
-            const int kp = tid & 31, d0 = 8 * (tid >> 5);
-            const unsigned e[4] = {stg[0].x, stg[0].y, stg[0].z, stg[0].w};
-            const unsigned o2[4] = {stg[1].x, stg[1].y, stg[1].z, stg[1].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                *reinterpret_cast<unsigned *>(&Ks[buf][d0 + 2 * j][2 * kp]) = (e[j] & 0xffffu) | (o2[j] << 16);
-                *reinterpret_cast<unsigned *>(&Ks[buf][d0 + 2 * j + 1][2 * kp]) = (e[j] >> 16) | (o2[j] & 0xffff0000u);
-            }
-        }
+        commit_transposed(Ks[buf], stg);
         __syncthreads();
-        if (st + 1 < NS) load_pairs(v, st + 1, stg);
+        if (st + 1 < NS) load_pairs(vm, base + KS * (st + 1), stg);
 #pragma unroll
-        for (int kt = 0; kt < 4; kt++) {
-            f32x4 p = acc[4 * st + kt];
+        for (int hf = 0; hf < 2; hf++) {
+            const f32x4 p0 = acc[4 * st + 2 * hf], p1 = acc[4 * st + 2 * hf + 1];
+            const uint4 pb = make_uint4(pack2(p0[0] * inv, p0[1] * inv), pack2(p0[2] * inv, p0[3] * inv),
+                                        pack2(p1[0] * inv, p1[1] * inv), pack2(p1[2] * inv, p1[3] * inv));
 #pragma unroll
-            for (int i = 0; i < 4; i++) p[i] *= inv;
-            const bf16x4 pb = pack4(p);
-            *reinterpret_cast<bf16x4 *>(&Pw[wave][r][16 * kt + 4 * g]) = pb;
+            for (int dt = 0; dt < 4; dt++) o[dt] = mfma32(ld_op(Ks[buf], 16 * dt, hf), pb, o[dt]);
+            // the lane's 8 weights are slots key0 - lsq .. + 7 of its query's row; keys after the
+            // query carry zeros, which the contract wants written while the slot exists
+            const int key0 = base + KS * st + 32 * hf + 8 * g, slot0 = key0 - lsq;
+            if (tq < s) {
+                if (slot0 >= 0 && slot0 + 8 <= ws) {
+                    __builtin_memcpy(wrow + slot0, &pb, 16);
+                } else if (slot0 + 8 > 0 && slot0 < ws) {
+                    const unsigned d[4] = {pb.x, pb.y, pb.z, pb.w};
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Ks[buf][16 * dt + r][16 * kt + 4 * g]);
-                o[dt] = mfma16(a, pb, o[dt]);
+                    for (int e = 0; e < 8; e++)
+                        if (slot0 + e >= 0 && slot0 + e < ws) wrow[slot0 + e] = (unsigned short)(d[e >> 1] >> (16 * (e & 1)));
+                }
             }
         }
-        // this stage's weights: one query row per instruction, 64 consecutive slots
-        // (the tile was written by this wave only; order the LDS stores before the loads)
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll 4
-        for (int qi = 0; qi < 16; qi++) {
-            const int tt = t0 + 16 * wave + qi, key = base + KS * st + l;
-            const int slot = key - max(tt + 1 - ws, 0);
-            if (tt < s && slot >= 0 && slot < ws) awb[(size_t)tt * ws + slot] = Pw[wave][qi][l];
-        }
-        asm volatile("" ::: "memory");
     }
     // slots whose keys lie beyond the block's last key (early queries only): zero
     if (t0 + QB < ws) {
+        unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
         for (int qi = 0; qi < 16; qi++) {
             const int tt = t0 + 16 * wave + qi;
             if (tt >= s) break;
@@ -226,18 +270,8 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
     if (tq < s) {
         unsigned short *ob = out + (row0 + tq) * total + hoff;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) *reinterpret_cast<bf16x4 *>(ob + 16 * dt + 4 * g) = pack4(o[dt]);
-    }
-}
-
-__device__ __forceinline__ float bf2f(unsigned short h) { return __uint_as_float(((unsigned)h) << 16); }
-// x = hi + lo with hi, lo bf16: the pair carries 16 mantissa bits through a bf16 product
-__device__ __forceinline__ void split4(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const unsigned short h = f2bf(x[i]);
-        hi[i] = (short)h;
-        lo[i] = (short)f2bf(x[i] - bf2f(h));
+        for (int dt = 0; dt < 4; dt++)
+            *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) = make_uint2(pack2(o[dt][0], o[dt][1]), pack2(o[dt][2], o[dt][3]));
     }
 }
 
@@ -248,17 +282,10 @@ __device__ __forceinline__ void split4(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
 // recomputes each dW tile next to its use, so no score tile outlives a stage.  dO and dS enter the
 // bf16 products as hi + lo pairs.  D_t goes to dvec for the key pass.
 //
-// The weights never pass through LDS.  Within a stage of 64 keys, element i of lane group g in
-// 16-key tile kt stands for key 32 (kt / 2) + 8 g + 4 (kt % 2) + i, so that the B operands of one
-// query for two tiles are 8 consecutive slots of its weight row: one 16-byte load (2-byte aligned)
-// per lane, kept in registers for the second sweep.  The LDS tiles of V and K are stored in that key
-// order (stage_pos).  Only the last stage, the one that holds the queries themselves, is read slot
-// by slot: its groups can end inside the 16 bytes, and a load that runs past the query's row would
-// leave the array at its last row.
-__device__ __forceinline__ int stage_pos(int key) {   // key 32 a + 8 g + 4 c + i -> 16 (2 a + c) + 4 g + i
-    return (key & 0x23) | ((key & 0x18) >> 1) | ((key & 0x04) << 2);
-}
-
+// The weights never pass through LDS: the B operand of one query for a 32-key half is one 16-byte
+// load of its weight row, kept in registers for the second sweep.  Only the last stage, the one that
+// holds the queries themselves, is read slot by slot: its groups can end inside the 16 bytes, and a
+// load that runs past the query's row would leave the array at its last row.
 __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
                                                                 const unsigned short *__restrict__ v,
                                                                 const unsigned short *__restrict__ attn_w,
@@ -266,7 +293,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
                                                                 float *__restrict__ d_q, float *__restrict__ dvec,
                                                                 int s, int H, int ws) {
     __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [stage_pos(key)][dim]
-    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][stage_pos(key)]: V (sweep 1), K (sweep 2)
+    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][key]: V (sweep 1), K (sweep 2)
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * QB, h = bc.h, b = bc.b;
@@ -277,55 +304,10 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
     const size_t row0 = (size_t)b * s;
     const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
     const unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
 
-    f32x4 dof[4];     // dO_t at dims 16 sp + 4 g .. +3: the positions of this lane in an O^T tile
-    bf16x4 doh[4], dol[4];
-#pragma unroll
-    for (int sp = 0; sp < 4; sp++) {
-        dof[sp] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (tq < s) dof[sp] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * sp + 4 * g);
-        split4(dof[sp], doh[sp], dol[sp]);
-    }
-
-    auto load_rows = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c, key = base + KS * stage + (chunk >> 3);
-            regs[c] = make_uint4(0, 0, 0, 0);
-            if (key >= 0 && key < s)
-                regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + 8 * (chunk & 7));
-        }
-    };
-    auto commit_rows = [&](int buf, const uint4 (&regs)[2]) {
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int chunk = tid + 256 * c;
-            *reinterpret_cast<uint4 *>(&Vr[buf][stage_pos(chunk >> 3)][8 * (chunk & 7)]) = regs[c];
-        }
-    };
-    // rows for a transposed stage: the thread takes 8 dims of two neighbouring keys, so that the
-    // transposed tile is written as 32-bit key pairs (bank = key pair: no conflicts)
-    auto load_pairs = [&](const unsigned short *src, int stage, uint4 (&regs)[2]) {
-        const int kp = tid & 31, d0 = 8 * (tid >> 5);
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int key = base + KS * stage + 2 * kp + c;
-            regs[c] = make_uint4(0, 0, 0, 0);
-            if (key >= 0 && key < s) regs[c] = *reinterpret_cast<const uint4 *>(src + (row0 + key) * total + hoff + d0);
-        }
-    };
-    auto commit_transposed = [&](int buf, const uint4 (&regs)[2]) {
-        const int col = stage_pos(2 * (tid & 31)), d0 = 8 * (tid >> 5);
-        const unsigned e[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
-        const unsigned o[4] = {regs[1].x, regs[1].y, regs[1].z, regs[1].w};
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j][col]) = (e[j] & 0xffffu) | (o[j] << 16);
-            *reinterpret_cast<unsigned *>(&Tt[buf][d0 + 2 * j + 1][col]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
-        }
-    };
-    // weights of this lane's query for the keys of its group in a stage: wv[stage][half] holds the
-    // 8 keys 32 half + 8 g .. + 7 (B operands of tiles 2 half and 2 half + 1), zero outside the window
+    // weights of this lane's query for the keys of its group in a stage: wv[stage][hf] holds the
+    // 8 keys 32 hf + 8 g .. + 7, zero outside the window
     uint4 wv[NS][2];
     auto fetch_weights = [&](int stage, uint4 (&w)[2]) {
 #pragma unroll
@@ -337,12 +319,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
                 if (tq < s && key0 + 7 >= lsq) {
                     uint4 x;
                     __builtin_memcpy(&x, wrow + (key0 - lsq), 16);
-                    const int cut = lsq - key0;   // elements below cut are outside the window
-                    x.x &= (cut > 0 ? 0u : 0xffffu) | (cut > 1 ? 0u : 0xffff0000u);
-                    x.y &= (cut > 2 ? 0u : 0xffffu) | (cut > 3 ? 0u : 0xffff0000u);
-                    x.z &= (cut > 4 ? 0u : 0xffffu) | (cut > 5 ? 0u : 0xffff0000u);
-                    x.w &= (cut > 6 ? 0u : 0xffffu) | (cut > 7 ? 0u : 0xffff0000u);
-                    w[hf] = x;
+                    w[hf] = mask_below(x, lsq - key0);
                 }
             } else {
                 unsigned d[4] = {0u, 0u, 0u, 0u};
@@ -357,12 +334,6 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
             }
         }
     };
-    auto b_operand = [&](const uint4 &w, int odd) {
-        const unsigned lo = odd ? w.z : w.x, hi = odd ? w.w : w.y;
-        bf16x4 pb;
-        pb[0] = (short)(lo & 0xffffu); pb[1] = (short)(lo >> 16); pb[2] = (short)(hi & 0xffffu); pb[3] = (short)(hi >> 16);
-        return pb;
-    };
     uint4 sv[2], sk[2];
 
     // ---- sweep 1: O^T = V^T P^T, then D = dO . O ----
@@ -371,70 +342,86 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
     for (int i = 0; i < 4; i++) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int st = 0; st < NS; st++) { wv[st][0] = make_uint4(0, 0, 0, 0); wv[st][1] = make_uint4(0, 0, 0, 0); }
-    load_pairs(v, st_lo, sv);
+    load_pairs(vm, base + KS * st_lo, sv);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
         const int buf = st & 1;
         fetch_weights(st, wv[st]);
-        commit_transposed(buf, sv);
+        commit_transposed(Tt[buf], sv);
         __syncthreads();
-        if (st + 1 < NS) load_pairs(v, st + 1, sv);
+        if (st + 1 < NS) load_pairs(vm, base + KS * (st + 1), sv);
 #pragma unroll
-        for (int kt = 0; kt < 4; kt++) {
-            const bf16x4 pb = b_operand(wv[st][kt >> 1], kt & 1);
+        for (int hf = 0; hf < 2; hf++)
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Tt[buf][16 * dt + r][16 * kt + 4 * g]);
-                ot[dt] = mfma16(a, pb, ot[dt]);
-            }
+            for (int dt = 0; dt < 4; dt++) ot[dt] = mfma32(ld_op(Tt[buf], 16 * dt, hf), wv[st][hf], ot[dt]);
+    }
+    // O^T tile dt holds dims 16 dt + 4 g + i of query r
+    float dsum = 0.f;
+    if (tq < s) {
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            const f32x4 x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * dt + 4 * g);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dsum = fmaf(x[i], ot[dt][i], dsum);
         }
     }
-    float dsum = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) dsum = fmaf(dof[dt][i], ot[dt][i], dsum);
     dsum += __shfl_xor(dsum, 16, 64);
     dsum += __shfl_xor(dsum, 32, 64);
     if (g == 0 && tq < s) dvec[(size_t)(b * H + h) * s + tq] = dsum;
 
     // ---- sweep 2: dW^T tiles recomputed, dS, d_q^T = K^T dS^T ----
+    uint4 doh[2], dol[2];   // dO_t, dims 32 ks + 8 g .. + 7, as hi + lo
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
+        if (tq < s) {
+            const float *p = d_out + (row0 + tq) * total + hoff + 32 * ks + 8 * g;
+            x0 = *reinterpret_cast<const f32x4 *>(p);
+            x1 = *reinterpret_cast<const f32x4 *>(p + 4);
+        }
+        split8(x0, x1, doh[ks], dol[ks]);
+    }
     f32x4 dq[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) dq[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     const float scale = 0.125f;
     __syncthreads();
-    load_rows(v, st_lo, sv);
-    load_pairs(k, st_lo, sk);
+    load_rows(vm, base + KS * st_lo, sv);
+    load_pairs(km, base + KS * st_lo, sk);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
         const int buf = st & 1;
-        commit_rows(buf, sv);
-        commit_transposed(buf, sk);
+        commit_rows_tiled(Vr[buf], sv);
+        commit_transposed(Tt[buf], sk);
         __syncthreads();
-        if (st + 1 < NS) { load_rows(v, st + 1, sv); load_pairs(k, st + 1, sk); }
+        if (st + 1 < NS) { load_rows(vm, base + KS * (st + 1), sv); load_pairs(km, base + KS * (st + 1), sk); }
 #pragma unroll
-        for (int kt = 0; kt < 4; kt++) {
-            f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key of (kt, g, i)][query r]
+        for (int hf = 0; hf < 2; hf++) {
+            f32x4 ds[2];
+            const unsigned wd[4] = {wv[st][hf].x, wv[st][hf].y, wv[st][hf].z, wv[st][hf].w};
 #pragma unroll
-            for (int sp = 0; sp < 4; sp++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Vr[buf][16 * kt + r][16 * sp + 4 * g]);
-                dw = mfma16(a, doh[sp], dw);
-                dw = mfma16(a, dol[sp], dw);
+            for (int c = 0; c < 2; c++) {
+                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key 32 hf + 8 g + 4 c + i][query r]
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    const uint4 a = ld_op(Vr[buf], 16 * (2 * hf + c), ks);
+                    dw = mfma32(a, doh[ks], dw);
+                    dw = mfma32(a, dol[ks], dw);
+                }
+                ds[c][0] = bf_lo(wd[2 * c]) * (dw[0] - dsum) * scale;
+                ds[c][1] = bf_hi(wd[2 * c]) * (dw[1] - dsum) * scale;
+                ds[c][2] = bf_lo(wd[2 * c + 1]) * (dw[2] - dsum) * scale;
+                ds[c][3] = bf_hi(wd[2 * c + 1]) * (dw[3] - dsum) * scale;
             }
-            const bf16x4 pb = b_operand(wv[st][kt >> 1], kt & 1);
-            f32x4 ds;
-#pragma unroll
-            for (int i = 0; i < 4; i++) ds[i] = bf2f((unsigned short)pb[i]) * (dw[i] - dsum) * scale;
-            bf16x4 dsh, dsl;
-            split4(ds, dsh, dsl);
+            uint4 dsh, dsl;
+            split8(ds[0], ds[1], dsh, dsl);
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const bf16x4 a = *reinterpret_cast<const bf16x4 *>(&Tt[buf][16 * dt + r][16 * kt + 4 * g]);
-                dq[dt] = mfma16(a, dsh, dq[dt]);
-                dq[dt] = mfma16(a, dsl, dq[dt]);
+                const uint4 a = ld_op(Tt[buf], 16 * dt, hf);
+                dq[dt] = mfma32(a, dsh, dq[dt]);
+                dq[dt] = mfma32(a, dsl, dq[dt]);
             }
         }
     }
@@ -448,8 +435,9 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
 // Backward, key pass (one workgroup per 64 keys, one wave per 16 keys): over the up to 575
 // queries t in [j, j + window) that see key j,
 //   d_v[j] += sum_t w[t,j] dO_t,   d_k[j] += sum_t dS[t,j] q_t,   dS recomputed from w, dO.v_j, D_t.
-// A tile of dS / w in accumulator layout (rows = queries, column = the lane's key) is exactly
-// the A operand of the products with Q^T / dO^T, which are staged transposed in LDS.
+// Two tiles of dS / w in accumulator layout (rows = queries, column = the lane's key) are the A
+// operand of the products with Q^T / dO^T, which are staged transposed in LDS; the rows of the
+// dO stage are stored in tile order (stage_pos) so that those 8 rows are 8 consecutive queries.
 __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned short *__restrict__ q,
                                                              const unsigned short *__restrict__ v,
                                                              const unsigned short *__restrict__ attn_w,
@@ -457,7 +445,7 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
                                                              const float *__restrict__ dvec,
                                                              float *__restrict__ d_k, float *__restrict__ d_v,
                                                              int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short Dh[KS][LDH], Dl[KS][LDH];      // dO hi / lo, [query][dim]
+    __shared__ __align__(16) unsigned short Dh[KS][LDH], Dl[KS][LDH];      // dO hi / lo, [stage_pos(query)][dim]
     __shared__ __align__(16) unsigned short DhT[HD][LDH], DlT[HD][LDH];    // transposed, [dim][query]
     __shared__ __align__(16) unsigned short QT[HD][LDH];                   // Q^T, [dim][query]
     __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
@@ -470,12 +458,13 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
     const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
     const float *dvb = dvec + (size_t)(b * H + h) * s;
+    const StageSrc qm{q, row0, total, hoff, s};
 
-    bf16x4 vf[4];
+    uint4 vf[2];
 #pragma unroll
-    for (int sp = 0; sp < 4; sp++) {
-        vf[sp] = bf16x4{0, 0, 0, 0};
-        if (kj < s) vf[sp] = *reinterpret_cast<const bf16x4 *>(v + (row0 + kj) * total + hoff + 16 * sp + 4 * g);
+    for (int ks = 0; ks < 2; ks++) {
+        vf[ks] = make_uint4(0, 0, 0, 0);
+        if (kj < s) vf[ks] = *reinterpret_cast<const uint4 *>(v + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
     }
     f32x4 dk[4], dv[4];
 #pragma unroll
@@ -487,13 +476,13 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     f32x4 gdo[4];
     uint4 gq[2];
     unsigned short gw[16];
+    uint4 gwv[2];
     float gd = 0.f;
-    const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // dO: query pair, first dim (+32 for the second half)
-    const int qpair = tid & 31, qd0 = 8 * (tid >> 5);                        // Q: query pair, first dim
+    // dO: query pair (2 rows) x 4 dims per load; pairs so that the transposed tiles are written as
+    // 32-bit words without bank conflicts
+    const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // query pair, first dim (+32 for the second half)
     auto fetch_stage = [&](int st) {
         const int qs0 = j0 + KS * st;
-        // dO: query pair (2 rows) x 4 dims per load, Q: query pair x 8 dims; pairs so that the
-        // transposed tiles are written as 32-bit words without bank conflicts
 #pragma unroll
         for (int cc = 0; cc < 2; cc++)
 #pragma unroll
@@ -502,19 +491,31 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
                 gdo[2 * cc + c] = f32x4{0.f, 0.f, 0.f, 0.f};
                 if (t < s) gdo[2 * cc + c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dd0 + 32 * cc);
             }
+        load_pairs(qm, qs0, gq);
+        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t).
+        // Past the first stage every query lies after all keys of the block, so a group of 8 keys
+        // never runs past the query's row: one 16-byte load (2-byte aligned) per group, the keys
+        // before the window masked.  The first stage is read slot by slot.
+        if (st == 0) {
 #pragma unroll
-        for (int c = 0; c < 2; c++) {
-            const int t = qs0 + 2 * qpair + c;
-            gq[c] = make_uint4(0, 0, 0, 0);
-            if (t < s) gq[c] = *reinterpret_cast<const uint4 *>(q + (row0 + t) * total + hoff + qd0);
-        }
-        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t)
+            for (int c = 0; c < 16; c++) {
+                const int t = qs0 + 4 * c + wave, key = j0 + l;
+                const int slot = key - max(t + 1 - ws, 0);
+                gw[c] = 0;
+                if (t < s && key <= t && slot >= 0 && slot < ws) gw[c] = awb[(size_t)t * ws + slot];
+            }
+        } else {
 #pragma unroll
-        for (int c = 0; c < 16; c++) {
-            const int t = qs0 + 4 * c + wave, key = j0 + l;
-            const int slot = key - max(t + 1 - ws, 0);
-            gw[c] = 0;
-            if (t < s && key <= t && slot >= 0 && slot < ws) gw[c] = awb[(size_t)t * ws + slot];
+            for (int c = 0; c < 2; c++) {
+                const int chunk = tid + 256 * c, t = qs0 + (chunk >> 3), key0 = j0 + 8 * (chunk & 7);
+                const int ls = max(t + 1 - ws, 0);
+                gwv[c] = make_uint4(0, 0, 0, 0);
+                if (t < s && key0 + 7 >= ls) {
+                    uint4 x;
+                    __builtin_memcpy(&x, awb + (size_t)t * ws + (key0 - ls), 16);
+                    gwv[c] = mask_below(x, ls - key0);
+                }
+            }
         }
         gd = (tid < KS && qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
     };
@@ -525,66 +526,71 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
         __syncthreads();   // previous stage's readers are done
 #pragma unroll
         for (int cc = 0; cc < 2; cc++) {
-            bf16x4 hi[2], lo[2];
+            unsigned hi[2][2], lo[2][2];
 #pragma unroll
             for (int c = 0; c < 2; c++) {
-                split4(gdo[2 * cc + c], hi[c], lo[c]);
-                *reinterpret_cast<bf16x4 *>(&Dh[2 * dpair + c][dd0 + 32 * cc]) = hi[c];
-                *reinterpret_cast<bf16x4 *>(&Dl[2 * dpair + c][dd0 + 32 * cc]) = lo[c];
+                const f32x4 x = gdo[2 * cc + c];
+                split2(x[0], x[1], hi[c][0], lo[c][0]);
+                split2(x[2], x[3], hi[c][1], lo[c][1]);
+                const int row = stage_pos(2 * dpair + c);
+                *reinterpret_cast<uint2 *>(&Dh[row][dd0 + 32 * cc]) = make_uint2(hi[c][0], hi[c][1]);
+                *reinterpret_cast<uint2 *>(&Dl[row][dd0 + 32 * cc]) = make_uint2(lo[c][0], lo[c][1]);
             }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
+                const unsigned h0 = hi[0][j >> 1], h1 = hi[1][j >> 1], l0 = lo[0][j >> 1], l1 = lo[1][j >> 1];
                 *reinterpret_cast<unsigned *>(&DhT[dd0 + 32 * cc + j][2 * dpair]) =
-                    (unsigned)(unsigned short)hi[0][j] | ((unsigned)(unsigned short)hi[1][j] << 16);
+                    (j & 1) ? ((h0 >> 16) | (h1 & 0xffff0000u)) : ((h0 & 0xffffu) | (h1 << 16));
                 *reinterpret_cast<unsigned *>(&DlT[dd0 + 32 * cc + j][2 * dpair]) =
-                    (unsigned)(unsigned short)lo[0][j] | ((unsigned)(unsigned short)lo[1][j] << 16);
+                    (j & 1) ? ((l0 >> 16) | (l1 & 0xffff0000u)) : ((l0 & 0xffffu) | (l1 << 16));
             }
         }
-        {
-            const unsigned e[4] = {gq[0].x, gq[0].y, gq[0].z, gq[0].w};
-            const unsigned o[4] = {gq[1].x, gq[1].y, gq[1].z, gq[1].w};
+        commit_transposed(QT, gq);
+        if (st == 0) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                *reinterpret_cast<unsigned *>(&QT[qd0 + 2 * j][2 * qpair]) = (e[j] & 0xffffu) | (o[j] << 16);
-                *reinterpret_cast<unsigned *>(&QT[qd0 + 2 * j + 1][2 * qpair]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
+            for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int chunk = tid + 256 * c;
+                *reinterpret_cast<uint4 *>(&Pt[chunk >> 3][8 * (chunk & 7)]) = gwv[c];
             }
         }
-#pragma unroll
-        for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
         if (tid < KS) Dv[tid] = gd;
         __syncthreads();
         if (qs0 + KS <= t_last) fetch_stage(st + 1);
 #pragma unroll
-        for (int qt = 0; qt < 4; qt++) {
-            f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int hf = 0; hf < 2; hf++) {
+            f32x4 ds[2];
+            unsigned pw[2][2];
 #pragma unroll
-            for (int sp = 0; sp < 4; sp++) {
-                const bf16x4 ah = *reinterpret_cast<const bf16x4 *>(&Dh[16 * qt + r][16 * sp + 4 * g]);
-                const bf16x4 al = *reinterpret_cast<const bf16x4 *>(&Dl[16 * qt + r][16 * sp + 4 * g]);
-                dw = mfma16(ah, vf[sp], dw);
-                dw = mfma16(al, vf[sp], dw);
-            }
-            // accumulator layout: rows = queries 16 qt + 4g + i, column = key r of this wave
-            bf16x4 pa;
-            f32x4 ds;
+            for (int c = 0; c < 2; c++) {
+                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW[query 32 hf + 8 g + 4 c + i][key r of this wave]
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int qi = 16 * qt + 4 * g + i;
-                const unsigned short pw = Pt[qi][16 * wave + r];
-                pa[i] = (short)pw;
-                ds[i] = bf2f(pw) * (dw[i] - Dv[qi]) * scale;
+                for (int ks = 0; ks < 2; ks++) {
+                    dw = mfma32(ld_op(Dh, 16 * (2 * hf + c), ks), vf[ks], dw);
+                    dw = mfma32(ld_op(Dl, 16 * (2 * hf + c), ks), vf[ks], dw);
+                }
+                unsigned short p4[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int qi = 32 * hf + 8 * g + 4 * c + i;
+                    p4[i] = Pt[qi][16 * wave + r];
+                    ds[c][i] = __uint_as_float((unsigned)p4[i] << 16) * (dw[i] - Dv[qi]) * scale;
+                }
+                pw[c][0] = (unsigned)p4[0] | ((unsigned)p4[1] << 16);
+                pw[c][1] = (unsigned)p4[2] | ((unsigned)p4[3] << 16);
             }
-            bf16x4 dsh, dsl;
-            split4(ds, dsh, dsl);
+            const uint4 pa = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
+            uint4 dsh, dsl;
+            split8(ds[0], ds[1], dsh, dsl);
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const bf16x4 bh = *reinterpret_cast<const bf16x4 *>(&DhT[16 * dt + r][16 * qt + 4 * g]);
-                const bf16x4 bl = *reinterpret_cast<const bf16x4 *>(&DlT[16 * dt + r][16 * qt + 4 * g]);
-                const bf16x4 bq = *reinterpret_cast<const bf16x4 *>(&QT[16 * dt + r][16 * qt + 4 * g]);
-                dv[dt] = mfma16(pa, bh, dv[dt]);
-                dv[dt] = mfma16(pa, bl, dv[dt]);
-                dk[dt] = mfma16(dsh, bq, dk[dt]);
-                dk[dt] = mfma16(dsl, bq, dk[dt]);
+                const uint4 bh = ld_op(DhT, 16 * dt, hf), bl = ld_op(DlT, 16 * dt, hf), bq = ld_op(QT, 16 * dt, hf);
+                dv[dt] = mfma32(pa, bh, dv[dt]);
+                dv[dt] = mfma32(pa, bl, dv[dt]);
+                dk[dt] = mfma32(dsh, bq, dk[dt]);
+                dk[dt] = mfma32(dsl, bq, dk[dt]);
             }
         }
     }
