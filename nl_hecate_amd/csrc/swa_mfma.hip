@@ -149,7 +149,7 @@ __device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int k
     return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
 }
 
-__global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
+__global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
                                                            const unsigned short *__restrict__ k,
                                                            const unsigned short *__restrict__ v,
                                                            unsigned short *__restrict__ out,
@@ -193,28 +193,42 @@ __global__ __launch_bounds__(256) void swa_fwd_mfma_kernel(const unsigned short 
             for (int ks = 0; ks < 2; ks++) acc[4 * st + kt] = mfma32(ld_op(Ks[buf], 16 * kt, ks), qf[ks], acc[4 * st + kt]);
     }
 
-    // ---- mask, scale, softmax over this lane's query column ----
-    const float scale = 0.125f;   // 1/sqrt(64)
+    // ---- mask and softmax over this lane's query column ----
+    // exp(scale (x - max)) = exp2(c x - c max) with c = scale log2(e): one fused multiply-add and
+    // one v_exp_f32 per score; exp2(-inf) = 0 takes care of the masked ones.  Only the stages at
+    // the two ends of the window hold masked keys; the others skip the test (block-uniform).
+    const float c2 = 0.125f * 1.44269504088896340736f;   // log2(e) / sqrt(64)
     const int lsq = max(tq + 1 - ws, 0);
+    const int ls_hi = max(t0 + QB - ws, 0);   // window start of the block's last query
     float mx = -INFINITY;
 #pragma unroll
-    for (int T = 0; T < NT; T++)
+    for (int st = 0; st < NS; st++) {
+        const int k0 = base + KS * st;
+        const bool full = k0 >= ls_hi && k0 + KS - 1 <= t0 && t0 + QB <= s;
+        if (!full) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int key = base + KS * (T >> 2) + tile_key(T & 3, g, i);
-            const bool ok = key >= lsq && key <= tq && tq < s;
-            const float x = ok ? acc[T][i] * scale : -INFINITY;
-            acc[T][i] = x;
-            mx = fmaxf(mx, x);
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = k0 + tile_key(kt, g, i);
+                    const bool ok = key >= lsq && key <= tq && tq < s;
+                    acc[4 * st + kt][i] = ok ? acc[4 * st + kt][i] : -INFINITY;
+                }
         }
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[4 * st + kt][i]);
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mc = mx == -INFINITY ? 0.f : mx * c2;
     float sum = 0.f;
 #pragma unroll
     for (int T = 0; T < NT; T++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float e = acc[T][i] == -INFINITY ? 0.f : expf(acc[T][i] - mx);
+            const float e = __builtin_amdgcn_exp2f(fmaf(acc[T][i], c2, -mc));
             acc[T][i] = e;
             sum += e;
         }
