@@ -103,6 +103,7 @@ class MagLayer:
         for lv, l in enumerate(self.p.levels):
             l.w_k, l.w_v, l.w_q = views[3 + 3 * lv], views[4 + 3 * lv], views[5 + 3 * lv]
         self.split_gemm = True
+        self.stack_levels = True   # chunkwise rule: active levels run as one batch of chains
         # per-level context memory, one matrix per (batch element, head); created on first use
         self.m_state: List[Optional[torch.Tensor]] = [None] * k
         self.s_state: List[Optional[torch.Tensor]] = [None] * k
@@ -144,11 +145,13 @@ class MagLayer:
         return torch.mm(xa, wb[index * d:(index + 1) * d].t(), out_dtype=torch.float32)
 
     def ensure_state(self, bs):
-        """Creates the (zero) context memories of every level for batch size bs if they do not exist."""
-        for lv in range(self.k):
-            if self.m_state[lv] is None:
-                self.m_state[lv] = _zeros(bs * self.nh, self.hd * self.hd)
-                self.s_state[lv] = _zeros(bs * self.nh, self.hd * self.hd)
+        """Creates the (zero) context memories of every level for batch size bs if they do not exist.
+        The levels' memories are slices of one tensor, so that a prefix of levels is one batch of chains."""
+        if self.m_state[0] is None:
+            self._m_all = _zeros(self.k, bs * self.nh, self.hd * self.hd)
+            self._s_all = _zeros(self.k, bs * self.nh, self.hd * self.hd)
+            for lv in range(self.k):
+                self.m_state[lv], self.s_state[lv] = self._m_all[lv], self._s_all[lv]
 
     # ── one level ────────────────────────────────────────────────────────────
     def _level_forward(self, lv, x2, bs, s, active, ops=None):
@@ -157,8 +160,7 @@ class MagLayer:
         lp = self.p.levels[lv]
         B = bs * nh
         n = bs * s
-        if self.m_state[lv] is None:
-            self.m_state[lv], self.s_state[lv] = _zeros(B, hd * hd), _zeros(B, hd * hd)
+        self.ensure_state(bs)
         y = _new(bs, s, d)
         if not active:
             # frozen level (gpu_memory_read_only, gpu_forward.rs:2906-2950): y = M_h q with the raw
@@ -167,23 +169,9 @@ class MagLayer:
             m_shared = self.m_state[lv][:nh].contiguous()
             D.call("memory_read_only_f32_rocm", q_raw, m_shared, y, n, nh, hd)
             return y, dict(active=False, m_shared=m_shared)
-        k_mem = self._project(ops, x2, lp.w_k, 3 + 3 * lv)
-        v_mem = self._project(ops, x2, lp.w_v, 4 + 3 * lv)
-        q_mem = self._project(ops, x2, lp.w_q, 5 + 3 * lv)
-        k_norms, q_norms = _new(n), _new(n)
-        D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
-        D.call("l2_normalize_rows_f32_cuda", q_mem, q_norms, n, d, 1e-8)
-        c = dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, k_norms=k_norms, q_norms=q_norms, active=active, ops=ops)
-        alpha, theta, eta = _new(n), _new(n), _new(n)
-        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_alpha, lp.b_alpha, alpha, n, d, 0)
-        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_theta, lp.b_theta, theta, n, d, 1)
-        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_eta, lp.b_eta, eta, n, d, 0)
         kh, vh, qh = _new(B, s, hd), _new(B, s, hd), _new(B, s, hd)
-        for src, dst in ((k_mem, kh), (v_mem, vh), (q_mem, qh)):
-            D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 1)
         ah, th, eh = _new(B, s), _new(B, s), _new(B, s)
-        for src, dst in ((alpha, ah), (theta, th), (eta, eh)):
-            D.call("broadcast_heads_f32_cuda", src, dst, bs, s, nh)
+        c = self._level_inputs(lv, x2, bs, s, ops, (kh, vh, qh, ah, th, eh))
         yh = _new(B, s, hd)
         C = self.chunk
         if self.rule == "exact":
@@ -202,8 +190,79 @@ class MagLayer:
         self.m_state[lv].copy_(mc[:, -1])
         self.s_state[lv].copy_(sc[:, -1])
         D.call("transpose_heads_f32_cuda", yh, y, bs, s, nh, hd, 0)
-        c.update(alpha=alpha, theta=theta, eta=eta, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc)
+        c.update(kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc)
         return y, c
+
+    def _level_inputs(self, lv, x2, bs, s, ops, dst):
+        """Projections, L2 norm, gates and head split of level lv; the head-major k, v, q [B, s, hd] and
+        gates [B, s] go to the six tensors of dst.  Returns the level's cache of token-major tensors."""
+        d, nh, hd = self.d, self.nh, self.hd
+        lp = self.p.levels[lv]
+        n = bs * s
+        k_mem = self._project(ops, x2, lp.w_k, 3 + 3 * lv)
+        v_mem = self._project(ops, x2, lp.w_v, 4 + 3 * lv)
+        q_mem = self._project(ops, x2, lp.w_q, 5 + 3 * lv)
+        k_norms, q_norms = _new(n), _new(n)
+        D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
+        D.call("l2_normalize_rows_f32_cuda", q_mem, q_norms, n, d, 1e-8)
+        alpha, theta, eta = _new(n), _new(n), _new(n)
+        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_alpha, lp.b_alpha, alpha, n, d, 0)
+        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_theta, lp.b_theta, theta, n, d, 1)
+        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_eta, lp.b_eta, eta, n, d, 0)
+        for src, dst_t in zip((k_mem, v_mem, q_mem), dst[:3]):
+            D.call("transpose_heads_f32_cuda", src, dst_t, bs, s, nh, hd, 1)
+        for src, dst_t in zip((alpha, theta, eta), dst[3:]):
+            D.call("broadcast_heads_f32_cuda", src, dst_t, bs, s, nh)
+        return dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, k_norms=k_norms, q_norms=q_norms, active=True, ops=ops,
+                    alpha=alpha, theta=theta, eta=eta)
+
+    # The active levels of the chunkwise rule as ONE batch of chains.  The levels are independent
+    # memories over the same tokens, and the chain kernels want at least 128 chains to fill the chip, so
+    # the head-major tensors of the active levels (always a prefix: the periods are nested) are stacked
+    # along the chain dimension and the rule runs once, forward and backward.
+    def _levels_forward_stacked(self, na, x2, bs, s, ops):
+        d, nh, hd, C = self.d, self.nh, self.hd, self.chunk
+        B = bs * nh
+        self.ensure_state(bs)
+        kh, vh, qh = _new(na * B, s, hd), _new(na * B, s, hd), _new(na * B, s, hd)
+        ah, th, eh = _new(na * B, s), _new(na * B, s), _new(na * B, s)
+        caches = []
+        for lv in range(na):
+            sl = slice(lv * B, (lv + 1) * B)
+            caches.append(self._level_inputs(lv, x2, bs, s, ops, tuple(t[sl] for t in (kh, vh, qh, ah, th, eh))))
+        nc = (s + C - 1) // C
+        mc, sc, yh = _new(na * B, nc + 1, hd * hd), _new(na * B, nc + 1, hd * hd), _new(na * B, s, hd)
+        kh, vh, qh = kh.to(torch.bfloat16), vh.to(torch.bfloat16), qh.to(torch.bfloat16)
+        m0, s0 = self._m_all[:na].view(na * B, hd * hd), self._s_all[:na].view(na * B, hd * hd)
+        D.call("titans_chunkwise_forward_bf16_rocm", kh, vh, qh, ah, th, eh, m0, s0, mc, sc, yh, s, hd, na * B, C)
+        m0.copy_(mc[:, -1])
+        s0.copy_(sc[:, -1])
+        ys = []
+        for lv in range(na):
+            y = _new(bs, s, d)
+            D.call("transpose_heads_f32_cuda", yh[lv * B:(lv + 1) * B], y, bs, s, nh, hd, 0)
+            ys.append(y)
+        return ys, caches, dict(na=na, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc)
+
+    def _levels_backward_stacked(self, st, caches, x2, d_y, bs, s, grads):
+        nh, hd, C, na = self.nh, self.hd, self.chunk, st["na"]
+        B = bs * nh
+        dyh = _new(na * B, s, hd)
+        D.call("transpose_heads_f32_cuda", d_y, dyh[:B], bs, s, nh, hd, 1)
+        for lv in range(1, na):   # every level sees the same upstream gradient
+            dyh[lv * B:(lv + 1) * B].copy_(dyh[:B])
+        dkh, dvh, dqh = _new(na * B, s, hd), _new(na * B, s, hd), _new(na * B, s, hd)
+        dah, dth, deh = _new(na * B, s), _new(na * B, s), _new(na * B, s)
+        dm, ds = _zeros(hd, hd), _zeros(hd, hd)
+        D.call("titans_chunkwise_backward_bf16_rocm", st["kh"], st["vh"], st["qh"], st["ah"], st["th"], st["eh"],
+               st["mc"], st["sc"], dyh, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, na * B, C)
+        d_x = None
+        for lv in range(na):
+            sl = slice(lv * B, (lv + 1) * B)
+            dx = self._level_param_grads(lv, caches[lv], x2, tuple(t[sl] for t in (dkh, dvh, dqh, dah, dth, deh)),
+                                         bs, s, grads)
+            d_x = dx if d_x is None else d_x.add_(dx)
+        return d_x
 
     def _level_backward(self, lv, c, x2, d_y, bs, s, grads):
         """gpu_memory_backward + accumulate_projection_grads; returns the level's d_x [bs*s, d]."""
@@ -228,6 +287,15 @@ class MagLayer:
         else:
             D.call("titans_chunkwise_backward_bf16_rocm", c["kh"], c["vh"], c["qh"], c["ah"], c["th"], c["eh"],
                    c["mc"], c["sc"], dyh, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, B, C)
+        return self._level_param_grads(lv, c, x2, (dkh, dvh, dqh, dah, dth, deh), bs, s, grads)
+
+    def _level_param_grads(self, lv, c, x2, head_grads, bs, s, grads):
+        """From the rule's head-major gradients (d_k, d_v, d_q [B, s, hd], d_alpha, d_theta, d_eta [B, s]) of
+        level lv: gate and projection weight gradients (accumulated into grads) and the level's d_x."""
+        d, nh, hd = self.d, self.nh, self.hd
+        lp, g = self.p.levels[lv], grads.levels[lv]
+        n = bs * s
+        dkh, dvh, dqh, dah, dth, deh = head_grads
         d_alpha, d_theta, d_eta = _new(n), _new(n), _new(n)
         for src, dst in ((dah, d_alpha), (dth, d_theta), (deh, d_eta)):
             D.call("sum_heads_f32_cuda", src, dst, bs, s, nh)
@@ -260,9 +328,13 @@ class MagLayer:
         attn_bf, aw = _new(bs, s, d, dtype=torch.bfloat16), _new(bs, nh, s, self.window, dtype=torch.bfloat16)
         D.call("swa_forward_f32_cuda", q, k, v, attn_bf, aw, s, nh, hd, self.window, bs, 0)
         attn = attn_bf.to(torch.float32)
-        ys, caches = [], []
-        for lv in range(self.k):
-            y, c = self._level_forward(lv, x2, bs, s, pulse.active_levels[lv], ops)
+        ys, caches, stack = [], [], None
+        active = [bool(a) for a in pulse.active_levels]
+        na = active.index(False) if False in active else self.k
+        if self.rule == "chunkwise" and self.stack_levels and na >= 2 and not any(active[na:]):
+            ys, caches, stack = self._levels_forward_stacked(na, x2, bs, s, ops)
+        for lv in range(len(ys), self.k):
+            y, c = self._level_forward(lv, x2, bs, s, active[lv], ops)
             ys.append(y)
             caches.append(c)
         y_comb, gate, gated = _new(bs, s, d), _new(bs, s, d), _new(bs, s, d)
@@ -271,7 +343,7 @@ class MagLayer:
                                   gated.data_ptr(), bs * s * d)
         out = (gated.view(bs * s, d) @ p.w_o.t()).view(bs, s, d)
         cache = dict(x=x, q=q, k=k, v=v, aw=aw, attn=attn, gate=gate, gated=gated, levels=caches, pulse=pulse,
-                     ys=ys, ops=ops)
+                     ys=ys, ops=ops, stack=stack)
         return out, cache
 
     def backward(self, cache, d_out):
@@ -288,8 +360,11 @@ class MagLayer:
         grads.w_o += _wgrad(do2, cache["gated"].view(n, d))
         d_attn, d_ycomb = _new(bs, s, d), _new(bs, s, d)
         D.call("cms_gate_backward_rocm", d_gated, cache["attn"], cache["gate"], self.k, d_attn, d_ycomb, n * d)
-        d_x = _zeros(n, d)
-        for lv in range(self.k):
+        d_x, first = _zeros(n, d), 0
+        if cache["stack"] is not None:
+            first = cache["stack"]["na"]
+            d_x += self._levels_backward_stacked(cache["stack"], cache["levels"], x2, d_ycomb, bs, s, grads)
+        for lv in range(first, self.k):
             d_x += self._level_backward(lv, cache["levels"][lv], x2, d_ycomb, bs, s, grads)
         dq, dk, dv = _new(bs, s, d), _zeros(bs, s, d), _zeros(bs, s, d)
         D.call("swa_backward_f32_cuda", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv, s, nh,
