@@ -24,6 +24,8 @@ Workloads (BASELINE.json `configs`):
   hope_selfref_c4   configs[3]: HOPE self-referential memory, 8 heads x 64, batch 8,
                     seq 2048, fp32, self-generated values, frozen snapshots per
                     64-token chunk; grads to x and to the six initial memories.
+  hebbian_c2        the Hebbian rule (M <- (1 - alpha) M + v k^T) at the shape of configs[1]:
+                    full-trajectory forward + whole-sequence segment backward.
 """
 import argparse
 import ctypes
@@ -198,7 +200,7 @@ def setup_titans_chunkwise_c3(torch, D, lib):
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16",
         flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_bwd=BYTES_CW_BWD,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
-        traffic_bwd=int((1707.6 + 522.3) * 2**20),   # measured for cw_grads_bf16_kernel: 1707.6 MiB read, 522.3 MiB written
+        traffic_bwd=int((1707.8 + 522.3) * 2**20),   # measured for cw_grads_bf16_kernel: 1707.8 MiB read, 522.3 MiB written
         kernel="cw_grads_bf16_kernel (the per-chunk gradient pass of the backward entry point)",
         kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
         config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
@@ -252,7 +254,7 @@ def setup_swa_c5(torch, D, lib):
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * heads * s, bound="hbm", dtype="bf16",
         flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_bwd=BYTES_SWA_BWD,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
-        traffic_bwd=int((1441.1 + 128.0 + 1057.9 + 65.0) * 2**20),   # measured: key pass + query pass
+        traffic_bwd=int((522.9 + 128.0 + 403.2 + 65.0) * 2**20),   # measured: key pass + query pass (read + written MiB each)
         kernel=None,
         kernel_names={"forward": "swa_forward", "backward": "swa_backward"},
         config={"workload": "BASELINE configs[4], attention branch: sliding-window attention, window 512, 8 heads x 64, "
@@ -392,9 +394,62 @@ def setup_hope_selfref_c4(torch, D, lib):
         cpu=lambda: cpu_baseline_hope(mems, x, dy, C))
 
 
+# Hebbian rule, per head-token at d=64 with the full trajectory the contract asks for: forward
+# k,v,q 768 + alpha 4 + y 256 + M_{t+1} 16 384 = 17 412 B, 6 d^2 flop; backward k,v,q,dY 1024 + alpha 4 +
+# M_t 16 384 + grads 772 = 18 184 B, 12 d^2 flop.
+BYTES_HEB_FWD, BYTES_HEB_BWD = 17412, 18184
+FLOP_HEB_FWD, FLOP_HEB_BWD = 6 * 64 * 64, 12 * 64 * 64
+
+
+def cpu_baseline_hebbian(x, heads, budget_s=12.0):
+    """Oracle of the Hebbian rule (dispatch.rs:1566-1660), one thread, whole sequences until the budget is used."""
+    from oracle import pyoracle as orc
+    B, s, d = x["k"].shape
+    npx = {n: t.numpy() for n, t in x.items()}
+    done = 0
+    t_start = time.perf_counter()
+    while done < B and time.perf_counter() - t_start < budget_s:
+        for b in range(done, done + heads):
+            a = [npx[n][b] for n in ("k", "v", "q", "alpha")]
+            y, ms = orc.hebbian_forward(*a, npx["m0"][b])
+            orc.hebbian_backward(*a, ms, npx["dy"][b])
+        done += heads
+    el = time.perf_counter() - t_start
+    return {"value": (done // heads) * s / el, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{done} of {B} chains ({done // heads} sequences of {s} tokens, all {heads} heads), "
+                      f"full-trajectory forward + backward, {el:.1f} s"}
+
+
+def setup_hebbian_c2(torch, D, lib):
+    bs, heads, d, s = 8, 8, 64, 2048
+    B = bs * heads
+    x = make_inputs(B, s, d, 0x5EED0006)
+    dv = {n: t.cuda() for n, t in x.items()}
+    z = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device="cuda")
+    ms, y = z(B, s + 1, d, d), z(B, s, d)
+    g = dict(dk=z(B, s, d), dv=z(B, s, d), dq=z(B, s, d), da=z(B, s), dm=z(B, d, d), seed=z(B, d, d))
+
+    def fwd():
+        D.hebbian_forward_dd(dv["k"], dv["v"], dv["q"], dv["alpha"], dv["m0"], ms, y, s, d, B, s, d * d)
+
+    def bwd():
+        D.hebbian_backward_dd_segment(dv["k"], dv["v"], dv["q"], dv["alpha"], ms, dv["dy"], g["seed"],
+                                      g["dk"], g["dv"], g["dq"], g["da"], g["dm"], 0, s, d, B, s)
+
+    return dict(
+        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm",
+        flop_fwd=FLOP_HEB_FWD, flop_bwd=FLOP_HEB_BWD, bytes_bwd=BYTES_HEB_BWD,
+        traffic_bwd=None, kernel=None,
+        kernel_names={"forward": "hebbian_forward", "backward": "hebbian_backward_segment"},
+        config={"workload": "Hebbian rule at the shape of BASELINE configs[1]: 8 heads x 64 (d=512), batch 8, "
+                            "seq 2048, fp32, full M trajectory, forward + whole-sequence segment backward",
+                "batch": bs, "heads": heads, "head_dim": d, "seq_len": s},
+        cpu=lambda: cpu_baseline_hebbian(x, heads))
+
+
 WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
              "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5,
-             "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5}
+             "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5, "hebbian_c2": setup_hebbian_c2}
 
 
 def main():

@@ -92,6 +92,30 @@ void titans_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, co
                                       int t_start, int t_end, int d, int batch_size, int seq_len,
                                       float error_clip);
 
+/* ── Hebbian rule: M <- (1 - alpha) M + v k^T (d in {8, 16, 32, 64, 128}) ────────── */
+/* core/src/cuda_ffi.rs:186 */
+void hebbian_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                              const float *alpha, const float *m_initial,
+                              float *m_states, float *y, int seq_len, int d, int batch_size,
+                              int input_stride, int m_stride);
+/* core/src/cuda_ffi.rs:202 (one chain; d_m_initial is overwritten) */
+void hebbian_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                               const float *alpha, const float *m_states, const float *d_y,
+                               float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                               float *d_alpha, float *d_m_initial, int seq_len, int d);
+/* core/src/cuda_ffi.rs:240 (one chain) */
+void hebbian_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                   const float *alpha, const float *m_initial,
+                                   float *m_states, float *y,
+                                   int seq_len, int d, int checkpoint_interval);
+/* core/src/cuda_ffi.rs:275 */
+void hebbian_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
+                                       const float *alpha, const float *m_states, const float *d_y,
+                                       const float *d_m_seed,
+                                       float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                       float *d_alpha, float *d_m_out,
+                                       int t_start, int t_end, int d, int batch_size, int seq_len);
+
 /* ── Delta rule (Titans without momentum) ────────────────────────────────── */
 /* core/src/cuda_ffi.rs:86 */
 void delta_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,

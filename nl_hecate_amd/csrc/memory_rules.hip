@@ -516,7 +516,7 @@ __global__ void finalize_parts_kernel(const float *ws_dq, const float *ws_dk, co
             ga += wg[0]; ge += wg[1]; gt += wg[2];
         }
         d_alpha[o] = ga;
-        d_theta[o] = gt;
+        if (d_theta) d_theta[o] = gt;
         if (d_eta) d_eta[o] = ge;
     }
 }

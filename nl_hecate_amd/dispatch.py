@@ -93,6 +93,38 @@ def titans_backward_dd_segment(k_mem, v_mem, q_mem, alpha, theta, eta, m_states,
          d_m_out, d_s_out, t_start, t_end, d, batch_size, seq_len, error_clip)
 
 
+# ── Hebbian rule ────────────────────────────────────────────────────────────
+def hebbian_forward_dd(k_mem, v_mem, q_mem, alpha, m_initial, m_states, y,
+                       seq_len, d, batch_size, input_stride, m_stride):
+    """dispatch.rs:2947."""
+    check_forward_strides(seq_len, d, batch_size, input_stride, m_stride)
+    call("hebbian_forward_f32_cuda", k_mem, v_mem, q_mem, alpha, m_initial, m_states, y,
+         seq_len, d, batch_size, input_stride, m_stride)
+
+
+def hebbian_backward_dd(k_mem, v_mem, q_mem, alpha, m_states, d_y,
+                        d_k_mem, d_v_mem, d_q_mem, d_alpha, d_m_initial, seq_len, d):
+    """dispatch.rs:2969 (one chain)."""
+    call("hebbian_backward_f32_cuda", k_mem, v_mem, q_mem, alpha, m_states, d_y,
+         d_k_mem, d_v_mem, d_q_mem, d_alpha, d_m_initial, seq_len, d)
+
+
+def hebbian_forward_dd_ckpt(k_mem, v_mem, q_mem, alpha, m_initial, m_states, y,
+                            seq_len, d, checkpoint_interval):
+    """dispatch.rs:3083 (one chain)."""
+    call("hebbian_forward_ckpt_f32_cuda", k_mem, v_mem, q_mem, alpha, m_initial, m_states, y,
+         seq_len, d, checkpoint_interval)
+
+
+def hebbian_backward_dd_segment(k_mem, v_mem, q_mem, alpha, m_states, d_y, d_m_seed,
+                                d_k_mem, d_v_mem, d_q_mem, d_alpha, d_m_out,
+                                t_start, t_end, d, batch_size, seq_len):
+    """dispatch.rs:3190."""
+    assert t_start < t_end and t_end <= seq_len and d > 0
+    call("hebbian_backward_segment_f32_cuda", k_mem, v_mem, q_mem, alpha, m_states, d_y, d_m_seed,
+         d_k_mem, d_v_mem, d_q_mem, d_alpha, d_m_out, t_start, t_end, d, batch_size, seq_len)
+
+
 # ── Delta rule ──────────────────────────────────────────────────────────────
 def delta_forward_dd(k_mem, v_mem, q_mem, alpha, theta, m_initial, m_states, y,
                      seq_len, d, batch_size, input_stride, m_stride, error_clip, m_norm_max):

@@ -137,6 +137,35 @@ def delta_backward(k, v, q, alpha, theta, m_states, d_y, error_clip=0.0,
     return g
 
 
+def hebbian_forward(k, v, q, alpha, m0, m_norm_max=F32_MAX, checkpoint_interval=0):
+    """rust_hebbian_forward (core/src/dispatch.rs:1566-1601); with checkpoint_interval > 0 m_states holds
+    M_0 and the states after every C-th token and the last one (hebbian_forward.cu:212-268)."""
+    dt = k.dtype
+    sfx, real = _sfx(dt)
+    s, d = k.shape
+    n = s + 1 if checkpoint_interval <= 0 else checkpoint_count(s, checkpoint_interval)
+    m_states = np.zeros((n, d, d), dt)
+    y = np.zeros((s, d), dt)
+    _call("orc_hebbian_forward" + sfx, _c(k, dt), _c(v, dt), _c(q, dt), _c(alpha, dt), _c(m0, dt),
+          m_states, y, s, d, float(m_norm_max), int(checkpoint_interval), real=real)
+    return y, m_states
+
+
+def hebbian_backward(k, v, q, alpha, m_states, d_y, t_lo=0, t_hi=None, d_m_seed=None):
+    """rust_hebbian_backward (core/src/dispatch.rs:1604-1660); segment form as in delta_backward."""
+    dt = k.dtype
+    sfx, real = _sfx(dt)
+    s, d = k.shape
+    t_hi = s if t_hi is None else t_hi
+    g = {n: np.zeros((s, d), dt) for n in ("d_k", "d_v", "d_q")}
+    g["d_alpha"] = np.zeros(s, dt)
+    g["d_m"] = np.zeros((d, d), dt) if d_m_seed is None else _c(d_m_seed, dt).copy()
+    _call("orc_hebbian_backward_range" + sfx, _c(k, dt), _c(v, dt), _c(q, dt), _c(alpha, dt),
+          _c(m_states, dt), _c(d_y, dt), g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_m"],
+          t_lo, t_hi, d, real=real)
+    return g
+
+
 def chunkwise_forward(k, v, q, alpha, theta, eta, m0, s0, chunk_size, has_s=True,
                       error_clip=0.0, m_norm_max=F32_MAX):
     dt = k.dtype
