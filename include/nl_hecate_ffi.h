@@ -548,6 +548,54 @@ void titans_phase2_backward_f32_cuda(const float *k_mem, const float *q_mem, con
                                      float *d_M0, float *m_recompute, float *s_recompute, int seq_len, int d,
                                      int batch_size, int chunk_size, int chunk_idx, float m_norm_max);
 
+/* ── around the memory path: normalisation, embedding, loss, TNT helpers, pooling, M3 helpers ── */
+/* core/src/cuda_ffi.rs:487 */
+void layer_norm_forward_cuda(const float *x, const float *gamma, const float *beta, float *out,
+                             float *mean_cache, float *rstd_cache, int n, int d, float eps);
+/* core/src/cuda_ffi.rs:495 (d_gamma, d_beta are accumulated: the caller zeroes them; d <= 2048) */
+void layer_norm_backward_cuda(const float *d_out, const float *x, const float *gamma, const float *mean_cache,
+                              const float *rstd_cache, float *d_x, float *d_gamma, float *d_beta, int n, int d);
+/* core/src/cuda_ffi.rs:523 */
+void embedding_gather_cuda(const float *w_embed, const int *input_ids, float *output, int seq_len, int d);
+/* core/src/cuda_ffi.rs:532 (d_embed is accumulated) */
+void embedding_scatter_add_cuda(const float *d_embedded, const int *input_ids, float *d_embed, int seq_len, int d);
+/* core/src/cuda_ffi.rs:542: dst[col * rows + row] = src[row * cols + col] */
+void transpose_copy_cuda(const float *src, float *dst, int rows, int cols);
+/* core/src/cuda_ffi.rs:766 (loss_out[0] = sum of the rows' NLL; rows with a target outside [0, vocab) are skipped) */
+void cross_entropy_forward_cuda(const float *logits, const int *target_ids, float *loss_out, int seq_len, int vocab);
+/* core/src/cuda_ffi.rs:772 */
+void cross_entropy_backward_cuda(const float *logits, const int *target_ids, float *d_logits, int seq_len, int vocab,
+                                 float inv_count);
+/* core/src/cuda_ffi.rs:616 */
+void tnt_broadcast_m_f32_cuda(const float *m_src, float *m_dst, int n_local, int d);
+/* core/src/cuda_ffi.rs:624 */
+void tnt_shard_summary_mean_f32_cuda(const float *local_y, float *k_sum, float *v_sum, int shard_len, int d);
+/* core/src/cuda_ffi.rs:633 */
+void tnt_global_update_f32_cuda(float *global_m, const float *k_sum, const float *v_sum, int d, float alpha);
+/* core/src/cuda_ffi.rs:642 (d_k_sum, d_v_sum are accumulated) */
+void tnt_global_update_backward_f32_cuda(const float *d_m_new, const float *k_sum, const float *v_sum,
+                                         float *d_m_old, float *d_k_sum, float *d_v_sum, int d, float alpha);
+/* core/src/cuda_ffi.rs:654 (d_local_y is accumulated) */
+void tnt_shard_summary_mean_backward_f32_cuda(const float *d_k_sum, const float *d_v_sum, float *d_local_y,
+                                              int shard_len, int d);
+/* core/src/cuda_ffi.rs:663 */
+void tnt_combine_gradients_f32_cuda(const float *d_y_upstream, const float *d_y_global, float *d_y_combined, int n);
+/* core/src/cuda_ffi.rs:1061, 1067, 1074 (d_x accumulated), 1081; tokens past the last full group of C are
+ * not read and not written */
+void mean_pool_1d_f32_cuda(const float *x, float *out, int bs, int s, int d, int C);
+void repeat_upsample_1d_f32_cuda(const float *x, float *out, int bs, int s, int d, int C);
+void mean_pool_1d_backward_f32_cuda(const float *d_out, float *d_x, int bs, int s, int d, int C);
+void repeat_upsample_1d_backward_f32_cuda(const float *d_out, float *d_x, int bs, int s, int d, int C);
+/* core/src/cuda_ffi.rs:722, 730, 740, 747, 753, 757; return 0 on success like the AdamW family */
+unsigned m3_ema_update_cuda(float *m1, float *m2, float *v, const float *g, int n, float beta1, float beta2,
+                            float beta3, int update_m2);
+unsigned m3_apply_1d_cuda(float *w, const float *m1, const float *m2, const float *v, int n, float lr, float alpha,
+                          float eps, float bc2);
+unsigned m3_apply_2d_cuda(float *w, const float *o1, const float *o2, int n, float lr, float alpha);
+unsigned frob_norm_sq_cuda(const float *x, float *partial_sums, int n, int *out_num_blocks);
+unsigned scale_buf_cuda(float *x, float scale, int n);
+unsigned m3_ns_poly_cuda(float *x, const float *y, const float *z, int n, float a, float b, float c);
+
 #ifdef __cplusplus
 }
 #endif

@@ -200,6 +200,38 @@ static unsigned launch_status(const char *what) {
 
 using namespace nlh;
 
+// ── M3 optimizer helpers (core/kernels/m3_optimizer.cu) ─────────────────────
+// m3_optimizer.cu:24-42: fast momentum, second moment, and (when update_m2) the slow momentum
+__global__ void m3_ema_kernel(float *__restrict__ m1, float *__restrict__ m2, float *__restrict__ v,
+                              const float *__restrict__ g, int n, float b1, float b2, float b3, int update_m2) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        const float gi = g[i];
+        m1[i] = b1 * m1[i] + (1.0f - b1) * gi;
+        v[i] = b2 * v[i] + (1.0f - b2) * gi * gi;
+        if (update_m2) m2[i] = b3 * m2[i] + (1.0f - b3) * gi;
+    }
+}
+// m3_optimizer.cu:66-80
+__global__ void m3_apply_1d_kernel(float *__restrict__ w, const float *__restrict__ m1, const float *__restrict__ m2,
+                                   const float *__restrict__ v, int n, float lr, float alpha, float eps, float bc2) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        const float combined = m1[i] + alpha * m2[i];
+        w[i] -= lr * combined / (sqrtf(v[i] / bc2) + eps);
+    }
+}
+// m3_optimizer.cu:103-114 (a = -lr, b = -lr alpha) and :204-215 (Newton-Schulz polynomial): x = a x' + b y + c z
+// with x' = x or, for the 2-D update, w itself with coefficient 1
+__global__ void axpbypcz_kernel(float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ z, int n,
+                                float a, float b, float c) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        x[i] = a * x[i] + b * y[i] + c * z[i];
+}
+__global__ void m3_apply_2d_kernel(float *__restrict__ w, const float *__restrict__ o1, const float *__restrict__ o2,
+                                   int n, float lr, float alpha) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        w[i] -= lr * (o1[i] + alpha * o2[i]);
+}
+
 extern "C" {
 
 unsigned adamw_update_cuda(float *w, const float *g, float *m, float *v, int n, float lr, float beta1,
@@ -323,6 +355,43 @@ unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, flo
         if (rc) return rc;
     }
     return 0;
+}
+
+
+// ── M3 optimizer helpers ────────────────────────────────────────────────────
+unsigned m3_ema_update_cuda(float *m1, float *m2, float *v, const float *g, int n, float beta1, float beta2,
+                            float beta3, int update_m2) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(m3_ema_kernel, dim3(opt_blocks(n)), dim3(kOptThreads), 0, stream(), m1, m2, v, g, n, beta1,
+                       beta2, beta3, update_m2);
+    return launch_status("m3_ema_update_cuda");
+}
+
+unsigned m3_apply_1d_cuda(float *w, const float *m1, const float *m2, const float *v, int n, float lr, float alpha,
+                          float eps, float bc2) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(m3_apply_1d_kernel, dim3(opt_blocks(n)), dim3(kOptThreads), 0, stream(), w, m1, m2, v, n, lr,
+                       alpha, eps, bc2);
+    return launch_status("m3_apply_1d_cuda");
+}
+
+unsigned m3_apply_2d_cuda(float *w, const float *o1, const float *o2, int n, float lr, float alpha) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(m3_apply_2d_kernel, dim3(opt_blocks(n)), dim3(kOptThreads), 0, stream(), w, o1, o2, n, lr, alpha);
+    return launch_status("m3_apply_2d_cuda");
+}
+
+// same partial-sum layout as grad_norm_sq_cuda: one partial per 256 elements (m3_optimizer.cu:141-178)
+unsigned frob_norm_sq_cuda(const float *x, float *partial_sums, int n, int *out_num_blocks) {
+    return grad_norm_sq_cuda(x, partial_sums, n, out_num_blocks);
+}
+
+unsigned scale_buf_cuda(float *x, float scale, int n) { return grad_scale_cuda(x, scale, n); }
+
+unsigned m3_ns_poly_cuda(float *x, const float *y, const float *z, int n, float a, float b, float c) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(axpbypcz_kernel, dim3(opt_blocks(n)), dim3(kOptThreads), 0, stream(), x, y, z, n, a, b, c);
+    return launch_status("m3_ns_poly_cuda");
 }
 
 }  // extern "C"
