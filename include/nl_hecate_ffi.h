@@ -548,6 +548,27 @@ void titans_phase2_backward_f32_cuda(const float *k_mem, const float *q_mem, con
                                      float *d_M0, float *m_recompute, float *s_recompute, int seq_len, int d,
                                      int batch_size, int chunk_size, int chunk_idx, float m_norm_max);
 
+/* ── one memory level's glue in one pass (no symbol in cuda_ffi.rs) ───────── */
+/* Replaces, in gpu_memory_forward (core/src/gpu_forward.rs:1197 ff.), l2_normalize_rows x2, gate_compute x3,
+ * transpose_heads x3, broadcast_heads x3 (and the f32 -> bf16 copies when heads_bf16 != 0).  k_mem and q_mem
+ * [bs*s, nh*hd] are normalised in place; alpha = sigmoid, theta = softplus, eta = sigmoid of
+ * w . [k | v] + b; k/v/q_heads are [bs*nh, s, hd] (bf16 bit patterns when heads_bf16, else float), the
+ * *_heads gates [bs*nh, s]. */
+void memory_inputs_fused_rocm(float *k_mem, const float *v_mem, float *q_mem, const float *w_alpha,
+                              const float *b_alpha, const float *w_theta, const float *b_theta, const float *w_eta,
+                              const float *b_eta, float *k_norms, float *q_norms, float *alpha, float *theta,
+                              float *eta, void *k_heads, void *v_heads, void *q_heads, float *alpha_heads,
+                              float *theta_heads, float *eta_heads, int bs, int s, int nh, int hd, float eps,
+                              int heads_bf16);
+/* Replaces, in gpu_memory_backward (core/src/gpu_backward.rs:2047 ff.), sum_heads x3, transpose_heads x3 and
+ * l2_normalize_backward x2: from the rule's head-major gradients to the token-major ones that the gate and
+ * projection gradients take.  k_norm / q_norm are the normalised rows, k_norms / q_norms their former norms. */
+void memory_grads_fused_rocm(const float *d_k_heads, const float *d_v_heads, const float *d_q_heads,
+                             const float *d_alpha_heads, const float *d_theta_heads, const float *d_eta_heads,
+                             const float *k_norm, const float *q_norm, const float *k_norms, const float *q_norms,
+                             float *d_k_in, float *d_v, float *d_q_in, float *d_alpha, float *d_theta, float *d_eta,
+                             int bs, int s, int nh, int hd, float eps);
+
 /* ── around the memory path: normalisation, embedding, loss, TNT helpers, pooling, M3 helpers ── */
 /* core/src/cuda_ffi.rs:487 */
 void layer_norm_forward_cuda(const float *x, const float *gamma, const float *beta, float *out,

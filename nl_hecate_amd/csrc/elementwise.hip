@@ -171,6 +171,105 @@ __global__ void gate_compute_kernel(const float *__restrict__ k, const float *__
     }
 }
 
+// ── the glue of one memory level's forward in one pass over the tokens ──────
+// gpu_memory_forward (core/src/gpu_forward.rs:1197 ff.) runs, per level: row L2 norm of k and q, three
+// gate projections on the normalised k and v, the head split of k, v, q and the per-head copies of the
+// gates: eleven launches that each stream [n, d] tensors.  Here one wave owns a token: it normalises k
+// and q in place (the backward needs them), writes the norms and the token-major gates, and emits the
+// head-major tensors directly (as bf16 when KV16: what the matrix-core chunkwise rule takes).  Sums run
+// over the same lane pattern as the separate kernels, so the results are the same numbers.
+template <bool KV16>
+__global__ void memory_inputs_fused_kernel(float *__restrict__ k, const float *__restrict__ v, float *__restrict__ q,
+                                           const float *__restrict__ w_alpha, const float *__restrict__ b_alpha,
+                                           const float *__restrict__ w_theta, const float *__restrict__ b_theta,
+                                           const float *__restrict__ w_eta, const float *__restrict__ b_eta,
+                                           float *__restrict__ k_norms, float *__restrict__ q_norms,
+                                           float *__restrict__ alpha, float *__restrict__ theta, float *__restrict__ eta,
+                                           void *__restrict__ kh, void *__restrict__ vh, void *__restrict__ qh,
+                                           float *__restrict__ ah, float *__restrict__ th, float *__restrict__ eh,
+                                           int bs, int s, int nh, int hd, float eps) {
+    const int lane = threadIdx.x & 63, d = nh * hd;
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
+    const float ba = b_alpha[0], bt = b_theta[0], be = b_eta[0];
+    for (int tok = wave; tok < bs * s; tok += nwaves) {
+        float *kr = k + (size_t)tok * d, *qr = q + (size_t)tok * d;
+        const float *vr = v + (size_t)tok * d;
+        float sk = 0.f, sq = 0.f;
+        for (int i = lane; i < d; i += 64) { const float a = kr[i], c = qr[i]; sk += a * a; sq += c * c; }
+        const float kn = sqrtf(wave_allreduce(sk)), qn = sqrtf(wave_allreduce(sq));
+        const float ki = 1.0f / fmaxf(kn, eps), qi = 1.0f / fmaxf(qn, eps);
+        const int b = tok / s, t = tok % s;
+        float ga = 0.f, gt = 0.f, ge = 0.f;
+        for (int i = lane; i < d; i += 64) {
+            const float kk = kr[i] * ki, qq = qr[i] * qi, vv = vr[i];
+            kr[i] = kk;
+            qr[i] = qq;
+            ga += kk * w_alpha[i] + vv * w_alpha[d + i];
+            gt += kk * w_theta[i] + vv * w_theta[d + i];
+            ge += kk * w_eta[i] + vv * w_eta[d + i];
+            const size_t o = (((size_t)b * nh + i / hd) * s + t) * hd + i % hd;
+            if (KV16) {
+                reinterpret_cast<__bf16 *>(kh)[o] = (__bf16)kk;
+                reinterpret_cast<__bf16 *>(vh)[o] = (__bf16)vv;
+                reinterpret_cast<__bf16 *>(qh)[o] = (__bf16)qq;
+            } else {
+                reinterpret_cast<float *>(kh)[o] = kk;
+                reinterpret_cast<float *>(vh)[o] = vv;
+                reinterpret_cast<float *>(qh)[o] = qq;
+            }
+        }
+        const float al = sigmoidf_(wave_allreduce(ga) + ba), tht = softplusf_(wave_allreduce(gt) + bt);
+        const float et = sigmoidf_(wave_allreduce(ge) + be);
+        if (lane == 0) { k_norms[tok] = kn; q_norms[tok] = qn; alpha[tok] = al; theta[tok] = tht; eta[tok] = et; }
+        for (int h = lane; h < nh; h += 64) {
+            const size_t o = ((size_t)b * nh + h) * s + t;
+            ah[o] = al; th[o] = tht; eh[o] = et;
+        }
+    }
+}
+
+// The glue of the level's backward between the rule and the projections: head sums of the gate
+// gradients, head merge of d_k, d_v, d_q and the backward of the two row normalisations
+// (gpu_memory_backward, core/src/gpu_backward.rs:2047 ff.: eight launches), one wave per token.
+__global__ void memory_grads_fused_kernel(const float *__restrict__ dkh, const float *__restrict__ dvh,
+                                          const float *__restrict__ dqh, const float *__restrict__ dah,
+                                          const float *__restrict__ dth, const float *__restrict__ deh,
+                                          const float *__restrict__ k_norm, const float *__restrict__ q_norm,
+                                          const float *__restrict__ k_norms, const float *__restrict__ q_norms,
+                                          float *__restrict__ dk_in, float *__restrict__ dv, float *__restrict__ dq_in,
+                                          float *__restrict__ d_alpha, float *__restrict__ d_theta,
+                                          float *__restrict__ d_eta, int bs, int s, int nh, int hd, float eps) {
+    const int lane = threadIdx.x & 63, d = nh * hd;
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
+    for (int tok = wave; tok < bs * s; tok += nwaves) {
+        const int b = tok / s, t = tok % s;
+        if (lane < 3) {   // sum_heads: serial over the heads, as the separate kernel
+            const float *src = lane == 0 ? dah : (lane == 1 ? dth : deh);
+            float acc = 0.f;
+            for (int h = 0; h < nh; h++) acc += src[((size_t)b * nh + h) * s + t];
+            (lane == 0 ? d_alpha : (lane == 1 ? d_theta : d_eta))[tok] = acc;
+        }
+        const float *kx = k_norm + (size_t)tok * d, *qx = q_norm + (size_t)tok * d;
+        float dk_dot = 0.f, dq_dot = 0.f;
+        for (int i = lane; i < d; i += 64) {
+            const size_t o = (((size_t)b * nh + i / hd) * s + t) * hd + i % hd;
+            dk_dot += dkh[o] * kx[i];
+            dq_dot += dqh[o] * qx[i];
+        }
+        dk_dot = wave_allreduce(dk_dot);
+        dq_dot = wave_allreduce(dq_dot);
+        const float kn = k_norms[tok], qn = q_norms[tok];
+        const float ki = 1.0f / fmaxf(kn, eps), qi = 1.0f / fmaxf(qn, eps), inv_eps = 1.0f / eps;
+        for (int i = lane; i < d; i += 64) {
+            const size_t o = (((size_t)b * nh + i / hd) * s + t) * hd + i % hd;
+            const float gk = dkh[o], gq = dqh[o];
+            dk_in[(size_t)tok * d + i] = kn >= eps ? (gk - kx[i] * dk_dot) * ki : gk * inv_eps;
+            dq_in[(size_t)tok * d + i] = qn >= eps ? (gq - qx[i] * dq_dot) * qi : gq * inv_eps;
+            dv[(size_t)tok * d + i] = dvh[o];
+        }
+    }
+}
+
 // ── gate backward: d_w[2D] and d_b for alpha / theta / eta ──────────────────
 // Stage 1: each workgroup owns a token range and every thread a set of the 2D
 // columns; stage 2 sums the per-workgroup partials in a fixed order.
@@ -464,6 +563,39 @@ void gate_compute_cuda(const float *k_mem, const float *v_mem, const float *w_ga
     hipLaunchKernelGGL(gate_compute_kernel, dim3(ew_blocks((long long)seq_len * 64)), dim3(kEwThreads), 0,
                        stream(), k_mem, v_mem, w_gate, bias_ptr, gate_out, seq_len, d, activation);
     check_launch("gate_compute_kernel");
+}
+
+void memory_inputs_fused_rocm(float *k_mem, const float *v_mem, float *q_mem, const float *w_alpha,
+                              const float *b_alpha, const float *w_theta, const float *b_theta, const float *w_eta,
+                              const float *b_eta, float *k_norms, float *q_norms, float *alpha, float *theta,
+                              float *eta, void *k_heads, void *v_heads, void *q_heads, float *alpha_heads,
+                              float *theta_heads, float *eta_heads, int bs, int s, int nh, int hd, float eps,
+                              int heads_bf16) {
+    const long long n = (long long)bs * s;
+    if (n <= 0 || nh <= 0 || hd <= 0) return;
+    const dim3 grid(ew_blocks(n * 64)), blk(kEwThreads);
+    if (heads_bf16)
+        hipLaunchKernelGGL(memory_inputs_fused_kernel<true>, grid, blk, 0, stream(), k_mem, v_mem, q_mem, w_alpha,
+                           b_alpha, w_theta, b_theta, w_eta, b_eta, k_norms, q_norms, alpha, theta, eta, k_heads, v_heads,
+                           q_heads, alpha_heads, theta_heads, eta_heads, bs, s, nh, hd, eps);
+    else
+        hipLaunchKernelGGL(memory_inputs_fused_kernel<false>, grid, blk, 0, stream(), k_mem, v_mem, q_mem, w_alpha,
+                           b_alpha, w_theta, b_theta, w_eta, b_eta, k_norms, q_norms, alpha, theta, eta, k_heads, v_heads,
+                           q_heads, alpha_heads, theta_heads, eta_heads, bs, s, nh, hd, eps);
+    check_launch("memory_inputs_fused_kernel");
+}
+
+void memory_grads_fused_rocm(const float *d_k_heads, const float *d_v_heads, const float *d_q_heads,
+                             const float *d_alpha_heads, const float *d_theta_heads, const float *d_eta_heads,
+                             const float *k_norm, const float *q_norm, const float *k_norms, const float *q_norms,
+                             float *d_k_in, float *d_v, float *d_q_in, float *d_alpha, float *d_theta, float *d_eta,
+                             int bs, int s, int nh, int hd, float eps) {
+    const long long n = (long long)bs * s;
+    if (n <= 0 || nh <= 0 || hd <= 0) return;
+    hipLaunchKernelGGL(memory_grads_fused_kernel, dim3(ew_blocks(n * 64)), dim3(kEwThreads), 0, stream(), d_k_heads,
+                       d_v_heads, d_q_heads, d_alpha_heads, d_theta_heads, d_eta_heads, k_norm, q_norm, k_norms, q_norms,
+                       d_k_in, d_v, d_q_in, d_alpha, d_theta, d_eta, bs, s, nh, hd, eps);
+    check_launch("memory_grads_fused_kernel");
 }
 
 void gate_backward_cuda(const float *d_alpha, const float *alpha, const float *d_theta,

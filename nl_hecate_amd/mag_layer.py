@@ -104,6 +104,7 @@ class MagLayer:
             l.w_k, l.w_v, l.w_q = views[3 + 3 * lv], views[4 + 3 * lv], views[5 + 3 * lv]
         self.split_gemm = True
         self.stack_levels = True   # chunkwise rule: active levels run as one batch of chains
+        self.fused_glue = True     # one pass per level for the glue either side of the rule
         # per-level context memory, one matrix per (batch element, head); created on first use
         self.m_state: List[Optional[torch.Tensor]] = [None] * k
         self.s_state: List[Optional[torch.Tensor]] = [None] * k
@@ -203,16 +204,21 @@ class MagLayer:
         v_mem = self._project(ops, x2, lp.w_v, 4 + 3 * lv)
         q_mem = self._project(ops, x2, lp.w_q, 5 + 3 * lv)
         k_norms, q_norms = _new(n), _new(n)
-        D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
-        D.call("l2_normalize_rows_f32_cuda", q_mem, q_norms, n, d, 1e-8)
         alpha, theta, eta = _new(n), _new(n), _new(n)
-        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_alpha, lp.b_alpha, alpha, n, d, 0)
-        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_theta, lp.b_theta, theta, n, d, 1)
-        D.call("gate_compute_cuda", k_mem, v_mem, lp.w_eta, lp.b_eta, eta, n, d, 0)
-        for src, dst_t in zip((k_mem, v_mem, q_mem), dst[:3]):
-            D.call("transpose_heads_f32_cuda", src, dst_t, bs, s, nh, hd, 1)
-        for src, dst_t in zip((alpha, theta, eta), dst[3:]):
-            D.call("broadcast_heads_f32_cuda", src, dst_t, bs, s, nh)
+        if self.fused_glue:   # the eleven launches below as one pass over the tokens
+            D.call("memory_inputs_fused_rocm", k_mem, v_mem, q_mem, lp.w_alpha, lp.b_alpha, lp.w_theta, lp.b_theta,
+                   lp.w_eta, lp.b_eta, k_norms, q_norms, alpha, theta, eta, *dst, bs, s, nh, hd, 1e-8,
+                   int(dst[0].dtype == torch.bfloat16))
+        else:
+            D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
+            D.call("l2_normalize_rows_f32_cuda", q_mem, q_norms, n, d, 1e-8)
+            D.call("gate_compute_cuda", k_mem, v_mem, lp.w_alpha, lp.b_alpha, alpha, n, d, 0)
+            D.call("gate_compute_cuda", k_mem, v_mem, lp.w_theta, lp.b_theta, theta, n, d, 1)
+            D.call("gate_compute_cuda", k_mem, v_mem, lp.w_eta, lp.b_eta, eta, n, d, 0)
+            for src, dst_t in zip((k_mem, v_mem, q_mem), dst[:3]):
+                D.call("transpose_heads_f32_cuda", src, dst_t, bs, s, nh, hd, 1)
+            for src, dst_t in zip((alpha, theta, eta), dst[3:]):
+                D.call("broadcast_heads_f32_cuda", src, dst_t, bs, s, nh)
         return dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, k_norms=k_norms, q_norms=q_norms, active=True, ops=ops,
                     alpha=alpha, theta=theta, eta=eta)
 
@@ -224,7 +230,8 @@ class MagLayer:
         d, nh, hd, C = self.d, self.nh, self.hd, self.chunk
         B = bs * nh
         self.ensure_state(bs)
-        kh, vh, qh = _new(na * B, s, hd), _new(na * B, s, hd), _new(na * B, s, hd)
+        hdt = torch.bfloat16 if self.fused_glue else torch.float32   # the fused glue writes bf16 heads itself
+        kh, vh, qh = (_new(na * B, s, hd, dtype=hdt) for _ in range(3))
         ah, th, eh = _new(na * B, s), _new(na * B, s), _new(na * B, s)
         caches = []
         for lv in range(na):
@@ -297,17 +304,21 @@ class MagLayer:
         n = bs * s
         dkh, dvh, dqh, dah, dth, deh = head_grads
         d_alpha, d_theta, d_eta = _new(n), _new(n), _new(n)
-        for src, dst in ((dah, d_alpha), (dth, d_theta), (deh, d_eta)):
-            D.call("sum_heads_f32_cuda", src, dst, bs, s, nh)
-        dk, dv, dq = _new(n, d), _new(n, d), _new(n, d)
-        for src, dst in ((dkh, dk), (dvh, dv), (dqh, dq)):
-            D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 0)
+        dk_in, dv, dq_in = _new(n, d), _new(n, d), _new(n, d)
+        if self.fused_glue:   # head sums, head merge and both normalisation backwards in one pass
+            D.call("memory_grads_fused_rocm", dkh, dvh, dqh, dah, dth, deh, c["k_mem"], c["q_mem"], c["k_norms"],
+                   c["q_norms"], dk_in, dv, dq_in, d_alpha, d_theta, d_eta, bs, s, nh, hd, 1e-8)
+        else:
+            for src, dst in ((dah, d_alpha), (dth, d_theta), (deh, d_eta)):
+                D.call("sum_heads_f32_cuda", src, dst, bs, s, nh)
+            dk, dq = _new(n, d), _new(n, d)
+            for src, dst in ((dkh, dk), (dvh, dv), (dqh, dq)):
+                D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 0)
+            D.call("l2_normalize_backward_f32_cuda", dk, c["k_mem"], c["k_norms"], dk_in, n, d, 1e-8)
+            D.call("l2_normalize_backward_f32_cuda", dq, c["q_mem"], c["q_norms"], dq_in, n, d, 1e-8)
         # gate projections (d_w, d_b) from the cached gate outputs
         D.call("gate_backward_cuda", d_alpha, c["alpha"], d_theta, c["theta"], d_eta, c["eta"], c["k_mem"],
                c["v_mem"], g.w_alpha, g.b_alpha, g.w_theta, g.b_theta, g.w_eta, g.b_eta, n, d, 1, 1)
-        dk_in, dq_in = _new(n, d), _new(n, d)
-        D.call("l2_normalize_backward_f32_cuda", dk, c["k_mem"], c["k_norms"], dk_in, n, d, 1e-8)
-        D.call("l2_normalize_backward_f32_cuda", dq, c["q_mem"], c["q_norms"], dq_in, n, d, 1e-8)
         g.w_k += _wgrad(dk_in, x2)
         g.w_v += _wgrad(dv, x2)
         g.w_q += _wgrad(dq_in, x2)

@@ -235,3 +235,65 @@ def test_multi_tensor_adamw_and_clip():
         orc.adamw_step(ws[i], gi, ms[i], vs[i], lr, b1, b2, eps, bc1[i], bc2[i], wd)
         assert_close(f"w[{i}]", host(dws[i]), ws[i], 1e-6)
         assert_close(f"v[{i}]", host(dvs[i]), vs[i], 1e-6)
+
+
+@pytest.mark.parametrize("bs,s,nh,hd,bf16", [(2, 37, 4, 16, False), (1, 100, 8, 64, True), (3, 5, 2, 24, True)])
+def test_fused_level_glue_equals_the_separate_kernels(bs, s, nh, hd, bf16):
+    """memory_inputs_fused_rocm / memory_grads_fused_rocm against the launches they replace
+    (l2_normalize_rows, gate_compute, transpose_heads, broadcast_heads, sum_heads, l2_normalize_backward):
+    same lane pattern in every sum, so equal to the last bit."""
+    d, n, B = nh * hd, bs * s, bs * nh
+    g = torch.Generator(device="cuda").manual_seed(5 + s)
+    rn = lambda *sh: torch.randn(*sh, device="cuda", generator=g)
+    k0, v, q0 = rn(n, d), rn(n, d), rn(n, d)
+    k0[3 % n] = 0.0   # a zero row takes the norm < eps branch of the backward
+    w = [0.1 * rn(2 * d) for _ in range(3)]
+    bias = [rn(1) for _ in range(3)]
+    # separate kernels
+    k1, q1 = k0.clone(), q0.clone()
+    kn1, qn1 = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    D.call("l2_normalize_rows_f32_cuda", k1, kn1, n, d, 1e-8)
+    D.call("l2_normalize_rows_f32_cuda", q1, qn1, n, d, 1e-8)
+    gates1 = [torch.zeros(n, device="cuda") for _ in range(3)]
+    for gt, ww, bb, act in zip(gates1, w, bias, (0, 1, 0)):
+        D.call("gate_compute_cuda", k1, v, ww, bb, gt, n, d, act)
+    heads1 = [torch.zeros(B, s, hd, device="cuda") for _ in range(3)]
+    for src, dst in zip((k1, v, q1), heads1):
+        D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 1)
+    gh1 = [torch.zeros(B, s, device="cuda") for _ in range(3)]
+    for src, dst in zip(gates1, gh1):
+        D.call("broadcast_heads_f32_cuda", src, dst, bs, s, nh)
+    # fused
+    k2, q2 = k0.clone(), q0.clone()
+    kn2, qn2 = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    gates2 = [torch.zeros(n, device="cuda") for _ in range(3)]
+    hdt = torch.bfloat16 if bf16 else torch.float32
+    heads2 = [torch.zeros(B, s, hd, device="cuda", dtype=hdt) for _ in range(3)]
+    gh2 = [torch.zeros(B, s, device="cuda") for _ in range(3)]
+    D.call("memory_inputs_fused_rocm", k2, v, q2, w[0], bias[0], w[1], bias[1], w[2], bias[2], kn2, qn2, *gates2,
+           *heads2, *gh2, bs, s, nh, hd, 1e-8, int(bf16))
+    torch.cuda.synchronize()
+    assert torch.equal(k1, k2) and torch.equal(q1, q2) and torch.equal(kn1, kn2) and torch.equal(qn1, qn2)
+    for a, b in zip(gates1 + gh1, gates2 + gh2):
+        assert torch.equal(a, b)
+    for a, b in zip(heads1, heads2):
+        assert torch.equal(a.to(hdt), b)
+    # backward glue
+    dh = [rn(B, s, hd) for _ in range(3)]
+    dg = [rn(B, s) for _ in range(3)]
+    tok1 = [torch.zeros(n, d, device="cuda") for _ in range(3)]
+    for src, dst in zip(dh, tok1):
+        D.call("transpose_heads_f32_cuda", src, dst, bs, s, nh, hd, 0)
+    dgs1 = [torch.zeros(n, device="cuda") for _ in range(3)]
+    for src, dst in zip(dg, dgs1):
+        D.call("sum_heads_f32_cuda", src, dst, bs, s, nh)
+    dk1, dq1 = torch.zeros(n, d, device="cuda"), torch.zeros(n, d, device="cuda")
+    D.call("l2_normalize_backward_f32_cuda", tok1[0], k1, kn1, dk1, n, d, 1e-8)
+    D.call("l2_normalize_backward_f32_cuda", tok1[2], q1, qn1, dq1, n, d, 1e-8)
+    dk2, dv2, dq2 = (torch.zeros(n, d, device="cuda") for _ in range(3))
+    dgs2 = [torch.zeros(n, device="cuda") for _ in range(3)]
+    D.call("memory_grads_fused_rocm", *dh, *dg, k1, q1, kn1, qn1, dk2, dv2, dq2, *dgs2, bs, s, nh, hd, 1e-8)
+    torch.cuda.synchronize()
+    assert torch.equal(dk1, dk2) and torch.equal(tok1[1], dv2) and torch.equal(dq1, dq2)
+    for a, b in zip(dgs1, dgs2):
+        assert torch.equal(a, b)
