@@ -103,6 +103,7 @@ class MagLayer:
         for lv, l in enumerate(self.p.levels):
             l.w_k, l.w_v, l.w_q = views[3 + 3 * lv], views[4 + 3 * lv], views[5 + 3 * lv]
         self.split_gemm = True
+        self.split_wgrad = True    # weight gradients of a projection group from the same packed operand
         self.stack_levels = True   # chunkwise rule: active levels run as one batch of chains
         self.fused_glue = True     # one pass per level for the glue either side of the rule
         # per-level context memory, one matrix per (batch element, head); created on first use
@@ -129,13 +130,34 @@ class MagLayer:
         wh = self._pack.to(torch.bfloat16)
         wl = (self._pack - wh.float()).to(torch.bfloat16)
         wht, wlt = (w.view(groups, 3 * d, d).transpose(1, 2) for w in (wh, wl))   # [group, d_in, 3 d_out]
-        return self._pack_split([x2]), torch.cat([wh, wh, wl], 1), torch.cat([wht, wht, wlt], 2).contiguous()
+        xa = self._pack_split([x2])                                               # [n, 3d]: xh | xl | xh
+        xw = torch.cat([xa[:, :d], xa[:, 2 * d:], xa[:, d:2 * d]], 1)             # [n, 3d]: xh | xh | xl
+        return xa, torch.cat([wh, wh, wl], 1), torch.cat([wht, wht, wlt], 2).contiguous(), xw
 
-    def _input_grad(self, ops, group, grads3, weights3):
-        """sum_s grads3[s] @ weights3[s] for projection group `group` (0: attention q, k, v; 1 + lv: level k, v, q)."""
-        if ops is None:
-            return grads3[0] @ weights3[0] + grads3[1] @ weights3[1] + grads3[2] @ weights3[2]
-        return torch.mm(self._pack_split(list(grads3)), ops[2][group].t(), out_dtype=torch.float32)
+    def _group_grads(self, ops, group, x2, grads3, weights3, wgrads3):
+        """Projection group `group` (0: attention q, k, v; 1 + lv: level k, v, q): adds the three weight gradients
+        grads3[s]^T x2 to wgrads3 and returns the input gradient sum_s grads3[s] @ weights3[s].
+        With split operands both come from ONE packing of the three upstream gradients, P = [H | L | H] (9d wide,
+        H / L the hi / lo bf16 parts of [g0 | g1 | g2]): the input gradient as P . [Wh^T | Wh^T | Wl^T], and the
+        weight gradients, the contraction now over tokens, by reading P as 3n rows (H_t, L_t, H_t) against the rows
+        (xh_t, xh_t, xl_t) of x: G^T x ~ H^T xh + L^T xh + H^T xl in one bf16 GEMM with fp32 accumulation, cut into
+        up to 16 slabs along the contraction like _wgrad."""
+        d = self.d
+        n = x2.shape[0]
+        if ops is None or not self.split_wgrad:
+            for g, w in zip(grads3, wgrads3):
+                w += _wgrad(g, x2)
+            if ops is None:
+                return grads3[0] @ weights3[0] + grads3[1] @ weights3[1] + grads3[2] @ weights3[2]
+            return torch.mm(self._pack_split(list(grads3)), ops[2][group].t(), out_dtype=torch.float32)
+        P = self._pack_split(list(grads3))
+        parts = next(p for p in (16, 8, 4, 2, 1) if (3 * n) % p == 0)
+        rows = 3 * n // parts
+        dw = torch.bmm(P.view(parts, rows, 3 * d).transpose(1, 2), ops[3].view(parts, rows, d),
+                       out_dtype=torch.float32).sum(0)                            # [3 d_out, d_in]
+        for i, w in enumerate(wgrads3):
+            w += dw[i * d:(i + 1) * d]
+        return torch.mm(P, ops[2][group].t(), out_dtype=torch.float32)
 
     def _project(self, ops, x2, w, index):
         """x2 @ w^T for the packed projection number `index` (w is its fp32 view)."""
@@ -319,10 +341,8 @@ class MagLayer:
         # gate projections (d_w, d_b) from the cached gate outputs
         D.call("gate_backward_cuda", d_alpha, c["alpha"], d_theta, c["theta"], d_eta, c["eta"], c["k_mem"],
                c["v_mem"], g.w_alpha, g.b_alpha, g.w_theta, g.b_theta, g.w_eta, g.b_eta, n, d, 1, 1)
-        g.w_k += _wgrad(dk_in, x2)
-        g.w_v += _wgrad(dv, x2)
-        g.w_q += _wgrad(dq_in, x2)
-        return self._input_grad(c.get("ops"), 1 + lv, (dk_in, dv, dq_in), (lp.w_k, lp.w_v, lp.w_q))
+        return self._group_grads(c.get("ops"), 1 + lv, x2, (dk_in, dv, dq_in), (lp.w_k, lp.w_v, lp.w_q),
+                                 (g.w_k, g.w_v, g.w_q))
 
     # ── the layer ────────────────────────────────────────────────────────────
     def forward(self, x):
@@ -381,10 +401,8 @@ class MagLayer:
         D.call("swa_backward_f32_cuda", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv, s, nh,
                hd, self.window, bs, 0)
         dq2, dk2, dv2 = dq.view(n, d), dk.view(n, d), dv.view(n, d)
-        grads.w_q += _wgrad(dq2, x2)
-        grads.w_k += _wgrad(dk2, x2)
-        grads.w_v += _wgrad(dv2, x2)
-        d_x += self._input_grad(cache["ops"], 0, (dq2, dk2, dv2), (p.w_q, p.w_k, p.w_v))
+        d_x += self._group_grads(cache["ops"], 0, x2, (dq2, dk2, dv2), (p.w_q, p.w_k, p.w_v),
+                                 (grads.w_q, grads.w_k, grads.w_v))
         return d_x.view(bs, s, d), grads
 
 
