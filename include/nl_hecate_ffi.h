@@ -569,6 +569,17 @@ void memory_grads_fused_rocm(const float *d_k_heads, const float *d_v_heads, con
                              float *d_k_in, float *d_v, float *d_q_in, float *d_alpha, float *d_theta, float *d_eta,
                              int bs, int s, int nh, int hd, float eps);
 
+/* ── SwiGLU MLP, device-to-device (the GEMMs go to rocBLAS on the library's stream) ── */
+/* core/src/cuda_ffi.rs:925 */
+void swiglu_forward_f32_cuda_dd(const float *x, const float *gate_proj, const float *up_proj, const float *down_proj,
+                                float *y, float *gate_buf, float *up_buf, float *fused_buf, float *cache_buf,
+                                int seq_len, int d_model, int intermediate);
+/* core/src/cuda_ffi.rs:945 (output gradients are written, not accumulated) */
+void swiglu_backward_f32_cuda_dd(const float *d_y, const float *x, const float *gate_proj, const float *up_proj,
+                                 const float *down_proj, const float *fused_buf, const float *gate_buf,
+                                 const float *up_buf, const float *cache_buf, float *d_x, float *d_gate_proj,
+                                 float *d_up_proj, float *d_down_proj, int seq_len, int d_model, int intermediate);
+
 /* ── around the memory path: normalisation, embedding, loss, TNT helpers, pooling, M3 helpers ── */
 /* core/src/cuda_ffi.rs:487 */
 void layer_norm_forward_cuda(const float *x, const float *gamma, const float *beta, float *out,

@@ -144,3 +144,19 @@ def m3_apply_2d(w, o1, o2, lr, alpha):
 def m3_ns_poly(x, y, z, a, b, c):
     f = x.dtype.type
     return f(a) * x + f(b) * y + f(c) * z
+
+
+# core/kernels/swiglu_forward.cu:144-158, 301-355; swiglu_backward.cu:174-197, 411-500
+def swiglu_forward(x, gate_proj, up_proj, down_proj):
+    gate, up = x @ gate_proj.T, x @ up_proj.T
+    sig = 1.0 / (1.0 + np.exp(-gate))
+    fused = gate * sig * up
+    return fused @ down_proj.T, gate, up, fused, sig
+
+
+def swiglu_backward(d_y, x, gate_proj, up_proj, down_proj, fused, gate, up, sig):
+    d_fused = d_y @ down_proj
+    d_down = d_y.T @ fused
+    d_gate = d_fused * up * (sig * (1.0 + gate * (1.0 - sig)))
+    d_up = d_fused * gate * sig
+    return d_gate @ gate_proj + d_up @ up_proj, d_gate.T @ x, d_up.T @ x, d_down

@@ -170,3 +170,22 @@ def test_m3_helpers():
     assert D.call("frob_norm_sq_cuda", dev(w), parts, n, ctypes.byref(nb)) == 0
     assert nb.value == (n + 255) // 256
     assert abs(float(host(parts).astype(np.float64).sum()) - float((w.astype(np.float64) ** 2).sum())) < 1e-4 * n
+
+
+@pytest.mark.parametrize("s,d,inter", [(37, 48, 100), (512, 512, 1408), (1, 8, 8)])
+def test_swiglu_forward_backward(s, d, inter):
+    rn = _r(s + inter)
+    x, wg, wu, wd, gy = rn(s, d), rn(inter, d) / d ** 0.5, rn(inter, d) / d ** 0.5, rn(d, inter) / inter ** 0.5, rn(s, d)
+    y, gate, up, fused, cache = zeros(s, d), zeros(s, inter), zeros(s, inter), zeros(s, inter), zeros(s, inter)
+    D.call("swiglu_forward_f32_cuda_dd", dev(x), dev(wg), dev(wu), dev(wd), y, gate, up, fused, cache, s, d, inter)
+    x64, g64, u64, d64 = (a.astype(np.float64) for a in (x, wg, wu, wd))
+    oy, og, ou, of, osig = G.swiglu_forward(x64, g64, u64, d64)
+    for name, got, want in (("y", y, oy), ("gate", gate, og), ("up", up, ou), ("fused", fused, of), ("sigmoid", cache, osig)):
+        assert_close(name, host(got), want)
+    dx = dev(np.full((s, d), 5.0, f32))   # written fresh, not accumulated
+    dg, du, dd = zeros(inter, d), zeros(inter, d), zeros(d, inter)
+    D.call("swiglu_backward_f32_cuda_dd", dev(gy), dev(x), dev(wg), dev(wu), dev(wd), fused, gate, up, cache, dx, dg, du,
+           dd, s, d, inter)
+    wx, wgg, wuu, wdd = G.swiglu_backward(gy.astype(np.float64), x64, g64, u64, d64, of, og, ou, osig)
+    for name, got, want in (("d_x", dx, wx), ("d_gate_proj", dg, wgg), ("d_up_proj", du, wuu), ("d_down_proj", dd, wdd)):
+        assert_close(name, host(got), want)

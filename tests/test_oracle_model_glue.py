@@ -109,3 +109,16 @@ def test_m3_helpers_closed_forms():
     assert np.allclose(G.m3_apply_1d(w, m1, m2, v, 0.1, 0.5, 1e-8, 0.7), w - 0.1 * (m1 + 0.5 * m2) / (np.sqrt(v / 0.7) + 1e-8))
     assert np.allclose(G.m3_apply_2d(w, m1, m2, 0.1, 0.5), w - 0.1 * (m1 + 0.5 * m2))
     assert np.allclose(G.m3_ns_poly(w, m1, m2, 3.4445, -4.775, 2.0315), 3.4445 * w - 4.775 * m1 + 2.0315 * m2)
+
+
+def test_swiglu_matches_torch_silu_mlp_and_autograd():
+    s, d, inter = 6, 5, 9
+    x, wg, wu, wd, gy = (R.standard_normal(sh) for sh in ((s, d), (inter, d), (inter, d), (d, inter), (s, d)))
+    y, gate, up, fused, sig = G.swiglu_forward(x, wg, wu, wd)
+    xt, gt, ut, dt = T(x, True), T(wg, True), T(wu, True), T(wd, True)
+    yt = (F.silu(xt @ gt.T) * (xt @ ut.T)) @ dt.T
+    assert np.allclose(y, yt.detach().numpy(), atol=1e-12)
+    yt.backward(T(gy))
+    dx, dg, du, dd = G.swiglu_backward(gy, x, wg, wu, wd, fused, gate, up, sig)
+    for got, want in ((dx, xt.grad), (dg, gt.grad), (du, ut.grad), (dd, dt.grad)):
+        assert np.allclose(got, want.numpy(), atol=1e-11)
