@@ -134,3 +134,34 @@ def test_graph_replayed_steps_match_eager_steps():
             assert torch.allclose(a, b, rtol=1e-5, atol=1e-7)
         for a, b in zip(graphed.layer.m_state, eager.layer.m_state):
             assert torch.allclose(a, b, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("frozen_second", [False, True])
+def test_decode_steps_reproduce_the_full_sequence_forward(frozen_second):
+    """Token-by-token decode with the KV cache (gpu_single_token_forward, gpu_forward.rs:3377 ff.) against one
+    forward over the whole sequence, exact rule: the recurrence is sequential and the attention row of the
+    newest token sees the same keys, so both give the same outputs and leave the same context memories.
+    Projections differ in the last bits (split-bf16 GEMM vs fp32), which can flip a bf16 rounding of q/k/v:
+    compared at the bf16 tolerance of the attention branch."""
+    from nl_hecate_amd.cms import Pulse
+    torch.manual_seed(3)
+    d, heads, s, window = 128, 2, 40, 16
+    mk = lambda: MagLayer(d, heads, 2, window, [1, 1], rule="exact", chunk=8, seed=21)
+    full, dec = mk(), mk()
+    x = torch.randn(1, s, d, device="cuda") / d ** 0.5
+    pulse = Pulse(0, [True, not frozen_second])
+    for layer in (full, dec):   # a non-trivial memory for the frozen level to read
+        layer.ensure_state(1)
+        layer.m_state[1].copy_(0.05 * torch.randn_like(layer.m_state[1]))
+    dec.m_state[1].copy_(full.m_state[1])
+    full.conductor.pulse = lambda: pulse
+    out_full, _ = full.forward(x)
+    dec.decode_reset(s)
+    outs = [dec.decode_step(x[0, t], pulse) for t in range(s)]
+    out_dec = torch.stack(outs)
+    torch.cuda.synchronize()
+    err = (out_dec - out_full[0]).abs().max().item() / out_full.abs().max().item()
+    assert err < 2e-2, err
+    for lv in range(2):
+        m_err = (dec.m_state[lv] - full.m_state[lv]).abs().max().item()
+        assert m_err <= 1e-4 * max(full.m_state[lv].abs().max().item(), 1e-6), (lv, m_err)
