@@ -439,7 +439,8 @@ def setup_hebbian_c2(torch, D, lib):
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm",
         flop_fwd=FLOP_HEB_FWD, flop_bwd=FLOP_HEB_BWD, bytes_bwd=BYTES_HEB_BWD,
-        traffic_bwd=None, kernel=None,
+        traffic_bwd=int((2178.6 + 297.6 + 264.0 + 64.5) * 2**20),   # measured: sweep + sum of the row parts (read + written MiB)
+        kernel=None,
         kernel_names={"forward": "hebbian_forward", "backward": "hebbian_backward_segment"},
         config={"workload": "Hebbian rule at the shape of BASELINE configs[1]: 8 heads x 64 (d=512), batch 8, "
                             "seq 2048, fp32, full M trajectory, forward + whole-sequence segment backward",
