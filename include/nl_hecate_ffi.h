@@ -569,6 +569,23 @@ void memory_grads_fused_rocm(const float *d_k_heads, const float *d_v_heads, con
                              float *d_k_in, float *d_v, float *d_q_in, float *d_alpha, float *d_theta, float *d_eta,
                              int bs, int s, int nh, int hd, float eps);
 
+/* ── Titans rule with an MLP memory: packed state [W1 (dh x d) | b1 (dh) | W2 (d x dh) | b2 (d)] ── */
+/* core/src/cuda_ffi.rs:854.  input_stride = elements between the chains' token tensors (seq_len * d),
+ * m_stride = elements between the chains' trajectories ((seq_len + 1) * state_size); activation 0 GELU,
+ * 1 SiLU, 2 ReLU. */
+void titans_mlp_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                 const float *theta, const float *eta, const float *m_initial, const float *s_initial,
+                                 float *m_states, float *s_states, float *y, int seq_len, int d, int d_hidden,
+                                 int batch_size, int input_stride, int m_stride, int activation, float m_norm_max);
+/* core/src/cuda_ffi.rs:887 (d_m_initial, d_s_initial [state_size] are summed over the batch into the
+ * caller's zeroed buffers) */
+void titans_mlp_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                  const float *theta, const float *eta, const float *m_states, const float *s_states,
+                                  const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem, float *d_alpha,
+                                  float *d_theta, float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len,
+                                  int d, int d_hidden, int batch_size, int input_stride, int m_stride, int activation,
+                                  float m_norm_max);
+
 /* ── SwiGLU MLP, device-to-device (the GEMMs go to rocBLAS on the library's stream) ── */
 /* core/src/cuda_ffi.rs:925 */
 void swiglu_forward_f32_cuda_dd(const float *x, const float *gate_proj, const float *up_proj, const float *down_proj,

@@ -40,6 +40,7 @@
 #define SQRT sqrtf
 #define EXP expf
 #define LOG logf
+#define TANH tanhf
 #include "rules.inc"
 #include "selfref.inc"
 #undef REAL
@@ -47,12 +48,14 @@
 #undef SQRT
 #undef EXP
 #undef LOG
+#undef TANH
 
 #define REAL double
 #define SFX _f64
 #define SQRT sqrt
 #define EXP exp
 #define LOG log
+#define TANH tanh
 #include "rules.inc"
 #include "selfref.inc"
 #undef REAL
@@ -60,6 +63,7 @@
 #undef SQRT
 #undef EXP
 #undef LOG
+#undef TANH
 
 /* ── SimpleRng: xorshift64, core/src/tensor.rs:380-408 ──────────────────── */
 void orc_simple_rng_fill_uniform(uint64_t seed, float scale, float *buf, int64_t n) {

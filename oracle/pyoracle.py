@@ -166,6 +166,40 @@ def hebbian_backward(k, v, q, alpha, m_states, d_y, t_lo=0, t_hi=None, d_m_seed=
     return g
 
 
+def mlp_state_size(d, dh):
+    """packed [W1 (dh x d) | b1 (dh) | W2 (d x dh) | b2 (d)]"""
+    return 2 * dh * d + dh + d
+
+
+def titans_mlp_forward(k, v, q, alpha, theta, eta, m0, s0, dh, act=0, m_norm_max=F32_MAX, actp_fix=None):
+    """core/kernels/titans_mlp_forward.cu:115-330, one chain.  actp_fix [s, dh]: values used in place of
+    act'(pre) in the inner gradient (for tests that freeze them)."""
+    dt = k.dtype
+    sfx, real = _sfx(dt)
+    s, d = k.shape
+    n = mlp_state_size(d, dh)
+    m_states, s_states, y = np.zeros((s + 1, n), dt), np.zeros((s + 1, n), dt), np.zeros((s, d), dt)
+    _call("orc_titans_mlp_forward" + sfx, _c(k, dt), _c(v, dt), _c(q, dt), _c(alpha, dt), _c(theta, dt), _c(eta, dt),
+          _c(m0, dt), _c(s0, dt), m_states, s_states, y, s, d, int(dh), int(act), float(m_norm_max),
+          None if actp_fix is None else _c(actp_fix, dt), real=real)
+    return y, m_states, s_states
+
+
+def titans_mlp_backward(k, v, q, alpha, theta, eta, m_states, s_states, d_y, dh, act=0):
+    """core/kernels/titans_mlp_backward.cu:100-560, one chain; d_m / d_s: gradients of the initial state."""
+    dt = k.dtype
+    sfx, real = _sfx(dt)
+    s, d = k.shape
+    n = mlp_state_size(d, dh)
+    g = {nm: np.zeros((s, d), dt) for nm in ("d_k", "d_v", "d_q")}
+    g.update({nm: np.zeros(s, dt) for nm in ("d_alpha", "d_theta", "d_eta")})
+    g["d_m"], g["d_s"] = np.zeros(n, dt), np.zeros(n, dt)
+    _call("orc_titans_mlp_backward" + sfx, _c(k, dt), _c(v, dt), _c(q, dt), _c(alpha, dt), _c(theta, dt), _c(eta, dt),
+          _c(m_states, dt), _c(s_states, dt), _c(d_y, dt), g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"],
+          g["d_eta"], g["d_m"], g["d_s"], s, d, int(dh), int(act), real=real)
+    return g
+
+
 def chunkwise_forward(k, v, q, alpha, theta, eta, m0, s0, chunk_size, has_s=True,
                       error_clip=0.0, m_norm_max=F32_MAX):
     dt = k.dtype
