@@ -586,6 +586,32 @@ void titans_mlp_backward_f32_cuda(const float *k_mem, const float *v_mem, const 
                                   int d, int d_hidden, int batch_size, int input_stride, int m_stride, int activation,
                                   float m_norm_max);
 
+/* ── MIRAS MLP memories (one chain): MONETA (l_p error, L_q / L2 retention), YAAD (Huber, local + L2) ── */
+/* core/src/cuda_ffi.rs:785.  w*_states [(seq_len + 1), d_hidden * d]: the full trajectories. */
+void mlp_forward_lp_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                             const float *theta, const float *w1_initial, const float *w2_initial, float *w1_states,
+                             float *w2_states, float *y, int seq_len, int d, int d_hidden, float lp_p,
+                             float sign_sharpness, float lambda_2, float lq_q);
+/* core/src/cuda_ffi.rs:799 */
+void mlp_forward_huber_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                const float *theta, const float *w1_initial, const float *w2_initial,
+                                const float *w1_boundary, const float *w2_boundary, float *w1_states, float *w2_states,
+                                float *y, int seq_len, int d, int d_hidden, float huber_delta, float lambda_local,
+                                float lambda_2);
+/* core/src/cuda_ffi.rs:813 (q = 2 only; d_k_mem is added to and d_v_mem subtracted from: the caller zeroes them) */
+void mlp_backward_lp_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                              const float *theta, const float *w1_states, const float *w2_states, const float *d_y,
+                              float *d_k_mem, float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta,
+                              float *d_w1_initial, float *d_w2_initial, int seq_len, int d, int d_hidden, float lp_p,
+                              float sign_sharpness, float lambda_2, float lq_q);
+/* core/src/cuda_ffi.rs:829 */
+void mlp_backward_huber_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                 const float *theta, const float *w1_states, const float *w2_states,
+                                 const float *w1_boundary, const float *w2_boundary, const float *d_y, float *d_k_mem,
+                                 float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta, float *d_w1_initial,
+                                 float *d_w2_initial, int seq_len, int d, int d_hidden, float huber_delta,
+                                 float lambda_local, float lambda_2);
+
 /* ── SwiGLU MLP, device-to-device (the GEMMs go to rocBLAS on the library's stream) ── */
 /* core/src/cuda_ffi.rs:925 */
 void swiglu_forward_f32_cuda_dd(const float *x, const float *gate_proj, const float *up_proj, const float *down_proj,

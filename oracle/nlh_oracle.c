@@ -41,6 +41,8 @@
 #define EXP expf
 #define LOG logf
 #define TANH tanhf
+#define FABS fabsf
+#define POW powf
 #include "rules.inc"
 #include "selfref.inc"
 #undef REAL
@@ -49,6 +51,8 @@
 #undef EXP
 #undef LOG
 #undef TANH
+#undef FABS
+#undef POW
 
 #define REAL double
 #define SFX _f64
@@ -56,6 +60,8 @@
 #define EXP exp
 #define LOG log
 #define TANH tanh
+#define FABS fabs
+#define POW pow
 #include "rules.inc"
 #include "selfref.inc"
 #undef REAL
@@ -64,6 +70,8 @@
 #undef EXP
 #undef LOG
 #undef TANH
+#undef FABS
+#undef POW
 
 /* ── SimpleRng: xorshift64, core/src/tensor.rs:380-408 ──────────────────── */
 void orc_simple_rng_fill_uniform(uint64_t seed, float scale, float *buf, int64_t n) {

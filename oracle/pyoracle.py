@@ -200,6 +200,37 @@ def titans_mlp_backward(k, v, q, alpha, theta, eta, m_states, s_states, d_y, dh,
     return g
 
 
+def miras_mlp_forward(mode, k, v, q, alpha, theta, w1, w2, dh, p1, p2, lambda_2, lq_q=2.0, boundary=None,
+                      slope_fix=None):
+    """MONETA (mode 0: p1 = lp_p, p2 = sign_sharpness) / YAAD (mode 1: p1 = huber_delta, p2 = lambda_local,
+    boundary = (w1_boundary, w2_boundary)) forward, core/kernels/moneta_forward.cu:100-430, one chain."""
+    dt = k.dtype
+    sfx, real = _sfx(dt)
+    s, d = k.shape
+    w1s, w2s, y = np.zeros((s + 1, dh, d), dt), np.zeros((s + 1, d, dh), dt), np.zeros((s, d), dt)
+    b1, b2 = (None, None) if boundary is None else (_c(boundary[0], dt), _c(boundary[1], dt))
+    _call("orc_miras_mlp_forward" + sfx, int(mode), _c(k, dt), _c(v, dt), _c(q, dt), _c(alpha, dt), _c(theta, dt),
+          _c(w1, dt), _c(w2, dt), b1, b2, w1s, w2s, y, s, d, int(dh), float(p1), float(p2), float(lambda_2),
+          float(lq_q), None if slope_fix is None else _c(slope_fix, dt), real=real)
+    return y, w1s, w2s
+
+
+def miras_mlp_backward(mode, k, v, q, alpha, theta, w1s, w2s, d_y, dh, p1, p2, lambda_2, boundary=None,
+                       d_k0=None, d_v0=None):
+    """core/kernels/moneta_backward.cu:96-520 (q = 2); d_k / d_v start from d_k0 / d_v0 (accumulate contract)."""
+    dt = k.dtype
+    sfx, real = _sfx(dt)
+    s, d = k.shape
+    g = dict(d_k=np.zeros((s, d), dt) if d_k0 is None else _c(d_k0, dt).copy(),
+             d_v=np.zeros((s, d), dt) if d_v0 is None else _c(d_v0, dt).copy(), d_q=np.zeros((s, d), dt),
+             d_alpha=np.zeros(s, dt), d_theta=np.zeros(s, dt), d_w1=np.zeros((dh, d), dt), d_w2=np.zeros((d, dh), dt))
+    b1, b2 = (None, None) if boundary is None else (_c(boundary[0], dt), _c(boundary[1], dt))
+    _call("orc_miras_mlp_backward" + sfx, int(mode), _c(k, dt), _c(v, dt), _c(q, dt), _c(alpha, dt), _c(theta, dt),
+          _c(w1s, dt), _c(w2s, dt), b1, b2, _c(d_y, dt), g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"],
+          g["d_w1"], g["d_w2"], s, d, int(dh), float(p1), float(p2), float(lambda_2), real=real)
+    return g
+
+
 def chunkwise_forward(k, v, q, alpha, theta, eta, m0, s0, chunk_size, has_s=True,
                       error_clip=0.0, m_norm_max=F32_MAX):
     dt = k.dtype

@@ -58,3 +58,18 @@ def test_product_package_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"\boracle\b", text), f"{f} mentions the oracle"
+
+
+def test_every_function_of_the_reference_ffi_is_exported():
+    """tests/golden/cuda_ffi_symbols.txt lists the `pub(crate) fn` names of core/src/cuda_ffi.rs (names only:
+    data, made with grep).  Each must be declared in the header and exported by the library."""
+    import ctypes
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    names = open(os.path.join(here, "golden", "cuda_ffi_symbols.txt")).read().split()
+    assert len(names) == 87
+    from nl_hecate_amd.ffi import LIB_PATH, parse_header
+    protos = parse_header()
+    cdll = ctypes.CDLL(LIB_PATH)
+    missing = [n for n in names if n not in protos or not hasattr(cdll, n)]
+    assert not missing, missing
