@@ -52,6 +52,9 @@ CASES = [  # B, s, d, C
     (2, 96, 64, 32),
     (2, 50, 64, 64),    # single partial chunk
     (1, 70, 64, 24),
+    (2, 130, 64, 64),   # full chunks plus a two-token chunk
+    (1, 100, 64, 80),   # chunks above 64 tokens take the trajectory path
+    (2, 150, 16, 70),
 ]
 
 
