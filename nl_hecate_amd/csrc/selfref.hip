@@ -457,6 +457,7 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
     __shared__ __align__(16) float sp[2][NW][2];
     __shared__ __align__(16) float sc[4][kTB];
     __shared__ __align__(16) float av[2][D];
+    __shared__ float dEA[2][kTB];  // de_t, da_t of the tile
     constexpr int RS = (LR && !SG) ? 6 : 4;  // vectors per token kept between the two passes of a chunk
 #define T_(a, tt, i) raw[((a) * kTB + (tt)) * TL + (i)]
 
@@ -470,12 +471,16 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
     float sig_base = 0.f, pend = 0.f;
     const int stt = tid / V4, sj = (tid % V4) * 4;  // staging slot: token, column
 
-    float dF[4][CP], accE[CP], accA[CP], dG[CP], dH[CP];
+    // dF_k, dF_v, dF_q, dF_mem live in the accumulator layout of the matrix cores (wave w owns rows
+    // 16 w .., lane (ml, kg) rows 4 kg + v of column 16 jt + ml); the equal rows of dF_eta, dF_alpha are
+    // rows 0 and 1 of accEA, wave w holding columns 16 w .. (lanes kg = 0).
+    const int ml = lane & 15, kg = lane >> 4, wr = 16 * wave;
+    f32x4 dFm[4][JT], accEA = f32x4{0.f, 0.f, 0.f, 0.f};
+    float dG[CP], dH[CP];
 #pragma unroll
-    for (int i = 0; i < CP; i++) {
-        dF[0][i] = dF[1][i] = dF[2][i] = dF[3][i] = 0.f;
-        accE[i] = accA[i] = dG[i] = dH[i] = 0.f;
-    }
+    for (int jt = 0; jt < JT; jt++) dFm[0][jt] = dFm[1][jt] = dFm[2][jt] = dFm[3][jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < CP; i++) dG[i] = dH[i] = 0.f;
 
     // Inputs of the next tile of the reverse sweep, requested one tile ahead (low-rank path).
     float4 pf_k, pf_v, pf_q, pf_x, pf_dy, pf_g, pf_p, pf_dq, pf_dp, pf_hx, pf_hq, pf_s;
@@ -640,21 +645,25 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
         if (LR) SWEEP_REQUEST(ntile - 1)
         if (ci < nc - 1) {
             float *Fs = raw, *Bm = raw + D * LD, *GLT = raw + 2 * D * LD;
-            const int ml = lane & 15, kg = lane >> 4, wr = 16 * wave;
 #pragma unroll
             for (int i = 0; i < CP; i++) GLT[(c0 + i) * LD + r] = G[i];
-            if (r == 0) { vec_store<CP>(&av[0][c0], accE); vec_store<CP>(&av[1][c0], accA); }
-            // rows of dF_eta, dF_alpha are all equal (accE, accA): rank-1 terms
+            if (kg == 0) { av[0][wr + ml] = accEA[0]; av[1][wr + ml] = accEA[1]; }
+            __syncthreads();
+            {   // rows of dF_eta, dF_alpha are all equal: rank-1 terms
+                float eE[CP], eA[CP];
+                lds_read<CP>(eE, &av[0][c0]);
+                lds_read<CP>(eA, &av[1][c0]);
 #pragma unroll
-            for (int i = 0; i < CP; i++) {
-                dG[i] = csE * accE[i] + csA * accA[i];
-                dH[i] = accE[i] + accA[i];
+                for (int i = 0; i < CP; i++) {
+                    dG[i] = csE * eE[i] + csA * eA[i];
+                    dH[i] = eE[i] + eA[i];
+                }
             }
             // The eight D x D products run on the matrix cores in fp32 (v_mfma_f32_16x16x4_f32: lane
             // (ml, kg) = (lane % 16, lane / 16) feeds A[ml][kg], B[kg][ml] and receives rows 4 kg + v of
             // column ml); wave w owns rows 16 w .. 16 w + 15 of both results, which are also the rows its
-            // lanes keep in registers, so the accumulators return to the row-quad layout through the
-            // wave's own rows of Bm without a workgroup barrier.
+            // lanes keep in the row-quad layout, so values change layout through the wave's own rows of Bm
+            // without a workgroup barrier.
             f32x4 accG[JT];
 #pragma unroll
             for (int jt = 0; jt < JT; jt++) accG[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -666,10 +675,16 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                     const int m = e / V4, j = (e % V4) * 4;
                     *reinterpret_cast<float4 *>(Fs + m * LD + j) = *reinterpret_cast<const float4 *>(fz + (size_t)c * DD + m * D + j);
                 }
-                vec_store<CP>(Bm + r * LD + c0, dF[comp]);
-                if (!SG) {
 #pragma unroll
-                    for (int i = 0; i < CP; i++) dH[i] += dF[comp][i];
+                for (int jt = 0; jt < JT; jt++) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) Bm[(wr + 4 * kg + v) * LD + 16 * jt + ml] = dFm[comp][jt][v];
+                }
+                if (!SG) {  // the wave's own rows, back in the row-quad layout
+                    float t[CP];
+                    lds_read<CP>(t, Bm + r * LD + c0);
+#pragma unroll
+                    for (int i = 0; i < CP; i++) dH[i] += t[i];
                 }
                 __syncthreads();
                 f32x4 accN[JT];
@@ -687,15 +702,11 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                         accN[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a2, b2, accN[jt], 0, 0, 0);
                     }
                 }
-                __syncthreads();  // every wave has read Bm
 #pragma unroll
-                for (int jt = 0; jt < JT; jt++) {
-#pragma unroll
-                    for (int v = 0; v < 4; v++) Bm[(wr + 4 * kg + v) * LD + 16 * jt + ml] = accN[jt][v];
-                }
-                lds_read<CP>(dF[comp], Bm + r * LD + c0);  // dF_c = dF'_c G_L^T
+                for (int jt = 0; jt < JT; jt++) dFm[comp][jt] = accN[jt];  // dF_c = dF'_c G_L^T
             }
-            {   // dG_L += sum_c F_c^T dF'_c, through the wave's rows of Bm again
+            __syncthreads();  // every wave has read Bm
+            {   // dG_L += sum_c F_c^T dF'_c, into the row-quad layout through the wave's own rows of Bm
 #pragma unroll
                 for (int jt = 0; jt < JT; jt++) {
 #pragma unroll
@@ -714,11 +725,7 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                     const float a = ml < 2 ? av[ml][k0 + kg] : 0.f;
                     accV = __builtin_amdgcn_mfma_f32_16x16x4f32(a, GLT[(k0 + kg) * LD + wr + ml], accV, 0, 0, 0);
                 }
-                __syncthreads();  // av has been read
-                if (kg == 0) { av[0][wr + ml] = accV[0]; av[1][wr + ml] = accV[1]; }
-                __syncthreads();
-                lds_read<CP>(accE, &av[0][c0]);
-                lds_read<CP>(accA, &av[1][c0]);
+                accEA = accV;
             }
             __syncthreads();
         }
@@ -900,23 +907,19 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                     if (!SG) pend += dh * T_(A_HX, tt, r) + dy_r * T_(A_HQ, tt, r);
                     pend *= 0.25f;  // the four lanes of a row hold the same values
                 }
-                float xc[CP], qc[CP], gc[CP], pc[CP];
+                float xc[CP], qc[CP];
                 lds_read<CP>(xc, &T_(A_X, tt, c0));
                 lds_read<CP>(qc, &T_(A_Q, tt, c0));
-                lds_read<CP>(gc, &T_(A_G, tt, c0));
-                lds_read<CP>(pc, &T_(A_P, tt, c0));
                 const float keep = 1.f - al;
 #pragma unroll
                 for (int i = 0; i < CP; i++) {
                     dG[i] = fmaf(dg, xc[i], fmaf(dp_r, qc[i], keep * dG[i]));
                     if (!SG) dH[i] = fmaf(dh, xc[i], fmaf(dy_r, qc[i], keep * dH[i]));
-                    dF[0][i] = fmaf(dk_r, gc[i], dF[0][i]);
-                    dF[1][i] = fmaf(dv_r, gc[i], dF[1][i]);
-                    dF[2][i] = fmaf(dq_r, gc[i], dF[2][i]);
-                    dF[3][i] = fmaf(dy_r, pc[i], dF[3][i]);
-                    accE[i] = fmaf(de, gc[i], accE[i]);
-                    accA[i] = fmaf(da, gc[i], accA[i]);
                 }
+                // dk_t, dv_t take the place of k_t, v_t (read by every wave before this token's barrier);
+                // the outer products with g_t, p_t follow for the whole tile after the loop
+                if (cq == 0) { T_(A_K, tt, r) = dk_r; T_(A_V, tt, r) = dv_r; }
+                if (tid == 0) { dEA[0][tt] = de; dEA[1][tt] = da; }
                 if (cq == 0) T_(A_DG, tt, r) = dg;
                 if (!SG && cq == 1) T_(A_DH, tt, r) = dh;
                 if (!LR && tt > 0) {
@@ -925,6 +928,25 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                 }
             }
             __syncthreads();
+            // the tile's outer products: dF_k += dk g^T, dF_v += dv g^T, dF_q += dq g^T, dF_mem += dy p^T,
+            // accE += sum_t de_t g_t, accA += sum_t da_t g_t (tokens are the contraction index)
+#pragma unroll
+            for (int k0 = 0; k0 < kTB; k0 += 4) {
+                const int tk = k0 + kg;
+                const bool ok = tk < nt;
+                const float a_k = ok ? T_(A_K, tk, wr + ml) : 0.f, a_v = ok ? T_(A_V, tk, wr + ml) : 0.f;
+                const float a_q = ok ? T_(A_DQ, tk, wr + ml) : 0.f, a_y = ok ? T_(A_DY, tk, wr + ml) : 0.f;
+                const float a_e = (ok && ml < 2) ? dEA[ml][tk] : 0.f;
+#pragma unroll
+                for (int jt = 0; jt < JT; jt++) {
+                    const float b_g = ok ? T_(A_G, tk, 16 * jt + ml) : 0.f, b_p = ok ? T_(A_P, tk, 16 * jt + ml) : 0.f;
+                    dFm[0][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_k, b_g, dFm[0][jt], 0, 0, 0);
+                    dFm[1][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_v, b_g, dFm[1][jt], 0, 0, 0);
+                    dFm[2][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_q, b_g, dFm[2][jt], 0, 0, 0);
+                    dFm[3][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_y, b_p, dFm[3][jt], 0, 0, 0);
+                }
+                accEA = __builtin_amdgcn_mfma_f32_16x16x4f32(a_e, ok ? T_(A_G, tk, wr + ml) : 0.f, accEA, 0, 0, 0);
+            }
             // d_x_t = G_t^T dg_t + H_t^T dh_t
             if (LR) {
                 if (stt < nt) {
@@ -956,13 +978,26 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
         }
     }
     // gradients of the initial memories; rows of d_M_eta / d_M_alpha are all equal
-    float *dmb = d_mems + b * 6 * DD + r * D + c0;
-    vec_store<CP>(dmb + 0 * DD, dF[0]);
-    vec_store<CP>(dmb + 1 * DD, dF[1]);
-    vec_store<CP>(dmb + 2 * DD, dF[2]);
-    vec_store<CP>(dmb + 3 * DD, accE);
-    vec_store<CP>(dmb + 4 * DD, accA);
-    vec_store<CP>(dmb + 5 * DD, dF[3]);
+    float *dmb = d_mems + b * 6 * DD;
+#pragma unroll
+    for (int comp = 0; comp < 4; comp++) {
+        float *dst = dmb + (comp < 3 ? comp : 5) * DD;
+#pragma unroll
+        for (int jt = 0; jt < JT; jt++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) dst[(wr + 4 * kg + v) * D + 16 * jt + ml] = dFm[comp][jt][v];
+        }
+    }
+    __syncthreads();
+    if (kg == 0) { av[0][wr + ml] = accEA[0]; av[1][wr + ml] = accEA[1]; }
+    __syncthreads();
+    {
+        float eE[CP], eA[CP];
+        lds_read<CP>(eE, &av[0][c0]);
+        lds_read<CP>(eA, &av[1][c0]);
+        vec_store<CP>(dmb + 3 * DD + r * D + c0, eE);
+        vec_store<CP>(dmb + 4 * DD + r * D + c0, eA);
+    }
 #undef T_
 }
 
