@@ -385,8 +385,8 @@ def setup_hope_selfref_c4(torch, D, lib):
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s,
         flop_fwd=FLOP_HOPE_FWD, flop_bwd=FLOP_HOPE_BWD, bytes_bwd=BYTES_HOPE_BWD,
-        traffic_bwd=int((4041.7 + 2214.0) * 2**20),  # measured: per-token G trajectory through HBM
-        kernel="selfref_bwd_kernel<64,true> (one launch of the backward entry point)",
+        traffic_bwd=int((542.2 + 38.0) * 2**20),  # measured, the sweep kernel alone
+        kernel="selfref_bwd_kernel<64,true,true> (the chain-sequential sweep of the backward entry point)",
         kernel_names={"forward": "selfref_forward", "backward": "selfref_backward"},
         config={"workload": "BASELINE configs[3]: HOPE self-referential memory, 8 heads x 64 (d=512), "
                             "batch 8, seq 2048, fp32, self-generated values, frozen snapshots per 64 tokens, fwd+bwd",

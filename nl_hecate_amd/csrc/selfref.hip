@@ -16,7 +16,11 @@
 //     G_0 = I, G_{t+1} = (1-a_t) G_t - th_t u_t k_t^T      u = k - v (self-generated
 //     H_0 = 0, H_{t+1} = (1-a_t) H_t + th_t v_t k_t^T       values: H == 0) or u = k
 // so the reverse sweep carries dG, dH (and the six dF) instead of six dM and six
-// dF, and only G_t, H_t have to be replayed per token.
+// dF.  Chunks of up to 64 tokens use the explicit (low-rank) form of G_t, H_t:
+// a chunk-parallel kernel prepares every product that does not depend on the
+// sweep, the sweep kernel keeps only the per-token recurrence, and a second
+// chunk-parallel kernel turns dg, dh into d_x.  Longer chunks replay G_t, H_t
+// into a per-chunk trajectory in scratch memory.
 #include <hip/hip_runtime.h>
 #include <math.h>
 
