@@ -51,6 +51,14 @@ __device__ __forceinline__ float sr_softplus(float x) {
 // core/src/chunkwise_self_ref.rs:95-218.  mems [B,6,D*D] is updated in place;
 // frozen [B,nc,6,D*D] receives the chunk-start snapshots; the per-token caches
 // are what the backward consumes.
+//
+// Inside a chunk the six memories are M_c,t = F_c G_t + H_t (F_c the chunk-start
+// snapshot, G and H as in the header), so a token costs two products with G
+// (g = G x, p = G q), six with the frozen F_c (k, v, q, the two gates = F_c g,
+// y = F_mem p) and one rank-1 update of G (and H) instead of eleven products
+// and six updates with the M_c themselves; M_c = F_c G_L + H_L is formed once
+// per chunk on the fp32 matrix cores.  Two LDS exchanges per token: (g_t, p_{t-1})
+// and (k_t, v_t, q_t, gate sums); y is written one token late.
 template <int D, bool SG>
 __global__ __launch_bounds__(4 * D) void selfref_fwd_kernel(
     float *__restrict__ mems, const float *__restrict__ emb, float *__restrict__ y,
@@ -58,24 +66,83 @@ __global__ __launch_bounds__(4 * D) void selfref_fwd_kernel(
     float *__restrict__ alpha_cache, float *__restrict__ theta_cache,
     float *__restrict__ amean_cache, float *__restrict__ emean_cache, float *__restrict__ frozen,
     int s, int C, int nc) {
-    constexpr int CP = D / 4, NT = 4 * D, NW = (NT + 63) / 64, DD = D * D;
+    constexpr int CP = D / 4, NT = 4 * D, NW = (NT + 63) / 64, DD = D * D, LD = D + 4, JT = D / 16;
     __shared__ __align__(16) float xt[2][kTB][D];
-    __shared__ __align__(16) float vec[2][3][D];
-    __shared__ __align__(16) float gpart[2][8];
+    __shared__ __align__(16) float vec[5][D];   // g, p | k, v, q in row order
+    __shared__ __align__(16) float gpart[4];      // per-wave sums of H x
+    __shared__ __align__(16) float csum[2][NW][D];  // per-wave column sums of F_eta, F_alpha
+    __shared__ __align__(16) float Gs[D * LD];  // G_L, then H-free staging of the chunk-end products
+    __shared__ __align__(16) float Fs[D * LD];  // a wave touches its own 16 rows only
 
     const int tid = threadIdx.x, r = tid >> 2, cq = tid & 3, wave = tid >> 6, lane = tid & 63;
+    const int c0 = cq * CP, ml = lane & 15, kg = lane >> 4, wr = 16 * wave;
     const size_t b = blockIdx.x;
-    float *mb = mems + b * 6 * DD + r * D + cq * CP;
+    float *mb = mems + b * 6 * DD + r * D + c0;
     const float *xb = emb + b * (size_t)s * D;
-    float *fb = frozen + b * (size_t)nc * 6 * DD + r * D + cq * CP;
+    float *fb = frozen + b * (size_t)nc * 6 * DD + r * D + c0;
 
-    float M[6][CP], F[6][CP];
+    float F[6][CP], G[CP], H[CP];
 #pragma unroll
-    for (int c = 0; c < 6; c++) {
-        lds_read<CP>(M[c], mb + c * DD);
+    for (int c = 0; c < 6; c++) lds_read<CP>(F[c], mb + c * DD);
 #pragma unroll
-        for (int i = 0; i < CP; i++) F[c][i] = 0.f;
-    }
+    for (int i = 0; i < CP; i++) { G[i] = (c0 + i == r) ? 1.f : 0.f; H[i] = 0.f; }
+
+    // F_c <- F_c G + H for the six memories; ends with every wave's F in registers.
+    auto fold = [&]() {
+        __syncthreads();
+        vec_store<CP>(Gs + r * LD + c0, G);
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 6; c++) {
+            vec_store<CP>(Fs + r * LD + c0, F[c]);
+            f32x4 acc[JT];
+#pragma unroll
+            for (int jt = 0; jt < JT; jt++) acc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int k0 = 0; k0 < D; k0 += 4) {
+                const float a = Fs[(wr + ml) * LD + k0 + kg];
+#pragma unroll
+                for (int jt = 0; jt < JT; jt++)
+                    acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Gs[(k0 + kg) * LD + 16 * jt + ml], acc[jt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int jt = 0; jt < JT; jt++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) Fs[(wr + 4 * kg + v) * LD + 16 * jt + ml] = acc[jt][v];
+            }
+            lds_read<CP>(F[c], Fs + r * LD + c0);
+#pragma unroll
+            for (int i = 0; i < CP; i++) F[c][i] += H[i];
+        }
+    };
+
+    // The gates are means over the rows of F_eta g + H x and F_alpha g + H x: the frozen parts are
+    // dots of g with the column means of F_eta, F_alpha, refreshed with each snapshot.
+    float cse[CP], csa[CP];
+    auto column_means = [&]() {
+        float eo[CP / 4], ao[CP / 4];
+        rows_reduce_scatter<CP>(F[3], eo);
+        rows_reduce_scatter<CP>(F[4], ao);
+        const int rho = lane >> 4, zoff = c0 + (CP / 2) * (rho >> 1) + (CP / 4) * (rho & 1);
+        __syncthreads();
+        if (((lane & 15) >> 2) == 0) {
+#pragma unroll
+            for (int i = 0; i < CP / 4; i++) { csum[0][wave][zoff + i] = eo[i]; csum[1][wave][zoff + i] = ao[i]; }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < CP; i++) cse[i] = csa[i] = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            float te[CP], ta[CP];
+            lds_read<CP>(te, &csum[0][w][c0]);
+            lds_read<CP>(ta, &csum[1][w][c0]);
+#pragma unroll
+            for (int i = 0; i < CP; i++) { cse[i] += te[i]; csa[i] += ta[i]; }
+        }
+#pragma unroll
+        for (int i = 0; i < CP; i++) { cse[i] *= 1.f / D; csa[i] *= 1.f / D; }
+    };
 
     // x tiles: one float4 per thread per tile of kTB tokens
     const int xtt = tid / (D / 4), xj = (tid % (D / 4)) * 4;
@@ -87,75 +154,104 @@ __global__ __launch_bounds__(4 * D) void selfref_fwd_kernel(
     *reinterpret_cast<float4 *>(&xt[0][xtt][xj]) = load_x(0);
     __syncthreads();
 
+    bool have_p = false;
+    float p_r = 0.f, hq_r = 0.f;
+    int chunk_t = 0, ci = 0;  // first token and index of the next chunk
+    // y_{t-1} = F_mem p_{t-1} + H_{t-1} q_{t-1} from the column form of p
+    auto emit_y = [&](int t_prev, bool valid) {
+        float pc[CP];
+        lds_read<CP>(pc, &vec[1][c0]);
+        const float y_r = quad_allreduce(dotn<CP>(F[5], pc)) + hq_r;
+        if (valid && cq == 3) y[(b * s + t_prev) * D + r] = y_r;
+    };
+
     for (int tile = 0; tile < ntiles; tile++) {
         const int xb_cur = tile & 1;
         float4 xnext = make_float4(0, 0, 0, 0);
         if (tile + 1 < ntiles) xnext = load_x(tile + 1);
         const int nt = min(kTB, s - tile * kTB);
         for (int tt = 0; tt < nt; tt++) {
-            const int t = tile * kTB + tt, pb = tt & 1;
-            if (t % C == 0) {
-                const int ci = t / C;
+            const int t = tile * kTB + tt;
+            if (t == chunk_t) {
+                if (t > 0) {
+                    if (cq == 1) vec[1][r] = p_r;
+                    lds_barrier();
+                    emit_y(t - 1, true);
+                    have_p = false;
+                    fold();
 #pragma unroll
-                for (int c = 0; c < 6; c++) {
-#pragma unroll
-                    for (int i = 0; i < CP; i++) F[c][i] = M[c][i];
-                    vec_store<CP>(fb + ((size_t)ci * 6 + c) * DD, F[c]);
+                    for (int i = 0; i < CP; i++) { G[i] = (c0 + i == r) ? 1.f : 0.f; H[i] = 0.f; }
                 }
+#pragma unroll
+                for (int c = 0; c < 6; c++) vec_store<CP>(fb + ((size_t)ci * 6 + c) * DD, F[c]);
+                column_means();
+                ci++;
+                chunk_t += C;
             }
             float xc[CP];
-            lds_read<CP>(xc, &xt[xb_cur][tt][cq * CP]);
-            float pr[5];
-#pragma unroll
-            for (int c = 0; c < 5; c++) pr[c] = quad_allreduce(dotn<CP>(M[c], xc));
-            const float k_r = pr[0], v_r = pr[1], q_r = pr[2];
-            // eta_raw in even-cq lanes, alpha_raw in odd-cq lanes: one reduction for both sums
-            const float gsum = rows_allreduce((cq & 1) ? pr[4] : pr[3]);
-            if (lane < 2) gpart[pb][wave * 2 + lane] = gsum;
-            if (cq < 3) {
-                const float val = cq == 0 ? k_r : cq == 1 ? v_r : q_r;
-                vec[pb][cq][r] = val;
-                float *dst = cq == 0 ? k_cache : cq == 1 ? v_cache : q_cache;
-                dst[(b * s + t) * D + r] = val;
+            lds_read<CP>(xc, &xt[xb_cur][tt][c0]);
+            const float g_r = quad_allreduce(dotn<CP>(G, xc));
+            const float hx_r = SG ? 0.f : quad_allreduce(dotn<CP>(H, xc));
+            if (!SG) {  // sum of H x over the rows, for both gate means
+                const float hs = rows_allreduce(hx_r);
+                if (lane == 0) gpart[wave] = hs;
             }
+            if (cq == 0) vec[0][r] = g_r;
+            if (cq == 1) vec[1][r] = p_r;
             lds_barrier();
-            float em = 0.f, am = 0.f;
+            emit_y(t - 1, have_p);  // no branch around it: its product overlaps the five below
+            float gc[CP];
+            lds_read<CP>(gc, &vec[0][c0]);
+            float pr[3];
 #pragma unroll
-            for (int w = 0; w < NW; w++) { em += gpart[pb][2 * w]; am += gpart[pb][2 * w + 1]; }
-            em *= 1.f / D; am *= 1.f / D;
+            for (int c = 0; c < 3; c++) pr[c] = quad_allreduce(dotn<CP>(F[c], gc)) + hx_r;
+            const float k_r = pr[0], v_r = pr[1], q_r = pr[2];
+            float em = quad_allreduce(dotn<CP>(cse, gc)), am = quad_allreduce(dotn<CP>(csa, gc));
+            if (!SG) {
+                float hm = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; w++) hm += gpart[w];
+                em = fmaf(hm, 1.f / D, em); am = fmaf(hm, 1.f / D, am);
+            }
             const float alpha = sr_sigmoid(am), theta = sr_softplus(em);
             if (tid == 0) {
                 alpha_cache[b * s + t] = alpha; theta_cache[b * s + t] = theta;
                 amean_cache[b * s + t] = am; emean_cache[b * s + t] = em;
             }
-            float kc[CP], uc[CP], qc[CP];
-            lds_read<CP>(kc, &vec[pb][0][cq * CP]);
-            lds_read<CP>(qc, &vec[pb][2][cq * CP]);
-            if (SG) {
-                lds_read<CP>(uc, &vec[pb][1][cq * CP]);
-#pragma unroll
-                for (int i = 0; i < CP; i++) uc[i] = kc[i] - uc[i];
+            if (cq < 3) {
+                const float val = cq == 0 ? k_r : cq == 1 ? v_r : q_r;
+                vec[2 + cq][r] = val;
+                float *dst = cq == 0 ? k_cache : cq == 1 ? v_cache : q_cache;
+                dst[(b * s + t) * D + r] = val;
             }
-            const float y_r = quad_allreduce(dotn<CP>(M[5], qc));  // read before the update (:138)
-            if (cq == 3) y[(b * s + t) * D + r] = y_r;
+            lds_barrier();
+            float kc[CP], qc[CP];
+            lds_read<CP>(kc, &vec[2][c0]);
+            lds_read<CP>(qc, &vec[4][c0]);
+            // the read uses the memory before this token's update (:138)
+            p_r = quad_allreduce(dotn<CP>(G, qc));
+            hq_r = SG ? 0.f : quad_allreduce(dotn<CP>(H, qc));
+            have_p = true;
             const float keep = 1.f - alpha;
+            // self-generated target F_c v: the error is F_c (k - v)  (:155-166, :200)
+            const float su = theta * (SG ? k_r - v_r : k_r), sv = theta * v_r;
 #pragma unroll
-            for (int c = 0; c < 6; c++) {
-                // self-generated target F_c v: the error is F_c (k - v)  (:155-166, :200)
-                float e = quad_allreduce(SG ? dotn<CP>(F[c], uc) : dotn<CP>(F[c], kc));
-                if (!SG) e -= v_r;
-                const float se = theta * e;
-#pragma unroll
-                for (int i = 0; i < CP; i++) M[c][i] = fmaf(-se, kc[i], keep * M[c][i]);
+            for (int i = 0; i < CP; i++) {
+                G[i] = fmaf(-su, kc[i], keep * G[i]);
+                if (!SG) H[i] = fmaf(sv, kc[i], keep * H[i]);
             }
         }
         if (tile + 1 < ntiles) {
             *reinterpret_cast<float4 *>(&xt[xb_cur ^ 1][xtt][xj]) = xnext;
-            __syncthreads();
+            lds_barrier();
         }
     }
+    if (cq == 1) vec[1][r] = p_r;
+    lds_barrier();
+    emit_y(s - 1, true);
+    fold();
 #pragma unroll
-    for (int c = 0; c < 6; c++) vec_store<CP>(mb + c * DD, M[c]);
+    for (int c = 0; c < 6; c++) vec_store<CP>(mb + c * DD, F[c]);
 }
 
 // ── backward ───────────────────────────────────────────────────────────────
