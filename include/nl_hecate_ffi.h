@@ -671,6 +671,59 @@ unsigned frob_norm_sq_cuda(const float *x, float *partial_sums, int n, int *out_
 unsigned scale_buf_cuda(float *x, float scale, int n);
 unsigned m3_ns_poly_cuda(float *x, const float *y, const float *z, int n, float a, float b, float c);
 
+/* ── host-slice dispatch: every pointer below is HOST memory ───────────────────────────────────
+ * The bodies of the reference's `*_dispatch` functions for a device feature: one chain is staged on
+ * the device (allocate, copy in, zero the outputs, launch with batch_size = 1, synchronise, copy out),
+ * as core/src/dispatch.rs:1665-2085 does with its own DevBuf.  Argument order = the Rust function's.
+ * These are what the rule structs and the opaque VJP blocks of the Wengert tape call on a CPU tape
+ * (core/src/opaque_adapters.rs:306-400 Delta, 402-590 Titans, 593-629 Hebbian, 966-1010 SWA,
+ * 1686-1725 DGD). */
+/* core/src/dispatch.rs:746 */
+void nlh_delta_forward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                const float *theta, const float *m_initial, float *m_states, float *y,
+                                int seq_len, int d, float error_clip, float m_norm_max);
+/* core/src/dispatch.rs:775 (gradients are overwritten) */
+void nlh_delta_backward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                 const float *theta, const float *m_states, const float *d_y, float *d_k_mem,
+                                 float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta,
+                                 float *d_m_initial, int seq_len, int d, float error_clip);
+/* core/src/dispatch.rs:810 */
+void nlh_titans_forward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                 const float *theta, const float *eta, const float *m_initial,
+                                 const float *s_initial, float *m_states, float *s_states, float *y,
+                                 int seq_len, int d, float error_clip, float m_norm_max);
+/* core/src/dispatch.rs:842 */
+void nlh_titans_backward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                  const float *theta, const float *eta, const float *m_states,
+                                  const float *s_states, const float *d_y, float *d_k_mem, float *d_v_mem,
+                                  float *d_q_mem, float *d_alpha, float *d_theta, float *d_eta,
+                                  float *d_m_initial, float *d_s_initial, int seq_len, int d, float error_clip);
+/* core/src/dispatch.rs:1083 (a finite positive m_norm_max is refused: the reference runs that case on the CPU) */
+void nlh_hebbian_forward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                  const float *m_initial, float *m_states, float *y, int seq_len, int d,
+                                  float m_norm_max);
+/* core/src/dispatch.rs:1110 */
+void nlh_hebbian_backward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                                   const float *m_states, const float *d_y, float *d_k_mem, float *d_v_mem,
+                                   float *d_q_mem, float *d_alpha, float *d_m_initial, int seq_len, int d);
+/* core/src/dispatch.rs:1153 */
+void nlh_dgd_forward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                              const float *theta, const float *m_initial, float *m_states, float *y, int seq_len,
+                              int d, float error_clip);
+/* core/src/dispatch.rs:1182 */
+void nlh_dgd_backward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
+                               const float *theta, const float *m_states, const float *d_y, float *d_k_mem,
+                               float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta, float *d_m_initial,
+                               int seq_len, int d, float error_clip);
+/* core/src/dispatch.rs:378 (float on the host, bf16 on the device; one sequence, no persistent tokens) */
+void nlh_swa_forward_dispatch(const float *q, const float *k, const float *v, float *out, float *attn_weights,
+                              int seq_len, int num_heads, int head_dim, int window_size);
+/* core/src/dispatch.rs:408 (the caller zeroes d_q, d_k, d_v as the reference asks: d_k, d_v are accumulated
+ * into, d_q is overwritten) */
+void nlh_swa_backward_dispatch(const float *q, const float *k, const float *v, const float *attn_weights,
+                               const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len,
+                               int num_heads, int head_dim, int window_size);
+
 #ifdef __cplusplus
 }
 #endif
