@@ -767,13 +767,29 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
             f32x4 accG[JT];
 #pragma unroll
             for (int jt = 0; jt < JT; jt++) accG[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            // F_c travels global -> registers -> Fs; the next one is requested before the products of the
+            // current one, so only the first request's latency is exposed.
+            f32x4 fnext[JT];  // D*D/4 vectors of four over 4*D threads
+#pragma unroll
+            for (int i = 0; i < JT; i++) {
+                const int e = tid + i * NT;
+                fnext[i] = *reinterpret_cast<const f32x4 *>(fz + (e / V4) * D + (e % V4) * 4);
+            }
 #pragma unroll
             for (int comp = 0; comp < 4; comp++) {
-                const int c = comp < 3 ? comp : 5;
                 __syncthreads();
-                for (int e = tid; e < DD / 4; e += NT) {
-                    const int m = e / V4, j = (e % V4) * 4;
-                    *reinterpret_cast<float4 *>(Fs + m * LD + j) = *reinterpret_cast<const float4 *>(fz + (size_t)c * DD + m * D + j);
+#pragma unroll
+                for (int i = 0; i < JT; i++) {
+                    const int e = tid + i * NT;
+                    *reinterpret_cast<f32x4 *>(Fs + (e / V4) * LD + (e % V4) * 4) = fnext[i];
+                }
+                if (comp < 3) {
+                    const float *nf = fz + (size_t)(comp < 2 ? comp + 1 : 5) * DD;
+#pragma unroll
+                    for (int i = 0; i < JT; i++) {
+                        const int e = tid + i * NT;
+                        fnext[i] = *reinterpret_cast<const f32x4 *>(nf + (e / V4) * D + (e % V4) * 4);
+                    }
                 }
 #pragma unroll
                 for (int jt = 0; jt < JT; jt++) {
@@ -862,8 +878,10 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                 }
                 if (tid < nt) {
                     sc[0][tid] = pf_s.x; sc[1][tid] = pf_s.y;
-                    const float sa = sr_sigmoid(pf_s.z);
-                    sc[2][tid] = sa * (1.f - sa) * (1.f / D);
+                    const float sa = sr_sigmoid(pf_s.z), keep_t = 1.f - pf_s.x;
+                    // sigmoid'(mean) / d, here already over (1 - a_t): the sweep forms (1 - a_t) <G_t, dG_{t+1}>;
+                    // a saturated gate (keep = 0) has no gradient
+                    sc[2][tid] = keep_t > 0.f ? sa * (1.f - sa) * (1.f / D) / keep_t : 0.f;
                     sc[3][tid] = sr_sigmoid(pf_s.w) * (1.f / D);
                 }
                 __syncthreads();
@@ -950,8 +968,7 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
                 for (int x = 0; x < NW; x++) { dal -= sp[pb][x][0]; dth -= sp[pb][x][1]; }
                 if (LR) {
                     const float keepalp = fmaf(-th, dth, sig_base - dal);  // sigma_{t+1} + th (u.w - v.wh)
-                    const float keep_t = 1.f - al;
-                    dal = keep_t > 0.f ? -keepalp / keep_t : 0.f;
+                    dal = -keepalp;  // times 1 / (1 - a_t), folded into sc[2]
                     sig_base = keepalp;
                 }
                 const float da = dal * sc[2][tt], de = dth * sc[3][tt];
