@@ -396,8 +396,9 @@ def setup_hope_selfref_c4(torch, D, lib):
 
 # Hebbian rule, per head-token at d=64 with the full trajectory the contract asks for: forward
 # k,v,q 768 + alpha 4 + y 256 + M_{t+1} 16 384 = 17 412 B, 6 d^2 flop; backward k,v,q,dY 1024 + alpha 4 +
-# M_t 16 384 + grads 772 = 18 184 B, 12 d^2 flop.
-BYTES_HEB_FWD, BYTES_HEB_BWD = 17412, 18184
+# grads 772 + the states the chunk-parallel form needs (one per 64 tokens: 16 384 / 64 = 256) = 2 056 B
+# (the reference's sequential backward reads M_t per token: 18 184 B), 12 d^2 flop.
+BYTES_HEB_FWD, BYTES_HEB_BWD = 17412, 2056
 FLOP_HEB_FWD, FLOP_HEB_BWD = 6 * 64 * 64, 12 * 64 * 64
 
 
@@ -439,7 +440,7 @@ def setup_hebbian_c2(torch, D, lib):
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm",
         flop_fwd=FLOP_HEB_FWD, flop_bwd=FLOP_HEB_BWD, bytes_bwd=BYTES_HEB_BWD,
-        traffic_bwd=int((2178.6 + 297.6 + 264.0 + 64.5) * 2**20),   # measured: sweep + sum of the row parts (read + written MiB)
+        traffic_bwd=int((192.7 + 96.5 + 65.1 + 32.1 + 33.1 + 33.0) * 2**20),   # measured: gradients + seed + scan kernels (read + written MiB)
         kernel=None,
         kernel_names={"forward": "hebbian_forward", "backward": "hebbian_backward_segment"},
         config={"workload": "Hebbian rule at the shape of BASELINE configs[1]: 8 heads x 64 (d=512), batch 8, "

@@ -349,8 +349,287 @@ void launch_bwd_d(const HebBwdArgs &a, int batch) {
     }
 }
 
+// ── backward in chunk-parallel matrix form (d = 64) ─────────────────────────
+// The rule is linear in M, so with r_t = 1 - alpha_t and, inside a chunk of up to 64 tokens that
+// starts at state M_0 and receives the gradient S from the tokens after it,
+//     rho(tau, t) = prod_{t < r <= tau} r_r,   A(t) = prod_{r < t} r_r,   rho_L(t) = rho(L - 1, t),
+//     E_t  = sum_{tau >= t} rho(tau, t) dy_tau q_tau^T + rho_L(t) S          (gradient w.r.t. M_{t+1})
+//     M_t  = A(t) M_0 + sum_{s < t} rho(t - 1, s) v_s k_s^T
+// every output is a product of 64 x 64 matrices:
+//     d_v = (R o K Q^T) dY + rho_L o (K S^T)        d_k = (R o V dY^T) Q + rho_L o (V S)
+//     d_q = (R o V dY^T)^T K + A(t+1) o (dY M_0)    d_alpha_t = -<M_t, E_t>  (four sums, below)
+// with R[t][tau] = rho(tau, t) for t <= tau < L and 0 elsewhere.  Only the states at chunk starts are
+// read (1/64 of the trajectory), no division is needed, and the chunks are independent once S is known:
+// S_{c-1} = P_c + gamma_c S_c with P_c = sum_tau A(tau+1) dy_tau q_tau^T, gamma_c = A(L), a scan over
+// the chunks of a chain that costs d*d multiply-adds per chunk.  Three launches: P and gamma per chunk,
+// the scan, the gradients per chunk; all products on v_mfma_f32_16x16x4_f32 (fp32 in and out).
+constexpr int kHC = 64;   // tokens per chunk
+constexpr int kHL = 68;   // LDS row stride (= 4 mod 64: the operand reads of a wave fall on 64 banks)
+
+// acc[jt] += A B for the wave's 16-row strip (rows wr ..) and the four 16-column tiles; AT / BT read
+// the operand transposed (A[i][k] = bufA[k][i], B[k][n] = bufB[n][k]).
+template <bool AT, bool BT>
+__device__ __forceinline__ void heb_strip_mma(const float *bufA, const float *bufB, f32x4 (&acc)[4], int wr, int ml,
+                                              int kg) {
+#pragma unroll 4
+    for (int k0 = 0; k0 < kHC; k0 += 4) {
+        const float av = AT ? bufA[(k0 + kg) * kHL + wr + ml] : bufA[(wr + ml) * kHL + k0 + kg];
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++) {
+            const float bv = BT ? bufB[(16 * jt + ml) * kHL + k0 + kg] : bufB[(k0 + kg) * kHL + 16 * jt + ml];
+            acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[jt], 0, 0, 0);
+        }
+    }
+}
+
+__device__ __forceinline__ void heb_clear(f32x4 (&acc)[4]) {
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) acc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// rows [0, L) of a [tokens, 64] block into an LDS matrix, zeros behind them
+__device__ __forceinline__ void heb_stage_rows(float *dst, const float *src, int L, int tid) {
+    for (int e = tid; e < kHC * 16; e += 256) {
+        const int row = e >> 4, j = (e & 15) * 4;
+        f32x4 x = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (row < L) x = *reinterpret_cast<const f32x4 *>(src + (size_t)row * 64 + j);
+        *reinterpret_cast<f32x4 *>(dst + row * kHL + j) = x;
+    }
+}
+
+// P_c and gamma_c of every chunk: one workgroup per (chain, chunk).
+__global__ __launch_bounds__(256) void heb_chunk_seed_kernel(HebBwdArgs a, float *P, float *gamma, int nch) {
+    __shared__ __align__(16) float sDY[kHC * kHL];
+    __shared__ __align__(16) float sQ[kHC * kHL];
+    __shared__ float sa[kHC + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wr = 16 * (tid >> 6), ml = lane & 15, kg = lane >> 4;
+    const int chunk = blockIdx.x % nch, b = blockIdx.x / nch;
+    const int t0 = a.t_start + chunk * kHC, L = min(kHC, a.t_end - t0);
+    const size_t tok = (size_t)b * a.seq_len + t0;
+    heb_stage_rows(sDY, a.d_y + tok * 64, L, tid);
+    heb_stage_rows(sQ, a.q + tok * 64, L, tid);
+    if (tid == 0) {
+        float p = 1.f;
+        sa[0] = 1.f;
+        for (int t = 0; t < kHC; t++) {
+            if (t < L) p *= 1.f - a.alpha[tok + t];
+            sa[t + 1] = p;   // A(t + 1); constant behind the chunk's last token
+        }
+    }
+    __syncthreads();
+    f32x4 acc[4];
+    heb_clear(acc);
+#pragma unroll 4
+    for (int k0 = 0; k0 < kHC; k0 += 4) {
+        const float av = sDY[(k0 + kg) * kHL + wr + ml] * sa[k0 + kg + 1];
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++)
+            acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, sQ[(k0 + kg) * kHL + 16 * jt + ml], acc[jt], 0, 0, 0);
+    }
+    float *dst = P + (size_t)blockIdx.x * 4096;
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) dst[(wr + 4 * kg + v) * 64 + 16 * jt + ml] = acc[jt][v];
+    }
+    if (tid == 0) gamma[blockIdx.x] = sa[L];
+}
+
+// S_c for every chunk of a chain (the gradient entering the chunk from the tokens after it) and the
+// gradient leaving the segment: element-wise over d*d, sequential over the chunks.
+__global__ __launch_bounds__(256) void heb_chunk_scan_kernel(const float *P, const float *gamma, const float *seed,
+                                                             float *S, float *d_m_out, int nch) {
+    const int b = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+    float sv = seed ? seed[(size_t)b * 4096 + e] : 0.f;
+    for (int c = nch - 1; c >= 0; c--) {
+        const size_t o = ((size_t)b * nch + c) * 4096 + e;
+        S[o] = sv;
+        sv = fmaf(gamma[b * nch + c], sv, P[o]);
+    }
+    d_m_out[(size_t)b * 4096 + e] = sv;
+}
+
+constexpr int kHebGradLds = (8 * kHC * kHL + 1024) * (int)sizeof(float);
+
+// The gradients of one chunk: one workgroup per (chain, chunk), wave w owning token rows 16 w ..
+__global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, const float *Sc, int nch) {
+    extern __shared__ __align__(16) float heb_lds[];
+    float *bK = heb_lds, *bV = bK + kHC * kHL, *bQ = bV + kHC * kHL, *bDY = bQ + kHC * kHL, *bM = bDY + kHC * kHL;
+    float *bW1 = bM + kHC * kHL, *bW2 = bW1 + kHC * kHL, *bR = bW2 + kHC * kHL;
+    float *rr = bR + kHC * kHL, *aa = rr + 64, *rhoL = aa + 80, *A1 = rhoL + 64, *gs = A1 + 64, *colp = gs + 64;
+    float *red = colp + 256;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, wr = 16 * wave, ml = lane & 15, kg = lane >> 4;
+    const int chunk = blockIdx.x % nch, b = blockIdx.x / nch;
+    const int seg = a.t_end - a.t_start;
+    const int t0 = a.t_start + chunk * kHC, L = min(kHC, a.t_end - t0);
+    const size_t tok = (size_t)b * a.seq_len + t0;
+    const float *m0 = a.m_states + ((size_t)b * (seg + 1) + (t0 - a.t_start)) * 4096;
+    const float *sc = Sc + (size_t)blockIdx.x * 4096;
+
+    heb_stage_rows(bK, a.k + tok * 64, L, tid);
+    heb_stage_rows(bV, a.v + tok * 64, L, tid);
+    heb_stage_rows(bQ, a.q + tok * 64, L, tid);
+    heb_stage_rows(bDY, a.d_y + tok * 64, L, tid);
+    heb_stage_rows(bM, sc, kHC, tid);   // S
+    if (tid < 64) rr[tid] = tid < L ? 1.f - a.alpha[tok + tid] : 1.f;
+    __syncthreads();
+    if (wave == 0) {
+        // lane t builds row t of R from its diagonal rightwards; tau runs in lock step over the wave
+        const int t = lane;
+        float p = 1.f;
+#pragma unroll 8
+        for (int tau = 0; tau < kHC; tau++) {
+            if (tau > t) p *= rr[tau];
+            bR[t * kHL + tau] = (tau >= t && tau < L && t < L) ? p : 0.f;
+        }
+        rhoL[t] = t < L ? bR[t * kHL + L - 1] : 0.f;
+    } else if (wave == 1) {
+        // A(t) for t = 0 .. 64
+        float p = 1.f;
+        for (int q = 0; q < lane; q++) p *= rr[q];
+        aa[lane] = p;
+        if (lane == 63) aa[64] = p * rr[63];
+    }
+    // <M_0, S>
+    {
+        float part = 0.f;
+        for (int e = tid; e < 1024; e += 256) {
+            const int row = e >> 4, j = (e & 15) * 4;
+            const f32x4 mv = *reinterpret_cast<const f32x4 *>(m0 + row * 64 + j);
+            const f32x4 sv = *reinterpret_cast<const f32x4 *>(bM + row * kHL + j);
+            part += mv[0] * sv[0] + mv[1] * sv[1] + mv[2] * sv[2] + mv[3] * sv[3];
+        }
+        part = wave_allreduce(part);
+        if (lane == 0) red[wave] = part;
+    }
+    // products with S: T1 = K S^T (rows of d_v), T2 = V S (rows of d_k), g_s = v_s^T S k_s
+    f32x4 dv[4], dk[4], dq[4];
+    heb_clear(dv); heb_clear(dk); heb_clear(dq);
+    heb_strip_mma<false, true>(bK, bM, dv, wr, ml, kg);
+    heb_strip_mma<false, false>(bV, bM, dk, wr, ml, kg);
+    __syncthreads();   // tables, red and every read of S are done
+    const float m0s = red[0] + red[1] + red[2] + red[3];
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int row = wr + 4 * kg + v;
+        float part = 0.f;
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++) part = fmaf(dk[jt][v], bK[row * kHL + 16 * jt + ml], part);
+        part = group_allreduce<16>(part);
+        if (ml == 0) gs[row] = part;
+        const float sL = rhoL[row];
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++) { dv[jt][v] *= sL; dk[jt][v] *= sL; }
+    }
+    heb_stage_rows(bM, m0, kHC, tid);   // M_0
+    __syncthreads();
+    // T3 = dY M_0: d_q starts as A(t+1) T3, and A1_tau = dy_tau^T M_0 q_tau
+    heb_strip_mma<false, false>(bDY, bM, dq, wr, ml, kg);
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int row = wr + 4 * kg + v;
+        float part = 0.f;
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++) part = fmaf(dq[jt][v], bQ[row * kHL + 16 * jt + ml], part);
+        part = group_allreduce<16>(part);
+        if (ml == 0) A1[row] = part;
+        const float sA = aa[row + 1];
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++) dq[jt][v] *= sA;
+    }
+    // G1 = K Q^T, G2 = V dY^T (token x token); W1 = R o G1, W2 = R o G2, and G1 o G2 for d_alpha
+    f32x4 g1[4], g2[4];
+    heb_clear(g1); heb_clear(g2);
+    heb_strip_mma<false, true>(bK, bQ, g1, wr, ml, kg);
+    heb_strip_mma<false, true>(bV, bDY, g2, wr, ml, kg);
+    __syncthreads();   // M_0 has been read
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int o = (wr + 4 * kg + v) * kHL + 16 * jt + ml;
+            const float rv = bR[o];
+            bW1[o] = rv * g1[jt][v];
+            bW2[o] = rv * g2[jt][v];
+            bM[o] = g1[jt][v] * g2[jt][v];
+        }
+    }
+    __syncthreads();
+    heb_strip_mma<false, false>(bW1, bDY, dv, wr, ml, kg);
+    heb_strip_mma<false, false>(bW2, bQ, dk, wr, ml, kg);
+    heb_strip_mma<true, false>(bW2, bK, dq, wr, ml, kg);
+    // U[s][t] = sum_{tau >= t} rho(tau, t) (v_s . dy_tau)(k_s . q_tau)
+    f32x4 u[4];
+    heb_clear(u);
+    heb_strip_mma<false, true>(bM, bR, u, wr, ml, kg);
+    float *dvo = a.d_v + tok * 64, *dko = a.d_k + tok * 64, *dqo = a.d_q + tok * 64;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int row = wr + 4 * kg + v;
+        if (row < L) {
+#pragma unroll
+            for (int jt = 0; jt < 4; jt++) {
+                dvo[(size_t)row * 64 + 16 * jt + ml] = dv[jt][v];
+                dko[(size_t)row * 64 + 16 * jt + ml] = dk[jt][v];
+                dqo[(size_t)row * 64 + 16 * jt + ml] = dq[jt][v];
+            }
+        }
+    }
+    // sum_{s < t} rho(t - 1, s) U[s][t]: columns of the wave's 16 rows, then over the waves
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+        const int t = 16 * jt + ml;
+        float part = 0.f;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int srow = wr + 4 * kg + v;
+            if (srow < t) part = fmaf(bR[srow * kHL + t - 1], u[jt][v], part);
+        }
+        part = stride_allreduce<16>(part);
+        if (kg == 0) colp[wave * 64 + t] = part;
+    }
+    __syncthreads();
+    if (tid < L) {
+        // d_alpha_t = -<M_t, E_t> = -( A(t) [sum_{tau>=t} rho(tau,t) A1_tau + rho_L(t) <M_0,S>]
+        //                             + sum_{s<t} rho(t-1,s) [U[s][t] + rho_L(t) g_s] )
+        const int t = tid;
+        float s1 = 0.f, s4 = 0.f;
+        for (int tau = t; tau < L; tau++) s1 = fmaf(bR[t * kHL + tau], A1[tau], s1);
+        for (int s2 = 0; s2 < t; s2++) s4 = fmaf(bR[s2 * kHL + t - 1], gs[s2], s4);
+        const float s3 = colp[t] + colp[64 + t] + colp[128 + t] + colp[192 + t];
+        const float x = aa[t] * fmaf(rhoL[t], m0s, s1) + s3 + rhoL[t] * s4;
+        a.d_alpha[tok + t] = -x;
+    }
+}
+
+// d = 64 only; false if the shape is not covered (the caller falls back to the sweep kernel).
+bool launch_bwd_chunks(const HebBwdArgs &a, int batch) {
+    const int seg = a.t_end - a.t_start;
+    if (seg <= 0) return false;
+    const int nch = (seg + kHC - 1) / kHC;
+    const size_t chunks = (size_t)batch * nch;
+    float *P = scratch(5, chunks * 4096 * sizeof(float));
+    float *gamma = scratch(6, chunks * sizeof(float));
+    float *S = scratch(7, chunks * 4096 * sizeof(float));
+    if (failed()) return true;
+    hipLaunchKernelGGL(heb_chunk_seed_kernel, dim3((unsigned)chunks), dim3(256), 0, stream(), a, P, gamma, nch);
+    check_launch("heb_chunk_seed_kernel");
+    hipLaunchKernelGGL(heb_chunk_scan_kernel, dim3(16, batch), dim3(256), 0, stream(), P, gamma, a.d_m_seed, S,
+                       a.d_m_out, nch);
+    check_launch("heb_chunk_scan_kernel");
+    check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(heb_chunk_grads_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kHebGradLds), "dynamic LDS size");
+    {
+        KernelTimer kt("hebbian_bwd_kernel");
+        hipLaunchKernelGGL(heb_chunk_grads_kernel, dim3((unsigned)chunks), dim3(256), kHebGradLds, stream(), a, S, nch);
+        check_launch("heb_chunk_grads_kernel");
+    }
+    return true;
+}
+
 bool launch_bwd(HebBwdArgs a, int d, int batch) {
     if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) return false;
+    if (d == 64 && launch_bwd_chunks(a, batch)) return true;
     a.rows = rows_per_workgroup(d, batch);
     const int parts = d / a.rows;
     if (parts > 1) {

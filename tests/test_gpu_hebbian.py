@@ -64,7 +64,8 @@ def test_reference_backward_recipe():
         assert_abs(n, host(g[n]), want[n], 1e-4)
 
 
-@pytest.mark.parametrize("B,s,d", [(3, 40, 16), (5, 33, 32), (6, 70, 64), (2, 9, 128), (2, 21, 8)])
+@pytest.mark.parametrize("B,s,d", [(3, 40, 16), (5, 33, 32), (6, 70, 64), (3, 257, 64), (2, 64, 64), (2, 9, 128),
+                                   (2, 21, 8)])
 def test_batched_forward_and_segment_backward_match_oracle(B, s, d):
     x = rule_inputs(B, s, d, 900 + d + s, m0_scale=0.3)
     y, ms = gpu_forward(x["k"], x["v"], x["q"], x["alpha"], x["m0"])
@@ -94,9 +95,9 @@ def test_forward_strides_select_a_window_of_a_longer_sequence():
     assert_close("m_states", ms, mo)
 
 
-@pytest.mark.parametrize("C", [4, 7, 64])
-def test_checkpointed_forward_and_segment_backward_compose(C):
-    s, d = 23, 32
+@pytest.mark.parametrize("s,d,C", [(23, 32, 4), (23, 32, 7), (23, 32, 64), (150, 64, 64), (150, 64, 100),
+                                   (150, 64, 9)])
+def test_checkpointed_forward_and_segment_backward_compose(s, d, C):
     x = rule_inputs(1, s, d, 31, m0_scale=0.3)
     k, v, q, alpha, m0, dy = (x[n][0] for n in ("k", "v", "q", "alpha", "m0", "dy"))
     yo, ck = orc.hebbian_forward(k, v, q, alpha, m0, checkpoint_interval=C)
