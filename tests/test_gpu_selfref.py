@@ -55,6 +55,10 @@ CASES = [  # B, s, d, C
     (2, 130, 64, 64),   # full chunks plus a two-token chunk
     (1, 100, 64, 80),   # chunks above 64 tokens take the trajectory path
     (2, 150, 16, 70),
+    (1, 1, 16, 4),      # one token
+    (1, 64, 64, 64),    # exactly one full chunk: no chunk boundary is crossed
+    (1, 65, 64, 64),    # a one-token chunk after a full one
+    (2, 128, 32, 64),
 ]
 
 
