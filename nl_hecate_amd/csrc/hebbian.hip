@@ -134,28 +134,35 @@ struct HebFwdArgs {
     float *m_states, *y;
     int seq_len, input_stride, m_stride, ckpt, rows;
     long long states_per_chain;   // matrices of m_states per chain
+    int chunks;                   // > 0: workgroup x is chunk x % chunks of chain x / chunks, m_initial holds the
+                                  // chunk-start states [chain][chunk][D*D] (trajectory mode only)
 };
+
+constexpr int kHC = 64;   // tokens per chunk of the chunk-parallel kernels
 
 template <int D, int STORE>
 __global__ __launch_bounds__(heb_threads(D)) void hebbian_fwd_kernel(HebFwdArgs a) {
     constexpr int CP = D / 4, T = 8;
     __shared__ __align__(16) float tile[2][T][3][D];   // k, q, v of a tile's tokens
     __shared__ float tal[2][T];
-    const int b = blockIdx.x, tid = threadIdx.x, cq = tid & 3, c0 = cq * CP;
+    const int tid = threadIdx.x, cq = tid & 3, c0 = cq * CP;
+    const int b = a.chunks ? blockIdx.x / a.chunks : blockIdx.x, chunk = a.chunks ? blockIdx.x % a.chunks : 0;
+    const int t_off = chunk * kHC, len = a.chunks ? min(kHC, a.seq_len - t_off) : a.seq_len;
+    const bool inner_chunk = a.chunks && chunk + 1 < a.chunks;   // its last state is the next chunk's first store
     const int rl = min(tid >> 2, a.rows - 1);          // lanes beyond the rows (d = 8) shadow the last row
     const bool valid = (tid >> 2) < a.rows;
     const int r = blockIdx.y * a.rows + rl;            // a.rows rows of the chain per workgroup
-    const size_t tok0 = (size_t)b * a.input_stride;
+    const size_t tok0 = (size_t)b * a.input_stride + t_off;
     const float *kb = a.k + tok0 * D, *qb = a.q + tok0 * D, *vb = a.v + tok0 * D;
     const float *ab = a.alpha + tok0;
-    float *ms = a.m_states + (size_t)b * a.states_per_chain * D * D + r * D + c0;
-    float *yb = a.y + (size_t)b * a.seq_len * D;
+    float *ms = a.m_states + ((size_t)b * a.states_per_chain + t_off) * D * D + r * D + c0;
+    float *yb = a.y + ((size_t)b * a.seq_len + t_off) * D;
     float M[CP];
-    gload<CP>(M, a.m_initial + (size_t)b * a.m_stride + r * D + c0);
+    gload<CP>(M, a.m_initial + (a.chunks ? (size_t)blockIdx.x * D * D : (size_t)b * a.m_stride) + r * D + c0);
     if (valid) gstore<CP>(ms, M);
-    if (a.seq_len == 0) return;
+    if (len == 0) return;
     int ck = 1;
-    const int last = a.seq_len - 1, ntile = (a.seq_len + T - 1) / T;
+    const int last = len - 1, ntile = (len + T - 1) / T;
     f32x4 stage[tile_per_lane(D, T, 3)];
     float stage_al;
     tile_fetch<D, T, 3>(stage, stage_al, kb, qb, vb, vb, ab, [&](int j) { return min(j, last); });
@@ -174,7 +181,7 @@ __global__ __launch_bounds__(heb_threads(D)) void hebbian_fwd_kernel(HebFwdArgs 
 #pragma unroll
             for (int i = 0; i < CP; i++) M[i] = ret * M[i] + v_r * kc[i];
             if (STORE == HEB_TRAJ) {
-                if (valid) gstore<CP>(ms + (size_t)(t + 1) * D * D, M);
+                if (valid && !(inner_chunk && t == last)) gstore<CP>(ms + (size_t)(t + 1) * D * D, M);
             } else if (((t + 1) % a.ckpt == 0) || (t + 1 == a.seq_len)) {
                 if (valid) gstore<CP>(ms + (size_t)ck * D * D, M);
                 ck++;
@@ -315,10 +322,22 @@ int rows_per_workgroup(int d, int batch) {
     return rows;
 }
 
+// Forward in chunks (d = 64, trajectory mode): the state at the start of chunk c+1 is
+// gamma_c M_{c,0} + P_c with P_c = sum_s rho(L-1, s) v_s k_s^T and gamma_c = A(L), so after one product
+// per chunk and a scan over the chunks every chunk of every chain writes its part of the trajectory in
+// its own workgroup (the trajectory is what the forward has to move: 16 KB per token and chain).
+__global__ __launch_bounds__(256) void heb_chunk_fwd_seed_kernel(HebFwdArgs a, float *P, float *gamma, int nch);
+__global__ __launch_bounds__(256) void heb_chunk_fwd_scan_kernel(const float *P, const float *gamma,
+                                                                 const float *m_initial, int m_stride, float *Mstart,
+                                                                 int nch);
+bool launch_fwd_chunks(HebFwdArgs a, int batch);
+
 template <int STORE>
 bool launch_fwd(HebFwdArgs a, int d, int batch) {
-    a.rows = rows_per_workgroup(d, batch);
-    const dim3 grid(batch, d / a.rows), block(4 * a.rows < 64 ? 64 : 4 * a.rows);
+    if (STORE == HEB_TRAJ && d == 64 && a.seq_len > 2 * kHC && a.chunks == 0 && launch_fwd_chunks(a, batch)) return true;
+    const int groups = a.chunks ? batch * a.chunks : batch;
+    a.rows = rows_per_workgroup(d, groups);
+    const dim3 grid(groups, d / a.rows), block(4 * a.rows < 64 ? 64 : 4 * a.rows);
     switch (d) {
         case 8: hipLaunchKernelGGL((hebbian_fwd_kernel<8, STORE>), grid, block, 0, stream(), a); break;
         case 16: hipLaunchKernelGGL((hebbian_fwd_kernel<16, STORE>), grid, block, 0, stream(), a); break;
@@ -363,7 +382,6 @@ void launch_bwd_d(const HebBwdArgs &a, int batch) {
 // S_{c-1} = P_c + gamma_c S_c with P_c = sum_tau A(tau+1) dy_tau q_tau^T, gamma_c = A(L), a scan over
 // the chunks of a chain that costs d*d multiply-adds per chunk.  Three launches: P and gamma per chunk,
 // the scan, the gradients per chunk; all products on v_mfma_f32_16x16x4_f32 (fp32 in and out).
-constexpr int kHC = 64;   // tokens per chunk
 constexpr int kHL = 68;   // LDS row stride (= 4 mod 64: the operand reads of a wave fall on 64 banks)
 
 // acc[jt] += A B for the wave's 16-row strip (rows wr ..) and the four 16-column tiles; AT / BT read
@@ -625,6 +643,73 @@ bool launch_bwd_chunks(const HebBwdArgs &a, int batch) {
         check_launch("heb_chunk_grads_kernel");
     }
     return true;
+}
+
+__global__ __launch_bounds__(256) void heb_chunk_fwd_seed_kernel(HebFwdArgs a, float *P, float *gamma, int nch) {
+    __shared__ __align__(16) float sV[kHC * kHL];
+    __shared__ __align__(16) float sK[kHC * kHL];
+    __shared__ float sb[kHC + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wr = 16 * (tid >> 6), ml = lane & 15, kg = lane >> 4;
+    const int chunk = blockIdx.x % nch, b = blockIdx.x / nch;
+    const int t0 = chunk * kHC, L = min(kHC, a.seq_len - t0);
+    const size_t tok = (size_t)b * a.input_stride + t0;
+    heb_stage_rows(sV, a.v + tok * 64, L, tid);
+    heb_stage_rows(sK, a.k + tok * 64, L, tid);
+    if (tid == 0) {
+        // sb[s] = rho(L-1, s) = prod_{s < r <= L-1} (1 - alpha_r); sb[kHC] = A(L)
+        float p = 1.f;
+        for (int t = kHC - 1; t >= 0; t--) {
+            sb[t] = t < L ? p : 0.f;
+            if (t < L) p *= 1.f - a.alpha[tok + t];
+        }
+        sb[kHC] = p;
+    }
+    __syncthreads();
+    f32x4 acc[4];
+    heb_clear(acc);
+#pragma unroll 4
+    for (int k0 = 0; k0 < kHC; k0 += 4) {
+        const float av = sV[(k0 + kg) * kHL + wr + ml] * sb[k0 + kg];
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++)
+            acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, sK[(k0 + kg) * kHL + 16 * jt + ml], acc[jt], 0, 0, 0);
+    }
+    float *dst = P + (size_t)blockIdx.x * 4096;
+#pragma unroll
+    for (int jt = 0; jt < 4; jt++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) dst[(wr + 4 * kg + v) * 64 + 16 * jt + ml] = acc[jt][v];
+    }
+    if (tid == 0) gamma[blockIdx.x] = sb[kHC];
+}
+
+__global__ __launch_bounds__(256) void heb_chunk_fwd_scan_kernel(const float *P, const float *gamma,
+                                                                 const float *m_initial, int m_stride, float *Mstart,
+                                                                 int nch) {
+    const int b = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+    float m = m_initial[(size_t)b * m_stride + e];
+    for (int c = 0; c < nch; c++) {
+        const size_t o = ((size_t)b * nch + c) * 4096 + e;
+        Mstart[o] = m;
+        m = fmaf(gamma[b * nch + c], m, P[o]);
+    }
+}
+
+bool launch_fwd_chunks(HebFwdArgs a, int batch) {
+    const int nch = (a.seq_len + kHC - 1) / kHC;
+    const size_t chunks = (size_t)batch * nch;
+    float *P = scratch(5, chunks * 4096 * sizeof(float));
+    float *gamma = scratch(6, chunks * sizeof(float));
+    float *Mstart = scratch(7, chunks * 4096 * sizeof(float));
+    if (failed()) return true;
+    hipLaunchKernelGGL(heb_chunk_fwd_seed_kernel, dim3((unsigned)chunks), dim3(256), 0, stream(), a, P, gamma, nch);
+    check_launch("heb_chunk_fwd_seed_kernel");
+    hipLaunchKernelGGL(heb_chunk_fwd_scan_kernel, dim3(16, batch), dim3(256), 0, stream(), P, gamma, a.m_initial,
+                       a.m_stride, Mstart, nch);
+    check_launch("heb_chunk_fwd_scan_kernel");
+    a.m_initial = Mstart;
+    a.chunks = nch;
+    return launch_fwd<HEB_TRAJ>(a, 64, batch);
 }
 
 bool launch_bwd(HebBwdArgs a, int d, int batch) {

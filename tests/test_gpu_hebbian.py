@@ -64,7 +64,7 @@ def test_reference_backward_recipe():
         assert_abs(n, host(g[n]), want[n], 1e-4)
 
 
-@pytest.mark.parametrize("B,s,d", [(3, 40, 16), (5, 33, 32), (6, 70, 64), (3, 257, 64), (2, 64, 64), (2, 9, 128),
+@pytest.mark.parametrize("B,s,d", [(3, 40, 16), (5, 33, 32), (6, 70, 64), (3, 257, 64), (2, 64, 64), (2, 129, 64), (1, 1000, 64), (2, 9, 128),
                                    (2, 21, 8)])
 def test_batched_forward_and_segment_backward_match_oracle(B, s, d):
     x = rule_inputs(B, s, d, 900 + d + s, m0_scale=0.3)
@@ -84,9 +84,9 @@ def test_batched_forward_and_segment_backward_match_oracle(B, s, d):
             assert_close(f"{n}[{b}]", host(g[n])[b], want[n])
 
 
-def test_forward_strides_select_a_window_of_a_longer_sequence():
+@pytest.mark.parametrize("B,S,s,d", [(3, 24, 10, 16), (2, 300, 200, 64)])
+def test_forward_strides_select_a_window_of_a_longer_sequence(B, S, s, d):
     """input_stride / m_stride as in the other rules' forwards (core/kernels/hebbian_forward.cu:75-90)."""
-    B, S, s, d = 3, 24, 10, 16
     x = rule_inputs(B, S, d, 77, m0_scale=0.2)
     pool = np.concatenate([x["m0"], x["s0"]], 1).reshape(B, 2 * d * d)   # states with stride 2 d^2
     y, ms = gpu_forward(x["k"], x["v"], x["q"], x["alpha"], pool, input_stride=S, m_stride=2 * d * d, s=s)
