@@ -754,7 +754,7 @@ void hebbian_forward_f32_cuda(const float *k_mem, const float *v_mem, const floa
                               int batch_size, int input_stride, int m_stride) {
     if (!check_dims("hebbian_forward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
     const HebFwdArgs a{k_mem, v_mem, q_mem, alpha, m_initial, m_states, y, seq_len, input_stride, m_stride, 1, 0,
-                       (long long)seq_len + 1};
+                       (long long)seq_len + 1, 0};
     if (!launch_fwd<HEB_TRAJ>(a, d, batch_size)) bad_d("hebbian_forward_f32_cuda", d);
 }
 
@@ -767,7 +767,7 @@ void hebbian_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const
         return;
     }
     const HebFwdArgs a{k_mem, v_mem, q_mem, alpha, m_initial, m_states, y, seq_len, seq_len, d * d,
-                       checkpoint_interval, 0, (long long)n_ckpt_count(seq_len, checkpoint_interval)};
+                       checkpoint_interval, 0, (long long)n_ckpt_count(seq_len, checkpoint_interval), 0};
     if (!launch_fwd<HEB_CKPT>(a, d, 1)) bad_d("hebbian_forward_ckpt_f32_cuda", d);
 }
 
