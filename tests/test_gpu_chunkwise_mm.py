@@ -4,7 +4,7 @@ runs in float32 on the same (bf16-rounded) values.  Stated tolerance for bf16-in
 fp32-accumulate paths is relative 2e-2.  The bf16 forward carries every fp32 operand as a
 hi + lo bf16 pair and is held to 1e-3; the bf16 backward feeds its fp32 operands to the
 matrix cores as single bf16 values (fp32 accumulation) and is held to 1e-2; the float
-entry points compute in fp32 throughout and are held to 1e-4 / 2e-4."""
+entry points compute in fp32 throughout and are held to 1e-4 (measured: below 3e-6)."""
 import numpy as np
 import pytest
 import torch
@@ -94,7 +94,7 @@ def test_backward_matches_oracle(B, s, C, bf16):
            g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], g["d_m_initial"],
            g["d_s_initial"], s, d, B, C)
     torch.cuda.synchronize()
-    tol = 1e-2 if bf16 else 2e-4
+    tol = 1e-2 if bf16 else 1e-4
     for n in g:
         assert_close(n, host(g[n]), want[n], tol)
 
@@ -109,8 +109,8 @@ def test_initial_state_gradients_accumulate():
     D.call("titans_chunkwise_backward_mm_f32_rocm", f["k"], f["v"], f["q"], f["al"], f["th"], f["et"],
            f["mc"], f["sc"], dev(x["dy"]), *junk, dm, ds, s, d, B, 32)
     torch.cuda.synchronize()
-    assert_close("d_m_initial", host(dm) - 1.0, want["d_m_initial"], 2e-4)
-    assert_close("d_s_initial", host(ds) - 1.0, want["d_s_initial"], 2e-4)
+    assert_close("d_m_initial", host(dm) - 1.0, want["d_m_initial"], 1e-4)
+    assert_close("d_s_initial", host(ds) - 1.0, want["d_s_initial"], 1e-4)
 
 
 def test_matrix_form_agrees_with_sequential_kernels_at_benchmark_shape():
@@ -163,10 +163,10 @@ def test_delta_matrix_form_matches_oracle(B, s, C, bf16):
              d_theta=zeros(B, s), d_m=zeros(d, d))
     D.call("delta_chunkwise_backward_" + sfx, k, v, q, al, th, mc, dev(x["dy"]), *[g[n] for n in g], s, d, B, C)
     torch.cuda.synchronize()
-    tol = 1e-3 if bf16 else 2e-4
+    tol = 1e-3 if bf16 else 1e-4
     assert_close("y", host(y), np.stack([f[0] for f in fw]), tol)
     assert_close("m_chunk_states", host(mc), np.stack([f[1] for f in fw]), tol)
-    tol = 1e-2 if bf16 else 2e-4
+    tol = 1e-2 if bf16 else 1e-4
     for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta"):
         assert_close(n, host(g[n]), np.stack([o[n] for o in bw]), tol)
     assert_close("d_m_initial", host(g["d_m"]), sum(o["d_m"] for o in bw), tol)
