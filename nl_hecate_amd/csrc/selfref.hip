@@ -35,16 +35,18 @@ namespace {
 constexpr int kTB = 16;  // tokens staged in LDS at a time
 using f32x4 = float __attribute__((ext_vector_type(4)));
 
-// core/src/tensor.rs:202-207, 221-227
+// core/src/tensor.rs:202-207, 221-227.  The gates sit on the per-token critical path of the forward,
+// so exp, log and the reciprocal are the hardware approximations (v_exp_f32, v_log_f32, v_rcp_f32: about
+// one ulp each, three orders of magnitude inside the parity bar) instead of the library routines.
 __device__ __forceinline__ float sr_sigmoid(float x) {
     if (x >= 15.f) return 1.f;
     if (x <= -15.f) return 0.f;
-    return 1.f / (1.f + expf(-x));
+    return __builtin_amdgcn_rcpf(1.f + __expf(-x));
 }
 __device__ __forceinline__ float sr_softplus(float x) {
     if (x >= 15.f) return x;
     if (x <= -15.f) return 0.f;
-    return logf(1.f + expf(x));
+    return __logf(1.f + __expf(x));
 }
 
 // ── forward ────────────────────────────────────────────────────────────────
