@@ -127,3 +127,27 @@ def test_checkpointed_forward_and_segment_backward_compose(s, d, C):
     for n in g:
         assert_close(n, host(g[n])[0], want[n])
     assert_close("d_m", host(seed)[0], want["d_m"])
+
+
+@pytest.mark.parametrize("d", [32, 64])
+def test_saturated_gates(d):
+    """alpha = 1 wipes the memory (retention 0) and alpha = 0 keeps it: the gradient of a wiped step still
+    depends on the state before it, so nothing in the backward may divide by the retention."""
+    B, s = 2, 150
+    x = rule_inputs(B, s, d, 4242, m0_scale=0.3)
+    x["alpha"][:, 5::17] = 1.0
+    x["alpha"][:, 9::23] = 0.0
+    x["alpha"][0, 63] = 1.0   # last token of a 64-token chunk
+    x["alpha"][1, 64] = 1.0   # first token of the next one
+    y, ms = gpu_forward(x["k"], x["v"], x["q"], x["alpha"], x["m0"])
+    yo, mo = oracle_forward(x["k"], x["v"], x["q"], x["alpha"], x["m0"])
+    assert_close("y", y, yo)
+    assert_close("m_states", ms, mo)
+    g = dict(d_k=zeros(B, s, d), d_v=zeros(B, s, d), d_q=zeros(B, s, d), d_alpha=zeros(B, s), d_m=zeros(B, d, d))
+    D.hebbian_backward_dd_segment(dev(x["k"]), dev(x["v"]), dev(x["q"]), dev(x["alpha"]), dev(mo), dev(x["dy"]),
+                                  None, g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_m"], 0, s, d, B, s)
+    torch.cuda.synchronize()
+    for b in range(B):
+        want = orc.hebbian_backward(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], mo[b], x["dy"][b])
+        for n in want:
+            assert_close(f"{n}[{b}]", host(g[n])[b], want[n])
