@@ -116,3 +116,33 @@ def test_bad_arguments_are_reported():
     finally:
         lib.nlh_clear_error()
         lib.nlh_set_error_mode(0)
+
+
+@pytest.mark.parametrize("sg", [True, False])
+@pytest.mark.parametrize("d,C,early", [(16, 8, True), (16, 8, False), (64, 64, True)])   # at d = 64 the large
+def test_saturated_decay_gate(sg, d, C, early):                                          # column diverges later on
+    """alpha = sigmoid(mean) is clamped to exactly 0 below -15 and exactly 1 above 15
+    (core/src/tensor.rs:202-207).  A constant feature with a large first column of M_alpha drives the
+    mean to about -20 at every token but one, where it is about +20: there alpha = 1 (exactly, when the
+    token comes early enough that M_alpha has not drifted) wipes all six memories (retention 0), whose
+    gradient has no factor to divide by; the tokens before it keep retention 1 exactly."""
+    B, s = 2, 3 * C // 2 + 3
+    wipe = 1 if early else C // 2 + 1
+    mems, x, dy = inputs(B, s, d, seed=77 + d)
+    mems[:, 4, :, 0] = 20.0
+    x[:, :, 0] = -1.0
+    x[:, wipe, 0] = 1.0
+    got = gpu_run(mems, x, dy, C, sg)
+    want = oracle_run(mems, x, dy, C, sg, np.float32)
+    assert (want["alpha"] == 0.0).any()
+    assert (want["alpha"] == 1.0).any() if early else want["alpha"].max() > 0.99
+    # A gate within 1e-3 of saturation makes the retention 1 - alpha ill-conditioned in the mean it comes
+    # from, so float32 rounding alone moves the results by more than the usual bar: the yardstick is the
+    # float64 oracle, and the float32 oracle's own distance to it bounds what rounding explains.
+    ref = oracle_run(mems, x, dy, C, sg, np.float64)
+    for n in ("y", "mems", "k", "v", "q", "alpha", "theta", "frozen", "d_emb", "d_mems"):
+        r = ref[n].astype(np.float64)
+        scale = max(float(np.abs(r).max()), 1e-30)
+        e_gpu = float(np.abs(got[n].reshape(r.shape) - r).max()) / scale
+        e_f32 = float(np.abs(want[n].reshape(r.shape) - r).max()) / scale
+        assert e_gpu <= max(1e-4, 4.0 * e_f32), f"{n}: {e_gpu:.2e} against float64, float32 oracle {e_f32:.2e}"
