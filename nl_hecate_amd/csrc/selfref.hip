@@ -1118,6 +1118,7 @@ __global__ __launch_bounds__(4 * D) void selfref_bwd_kernel(
         vec_store<CP>(dmb + 4 * DD + r * D + c0, eA);
     }
 #undef T_
+#undef SWEEP_REQUEST
 }
 
 template <int D>
