@@ -11,6 +11,9 @@
 // and has two column sums (d_q = M_{t+1}^T dy, d_k = dM^T v) and one full sum (d_alpha) per token:
 // reduced inside the wave with DPP, across waves through a double-buffered LDS tile: one barrier per
 // token.  With the rows split, each part writes partial sums and one more launch adds the parts.
+// At d = 64 both directions take a chunk-parallel form instead (64-token chunks, a scan over the chunks,
+// 64 x 64 products on the matrix cores), described at those kernels; the per-token kernels
+// remain the path of every other width and of short sequences.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
