@@ -376,6 +376,57 @@ def test_checkpointed_backward_one_call(entry, B, s, d, C):
             assert_close(f"{n} has_s={has_s}", g[n], go[n])
 
 
+def _saturate(x, s, C):
+    """alpha exactly 0 and 1 (retention 1 and 0), eta exactly 0 and 1, theta 0: at segment edges, inside
+    segments, at the first and the last token, and in runs."""
+    spots = {0: (0.0, 1.0, None), 3: (1.0, 0.0, None), C - 1: (1.0, 1.0, 0.0), C: (0.0, 0.0, None),
+             C + 7: (1.0, None, None), 2 * C: (None, 0.0, 0.0), s - 1: (1.0, 1.0, None)}
+    for t, (a, e, th) in spots.items():
+        if a is not None: x["alpha"][:, t] = a
+        if e is not None: x["eta"][:, t] = e
+        if th is not None: x["theta"][:, t] = th
+    x["alpha"][1, 10:20] = 0.0
+    x["eta"][1, C + 10:C + 20] = 1.0
+    return x
+
+
+@pytest.mark.parametrize("d", [16, 64])
+def test_saturated_gates_full_trajectory(d):
+    B, s = 2, 70
+    x = _saturate(rule_inputs(B, s, d, 7300 + d, m0_scale=0.2), s, 32)
+    y, ms, ss = gpu_titans_forward(x)
+    yo, mo, so = orc.titans_forward_batch(x["k"], x["v"], x["q"], x["alpha"], x["theta"], x["eta"],
+                                          x["m0"], x["s0"])
+    assert_close("y", y, yo)
+    assert_close("m_states", ms, mo)
+    assert_close("s_states", ss, so)
+    g = gpu_titans_backward(x, mo, so)
+    go = orc.titans_backward_batch(x["k"], x["v"], x["q"], x["alpha"], x["theta"], x["eta"], mo, so, x["dy"])
+    for n in go:
+        assert np.isfinite(g[n]).all(), n
+        assert_close(n, g[n], go[n])
+    yd, md = gpu_delta_forward(x)
+    ydo, mdo = orc.delta_forward_batch(x["k"], x["v"], x["q"], x["alpha"], x["theta"], x["m0"])
+    assert_close("delta y", yd, ydo)
+    gd = gpu_delta_backward(x, mdo)
+    gdo = orc.delta_backward_batch(x["k"], x["v"], x["q"], x["alpha"], x["theta"], mdo, x["dy"])
+    for n in gdo:
+        assert_close("delta " + n, gd[n], gdo[n])
+
+
+@pytest.mark.parametrize("entry", ["", "_replay"])
+@pytest.mark.parametrize("d,C", [(64, 64), (16, 8)])
+def test_saturated_gates_checkpointed(entry, d, C):
+    B, s = 2, 3 * C + 5
+    x = _saturate(rule_inputs(B, s, d, 7400 + d, m0_scale=0.2), s, C)
+    for has_s in (True, False):
+        g = _gpu_ckpt_fwd_bwd(x, C, has_s, entry)
+        go = _oracle_ckpt_grads(x, C, has_s)
+        for n in g:
+            assert np.isfinite(g[n]).all(), n
+            assert_close(f"{n} has_s={has_s}", g[n], go[n])
+
+
 def test_checkpointed_backward_with_clip_takes_replay_schedule():
     x = rule_inputs(2, 40, 64, 7100, m0_scale=0.3)
     x["v"] *= 2.0
