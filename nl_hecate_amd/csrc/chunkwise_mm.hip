@@ -139,7 +139,7 @@ __device__ __forceinline__ void for_c(Strip &acc, F f) {
 // strip row 4*(l/16) + i.
 __device__ __forceinline__ void strip_row_sums(Strip &x) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) x.t[0][i] = group_allreduce<16>(x.t[0][i] + 0.f) + group_allreduce<16>(x.t[1][i] + 0.f);
+    for (int i = 0; i < 4; i++) x.t[0][i] = group_allreduce<16>(x.t[0][i] + x.t[1][i]);
 }
 // lanes that publish the row sums (one per 16-lane group), and the strip rows they hold
 __device__ __forceinline__ bool row_writer() { return (threadIdx.x & 15) == 0; }
