@@ -70,6 +70,24 @@ void titans_backward_f32_cuda(const float *k_mem, const float *v_mem, const floa
                               float *d_alpha, float *d_theta, float *d_eta,
                               float *d_m_initial, float *d_s_initial,
                               int seq_len, int d, int batch_size, float error_clip);
+/* No counterpart in the reference.  titans_backward_f32_cuda for callers that
+ * cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same
+ * results to 1e-4, but its work buffers (per-chain dM / dS [batch, d*d] each,
+ * and for d = 128 the partial sums of a chain's four workgroups,
+ * 4*batch*seq_len*(2d+4) floats) live in a fixed 8 MiB device array inside the
+ * library, so the call makes no hipMalloc / hipFree.  d in {8,16,32,64,128};
+ * 2*batch*d*d (+ partial sums) must not exceed 2 097 152 floats (256 chains at
+ * d = 64), otherwise the call fails with a message and launches nothing.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one
+ * GPU (two streams, two threads) race. */
+void titans_backward_noalloc_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                      const float *alpha, const float *theta, const float *eta,
+                                      const float *m_states, const float *s_states, const float *d_y,
+                                      float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                      float *d_alpha, float *d_theta, float *d_eta,
+                                      float *d_m_initial, float *d_s_initial,
+                                      int seq_len, int d, int batch_size, float error_clip);
 /* core/src/cuda_ffi.rs:230.  One chain; stores M/S at slot 0 and after every
  * token with (t+1)%C==0 or t+1==seq_len. */
 void titans_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,

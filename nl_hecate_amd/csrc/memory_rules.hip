@@ -607,17 +607,36 @@ static void launch_bwd_c(const BwdArgs &a, bool coupled) {
     check_launch("rule_bwd_traj_kernel");
 }
 
+// rows-per-lane of the backward launch: `whole_chain` keeps a chain in as few workgroups as the
+// kernels allow (one for d <= 64), whatever the batch
+static int bwd_rpl(int d, int batch, bool coupled, bool whole_chain) {
+    return (whole_chain && d == 64) ? 4 : pick_rpl(d, batch, coupled);
+}
+
+// floats of partial-sum workspace a backward launch needs (0 when a chain is one workgroup)
+static size_t bwd_partial_floats(int d, int batch, int seq_len, int rpl) {
+    const int parts = ceil_div(d, rows_per_wg(d, rpl));
+    return parts > 1 ? (size_t)parts * batch * seq_len * (2 * (size_t)d + 4) : 0;
+}
+
+// ws == nullptr: partial sums come from the arena; otherwise from ws (bwd_partial_floats floats)
 template <bool HAS_S, bool FROZEN = false>
-static bool launch_bwd(BwdArgs a, int d) {
+static bool launch_bwd(BwdArgs a, int d, float *ws = nullptr, bool whole_chain = false) {
     const bool coupled = a.error_clip > 0.f;
-    const int rpl = pick_rpl(d, a.batch, coupled);
+    const int rpl = bwd_rpl(d, a.batch, coupled, whole_chain);
     a.parts = ceil_div(d, rows_per_wg(d, rpl));
     if (coupled && a.parts != 1) return false;
     if (a.parts > 1) {
         size_t n = (size_t)a.parts * a.batch * a.seq_len;
-        a.ws_dq = scratch(2, n * d * sizeof(float));
-        a.ws_dk = scratch(3, n * d * sizeof(float));
-        a.ws_gate = scratch(4, n * 4 * sizeof(float));
+        if (ws) {
+            a.ws_dq = ws;
+            a.ws_dk = ws + n * d;
+            a.ws_gate = ws + 2 * n * d;
+        } else {
+            a.ws_dq = scratch(2, n * d * sizeof(float));
+            a.ws_dk = scratch(3, n * d * sizeof(float));
+            a.ws_gate = scratch(4, n * 4 * sizeof(float));
+        }
         if (failed()) return true;
     }
     switch (d) {
@@ -642,6 +661,31 @@ void accumulate_over_batch(const float *src, float *dst, int batch, int n) {
     hipLaunchKernelGGL(accumulate_over_batch_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream(),
                        src, dst, batch, n);
     check_launch("accumulate_over_batch_kernel");
+}
+
+// Work space of the entry point that allocates nothing: a fixed device array (each GPU the
+// library runs on holds its own copy until the process ends).  Host code never uses the array's
+// name as an address: the device address is looked up once per device and kept.
+constexpr size_t kNoAllocFloats = (size_t)2 << 20;   // 8 MiB
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float g_noalloc_scratch[kNoAllocFloats];
+static float *g_noalloc_ptr[kMaxDevices] = {nullptr};
+
+static float *noalloc_base() {
+    int dev = 0;
+    check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (failed()) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) { fail("device ordinal %d out of range", dev); return nullptr; }
+    if (!g_noalloc_ptr[dev]) {
+        float *p = nullptr;
+        hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(g_noalloc_scratch));
+        if (e != hipSuccess || !p) {
+            fail("hipGetSymbolAddress(g_noalloc_scratch): %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_noalloc_ptr[dev] = p;
+    }
+    return g_noalloc_ptr[dev];
 }
 
 int n_ckpt_count(int seq_len, int c) {  // core/src/gpu_forward.rs:2885-2897
@@ -914,6 +958,39 @@ void titans_backward_f32_cuda(const float *k_mem, const float *v_mem, const floa
               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
               dm, ds, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
     if (!launch_bwd<true>(a, d)) { unsupported("titans_backward_f32_cuda", d, error_clip > 0.f); return; }
+    accumulate_over_batch(dm, d_m_initial, batch_size, (int)dd);
+    accumulate_over_batch(ds, d_s_initial, batch_size, (int)dd);
+}
+
+// Same contract and kernels as titans_backward_f32_cuda for callers that cannot allocate device
+// memory: the work buffers (per-chain dM / dS and, for d = 128, the partial sums of a chain's
+// workgroups) live in a file-scope device array of fixed size.
+void titans_backward_noalloc_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
+                                      const float *alpha, const float *theta, const float *eta,
+                                      const float *m_states, const float *s_states, const float *d_y,
+                                      float *d_k_mem, float *d_v_mem, float *d_q_mem,
+                                      float *d_alpha, float *d_theta, float *d_eta,
+                                      float *d_m_initial, float *d_s_initial,
+                                      int seq_len, int d, int batch_size, float error_clip) {
+    const char *fn = "titans_backward_noalloc_f32_rocm";
+    if (!check_dims(fn, seq_len, d, batch_size) || batch_size == 0) return;
+    if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) { unsupported(fn, d, error_clip > 0.f); return; }
+    const size_t dd = (size_t)d * d;
+    const bool coupled = error_clip > 0.f;
+    const size_t state_floats = 2 * (size_t)batch_size * dd;
+    const size_t need = state_floats + bwd_partial_floats(d, batch_size, seq_len, bwd_rpl(d, batch_size, coupled, true));
+    if (need > kNoAllocFloats) {
+        fail("%s: batch_size=%d, d=%d, seq_len=%d need %zu floats of work space; the fixed buffer holds %zu "
+             "(use titans_backward_f32_cuda).", fn, batch_size, d, seq_len, need, kNoAllocFloats);
+        return;
+    }
+    float *base = noalloc_base();
+    if (!base) return;
+    float *dm = base, *ds = base + (size_t)batch_size * dd;
+    BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_states, s_states, d_y, nullptr, nullptr,
+              d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
+              dm, ds, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
+    if (!launch_bwd<true>(a, d, base + state_floats, true)) { unsupported(fn, d, coupled); return; }
     accumulate_over_batch(dm, d_m_initial, batch_size, (int)dd);
     accumulate_over_batch(ds, d_s_initial, batch_size, (int)dd);
 }
