@@ -33,6 +33,12 @@ const char *nlh_last_error(void);      /* "" when no error is recorded */
 void nlh_clear_error(void);
 void nlh_set_stream(void *hip_stream); /* hipStream_t; NULL = null stream */
 void nlh_release_workspace(void);      /* frees the library's device scratch */
+/* Bumped whenever a scratch buffer is freed (a slot grew, or nlh_release_workspace
+ * ran).  A HIP graph captured from calls into this library holds scratch addresses:
+ * record the value at capture, and when it has changed drop the graph and capture
+ * again instead of replaying it.  A slot never grows while the launch stream is
+ * being captured: such a call fails with a message instead. */
+unsigned long long nlh_workspace_generation(void);
 /* hipEvent pair on the launch stream: start, then stop returns elapsed ms
  * (blocks until the stop event completes); negative on failure. */
 int nlh_timer_start(void);

@@ -201,6 +201,7 @@ constexpr size_t kAdjointLds = (6 * BMAT + 12 * HMAT) * sizeof(u16) + (5 * CW + 
 bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
                             const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
                             int chunk_size, bool has_s) {
+    const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size);
     static bool attr_set = false;
     if (!attr_set) {
@@ -210,7 +211,7 @@ bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kAdjointLds), "dynamic LDS size");
         attr_set = true;
     }
-    if (failed()) return true;
+    if (es.failed()) return true;
     const int tabf = (int)chunkwise_grads_table_floats(), vecf = (int)chunkwise_grads_vec_floats();
     if (has_s)
         hipLaunchKernelGGL(cw_adjoint_chain_kernel<true>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,

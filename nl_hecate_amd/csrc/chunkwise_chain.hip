@@ -385,6 +385,7 @@ template <bool HAS_S>
 void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, const float *alpha, const float *theta,
                     const float *eta, const float *m_initial, const float *s_initial, float *m_states,
                     float *s_states, float *y, int seq_len, int batch, int chunk_size) {
+    const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), nchunks = batch * nc;
     float *table = scratch(3, (size_t)nchunks * kTableFloats * sizeof(float));
     float *vecs = scratch(4, (size_t)nchunks * kVecFloats * sizeof(float));
@@ -395,7 +396,7 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
                   "dynamic LDS size");
         attr_set = true;
     }
-    if (failed()) return;
+    if (es.failed()) return;
     hipLaunchKernelGGL(cw_coef_kernel<HAS_S>, dim3(ceil_div(nchunks, 2)), dim3(256), 0, stream(), alpha, theta, eta,
                        table, vecs, seq_len, chunk_size, nc, nchunks);
     check_launch("cw_coef_kernel");

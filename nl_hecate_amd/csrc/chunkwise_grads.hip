@@ -605,6 +605,7 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid) {
+    const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     static bool attr_set = false;
     if (!attr_set) {
@@ -614,7 +615,7 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
         attr_set = true;
     }
-    if (failed()) return true;
+    if (es.failed()) return true;
     KernelTimer kt("cw_grads_bf16_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,

@@ -954,10 +954,11 @@ template <class TIn>
 void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const float *alpha, const float *theta,
                 const float *eta, const float *m_initial, const float *s_initial, float *m_states, float *s_states,
                 float *y, int seq_len, int d, int batch, int chunk_size, bool has_s) {
+    const ErrorScope es;
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
     const int nc = ceil_div(seq_len, chunk_size);
     Scratch sc = local_scratch(batch, nc);
-    if (failed()) return;
+    if (es.failed()) return;
     static bool attr_set = false;
     if (!attr_set) {
         const size_t lds = kOutFwdLds;
@@ -990,6 +991,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                  const float *eta, const float *m_states, const float *s_states, const float *d_y, float *d_k,
                  float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                  float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s) {
+    const ErrorScope es;
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
     const int nc = ceil_div(seq_len, chunk_size);
     Scratch sc{nullptr, nullptr};
@@ -1000,7 +1002,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     float *xs = scratch(7, (size_t)batch * nc * CW * CW * sizeof(float));
     float *pvec = scratch(8, (size_t)batch * seq_len * 4 * sizeof(float));
     float *scal = scratch(9, (size_t)batch * nc * 4 * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     static bool attr_set = false;
     if (!attr_set) {
         set_lds(cw_local_bwd_kernel<float>, kLocalBwdLds);
@@ -1017,7 +1019,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         float *tab_a = scratch(12, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *tab_b = scratch(13, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
-        if (failed()) return;
+        if (es.failed()) return;
         chunkwise_backward_coefficients(alpha, theta, eta, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s);
         chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_states, ds_states, seq_len, batch, chunk_size, has_s);
         chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec, xs,
@@ -1048,7 +1050,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
     const int per = 8, rows = ceil_div(batch, per);
     float *tmp = scratch(10, (size_t)rows * HD * HD * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     for (int which = 0; which < (has_s && d_s_initial ? 2 : 1); which++) {
         hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows), dim3(256), 0, stream(),
                            which ? ds_states : dm_states, tmp, batch, per, chain_stride);

@@ -603,11 +603,12 @@ void gate_backward_cuda(const float *d_alpha, const float *alpha, const float *d
                         const float *k_mem, const float *v_mem,
                         float *d_w_alpha, float *d_b_alpha, float *d_w_theta, float *d_b_theta,
                         float *d_w_eta, float *d_b_eta, int T, int D, int has_theta, int has_eta) {
+    const ErrorScope es;
     if (D <= 0) { fail("gate_backward_cuda: D=%d must be > 0.", D); return; }
     const int twoD = 2 * D;
     const int nblk = T > 0 ? ceil_div(T, kGateTok) : 0;
     float *part = scratch(10, (size_t)(nblk > 0 ? nblk : 1) * 3 * (twoD + 1) * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     if (nblk > 0) {
         hipLaunchKernelGGL(gate_backward_stage1, dim3(nblk), dim3(kEwThreads), 0, stream(), d_alpha, alpha,
                            d_theta, theta, d_eta, eta, k_mem, v_mem, part, T, D, has_theta, has_eta);

@@ -62,6 +62,7 @@ extern "C" void titans_fused_forward_f32_cuda(float *k_mem, const float *v_mem, 
                                               float *theta_out, float *eta_out, float *k_norms_out,
                                               float *q_norms_out, int seq_len, int d, int batch_size,
                                               float error_clip, float m_norm_max) {
+    const ErrorScope es;
     if (seq_len <= 0 || d <= 0 || batch_size <= 0) {
         fail("titans_fused_forward_f32_cuda: seq_len, d and batch_size must be positive");
         return;
@@ -74,7 +75,7 @@ extern "C" void titans_fused_forward_f32_cuda(float *k_mem, const float *v_mem, 
     gate_compute_cuda(k_mem, v_mem, w_theta, b_theta_ptr, theta_out, rows, d, 1);
     clamp_f32_cuda(theta_out, rows, theta_floor, theta_ceil);
     gate_compute_cuda(k_mem, v_mem, w_eta, b_eta_ptr, eta_out, rows, d, 0);
-    if (failed()) return;
+    if (es.failed()) return;
     titans_forward_f32_cuda(k_mem, v_mem, q_mem, alpha_out, theta_out, eta_out, m_initial, s_initial, m_states,
                             s_states, y, seq_len, d, batch_size, seq_len, d * d, error_clip, m_norm_max);
 }
@@ -85,6 +86,7 @@ extern "C" void dgd_fused_forward_f32_cuda(float *k_mem, const float *v_mem, flo
                                            const float *m_initial, float *m_states, float *y, float *alpha_out,
                                            float *theta_out, float *k_norms_out, float *q_norms_out, int seq_len,
                                            int d, int batch_size, float error_clip) {
+    const ErrorScope es;
     if (seq_len <= 0 || d <= 0 || batch_size <= 0) {
         fail("dgd_fused_forward_f32_cuda: seq_len, d and batch_size must be positive");
         return;
@@ -96,7 +98,7 @@ extern "C" void dgd_fused_forward_f32_cuda(float *k_mem, const float *v_mem, flo
     clamp_f32_cuda(alpha_out, rows, alpha_floor, alpha_ceil);
     gate_compute_cuda(k_mem, v_mem, w_theta, b_theta_ptr, theta_out, rows, d, 1);
     clamp_f32_cuda(theta_out, rows, theta_floor, theta_ceil);
-    if (failed()) return;
+    if (es.failed()) return;
     dgd_forward_f32_cuda(k_mem, v_mem, q_mem, alpha_out, theta_out, m_initial, m_states, y, seq_len, d, batch_size,
                          seq_len, d * d, error_clip);
 }

@@ -625,6 +625,7 @@ __global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, cons
 
 // d = 64 only; false if the shape is not covered (the caller falls back to the sweep kernel).
 bool launch_bwd_chunks(const HebBwdArgs &a, int batch) {
+    const ErrorScope es;
     const int seg = a.t_end - a.t_start;
     if (seg <= 0) return false;
     const int nch = (seg + kHC - 1) / kHC;
@@ -632,7 +633,7 @@ bool launch_bwd_chunks(const HebBwdArgs &a, int batch) {
     float *P = scratch(5, chunks * 4096 * sizeof(float));
     float *gamma = scratch(6, chunks * sizeof(float));
     float *S = scratch(7, chunks * 4096 * sizeof(float));
-    if (failed()) return true;
+    if (es.failed()) return true;
     hipLaunchKernelGGL(heb_chunk_seed_kernel, dim3((unsigned)chunks), dim3(256), 0, stream(), a, P, gamma, nch);
     check_launch("heb_chunk_seed_kernel");
     hipLaunchKernelGGL(heb_chunk_scan_kernel, dim3(16, batch), dim3(256), 0, stream(), P, gamma, a.d_m_seed, S,
@@ -699,12 +700,13 @@ __global__ __launch_bounds__(256) void heb_chunk_fwd_scan_kernel(const float *P,
 }
 
 bool launch_fwd_chunks(HebFwdArgs a, int batch) {
+    const ErrorScope es;
     const int nch = (a.seq_len + kHC - 1) / kHC;
     const size_t chunks = (size_t)batch * nch;
     float *P = scratch(5, chunks * 4096 * sizeof(float));
     float *gamma = scratch(6, chunks * sizeof(float));
     float *Mstart = scratch(7, chunks * 4096 * sizeof(float));
-    if (failed()) return true;
+    if (es.failed()) return true;
     hipLaunchKernelGGL(heb_chunk_fwd_seed_kernel, dim3((unsigned)chunks), dim3(256), 0, stream(), a, P, gamma, nch);
     check_launch("heb_chunk_fwd_seed_kernel");
     hipLaunchKernelGGL(heb_chunk_fwd_scan_kernel, dim3(16, batch), dim3(256), 0, stream(), P, gamma, a.m_initial,
@@ -716,6 +718,7 @@ bool launch_fwd_chunks(HebFwdArgs a, int batch) {
 }
 
 bool launch_bwd(HebBwdArgs a, int d, int batch) {
+    const ErrorScope es;
     if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) return false;
     if (d == 64 && launch_bwd_chunks(a, batch)) return true;
     a.rows = rows_per_workgroup(d, batch);
@@ -725,7 +728,7 @@ bool launch_bwd(HebBwdArgs a, int d, int batch) {
         a.ws_dq = scratch(2, n * d * sizeof(float));
         a.ws_dk = scratch(3, n * d * sizeof(float));
         a.ws_gate = scratch(4, n * 4 * sizeof(float));
-        if (failed()) return true;
+        if (es.failed()) return true;
     }
     switch (d) {
         case 8: launch_bwd_d<8>(a, batch); break;

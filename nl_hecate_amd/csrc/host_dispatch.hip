@@ -96,10 +96,11 @@ extern "C" void nlh_delta_forward_dispatch(const float *k_mem, const float *v_me
                                            const float *alpha, const float *theta, const float *m_initial,
                                            float *m_states, float *y, int seq_len, int d, float error_clip,
                                            float m_norm_max) {
+    const ErrorScope es;
     if (!positive("nlh_delta_forward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), th(seq_len), m0(dd), ms((seq_len + 1) * dd), yy(sd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem);
     al.from_host(alpha); th.from_host(theta); m0.from_host(m_initial);
     ms.zero(); yy.zero();
@@ -114,11 +115,12 @@ extern "C" void nlh_delta_backward_dispatch(const float *k_mem, const float *v_m
                                             const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
                                             float *d_alpha, float *d_theta, float *d_m_initial, int seq_len, int d,
                                             float error_clip) {
+    const ErrorScope es;
     if (!positive("nlh_delta_backward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), th(seq_len), ms((seq_len + 1) * dd), dy(sd);
     Staged<float> dk(sd), dv(sd), dq(sd), da(seq_len), dt(seq_len), dm(dd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem);
     al.from_host(alpha); th.from_host(theta); ms.from_host(m_states); dy.from_host(d_y);
     dk.zero(); dv.zero(); dq.zero(); da.zero(); dt.zero(); dm.zero();
@@ -135,11 +137,12 @@ extern "C" void nlh_titans_forward_dispatch(const float *k_mem, const float *v_m
                                             const float *m_initial, const float *s_initial, float *m_states,
                                             float *s_states, float *y, int seq_len, int d, float error_clip,
                                             float m_norm_max) {
+    const ErrorScope es;
     if (!positive("nlh_titans_forward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), th(seq_len), et(seq_len), m0(dd), s0(dd);
     Staged<float> ms((seq_len + 1) * dd), ss((seq_len + 1) * dd), yy(sd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem);
     al.from_host(alpha); th.from_host(theta); et.from_host(eta);
     m0.from_host(m_initial); s0.from_host(s_initial);
@@ -156,12 +159,13 @@ extern "C" void nlh_titans_backward_dispatch(const float *k_mem, const float *v_
                                              float *d_k_mem, float *d_v_mem, float *d_q_mem, float *d_alpha,
                                              float *d_theta, float *d_eta, float *d_m_initial, float *d_s_initial,
                                              int seq_len, int d, float error_clip) {
+    const ErrorScope es;
     if (!positive("nlh_titans_backward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), th(seq_len), et(seq_len);
     Staged<float> ms((seq_len + 1) * dd), ss((seq_len + 1) * dd), dy(sd);
     Staged<float> dk(sd), dv(sd), dq(sd), da(seq_len), dt(seq_len), de(seq_len), dm(dd), ds(dd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem);
     al.from_host(alpha); th.from_host(theta); et.from_host(eta);
     ms.from_host(m_states); ss.from_host(s_states); dy.from_host(d_y);
@@ -181,6 +185,7 @@ extern "C" void nlh_titans_backward_dispatch(const float *k_mem, const float *v_
 extern "C" void nlh_hebbian_forward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem,
                                              const float *alpha, const float *m_initial, float *m_states, float *y,
                                              int seq_len, int d, float m_norm_max) {
+    const ErrorScope es;
     if (!positive("nlh_hebbian_forward_dispatch", seq_len, d)) return;
     if (m_norm_max > 0.f && m_norm_max < 3.4028234e38f) {
         fail("nlh_hebbian_forward_dispatch: the Hebbian kernel has no norm clamp (m_norm_max=%g)", (double)m_norm_max);
@@ -188,7 +193,7 @@ extern "C" void nlh_hebbian_forward_dispatch(const float *k_mem, const float *v_
     }
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), m0(dd), ms((seq_len + 1) * dd), yy(sd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem); al.from_host(alpha); m0.from_host(m_initial);
     ms.zero(); yy.zero();
     hebbian_forward_f32_cuda(km.ptr, vm.ptr, qm.ptr, al.ptr, m0.ptr, ms.ptr, yy.ptr, seq_len, d, 1, seq_len, (int)dd);
@@ -200,11 +205,12 @@ extern "C" void nlh_hebbian_backward_dispatch(const float *k_mem, const float *v
                                               const float *alpha, const float *m_states, const float *d_y,
                                               float *d_k_mem, float *d_v_mem, float *d_q_mem, float *d_alpha,
                                               float *d_m_initial, int seq_len, int d) {
+    const ErrorScope es;
     if (!positive("nlh_hebbian_backward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), ms((seq_len + 1) * dd), dy(sd);
     Staged<float> dk(sd), dv(sd), dq(sd), da(seq_len), dm(dd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem); al.from_host(alpha);
     ms.from_host(m_states); dy.from_host(d_y);
     dk.zero(); dv.zero(); dq.zero(); da.zero(); dm.zero();
@@ -218,10 +224,11 @@ extern "C" void nlh_hebbian_backward_dispatch(const float *k_mem, const float *v
 extern "C" void nlh_dgd_forward_dispatch(const float *k_mem, const float *v_mem, const float *q_mem,
                                          const float *alpha, const float *theta, const float *m_initial,
                                          float *m_states, float *y, int seq_len, int d, float error_clip) {
+    const ErrorScope es;
     if (!positive("nlh_dgd_forward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), th(seq_len), m0(dd), ms((seq_len + 1) * dd), yy(sd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem);
     al.from_host(alpha); th.from_host(theta); m0.from_host(m_initial);
     ms.zero(); yy.zero();
@@ -236,11 +243,12 @@ extern "C" void nlh_dgd_backward_dispatch(const float *k_mem, const float *v_mem
                                           const float *d_y, float *d_k_mem, float *d_v_mem, float *d_q_mem,
                                           float *d_alpha, float *d_theta, float *d_m_initial, int seq_len, int d,
                                           float error_clip) {
+    const ErrorScope es;
     if (!positive("nlh_dgd_backward_dispatch", seq_len, d)) return;
     const size_t sd = (size_t)seq_len * d, dd = (size_t)d * d;
     Staged<float> km(sd), vm(sd), qm(sd), al(seq_len), th(seq_len), ms((seq_len + 1) * dd), dy(sd);
     Staged<float> dk(sd), dv(sd), dq(sd), da(seq_len), dt(seq_len), dm(dd);
-    if (failed()) return;
+    if (es.failed()) return;
     km.from_host(k_mem); vm.from_host(v_mem); qm.from_host(q_mem);
     al.from_host(alpha); th.from_host(theta); ms.from_host(m_states); dy.from_host(d_y);
     dk.zero(); dv.zero(); dq.zero(); da.zero(); dt.zero(); dm.zero();
@@ -257,11 +265,12 @@ extern "C" void nlh_dgd_backward_dispatch(const float *k_mem, const float *v_mem
 extern "C" void nlh_swa_forward_dispatch(const float *q, const float *k, const float *v, float *out,
                                          float *attn_weights, int seq_len, int num_heads, int head_dim,
                                          int window_size) {
+    const ErrorScope es;
     if (!positive("nlh_swa_forward_dispatch", seq_len, head_dim) || !swa_head_dim_ok("nlh_swa_forward_dispatch", head_dim))
         return;
     const size_t total = (size_t)seq_len * num_heads * head_dim, aw_total = (size_t)num_heads * seq_len * window_size;
     StagedBf16 dq(total), dk(total), dv(total), dout(total), daw(aw_total);
-    if (failed()) return;
+    if (es.failed()) return;
     dq.from_host_f32(q); dk.from_host_f32(k); dv.from_host_f32(v);
     dout.dev.zero(); daw.dev.zero();
     swa_forward_f32_cuda(dq.dev.ptr, dk.dev.ptr, dv.dev.ptr, dout.dev.ptr, daw.dev.ptr, seq_len, num_heads, head_dim,
@@ -274,12 +283,13 @@ extern "C" void nlh_swa_forward_dispatch(const float *q, const float *k, const f
 extern "C" void nlh_swa_backward_dispatch(const float *q, const float *k, const float *v, const float *attn_weights,
                                           const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len,
                                           int num_heads, int head_dim, int window_size) {
+    const ErrorScope es;
     if (!positive("nlh_swa_backward_dispatch", seq_len, head_dim) || !swa_head_dim_ok("nlh_swa_backward_dispatch", head_dim))
         return;
     const size_t total = (size_t)seq_len * num_heads * head_dim, aw_total = (size_t)num_heads * seq_len * window_size;
     StagedBf16 bq(total), bk(total), bv(total), baw(aw_total);
     Staged<float> dao(total), gq(total), gk(total), gv(total);
-    if (failed()) return;
+    if (es.failed()) return;
     bq.from_host_f32(q); bk.from_host_f32(k); bv.from_host_f32(v); baw.from_host_f32(attn_weights);
     dao.from_host(d_attn_out); gq.from_host(d_q); gk.from_host(d_k); gv.from_host(d_v);
     swa_backward_f32_cuda(bq.dev.ptr, bk.dev.ptr, bv.dev.ptr, baw.dev.ptr, dao.ptr, gq.ptr, gk.ptr, gv.ptr, seq_len,

@@ -622,6 +622,7 @@ static size_t bwd_partial_floats(int d, int batch, int seq_len, int rpl) {
 // ws == nullptr: partial sums come from the arena; otherwise from ws (bwd_partial_floats floats)
 template <bool HAS_S, bool FROZEN = false>
 static bool launch_bwd(BwdArgs a, int d, float *ws = nullptr, bool whole_chain = false) {
+    const ErrorScope es;
     const bool coupled = a.error_clip > 0.f;
     const int rpl = bwd_rpl(d, a.batch, coupled, whole_chain);
     a.parts = ceil_div(d, rows_per_wg(d, rpl));
@@ -637,7 +638,7 @@ static bool launch_bwd(BwdArgs a, int d, float *ws = nullptr, bool whole_chain =
             a.ws_dk = scratch(3, n * d * sizeof(float));
             a.ws_gate = scratch(4, n * 4 * sizeof(float));
         }
-        if (failed()) return true;
+        if (es.failed()) return true;
     }
     switch (d) {
         case 8: launch_bwd_c<8, 1, HAS_S, FROZEN>(a, coupled); break;
@@ -672,9 +673,10 @@ static __device__ __align__(256) float g_noalloc_scratch[kNoAllocFloats];
 static float *g_noalloc_ptr[kMaxDevices] = {nullptr};
 
 static float *noalloc_base() {
+    const ErrorScope es;
     int dev = 0;
     check_hip(hipGetDevice(&dev), "hipGetDevice");
-    if (failed()) return nullptr;
+    if (es.failed()) return nullptr;
     if (dev < 0 || dev >= kMaxDevices) { fail("device ordinal %d out of range", dev); return nullptr; }
     if (!g_noalloc_ptr[dev]) {
         float *p = nullptr;
@@ -721,6 +723,7 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
                                  float *d_m_initial, float *d_s_initial,
                                  int seq_len, int d, int batch, int C,
                                  float error_clip, float m_norm_max, const char *fn) {
+    const ErrorScope es;
     const size_t dd = (size_t)d * d;
     const int nck = n_ckpt_count(seq_len, C);
     const int max_seg = C < seq_len ? C : seq_len;
@@ -730,7 +733,7 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
     float *ly = scratch(7, (size_t)batch * max_seg * d * sizeof(float));
     float *seed_m = scratch(8, 2 * batch * dd * sizeof(float));
     float *seed_s = HAS_S ? scratch(9, 2 * batch * dd * sizeof(float)) : nullptr;
-    if (failed()) return;
+    if (es.failed()) return;
     // cleared by a kernel, not a memset node: the call stays replayable inside a captured graph
     const size_t nseed = (size_t)batch * dd;
     hipLaunchKernelGGL(zero_fill_kernel, dim3(ceil_div(nseed, 256)), dim3(256), 0, stream(), seed_m, nseed);
@@ -949,11 +952,12 @@ void titans_backward_f32_cuda(const float *k_mem, const float *v_mem, const floa
                               float *d_alpha, float *d_theta, float *d_eta,
                               float *d_m_initial, float *d_s_initial,
                               int seq_len, int d, int batch_size, float error_clip) {
+    const ErrorScope es;
     if (!check_dims("titans_backward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
     const size_t dd = (size_t)d * d;
     float *dm = scratch(0, (size_t)batch_size * dd * sizeof(float));
     float *ds = scratch(1, (size_t)batch_size * dd * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_states, s_states, d_y, nullptr, nullptr,
               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
               dm, ds, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
@@ -1001,10 +1005,11 @@ void delta_backward_f32_cuda(const float *k_mem, const float *v_mem, const float
                              float *d_k_mem, float *d_v_mem, float *d_q_mem,
                              float *d_alpha, float *d_theta, float *d_m_initial,
                              int seq_len, int d, int batch_size, float error_clip) {
+    const ErrorScope es;
     if (!check_dims("delta_backward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
     const size_t dd = (size_t)d * d;
     float *dm = scratch(0, (size_t)batch_size * dd * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     BwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_states, nullptr, d_y, nullptr, nullptr,
               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, nullptr, nullptr, nullptr, nullptr,
               dm, nullptr, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};

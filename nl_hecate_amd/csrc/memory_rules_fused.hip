@@ -351,6 +351,7 @@ static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q
                                   float *d_alpha, float *d_theta, float *d_eta,
                                   float *d_m_initial, float *d_s_initial,
                                   int seq_len, int d, int batch, int C) {
+    const ErrorScope es;
     if (C > C_MAX) return false;
     if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) return false;
     const size_t dd = (size_t)d * d;
@@ -366,7 +367,7 @@ static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q
         a.ws_dk = scratch(3, n * d * sizeof(float));
         a.ws_gate = scratch(4, n * 4 * sizeof(float));
     }
-    if (failed()) return true;
+    if (es.failed()) return true;
     switch (d) {
         case 8: launch_fused_d<8, HAS_S, FROZEN>(a); break;
         case 16: launch_fused_d<16, HAS_S, FROZEN>(a); break;

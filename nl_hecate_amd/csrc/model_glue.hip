@@ -344,6 +344,7 @@ void layer_norm_forward_cuda(const float *x, const float *gamma, const float *be
 
 void layer_norm_backward_cuda(const float *d_out, const float *x, const float *gamma, const float *mean_cache,
                               const float *rstd_cache, float *d_x, float *d_gamma, float *d_beta, int n, int d) {
+    const ErrorScope es;
     if (n <= 0 || d <= 0) return;
     const size_t lds = (size_t)(kThreads / 64) * 2 * d * sizeof(float);
     if (lds > 64 * 1024) {
@@ -352,7 +353,7 @@ void layer_norm_backward_cuda(const float *d_out, const float *x, const float *g
     }
     const int nblk = blocks_for(n, 64);   // some 64 rows per workgroup, at most 2048 partial rows
     float *part = scratch(5, (size_t)2 * nblk * d * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     hipLaunchKernelGGL(layer_norm_bwd_kernel, dim3(nblk), dim3(kThreads), lds, stream(), d_out, x,
                        gamma, mean_cache, rstd_cache, d_x, part, n, d);
     check_launch("layer_norm_bwd_kernel");
@@ -384,15 +385,16 @@ void transpose_copy_cuda(const float *src, float *dst, int rows, int cols) {
 }
 
 void cross_entropy_forward_cuda(const float *logits, const int *target_ids, float *loss_out, int seq_len, int vocab) {
+    const ErrorScope es;
     if (seq_len <= 0 || vocab <= 0) {   // the reference zeroes the loss before anything else
         float *z = scratch(5, sizeof(float));
-        if (failed()) return;
+        if (es.failed()) return;
         hipLaunchKernelGGL(sum_to_scalar_kernel, dim3(1), dim3(kThreads), 0, stream(), z, loss_out, 0);
         check_launch("sum_to_scalar_kernel");
         return;
     }
     float *nll = scratch(5, (size_t)seq_len * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     hipLaunchKernelGGL(cross_entropy_fwd_kernel, dim3(blocks_for(seq_len, 1)), dim3(kThreads), 0, stream(), logits,
                        target_ids, nll, seq_len, vocab);
     check_launch("cross_entropy_fwd_kernel");

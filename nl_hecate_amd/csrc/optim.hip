@@ -246,11 +246,12 @@ unsigned adamw_update_multi_rocm(float *const *w, const float *const *g, float *
                                  const int *n, const float *bc1_inv, const float *bc2_inv, int count,
                                  float lr, float beta1, float beta2, float eps, float weight_decay) {
     const AdamwHyper h{lr, beta1, beta2, eps, weight_decay};
+    // a batch is the next kMaxTensors input slots (empty ones skipped), so no tensor is seen twice
     for (int first = 0; first < count; first += kMaxTensors) {
         AdamwBatch b;
         b.count = 0;
         int blocks = 0;
-        for (int i = first; i < count && b.count < kMaxTensors; i++) {
+        for (int i = first; i < count && i < first + kMaxTensors; i++) {
             if (n[i] <= 0) continue;
             const int c = b.count++;
             b.w[c] = w[i]; b.g[c] = g[i]; b.m[c] = m[i]; b.v[c] = v[i]; b.n[c] = n[i];
@@ -310,11 +311,12 @@ unsigned grad_scale_conditional_cuda(float *g, const float *scale_ptr, int n) {
 
 unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, float max_grad_norm,
                                    float *out_norm, float *out_scale) {
+    const ErrorScope es;
     // pass 1: partial sums of every tensor into one scratch array
     long long total_blocks = 0;
     for (int i = 0; i < count; i++) total_blocks += n[i] > 0 ? (n[i] + 255) / 256 : 0;
     float *partial = scratch(11, (size_t)(total_blocks > 0 ? total_blocks : 1) * sizeof(float));
-    if (failed()) return 1;
+    if (es.failed()) return 1;
     int off = 0;
     for (int first = 0; first < count; first += kMaxTensors) {
         PtrBatch b;

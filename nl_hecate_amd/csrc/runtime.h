@@ -12,6 +12,14 @@ namespace nlh {
 // without launching, so callers and tests can observe argument errors.
 void fail(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 bool failed();          // an error was recorded since the last nlh_clear_error()
+// Errors recorded so far in this process.  An entry point that must stop after a failed argument
+// check, allocation or launch of its own opens an ErrorScope first and asks that: an error an earlier
+// call left behind (record mode keeps its message until nlh_clear_error) does not stop later calls.
+unsigned long long error_count();
+struct ErrorScope {
+    unsigned long long at = error_count();
+    bool failed() const { return error_count() != at; }
+};
 void check_hip(hipError_t e, const char *what);
 void check_launch(const char *kernel);
 
@@ -19,7 +27,11 @@ hipStream_t stream();   // launch stream (the null stream unless nlh_set_stream 
 
 // Scratch arena: one device allocation per slot, grown on demand, kept until
 // nlh_release_workspace().  Slots let one entry point hold several buffers.
-// Work on the launch stream is ordered, so reuse across calls is safe.
+// Work on the launch stream is ordered, so reuse across calls is safe; calls issued on different
+// streams (nlh_set_stream between them) share the slots and are NOT ordered against each other.
+// Growing a slot frees the old buffer and bumps the arena generation (nlh_workspace_generation):
+// a HIP graph captured earlier still holds the old address and must be dropped, not replayed.
+// While the launch stream is being captured a slot cannot grow: the call fails instead.
 float *scratch(int slot, size_t bytes);
 constexpr int kScratchSlots = 16;
 

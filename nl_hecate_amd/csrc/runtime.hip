@@ -20,6 +20,8 @@ static char g_kt_name[128] = {0};
 
 static int g_error_mode = 0;
 static bool g_failed = false;
+static unsigned long long g_error_count = 0;
+static unsigned long long g_arena_generation = 0;
 static char g_error[512] = "";
 static hipStream_t g_stream = nullptr;
 
@@ -36,6 +38,7 @@ void fail(const char *fmt, ...) {
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
     va_end(ap);
     g_failed = true;
+    g_error_count++;
     if (g_error_mode == 0) {
         fprintf(stderr, "[nl_hecate_rocm FATAL] %s\n", g_error);
         abort();
@@ -43,6 +46,7 @@ void fail(const char *fmt, ...) {
 }
 
 bool failed() { return g_failed; }
+unsigned long long error_count() { return g_error_count; }
 
 void check_hip(hipError_t e, const char *what) {
     if (e != hipSuccess) fail("%s: %s", what, hipGetErrorString(e));
@@ -63,18 +67,27 @@ float *scratch(int slot, size_t bytes) {
     int dev = 0;
     check_hip(hipGetDevice(&dev), "hipGetDevice");
     Slot &s = g_slots[slot];
-    if (s.ptr && (s.device != dev || s.bytes < bytes)) {
-        // Earlier launches may still read the old buffer.
+    if (s.ptr && s.device == dev && s.bytes >= bytes) return (float *)s.ptr;
+    // The slot has to be (re)allocated.  Not while the launch stream is being captured: hipMalloc,
+    // hipFree and the synchronisation below would invalidate the capture.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(g_stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) {
+        fail("scratch slot %d needs %zu bytes but holds %zu and the launch stream is being captured: run the "
+             "same call once before the capture", slot, bytes, s.ptr ? s.bytes : (size_t)0);
+        return nullptr;
+    }
+    if (s.ptr) {
+        // Earlier launches may still read the old buffer; graphs captured earlier keep its address.
         check_hip(hipDeviceSynchronize(), "scratch: hipDeviceSynchronize");
         check_hip(hipFree(s.ptr), "scratch: hipFree");
         s = Slot();
+        g_arena_generation++;
     }
-    if (!s.ptr) {
-        size_t want = bytes < 256 ? 256 : bytes;
-        check_hip(hipMalloc(&s.ptr, want), "scratch: hipMalloc");
-        s.bytes = want;
-        s.device = dev;
-    }
+    size_t want = bytes < 256 ? 256 : bytes;
+    check_hip(hipMalloc(&s.ptr, want), "scratch: hipMalloc");
+    if (!s.ptr) return nullptr;
+    s.bytes = want;
+    s.device = dev;
     return (float *)s.ptr;
 }
 
@@ -109,7 +122,10 @@ void nlh_clear_error(void) {
 
 void nlh_set_stream(void *hip_stream) { nlh::g_stream = (hipStream_t)hip_stream; }
 
+unsigned long long nlh_workspace_generation(void) { return nlh::g_arena_generation; }
+
 void nlh_release_workspace(void) {
+    nlh::g_arena_generation++;
     for (auto &s : nlh::g_slots) {
         if (s.ptr) {
             (void)hipDeviceSynchronize();

@@ -1216,6 +1216,7 @@ extern "C" void selfref_chunkwise_backward_f32_rocm(const float *embedded, const
                                                     const float *frozen, float *d_embedded, float *d_mems,
                                                     int seq_len, int d, int batch_size, int chunk_size,
                                                     int self_generated_values) {
+    const ErrorScope es;
     if (!check_args("selfref_chunkwise_backward_f32_rocm", seq_len, d, batch_size, chunk_size)) return;
     const int C = chunk_size > seq_len ? seq_len : chunk_size;
     const int nc = (seq_len + chunk_size - 1) / chunk_size;
@@ -1244,6 +1245,6 @@ extern "C" void selfref_chunkwise_backward_f32_rocm(const float *embedded, const
         a.csv = scratch(4, chunks * 2 * d * sizeof(float));
         a.dh = sg ? nullptr : scratch(5, tokens * d * sizeof(float));
     }
-    if (failed()) return;
+    if (es.failed()) return;
     if (d == 16) launch_bwd<16>(a); else if (d == 32) launch_bwd<32>(a); else launch_bwd<64>(a);
 }

@@ -348,6 +348,7 @@ void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t 
                            const uint16_t *attn_weights, const float *d_attn_out,
                            float *d_q, float *d_k, float *d_v, int seq_len, int num_heads, int head_dim,
                            int window_size, int batch_size, int n_persistent) {
+    const ErrorScope es;
     if (!swa_check("swa_backward_f32_cuda", seq_len, num_heads, head_dim, window_size, batch_size, n_persistent))
         return;
     if (swa_backward_mfma(q, k, v, attn_weights, d_attn_out, d_q, d_k, d_v, seq_len, num_heads, head_dim,
@@ -356,7 +357,7 @@ void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t 
     const long long nq = (long long)batch_size * num_heads * seq_len;
     const int aw = n_persistent + window_size;
     float *ds = scratch(0, (size_t)nq * aw * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     const size_t lds = (size_t)kSwaWaves * (((head_dim + 3) & ~3) + aw) * sizeof(float);
     const dim3 grid((unsigned)((nq + kSwaWaves - 1) / kSwaWaves)), blk(kSwaWaves * 64);
     hipLaunchKernelGGL(swa_backward_query_kernel, grid, blk, lds, stream(), k, v, attn_weights, d_attn_out,

@@ -640,9 +640,10 @@ namespace nlh {
 bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *attn_weights,
                        const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
                        int head_dim, int window, int batch, int n_persistent) {
+    const ErrorScope es;
     if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
     float *dvec = scratch(1, (size_t)batch * num_heads * seq_len * sizeof(float));
-    if (failed()) return true;
+    if (es.failed()) return true;
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
     hipLaunchKernelGGL(swa_bwd_q_mfma_kernel, grid, dim3(256), 0, stream(), k, v, attn_weights, d_attn_out, d_q, dvec,
                        seq_len, num_heads, window);

@@ -113,13 +113,14 @@ void swiglu_backward_f32_cuda_dd(const float *d_y, const float *x, const float *
                                  const float *down_proj, const float *fused_buf, const float *gate_buf,
                                  const float *up_buf, const float *cache_buf, float *d_x, float *d_gate_proj,
                                  float *d_up_proj, float *d_down_proj, int seq_len, int d_model, int intermediate) {
+    const ErrorScope es;
     if (!dims_ok("swiglu_backward_f32_cuda_dd", seq_len, d_model, intermediate)) return;
     const rocblas_operation N = rocblas_operation_none, T = rocblas_operation_transpose;
     const size_t n = (size_t)seq_len * intermediate;
     float *d_fused = scratch(6, n * sizeof(float));
     float *d_gate = scratch(7, n * sizeof(float));
     float *d_up = scratch(8, n * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     // d_fused = dY Wd;  d_Wd = dY^T fused
     if (!gemm("d_fused", N, N, intermediate, seq_len, d_model, down_proj, intermediate, d_y, d_model, 0.f, d_fused, intermediate)) return;
     if (!gemm("d_down_proj", N, T, intermediate, d_model, seq_len, fused_buf, intermediate, d_y, d_model, 0.f, d_down_proj, intermediate)) return;

@@ -436,6 +436,7 @@ __global__ __launch_bounds__(kMlpThreads) void miras_mlp_bwd_kernel(MirasArgs a,
 
 void miras_forward(const char *fn, MirasArgs a, const float *w1_initial, const float *w2_initial, float *w1_states,
                    float *w2_states, float *y) {
+    const ErrorScope es;
     if (a.d <= 0 || a.dh <= 0) { fail("%s: d=%d, d_hidden=%d must be > 0.", fn, a.d, a.dh); return; }
     if (a.seq_len < 0) { fail("%s: seq_len=%d must be >= 0.", fn, a.seq_len); return; }
     const size_t lds = (size_t)(2 * a.d + 3 * a.dh + kMlpWaves) * sizeof(float);
@@ -445,7 +446,7 @@ void miras_forward(const char *fn, MirasArgs a, const float *w1_initial, const f
         const size_t bytes = (size_t)a.dh * a.d * sizeof(float);
         a1 = scratch(6, bytes);
         a2 = scratch(7, bytes);
-        if (failed()) return;
+        if (es.failed()) return;
     }
     hipLaunchKernelGGL(miras_mlp_fwd_kernel, dim3(1), dim3(kMlpThreads), lds, stream(), a, w1_initial, w2_initial,
                        w1_states, w2_states, y, a1, a2);
@@ -455,13 +456,14 @@ void miras_forward(const char *fn, MirasArgs a, const float *w1_initial, const f
 void miras_backward(const char *fn, MirasArgs a, const float *w1_states, const float *w2_states, const float *d_y,
                     float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_w1_initial,
                     float *d_w2_initial) {
+    const ErrorScope es;
     if (a.d <= 0 || a.dh <= 0) { fail("%s: d=%d, d_hidden=%d must be > 0.", fn, a.d, a.dh); return; }
     if (a.seq_len < 0) { fail("%s: seq_len=%d must be >= 0.", fn, a.seq_len); return; }
     const size_t lds = (size_t)(5 * a.d + 5 * a.dh + kMlpWaves) * sizeof(float);
     if (lds > 64 * 1024) { fail("%s: d=%d d_hidden=%d need %zu bytes of LDS (limit 65536).", fn, a.d, a.dh, lds); return; }
     const size_t bytes = (size_t)a.dh * a.d * sizeof(float);
     float *dW1 = scratch(6, bytes), *dW2 = scratch(7, bytes);
-    if (failed()) return;
+    if (es.failed()) return;
     hipLaunchKernelGGL(miras_mlp_bwd_kernel, dim3(1), dim3(kMlpThreads), lds, stream(), a, w1_states, w2_states, d_y,
                        d_k, d_v, d_q, d_alpha, d_theta, d_w1_initial, d_w2_initial, dW1, dW2);
     check_launch("miras_mlp_bwd_kernel");
@@ -500,6 +502,7 @@ void titans_mlp_backward_f32_cuda(const float *k_mem, const float *v_mem, const 
                                   float *d_theta, float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len,
                                   int d, int d_hidden, int batch_size, int input_stride, int m_stride, int activation,
                                   float m_norm_max) {
+    const ErrorScope es;
     (void)m_norm_max;   // the projection is the identity in the backward (titans_mlp_backward.cu: no use either)
     if (!mlp_args_ok("titans_mlp_backward_f32_cuda", seq_len, d, d_hidden, batch_size, activation) || batch_size == 0) return;
     const size_t lds = (size_t)(4 * d + 5 * d_hidden + kMlpWaves) * sizeof(float);
@@ -507,7 +510,7 @@ void titans_mlp_backward_f32_cuda(const float *k_mem, const float *v_mem, const 
     const size_t n = MlpDims{d, d_hidden}.n();
     float *dM = scratch(6, (size_t)batch_size * n * sizeof(float));
     float *dS = scratch(7, (size_t)batch_size * n * sizeof(float));
-    if (failed()) return;
+    if (es.failed()) return;
     const MlpBwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_states, s_states, d_y, d_k_mem, d_v_mem, d_q_mem,
                        d_alpha, d_theta, d_eta, dM, dS, seq_len, d, d_hidden, input_stride, m_stride, activation};
     hipLaunchKernelGGL(titans_mlp_bwd_kernel, dim3(batch_size), dim3(kMlpThreads), lds, stream(), a);

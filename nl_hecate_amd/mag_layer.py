@@ -439,6 +439,32 @@ class MagLayer:
         return d_x.view(bs, s, d), grads
 
 
+class GraphCache:
+    """Captured graphs keyed by (pulse pattern, shape), valid for one generation of the library's
+    scratch arena: a graph holds the scratch addresses of the calls it recorded, and when a slot has
+    been reallocated since (a larger shape, nlh_release_workspace) those addresses are dead, so every
+    cached graph is dropped and captured again rather than replayed."""
+
+    def __init__(self, generation_fn):
+        self._gen_fn, self._gen, self._graphs = generation_fn, None, {}
+
+    def get(self, key):
+        if self._gen != self._gen_fn():
+            self._graphs.clear()
+        return self._graphs.get(key)
+
+    def put(self, key, value):
+        """Call after the capture: the generation that the captured addresses belong to is read here."""
+        gen = self._gen_fn()
+        if self._gen != gen:
+            self._graphs.clear()
+            self._gen = gen
+        self._graphs[key] = value
+
+    def __len__(self):
+        return len(self._graphs)
+
+
 class MagTrainer:
     """forward + backward + frequency-aware AdamW step (core/src/gpu_optimizer.rs:403-515)."""
 
@@ -455,7 +481,10 @@ class MagTrainer:
         for grp, w, g in zip(groups, p.tensors(), self.grads.tensors()):
             m, v = torch.zeros_like(w), torch.zeros_like(w)
             self.state.append((m, v))
-            self.opt.add_tensor(grp, w, g, m, v)
+            tid = self.opt.add_tensor(grp, w, g, m, v)
+            # b_theta is held in [-10, 2] after every level update (gpu_optimizer.rs:491-493)
+            if grp >= 0 and any(w is lp.b_theta for lp in p.levels):
+                self.opt.set_clamp(tid, -10.0, 2.0)
         self.scale = torch.zeros(2, dtype=torch.float32, device="cuda")
 
     def _forward_backward(self, x, d_out):
@@ -474,8 +503,9 @@ class MagTrainer:
         layer.conductor.set_seq_len(x.shape[1])
         pulse = layer.conductor.pulse()
         key = (tuple(bool(a) for a in pulse.active_levels), tuple(x.shape))
-        graphs = self.__dict__.setdefault("_graphs", {})
-        if key not in graphs:
+        graphs = self.__dict__.setdefault("_graphs", GraphCache(lib.nlh_workspace_generation))
+        entry = graphs.get(key)
+        if entry is None:
             xs, ds = x.clone(), d_out.clone()
             # Warm-up on a side stream sizes every scratch buffer (nothing may allocate while a graph
             # is captured); it advances the context memories, which are put back afterwards.
@@ -494,8 +524,9 @@ class MagTrainer:
                 lib.nlh_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
                 out = self._forward_backward(xs, ds)
             lib.nlh_set_stream(None)
-            graphs[key] = (graph, xs, ds, out)
-        graph, xs, ds, out = graphs[key]
+            entry = (graph, xs, ds, out)
+            graphs.put(key, entry)
+        graph, xs, ds, out = entry
         xs.copy_(x)
         ds.copy_(d_out)
         graph.replay()

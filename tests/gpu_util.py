@@ -52,9 +52,20 @@ def rel_err(got, want):
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
 
 
+def l2_rel_err(got, want):
+    """||got - want||_2 / ||want||_2: a tensor whose small entries are all wrong fails this one even
+    when a few large entries keep the max-norm figure low."""
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    return float(np.sqrt(np.sum((got - want) ** 2)) / max(np.sqrt(np.sum(want ** 2)), 1e-30))
+
+
 def assert_close(name, got, want, tol=REL_TOL_F32):
+    """Both figures must hold: max|a-b| / max|b| and ||a-b||_2 / ||b||_2."""
     e = rel_err(got, want)
     assert e <= tol, f"{name}: rel err {e:.3e} > {tol:.0e}"
+    e2 = l2_rel_err(got, want)
+    assert e2 <= tol, f"{name}: L2-relative err {e2:.3e} > {tol:.0e}"
     return e
 
 

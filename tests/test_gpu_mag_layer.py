@@ -109,6 +109,23 @@ def test_training_step_changes_only_active_levels():
     assert tr.opt.level_step(0) == 2 and tr.opt.level_step(1) == 1
 
 
+def test_trainer_clamps_b_theta_after_every_level_update():
+    """gpu_optimizer.rs:491-493: b_theta of an updated level is held in [-10, 2]."""
+    d, nh, k = 32, 2, 2
+    layer = MagLayer(d, nh, k, 4, [1, 8], rule="exact", chunk=4, seed=12)
+    with torch.no_grad():
+        layer.p.levels[0].b_theta.fill_(7.5)
+        layer.p.levels[1].b_theta.fill_(-30.0)
+    tr = MagTrainer(layer)
+    x = (torch.randn(1, 6, d, generator=torch.Generator().manual_seed(1)) / math.sqrt(d)).cuda()
+    tr.step(x, lambda out: torch.ones_like(out))
+    torch.cuda.synchronize()
+    assert float(layer.p.levels[0].b_theta.max()) <= 2.0
+    assert float(layer.p.levels[1].b_theta.min()) >= -10.0
+    for lp in layer.p.levels:   # the other biases are not clamped
+        assert torch.isfinite(lp.b_alpha).all() and torch.isfinite(lp.b_eta).all()
+
+
 def test_graph_replayed_steps_match_eager_steps():
     """Three training steps from a captured HIP graph (forward + backward replayed, optimizer eager)
     against three eager steps from the same start, with different inputs per step and eager work on
