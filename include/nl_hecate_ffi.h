@@ -51,6 +51,11 @@ int nlh_kernel_timer_enable(int on);
 float nlh_kernel_timer_read_ms(int *launches, char *name, int name_len);
 /* Runs the cross-lane primitives on known data; returns 0 when all agree. */
 int nlh_selftest_lane_ops(void);
+/* Gate coefficients of one chunk (L <= 64 device-resident gates each) from the in-kernel generator:
+ * tj, jt [3][64][64] = c, bb, r indexed [t][j] from the two tile orders; vecs [9][64] = a, beta, h,
+ * cl, bl, rl, keep, eta, theta, then a_L, beta_L, h_L.  0 on success.  For tests. */
+int nlh_selftest_chunk_coef(const float *alpha, const float *theta, const float *eta, int L, float *tj,
+                            float *jt, float *vecs);
 
 /* ── Titans LMM, exact per-token rule ───────────────────────────────────────
  * Per token: e = clip(M k - v); S = eta S - theta e k^T; M = (1-alpha) M + S;

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "../../include/nl_hecate_ffi.h"
+#include "chunk_coef.h"
 #include "lane_ops.h"
 #include "runtime.h"
 
@@ -120,4 +121,39 @@ extern "C" int nlh_selftest_lane_ops(void) {
         bad += nb;
     }
     return bad;
+}
+
+namespace nlh {
+// c, bb, r of one chunk from both tile generators, as dense [kind][t][j] tables, and the vectors.
+__global__ void chunk_coef_kernel(const float *alpha, const float *theta, const float *eta, int L, float *tj,
+                                  float *jt, float *vecs) {
+    __shared__ ChunkCoef cc;
+    const int l = threadIdx.x, g = l >> 4, c16 = l & 15;
+    coef_scan(cc, alpha[l], theta[l], eta[l], L);
+    __syncthreads();
+    for (int T = 0; T < 4; T++)
+        for (int J = 0; J < 4; J++) {
+            const cf32x4 a[3] = {coef_tile_tj<COEF_C>(cc, T, J, L), coef_tile_tj<COEF_BB>(cc, T, J, L),
+                                 coef_tile_tj<COEF_R>(cc, T, J, L)};
+            const cf32x4 b[3] = {coef_tile_jt<COEF_C>(cc, J, T, L), coef_tile_jt<COEF_BB>(cc, J, T, L),
+                                 coef_tile_jt<COEF_R>(cc, J, T, L)};
+            for (int kd = 0; kd < 3; kd++)
+                for (int i = 0; i < 4; i++) {
+                    tj[(kd * 64 + 16 * T + 4 * g + i) * 64 + 16 * J + c16] = a[kd][i];
+                    jt[(kd * 64 + 16 * T + c16) * 64 + 16 * J + 4 * g + i] = b[kd][i];
+                }
+        }
+    const float *src[9] = {cc.a, cc.beta, cc.h, cc.cl, cc.bl, cc.rl, cc.keep, cc.eta, cc.th};
+    for (int v = 0; v < 9; v++) vecs[v * 64 + l] = src[v][l];
+    if (l < 3) vecs[9 * 64 + l] = cc.last[l];
+}
+}  // namespace nlh
+
+// tj, jt: [3][64][64] (c, bb, r indexed [t][j]); vecs: [9][64] a, beta, h, cl, bl, rl, keep, eta, theta, then a_L, beta_L, h_L
+extern "C" int nlh_selftest_chunk_coef(const float *alpha, const float *theta, const float *eta, int L, float *tj,
+                                       float *jt, float *vecs) {
+    using namespace nlh;
+    if (L < 1 || L > 64) return -1;
+    hipLaunchKernelGGL(chunk_coef_kernel, dim3(1), dim3(64), 0, stream(), alpha, theta, eta, L, tj, jt, vecs);
+    return hipGetLastError() == hipSuccess ? 0 : -2;
 }
