@@ -1,0 +1,142 @@
+// Backward of the frozen-M0 chunkwise Titans / Delta rule: the gate gradients d_alpha, d_eta.
+//
+//   d_alpha_s = -<M_(s-1), A_s>,   d_eta_s = <S_(s-1), B_s>
+// with A_s, B_s the adjoints of M_s, S_s inside the chunk (core/kernels/titans_chunkwise_backward.cu:
+// 118-358 accumulates the same inner products token by token on full d x d matrices):
+//   A_s = sum_(t >= s) r[s][t] dy_t q_t^T + r[s][L-1] dMo
+//   B_s = sum_(t >= s) c[t][s] dy_t q_t^T + c[L-1][s] dMo + bb[s][L-1] dSo
+// Every inner product of a state with a rank-1 term is a scalar that obeys the rule's own recurrence:
+// with u_s(t) = <M_s, dy_t q_t^T>, v_s(t) = <S_s, dy_t q_t^T>,
+//   v_s(t) = eta_s v_(s-1)(t) + xs[s][t],   u_s(t) = keep_s u_(s-1)(t) + v_s(t),   u_(-1) = p0[t], v_(-1) = ps[t]
+// where xs[s][t] = -theta_s (dy_t . e_s)(q_t . k_s) and p0, ps come from the gradient pass; the same holds
+// for <M_s, dMo>, <S_s, dMo>, <S_s, dSo> with -theta_s e_s^T dMo k_s and -theta_s e_s^T dSo k_s as the
+// per-token terms.  The weights r, c, bb obey forward recurrences in t.  So a chunk costs two sweeps of
+// 64 steps on ONE wave and no matrix product, no coefficient table and no division:
+//   sweep 1 (lane = t): u, v for s = 0..63, parked in LDS as rows s + 1
+//   sweep 2 (lane = s): the weighted sums over t >= s with the weights advanced step by step.
+// Gates travel as wave-uniform values (v_readlane); tokens beyond a short chunk carry keep = 1, eta = 0
+// and zero terms.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "chunkwise_grads.h"
+#include "runtime.h"
+
+namespace nlh {
+namespace {
+
+constexpr int GW = 64;            // tokens per chunk tile
+constexpr int GLD = 65;           // LDS row stride (floats): rows and columns conflict-free
+constexpr int kGateWaves = 4;     // chunks per workgroup, one wave each
+
+__device__ __forceinline__ float bcast(float x, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+
+template <bool HAS_S>
+__global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
+    const float *__restrict__ alpha, const float *__restrict__ eta, const float *__restrict__ pvec,
+    const float *__restrict__ xs, const float *__restrict__ scal, float *__restrict__ d_alpha,
+    float *__restrict__ d_eta, int s, int C, int nc, int ntask) {
+    extern __shared__ float smem[];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int task = blockIdx.x * kGateWaves + wv;
+    if (task >= ntask) return;   // no barrier below: waves are independent
+    float *U = smem + (size_t)wv * (HAS_S ? 2 : 1) * GW * GLD, *V = U + GW * GLD;
+    const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0;
+    const bool in = lane < L;
+    const float keep_l = in ? 1.f - alpha[tok + lane] : 1.f;
+    const float eta_l = (HAS_S && in) ? eta[tok + lane] : 0.f;
+    const float4 pv = in ? *reinterpret_cast<const float4 *>(pvec + (tok + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    const float m0dm = scal[(size_t)task * 4 + 0], s0dm = scal[(size_t)task * 4 + 1], s0ds = scal[(size_t)task * 4 + 2];
+    const float *x = xs + (size_t)task * GW * GW + lane;
+
+    // ── sweep 1: lane = t ──
+    float u = pv.x, v = pv.y;              // <M_s, dy_t q_t^T>, <S_s, dy_t q_t^T>
+    float um = m0dm, vm = s0dm, vs = s0ds; // <M_s, dMo>, <S_s, dMo>, <S_s, dSo> (wave-uniform)
+    float pum = um, pvm = vm, pvs = vs;    // their values at s = lane - 1
+    U[lane] = u;
+    if (HAS_S) V[lane] = v;
+    constexpr int PF = GW;                 // the whole column of per-token terms is requested up front
+    float xr[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) xr[i] = x[i * GW];
+#pragma unroll
+    for (int sx = 0; sx < GW; sx++) {
+        const float xv = xr[sx % PF];
+        if (sx + PF < GW) xr[sx % PF] = x[(sx + PF) * GW];
+        const float kp = bcast(keep_l, sx), g1 = bcast(pv.z, sx);
+        if (HAS_S) {
+            const float et = bcast(eta_l, sx), g2 = bcast(pv.w, sx);
+            v = fmaf(et, v, xv);
+            vm = fmaf(et, vm, g1);
+            vs = fmaf(et, vs, g2);
+        } else {
+            v = xv;
+            vm = g1;
+        }
+        u = fmaf(kp, u, v);
+        um = fmaf(kp, um, vm);
+        if (sx + 1 < GW) {
+            U[(sx + 1) * GLD + lane] = u;
+            if (HAS_S) V[(sx + 1) * GLD + lane] = v;
+            if (lane == sx + 1) { pum = um; pvm = vm; pvs = vs; }
+        }
+    }
+    // the rows are read back by other lanes of the same wave
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ── sweep 2: lane = s; weights r[s][t], c[t][s], bb[s][t] advance with t ──
+    float rho = 1.f, cc = 1.f, bb = 1.f, accA = 0.f, accE = 0.f;
+    const float *Ur = U + lane * GLD, *Vr = V + lane * GLD;
+#pragma unroll
+    for (int t = 0; t < GW; t++) {
+        const float kp = bcast(keep_l, t);
+        const bool after = t > lane && t < L, on = t >= lane;   // tokens beyond a short chunk change no weight
+        rho *= after ? kp : 1.f;
+        accA = fmaf(on ? rho : 0.f, Ur[t], accA);
+        if (HAS_S) {
+            const float et = bcast(eta_l, t);
+            bb *= after ? et : 1.f;
+            cc = after ? fmaf(kp, cc, bb) : cc;
+            accE = fmaf(on ? cc : 0.f, Vr[t], accE);
+        }
+    }
+    if (in) {
+        d_alpha[tok + lane] = -fmaf(rho, pum, accA);
+        if (HAS_S) d_eta[tok + lane] = accE + cc * pvm + bb * pvs;
+    }
+}
+
+}  // namespace
+
+void chunkwise_gate_gradients(const float *alpha, const float *eta, const float *pvec, const float *xs,
+                              const float *scal, float *d_alpha, float *d_eta, int seq_len, int batch,
+                              int chunk_size, bool has_s) {
+    const ErrorScope es;
+    const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
+    const size_t lds = (size_t)kGateWaves * (has_s ? 2 : 1) * GW * GLD * sizeof(float);
+    static bool attr_set = false;
+    if (!attr_set) {
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_gates_sweep_kernel<true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kGateWaves * 2 * GW * GLD * 4)),
+                  "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_gates_sweep_kernel<false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kGateWaves * GW * GLD * 4)),
+                  "dynamic LDS size");
+        attr_set = true;
+    }
+    if (es.failed()) return;
+    const dim3 grid(ceil_div(ntask, kGateWaves)), block(64 * kGateWaves);
+    if (has_s)
+        hipLaunchKernelGGL(cw_gates_sweep_kernel<true>, grid, block, lds, stream(), alpha, eta, pvec, xs, scal, d_alpha,
+                           d_eta, seq_len, chunk_size, nc, ntask);
+    else
+        hipLaunchKernelGGL(cw_gates_sweep_kernel<false>, grid, block, lds, stream(), alpha, nullptr, pvec, xs, scal,
+                           d_alpha, nullptr, seq_len, chunk_size, nc, ntask);
+    check_launch("cw_gates_sweep_kernel");
+}
+
+}  // namespace nlh

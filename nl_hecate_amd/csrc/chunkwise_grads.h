@@ -4,8 +4,10 @@
 //     chunk) and vectors vecs (vec_floats per chunk) from the gates
 //   chunkwise_adjoint_bf16: the adjoint scan; dm_states / ds_states [batch][num_chunks + 1][64*64],
 //     slot c = adjoint of the state at the start of chunk c
-//   chunkwise_grads_bf16: d_q, d_k, d_v, d_theta, and for the gate pass pvec [token][4], xs
-//     [chunk][64*64] in accumulator-tile order, scal [chunk][4]
+//   chunkwise_grads_bf16: d_q, d_k, d_v, d_theta, and for the gate pass
+//     pvec [token][4] = p0_t = dy_t^T M0 q_t, ps_t = dy_t^T S0 q_t, -theta_t e_t^T dMo k_t, -theta_t e_t^T dSo k_t
+//     xs [chunk][j][t] = -theta_j (dy_t . e_j)(q_t . k_j)      scal [chunk][4] = <M0,dMo>, <S0,dMo>, <S0,dSo>
+//   chunkwise_gate_gradients: d_alpha, d_eta from those (chunkwise_gates.hip; also serves the fp32 path)
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -27,5 +29,9 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid);
+
+void chunkwise_gate_gradients(const float *alpha, const float *eta, const float *pvec, const float *xs,
+                              const float *scal, float *d_alpha, float *d_eta, int seq_len, int batch,
+                              int chunk_size, bool has_s);
 
 }  // namespace nlh

@@ -381,8 +381,9 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int rt = 0; rt < 2; rt++)
 #pragma unroll
                     for (int ct = 0; ct < 2; ct++) {
-                        *reinterpret_cast<f32x4 *>(xo + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4) = rr[rt][ct] * keep[rt][ct];
                         const int off = (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g;   // [j][t .. t+3]
+                        *reinterpret_cast<f32x4 *>(xo + (bn + 16 * ct + r16) * CW + bm + 16 * rt + 4 * g) =
+                            -cvec[4 * CW + bn + 16 * ct + r16] * (rr[rt][ct] * keep[rt][ct]);
                         bf16_store(CPt, off, ntab[rt][ct] * keep[rt][ct]);
                         bf16_store(CRt, off, ntab[rt][ct] * rr[rt][ct]);
                     }
@@ -570,9 +571,10 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
         } else if (tid < L) {
             const int t = tid;
             d_theta[tok + t] = -(part[(2 * 2) * CW + t] + part[(2 * 2 + 1) * CW + t]);
+            const float nth = -cvec[4 * CW + t];
             *reinterpret_cast<f32x4 *>(pvec + (tok + t) * 4) =
                 f32x4{part[t] + part[CW + t], part[2 * CW + t] + part[3 * CW + t],
-                      part[6 * CW + t] + part[7 * CW + t], part[8 * CW + t] + part[9 * CW + t]};
+                      nth * (part[6 * CW + t] + part[7 * CW + t]), nth * (part[8 * CW + t] + part[9 * CW + t])};
         } else if (tid >= 64 && tid < 67) {
             const float *p = dots + 8 * (tid - 64);
             scal[(size_t)task * 4 + (tid - 64)] = p[0] + p[1] + p[2] + p[3] + p[4] + p[5] + p[6] + p[7];

@@ -581,7 +581,7 @@ __global__ __launch_bounds__(256) void cw_state_dots_kernel(const float *__restr
 }
 
 // ── backward, main per-chunk pass: dQ, dK, dV, dtheta; exports for the gate pass ──
-//   pvec [chain][token][4] = p0, ps, g1, g2   xs [chain][chunk][64][64] = X[t][j] = (dy_t.e_j)(q_t.k_j)
+//   pvec [chain][token][4] = p0, ps, -theta g1, -theta g2   xs [chain][chunk][j][t] = -theta_j (dy_t.e_j)(q_t.k_j)
 template <class TIn>
 __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     const TIn *__restrict__ k, const TIn *__restrict__ v, const TIn *__restrict__ q, const float *__restrict__ d_y,
@@ -679,7 +679,7 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
             for (int i = 0; i < 4; i++) {
                 const int row = m0 + row_of(i), col = n0 + 16 * tl + (threadIdx.x & 15);
                 const float c = Cc[row * LDM + col], pv = p.t[tl][i], rv = r.t[tl][i];
-                xo[row * CW + col] = rv * pv;
+                xo[col * CW + row] = -cf.th[col] * rv * pv;   // [j][t], scaled for the gate pass
                 CP[row * LDM + col] = c * pv;
                 CR[row * LDM + col] = c * rv;
             }
@@ -755,149 +755,12 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
         float *pv = pvec + (tok + t) * 4;
         pv[0] = part[0][0][t] + part[0][1][t];
         pv[1] = part[1][0][t] + part[1][1][t];
-        pv[2] = part[3][0][t] + part[3][1][t];
-        pv[3] = part[4][0][t] + part[4][1][t];
+        pv[2] = -cf.th[t] * (part[3][0][t] + part[3][1][t]);
+        pv[3] = -cf.th[t] * (part[4][0][t] + part[4][1][t]);
     }
     }
 }
 constexpr size_t kGradsBwdLds = 9 * MAT * sizeof(float);
-
-// ── backward, gate pass: d_alpha, d_eta of one chunk ────────────────────────
-//   d_alpha_t = -<M_{t-1}, A_t>,  d_eta_t = <S_{t-1}, B_t>  with A, B the adjoints of M_t, S_t:
-//   <M_tau, dy_t' q_t'^T> = a_tau p0[t'] + beta_tau ps[t'] + sum_j W[tau][j] X[t'][j]
-//   <S_tau, dy_t' q_t'^T> = h_tau ps[t'] + sum_j Ws[tau][j] X[t'][j],  Ws[tau][j] = -theta_j bb[j][tau]
-//   and the same with dMo / dSo in place of dy q^T (g1, g2 and the three state dots).
-__global__ __launch_bounds__(kThr, 4) void cw_gates_bwd_kernel(const float *__restrict__ alpha,
-                                                            const float *__restrict__ theta,
-                                                            const float *__restrict__ eta,
-                                                            const float *__restrict__ pvec,
-                                                            const float *__restrict__ xs,
-                                                            const float *__restrict__ scal,
-                                                            float *__restrict__ d_alpha, float *__restrict__ d_eta,
-                                                            int s, int C, int nc, int has_s, int xs_tiled, int ntask) {
-    extern __shared__ float smem[];
-    float *Xs = smem, *Cc = Xs + MAT, *Bb = Cc + MAT, *Rr = Bb + MAT;   // Xs[t'][j] = -theta_j X[t'][j]
-    __shared__ Coef cf;
-    __shared__ float p0[CW], ps[CW], g1[CW], g2[CW], um[CW], usm[CW], uss[CW];   // g1, g2 scaled by -theta_j
-    __shared__ float part[2][2][CW];
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    // Persistent over chunk tasks; the small inputs of the next task are fetched into registers
-    // while the current one computes.
-    // xs is row-major [t][j], or (xs_tiled) in the accumulator-tile order of the bf16 pass:
-    // [block bi][rt][ct][lane][r] holds X[32 (bi/2) + 16 rt + 4 (lane/16) + r][32 (bi%2) + 16 ct + lane%16]
-    Tile<float> tx;
-    Gates gt;
-    float4 pv;
-    float sc0 = 0.f, sc1 = 0.f, sc2 = 0.f;
-    auto fetch_task = [&](int task) {
-        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
-        const size_t tok = (size_t)chain * s + t0;
-        fetch(tx, xs + (size_t)task * CW * CW, 64);
-        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        pv = *reinterpret_cast<const float4 *>(pvec + (tok + min(lane, L - 1)) * 4);
-        sc0 = scal[(size_t)task * 4 + 0]; sc1 = scal[(size_t)task * 4 + 1]; sc2 = scal[(size_t)task * 4 + 2];
-    };
-    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per,
-              task_hi = min(ntask, task_lo + per);
-    if (task_lo >= task_hi) return;
-    fetch_task(task_lo);
-    for (int task = task_lo; task < task_hi; task++) {
-    const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0;
-    const float m0dm = sc0, s0dm = sc1, s0ds = sc2;
-    load_gates(cf, gt);
-    if (wv == 4) {
-        const bool in = lane < L;
-        p0[lane] = in ? pv.x : 0.f; ps[lane] = in ? pv.y : 0.f;
-        g1[lane] = in ? -gt.th * pv.z : 0.f; g2[lane] = in ? -gt.th * pv.w : 0.f;
-    }
-    coefficients(cf, gt, L, Cc, Bb, Rr);
-    if (xs_tiled) {
-#pragma unroll
-        for (int it = 0; it < 2; it++) {
-            const int qd = it * kThr + threadIdx.x, ln = qd & 63, ct = (qd >> 6) & 1, rt = (qd >> 7) & 1, bi = qd >> 8;
-            const int t = 32 * (bi >> 1) + 16 * rt + 4 * (ln >> 4), j = 32 * (bi & 1) + 16 * ct + (ln & 15);
-            const float nth = -__shfl(gt.th, j);
-            Xs[t * LDM + j] = nth * tx.x[it].x; Xs[(t + 1) * LDM + j] = nth * tx.x[it].y;
-            Xs[(t + 2) * LDM + j] = nth * tx.x[it].z; Xs[(t + 3) * LDM + j] = nth * tx.x[it].w;
-        }
-    } else {
-#pragma unroll
-        for (int it = 0; it < 2; it++) {
-            const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
-            float *p = Xs + rr * LDM + cc;
-            p[0] = -__shfl(gt.th, cc) * tx.x[it].x; p[1] = -__shfl(gt.th, cc + 1) * tx.x[it].y;
-            p[2] = -__shfl(gt.th, cc + 2) * tx.x[it].z; p[3] = -__shfl(gt.th, cc + 3) * tx.x[it].w;
-        }
-    }
-    __syncthreads();
-    if (task + 1 < task_hi) fetch_task(task + 1);
-    {   // mat-vecs with c and bb: thread (tau, segment of 8 tokens j), then a sum over the 8 segments
-        const int tau = threadIdx.x >> 3, j0 = (threadIdx.x & 7) * 8;
-        float x0 = 0.f, x1 = 0.f, x2 = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int j = j0 + i;   // entries beyond the diagonal or beyond L are stored as zero
-            const float wf = Cc[tau * LDM + j], wsv = Bb[j * LDM + tau];
-            x0 = fmaf(wf, g1[j], x0); x1 = fmaf(wsv, g1[j], x1); x2 = fmaf(wsv, g2[j], x2);
-        }
-#pragma unroll
-        for (int m = 1; m < 8; m <<= 1) { x0 += __shfl_xor(x0, m); x1 += __shfl_xor(x1, m); x2 += __shfl_xor(x2, m); }
-        if ((threadIdx.x & 7) == 0) {
-            um[tau] = cf.a[tau] * m0dm + cf.beta[tau] * s0dm + x0;
-            usm[tau] = cf.h[tau] * s0dm + x1;
-            uss[tau] = cf.h[tau] * s0ds + x2;
-        }
-    }
-    NLH_STRIP_ORIGIN();
-    Strip ua = zero_strip(), us = zero_strip();
-    mma(ua, [&](int m, int kk) { return Cc[(m0 + m) * LDM + kk]; },
-        [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
-    if (has_s)
-        mma(us, [&](int m, int kk) { return Bb[kk * LDM + m0 + m]; },
-            [&](int kk, int n) { return Xs[(n0 + n) * LDM + kk]; });
-    // row tau feeds token tau+1: weights r[tau+1][t'] (d_alpha) and c[t'][tau+1] (d_eta), zero for t' <= tau
-#pragma unroll
-    for (int tl = 0; tl < 2; tl++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int tau = m0 + row_of(i), tp = n0 + 16 * tl + (threadIdx.x & 15);
-            const float uM = cf.a[tau] * p0[tp] + cf.beta[tau] * ps[tp] + ua.t[tl][i];
-            const float uS = cf.h[tau] * ps[tp] + us.t[tl][i];
-            const bool ok = tau + 1 < CW;
-            ua.t[tl][i] = ok ? Rr[(tau + 1) * LDM + tp] * uM : 0.f;
-            us.t[tl][i] = ok ? Cc[tp * LDM + tau + 1] * uS : 0.f;
-        }
-    strip_row_sums(ua);
-    strip_row_sums(us);
-    if (row_writer()) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) { part[0][nh][m0 + row_of(i)] = ua.t[0][i]; part[1][nh][m0 + row_of(i)] = us.t[0][i]; }
-    }
-    // token 0 has no predecessor row: its sums run over the first column of r and c (one wave)
-    float da0 = 0.f, de0 = 0.f;
-    if (wv == 0) {
-        da0 = wave_allreduce(lane < L ? Rr[lane] * p0[lane] : 0.f);
-        de0 = wave_allreduce(lane < L ? Cc[lane * LDM] * ps[lane] : 0.f);
-    }
-    __syncthreads();
-    if (threadIdx.x < L) {
-        const int t = threadIdx.x;
-        float da, de;
-        if (t == 0) {
-            da = Rr[L - 1] * m0dm + da0;
-            de = cf.cl[0] * s0dm + cf.bl[0] * s0ds + de0;
-        } else {
-            da = part[0][0][t - 1] + part[0][1][t - 1] + Rr[t * LDM + L - 1] * um[t - 1];
-            de = part[1][0][t - 1] + part[1][1][t - 1] + cf.cl[t] * usm[t - 1] + cf.bl[t] * uss[t - 1];
-        }
-        d_alpha[tok + t] = -da;
-        if (has_s) d_eta[tok + t] = de;
-    }
-    __syncthreads();   // LDS is rewritten by the next task
-    }
-}
-constexpr size_t kGatesBwdLds = 4 * MAT * sizeof(float);
 
 // Sum over chains of st[chain][slot 0][.]: stage 1 sums `per` chains per block row into
 // tmp[rows][4096]; stage 2 adds the rows to dst (+=).
@@ -1009,10 +872,8 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         set_lds(cw_local_bwd_kernel<uint16_t>, kLocalBwdLds);
         set_lds(cw_grads_bwd_kernel<float>, kGradsBwdLds);
         set_lds(cw_grads_bwd_kernel<uint16_t>, kGradsBwdLds);
-        set_lds(cw_gates_bwd_kernel, kGatesBwdLds);
         attr_set = true;
     }
-    int xs_tiled = 0;
     if constexpr (sizeof(TIn) == 2) {
         // bf16 tokens: coefficient pre-pass, adjoint scan and per-chunk gradients on the bf16 matrix cores
         const size_t nchunks = (size_t)batch * nc;
@@ -1025,7 +886,6 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec, xs,
                              scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
                              persistent_grid(batch * nc));
-        xs_tiled = 1;
     } else {
         hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
                            stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc,
@@ -1043,10 +903,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                            d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc);
         check_launch("cw_grads_bwd_kernel");
     }
-    hipLaunchKernelGGL(cw_gates_bwd_kernel, dim3(min(batch * nc, 2 * persistent_grid(1 << 30))), dim3(kThr),
-                       kGatesBwdLds, stream(), alpha, theta, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, chunk_size,
-                       nc, (int)has_s, xs_tiled, batch * nc);
-    check_launch("cw_gates_bwd_kernel");
+    chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s);
     const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
     const int per = 8, rows = ceil_div(batch, per);
     float *tmp = scratch(10, (size_t)rows * HD * HD * sizeof(float));
