@@ -74,7 +74,8 @@ def make_inputs(B, s, d, seed):
 # read, and per memory: target, error, update), forward + backward 260 d^2.
 FLOP_HOPE_FWD = 54 * D_HEAD * D_HEAD
 FLOP_HOPE_BWD = 206 * D_HEAD * D_HEAD
-BYTES_HOPE_BWD = 4 * 4 * D_HEAD + 2 * 6 * D_HEAD * D_HEAD * 4 // 64   # x, dy, d_x + caches; snapshots / 64 tokens
+BYTES_HOPE_FWD = 2 * 4 * D_HEAD + 6 * D_HEAD * D_HEAD * 4 // 64   # x, y; snapshots written once per 64 tokens
+BYTES_HOPE_BWD = 2 * 4 * D_HEAD + 6 * D_HEAD * D_HEAD * 4 // 64   # dy, d_x; snapshots read
 
 
 def cpu_baseline(x, heads, budget_s=12.0):
@@ -99,6 +100,37 @@ def cpu_baseline(x, heads, budget_s=12.0):
     return {"value": tokens / el, "unit": "tokens/s", "cores": 1, "kind": "port",
             "sample": f"{done} of {B} chains ({done // heads} sequences of {s} tokens, all {heads} heads), "
                       f"full-trajectory forward + backward, {el:.1f} s"}
+
+
+def host_threads():
+    """Threads for the all-cores CPU leg: the host cores this process may use (the GPU boxes export
+    their CPU share as OMP_NUM_THREADS)."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, int(os.environ.get("OMP_NUM_THREADS", n)))
+    except ValueError:
+        pass
+    return max(1, n)
+
+
+def cpu_all_cores(chain_fn, n_chains, seq_len, chains_per_token_row, what, budget_s=10.0):
+    """The same oracle over whole chains on every host core: chains are independent, the oracle is a C
+    library called through ctypes (the interpreter lock is released during a call), so a thread pool
+    scales like the reference's loops would under a chain-parallel driver.  Chains are handed out until
+    the time budget is used."""
+    from concurrent.futures import ThreadPoolExecutor
+    n_thr = host_threads()
+    done = 0
+    t_start = time.perf_counter()
+    with ThreadPoolExecutor(n_thr) as pool:
+        while done < n_chains and time.perf_counter() - t_start < budget_s:
+            batch = list(range(done, min(n_chains, done + n_thr)))
+            list(pool.map(chain_fn, batch))
+            done += len(batch)
+    el = time.perf_counter() - t_start
+    return {"value": done * seq_len / chains_per_token_row / el, "unit": "tokens/s", "cores": n_thr, "kind": "port",
+            "sample": f"{done} of {n_chains} chains of {seq_len} tokens ({chains_per_token_row} chains = one sequence "
+                      f"of d=512), {what}, {n_thr} threads, {el:.1f} s"}
 
 
 # Chunkwise (matrix form), per head-token at d=64, C=64: compulsory HBM bytes forward 1164
@@ -162,12 +194,19 @@ def setup_titans_exact_c2(torch, D, lib):
                dv["eta"], mc, sc, dv["dy"], g["dk"], g["dv"], g["dq"], g["da"], g["dt"], g["de"],
                g["dm"], g["ds"], s, d, B, C, 0.0, F32_MAX)
 
+    def chain(b):
+        from oracle import pyoracle as orc
+        a = [x[n][b].numpy() for n in ("k", "v", "q", "alpha", "theta", "eta")]
+        y, ms, ss = orc.titans_forward(*a, x["m0"][b].numpy(), x["s0"][b].numpy())
+        orc.titans_backward(*a, ms, ss, x["dy"][b].numpy())
+
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s,
-        flop_fwd=FLOP_FWD, flop_bwd=FLOP_BWD, bytes_bwd=BYTES_BWD,
-        traffic_bwd=int((193.7 + 298.0) * 2**20),   # measured: 193.7 MiB read, 298.0 MiB written
-        kernel="rule_bwd_fused_kernel<64,true> (+ finalize, per launch of the backward entry point)",
+        flop_fwd=FLOP_FWD, flop_bwd=FLOP_BWD, bytes_fwd=BYTES_FWD, bytes_bwd=BYTES_BWD,
+        # own algorithmic flops per head-token of the instrumented kernels
+        kernel_work={"rule_fwd_kernel": FLOP_FWD, "rule_bwd_fused_kernel": FLOP_BWD},
         kernel_names={"forward": "forward_ckpt", "backward": "backward_ckpt_fused"},
+        cpu_all=lambda: cpu_all_cores(chain, B, s, heads, "full-trajectory forward + backward"),
         config={"workload": "BASELINE configs[1]: Titans LMM exact recurrence, 8 heads x 64 (d=512), "
                             "batch 8, seq 2048, fp32 state, checkpoints every 64 tokens, fwd+bwd",
                 "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "checkpoint_interval": C},
@@ -196,13 +235,27 @@ def setup_titans_chunkwise_c3(torch, D, lib):
                dv["eta"], mc, sc, dv["dy"], g["dk"], g["dv"], g["dq"], g["da"], g["dt"], g["de"],
                g["dm"], g["ds"], s, d, B, C)
 
+    def chain(b):
+        from oracle import pyoracle as orc
+        a = [x[n][b].float().numpy() for n in ("k", "v", "q", "alpha", "theta", "eta")]
+        y, mco, sco = orc.chunkwise_forward(*a, x["m0"][b].numpy(), x["s0"][b].numpy(), C, True)
+        orc.chunkwise_backward(*a, mco, sco, x["dy"][b].numpy(), C, True)
+
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16",
-        flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_bwd=BYTES_CW_BWD,
+        flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_fwd=BYTES_CW_FWD, bytes_bwd=BYTES_CW_BWD,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
-        traffic_bwd=int((1707.8 + 522.3) * 2**20),   # measured for cw_grads_bf16_kernel: 1707.8 MiB read, 522.3 MiB written
-        kernel="cw_grads_bf16_kernel (the per-chunk gradient pass of the backward entry point)",
+        # each kernel's OWN compulsory bytes per head-token (what it must read and write given its role in
+        # the split; intermediates between kernels count for both sides, so these do not add up to 3108):
+        #   forward chain: the forward's 1164
+        #   adjoint scan: k, q 256 + dY 256 + gates 12 + adjoint snapshots 2 x 16384 / 64
+        #   gradients: k, v, q 384 + dY 256 + gates 12 + states 512 + adjoints 512 + d_k, d_v, d_q 768 + d_theta 4
+        #              + per-token terms for the gate pass 256 + 16
+        #   gate sweeps: those 256 + 16, gates 8, d_alpha, d_eta 8
+        kernel_work={"cw_chain_fwd_kernel": BYTES_CW_FWD, "cw_adjoint_chain_kernel": 1036,
+                     "cw_grads_bf16_kernel": 2720, "cw_gates_sweep_kernel": 288},
         kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
+        cpu_all=lambda: cpu_all_cores(chain, B, s, heads, "chunkwise forward + backward"),
         config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
                             "batch 16, seq 4096, bf16 k/v/q with fp32 accumulate and fp32 M/S, fwd+bwd",
                 "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "chunk_size": C},
@@ -212,6 +265,7 @@ def setup_titans_chunkwise_c3(torch, D, lib):
 # SWA per head-token at window 512, hd 64: forward 4*ws*hd flop, backward ~2.5x; compulsory bytes
 # bf16 q,k,v,out 512 + weights 2*1024 + fp32 d_out,dq,dk,dv 1024.
 FLOP_SWA_FWD, FLOP_SWA_BWD = 4 * 512 * 64, 10 * 512 * 64
+BYTES_SWA_FWD = 4 * 128 + 1024           # q, k, v in, out and the weights out
 BYTES_SWA_BWD = 3 * 128 + 1024 + 4 * 256
 
 
@@ -252,15 +306,64 @@ def setup_swa_c5(torch, D, lib):
 
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * heads * s, bound="hbm", dtype="bf16",
-        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_bwd=BYTES_SWA_BWD,
+        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_fwd=BYTES_SWA_FWD, bytes_bwd=BYTES_SWA_BWD,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
-        traffic_bwd=int((522.9 + 128.0 + 403.2 + 65.0) * 2**20),   # measured: key pass + query pass (read + written MiB each)
-        kernel=None,
         kernel_names={"forward": "swa_forward", "backward": "swa_backward"},
         config={"workload": "BASELINE configs[4], attention branch: sliding-window attention, window 512, 8 heads x 64, "
                             "bf16 storage with fp32 softmax, batch 8, seq 4096, fwd+bwd",
                 "batch": bs, "heads": heads, "head_dim": hd, "seq_len": s, "window": window},
         cpu=lambda: cpu_baseline_swa(q, k, v, d_out, window, heads))
+
+
+def cpu_baseline_mag_layer(bs, s, d, heads, k, window):
+    """The layer's CPU cost as the sum of its parts, each on a bounded sample, one thread: the chunkwise
+    rule (oracle, k levels x heads chains), sliding-window attention (oracle), the dense projections
+    (numpy fp32 GEMMs held to one BLAS thread) and AdamW (oracle) amortised over the step's tokens.
+    The glue between them (row norms, gate dot products, head transposes) is left out: the figure
+    overstates the CPU rate."""
+    import torch
+    from threadpoolctl import threadpool_limits
+    from oracle import pyoracle as orc
+    hd, C, n = d // heads, 64, 1024
+    xin = make_inputs(k * heads, n, hd, 0x5EED0009)
+    npx = {nm: t.numpy() for nm, t in xin.items()}
+    t0 = time.perf_counter()
+    for b in range(k * heads):
+        a = [npx[nm][b] for nm in ("k", "v", "q", "alpha", "theta", "eta")]
+        y, mc, sc = orc.chunkwise_forward(*a, npx["m0"][b], npx["s0"][b], C, True)
+        orc.chunkwise_backward(*a, mc, sc, npx["dy"][b], C, True)
+    t_rule = (time.perf_counter() - t0) / n
+    g = torch.Generator(device="cpu").manual_seed(0x5EED000A)
+    ns = 1024
+    q, kk, v = (torch.randn(1, ns, d, generator=g).to(torch.bfloat16).view(torch.uint16).numpy() for _ in range(3))
+    do = torch.randn(1, ns, d, generator=g).numpy()
+    t0 = time.perf_counter()
+    out, aw = orc.swa_forward(q, kk, v, window, heads, 0)
+    orc.swa_backward(q, kk, v, aw, do, window, heads, 0)
+    t_swa = (time.perf_counter() - t0) / ns
+    rs = np.random.default_rng(5)
+    xm, wm = rs.standard_normal((n, d), dtype=np.float32), rs.standard_normal((d, d), dtype=np.float32)
+    n_proj = 3 + 3 * k + 1            # q, k, v, per level k, v, q, and W_o
+    with threadpool_limits(limits=1):
+        t0 = time.perf_counter()
+        for _ in range(n_proj):
+            yv = xm @ wm.T            # forward
+            _ = yv @ wm               # input gradient
+            _ = yv.T @ xm             # weight gradient
+        t_proj = (time.perf_counter() - t0) / n
+    n_par = (4 + 3 * k) * d * d + 3 * k * (2 * d + 1)
+    w, gr, m, vv = (rs.standard_normal(n_par, dtype=np.float32) for _ in range(4))
+    vv = np.abs(vv)
+    t0 = time.perf_counter()
+    orc.grad_norm_clip([gr], 1.0)
+    orc.adamw_step(w, gr, m, vv, 3e-4, 0.9, 0.95, 1e-8, 10.0, 20.0, 0.1)
+    t_opt = (time.perf_counter() - t0) / (bs * s)
+    per_token = t_rule + t_swa + t_proj + t_opt
+    return {"value": 1.0 / per_token, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"sum of parts per token: chunkwise rule {k} levels x {heads} heads on {n} tokens "
+                      f"({t_rule * 1e6:.0f} us/token), attention on {ns} tokens ({t_swa * 1e6:.0f}), {n_proj} projection "
+                      f"GEMM triples on {n} tokens ({t_proj * 1e6:.0f}), AdamW over {n_par} parameters per step of "
+                      f"{bs * s} tokens ({t_opt * 1e6:.1f}); glue kernels not counted"}
 
 
 def setup_mag_layer_c5(torch, D, lib):
@@ -291,7 +394,8 @@ def setup_mag_layer_c5(torch, D, lib):
     return dict(
         fwd=fwd, bwd=bwd, step=step, tokens=bs * s, head_tokens=bs * s, bound="hbm", dtype="bf16",
         flop_fwd=4 * 8 * FLOP_CW_FWD + 8 * FLOP_SWA_FWD, flop_bwd=4 * 8 * FLOP_CW_BWD + 8 * FLOP_SWA_BWD,
-        bytes_bwd=4 * 8 * BYTES_CW_BWD + 8 * BYTES_SWA_BWD, traffic_bwd=None, kernel=None,
+        bytes_fwd=4 * 8 * BYTES_CW_FWD + 8 * BYTES_SWA_FWD, bytes_bwd=4 * 8 * BYTES_CW_BWD + 8 * BYTES_SWA_BWD,
+        step_eager=lambda: (fwd(), bwd()),
         kernel_names={"forward": "layer_forward", "backward": "layer_backward_and_adamw"},
         config={"workload": "BASELINE configs[4]: full layer, CMS k=4 Titans levels at periods [1,8,64,512] (chunkwise "
                             "rule, chunk 64, bf16 k/v/q) with MAG sigmoid gating over sliding-window attention "
@@ -299,8 +403,7 @@ def setup_mag_layer_c5(torch, D, lib):
                             "Xavier weights; forward + backward (replayed from a HIP graph) + AdamW (lr 3e-4, betas "
                             "0.9/0.95, wd 0.1); the dense projections are library GEMMs",
                 "batch": bs, "heads": heads, "d_model": d, "seq_len": s, "levels": k, "window": window},
-        cpu=lambda: {"value": None, "unit": "tokens/s", "cores": 1, "kind": "port",
-                     "sample": "not timed: the layer has no CPU restatement beyond its parts (see the per-part workloads)"})
+        cpu=lambda: cpu_baseline_mag_layer(bs, s, d, heads, k, window))
 
 
 def cpu_baseline_adamw(tensors, budget_s=12.0):
@@ -354,7 +457,7 @@ def setup_adamw_c5(torch, D, lib):
 
     return dict(
         fwd=fwd, bwd=bwd, tokens=n, head_tokens=n, bound="hbm", dtype="f32", unit="params/s",
-        flop_fwd=0, flop_bwd=12, bytes_bwd=28, traffic_bwd=None, kernel=None,
+        flop_fwd=0, flop_bwd=12, bytes_fwd=0, bytes_bwd=28,
         kernel_names={"forward": "none", "backward": "adamw_step"},
         config={"workload": "BASELINE configs[4], optimizer step: frequency-aware AdamW (lr 3e-4, betas 0.9/0.95, wd 0.1) "
                             "with gradient-norm clip over the layer's parameters, d=512, k=4 levels, all firing",
@@ -384,9 +487,7 @@ def setup_hope_selfref_c4(torch, D, lib):
 
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s,
-        flop_fwd=FLOP_HOPE_FWD, flop_bwd=FLOP_HOPE_BWD, bytes_bwd=BYTES_HOPE_BWD,
-        traffic_bwd=int((542.2 + 38.0) * 2**20),  # measured, the sweep kernel alone
-        kernel="selfref_bwd_kernel<64,true,true> (the chain-sequential sweep of the backward entry point)",
+        flop_fwd=FLOP_HOPE_FWD, flop_bwd=FLOP_HOPE_BWD, bytes_fwd=BYTES_HOPE_FWD, bytes_bwd=BYTES_HOPE_BWD,
         kernel_names={"forward": "selfref_forward", "backward": "selfref_backward"},
         config={"workload": "BASELINE configs[3]: HOPE self-referential memory, 8 heads x 64 (d=512), "
                             "batch 8, seq 2048, fp32, self-generated values, frozen snapshots per 64 tokens, fwd+bwd",
@@ -439,9 +540,7 @@ def setup_hebbian_c2(torch, D, lib):
 
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm",
-        flop_fwd=FLOP_HEB_FWD, flop_bwd=FLOP_HEB_BWD, bytes_bwd=BYTES_HEB_BWD,
-        traffic_bwd=int((192.7 + 96.5 + 65.1 + 32.1 + 33.1 + 33.0) * 2**20),   # measured: gradients + seed + scan kernels (read + written MiB)
-        kernel=None,
+        flop_fwd=FLOP_HEB_FWD, flop_bwd=FLOP_HEB_BWD, bytes_fwd=BYTES_HEB_FWD, bytes_bwd=BYTES_HEB_BWD,
         kernel_names={"forward": "hebbian_forward", "backward": "hebbian_backward_segment"},
         config={"workload": "Hebbian rule at the shape of BASELINE configs[1]: 8 heads x 64 (d=512), batch 8, "
                             "seq 2048, fp32, full M trajectory, forward + whole-sequence segment backward",
@@ -454,6 +553,131 @@ WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2"
              "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5, "hebbian_c2": setup_hebbian_c2}
 
 
+def source_hash():
+    """sha256 over the kernel sources and the C ABI header: what a traffic profile belongs to."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(ROOT, "nl_hecate_amd", "csrc", "*.hip")) +
+                   glob.glob(os.path.join(ROOT, "nl_hecate_amd", "csrc", "*.h")) +
+                   [os.path.join(ROOT, "include", "nl_hecate_ffi.h")])
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()
+
+
+def git_head():
+    import subprocess
+    try:
+        return subprocess.check_output(["git", "-C", ROOT, "rev-parse", "--short=12", "HEAD"],
+                                       stderr=subprocess.DEVNULL).decode().strip()
+    except Exception:
+        return None
+
+
+def profile_sidecar(workload):
+    """profiles/<workload>.json, written by `bench.py --write-profile` from rocprofv3 counter runs:
+    per-kernel FETCH_SIZE / WRITE_SIZE bytes per launch, stamped with the sources they were measured on."""
+    path = os.path.join(ROOT, "profiles", workload + ".json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f)
+
+
+def short_kernel_name(n):
+    n = n.replace("void ", "").replace("nlh::(anonymous namespace)::", "").replace("nlh::", "")
+    return n.split("(")[0]
+
+
+def write_profile(workload, raw):
+    """Summarise the rocprofv3 runs found under `raw` (trace_<w>/, pmc_FETCH_SIZE_<w>/, pmc_WRITE_SIZE_<w>/,
+    pmc_FETCH_SIZE_calib/, pmc_WRITE_SIZE_calib/, optional pmc_MFMA_<w>/) into
+    profiles/<workload>_kernels_and_hbm_traffic.txt and the sidecar profiles/<workload>.json."""
+    import collections
+    import csv
+    import glob
+
+    def find(sub, name):
+        hits = glob.glob(os.path.join(raw, sub, "**", name), recursive=True)
+        if not hits:
+            sys.exit(f"--write-profile: {name} not found under {os.path.join(raw, sub)}")
+        return hits[0]
+
+    def pmc(path):
+        agg = collections.defaultdict(lambda: [0, 0.0])
+        for row in csv.DictReader(open(path)):
+            k = (row["Kernel_Name"], row["Counter_Name"])
+            agg[k][0] += 1
+            agg[k][1] += float(row["Counter_Value"])
+        return {k: v / n for k, (n, v) in agg.items()}
+
+    cal_f = [v for (k, c), v in pmc(find("pmc_FETCH_SIZE_calib", "p_counter_collection.csv")).items() if "map_kernel" in k][0]
+    cal_w = [v for (k, c), v in pmc(find("pmc_WRITE_SIZE_calib", "p_counter_collection.csv")).items() if "map_kernel" in k][0]
+    kib = 262144.0
+    ff, fw = kib / cal_f, kib / cal_w
+    stats = list(csv.DictReader(open(find("trace_" + workload, "t_kernel_stats.csv"))))
+    pf = pmc(find("pmc_FETCH_SIZE_" + workload, "p_counter_collection.csv"))
+    pw = pmc(find("pmc_WRITE_SIZE_" + workload, "p_counter_collection.csv"))
+    cmd = f"python3 bench.py --workload {workload}"
+    lines = [f"{workload}: per-kernel time and HBM traffic on one MI355X (rocprofv3, ROCm 7.2)", "",
+             "commands (from /tmp, TMPDIR=/tmp; one run each; the summary below was written by "
+             f"`python3 bench.py --workload {workload} --write-profile <dir holding the runs' output>`):",
+             f"  rocprofv3 --kernel-trace --stats --output-format csv -d <out>/trace_{workload} -o t -- {cmd} --steps 10 --warmup 3 --no-cpu-baseline",
+             f"  rocprofv3 --pmc FETCH_SIZE --output-format csv -d <out>/pmc_FETCH_SIZE_{workload} -o p -- {cmd} --steps 2 --warmup 1 --no-cpu-baseline",
+             f"  rocprofv3 --pmc WRITE_SIZE --output-format csv -d <out>/pmc_WRITE_SIZE_{workload} -o p -- {cmd} --steps 2 --warmup 1 --no-cpu-baseline",
+             "  rocprofv3 --pmc FETCH_SIZE (then WRITE_SIZE) --output-format csv -d <out>/pmc_<counter>_calib -o p -- python3 bench.py --calibrate-copy"
+             "   (plain map kernel: 262144 KiB read, 262144 KiB written per launch)", "",
+             f"sources: git {git_head()}, sha256 of csrc/*.hip, csrc/*.h and the C header {source_hash()[:16]}", "",
+             "kernel trace (warm-up + timed steps + the per-entry-point and per-kernel timing launches of bench.py)",
+             f"{'kernel':62s} {'calls':>6s} {'total_us':>11s} {'avg_us':>10s} {'pct':>6s}"]
+    kernels = {}
+    for r in stats[:24]:
+        nm = short_kernel_name(r["Name"])
+        lines.append(f"{nm[:62]:62s} {int(r['Calls']):6d} {float(r['TotalDurationNs']) / 1e3:11.1f} "
+                     f"{float(r['AverageNs']) / 1e3:10.2f} {float(r['Percentage']):6.2f}")
+        kernels.setdefault(nm, {})["avg_us"] = float(r["AverageNs"]) / 1e3
+    lines += ["", f"counter calibration: the map kernel reads FETCH_SIZE={cal_f:.1f} for 262144 KiB read (factor {ff:.3f}) "
+                  f"and WRITE_SIZE={cal_w:.1f} for 262144 KiB written (factor {fw:.3f})", "",
+              f"{'kernel':62s} {'FETCH_SIZE':>12s} {'WRITE_SIZE':>12s} {'read_MiB':>10s} {'written_MiB':>11s}"]
+    names = sorted({k for (k, c) in pf if "nlh::" in k}, key=lambda k: -pf[(k, "FETCH_SIZE")])
+    for k in names:
+        a, b = pf[(k, "FETCH_SIZE")], pw.get((k, "WRITE_SIZE"), 0.0)
+        nm = short_kernel_name(k)
+        lines.append(f"{nm[:62]:62s} {a:12.1f} {b:12.1f} {a * ff / 1024:10.1f} {b * fw / 1024:11.1f}")
+        kernels.setdefault(nm, {}).update(fetch_bytes=int(a * ff * 1024), write_bytes=int(b * fw * 1024))
+    mp = glob.glob(os.path.join(raw, "pmc_MFMA_" + workload, "**", "p_counter_collection.csv"), recursive=True)
+    if mp:
+        pm = pmc(mp[0])
+        lines += ["", "matrix-core counters (one more run): rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES "
+                      "SQ_INSTS_VALU_MFMA_MOPS_BF16 SQ_INSTS_VALU_MFMA_MOPS_F32 GRBM_GUI_ACTIVE --output-format csv "
+                      f"-d <out>/pmc_MFMA_{workload} -o p -- {cmd} --steps 2 --warmup 1 --no-cpu-baseline",
+                  "per launch; GRBM_GUI_ACTIVE is summed over the 8 XCDs, SQ_VALU_MFMA_BUSY_CYCLES over the 1024 SIMDs; "
+                  "MOPS counters are in units of 512 flop; mfma_busy = MFMA_BUSY / 1024 / (GUI_ACTIVE / 8)",
+                  f"{'kernel':62s} {'GUI_ACTIVE':>12s} {'MFMA_BUSY':>13s} {'MOPS_BF16':>12s} {'MOPS_F32':>12s} {'mfma_busy':>10s}"]
+        for k in sorted({k for (k, c) in pm if "nlh::" in k}, key=lambda k: -pm.get((k, "GRBM_GUI_ACTIVE"), 0)):
+            ga = pm.get((k, "GRBM_GUI_ACTIVE"), 0)
+            if ga <= 0:
+                continue
+            mb = pm.get((k, "SQ_VALU_MFMA_BUSY_CYCLES"), 0)
+            nm = short_kernel_name(k)
+            lines.append(f"{nm[:62]:62s} {ga:12.0f} {mb:13.0f} {pm.get((k, 'SQ_INSTS_VALU_MFMA_MOPS_BF16'), 0):12.0f} "
+                         f"{pm.get((k, 'SQ_INSTS_VALU_MFMA_MOPS_F32'), 0):12.0f} {mb / 1024 / (ga / 8):10.3f}")
+            kernels.setdefault(nm, {})["mfma_busy"] = mb / 1024 / (ga / 8)
+    out_txt = os.path.join(ROOT, "profiles", workload + "_kernels_and_hbm_traffic.txt")
+    with open(out_txt, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    side = {"workload": workload, "git_head": git_head(), "source_sha256": source_hash(),
+            "calibration": {"fetch_factor": ff, "write_factor": fw,
+                            "note": "counter KiB per dispatch x factor = KiB moved; factors from a map kernel of known size"},
+            "kernels": kernels}
+    with open(os.path.join(ROOT, "profiles", workload + ".json"), "w") as f:
+        json.dump(side, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(open(out_txt).read())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -464,9 +688,15 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch a plain map kernel (256 MiB read, 256 MiB written) 5 times and exit: "
                          "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--write-profile", metavar="DIR",
+                    help="no GPU work: summarise the rocprofv3 runs of this workload found under DIR into "
+                         "profiles/<workload>_kernels_and_hbm_traffic.txt and profiles/<workload>.json")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
+    if args.write_profile:
+        write_profile(args.workload, args.write_profile)
+        return
 
     import torch
     from nl_hecate_amd import dispatch as D
@@ -506,59 +736,106 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = wall_ms / args.steps
     value = w["tokens"] / (ms_per_step * 1e-3)
+    ev_step_ms = ev_ms / args.steps
 
-    # per-kernel durations with events on the launch stream (outside the timed region)
+    # per-entry-point durations with events on the launch stream (outside the timed region)
     def avg_ms(fn, n=10):
         lib.nlh_timer_start()
         for _ in range(n):
             fn()
         return lib.nlh_timer_stop_ms() / n
     fwd_ms, bwd_ms = avg_ms(fwd), avg_ms(bwd)
-    # the dominant kernel alone: event pairs around its launches inside the entry point
-    if w["kernel"] is None:      # the entry point is the unit: its kernels are timed together
-        kern_ms, w["kernel"] = bwd_ms, w["kernel_names"]["backward"] + " entry point (all its kernels)"
-    else:
-        lib.nlh_kernel_timer_enable(1)
-        for _ in range(10):
-            bwd()
-        n_launch, name = ctypes.c_int(0), ctypes.create_string_buffer(128)
-        kern_ms = lib.nlh_kernel_timer_read_ms(ctypes.byref(n_launch), name, 128) / max(n_launch.value, 1)
-        lib.nlh_kernel_timer_enable(0)
-        assert n_launch.value == 10 and name.value.decode() in w["kernel"], (n_launch.value, name.value)
+    # every instrumented kernel on its own: event pairs around its launches inside the entry points
+    reps = 5
+    lib.nlh_kernel_timer_enable(1)
+    buf = ctypes.create_string_buffer(8192)
+    timed = {}
+    for _ in range(reps):
+        (w.get("step_eager") or (lambda: (fwd(), bwd())))()
+        assert lib.nlh_kernel_timer_report(buf, len(buf)) >= 0
+        for item in buf.value.decode().split(";"):
+            if item:
+                nm, launches, ms = item.rsplit(":", 2)
+                t = timed.setdefault(nm, [0, 0.0])
+                t[0] += int(launches)
+                t[1] += float(ms)
+    lib.nlh_kernel_timer_enable(0)
+
     head_tokens = w["head_tokens"]
-    bwd_tflops = w["flop_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e12
-    bwd_gbs = w["bytes_bwd"] * head_tokens / (kern_ms * 1e-3) / 1e9
     hbm_bound = w.get("bound") == "hbm"
-    roofline = {"kernel": w["kernel"],
-                "bound": "hbm" if hbm_bound else "mfma",
-                "achieved": bwd_gbs if hbm_bound else bwd_tflops,
-                "peak": PEAK_HBM_GBS if hbm_bound else PEAK_FP32_TFLOPS,
-                "unit": "GB/s" if hbm_bound else "TFLOP/s",
-                "frac": bwd_gbs / PEAK_HBM_GBS if hbm_bound else bwd_tflops / PEAK_FP32_TFLOPS,
-                "traffic": w["traffic_bwd"],
-                "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel; "
-                                "see profiles/" + args.workload + "_kernels_and_hbm_traffic.txt)",
-                "algorithmic_bytes": w["bytes_bwd"] * head_tokens,
-                "avg_launch_ms": kern_ms, "entry_point_ms": bwd_ms,
-                "hbm": {"achieved": bwd_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s"},
-                w.get("matrix", "fp32_matrix"): {"achieved": bwd_tflops, "peak": w.get("matrix_peak", PEAK_FP32_TFLOPS),
-                                                 "unit": "TFLOP/s",
-                                                 "frac": bwd_tflops / w.get("matrix_peak", PEAK_FP32_TFLOPS)},
-                "entry_point": {"achieved": w["bytes_bwd"] * head_tokens / (bwd_ms * 1e-3) / 1e9, "unit": "GB/s",
-                                "frac": w["bytes_bwd"] * head_tokens / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}}
+    peak = PEAK_HBM_GBS if hbm_bound else PEAK_FP32_TFLOPS
+    unit = "GB/s" if hbm_bound else "TFLOP/s"
+    per_ht = (lambda b, f: b) if hbm_bound else (lambda b, f: f)   # algorithmic work per head-token: bytes or flops
+    scale = 1e9 if hbm_bound else 1e12
+
+    def rate(work_per_ht, ms):
+        return work_per_ht * head_tokens / (max(ms, 1e-9) * 1e-3) / scale
+
+    side = profile_sidecar(args.workload)
+    stale = None if side is None else side.get("source_sha256") != source_hash()
+    side_k = {} if side is None else side["kernels"]
+
+    def kernel_traffic(nm):   # bytes per launch from the sidecar: the profile's kernel whose name starts with nm
+        for pn, rec in side_k.items():
+            if pn.startswith(nm) and "fetch_bytes" in rec:
+                return rec["fetch_bytes"] + rec.get("write_bytes", 0)
+        return None
+
+    kernels = []
+    for nm, (launches, ms) in sorted(timed.items(), key=lambda kv: -kv[1][1]):
+        own = w.get("kernel_work", {}).get(nm)
+        rec = {"name": nm, "launches_per_step": launches / reps, "avg_launch_ms": ms / launches,
+               "ms_per_step": ms / reps, "traffic": kernel_traffic(nm)}
+        if own is not None:
+            rec.update(algorithmic=own * head_tokens, achieved=rate(own, ms / reps),
+                       frac=rate(own, ms / reps) / peak, unit=unit)
+        kernels.append(rec)
+    step_traffic = None
+    if kernels and all(k["traffic"] is not None for k in kernels):
+        step_traffic = int(sum(k["traffic"] * k["launches_per_step"] for k in kernels))
+    work_step = per_ht(w.get("bytes_fwd", 0) + w["bytes_bwd"], w["flop_fwd"] + w["flop_bwd"])
+    work_bwd = per_ht(w["bytes_bwd"], w["flop_bwd"])
+    work_fwd = per_ht(w.get("bytes_fwd", 0), w["flop_fwd"])
+    roofline = {
+        "unit_timed": "the whole step (every kernel of the forward and backward entry points), HIP events on the "
+                      "launch stream around the timed steps",
+        "bound": "hbm" if hbm_bound else "mfma",
+        "achieved": rate(work_step, ev_step_ms), "peak": peak, "unit": unit,
+        "frac": rate(work_step, ev_step_ms) / peak,
+        "algorithmic": work_step * head_tokens,
+        "algorithmic_unit": "bytes per step" if hbm_bound else "flop per step",
+        "avg_launch_ms": ev_step_ms,
+        "traffic": step_traffic,
+        "traffic_unit": "HBM bytes per step: sum over kernels of (FETCH_SIZE + WRITE_SIZE per launch, scaled by a copy "
+                        "kernel) x launches per step, from profiles/" + args.workload + ".json",
+        "traffic_stale": stale,
+        "traffic_measured_at": None if side is None else side.get("git_head"),
+        "entry_points": {
+            "forward": {"ms": fwd_ms, "achieved": rate(work_fwd, fwd_ms), "frac": rate(work_fwd, fwd_ms) / peak},
+            "backward": {"ms": bwd_ms, "achieved": rate(work_bwd, bwd_ms), "frac": rate(work_bwd, bwd_ms) / peak}},
+        "kernels": kernels,
+        "dominant_kernel": kernels[0] if kernels else None,
+    }
+    if "matrix" in w:   # matrix-core rate of the whole step beside the memory figure
+        tf = (w["flop_fwd"] + w["flop_bwd"]) * head_tokens / (ev_step_ms * 1e-3) / 1e12
+        roofline[w["matrix"]] = {"achieved": tf, "peak": w["matrix_peak"], "unit": "TFLOP/s", "frac": tf / w["matrix_peak"]}
+    if not hbm_bound:
+        gbs = (w.get("bytes_fwd", 0) + w["bytes_bwd"]) * head_tokens / (ev_step_ms * 1e-3) / 1e9
+        roofline["hbm"] = {"achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS}
     out = {
         "metric": METRIC, "value": value, "unit": w.get("unit", "tokens/s"), "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.get("dtype", "f32"), "data": "synthetic",
         "config": w["config"],
-        "event_ms_per_step": ev_ms / args.steps,
+        "event_ms_per_step": ev_step_ms,
         "kernels_ms": {w["kernel_names"]["forward"]: fwd_ms, w["kernel_names"]["backward"]: bwd_ms},
-        "fwd_tflops": w["flop_fwd"] * head_tokens / (max(fwd_ms, 1e-9) * 1e-3) / 1e12,
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = w["cpu"]()
+        if "cpu_all" in w:
+            out["cpu_baseline_all_cores"] = w["cpu_all"]()
     print(json.dumps(out))
 
 

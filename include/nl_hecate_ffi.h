@@ -43,12 +43,14 @@ unsigned long long nlh_workspace_generation(void);
  * (blocks until the stop event completes); negative on failure. */
 int nlh_timer_start(void);
 float nlh_timer_stop_ms(void);
-/* Per-kernel timing of the dominant kernel of an entry point (the fused checkpointed
- * backward, the self-referential backward): while enabled, each such launch is bracketed
- * by an event pair on the launch stream (at most 256 between reads).  read_ms waits for
- * them, returns their summed duration, the launch count and the kernel's name, and resets. */
+/* Per-kernel timing: while enabled, every launch of the kernels the library instruments (those
+ * of the memory-rule entry points) is bracketed by an event pair on the launch stream (at most
+ * 256 between reads).  read_ms waits for them, returns their summed duration, the launch count
+ * and the name of the last kernel, and resets.  report writes "name:launches:total_ms;" per
+ * kernel name into buf, returns the number of names (< 0 on error) and resets. */
 int nlh_kernel_timer_enable(int on);
 float nlh_kernel_timer_read_ms(int *launches, char *name, int name_len);
+int nlh_kernel_timer_report(char *buf, int buf_len);
 /* Runs the cross-lane primitives on known data; returns 0 when all agree. */
 int nlh_selftest_lane_ops(void);
 /* Gate coefficients of one chunk (L <= 64 device-resident gates each) from the in-kernel generator:

@@ -213,6 +213,7 @@ bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d
     }
     if (es.failed()) return true;
     const int tabf = (int)chunkwise_grads_table_floats(), vecf = (int)chunkwise_grads_vec_floats();
+    KernelTimer kt("cw_adjoint_chain_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_adjoint_chain_kernel<true>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
                            d_y, tab_b, vecs, dm_states, ds_states, seq_len, chunk_size, nc, batch, tabf, vecf);

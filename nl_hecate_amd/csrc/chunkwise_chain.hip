@@ -397,11 +397,17 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
         attr_set = true;
     }
     if (es.failed()) return;
-    hipLaunchKernelGGL(cw_coef_kernel<HAS_S>, dim3(ceil_div(nchunks, 2)), dim3(256), 0, stream(), alpha, theta, eta,
-                       table, vecs, seq_len, chunk_size, nc, nchunks);
+    {
+        KernelTimer kt("cw_coef_kernel");
+        hipLaunchKernelGGL(cw_coef_kernel<HAS_S>, dim3(ceil_div(nchunks, 2)), dim3(256), 0, stream(), alpha, theta, eta,
+                           table, vecs, seq_len, chunk_size, nc, nchunks);
+    }
     check_launch("cw_coef_kernel");
-    hipLaunchKernelGGL(cw_chain_fwd_kernel<HAS_S>, dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k, v, q,
-                       table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch);
+    {
+        KernelTimer kt("cw_chain_fwd_kernel");
+        hipLaunchKernelGGL(cw_chain_fwd_kernel<HAS_S>, dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k, v, q,
+                           table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch);
+    }
     check_launch(fn);
 }
 

@@ -130,6 +130,7 @@ void chunkwise_gate_gradients(const float *alpha, const float *eta, const float 
     }
     if (es.failed()) return;
     const dim3 grid(ceil_div(ntask, kGateWaves)), block(64 * kGateWaves);
+    KernelTimer kt("cw_gates_sweep_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_gates_sweep_kernel<true>, grid, block, lds, stream(), alpha, eta, pvec, xs, scal, d_alpha,
                            d_eta, seq_len, chunk_size, nc, ntask);

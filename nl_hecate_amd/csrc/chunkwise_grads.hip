@@ -593,6 +593,7 @@ size_t chunkwise_grads_vec_floats() { return kVecB; }
 void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta, float *tab_a,
                                      float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s) {
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
+    KernelTimer kt("cw_coef_bwd_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
                            eta, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);

@@ -909,8 +909,12 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     float *tmp = scratch(10, (size_t)rows * HD * HD * sizeof(float));
     if (es.failed()) return;
     for (int which = 0; which < (has_s && d_s_initial ? 2 : 1); which++) {
-        hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows), dim3(256), 0, stream(),
-                           which ? ds_states : dm_states, tmp, batch, per, chain_stride);
+        {
+            KernelTimer kt("cw_sum_slot0_kernel");
+            hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows), dim3(256), 0, stream(),
+                               which ? ds_states : dm_states, tmp, batch, per, chain_stride);
+        }
+        KernelTimer kt("cw_add_rows_kernel");
         hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), tmp,
                            which ? d_s_initial : d_m_initial, rows);
     }

@@ -537,6 +537,7 @@ void finalize_parts(const float *ws_dq, const float *ws_dk, const float *ws_gate
                     float *d_q, float *d_k, float *d_alpha, float *d_theta, float *d_eta,
                     int parts, int batch, int seq_len, int d, int t_start, int t_end) {
     dim3 grid(ceil_div((long long)(t_end - t_start) * d, 256), batch);
+    KernelTimer kt("finalize_parts_kernel");
     hipLaunchKernelGGL(finalize_parts_kernel, grid, dim3(256), 0, stream(), ws_dq, ws_dk, ws_gate,
                        d_q, d_k, d_alpha, d_theta, d_eta, parts, batch, seq_len, d, t_start, t_end);
     check_launch("finalize_parts_kernel");
@@ -570,6 +571,7 @@ static int pick_rpl(int d, int batch, bool coupled) {
 template <int D, int RPL, bool HAS_S, int STORE, bool FROZEN>
 static void launch_fwd_c(const FwdArgs &a, int batch, bool coupled) {
     dim3 grid(batch * a.parts), block(kThreads);
+    KernelTimer kt("rule_fwd_kernel");
     if (coupled)
         hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, true, FROZEN>), grid, block, 0, stream(), a);
     else
@@ -659,6 +661,7 @@ static bool launch_bwd(BwdArgs a, int d, float *ws = nullptr, bool whole_chain =
 }
 
 void accumulate_over_batch(const float *src, float *dst, int batch, int n) {
+    KernelTimer kt("accumulate_over_batch_kernel");
     hipLaunchKernelGGL(accumulate_over_batch_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream(),
                        src, dst, batch, n);
     check_launch("accumulate_over_batch_kernel");

@@ -16,6 +16,7 @@ static int g_kt_used = 0;
 static hipEvent_t g_kt_ev[kKtMax][2];
 static int g_kt_created = 0;
 static char g_kt_name[128] = {0};
+static const char *g_kt_names[kKtMax] = {nullptr};   // string literals of the call sites
 
 
 static int g_error_mode = 0;
@@ -100,6 +101,7 @@ KernelTimer::KernelTimer(const char *name) : slot(-1) {
         g_kt_created++;
     }
     slot = g_kt_used++;
+    g_kt_names[slot] = name;
     snprintf(g_kt_name, sizeof(g_kt_name), "%s", name);
     (void)hipEventRecord(g_kt_ev[slot][0], stream());
 }
@@ -172,6 +174,36 @@ float nlh_kernel_timer_read_ms(int *launches, char *name, int name_len) {
     if (name && name_len > 0) snprintf(name, name_len, "%s", nlh::g_kt_name);
     nlh::g_kt_used = 0;
     return total;
+}
+
+int nlh_kernel_timer_report(char *buf, int buf_len) {
+    if (!buf || buf_len <= 0) return -1;
+    struct Row { const char *name; int launches; float ms; };
+    Row rows[64];
+    int nrows = 0;
+    for (int i = 0; i < nlh::g_kt_used; i++) {
+        float ms = 0.f;
+        if (hipEventSynchronize(nlh::g_kt_ev[i][1]) != hipSuccess ||
+            hipEventElapsedTime(&ms, nlh::g_kt_ev[i][0], nlh::g_kt_ev[i][1]) != hipSuccess)
+            return -1;
+        int r = 0;
+        while (r < nrows && strcmp(rows[r].name, nlh::g_kt_names[i]) != 0) r++;
+        if (r == nrows) {
+            if (nrows == 64) continue;
+            rows[nrows++] = Row{nlh::g_kt_names[i], 0, 0.f};
+        }
+        rows[r].launches++;
+        rows[r].ms += ms;
+    }
+    int off = 0;
+    buf[0] = 0;
+    for (int r = 0; r < nrows; r++) {
+        int n = snprintf(buf + off, buf_len - off, "%s:%d:%.6f;", rows[r].name, rows[r].launches, rows[r].ms);
+        if (n < 0 || n >= buf_len - off) return -2;
+        off += n;
+    }
+    nlh::g_kt_used = 0;
+    return nrows;
 }
 
 const char *nlh_version(void) { return "nl_hecate_rocm 0.1 (gfx950)"; }
