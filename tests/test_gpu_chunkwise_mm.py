@@ -182,8 +182,9 @@ def test_initial_state_gradients_accumulate():
 
 
 def test_matrix_form_agrees_with_sequential_kernels_at_benchmark_shape():
-    """B' = 16 chains of the config-3 shape (seq 4096, C = 64) are too long for the CPU
-    oracle; the sequential frozen-M0 kernels (parity-tested against it) are the yardstick.
+    """A second opinion beside the oracle (which checks all 128 chains of this shape in
+    test_gpu_fullsize_values.py): B' = 16 chains of the config-3 shape (seq 4096, C = 64) against the
+    sequential frozen-M0 kernels of the library.
     The reference-named symbols take the matrix form themselves when no clip is set, so the
     yardstick is called with an error clip that is active and never reached (1e30): that
     selects the sequential kernels and leaves every error unchanged."""

@@ -1,6 +1,7 @@
 """Properties of the bf16 chunkwise path at the full size of BASELINE configs[2] (128 chains of
-4096 tokens, chunk 64), where the CPU oracle is too slow to be the yardstick.  The kernels
-contain no atomics and no data-dependent scheduling, so each property holds bit for bit:
+4096 tokens, chunk 64), beside the value check against the oracle at the same size
+(test_gpu_fullsize_values.py).  The kernels contain no atomics and no data-dependent scheduling, so
+each property holds bit for bit:
 
 * chain independence: a chain's results do not depend on which other chains share the launch;
 * causality: outputs and chunk states before a chunk do not depend on its tokens;
@@ -8,7 +9,7 @@ contain no atomics and no data-dependent scheduling, so each property holds bit 
   path (fp32, bf16 and hi + lo pairs of bf16).
 
 A wrong index, a race between workgroups of one chain or a dependence on launch geometry breaks
-one of them.  Values are checked against the oracle at small sizes in test_gpu_chunkwise_mm.py."""
+one of them."""
 import pytest
 import torch
 

@@ -1,5 +1,5 @@
-"""Properties of the HOPE self-referential path at the launch size of BASELINE configs[3], where the
-CPU oracle is too slow to be the yardstick.  configs[3] is 64 chains of 2048 tokens = 2048 chunks of
+"""Properties of the HOPE self-referential path at the launch size of BASELINE configs[3] (values
+against the oracle at that size: test_gpu_fullsize_values.py).  configs[3] is 64 chains of 2048 tokens = 2048 chunks of
 64 tokens; with its distributions (x ~ N(0, 1/d), so alpha = sigmoid(~0) = 1/2 at every token) every
 memory halves per token and is exactly zero in fp32 after about 150 tokens, in the reference's
 equations as here, so all later chunks of a chain carry zeros.  To keep every chunk's data alive the
@@ -12,7 +12,7 @@ data-dependent scheduling, so each property holds bit for bit:
 * exact scaling: the backward is linear in dY and a factor of 2 is exact in fp32 (above the
   underflow threshold).
 
-Values are checked against the oracle at small sizes in test_gpu_selfref.py."""
+Small sizes against the oracle: test_gpu_selfref.py."""
 import pytest
 import torch
 

@@ -21,7 +21,10 @@ def ref_params(p, dtype=torch.float64):
                 levels=[{n: leaf(getattr(l, n)) for n in names} for l in p.levels])
 
 
-def run_case(bs, s, d, nh, k, window, periods, rule, chunk, seed, steps=1):
+def run_case(bs, s, d, nh, k, window, periods, rule, chunk, seed, steps=1, bias_scale=False):
+    """bias_scale: a gate bias gradient is one scalar, a sum over all tokens of signed terms that can
+    nearly cancel; its error is then taken relative to max(|reference|, ||gradient of the matching gate
+    weight vector||), the size of the sums it belongs to, instead of to its own (possibly tiny) value."""
     torch.manual_seed(seed)
     p = init_params(d, k, seed)
     layer = MagLayer(d, nh, k, window, periods, rule=rule, chunk=chunk, params=p)
@@ -55,6 +58,10 @@ def run_case(bs, s, d, nh, k, window, periods, rule, chunk, seed, steps=1):
                     chk[f"L{lv}.d_{n}"] = (getattr(grads.levels[lv], n), t.grad)
         for n, (a, b) in chk.items():
             e = rel_err(a.detach().cpu().numpy().reshape(b.shape), b.detach().numpy())
+            if bias_scale and ".d_b_" in n:
+                wref = chk[n.replace(".d_b_", ".d_w_")][1]
+                e = float((a.detach().cpu().double().reshape(b.shape) - b.detach()).abs().max()
+                          / max(float(b.detach().abs().max()), float(wref.detach().norm())))
             worst[n] = max(worst.get(n, 0.0), e)
     return worst
 
