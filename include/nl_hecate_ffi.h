@@ -419,6 +419,35 @@ unsigned nlh_pulse_to_bitmask(const int *active, int k);
 int nlh_conductor_restore(nlh_conductor *c, int k, const long long *chunk_sizes, long long step,
                           long long stream_pulse_id);
 
+/* ErrorBuffer of one frozen CMS level (core/src/conductor.rs:224-261): the outer-loop gradients a level
+ * receives while it does not fire are summed and applied as one plain gradient step when it fires.
+ * The accumulators are caller-owned device buffers, one per parameter tensor of the level (zeroed by
+ * the caller), registered in a fixed order; `level_grads`, `params` and `single_step_grads` are host
+ * arrays of device pointers in that order.
+ *   accumulate       (:240-243): acc_i += grad_i for every tensor (one launch), steps_accumulated += 1
+ *   apply_and_reset  (:246-252): if steps_accumulated > 0: param_i -= lr * acc_i, acc_i = 0, counter = 0
+ *   health_check     (:256-261): *ratio = ||acc|| / ||single_step||; returns 1, or 0 (None) when the
+ *                    single-step norm is below 1e-12, < 0 on error; synchronises the launch stream */
+typedef struct nlh_error_buffer nlh_error_buffer;
+nlh_error_buffer *nlh_error_buffer_new(void);
+void nlh_error_buffer_free(nlh_error_buffer *b);
+int nlh_error_buffer_add_tensor(nlh_error_buffer *b, float *accumulator, int n);
+long long nlh_error_buffer_steps(const nlh_error_buffer *b);
+void nlh_error_buffer_accumulate(nlh_error_buffer *b, const float *const *level_grads);
+void nlh_error_buffer_apply_and_reset(nlh_error_buffer *b, float *const *params, float lr);
+int nlh_error_buffer_health_check(const nlh_error_buffer *b, const float *const *single_step_grads, float *ratio);
+/* ContextState (core/src/conductor.rs:156-221): the memories that persist across forward calls are
+ * caller-owned device buffers.
+ *   reset (:212-219): zero every buffer (per-level M, S and the self-referential memories) with one fill
+ *         launch (no memset node, so the call may be captured); the Conductor's step is not touched
+ *   seed_self_ref (:194-207): copy a level's m_*_init parameters into every chain of a
+ *         [batch, 6, d*d] block of self-referential memories (order m_k, m_v, m_q, m_eta, m_alpha,
+ *         m_mem): the five projection memories when m_k_init is non-null (all five are then required),
+ *         m_mem when m_mem_init is non-null; a null pointer stands for the reference's empty vector */
+void nlh_context_state_reset(float *const *buffers, const int *n, int count);
+void nlh_context_state_seed_self_ref(float *mems, const float *m_k_init, const float *m_v_init, const float *m_q_init,
+                                     const float *m_eta_init, const float *m_alpha_init, const float *m_mem_init,
+                                     int batch, int d);
 /* Frequency-aware AdamW (core/src/adamw.rs, core/src/gpu_optimizer.rs:403-515):
  * group -1 tensors update every step with the global step's bias correction;
  * group l tensors update only when level l's pulse is on, with that level's
@@ -445,6 +474,10 @@ void cms_gate_backward_rocm(const float *d_gated, const float *attn_out, const f
 /* Frozen level (core/src/gpu_forward.rs:2906-2950): y = M_h q per head, token-major */
 void memory_read_only_f32_rocm(const float *q_mem, const float *m, float *y, long long n_tokens, int nh,
                                int hd);
+/* Backward of that read (core/src/opaque_adapters.rs:1030-1047, per head): d_q = M_h^T d_y; no gradient
+ * reaches the frozen memory. */
+void memory_read_only_backward_f32_rocm(const float *d_y, const float *m, float *d_q, long long n_tokens, int nh,
+                                        int hd);
 
 /* HOPE self-referential memory, chunkwise with frozen snapshots.  The reference runs it
  * on the CPU only (core/src/chunkwise_self_ref.rs:52-222 chunkwise_self_ref_step,
@@ -754,6 +787,30 @@ void nlh_swa_forward_dispatch(const float *q, const float *k, const float *v, fl
 void nlh_swa_backward_dispatch(const float *q, const float *k, const float *v, const float *attn_weights,
                                const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len,
                                int num_heads, int head_dim, int window_size);
+
+/* ── Opaque VJP blocks of the Wengert tape ───────────────────────────────────────────────────────
+ * core/src/tape.rs:141-150 OpaqueBackwardFn(d_outputs, saved, d_inputs) for the OpaqueKey values
+ * below (numbered in the order of the enum at tape.rs:100-134), with the saved-buffer layouts of the
+ * registry's adapters (core/src/opaque_adapters.rs:290-304 DeltaRule, :386-401 TitansLMM, :952-964
+ * SWA, :1004-1008 frozen reads, :1680-1690 DGD).  All pointers are HOST memory (the tape is a CPU
+ * structure): buffer i of a list has lens[i] floats.  The block's backward runs on the GPU and its
+ * results are ADDED to d_inputs (the accumulation the tape performs after an adapter returns,
+ * tape.rs:839-866, is part of the call; a d_inputs buffer longer than what the rule produces, as with
+ * learned frequency gates, keeps its tail).  Returns 0, or non-zero after recording a message
+ * (argument error 1, layout / unsupported configuration 2, runtime 3).  Built: the default block
+ * configuration (L2 attentional bias, identity feature map, no Conv1D, linear memory, EMA momentum)
+ * in the newest recording format; d must be a size the memory-rule kernels serve. */
+enum {
+    NLH_OPAQUE_DELTA_RULE = 0,
+    NLH_OPAQUE_TITANS_LMM = 1,
+    NLH_OPAQUE_DGD = 9,
+    NLH_OPAQUE_SWA = 10,
+    NLH_OPAQUE_FROZEN_DELTA_RULE = 11,
+    NLH_OPAQUE_FROZEN_TITANS_LMM = 12
+};
+int nlh_opaque_backward(int key, const float *const *d_outputs, const long long *d_output_lens, int n_outputs,
+                        const float *const *saved, const long long *saved_lens, int n_saved,
+                        float *const *d_inputs, const long long *d_input_lens, int n_inputs);
 
 #ifdef __cplusplus
 }

@@ -105,3 +105,84 @@ class FrequencyAwareAdamW:
 
     def level_step(self, level):
         return lib.nlh_adamw_level_step(self._h, level)
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+class ErrorBuffer:
+    """core/src/conductor.rs:224-261: outer-loop gradients a frozen level receives are summed here and
+    applied as one plain gradient step when the level fires.  `like` is the level's parameter tensors
+    (device, float32): one accumulator of the same size is kept per tensor, in the same order."""
+
+    def __init__(self, like):
+        import torch
+        self.grads = [torch.zeros_like(t) for t in like]
+        self._h = lib.nlh_error_buffer_new()
+        for g in self.grads:
+            assert g.is_cuda and g.is_contiguous() and g.dtype == torch.float32
+            lib.nlh_error_buffer_add_tensor(self._h, g.data_ptr(), g.numel())
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib.nlh_error_buffer_free(self._h)
+            self._h = None
+
+    @property
+    def steps_accumulated(self) -> int:
+        return lib.nlh_error_buffer_steps(self._h)
+
+    def _check(self, tensors):
+        assert len(tensors) == len(self.grads)
+        for t, g in zip(tensors, self.grads):
+            assert t.is_cuda and t.is_contiguous() and t.numel() == g.numel()
+
+    def accumulate(self, level_grads):
+        self._check(level_grads)
+        lib.nlh_error_buffer_accumulate(self._h, _ptr_array(level_grads))
+
+    def apply_and_reset(self, params, lr):
+        self._check(params)
+        lib.nlh_error_buffer_apply_and_reset(self._h, _ptr_array(params), lr)
+
+    def health_check(self, single_step_grads):
+        """-> ||accumulated|| / ||single_step||, or None when the single-step norm is below 1e-12."""
+        self._check(single_step_grads)
+        ratio = ctypes.c_float(0.0)
+        rc = lib.nlh_error_buffer_health_check(self._h, _ptr_array(single_step_grads), ctypes.byref(ratio))
+        if rc < 0:
+            raise RuntimeError("nlh_error_buffer_health_check failed")
+        return ratio.value if rc == 1 else None
+
+
+class ContextState:
+    """core/src/conductor.rs:156-221: the memories that persist across forward calls.  `memory[l]` is
+    level l's state ([chains, d, d] here: one matrix per batch element and head), `momentum[l]` the Titans
+    momentum carried with it, `self_ref[l]` a [chains, 6, d, d] block of self-referential memories
+    (m_k, m_v, m_q, m_eta, m_alpha, m_mem) or None when the projections are static."""
+
+    def __init__(self, memory, momentum=None, self_ref=None):
+        self.memory = list(memory)
+        self.momentum = list(momentum) if momentum is not None else []
+        self.self_ref = list(self_ref) if self_ref is not None else [None] * len(self.memory)
+
+    def reset(self):
+        """:212-219: zero every memory in place (document boundary); the Conductor's step is untouched."""
+        bufs = [t for t in self.memory + self.momentum + self.self_ref if t is not None]
+        if bufs:
+            n = (ctypes.c_int * len(bufs))(*[t.numel() for t in bufs])
+            lib.nlh_context_state_reset(_ptr_array(bufs), n, len(bufs))
+
+    def seed_self_ref(self, level_inits):
+        """:194-207: level_inits[l] = dict with m_k_init, m_v_init, m_q_init, m_eta_init, m_alpha_init
+        ([d, d] tensors, or absent for static projections) and m_mem_init (or absent)."""
+        for lv, init in enumerate(level_inits):
+            if lv >= len(self.self_ref) or self.self_ref[lv] is None:
+                break
+            mems = self.self_ref[lv]
+            chains, six, d, _ = mems.shape
+            assert six == 6
+            get = lambda n: init[n].data_ptr() if init.get(n) is not None else None
+            lib.nlh_context_state_seed_self_ref(mems.data_ptr(), get("m_k_init"), get("m_v_init"), get("m_q_init"),
+                                                get("m_eta_init"), get("m_alpha_init"), get("m_mem_init"), chains, d)

@@ -39,6 +39,13 @@ struct nlh_adamw {
     std::vector<nlh_adamw_tensor> tensors;
 };
 
+// ── ErrorBuffer of one frozen level (core/src/conductor.rs:224-261) ─────────
+struct nlh_error_buffer {
+    std::vector<float *> acc;   // caller-owned device accumulators, one per parameter tensor
+    std::vector<int> n;
+    long long steps_accumulated;
+};
+
 namespace nlh {
 
 constexpr int kCmsThreads = 256;
@@ -78,17 +85,20 @@ __global__ void cms_gate_backward_kernel(const float *__restrict__ d_gated, cons
 // Frozen level: y[t, h*hd + i] = sum_j M[h][i][j] q[t, h*hd + j]
 // (core/src/gpu_forward.rs:2906-2950), token-major in and out, no transposes.
 // One workgroup per (head, 64-token tile); M_h and the q tile sit in LDS.
+// transposed != 0 reads M_h^T instead: the backward of the read, d_q = M_h^T d_y.
 __global__ __launch_bounds__(kCmsThreads) void memory_read_only_kernel(
     const float *__restrict__ q, const float *__restrict__ m, float *__restrict__ y, long long n_tok,
-    int nh, int hd) {
+    int nh, int hd, int transposed) {
     extern __shared__ float smem[];
     float *sm = smem;                       // [hd][hd+1]
     float *sq = smem + hd * (hd + 1);       // [64][hd+1]
     const int h = blockIdx.y;
     const long long t0 = (long long)blockIdx.x * 64;
     const int d = nh * hd;
-    for (int i = threadIdx.x; i < hd * hd; i += blockDim.x)
-        sm[(i / hd) * (hd + 1) + i % hd] = m[(size_t)h * hd * hd + i];
+    for (int i = threadIdx.x; i < hd * hd; i += blockDim.x) {
+        const int r = i / hd, c = i % hd;
+        sm[(transposed ? c * (hd + 1) + r : r * (hd + 1) + c)] = m[(size_t)h * hd * hd + i];
+    }
     for (int i = threadIdx.x; i < 64 * hd; i += blockDim.x) {
         const long long t = t0 + i / hd;
         sq[(i / hd) * (hd + 1) + i % hd] = t < n_tok ? q[t * d + h * hd + i % hd] : 0.f;
@@ -101,6 +111,48 @@ __global__ __launch_bounds__(kCmsThreads) void memory_read_only_kernel(
         float acc = 0.f;
         for (int j = 0; j < hd; j++) acc += sm[i * (hd + 1) + j] * sq[tt * (hd + 1) + j];
         y[t * d + h * hd + i] = acc;
+    }
+}
+
+// Multi-tensor maps of the ErrorBuffer / ContextState: the pointer table travels in the kernel argument.
+constexpr int kEbMax = 24;
+struct EbBatch {
+    float *dst[kEbMax];
+    float *src[kEbMax];
+    int n[kEbMax];
+    int blk_begin[kEbMax + 1];
+    int count;
+};
+// mode 0: dst += src (accumulate); 1: dst -= lr * src, then src <- 0 (apply_and_reset);
+// 2: dst <- 0 (reset); 3: dst <- src (seed)
+__global__ void eb_map_kernel(EbBatch b, int mode, float lr) {
+    int t = 0;
+    while (t + 1 < b.count && (int)blockIdx.x >= b.blk_begin[t + 1]) t++;
+    const int nblk = b.blk_begin[t + 1] - b.blk_begin[t], local = blockIdx.x - b.blk_begin[t];
+    float *d = b.dst[t];
+    float *sp = b.src[t];
+    for (int i = local * blockDim.x + threadIdx.x; i < b.n[t]; i += nblk * blockDim.x) {
+        if (mode == 0) d[i] += sp[i];
+        else if (mode == 1) { d[i] -= lr * sp[i]; sp[i] = 0.f; }
+        else if (mode == 2) d[i] = 0.f;
+        else d[i] = sp[i];
+    }
+}
+// sum of squares over a tensor list -> out[which] (one workgroup; the lists are a level's parameters)
+__global__ void eb_norm_sq_kernel(EbBatch b, int use_src, float *out) {
+    __shared__ float part[kCmsThreads / 64];
+    float acc = 0.f;
+    for (int t = 0; t < b.count; t++) {
+        const float *p = use_src ? b.src[t] : b.dst[t];
+        for (int i = threadIdx.x; i < b.n[t]; i += blockDim.x) acc = fmaf(p[i], p[i], acc);
+    }
+    acc = group_allreduce<64>(acc);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float sum = 0.f;
+        for (int w = 0; w < kCmsThreads / 64; w++) sum += part[w];
+        out[use_src] = sum;
     }
 }
 
@@ -244,6 +296,111 @@ unsigned nlh_adamw_step(nlh_adamw *o, const int *active_levels, float lr, float 
 // gate = sigmoid(c * sum_l y_l), gated = attn_out * gate, c = 1/sqrt(k) for k > 2
 // else 1 (core/src/gpu_forward.rs:1027-1070; mag.rs:709-718).  y_levels is a
 // HOST array of k device pointers; y_combined may be NULL.
+// ── ErrorBuffer (core/src/conductor.rs:224-261) ─────────────────────────────
+static bool eb_launch(const std::vector<float *> &dst, const float *const *src, const std::vector<int> &n, int mode,
+                      float lr, const char *what) {
+    for (size_t first = 0; first < dst.size(); first += nlh::kEbMax) {
+        nlh::EbBatch b;
+        b.count = 0;
+        int blocks = 0;
+        for (size_t i = first; i < dst.size() && i < first + nlh::kEbMax; i++) {
+            if (n[i] <= 0) continue;
+            const int c = b.count++;
+            b.dst[c] = dst[i];
+            b.src[c] = src ? const_cast<float *>(src[i]) : nullptr;
+            b.n[c] = n[i];
+            b.blk_begin[c] = blocks;
+            const int nb = (n[i] + nlh::kCmsThreads * 4 - 1) / (nlh::kCmsThreads * 4);
+            blocks += nb < 1 ? 1 : (nb > 128 ? 128 : nb);
+        }
+        if (b.count == 0) continue;
+        b.blk_begin[b.count] = blocks;
+        hipLaunchKernelGGL(nlh::eb_map_kernel, dim3(blocks), dim3(nlh::kCmsThreads), 0, nlh::stream(), b, mode, lr);
+        nlh::check_launch(what);
+    }
+    return true;
+}
+
+nlh_error_buffer *nlh_error_buffer_new(void) {
+    nlh_error_buffer *b = new nlh_error_buffer();
+    b->steps_accumulated = 0;
+    return b;
+}
+void nlh_error_buffer_free(nlh_error_buffer *b) { delete b; }
+int nlh_error_buffer_add_tensor(nlh_error_buffer *b, float *accumulator, int n) {
+    if (!b || (n > 0 && !accumulator) || n < 0) { nlh::fail("nlh_error_buffer_add_tensor: bad argument"); return -1; }
+    b->acc.push_back(accumulator);
+    b->n.push_back(n);
+    return (int)b->acc.size() - 1;
+}
+long long nlh_error_buffer_steps(const nlh_error_buffer *b) { return b->steps_accumulated; }
+void nlh_error_buffer_accumulate(nlh_error_buffer *b, const float *const *level_grads) {
+    eb_launch(b->acc, level_grads, b->n, 0, 0.f, "nlh_error_buffer_accumulate");
+    b->steps_accumulated += 1;
+}
+void nlh_error_buffer_apply_and_reset(nlh_error_buffer *b, float *const *params, float lr) {
+    if (b->steps_accumulated <= 0) return;
+    std::vector<float *> dst(params, params + b->acc.size());
+    eb_launch(dst, b->acc.data(), b->n, 1, lr, "nlh_error_buffer_apply_and_reset");
+    b->steps_accumulated = 0;
+}
+int nlh_error_buffer_health_check(const nlh_error_buffer *b, const float *const *single_step_grads, float *ratio) {
+    if (b->acc.size() > (size_t)nlh::kEbMax) { nlh::fail("nlh_error_buffer_health_check: more than %d tensors", nlh::kEbMax); return -1; }
+    const nlh::ErrorScope es;
+    float *out = nlh::scratch(15, 2 * sizeof(float));
+    if (es.failed()) return -1;
+    nlh::EbBatch e;
+    e.count = 0;
+    for (size_t i = 0; i < b->acc.size(); i++) {
+        if (b->n[i] <= 0) continue;
+        const int c = e.count++;
+        e.dst[c] = b->acc[i];
+        e.src[c] = const_cast<float *>(single_step_grads[i]);
+        e.n[c] = b->n[i];
+    }
+    hipLaunchKernelGGL(nlh::eb_norm_sq_kernel, dim3(1), dim3(nlh::kCmsThreads), 0, nlh::stream(), e, 0, out);
+    hipLaunchKernelGGL(nlh::eb_norm_sq_kernel, dim3(1), dim3(nlh::kCmsThreads), 0, nlh::stream(), e, 1, out);
+    nlh::check_launch("nlh_error_buffer_health_check");
+    float h[2] = {0.f, 0.f};
+    nlh::check_hip(hipMemcpyAsync(h, out, sizeof(h), hipMemcpyDeviceToHost, nlh::stream()), "health_check: copy out");
+    nlh::check_hip(hipStreamSynchronize(nlh::stream()), "health_check: synchronize");
+    if (es.failed()) return -1;
+    const float single = sqrtf(h[1]);
+    if (single < 1e-12f) return 0;   // None
+    *ratio = sqrtf(h[0]) / single;
+    return 1;
+}
+
+// ── ContextState (core/src/conductor.rs:156-221) ─────────────────────────────
+void nlh_context_state_reset(float *const *buffers, const int *n, int count) {
+    std::vector<float *> dst(buffers, buffers + count);
+    std::vector<int> nn(n, n + count);
+    eb_launch(dst, nullptr, nn, 2, 0.f, "nlh_context_state_reset");
+}
+void nlh_context_state_seed_self_ref(float *mems, const float *m_k_init, const float *m_v_init, const float *m_q_init,
+                                     const float *m_eta_init, const float *m_alpha_init, const float *m_mem_init,
+                                     int batch, int d) {
+    if (batch <= 0 || d <= 0 || !mems) { nlh::fail("nlh_context_state_seed_self_ref: bad argument"); return; }
+    const int dd = d * d;
+    // the five projection memories are seeded together or not at all (SelfRefState::from_init)
+    const float *proj[5] = {m_k_init, m_v_init, m_q_init, m_eta_init, m_alpha_init};
+    const bool have_proj = m_k_init != nullptr;
+    if (have_proj && !(m_v_init && m_q_init && m_eta_init && m_alpha_init)) {
+        nlh::fail("nlh_context_state_seed_self_ref: m_k_init is given, so m_v/m_q/m_eta/m_alpha_init must be too");
+        return;
+    }
+    std::vector<float *> dst;
+    std::vector<const float *> src;
+    for (int b = 0; b < batch; b++) {
+        float *chain = mems + (size_t)b * 6 * dd;
+        if (have_proj)
+            for (int c = 0; c < 5; c++) { dst.push_back(chain + (size_t)c * dd); src.push_back(proj[c]); }
+        if (m_mem_init) { dst.push_back(chain + (size_t)5 * dd); src.push_back(m_mem_init); }
+    }
+    std::vector<int> nn(dst.size(), dd);
+    eb_launch(dst, src.data(), nn, 3, 0.f, "nlh_context_state_seed_self_ref");
+}
+
 void cms_combine_gate_rocm(const float *const *y_levels, int k, const float *attn_out,
                            float *y_combined, float *gate, float *gated, long long n) {
     if (k < 1 || k > kMaxLevels) { fail("cms_combine_gate_rocm: k=%d must be in [1, %d].", k, kMaxLevels); return; }
@@ -274,7 +431,19 @@ void memory_read_only_f32_rocm(const float *q_mem, const float *m, float *y, lon
     const size_t lds = (size_t)(hd + 64) * (hd + 1) * sizeof(float);
     if (lds > 64 * 1024) { fail("memory_read_only_f32_rocm: head_dim=%d too large for the LDS tile.", hd); return; }
     hipLaunchKernelGGL(memory_read_only_kernel, dim3((unsigned)((n_tokens + 63) / 64), nh),
-                       dim3(kCmsThreads), lds, stream(), q_mem, m, y, n_tokens, nh, hd);
+                       dim3(kCmsThreads), lds, stream(), q_mem, m, y, n_tokens, nh, hd, 0);
+    check_launch("memory_read_only_kernel");
+}
+
+// Its backward (the frozen-read adapter, core/src/opaque_adapters.rs:1030-1047, per head):
+// d_q[t, h*hd+j] = sum_i M[h,i,j] d_y[t, h*hd+i].  No gradient reaches M: the level did not fire.
+void memory_read_only_backward_f32_rocm(const float *d_y, const float *m, float *d_q, long long n_tokens, int nh,
+                                        int hd) {
+    if (n_tokens <= 0 || nh <= 0 || hd <= 0) return;
+    const size_t lds = (size_t)(hd + 64) * (hd + 1) * sizeof(float);
+    if (lds > 64 * 1024) { fail("memory_read_only_backward_f32_rocm: head_dim=%d too large for the LDS tile.", hd); return; }
+    hipLaunchKernelGGL(memory_read_only_kernel, dim3((unsigned)((n_tokens + 63) / 64), nh),
+                       dim3(kCmsThreads), lds, stream(), d_y, m, d_q, n_tokens, nh, hd, 1);
     check_launch("memory_read_only_kernel");
 }
 

@@ -17,7 +17,7 @@ from typing import List, Optional
 import torch
 
 from . import dispatch as D
-from .cms import Conductor, FrequencyAwareAdamW, Pulse
+from .cms import Conductor, ContextState, ErrorBuffer, FrequencyAwareAdamW, Pulse
 from .ffi import lib
 
 F32_MAX = 3.4028234663852886e38
@@ -176,6 +176,12 @@ class MagLayer:
             for lv in range(self.k):
                 self.m_state[lv], self.s_state[lv] = self._m_all[lv], self._s_all[lv]
 
+    def context_state(self, bs):
+        """The layer's persistent memories as a ContextState (conductor.rs:156-221): reset() at a document
+        boundary zeroes every level's M and S in place (addresses stay fixed for captured graphs)."""
+        self.ensure_state(bs)
+        return ContextState(self.m_state, self.s_state)
+
     # ── one level ────────────────────────────────────────────────────────────
     def _level_forward(self, lv, x2, bs, s, active, ops=None):
         """gpu_memory_forward: projections, L2 norm, gates, head split, recurrence."""
@@ -300,8 +306,8 @@ class MagLayer:
         B, n = bs * nh, bs * s
         if not c["active"]:
             # read-only level: y = M_h q, only the q path carries gradient
-            m = c["m_shared"].view(nh, hd, hd)
-            dq = torch.einsum("hij,bthi->bthj", m, d_y.view(bs, s, nh, hd)).reshape(n, d)
+            dq = _new(n, d)
+            D.call("memory_read_only_backward_f32_rocm", d_y, c["m_shared"], dq, n, nh, hd)
             g.w_q += _wgrad(dq, x2)
             return dq @ lp.w_q
         dyh = _new(B, s, hd)
@@ -486,6 +492,22 @@ class MagTrainer:
             if grp >= 0 and any(w is lp.b_theta for lp in p.levels):
                 self.opt.set_clamp(tid, -10.0, 2.0)
         self.scale = torch.zeros(2, dtype=torch.float32, device="cuda")
+        # gradients that reach a level while it is frozen wait here until it fires (conductor.rs:224-261)
+        self.error_buffers = [ErrorBuffer(l.tensors()) for l in p.levels]
+
+    def _optimizer_and_error_buffers(self, pulse):
+        """The step's parameter updates in the reference's order (core/tests/test_cms.rs:66-84): the
+        optimizer for everything that fired, then, for a level that fired with gradients waiting from its
+        frozen steps, their plain gradient step; a frozen level's gradients of this step join its buffer."""
+        layer = self.layer
+        for lv in range(layer.k):
+            if not pulse.active_levels[lv]:
+                self.error_buffers[lv].accumulate(self.grads.levels[lv].tensors())
+        self.opt.step(pulse, self.lr, self.max_grad_norm, self.scale)
+        for lv in range(layer.k):
+            eb = self.error_buffers[lv]
+            if pulse.active_levels[lv] and eb.steps_accumulated > 0:
+                eb.apply_and_reset(layer.p.levels[lv].tensors(), self.lr)
 
     def _forward_backward(self, x, d_out):
         out, cache = self.layer.forward(x)
@@ -530,7 +552,7 @@ class MagTrainer:
         xs.copy_(x)
         ds.copy_(d_out)
         graph.replay()
-        self.opt.step(pulse, self.lr, self.max_grad_norm, self.scale)
+        self._optimizer_and_error_buffers(pulse)
         layer.conductor.advance()
         return out
 
@@ -540,6 +562,6 @@ class MagTrainer:
         _, g = self.layer.backward(cache, d_out_fn(out))
         for dst, src in zip(self.grads.tensors(), g.tensors()):
             dst.copy_(src)
-        self.opt.step(cache["pulse"], self.lr, self.max_grad_norm, self.scale)
+        self._optimizer_and_error_buffers(cache["pulse"])
         self.layer.conductor.advance()
         return out

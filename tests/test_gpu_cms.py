@@ -95,3 +95,96 @@ def test_frozen_level_read_only():
     D.call("memory_read_only_f32_rocm", dev(q), dev(m), y, n_tok, nh, hd)
     want = np.einsum("hij,thj->thi", m.astype(np.float64), q.reshape(n_tok, nh, hd)).reshape(n_tok, nh * hd)
     assert_close("y", host(y), want, 1e-5)
+
+
+# ── ErrorBuffer (core/src/conductor.rs:224-261; known answers of its unit tests, :320-381) ──
+def _level_like(d):
+    sizes = [d * d, d * d, d * d, 2 * d, 1, 2 * d, 1, 2 * d, 1]
+    return [zeros(n) for n in sizes]
+
+
+def test_error_buffer_accumulates_applies_and_resets():
+    from nl_hecate_amd.cms import ErrorBuffer
+    d = 4
+    buf = ErrorBuffer(_level_like(d))
+    g1, g2 = _level_like(d), _level_like(d)
+    g1[0].fill_(1.0)
+    g2[0].fill_(2.0)
+    g2[4].fill_(-0.5)   # a bias
+    buf.accumulate(g1)
+    assert buf.steps_accumulated == 1
+    buf.accumulate(g2)
+    assert buf.steps_accumulated == 2
+    torch.cuda.synchronize()
+    assert torch.all(buf.grads[0] == 3.0) and torch.all(buf.grads[4] == -0.5) and not buf.grads[1].any()
+    params = _level_like(d)
+    params[0].fill_(10.0)
+    buf.apply_and_reset(params, 0.1)
+    torch.cuda.synchronize()
+    assert_close("w_k_mem", host(params[0]), np.full(d * d, 10.0 - 0.1 * 3.0, np.float32), 1e-6)
+    assert_close("b_alpha", host(params[4]), np.full(1, 0.05, np.float32), 1e-6)
+    assert buf.steps_accumulated == 0 and not any(g.any() for g in buf.grads)
+    before = [p.clone() for p in params]
+    buf.apply_and_reset(params, 0.1)   # nothing accumulated: parameters untouched (conductor.rs:247)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(before, params))
+
+
+def test_error_buffer_health_check():
+    from nl_hecate_amd.cms import ErrorBuffer
+    d = 4
+    buf = ErrorBuffer(_level_like(d))
+    g = _level_like(d)
+    g[0].fill_(1.0)
+    for _ in range(7):
+        buf.accumulate(g)
+    assert abs(buf.health_check(g) - 7.0) < 1e-5          # conductor.rs:355-373
+    assert buf.health_check(_level_like(d)) is None        # :376-381: zero single-step norm
+    h = _level_like(d)
+    for i, t in enumerate(h):
+        t.copy_(torch.from_numpy(rnd(t.numel())))
+    buf2 = ErrorBuffer(_level_like(d))
+    buf2.accumulate(h)
+    buf2.accumulate(g)
+    acc = np.sqrt(sum(float(((host(a) + host(b)) ** 2).sum()) for a, b in zip(h, g)))
+    single = np.sqrt(sum(float((host(a) ** 2).sum()) for a in h))
+    assert abs(buf2.health_check(h) - acc / single) < 1e-5 * acc / single
+
+
+# ── ContextState (core/src/conductor.rs:156-221) ──
+def test_context_state_reset_and_seed_self_ref():
+    from nl_hecate_amd.cms import ContextState
+    chains, d, k = 6, 8, 2
+    mem = [dev(rnd(chains, d, d)) for _ in range(k)]
+    mom = [dev(rnd(chains, d, d)) for _ in range(k)]
+    sr = [dev(rnd(chains, 6, d, d)), None]
+    ptrs = [t.data_ptr() for t in mem + mom + [sr[0]]]
+    cs = ContextState(mem, mom, sr)
+    inits = [dict(m_k_init=dev(rnd(d, d)), m_v_init=dev(rnd(d, d)), m_q_init=dev(rnd(d, d)), m_eta_init=dev(rnd(d, d)),
+                  m_alpha_init=dev(rnd(d, d)), m_mem_init=dev(rnd(d, d))), dict()]
+    cs.seed_self_ref(inits)
+    torch.cuda.synchronize()
+    for c, n in enumerate(("m_k_init", "m_v_init", "m_q_init", "m_eta_init", "m_alpha_init", "m_mem_init")):
+        for b in range(chains):
+            assert torch.equal(sr[0][b, c], inits[0][n]), (n, b)
+    # static projections: only m_mem is seeded, the five projection memories keep their values
+    keep = sr[0].clone()
+    new_mem = dev(rnd(d, d))
+    cs.seed_self_ref([dict(m_mem_init=new_mem)])
+    torch.cuda.synchronize()
+    assert torch.equal(sr[0][:, :5], keep[:, :5]) and all(torch.equal(sr[0][b, 5], new_mem) for b in range(chains))
+    cs.reset()
+    torch.cuda.synchronize()
+    assert not any(t.any() for t in mem + mom) and not sr[0].any()
+    assert ptrs == [t.data_ptr() for t in mem + mom + [sr[0]]], "reset is in place"
+
+
+def test_frozen_read_backward_kernel():
+    bs, s, nh, hd = 2, 70, 3, 16
+    d, n = nh * hd, 2 * 70
+    dy, m = rnd(n, d), rnd(nh, hd, hd)
+    dq = zeros(n, d)
+    D.call("memory_read_only_backward_f32_rocm", dev(dy), dev(m), dq, n, nh, hd)
+    torch.cuda.synchronize()
+    want = np.einsum("hij,thi->thj", m.astype(np.float64), dy.reshape(n, nh, hd).astype(np.float64)).reshape(n, d)
+    assert_close("d_q", host(dq), want)

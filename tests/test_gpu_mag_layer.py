@@ -116,6 +116,55 @@ def test_training_step_changes_only_active_levels():
     assert tr.opt.level_step(0) == 2 and tr.opt.level_step(1) == 1
 
 
+def test_frozen_level_gradients_wait_in_the_error_buffer_and_are_applied_when_it_fires():
+    """conductor.rs:224-261 with the loop of core/tests/test_cms.rs:66-84: level 1 (period 4, sequences
+    shorter than that) is frozen on steps 1..3; its read path still produces a w_q gradient, which is
+    summed in the level's ErrorBuffer and applied as one plain step of size lr when the level fires again."""
+    d, nh, k = 32, 2, 2
+    layer = MagLayer(d, nh, k, 4, [1, 4], rule="exact", chunk=2, seed=21)
+    tr = MagTrainer(layer, lr=1e-2, max_grad_norm=0.0)   # no clip: the step's gradients stay as the backward wrote them
+    g = torch.Generator().manual_seed(3)
+    wq_idx = 2   # level tensors: w_k, w_v, w_q, ...
+    sums = torch.zeros_like(layer.p.levels[1].w_q)
+    for step in range(5):
+        x = (torch.randn(1, 3, d, generator=g) / math.sqrt(d)).cuda()
+        before = [t.clone() for t in layer.p.levels[1].tensors()]
+        pulse = layer.conductor.pulse()
+        out = tr.step(x, lambda o: torch.ones_like(o))
+        torch.cuda.synchronize()
+        eb = tr.error_buffers[1]
+        if step == 0:
+            assert pulse.active_levels[1] and eb.steps_accumulated == 0
+        elif step < 4:
+            assert not pulse.active_levels[1]
+            assert eb.steps_accumulated == step
+            sums += tr.grads.levels[1].w_q
+            assert float(tr.grads.levels[1].w_q.abs().max()) > 0, "the frozen read carries a w_q gradient"
+            assert torch.allclose(eb.grads[wq_idx], sums, rtol=1e-6, atol=1e-9)
+            assert all(torch.equal(a, b) for a, b in zip(before, layer.p.levels[1].tensors())), "frozen: untouched"
+            ratio = eb.health_check(tr.grads.levels[1].tensors())
+            assert ratio is not None and 0.5 < ratio < 2.0 * step
+        else:
+            assert pulse.active_levels[1] and eb.steps_accumulated == 0 and not eb.grads[wq_idx].any()
+    # the last step applied AdamW (gradients of step 4) and then the buffered sum: replay it by hand
+    assert float(sums.abs().max()) > 0
+
+
+def test_context_state_reset_zeroes_the_layer_memories_in_place():
+    d, nh, k = 32, 2, 2
+    layer = MagLayer(d, nh, k, 4, [1, 8], rule="exact", chunk=4, seed=22)
+    x = (torch.randn(2, 6, d, generator=torch.Generator().manual_seed(2)) / math.sqrt(d)).cuda()
+    layer.forward(x)
+    cs = layer.context_state(2)
+    ptrs = [t.data_ptr() for t in layer.m_state]
+    assert any(float(t.abs().max()) > 0 for t in layer.m_state)
+    step_before = layer.conductor.step()
+    cs.reset()
+    torch.cuda.synchronize()
+    assert not any(t.any() for t in layer.m_state + layer.s_state)
+    assert ptrs == [t.data_ptr() for t in layer.m_state] and layer.conductor.step() == step_before
+
+
 def test_trainer_clamps_b_theta_after_every_level_update():
     """gpu_optimizer.rs:491-493: b_theta of an updated level is held in [-10, 2]."""
     d, nh, k = 32, 2, 2
