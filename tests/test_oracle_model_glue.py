@@ -98,17 +98,104 @@ def test_pooling_pair_against_torch(C=3):
     assert np.allclose(G.repeat_upsample_1d_backward(gu, C), pt.grad.numpy(), atol=1e-14)
 
 
-def test_m3_helpers_closed_forms():
-    n = 8
-    g, m1, m2, v, w = (R.standard_normal(n) for _ in range(5))
-    v = np.abs(v)
-    a, b, c = G.m3_ema_update(m1, m2, v, g, 0.9, 0.99, 0.999, True)
-    assert np.allclose(a, 0.9 * m1 + 0.1 * g) and np.allclose(c, 0.99 * v + 0.01 * g * g)
-    assert np.allclose(b, 0.999 * m2 + 0.001 * g)
-    assert np.array_equal(G.m3_ema_update(m1, m2, v, g, 0.9, 0.99, 0.999, False)[1], m2)
-    assert np.allclose(G.m3_apply_1d(w, m1, m2, v, 0.1, 0.5, 1e-8, 0.7), w - 0.1 * (m1 + 0.5 * m2) / (np.sqrt(v / 0.7) + 1e-8))
-    assert np.allclose(G.m3_apply_2d(w, m1, m2, 0.1, 0.5), w - 0.1 * (m1 + 0.5 * m2))
-    assert np.allclose(G.m3_ns_poly(w, m1, m2, 3.4445, -4.775, 2.0315), 3.4445 * w - 4.775 * m1 + 2.0315 * m2)
+def _golden_m3():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "m3_known_answers.json")) as f:
+        return json.load(f)
+
+
+def test_m3_moment_updates_match_torch_adam_state_and_the_reference_known_answers():
+    """m3_ema_update is Adam's pair of moment updates plus a slow first moment: checked against the state
+    torch.optim.Adam keeps (exp_avg, exp_avg_sq) over three steps, and against the known answers of the
+    reference's own tests (first step from zero = theta * grad with theta = 1 - eta; constant gradient
+    converges to it)."""
+    n, b1, b2, b3 = 11, 0.9, 0.99, 0.999
+    w = torch.nn.Parameter(torch.zeros(n, dtype=torch.float64))
+    opt = torch.optim.Adam([w], lr=1e-3, betas=(b1, b2), eps=1e-8)
+    slow = torch.optim.Adam([torch.nn.Parameter(torch.zeros(n, dtype=torch.float64))], lr=1e-3, betas=(b3, b2))
+    m1, m2, v = np.zeros(n), np.zeros(n), np.zeros(n)
+    for step in range(3):
+        g = R.standard_normal(n)
+        for o in (opt, slow):
+            o.param_groups[0]["params"][0].grad = T(g)
+            o.step()
+        m1, m2, v = G.m3_ema_update(m1, m2, v, g, b1, b2, b3, True)
+        st = opt.state[w]
+        assert np.allclose(m1, st["exp_avg"].numpy(), atol=1e-15) and np.allclose(v, st["exp_avg_sq"].numpy(), atol=1e-15)
+        assert np.allclose(m2, slow.state[slow.param_groups[0]["params"][0]]["exp_avg"].numpy(), atol=1e-15)
+    keep = m2.copy()
+    assert np.array_equal(G.m3_ema_update(m1, m2, v, g, b1, b2, b3, False)[1], keep), "update_m2 = 0 leaves the slow moment"
+    ka = _golden_m3()
+    one = ka["single_step"]
+    z = np.zeros(3)
+    got = G.m3_ema_update(z, z, z, np.array(one["grad"]), one["eta"], 0.99, 0.999, True)[0]
+    assert np.abs(got - np.array(one["update"])).max() < one["abs_tol"]
+    cv = ka["ema_convergence"]
+    m = np.zeros(1)
+    for _ in range(cv["steps"]):
+        m = G.m3_ema_update(m, m, m, np.array([cv["grad"]]), cv["eta"], 0.99, 0.999, False)[0]
+    assert abs(m[0] - cv["expected"]) < cv["abs_tol"]
+
+
+def test_m3_parameter_updates_match_torch_adam_and_sgd_steps():
+    """m3_apply_1d with alpha = 0 is Adam's parameter update with the first-moment bias correction folded
+    into lr (torch: step = lr / bc1 * m / (sqrt(v) / sqrt(bc2) + eps)); the slow moment enters linearly
+    (alpha).  m3_apply_2d is a plain gradient step on o1 + alpha o2."""
+    n, b1, b2, lr, eps = 9, 0.9, 0.95, 3e-3, 1e-8
+    w0 = R.standard_normal(n)
+    w = torch.nn.Parameter(T(w0).clone())
+    opt = torch.optim.Adam([w], lr=lr, betas=(b1, b2), eps=eps)
+    ours, m1, m2, v = w0.copy(), np.zeros(n), np.zeros(n), np.zeros(n)
+    for step in range(1, 4):
+        g = R.standard_normal(n)
+        w.grad = T(g)
+        opt.step()
+        m1, m2, v = G.m3_ema_update(m1, m2, v, g, b1, b2, 0.999, True)
+        ours = G.m3_apply_1d(ours, m1, m2, v, lr / (1 - b1 ** step), 0.0, eps, 1 - b2 ** step)
+        assert np.allclose(ours, w.detach().numpy(), atol=1e-13)
+    al = 0.37
+    assert np.allclose(G.m3_apply_1d(w0, m1, m2, v, lr, al, eps, 0.7), G.m3_apply_1d(w0, m1 + al * m2, 0 * m2, v, lr, 0.0, eps, 0.7),
+                       atol=1e-15)
+    ws = torch.nn.Parameter(T(w0).clone())
+    sgd = torch.optim.SGD([ws], lr=lr)
+    ws.grad = T(m1 + al * m2)
+    sgd.step()
+    assert np.allclose(G.m3_apply_2d(w0, m1, m2, lr, al), ws.detach().numpy(), atol=1e-15)
+
+
+def _newton_schulz(m, iters, coef):
+    """The loop around m3_ns_poly (core/src/gpu_optimizer.rs:975-1000): X <- a X + b (X X^T) X + c (X X^T)^2 X."""
+    x = m.copy()
+    for _ in range(iters):
+        ata = x @ x.T
+        ax = ata @ x
+        x = G.m3_ns_poly(x, ax, ata @ ax, coef["a"], coef["b"], coef["c"])
+    return x
+
+
+def test_m3_newton_schulz_polynomial():
+    """On a scaled orthogonal matrix sigma Q one step must give p(sigma) Q with p(s) = a s + b s^3 + c s^5
+    (X X^T = sigma^2 I): a closed form that a swapped or mis-signed coefficient breaks.  Iterated on the
+    reference's test matrix the singular values move into the band around 1 the quintic is built for, and
+    its known answers hold (finite, non-zero, modified; zero iterations change nothing)."""
+    ka = _golden_m3()
+    co, ns = ka["coefficients"], ka["newton_schulz"]
+    q, _ = np.linalg.qr(R.standard_normal((5, 5)))
+    for sigma in (0.3, 0.8, 1.1):
+        got = _newton_schulz(sigma * q, 1, co)
+        p = co["a"] * sigma + co["b"] * sigma ** 3 + co["c"] * sigma ** 5
+        assert np.allclose(got, p * q, atol=1e-12)
+    d = ns["d"]
+    m = np.array([np.sin(0.37 * i + 0.1) * 0.5 for i in range(d * d)]).reshape(d, d)
+    x0 = m / np.linalg.norm(m)
+    out = _newton_schulz(x0, ns["iterations"], co)
+    assert np.isfinite(out).all() and np.linalg.norm(out) > ns["min_frobenius"] and np.abs(out - m).sum() > ns["min_l1_change"]
+    sv = np.linalg.svd(out, compute_uv=False)
+    big = np.linalg.svd(x0, compute_uv=False) > 1e-3
+    assert np.all((sv[big] > 0.6) & (sv[big] < 1.3)), sv
+    z = np.array(ns["zero_iterations_matrix"], float).reshape(3, 3)
+    assert np.array_equal(_newton_schulz(z, 0, co), z)
 
 
 def test_swiglu_matches_torch_silu_mlp_and_autograd():
