@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "../../include/nl_hecate_ffi.h"
+#include "rule_args.h"
 #include "rule_common.h"
 
 namespace nlh {
@@ -36,17 +37,6 @@ static __global__ void zero_fill_kernel(float *__restrict__ p, size_t n) {
 }
 
 // ───────────────────────────── forward ─────────────────────────────────────
-struct FwdArgs {
-    const float *k, *v, *q, *alpha, *theta, *eta, *m_initial, *s_initial;
-    float *m_out, *s_out, *y;
-    int seq_len, input_stride, ckpt_interval, parts;
-    long long m_stride;      // elements between chains in m_initial / s_initial
-    long long state_stride;  // elements between chains in m_out / s_out
-    float error_clip, m_norm_max;
-};
-
-enum { STORE_NONE = 0, STORE_TRAJ = 1, STORE_CKPT = 2 };
-
 // FROZEN: the frozen-M0 chunkwise rule (core/kernels/titans_chunkwise_forward.cu):
 // errors of a chunk are taken against the chunk-start M; ckpt_interval is the
 // chunk size and the stored checkpoints are the chunk-boundary states.
@@ -246,17 +236,6 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
 // Reverse sweep over [t_start, t_end) of every chain, reading the trajectory
 // M_{t_start..t_end}, S_{t_start..t_end-1} from memory (the reference's
 // *_backward and *_backward_segment contract).
-struct BwdArgs {
-    const float *k, *v, *q, *alpha, *theta, *eta, *m_states, *s_states, *d_y;
-    const float *d_m_seed, *d_s_seed;      // [B, dd] or null (zero)
-    float *d_k, *d_v, *d_q, *d_alpha, *d_theta, *d_eta;
-    float *ws_dq, *ws_dk, *ws_gate;        // partial sums when parts > 1
-    float *d_m_out, *d_s_out;              // [B, dd]
-    int seq_len, t_start, t_end, parts, batch;
-    long long traj_stride;                 // elements between chains in m_states
-    float error_clip;
-};
-
 // FROZEN: the range is one chunk of the frozen-M0 rule
 // (core/kernels/titans_chunkwise_backward.cu): errors and M^T d_err use the
 // chunk-start M (m_states slot 0), d_M propagates by retention only, and the
@@ -579,12 +558,22 @@ static void launch_fwd_c(const FwdArgs &a, int batch, bool coupled) {
     check_launch("rule_fwd_kernel");
 }
 
+// head sizes with register-resident kernels
+static bool tiled_size(int d) { return d == 8 || d == 16 || d == 32 || d == 64 || d == 128; }
+
+// Always launches (returns true) for d >= 1: head sizes without a tiled kernel, and clip / projection
+// where the tiled layout would split a chain over workgroups (d = 128), take the general kernels.
 template <bool HAS_S, int STORE, bool FROZEN = false>
 static bool launch_fwd(FwdArgs a, int d, int batch) {
+    if (d < 1) return false;
     const bool coupled = coupled_needed(a.error_clip, a.m_norm_max);
-    const int rpl = pick_rpl(d, batch, coupled);
-    a.parts = ceil_div(d, rows_per_wg(d, rpl));
-    if (coupled && a.parts != 1) return false;
+    const int rpl = tiled_size(d) ? pick_rpl(d, batch, coupled) : 1;
+    a.parts = tiled_size(d) ? ceil_div(d, rows_per_wg(d, rpl)) : 1;
+    if (!tiled_size(d) || (coupled && a.parts != 1)) {
+        a.parts = 1;
+        launch_fwd_generic(a, d, batch, HAS_S, STORE, FROZEN);
+        return true;
+    }
     switch (d) {
         case 8: launch_fwd_c<8, 1, HAS_S, STORE, FROZEN>(a, batch, coupled); return true;
         case 16: launch_fwd_c<16, 1, HAS_S, STORE, FROZEN>(a, batch, coupled); return true;
@@ -625,10 +614,15 @@ static size_t bwd_partial_floats(int d, int batch, int seq_len, int rpl) {
 template <bool HAS_S, bool FROZEN = false>
 static bool launch_bwd(BwdArgs a, int d, float *ws = nullptr, bool whole_chain = false) {
     const ErrorScope es;
+    if (d < 1) return false;
     const bool coupled = a.error_clip > 0.f;
-    const int rpl = bwd_rpl(d, a.batch, coupled, whole_chain);
-    a.parts = ceil_div(d, rows_per_wg(d, rpl));
-    if (coupled && a.parts != 1) return false;
+    const int rpl = tiled_size(d) ? bwd_rpl(d, a.batch, coupled, whole_chain) : 1;
+    a.parts = tiled_size(d) ? ceil_div(d, rows_per_wg(d, rpl)) : 1;
+    if (!tiled_size(d) || (coupled && a.parts != 1)) {
+        a.parts = 1;
+        launch_bwd_generic(a, d, HAS_S, FROZEN);
+        return true;
+    }
     if (a.parts > 1) {
         size_t n = (size_t)a.parts * a.batch * a.seq_len;
         if (ws) {
@@ -706,8 +700,8 @@ bool check_dims(const char *fn, int seq_len, int d, int batch) {
 }
 
 void unsupported(const char *fn, int d, bool coupled) {
-    fail("%s: d=%d%s is not supported by the gfx950 kernels (d in {8,16,32,64,128}; "
-         "clip / M-norm projection need d <= 64).", fn, d, coupled ? " with clip/projection" : "");
+    fail("%s: d=%d%s is not served by this entry point (the tiled kernels cover d in {8,16,32,64,128}, "
+         "the general ones any d >= 1 within their LDS limit).", fn, d, coupled ? " with clip/projection" : "");
 }
 
 

@@ -94,8 +94,8 @@ def test_titans_forward_reference_recipe():
 
 
 def test_titans_forward_seq_len_1():
-    """test_cuda_titans.rs:99-128: d=4 is below the tiled kernels' range -> d=8 here."""
-    x = _ref_recipe(1, 8, (400, 500, 600))
+    """test_cuda_titans.rs:99-128: d=4, s=1, seeds 400/500/600 (the general-head-size kernels)."""
+    x = _ref_recipe(1, 4, (400, 500, 600))
     y, ms, ss = gpu_titans_forward(x)
     yo, mo, so = orc.titans_forward_batch(x["k"], x["v"], x["q"], x["alpha"], x["theta"], x["eta"],
                                           x["m0"], x["s0"])
@@ -313,8 +313,9 @@ def test_argument_errors_are_reported():
         D.call("titans_forward_f32_cuda", z, z, z, z, z, z, z, z, z, z, z, 4, 0, 1, 4, 0, 0.0, 0.0)
         assert b"d=0" in lib.nlh_last_error()
         lib.nlh_clear_error()
-        D.call("titans_forward_f32_cuda", z, z, z, z, z, z, z, z, z, z, z, 4, 24, 1, 4, 576, 0.0, 0.0)
-        assert b"not supported" in lib.nlh_last_error()
+        # refused before any launch: the per-token vectors of this head size do not fit in LDS
+        D.call("titans_forward_f32_cuda", z, z, z, z, z, z, z, z, z, z, z, 4, 20000, 1, 4, 0, 0.0, 0.0)
+        assert b"beyond the general kernels" in lib.nlh_last_error()
         lib.nlh_clear_error()
         D.call("titans_forward_ckpt_f32_cuda", z, z, z, z, z, z, z, z, z, z, z, 4, 8, 0, 0.0, 0.0)
         assert b"checkpoint_interval" in lib.nlh_last_error()
