@@ -633,6 +633,50 @@ void memory_grads_fused_rocm(const float *d_k_heads, const float *d_v_heads, con
                              float *d_k_in, float *d_v, float *d_q_in, float *d_alpha, float *d_theta, float *d_eta,
                              int bs, int s, int nh, int hd, float eps);
 
+/* ── the layer step's glue with strided operands (no symbols in cuda_ffi.rs) ───────────────────────────
+ * The reference's layer step (core/src/gpu_forward.rs:864-1071, gpu_backward.rs:212-435) runs its projections as
+ * one cuBLAS call each and streams every [tokens, d] tensor through a dozen small kernels.  Here the projections
+ * of x are split-bf16 GEMMs over packed operands; these entry points let several producers fill column slabs of
+ * ONE operand, and read projection outputs in place as column ranges of a wider GEMM output (row stride ld). */
+/* As split_pack_bf16_rocm with row strides: source rows src_ld floats apart; in row r of out (out_ld bf16 values
+ * apart) source i, column c goes to i*d + c, its hi part at off_h1 + and off_h2 +, its lo part at off_l +. */
+void split_pack_bf16_ld_rocm(const float *const *srcs, int count, long long src_ld, uint16_t *out, long long n, int d,
+                             long long out_ld, long long off_h1, long long off_l, long long off_h2);
+/* The packed fp32 weight rows [rows, d] -> wb [rows, 3d] = (Wh | Wl | Wh) per row, the right operand of the
+ * forward projections against x packed as (xh | xh | xl), and wstack [3*rows_stack, d] = (Wh ; Wh ; Wl) of the
+ * first rows_stack rows, the right operand of d_x = P . wstack for P packed as (H | L | H). */
+void split_pack_weights_rocm(const float *pack, int rows, int rows_stack, int d, uint16_t *wb, uint16_t *wstack);
+/* memory_inputs_fused_rocm on k_mem, v_mem, q_mem with row stride ld (floats); 16-byte accesses, so head_dim must
+ * be a multiple of 4 and nh*hd <= 1024.  Sums run in another order than in memory_inputs_fused_rocm.
+ * normalise_in_place == 0 leaves k_mem and q_mem as they came (the heads still get the normalised rows): a
+ * backward that divides by k_norms / q_norms again (level_grads_packed_rocm, inputs_raw) saves the write. */
+void level_inputs_fused_rocm(float *k_mem, const float *v_mem, float *q_mem, long long ld, const float *w_alpha,
+                             const float *b_alpha, const float *w_theta, const float *b_theta, const float *w_eta,
+                             const float *b_eta, float *k_norms, float *q_norms, float *alpha, float *theta, float *eta,
+                             void *k_heads, void *v_heads, void *q_heads, float *alpha_heads, float *theta_heads,
+                             float *eta_heads, int bs, int s, int nh, int hd, float eps, int heads_bf16,
+                             int normalise_in_place);
+/* memory_grads_fused_rocm + gate_backward_cuda + split_pack_bf16_rocm in one pass (gpu_backward.rs:2047-2115):
+ * from the rule's head-major gradients to (a) the packed operand of the projection-gradient GEMMs, written into
+ * p_out (row stride p_ld) with d_k_in at column 0, d_v at d, d_q_in at 2d of each of the three positions
+ * off_h1 / off_l / off_h2, and (b) the gate projections' weight [2d] and bias [1] gradients, assigned.
+ * k_norm, v_mem, q_norm: the level's normalised k, its v and normalised q, row stride ld (inputs_raw != 0: k and
+ * q as projected, normalised here with k_norms / q_norms); alpha, theta, eta [bs*s]: the gate outputs. */
+void level_grads_packed_rocm(const float *d_k_heads, const float *d_v_heads, const float *d_q_heads,
+                             const float *d_alpha_heads, const float *d_theta_heads, const float *d_eta_heads,
+                             const float *k_norm, const float *v_mem, const float *q_norm, long long ld,
+                             const float *k_norms, const float *q_norms, const float *alpha, const float *theta,
+                             const float *eta, uint16_t *p_out, long long p_ld, long long off_h1, long long off_l,
+                             long long off_h2, float *d_w_alpha, float *d_b_alpha, float *d_w_theta, float *d_b_theta,
+                             float *d_w_eta, float *d_b_eta, int bs, int s, int nh, int hd, float eps, int inputs_raw);
+/* cms_combine_gate_rocm / cms_gate_backward_rocm with the attention output in bf16 (what the attention kernels
+ * write) and no y_combined copy; n a multiple of 4.  gated (fp32) and gated_packed ([n / d, 3d] bf16: hi | hi | lo of
+ * each row, the left operand of the output projection as a split-bf16 GEMM) may each be null. */
+void cms_combine_gate_bf16_rocm(const float *const *y_levels, int k, const uint16_t *attn_out, float *gate, float *gated,
+                                uint16_t *gated_packed, int d, long long n);
+void cms_gate_backward_bf16_rocm(const float *d_gated, const uint16_t *attn_out, const float *gate, int k, float *d_attn,
+                                 float *d_y_combined, long long n);
+
 /* ── Titans rule with an MLP memory: packed state [W1 (dh x d) | b1 (dh) | W2 (d x dh) | b2 (d)] ── */
 /* core/src/cuda_ffi.rs:854.  input_stride = elements between the chains' token tensors (seq_len * d),
  * m_stride = elements between the chains' trajectories ((seq_len + 1) * state_size); activation 0 GELU,

@@ -48,6 +48,8 @@ class MagParams:
     w_v: torch.Tensor
     w_o: torch.Tensor
     levels: List[MemoryLevelParams] = field(default_factory=list)
+    flat: Optional[torch.Tensor] = None    # gradients only: the one buffer all tensors are views of
+    pack: Optional[torch.Tensor] = None    # gradients only: the projection matrices' rows, [3(1+k)d, d]
 
     def tensors(self):
         return [self.w_q, self.w_k, self.w_v, self.w_o] + [t for l in self.levels for t in l.tensors()]
@@ -94,12 +96,13 @@ class MagLayer:
         self.rule, self.chunk = rule, chunk
         self.p = params if params is not None else init_params(d, k, seed)
         self.conductor = Conductor(k, list(periods))
-        # The 3 + 3k projections of x share one packed weight tensor (the parameters become views of
+        # The 3 + 3k projections of x and the output projection share one packed weight tensor (the parameters become views of
         # it), so that one pass per step produces their bf16 operand copies (see _split_operands).
-        tens = [self.p.w_q, self.p.w_k, self.p.w_v] + [w for l in self.p.levels for w in (l.w_k, l.w_v, l.w_q)]
+        tens = ([self.p.w_q, self.p.w_k, self.p.w_v] + [w for l in self.p.levels for w in (l.w_k, l.w_v, l.w_q)]
+                + [self.p.w_o])
         self._pack = torch.cat([w.reshape(d, d) for w in tens], 0).contiguous()
         views = [self._pack[i * d:(i + 1) * d] for i in range(len(tens))]
-        self.p.w_q, self.p.w_k, self.p.w_v = views[0], views[1], views[2]
+        self.p.w_q, self.p.w_k, self.p.w_v, self.p.w_o = views[0], views[1], views[2], views[-1]
         for lv, l in enumerate(self.p.levels):
             l.w_k, l.w_v, l.w_q = views[3 + 3 * lv], views[4 + 3 * lv], views[5 + 3 * lv]
         self.split_gemm = True
@@ -111,11 +114,13 @@ class MagLayer:
         self.s_state: List[Optional[torch.Tensor]] = [None] * k
 
     # Projections of x as "3 x bf16" products: x = xh + xl, W = Wh + Wl (bf16 pairs, 16 mantissa bits),
-    # x W^T ~ xh Wh^T + xl Wh^T + xh Wl^T as ONE bf16 GEMM with fp32 accumulation and fp32 output over the
-    # tripled contraction [xh | xl | xh] . [Wh | Wh | Wl]^T.  Agrees with the fp32 GEMM to 5e-6 and runs
-    # about three times faster on the bf16 matrix cores; the operand copies are made once per step.
-    # The backward's d_x = sum_s d_s W_s of a group of three projections is the same construction with
-    # the three upstream gradients side by side: [H | L | H] (9d wide) against [Wh^T | Wh^T | Wl^T].
+    # x W^T ~ xh Wh^T + xh Wl^T + xl Wh^T as ONE bf16 GEMM with fp32 accumulation over the tripled
+    # contraction [xh | xh | xl] . [Wh | Wl | Wh]^T.  Agrees with the fp32 GEMM to 5e-6 and runs about
+    # three times faster on the bf16 matrix cores; the operand copies are made once per step.
+    # The backward's d_x = sum_j g_j W_j over a set of projections j is the same construction with the
+    # upstream gradients side by side: P = [H | L | H] (H, L the hi / lo parts of [g_0 | g_1 | ...])
+    # against the rows [Wh ; Wh ; Wl] of those projections; and the weight gradients g_j^T x come from
+    # the same P as H^T xh + L^T xh + H^T xl.
     @staticmethod
     def _pack_split(srcs):
         """[n, d] float tensors -> [n, 3*len*d] bf16: [hi(all) | lo(all) | hi(all)] (one pass)."""
@@ -125,47 +130,78 @@ class MagLayer:
         lib.split_pack_bf16_rocm(ptrs, len(srcs), out.data_ptr(), n, d)
         return out
 
-    def _split_operands(self, x2):
-        d, groups = self.d, 1 + self.k
-        wh = self._pack.to(torch.bfloat16)
-        wl = (self._pack - wh.float()).to(torch.bfloat16)
-        wht, wlt = (w.view(groups, 3 * d, d).transpose(1, 2) for w in (wh, wl))   # [group, d_in, 3 d_out]
-        xa = self._pack_split([x2])                                               # [n, 3d]: xh | xl | xh
-        xw = torch.cat([xa[:, :d], xa[:, 2 * d:], xa[:, d:2 * d]], 1)             # [n, 3d]: xh | xh | xl
-        return xa, torch.cat([wh, wh, wl], 1), torch.cat([wht, wht, wlt], 2).contiguous(), xw
+    def _split_operands(self, x2, rows_stack=0):
+        """The step's packed operands: xa [n, 3d] = (xh | xh | xl); wb [15d.., 3d] = (Wh | Wl | Wh) per
+        weight row; wstack [3 * rows_stack, d] = (Wh ; Wh ; Wl) of the first rows_stack weight rows."""
+        d, n, rows = self.d, x2.shape[0], self._pack.shape[0]
+        xa = _new(n, 3 * d, dtype=torch.bfloat16)
+        ptrs = (ctypes.c_void_p * 1)(x2.data_ptr())
+        lib.split_pack_bf16_ld_rocm(ptrs, 1, d, xa.data_ptr(), n, d, 3 * d, 0, 2 * d, d)
+        wb = _new(rows, 3 * d, dtype=torch.bfloat16)
+        wstack = _new(max(3 * rows_stack, 1), d, dtype=torch.bfloat16)
+        lib.split_pack_weights_rocm(self._pack.data_ptr(), rows, rows_stack, d, wb.data_ptr(), wstack.data_ptr())
+        return dict(xa=xa, wb=wb, wstack=wstack, rows_stack=rows_stack)
 
     def _group_grads(self, ops, group, x2, grads3, weights3, wgrads3):
         """Projection group `group` (0: attention q, k, v; 1 + lv: level k, v, q): adds the three weight gradients
         grads3[s]^T x2 to wgrads3 and returns the input gradient sum_s grads3[s] @ weights3[s].
-        With split operands both come from ONE packing of the three upstream gradients, P = [H | L | H] (9d wide,
-        H / L the hi / lo bf16 parts of [g0 | g1 | g2]): the input gradient as P . [Wh^T | Wh^T | Wl^T], and the
-        weight gradients, the contraction now over tokens, by reading P as 3n rows (H_t, L_t, H_t) against the rows
-        (xh_t, xh_t, xl_t) of x: G^T x ~ H^T xh + L^T xh + H^T xl in one bf16 GEMM with fp32 accumulation, cut into
-        up to 16 slabs along the contraction like _wgrad."""
+        With split operands both come from ONE packing of the three upstream gradients, P = [H | L | H] (9d wide):
+        the input gradient as P . [Wh ; Wh ; Wl], and the weight gradients, the contraction now over tokens, by
+        reading P as 3n rows (H_t, L_t, H_t) against the rows (xh_t, xh_t, xl_t) of the packed x:
+        G^T x ~ H^T xh + L^T xh + H^T xl in one bf16 GEMM with fp32 accumulation, cut into up to 16 slabs along the
+        contraction like _wgrad."""
         d = self.d
         n = x2.shape[0]
-        if ops is None or not self.split_wgrad:
+        if ops is None:
             for g, w in zip(grads3, wgrads3):
                 w += _wgrad(g, x2)
-            if ops is None:
-                return grads3[0] @ weights3[0] + grads3[1] @ weights3[1] + grads3[2] @ weights3[2]
-            return torch.mm(self._pack_split(list(grads3)), ops[2][group].t(), out_dtype=torch.float32)
+            return grads3[0] @ weights3[0] + grads3[1] @ weights3[1] + grads3[2] @ weights3[2]
         P = self._pack_split(list(grads3))
+        wg = ops["wb"][group * 3 * d:(group + 1) * 3 * d]
+        stack = torch.cat([wg[:, :d], wg[:, :d], wg[:, d:2 * d]], 0)              # [9d, d]: Wh ; Wh ; Wl
+        if not self.split_wgrad:
+            for g, w in zip(grads3, wgrads3):
+                w += _wgrad(g, x2)
+            return torch.mm(P, stack, out_dtype=torch.float32)
         parts = next(p for p in (16, 8, 4, 2, 1) if (3 * n) % p == 0)
         rows = 3 * n // parts
-        dw = torch.bmm(P.view(parts, rows, 3 * d).transpose(1, 2), ops[3].view(parts, rows, d),
+        dw = torch.bmm(P.view(parts, rows, 3 * d).transpose(1, 2), ops["xa"].view(parts, rows, d),
                        out_dtype=torch.float32).sum(0)                            # [3 d_out, d_in]
         for i, w in enumerate(wgrads3):
             w += dw[i * d:(i + 1) * d]
-        return torch.mm(P, ops[2][group].t(), out_dtype=torch.float32)
+        return torch.mm(P, stack, out_dtype=torch.float32)
 
-    def _project(self, ops, x2, w, index):
-        """x2 @ w^T for the packed projection number `index` (w is its fp32 view)."""
+    def _project(self, ops, x2, w, index, bf16_out=False):
+        """x2 @ w^T for the packed projection number `index` (w is its fp32 view); bf16_out: rounded once, at
+        the GEMM's store (what the attention kernels take)."""
         if ops is None:
-            return x2 @ w.t()
-        xa, wb = ops[0], ops[1]
+            y = x2 @ w.t()
+            return y.to(torch.bfloat16) if bf16_out else y
         d = self.d
-        return torch.mm(xa, wb[index * d:(index + 1) * d].t(), out_dtype=torch.float32)
+        wt = ops["wb"][index * d:(index + 1) * d].t()
+        return torch.mm(ops["xa"], wt) if bf16_out else torch.mm(ops["xa"], wt, out_dtype=torch.float32)
+
+    def new_grads(self):
+        """A MagParams of zeroed gradients whose tensors are views of ONE buffer (`flat`): the 3 + 3k projection
+        matrices and w_o first, in the order of the packed weights, then the gate vectors."""
+        d, k = self.d, self.k
+        rows = self._pack.shape[0]
+        sizes = [rows * d] + [2 * d, 4, 2 * d, 4, 2 * d, 4] * k
+        flat = _zeros(sum(sizes))
+        offs = [0]
+        for z in sizes:
+            offs.append(offs[-1] + z)
+        gp = flat[:rows * d].view(rows, d)
+        mats = [gp[i * d:(i + 1) * d] for i in range(rows // d)]
+        levels = []
+        for lv in range(k):
+            o = offs[1 + 6 * lv:1 + 6 * lv + 6]
+            gate = [flat[o[0]:o[0] + 2 * d], flat[o[1]:o[1] + 1], flat[o[2]:o[2] + 2 * d], flat[o[3]:o[3] + 1],
+                    flat[o[4]:o[4] + 2 * d], flat[o[5]:o[5] + 1]]
+            levels.append(MemoryLevelParams(mats[3 + 3 * lv], mats[4 + 3 * lv], mats[5 + 3 * lv], *gate))
+        g = MagParams(mats[0], mats[1], mats[2], mats[-1], levels=levels)
+        g.flat, g.pack = flat, gp
+        return g
 
     def ensure_state(self, bs):
         """Creates the (zero) context memories of every level for batch size bs if they do not exist.
@@ -256,18 +292,29 @@ class MagLayer:
     # along the chain dimension and the rule runs once, forward and backward.
     def _levels_forward_stacked(self, na, x2, bs, s, ops):
         d, nh, hd, C = self.d, self.nh, self.hd, self.chunk
-        B = bs * nh
+        B, n = bs * nh, bs * s
         self.ensure_state(bs)
-        hdt = torch.bfloat16 if self.fused_glue else torch.float32   # the fused glue writes bf16 heads itself
-        kh, vh, qh = (_new(na * B, s, hd, dtype=hdt) for _ in range(3))
+        # k, v, q of every active level from one GEMM: [n, 3 na d], level lv at columns 3 lv d ..
+        ld = 3 * na * d
+        proj = torch.mm(ops["xa"], ops["wb"][3 * d:3 * d + ld].t(), out_dtype=torch.float32)
+        kh, vh, qh = (_new(na * B, s, hd, dtype=torch.bfloat16) for _ in range(3))
         ah, th, eh = _new(na * B, s), _new(na * B, s), _new(na * B, s)
         caches = []
         for lv in range(na):
+            lp = self.p.levels[lv]
             sl = slice(lv * B, (lv + 1) * B)
-            caches.append(self._level_inputs(lv, x2, bs, s, ops, tuple(t[sl] for t in (kh, vh, qh, ah, th, eh))))
+            k_mem, v_mem, q_mem = (proj[:, (3 * lv + i) * d:(3 * lv + i + 1) * d] for i in range(3))
+            k_norms, q_norms, alpha, theta, eta = (_new(n) for _ in range(5))
+            lib.level_inputs_fused_rocm(
+                k_mem.data_ptr(), v_mem.data_ptr(), q_mem.data_ptr(), ld, lp.w_alpha.data_ptr(), lp.b_alpha.data_ptr(),
+                lp.w_theta.data_ptr(), lp.b_theta.data_ptr(), lp.w_eta.data_ptr(), lp.b_eta.data_ptr(),
+                k_norms.data_ptr(), q_norms.data_ptr(), alpha.data_ptr(), theta.data_ptr(), eta.data_ptr(),
+                kh[sl].data_ptr(), vh[sl].data_ptr(), qh[sl].data_ptr(), ah[sl].data_ptr(), th[sl].data_ptr(),
+                eh[sl].data_ptr(), bs, s, nh, hd, 1e-8, 1, 0)
+            caches.append(dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, ld=ld, k_norms=k_norms, q_norms=q_norms,
+                               active=True, ops=ops, alpha=alpha, theta=theta, eta=eta))
         nc = (s + C - 1) // C
         mc, sc, yh = _new(na * B, nc + 1, hd * hd), _new(na * B, nc + 1, hd * hd), _new(na * B, s, hd)
-        kh, vh, qh = kh.to(torch.bfloat16), vh.to(torch.bfloat16), qh.to(torch.bfloat16)
         m0, s0 = self._m_all[:na].view(na * B, hd * hd), self._s_all[:na].view(na * B, hd * hd)
         D.call("titans_chunkwise_forward_bf16_rocm", kh, vh, qh, ah, th, eh, m0, s0, mc, sc, yh, s, hd, na * B, C)
         m0.copy_(mc[:, -1])
@@ -277,10 +324,12 @@ class MagLayer:
             y = _new(bs, s, d)
             D.call("transpose_heads_f32_cuda", yh[lv * B:(lv + 1) * B], y, bs, s, nh, hd, 0)
             ys.append(y)
-        return ys, caches, dict(na=na, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc)
+        return ys, caches, dict(na=na, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc, proj=proj)
 
-    def _levels_backward_stacked(self, st, caches, x2, d_y, bs, s, grads):
-        nh, hd, C, na = self.nh, self.hd, self.chunk, st["na"]
+    def _levels_backward_stacked(self, st, caches, d_y, bs, s, grads, P, rows_stack):
+        """Rule backward of the stacked levels; every level's projection-input gradients go straight into its
+        column slab of the packed operand P [n, 3 rows_stack] (see backward), its gate gradients into grads."""
+        d, nh, hd, C, na = self.d, self.nh, self.hd, self.chunk, st["na"]
         B = bs * nh
         dyh = _new(na * B, s, hd)
         D.call("transpose_heads_f32_cuda", d_y, dyh[:B], bs, s, nh, hd, 1)
@@ -291,13 +340,17 @@ class MagLayer:
         dm, ds = _zeros(hd, hd), _zeros(hd, hd)
         D.call("titans_chunkwise_backward_bf16_rocm", st["kh"], st["vh"], st["qh"], st["ah"], st["th"], st["eh"],
                st["mc"], st["sc"], dyh, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, na * B, C)
-        d_x = None
         for lv in range(na):
+            c, g = caches[lv], grads.levels[lv]
             sl = slice(lv * B, (lv + 1) * B)
-            dx = self._level_param_grads(lv, caches[lv], x2, tuple(t[sl] for t in (dkh, dvh, dqh, dah, dth, deh)),
-                                         bs, s, grads)
-            d_x = dx if d_x is None else d_x.add_(dx)
-        return d_x
+            col = (3 + 3 * lv) * d
+            lib.level_grads_packed_rocm(
+                dkh[sl].data_ptr(), dvh[sl].data_ptr(), dqh[sl].data_ptr(), dah[sl].data_ptr(), dth[sl].data_ptr(),
+                deh[sl].data_ptr(), c["k_mem"].data_ptr(), c["v_mem"].data_ptr(), c["q_mem"].data_ptr(), c["ld"],
+                c["k_norms"].data_ptr(), c["q_norms"].data_ptr(), c["alpha"].data_ptr(), c["theta"].data_ptr(),
+                c["eta"].data_ptr(), P.data_ptr(), 3 * rows_stack, col, rows_stack + col, 2 * rows_stack + col,
+                g.w_alpha.data_ptr(), g.b_alpha.data_ptr(), g.w_theta.data_ptr(), g.b_theta.data_ptr(),
+                g.w_eta.data_ptr(), g.b_eta.data_ptr(), bs, s, nh, hd, 1e-8, 1)
 
     def _level_backward(self, lv, c, x2, d_y, bs, s, grads):
         """gpu_memory_backward + accumulate_projection_grads; returns the level's d_x [bs*s, d]."""
@@ -358,27 +411,37 @@ class MagLayer:
         x2 = x.reshape(bs * s, d)
         self.conductor.set_seq_len(s)
         pulse = self.conductor.pulse()
-        ops = self._split_operands(x2) if self.split_gemm else None
-        q = self._project(ops, x2, p.w_q, 0).to(torch.bfloat16).view(bs, s, d)
-        k = self._project(ops, x2, p.w_k, 1).to(torch.bfloat16).view(bs, s, d)
-        v = self._project(ops, x2, p.w_v, 2).to(torch.bfloat16).view(bs, s, d)
-        attn_bf, aw = _new(bs, s, d, dtype=torch.bfloat16), _new(bs, nh, s, self.window, dtype=torch.bfloat16)
-        D.call("swa_forward_f32_cuda", q, k, v, attn_bf, aw, s, nh, hd, self.window, bs, 0)
-        attn = attn_bf.to(torch.float32)
-        ys, caches, stack = [], [], None
         active = [bool(a) for a in pulse.active_levels]
         na = active.index(False) if False in active else self.k
-        if self.rule == "chunkwise" and self.stack_levels and na >= 2 and not any(active[na:]):
+        stacked = (self.rule == "chunkwise" and self.stack_levels and self.split_gemm and self.fused_glue
+                   and na >= 2 and not any(active[na:]) and hd % 4 == 0 and d <= 1024)
+        ops = self._split_operands(x2, 3 * d * (1 + na) if stacked else 0) if self.split_gemm else None
+        q = self._project(ops, x2, p.w_q, 0, bf16_out=True).view(bs, s, d)
+        k = self._project(ops, x2, p.w_k, 1, bf16_out=True).view(bs, s, d)
+        v = self._project(ops, x2, p.w_v, 2, bf16_out=True).view(bs, s, d)
+        attn, aw = _new(bs, s, d, dtype=torch.bfloat16), _new(bs, nh, s, self.window, dtype=torch.bfloat16)
+        D.call("swa_forward_f32_cuda", q, k, v, attn, aw, s, nh, hd, self.window, bs, 0)
+        ys, caches, stack = [], [], None
+        if stacked:
             ys, caches, stack = self._levels_forward_stacked(na, x2, bs, s, ops)
         for lv in range(len(ys), self.k):
             y, c = self._level_forward(lv, x2, bs, s, active[lv], ops)
             ys.append(y)
             caches.append(c)
-        y_comb, gate, gated = _new(bs, s, d), _new(bs, s, d), _new(bs, s, d)
+        gate = _new(bs, s, d)
         ptrs = (ctypes.c_void_p * self.k)(*[y.data_ptr() for y in ys])
-        lib.cms_combine_gate_rocm(ptrs, self.k, attn.data_ptr(), y_comb.data_ptr(), gate.data_ptr(),
-                                  gated.data_ptr(), bs * s * d)
-        out = (gated.view(bs * s, d) @ p.w_o.t()).view(bs, s, d)
+        if d % 4 == 0 and ops is not None:
+            # the attention output is consumed as bf16; gated leaves as the packed operand of the output
+            # projection (hi | hi | lo), which is the last d rows of the packed weights
+            gated = _new(bs * s, 3 * d, dtype=torch.bfloat16)
+            lib.cms_combine_gate_bf16_rocm(ptrs, self.k, attn.data_ptr(), gate.data_ptr(), None, gated.data_ptr(), d,
+                                           bs * s * d)
+            out = torch.mm(gated, ops["wb"][-d:].t(), out_dtype=torch.float32).view(bs, s, d)
+        else:
+            gated = _new(bs, s, d)
+            lib.cms_combine_gate_rocm(ptrs, self.k, attn.to(torch.float32).data_ptr(), None, gate.data_ptr(),
+                                      gated.data_ptr(), bs * s * d)
+            out = (gated.view(bs * s, d) @ p.w_o.t()).view(bs, s, d)
         cache = dict(x=x, q=q, k=k, v=v, aw=aw, attn=attn, gate=gate, gated=gated, levels=caches, pulse=pulse,
                      ys=ys, ops=ops, stack=stack)
         return out, cache
@@ -416,32 +479,70 @@ class MagLayer:
                                   gated.data_ptr(), d)
         return (gated.view(1, d) @ p.w_o.t()).view(d)
 
-    def backward(self, cache, d_out):
-        """-> (d_x [bs, s, d], grads: MagParams of gradients)."""
+    def backward(self, cache, d_out, grads=None):
+        """-> (d_x [bs, s, d], grads: MagParams of gradients).  `grads`: a MagParams from new_grads() to write
+        into (zeroed here first); a new one is made otherwise."""
         x = cache["x"]
         bs, s, d = x.shape
         p, nh, hd = self.p, self.nh, self.hd
         n = bs * s
         x2 = x.reshape(n, d)
         do2 = d_out.reshape(n, d)
-        grads = MagParams(*[torch.zeros_like(t) for t in (p.w_q, p.w_k, p.w_v, p.w_o)],
-                          levels=[MemoryLevelParams(*[torch.zeros_like(t) for t in l.tensors()]) for l in p.levels])
-        d_gated = do2 @ p.w_o
-        grads.w_o += _wgrad(do2, cache["gated"].view(n, d))
+        if grads is None:
+            grads = self.new_grads()
+        else:
+            grads.flat.zero_()
+        ops, stack = cache["ops"], cache["stack"]
+        if cache["gated"].dtype == torch.bfloat16:
+            # d_gated = d_out W_o and d_W_o = d_out^T gated from one packing (H | L | H) of d_out
+            Pd, wo = self._pack_split([do2]), ops["wb"][-d:]
+            d_gated = torch.mm(Pd, torch.cat([wo[:, :d], wo[:, :d], wo[:, d:2 * d]], 0), out_dtype=torch.float32)
+            parts = next(q_ for q_ in (16, 8, 4, 2, 1) if (3 * n) % q_ == 0)
+            rows = 3 * n // parts
+            torch.sum(torch.bmm(Pd.view(parts, rows, d).transpose(1, 2), cache["gated"].view(parts, rows, d),
+                                out_dtype=torch.float32), 0, out=grads.w_o)
+        else:
+            d_gated = do2 @ p.w_o
+            grads.w_o += _wgrad(do2, cache["gated"].view(n, d))
         d_attn, d_ycomb = _new(bs, s, d), _new(bs, s, d)
-        D.call("cms_gate_backward_rocm", d_gated, cache["attn"], cache["gate"], self.k, d_attn, d_ycomb, n * d)
-        d_x, first = _zeros(n, d), 0
-        if cache["stack"] is not None:
-            first = cache["stack"]["na"]
-            d_x += self._levels_backward_stacked(cache["stack"], cache["levels"], x2, d_ycomb, bs, s, grads)
+        if d % 4 == 0:
+            lib.cms_gate_backward_bf16_rocm(d_gated.data_ptr(), cache["attn"].data_ptr(), cache["gate"].data_ptr(),
+                                            self.k, d_attn.data_ptr(), d_ycomb.data_ptr(), n * d)
+        else:
+            D.call("cms_gate_backward_rocm", d_gated, cache["attn"].to(torch.float32), cache["gate"], self.k, d_attn,
+                   d_ycomb, n * d)
+        first, P, rows_stack, d_x = 0, None, 0, None
+        if stack is not None:
+            # ONE packed operand for the attention group and every stacked level: P = (H | L | H), each third
+            # rows_stack wide with the projections in the order of the packed weights
+            first, rows_stack = stack["na"], ops["rows_stack"]
+            P = _new(n, 3 * rows_stack, dtype=torch.bfloat16)
+            self._levels_backward_stacked(stack, cache["levels"], d_ycomb, bs, s, grads, P, rows_stack)
         for lv in range(first, self.k):
-            d_x += self._level_backward(lv, cache["levels"][lv], x2, d_ycomb, bs, s, grads)
+            dx = self._level_backward(lv, cache["levels"][lv], x2, d_ycomb, bs, s, grads)
+            d_x = dx if d_x is None else d_x.add_(dx)
         dq, dk, dv = _new(bs, s, d), _zeros(bs, s, d), _zeros(bs, s, d)
         D.call("swa_backward_f32_cuda", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv, s, nh,
                hd, self.window, bs, 0)
         dq2, dk2, dv2 = dq.view(n, d), dk.view(n, d), dv.view(n, d)
-        d_x += self._group_grads(cache["ops"], 0, x2, (dq2, dk2, dv2), (p.w_q, p.w_k, p.w_v),
-                                 (grads.w_q, grads.w_k, grads.w_v))
+        if P is None:
+            dx = self._group_grads(ops, 0, x2, (dq2, dk2, dv2), (p.w_q, p.w_k, p.w_v),
+                                   (grads.w_q, grads.w_k, grads.w_v))
+            d_x = dx if d_x is None else d_x.add_(dx)
+            return d_x.view(bs, s, d), grads
+        ptrs = (ctypes.c_void_p * 3)(dq2.data_ptr(), dk2.data_ptr(), dv2.data_ptr())
+        lib.split_pack_bf16_ld_rocm(ptrs, 3, d, P.data_ptr(), n, d, 3 * rows_stack, 0, rows_stack, 2 * rows_stack)
+        dx = torch.mm(P, ops["wstack"], out_dtype=torch.float32)
+        d_x = dx if d_x is None else d_x.add_(dx)
+        # weight gradients of all these projections: (H^T xh + L^T xh) and H^T xl, the contraction over the
+        # tokens cut into slabs that run as one batched GEMM and are summed
+        parts = next(q_ for q_ in (4, 2, 1) if n % q_ == 0)
+        Pv, xv = P.view(parts, n // parts, 3 * rows_stack), ops["xa"].view(parts, n // parts, 3 * d)
+        dw_hl = torch.bmm(Pv[:, :, :2 * rows_stack].transpose(1, 2), xv[:, :, :d], out_dtype=torch.float32).sum(0)
+        dw_h = torch.bmm(Pv[:, :, 2 * rows_stack:].transpose(1, 2), xv[:, :, 2 * d:], out_dtype=torch.float32).sum(0)
+        gp = grads.pack[:rows_stack]
+        torch.add(dw_hl[:rows_stack], dw_hl[rows_stack:], out=gp)
+        gp += dw_h
         return d_x.view(bs, s, d), grads
 
 
@@ -478,9 +579,7 @@ class MagTrainer:
                  max_grad_norm=1.0):
         self.layer, self.lr, self.max_grad_norm = layer, lr, max_grad_norm
         p = layer.p
-        self.grads = MagParams(*[torch.zeros_like(t) for t in (p.w_q, p.w_k, p.w_v, p.w_o)],
-                               levels=[MemoryLevelParams(*[torch.zeros_like(t) for t in l.tensors()])
-                                       for l in p.levels])
+        self.grads = layer.new_grads()
         self.opt = FrequencyAwareAdamW(layer.k, beta1, beta2, eps, weight_decay)
         self.state = []
         groups = [-1] * 4 + [lv for lv in range(layer.k) for _ in range(9)]
@@ -511,9 +610,7 @@ class MagTrainer:
 
     def _forward_backward(self, x, d_out):
         out, cache = self.layer.forward(x)
-        _, g = self.layer.backward(cache, d_out)
-        for dst, src in zip(self.grads.tensors(), g.tensors()):
-            dst.copy_(src)
+        self.layer.backward(cache, d_out, self.grads)
         return out
 
     def step_graphed(self, x, d_out):
@@ -559,9 +656,7 @@ class MagTrainer:
     def step(self, x, d_out_fn):
         """One training step; d_out_fn(out) gives the upstream gradient.  Returns out."""
         out, cache = self.layer.forward(x)
-        _, g = self.layer.backward(cache, d_out_fn(out))
-        for dst, src in zip(self.grads.tensors(), g.tensors()):
-            dst.copy_(src)
+        self.layer.backward(cache, d_out_fn(out), self.grads)
         self._optimizer_and_error_buffers(cache["pulse"])
         self.layer.conductor.advance()
         return out
