@@ -528,6 +528,24 @@ void titans_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const uint16_t *
                                          float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                                          float *d_s_initial, int seq_len, int d, int batch_size,
                                          int chunk_size);
+/* The same pair for a layer that keeps its tensors token-major (no counterpart in the reference, whose
+ * gpu_memory_forward / gpu_memory_backward transpose between the layouts, core/src/gpu_forward.rs:1197 ff.):
+ * chain c = (level, batch element, head), batch_size = levels * bs * heads; y_tokens [levels, bs, seq_len, heads*d]
+ * is written directly; d_y_tokens has that shape (d_y_per_level != 0) or is ONE [bs, seq_len, heads*d] gradient
+ * that every level reads.  k, v, q, the gates and the gradients stay head-major.  d = 64, chunk_size <= 64. */
+void titans_chunkwise_forward_bf16_tokens_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                               const float *alpha, const float *theta, const float *eta,
+                                               const float *m_initial, const float *s_initial, float *m_chunk_states,
+                                               float *s_chunk_states, float *y_tokens, int seq_len, int d,
+                                               int batch_size, int chunk_size, int heads, int levels);
+void titans_chunkwise_backward_bf16_tokens_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                                const float *alpha, const float *theta, const float *eta,
+                                                const float *m_chunk_states, const float *s_chunk_states,
+                                                const float *d_y_tokens, float *d_k_mem, float *d_v_mem,
+                                                float *d_q_mem, float *d_alpha, float *d_theta, float *d_eta,
+                                                float *d_m_initial, float *d_s_initial, int seq_len, int d,
+                                                int batch_size, int chunk_size, int heads, int levels,
+                                                int d_y_per_level);
 void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
                                            const float *alpha, const float *theta, const float *eta,
                                            const float *m_chunk_states, const float *s_chunk_states,
@@ -639,7 +657,8 @@ void memory_grads_fused_rocm(const float *d_k_heads, const float *d_v_heads, con
  * of x are split-bf16 GEMMs over packed operands; these entry points let several producers fill column slabs of
  * ONE operand, and read projection outputs in place as column ranges of a wider GEMM output (row stride ld). */
 /* As split_pack_bf16_rocm with row strides: source rows src_ld floats apart; in row r of out (out_ld bf16 values
- * apart) source i, column c goes to i*d + c, its hi part at off_h1 + and off_h2 +, its lo part at off_l +. */
+ * apart) source i, column c goes to i*d + c, its hi part at off_h1 + and off_h2 +, its lo part at off_l +.
+ * off_h2 < 0 (here and in level_grads_packed_rocm): the hi part is written once. */
 void split_pack_bf16_ld_rocm(const float *const *srcs, int count, long long src_ld, uint16_t *out, long long n, int d,
                              long long out_ld, long long off_h1, long long off_l, long long off_h2);
 /* The packed fp32 weight rows [rows, d] -> wb [rows, 3d] = (Wh | Wl | Wh) per row, the right operand of the

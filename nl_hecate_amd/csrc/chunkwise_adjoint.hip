@@ -29,7 +29,7 @@ template <bool HAS_S>
 __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ q, const float *__restrict__ d_y,
     const float *__restrict__ tab_b, const float *__restrict__ vecs, float *__restrict__ dm_states,
-    float *__restrict__ ds_states, int s, int C, int nc, int batch, int tab_floats, int vec_floats) {
+    float *__restrict__ ds_states, int s, int C, int nc, int batch, int tab_floats, int vec_floats, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Kt = Kr + BMAT;   // K [j][c], K^T [c][j]
     u16 *Qr = Kt + BMAT, *Qt = Qr + BMAT;                            // Q [t][c], Q^T [c][t]
@@ -45,6 +45,7 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
     const int chain = blockIdx.x % batch, half = blockIdx.x / batch, i0 = 32 * half;
     const size_t chain_tok = (size_t)chain * s, state0 = (size_t)chain * (nc + 1) * HD * HD;
+    const size_t dy_off = dyr.offset(chain);
     const int st_t = 16 * (w & 3) + (l & 15), st_cb = 4 * (w >> 2) + (l >> 4);   // bf16 tile: row, 8-element block
     const int yt = tid >> 3, yg = tid & 7;                                        // dY tile: row t, 4-element block
 
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
         const size_t row = tok + min(st_t, L - 1);
         nK = *reinterpret_cast<const uint4 *>(k + row * HD + st_cb * 8);
         nQ = *reinterpret_cast<const uint4 *>(q + row * HD + st_cb * 8);
-        ndY = *reinterpret_cast<const f32x4 *>(d_y + (tok + min(yt, L - 1)) * HD + i0 + yg * 4);
+        ndY = *reinterpret_cast<const f32x4 *>(d_y + dy_off + (size_t)(c * C + min(yt, L - 1)) * dyr.row_stride + i0 +
+                                               yg * 4);
         const size_t chunk = (size_t)chain * nc + c;
         const float *vo = vecs + chunk * vec_floats, *tb = tab_b + chunk * tab_floats;
         na = vo[yt];
@@ -200,9 +202,10 @@ constexpr size_t kAdjointLds = (6 * BMAT + 12 * HMAT) * sizeof(u16) + (5 * CW + 
 
 bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
                             const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
-                            int chunk_size, bool has_s) {
+                            int chunk_size, bool has_s, const HeadRows *dy_rows) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size);
+    const HeadRows dyr = dy_rows ? *dy_rows : head_major_rows(seq_len, HD);
     static bool attr_set = false;
     if (!attr_set) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_adjoint_chain_kernel<true>),
@@ -216,10 +219,10 @@ bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d
     KernelTimer kt("cw_adjoint_chain_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_adjoint_chain_kernel<true>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
-                           d_y, tab_b, vecs, dm_states, ds_states, seq_len, chunk_size, nc, batch, tabf, vecf);
+                           d_y, tab_b, vecs, dm_states, ds_states, seq_len, chunk_size, nc, batch, tabf, vecf, dyr);
     else
         hipLaunchKernelGGL(cw_adjoint_chain_kernel<false>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
-                           d_y, tab_b, vecs, dm_states, nullptr, seq_len, chunk_size, nc, batch, tabf, vecf);
+                           d_y, tab_b, vecs, dm_states, nullptr, seq_len, chunk_size, nc, batch, tabf, vecf, dyr);
     check_launch("cw_adjoint_chain_kernel");
     return true;
 }

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q,
     const float *__restrict__ table, const float *__restrict__ vecs, const float *__restrict__ m_initial,
     const float *__restrict__ s_initial, float *__restrict__ m_states, float *__restrict__ s_states,
-    float *__restrict__ y, int s, int C, int nc, int batch) {
+    float *__restrict__ y, int s, int C, int nc, int batch, HeadRows yr) {
     constexpr int HMAT = 32 * LDB;   // a 32-row matrix
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *Kr = reinterpret_cast<u16 *>(smem_raw);   // K [t][c]
@@ -145,6 +145,7 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
     const int bi = w & 3, bm = 32 * (bi >> 1), bn = 32 * (bi & 1);   // group Y: 32x32 block of P^T; group X: strip bi
     const size_t chain_tok = (size_t)chain * s;
     const size_t state0 = (size_t)chain * (nc + 1) * HD * HD;
+    const size_t y_off = yr.offset(chain);
 
     // -V enters E = K M0^T - V as one more step of the product: A = V (rows t, this half's 32
     // columns as contraction), B = -identity: column 16 ct + l%16 meets contraction index 8 (l/16) + e.
@@ -366,7 +367,7 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
             if (t < L) {
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++)
-                    *reinterpret_cast<f32x4 *>(y + (tok + t) * HD + i0 + 16 * rt + 4 * g) = y2[rt];
+                    *reinterpret_cast<f32x4 *>(y + y_off + (size_t)(t0 + t) * yr.row_stride + i0 + 16 * rt + 4 * g) = y2[rt];
             }
         } else {
             publish_state(c + 1);
@@ -384,7 +385,7 @@ constexpr size_t kChainFwdLds = (7 * BMAT + 10 * 32 * LDB) * sizeof(u16) + (4 * 
 template <bool HAS_S>
 void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, const float *alpha, const float *theta,
                     const float *eta, const float *m_initial, const float *s_initial, float *m_states,
-                    float *s_states, float *y, int seq_len, int batch, int chunk_size) {
+                    float *s_states, float *y, int seq_len, int batch, int chunk_size, const HeadRows &yr) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), nchunks = batch * nc;
     float *table = scratch(3, (size_t)nchunks * kTableFloats * sizeof(float));
@@ -406,7 +407,7 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
     {
         KernelTimer kt("cw_chain_fwd_kernel");
         hipLaunchKernelGGL(cw_chain_fwd_kernel<HAS_S>, dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k, v, q,
-                           table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch);
+                           table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch, yr);
     }
     check_launch(fn);
 }
@@ -416,14 +417,15 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
 bool chunkwise_chain_forward_bf16(const char *fn, const uint16_t *k, const uint16_t *v, const uint16_t *q,
                                   const float *alpha, const float *theta, const float *eta, const float *m_initial,
                                   const float *s_initial, float *m_states, float *s_states, float *y, int seq_len,
-                                  int d, int batch, int chunk_size, bool has_s) {
+                                  int d, int batch, int chunk_size, bool has_s, const HeadRows *y_rows) {
     if (d != HD || chunk_size < 1 || chunk_size > CW || seq_len <= 0 || batch <= 0) return false;
+    const HeadRows yr = y_rows ? *y_rows : head_major_rows(seq_len, HD);
     if (has_s)
         launch_forward<true>(fn, k, v, q, alpha, theta, eta, m_initial, s_initial, m_states, s_states, y, seq_len,
-                             batch, chunk_size);
+                             batch, chunk_size, yr);
     else
         launch_forward<false>(fn, k, v, q, alpha, theta, nullptr, m_initial, nullptr, m_states, nullptr, y, seq_len,
-                              batch, chunk_size);
+                              batch, chunk_size, yr);
     return true;
 }
 

@@ -12,6 +12,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "head_rows.h"
+
 namespace nlh {
 
 size_t chunkwise_grads_table_floats();
@@ -22,13 +24,14 @@ void chunkwise_backward_coefficients(const float *alpha, const float *theta, con
 
 bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
                             const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
-                            int chunk_size, bool has_s);
+                            int chunk_size, bool has_s, const HeadRows *dy_rows = nullptr);
 
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
                           const float *m_states, const float *s_states, const float *dm_states,
                           const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
-                          int seq_len, int batch, int chunk_size, bool has_s, int grid);
+                          int seq_len, int batch, int chunk_size, bool has_s, int grid,
+                          const HeadRows *dy_rows = nullptr);
 
 void chunkwise_gate_gradients(const float *alpha, const float *eta, const float *pvec, const float *xs,
                               const float *scal, float *d_alpha, float *d_eta, int seq_len, int batch,

@@ -132,7 +132,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
     const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
-    int C, int nc, int ntask) {
+    int C, int nc, int ntask, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Kt = Kr + BMAT;   // K [t][c], K^T [c][t]
     u16 *Qr = Kt + BMAT, *Qt = Qr + BMAT;                            // Q, Q^T
@@ -165,15 +165,16 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     float nvec = 0.f;
     auto fetch = [&](int task) {
         const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
-        const size_t tok = (size_t)chain * s + t0, row = tok + min(st_t, L - 1), frow = tok + min(ft, L - 1);
+        const size_t tok = (size_t)chain * s + t0, row = tok + min(st_t, L - 1);
         nK = *reinterpret_cast<const uint4 *>(k + row * HD + st_cb * 8);
         nQ = *reinterpret_cast<const uint4 *>(q + row * HD + st_cb * 8);
         nV = *reinterpret_cast<const uint4 *>(v + row * HD + st_cb * 8);
         const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD + ft * HD, st1 = st0 + HD * HD;
+        const float *dy_row = d_y + dyr.offset(chain) + (size_t)(t0 + min(ft, L - 1)) * dyr.row_stride;
 #pragma unroll
         for (int it = 0; it < 2; it++) {
             const int c4 = (fg0 + 8 * it) * 4;
-            ndY[it] = *reinterpret_cast<const f32x4 *>(d_y + frow * HD + c4);
+            ndY[it] = *reinterpret_cast<const f32x4 *>(dy_row + c4);
             nM0[it] = *reinterpret_cast<const f32x4 *>(m_states + st0 + c4);
             ndM[it] = *reinterpret_cast<const f32x4 *>(dm_states + st1 + c4);
             if (HAS_S) {
@@ -214,7 +215,8 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 return base + (tok + min(ln & 63, L - 1)) * HD;
             }
             const int f = (ln - 192) >> 7, o = (ln - 192) & 127;   // line o of fp32 tile f: row o/2, half o%2
-            if (f == 0) return d_y + (tok + min(o >> 1, L - 1)) * HD + (o & 1) * 32;
+            if (f == 0)
+                return d_y + dyr.offset(chain) + (size_t)(t0 + min(o >> 1, L - 1)) * dyr.row_stride + (o & 1) * 32;
             const float *base = f == 1 ? m_states + st0 : (f == 2 ? (HAS_S ? s_states + st0 : m_states + st0)
                                 : (f == 3 ? dm_states + st1 : (HAS_S ? ds_states + st1 : dm_states + st1)));
             return base + o * 32;
@@ -607,9 +609,10 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           const float *m_states, const float *s_states, const float *dm_states,
                           const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
-                          int seq_len, int batch, int chunk_size, bool has_s, int grid) {
+                          int seq_len, int batch, int chunk_size, bool has_s, int grid, const HeadRows *dy_rows) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
+    const HeadRows dyr = dy_rows ? *dy_rows : head_major_rows(seq_len, HD);
     static bool attr_set = false;
     if (!attr_set) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_grads_bf16_kernel<true>),
@@ -623,11 +626,11 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
     if (has_s)
         hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
                            tab_a, tab_b, vecs, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec,
-                           xs, scal, seq_len, chunk_size, nc, ntask);
+                           xs, scal, seq_len, chunk_size, nc, ntask, dyr);
     else
         hipLaunchKernelGGL(cw_grads_bf16_kernel<false>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
                            tab_a, tab_b, vecs, m_states, nullptr, dm_states, nullptr, d_k, d_v, d_q, d_theta, pvec,
-                           xs, scal, seq_len, chunk_size, nc, ntask);
+                           xs, scal, seq_len, chunk_size, nc, ntask, dyr);
     check_launch("cw_grads_bf16_kernel");
     return true;
 }

@@ -853,9 +853,11 @@ template <class TIn>
 void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const float *alpha, const float *theta,
                  const float *eta, const float *m_states, const float *s_states, const float *d_y, float *d_k,
                  float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
-                 float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s) {
+                 float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s,
+                 const HeadRows *dy_rows = nullptr) {
     const ErrorScope es;
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
+    if (dy_rows && sizeof(TIn) != 2) { fail("%s: token-major d_y is served for bf16 tokens only.", fn); return; }
     const int nc = ceil_div(seq_len, chunk_size);
     Scratch sc{nullptr, nullptr};
     if constexpr (sizeof(TIn) == 4) sc = local_scratch(batch, nc);
@@ -882,10 +884,11 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
         if (es.failed()) return;
         chunkwise_backward_coefficients(alpha, theta, eta, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s);
-        chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_states, ds_states, seq_len, batch, chunk_size, has_s);
+        chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_states, ds_states, seq_len, batch, chunk_size, has_s,
+                               dy_rows);
         chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec, xs,
                              scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
-                             persistent_grid(batch * nc));
+                             persistent_grid(batch * nc), dy_rows);
     } else {
         hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
                            stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc,
@@ -959,6 +962,52 @@ extern "C" void titans_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const
     backward_mm<uint16_t>("titans_chunkwise_backward_bf16_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
                           m_chunk_states, s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta,
                           d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, true);
+}
+
+// The same rule for a layer that keeps its tensors token-major: chain c = (level, batch element, head) with
+// batch_size = levels * bs * heads chains; y_tokens [levels, bs, seq_len, heads * d] is written directly, and
+// d_y_tokens is [levels, ...] of that shape (d_y_per_level != 0) or ONE [bs, seq_len, heads * d] gradient that
+// every level reads.  The head-major k, v, q, gates and the gradients keep the layout of the entry points above.
+static bool token_rows_ok(const char *fn, int d, int batch_size, int chunk_size, int heads, int levels) {
+    if (d != HD || chunk_size < 1 || chunk_size > CW) {
+        fail("%s: needs d=%d == %d and chunk_size=%d in [1, %d].", fn, d, HD, chunk_size, CW);
+        return false;
+    }
+    if (heads < 1 || levels < 1 || batch_size % (heads * levels)) {
+        fail("%s: batch_size=%d must be a multiple of heads=%d * levels=%d.", fn, batch_size, heads, levels);
+        return false;
+    }
+    return true;
+}
+
+extern "C" void titans_chunkwise_forward_bf16_tokens_rocm(const uint16_t *k_mem, const uint16_t *v_mem,
+                                                          const uint16_t *q_mem, const float *alpha,
+                                                          const float *theta, const float *eta,
+                                                          const float *m_initial, const float *s_initial,
+                                                          float *m_chunk_states, float *s_chunk_states,
+                                                          float *y_tokens, int seq_len, int d, int batch_size,
+                                                          int chunk_size, int heads, int levels) {
+    const char *fn = "titans_chunkwise_forward_bf16_tokens_rocm";
+    if (seq_len <= 0 || batch_size <= 0) return;
+    if (!token_rows_ok(fn, d, batch_size, chunk_size, heads, levels)) return;
+    const HeadRows yr = token_major_rows(seq_len, HD, heads, batch_size / levels, true);
+    chunkwise_chain_forward_bf16(fn, k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial, m_chunk_states,
+                                 s_chunk_states, y_tokens, seq_len, d, batch_size, chunk_size, true, &yr);
+}
+
+extern "C" void titans_chunkwise_backward_bf16_tokens_rocm(
+    const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem, const float *alpha, const float *theta,
+    const float *eta, const float *m_chunk_states, const float *s_chunk_states, const float *d_y_tokens,
+    float *d_k_mem, float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta, float *d_eta,
+    float *d_m_initial, float *d_s_initial, int seq_len, int d, int batch_size, int chunk_size, int heads, int levels,
+    int d_y_per_level) {
+    const char *fn = "titans_chunkwise_backward_bf16_tokens_rocm";
+    if (seq_len <= 0 || batch_size <= 0) return;
+    if (!token_rows_ok(fn, d, batch_size, chunk_size, heads, levels)) return;
+    const HeadRows dyr = token_major_rows(seq_len, HD, heads, batch_size / levels, d_y_per_level != 0);
+    backward_mm<uint16_t>(fn, k_mem, v_mem, q_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, d_y_tokens,
+                          d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d,
+                          batch_size, chunk_size, true, &dyr);
 }
 
 extern "C" void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,

@@ -33,13 +33,13 @@ __device__ __forceinline__ bf4 lo4(const float4 &x, const bf4 &h) {
     return bf4{(__bf16)(x.x - (float)h[0]), (__bf16)(x.y - (float)h[1]), (__bf16)(x.z - (float)h[2]),
                (__bf16)(x.w - (float)h[3])};
 }
-// x = hi + lo in bf16; hi goes to two column positions of the row, lo to one
+// x = hi + lo in bf16; hi goes to two column positions of the row (one when off_h2 < 0), lo to one
 __device__ __forceinline__ void store_split(uint16_t *row, long long col, long long off_h1, long long off_l,
                                             long long off_h2, const float4 &x) {
     const bf4 h = hi4(x), l = lo4(x, h);
     *reinterpret_cast<bf4 *>(row + off_h1 + col) = h;
     *reinterpret_cast<bf4 *>(row + off_l + col) = l;
-    *reinterpret_cast<bf4 *>(row + off_h2 + col) = h;
+    if (off_h2 >= 0) *reinterpret_cast<bf4 *>(row + off_h2 + col) = h;
 }
 
 struct SplitSrcs4 { const float *p[4]; };
@@ -376,7 +376,7 @@ extern "C" {
 void split_pack_bf16_ld_rocm(const float *const *srcs, int count, long long src_ld, uint16_t *out, long long n, int d,
                              long long out_ld, long long off_h1, long long off_l, long long off_h2) {
     if (n <= 0) return;
-    if (count < 1 || count > 4 || d <= 0 || d % 4 || src_ld % 4 || out_ld % 4 || off_h1 % 4 || off_l % 4 || off_h2 % 4 ||
+    if (count < 1 || count > 4 || d <= 0 || d % 4 || src_ld % 4 || out_ld % 4 || off_h1 % 4 || off_l % 4 || (off_h2 >= 0 && off_h2 % 4) ||
         !al8(out)) {
         fail("split_pack_bf16_ld_rocm: count=%d must be 1..4, d=%d, the strides and the offsets multiples of 4.", count, d);
         return;
@@ -444,7 +444,7 @@ void level_grads_packed_rocm(const float *d_k_heads, const float *d_v_heads, con
     const long long n = (long long)bs * s;
     if (n <= 0 || nh <= 0 || hd <= 0) return;
     const int d = nh * hd;
-    if (hd % 4 || d > 1024 || ld % 4 || ld < d || p_ld % 4 || off_h1 % 4 || off_l % 4 || off_h2 % 4 || !al16(d_k_heads) ||
+    if (hd % 4 || d > 1024 || ld % 4 || ld < d || p_ld % 4 || off_h1 % 4 || off_l % 4 || (off_h2 >= 0 && off_h2 % 4) || !al16(d_k_heads) ||
         !al16(d_v_heads) || !al16(d_q_heads) || !al16(k_norm) || !al16(v_mem) || !al16(q_norm) || !al8(p_out)) {
         fail("level_grads_packed_rocm: needs head_dim=%d a multiple of 4, nh*hd=%d <= 1024, strides and offsets multiples "
              "of 4, ld=%lld >= nh*hd, and aligned buffers.", hd, d, ld);

@@ -314,32 +314,27 @@ class MagLayer:
             caches.append(dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, ld=ld, k_norms=k_norms, q_norms=q_norms,
                                active=True, ops=ops, alpha=alpha, theta=theta, eta=eta))
         nc = (s + C - 1) // C
-        mc, sc, yh = _new(na * B, nc + 1, hd * hd), _new(na * B, nc + 1, hd * hd), _new(na * B, s, hd)
+        mc, sc = _new(na * B, nc + 1, hd * hd), _new(na * B, nc + 1, hd * hd)
         m0, s0 = self._m_all[:na].view(na * B, hd * hd), self._s_all[:na].view(na * B, hd * hd)
-        D.call("titans_chunkwise_forward_bf16_rocm", kh, vh, qh, ah, th, eh, m0, s0, mc, sc, yh, s, hd, na * B, C)
+        y_all = _new(na, bs, s, d)   # the rule writes every level's output token-major: no head transposes
+        D.call("titans_chunkwise_forward_bf16_tokens_rocm", kh, vh, qh, ah, th, eh, m0, s0, mc, sc, y_all, s, hd,
+               na * B, C, nh, na)
         m0.copy_(mc[:, -1])
         s0.copy_(sc[:, -1])
-        ys = []
-        for lv in range(na):
-            y = _new(bs, s, d)
-            D.call("transpose_heads_f32_cuda", yh[lv * B:(lv + 1) * B], y, bs, s, nh, hd, 0)
-            ys.append(y)
+        ys = [y_all[lv] for lv in range(na)]
         return ys, caches, dict(na=na, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, mc=mc, sc=sc, proj=proj)
 
     def _levels_backward_stacked(self, st, caches, d_y, bs, s, grads, P, rows_stack):
         """Rule backward of the stacked levels; every level's projection-input gradients go straight into its
-        column slab of the packed operand P [n, 3 rows_stack] (see backward), its gate gradients into grads."""
+        column slab of the packed operand P [n, 2 rows_stack] (see backward), its gate gradients into grads."""
         d, nh, hd, C, na = self.d, self.nh, self.hd, self.chunk, st["na"]
         B = bs * nh
-        dyh = _new(na * B, s, hd)
-        D.call("transpose_heads_f32_cuda", d_y, dyh[:B], bs, s, nh, hd, 1)
-        for lv in range(1, na):   # every level sees the same upstream gradient
-            dyh[lv * B:(lv + 1) * B].copy_(dyh[:B])
         dkh, dvh, dqh = _new(na * B, s, hd), _new(na * B, s, hd), _new(na * B, s, hd)
         dah, dth, deh = _new(na * B, s), _new(na * B, s), _new(na * B, s)
         dm, ds = _zeros(hd, hd), _zeros(hd, hd)
-        D.call("titans_chunkwise_backward_bf16_rocm", st["kh"], st["vh"], st["qh"], st["ah"], st["th"], st["eh"],
-               st["mc"], st["sc"], dyh, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, na * B, C)
+        # every level reads the one token-major upstream gradient in place
+        D.call("titans_chunkwise_backward_bf16_tokens_rocm", st["kh"], st["vh"], st["qh"], st["ah"], st["th"],
+               st["eh"], st["mc"], st["sc"], d_y, dkh, dvh, dqh, dah, dth, deh, dm, ds, s, hd, na * B, C, nh, na, 0)
         for lv in range(na):
             c, g = caches[lv], grads.levels[lv]
             sl = slice(lv * B, (lv + 1) * B)
@@ -348,7 +343,7 @@ class MagLayer:
                 dkh[sl].data_ptr(), dvh[sl].data_ptr(), dqh[sl].data_ptr(), dah[sl].data_ptr(), dth[sl].data_ptr(),
                 deh[sl].data_ptr(), c["k_mem"].data_ptr(), c["v_mem"].data_ptr(), c["q_mem"].data_ptr(), c["ld"],
                 c["k_norms"].data_ptr(), c["q_norms"].data_ptr(), c["alpha"].data_ptr(), c["theta"].data_ptr(),
-                c["eta"].data_ptr(), P.data_ptr(), 3 * rows_stack, col, rows_stack + col, 2 * rows_stack + col,
+                c["eta"].data_ptr(), P.data_ptr(), 2 * rows_stack, col, rows_stack + col, -1,
                 g.w_alpha.data_ptr(), g.b_alpha.data_ptr(), g.w_theta.data_ptr(), g.b_theta.data_ptr(),
                 g.w_eta.data_ptr(), g.b_eta.data_ptr(), bs, s, nh, hd, 1e-8, 1)
 
@@ -414,7 +409,7 @@ class MagLayer:
         active = [bool(a) for a in pulse.active_levels]
         na = active.index(False) if False in active else self.k
         stacked = (self.rule == "chunkwise" and self.stack_levels and self.split_gemm and self.fused_glue
-                   and na >= 2 and not any(active[na:]) and hd % 4 == 0 and d <= 1024)
+                   and na >= 2 and not any(active[na:]) and hd == 64 and self.chunk <= 64 and d <= 1024)
         ops = self._split_operands(x2, 3 * d * (1 + na) if stacked else 0) if self.split_gemm else None
         q = self._project(ops, x2, p.w_q, 0, bf16_out=True).view(bs, s, d)
         k = self._project(ops, x2, p.w_k, 1, bf16_out=True).view(bs, s, d)
@@ -513,10 +508,10 @@ class MagLayer:
                    d_ycomb, n * d)
         first, P, rows_stack, d_x = 0, None, 0, None
         if stack is not None:
-            # ONE packed operand for the attention group and every stacked level: P = (H | L | H), each third
+            # ONE packed operand for the attention group and every stacked level: P = (H | L), each half
             # rows_stack wide with the projections in the order of the packed weights
             first, rows_stack = stack["na"], ops["rows_stack"]
-            P = _new(n, 3 * rows_stack, dtype=torch.bfloat16)
+            P = _new(n, 2 * rows_stack, dtype=torch.bfloat16)
             self._levels_backward_stacked(stack, cache["levels"], d_ycomb, bs, s, grads, P, rows_stack)
         for lv in range(first, self.k):
             dx = self._level_backward(lv, cache["levels"][lv], x2, d_ycomb, bs, s, grads)
@@ -531,15 +526,18 @@ class MagLayer:
             d_x = dx if d_x is None else d_x.add_(dx)
             return d_x.view(bs, s, d), grads
         ptrs = (ctypes.c_void_p * 3)(dq2.data_ptr(), dk2.data_ptr(), dv2.data_ptr())
-        lib.split_pack_bf16_ld_rocm(ptrs, 3, d, P.data_ptr(), n, d, 3 * rows_stack, 0, rows_stack, 2 * rows_stack)
-        dx = torch.mm(P, ops["wstack"], out_dtype=torch.float32)
+        lib.split_pack_bf16_ld_rocm(ptrs, 3, d, P.data_ptr(), n, d, 2 * rows_stack, 0, rows_stack, -1)
+        # d_x = H Wh + L Wh + H Wl: (H | L) . (Wh ; Wh), then H . Wl added by a second GEMM on the H columns
+        ws = ops["wstack"]
+        dx = torch.mm(P, ws[:2 * rows_stack], out_dtype=torch.float32)
+        dx = torch.addmm(dx, P[:, :rows_stack], ws[2 * rows_stack:], out_dtype=torch.float32)
         d_x = dx if d_x is None else d_x.add_(dx)
-        # weight gradients of all these projections: (H^T xh + L^T xh) and H^T xl, the contraction over the
+        # weight gradients of all these projections: (H^T xh ; L^T xh) and H^T xl, the contraction over the
         # tokens cut into slabs that run as one batched GEMM and are summed
         parts = next(q_ for q_ in (4, 2, 1) if n % q_ == 0)
-        Pv, xv = P.view(parts, n // parts, 3 * rows_stack), ops["xa"].view(parts, n // parts, 3 * d)
-        dw_hl = torch.bmm(Pv[:, :, :2 * rows_stack].transpose(1, 2), xv[:, :, :d], out_dtype=torch.float32).sum(0)
-        dw_h = torch.bmm(Pv[:, :, 2 * rows_stack:].transpose(1, 2), xv[:, :, 2 * d:], out_dtype=torch.float32).sum(0)
+        Pv, xv = P.view(parts, n // parts, 2 * rows_stack), ops["xa"].view(parts, n // parts, 3 * d)
+        dw_hl = torch.bmm(Pv.transpose(1, 2), xv[:, :, :d], out_dtype=torch.float32).sum(0)
+        dw_h = torch.bmm(Pv[:, :, :rows_stack].transpose(1, 2), xv[:, :, 2 * d:], out_dtype=torch.float32).sum(0)
         gp = grads.pack[:rows_stack]
         torch.add(dw_hl[:rows_stack], dw_hl[rows_stack:], out=gp)
         gp += dw_h

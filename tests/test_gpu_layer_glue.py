@@ -170,3 +170,40 @@ def test_combine_gate_with_bf16_attention_matches_the_fp32_kernels():
     torch.cuda.synchronize()
     assert torch.equal(da1, da2)
     _close("d_y", dy2, dy1, 1e-6)
+
+
+@pytest.mark.parametrize("levels,bs,nh,s,C,per_level", [(3, 2, 4, 150, 64, False), (2, 1, 8, 70, 16, True)])
+def test_chunkwise_rule_on_token_major_rows_equals_the_head_major_entry_points(levels, bs, nh, s, C, per_level):
+    """titans_chunkwise_{forward,backward}_bf16_tokens_rocm write y / read d_y in [levels, bs, s, nh*64] (d_y
+    optionally shared by the levels); same kernels, other addresses: bit-equal to the head-major pair."""
+    hd, B = 64, bs * nh
+    nb, nc = levels * B, (s + C - 1) // C
+    g = torch.Generator(device="cuda").manual_seed(77 + s)
+    k, v, q = (_rn(g, nb, s, hd).to(torch.bfloat16) for _ in range(3))
+    al, th, et = (torch.rand(nb, s, device="cuda", generator=g) * sc for sc in (0.1, 0.05, 0.9))
+    m0, s0 = 0.1 * _rn(g, nb, hd * hd), 0.1 * _rn(g, nb, hd * hd)
+    z = lambda *sh: torch.zeros(*sh, device="cuda")
+    mc1, sc1, y1 = z(nb, nc + 1, hd * hd), z(nb, nc + 1, hd * hd), z(nb, s, hd)
+    D.call("titans_chunkwise_forward_bf16_rocm", k, v, q, al, th, et, m0, s0, mc1, sc1, y1, s, hd, nb, C)
+    mc2, sc2, y2 = z(nb, nc + 1, hd * hd), z(nb, nc + 1, hd * hd), z(levels, bs, s, nh * hd)
+    D.call("titans_chunkwise_forward_bf16_tokens_rocm", k, v, q, al, th, et, m0, s0, mc2, sc2, y2, s, hd, nb, C, nh,
+           levels)
+    torch.cuda.synchronize()
+    assert torch.equal(mc1, mc2) and torch.equal(sc1, sc2)
+    assert torch.equal(y1.view(levels, bs, nh, s, hd).permute(0, 1, 3, 2, 4).reshape(levels, bs, s, nh * hd), y2)
+    # backward
+    dy_tok = _rn(g, levels if per_level else 1, bs, s, nh * hd)
+    dy_heads = dy_tok.expand(levels, bs, s, nh * hd).reshape(levels, bs, s, nh, hd).permute(0, 1, 3, 2, 4)
+    dy_heads = dy_heads.reshape(nb, s, hd).contiguous()
+    outs = []
+    for tokens in (False, True):
+        gr = [z(nb, s, hd) for _ in range(3)] + [z(nb, s) for _ in range(3)] + [z(hd, hd), z(hd, hd)]
+        if tokens:
+            D.call("titans_chunkwise_backward_bf16_tokens_rocm", k, v, q, al, th, et, mc1, sc1, dy_tok, *gr, s, hd, nb,
+                   C, nh, levels, int(per_level))
+        else:
+            D.call("titans_chunkwise_backward_bf16_rocm", k, v, q, al, th, et, mc1, sc1, dy_heads, *gr, s, hd, nb, C)
+        outs.append(gr)
+    torch.cuda.synchronize()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
