@@ -511,6 +511,26 @@ __global__ void accumulate_over_batch_kernel(const float *src, float *dst, int b
     dst[i] += s;
 }
 
+// The same for up to two [batch, n] sources in one launch (blockIdx.y picks the pair); the batch is
+// summed in four interleaved partial sums (independent loads in flight), combined in a fixed order.
+__global__ void accumulate_over_batch2_kernel(const float *src_a, float *dst_a, const float *src_b, float *dst_b,
+                                              int batch, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float *src = blockIdx.y ? src_b : src_a;
+    float *dst = blockIdx.y ? dst_b : dst_a;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int b = 0;
+    for (; b + 4 <= batch; b += 4) {
+        s0 += src[(size_t)b * n + i];
+        s1 += src[(size_t)(b + 1) * n + i];
+        s2 += src[(size_t)(b + 2) * n + i];
+        s3 += src[(size_t)(b + 3) * n + i];
+    }
+    for (; b < batch; b++) s0 += src[(size_t)b * n + i];
+    dst[i] += (s0 + s1) + (s2 + s3);
+}
+
 // ───────────────────────────── host dispatch ───────────────────────────────
 void finalize_parts(const float *ws_dq, const float *ws_dk, const float *ws_gate,
                     float *d_q, float *d_k, float *d_alpha, float *d_theta, float *d_eta,
@@ -520,6 +540,13 @@ void finalize_parts(const float *ws_dq, const float *ws_dk, const float *ws_gate
     hipLaunchKernelGGL(finalize_parts_kernel, grid, dim3(256), 0, stream(), ws_dq, ws_dk, ws_gate,
                        d_q, d_k, d_alpha, d_theta, d_eta, parts, batch, seq_len, d, t_start, t_end);
     check_launch("finalize_parts_kernel");
+}
+
+void accumulate_over_batch2(const float *src_a, float *dst_a, const float *src_b, float *dst_b, int batch, int n) {
+    KernelTimer kt("accumulate_over_batch_kernel");
+    hipLaunchKernelGGL(accumulate_over_batch2_kernel, dim3(ceil_div(n, 64), src_b ? 2 : 1), dim3(64), 0, stream(),
+                       src_a, dst_a, src_b, dst_b, batch, n);
+    check_launch("accumulate_over_batch2_kernel");
 }
 
 bool coupled_needed(float error_clip, float m_norm_max) {
@@ -959,8 +986,7 @@ void titans_backward_f32_cuda(const float *k_mem, const float *v_mem, const floa
               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
               dm, ds, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
     if (!launch_bwd<true>(a, d)) { unsupported("titans_backward_f32_cuda", d, error_clip > 0.f); return; }
-    accumulate_over_batch(dm, d_m_initial, batch_size, (int)dd);
-    accumulate_over_batch(ds, d_s_initial, batch_size, (int)dd);
+    accumulate_over_batch2(dm, d_m_initial, ds, d_s_initial, batch_size, (int)dd);
 }
 
 // Same contract and kernels as titans_backward_f32_cuda for callers that cannot allocate device
@@ -992,8 +1018,7 @@ void titans_backward_noalloc_f32_rocm(const float *k_mem, const float *v_mem, co
               d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, nullptr, nullptr, nullptr,
               dm, ds, seq_len, 0, seq_len, 1, batch_size, (long long)((seq_len + 1) * dd), error_clip};
     if (!launch_bwd<true>(a, d, base + state_floats, true)) { unsupported(fn, d, coupled); return; }
-    accumulate_over_batch(dm, d_m_initial, batch_size, (int)dd);
-    accumulate_over_batch(ds, d_s_initial, batch_size, (int)dd);
+    accumulate_over_batch2(dm, d_m_initial, ds, d_s_initial, batch_size, (int)dd);
 }
 
 void delta_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,

@@ -378,8 +378,7 @@ static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q
     if (a.parts > 1)
         finalize_parts(a.ws_dq, a.ws_dk, a.ws_gate, d_q, d_k, d_alpha, d_theta,
                        HAS_S ? d_eta : nullptr, a.parts, batch, seq_len, d, 0, seq_len);
-    accumulate_over_batch(a.d_m_out, d_m_initial, batch, (int)dd);
-    if (HAS_S) accumulate_over_batch(a.d_s_out, d_s_initial, batch, (int)dd);
+    accumulate_over_batch2(a.d_m_out, d_m_initial, HAS_S ? a.d_s_out : nullptr, d_s_initial, batch, (int)dd);
     return true;
 }
 

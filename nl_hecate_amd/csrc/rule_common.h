@@ -58,6 +58,8 @@ void unsupported(const char *fn, int d, bool coupled);
 bool coupled_needed(float error_clip, float m_norm_max);
 // dst[i] += sum_b src[b, i]
 void accumulate_over_batch(const float *src, float *dst, int batch, int n);
+// the same for two pairs in one launch (src_b may be null)
+void accumulate_over_batch2(const float *src_a, float *dst_a, const float *src_b, float *dst_b, int batch, int n);
 // d_q/d_k/gates = sum over parts of the partial buffers, tokens [t_start, t_end)
 void finalize_parts(const float *ws_dq, const float *ws_dk, const float *ws_gate,
                     float *d_q, float *d_k, float *d_alpha, float *d_theta, float *d_eta,
