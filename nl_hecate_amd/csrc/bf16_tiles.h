@@ -59,6 +59,21 @@ __device__ __forceinline__ Gates fetch_gates(const float *alpha, const float *th
     return g;
 }
 
+// Workgroup -> (chain, half of its rows) for the chain-resident kernels (grid = 2 * batch).  Workgroups go
+// to the 8 XCDs round robin in linear order and each XCD has its own L2: the two halves of a chain read the
+// same K, Q and coefficient tables, so they get linear ids 8 apart (same XCD, dispatched together; with more
+// workgroups than fit at once they also run in the same round and the second reader hits L2).
+__device__ __forceinline__ void chain_half_of_block(int batch, int &chain, int &half) {
+    const int id = blockIdx.x;
+    if ((batch & 7) == 0) {
+        chain = (id >> 4) * 8 + (id & 7);
+        half = (id >> 3) & 1;
+    } else {
+        chain = id % batch;
+        half = id / batch;
+    }
+}
+
 // Store of four consecutive elements as bf16 (round to nearest even).
 __device__ __forceinline__ void bf16_store(u16 *X, int off, f32x4 x) {
     bf16x4 h;

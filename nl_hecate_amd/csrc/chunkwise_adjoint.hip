@@ -43,7 +43,9 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     float *cvec = reinterpret_cast<float *>(dEl + HMAT);             // a, beta, cl, bl, theta [64] each, .., h_L
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
-    const int chain = blockIdx.x % batch, half = blockIdx.x / batch, i0 = 32 * half;
+    int chain, half;
+    chain_half_of_block(batch, chain, half);
+    const int i0 = 32 * half;
     const size_t chain_tok = (size_t)chain * s, state0 = (size_t)chain * (nc + 1) * HD * HD;
     const size_t dy_off = dyr.offset(chain);
     const int st_t = 16 * (w & 3) + (l & 15), st_cb = 4 * (w >> 2) + (l >> 4);   // bf16 tile: row, 8-element block

@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void cw_coef_kernel(const float *__restrict__ 
 // repeat the last chunk): memory waits are placed per program point, not per path.
 //
 // The rows of M and S never mix, so a chain is split over two workgroups of 32 rows each
-// (workgroup = blockIdx.x / batch picks the half, so both halves of a chain share an XCD's L2
+// (chain_half_of_block: both halves of a chain share an XCD's L2 and are dispatched together
 // for K, Q and W).  Waves 0..3 (group X): E, then Y^T, one 16-token strip each.  Waves 4..7
 // (group Y): one 32x32 block of W.P each, then one 16-column strip of the transposed state
 // update; they hold the fp32 master state.
@@ -140,7 +140,9 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
     float *cvec = reinterpret_cast<float *>(ESl + HMAT);   // a, beta, wM, wS [64] each, then a_L, beta_L, h_L
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
-    const int chain = blockIdx.x % batch, i0 = 32 * (blockIdx.x / batch);
+    int chain, half;
+    chain_half_of_block(batch, chain, half);
+    const int i0 = 32 * half;
     const bool grpX = w < 4;
     const int bi = w & 3, bm = 32 * (bi >> 1), bn = 32 * (bi & 1);   // group Y: 32x32 block of P^T; group X: strip bi
     const size_t chain_tok = (size_t)chain * s;

@@ -2,6 +2,9 @@
 (LayerNorm, embedding, transpose copy, cross-entropy, TNT helpers, 1-D pooling, M3 helpers).  Each function
 cites the reference lines it follows and computes in the dtype of its inputs (float32 = the arithmetic the
 reference runs, float64 for pinning).  Only tests/, the smoke check and bench.py's CPU baseline may import it.
+Pinned by tests/test_oracle_model_glue.py: torch's library routines and autograd in float64, and for the M3
+helpers the known answers that the reference's own tests hold (core/tests/test_m3.rs), kept as
+tests/golden/m3_known_answers.json.
 """
 import numpy as np
 
