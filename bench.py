@@ -15,6 +15,8 @@ Workloads (BASELINE.json `configs`):
                     tokens (checkpointed forward + fused checkpointed backward).
   swa_c5            the attention branch of configs[4]: sliding-window attention, window 512,
                     8 heads x 64, bf16 storage, fp32 softmax, batch 8, seq 4096, fwd+bwd.
+  swa_stats_c5      the same attention through the pair that keeps two softmax statistics per query
+                    instead of the weight tensor (what the layer calls).
   mag_layer_c5      configs[4]: the full layer — CMS of k=4 Titans levels (periods 1, 8, 64, 512;
                     chunkwise rule, chunk 64) gating sliding-window attention (window 512), 8 heads
                     x 64, batch 8, seq 4096: forward + backward + frequency-aware AdamW step.
@@ -295,7 +297,7 @@ def cpu_baseline_swa(q, k, v, d_out, window, heads, budget_s=12.0):
                       f"filled, so this overstates the CPU rate), forward + backward, {el:.1f} s"}
 
 
-def setup_swa_c5(torch, D, lib):
+def setup_swa_c5(torch, D, lib, lse=False):
     bs, heads, hd, s, window = 8, 8, 64, 4096, 512
     td = heads * hd
     g = torch.Generator(device="cpu").manual_seed(0x5EED0005)
@@ -306,20 +308,32 @@ def setup_swa_c5(torch, D, lib):
     aw = torch.zeros(bs, heads, s, window, dtype=torch.bfloat16, device="cuda")
     dq, dk, dv = (torch.zeros(bs, s, td, dtype=torch.float32, device="cuda") for _ in range(3))
 
+    stats = torch.zeros(bs, heads, s, 2, dtype=torch.float32, device="cuda")
+
     def fwd():
-        D.call("swa_forward_f32_cuda", qd, kd, vd, out, aw, s, heads, hd, window, bs, 0)
+        if lse:
+            D.call("swa_forward_lse_bf16_rocm", qd, kd, vd, out, stats, s, heads, hd, window, bs)
+        else:
+            D.call("swa_forward_f32_cuda", qd, kd, vd, out, aw, s, heads, hd, window, bs, 0)
 
     def bwd():
         dk.zero_(); dv.zero_()
-        D.call("swa_backward_f32_cuda", qd, kd, vd, aw, dod, dq, dk, dv, s, heads, hd, window, bs, 0)
+        if lse:
+            D.call("swa_backward_lse_bf16_rocm", qd, kd, vd, stats, dod, dq, dk, dv, s, heads, hd, window, bs)
+        else:
+            D.call("swa_backward_f32_cuda", qd, kd, vd, aw, dod, dq, dk, dv, s, heads, hd, window, bs, 0)
 
+    # the statistics pair moves 8 bytes per head-token where the contract pair moves the 1024-byte weight row
+    wbytes = 8 if lse else 1024
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * heads * s, bound="hbm", dtype="bf16",
-        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD, bytes_fwd=BYTES_SWA_FWD, bytes_bwd=BYTES_SWA_BWD,
+        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD + (FLOP_SWA_FWD if lse else 0),
+        bytes_fwd=BYTES_SWA_FWD - 1024 + wbytes, bytes_bwd=BYTES_SWA_BWD - 1024 + wbytes,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
         kernel_names={"forward": "swa_forward", "backward": "swa_backward"},
         config={"workload": "BASELINE configs[4], attention branch: sliding-window attention, window 512, 8 heads x 64, "
-                            "bf16 storage with fp32 softmax, batch 8, seq 4096, fwd+bwd",
+                            "bf16 storage with fp32 softmax, batch 8, seq 4096, fwd+bwd"
+                            + (", per-query softmax statistics kept instead of the weight tensor" if lse else ""),
                 "batch": bs, "heads": heads, "head_dim": hd, "seq_len": s, "window": window},
         cpu=lambda: cpu_baseline_swa(q, k, v, d_out, window, heads))
 
@@ -560,6 +574,7 @@ def setup_hebbian_c2(torch, D, lib):
 
 WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
              "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5,
+             "swa_stats_c5": lambda torch, D, lib: setup_swa_c5(torch, D, lib, lse=True),
              "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5, "hebbian_c2": setup_hebbian_c2}
 
 

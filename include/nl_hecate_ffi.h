@@ -369,6 +369,18 @@ void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t 
                            float *d_q, float *d_k, float *d_v, int seq_len, int num_heads, int head_dim,
                            int window_size, int batch_size, int n_persistent);
 
+/* No counterpart in the reference (its backward, core/src/cuda_ffi.rs:62, reads the weight tensor the forward
+ * stored): the same attention with the weight tensor left out.  The forward stores per query only
+ * stats [batch, heads, seq, 2] fp32 = (max_j score * log2(e) / sqrt(hd), 1 / sum_j exp(...)); the backward rebuilds
+ * each weight from q . k and those two numbers, rounded to bf16 as the stored tensor would hold it.
+ * head_dim 64, window_size <= 512, no persistent prefix; other shapes are an error.  out, d_q, d_k, d_v as in
+ * the pair above (d_k, d_v accumulated). */
+void swa_forward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, float *stats,
+                               int seq_len, int num_heads, int head_dim, int window_size, int batch_size);
+void swa_backward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, const float *stats,
+                                const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len,
+                                int num_heads, int head_dim, int window_size, int batch_size);
+
 /* ── AdamW and gradient clipping; return hipError_t as unsigned, 0 = success ─ */
 /* core/src/cuda_ffi.rs:674 */
 unsigned adamw_update_cuda(float *w, const float *g, float *m, float *v, int n, float lr, float beta1,
@@ -487,7 +499,8 @@ void memory_read_only_backward_f32_rocm(const float *d_y, const float *m, float 
  *   embedded  [batch, seq_len, d]
  *   y, k/v/q_cache [batch, seq_len, d];  alpha/theta/alpha_mean/eta_mean_cache [batch, seq_len]
  *   frozen    [batch, num_chunks, 6, d*d], num_chunks = ceil(seq_len / chunk_size)
- * d in {16, 32, 64}. */
+ * d = 16, 32, 64 run on the tiled kernels; every other d from 1 to 512 on general ones (the reference's own
+ * tests use d = 4, core/src/chunkwise_self_ref.rs:662); larger d is an error. */
 void selfref_chunkwise_forward_f32_rocm(float *mems, const float *embedded, float *y, float *k_cache,
                                         float *v_cache, float *q_cache, float *alpha_cache,
                                         float *theta_cache, float *alpha_mean_cache, float *eta_mean_cache,

@@ -128,17 +128,26 @@ __global__ void scale_kernel(float *g, float scale, const float *scale_ptr, int 
 }
 
 // norm = sqrt(sum partials); scale = min(1, max/norm) (core/kernels/adamw.cu:203-236)
-__global__ void reduce_partials_clip_kernel(const float *__restrict__ partial, int total,
-                                            float max_grad_norm, float *out_norm, float *out_scale) {
-    __shared__ float part[kOptThreads / 64];
-    float acc = 0.f;
-    for (int i = threadIdx.x; i < total; i += blockDim.x) acc += partial[i];
-    acc = wave_allreduce(acc);
+constexpr int kClipThreads = 1024;   // one workgroup; four independent partial sums per thread
+__global__ __launch_bounds__(kClipThreads) void reduce_partials_clip_kernel(const float *__restrict__ partial, int total,
+                                                                            float max_grad_norm, float *out_norm,
+                                                                            float *out_scale) {
+    __shared__ float part[kClipThreads / 64];
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int i = threadIdx.x;
+    for (; i + 3 * kClipThreads < total; i += 4 * kClipThreads) {
+        a0 += partial[i];
+        a1 += partial[i + kClipThreads];
+        a2 += partial[i + 2 * kClipThreads];
+        a3 += partial[i + 3 * kClipThreads];
+    }
+    for (; i < total; i += kClipThreads) a0 += partial[i];
+    float acc = wave_allreduce((a0 + a1) + (a2 + a3));
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0) {
         float t = 0.f;
-        for (int w = 0; w < kOptThreads / 64; w++) t += part[w];
+        for (int w = 0; w < kClipThreads / 64; w++) t += part[w];
         const float norm = sqrtf(t);
         *out_norm = norm;
         *out_scale = (norm > max_grad_norm && max_grad_norm > 0.0f) ? (max_grad_norm / norm) : 1.0f;
@@ -298,7 +307,7 @@ unsigned grad_scale_cuda(float *g, float scale, int n) {
 
 unsigned reduce_partials_clip_cuda(const float *partial_sums, int total_partials, float max_grad_norm,
                                    float *out_norm, float *out_scale) {
-    hipLaunchKernelGGL(reduce_partials_clip_kernel, dim3(1), dim3(kOptThreads), 0, stream(), partial_sums,
+    hipLaunchKernelGGL(reduce_partials_clip_kernel, dim3(1), dim3(kClipThreads), 0, stream(), partial_sums,
                        total_partials, max_grad_norm, out_norm, out_scale);
     return launch_status("reduce_partials_clip_cuda");
 }

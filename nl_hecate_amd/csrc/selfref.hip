@@ -28,6 +28,7 @@
 #include "lane_ops.h"
 #include "quad_rows.h"
 #include "runtime.h"
+#include "selfref_generic.h"
 
 namespace nlh {
 namespace {
@@ -1182,10 +1183,13 @@ void launch_bwd(const BwdArgs &a) {
     else launch_bwd_sg<D, false>(a);
 }
 
+// head sizes of the tiled kernels; every other one takes the general kernels of selfref_generic.hip
+bool tiled_head_size(int d) { return d == 16 || d == 32 || d == 64; }
+
 bool check_args(const char *fn, int seq_len, int d, int batch, int chunk_size) {
     if (seq_len <= 0 || batch <= 0) { fail("%s: seq_len and batch_size must be positive", fn); return false; }
     if (chunk_size < 1) { fail("%s: chunk_size must be >= 1", fn); return false; }
-    if (d != 16 && d != 32 && d != 64) { fail("%s: d=%d unsupported (16, 32, 64)", fn, d); return false; }
+    if (!tiled_head_size(d) && !selfref_generic_check(fn, d)) return false;
     return true;
 }
 
@@ -1203,6 +1207,11 @@ extern "C" void selfref_chunkwise_forward_f32_rocm(float *mems, const float *emb
     const int C = chunk_size > seq_len ? seq_len : chunk_size;
     const int nc = (seq_len + chunk_size - 1) / chunk_size;
     const bool sg = self_generated_values != 0;
+    if (!tiled_head_size(d)) {
+        selfref_forward_generic(mems, embedded, y, k_cache, v_cache, q_cache, alpha_cache, theta_cache,
+                                alpha_mean_cache, eta_mean_cache, frozen, seq_len, d, batch_size, C, nc, sg);
+        return;
+    }
 #define NLH_FWD(DV) launch_fwd<DV>(sg, batch_size, mems, embedded, y, k_cache, v_cache, q_cache, alpha_cache, \
                                    theta_cache, alpha_mean_cache, eta_mean_cache, frozen, seq_len, C, nc)
     if (d == 16) NLH_FWD(16); else if (d == 32) NLH_FWD(32); else NLH_FWD(64);
@@ -1221,6 +1230,11 @@ extern "C" void selfref_chunkwise_backward_f32_rocm(const float *embedded, const
     const int C = chunk_size > seq_len ? seq_len : chunk_size;
     const int nc = (seq_len + chunk_size - 1) / chunk_size;
     const bool sg = self_generated_values != 0;
+    if (!tiled_head_size(d)) {
+        selfref_backward_generic(embedded, d_y, k_cache, v_cache, q_cache, alpha_cache, theta_cache, alpha_mean_cache,
+                                 eta_mean_cache, frozen, d_embedded, d_mems, seq_len, d, batch_size, C, nc, sg);
+        return;
+    }
     const size_t dd = (size_t)d * d;
     const size_t traj_bytes = (size_t)batch_size * C * dd * sizeof(float);
     if (C > kLrC && traj_bytes > ((size_t)32 << 30)) {

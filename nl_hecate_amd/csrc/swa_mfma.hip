@@ -149,12 +149,15 @@ __device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int k
     return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
 }
 
+// LSE: the weights are not written; the query's softmax statistics (its maximum in exp2 units and the
+// reciprocal of its sum) go to stats [batch * H, s] instead, from which the backward rebuilds the weights.
+template <bool LSE>
 __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
                                                            const unsigned short *__restrict__ k,
                                                            const unsigned short *__restrict__ v,
                                                            unsigned short *__restrict__ out,
-                                                           unsigned short *__restrict__ attn_w, int s, int H,
-                                                           int ws) {
+                                                           unsigned short *__restrict__ attn_w,
+                                                           float2 *__restrict__ stats, int s, int H, int ws) {
     __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage [stage_pos(key)][dim], then V^T stage [dim][key]
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
@@ -235,12 +238,13 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+    if (LSE && g == 0 && tq < s) stats[(size_t)(b * H + h) * s + tq] = make_float2(mc, inv);
 
     // ---- pass B: O^T = V^T P^T, weights out ----
     f32x4 o[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+    unsigned short *wrow = LSE ? nullptr : attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
     __syncthreads();   // every wave is done with the last K stage
     load_pairs(vm, base + KS * st_lo, stg);
 #pragma unroll
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
             // the lane's 8 weights are slots key0 - lsq .. + 7 of its query's row; keys after the
             // query carry zeros, which the contract wants written while the slot exists
             const int key0 = base + KS * st + 32 * hf + 8 * g, slot0 = key0 - lsq;
-            if (tq < s) {
+            if (!LSE && tq < s) {
                 if (slot0 >= 0 && slot0 + 8 <= ws) {
                     __builtin_memcpy(wrow + slot0, &pb, 16);
                 } else if (slot0 + 8 > 0 && slot0 < ws) {
@@ -273,7 +277,7 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
         }
     }
     // slots whose keys lie beyond the block's last key (early queries only): zero
-    if (t0 + QB < ws) {
+    if (!LSE && t0 + QB < ws) {
         unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
         for (int qi = 0; qi < 16; qi++) {
             const int tt = t0 + 16 * wave + qi;
@@ -300,9 +304,14 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
 // load of its weight row, kept in registers for the second sweep.  Only the last stage, the one that
 // holds the queries themselves, is read slot by slot: its groups can end inside the 16 bytes, and a
 // load that runs past the query's row would leave the array at its last row.
-__global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
+// LSE: the weights of a stage are rebuilt from the scores (the forward's own sequence of matrix-core steps on the
+// K stage, which takes the place of the V stage that sweep 1 does not use) and the query's statistics.
+template <bool LSE>
+__global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ q,
+                                                                const unsigned short *__restrict__ k,
                                                                 const unsigned short *__restrict__ v,
                                                                 const unsigned short *__restrict__ attn_w,
+                                                                const float2 *__restrict__ stats,
                                                                 const float *__restrict__ d_out,
                                                                 float *__restrict__ d_q, float *__restrict__ dvec,
                                                                 int s, int H, int ws) {
@@ -317,8 +326,41 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
     const int lsq = max(tq + 1 - ws, 0);
     const size_t row0 = (size_t)b * s;
     const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
-    const unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+    const unsigned short *wrow = LSE ? nullptr : attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
     const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
+    uint4 qf[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    float q_mc = 0.f, q_inv = 0.f;
+    if (LSE && tq < s) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+            qf[ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
+        const float2 st2 = stats[(size_t)(b * H + h) * s + tq];
+        q_mc = st2.x;
+        q_inv = st2.y;
+    }
+    // LSE: weights of stage `stage` from its K rows in T (tile order): scores, mask, exp2, normalise, bf16
+    auto rebuild_weights = [&](unsigned short (*T)[LDH], int stage, uint4 (&w)[2]) {
+        const float c2 = 0.125f * 1.44269504088896340736f;
+        const int k0 = base + KS * stage;
+        f32x4 a[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+            a[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) a[kt] = mfma32(ld_op(T, 16 * kt, ks), qf[ks], a[kt]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int key = k0 + tile_key(kt, g, i);
+                const bool ok = key >= lsq && key <= tq && tq < s;
+                a[kt][i] = ok ? __builtin_amdgcn_exp2f(fmaf(a[kt][i], c2, -q_mc)) * q_inv : 0.f;
+            }
+        }
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            const f32x4 p0 = a[2 * hf], p1 = a[2 * hf + 1];
+            w[hf] = make_uint4(pack2(p0[0], p0[1]), pack2(p0[2], p0[3]), pack2(p1[0], p1[1]), pack2(p1[2], p1[3]));
+        }
+    };
 
     // weights of this lane's query for the keys of its group in a stage: wv[stage][hf] holds the
     // 8 keys 32 hf + 8 g .. + 7, zero outside the window
@@ -357,14 +399,20 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
 #pragma unroll
     for (int st = 0; st < NS; st++) { wv[st][0] = make_uint4(0, 0, 0, 0); wv[st][1] = make_uint4(0, 0, 0, 0); }
     load_pairs(vm, base + KS * st_lo, sv);
+    if (LSE) load_rows(km, base + KS * st_lo, sk);
 #pragma unroll
     for (int st = 0; st < NS; st++) {
         if (st < st_lo) continue;
         const int buf = st & 1;
-        fetch_weights(st, wv[st]);
+        if (!LSE) fetch_weights(st, wv[st]);
         commit_transposed(Tt[buf], sv);
+        if (LSE) commit_rows_tiled(Vr[buf], sk);
         __syncthreads();
-        if (st + 1 < NS) load_pairs(vm, base + KS * (st + 1), sv);
+        if (st + 1 < NS) {
+            load_pairs(vm, base + KS * (st + 1), sv);
+            if (LSE) load_rows(km, base + KS * (st + 1), sk);
+        }
+        if (LSE) rebuild_weights(Vr[buf], st, wv[st]);
 #pragma unroll
         for (int hf = 0; hf < 2; hf++)
 #pragma unroll
@@ -452,9 +500,14 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
 // Two tiles of dS / w in accumulator layout (rows = queries, column = the lane's key) are the A
 // operand of the products with Q^T / dO^T, which are staged transposed in LDS; the rows of the
 // dO stage are stored in tile order (stage_pos) so that those 8 rows are 8 consecutive queries.
+// LSE: the weights are rebuilt per tile from Q K^T (the Q rows of the stage take the LDS matrix of the stored
+// weights, K of the block's keys sits in registers) and the queries' statistics.
+template <bool LSE>
 __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned short *__restrict__ q,
+                                                             const unsigned short *__restrict__ k,
                                                              const unsigned short *__restrict__ v,
                                                              const unsigned short *__restrict__ attn_w,
+                                                             const float2 *__restrict__ stats,
                                                              const float *__restrict__ d_out,
                                                              const float *__restrict__ dvec,
                                                              float *__restrict__ d_k, float *__restrict__ d_v,
@@ -464,21 +517,25 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     __shared__ __align__(16) unsigned short QT[HD][LDH];                   // Q^T, [dim][query]
     __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
     __shared__ float Dv[KS];
+    __shared__ float2 Qst[KS];   // LSE: statistics of the stage's queries
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int j0 = bc.x * QB, h = bc.h, b = bc.b;
     const int total = H * HD, hoff = h * HD;
     const size_t row0 = (size_t)b * s;
     const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
-    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+    const unsigned short *awb = LSE ? nullptr : attn_w + ((size_t)(b * H + h) * s) * ws;
     const float *dvb = dvec + (size_t)(b * H + h) * s;
+    const float2 *stb = LSE ? stats + (size_t)(b * H + h) * s : nullptr;
     const StageSrc qm{q, row0, total, hoff, s};
 
-    uint4 vf[2];
+    uint4 vf[2], kf[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         vf[ks] = make_uint4(0, 0, 0, 0);
+        kf[ks] = make_uint4(0, 0, 0, 0);
         if (kj < s) vf[ks] = *reinterpret_cast<const uint4 *>(v + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
+        if (LSE && kj < s) kf[ks] = *reinterpret_cast<const uint4 *>(k + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
     }
     f32x4 dk[4], dv[4];
 #pragma unroll
@@ -490,8 +547,9 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     f32x4 gdo[4];
     uint4 gq[2];
     unsigned short gw[16];
-    uint4 gwv[2];
+    uint4 gwv[2], gqr[2];
     float gd = 0.f;
+    float2 gst = make_float2(0.f, 0.f);
     // dO: query pair (2 rows) x 4 dims per load; pairs so that the transposed tiles are written as
     // 32-bit words without bank conflicts
     const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // query pair, first dim (+32 for the second half)
@@ -506,6 +564,10 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
                 if (t < s) gdo[2 * cc + c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dd0 + 32 * cc);
             }
         load_pairs(qm, qs0, gq);
+        if (LSE) {   // the stage's Q rows once more, for the tile-ordered copy, and the queries' statistics
+            load_rows(qm, qs0, gqr);
+            gst = (tid < KS && qs0 + tid < s) ? stb[qs0 + tid] : make_float2(0.f, 0.f);
+        } else
         // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t).
         // Past the first stage every query lies after all keys of the block, so a group of 8 keys
         // never runs past the query's row: one 16-byte load (2-byte aligned) per group, the keys
@@ -560,7 +622,10 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
             }
         }
         commit_transposed(QT, gq);
-        if (st == 0) {
+        if (LSE) {
+            commit_rows_tiled(Pt, gqr);
+            if (tid < KS) Qst[tid] = gst;
+        } else if (st == 0) {
 #pragma unroll
             for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
         } else {
@@ -586,10 +651,23 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
                     dw = mfma32(ld_op(Dl, 16 * (2 * hf + c), ks), vf[ks], dw);
                 }
                 unsigned short p4[4];
+                f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};   // LSE: scores of the same tile
+                if (LSE) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ks++) sc = mfma32(ld_op(Pt, 16 * (2 * hf + c), ks), kf[ks], sc);
+                }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int qi = 32 * hf + 8 * g + 4 * c + i;
-                    p4[i] = Pt[qi][16 * wave + r];
+                    if (LSE) {
+                        const int t = qs0 + qi;
+                        const float2 st2 = Qst[qi];
+                        const bool ok = t < s && kj <= t && kj >= max(t + 1 - ws, 0);
+                        const float pf = ok ? __builtin_amdgcn_exp2f(fmaf(sc[i], 0.125f * 1.44269504088896340736f, -st2.x)) * st2.y : 0.f;
+                        p4[i] = (unsigned short)(pack2(pf, 0.f) & 0xffffu);
+                    } else {
+                        p4[i] = Pt[qi][16 * wave + r];
+                    }
                     ds[c][i] = __uint_as_float((unsigned)p4[i] << 16) * (dw[i] - Dv[qi]) * scale;
                 }
                 pw[c][0] = (unsigned)p4[0] | ((unsigned)p4[1] << 16);
@@ -625,11 +703,16 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
 }  // namespace
 
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
-                      int seq_len, int num_heads, int head_dim, int window, int batch, int n_persistent) {
+                      int seq_len, int num_heads, int head_dim, int window, int batch, int n_persistent, float *stats) {
     if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
-    hipLaunchKernelGGL(swa_fwd_mfma_kernel, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, seq_len,
-                       num_heads, window);
+    KernelTimer kt("swa_fwd_mfma_kernel");
+    if (stats)
+        hipLaunchKernelGGL(swa_fwd_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, out, nullptr,
+                           reinterpret_cast<float2 *>(stats), seq_len, num_heads, window);
+    else
+        hipLaunchKernelGGL(swa_fwd_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, nullptr,
+                           seq_len, num_heads, window);
     check_launch("swa_fwd_mfma_kernel");
     return true;
 }
@@ -639,17 +722,30 @@ bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, u
 namespace nlh {
 bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *attn_weights,
                        const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
-                       int head_dim, int window, int batch, int n_persistent) {
+                       int head_dim, int window, int batch, int n_persistent, const float *stats) {
     const ErrorScope es;
     if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
     float *dvec = scratch(1, (size_t)batch * num_heads * seq_len * sizeof(float));
     if (es.failed()) return true;
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
-    hipLaunchKernelGGL(swa_bwd_q_mfma_kernel, grid, dim3(256), 0, stream(), k, v, attn_weights, d_attn_out, d_q, dvec,
-                       seq_len, num_heads, window);
-    check_launch("swa_bwd_q_mfma_kernel");
-    hipLaunchKernelGGL(swa_bwd_k_mfma_kernel, grid, dim3(256), 0, stream(), q, v, attn_weights, d_attn_out, dvec, d_k,
-                       d_v, seq_len, num_heads, window);
+    const float2 *st2 = reinterpret_cast<const float2 *>(stats);
+    {
+        KernelTimer kt("swa_bwd_q_mfma_kernel");
+        if (stats)
+            hipLaunchKernelGGL(swa_bwd_q_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, nullptr, st2,
+                               d_attn_out, d_q, dvec, seq_len, num_heads, window);
+        else
+            hipLaunchKernelGGL(swa_bwd_q_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, attn_weights, nullptr,
+                               d_attn_out, d_q, dvec, seq_len, num_heads, window);
+        check_launch("swa_bwd_q_mfma_kernel");
+    }
+    KernelTimer kt("swa_bwd_k_mfma_kernel");
+    if (stats)
+        hipLaunchKernelGGL(swa_bwd_k_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, nullptr, st2, d_attn_out,
+                           dvec, d_k, d_v, seq_len, num_heads, window);
+    else
+        hipLaunchKernelGGL(swa_bwd_k_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, attn_weights, nullptr,
+                           d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
     check_launch("swa_bwd_k_mfma_kernel");
     return true;
 }

@@ -414,8 +414,14 @@ class MagLayer:
         q = self._project(ops, x2, p.w_q, 0, bf16_out=True).view(bs, s, d)
         k = self._project(ops, x2, p.w_k, 1, bf16_out=True).view(bs, s, d)
         v = self._project(ops, x2, p.w_v, 2, bf16_out=True).view(bs, s, d)
-        attn, aw = _new(bs, s, d, dtype=torch.bfloat16), _new(bs, nh, s, self.window, dtype=torch.bfloat16)
-        D.call("swa_forward_f32_cuda", q, k, v, attn, aw, s, nh, hd, self.window, bs, 0)
+        attn = _new(bs, s, d, dtype=torch.bfloat16)
+        if hd == 64 and self.window <= 512:
+            # per-query softmax statistics instead of the [bs, nh, s, window] weight tensor
+            aw = _new(bs, nh, s, 2)
+            D.call("swa_forward_lse_bf16_rocm", q, k, v, attn, aw, s, nh, hd, self.window, bs)
+        else:
+            aw = _new(bs, nh, s, self.window, dtype=torch.bfloat16)
+            D.call("swa_forward_f32_cuda", q, k, v, attn, aw, s, nh, hd, self.window, bs, 0)
         ys, caches, stack = [], [], None
         if stacked:
             ys, caches, stack = self._levels_forward_stacked(na, x2, bs, s, ops)
@@ -517,8 +523,12 @@ class MagLayer:
             dx = self._level_backward(lv, cache["levels"][lv], x2, d_ycomb, bs, s, grads)
             d_x = dx if d_x is None else d_x.add_(dx)
         dq, dk, dv = _new(bs, s, d), _zeros(bs, s, d), _zeros(bs, s, d)
-        D.call("swa_backward_f32_cuda", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv, s, nh,
-               hd, self.window, bs, 0)
+        if cache["aw"].dtype == torch.float32:
+            D.call("swa_backward_lse_bf16_rocm", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv,
+                   s, nh, hd, self.window, bs)
+        else:
+            D.call("swa_backward_f32_cuda", cache["q"], cache["k"], cache["v"], cache["aw"], d_attn, dq, dk, dv, s,
+                   nh, hd, self.window, bs, 0)
         dq2, dk2, dv2 = dq.view(n, d), dk.view(n, d), dv.view(n, d)
         if P is None:
             dx = self._group_grads(ops, 0, x2, (dq2, dk2, dv2), (p.w_q, p.w_k, p.w_v),

@@ -59,6 +59,11 @@ CASES = [  # B, s, d, C
     (1, 64, 64, 64),    # exactly one full chunk: no chunk boundary is crossed
     (1, 65, 64, 64),    # a one-token chunk after a full one
     (2, 128, 32, 64),
+    # head sizes outside 16 / 32 / 64 take the general kernels; d = 4 is the size of the reference's own tests
+    # (core/src/chunkwise_self_ref.rs:662-1061: s = 4..12, C in {1, 2, 3, 4, s})
+    (1, 4, 4, 1), (1, 8, 4, 2), (1, 12, 4, 4), (2, 7, 4, 3), (1, 6, 4, 6), (1, 5, 4, 8),
+    (2, 33, 1, 4), (2, 40, 5, 7), (1, 50, 12, 16), (2, 45, 24, 64), (1, 70, 48, 20), (1, 30, 100, 9),
+    (1, 150, 8, 70),
 ]
 
 
@@ -110,9 +115,9 @@ def test_bad_arguments_are_reported():
     lib.nlh_set_error_mode(1)
     try:
         lib.nlh_clear_error()
-        mems, x, dy = inputs(1, 8, 24, 0)
+        mems, x, dy = inputs(1, 8, 600, 0)
         SR.chunkwise_self_ref_step(dev(mems), dev(x), 4, True)
-        assert b"unsupported" in lib.nlh_last_error()
+        assert b"beyond the general kernels" in lib.nlh_last_error()
     finally:
         lib.nlh_clear_error()
         lib.nlh_set_error_mode(0)

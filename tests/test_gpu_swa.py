@@ -93,3 +93,66 @@ def test_swa_backward_accumulates_dk_dv_and_overwrites_dq():
     assert_close("d_q", host(dq), oq, 1e-4)
     assert_close("d_k", host(dk) - 1.0, ok, 1e-4)
     assert_close("d_v", host(dv) - 2.0, ov, 1e-4)
+
+
+@pytest.mark.parametrize("B,s,H,ws", [(2, 40, 2, 16), (1, 600, 2, 512), (2, 200, 2, 101), (1, 1100, 1, 300),
+                                      (1, 2, 1, 2), (8, 130, 2, 64), (1, 64, 1, 64), (1, 65, 3, 2)])
+def test_swa_without_weight_tensor(B, s, H, ws):
+    """The pair that keeps per-query softmax statistics instead of the weight tensor: same output bits as the
+    weight-storing forward, statistics against the oracle's scores, gradients against the weight-storing
+    backward (same rounding of the weights: fp32 round-off) and the oracle (bf16 tolerance)."""
+    hd = 64
+    q, k, v, go = _case(B, s, H, hd, 300 + s + ws)
+    out_w, aw = gpu_forward(q, k, v, ws, H, 0)
+    out = torch.zeros(B, s, H * hd, dtype=torch.uint16, device="cuda")
+    stats = torch.full((B, H, s, 2), float("nan"), device="cuda")
+    D.call("swa_forward_lse_bf16_rocm", _u16(q), _u16(k), _u16(v), out, stats, s, H, hd, ws, B)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), out_w)
+    # statistics from the scores in float64
+    qf, kf = (orc.bf16_to_f32(a).astype(np.float64).reshape(B, s, H, hd) for a in (q, k))
+    st = host(stats)
+    for b in range(B):
+        for h in range(H):
+            sc = qf[b, :, h] @ kf[b, :, h].T / 8.0
+            for t in range(0, s, max(1, s // 37)):
+                row = sc[t, max(t + 1 - ws, 0):t + 1]
+                assert abs(st[b, h, t, 0] - row.max() * np.log2(np.e)) < 1e-3 * max(1.0, abs(row.max()))
+                assert abs(st[b, h, t, 1] * np.exp(row - row.max()).sum() - 1.0) < 1e-4
+    dq, dk, dv = zeros(B, s, H * hd), zeros(B, s, H * hd), zeros(B, s, H * hd)
+    D.call("swa_backward_lse_bf16_rocm", _u16(q), _u16(k), _u16(v), stats, dev(go), dq, dk, dv, s, H, hd, ws, B)
+    torch.cuda.synchronize()
+    wq, wk, wv = gpu_backward(q, k, v, aw, go, ws, H, 0)
+    # a weight rebuilt from a score that differs in its last bit may round to the neighbouring bf16
+    assert_close("d_q vs stored weights", host(dq), wq, 2e-3)
+    assert_close("d_k vs stored weights", host(dk), wk, 2e-3)
+    assert_close("d_v vs stored weights", host(dv), wv, 2e-3)
+    oo, awo = orc.swa_forward(q, k, v, ws, H, 0)
+    oq, ok, ov = orc.swa_backward(q, k, v, awo, go, ws, H, 0)
+    assert_close("d_q", host(dq), oq, REL_TOL_BF16)
+    assert_close("d_k", host(dk), ok, REL_TOL_BF16)
+    assert_close("d_v", host(dv), ov, REL_TOL_BF16)
+    # d_k and d_v are accumulated into, d_q is overwritten: a second call doubles the first two only
+    q1, k1, v1 = host(dq), host(dk), host(dv)
+    D.call("swa_backward_lse_bf16_rocm", _u16(q), _u16(k), _u16(v), stats, dev(go), dq, dk, dv, s, H, hd, ws, B)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(dq), q1)
+    assert np.array_equal(host(dk), 2 * k1) and np.array_equal(host(dv), 2 * v1)
+
+
+def test_swa_without_weight_tensor_rejects_other_shapes():
+    from nl_hecate_amd.ffi import lib
+    z = torch.zeros(1, 8, 32, dtype=torch.uint16, device="cuda")
+    st = torch.zeros(1, 1, 8, 2, device="cuda")
+    lib.nlh_set_error_mode(1)
+    try:
+        lib.nlh_clear_error()
+        D.call("swa_forward_lse_bf16_rocm", z, z, z, z, st, 8, 1, 32, 4, 1)
+        assert b"head_dim 64" in lib.nlh_last_error()
+        lib.nlh_clear_error()
+        g = torch.zeros(1, 8, 32, device="cuda")
+        D.call("swa_backward_lse_bf16_rocm", z, z, z, st, g, g, g, g, 8, 1, 32, 4, 1)
+        assert b"head_dim 64" in lib.nlh_last_error()
+    finally:
+        lib.nlh_clear_error()
+        lib.nlh_set_error_mode(0)
