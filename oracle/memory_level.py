@@ -1,0 +1,235 @@
+"""TEST INFRASTRUCTURE ONLY — one CMS memory level end to end on the CPU.
+
+The composition the reference's host code makes around its rule kernels, for the matrix memories:
+gpu_memory_forward (core/src/gpu_forward.rs:1197-1705: projections, L2 normalisation of k and q, gate
+projections and clamps, per-head layout, the rule, carry of the final memory with its Frobenius clamp) and
+gpu_memory_backward (core/src/gpu_backward.rs:459-1200) with accumulate_projection_grads (:2047-2117).
+The rules themselves are the C oracle's (oracle/rules.inc through pyoracle); the glue is written here in
+numpy in the dtype of the inputs, so the whole level also runs in float64 and its backward can be checked
+against finite differences of its forward.  tests/test_oracle_memory_level.py pins the glue against the C
+oracle's float32 glue (orc_gate_compute, orc_l2_normalize_*, orc_gate_backward) and the backward against
+central differences of the float64 forward.
+
+cfg: any object with the attributes of nl_hecate_amd.memory_level.LevelConfig.
+p: dict of numpy arrays w_k, w_v, w_q [d, d], w_alpha, w_theta, w_eta [2d], b_alpha, b_theta, b_eta [1].
+"""
+import numpy as np
+
+from . import pyoracle as orc
+
+F32_MAX = 3.4028234663852886e38
+EPS = 1e-8
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def softplus(x):
+    """core/kernels/elementwise.cu:47: identity above 20."""
+    return np.where(x > 20.0, x, np.log1p(np.exp(np.minimum(x, 20.0))))
+
+
+def l2_normalize(x):
+    """core/kernels/elementwise.cu l2_normalize_rows: x / max(|x|, eps), norms before normalisation."""
+    n = np.sqrt((x * x).sum(-1))
+    return x / np.maximum(n, EPS)[:, None], n
+
+
+def l2_normalize_backward(d_out, x_norm, norms):
+    """d_in = (d_out - x_norm (x_norm . d_out)) / norm for norm >= eps, d_out / eps below it."""
+    dot = (d_out * x_norm).sum(-1, keepdims=True)
+    big = (d_out - x_norm * dot) / np.maximum(norms, EPS)[:, None]
+    return np.where((norms >= EPS)[:, None], big, d_out / EPS)
+
+
+def gate(k, v, w, b, act):
+    d = k.shape[1]
+    z = k @ w[:d] + v @ w[d:] + b[0]
+    return sigmoid(z) if act == 0 else softplus(z)
+
+
+def to_heads(x, bs, s, nh, hd):
+    """[bs*s, nh*hd] -> [bs*nh, s, hd] (reshape_to_per_head, gpu_forward.rs:1133)."""
+    return np.ascontiguousarray(x.reshape(bs, s, nh, hd).transpose(0, 2, 1, 3).reshape(bs * nh, s, hd))
+
+
+def from_heads(x, bs, s, nh, hd):
+    return np.ascontiguousarray(x.reshape(bs, nh, s, hd).transpose(0, 2, 1, 3).reshape(bs * s, nh * hd))
+
+
+def gates_to_heads(g, bs, s, nh):
+    """[bs*s] -> [bs*nh, s] (broadcast_gates, gpu_forward.rs:1161)."""
+    return np.ascontiguousarray(np.repeat(g.reshape(bs, 1, s), nh, axis=1).reshape(bs * nh, s))
+
+
+def gates_from_heads(g, bs, s, nh):
+    return g.reshape(bs, nh, s).sum(1).reshape(bs * s)
+
+
+def frobenius_clamp(m, m_norm_max):
+    """m_norm_clamp_batch_f32_cuda: each [hd, hd] block scaled back onto the ball; off for max <= 0 or >= 1e30."""
+    if not 0 < m_norm_max < 1e30:
+        return m
+    out = m.copy()
+    for i in range(out.shape[0]):
+        n = np.sqrt((out[i] * out[i]).sum())
+        if n > m_norm_max:
+            out[i] *= m_norm_max / n
+    return out
+
+
+def _clamped(cfg):
+    return (cfg.alpha_floor > 0.0 or cfg.alpha_ceil < 1.0), (cfg.theta_floor > 0.0 or cfg.theta_ceil < F32_MAX)
+
+
+def level_forward(p, cfg, x, m0, gates=None):
+    """x [bs, s, d], m0 [bs*nh, hd, hd] -> y [bs, s, d], cache, carried memory [bs*nh, hd, hd].
+    gates: (alpha, theta, eta) to use instead of the computed ones (the reference's backward sends no gradient
+    from the gates into k and v, so a finite-difference check of the k, v, q path holds them fixed)."""
+    bs, s, d = x.shape
+    nh, hd = cfg.num_heads, cfg.head_dim
+    dt = x.dtype
+    x2 = x.reshape(bs * s, d)
+    k_raw, v, q_raw = x2 @ p["w_k"].T, x2 @ p["w_v"].T, x2 @ p["w_q"].T
+    k, k_norms = l2_normalize(k_raw)
+    q, q_norms = l2_normalize(q_raw)
+    alpha = gate(k, v, p["w_alpha"], p["b_alpha"], 0)
+    theta = gate(k, v, p["w_theta"], p["b_theta"], 1)
+    ca, ct = _clamped(cfg)
+    if ca:
+        alpha = np.clip(alpha, cfg.alpha_floor, cfg.alpha_ceil)
+    if ct:
+        theta = np.clip(theta, cfg.theta_floor, cfg.theta_ceil)
+    rule = cfg.memory_rule
+    eta = gate(k, v, p["w_eta"], p["b_eta"], 0) if rule == "titans" else None
+    if gates is not None:
+        alpha, theta, eta = gates
+    kh, vh, qh = (to_heads(t, bs, s, nh, hd) for t in (k, v, q))
+    ah, th = gates_to_heads(alpha, bs, s, nh), gates_to_heads(theta, bs, s, nh)
+    eh = gates_to_heads(eta, bs, s, nh) if eta is not None else None
+    B = bs * nh
+    z = np.zeros((hd, hd), dt)
+    clip = cfg.error_clip
+    # DGD: the Delta update without the per-token projection (core/kernels/dgd_forward.cu:6-11)
+    mx = F32_MAX if rule == "dgd" else cfg.m_norm_max
+    C = cfg.checkpoint_interval
+    ys, ms, ss = [], [], []
+    for b in range(B):
+        if C is not None:
+            if rule == "hebbian":
+                y, m = orc.hebbian_forward(kh[b], vh[b], qh[b], ah[b], m0[b], checkpoint_interval=C)
+                sst = None
+            else:
+                y, m, sst = orc.forward_ckpt(kh[b], vh[b], qh[b], ah[b], th[b], None if eh is None else eh[b], m0[b],
+                                             z, C, has_s=rule == "titans", error_clip=clip, m_norm_max=mx)
+        elif cfg.proxy and rule in ("delta", "titans"):
+            cs = cfg.chunk_size or s
+            y, m, sst = orc.chunkwise_forward(kh[b], vh[b], qh[b], ah[b], th[b], None if eh is None else eh[b], m0[b],
+                                              z, cs, has_s=rule == "titans", error_clip=clip, m_norm_max=mx)
+        elif rule == "titans":
+            y, m, sst = orc.titans_forward(kh[b], vh[b], qh[b], ah[b], th[b], eh[b], m0[b], z, clip, mx)
+        elif rule == "hebbian":
+            y, m = orc.hebbian_forward(kh[b], vh[b], qh[b], ah[b], m0[b])
+            sst = None
+        else:
+            y, m = orc.delta_forward(kh[b], vh[b], qh[b], ah[b], th[b], m0[b], clip, mx)
+            sst = None
+        ys.append(y); ms.append(m); ss.append(sst)
+    y = from_heads(np.stack(ys), bs, s, nh, hd).reshape(bs, s, d)
+    m_states = np.stack(ms)
+    carried = frobenius_clamp(m_states[:, -1], cfg.m_norm_max)
+    cache = dict(k=k, v=v, q=q, alpha=alpha, theta=theta, eta=eta, k_norms=k_norms, q_norms=q_norms,
+                 m_states=m_states, s_states=None if ss[0] is None else np.stack(ss))
+    return y.astype(dt), cache, carried
+
+
+def level_backward(p, cfg, cache, d_y, x):
+    """-> (grads: dict like p, d_x [bs, s, d])."""
+    bs, s, d = x.shape
+    nh, hd = cfg.num_heads, cfg.head_dim
+    dt = x.dtype
+    rule = cfg.memory_rule
+    c = cache
+    kh, vh, qh = (to_heads(c[n], bs, s, nh, hd) for n in ("k", "v", "q"))
+    dyh = to_heads(d_y.reshape(bs * s, d), bs, s, nh, hd)
+    ah, th = gates_to_heads(c["alpha"], bs, s, nh), gates_to_heads(c["theta"], bs, s, nh)
+    eh = gates_to_heads(c["eta"], bs, s, nh) if c["eta"] is not None else None
+    B = bs * nh
+    clip = cfg.error_clip
+    mx = F32_MAX if rule == "dgd" else cfg.m_norm_max
+    C = cfg.checkpoint_interval
+    gs = []
+    for b in range(B):
+        m = c["m_states"][b]
+        sst = None if c["s_states"] is None else c["s_states"][b]
+        if C is not None:
+            if rule == "hebbian":
+                # replay each segment from its checkpoint, then the segment backward
+                # (hebbian_backward_checkpointed, gpu_backward.rs:1967-2035)
+                g = None
+                seed = None
+                t_ends = list(range(0, s, C))
+                for ci in reversed(range(len(t_ends))):
+                    t0, t1 = t_ends[ci], min(t_ends[ci] + C, s)
+                    _, traj = orc.hebbian_forward(kh[b][t0:t1], vh[b][t0:t1], qh[b][t0:t1], ah[b][t0:t1], m[ci])
+                    gi = orc.hebbian_backward(kh[b], vh[b], qh[b], ah[b], traj, dyh[b], t0, t1, seed)
+                    seed = gi["d_m"]
+                    if g is None:
+                        g = gi
+                    else:
+                        for n in ("d_k", "d_v", "d_q", "d_alpha"):
+                            g[n] = g[n] + gi[n]
+            else:
+                g = orc.backward_ckpt(kh[b], vh[b], qh[b], ah[b], th[b], None if eh is None else eh[b], m, sst,
+                                      dyh[b], C, has_s=rule == "titans", error_clip=clip, m_norm_max=mx)
+        elif cfg.proxy and rule in ("delta", "titans"):
+            cs = cfg.chunk_size or s
+            g = orc.chunkwise_backward(kh[b], vh[b], qh[b], ah[b], th[b], None if eh is None else eh[b], m, sst,
+                                       dyh[b], cs, has_s=rule == "titans", error_clip=clip, m_norm_max=mx)
+        elif rule == "titans":
+            g = orc.titans_backward(kh[b], vh[b], qh[b], ah[b], th[b], eh[b], m, sst, dyh[b], clip)
+        elif rule == "hebbian":
+            g = orc.hebbian_backward(kh[b], vh[b], qh[b], ah[b], m, dyh[b])
+        else:
+            g = orc.delta_backward(kh[b], vh[b], qh[b], ah[b], th[b], m, dyh[b], clip)
+        gs.append(g)
+    stack = lambda n: np.stack([g[n] for g in gs])
+    d_k, d_v, d_q = (from_heads(stack(n), bs, s, nh, hd) for n in ("d_k", "d_v", "d_q"))
+    d_alpha = gates_from_heads(stack("d_alpha"), bs, s, nh)
+    has_theta, has_eta = rule != "hebbian", rule == "titans"
+    d_theta = gates_from_heads(stack("d_theta"), bs, s, nh) if has_theta else None
+    d_eta = gates_from_heads(stack("d_eta"), bs, s, nh) if has_eta else None
+    # straight-through clamps: no gradient where the gate sits on a bound (theta_clamp_mask_cuda)
+    ca, ct = _clamped(cfg)
+    if ca:
+        d_alpha = np.where((c["alpha"] <= cfg.alpha_floor) | (c["alpha"] >= cfg.alpha_ceil), 0.0, d_alpha)
+    if ct and has_theta:
+        d_theta = np.where((c["theta"] <= cfg.theta_floor) | (c["theta"] >= cfg.theta_ceil), 0.0, d_theta)
+    return projection_grads(p, x, c, d_k, d_v, d_q, d_alpha, d_theta, d_eta)
+
+
+def projection_grads(p, x, c, d_k, d_v, d_q, d_alpha, d_theta, d_eta):
+    """accumulate_projection_grads (gpu_backward.rs:2047-2117).  As there, the gate gradients reach the gate
+    weights only: the gates' own inputs k, v receive no gradient from them."""
+    bs, s, d = x.shape
+    x2 = x.reshape(bs * s, d)
+    d_k_raw = l2_normalize_backward(d_k, c["k"], c["k_norms"])
+    d_q_raw = l2_normalize_backward(d_q, c["q"], c["q_norms"])
+    g = dict(w_k=d_k_raw.T @ x2, w_v=d_v.T @ x2, w_q=d_q_raw.T @ x2)
+    d_x = d_k_raw @ p["w_k"] + d_v @ p["w_v"] + d_q_raw @ p["w_q"]
+    kv = np.concatenate([c["k"], c["v"]], axis=1)
+    pre = d_alpha * c["alpha"] * (1.0 - c["alpha"])
+    g["w_alpha"], g["b_alpha"] = pre @ kv, np.array([pre.sum()])
+    z2, z1 = np.zeros(2 * d, x.dtype), np.zeros(1, x.dtype)
+    if d_theta is not None:
+        pre = d_theta * (1.0 - np.exp(-c["theta"]))
+        g["w_theta"], g["b_theta"] = pre @ kv, np.array([pre.sum()])
+    else:
+        g["w_theta"], g["b_theta"] = z2, z1
+    if d_eta is not None:
+        pre = d_eta * c["eta"] * (1.0 - c["eta"])
+        g["w_eta"], g["b_eta"] = pre @ kv, np.array([pre.sum()])
+    else:
+        g["w_eta"], g["b_eta"] = z2, z1
+    return g, d_x.reshape(bs, s, d)
