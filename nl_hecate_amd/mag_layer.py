@@ -449,9 +449,9 @@ class MagLayer:
 
     # ── decode: one token with a KV cache ────────────────────────────────────
     def decode_reset(self, max_len):
-        """Empties the bf16 KV cache of the attention branch (room for max_len tokens)."""
-        self._kv = (torch.zeros(max_len, self.d, dtype=torch.bfloat16, device="cuda"),
-                    torch.zeros(max_len, self.d, dtype=torch.bfloat16, device="cuda"), 0)
+        """A new, empty bf16 KV cache of the attention branch (room for max_len tokens)."""
+        from .serving import GpuKVCache   # serving imports this module
+        self._kv = GpuKVCache(max_len, self.d, 1)
 
     def decode_step(self, x_t, pulse=None):
         """One token of one sequence, x_t [d] -> out [d]: the layer part of gpu_single_token_forward
@@ -460,18 +460,16 @@ class MagLayer:
         rule on the carried context memory, frozen: read-only), combine, sigmoid gate, W_o.  The caller advances
         the Conductor; `pulse` defaults to its current one."""
         d, nh, hd, p = self.d, self.nh, self.hd, self.p
-        kc, vc, n = self._kv
-        assert n < kc.shape[0], "KV cache full"
+        kv = self._kv
+        assert kv.len < kv.max_len, "KV cache full"
         if pulse is None:
             self.conductor.set_seq_len(1)
             pulse = self.conductor.pulse()
         x2 = x_t.reshape(1, d)
         q = (x2 @ p.w_q.t()).to(torch.bfloat16)
-        kc[n] = (x2 @ p.w_k.t()).to(torch.bfloat16)[0]
-        vc[n] = (x2 @ p.w_v.t()).to(torch.bfloat16)[0]
-        self._kv = (kc, vc, n + 1)
+        kv.append_f32(x2 @ p.w_k.t(), x2 @ p.w_v.t(), 1)
         attn_bf = _new(1, d, dtype=torch.bfloat16)
-        D.call("swa_single_token_cuda", q, kc, vc, attn_bf, n + 1, nh, hd, self.window, 0)
+        D.call("swa_single_token_cuda", q, kv.k_cache_bf16, kv.v_cache_bf16, attn_bf, kv.len, nh, hd, self.window, 0)
         ys = [self._level_forward(lv, x2, 1, 1, bool(pulse.active_levels[lv]))[0] for lv in range(self.k)]
         y_comb, gate, gated = _new(1, 1, d), _new(1, 1, d), _new(1, 1, d)
         ptrs = (ctypes.c_void_p * self.k)(*[y.data_ptr() for y in ys])
