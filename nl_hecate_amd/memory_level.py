@@ -6,6 +6,9 @@ GpuMemoryCache variants of the matrix memories (gpu_forward.rs:129-312):
     Delta, Titans, Hebbian, DGD                  full trajectory  [bs*nh, s+1, hd*hd]
     DeltaCkpt, TitansCkpt, HebbianCkpt, DGDCkpt  checkpoints      [bs*nh, n_ckpt, hd*hd]
     DeltaChunkwise, TitansChunkwise              chunk states     [bs*nh, n_chunks+1, hd*hd]
+    TitansMlp                                    packed MLP state [bs*nh, s+1, 2*hd*dh + dh + hd] per head
+    Mlp (MONETA, YAAD)                           W1 / W2 trajectories [s+1, dh*d], [s+1, d*dh], batch 1
+    SwiGlu                                       the stateless MLP's four activation buffers
 
 Same order of operations and the same cached tensors as the reference: projections of the input,
 L2 normalisation of k and q, gate projections with their clamps, per-head layout, the rule, the final
@@ -29,7 +32,8 @@ from . import dispatch as D
 from .mag_layer import MemoryLevelParams
 
 F32_MAX = 3.4028234663852886e38
-RULES = ("delta", "titans", "hebbian", "dgd")
+RULES = ("delta", "titans", "hebbian", "dgd", "moneta", "yaad", "swiglu")
+ACTIVATIONS = {"gelu": 0, "silu": 1, "relu": 2}   # MemoryActivation -> the kernels' activation id
 
 
 @dataclass
@@ -47,25 +51,42 @@ class LevelConfig:
     theta_ceil: float = F32_MAX
     error_clip: float = 0.0                     # error_clip_for_level(level); 0 = off
     m_norm_max: float = F32_MAX                 # max_m_norm(level)
+    memory_layers: int = 1                      # 2 with "titans": the memory is a two-layer MLP per head
+    memory_expansion_factor: int = 4            # its hidden size = factor * head_dim
+    memory_activation: str = "gelu"             # "gelu", "silu", "relu"
+    d_hidden: int = 0                           # MONETA / YAAD hidden size
+    lp_p: float = 2.0                           # MONETA
+    sign_sharpness: float = 10.0
+    lambda_2: float = 0.0                       # MONETA and YAAD
+    lq_q: float = 2.0
+    delta: float = 1.0                          # YAAD: Huber threshold
+    lambda_local: float = 0.0
+    intermediate_size: int = 0                  # SwiGLU
 
     def __post_init__(self):
         if self.memory_rule not in RULES:
             raise ValueError(f"memory_rule {self.memory_rule!r}: expected one of {RULES}")
         if self.checkpoint_interval is not None and self.checkpoint_interval < 1:
             raise ValueError("checkpoint_interval must be > 0")
+        if self.memory_activation not in ACTIVATIONS:
+            raise ValueError(f"memory_activation {self.memory_activation!r}: expected one of {tuple(ACTIVATIONS)}")
+
+    @property
+    def is_mlp_mem(self):
+        return self.memory_layers == 2 and self.memory_rule == "titans"
 
 
 @dataclass
 class GpuMemoryCache:
     """One of the reference's enum variants; `kind` is the variant's name."""
     kind: str
-    k_mem: torch.Tensor                 # [bs*s, d] normalised
-    v_mem: torch.Tensor
-    q_mem: torch.Tensor                 # [bs*s, d] normalised
-    alpha: torch.Tensor                 # [bs*s]
-    k_norms: torch.Tensor
-    q_norms: torch.Tensor
-    m_states: torch.Tensor              # trajectory, checkpoints or chunk states (see the module text)
+    k_mem: Optional[torch.Tensor] = None      # [bs*s, d] normalised
+    v_mem: Optional[torch.Tensor] = None
+    q_mem: Optional[torch.Tensor] = None      # [bs*s, d] normalised
+    alpha: Optional[torch.Tensor] = None      # [bs*s]
+    k_norms: Optional[torch.Tensor] = None
+    q_norms: Optional[torch.Tensor] = None
+    m_states: Optional[torch.Tensor] = None   # trajectory, checkpoints or chunk states (see the module text)
     theta: Optional[torch.Tensor] = None
     eta: Optional[torch.Tensor] = None
     s_states: Optional[torch.Tensor] = None
@@ -73,11 +94,21 @@ class GpuMemoryCache:
     chunk_size: Optional[int] = None
     num_chunks: Optional[int] = None
     proxy: bool = False
+    d_hidden: Optional[int] = None            # TitansMlp
+    activation: Optional[int] = None
+    w1_states: Optional[torch.Tensor] = None  # Mlp
+    w2_states: Optional[torch.Tensor] = None
+    w1_boundary: Optional[torch.Tensor] = None   # YAAD only: the memory at the start of the call
+    w2_boundary: Optional[torch.Tensor] = None
+    gate_buf: Optional[torch.Tensor] = None   # SwiGlu
+    up_buf: Optional[torch.Tensor] = None
+    fused_buf: Optional[torch.Tensor] = None
+    cache_buf: Optional[torch.Tensor] = None
 
     def dgd_delta_norm(self, s, d, batch_size, num_heads):
         """|M k - v|_2 of the last token against the memory that token was written into
         (gpu_forward.rs:328-437): 0 for several heads, for Hebbian, and without tokens."""
-        if num_heads > 1 or s == 0 or self.kind.startswith("Hebbian"):
+        if num_heads > 1 or s == 0 or self.kind.startswith("Hebbian") or self.kind in ("TitansMlp", "Mlp", "SwiGlu"):
             return 0.0
         assert batch_size <= 1, "dgd_delta_norm reads batch slot 0 only"
         if self.kind.endswith("Chunkwise"):
@@ -97,7 +128,7 @@ class GpuMemoryCache:
 
     def alpha_stats(self, alpha_floor):
         """gpu_forward.rs:440-503."""
-        return GateStats.from_slice(self.alpha.cpu().numpy(), alpha_floor, True)
+        return None if self.alpha is None else GateStats.from_slice(self.alpha.cpu().numpy(), alpha_floor, True)
 
     def eta_stats(self):
         """gpu_forward.rs:505-564: only the Titans variants have a momentum gate."""
@@ -154,11 +185,25 @@ class LevelGrads:
     d_b_theta: torch.Tensor
     d_w_eta: torch.Tensor
     d_b_eta: torch.Tensor
+    d_gate_proj: Optional[torch.Tensor] = None   # SwiGLU levels ([inter, d], [inter, d], [d, inter])
+    d_up_proj: Optional[torch.Tensor] = None
+    d_down_proj: Optional[torch.Tensor] = None
 
     @staticmethod
-    def zeros(d, device="cuda"):
+    def zeros(d, device="cuda", intermediate=0):
         z = lambda *sh: torch.zeros(*sh, dtype=torch.float32, device=device)
-        return LevelGrads(z(d, d), z(d, d), z(d, d), z(2 * d), z(1), z(2 * d), z(1), z(2 * d), z(1))
+        g = LevelGrads(z(d, d), z(d, d), z(d, d), z(2 * d), z(1), z(2 * d), z(1), z(2 * d), z(1))
+        if intermediate:
+            g.d_gate_proj, g.d_up_proj, g.d_down_proj = z(intermediate, d), z(intermediate, d), z(d, intermediate)
+        return g
+
+
+@dataclass
+class SwiGluLevelParams:
+    """The parameters a SwiGLU level reads (GpuMemoryLevelParams gate_proj / up_proj / down_proj)."""
+    gate_proj: torch.Tensor    # [intermediate, d]
+    up_proj: torch.Tensor      # [intermediate, d]
+    down_proj: torch.Tensor    # [d, intermediate]
 
 
 def checkpoint_count(seq_len, c):
@@ -211,8 +256,23 @@ def gpu_memory_forward(level_params: MemoryLevelParams, cfg: LevelConfig, embedd
     lp, bs, nh, hd = level_params, batch_size, cfg.num_heads, cfg.head_dim
     assert nh * hd == d, "num_heads * head_dim must equal d"
     n, B, dd = bs * s, bs * nh, hd * hd
-    assert tuple(embedded.shape) == (n, d) and tuple(context_m.shape) == (B, dd)
+    assert tuple(embedded.shape) == (n, d)
     rule = cfg.memory_rule
+    if rule == "swiglu":   # stateless: no projections, no memory (gpu_forward.rs:1705-1727)
+        inter = cfg.intermediate_size
+        bufs = [_new(n, inter) for _ in range(4)]
+        y = _new(n, d)
+        D.call("swiglu_forward_f32_cuda_dd", embedded, lp.gate_proj, lp.up_proj, lp.down_proj, y, *bufs, n, d, inter)
+        return y, GpuMemoryCache("SwiGlu", gate_buf=bufs[0], up_buf=bufs[1], fused_buf=bufs[2], cache_buf=bufs[3])
+    if cfg.is_mlp_mem and (cfg.checkpoint_interval is not None or cfg.proxy):
+        raise ValueError("MLP memory (memory_layers >= 2) supports neither checkpointing nor the proxy strategy")
+    if rule in ("moneta", "yaad"):
+        if cfg.checkpoint_interval is not None:
+            raise ValueError(f"checkpointed forward is not supported for {rule}: use checkpoint_interval=None")
+        if bs != 1:
+            raise ValueError(f"{rule} forward with batch_size > 1 is not supported")
+    elif not cfg.is_mlp_mem:
+        assert tuple(context_m.shape) == (B, dd)
     k_mem, v_mem, q_mem = embedded @ lp.w_k.t(), embedded @ lp.w_v.t(), embedded @ lp.w_q.t()
     k_norms, q_norms = _new(n), _new(n)
     D.call("l2_normalize_rows_f32_cuda", k_mem, k_norms, n, d, 1e-8)
@@ -224,6 +284,9 @@ def gpu_memory_forward(level_params: MemoryLevelParams, cfg: LevelConfig, embedd
         D.call("clamp_f32_cuda", alpha, n, cfg.alpha_floor, cfg.alpha_ceil)
     if cfg.theta_floor > 0.0 or cfg.theta_ceil < F32_MAX:
         D.call("clamp_f32_cuda", theta, n, cfg.theta_floor, cfg.theta_ceil)
+    common = dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, alpha=alpha, k_norms=k_norms, q_norms=q_norms)
+    if rule in ("moneta", "yaad"):
+        return _mlp_forward(cfg, context_m, theta, common, s, d)
     kh, vh, qh = (_heads(cfg, t, bs, s) for t in (k_mem, v_mem, q_mem))
     ah, th = _gate_heads(cfg, alpha, bs, s), _gate_heads(cfg, theta, bs, s)
     eta = eh = None
@@ -233,8 +296,21 @@ def gpu_memory_forward(level_params: MemoryLevelParams, cfg: LevelConfig, embedd
         eh = _gate_heads(cfg, eta, bs, s)
     yh = _new(B, s, hd)
     clip, mx, C = cfg.error_clip, cfg.m_norm_max, cfg.checkpoint_interval
-    common = dict(k_mem=k_mem, v_mem=v_mem, q_mem=q_mem, alpha=alpha, k_norms=k_norms, q_norms=q_norms)
     s_states = None
+    if cfg.is_mlp_mem:
+        # the memory of a head is {W1, b1, W2, b2} packed; the kernel projects per token, so the carried state
+        # needs no clamp afterwards (gpu_forward.rs:1473-1510)
+        d_h = cfg.memory_expansion_factor * hd
+        n_state = 2 * hd * d_h + d_h + hd
+        assert tuple(context_m.shape) == (B, n_state)
+        act = ACTIVATIONS[cfg.memory_activation]
+        m_states, s_states = _new(B, s + 1, n_state), _new(B, s + 1, n_state)
+        D.call("titans_mlp_forward_f32_cuda", kh, vh, qh, ah, th, eh, context_m, _zeros(B, n_state), m_states, s_states,
+               yh, s, hd, d_h, B, s * hd, (s + 1) * n_state, act, mx)
+        context_m.copy_(m_states[:, -1])
+        cache = GpuMemoryCache("TitansMlp", theta=theta, eta=eta, m_states=m_states, s_states=s_states, d_hidden=d_h,
+                               activation=act, **common)
+        return _tokens(cfg, yh, bs, s), cache
     if C is not None:
         n_ck = checkpoint_count(s, C)
         m_states = _new(B, n_ck, dd)
@@ -288,6 +364,32 @@ def gpu_memory_forward(level_params: MemoryLevelParams, cfg: LevelConfig, embedd
     return _tokens(cfg, yh, bs, s), cache
 
 
+def _mlp_forward(cfg, context_m, theta, common, s, d):
+    """MONETA / YAAD: an MLP memory at model width, one sequence; context_m = [W1 (dh x d) | W2 (d x dh)]
+    (gpu_forward.rs:1729-1852)."""
+    dh = cfg.d_hidden
+    w1_size, w2_size = dh * d, d * dh
+    flat = context_m.view(-1)
+    if flat.numel() < w1_size + w2_size:
+        raise ValueError(f"{cfg.memory_rule}: context_m too small ({flat.numel()} elements) for [W1|W2] = "
+                         f"{w1_size + w2_size} (d_hidden={dh}, d={d})")
+    w1, w2 = flat[:w1_size], flat[w1_size:w1_size + w2_size]
+    w1_states, w2_states, y = _new(s + 1, w1_size), _new(s + 1, w2_size), _new(s, d)
+    c = common
+    b1 = b2 = None
+    if cfg.memory_rule == "yaad":   # the memory at the start of the call anchors the local retention
+        b1, b2 = w1.clone(), w2.clone()
+        D.call("mlp_forward_huber_f32_cuda", c["k_mem"], c["v_mem"], c["q_mem"], c["alpha"], theta, w1, w2, b1, b2,
+               w1_states, w2_states, y, s, d, dh, cfg.delta, cfg.lambda_local, cfg.lambda_2)
+    else:
+        D.call("mlp_forward_lp_f32_cuda", c["k_mem"], c["v_mem"], c["q_mem"], c["alpha"], theta, w1, w2, w1_states,
+               w2_states, y, s, d, dh, cfg.lp_p, cfg.sign_sharpness, cfg.lambda_2, cfg.lq_q)
+    w1.copy_(w1_states[s])
+    w2.copy_(w2_states[s])
+    return y, GpuMemoryCache("Mlp", theta=theta, w1_states=w1_states, w2_states=w2_states, w1_boundary=b1,
+                             w2_boundary=b2, **common)
+
+
 def gpu_memory_backward(level_params: MemoryLevelParams, cfg: LevelConfig, mem_cache: GpuMemoryCache, d_y, embedded,
                         level_grads: LevelGrads, s, d, batch_size):
     """d_y, embedded [bs*s, d].  Writes the level's parameter gradients into level_grads and returns
@@ -295,6 +397,15 @@ def gpu_memory_backward(level_params: MemoryLevelParams, cfg: LevelConfig, mem_c
     c, bs, nh, hd = mem_cache, batch_size, cfg.num_heads, cfg.head_dim
     n, B, dd = bs * s, bs * nh, hd * hd
     kind = c.kind
+    if kind == "SwiGlu":   # direct weight gradients, d_x returned (gpu_backward.rs:1736-1760)
+        inter = cfg.intermediate_size
+        d_x = _new(n, d)
+        D.call("swiglu_backward_f32_cuda_dd", d_y, embedded, level_params.gate_proj, level_params.up_proj,
+               level_params.down_proj, c.fused_buf, c.gate_buf, c.up_buf, c.cache_buf, d_x, level_grads.d_gate_proj,
+               level_grads.d_up_proj, level_grads.d_down_proj, n, d, inter)
+        return d_x
+    if kind == "Mlp":
+        return _mlp_backward(level_params, cfg, c, d_y, embedded, level_grads, s, d, bs)
     has_theta, has_eta = not kind.startswith("Hebbian"), kind.startswith("Titans")
     dyh = _heads(cfg, d_y, bs, s)
     kh, vh, qh = (_heads(cfg, t, bs, s) for t in (c.k_mem, c.v_mem, c.q_mem))
@@ -329,6 +440,11 @@ def gpu_memory_backward(level_params: MemoryLevelParams, cfg: LevelConfig, mem_c
         # the DGD replay leaves the projection off as its forward did (:1156-1161)
         D.call("delta_backward_ckpt_f32_rocm", kh, vh, qh, ah, th, c.m_states, dyh, dkh, dvh, dqh, dah, dth, d_m0, s,
                hd, B, c.checkpoint_interval, clip, F32_MAX if kind == "DGDCkpt" else mx)
+    elif kind == "TitansMlp":
+        n_state = c.m_states.shape[-1]
+        D.call("titans_mlp_backward_f32_cuda", kh, vh, qh, ah, th, eh, c.m_states, c.s_states, dyh, dkh, dvh, dqh, dah,
+               dth, deh, _zeros(n_state), _zeros(n_state), s, hd, c.d_hidden, B, s * hd, (s + 1) * n_state,
+               c.activation, mx)
     elif kind == "TitansCkpt":
         D.call("titans_backward_ckpt_f32_rocm", kh, vh, qh, ah, th, eh, c.m_states, c.s_states, dyh, dkh, dvh, dqh,
                dah, dth, deh, d_m0, d_s0, s, hd, B, c.checkpoint_interval, clip, mx)
@@ -348,6 +464,36 @@ def gpu_memory_backward(level_params: MemoryLevelParams, cfg: LevelConfig, mem_c
     d_k, d_v, d_q = (_tokens(cfg, t, bs, s) for t in (dkh, dvh, dqh))
     return accumulate_projection_grads(level_params, embedded, c, d_k, d_v, d_q, d_alpha, d_theta, d_eta, level_grads,
                                        s, d, bs)
+
+
+def _mlp_backward(level_params, cfg, c, d_y, embedded, level_grads, s, d, bs):
+    """MONETA (L2 retention only: lq_q = 2) / YAAD backward at model width, one sequence
+    (gpu_backward.rs:1635-1733).  As in the reference the gradients of the initial W1, W2 are computed and
+    not used."""
+    if bs != 1:
+        raise ValueError("MLP memory backward with batch_size > 1 is not supported")
+    dh = cfg.d_hidden
+    d_k, d_v, d_q = _zeros(s, d), _zeros(s, d), _zeros(s, d)
+    d_alpha, d_theta = _zeros(s), _zeros(s)
+    d_w1, d_w2 = _zeros(dh * d), _zeros(d * dh)
+    if (c.w1_boundary is None) != (c.w2_boundary is None):
+        raise ValueError("MLP backward: W1 and W2 boundaries must both be present (YAAD) or both absent (MONETA)")
+    if c.w1_boundary is not None:
+        D.call("mlp_backward_huber_f32_cuda", c.k_mem, c.v_mem, c.q_mem, c.alpha, c.theta, c.w1_states, c.w2_states,
+               c.w1_boundary, c.w2_boundary, d_y, d_k, d_v, d_q, d_alpha, d_theta, d_w1, d_w2, s, d, dh, cfg.delta,
+               cfg.lambda_local, cfg.lambda_2)
+    else:
+        if abs(cfg.lq_q - 2.0) >= 1e-6:
+            raise ValueError(f"MONETA backward only supports lq_q=2.0 (L2 retention); got {cfg.lq_q}")
+        D.call("mlp_backward_lp_f32_cuda", c.k_mem, c.v_mem, c.q_mem, c.alpha, c.theta, c.w1_states, c.w2_states, d_y,
+               d_k, d_v, d_q, d_alpha, d_theta, d_w1, d_w2, s, d, dh, cfg.lp_p, cfg.sign_sharpness, cfg.lambda_2,
+               cfg.lq_q)
+    if cfg.alpha_floor > 0.0 or cfg.alpha_ceil < 1.0:
+        D.call("theta_clamp_mask_cuda", c.alpha, d_alpha, s, cfg.alpha_floor, cfg.alpha_ceil)
+    if cfg.theta_floor > 0.0 or cfg.theta_ceil < F32_MAX:
+        D.call("theta_clamp_mask_cuda", c.theta, d_theta, s, cfg.theta_floor, cfg.theta_ceil)
+    return accumulate_projection_grads(level_params, embedded, c, d_k, d_v, d_q, d_alpha, d_theta, None, level_grads, s,
+                                       d, 1)
 
 
 def _hebbian_backward_checkpointed(kh, vh, qh, ah, m_ckpt, dyh, dkh, dvh, dqh, dah, s, hd, c, B):

@@ -15,6 +15,7 @@ p: dict of numpy arrays w_k, w_v, w_q [d, d], w_alpha, w_theta, w_eta [2d], b_al
 """
 import numpy as np
 
+from . import model_glue as glue
 from . import pyoracle as orc
 
 F32_MAX = 3.4028234663852886e38
@@ -91,6 +92,9 @@ def level_forward(p, cfg, x, m0, gates=None):
     nh, hd = cfg.num_heads, cfg.head_dim
     dt = x.dtype
     x2 = x.reshape(bs * s, d)
+    if cfg.memory_rule == "swiglu":   # stateless MLP level (gpu_forward.rs:1705-1727)
+        y, gate_b, up_b, fused, sig = glue.swiglu_forward(x2, p["gate_proj"], p["up_proj"], p["down_proj"])
+        return y.reshape(bs, s, d).astype(dt), dict(gate=gate_b, up=up_b, fused=fused, sig=sig), m0
     k_raw, v, q_raw = x2 @ p["w_k"].T, x2 @ p["w_v"].T, x2 @ p["w_q"].T
     k, k_norms = l2_normalize(k_raw)
     q, q_norms = l2_normalize(q_raw)
@@ -105,6 +109,21 @@ def level_forward(p, cfg, x, m0, gates=None):
     eta = gate(k, v, p["w_eta"], p["b_eta"], 0) if rule == "titans" else None
     if gates is not None:
         alpha, theta, eta = gates
+    base = dict(k=k, v=v, q=q, alpha=alpha, theta=theta, eta=eta, k_norms=k_norms, q_norms=q_norms)
+    if rule in ("moneta", "yaad"):
+        # an MLP memory at model width, one sequence; m0 = (W1 [dh, d], W2 [d, dh]) (gpu_forward.rs:1729-1852)
+        assert bs == 1
+        w1, w2 = m0
+        dh = cfg.d_hidden
+        if rule == "yaad":
+            y, w1s, w2s = orc.miras_mlp_forward(1, k, v, q, alpha, theta, w1, w2, dh, cfg.delta, cfg.lambda_local,
+                                                cfg.lambda_2, boundary=(w1, w2))
+            bnd = (w1, w2)
+        else:
+            y, w1s, w2s = orc.miras_mlp_forward(0, k, v, q, alpha, theta, w1, w2, dh, cfg.lp_p, cfg.sign_sharpness,
+                                                cfg.lambda_2, cfg.lq_q)
+            bnd = None
+        return y.reshape(1, s, d).astype(dt), dict(base, w1_states=w1s, w2_states=w2s, boundary=bnd), (w1s[s], w2s[s])
     kh, vh, qh = (to_heads(t, bs, s, nh, hd) for t in (k, v, q))
     ah, th = gates_to_heads(alpha, bs, s, nh), gates_to_heads(theta, bs, s, nh)
     eh = gates_to_heads(eta, bs, s, nh) if eta is not None else None
@@ -115,8 +134,14 @@ def level_forward(p, cfg, x, m0, gates=None):
     mx = F32_MAX if rule == "dgd" else cfg.m_norm_max
     C = cfg.checkpoint_interval
     ys, ms, ss = [], [], []
+    mlp_mem = rule == "titans" and getattr(cfg, "memory_layers", 1) == 2
     for b in range(B):
-        if C is not None:
+        if mlp_mem:   # per head, the memory a packed two-layer MLP (gpu_forward.rs:1473-1510); no carried clamp
+            d_h = cfg.memory_expansion_factor * hd
+            act = {"gelu": 0, "silu": 1, "relu": 2}[cfg.memory_activation]
+            y, m, sst = orc.titans_mlp_forward(kh[b], vh[b], qh[b], ah[b], th[b], eh[b], m0[b], np.zeros_like(m0[b]),
+                                               d_h, act, mx)
+        elif C is not None:
             if rule == "hebbian":
                 y, m = orc.hebbian_forward(kh[b], vh[b], qh[b], ah[b], m0[b], checkpoint_interval=C)
                 sst = None
@@ -138,9 +163,8 @@ def level_forward(p, cfg, x, m0, gates=None):
         ys.append(y); ms.append(m); ss.append(sst)
     y = from_heads(np.stack(ys), bs, s, nh, hd).reshape(bs, s, d)
     m_states = np.stack(ms)
-    carried = frobenius_clamp(m_states[:, -1], cfg.m_norm_max)
-    cache = dict(k=k, v=v, q=q, alpha=alpha, theta=theta, eta=eta, k_norms=k_norms, q_norms=q_norms,
-                 m_states=m_states, s_states=None if ss[0] is None else np.stack(ss))
+    carried = m_states[:, -1] if mlp_mem else frobenius_clamp(m_states[:, -1], cfg.m_norm_max)
+    cache = dict(base, m_states=m_states, s_states=None if ss[0] is None else np.stack(ss))
     return y.astype(dt), cache, carried
 
 
@@ -151,6 +175,23 @@ def level_backward(p, cfg, cache, d_y, x):
     dt = x.dtype
     rule = cfg.memory_rule
     c = cache
+    if rule == "swiglu":
+        d_x, dg, du, dd = glue.swiglu_backward(d_y.reshape(bs * s, d), x.reshape(bs * s, d), p["gate_proj"],
+                                               p["up_proj"], p["down_proj"], c["fused"], c["gate"], c["up"], c["sig"])
+        return dict(gate_proj=dg, up_proj=du, down_proj=dd), d_x.reshape(bs, s, d)
+    if rule in ("moneta", "yaad"):
+        mode = 1 if rule == "yaad" else 0
+        p1, p2 = (cfg.delta, cfg.lambda_local) if mode else (cfg.lp_p, cfg.sign_sharpness)
+        g = orc.miras_mlp_backward(mode, c["k"], c["v"], c["q"], c["alpha"], c["theta"], c["w1_states"],
+                                   c["w2_states"], d_y.reshape(s, d), cfg.d_hidden, p1, p2, cfg.lambda_2, c["boundary"])
+        d_alpha, d_theta = g["d_alpha"], g["d_theta"]
+        ca, ct = _clamped(cfg)
+        if ca:
+            d_alpha = np.where((c["alpha"] <= cfg.alpha_floor) | (c["alpha"] >= cfg.alpha_ceil), 0.0, d_alpha)
+        if ct:
+            d_theta = np.where((c["theta"] <= cfg.theta_floor) | (c["theta"] >= cfg.theta_ceil), 0.0, d_theta)
+        return projection_grads(p, x, c, g["d_k"], g["d_v"], g["d_q"], d_alpha, d_theta, None)
+    mlp_mem = rule == "titans" and getattr(cfg, "memory_layers", 1) == 2
     kh, vh, qh = (to_heads(c[n], bs, s, nh, hd) for n in ("k", "v", "q"))
     dyh = to_heads(d_y.reshape(bs * s, d), bs, s, nh, hd)
     ah, th = gates_to_heads(c["alpha"], bs, s, nh), gates_to_heads(c["theta"], bs, s, nh)
@@ -163,7 +204,11 @@ def level_backward(p, cfg, cache, d_y, x):
     for b in range(B):
         m = c["m_states"][b]
         sst = None if c["s_states"] is None else c["s_states"][b]
-        if C is not None:
+        if mlp_mem:
+            d_h = cfg.memory_expansion_factor * hd
+            act = {"gelu": 0, "silu": 1, "relu": 2}[cfg.memory_activation]
+            g = orc.titans_mlp_backward(kh[b], vh[b], qh[b], ah[b], th[b], eh[b], m, sst, dyh[b], d_h, act)
+        elif C is not None:
             if rule == "hebbian":
                 # replay each segment from its checkpoint, then the segment backward
                 # (hebbian_backward_checkpointed, gpu_backward.rs:1967-2035)

@@ -9,6 +9,7 @@ import torch
 from nl_hecate_amd import memory_level as GL
 from nl_hecate_amd.mag_layer import MemoryLevelParams
 from oracle import memory_level as ML
+from oracle import pyoracle as orc
 from tests.gpu_util import assert_close, dev, host
 
 pytestmark = pytest.mark.gpu
@@ -149,3 +150,100 @@ def test_gate_statistics_and_delta_norm():
     assert abs(cache.dgd_delta_norm(11, 16, 1, 1) - want) <= 1e-4 * want
     assert cache.eta_stats().count == 11
     assert GL.LevelConfig("hebbian", 2, 8) and out["cache"][0].dgd_delta_norm(11, 16, 1, 2) == 0.0
+
+
+@pytest.mark.parametrize("act", ["gelu", "silu", "relu"])
+@pytest.mark.parametrize("bs,s,nh,hd,factor", [(1, 6, 2, 8, 4), (2, 9, 1, 8, 3)])
+def test_titans_with_an_mlp_memory(act, bs, s, nh, hd, factor):
+    """memory_layers = 2: the packed {W1, b1, W2, b2} state per head (gpu_forward.rs:1473-1510)."""
+    cfg = GL.LevelConfig("titans", nh, hd, memory_layers=2, memory_expansion_factor=factor, memory_activation=act)
+    d, dh = nh * hd, factor * hd
+    n_state = orc.mlp_state_size(hd, dh)
+    r = np.random.default_rng(31 + s)
+    p = params(d, 32)
+    x = (r.standard_normal((bs, s, d)) / np.sqrt(d)).astype(np.float32)
+    m0 = (0.3 * r.standard_normal((bs * nh, n_state)) / np.sqrt(hd)).astype(np.float32)
+    dy = r.standard_normal((bs, s, d)).astype(np.float32)
+    y_o, c_o, carried_o = ML.level_forward(p, cfg, x, m0)
+    g_o, dx_o = ML.level_backward(p, cfg, c_o, dy, x)
+    lp = MemoryLevelParams(*[dev(p[n]) for n in NAMES])
+    ctx, emb = dev(m0), dev(x.reshape(bs * s, d))
+    y, cache = GL.gpu_memory_forward(lp, cfg, emb, ctx, s, d, bs)
+    grads = GL.LevelGrads.zeros(d)
+    d_emb = GL.gpu_memory_backward(lp, cfg, cache, dev(dy.reshape(bs * s, d)), emb, grads, s, d, bs)
+    torch.cuda.synchronize()
+    assert cache.kind == "TitansMlp" and cache.d_hidden == dh
+    out = dict(y=(host(y).reshape(bs, s, d), y_o), cache=(cache, c_o), carried=(host(ctx), carried_o),
+               grads=(grads, g_o), d_x=(host(d_emb).reshape(bs, s, d), dx_o))
+    check(out, "TitansMlp", tol=2e-4, has_eta=True)
+    assert cache.dgd_delta_norm(s, d, 1, 1) == 0.0
+    with pytest.raises(ValueError):
+        GL.gpu_memory_forward(lp, GL.LevelConfig("titans", nh, hd, memory_layers=2, checkpoint_interval=4), emb, ctx, s,
+                              d, bs)
+
+
+@pytest.mark.parametrize("rule", ["moneta", "yaad"])
+@pytest.mark.parametrize("s,d,dh", [(7, 16, 24), (12, 8, 32)])
+def test_mlp_memories_at_model_width(rule, s, d, dh):
+    """MONETA / YAAD levels (gpu_forward.rs:1729-1852, gpu_backward.rs:1635-1733): one sequence, context_m = [W1|W2]."""
+    cfg = GL.LevelConfig(rule, 1, d, d_hidden=dh, lp_p=3.0, sign_sharpness=8.0, lambda_2=0.02, delta=0.5,
+                         lambda_local=0.05, theta_ceil=0.4)
+    r = np.random.default_rng(50 + s)
+    p = params(d, 51)
+    x = (r.standard_normal((1, s, d)) / np.sqrt(d)).astype(np.float32)
+    w1 = (r.standard_normal((dh, d)) / np.sqrt(d)).astype(np.float32)
+    w2 = (r.standard_normal((d, dh)) / np.sqrt(dh)).astype(np.float32)
+    dy = r.standard_normal((1, s, d)).astype(np.float32)
+    y_o, c_o, (w1_f, w2_f) = ML.level_forward(p, cfg, x, (w1, w2))
+    g_o, dx_o = ML.level_backward(p, cfg, c_o, dy, x)
+    lp = MemoryLevelParams(*[dev(p[n]) for n in NAMES])
+    ctx = dev(np.concatenate([w1.ravel(), w2.ravel()]))
+    emb = dev(x.reshape(s, d))
+    y, cache = GL.gpu_memory_forward(lp, cfg, emb, ctx, s, d, 1)
+    grads = GL.LevelGrads.zeros(d)
+    d_emb = GL.gpu_memory_backward(lp, cfg, cache, dev(dy.reshape(s, d)), emb, grads, s, d, 1)
+    torch.cuda.synchronize()
+    assert cache.kind == "Mlp" and (cache.w1_boundary is not None) == (rule == "yaad")
+    assert_close("y", host(y), y_o[0], 2e-4)
+    assert_close("w1_states", host(cache.w1_states).reshape(c_o["w1_states"].shape), c_o["w1_states"], 2e-4)
+    assert_close("w2_states", host(cache.w2_states).reshape(c_o["w2_states"].shape), c_o["w2_states"], 2e-4)
+    got = host(ctx)
+    assert_close("carried W1", got[:dh * d].reshape(dh, d), w1_f, 2e-4)
+    assert_close("carried W2", got[dh * d:].reshape(d, dh), w2_f, 2e-4)
+    for n in ("w_k", "w_v", "w_q"):
+        assert_close("d_" + n, host(getattr(grads, f"d_{n}_mem")), g_o[n], 5e-4)
+    for n in ("alpha", "theta"):
+        assert_close("d_w_" + n, host(getattr(grads, "d_w_" + n)), g_o["w_" + n], 5e-4)
+        assert_close("d_b_" + n, host(getattr(grads, "d_b_" + n)), g_o["b_" + n], 5e-4)
+    assert_close("d_embedded", host(d_emb), dx_o[0], 5e-4)
+    with pytest.raises(ValueError):
+        GL.gpu_memory_forward(lp, cfg, dev(np.zeros((2 * s, d), np.float32)), ctx, s, d, 2)
+    with pytest.raises(ValueError):
+        GL.gpu_memory_forward(lp, cfg, emb, dev(np.zeros(10, np.float32)), s, d, 1)
+
+
+def test_swiglu_level():
+    """The stateless MLP level (gpu_forward.rs:1705-1727, gpu_backward.rs:1736-1760): no memory, direct gradients."""
+    bs, s, d, inter = 2, 9, 16, 40
+    r = np.random.default_rng(70)
+    f = np.float32
+    p = dict(gate_proj=(r.standard_normal((inter, d)) / np.sqrt(d)).astype(f),
+             up_proj=(r.standard_normal((inter, d)) / np.sqrt(d)).astype(f),
+             down_proj=(r.standard_normal((d, inter)) / np.sqrt(inter)).astype(f))
+    x, dy = r.standard_normal((bs, s, d)).astype(f), r.standard_normal((bs, s, d)).astype(f)
+    cfg = GL.LevelConfig("swiglu", 2, 8, intermediate_size=inter)
+    y_o, c_o, _ = ML.level_forward(p, cfg, x, None)
+    g_o, dx_o = ML.level_backward(p, cfg, c_o, dy, x)
+    lp = GL.SwiGluLevelParams(dev(p["gate_proj"]), dev(p["up_proj"]), dev(p["down_proj"]))
+    ctx = dev(np.full((4, 64), 7.0, f))
+    emb = dev(x.reshape(bs * s, d))
+    y, cache = GL.gpu_memory_forward(lp, cfg, emb, ctx, s, d, bs)
+    grads = GL.LevelGrads.zeros(d, intermediate=inter)
+    d_emb = GL.gpu_memory_backward(lp, cfg, cache, dev(dy.reshape(bs * s, d)), emb, grads, s, d, bs)
+    torch.cuda.synchronize()
+    assert cache.kind == "SwiGlu" and cache.alpha_stats(0.0) is None
+    assert np.all(host(ctx) == 7.0), "a SwiGLU level leaves context_m alone"
+    assert_close("y", host(y).reshape(bs, s, d), y_o, 1e-4)
+    assert_close("d_x", host(d_emb).reshape(bs, s, d), dx_o, 1e-4)
+    for n in ("gate_proj", "up_proj", "down_proj"):
+        assert_close("d_" + n, host(getattr(grads, "d_" + n)), g_o[n], 1e-4)
