@@ -110,6 +110,8 @@ class GpuMemoryCache:
         (gpu_forward.rs:328-437): 0 for several heads, for Hebbian, and without tokens."""
         if num_heads > 1 or s == 0 or self.kind.startswith("Hebbian") or self.kind in ("TitansMlp", "Mlp", "SwiGlu"):
             return 0.0
+        if self.proxy:   # only final states are kept (the TNT inner caches of a proxy level)
+            return 0.0
         assert batch_size <= 1, "dgd_delta_norm reads batch slot 0 only"
         if self.kind.endswith("Chunkwise"):
             if not self.num_chunks:
@@ -122,8 +124,8 @@ class GpuMemoryCache:
         else:
             slot = s - 1
         out = torch.zeros(1, device=self.k_mem.device)
-        D.call("dgd_delta_norm_cuda", self.m_states[0, slot].contiguous(), self.k_mem[s - 1].contiguous(),
-               self.v_mem[s - 1].contiguous(), out, d)
+        D.call("dgd_delta_norm_cuda", self.m_states[0, slot].contiguous(), self.k_mem.reshape(-1, d)[s - 1].contiguous(),
+               self.v_mem.reshape(-1, d)[s - 1].contiguous(), out, d)
         return float(out.item())
 
     def alpha_stats(self, alpha_floor):

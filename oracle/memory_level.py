@@ -278,3 +278,144 @@ def projection_grads(p, x, c, d_k, d_v, d_q, d_alpha, d_theta, d_eta):
     else:
         g["w_eta"], g["b_eta"] = z2, z1
     return g, d_x.reshape(bs, s, d)
+
+
+# ── TNT: shards of local chunks around a global memory (gpu_forward.rs:1878-2293, gpu_backward.rs:1201-1632) ──
+GLOBAL_RETENTION = 0.95
+
+
+def _pad(t, n, padded):
+    """[nh, n, ...] -> [nh, padded, ...], zeros behind."""
+    out = np.zeros((t.shape[0], padded) + t.shape[2:], t.dtype)
+    out[:, :n] = t
+    return out
+
+
+def tnt_forward(p, cfg, x, m0, cg, cl, gates=None):
+    """x [s, d], m0 [nh, hd, hd] (global memory per head) -> y [s, d], cache (list of per-shard dicts), final
+    global memory.  gates: per-shard list of (alpha, theta, eta) to use instead of the computed ones."""
+    s, d = x.shape
+    nh, hd = cfg.num_heads, cfg.head_dim
+    dt = x.dtype
+    titans = cfg.memory_rule == "titans"
+    m_glob = m0.copy()
+    y_full = np.zeros((s, d), dt)
+    shards = []
+    for si, t0 in enumerate(range(0, s, cg)):
+        t1 = min(t0 + cg, s)
+        n = t1 - t0
+        n_batch = -(-n // cl)
+        padded = n_batch * cl
+        xs = x[t0:t1]
+        k, k_norms = l2_normalize(xs @ p["w_k"].T)
+        q, q_norms = l2_normalize(xs @ p["w_q"].T)
+        v = xs @ p["w_v"].T
+        alpha = gate(k, v, p["w_alpha"], p["b_alpha"], 0)
+        theta = gate(k, v, p["w_theta"], p["b_theta"], 1)
+        ca, ct = _clamped(cfg)
+        if ca:
+            alpha = np.clip(alpha, cfg.alpha_floor, cfg.alpha_ceil)
+        if ct:
+            theta = np.clip(theta, cfg.theta_floor, cfg.theta_ceil)
+        eta = gate(k, v, p["w_eta"], p["b_eta"], 0) if titans else None
+        if gates is not None:
+            alpha, theta, eta = gates[si]
+        kh, vh, qh = (_pad(to_heads(t, 1, n, nh, hd), n, padded) for t in (k, v, q))
+        ah, th = (_pad(gates_to_heads(g, 1, n, nh), n, padded) for g in (alpha, theta))
+        eh = _pad(gates_to_heads(eta, 1, n, nh), n, padded) if titans else None
+        y_local = np.zeros((nh, padded, hd), dt)
+        ms, ss = [], []
+        z = np.zeros((hd, hd), dt)
+        for h in range(nh):
+            for b in range(n_batch):
+                sl = slice(b * cl, (b + 1) * cl)
+                if titans:
+                    y, m, sst = orc.titans_forward(kh[h, sl], vh[h, sl], qh[h, sl], ah[h, sl], th[h, sl], eh[h, sl],
+                                                   m_glob[h], z, cfg.error_clip, cfg.m_norm_max)
+                    ss.append(sst)
+                else:
+                    y, m = orc.delta_forward(kh[h, sl], vh[h, sl], qh[h, sl], ah[h, sl], th[h, sl], m_glob[h],
+                                             cfg.error_clip, cfg.m_norm_max)
+                y_local[h, sl] = y
+                ms.append(m)
+        y_full[t0:t1] = from_heads(y_local, 1, padded, nh, hd)[:n]
+        mean = y_local[:, :n].sum(1) / dt.type(n)          # [nh, hd]: key and value summary alike
+        m_glob = dt.type(GLOBAL_RETENTION) * m_glob + np.einsum("hi,hj->hij", mean, mean)
+        m_glob = frobenius_clamp(m_glob, cfg.m_norm_max)
+        shards.append(dict(t0=t0, n=n, n_batch=n_batch, padded=padded, k=k, v=v, q=q, k_norms=k_norms, q_norms=q_norms,
+                           alpha=alpha, theta=theta, eta=eta, kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh,
+                           m_states=np.stack(ms), s_states=np.stack(ss) if titans else None, summary=mean))
+    return y_full, shards, m_glob
+
+
+def tnt_backward(p, cfg, shards, d_y, x, cl, first_retained=0):
+    """-> (grads, d_x).  The rule's backward returns the gradient of the initial memory summed over the chains of
+    a call; as in the reference (gpu_backward.rs:1408-1418) the whole sum is added to head 0's global memory
+    gradient — the gradient itself for one head."""
+    s, d = x.shape
+    nh, hd = cfg.num_heads, cfg.head_dim
+    dt = x.dtype
+    titans = cfg.memory_rule == "titans"
+    d_k_tot, d_v_tot, d_q_tot = np.zeros((s, d), dt), np.zeros((s, d), dt), np.zeros((s, d), dt)
+    g = {n: np.zeros(2 * d, dt) for n in ("w_alpha", "w_theta", "w_eta")}
+    g.update({n: np.zeros(1, dt) for n in ("b_alpha", "b_theta", "b_eta")})
+    d_m_carry = np.zeros((nh, hd, hd), dt)
+    for si in reversed(range(len(shards))):
+        c = shards[si]
+        n, n_batch, padded, t0 = c["n"], c["n_batch"], c["padded"], c["t0"]
+        mean = c["summary"]
+        d_m_old = dt.type(GLOBAL_RETENTION) * d_m_carry
+        d_k_sum = np.einsum("hij,hi->hj", d_m_carry, mean)      # M_new = a M + v_sum k_sum^T
+        d_v_sum = np.einsum("hij,hj->hi", d_m_carry, mean)
+        if si < first_retained:
+            d_m_carry = d_m_old
+            continue
+        d_local = np.repeat(((d_k_sum + d_v_sum) / dt.type(n))[:, None, :], n, axis=1)   # [nh, n, hd]
+        d_y_comb = d_y[t0:t0 + n] + from_heads(d_local, 1, n, nh, hd)
+        dyh = _pad(to_heads(d_y_comb, 1, n, nh, hd), n, padded)
+        dk, dv, dq = (np.zeros((nh, padded, hd), dt) for _ in range(3))
+        da, dth, de = (np.zeros((nh, padded), dt) for _ in range(3))
+        d_m_sum = np.zeros((hd, hd), dt)
+        for h in range(nh):
+            for b in range(n_batch):
+                sl = slice(b * cl, (b + 1) * cl)
+                i = h * n_batch + b
+                m_i = c["m_states"][i]
+                s_i = c["s_states"][i] if titans else None
+                if cfg.proxy:   # a proxy level keeps the final states only; they stand in for every state
+                    m_i = np.ascontiguousarray(np.broadcast_to(m_i[-1], m_i.shape))
+                    s_i = np.ascontiguousarray(np.broadcast_to(s_i[-1], s_i.shape)) if titans else None
+                if titans:
+                    gi = orc.titans_backward(c["kh"][h, sl], c["vh"][h, sl], c["qh"][h, sl], c["ah"][h, sl], c["th"][h, sl],
+                                             c["eh"][h, sl], m_i, s_i, dyh[h, sl], cfg.error_clip)
+                    de[h, sl] = gi["d_eta"]
+                else:
+                    gi = orc.delta_backward(c["kh"][h, sl], c["vh"][h, sl], c["qh"][h, sl], c["ah"][h, sl], c["th"][h, sl],
+                                            m_i, dyh[h, sl], cfg.error_clip)
+                dk[h, sl], dv[h, sl], dq[h, sl] = gi["d_k"], gi["d_v"], gi["d_q"]
+                da[h, sl], dth[h, sl] = gi["d_alpha"], gi["d_theta"]
+                d_m_sum += gi["d_m"]
+        if not cfg.proxy:
+            d_m_old[0] += d_m_sum
+        ca, ct = _clamped(cfg)
+        if ca:
+            da = np.where((c["ah"] <= cfg.alpha_floor) | (c["ah"] >= cfg.alpha_ceil), 0.0, da)
+        if ct:
+            dth = np.where((c["th"] <= cfg.theta_floor) | (c["th"] >= cfg.theta_ceil), 0.0, dth)
+        dk_dm, dv_dm, dq_dm = (from_heads(t, 1, padded, nh, hd)[:n] for t in (dk, dv, dq))
+        da_dm, dth_dm, de_dm = (t.sum(0)[:n] for t in (da, dth, de))
+        d_k_tot[t0:t0 + n] += l2_normalize_backward(dk_dm, c["k"], c["k_norms"])
+        d_v_tot[t0:t0 + n] += dv_dm
+        d_q_tot[t0:t0 + n] += l2_normalize_backward(dq_dm, c["q"], c["q_norms"])
+        kv = np.concatenate([c["k"], c["v"]], axis=1)
+        pre = da_dm * c["alpha"] * (1.0 - c["alpha"])
+        g["w_alpha"] += pre @ kv; g["b_alpha"] += pre.sum()
+        pre = dth_dm * (1.0 - np.exp(-c["theta"]))
+        g["w_theta"] += pre @ kv; g["b_theta"] += pre.sum()
+        if titans:
+            pre = de_dm * c["eta"] * (1.0 - c["eta"])
+            g["w_eta"] += pre @ kv; g["b_eta"] += pre.sum()
+        d_m_carry = d_m_old
+    g["w_k"], g["w_v"], g["w_q"] = d_k_tot.T @ x, d_v_tot.T @ x, d_q_tot.T @ x
+    d_x = d_k_tot @ p["w_k"] + d_v_tot @ p["w_v"] + d_q_tot @ p["w_q"]
+    return g, d_x

@@ -161,3 +161,62 @@ def test_carried_memory_is_clamped():
     _, cache, carried = ML.level_forward(p, cfg, x, m0)
     assert np.sqrt((cache["m_states"][0, -1] ** 2).sum()) > 0.5
     assert abs(np.sqrt((carried[0] ** 2).sum()) - 0.5) < 1e-12
+
+
+@pytest.mark.parametrize("rule", ["delta", "titans"])
+def test_tnt_backward_is_the_gradient_of_the_forward(rule):
+    """TNT level (shards of local chunks around a global memory), one head, float64: central differences of
+    L = sum(y * dY) + sum(M_final * dM) are not needed — the reference's backward starts from a zero gradient of the
+    final global memory, so L = sum(y * dY).  Ragged last shard and a padded last local chunk included."""
+    nh, hd, s, cg, cl = 1, 4, 11, 4, 3        # shards of 4, 4, 3 tokens; local chunks of 3 (+ padding)
+    d = nh * hd
+    cfg = cfg_of(rule, nh, hd)
+    r = np.random.default_rng(21)
+    p = params(d, 22)
+    x = r.standard_normal((s, d)) / np.sqrt(d)
+    m0 = 0.3 * r.standard_normal((nh, hd, hd))
+    dy = r.standard_normal((s, d))
+    y, shards, m_fin = ML.tnt_forward(p, cfg, x, m0, cg, cl)
+    assert len(shards) == 3 and shards[0]["padded"] == 6 and shards[2]["padded"] == 3
+    grads, d_x = ML.tnt_backward(p, cfg, shards, dy, x, cl)
+    gates = [(c["alpha"], c["theta"], c["eta"]) for c in shards]
+    eps = 1e-6
+
+    def loss(pp, xx, frozen):
+        return float((ML.tnt_forward(pp, cfg, xx, m0, cg, cl, gates if frozen else None)[0] * dy).sum())
+
+    def fd_param(name, idx, frozen):
+        lo, hi = {**p}, {**p}
+        lo[name], hi[name] = p[name].copy(), p[name].copy()
+        lo[name][idx] -= eps
+        hi[name][idx] += eps
+        return (loss(hi, x, frozen) - loss(lo, x, frozen)) / (2 * eps)
+
+    names = ["w_alpha", "b_alpha", "w_theta", "b_theta"] + (["w_eta", "b_eta"] if rule == "titans" else [])
+    for name in names:
+        for idx in ([(0,)] if name[0] == "b" else [(1,), (d + 2,)]):
+            want = fd_param(name, idx, False)
+            assert abs(grads[name][idx] - want) <= 1e-6 + 1e-5 * abs(want), (name, idx, grads[name][idx], want)
+    for name in ("w_k", "w_v", "w_q"):
+        for idx in [(0, 0), (3, 1)]:
+            want = fd_param(name, idx, True)
+            assert abs(grads[name][idx] - want) <= 1e-6 + 1e-5 * abs(want), (name, idx, grads[name][idx], want)
+    for idx in [(0, 0), (5, 2), (s - 1, d - 1)]:
+        lo, hi = x.copy(), x.copy()
+        lo[idx] -= eps
+        hi[idx] += eps
+        want = (loss(p, hi, True) - loss(p, lo, True)) / (2 * eps)
+        assert abs(d_x[idx] - want) <= 1e-6 + 1e-5 * abs(want), (idx, d_x[idx], want)
+
+
+def test_tnt_with_one_shard_and_one_chunk_is_the_plain_level():
+    nh, hd, s = 2, 4, 6
+    d = nh * hd
+    cfg = cfg_of("titans", nh, hd)
+    r = np.random.default_rng(23)
+    p = params(d, 24)
+    x = r.standard_normal((s, d)) / np.sqrt(d)
+    m0 = 0.3 * r.standard_normal((nh, hd, hd))
+    y_t, _, _ = ML.tnt_forward(p, cfg, x, m0, s, s)
+    y_l, _, _ = ML.level_forward(p, cfg, x[None], m0)
+    assert np.allclose(y_t, y_l[0], rtol=1e-12, atol=1e-14)
