@@ -123,7 +123,8 @@ void titans_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, co
                                       int t_start, int t_end, int d, int batch_size, int seq_len,
                                       float error_clip);
 
-/* ── Hebbian rule: M <- (1 - alpha) M + v k^T (d in {8, 16, 32, 64, 128}) ────────── */
+/* ── Hebbian rule: M <- (1 - alpha) M + v k^T.  d = 8, 16, 32, 64, 128 on tiled kernels, every other d from 1 to
+ * 3840 on general ones (the reference runs these at d = 2048, core/tests/test_cuda_large_d.rs:353) ─────────── */
 /* core/src/cuda_ffi.rs:186 */
 void hebbian_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
                               const float *alpha, const float *m_initial,

@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "hebbian_generic.h"
 #include "quad_rows.h"
 #include "rule_common.h"
 #include "runtime.h"
@@ -337,6 +338,7 @@ bool launch_fwd_chunks(HebFwdArgs a, int batch);
 
 template <int STORE>
 bool launch_fwd(HebFwdArgs a, int d, int batch) {
+    if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) return false;
     if (STORE == HEB_TRAJ && d == 64 && a.seq_len > 2 * kHC && a.chunks == 0 && launch_fwd_chunks(a, batch)) return true;
     const int groups = a.chunks ? batch * a.chunks : batch;
     a.rows = rows_per_workgroup(d, groups);
@@ -744,10 +746,6 @@ bool launch_bwd(HebBwdArgs a, int d, int batch) {
     return true;
 }
 
-void bad_d(const char *fn, int d) {
-    fail("%s: d=%d is not supported by the gfx950 kernels (d in {8, 16, 32, 64, 128}).", fn, d);
-}
-
 }  // namespace
 }  // namespace nlh
 
@@ -761,7 +759,10 @@ void hebbian_forward_f32_cuda(const float *k_mem, const float *v_mem, const floa
     if (!check_dims("hebbian_forward_f32_cuda", seq_len, d, batch_size) || batch_size == 0) return;
     const HebFwdArgs a{k_mem, v_mem, q_mem, alpha, m_initial, m_states, y, seq_len, input_stride, m_stride, 1, 0,
                        (long long)seq_len + 1, 0};
-    if (!launch_fwd<HEB_TRAJ>(a, d, batch_size)) bad_d("hebbian_forward_f32_cuda", d);
+    if (launch_fwd<HEB_TRAJ>(a, d, batch_size)) return;
+    if (hebbian_generic_check("hebbian_forward_f32_cuda", d))
+        hebbian_forward_generic(k_mem, v_mem, q_mem, alpha, m_initial, m_states, y, seq_len, d, batch_size, input_stride,
+                                m_stride, 0, (long long)seq_len + 1);
 }
 
 void hebbian_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
@@ -774,7 +775,10 @@ void hebbian_forward_ckpt_f32_cuda(const float *k_mem, const float *v_mem, const
     }
     const HebFwdArgs a{k_mem, v_mem, q_mem, alpha, m_initial, m_states, y, seq_len, seq_len, d * d,
                        checkpoint_interval, 0, (long long)n_ckpt_count(seq_len, checkpoint_interval), 0};
-    if (!launch_fwd<HEB_CKPT>(a, d, 1)) bad_d("hebbian_forward_ckpt_f32_cuda", d);
+    if (launch_fwd<HEB_CKPT>(a, d, 1)) return;
+    if (hebbian_generic_check("hebbian_forward_ckpt_f32_cuda", d))
+        hebbian_forward_generic(k_mem, v_mem, q_mem, alpha, m_initial, m_states, y, seq_len, d, 1, seq_len, d * d,
+                                checkpoint_interval, (long long)n_ckpt_count(seq_len, checkpoint_interval));
 }
 
 void hebbian_backward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem, const float *alpha,
@@ -783,7 +787,10 @@ void hebbian_backward_f32_cuda(const float *k_mem, const float *v_mem, const flo
     if (!check_dims("hebbian_backward_f32_cuda", seq_len, d, 1)) return;
     const HebBwdArgs a{k_mem, v_mem, q_mem, alpha, m_states, d_y, nullptr, d_k_mem, d_v_mem, d_q_mem, d_alpha,
                        d_m_initial, nullptr, nullptr, nullptr, seq_len, 0, seq_len, 0};
-    if (!launch_bwd(a, d, 1)) bad_d("hebbian_backward_f32_cuda", d);
+    if (launch_bwd(a, d, 1)) return;
+    if (hebbian_generic_check("hebbian_backward_f32_cuda", d))
+        hebbian_backward_generic(k_mem, v_mem, q_mem, alpha, m_states, d_y, nullptr, d_k_mem, d_v_mem, d_q_mem, d_alpha,
+                                 d_m_initial, seq_len, 0, seq_len, d, 1);
 }
 
 void hebbian_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
@@ -798,7 +805,10 @@ void hebbian_backward_segment_f32_cuda(const float *k_mem, const float *v_mem, c
     }
     const HebBwdArgs a{k_mem, v_mem, q_mem, alpha, m_states, d_y, d_m_seed, d_k_mem, d_v_mem, d_q_mem, d_alpha,
                        d_m_out, nullptr, nullptr, nullptr, seq_len, t_start, t_end, 0};
-    if (!launch_bwd(a, d, batch_size)) bad_d("hebbian_backward_segment_f32_cuda", d);
+    if (launch_bwd(a, d, batch_size)) return;
+    if (hebbian_generic_check("hebbian_backward_segment_f32_cuda", d))
+        hebbian_backward_generic(k_mem, v_mem, q_mem, alpha, m_states, d_y, d_m_seed, d_k_mem, d_v_mem, d_q_mem, d_alpha,
+                                 d_m_out, seq_len, t_start, t_end, d, batch_size);
 }
 
 }  // extern "C"
