@@ -13,6 +13,7 @@
 
 #include "../../include/nl_hecate_ffi.h"
 #include "lane_ops.h"
+#include "optim_steps.h"
 #include "runtime.h"
 
 // ── Conductor (core/src/conductor.rs:36-155) ────────────────────────────────
@@ -257,12 +258,21 @@ unsigned nlh_adamw_step(nlh_adamw *o, const int *active_levels, float lr, float 
     std::vector<float *> w, g, m, v;
     std::vector<int> n;
     std::vector<float> bc1, bc2;
-    if (max_grad_norm > 0.0f) {
+    const bool clip = max_grad_norm > 0.0f;
+    if (clip) {
+        // the clip factor stays on the device; the update below applies it to the gradients it reads (and writes
+        // them back scaled), so only the tensors that take no update this step need a scaling pass of their own
         if (!norm_scale) { fail("nlh_adamw_step: norm_scale must be a device buffer of 2 floats when clipping."); return 1; }
         for (auto &t : o->tensors) { g.push_back(t.g); n.push_back(t.n); }
-        unsigned rc = grad_norm_clip_multi_rocm(g.data(), n.data(), (int)nt, max_grad_norm, norm_scale,
-                                                norm_scale + 1);
+        unsigned rc = nlh::grad_norm_scale_multi(g.data(), n.data(), (int)nt, max_grad_norm, norm_scale, norm_scale + 1);
         if (rc) return rc;
+        g.clear(); n.clear();
+        for (auto &t : o->tensors)
+            if (t.group >= 0 && (!active_levels || !active_levels[t.group])) { g.push_back(t.g); n.push_back(t.n); }
+        if (!g.empty()) {
+            rc = nlh::grad_scale_multi(g.data(), n.data(), (int)g.size(), norm_scale + 1);
+            if (rc) return rc;
+        }
         g.clear(); n.clear();
     }
     o->step += 1;
@@ -282,9 +292,9 @@ unsigned nlh_adamw_step(nlh_adamw *o, const int *active_levels, float lr, float 
         bc1.push_back(t.group < 0 ? sbc1 : lbc1[t.group]);
         bc2.push_back(t.group < 0 ? sbc2 : lbc2[t.group]);
     }
-    unsigned rc = adamw_update_multi_rocm(w.data(), (const float *const *)g.data(), m.data(), v.data(),
-                                          n.data(), bc1.data(), bc2.data(), (int)w.size(), lr, o->beta1,
-                                          o->beta2, o->eps, o->weight_decay);
+    unsigned rc = nlh::adamw_update_multi_scaled(w.data(), (const float *const *)g.data(), m.data(), v.data(),
+                                                 n.data(), bc1.data(), bc2.data(), (int)w.size(), lr, o->beta1,
+                                                 o->beta2, o->eps, o->weight_decay, clip ? norm_scale + 1 : nullptr);
     if (rc) return rc;
     for (auto &t : o->tensors)
         if (t.clamp && (t.group < 0 || (active_levels && active_levels[t.group])))

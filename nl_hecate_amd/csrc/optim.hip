@@ -12,6 +12,7 @@
 
 #include "../../include/nl_hecate_ffi.h"
 #include "lane_ops.h"
+#include "optim_steps.h"
 #include "runtime.h"
 
 namespace nlh {
@@ -31,15 +32,27 @@ __device__ __forceinline__ void adamw_one(float &w, float g, float &m, float &v,
 
 struct AdamwHyper { float lr, b1, b2, eps, wd; };
 
+// SCALE: the gradient is first multiplied by *scale_ptr when that is below 1 (the clip factor, still on the
+// device) and written back, which is what a separate in-place scaling pass before the update would leave.
+template <bool SCALE>
 __device__ __forceinline__ void adamw_span(float *w, const float *g, float *m, float *v, int n,
-                                           int start, int stride, const AdamwHyper &h, float bc1, float bc2) {
+                                           int start, int stride, const AdamwHyper &h, float bc1, float bc2,
+                                           const float *scale_ptr = nullptr) {
     const bool vec = ((((uintptr_t)w) | ((uintptr_t)g) | ((uintptr_t)m) | ((uintptr_t)v)) & 15) == 0;
+    float sc = 1.0f;
+    if (SCALE) sc = *scale_ptr;
+    const bool scaled = SCALE && sc < 1.0f;
+    float *gw = const_cast<float *>(g);
     if (vec) {
         const int n4 = n >> 2;
         for (int j = start; j < n4; j += stride) {
             float4 W = reinterpret_cast<float4 *>(w)[j], M = reinterpret_cast<float4 *>(m)[j];
             float4 V = reinterpret_cast<float4 *>(v)[j];
-            const float4 G = reinterpret_cast<const float4 *>(g)[j];
+            float4 G = reinterpret_cast<const float4 *>(g)[j];
+            if (scaled) {
+                G.x *= sc; G.y *= sc; G.z *= sc; G.w *= sc;
+                reinterpret_cast<float4 *>(gw)[j] = G;
+            }
             adamw_one(W.x, G.x, M.x, V.x, h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
             adamw_one(W.y, G.y, M.y, V.y, h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
             adamw_one(W.z, G.z, M.z, V.z, h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
@@ -48,17 +61,23 @@ __device__ __forceinline__ void adamw_span(float *w, const float *g, float *m, f
             reinterpret_cast<float4 *>(m)[j] = M;
             reinterpret_cast<float4 *>(v)[j] = V;
         }
-        for (int i = (n4 << 2) + start; i < n; i += stride)
-            adamw_one(w[i], g[i], m[i], v[i], h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
+        for (int i = (n4 << 2) + start; i < n; i += stride) {
+            float gi = g[i];
+            if (scaled) { gi *= sc; gw[i] = gi; }
+            adamw_one(w[i], gi, m[i], v[i], h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
+        }
     } else {
-        for (int i = start; i < n; i += stride)
-            adamw_one(w[i], g[i], m[i], v[i], h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
+        for (int i = start; i < n; i += stride) {
+            float gi = g[i];
+            if (scaled) { gi *= sc; gw[i] = gi; }
+            adamw_one(w[i], gi, m[i], v[i], h.lr, h.b1, h.b2, h.eps, bc1, bc2, h.wd);
+        }
     }
 }
 
 __global__ void adamw_kernel(float *w, const float *g, float *m, float *v, int n, AdamwHyper h,
                              float bc1, float bc2) {
-    adamw_span(w, g, m, v, n, blockIdx.x * blockDim.x + threadIdx.x, gridDim.x * blockDim.x, h, bc1, bc2);
+    adamw_span<false>(w, g, m, v, n, blockIdx.x * blockDim.x + threadIdx.x, gridDim.x * blockDim.x, h, bc1, bc2);
 }
 
 // Up to kMaxTensors tensors per launch, passed by value in the kernel argument.
@@ -74,13 +93,14 @@ struct AdamwBatch {
     int count;
 };
 
-__global__ void adamw_multi_kernel(AdamwBatch b, AdamwHyper h) {
+template <bool SCALE>
+__global__ void adamw_multi_kernel(AdamwBatch b, AdamwHyper h, const float *scale_ptr) {
     int t = 0;
     while (t + 1 < b.count && (int)blockIdx.x >= b.blk_begin[t + 1]) t++;
     const int nblk = b.blk_begin[t + 1] - b.blk_begin[t];
     const int lb = blockIdx.x - b.blk_begin[t];
-    adamw_span(b.w[t], b.g[t], b.m[t], b.v[t], b.n[t], lb * blockDim.x + threadIdx.x, nblk * blockDim.x, h,
-               b.bc1[t], b.bc2[t]);
+    adamw_span<SCALE>(b.w[t], b.g[t], b.m[t], b.v[t], b.n[t], lb * blockDim.x + threadIdx.x, nblk * blockDim.x, h,
+                      b.bc1[t], b.bc2[t], scale_ptr);
 }
 
 // One partial per 256 elements (the reference's layout, core/kernels/adamw.cu:86-127):
@@ -157,9 +177,13 @@ __global__ __launch_bounds__(kClipThreads) void reduce_partials_clip_kernel(cons
 struct PtrBatch {
     float *p[kMaxTensors];
     int n[kMaxTensors];
-    int blk_begin[kMaxTensors + 1];  // in units of 256-element blocks (norm) or workgroups (scale)
+    int blk_begin[kMaxTensors + 1];  // in units of kNormBlock-element blocks (norm) or workgroups (scale)
     int count;
 };
+
+// elements per partial sum of the multi-tensor norm: eight 16-byte loads per lane in flight before the one
+// reduction (one load per reduction left the pass at 1.4 TB/s)
+constexpr int kNormBlock = 2048;
 
 __global__ void norm_sq_multi_kernel(PtrBatch b, float *__restrict__ partial) {
     const int lane = threadIdx.x & 63;
@@ -170,13 +194,21 @@ __global__ void norm_sq_multi_kernel(PtrBatch b, float *__restrict__ partial) {
         int t = 0;
         while (t + 1 < b.count && blk >= b.blk_begin[t + 1]) t++;
         const float *a = b.p[t];
-        const int n = b.n[t], base = (blk - b.blk_begin[t]) * 256;
+        const int n = b.n[t], base = (blk - b.blk_begin[t]) * kNormBlock;
         float s = 0.f;
-        if (((((uintptr_t)a) & 15) == 0) && base + 256 <= n) {
-            const float4 x = reinterpret_cast<const float4 *>(a + base)[lane];
-            s = x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+        if (((((uintptr_t)a) & 15) == 0) && base + kNormBlock <= n) {
+            float4 x[kNormBlock / 256];
+#pragma unroll
+            for (int r = 0; r < kNormBlock / 256; r++) x[r] = reinterpret_cast<const float4 *>(a + base + 256 * r)[lane];
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int r = 0; r < kNormBlock / 256; r += 2) {
+                s0 += x[r].x * x[r].x + x[r].y * x[r].y + x[r].z * x[r].z + x[r].w * x[r].w;
+                s1 += x[r + 1].x * x[r + 1].x + x[r + 1].y * x[r + 1].y + x[r + 1].z * x[r + 1].z + x[r + 1].w * x[r + 1].w;
+            }
+            s = s0 + s1;
         } else {
-            for (int i = base + lane; i < min(base + 256, n); i += 64) s += a[i] * a[i];
+            for (int i = base + lane; i < min(base + kNormBlock, n); i += 64) s += a[i] * a[i];
         }
         s = wave_allreduce(s);
         if (lane == 0) partial[blk] = s;
@@ -254,6 +286,16 @@ unsigned adamw_update_cuda(float *w, const float *g, float *m, float *v, int n, 
 unsigned adamw_update_multi_rocm(float *const *w, const float *const *g, float *const *m, float *const *v,
                                  const int *n, const float *bc1_inv, const float *bc2_inv, int count,
                                  float lr, float beta1, float beta2, float eps, float weight_decay) {
+    return nlh::adamw_update_multi_scaled(w, g, m, v, n, bc1_inv, bc2_inv, count, lr, beta1, beta2, eps, weight_decay,
+                                          nullptr);
+}
+
+}  // extern "C"
+
+unsigned nlh::adamw_update_multi_scaled(float *const *w, const float *const *g, float *const *m, float *const *v,
+                                        const int *n, const float *bc1_inv, const float *bc2_inv, int count, float lr,
+                                        float beta1, float beta2, float eps, float weight_decay,
+                                        const float *scale_ptr) {
     const AdamwHyper h{lr, beta1, beta2, eps, weight_decay};
     // a batch is the next kMaxTensors input slots (empty ones skipped), so no tensor is seen twice
     for (int first = 0; first < count; first += kMaxTensors) {
@@ -271,12 +313,17 @@ unsigned adamw_update_multi_rocm(float *const *w, const float *const *g, float *
         }
         if (b.count == 0) continue;
         b.blk_begin[b.count] = blocks;
-        hipLaunchKernelGGL(adamw_multi_kernel, dim3(blocks), dim3(kOptThreads), 0, stream(), b, h);
+        if (scale_ptr)
+            hipLaunchKernelGGL(adamw_multi_kernel<true>, dim3(blocks), dim3(kOptThreads), 0, stream(), b, h, scale_ptr);
+        else
+            hipLaunchKernelGGL(adamw_multi_kernel<false>, dim3(blocks), dim3(kOptThreads), 0, stream(), b, h, scale_ptr);
         unsigned rc = launch_status("adamw_update_multi_rocm");
         if (rc) return rc;
     }
     return 0;
 }
+
+extern "C" {
 
 unsigned grad_norm_sq_cuda(const float *g, float *partial_sums, int n, int *out_num_blocks) {
     const int nblk = (n + 255) / 256;
@@ -320,10 +367,20 @@ unsigned grad_scale_conditional_cuda(float *g, const float *scale_ptr, int n) {
 
 unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, float max_grad_norm,
                                    float *out_norm, float *out_scale) {
+    unsigned rc = nlh::grad_norm_scale_multi(g, n, count, max_grad_norm, out_norm, out_scale);
+    if (rc) return rc;
+    return nlh::grad_scale_multi(g, n, count, out_scale);
+}
+
+}  // extern "C"
+
+// norm and clip factor of a set of tensors, left on the device: {norm} -> out_norm, {min(1, max / norm)} -> out_scale
+unsigned nlh::grad_norm_scale_multi(float *const *g, const int *n, int count, float max_grad_norm, float *out_norm,
+                                    float *out_scale) {
     const ErrorScope es;
     // pass 1: partial sums of every tensor into one scratch array
     long long total_blocks = 0;
-    for (int i = 0; i < count; i++) total_blocks += n[i] > 0 ? (n[i] + 255) / 256 : 0;
+    for (int i = 0; i < count; i++) total_blocks += n[i] > 0 ? (n[i] + kNormBlock - 1) / kNormBlock : 0;
     float *partial = scratch(11, (size_t)(total_blocks > 0 ? total_blocks : 1) * sizeof(float));
     if (es.failed()) return 1;
     int off = 0;
@@ -335,19 +392,22 @@ unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, flo
             if (n[i] <= 0) continue;
             const int c = b.count++;
             b.p[c] = g[i]; b.n[c] = n[i]; b.blk_begin[c] = blocks;
-            blocks += (n[i] + 255) / 256;
+            blocks += (n[i] + kNormBlock - 1) / kNormBlock;
         }
         if (b.count == 0) continue;
         b.blk_begin[b.count] = blocks;
-        const int grid = blocks < 4 ? 1 : (blocks / 4 > 2048 ? 2048 : blocks / 4);
+        const int grid = blocks < 4 ? 1 : ((blocks + 3) / 4 > 2048 ? 2048 : (blocks + 3) / 4);   // a wave per block
         hipLaunchKernelGGL(norm_sq_multi_kernel, dim3(grid), dim3(kOptThreads), 0, stream(), b, partial + off);
         unsigned rc = launch_status("grad_norm_clip_multi_rocm/norm");
         if (rc) return rc;
         off += blocks;
     }
-    unsigned rc = reduce_partials_clip_cuda(partial, off, max_grad_norm, out_norm, out_scale);
-    if (rc) return rc;
-    // pass 2: scale in place when the device-side scale is < 1
+    return reduce_partials_clip_cuda(partial, off, max_grad_norm, out_norm, out_scale);
+}
+
+// every tensor times *scale_ptr, in place, when that is below 1
+unsigned nlh::grad_scale_multi(float *const *g, const int *n, int count, const float *out_scale) {
+    unsigned rc = 0;
     for (int first = 0; first < count; first += kMaxTensors) {
         PtrBatch b;
         b.count = 0;
@@ -368,6 +428,8 @@ unsigned grad_norm_clip_multi_rocm(float *const *g, const int *n, int count, flo
     return 0;
 }
 
+
+extern "C" {
 
 // ── M3 optimizer helpers ────────────────────────────────────────────────────
 unsigned m3_ema_update_cuda(float *m1, float *m2, float *v, const float *g, int n, float beta1, float beta2,
