@@ -53,9 +53,11 @@ __global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restric
                                                           const float *__restrict__ eta, float *__restrict__ tab_a,
                                                           float *__restrict__ tab_b, float *__restrict__ vecs,
                                                           int s, int C, int nc, int nchunks) {
-    // One chunk per workgroup of two waves; both tables are assembled in LDS and leave as 16-byte
-    // stores of consecutive lanes.
-    __shared__ __align__(16) float stage[2][kTab];
+    // One chunk per workgroup of two waves.  tab_a is assembled in LDS and leaves as 16-byte stores of
+    // consecutive lanes; tab_b holds the same numbers in the other tile orientation and is gathered from
+    // the same LDS copy on the way out (one table of LDS instead of two: twice the workgroups per CU for a
+    // kernel that is one serial 64-step loop per chunk).
+    __shared__ __align__(16) float stage[kTab];
     const int chunk = blockIdx.x, role = threadIdx.x >> 6, j = threadIdx.x & 63;
     const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
     const Gates g = fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, L);
@@ -63,11 +65,10 @@ __global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restric
     const float eta_j = g.et;          // 0 beyond L
     float *vo = vecs + (size_t)chunk * kVecB;
     if (role == 0) {
-        float *ta = stage[0], *tb = stage[1];
+        float *ta = stage;
         float b = 1.f, cc = 1.f, blv = 0.f;
         const bool jv = j < L;
         const int ja = (j >> 5) * 2048 + ((j >> 4) & 1) * 512 + ((j & 15) >> 2) * 64 + (j & 3);
-        const int jb = (j >> 5) * 1024 + ((j >> 4) & 1) * 256 + (j & 15) * 4;
 #pragma unroll
         for (int t = 0; t < CW; t++) {
             const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
@@ -78,7 +79,6 @@ __global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restric
             if ((t >> 4) >= (j >> 4)) {
                 const float x = (jv && t >= j && t < L) ? cc : 0.f;
                 ta[ja + (t >> 5) * 1024 + ((t >> 4) & 1) * 256 + (t & 15) * 4] = x;
-                tb[jb + (t >> 5) * 2048 + ((t >> 4) & 1) * 512 + ((t & 15) >> 2) * 64 + (t & 3)] = x;
             }
         }
         vo[2 * CW + j] = jv ? cc : 0.f;
@@ -103,8 +103,15 @@ __global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restric
     float *oa = tab_a + (size_t)chunk * kTab, *ob = tab_b + (size_t)chunk * kTab;
     for (int qd = threadIdx.x; qd < kTab / 4; qd += 128) {
         const int tile = qd >> 6, bi = tile >> 2, rt = (tile >> 1) & 1, ct = tile & 1;
-        if (live_a(bi, rt, ct)) *reinterpret_cast<f32x4 *>(oa + qd * 4) = *reinterpret_cast<const f32x4 *>(stage[0] + qd * 4);
-        if (live_b(bi, rt, ct)) *reinterpret_cast<f32x4 *>(ob + qd * 4) = *reinterpret_cast<const f32x4 *>(stage[1] + qd * 4);
+        if (live_a(bi, rt, ct)) *reinterpret_cast<f32x4 *>(oa + qd * 4) = *reinterpret_cast<const f32x4 *>(stage + qd * 4);
+        if (live_b(bi, rt, ct)) {
+            // element X = 4 qd + r of tab_b is c[t][j] with t = 32 X[11] + 16 X[9] + 4 X[7:6] + r, j = 32 X[10] +
+            // 16 X[8] + X[5:2]; in tab_a that pair sits at the index below, consecutive t four floats apart
+            const int X = qd * 4;
+            const int jl = (X >> 2) & 15, a0 = ((X >> 10) & 1) * 2048 + ((X >> 11) & 1) * 1024 + ((X >> 8) & 1) * 512 +
+                                              ((X >> 9) & 1) * 256 + (jl >> 2) * 64 + ((X >> 6) & 3) * 16 + (jl & 3);
+            *reinterpret_cast<f32x4 *>(ob + X) = f32x4{stage[a0], stage[a0 + 4], stage[a0 + 8], stage[a0 + 12]};
+        }
     }
 }
 

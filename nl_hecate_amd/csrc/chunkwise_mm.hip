@@ -763,18 +763,22 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
 constexpr size_t kGradsBwdLds = 9 * MAT * sizeof(float);
 
 // Sum over chains of st[chain][slot 0][.]: stage 1 sums `per` chains per block row into
-// tmp[rows][4096]; stage 2 adds the rows to dst (+=).
-__global__ void cw_sum_slot0_kernel(const float *__restrict__ st, float *__restrict__ tmp, int batch, int per,
-                                    size_t chain_stride) {
+// tmp[which][rows][4096]; stage 2 adds the rows to dst (+=).  blockIdx.z = which: the M adjoint (0) and the S
+// adjoint (1) share the two launches.
+__global__ void cw_sum_slot0_kernel(const float *__restrict__ st0, const float *__restrict__ st1,
+                                    float *__restrict__ tmp, int batch, int per, size_t chain_stride) {
+    const float *st = blockIdx.z ? st1 : st0;
     const int e = blockIdx.x * blockDim.x + threadIdx.x, b0 = blockIdx.y * per, b1 = min(batch, b0 + per);
     float x = 0.f;
     for (int b = b0; b < b1; b++) x += st[(size_t)b * chain_stride + e];
-    tmp[(size_t)blockIdx.y * HD * HD + e] = x;
+    tmp[((size_t)blockIdx.z * gridDim.y + blockIdx.y) * HD * HD + e] = x;
 }
-__global__ void cw_add_rows_kernel(const float *__restrict__ tmp, float *__restrict__ dst, int rows) {
+__global__ void cw_add_rows_kernel(const float *__restrict__ tmp, float *__restrict__ dst0, float *__restrict__ dst1,
+                                   int rows) {
+    float *dst = blockIdx.z ? dst1 : dst0;
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     float x = 0.f;
-    for (int r = 0; r < rows; r++) x += tmp[(size_t)r * HD * HD + e];
+    for (int r = 0; r < rows; r++) x += tmp[((size_t)blockIdx.z * rows + r) * HD * HD + e];
     dst[e] += x;
 }
 
@@ -909,19 +913,19 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s);
     const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
     const int per = 8, rows = ceil_div(batch, per);
-    float *tmp = scratch(10, (size_t)rows * HD * HD * sizeof(float));
+    const int nsum = has_s && d_s_initial ? 2 : 1;
+    float *tmp = scratch(10, (size_t)nsum * rows * HD * HD * sizeof(float));
     if (es.failed()) return;
-    for (int which = 0; which < (has_s && d_s_initial ? 2 : 1); which++) {
-        {
-            KernelTimer kt("cw_sum_slot0_kernel");
-            hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows), dim3(256), 0, stream(),
-                               which ? ds_states : dm_states, tmp, batch, per, chain_stride);
-        }
-        KernelTimer kt("cw_add_rows_kernel");
-        hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256), dim3(256), 0, stream(), tmp,
-                           which ? d_s_initial : d_m_initial, rows);
+    {
+        KernelTimer kt("cw_sum_slot0_kernel");
+        hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows, nsum), dim3(256), 0, stream(), dm_states,
+                           ds_states, tmp, batch, per, chain_stride);
     }
     check_launch("cw_sum_slot0_kernel");
+    KernelTimer kt("cw_add_rows_kernel");
+    hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256, 1, nsum), dim3(256), 0, stream(), tmp, d_m_initial,
+                       d_s_initial, rows);
+    check_launch("cw_add_rows_kernel");
 }
 
 }  // namespace
