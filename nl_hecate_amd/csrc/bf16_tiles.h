@@ -30,6 +30,23 @@ __device__ __forceinline__ bf16x8 ld_op(const u16 *X, int row0, int ks) {
     const int l = threadIdx.x & 63;
     return *reinterpret_cast<const bf16x8 *>(X + (row0 + (l & 15)) * LDB + 32 * ks + 8 * (l >> 4));
 }
+// The same operand from a matrix stored the other way round (element (contraction index k, row n) at
+// X[k * STRIDE + n]), with no transposed copy: ds_read_b64_tr_b16 works on groups of 16 lanes; when lane s of
+// a group addresses the four elements X[k0 + s/4][n0 + 4 (s%4) .. + 3], lane i receives X[k0 .. k0 + 3][n0 + i].
+// Two such reads give the eight contraction indices 32*ks + 8*(l/16) .. + 8 of row row0 + l%16.  STRIDE in
+// elements, a multiple of 4; conflict-free inside a group when STRIDE / 2 is 8 modulo 16 (48, 80, ..).
+template <int STRIDE>
+__device__ __forceinline__ bf16x8 ld_op_tr(const u16 *X, int row0, int ks) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 *lds_ptr;
+    const int l = threadIdx.x & 63, sl = l & 15;
+    const u16 *p = X + (32 * ks + 8 * (l >> 4) + (sl >> 2)) * STRIDE + row0 + 4 * (sl & 3);
+    const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p);
+    const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * STRIDE));
+    const s16x8 ab = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, ab);
+}
 // x = hi + lo with hi, lo bf16; both stored as four consecutive elements at off.
 __device__ __forceinline__ void split_store(u16 *H, u16 *Lo, int off, f32x4 x) {
     bf16x4 h, lo;

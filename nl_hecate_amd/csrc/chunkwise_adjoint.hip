@@ -24,6 +24,10 @@ namespace nlh {
 namespace {
 
 constexpr int HMAT = 32 * LDB;   // elements of a 32-row bf16 matrix
+constexpr int DYS = 48;          // row stride of a [token][32 rows] bf16 matrix (read through ld_op_tr)
+constexpr int DYM = 64 * DYS;
+constexpr int kLate = 2 * BMAT + 4 * DYM;   // elements of one copy of the last phase's operands
+constexpr int kCvec = 5 * CW + 8;
 
 template <bool HAS_S>
 __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
@@ -31,17 +35,16 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     const float *__restrict__ tab_b, const float *__restrict__ vecs, float *__restrict__ dm_states,
     float *__restrict__ ds_states, int s, int C, int nc, int batch, int tab_floats, int vec_floats, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Kt = Kr + BMAT;   // K [j][c], K^T [c][j]
-    u16 *Qr = Kt + BMAT, *Qt = Qr + BMAT;                            // Q [t][c], Q^T [c][t]
-    u16 *WPh = Qt + BMAT, *WPl = WPh + BMAT;                         // (W.P)^T [j][t]
-    u16 *dYh = WPl + BMAT, *dYl = dYh + HMAT;                        // dY^T [i][t] (this workgroup's 32 rows i)
-    u16 *dYah = dYl + HMAT, *dYal = dYah + HMAT;                     // (a.dY)^T
-    u16 *dYbh = dYal + HMAT, *dYbl = dYbh + HMAT;                    // (beta.dY)^T
-    u16 *dMh = dYbl + HMAT, *dMl = dMh + HMAT;                       // dMo [i][c]
-    u16 *dSh = dMl + HMAT, *dSl = dSh + HMAT;                        // dSo [i][c]
-    u16 *dEh = dSl + HMAT, *dEl = dEh + HMAT;                        // dE^T [i][j]
-    float *cvec = reinterpret_cast<float *>(dEl + HMAT);             // a, beta, cl, bl, theta [64] each, .., h_L
-
+    u16 *WPh = reinterpret_cast<u16 *>(smem_raw), *WPl = WPh + BMAT;   // (W.P)^T [j][t]
+    u16 *dYh = WPl + BMAT, *dYl = dYh + DYM;                           // dY [t][i] (this workgroup's 32 rows i)
+    u16 *dMh = dYl + DYM, *dMl = dMh + HMAT;                           // dMo [i][c]
+    u16 *dSh = dMl + HMAT, *dSl = dSh + HMAT;                          // dSo [i][c]
+    u16 *dEh = dSl + HMAT, *dEl = dEh + HMAT;                          // dE^T [i][j]
+    // What the last phase of a step reads exists twice, so that the next step's copy is written while
+    // this step's is still in use: K [j][c], Q [t][c], a.dY hi / lo, beta.dY hi / lo [t][i], and the
+    // vectors a, beta, cl, bl, theta [64] each, .., h_L
+    u16 *late = dEl + HMAT;
+    float *cvecs = reinterpret_cast<float *>(late + 2 * kLate);
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
     int chain, half;
     chain_half_of_block(batch, chain, half);
@@ -59,7 +62,7 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
 
     // registers of the next step (chunk c - 1)
     uint4 nK, nQ;
-    f32x4 ndY, ntab[2];
+    f32x4 ndY;
     float na = 0.f, nb = 0.f, nvec = 0.f;
     const int tt = w >> 1, jt0 = 2 * (w & 1);   // phase A: P tiles (tt, jt0) and (tt, jt0 + 1)
     auto fetch = [&](int c) {
@@ -71,47 +74,41 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
         ndY = *reinterpret_cast<const f32x4 *>(d_y + dy_off + (size_t)(c * C + min(yt, L - 1)) * dyr.row_stride + i0 +
                                                yg * 4);
         const size_t chunk = (size_t)chain * nc + c;
-        const float *vo = vecs + chunk * vec_floats, *tb = tab_b + chunk * tab_floats;
+        const float *vo = vecs + chunk * vec_floats;
         na = vo[yt];
         nb = vo[CW + yt];
         nvec = vo[min(tid, 5 * CW + 7)];
+    };
+    // The coefficient tiles are used by the first phase of a step only; the next step's are requested right
+    // after that use, into the same registers (a value that had to outlive the next request would be copied at
+    // the bottom of the loop, behind a wait for that request).
+    f32x4 ctab[2];
+    auto fetch_tab = [&](int c) {
+        const size_t chunk = (size_t)chain * nc + c;
+        const float *vo = vecs + chunk * vec_floats, *tb = tab_b + chunk * tab_floats;
 #pragma unroll
         for (int x = 0; x < 2; x++) {
             const int jt = jt0 + x, bi = 2 * (tt >> 1) + (jt >> 1);
-            ntab[x] = *reinterpret_cast<const f32x4 *>(
+            ctab[x] = *reinterpret_cast<const f32x4 *>(
                 jt <= tt ? tb + (((bi * 2 + (tt & 1)) * 2 + (jt & 1)) * 64 + l) * 4 : vo + 5 * CW);
         }
     };
-    f32x4 ctab[2];
-    auto commit = [&](int c) {
+    // Registers -> LDS, everything in the order it arrives (rows = tokens): the products that contract over
+    // tokens read their operands through ld_op_tr.  Called in the last phase of the step before: dY is no
+    // longer read there, and the rest goes to the copy that this step does not use.
+    auto commit = [&](int c, int par) {
         const int L = min(C, s - c * C);
+        u16 *Kr = late + par * kLate, *Qr = Kr + BMAT;
+        u16 *dYah = Qr + BMAT, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
         if (st_t >= L) { nK = make_uint4(0, 0, 0, 0); nQ = nK; }
         if (yt >= L) ndY = zero4();
         *reinterpret_cast<uint4 *>(Kr + st_t * LDB + st_cb * 8) = nK;
         *reinterpret_cast<uint4 *>(Qr + st_t * LDB + st_cb * 8) = nQ;
-        const unsigned kw[4] = {nK.x, nK.y, nK.z, nK.w}, qw[4] = {nQ.x, nQ.y, nQ.z, nQ.w};
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            Kt[(st_cb * 8 + 2 * e) * LDB + st_t] = (u16)(kw[e] & 0xffffu);
-            Kt[(st_cb * 8 + 2 * e + 1) * LDB + st_t] = (u16)(kw[e] >> 16);
-            Qt[(st_cb * 8 + 2 * e) * LDB + st_t] = (u16)(qw[e] & 0xffffu);
-            Qt[(st_cb * 8 + 2 * e + 1) * LDB + st_t] = (u16)(qw[e] >> 16);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int off = (yg * 4 + e) * LDB + yt;
-            auto put = [&](u16 *H, u16 *Lo, float x) {
-                const __bf16 hb = (__bf16)x;
-                reinterpret_cast<__bf16 *>(H)[off] = hb;
-                reinterpret_cast<__bf16 *>(Lo)[off] = (__bf16)(x - (float)hb);
-            };
-            put(dYh, dYl, ndY[e]);
-            put(dYah, dYal, na * ndY[e]);
-            if (HAS_S) put(dYbh, dYbl, nb * ndY[e]);
-        }
-        if (tid < 5 * CW + 8) cvec[tid] = nvec;
-        ctab[0] = ntab[0];
-        ctab[1] = ntab[1];
+        const int off = yt * DYS + yg * 4;
+        split_store(dYh, dYl, off, ndY);
+        split_store(dYah, dYal, off, na * ndY);
+        if (HAS_S) split_store(dYbh, dYbl, off, nb * ndY);
+        if (tid < kCvec) cvecs[par * kCvec + tid] = nvec;
     };
 
     // fp32 master: transposed tile rows c = 16 (w/2) + 4 (l/16) + r, column i = 16 (w%2) + l%16
@@ -127,12 +124,16 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     };
 
     fetch(nc - 1);
+    fetch_tab(nc - 1);
     publish(nc);
+    commit(nc - 1, (nc - 1) & 1);
+    fetch(max(nc - 2, 0));
+    __syncthreads();
     for (int c = nc - 1; c >= 0; c--) {
-        const int L = min(C, s - c * C);
-        commit(c);
-        __syncthreads();
-        fetch(max(c - 1, 0));
+        const int L = min(C, s - c * C), par = c & 1;
+        const float *cvec = cvecs + par * kCvec;
+        const u16 *Kr = late + par * kLate, *Qr = Kr + BMAT;
+        const u16 *dYah = Qr + BMAT, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
         // ── (W.P)^T: this wave's two tiles of P[t][j] ──
         {
             const bf16x8 aq[2] = {ld_op(Qr, 16 * tt, 0), ld_op(Qr, 16 * tt, 1)};
@@ -148,6 +149,7 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
                 }
             }
         }
+        fetch_tab(max(c - 1, 0));
         __syncthreads();
         // ── dE[j][i]: tile rows j = 16 rt.., columns i = 16 ct.. ──
         {
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 const bf16x8 wh = ld_op(WPh, 16 * rt, ks), wl = ld_op(WPl, 16 * rt, ks), ak = ld_op(Kr, 16 * rt, ks);
-                const bf16x8 yh = ld_op(dYh, 16 * ct, ks), yl = ld_op(dYl, 16 * ct, ks);
+                const bf16x8 yh = ld_op_tr<DYS>(dYh, 16 * ct, ks), yl = ld_op_tr<DYS>(dYl, 16 * ct, ks);
                 e1 = mfma32(wh, yh, e1);
                 e1 = mfma32(wl, yh, e1);
                 e1 = mfma32(wh, yl, e1);
@@ -173,19 +175,23 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
             split_store(dEh, dEl, (16 * ct + r16) * LDB + j4, e1 - th * (cl * e2 + bl * e3));   // [i][j .. j+3]
         }
         __syncthreads();
+        // ── the inputs of the next step (chunk c - 1; chunk 0 once more after the last) go to LDS, those of
+        //    the one after are requested ──
+        commit(max(c - 1, 0), par ^ 1);
+        fetch(max(c - 2, 0));
         // ── dM0^T, dS0^T: tile rows c = 16 rt.., columns i = 16 ct.. ──
         {
             f32x4 am = zero4(), as = zero4();
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                const bf16x8 aq = ld_op(Qt, 16 * rt, ks), ak = ld_op(Kt, 16 * rt, ks);
-                am = mfma32(aq, ld_op(dYah, 16 * ct, ks), am);
-                am = mfma32(aq, ld_op(dYal, 16 * ct, ks), am);
+                const bf16x8 aq = ld_op_tr<LDB>(Qr, 16 * rt, ks), ak = ld_op_tr<LDB>(Kr, 16 * rt, ks);   // Q^T, K^T
+                am = mfma32(aq, ld_op_tr<DYS>(dYah, 16 * ct, ks), am);
+                am = mfma32(aq, ld_op_tr<DYS>(dYal, 16 * ct, ks), am);
                 am = mfma32(ak, ld_op(dEh, 16 * ct, ks), am);
                 am = mfma32(ak, ld_op(dEl, 16 * ct, ks), am);
                 if (HAS_S) {
-                    as = mfma32(aq, ld_op(dYbh, 16 * ct, ks), as);
-                    as = mfma32(aq, ld_op(dYbl, 16 * ct, ks), as);
+                    as = mfma32(aq, ld_op_tr<DYS>(dYbh, 16 * ct, ks), as);
+                    as = mfma32(aq, ld_op_tr<DYS>(dYbl, 16 * ct, ks), as);
                 }
             }
             const float aL = cvec[L - 1], betaL = cvec[CW + L - 1], hL = cvec[5 * CW + 4];
@@ -198,7 +204,7 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     }
 }
 
-constexpr size_t kAdjointLds = (6 * BMAT + 12 * HMAT) * sizeof(u16) + (5 * CW + 8) * sizeof(float);
+constexpr size_t kAdjointLds = (2 * BMAT + 2 * DYM + 6 * HMAT + 2 * kLate) * sizeof(u16) + 2 * kCvec * sizeof(float);
 
 }  // namespace
 

@@ -14,6 +14,11 @@
 // 64 steps on ONE wave and no matrix product, no coefficient table and no division:
 //   sweep 1 (lane = t): u, v for s = 0..63, parked in LDS as rows s + 1
 //   sweep 2 (lane = s): the weighted sums over t >= s with the weights advanced step by step.
+// Row s is only ever read at t >= s, so the rows are packed as a triangle (row s starts at
+// 64 s - s (s - 1) / 2 and holds t = s .. 63): half the LDS of a square, which is what decides how many
+// chunks a compute unit works on at once.  Sweep 1 writes a row at consecutive addresses; in sweep 2
+// lane s reads address 63 s - s (s - 1) / 2 + t, whose bank is t minus a triangular number: the
+// triangular numbers of 32 consecutive s fall on 32 different banks.
 // Gates travel as wave-uniform values (v_readlane); tokens beyond a short chunk carry keep = 1, eta = 0
 // and zero terms.
 #include <hip/hip_runtime.h>
@@ -26,8 +31,9 @@ namespace nlh {
 namespace {
 
 constexpr int GW = 64;            // tokens per chunk tile
-constexpr int GLD = 65;           // LDS row stride (floats): rows and columns conflict-free
+constexpr int GTRI = GW * (GW + 1) / 2;   // floats of one packed triangle
 constexpr int kGateWaves = 4;     // chunks per workgroup, one wave each
+__host__ __device__ constexpr int tri_row(int r) { return GW * r - r * (r - 1) / 2; }
 
 __device__ __forceinline__ float bcast(float x, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
@@ -42,7 +48,7 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int task = blockIdx.x * kGateWaves + wv;
     if (task >= ntask) return;   // no barrier below: waves are independent
-    float *U = smem + (size_t)wv * (HAS_S ? 2 : 1) * GW * GLD, *V = U + GW * GLD;
+    float *U = smem + (size_t)wv * (HAS_S ? 2 : 1) * GTRI, *V = U + GTRI;
     const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0;
     const bool in = lane < L;
@@ -79,8 +85,10 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
         u = fmaf(kp, u, v);
         um = fmaf(kp, um, vm);
         if (sx + 1 < GW) {
-            U[(sx + 1) * GLD + lane] = u;
-            if (HAS_S) V[(sx + 1) * GLD + lane] = v;
+            if (lane >= sx + 1) {   // row sx + 1, columns t >= sx + 1
+                U[tri_row(sx + 1) - (sx + 1) + lane] = u;
+                if (HAS_S) V[tri_row(sx + 1) - (sx + 1) + lane] = v;
+            }
             if (lane == sx + 1) { pum = um; pvm = vm; pvs = vs; }
         }
     }
@@ -90,7 +98,8 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
 
     // ── sweep 2: lane = s; weights r[s][t], c[t][s], bb[s][t] advance with t ──
     float rho = 1.f, cc = 1.f, bb = 1.f, accA = 0.f, accE = 0.f;
-    const float *Ur = U + lane * GLD, *Vr = V + lane * GLD;
+    // row s seen from column 0: what it reads at t < s belongs to earlier rows and is weighted by zero
+    const float *Ur = U + tri_row(lane) - lane, *Vr = V + tri_row(lane) - lane;
 #pragma unroll
     for (int t = 0; t < GW; t++) {
         const float kp = bcast(keep_l, t);
@@ -117,14 +126,14 @@ void chunkwise_gate_gradients(const float *alpha, const float *eta, const float 
                               int chunk_size, bool has_s) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
-    const size_t lds = (size_t)kGateWaves * (has_s ? 2 : 1) * GW * GLD * sizeof(float);
+    const size_t lds = (size_t)kGateWaves * (has_s ? 2 : 1) * GTRI * sizeof(float);
     static bool attr_set = false;
     if (!attr_set) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_gates_sweep_kernel<true>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kGateWaves * 2 * GW * GLD * 4)),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kGateWaves * 2 * GTRI * 4)),
                   "dynamic LDS size");
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_gates_sweep_kernel<false>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kGateWaves * GW * GLD * 4)),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kGateWaves * GTRI * 4)),
                   "dynamic LDS size");
         attr_set = true;
     }
