@@ -141,17 +141,16 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
     int C, int nc, int ntask, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Kt = Kr + BMAT;   // K [t][c], K^T [c][t]
-    u16 *Qr = Kt + BMAT, *Qt = Qr + BMAT;                            // Q, Q^T
-    u16 *Vr = Qt + BMAT;                                             // V [t][i]
-    u16 *dYr = Vr + BMAT, *dYt = dYr + BMAT;                         // dY [t][i], dY^T [i][t]
-    u16 *M0h = dYt + BMAT, *M0l = M0h + BMAT, *M0t = M0l + BMAT;     // M0 [i][c] hi / lo, M0^T [c][i]
-    u16 *S0t = M0t + BMAT;                                           // S0^T [c][i]
-    u16 *dMr = S0t + BMAT, *dMt = dMr + BMAT;                        // dMo [i][c], dMo^T [c][i]
-    u16 *dSr = dMt + BMAT, *dSt = dSr + BMAT;                        // dSo
-    u16 *Er = dSt + BMAT;                                            // E [t][i]
-    u16 *CPt = Vr, *CRt = M0h, *ThCR = M0l, *dEr = S0t;              // reuse once their first tenants are dead
-    float *cvec = reinterpret_cast<float *>(Er + BMAT);              // a, beta, cl, bl, theta [64] each
+    // Every input is staged once, in the order it arrives (rows = tokens or state rows); a product that contracts
+    // over the row index reads its operand through ld_op_tr.
+    u16 *Kr = reinterpret_cast<u16 *>(smem_raw), *Qr = Kr + BMAT;   // K [t][c], Q [t][c]
+    u16 *Vr = Qr + BMAT, *dYr = Vr + BMAT;                           // V [t][i], dY [t][i]
+    u16 *M0h = dYr + BMAT, *M0l = M0h + BMAT;                        // M0 [i][c] hi / lo
+    u16 *S0r = M0l + BMAT;                                           // S0 [i][c]
+    u16 *dMr = S0r + BMAT, *dSr = dMr + BMAT;                        // dMo [i][c], dSo [i][c]
+    u16 *Er = dSr + BMAT, *CRt = Er + BMAT;                          // E [t][i]; (c.R)^T [j][t]
+    u16 *CPt = Vr, *ThCR = M0l, *dEr = S0r;                          // reuse once their first tenants are dead
+    float *cvec = reinterpret_cast<float *>(CRt + BMAT);             // a, beta, cl, bl, theta [64] each
     float *part = cvec + 5 * CW;                                     // [5][2][64]: p0, ps, rt, g1, g2 per half
     float *dots = part + 5 * 2 * CW;                                 // [3][8]
 
@@ -248,14 +247,6 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
             *reinterpret_cast<uint4 *>(Kr + st_t * LDB + st_cb * 8) = nK;
             *reinterpret_cast<uint4 *>(Qr + st_t * LDB + st_cb * 8) = nQ;
             *reinterpret_cast<uint4 *>(Vr + st_t * LDB + st_cb * 8) = nV;
-            const unsigned kw[4] = {nK.x, nK.y, nK.z, nK.w}, qw[4] = {nQ.x, nQ.y, nQ.z, nQ.w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                Kt[(st_cb * 8 + 2 * i) * LDB + st_t] = (u16)(kw[i] & 0xffffu);
-                Kt[(st_cb * 8 + 2 * i + 1) * LDB + st_t] = (u16)(kw[i] >> 16);
-                Qt[(st_cb * 8 + 2 * i) * LDB + st_t] = (u16)(qw[i] & 0xffffu);
-                Qt[(st_cb * 8 + 2 * i + 1) * LDB + st_t] = (u16)(qw[i] >> 16);
-            }
             float d0 = 0.f, d1 = 0.f, d2 = 0.f;
 #pragma unroll
             for (int it = 0; it < 2; it++) {
@@ -263,17 +254,12 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 bf16_store(dYr, off, ndY[it]);
                 split_store(M0h, M0l, off, nM0[it]);
                 bf16_store(dMr, off, ndM[it]);
-                if (HAS_S) bf16_store(dSr, off, ndS[it]);
+                if (HAS_S) {
+                    bf16_store(dSr, off, ndS[it]);
+                    bf16_store(S0r, off, nS0[it]);
+                }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int toff = (c4 + i) * LDB + ft;
-                    reinterpret_cast<__bf16 *>(dYt)[toff] = (__bf16)ndY[it][i];
-                    reinterpret_cast<__bf16 *>(M0t)[toff] = (__bf16)nM0[it][i];
-                    reinterpret_cast<__bf16 *>(dMt)[toff] = (__bf16)ndM[it][i];
-                    if (HAS_S) {
-                        reinterpret_cast<__bf16 *>(S0t)[toff] = (__bf16)nS0[it][i];
-                        reinterpret_cast<__bf16 *>(dSt)[toff] = (__bf16)ndS[it][i];
-                    }
                     d0 = fmaf(nM0[it][i], ndM[it][i], d0);
                     if (HAS_S) { d1 = fmaf(nS0[it][i], ndM[it][i], d1); d2 = fmaf(nS0[it][i], ndS[it][i], d2); }
                 }
@@ -330,7 +316,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
             }
         } else {
             // one product at a time: its row sums and its share of dQ^T, then the accumulators are free
-            auto half = [&](const u16 *St, int which, int voff) {
+            auto half = [&](const u16 *Sr, int which, int voff) {   // Sr [i][c]: read as S^T
                 f32x4 ym[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++) {
@@ -339,7 +325,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                     for (int ct = 0; ct < 2; ct++) bD[ct] = ld_op(dYr, bn + 16 * ct, ks);
 #pragma unroll
                     for (int rt = 0; rt < 2; rt++) {
-                        const bf16x8 am = ld_op(St, bm + 16 * rt, ks);
+                        const bf16x8 am = ld_op_tr<LDB>(Sr, bm + 16 * rt, ks);
 #pragma unroll
                         for (int ct = 0; ct < 2; ct++) ym[rt][ct] = mfma32(am, bD[ct], ym[rt][ct]);   // [c][t]
                     }
@@ -360,9 +346,9 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                     if (g == 0) part[(which * 2 + (bi >> 1)) * CW + t] = p0;
                 }
             };
-            half(M0t, 0, 0);
+            half(M0h, 0, 0);
             if (HAS_S) {
-                half(S0t, 1, CW);
+                half(S0r, 1, CW);
             } else {
 #pragma unroll
                 for (int ct = 0; ct < 2; ct++)
@@ -446,7 +432,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int ct = 0; ct < 2; ct++) bP[ct] = ld_op(CPt, bn + 16 * ct, ks);
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
-                    const bf16x8 ay = ld_op(dYt, bm + 16 * rt, ks);
+                    const bf16x8 ay = ld_op_tr<LDB>(dYr, bm + 16 * rt, ks);   // dY^T
 #pragma unroll
                     for (int ct = 0; ct < 2; ct++) dk[rt][ct] = mfma32(ay, bP[ct], dk[rt][ct]);
                 }
@@ -467,7 +453,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 rs = sum_groups(rs);
                 if (g == 0) part[(2 * 2 + (bi >> 1)) * CW + j] = rs;
             }
-            // S0^T was last read two barriers ago: dE may take its place now
+            // S0 was last read two barriers ago: dE may take its place now
 #pragma unroll
             for (int ct = 0; ct < 2; ct++) {
                 const int j = bn + 16 * ct + r16;
@@ -486,7 +472,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int ct = 0; ct < 2; ct++) bT[ct] = ld_op(ThCR, bn + 16 * ct, ks);
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
-                    const bf16x8 ak = ld_op(Kt, bm + 16 * rt, ks);
+                    const bf16x8 ak = ld_op_tr<LDB>(Kr, bm + 16 * rt, ks);   // K^T
 #pragma unroll
                     for (int ct = 0; ct < 2; ct++) keep[rt][ct] = mfma32(ak, bT[ct], keep[rt][ct]);
                 }
@@ -500,7 +486,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                         *reinterpret_cast<f32x4 *>(d_q + (tok + t) * HD + bm + 16 * rt + 4 * g) = keep[rt][ct];
                 }
             }
-            auto state_term = [&](const u16 *At, int which, int voff) {   // dte += cvec[voff + j] . (At E^T); g sums
+            auto state_term = [&](const u16 *Ar, int which, int voff) {   // dte += cvec[voff + j] . (Ar^T E^T); g sums
                 f32x4 t3[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++) {
@@ -509,7 +495,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                     for (int ct = 0; ct < 2; ct++) bE[ct] = ld_op(Er, bn + 16 * ct, ks);
 #pragma unroll
                     for (int rt = 0; rt < 2; rt++) {
-                        const bf16x8 am = ld_op(At, bm + 16 * rt, ks);
+                        const bf16x8 am = ld_op_tr<LDB>(Ar, bm + 16 * rt, ks);
 #pragma unroll
                         for (int ct = 0; ct < 2; ct++) t3[rt][ct] = mfma32(am, bE[ct], t3[rt][ct]);
                     }
@@ -530,9 +516,9 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                     if (g == 0) part[(which * 2 + (bi >> 1)) * CW + j] = g1;
                 }
             };
-            state_term(dMt, 3, 2 * CW);
+            state_term(dMr, 3, 2 * CW);
             if (HAS_S) {
-                state_term(dSt, 4, 3 * CW);
+                state_term(dSr, 4, 3 * CW);
             } else {
 #pragma unroll
                 for (int ct = 0; ct < 2; ct++)
@@ -545,7 +531,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int ct = 0; ct < 2; ct++) bC[ct] = ld_op(CRt, bn + 16 * ct, ks);
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
-                    const bf16x8 aq = ld_op(Qt, bm + 16 * rt, ks);
+                    const bf16x8 aq = ld_op_tr<LDB>(Qr, bm + 16 * rt, ks);   // Q^T
 #pragma unroll
                     for (int ct = 0; ct < 2; ct++) dte[rt][ct] = mfma32(aq, bC[ct], dte[rt][ct]);
                 }
@@ -564,7 +550,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int ct = 0; ct < 2; ct++) bE[ct] = ld_op(dEr, bn + 16 * ct, ks);
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
-                    const bf16x8 am = ld_op(M0t, bm + 16 * rt, ks);
+                    const bf16x8 am = ld_op_tr<LDB>(M0h, bm + 16 * rt, ks);   // M0^T
 #pragma unroll
                     for (int ct = 0; ct < 2; ct++) em[rt][ct] = mfma32(am, bE[ct], em[rt][ct]);
                 }
@@ -595,7 +581,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     }
 }
 
-constexpr size_t kGradsLds = 16 * BMAT * sizeof(u16) + (5 * CW + 10 * CW + 24) * sizeof(float);
+constexpr size_t kGradsLds = 11 * BMAT * sizeof(u16) + (5 * CW + 10 * CW + 24) * sizeof(float);
 
 }  // namespace
 
