@@ -9,8 +9,9 @@
 // matrices).  The rows of dM, dS never mix, so a chain is split over two workgroups of 32 rows
 // each; each walks all chunks with its rows of dM and dS in registers (fp32) and, as bf16
 // hi + lo pairs, in LDS as operands of the next step.  HBM sees k, q, dY and the coefficient
-// table once per step and receives one adjoint snapshot per chunk: dm_states[chain][c] is the
-// adjoint of the state at the start of chunk c (slot num_chunks = 0).
+// table once per step and receives one adjoint snapshot per chunk, in bf16: dm_snap[chain][c] is the
+// adjoint of the state at the start of chunk c (slot num_chunks = 0), rounded as the gradient pass
+// would round it; slot 0, the gradient of the initial state, leaves in fp32 (dm_first).
 //
 // Every fp32 operand enters the bf16 matrix cores as a hi + lo pair: this path is recurrent.
 #include <hip/hip_runtime.h>
@@ -32,8 +33,8 @@ constexpr int kCvec = 5 * CW + 8;
 template <bool HAS_S>
 __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ q, const float *__restrict__ d_y,
-    const float *__restrict__ tab_b, const float *__restrict__ vecs, float *__restrict__ dm_states,
-    float *__restrict__ ds_states, int s, int C, int nc, int batch, int tab_floats, int vec_floats, HeadRows dyr) {
+    const float *__restrict__ tab_b, const float *__restrict__ vecs, u16 *__restrict__ dm_snap,
+    u16 *__restrict__ ds_snap, float *__restrict__ dm_first, float *__restrict__ ds_first, int s, int C, int nc, int batch, int tab_floats, int vec_floats, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *WPh = reinterpret_cast<u16 *>(smem_raw), *WPl = WPh + BMAT;   // (W.P)^T [j][t]
     u16 *dYh = WPl + BMAT, *dYl = dYh + DYM;                           // dY [t][i] (this workgroup's 32 rows i)
@@ -114,13 +115,26 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     // fp32 master: transposed tile rows c = 16 (w/2) + 4 (l/16) + r, column i = 16 (w%2) + l%16
     const int rt = w >> 1, ct = w & 1;
     f32x4 dM = zero4(), dS = zero4();
+    // The snapshot a later pass reads is the bf16 value that this scan itself uses as the hi operand; the
+    // gradient of the initial state (slot 0) leaves in fp32.
     auto publish = [&](int slot) {
-        const size_t o = state0 + (size_t)slot * HD * HD + (i0 + 16 * ct + r16) * HD + 16 * rt + 4 * g;
-        *reinterpret_cast<f32x4 *>(dm_states + o) = dM;
-        if (HAS_S) *reinterpret_cast<f32x4 *>(ds_states + o) = dS;
-        const int off = (16 * ct + r16) * LDB + 16 * rt + 4 * g;
-        split_store(dMh, dMl, off, dM);
-        if (HAS_S) split_store(dSh, dSl, off, dS);
+        const int e = (i0 + 16 * ct + r16) * HD + 16 * rt + 4 * g, off = (16 * ct + r16) * LDB + 16 * rt + 4 * g;
+        const size_t o = state0 + (size_t)slot * HD * HD + e;
+        auto one = [&](u16 *H, u16 *Lo, u16 *snap, float *first, const f32x4 &x) {
+            bf16x4 h, lo;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const __bf16 hb = (__bf16)x[i];
+                h[i] = hb;
+                lo[i] = (__bf16)(x[i] - (float)hb);
+            }
+            *reinterpret_cast<bf16x4 *>(H + off) = h;
+            *reinterpret_cast<bf16x4 *>(Lo + off) = lo;
+            if (slot) *reinterpret_cast<bf16x4 *>(snap + o) = h;
+            else *reinterpret_cast<f32x4 *>(first + (size_t)chain * HD * HD + e) = x;
+        };
+        one(dMh, dMl, dm_snap, dm_first, dM);
+        if (HAS_S) one(dSh, dSl, ds_snap, ds_first, dS);
     };
 
     fetch(nc - 1);
@@ -209,8 +223,9 @@ constexpr size_t kAdjointLds = (2 * BMAT + 2 * DYM + 6 * HMAT + 2 * kLate) * siz
 }  // namespace
 
 bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
-                            const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
-                            int chunk_size, bool has_s, const HeadRows *dy_rows) {
+                            const float *vecs, uint16_t *dm_snap, uint16_t *ds_snap, float *dm_first,
+                            float *ds_first, int seq_len, int batch, int chunk_size, bool has_s,
+                            const HeadRows *dy_rows) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size);
     const HeadRows dyr = dy_rows ? *dy_rows : head_major_rows(seq_len, HD);
@@ -227,10 +242,12 @@ bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d
     KernelTimer kt("cw_adjoint_chain_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_adjoint_chain_kernel<true>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
-                           d_y, tab_b, vecs, dm_states, ds_states, seq_len, chunk_size, nc, batch, tabf, vecf, dyr);
+                           d_y, tab_b, vecs, dm_snap, ds_snap, dm_first, ds_first, seq_len, chunk_size, nc, batch, tabf,
+                           vecf, dyr);
     else
         hipLaunchKernelGGL(cw_adjoint_chain_kernel<false>, dim3(2 * batch), dim3(kTileThr), kAdjointLds, stream(), k, q,
-                           d_y, tab_b, vecs, dm_states, nullptr, seq_len, chunk_size, nc, batch, tabf, vecf, dyr);
+                           d_y, tab_b, vecs, dm_snap, nullptr, dm_first, nullptr, seq_len, chunk_size, nc, batch, tabf,
+                           vecf, dyr);
     check_launch("cw_adjoint_chain_kernel");
     return true;
 }

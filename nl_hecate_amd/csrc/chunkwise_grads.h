@@ -2,8 +2,10 @@
 // launches on the library's stream:
 //   chunkwise_backward_coefficients: per-chunk coefficient tables tab_a, tab_b (table_floats per
 //     chunk) and vectors vecs (vec_floats per chunk) from the gates
-//   chunkwise_adjoint_bf16: the adjoint scan; dm_states / ds_states [batch][num_chunks + 1][64*64],
-//     slot c = adjoint of the state at the start of chunk c
+//   chunkwise_adjoint_bf16: the adjoint scan; dm_snap / ds_snap [batch][num_chunks + 1][64*64] in bf16,
+//     slot c = adjoint of the state at the start of chunk c as the gradient pass takes it (one bf16
+//     operand; slot 0 is not written), and dm_first / ds_first [batch][64*64] in fp32 = slot 0, the
+//     gradient of the initial state
 //   chunkwise_grads_bf16: d_q, d_k, d_v, d_theta, and for the gate pass
 //     pvec [token][4] = p0_t = dy_t^T M0 q_t, ps_t = dy_t^T S0 q_t, -theta_t e_t^T dMo k_t, -theta_t e_t^T dSo k_t
 //     xs [chunk][j][t] = -theta_j (dy_t . e_j)(q_t . k_j)      scal [chunk][4] = <M0,dMo>, <S0,dMo>, <S0,dSo>
@@ -23,12 +25,13 @@ void chunkwise_backward_coefficients(const float *alpha, const float *theta, con
                                      float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s);
 
 bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
-                            const float *vecs, float *dm_states, float *ds_states, int seq_len, int batch,
-                            int chunk_size, bool has_s, const HeadRows *dy_rows = nullptr);
+                            const float *vecs, uint16_t *dm_snap, uint16_t *ds_snap, float *dm_first,
+                            float *ds_first, int seq_len, int batch, int chunk_size, bool has_s,
+                            const HeadRows *dy_rows = nullptr);
 
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
-                          const float *m_states, const float *s_states, const float *dm_states,
-                          const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
+                          const float *m_states, const float *s_states, const uint16_t *dm_snap,
+                          const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid,
                           const HeadRows *dy_rows = nullptr);

@@ -19,10 +19,11 @@
 // accumulate in fp32.  That is the bf16-input / fp32-accumulate contract: results agree with
 // an fp32 evaluation of the same rule to a few 1e-3, inside the 2e-2 stated for this path.
 //
-// One workgroup per compute unit walks over chunks.  While one chunk computes, the lines of the
-// next chunk's bf16 token tiles are touched by one 4-byte load each, so that the first loads at the
-// top of the next step come from the L2 cache; holding the inputs themselves in registers
-// across a step would not fit beside the accumulators.  Every output tile is computed transposed
+// One workgroup per compute unit walks over chunks.  The inputs of the next chunk are requested right
+// after this chunk's have been staged and stay in registers for the rest of the step (the staged copies
+// need 11 LDS matrices and no transposed ones, which leaves the registers for that).  The pass moves
+// 1.6 GB per launch at configuration size and is bound by that traffic; the adjoint snapshots arrive as
+// bf16, as the scan's own hi operand.  Every output tile is computed transposed
 // (rows = feature, columns = token) so that a lane ends up with four consecutive features of
 // one token: 16-byte stores.  Waves 0..3 (group A) hold P and produce X, c.P, c.R, Dk; waves
 // 4..7 (group B) hold dQ and produce -theta c.R, dQ, DTe, dK.
@@ -126,18 +127,18 @@ __device__ __forceinline__ float sum_wave(float x) {
     for (int m = 1; m < 64; m <<= 1) x += __shfl_xor(x, m);
     return x;
 }
-__device__ __forceinline__ f32x4 bf4_to_f32(const u16 *p) {
-    const uint2 b = *reinterpret_cast<const uint2 *>(p);
+__device__ __forceinline__ f32x4 bf4_to_f32(const uint2 b) {
     return f32x4{__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u), __uint_as_float(b.y << 16),
                  __uint_as_float(b.y & 0xffff0000u)};
 }
+__device__ __forceinline__ f32x4 bf4_to_f32(const u16 *p) { return bf4_to_f32(*reinterpret_cast<const uint2 *>(p)); }
 
 template <bool HAS_S>
 __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q, const float *__restrict__ d_y,
     const float *__restrict__ tab_a, const float *__restrict__ tab_b, const float *__restrict__ vecs,
-    const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
-    const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
+    const float *__restrict__ m_states, const float *__restrict__ s_states, const u16 *__restrict__ dm_snap,
+    const u16 *__restrict__ ds_snap, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
     int C, int nc, int ntask, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -158,8 +159,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const bool grpA = w < 4;
     const int bi = w & 3, bm = 32 * (bi >> 1), bn = 32 * (bi & 1);
     // Staging maps.  A wave instruction reads whole or half 128-byte lines (the rate of line
-    // requests, not bytes, bounds a compute unit), and the 2-byte transposed LDS writes of a
-    // wave land on 16 different banks.
+    // requests, not bytes, bounds a compute unit).
     //   bf16 tile: row st_t, 8-element block st_cb (16 rows x 64 bytes per wave)
     //   fp32 tile: row ft, 4-element blocks fg0 and fg0 + 8 (8 rows x 128 bytes per wave and pass)
     const int st_t = 16 * (w & 3) + (l & 15), st_cb = 4 * (w >> 2) + (l >> 4);
@@ -167,7 +167,8 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
 
     // inputs of the current task in registers (only while they are staged)
     uint4 nK, nQ, nV;
-    f32x4 ndY[2], nM0[2], nS0[2], ndM[2], ndS[2], ntab[2][2];
+    f32x4 ndY[2], nM0[2], nS0[2], ntab[2][2];
+    uint2 ndM[2], ndS[2];   // four bf16 each
     float nvec = 0.f;
     auto fetch = [&](int task) {
         const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
@@ -182,10 +183,10 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
             const int c4 = (fg0 + 8 * it) * 4;
             ndY[it] = *reinterpret_cast<const f32x4 *>(dy_row + c4);
             nM0[it] = *reinterpret_cast<const f32x4 *>(m_states + st0 + c4);
-            ndM[it] = *reinterpret_cast<const f32x4 *>(dm_states + st1 + c4);
+            ndM[it] = *reinterpret_cast<const uint2 *>(dm_snap + st1 + c4);
             if (HAS_S) {
                 nS0[it] = *reinterpret_cast<const f32x4 *>(s_states + st0 + c4);
-                ndS[it] = *reinterpret_cast<const f32x4 *>(ds_states + st1 + c4);
+                ndS[it] = *reinterpret_cast<const uint2 *>(ds_snap + st1 + c4);
             }
         }
         nvec = vecs[(size_t)task * kVecB + min(tid, 5 * CW - 1)];
@@ -208,39 +209,13 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per,
               task_hi = min(ntask, task_lo + per);
     if (task_lo >= task_hi) return;
-    // One load per 128-byte line of a task's inputs: 3 bf16 tiles of 64 lines, then 5 fp32 tiles of
-    // 128 lines; thread tid takes lines tid and tid + 512.
-    float touched0 = 0.f, touched1 = 0.f;
-    auto touch = [&](int task) {
-        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
-        const size_t tok = (size_t)chain * s + t0;
-        const size_t st0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, st1 = st0 + HD * HD;
-        auto line = [&](int ln) -> const void * {
-            if (ln < 192) {
-                const u16 *base = ln < 64 ? k : (ln < 128 ? q : v);
-                return base + (tok + min(ln & 63, L - 1)) * HD;
-            }
-            const int f = (ln - 192) >> 7, o = (ln - 192) & 127;   // line o of fp32 tile f: row o/2, half o%2
-            if (f == 0)
-                return d_y + dyr.offset(chain) + (size_t)(t0 + min(o >> 1, L - 1)) * dyr.row_stride + (o & 1) * 32;
-            const float *base = f == 1 ? m_states + st0 : (f == 2 ? (HAS_S ? s_states + st0 : m_states + st0)
-                                : (f == 3 ? dm_states + st1 : (HAS_S ? ds_states + st1 : dm_states + st1)));
-            return base + o * 32;
-        };
-        // Only the three bf16 token tiles (lines 0..191) are touched.  A compute unit's share of the XCD's
-        // L2 (128 KB) is smaller than a task's inputs (136 KB): touched fp32 lines were evicted before
-        // their use and fetched twice (measured: all 832 lines touched 341 us, none 320 us, the token
-        // tiles only 315 us).
-        if (tid < 192) touched0 = *reinterpret_cast<const float *>(line(tid));
-    };
     fetch_tab(task_lo);
+    fetch(task_lo);
 
     for (int task = task_lo; task < task_hi; task++) {
         const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
         const size_t tok = (size_t)chain * s + t0;
         // ── load and stage everything ──
-        asm volatile("" ::"v"(touched0), "v"(touched1));   // the touches of this task end here
-        fetch(task);
         {
             if (st_t >= L) { nK = make_uint4(0, 0, 0, 0); nQ = nK; nV = nK; }
             if (ft >= L) { ndY[0] = zero4(); ndY[1] = zero4(); }
@@ -253,15 +228,18 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 const int c4 = (fg0 + 8 * it) * 4, off = ft * LDB + c4;
                 bf16_store(dYr, off, ndY[it]);
                 split_store(M0h, M0l, off, nM0[it]);
-                bf16_store(dMr, off, ndM[it]);
+                *reinterpret_cast<uint2 *>(dMr + off) = ndM[it];
+                const f32x4 fdM = bf4_to_f32(ndM[it]);
+                f32x4 fdS = zero4();
                 if (HAS_S) {
-                    bf16_store(dSr, off, ndS[it]);
+                    *reinterpret_cast<uint2 *>(dSr + off) = ndS[it];
                     bf16_store(S0r, off, nS0[it]);
+                    fdS = bf4_to_f32(ndS[it]);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    d0 = fmaf(nM0[it][i], ndM[it][i], d0);
-                    if (HAS_S) { d1 = fmaf(nS0[it][i], ndM[it][i], d1); d2 = fmaf(nS0[it][i], ndS[it][i], d2); }
+                    d0 = fmaf(nM0[it][i], fdM[i], d0);
+                    if (HAS_S) { d1 = fmaf(nS0[it][i], fdM[i], d1); d2 = fmaf(nS0[it][i], fdS[i], d2); }
                 }
             }
             d0 = sum_wave(d0); d1 = sum_wave(d1); d2 = sum_wave(d2);
@@ -269,7 +247,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
             if (tid < 5 * CW) cvec[tid] = nvec;
         }
         __syncthreads();
-        touch(min(task + 1, task_hi - 1));
+        fetch(min(task + 1, task_hi - 1));
 
         // ── P, E^T (group A); dQ^T = a.(M0^T dY^T) + beta.(S0^T dY^T), p0, ps (group B) ──
         f32x4 keep[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};   // group A: P [t][j]; group B: dQ^T [c][t]
@@ -602,8 +580,8 @@ void chunkwise_backward_coefficients(const float *alpha, const float *theta, con
 }
 
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
-                          const float *m_states, const float *s_states, const float *dm_states,
-                          const float *ds_states, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
+                          const float *m_states, const float *s_states, const uint16_t *dm_snap,
+                          const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid, const HeadRows *dy_rows) {
     const ErrorScope es;
@@ -621,11 +599,11 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
     KernelTimer kt("cw_grads_bf16_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
-                           tab_a, tab_b, vecs, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec,
+                           tab_a, tab_b, vecs, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec,
                            xs, scal, seq_len, chunk_size, nc, ntask, dyr);
     else
         hipLaunchKernelGGL(cw_grads_bf16_kernel<false>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
-                           tab_a, tab_b, vecs, m_states, nullptr, dm_states, nullptr, d_k, d_v, d_q, d_theta, pvec,
+                           tab_a, tab_b, vecs, m_states, nullptr, dm_snap, nullptr, d_k, d_v, d_q, d_theta, pvec,
                            xs, scal, seq_len, chunk_size, nc, ntask, dyr);
     check_launch("cw_grads_bf16_kernel");
     return true;

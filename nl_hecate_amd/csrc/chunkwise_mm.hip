@@ -865,7 +865,10 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     const int nc = ceil_div(seq_len, chunk_size);
     Scratch sc{nullptr, nullptr};
     if constexpr (sizeof(TIn) == 4) sc = local_scratch(batch, nc);
-    const size_t st_bytes = (size_t)batch * (nc + 1) * HD * HD * sizeof(float);
+    // adjoint snapshots: fp32 [batch][nc + 1][d*d] on the fp32 path; on the bf16 path the same slots hold bf16
+    // snapshots followed by the fp32 gradient of the initial state [batch][d*d]
+    const size_t n_snap = (size_t)batch * (nc + 1) * HD * HD, n_first = (size_t)batch * HD * HD;
+    const size_t st_bytes = sizeof(TIn) == 2 ? n_snap * sizeof(uint16_t) + n_first * sizeof(float) : n_snap * sizeof(float);
     float *dm_states = scratch(5, st_bytes);
     float *ds_states = scratch(6, st_bytes);
     float *xs = scratch(7, (size_t)batch * nc * CW * CW * sizeof(float));
@@ -888,9 +891,10 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
         if (es.failed()) return;
         chunkwise_backward_coefficients(alpha, theta, eta, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s);
-        chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_states, ds_states, seq_len, batch, chunk_size, has_s,
-                               dy_rows);
-        chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta, pvec, xs,
+        uint16_t *dm_snap = reinterpret_cast<uint16_t *>(dm_states), *ds_snap = reinterpret_cast<uint16_t *>(ds_states);
+        chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_snap, ds_snap, reinterpret_cast<float *>(dm_snap + n_snap),
+                               reinterpret_cast<float *>(ds_snap + n_snap), seq_len, batch, chunk_size, has_s, dy_rows);
+        chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec, xs,
                              scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
                              persistent_grid(batch * nc), dy_rows);
     } else {
@@ -911,15 +915,20 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         check_launch("cw_grads_bwd_kernel");
     }
     chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s);
-    const size_t chain_stride = (size_t)(nc + 1) * HD * HD;
+    const bool packed = sizeof(TIn) == 2;   // where the gradient of the initial state sits (see above)
+    const size_t chain_stride = packed ? (size_t)HD * HD : (size_t)(nc + 1) * HD * HD;
+    const float *dm_first = packed ? reinterpret_cast<const float *>(reinterpret_cast<const uint16_t *>(dm_states) + n_snap)
+                                   : dm_states;
+    const float *ds_first = packed ? reinterpret_cast<const float *>(reinterpret_cast<const uint16_t *>(ds_states) + n_snap)
+                                   : ds_states;
     const int per = 8, rows = ceil_div(batch, per);
     const int nsum = has_s && d_s_initial ? 2 : 1;
     float *tmp = scratch(10, (size_t)nsum * rows * HD * HD * sizeof(float));
     if (es.failed()) return;
     {
         KernelTimer kt("cw_sum_slot0_kernel");
-        hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows, nsum), dim3(256), 0, stream(), dm_states,
-                           ds_states, tmp, batch, per, chain_stride);
+        hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows, nsum), dim3(256), 0, stream(), dm_first,
+                           ds_first, tmp, batch, per, chain_stride);
     }
     check_launch("cw_sum_slot0_kernel");
     KernelTimer kt("cw_add_rows_kernel");
