@@ -1,6 +1,6 @@
 // Backward of the chunkwise rule on bf16 tokens (head size 64, chunks of up to 64 tokens), three
 // launches on the library's stream:
-//   chunkwise_backward_coefficients: per-chunk coefficient tables tab_a, tab_b (table_floats per
+//   chunkwise_backward_coefficients: per-chunk coefficient table tab_b (table_floats per
 //     chunk) and vectors vecs (vec_floats per chunk) from the gates
 //   chunkwise_adjoint_bf16: the adjoint scan; dm_snap / ds_snap [batch][num_chunks + 1][64*64] in bf16,
 //     slot c = adjoint of the state at the start of chunk c as the gradient pass takes it (one bf16
@@ -21,7 +21,7 @@ namespace nlh {
 size_t chunkwise_grads_table_floats();
 size_t chunkwise_grads_vec_floats();
 
-void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta, float *tab_a,
+void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta,
                                      float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s);
 
 bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d_y, const float *tab_b,
@@ -32,7 +32,7 @@ bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
                           const float *m_states, const float *s_states, const uint16_t *dm_snap,
                           const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
-                          float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
+                          float *xs, float *scal, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid,
                           const HeadRows *dy_rows = nullptr);
 

@@ -38,26 +38,24 @@ namespace nlh {
 namespace {
 
 // Per-chunk coefficients in HBM, written by cw_coef_bwd_kernel:
-//   tab_a [chunk][block bi][rt][ct][lane l][r]: c[t][j] (zero outside j <= t < L) at
-//         j = 32 (bi/2) + 16 rt + 4 (l/16) + r, t = 32 (bi%2) + 16 ct + l%16   (group B: R^T)
-//   tab_b same for t = 32 (bi/2) + 16 rt + 4 (l/16) + r, j = 32 (bi%2) + 16 ct + l%16  (group A: P, R)
+//   tab_b [chunk][block bi][rt][ct][lane l][r]: c[t][j] (zero outside j <= t < L) at
+//         t = 32 (bi/2) + 16 rt + 4 (l/16) + r, j = 32 (bi%2) + 16 ct + l%16  (the order in which group A holds P, R)
 //   vecs  [chunk][kVecB]: a_t, beta_t, cl_j, bl_j, theta_j, then four zeros and h_L
 // Tiles entirely above the diagonal are neither written nor read.
 constexpr int kTab = CW * CW;
 constexpr int kVecB = 5 * CW + 16;
-__device__ __forceinline__ bool live_a(int bi, int rt, int ct) { return 2 * (bi & 1) + ct >= 2 * (bi >> 1) + rt; }
+constexpr int kCtLd = CW + 4;   // row stride (floats) of the coefficient copy in LDS
 __device__ __forceinline__ bool live_b(int bi, int rt, int ct) { return 2 * (bi >> 1) + rt >= 2 * (bi & 1) + ct; }
 
 template <bool HAS_S>
 __global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restrict__ alpha,
                                                           const float *__restrict__ theta,
-                                                          const float *__restrict__ eta, float *__restrict__ tab_a,
+                                                          const float *__restrict__ eta,
                                                           float *__restrict__ tab_b, float *__restrict__ vecs,
                                                           int s, int C, int nc, int nchunks) {
-    // One chunk per workgroup of two waves.  tab_a is assembled in LDS and leaves as 16-byte stores of
-    // consecutive lanes; tab_b holds the same numbers in the other tile orientation and is gathered from
-    // the same LDS copy on the way out (one table of LDS instead of two: twice the workgroups per CU for a
-    // kernel that is one serial 64-step loop per chunk).
+    // One chunk per workgroup of two waves.  The loop's lanes own columns j, the consumers' lanes own tokens t:
+    // the table is assembled in LDS in the loop's order and gathered in the consumers' order on the way out, as
+    // 16-byte stores of consecutive lanes.
     __shared__ __align__(16) float stage[kTab];
     const int chunk = blockIdx.x, role = threadIdx.x >> 6, j = threadIdx.x & 63;
     const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
@@ -101,13 +99,12 @@ __global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restric
         if (j == L - 1) vo[5 * CW + 4] = kh;
     }
     __syncthreads();
-    float *oa = tab_a + (size_t)chunk * kTab, *ob = tab_b + (size_t)chunk * kTab;
+    float *ob = tab_b + (size_t)chunk * kTab;
     for (int qd = threadIdx.x; qd < kTab / 4; qd += 128) {
         const int tile = qd >> 6, bi = tile >> 2, rt = (tile >> 1) & 1, ct = tile & 1;
-        if (live_a(bi, rt, ct)) *reinterpret_cast<f32x4 *>(oa + qd * 4) = *reinterpret_cast<const f32x4 *>(stage + qd * 4);
         if (live_b(bi, rt, ct)) {
             // element X = 4 qd + r of tab_b is c[t][j] with t = 32 X[11] + 16 X[9] + 4 X[7:6] + r, j = 32 X[10] +
-            // 16 X[8] + X[5:2]; in tab_a that pair sits at the index below, consecutive t four floats apart
+            // 16 X[8] + X[5:2]; in the staged copy that pair sits at the index below, consecutive t four floats apart
             const int X = qd * 4;
             const int jl = (X >> 2) & 15, a0 = ((X >> 10) & 1) * 2048 + ((X >> 11) & 1) * 1024 + ((X >> 8) & 1) * 512 +
                                               ((X >> 9) & 1) * 256 + (jl >> 2) * 64 + ((X >> 6) & 3) * 16 + (jl & 3);
@@ -136,7 +133,7 @@ __device__ __forceinline__ f32x4 bf4_to_f32(const u16 *p) { return bf4_to_f32(*r
 template <bool HAS_S>
 __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q, const float *__restrict__ d_y,
-    const float *__restrict__ tab_a, const float *__restrict__ tab_b, const float *__restrict__ vecs,
+    const float *__restrict__ tab_b, const float *__restrict__ vecs,
     const float *__restrict__ m_states, const float *__restrict__ s_states, const u16 *__restrict__ dm_snap,
     const u16 *__restrict__ ds_snap, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
@@ -154,6 +151,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     float *cvec = reinterpret_cast<float *>(CRt + BMAT);             // a, beta, cl, bl, theta [64] each
     float *part = cvec + 5 * CW;                                     // [5][2][64]: p0, ps, rt, g1, g2 per half
     float *dots = part + 5 * 2 * CW;                                 // [3][8]
+    float *Ctj = dots + 24;                                          // c [t][j], row stride kCtLd: group A -> group B
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, g = l >> 4, r16 = l & 15;
     const bool grpA = w < 4;
@@ -191,18 +189,19 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
         }
         nvec = vecs[(size_t)task * kVecB + min(tid, 5 * CW - 1)];
     };
-    // the coefficient table of a task is requested separately, once the previous one has been used
+    // The coefficient table of a task is requested separately, once the previous one has been used, by group A
+    // only: group B wants the same numbers with the roles of t and j exchanged and takes them from the copy that
+    // group A leaves in LDS.
     auto fetch_tab = [&](int task) {
+        if (!grpA) return;
         const float *zero = vecs + (size_t)task * kVecB + 5 * CW;
-        const float *tb = (grpA ? tab_b : tab_a) + (size_t)task * kTab;
+        const float *tb = tab_b + (size_t)task * kTab;
 #pragma unroll
         for (int rt = 0; rt < 2; rt++)
 #pragma unroll
-            for (int ct = 0; ct < 2; ct++) {
-                const bool live = grpA ? live_b(bi, rt, ct) : live_a(bi, rt, ct);
-                ntab[rt][ct] =
-                    *reinterpret_cast<const f32x4 *>(live ? tb + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4 : zero);
-            }
+            for (int ct = 0; ct < 2; ct++)
+                ntab[rt][ct] = *reinterpret_cast<const f32x4 *>(
+                    live_b(bi, rt, ct) ? tb + (((bi * 2 + rt) * 2 + ct) * 64 + l) * 4 : zero);
     };
 
     // contiguous task range per workgroup: consecutive chunks of a chain share pages and cache lines
@@ -245,6 +244,15 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
             d0 = sum_wave(d0); d1 = sum_wave(d1); d2 = sum_wave(d2);
             if (l == 0) { dots[w] = d0; dots[8 + w] = d1; dots[16 + w] = d2; }
             if (tid < 5 * CW) cvec[tid] = nvec;
+            if (grpA) {   // c[t .. t+3][j] of this wave's block
+#pragma unroll
+                for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            Ctj[(bm + 16 * rt + 4 * g + r) * kCtLd + bn + 16 * ct + r16] = ntab[rt][ct][r];
+            }
         }
         __syncthreads();
         fetch(min(task + 1, task_hi - 1));
@@ -368,9 +376,11 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int rt = 0; rt < 2; rt++) {
                     const f32x4 th = *reinterpret_cast<const f32x4 *>(cvec + 4 * CW + bm + 16 * rt + 4 * g);
 #pragma unroll
-                    for (int ct = 0; ct < 2; ct++)   // [t][j .. j+3]
-                        bf16_store(ThCR, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g,
-                                   -(th * ntab[rt][ct] * rr[rt][ct]));
+                    for (int ct = 0; ct < 2; ct++) {   // [t][j .. j+3]
+                        const f32x4 c4 = *reinterpret_cast<const f32x4 *>(Ctj + (bn + 16 * ct + r16) * kCtLd + bm +
+                                                                          16 * rt + 4 * g);
+                        bf16_store(ThCR, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g, -(th * c4 * rr[rt][ct]));
+                    }
                 }
             }
         }
@@ -559,30 +569,30 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     }
 }
 
-constexpr size_t kGradsLds = 11 * BMAT * sizeof(u16) + (5 * CW + 10 * CW + 24) * sizeof(float);
+constexpr size_t kGradsLds = 11 * BMAT * sizeof(u16) + (5 * CW + 10 * CW + 24 + CW * kCtLd) * sizeof(float);
 
 }  // namespace
 
 size_t chunkwise_grads_table_floats() { return kTab; }
 size_t chunkwise_grads_vec_floats() { return kVecB; }
 
-void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta, float *tab_a,
+void chunkwise_backward_coefficients(const float *alpha, const float *theta, const float *eta,
                                      float *tab_b, float *vecs, int seq_len, int batch, int chunk_size, bool has_s) {
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     KernelTimer kt("cw_coef_bwd_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
-                           eta, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
+                           eta, tab_b, vecs, seq_len, chunk_size, nc, ntask);
     else
         hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
-                           nullptr, tab_a, tab_b, vecs, seq_len, chunk_size, nc, ntask);
+                           nullptr, tab_b, vecs, seq_len, chunk_size, nc, ntask);
     check_launch("cw_coef_bwd_kernel");
 }
 
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
                           const float *m_states, const float *s_states, const uint16_t *dm_snap,
                           const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
-                          float *xs, float *scal, const float *tab_a, const float *tab_b, const float *vecs,
+                          float *xs, float *scal, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid, const HeadRows *dy_rows) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
@@ -599,11 +609,11 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
     KernelTimer kt("cw_grads_bf16_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
-                           tab_a, tab_b, vecs, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec,
+                           tab_b, vecs, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec,
                            xs, scal, seq_len, chunk_size, nc, ntask, dyr);
     else
         hipLaunchKernelGGL(cw_grads_bf16_kernel<false>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
-                           tab_a, tab_b, vecs, m_states, nullptr, dm_snap, nullptr, d_k, d_v, d_q, d_theta, pvec,
+                           tab_b, vecs, m_states, nullptr, dm_snap, nullptr, d_k, d_v, d_q, d_theta, pvec,
                            xs, scal, seq_len, chunk_size, nc, ntask, dyr);
     check_launch("cw_grads_bf16_kernel");
     return true;

@@ -886,16 +886,15 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     if constexpr (sizeof(TIn) == 2) {
         // bf16 tokens: coefficient pre-pass, adjoint scan and per-chunk gradients on the bf16 matrix cores
         const size_t nchunks = (size_t)batch * nc;
-        float *tab_a = scratch(12, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *tab_b = scratch(13, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
         if (es.failed()) return;
-        chunkwise_backward_coefficients(alpha, theta, eta, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s);
+        chunkwise_backward_coefficients(alpha, theta, eta, tab_b, vecs, seq_len, batch, chunk_size, has_s);
         uint16_t *dm_snap = reinterpret_cast<uint16_t *>(dm_states), *ds_snap = reinterpret_cast<uint16_t *>(ds_states);
         chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_snap, ds_snap, reinterpret_cast<float *>(dm_snap + n_snap),
                                reinterpret_cast<float *>(ds_snap + n_snap), seq_len, batch, chunk_size, has_s, dy_rows);
         chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec, xs,
-                             scal, tab_a, tab_b, vecs, seq_len, batch, chunk_size, has_s,
+                             scal, tab_b, vecs, seq_len, batch, chunk_size, has_s,
                              persistent_grid(batch * nc), dy_rows);
     } else {
         hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
