@@ -64,14 +64,14 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
     float pum = um, pvm = vm, pvs = vs;    // their values at s = lane - 1
     U[lane] = u;
     if (HAS_S) V[lane] = v;
-    constexpr int PF = GW;                 // the whole column of per-token terms is requested up front
-    float xr[PF];
+    // The whole column of per-token terms is requested up front.  Row s is used at t >= s only, and the
+    // producer leaves out the 16 x 16 tiles that lie entirely below that: those are neither read nor used.
+    float xr[GW];
 #pragma unroll
-    for (int i = 0; i < PF; i++) xr[i] = x[i * GW];
+    for (int i = 0; i < GW; i++) xr[i] = (lane >> 4) >= (i >> 4) ? x[i * GW] : 0.f;
 #pragma unroll
     for (int sx = 0; sx < GW; sx++) {
-        const float xv = xr[sx % PF];
-        if (sx + PF < GW) xr[sx % PF] = x[(sx + PF) * GW];
+        const float xv = xr[sx];
         const float kp = bcast(keep_l, sx), g1 = bcast(pv.z, sx);
         if (HAS_S) {
             const float et = bcast(eta_l, sx), g2 = bcast(pv.w, sx);

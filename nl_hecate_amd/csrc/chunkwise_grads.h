@@ -8,7 +8,8 @@
 //     gradient of the initial state
 //   chunkwise_grads_bf16: d_q, d_k, d_v, d_theta, and for the gate pass
 //     pvec [token][4] = p0_t = dy_t^T M0 q_t, ps_t = dy_t^T S0 q_t, -theta_t e_t^T dMo k_t, -theta_t e_t^T dSo k_t
-//     xs [chunk][j][t] = -theta_j (dy_t . e_j)(q_t . k_j)      scal [chunk][4] = <M0,dMo>, <S0,dMo>, <S0,dSo>
+//     xs [chunk][j][t] = -theta_j (dy_t . e_j)(q_t . k_j) (16 x 16 tiles with every t < j are not written)
+//     scal [chunk][4] = <M0,dMo>, <S0,dMo>, <S0,dSo>
 //   chunkwise_gate_gradients: d_alpha, d_eta from those (chunkwise_gates.hip; also serves the fp32 path)
 #pragma once
 #include <stddef.h>

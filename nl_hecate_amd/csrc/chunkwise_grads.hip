@@ -366,8 +366,9 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
 #pragma unroll
                     for (int ct = 0; ct < 2; ct++) {
                         const int off = (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g;   // [j][t .. t+3]
-                        *reinterpret_cast<f32x4 *>(xo + (bn + 16 * ct + r16) * CW + bm + 16 * rt + 4 * g) =
-                            -cvec[4 * CW + bn + 16 * ct + r16] * (rr[rt][ct] * keep[rt][ct]);
+                        if (live_b(bi, rt, ct))   // tiles with every t < j are never read
+                            *reinterpret_cast<f32x4 *>(xo + (bn + 16 * ct + r16) * CW + bm + 16 * rt + 4 * g) =
+                                -cvec[4 * CW + bn + 16 * ct + r16] * (rr[rt][ct] * keep[rt][ct]);
                         bf16_store(CPt, off, ntab[rt][ct] * keep[rt][ct]);
                         bf16_store(CRt, off, ntab[rt][ct] * rr[rt][ct]);
                     }
