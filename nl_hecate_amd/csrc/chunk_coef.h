@@ -203,5 +203,76 @@ __device__ __forceinline__ cf32x4 coef_tile_jt(const ChunkCoef &cc, int J, int T
     return out;
 }
 
+
+// ── Coefficient tables written to HBM by a pre-pass (one wave per chunk) ──
+// The vectors of a chunk from two scans of composed maps instead of 64-step loops:
+//   a, beta, h = R, X, H of G(0..t);  cl, bl = R + X, H of G(t+1..63)   (tokens beyond L: identity map)
+struct ChunkVectors { float a, beta, h, cl, bl; };
+__device__ __forceinline__ ChunkVectors coef_vectors(float keep, float et, bool in) {
+    const int t = threadIdx.x & 63;
+    const Map3 g = in ? Map3{keep, et, et} : map_identity();
+    Map3 hd = g;
+    hd = compose(hd, map_shr<1>(hd));
+    hd = compose(hd, map_shr<2>(hd));
+    hd = compose(hd, map_shr<4>(hd));
+    hd = compose(hd, map_shr<8>(hd));
+    Map3 sf = g;
+    sf = compose(map_shl<1>(sf), sf);
+    sf = compose(map_shl<2>(sf), sf);
+    sf = compose(map_shl<4>(sf), sf);
+    sf = compose(map_shl<8>(sf), sf);
+    const Map3 tl = map_shl<1>(sf);
+    Map3 blk[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+        blk[b] = Map3{coef_readlane(hd.R, 16 * b + 15), coef_readlane(hd.X, 16 * b + 15), coef_readlane(hd.H, 16 * b + 15)};
+    const Map3 pre1 = blk[0], pre2 = compose(blk[1], blk[0]), pre3 = compose(blk[2], pre2);
+    const Map3 post2 = blk[3], post1 = compose(blk[3], blk[2]), post0 = compose(post1, blk[1]);
+    const int T = t >> 4;
+    const Map3 pre = T == 0 ? map_identity() : (T == 1 ? pre1 : (T == 2 ? pre2 : pre3));
+    const Map3 post = T == 3 ? map_identity() : (T == 2 ? post2 : (T == 1 ? post1 : post0));
+    const Map3 pf = compose(hd, pre), sx = compose(post, tl);
+    return ChunkVectors{pf.R, pf.X, pf.H, sx.R + sx.X, sx.H};
+}
+
+// stage[t * LD + j] = scale_j c[t][j] for j <= t < L and zero elsewhere (64 rows of LD floats, LD a multiple of 4,
+// and one spare row behind them).
+// One wave, lane = j.  Lane j walks t = j, j + 1, .. on its own: at step i every lane multiplies (no lane waits
+// for its column to start), the gates of token j + i come from LDS (gk, ge: 128 floats each, identity from 64
+// on) at an immediate offset, and the destination is base + i * LD.  A step is two multiply-adds and a store
+// per lane, against a dozen instructions when the lanes advance through t together.
+template <int LD, bool SCALED>
+__device__ __forceinline__ void coef_table_columns(float *stage, float *gk, float *ge, float keep, float et,
+                                                   float scale, int L) {
+    const int j = threadIdx.x & 63;
+    gk[j] = keep; gk[64 + j] = 1.f;   // the caller passes keep = 1, eta = 0 beyond L
+    ge[j] = et;   ge[64 + j] = 0.f;
+    for (int e = j; e < 64 * LD / 4; e += 64) reinterpret_cast<cf32x4 *>(stage)[e] = cf32x4{0.f, 0.f, 0.f, 0.f};
+    // the gates of tokens j + 1 .. j + 63 in registers (requested in one go: no step waits for LDS), and every
+    // lane stores at every step (a lane whose column has ended stores to a spare row): no branch inside the walk
+    float kk[64], ee[64];
+#pragma unroll
+    for (int i = 1; i < 64; i++) { kk[i] = gk[j + i]; ee[i] = ge[j + i]; }
+    float b = 1.f, c = 1.f;
+    float *dst = stage + j * (LD + 1), *spare = stage + 64 * LD + j;
+    const bool jv = j < L;
+    dst[0] = jv ? (SCALED ? scale : 1.f) : 0.f;
+    if (L == 64) {
+#pragma unroll
+        for (int i = 1; i < 64; i++) {
+            b *= ee[i];
+            c = fmaf(kk[i], c, b);
+            *(j < 64 - i ? dst + i * LD : spare) = SCALED ? scale * c : c;
+        }
+    } else {
+#pragma unroll
+        for (int i = 1; i < 64; i++) {
+            b *= ee[i];
+            c = fmaf(kk[i], c, b);
+            *(j < 64 - i ? dst + i * LD : spare) = (jv && j < L - i) ? (SCALED ? scale * c : c) : 0.f;
+        }
+    }
+}
+
 }  // namespace
 }  // namespace nlh

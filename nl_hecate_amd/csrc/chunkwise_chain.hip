@@ -23,6 +23,7 @@
 #include <stdint.h>
 
 #include "bf16_tiles.h"
+#include "chunk_coef.h"
 #include "chunkwise_chain.h"
 #include "runtime.h"
 
@@ -45,67 +46,53 @@ constexpr int kChainThr = 512;     // 8 waves
 //         then a_L, beta_L, h_L, one unused float and four zeros
 constexpr int kTableFloats = CW * CW;
 constexpr int kVecFloats = 4 * CW + 16;
+constexpr int kStageLd = CW + 4;   // row stride (floats) of the table while it is assembled in LDS
+constexpr int kCoefChunksPerWave = 4;
 __device__ __forceinline__ bool tile_live(int bi, int rt, int ct) { return 2 * (bi & 1) + ct >= 2 * (bi >> 1) + rt; }
 
-// Coefficients of one chunk from its gates: two waves per chunk.  Wave role 0 (lane j): the
-// column recurrences c[t][j], bb[j][t] over t.  Role 1 (lane t): a_t, beta_t, h_t.
+// Coefficients of one chunk from its gates: one wave per chunk, lane = token.  The vectors come from two scans
+// of composed maps, the table from coef_table_columns; it is assembled in LDS as W[t][j] and leaves in the
+// consumers' order as 16-byte stores of consecutive lanes.
 template <bool HAS_S>
-__global__ __launch_bounds__(256) void cw_coef_kernel(const float *__restrict__ alpha,
-                                                      const float *__restrict__ theta,
-                                                      const float *__restrict__ eta, float *__restrict__ table,
-                                                      float *__restrict__ vecs, int s, int C, int nc, int nchunks) {
-    // The table is assembled in LDS and leaves as 16-byte stores of consecutive lanes.
-    __shared__ __align__(16) float stage[2][kTableFloats];
-    const int chunk = min(blockIdx.x * 2 + (int)(threadIdx.x >> 7), nchunks - 1);   // an odd tail is done twice
-    const int role = (threadIdx.x >> 6) & 1, j = threadIdx.x & 63;
-    const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
-    const Gates g = fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, L);
-    const float keep_j = 1.f - g.al;   // 1 beyond L
-    const float eta_j = g.et;          // 0 beyond L
-    float *vo = vecs + (size_t)chunk * kVecFloats;
-    if (role == 0) {
-        float *to = stage[threadIdx.x >> 7];
-        float b = 1.f, cc = 1.f, blv = 0.f;
+__global__ __launch_bounds__(64) void cw_coef_kernel(const float *__restrict__ alpha,
+                                                     const float *__restrict__ theta,
+                                                     const float *__restrict__ eta, float *__restrict__ table,
+                                                     float *__restrict__ vecs, int s, int C, int nc, int nchunks) {
+    __shared__ __align__(16) float stage[(CW + 1) * kStageLd];
+    __shared__ float gk[2 * CW], ge[2 * CW];
+    const int j = threadIdx.x, first = blockIdx.x * kCoefChunksPerWave, last = min(nchunks, first + kCoefChunksPerWave);
+    auto gates_of = [&](int chunk) {
+        const int chain = chunk / nc, t0 = (chunk % nc) * C;
+        return fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, min(C, s - t0));
+    };
+    // a wave walks over a few chunks with the next chunk's gates in flight: a wave per chunk would spend most of
+    // its life waiting for its three loads, and LDS allows only eight waves per compute unit
+    Gates gn = gates_of(first);
+    for (int chunk = first; chunk < last; chunk++) {
+        const int L = min(C, s - (chunk % nc) * C);
+        const Gates g = gn;
+        gn = gates_of(min(chunk + 1, last - 1));
         const bool jv = j < L;
-        const float nth = -g.th;
-        // destination of W[t][j]: block 2 (j/32) + t/32, rt = (j/16)%2, ct = (t/16)%2,
-        // lane 16 ((j%16)/4) + t%16, element j%4
-        const int jbase = (j >> 5) * 2048 + ((j >> 4) & 1) * 512 + ((j & 15) >> 2) * 64 + (j & 3);
-#pragma unroll
-        for (int t = 0; t < CW; t++) {
-            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
-            const bool after = t > j;
-            b *= after ? et : 1.f;
-            cc = after ? fmaf(keep, cc, b) : cc;
-            blv = (t == L - 1) ? b : blv;
-            if ((t >> 4) >= (j >> 4))
-                to[jbase + (t >> 5) * 1024 + ((t >> 4) & 1) * 256 + (t & 15) * 4] =
-                    (jv && t >= j && t < L) ? nth * cc : 0.f;
-        }
-        vo[2 * CW + j] = jv ? nth * cc : 0.f;
-        vo[3 * CW + j] = jv ? nth * blv : 0.f;
-    } else {
-        float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f, kh = 0.f;
-#pragma unroll
-        for (int t = 0; t < CW; t++) {
-            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
-            a *= keep;
-            h *= et;
-            beta = fmaf(keep, beta, h);
-            if (t == j) { ka = a; kb = beta; kh = h; }
-        }
-        vo[j] = j < L ? ka : 0.f;
-        vo[CW + j] = j < L ? kb : 0.f;
-        if (j == L - 1) { vo[4 * CW] = ka; vo[4 * CW + 1] = kb; vo[4 * CW + 2] = kh; }
+        const float keep = 1.f - g.al, et = g.et, nth = -g.th;   // 1, 0, 0 beyond L
+        const ChunkVectors cv = coef_vectors(keep, et, jv);
+        float *vo = vecs + (size_t)chunk * kVecFloats;
+        vo[j] = jv ? cv.a : 0.f;
+        vo[CW + j] = jv ? cv.beta : 0.f;
+        vo[2 * CW + j] = nth * cv.cl;
+        vo[3 * CW + j] = nth * cv.bl;
+        if (j == 63) { vo[4 * CW] = cv.a; vo[4 * CW + 1] = cv.beta; vo[4 * CW + 2] = cv.h; }   // the values at token L - 1
         if (j < 4) vo[4 * CW + 4 + j] = 0.f;   // zero pad: what tiles of W above the diagonal read
-    }
-    __syncthreads();
-    const float *from = stage[threadIdx.x >> 7];
-    float *out = table + (size_t)chunk * kTableFloats;
-    for (int qd = threadIdx.x & 127; qd < kTableFloats / 4; qd += 128) {
-        const int tile = qd >> 6;   // (bi, rt, ct) = (tile / 4, tile / 2 % 2, tile % 2)
-        if (tile_live(tile >> 2, (tile >> 1) & 1, tile & 1))
-            *reinterpret_cast<f32x4 *>(out + qd * 4) = *reinterpret_cast<const f32x4 *>(from + qd * 4);
+        coef_table_columns<kStageLd, true>(stage, gk, ge, keep, et, nth, L);
+        float *out = table + (size_t)chunk * kTableFloats;
+        // the ten 16 x 16 tiles on or below the diagonal (token tile T >= column tile J), one 16-byte piece per lane each
+#pragma unroll
+        for (int T = 0; T < 4; T++)
+#pragma unroll
+            for (int J = 0; J <= T; J++) {
+                const int tile = ((J >> 1) * 2 + (T >> 1)) * 4 + (J & 1) * 2 + (T & 1);   // (bi, rt, ct) of the layout above
+                *reinterpret_cast<f32x4 *>(out + (tile * 64 + j) * 4) =
+                    *reinterpret_cast<const f32x4 *>(stage + (16 * T + (j & 15)) * kStageLd + 16 * J + 4 * (j >> 4));
+            }
     }
 }
 
@@ -402,7 +389,7 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
     if (es.failed()) return;
     {
         KernelTimer kt("cw_coef_kernel");
-        hipLaunchKernelGGL(cw_coef_kernel<HAS_S>, dim3(ceil_div(nchunks, 2)), dim3(256), 0, stream(), alpha, theta, eta,
+        hipLaunchKernelGGL(cw_coef_kernel<HAS_S>, dim3(ceil_div(nchunks, kCoefChunksPerWave)), dim3(64), 0, stream(), alpha, theta, eta,
                            table, vecs, seq_len, chunk_size, nc, nchunks);
     }
     check_launch("cw_coef_kernel");

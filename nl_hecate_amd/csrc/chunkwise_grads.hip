@@ -31,6 +31,7 @@
 #include <stdint.h>
 
 #include "bf16_tiles.h"
+#include "chunk_coef.h"
 #include "chunkwise_grads.h"
 #include "runtime.h"
 
@@ -45,71 +46,54 @@ namespace {
 constexpr int kTab = CW * CW;
 constexpr int kVecB = 5 * CW + 16;
 constexpr int kCtLd = CW + 4;   // row stride (floats) of the coefficient copy in LDS
+constexpr int kCoefChunksPerWave = 4;
 __device__ __forceinline__ bool live_b(int bi, int rt, int ct) { return 2 * (bi >> 1) + rt >= 2 * (bi & 1) + ct; }
 
+// One wave per chunk, lane = token: the vectors from two scans of composed maps, the table from
+// coef_table_columns, assembled in LDS as c[t][j] and gathered in the consumers' order on the way out, as
+// 16-byte stores of consecutive lanes.
 template <bool HAS_S>
-__global__ __launch_bounds__(128) void cw_coef_bwd_kernel(const float *__restrict__ alpha,
-                                                          const float *__restrict__ theta,
-                                                          const float *__restrict__ eta,
-                                                          float *__restrict__ tab_b, float *__restrict__ vecs,
-                                                          int s, int C, int nc, int nchunks) {
-    // One chunk per workgroup of two waves.  The loop's lanes own columns j, the consumers' lanes own tokens t:
-    // the table is assembled in LDS in the loop's order and gathered in the consumers' order on the way out, as
-    // 16-byte stores of consecutive lanes.
-    __shared__ __align__(16) float stage[kTab];
-    const int chunk = blockIdx.x, role = threadIdx.x >> 6, j = threadIdx.x & 63;
-    const int chain = chunk / nc, ci = chunk % nc, t0 = ci * C, L = min(C, s - t0);
-    const Gates g = fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, L);
-    const float keep_j = 1.f - g.al;   // 1 beyond L
-    const float eta_j = g.et;          // 0 beyond L
-    float *vo = vecs + (size_t)chunk * kVecB;
-    if (role == 0) {
-        float *ta = stage;
-        float b = 1.f, cc = 1.f, blv = 0.f;
+__global__ __launch_bounds__(64) void cw_coef_bwd_kernel(const float *__restrict__ alpha,
+                                                         const float *__restrict__ theta,
+                                                         const float *__restrict__ eta,
+                                                         float *__restrict__ tab_b, float *__restrict__ vecs,
+                                                         int s, int C, int nc, int nchunks) {
+    __shared__ __align__(16) float stage[(CW + 1) * kCtLd];
+    __shared__ float gk[2 * CW], ge[2 * CW];
+    const int j = threadIdx.x, first = blockIdx.x * kCoefChunksPerWave, last = min(nchunks, first + kCoefChunksPerWave);
+    auto gates_of = [&](int chunk) {
+        const int chain = chunk / nc, t0 = (chunk % nc) * C;
+        return fetch_gates<HAS_S>(alpha, theta, eta, (size_t)chain * s + t0, min(C, s - t0));
+    };
+    // a wave walks over a few chunks with the next chunk's gates in flight (a wave per chunk would spend most of
+    // its life waiting for its three loads, and LDS allows only eight waves per compute unit)
+    Gates gn = gates_of(first);
+    for (int chunk = first; chunk < last; chunk++) {
+        const int L = min(C, s - (chunk % nc) * C);
+        const Gates g = gn;
+        gn = gates_of(min(chunk + 1, last - 1));
         const bool jv = j < L;
-        const int ja = (j >> 5) * 2048 + ((j >> 4) & 1) * 512 + ((j & 15) >> 2) * 64 + (j & 3);
-#pragma unroll
-        for (int t = 0; t < CW; t++) {
-            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
-            const bool after = t > j;
-            b *= after ? et : 1.f;
-            cc = after ? fmaf(keep, cc, b) : cc;
-            blv = (t == L - 1) ? b : blv;
-            if ((t >> 4) >= (j >> 4)) {
-                const float x = (jv && t >= j && t < L) ? cc : 0.f;
-                ta[ja + (t >> 5) * 1024 + ((t >> 4) & 1) * 256 + (t & 15) * 4] = x;
-            }
-        }
-        vo[2 * CW + j] = jv ? cc : 0.f;
-        vo[3 * CW + j] = jv ? blv : 0.f;
+        const float keep = 1.f - g.al, et = g.et;   // 1, 0 beyond L
+        const ChunkVectors cv = coef_vectors(keep, et, jv);
+        float *vo = vecs + (size_t)chunk * kVecB;
+        vo[j] = jv ? cv.a : 0.f;
+        vo[CW + j] = jv ? cv.beta : 0.f;
+        vo[2 * CW + j] = jv ? cv.cl : 0.f;
+        vo[3 * CW + j] = jv ? cv.bl : 0.f;
         vo[4 * CW + j] = g.th;
-    } else {
-        float a = 1.f, h = 1.f, beta = 0.f, ka = 0.f, kb = 0.f, kh = 0.f;
-#pragma unroll
-        for (int t = 0; t < CW; t++) {
-            const float keep = lane_bcast(keep_j, t), et = lane_bcast(eta_j, t);
-            a *= keep;
-            h *= et;
-            beta = fmaf(keep, beta, h);
-            if (t == j) { ka = a; kb = beta; kh = h; }
-        }
-        vo[j] = j < L ? ka : 0.f;
-        vo[CW + j] = j < L ? kb : 0.f;
         if (j < 4) vo[5 * CW + j] = 0.f;   // what tiles above the diagonal read
-        if (j == L - 1) vo[5 * CW + 4] = kh;
-    }
-    __syncthreads();
-    float *ob = tab_b + (size_t)chunk * kTab;
-    for (int qd = threadIdx.x; qd < kTab / 4; qd += 128) {
-        const int tile = qd >> 6, bi = tile >> 2, rt = (tile >> 1) & 1, ct = tile & 1;
-        if (live_b(bi, rt, ct)) {
-            // element X = 4 qd + r of tab_b is c[t][j] with t = 32 X[11] + 16 X[9] + 4 X[7:6] + r, j = 32 X[10] +
-            // 16 X[8] + X[5:2]; in the staged copy that pair sits at the index below, consecutive t four floats apart
-            const int X = qd * 4;
-            const int jl = (X >> 2) & 15, a0 = ((X >> 10) & 1) * 2048 + ((X >> 11) & 1) * 1024 + ((X >> 8) & 1) * 512 +
-                                              ((X >> 9) & 1) * 256 + (jl >> 2) * 64 + ((X >> 6) & 3) * 16 + (jl & 3);
-            *reinterpret_cast<f32x4 *>(ob + X) = f32x4{stage[a0], stage[a0 + 4], stage[a0 + 8], stage[a0 + 12]};
-        }
+        if (j == 63) vo[5 * CW + 4] = cv.h;   // h at token L - 1
+        coef_table_columns<kCtLd, false>(stage, gk, ge, keep, et, 1.f, L);
+        float *ob = tab_b + (size_t)chunk * kTab;
+        // the ten 16 x 16 tiles on or below the diagonal (token tile T >= column tile J), one 16-byte piece per lane each
+#pragma unroll
+        for (int T = 0; T < 4; T++)
+#pragma unroll
+            for (int J = 0; J <= T; J++) {
+                const int tile = ((T >> 1) * 2 + (J >> 1)) * 4 + (T & 1) * 2 + (J & 1);   // (bi, rt, ct) of the layout above
+                const float *p = stage + (16 * T + 4 * (j >> 4)) * kCtLd + 16 * J + (j & 15);
+                *reinterpret_cast<f32x4 *>(ob + (tile * 64 + j) * 4) = f32x4{p[0], p[kCtLd], p[2 * kCtLd], p[3 * kCtLd]};
+            }
     }
 }
 
@@ -582,10 +566,10 @@ void chunkwise_backward_coefficients(const float *alpha, const float *theta, con
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     KernelTimer kt("cw_coef_bwd_kernel");
     if (has_s)
-        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<true>, dim3(ceil_div(ntask, kCoefChunksPerWave)), dim3(64), 0, stream(), alpha, theta,
                            eta, tab_b, vecs, seq_len, chunk_size, nc, ntask);
     else
-        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ntask), dim3(128), 0, stream(), alpha, theta,
+        hipLaunchKernelGGL(cw_coef_bwd_kernel<false>, dim3(ceil_div(ntask, kCoefChunksPerWave)), dim3(64), 0, stream(), alpha, theta,
                            nullptr, tab_b, vecs, seq_len, chunk_size, nc, ntask);
     check_launch("cw_coef_bwd_kernel");
 }
