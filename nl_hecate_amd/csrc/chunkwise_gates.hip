@@ -39,12 +39,34 @@ __device__ __forceinline__ float bcast(float x, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
 }
 
+// The launch carries a second, unrelated piece of the same backward in its last workgroups: the first stage of
+// the sum over the batch of the gradient of the initial state (it depends on the adjoint scan only, is far too
+// small for a launch of its own, and runs beside the sweeps): workgroup (e, y, z) adds `per` chains' matrices
+// z (0: M, 1: S), elements 256 e .. 256 e + 255, into tmp[z][y]; a second launch adds the rows of tmp in a fixed order.
+struct FirstSum {
+    const float *src[2];   // [batch][chain_stride]: gradient of the initial M / S per chain
+    float *tmp;            // [nsum][rows][d*d]
+    size_t chain_stride;
+    int batch, per, rows, nsum;
+};
+constexpr int kSumElems = 64 * 64;
+
 template <bool HAS_S>
 __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
     const float *__restrict__ alpha, const float *__restrict__ eta, const float *__restrict__ pvec,
     const float *__restrict__ xs, const float *__restrict__ scal, float *__restrict__ d_alpha,
-    float *__restrict__ d_eta, int s, int C, int nc, int ntask) {
+    float *__restrict__ d_eta, int s, int C, int nc, int ntask, int sweep_blocks, FirstSum fs) {
     extern __shared__ float smem[];
+    if ((int)blockIdx.x >= sweep_blocks) {
+        const int bid = blockIdx.x - sweep_blocks, eb = bid % (kSumElems / 256), y = (bid / (kSumElems / 256)) % fs.rows,
+                  z = bid / ((kSumElems / 256) * fs.rows);
+        const float *st = fs.src[z];
+        const int e = eb * 256 + threadIdx.x, b0 = y * fs.per, b1 = min(fs.batch, b0 + fs.per);
+        float x = 0.f;
+        for (int b = b0; b < b1; b++) x += st[(size_t)b * fs.chain_stride + e];
+        fs.tmp[((size_t)z * fs.rows + y) * kSumElems + e] = x;
+        return;
+    }
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int task = blockIdx.x * kGateWaves + wv;
     if (task >= ntask) return;   // no barrier below: waves are independent
@@ -123,7 +145,8 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
 
 void chunkwise_gate_gradients(const float *alpha, const float *eta, const float *pvec, const float *xs,
                               const float *scal, float *d_alpha, float *d_eta, int seq_len, int batch,
-                              int chunk_size, bool has_s) {
+                              int chunk_size, bool has_s, const float *dm_first, const float *ds_first,
+                              size_t chain_stride, int per, int nsum, float *tmp) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     const size_t lds = (size_t)kGateWaves * (has_s ? 2 : 1) * GTRI * sizeof(float);
@@ -138,14 +161,17 @@ void chunkwise_gate_gradients(const float *alpha, const float *eta, const float 
         attr_set = true;
     }
     if (es.failed()) return;
-    const dim3 grid(ceil_div(ntask, kGateWaves)), block(64 * kGateWaves);
+    static_assert(64 * kGateWaves == 256, "the sum workgroups take 256 elements each");
+    const int sweep_blocks = ceil_div(ntask, kGateWaves), rows = ceil_div(batch, per);
+    const FirstSum fs{{dm_first, ds_first}, tmp, chain_stride, batch, per, rows, nsum};
+    const dim3 grid(sweep_blocks + (kSumElems / 256) * rows * nsum), block(64 * kGateWaves);
     KernelTimer kt("cw_gates_sweep_kernel");
     if (has_s)
         hipLaunchKernelGGL(cw_gates_sweep_kernel<true>, grid, block, lds, stream(), alpha, eta, pvec, xs, scal, d_alpha,
-                           d_eta, seq_len, chunk_size, nc, ntask);
+                           d_eta, seq_len, chunk_size, nc, ntask, sweep_blocks, fs);
     else
         hipLaunchKernelGGL(cw_gates_sweep_kernel<false>, grid, block, lds, stream(), alpha, nullptr, pvec, xs, scal,
-                           d_alpha, nullptr, seq_len, chunk_size, nc, ntask);
+                           d_alpha, nullptr, seq_len, chunk_size, nc, ntask, sweep_blocks, fs);
     check_launch("cw_gates_sweep_kernel");
 }
 

@@ -37,8 +37,11 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           int seq_len, int batch, int chunk_size, bool has_s, int grid,
                           const HeadRows *dy_rows = nullptr);
 
+// also runs the first stage of the batch sum of the initial-state gradients: tmp [nsum][ceil(batch / per)][64*64]
+// receives the sums of `per` consecutive chains of dm_first (and ds_first when nsum = 2), [batch][chain_stride]
 void chunkwise_gate_gradients(const float *alpha, const float *eta, const float *pvec, const float *xs,
                               const float *scal, float *d_alpha, float *d_eta, int seq_len, int batch,
-                              int chunk_size, bool has_s);
+                              int chunk_size, bool has_s, const float *dm_first, const float *ds_first,
+                              size_t chain_stride, int per, int nsum, float *tmp);
 
 }  // namespace nlh

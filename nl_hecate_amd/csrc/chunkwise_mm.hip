@@ -765,14 +765,6 @@ constexpr size_t kGradsBwdLds = 9 * MAT * sizeof(float);
 // Sum over chains of st[chain][slot 0][.]: stage 1 sums `per` chains per block row into
 // tmp[which][rows][4096]; stage 2 adds the rows to dst (+=).  blockIdx.z = which: the M adjoint (0) and the S
 // adjoint (1) share the two launches.
-__global__ void cw_sum_slot0_kernel(const float *__restrict__ st0, const float *__restrict__ st1,
-                                    float *__restrict__ tmp, int batch, int per, size_t chain_stride) {
-    const float *st = blockIdx.z ? st1 : st0;
-    const int e = blockIdx.x * blockDim.x + threadIdx.x, b0 = blockIdx.y * per, b1 = min(batch, b0 + per);
-    float x = 0.f;
-    for (int b = b0; b < b1; b++) x += st[(size_t)b * chain_stride + e];
-    tmp[((size_t)blockIdx.z * gridDim.y + blockIdx.y) * HD * HD + e] = x;
-}
 __global__ void cw_add_rows_kernel(const float *__restrict__ tmp, float *__restrict__ dst0, float *__restrict__ dst1,
                                    int rows) {
     float *dst = blockIdx.z ? dst1 : dst0;
@@ -913,7 +905,6 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                            d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc);
         check_launch("cw_grads_bwd_kernel");
     }
-    chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s);
     const bool packed = sizeof(TIn) == 2;   // where the gradient of the initial state sits (see above)
     const size_t chain_stride = packed ? (size_t)HD * HD : (size_t)(nc + 1) * HD * HD;
     const float *dm_first = packed ? reinterpret_cast<const float *>(reinterpret_cast<const uint16_t *>(dm_states) + n_snap)
@@ -924,12 +915,9 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     const int nsum = has_s && d_s_initial ? 2 : 1;
     float *tmp = scratch(10, (size_t)nsum * rows * HD * HD * sizeof(float));
     if (es.failed()) return;
-    {
-        KernelTimer kt("cw_sum_slot0_kernel");
-        hipLaunchKernelGGL(cw_sum_slot0_kernel, dim3(HD * HD / 256, rows, nsum), dim3(256), 0, stream(), dm_first,
-                           ds_first, tmp, batch, per, chain_stride);
-    }
-    check_launch("cw_sum_slot0_kernel");
+    // d_alpha, d_eta, and in the same launch the first stage of the deterministic sum of d_m_initial, d_s_initial
+    chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s, dm_first,
+                             ds_first, chain_stride, per, nsum, tmp);
     KernelTimer kt("cw_add_rows_kernel");
     hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256, 1, nsum), dim3(256), 0, stream(), tmp, d_m_initial,
                        d_s_initial, rows);
