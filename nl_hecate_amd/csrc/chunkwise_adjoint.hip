@@ -115,26 +115,23 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     // fp32 master: transposed tile rows c = 16 (w/2) + 4 (l/16) + r, column i = 16 (w%2) + l%16
     const int rt = w >> 1, ct = w & 1;
     f32x4 dM = zero4(), dS = zero4();
-    // The snapshot a later pass reads is the bf16 value that this scan itself uses as the hi operand; the
-    // gradient of the initial state (slot 0) leaves in fp32.
+    // The snapshot a later pass reads is the bf16 value that this scan itself uses as the hi operand: it leaves
+    // from the LDS copy at the top of the next step, as whole 128-byte rows (from the accumulator layout a wave
+    // would store 32-byte pieces of 16 different lines).  The gradient of the initial state (slot 0) leaves in fp32.
     auto publish = [&](int slot) {
         const int e = (i0 + 16 * ct + r16) * HD + 16 * rt + 4 * g, off = (16 * ct + r16) * LDB + 16 * rt + 4 * g;
-        const size_t o = state0 + (size_t)slot * HD * HD + e;
-        auto one = [&](u16 *H, u16 *Lo, u16 *snap, float *first, const f32x4 &x) {
-            bf16x4 h, lo;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const __bf16 hb = (__bf16)x[i];
-                h[i] = hb;
-                lo[i] = (__bf16)(x[i] - (float)hb);
-            }
-            *reinterpret_cast<bf16x4 *>(H + off) = h;
-            *reinterpret_cast<bf16x4 *>(Lo + off) = lo;
-            if (slot) *reinterpret_cast<bf16x4 *>(snap + o) = h;
-            else *reinterpret_cast<f32x4 *>(first + (size_t)chain * HD * HD + e) = x;
-        };
-        one(dMh, dMl, dm_snap, dm_first, dM);
-        if (HAS_S) one(dSh, dSl, ds_snap, ds_first, dS);
+        split_store(dMh, dMl, off, dM);
+        if (HAS_S) split_store(dSh, dSl, off, dS);
+        if (slot == 0) {
+            *reinterpret_cast<f32x4 *>(dm_first + (size_t)chain * HD * HD + e) = dM;
+            if (HAS_S) *reinterpret_cast<f32x4 *>(ds_first + (size_t)chain * HD * HD + e) = dS;
+        }
+    };
+    auto store_snapshot = [&](int slot) {   // threads 0..255: a row piece of dMo, 256..511: of dSo
+        const int which = tid >> 8, row = (tid & 255) >> 3, c8 = (tid & 7) * 8;
+        if (which && !HAS_S) return;
+        const uint4 x = *reinterpret_cast<const uint4 *>((which ? dSh : dMh) + row * LDB + c8);
+        *reinterpret_cast<uint4 *>((which ? ds_snap : dm_snap) + state0 + (size_t)slot * HD * HD + (i0 + row) * HD + c8) = x;
     };
 
     fetch(nc - 1);
@@ -148,6 +145,7 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
         const float *cvec = cvecs + par * kCvec;
         const u16 *Kr = late + par * kLate, *Qr = Kr + BMAT;
         const u16 *dYah = Qr + BMAT, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
+        store_snapshot(c + 1);
         // ── (W.P)^T: this wave's two tiles of P[t][j] ──
         {
             const bf16x8 aq[2] = {ld_op(Qr, 16 * tt, 0), ld_op(Qr, 16 * tt, 1)};
