@@ -31,7 +31,7 @@ namespace nlh {
 namespace {
 
 constexpr int GW = 64;            // tokens per chunk tile
-constexpr int GTRI = GW * (GW + 1) / 2;   // floats of one packed triangle
+constexpr int GTRI = GW * (GW + 1) / 2 + GW;   // floats of one packed triangle, and a spare row behind it
 constexpr int kGateWaves = 4;     // chunks per workgroup, one wave each
 __host__ __device__ constexpr int tri_row(int r) { return GW * r - r * (r - 1) / 2; }
 
@@ -90,7 +90,13 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
     // producer leaves out the 16 x 16 tiles that lie entirely below that: those are neither read nor used.
     float xr[GW];
 #pragma unroll
-    for (int i = 0; i < GW; i++) xr[i] = (lane >> 4) >= (i >> 4) ? x[i * GW] : 0.f;
+    for (int i = 0; i < GW; i++) xr[i] = 0.f;
+#pragma unroll
+    for (int b = 0; b < GW / 16; b++)
+        if ((lane >> 4) >= b) {
+#pragma unroll
+            for (int i = 16 * b; i < 16 * b + 16; i++) xr[i] = x[i * GW];
+        }
 #pragma unroll
     for (int sx = 0; sx < GW; sx++) {
         const float xv = xr[sx];
@@ -107,10 +113,10 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
         u = fmaf(kp, u, v);
         um = fmaf(kp, um, vm);
         if (sx + 1 < GW) {
-            if (lane >= sx + 1) {   // row sx + 1, columns t >= sx + 1
-                U[tri_row(sx + 1) - (sx + 1) + lane] = u;
-                if (HAS_S) V[tri_row(sx + 1) - (sx + 1) + lane] = v;
-            }
+            // row sx + 1, columns t >= sx + 1; the other lanes store to the spare row (no branch in the sweep)
+            const int dst = lane >= sx + 1 ? tri_row(sx + 1) - (sx + 1) + lane : GTRI - GW + lane;
+            U[dst] = u;
+            if (HAS_S) V[dst] = v;
             if (lane == sx + 1) { pum = um; pvm = vm; pvs = vs; }
         }
     }
