@@ -27,7 +27,7 @@ namespace {
 constexpr int HMAT = 32 * LDB;   // elements of a 32-row bf16 matrix
 constexpr int DYS = 48;          // row stride of a [token][32 rows] bf16 matrix (read through ld_op_tr)
 constexpr int DYM = 64 * DYS;
-constexpr int kLate = 2 * BMAT + 4 * DYM;   // elements of one copy of the last phase's operands
+constexpr int kLate = 2 * BMAT + 6 * DYM;   // elements of one copy of a chunk's staged inputs
 constexpr int kCvec = 5 * CW + 8;
 
 template <bool HAS_S>
@@ -37,12 +37,11 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
     u16 *__restrict__ ds_snap, float *__restrict__ dm_first, float *__restrict__ ds_first, int s, int C, int nc, int batch, int tab_floats, int vec_floats, HeadRows dyr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *WPh = reinterpret_cast<u16 *>(smem_raw), *WPl = WPh + BMAT;   // (W.P)^T [j][t]
-    u16 *dYh = WPl + BMAT, *dYl = dYh + DYM;                           // dY [t][i] (this workgroup's 32 rows i)
-    u16 *dMh = dYl + DYM, *dMl = dMh + HMAT;                           // dMo [i][c]
+    u16 *dMh = WPl + BMAT, *dMl = dMh + HMAT;                          // dMo [i][c]
     u16 *dSh = dMl + HMAT, *dSl = dSh + HMAT;                          // dSo [i][c]
     u16 *dEh = dSl + HMAT, *dEl = dEh + HMAT;                          // dE^T [i][j]
-    // What the last phase of a step reads exists twice, so that the next step's copy is written while
-    // this step's is still in use: K [j][c], Q [t][c], a.dY hi / lo, beta.dY hi / lo [t][i], and the
+    // The staged inputs of a chunk exist twice, so that the next step's copy is written while this step's is
+    // still in use: K [j][c], Q [t][c], dY, a.dY, beta.dY hi / lo [t][i] (this workgroup's 32 rows i), and the
     // vectors a, beta, cl, bl, theta [64] each, .., h_L
     u16 *late = dEl + HMAT;
     float *cvecs = reinterpret_cast<float *>(late + 2 * kLate);
@@ -95,12 +94,12 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
         }
     };
     // Registers -> LDS, everything in the order it arrives (rows = tokens): the products that contract over
-    // tokens read their operands through ld_op_tr.  Called in the last phase of the step before: dY is no
-    // longer read there, and the rest goes to the copy that this step does not use.
+    // tokens read their operands through ld_op_tr.  Called during the step before, into the copy that step
+    // does not use.
     auto commit = [&](int c, int par) {
         const int L = min(C, s - c * C);
         u16 *Kr = late + par * kLate, *Qr = Kr + BMAT;
-        u16 *dYah = Qr + BMAT, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
+        u16 *dYh = Qr + BMAT, *dYl = dYh + DYM, *dYah = dYl + DYM, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
         if (st_t >= L) { nK = make_uint4(0, 0, 0, 0); nQ = nK; }
         if (yt >= L) ndY = zero4();
         *reinterpret_cast<uint4 *>(Kr + st_t * LDB + st_cb * 8) = nK;
@@ -134,35 +133,44 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
         *reinterpret_cast<uint4 *>((which ? ds_snap : dm_snap) + state0 + (size_t)slot * HD * HD + (i0 + row) * HD + c8) = x;
     };
 
+    // (W.P)^T of chunk c from its staged K, Q (copy par): this wave's two tiles of P[t][j].  It does not depend
+    // on the scan, so it is computed a step ahead, in the shadow of the step's last phase.
+    auto weights = [&](int par) {
+        const float *cvec = cvecs + par * kCvec;
+        const u16 *Kr = late + par * kLate, *Qr = Kr + BMAT;
+        const bf16x8 aq[2] = {ld_op(Qr, 16 * tt, 0), ld_op(Qr, 16 * tt, 1)};
+#pragma unroll
+        for (int x = 0; x < 2; x++) {
+            const int jt = jt0 + x;
+            if (jt <= tt) {
+                f32x4 p = zero4();
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) p = mfma32(aq[ks], ld_op(Kr, 16 * jt, ks), p);
+                const float nth = -cvec[4 * CW + 16 * jt + r16];
+                split_store(WPh, WPl, (16 * jt + r16) * LDB + 16 * tt + 4 * g, nth * ctab[x] * p);   // [j][t .. t+3]
+            }
+        }
+    };
+
+    // Two barriers per step.  First phase: the next chunk's inputs go to LDS (requested a step earlier), the ones
+    // after that are requested, dE.  Second phase: dM0, dS0, the next chunk's (W.P)^T, the new state to LDS.
     fetch(nc - 1);
     fetch_tab(nc - 1);
     publish(nc);
     commit(nc - 1, (nc - 1) & 1);
     fetch(max(nc - 2, 0));
     __syncthreads();
+    weights((nc - 1) & 1);
+    fetch_tab(max(nc - 2, 0));
+    __syncthreads();
     for (int c = nc - 1; c >= 0; c--) {
         const int L = min(C, s - c * C), par = c & 1;
         const float *cvec = cvecs + par * kCvec;
         const u16 *Kr = late + par * kLate, *Qr = Kr + BMAT;
-        const u16 *dYah = Qr + BMAT, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
+        const u16 *dYh = Qr + BMAT, *dYl = dYh + DYM, *dYah = dYl + DYM, *dYal = dYah + DYM, *dYbh = dYal + DYM, *dYbl = dYbh + DYM;
         store_snapshot(c + 1);
-        // ── (W.P)^T: this wave's two tiles of P[t][j] ──
-        {
-            const bf16x8 aq[2] = {ld_op(Qr, 16 * tt, 0), ld_op(Qr, 16 * tt, 1)};
-#pragma unroll
-            for (int x = 0; x < 2; x++) {
-                const int jt = jt0 + x;
-                if (jt <= tt) {
-                    f32x4 p = zero4();
-#pragma unroll
-                    for (int ks = 0; ks < 2; ks++) p = mfma32(aq[ks], ld_op(Kr, 16 * jt, ks), p);
-                    const float nth = -cvec[4 * CW + 16 * jt + r16];
-                    split_store(WPh, WPl, (16 * jt + r16) * LDB + 16 * tt + 4 * g, nth * ctab[x] * p);   // [j][t .. t+3]
-                }
-            }
-        }
-        fetch_tab(max(c - 1, 0));
-        __syncthreads();
+        commit(max(c - 1, 0), par ^ 1);
+        fetch(max(c - 2, 0));
         // ── dE[j][i]: tile rows j = 16 rt.., columns i = 16 ct.. ──
         {
             f32x4 e1 = zero4(), e2 = zero4(), e3 = zero4();
@@ -187,10 +195,6 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
             split_store(dEh, dEl, (16 * ct + r16) * LDB + j4, e1 - th * (cl * e2 + bl * e3));   // [i][j .. j+3]
         }
         __syncthreads();
-        // ── the inputs of the next step (chunk c - 1; chunk 0 once more after the last) go to LDS, those of
-        //    the one after are requested ──
-        commit(max(c - 1, 0), par ^ 1);
-        fetch(max(c - 2, 0));
         // ── dM0^T, dS0^T: tile rows c = 16 rt.., columns i = 16 ct.. ──
         {
             f32x4 am = zero4(), as = zero4();
@@ -212,11 +216,14 @@ __global__ __launch_bounds__(kTileThr) void cw_adjoint_chain_kernel(
             dM = dMn;
         }
         publish(c);
+        // (W.P)^T of the next step's chunk (staged during this step's first phase), then the tiles after it
+        weights(par ^ 1);
+        fetch_tab(max(c - 2, 0));
         __syncthreads();
     }
 }
 
-constexpr size_t kAdjointLds = (2 * BMAT + 2 * DYM + 6 * HMAT + 2 * kLate) * sizeof(u16) + 2 * kCvec * sizeof(float);
+constexpr size_t kAdjointLds = (2 * BMAT + 6 * HMAT + 2 * kLate) * sizeof(u16) + 2 * kCvec * sizeof(float);
 
 }  // namespace
 
