@@ -259,12 +259,12 @@ def setup_titans_chunkwise_c3(torch, D, lib):
         # each kernel's OWN compulsory bytes per head-token (what it must read and write given its role in
         # the split; intermediates between kernels count for both sides, so these do not add up to 3108):
         #   forward chain: the forward's 1164
-        #   adjoint scan: k, q 256 + dY 256 + gates 12 + adjoint snapshots 2 x 16384 / 64
-        #   gradients: k, v, q 384 + dY 256 + gates 12 + states 512 + adjoints 512 + d_k, d_v, d_q 768 + d_theta 4
-        #              + per-token terms for the gate pass 256 + 16
+        #   adjoint scan: k, q 256 + dY 256 + gates 12 + adjoint snapshots (bf16) 2 x 8192 / 64
+        #   gradients: k, v, q 384 + dY 256 + gates 12 + states 512 + adjoints (bf16) 256 + d_k, d_v, d_q 768
+        #              + d_theta 4 + per-token terms for the gate pass 256 + 16
         #   gate sweeps: those 256 + 16, gates 8, d_alpha, d_eta 8
-        kernel_work={"cw_chain_fwd_kernel": BYTES_CW_FWD, "cw_adjoint_chain_kernel": 1036,
-                     "cw_grads_bf16_kernel": 2720, "cw_gates_sweep_kernel": 288},
+        kernel_work={"cw_chain_fwd_kernel": BYTES_CW_FWD, "cw_adjoint_chain_kernel": 780,
+                     "cw_grads_bf16_kernel": 2464, "cw_gates_sweep_kernel": 288},
         kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
         cpu_all=lambda: cpu_all_cores(chain, B, s, heads, "chunkwise forward + backward"),
         config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
