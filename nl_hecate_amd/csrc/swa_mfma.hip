@@ -293,6 +293,160 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
     }
 }
 
+// Forward that keeps statistics instead of weights, in blocks of keys with a running maximum (no score
+// outlives its 64-key stage, so a lane holds 32 scores instead of 144 and four workgroups fit a compute unit
+// instead of two).  One workgroup per (128 queries, head, batch), one wave per 32 queries; per stage a wave
+// forms S^T = K Q^T for its two query tiles (32 matrix-core steps with the products of the second half, against
+// 8 per barrier in the kernel above), rescales O^T by exp2(old maximum - new maximum) and adds V^T P^T with the
+// unnormalised weights; the division by the sum happens once at the end.  K and V rows are staged as they
+// arrive; V^T is read through ds_read_b64_tr_b16: group g of a wave takes keys 32 hf + 4 g .. + 3 and
+// 32 hf + 16 + 4 g .. + 3, which are exactly the rows that the two score tiles of that half leave in its lanes.
+constexpr int FQ = 128;    // queries per workgroup
+constexpr int LDV = 80;    // row stride of the V stage (160 B: the transposing reads of a group fall on 32 banks)
+
+__device__ __forceinline__ uint4 ld_tr2(const unsigned short (*T)[LDV], int row_a, int row_b, int col0) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 *lds_ptr;
+    const int sl = threadIdx.x & 15;
+    const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)&T[row_a + (sl >> 2)][col0 + 4 * (sl & 3)]);
+    const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)&T[row_b + (sl >> 2)][col0 + 4 * (sl & 3)]);
+    const uint2 ua = __builtin_bit_cast(uint2, a), ub = __builtin_bit_cast(uint2, b);
+    return make_uint4(ua.x, ua.y, ub.x, ub.y);
+}
+
+__global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned short *__restrict__ q,
+                                                            const unsigned short *__restrict__ k,
+                                                            const unsigned short *__restrict__ v,
+                                                            unsigned short *__restrict__ out,
+                                                            float2 *__restrict__ stats, int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage [key][dim]
+    __shared__ __align__(16) unsigned short Vs[2][KS][LDV];   // V stage [key][dim]
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int qlo = t0 + 32 * wave, qhi = qlo + 31;           // this wave's queries
+    const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
+
+    uint4 qf[2][2];   // B operand: query qlo + 16 qt + r, dims 32 ks + 8 g ..
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const int tq = qlo + 16 * qt + r;
+            qf[qt][ks] = make_uint4(0, 0, 0, 0);
+            if (tq < s) qf[qt][ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
+        }
+    f32x4 o[2][4];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mrun[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};   // running maximum (exp2 units), this lane's share of the sum
+    const float c2 = 0.125f * 1.44269504088896340736f;   // log2(e) / sqrt(64)
+
+    uint4 kreg[2], vreg[2];
+    load_rows(km, KS * st_lo, kreg);
+    load_rows(vm, KS * st_lo, vreg);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, k0 = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = kreg[c];
+            *reinterpret_cast<uint4 *>(&Vs[buf][chunk >> 3][8 * (chunk & 7)]) = vreg[c];
+        }
+        __syncthreads();   // also: every wave is done with the stage before the previous one, whose buffer comes next
+        if (st < st_hi) {
+            load_rows(km, k0 + KS, kreg);
+            load_rows(vm, k0 + KS, vreg);
+        }
+        if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;   // no key of this stage is seen by this wave's queries
+        f32x4 sc[4][2];
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+            const uint4 a0 = ld_op(Ks[buf], 16 * kt, 0), a1 = ld_op(Ks[buf], 16 * kt, 1);
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                sc[kt][qt] = mfma32(a0, qf[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                sc[kt][qt] = mfma32(a1, qf[qt][1], sc[kt][qt]);
+            }
+        }
+        const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;   // wave-uniform: nothing to mask
+        if (!full) {
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int key = k0 + 16 * kt + 4 * g + i, tq = qlo + 16 * qt + r;
+                        const bool ok = key <= tq && key >= tq + 1 - ws && tq < s;
+                        sc[kt][qt][i] = ok ? sc[kt][qt][i] : -INFINITY;
+                    }
+        }
+#pragma unroll
+        for (int qt = 0; qt < 2; qt++) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) mx = fmaxf(mx, sc[kt][qt][i]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float mnew = fmaxf(mrun[qt], mx * c2);
+            const float mref = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = __builtin_amdgcn_exp2f(mrun[qt] - mref);
+            mrun[qt] = mnew;
+            float part = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float e = __builtin_amdgcn_exp2f(fmaf(sc[kt][qt][i], c2, -mref));
+                    sc[kt][qt][i] = e;
+                    part += e;
+                }
+            lsum[qt] = fmaf(lsum[qt], alpha, part);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) o[qt][dt] = o[qt][dt] * alpha;
+        }
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            uint4 pb[2];
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                const f32x4 p0 = sc[2 * hf][qt], p1 = sc[2 * hf + 1][qt];
+                pb[qt] = make_uint4(pack2(p0[0], p0[1]), pack2(p0[2], p0[3]), pack2(p1[0], p1[1]), pack2(p1[2], p1[3]));
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 av = ld_tr2(Vs[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++) o[qt][dt] = mfma32(av, pb[qt], o[qt][dt]);
+            }
+        }
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        float sum = lsum[qt];
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+        if (tq < s) {
+            if (g == 0) stats[(size_t)(b * H + h) * s + tq] = make_float2(mrun[qt] == -INFINITY ? 0.f : mrun[qt], inv);
+            unsigned short *ob = out + (row0 + tq) * total + hoff;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+                *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) =
+                    make_uint2(pack2(o[qt][dt][0] * inv, o[qt][dt][1] * inv), pack2(o[qt][dt][2] * inv, o[qt][dt][3] * inv));
+        }
+    }
+}
+
 // Backward, query pass (one workgroup per 64 queries, one wave per 16 queries):
 //   D_t = sum_j w dW = dO_t . O_t with O_t = sum_j w[t,j] v_j recomputed from the stored (bf16) weights,
 //   dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd),  d_q[t] = sum_j dS[t,j] k_j.
@@ -705,14 +859,17 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
                       int seq_len, int num_heads, int head_dim, int window, int batch, int n_persistent, float *stats) {
     if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
+    if (stats) {
+        KernelTimer kt("swa_fwd_stats_kernel");
+        hipLaunchKernelGGL(swa_fwd_stats_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+                           k, v, out, reinterpret_cast<float2 *>(stats), seq_len, num_heads, window);
+        check_launch("swa_fwd_stats_kernel");
+        return true;
+    }
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
     KernelTimer kt("swa_fwd_mfma_kernel");
-    if (stats)
-        hipLaunchKernelGGL(swa_fwd_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, out, nullptr,
-                           reinterpret_cast<float2 *>(stats), seq_len, num_heads, window);
-    else
-        hipLaunchKernelGGL(swa_fwd_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, nullptr,
-                           seq_len, num_heads, window);
+    hipLaunchKernelGGL(swa_fwd_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, nullptr,
+                       seq_len, num_heads, window);
     check_launch("swa_fwd_mfma_kernel");
     return true;
 }

@@ -98,8 +98,8 @@ def test_swa_backward_accumulates_dk_dv_and_overwrites_dq():
 @pytest.mark.parametrize("B,s,H,ws", [(2, 40, 2, 16), (1, 600, 2, 512), (2, 200, 2, 101), (1, 1100, 1, 300),
                                       (1, 2, 1, 2), (8, 130, 2, 64), (1, 64, 1, 64), (1, 65, 3, 2)])
 def test_swa_without_weight_tensor(B, s, H, ws):
-    """The pair that keeps per-query softmax statistics instead of the weight tensor: same output bits as the
-    weight-storing forward, statistics against the oracle's scores, gradients against the weight-storing
+    """The pair that keeps per-query softmax statistics instead of the weight tensor: output against the
+    weight-storing forward and the oracle, statistics against the oracle's scores, gradients against the weight-storing
     backward (same rounding of the weights: fp32 round-off) and the oracle (bf16 tolerance)."""
     hd = 64
     q, k, v, go = _case(B, s, H, hd, 300 + s + ws)
@@ -108,7 +108,11 @@ def test_swa_without_weight_tensor(B, s, H, ws):
     stats = torch.full((B, H, s, 2), float("nan"), device="cuda")
     D.call("swa_forward_lse_bf16_rocm", _u16(q), _u16(k), _u16(v), out, stats, s, H, hd, ws, B)
     torch.cuda.synchronize()
-    assert np.array_equal(out.cpu().numpy(), out_w)
+    # blocked softmax with a running maximum: the output agrees with the weight-storing forward to bf16 rounding
+    # (its weights are rounded before the product with V, here the unnormalised ones are) and with the oracle
+    assert_close("out vs stored weights", orc.bf16_to_f32(out.cpu().numpy()), orc.bf16_to_f32(out_w), REL_TOL_BF16)
+    assert_close("out", orc.bf16_to_f32(out.cpu().numpy()), orc.bf16_to_f32(orc.swa_forward(q, k, v, ws, H, 0)[0]),
+                 REL_TOL_BF16)
     # statistics from the scores in float64
     qf, kf = (orc.bf16_to_f32(a).astype(np.float64).reshape(B, s, H, hd) for a in (q, k))
     st = host(stats)
