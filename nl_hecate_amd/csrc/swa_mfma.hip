@@ -304,7 +304,8 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
 constexpr int FQ = 128;    // queries per workgroup
 constexpr int LDV = 80;    // row stride of the V stage (160 B: the transposing reads of a group fall on 32 banks)
 
-__device__ __forceinline__ uint4 ld_tr2(const unsigned short (*T)[LDV], int row_a, int row_b, int col0) {
+template <int LD>
+__device__ __forceinline__ uint4 ld_tr2(const unsigned short (*T)[LD], int row_a, int row_b, int col0) {
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 *lds_ptr;
     const int sl = threadIdx.x & 15;
@@ -423,7 +424,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
             }
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const uint4 av = ld_tr2(Vs[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
+                const uint4 av = ld_tr2<LDV>(Vs[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
 #pragma unroll
                 for (int qt = 0; qt < 2; qt++) o[qt][dt] = mfma32(av, pb[qt], o[qt][dt]);
             }
@@ -645,6 +646,145 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned s
         float *ob = d_q + (row0 + tq) * total + hoff;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = dq[dt];
+    }
+}
+
+// Query pass on statistics, in key blocks like swa_fwd_stats_kernel (one workgroup per 128 queries, one wave per
+// 32), in ONE sweep over the window.  dS = w (dW - D) needs D_t = sum_j w dW of the whole window, so the sweep
+// accumulates the two sums that do not:  A^T = K^T (w dW)^T and B^T = K^T w^T, and D itself, and ends with
+//   d_q = (A - D B) / sqrt(hd)
+// (the same numbers as sum_j dS k_j; no sweep that rebuilds O first, and D as exact as before — taking D from
+// the forward's bf16 output instead moves it by 2^-9 and, where the window holds few keys, d_q by 5e-3).
+// Per stage a wave forms S^T = K Q^T, the weights w = bf16(exp2(s c - m) / sum) as the weight tensor would hold
+// them, dW^T = V dO^T; dO and w dW enter as hi + lo pairs, w is exact in bf16.  K^T is read from the K rows
+// through ds_read_b64_tr_b16 in the key order that the score tiles leave in the lanes.  D goes to dvec.
+__global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned short *__restrict__ q,
+                                                                 const unsigned short *__restrict__ k,
+                                                                 const unsigned short *__restrict__ v,
+                                                                 const float2 *__restrict__ stats,
+                                                                 const float *__restrict__ d_out,
+                                                                 float *__restrict__ d_q, float *__restrict__ dvec,
+                                                                 int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Ks[2][KS][LDH], Vs[2][KS][LDH];   // stages [key][dim]
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int qlo = t0 + 32 * wave, qhi = qlo + 31;
+    const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
+    const float c2 = 0.125f * 1.44269504088896340736f, scale = 0.125f;
+
+    uint4 qf[2][2], doh[2][2], dol[2][2];
+    float mc[2], inv[2], dpart[2] = {0.f, 0.f};
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        mc[qt] = 0.f; inv[qt] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            qf[qt][ks] = make_uint4(0, 0, 0, 0);
+            f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
+            if (tq < s) {
+                const size_t o = (row0 + tq) * total + hoff + 32 * ks + 8 * g;
+                qf[qt][ks] = *reinterpret_cast<const uint4 *>(q + o);
+                x0 = *reinterpret_cast<const f32x4 *>(d_out + o);
+                x1 = *reinterpret_cast<const f32x4 *>(d_out + o + 4);
+            }
+            split8(x0, x1, doh[qt][ks], dol[qt][ks]);
+        }
+        if (tq < s) {
+            const float2 st2 = stats[(size_t)(b * H + h) * s + tq];
+            mc[qt] = st2.x;
+            inv[qt] = st2.y;
+        }
+    }
+    f32x4 aq[2][4], bq[2][4];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) { aq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; bq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+    uint4 kreg[2], vreg[2];
+    load_rows(km, KS * st_lo, kreg);
+    load_rows(vm, KS * st_lo, vreg);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, k0 = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = kreg[c];
+            *reinterpret_cast<uint4 *>(&Vs[buf][chunk >> 3][8 * (chunk & 7)]) = vreg[c];
+        }
+        __syncthreads();
+        if (st < st_hi) {
+            load_rows(km, k0 + KS, kreg);
+            load_rows(vm, k0 + KS, vreg);
+        }
+        if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
+        const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            uint4 xh[2], xl[2], wb[2];
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                f32x4 x[2];
+                unsigned wp[2][2];
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const int kt = 2 * hf + c;
+                    const uint4 ak0 = ld_op(Ks[buf], 16 * kt, 0), ak1 = ld_op(Ks[buf], 16 * kt, 1);
+                    const uint4 av0 = ld_op(Vs[buf], 16 * kt, 0), av1 = ld_op(Vs[buf], 16 * kt, 1);
+                    f32x4 sc = mfma32(ak0, qf[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                    sc = mfma32(ak1, qf[qt][1], sc);
+                    f32x4 dw = mfma32(av0, doh[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                    dw = mfma32(av0, dol[qt][0], dw);
+                    dw = mfma32(av1, doh[qt][1], dw);
+                    dw = mfma32(av1, dol[qt][1], dw);
+                    f32x4 w;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int key = k0 + 16 * kt + 4 * g + i, tq = qlo + 16 * qt + r;
+                        const bool ok = full || (key <= tq && key >= tq + 1 - ws && tq < s);
+                        w[i] = ok ? __builtin_amdgcn_exp2f(fmaf(sc[i], c2, -mc[qt])) * inv[qt] : 0.f;
+                    }
+                    wp[c][0] = pack2(w[0], w[1]);   // as the weight tensor holds them
+                    wp[c][1] = pack2(w[2], w[3]);
+                    x[c][0] = bf_lo(wp[c][0]) * dw[0];
+                    x[c][1] = bf_hi(wp[c][0]) * dw[1];
+                    x[c][2] = bf_lo(wp[c][1]) * dw[2];
+                    x[c][3] = bf_hi(wp[c][1]) * dw[3];
+                    dpart[qt] += (x[c][0] + x[c][1]) + (x[c][2] + x[c][3]);
+                }
+                split8(x[0], x[1], xh[qt], xl[qt]);
+                wb[qt] = make_uint4(wp[0][0], wp[0][1], wp[1][0], wp[1][1]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 a = ld_tr2<LDH>(Ks[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++) {
+                    aq[qt][dt] = mfma32(a, xh[qt], aq[qt][dt]);
+                    aq[qt][dt] = mfma32(a, xl[qt], aq[qt][dt]);
+                    bq[qt][dt] = mfma32(a, wb[qt], bq[qt][dt]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        float dsum = dpart[qt];
+        dsum += __shfl_xor(dsum, 16, 64);
+        dsum += __shfl_xor(dsum, 32, 64);
+        if (tq < s) {
+            if (g == 0) dvec[(size_t)(b * H + h) * s + tq] = dsum;
+            float *ob = d_q + (row0 + tq) * total + hoff;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+                *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
+        }
     }
 }
 
@@ -886,9 +1026,14 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
     if (es.failed()) return true;
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
     const float2 *st2 = reinterpret_cast<const float2 *>(stats);
-    {
+    if (stats) {
+        KernelTimer kt("swa_bwd_q_stats_kernel");
+        hipLaunchKernelGGL(swa_bwd_q_stats_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(),
+                           q, k, v, st2, d_attn_out, d_q, dvec, seq_len, num_heads, window);
+        check_launch("swa_bwd_q_stats_kernel");
+    } else {
         KernelTimer kt("swa_bwd_q_mfma_kernel");
-        if (stats)
+        if (false)
             hipLaunchKernelGGL(swa_bwd_q_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, nullptr, st2,
                                d_attn_out, d_q, dvec, seq_len, num_heads, window);
         else
