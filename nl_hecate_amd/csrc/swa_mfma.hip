@@ -994,6 +994,162 @@ __global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned shor
     }
 }
 
+// Key pass on statistics, in query blocks (one workgroup per 128 keys, one wave per 32): over the stages of 64
+// queries that see the block's keys, a wave forms S = Q K^T for its two key tiles (rows = queries, column = the
+// lane's key), the weights from the queries' statistics, dW = dO V^T, dS = w (dW - D_t) / sqrt(hd), and
+// accumulates d_v^T += dO^T w and d_k^T += Q^T dS.  The Q and dO rows of a stage are staged as they arrive (dO as
+// hi + lo); the products that contract over queries read them through ds_read_b64_tr_b16 in the query order
+// that the score tiles leave in the lanes.  K and V of the wave's keys sit in registers.
+__global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned short *__restrict__ q,
+                                                                 const unsigned short *__restrict__ k,
+                                                                 const unsigned short *__restrict__ v,
+                                                                 const float2 *__restrict__ stats,
+                                                                 const float *__restrict__ d_out,
+                                                                 const float *__restrict__ dvec,
+                                                                 float *__restrict__ d_k, float *__restrict__ d_v,
+                                                                 int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Qs[2][KS][LDH], Dh[2][KS][LDH], Dl[2][KS][LDH];   // [query][dim]
+    __shared__ __align__(16) float Mc[2][KS], Iv[2][KS], Dd[2][KS];   // the stage's queries: maximum, 1 / sum, D
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int j0 = bc.x * FQ, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int jlo = j0 + 32 * wave, jhi = jlo + 31;            // this wave's keys
+    const int st_lo = j0 / KS, st_hi = min(s - 1, j0 + FQ - 1 + ws - 1) / KS;
+    const float *dvb = dvec + (size_t)(b * H + h) * s;
+    const float2 *stb = stats + (size_t)(b * H + h) * s;
+    const StageSrc qm{q, row0, total, hoff, s};
+    const float c2 = 0.125f * 1.44269504088896340736f, scale = 0.125f;
+
+    uint4 kf[2][2], vf[2][2];   // B operands: key jlo + 16 jt + r, dims 32 ks + 8 g ..
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const int key = jlo + 16 * jt + r;
+            kf[jt][ks] = make_uint4(0, 0, 0, 0);
+            vf[jt][ks] = make_uint4(0, 0, 0, 0);
+            if (key < s) {
+                const size_t o = (row0 + key) * total + hoff + 32 * ks + 8 * g;
+                kf[jt][ks] = *reinterpret_cast<const uint4 *>(k + o);
+                vf[jt][ks] = *reinterpret_cast<const uint4 *>(v + o);
+            }
+        }
+    f32x4 dk[2][4], dv[2][4];   // d_k^T, d_v^T: rows = dims 16 dt + 4 g + i, column = key
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) { dk[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+    // one stage ahead in registers: Q rows (two 16-byte pieces per thread), dO rows (thread = quarter row)
+    uint4 qreg[2];
+    f32x4 dreg[4];
+    float2 streg = make_float2(0.f, 0.f);
+    float ddreg = 0.f;
+    const int drow = tid >> 2, dcol = 16 * (tid & 3);
+    auto fetch_stage = [&](int t_lo) {
+        load_rows(qm, t_lo, qreg);
+        const int t = t_lo + drow;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            dreg[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (t < s) dreg[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dcol + 4 * c);
+        }
+        streg = make_float2(0.f, 0.f);
+        ddreg = 0.f;
+        if (tid < KS && t_lo + tid < s) { streg = stb[t_lo + tid]; ddreg = dvb[t_lo + tid]; }
+    };
+    fetch_stage(KS * st_lo);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, t_lo = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Qs[buf][chunk >> 3][8 * (chunk & 7)]) = qreg[c];
+            uint4 hi, lo;
+            split8(dreg[2 * c], dreg[2 * c + 1], hi, lo);
+            *reinterpret_cast<uint4 *>(&Dh[buf][drow][dcol + 8 * c]) = hi;
+            *reinterpret_cast<uint4 *>(&Dl[buf][drow][dcol + 8 * c]) = lo;
+        }
+        if (tid < KS) { Mc[buf][tid] = streg.x; Iv[buf][tid] = streg.y; Dd[buf][tid] = ddreg; }
+        __syncthreads();
+        if (st < st_hi) fetch_stage(t_lo + KS);
+        if (t_lo + KS - 1 < jlo || t_lo > jhi + ws - 1) continue;   // no query of this stage sees a key of this wave
+        const bool full = t_lo >= jhi && t_lo + KS - 1 <= jlo + ws - 1 && t_lo + KS - 1 < s && jhi < s;
+#pragma unroll
+        for (int hq = 0; hq < 2; hq++) {
+            uint4 wpk[2], dsh[2], dsl[2];
+            f32x4 ds[2][2];
+            unsigned wp[2][2][2];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int qt = 2 * hq + c;
+                const uint4 aq0 = ld_op(Qs[buf], 16 * qt, 0), aq1 = ld_op(Qs[buf], 16 * qt, 1);
+                const uint4 ah0 = ld_op(Dh[buf], 16 * qt, 0), ah1 = ld_op(Dh[buf], 16 * qt, 1);
+                const uint4 al0 = ld_op(Dl[buf], 16 * qt, 0), al1 = ld_op(Dl[buf], 16 * qt, 1);
+                const f32x4 m4 = *reinterpret_cast<const f32x4 *>(&Mc[buf][16 * qt + 4 * g]);
+                const f32x4 i4 = *reinterpret_cast<const f32x4 *>(&Iv[buf][16 * qt + 4 * g]);
+                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&Dd[buf][16 * qt + 4 * g]);
+#pragma unroll
+                for (int jt = 0; jt < 2; jt++) {
+                    f32x4 sc = mfma32(aq0, kf[jt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                    sc = mfma32(aq1, kf[jt][1], sc);
+                    f32x4 dw = mfma32(ah0, vf[jt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                    dw = mfma32(al0, vf[jt][0], dw);
+                    dw = mfma32(ah1, vf[jt][1], dw);
+                    dw = mfma32(al1, vf[jt][1], dw);
+                    f32x4 w;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int t = t_lo + 16 * qt + 4 * g + i, key = jlo + 16 * jt + r;
+                        const bool ok = full || (key <= t && t <= key + ws - 1 && t < s && key < s);
+                        w[i] = ok ? __builtin_amdgcn_exp2f(fmaf(sc[i], c2, -m4[i])) * i4[i] : 0.f;
+                    }
+                    wp[jt][c][0] = pack2(w[0], w[1]);   // as the weight tensor holds them
+                    wp[jt][c][1] = pack2(w[2], w[3]);
+                    ds[jt][c][0] = bf_lo(wp[jt][c][0]) * (dw[0] - d4[0]) * scale;
+                    ds[jt][c][1] = bf_hi(wp[jt][c][0]) * (dw[1] - d4[1]) * scale;
+                    ds[jt][c][2] = bf_lo(wp[jt][c][1]) * (dw[2] - d4[2]) * scale;
+                    ds[jt][c][3] = bf_hi(wp[jt][c][1]) * (dw[3] - d4[3]) * scale;
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 2; jt++) {
+                wpk[jt] = make_uint4(wp[jt][0][0], wp[jt][0][1], wp[jt][1][0], wp[jt][1][1]);
+                split8(ds[jt][0], ds[jt][1], dsh[jt], dsl[jt]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const int ra = 32 * hq + 4 * g, rb = ra + 16;
+                const uint4 aq = ld_tr2<LDH>(Qs[buf], ra, rb, 16 * dt);    // Q^T [dim][query]
+                const uint4 ah = ld_tr2<LDH>(Dh[buf], ra, rb, 16 * dt);    // dO^T hi / lo
+                const uint4 al = ld_tr2<LDH>(Dl[buf], ra, rb, 16 * dt);
+#pragma unroll
+                for (int jt = 0; jt < 2; jt++) {
+                    dk[jt][dt] = mfma32(aq, dsh[jt], dk[jt][dt]);
+                    dk[jt][dt] = mfma32(aq, dsl[jt], dk[jt][dt]);
+                    dv[jt][dt] = mfma32(ah, wpk[jt], dv[jt][dt]);
+                    dv[jt][dt] = mfma32(al, wpk[jt], dv[jt][dt]);
+                }
+            }
+        }
+    }
+    // accumulate: column = key jlo + 16 jt + r, rows = dims 16 dt + 4 g ..
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+        const int key = jlo + 16 * jt + r;
+        if (key >= s) continue;
+        float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            f32x4 *ck = reinterpret_cast<f32x4 *>(pk + 16 * dt + 4 * g), *cv = reinterpret_cast<f32x4 *>(pv + 16 * dt + 4 * g);
+            *ck = *ck + dk[jt][dt];
+            *cv = *cv + dv[jt][dt];
+        }
+    }
+}
+
 }  // namespace
 
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
@@ -1041,8 +1197,15 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
                                d_attn_out, d_q, dvec, seq_len, num_heads, window);
         check_launch("swa_bwd_q_mfma_kernel");
     }
+    if (stats) {
+        KernelTimer kt("swa_bwd_k_stats_kernel");
+        hipLaunchKernelGGL(swa_bwd_k_stats_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(),
+                           q, k, v, st2, d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
+        check_launch("swa_bwd_k_stats_kernel");
+        return true;
+    }
     KernelTimer kt("swa_bwd_k_mfma_kernel");
-    if (stats)
+    if (false)
         hipLaunchKernelGGL(swa_bwd_k_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, nullptr, st2, d_attn_out,
                            dvec, d_k, d_v, seq_len, num_heads, window);
     else
