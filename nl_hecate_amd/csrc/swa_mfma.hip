@@ -26,6 +26,8 @@
 // O^T = V^T P^T: no shuffles between the two products.  V tiles are staged
 // transposed in LDS.  The normalised weights (part of the contract) leave straight
 // from the operand registers.
+// The pair that keeps two statistics per query instead of the weight tensor (swa_*_stats_kernel, at the end of
+// this file) works in blocks with a running maximum and shares only the helpers with the kernels of the contract.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -149,15 +151,12 @@ __device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int k
     return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
 }
 
-// LSE: the weights are not written; the query's softmax statistics (its maximum in exp2 units and the
-// reciprocal of its sum) go to stats [batch * H, s] instead, from which the backward rebuilds the weights.
-template <bool LSE>
 __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
                                                            const unsigned short *__restrict__ k,
                                                            const unsigned short *__restrict__ v,
                                                            unsigned short *__restrict__ out,
-                                                           unsigned short *__restrict__ attn_w,
-                                                           float2 *__restrict__ stats, int s, int H, int ws) {
+                                                           unsigned short *__restrict__ attn_w, int s, int H,
+                                                           int ws) {
     __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage [stage_pos(key)][dim], then V^T stage [dim][key]
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
@@ -238,13 +237,12 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     const float inv = sum > 0.f ? 1.0f / sum : 0.f;
-    if (LSE && g == 0 && tq < s) stats[(size_t)(b * H + h) * s + tq] = make_float2(mc, inv);
 
     // ---- pass B: O^T = V^T P^T, weights out ----
     f32x4 o[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    unsigned short *wrow = LSE ? nullptr : attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+    unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
     __syncthreads();   // every wave is done with the last K stage
     load_pairs(vm, base + KS * st_lo, stg);
 #pragma unroll
@@ -264,7 +262,7 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
             // the lane's 8 weights are slots key0 - lsq .. + 7 of its query's row; keys after the
             // query carry zeros, which the contract wants written while the slot exists
             const int key0 = base + KS * st + 32 * hf + 8 * g, slot0 = key0 - lsq;
-            if (!LSE && tq < s) {
+            if (tq < s) {
                 if (slot0 >= 0 && slot0 + 8 <= ws) {
                     __builtin_memcpy(wrow + slot0, &pb, 16);
                 } else if (slot0 + 8 > 0 && slot0 < ws) {
@@ -277,7 +275,7 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
         }
     }
     // slots whose keys lie beyond the block's last key (early queries only): zero
-    if (!LSE && t0 + QB < ws) {
+    if (t0 + QB < ws) {
         unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
         for (int qi = 0; qi < 16; qi++) {
             const int tt = t0 + 16 * wave + qi;
@@ -290,6 +288,339 @@ __global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned sho
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
             *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) = make_uint2(pack2(o[dt][0], o[dt][1]), pack2(o[dt][2], o[dt][3]));
+    }
+}
+
+// Backward, query pass (one workgroup per 64 queries, one wave per 16 queries):
+//   D_t = sum_j w dW = dO_t . O_t with O_t = sum_j w[t,j] v_j recomputed from the stored (bf16) weights,
+//   dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd),  d_q[t] = sum_j dS[t,j] k_j.
+// Two sweeps over the window: the first rebuilds O^T (four accumulators) and from it D; the second
+// recomputes each dW tile next to its use, so no score tile outlives a stage.  dO and dS enter the
+// bf16 products as hi + lo pairs.  D_t goes to dvec for the key pass.
+//
+// The weights never pass through LDS: the B operand of one query for a 32-key half is one 16-byte
+// load of its weight row, kept in registers for the second sweep.  Only the last stage, the one that
+// holds the queries themselves, is read slot by slot: its groups can end inside the 16 bytes, and a
+// load that runs past the query's row would leave the array at its last row.
+__global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
+                                                                const unsigned short *__restrict__ v,
+                                                                const unsigned short *__restrict__ attn_w,
+                                                                const float *__restrict__ d_out,
+                                                                float *__restrict__ d_q, float *__restrict__ dvec,
+                                                                int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [stage_pos(key)][dim]
+    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][key]: V (sweep 1), K (sweep 2)
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * QB, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const int base = t0 + QB - NS * KS;
+    const int tq = t0 + 16 * wave + r;
+    const int lsq = max(tq + 1 - ws, 0);
+    const size_t row0 = (size_t)b * s;
+    const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
+    const unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
+
+    // weights of this lane's query for the keys of its group in a stage: wv[stage][hf] holds the
+    // 8 keys 32 hf + 8 g .. + 7, zero outside the window
+    uint4 wv[NS][2];
+    auto fetch_weights = [&](int stage, uint4 (&w)[2]) {
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            const int key0 = base + KS * stage + 32 * hf + 8 * g;
+            w[hf] = make_uint4(0, 0, 0, 0);
+            if (stage < NS - 1) {
+                // keys below t0: the group never runs past the query; it may start before the window
+                if (tq < s && key0 + 7 >= lsq) {
+                    uint4 x;
+                    __builtin_memcpy(&x, wrow + (key0 - lsq), 16);
+                    w[hf] = mask_below(x, lsq - key0);
+                }
+            } else {
+                unsigned d[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int key = key0 + e;
+                    unsigned x = 0;
+                    if (tq < s && key >= lsq && key <= tq) x = wrow[key - lsq];
+                    d[e >> 1] |= x << (16 * (e & 1));
+                }
+                w[hf] = make_uint4(d[0], d[1], d[2], d[3]);
+            }
+        }
+    };
+    uint4 sv[2], sk[2];
+
+    // ---- sweep 1: O^T = V^T P^T, then D = dO . O ----
+    f32x4 ot[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < NS; st++) { wv[st][0] = make_uint4(0, 0, 0, 0); wv[st][1] = make_uint4(0, 0, 0, 0); }
+    load_pairs(vm, base + KS * st_lo, sv);
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        if (st < st_lo) continue;
+        const int buf = st & 1;
+        fetch_weights(st, wv[st]);
+        commit_transposed(Tt[buf], sv);
+        __syncthreads();
+        if (st + 1 < NS) load_pairs(vm, base + KS * (st + 1), sv);
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) ot[dt] = mfma32(ld_op(Tt[buf], 16 * dt, hf), wv[st][hf], ot[dt]);
+    }
+    // O^T tile dt holds dims 16 dt + 4 g + i of query r
+    float dsum = 0.f;
+    if (tq < s) {
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            const f32x4 x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * dt + 4 * g);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dsum = fmaf(x[i], ot[dt][i], dsum);
+        }
+    }
+    dsum += __shfl_xor(dsum, 16, 64);
+    dsum += __shfl_xor(dsum, 32, 64);
+    if (g == 0 && tq < s) dvec[(size_t)(b * H + h) * s + tq] = dsum;
+
+    // ---- sweep 2: dW^T tiles recomputed, dS, d_q^T = K^T dS^T ----
+    uint4 doh[2], dol[2];   // dO_t, dims 32 ks + 8 g .. + 7, as hi + lo
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
+        if (tq < s) {
+            const float *p = d_out + (row0 + tq) * total + hoff + 32 * ks + 8 * g;
+            x0 = *reinterpret_cast<const f32x4 *>(p);
+            x1 = *reinterpret_cast<const f32x4 *>(p + 4);
+        }
+        split8(x0, x1, doh[ks], dol[ks]);
+    }
+    f32x4 dq[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) dq[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float scale = 0.125f;
+    __syncthreads();
+    load_rows(vm, base + KS * st_lo, sv);
+    load_pairs(km, base + KS * st_lo, sk);
+#pragma unroll
+    for (int st = 0; st < NS; st++) {
+        if (st < st_lo) continue;
+        const int buf = st & 1;
+        commit_rows_tiled(Vr[buf], sv);
+        commit_transposed(Tt[buf], sk);
+        __syncthreads();
+        if (st + 1 < NS) { load_rows(vm, base + KS * (st + 1), sv); load_pairs(km, base + KS * (st + 1), sk); }
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            f32x4 ds[2];
+            const unsigned wd[4] = {wv[st][hf].x, wv[st][hf].y, wv[st][hf].z, wv[st][hf].w};
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key 32 hf + 8 g + 4 c + i][query r]
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    const uint4 a = ld_op(Vr[buf], 16 * (2 * hf + c), ks);
+                    dw = mfma32(a, doh[ks], dw);
+                    dw = mfma32(a, dol[ks], dw);
+                }
+                ds[c][0] = bf_lo(wd[2 * c]) * (dw[0] - dsum) * scale;
+                ds[c][1] = bf_hi(wd[2 * c]) * (dw[1] - dsum) * scale;
+                ds[c][2] = bf_lo(wd[2 * c + 1]) * (dw[2] - dsum) * scale;
+                ds[c][3] = bf_hi(wd[2 * c + 1]) * (dw[3] - dsum) * scale;
+            }
+            uint4 dsh, dsl;
+            split8(ds[0], ds[1], dsh, dsl);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 a = ld_op(Tt[buf], 16 * dt, hf);
+                dq[dt] = mfma32(a, dsh, dq[dt]);
+                dq[dt] = mfma32(a, dsl, dq[dt]);
+            }
+        }
+    }
+    if (tq < s) {
+        float *ob = d_q + (row0 + tq) * total + hoff;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = dq[dt];
+    }
+}
+
+// Backward, key pass (one workgroup per 64 keys, one wave per 16 keys): over the up to 575
+// queries t in [j, j + window) that see key j,
+//   d_v[j] += sum_t w[t,j] dO_t,   d_k[j] += sum_t dS[t,j] q_t,   dS recomputed from w, dO.v_j, D_t.
+// Two tiles of dS / w in accumulator layout (rows = queries, column = the lane's key) are the A
+// operand of the products with Q^T / dO^T, which are staged transposed in LDS; the rows of the
+// dO stage are stored in tile order (stage_pos) so that those 8 rows are 8 consecutive queries.
+__global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned short *__restrict__ q,
+                                                             const unsigned short *__restrict__ v,
+                                                             const unsigned short *__restrict__ attn_w,
+                                                             const float *__restrict__ d_out,
+                                                             const float *__restrict__ dvec,
+                                                             float *__restrict__ d_k, float *__restrict__ d_v,
+                                                             int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Dh[KS][LDH], Dl[KS][LDH];      // dO hi / lo, [stage_pos(query)][dim]
+    __shared__ __align__(16) unsigned short DhT[HD][LDH], DlT[HD][LDH];    // transposed, [dim][query]
+    __shared__ __align__(16) unsigned short QT[HD][LDH];                   // Q^T, [dim][query]
+    __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
+    __shared__ float Dv[KS];
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int j0 = bc.x * QB, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
+    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+    const float *dvb = dvec + (size_t)(b * H + h) * s;
+    const StageSrc qm{q, row0, total, hoff, s};
+
+    uint4 vf[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        vf[ks] = make_uint4(0, 0, 0, 0);
+        if (kj < s) vf[ks] = *reinterpret_cast<const uint4 *>(v + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
+    }
+    f32x4 dk[4], dv[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { dk[i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+    const float scale = 0.125f;
+    const int t_last = min(s - 1, j0 + QB - 1 + ws - 1);
+
+    // global -> register fetch of one stage (64 queries), issued one stage ahead of its use
+    f32x4 gdo[4];
+    uint4 gq[2];
+    unsigned short gw[16];
+    uint4 gwv[2];
+    float gd = 0.f;
+    // dO: query pair (2 rows) x 4 dims per load; pairs so that the transposed tiles are written as
+    // 32-bit words without bank conflicts
+    const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // query pair, first dim (+32 for the second half)
+    auto fetch_stage = [&](int st) {
+        const int qs0 = j0 + KS * st;
+#pragma unroll
+        for (int cc = 0; cc < 2; cc++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int t = qs0 + 2 * dpair + c;
+                gdo[2 * cc + c] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (t < s) gdo[2 * cc + c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dd0 + 32 * cc);
+            }
+        load_pairs(qm, qs0, gq);
+        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t).
+        // Past the first stage every query lies after all keys of the block, so a group of 8 keys
+        // never runs past the query's row: one 16-byte load (2-byte aligned) per group, the keys
+        // before the window masked.  The first stage is read slot by slot.
+        if (st == 0) {
+#pragma unroll
+            for (int c = 0; c < 16; c++) {
+                const int t = qs0 + 4 * c + wave, key = j0 + l;
+                const int slot = key - max(t + 1 - ws, 0);
+                gw[c] = 0;
+                if (t < s && key <= t && slot >= 0 && slot < ws) gw[c] = awb[(size_t)t * ws + slot];
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int chunk = tid + 256 * c, t = qs0 + (chunk >> 3), key0 = j0 + 8 * (chunk & 7);
+                const int ls = max(t + 1 - ws, 0);
+                gwv[c] = make_uint4(0, 0, 0, 0);
+                if (t < s && key0 + 7 >= ls) {
+                    uint4 x;
+                    __builtin_memcpy(&x, awb + (size_t)t * ws + (key0 - ls), 16);
+                    gwv[c] = mask_below(x, ls - key0);
+                }
+            }
+        }
+        gd = (tid < KS && qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
+    };
+    fetch_stage(0);
+    for (int st = 0; st < NS; st++) {
+        const int qs0 = j0 + KS * st;
+        if (qs0 > t_last) break;
+        __syncthreads();   // previous stage's readers are done
+#pragma unroll
+        for (int cc = 0; cc < 2; cc++) {
+            unsigned hi[2][2], lo[2][2];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const f32x4 x = gdo[2 * cc + c];
+                split2(x[0], x[1], hi[c][0], lo[c][0]);
+                split2(x[2], x[3], hi[c][1], lo[c][1]);
+                const int row = stage_pos(2 * dpair + c);
+                *reinterpret_cast<uint2 *>(&Dh[row][dd0 + 32 * cc]) = make_uint2(hi[c][0], hi[c][1]);
+                *reinterpret_cast<uint2 *>(&Dl[row][dd0 + 32 * cc]) = make_uint2(lo[c][0], lo[c][1]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const unsigned h0 = hi[0][j >> 1], h1 = hi[1][j >> 1], l0 = lo[0][j >> 1], l1 = lo[1][j >> 1];
+                *reinterpret_cast<unsigned *>(&DhT[dd0 + 32 * cc + j][2 * dpair]) =
+                    (j & 1) ? ((h0 >> 16) | (h1 & 0xffff0000u)) : ((h0 & 0xffffu) | (h1 << 16));
+                *reinterpret_cast<unsigned *>(&DlT[dd0 + 32 * cc + j][2 * dpair]) =
+                    (j & 1) ? ((l0 >> 16) | (l1 & 0xffff0000u)) : ((l0 & 0xffffu) | (l1 << 16));
+            }
+        }
+        commit_transposed(QT, gq);
+        if (st == 0) {
+#pragma unroll
+            for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int chunk = tid + 256 * c;
+                *reinterpret_cast<uint4 *>(&Pt[chunk >> 3][8 * (chunk & 7)]) = gwv[c];
+            }
+        }
+        if (tid < KS) Dv[tid] = gd;
+        __syncthreads();
+        if (qs0 + KS <= t_last) fetch_stage(st + 1);
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            f32x4 ds[2];
+            unsigned pw[2][2];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW[query 32 hf + 8 g + 4 c + i][key r of this wave]
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    dw = mfma32(ld_op(Dh, 16 * (2 * hf + c), ks), vf[ks], dw);
+                    dw = mfma32(ld_op(Dl, 16 * (2 * hf + c), ks), vf[ks], dw);
+                }
+                unsigned short p4[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int qi = 32 * hf + 8 * g + 4 * c + i;
+                    p4[i] = Pt[qi][16 * wave + r];
+                    ds[c][i] = __uint_as_float((unsigned)p4[i] << 16) * (dw[i] - Dv[qi]) * scale;
+                }
+                pw[c][0] = (unsigned)p4[0] | ((unsigned)p4[1] << 16);
+                pw[c][1] = (unsigned)p4[2] | ((unsigned)p4[3] << 16);
+            }
+            const uint4 pa = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
+            uint4 dsh, dsl;
+            split8(ds[0], ds[1], dsh, dsl);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 bh = ld_op(DhT, 16 * dt, hf), bl = ld_op(DlT, 16 * dt, hf), bq = ld_op(QT, 16 * dt, hf);
+                dv[dt] = mfma32(pa, bh, dv[dt]);
+                dv[dt] = mfma32(pa, bl, dv[dt]);
+                dk[dt] = mfma32(dsh, bq, dk[dt]);
+                dk[dt] = mfma32(dsl, bq, dk[dt]);
+            }
+        }
+    }
+    // accumulate: rows = keys 16 wave + 4g + i, column = dim 16 dt + r
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int key = j0 + 16 * wave + 4 * g + i;
+        if (key >= s) continue;
+        float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            pk[16 * dt + r] += dk[dt][i];
+            pv[16 * dt + r] += dv[dt][i];
+        }
     }
 }
 
@@ -448,207 +779,6 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
     }
 }
 
-// Backward, query pass (one workgroup per 64 queries, one wave per 16 queries):
-//   D_t = sum_j w dW = dO_t . O_t with O_t = sum_j w[t,j] v_j recomputed from the stored (bf16) weights,
-//   dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd),  d_q[t] = sum_j dS[t,j] k_j.
-// Two sweeps over the window: the first rebuilds O^T (four accumulators) and from it D; the second
-// recomputes each dW tile next to its use, so no score tile outlives a stage.  dO and dS enter the
-// bf16 products as hi + lo pairs.  D_t goes to dvec for the key pass.
-//
-// The weights never pass through LDS: the B operand of one query for a 32-key half is one 16-byte
-// load of its weight row, kept in registers for the second sweep.  Only the last stage, the one that
-// holds the queries themselves, is read slot by slot: its groups can end inside the 16 bytes, and a
-// load that runs past the query's row would leave the array at its last row.
-// LSE: the weights of a stage are rebuilt from the scores (the forward's own sequence of matrix-core steps on the
-// K stage, which takes the place of the V stage that sweep 1 does not use) and the query's statistics.
-template <bool LSE>
-__global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ q,
-                                                                const unsigned short *__restrict__ k,
-                                                                const unsigned short *__restrict__ v,
-                                                                const unsigned short *__restrict__ attn_w,
-                                                                const float2 *__restrict__ stats,
-                                                                const float *__restrict__ d_out,
-                                                                float *__restrict__ d_q, float *__restrict__ dvec,
-                                                                int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [stage_pos(key)][dim]
-    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][key]: V (sweep 1), K (sweep 2)
-    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const BlockCoord bc = xcd_block_coord(H);
-    const int t0 = bc.x * QB, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
-    const int base = t0 + QB - NS * KS;
-    const int tq = t0 + 16 * wave + r;
-    const int lsq = max(tq + 1 - ws, 0);
-    const size_t row0 = (size_t)b * s;
-    const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
-    const unsigned short *wrow = LSE ? nullptr : attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
-    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
-    uint4 qf[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-    float q_mc = 0.f, q_inv = 0.f;
-    if (LSE && tq < s) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++)
-            qf[ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
-        const float2 st2 = stats[(size_t)(b * H + h) * s + tq];
-        q_mc = st2.x;
-        q_inv = st2.y;
-    }
-    // LSE: weights of stage `stage` from its K rows in T (tile order): scores, mask, exp2, normalise, bf16
-    auto rebuild_weights = [&](unsigned short (*T)[LDH], int stage, uint4 (&w)[2]) {
-        const float c2 = 0.125f * 1.44269504088896340736f;
-        const int k0 = base + KS * stage;
-        f32x4 a[4];
-#pragma unroll
-        for (int kt = 0; kt < 4; kt++) {
-            a[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++) a[kt] = mfma32(ld_op(T, 16 * kt, ks), qf[ks], a[kt]);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int key = k0 + tile_key(kt, g, i);
-                const bool ok = key >= lsq && key <= tq && tq < s;
-                a[kt][i] = ok ? __builtin_amdgcn_exp2f(fmaf(a[kt][i], c2, -q_mc)) * q_inv : 0.f;
-            }
-        }
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            const f32x4 p0 = a[2 * hf], p1 = a[2 * hf + 1];
-            w[hf] = make_uint4(pack2(p0[0], p0[1]), pack2(p0[2], p0[3]), pack2(p1[0], p1[1]), pack2(p1[2], p1[3]));
-        }
-    };
-
-    // weights of this lane's query for the keys of its group in a stage: wv[stage][hf] holds the
-    // 8 keys 32 hf + 8 g .. + 7, zero outside the window
-    uint4 wv[NS][2];
-    auto fetch_weights = [&](int stage, uint4 (&w)[2]) {
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            const int key0 = base + KS * stage + 32 * hf + 8 * g;
-            w[hf] = make_uint4(0, 0, 0, 0);
-            if (stage < NS - 1) {
-                // keys below t0: the group never runs past the query; it may start before the window
-                if (tq < s && key0 + 7 >= lsq) {
-                    uint4 x;
-                    __builtin_memcpy(&x, wrow + (key0 - lsq), 16);
-                    w[hf] = mask_below(x, lsq - key0);
-                }
-            } else {
-                unsigned d[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int key = key0 + e;
-                    unsigned x = 0;
-                    if (tq < s && key >= lsq && key <= tq) x = wrow[key - lsq];
-                    d[e >> 1] |= x << (16 * (e & 1));
-                }
-                w[hf] = make_uint4(d[0], d[1], d[2], d[3]);
-            }
-        }
-    };
-    uint4 sv[2], sk[2];
-
-    // ---- sweep 1: O^T = V^T P^T, then D = dO . O ----
-    f32x4 ot[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int st = 0; st < NS; st++) { wv[st][0] = make_uint4(0, 0, 0, 0); wv[st][1] = make_uint4(0, 0, 0, 0); }
-    load_pairs(vm, base + KS * st_lo, sv);
-    if (LSE) load_rows(km, base + KS * st_lo, sk);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
-        const int buf = st & 1;
-        if (!LSE) fetch_weights(st, wv[st]);
-        commit_transposed(Tt[buf], sv);
-        if (LSE) commit_rows_tiled(Vr[buf], sk);
-        __syncthreads();
-        if (st + 1 < NS) {
-            load_pairs(vm, base + KS * (st + 1), sv);
-            if (LSE) load_rows(km, base + KS * (st + 1), sk);
-        }
-        if (LSE) rebuild_weights(Vr[buf], st, wv[st]);
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++)
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) ot[dt] = mfma32(ld_op(Tt[buf], 16 * dt, hf), wv[st][hf], ot[dt]);
-    }
-    // O^T tile dt holds dims 16 dt + 4 g + i of query r
-    float dsum = 0.f;
-    if (tq < s) {
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            const f32x4 x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * dt + 4 * g);
-#pragma unroll
-            for (int i = 0; i < 4; i++) dsum = fmaf(x[i], ot[dt][i], dsum);
-        }
-    }
-    dsum += __shfl_xor(dsum, 16, 64);
-    dsum += __shfl_xor(dsum, 32, 64);
-    if (g == 0 && tq < s) dvec[(size_t)(b * H + h) * s + tq] = dsum;
-
-    // ---- sweep 2: dW^T tiles recomputed, dS, d_q^T = K^T dS^T ----
-    uint4 doh[2], dol[2];   // dO_t, dims 32 ks + 8 g .. + 7, as hi + lo
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
-        if (tq < s) {
-            const float *p = d_out + (row0 + tq) * total + hoff + 32 * ks + 8 * g;
-            x0 = *reinterpret_cast<const f32x4 *>(p);
-            x1 = *reinterpret_cast<const f32x4 *>(p + 4);
-        }
-        split8(x0, x1, doh[ks], dol[ks]);
-    }
-    f32x4 dq[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) dq[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const float scale = 0.125f;
-    __syncthreads();
-    load_rows(vm, base + KS * st_lo, sv);
-    load_pairs(km, base + KS * st_lo, sk);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
-        const int buf = st & 1;
-        commit_rows_tiled(Vr[buf], sv);
-        commit_transposed(Tt[buf], sk);
-        __syncthreads();
-        if (st + 1 < NS) { load_rows(vm, base + KS * (st + 1), sv); load_pairs(km, base + KS * (st + 1), sk); }
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            f32x4 ds[2];
-            const unsigned wd[4] = {wv[st][hf].x, wv[st][hf].y, wv[st][hf].z, wv[st][hf].w};
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key 32 hf + 8 g + 4 c + i][query r]
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++) {
-                    const uint4 a = ld_op(Vr[buf], 16 * (2 * hf + c), ks);
-                    dw = mfma32(a, doh[ks], dw);
-                    dw = mfma32(a, dol[ks], dw);
-                }
-                ds[c][0] = bf_lo(wd[2 * c]) * (dw[0] - dsum) * scale;
-                ds[c][1] = bf_hi(wd[2 * c]) * (dw[1] - dsum) * scale;
-                ds[c][2] = bf_lo(wd[2 * c + 1]) * (dw[2] - dsum) * scale;
-                ds[c][3] = bf_hi(wd[2 * c + 1]) * (dw[3] - dsum) * scale;
-            }
-            uint4 dsh, dsl;
-            split8(ds[0], ds[1], dsh, dsl);
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const uint4 a = ld_op(Tt[buf], 16 * dt, hf);
-                dq[dt] = mfma32(a, dsh, dq[dt]);
-                dq[dt] = mfma32(a, dsl, dq[dt]);
-            }
-        }
-    }
-    if (tq < s) {
-        float *ob = d_q + (row0 + tq) * total + hoff;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = dq[dt];
-    }
-}
-
 // Query pass on statistics, in key blocks like swa_fwd_stats_kernel (one workgroup per 128 queries, one wave per
 // 32), in ONE sweep over the window.  dS = w (dW - D) needs D_t = sum_j w dW of the whole window, so the sweep
 // accumulates the two sums that do not:  A^T = K^T (w dW)^T and B^T = K^T w^T, and D itself, and ends with
@@ -784,212 +914,6 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
 #pragma unroll
             for (int dt = 0; dt < 4; dt++)
                 *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
-        }
-    }
-}
-
-// Backward, key pass (one workgroup per 64 keys, one wave per 16 keys): over the up to 575
-// queries t in [j, j + window) that see key j,
-//   d_v[j] += sum_t w[t,j] dO_t,   d_k[j] += sum_t dS[t,j] q_t,   dS recomputed from w, dO.v_j, D_t.
-// Two tiles of dS / w in accumulator layout (rows = queries, column = the lane's key) are the A
-// operand of the products with Q^T / dO^T, which are staged transposed in LDS; the rows of the
-// dO stage are stored in tile order (stage_pos) so that those 8 rows are 8 consecutive queries.
-// LSE: the weights are rebuilt per tile from Q K^T (the Q rows of the stage take the LDS matrix of the stored
-// weights, K of the block's keys sits in registers) and the queries' statistics.
-template <bool LSE>
-__global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned short *__restrict__ q,
-                                                             const unsigned short *__restrict__ k,
-                                                             const unsigned short *__restrict__ v,
-                                                             const unsigned short *__restrict__ attn_w,
-                                                             const float2 *__restrict__ stats,
-                                                             const float *__restrict__ d_out,
-                                                             const float *__restrict__ dvec,
-                                                             float *__restrict__ d_k, float *__restrict__ d_v,
-                                                             int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short Dh[KS][LDH], Dl[KS][LDH];      // dO hi / lo, [stage_pos(query)][dim]
-    __shared__ __align__(16) unsigned short DhT[HD][LDH], DlT[HD][LDH];    // transposed, [dim][query]
-    __shared__ __align__(16) unsigned short QT[HD][LDH];                   // Q^T, [dim][query]
-    __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
-    __shared__ float Dv[KS];
-    __shared__ float2 Qst[KS];   // LSE: statistics of the stage's queries
-    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const BlockCoord bc = xcd_block_coord(H);
-    const int j0 = bc.x * QB, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
-    const size_t row0 = (size_t)b * s;
-    const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
-    const unsigned short *awb = LSE ? nullptr : attn_w + ((size_t)(b * H + h) * s) * ws;
-    const float *dvb = dvec + (size_t)(b * H + h) * s;
-    const float2 *stb = LSE ? stats + (size_t)(b * H + h) * s : nullptr;
-    const StageSrc qm{q, row0, total, hoff, s};
-
-    uint4 vf[2], kf[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        vf[ks] = make_uint4(0, 0, 0, 0);
-        kf[ks] = make_uint4(0, 0, 0, 0);
-        if (kj < s) vf[ks] = *reinterpret_cast<const uint4 *>(v + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
-        if (LSE && kj < s) kf[ks] = *reinterpret_cast<const uint4 *>(k + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
-    }
-    f32x4 dk[4], dv[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) { dk[i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-    const float scale = 0.125f;
-    const int t_last = min(s - 1, j0 + QB - 1 + ws - 1);
-
-    // global -> register fetch of one stage (64 queries), issued one stage ahead of its use
-    f32x4 gdo[4];
-    uint4 gq[2];
-    unsigned short gw[16];
-    uint4 gwv[2], gqr[2];
-    float gd = 0.f;
-    float2 gst = make_float2(0.f, 0.f);
-    // dO: query pair (2 rows) x 4 dims per load; pairs so that the transposed tiles are written as
-    // 32-bit words without bank conflicts
-    const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // query pair, first dim (+32 for the second half)
-    auto fetch_stage = [&](int st) {
-        const int qs0 = j0 + KS * st;
-#pragma unroll
-        for (int cc = 0; cc < 2; cc++)
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int t = qs0 + 2 * dpair + c;
-                gdo[2 * cc + c] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (t < s) gdo[2 * cc + c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dd0 + 32 * cc);
-            }
-        load_pairs(qm, qs0, gq);
-        if (LSE) {   // the stage's Q rows once more, for the tile-ordered copy, and the queries' statistics
-            load_rows(qm, qs0, gqr);
-            gst = (tid < KS && qs0 + tid < s) ? stb[qs0 + tid] : make_float2(0.f, 0.f);
-        } else
-        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t).
-        // Past the first stage every query lies after all keys of the block, so a group of 8 keys
-        // never runs past the query's row: one 16-byte load (2-byte aligned) per group, the keys
-        // before the window masked.  The first stage is read slot by slot.
-        if (st == 0) {
-#pragma unroll
-            for (int c = 0; c < 16; c++) {
-                const int t = qs0 + 4 * c + wave, key = j0 + l;
-                const int slot = key - max(t + 1 - ws, 0);
-                gw[c] = 0;
-                if (t < s && key <= t && slot >= 0 && slot < ws) gw[c] = awb[(size_t)t * ws + slot];
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int chunk = tid + 256 * c, t = qs0 + (chunk >> 3), key0 = j0 + 8 * (chunk & 7);
-                const int ls = max(t + 1 - ws, 0);
-                gwv[c] = make_uint4(0, 0, 0, 0);
-                if (t < s && key0 + 7 >= ls) {
-                    uint4 x;
-                    __builtin_memcpy(&x, awb + (size_t)t * ws + (key0 - ls), 16);
-                    gwv[c] = mask_below(x, ls - key0);
-                }
-            }
-        }
-        gd = (tid < KS && qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
-    };
-    fetch_stage(0);
-    for (int st = 0; st < NS; st++) {
-        const int qs0 = j0 + KS * st;
-        if (qs0 > t_last) break;
-        __syncthreads();   // previous stage's readers are done
-#pragma unroll
-        for (int cc = 0; cc < 2; cc++) {
-            unsigned hi[2][2], lo[2][2];
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const f32x4 x = gdo[2 * cc + c];
-                split2(x[0], x[1], hi[c][0], lo[c][0]);
-                split2(x[2], x[3], hi[c][1], lo[c][1]);
-                const int row = stage_pos(2 * dpair + c);
-                *reinterpret_cast<uint2 *>(&Dh[row][dd0 + 32 * cc]) = make_uint2(hi[c][0], hi[c][1]);
-                *reinterpret_cast<uint2 *>(&Dl[row][dd0 + 32 * cc]) = make_uint2(lo[c][0], lo[c][1]);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const unsigned h0 = hi[0][j >> 1], h1 = hi[1][j >> 1], l0 = lo[0][j >> 1], l1 = lo[1][j >> 1];
-                *reinterpret_cast<unsigned *>(&DhT[dd0 + 32 * cc + j][2 * dpair]) =
-                    (j & 1) ? ((h0 >> 16) | (h1 & 0xffff0000u)) : ((h0 & 0xffffu) | (h1 << 16));
-                *reinterpret_cast<unsigned *>(&DlT[dd0 + 32 * cc + j][2 * dpair]) =
-                    (j & 1) ? ((l0 >> 16) | (l1 & 0xffff0000u)) : ((l0 & 0xffffu) | (l1 << 16));
-            }
-        }
-        commit_transposed(QT, gq);
-        if (LSE) {
-            commit_rows_tiled(Pt, gqr);
-            if (tid < KS) Qst[tid] = gst;
-        } else if (st == 0) {
-#pragma unroll
-            for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
-        } else {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int chunk = tid + 256 * c;
-                *reinterpret_cast<uint4 *>(&Pt[chunk >> 3][8 * (chunk & 7)]) = gwv[c];
-            }
-        }
-        if (tid < KS) Dv[tid] = gd;
-        __syncthreads();
-        if (qs0 + KS <= t_last) fetch_stage(st + 1);
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            f32x4 ds[2];
-            unsigned pw[2][2];
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW[query 32 hf + 8 g + 4 c + i][key r of this wave]
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++) {
-                    dw = mfma32(ld_op(Dh, 16 * (2 * hf + c), ks), vf[ks], dw);
-                    dw = mfma32(ld_op(Dl, 16 * (2 * hf + c), ks), vf[ks], dw);
-                }
-                unsigned short p4[4];
-                f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};   // LSE: scores of the same tile
-                if (LSE) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ks++) sc = mfma32(ld_op(Pt, 16 * (2 * hf + c), ks), kf[ks], sc);
-                }
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int qi = 32 * hf + 8 * g + 4 * c + i;
-                    if (LSE) {
-                        const int t = qs0 + qi;
-                        const float2 st2 = Qst[qi];
-                        const bool ok = t < s && kj <= t && kj >= max(t + 1 - ws, 0);
-                        const float pf = ok ? __builtin_amdgcn_exp2f(fmaf(sc[i], 0.125f * 1.44269504088896340736f, -st2.x)) * st2.y : 0.f;
-                        p4[i] = (unsigned short)(pack2(pf, 0.f) & 0xffffu);
-                    } else {
-                        p4[i] = Pt[qi][16 * wave + r];
-                    }
-                    ds[c][i] = __uint_as_float((unsigned)p4[i] << 16) * (dw[i] - Dv[qi]) * scale;
-                }
-                pw[c][0] = (unsigned)p4[0] | ((unsigned)p4[1] << 16);
-                pw[c][1] = (unsigned)p4[2] | ((unsigned)p4[3] << 16);
-            }
-            const uint4 pa = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
-            uint4 dsh, dsl;
-            split8(ds[0], ds[1], dsh, dsl);
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const uint4 bh = ld_op(DhT, 16 * dt, hf), bl = ld_op(DlT, 16 * dt, hf), bq = ld_op(QT, 16 * dt, hf);
-                dv[dt] = mfma32(pa, bh, dv[dt]);
-                dv[dt] = mfma32(pa, bl, dv[dt]);
-                dk[dt] = mfma32(dsh, bq, dk[dt]);
-                dk[dt] = mfma32(dsl, bq, dk[dt]);
-            }
-        }
-    }
-    // accumulate: rows = keys 16 wave + 4g + i, column = dim 16 dt + r
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int key = j0 + 16 * wave + 4 * g + i;
-        if (key >= s) continue;
-        float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            pk[16 * dt + r] += dk[dt][i];
-            pv[16 * dt + r] += dv[dt][i];
         }
     }
 }
@@ -1164,15 +1088,12 @@ bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, u
     }
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
     KernelTimer kt("swa_fwd_mfma_kernel");
-    hipLaunchKernelGGL(swa_fwd_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, nullptr,
-                       seq_len, num_heads, window);
+    hipLaunchKernelGGL(swa_fwd_mfma_kernel, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, seq_len, num_heads,
+                       window);
     check_launch("swa_fwd_mfma_kernel");
     return true;
 }
 
-}  // namespace nlh
-
-namespace nlh {
 bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *attn_weights,
                        const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
                        int head_dim, int window, int batch, int n_persistent, const float *stats) {
@@ -1180,38 +1101,33 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
     if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
     float *dvec = scratch(1, (size_t)batch * num_heads * seq_len * sizeof(float));
     if (es.failed()) return true;
-    const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
-    const float2 *st2 = reinterpret_cast<const float2 *>(stats);
     if (stats) {
-        KernelTimer kt("swa_bwd_q_stats_kernel");
-        hipLaunchKernelGGL(swa_bwd_q_stats_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(),
-                           q, k, v, st2, d_attn_out, d_q, dvec, seq_len, num_heads, window);
-        check_launch("swa_bwd_q_stats_kernel");
-    } else {
-        KernelTimer kt("swa_bwd_q_mfma_kernel");
-        if (false)
-            hipLaunchKernelGGL(swa_bwd_q_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, nullptr, st2,
-                               d_attn_out, d_q, dvec, seq_len, num_heads, window);
-        else
-            hipLaunchKernelGGL(swa_bwd_q_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, attn_weights, nullptr,
-                               d_attn_out, d_q, dvec, seq_len, num_heads, window);
-        check_launch("swa_bwd_q_mfma_kernel");
-    }
-    if (stats) {
+        const float2 *st2 = reinterpret_cast<const float2 *>(stats);
+        const dim3 grid((seq_len + FQ - 1) / FQ, num_heads, batch);
+        {
+            KernelTimer kt("swa_bwd_q_stats_kernel");
+            hipLaunchKernelGGL(swa_bwd_q_stats_kernel, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, dvec,
+                               seq_len, num_heads, window);
+            check_launch("swa_bwd_q_stats_kernel");
+        }
         KernelTimer kt("swa_bwd_k_stats_kernel");
-        hipLaunchKernelGGL(swa_bwd_k_stats_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(),
-                           q, k, v, st2, d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
+        hipLaunchKernelGGL(swa_bwd_k_stats_kernel, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec, d_k, d_v,
+                           seq_len, num_heads, window);
         check_launch("swa_bwd_k_stats_kernel");
         return true;
     }
+    const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
+    {
+        KernelTimer kt("swa_bwd_q_mfma_kernel");
+        hipLaunchKernelGGL(swa_bwd_q_mfma_kernel, grid, dim3(256), 0, stream(), k, v, attn_weights, d_attn_out, d_q, dvec,
+                           seq_len, num_heads, window);
+        check_launch("swa_bwd_q_mfma_kernel");
+    }
     KernelTimer kt("swa_bwd_k_mfma_kernel");
-    if (false)
-        hipLaunchKernelGGL(swa_bwd_k_mfma_kernel<true>, grid, dim3(256), 0, stream(), q, k, v, nullptr, st2, d_attn_out,
-                           dvec, d_k, d_v, seq_len, num_heads, window);
-    else
-        hipLaunchKernelGGL(swa_bwd_k_mfma_kernel<false>, grid, dim3(256), 0, stream(), q, k, v, attn_weights, nullptr,
-                           d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
+    hipLaunchKernelGGL(swa_bwd_k_mfma_kernel, grid, dim3(256), 0, stream(), q, v, attn_weights, d_attn_out, dvec, d_k,
+                       d_v, seq_len, num_heads, window);
     check_launch("swa_bwd_k_mfma_kernel");
     return true;
 }
+
 }  // namespace nlh
