@@ -18,16 +18,11 @@
 // access).  A tile's rows come from an LDS matrix whose rows are stored in that
 // order (stage_pos).
 //
-// Forward.  One workgroup per (64 queries, head, batch), one wave per 16 queries.
-// The wave computes S^T = K Q^T for its 16 queries against the 576 keys
-// [t0-512, t0+64) that the block can see, 36 tiles kept in registers.  A lane owns
-// ONE query column and 144 of its keys, so the softmax is a per-lane reduction plus
-// two exchanges, and the normalised tiles are already the B operand of
-// O^T = V^T P^T: no shuffles between the two products.  V tiles are staged
-// transposed in LDS.  The normalised weights (part of the contract) leave straight
-// from the operand registers.
-// The pair that keeps two statistics per query instead of the weight tensor (swa_*_stats_kernel, at the end of
-// this file) works in blocks with a running maximum and shares only the helpers with the kernels of the contract.
+// That order serves the two backward kernels of the contract, which read the stored weights 16 bytes at a time.
+// The forward of the contract (swa_fwd_blocked_kernel) and the pair that keeps two statistics per query instead
+// of the weight tensor (swa_*_stats_kernel) work in blocks of 64 keys with a running maximum, stage every row
+// block as it arrives and read transposed operands through ds_read_b64_tr_b16; they share only the helpers with
+// the two kernels above them.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -149,146 +144,6 @@ __device__ __forceinline__ void commit_transposed(unsigned short (*T)[LDH], cons
 __device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int ks) {
     const int l = threadIdx.x & 63;
     return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
-}
-
-__global__ __launch_bounds__(256, 2) void swa_fwd_mfma_kernel(const unsigned short *__restrict__ q,
-                                                           const unsigned short *__restrict__ k,
-                                                           const unsigned short *__restrict__ v,
-                                                           unsigned short *__restrict__ out,
-                                                           unsigned short *__restrict__ attn_w, int s, int H,
-                                                           int ws) {
-    __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage [stage_pos(key)][dim], then V^T stage [dim][key]
-    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const BlockCoord bc = xcd_block_coord(H);
-    const int t0 = bc.x * QB, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
-    const int base = t0 + QB - NS * KS;               // first key of stage 0 (may be negative)
-    const int tq = t0 + 16 * wave + r;                // this lane's query (column of S^T)
-    const size_t row0 = (size_t)b * s;
-    const int first_key = max(t0 + 1 - ws, 0);        // smallest key any query of the block sees
-    const int st_lo = max(0, (first_key - base) / KS);   // stages before it hold masked keys only
-    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
-
-    uint4 qf[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        qf[ks] = make_uint4(0, 0, 0, 0);
-        if (tq < s) qf[ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
-    }
-    f32x4 acc[NT];
-#pragma unroll
-    for (int i = 0; i < NT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    uint4 stg[2];
-
-    // ---- pass A: S^T tiles ----
-    load_rows(km, base + KS * st_lo, stg);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
-        const int buf = st & 1;
-        commit_rows_tiled(Ks[buf], stg);
-        __syncthreads();
-        if (st + 1 < NS) load_rows(km, base + KS * (st + 1), stg);
-#pragma unroll
-        for (int kt = 0; kt < 4; kt++)
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++) acc[4 * st + kt] = mfma32(ld_op(Ks[buf], 16 * kt, ks), qf[ks], acc[4 * st + kt]);
-    }
-
-    // ---- mask and softmax over this lane's query column ----
-    // exp(scale (x - max)) = exp2(c x - c max) with c = scale log2(e): one fused multiply-add and
-    // one v_exp_f32 per score; exp2(-inf) = 0 takes care of the masked ones.  Only the stages at
-    // the two ends of the window hold masked keys; the others skip the test (block-uniform).
-    const float c2 = 0.125f * 1.44269504088896340736f;   // log2(e) / sqrt(64)
-    const int lsq = max(tq + 1 - ws, 0);
-    const int ls_hi = max(t0 + QB - ws, 0);   // window start of the block's last query
-    float mx = -INFINITY;
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        const int k0 = base + KS * st;
-        const bool full = k0 >= ls_hi && k0 + KS - 1 <= t0 && t0 + QB <= s;
-        if (!full) {
-#pragma unroll
-            for (int kt = 0; kt < 4; kt++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int key = k0 + tile_key(kt, g, i);
-                    const bool ok = key >= lsq && key <= tq && tq < s;
-                    acc[4 * st + kt][i] = ok ? acc[4 * st + kt][i] : -INFINITY;
-                }
-        }
-#pragma unroll
-        for (int kt = 0; kt < 4; kt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[4 * st + kt][i]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mc = mx == -INFINITY ? 0.f : mx * c2;
-    float sum = 0.f;
-#pragma unroll
-    for (int T = 0; T < NT; T++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float e = __builtin_amdgcn_exp2f(fmaf(acc[T][i], c2, -mc));
-            acc[T][i] = e;
-            sum += e;
-        }
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
-    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
-
-    // ---- pass B: O^T = V^T P^T, weights out ----
-    f32x4 o[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
-    __syncthreads();   // every wave is done with the last K stage
-    load_pairs(vm, base + KS * st_lo, stg);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
-        const int buf = st & 1;
-        commit_transposed(Ks[buf], stg);
-        __syncthreads();
-        if (st + 1 < NS) load_pairs(vm, base + KS * (st + 1), stg);
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            const f32x4 p0 = acc[4 * st + 2 * hf], p1 = acc[4 * st + 2 * hf + 1];
-            const uint4 pb = make_uint4(pack2(p0[0] * inv, p0[1] * inv), pack2(p0[2] * inv, p0[3] * inv),
-                                        pack2(p1[0] * inv, p1[1] * inv), pack2(p1[2] * inv, p1[3] * inv));
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) o[dt] = mfma32(ld_op(Ks[buf], 16 * dt, hf), pb, o[dt]);
-            // the lane's 8 weights are slots key0 - lsq .. + 7 of its query's row; keys after the
-            // query carry zeros, which the contract wants written while the slot exists
-            const int key0 = base + KS * st + 32 * hf + 8 * g, slot0 = key0 - lsq;
-            if (tq < s) {
-                if (slot0 >= 0 && slot0 + 8 <= ws) {
-                    __builtin_memcpy(wrow + slot0, &pb, 16);
-                } else if (slot0 + 8 > 0 && slot0 < ws) {
-                    const unsigned d[4] = {pb.x, pb.y, pb.z, pb.w};
-#pragma unroll
-                    for (int e = 0; e < 8; e++)
-                        if (slot0 + e >= 0 && slot0 + e < ws) wrow[slot0 + e] = (unsigned short)(d[e >> 1] >> (16 * (e & 1)));
-                }
-            }
-        }
-    }
-    // slots whose keys lie beyond the block's last key (early queries only): zero
-    if (t0 + QB < ws) {
-        unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
-        for (int qi = 0; qi < 16; qi++) {
-            const int tt = t0 + 16 * wave + qi;
-            if (tt >= s) break;
-            for (int slot = t0 + QB + l; slot < ws; slot += 64) awb[(size_t)tt * ws + slot] = 0;
-        }
-    }
-    if (tq < s) {
-        unsigned short *ob = out + (row0 + tq) * total + hoff;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-            *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) = make_uint2(pack2(o[dt][0], o[dt][1]), pack2(o[dt][2], o[dt][3]));
-    }
 }
 
 // Backward, query pass (one workgroup per 64 queries, one wave per 16 queries):
@@ -779,6 +634,205 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
     }
 }
 
+// Forward of the contract (normalised weights stored) in the same blocks: the weights need the final maximum
+// and sum, so the window is swept twice — scores and running statistics first, then scores again, the weights
+// w = bf16(exp2(s c - m) / sum) to their slot rows (four consecutive slots per lane and tile: 8-byte stores at
+// 2-byte alignment) and O^T += V^T w^T.  Slots behind an early query's own key (t < window - 1) are zeroed at
+// the end.
+__global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned short *__restrict__ q,
+                                                              const unsigned short *__restrict__ k,
+                                                              const unsigned short *__restrict__ v,
+                                                              unsigned short *__restrict__ out,
+                                                              unsigned short *__restrict__ attn_w, int s, int H,
+                                                              int ws) {
+    __shared__ __align__(16) unsigned short Ks[2][KS][LDH];   // K stage [key][dim]
+    __shared__ __align__(16) unsigned short Vs[2][KS][LDV];   // V stage [key][dim]
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int qlo = t0 + 32 * wave, qhi = qlo + 31;
+    const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
+    const float c2 = 0.125f * 1.44269504088896340736f;
+
+    uint4 qf[2][2];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const int tq = qlo + 16 * qt + r;
+            qf[qt][ks] = make_uint4(0, 0, 0, 0);
+            if (tq < s) qf[qt][ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
+        }
+    // scores of one stage for this wave's two query tiles, masked keys at -inf
+    auto scores = [&](int buf, int k0, f32x4 (&sc)[4][2]) {
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+            const uint4 a0 = ld_op(Ks[buf], 16 * kt, 0), a1 = ld_op(Ks[buf], 16 * kt, 1);
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                sc[kt][qt] = mfma32(a0, qf[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                sc[kt][qt] = mfma32(a1, qf[qt][1], sc[kt][qt]);
+            }
+        }
+        const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;
+        if (!full) {
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int key = k0 + 16 * kt + 4 * g + i, tq = qlo + 16 * qt + r;
+                        const bool ok = key <= tq && key >= tq + 1 - ws && tq < s;
+                        sc[kt][qt][i] = ok ? sc[kt][qt][i] : -INFINITY;
+                    }
+        }
+    };
+
+    // ---- sweep 1: running maximum and sum ----
+    float mrun[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
+    uint4 kreg[2], vreg[2];
+    load_rows(km, KS * st_lo, kreg);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, k0 = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = kreg[c];
+        }
+        __syncthreads();
+        if (st < st_hi) load_rows(km, k0 + KS, kreg);
+        if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
+        f32x4 sc[4][2];
+        scores(buf, k0, sc);
+#pragma unroll
+        for (int qt = 0; qt < 2; qt++) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) mx = fmaxf(mx, sc[kt][qt][i]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float mnew = fmaxf(mrun[qt], mx * c2);
+            const float mref = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = __builtin_amdgcn_exp2f(mrun[qt] - mref);
+            mrun[qt] = mnew;
+            float part = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) part += __builtin_amdgcn_exp2f(fmaf(sc[kt][qt][i], c2, -mref));
+            lsum[qt] = fmaf(lsum[qt], alpha, part);
+        }
+    }
+    float mc[2], inv[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        float sum = lsum[qt];
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        inv[qt] = sum > 0.f ? 1.0f / sum : 0.f;
+        mc[qt] = mrun[qt] == -INFINITY ? 0.f : mrun[qt];
+    }
+
+    // ---- sweep 2: weights out, O^T = V^T w^T ----
+    f32x4 o[2][4];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    unsigned short *wrow[2];
+    int lsq[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        lsq[qt] = max(tq + 1 - ws, 0);
+        wrow[qt] = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+    }
+    __syncthreads();   // every wave is done with the buffers of sweep 1
+    load_rows(km, KS * st_lo, kreg);
+    load_rows(vm, KS * st_lo, vreg);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, k0 = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = kreg[c];
+            *reinterpret_cast<uint4 *>(&Vs[buf][chunk >> 3][8 * (chunk & 7)]) = vreg[c];
+        }
+        __syncthreads();
+        if (st < st_hi) {
+            load_rows(km, k0 + KS, kreg);
+            load_rows(vm, k0 + KS, vreg);
+        }
+        if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
+        f32x4 sc[4][2];
+        scores(buf, k0, sc);
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            uint4 pb[2];
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                const int tq = qlo + 16 * qt + r;
+                unsigned wp[2][2];
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const f32x4 x = sc[2 * hf + c][qt];
+                    float w[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) w[i] = __builtin_amdgcn_exp2f(fmaf(x[i], c2, -mc[qt])) * inv[qt];
+                    wp[c][0] = pack2(w[0], w[1]);
+                    wp[c][1] = pack2(w[2], w[3]);
+                    // keys key0 .. key0 + 3 of query tq sit in slots key0 - lsq ..; only keys of the window have one
+                    const int key0 = k0 + 16 * (2 * hf + c) + 4 * g;
+                    if (tq < s) {
+                        if (key0 >= lsq[qt] && key0 + 3 <= tq) {
+                            const uint2 pr = make_uint2(wp[c][0], wp[c][1]);
+                            __builtin_memcpy(wrow[qt] + (key0 - lsq[qt]), &pr, 8);
+                        } else if (key0 + 3 >= lsq[qt] && key0 <= tq) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++)
+                                if (key0 + i >= lsq[qt] && key0 + i <= tq)
+                                    wrow[qt][key0 + i - lsq[qt]] = (unsigned short)(wp[c][i >> 1] >> (16 * (i & 1)));
+                        }
+                    }
+                }
+                pb[qt] = make_uint4(wp[0][0], wp[0][1], wp[1][0], wp[1][1]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 av = ld_tr2<LDV>(Vs[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++) o[qt][dt] = mfma32(av, pb[qt], o[qt][dt]);
+            }
+        }
+    }
+    // early queries: the slots behind the query's own key hold zeros
+    if (qlo < ws - 1) {
+        unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+        for (int qi = 0; qi < 32; qi++) {
+            const int tt = qlo + qi;
+            if (tt >= s || tt >= ws - 1) break;
+            for (int slot = tt + 1 + l; slot < ws; slot += 64) awb[(size_t)tt * ws + slot] = 0;
+        }
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        if (tq < s) {
+            unsigned short *ob = out + (row0 + tq) * total + hoff;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+                *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) =
+                    make_uint2(pack2(o[qt][dt][0], o[qt][dt][1]), pack2(o[qt][dt][2], o[qt][dt][3]));
+        }
+    }
+}
+
 // Query pass on statistics, in key blocks like swa_fwd_stats_kernel (one workgroup per 128 queries, one wave per
 // 32), in ONE sweep over the window.  dS = w (dW - D) needs D_t = sum_j w dW of the whole window, so the sweep
 // accumulates the two sums that do not:  A^T = K^T (w dW)^T and B^T = K^T w^T, and D itself, and ends with
@@ -1086,11 +1140,10 @@ bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, u
         check_launch("swa_fwd_stats_kernel");
         return true;
     }
-    const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
-    KernelTimer kt("swa_fwd_mfma_kernel");
-    hipLaunchKernelGGL(swa_fwd_mfma_kernel, grid, dim3(256), 0, stream(), q, k, v, out, attn_weights, seq_len, num_heads,
-                       window);
-    check_launch("swa_fwd_mfma_kernel");
+    KernelTimer kt("swa_fwd_blocked_kernel");
+    hipLaunchKernelGGL(swa_fwd_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+                       k, v, out, attn_weights, seq_len, num_heads, window);
+    check_launch("swa_fwd_blocked_kernel");
     return true;
 }
 
