@@ -146,163 +146,6 @@ __device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int k
     return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
 }
 
-// Backward, query pass (one workgroup per 64 queries, one wave per 16 queries):
-//   D_t = sum_j w dW = dO_t . O_t with O_t = sum_j w[t,j] v_j recomputed from the stored (bf16) weights,
-//   dW[t,j] = dO_t . v_j,  dS = w (dW - D_t) / sqrt(hd),  d_q[t] = sum_j dS[t,j] k_j.
-// Two sweeps over the window: the first rebuilds O^T (four accumulators) and from it D; the second
-// recomputes each dW tile next to its use, so no score tile outlives a stage.  dO and dS enter the
-// bf16 products as hi + lo pairs.  D_t goes to dvec for the key pass.
-//
-// The weights never pass through LDS: the B operand of one query for a 32-key half is one 16-byte
-// load of its weight row, kept in registers for the second sweep.  Only the last stage, the one that
-// holds the queries themselves, is read slot by slot: its groups can end inside the 16 bytes, and a
-// load that runs past the query's row would leave the array at its last row.
-__global__ __launch_bounds__(256, 2) void swa_bwd_q_mfma_kernel(const unsigned short *__restrict__ k,
-                                                                const unsigned short *__restrict__ v,
-                                                                const unsigned short *__restrict__ attn_w,
-                                                                const float *__restrict__ d_out,
-                                                                float *__restrict__ d_q, float *__restrict__ dvec,
-                                                                int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short Vr[2][KS][LDH];   // V stage, [stage_pos(key)][dim]
-    __shared__ __align__(16) unsigned short Tt[2][HD][LDH];   // transposed stage [dim][key]: V (sweep 1), K (sweep 2)
-    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const BlockCoord bc = xcd_block_coord(H);
-    const int t0 = bc.x * QB, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
-    const int base = t0 + QB - NS * KS;
-    const int tq = t0 + 16 * wave + r;
-    const int lsq = max(tq + 1 - ws, 0);
-    const size_t row0 = (size_t)b * s;
-    const int st_lo = max(0, (max(t0 + 1 - ws, 0) - base) / KS);
-    const unsigned short *wrow = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
-    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
-
-    // weights of this lane's query for the keys of its group in a stage: wv[stage][hf] holds the
-    // 8 keys 32 hf + 8 g .. + 7, zero outside the window
-    uint4 wv[NS][2];
-    auto fetch_weights = [&](int stage, uint4 (&w)[2]) {
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            const int key0 = base + KS * stage + 32 * hf + 8 * g;
-            w[hf] = make_uint4(0, 0, 0, 0);
-            if (stage < NS - 1) {
-                // keys below t0: the group never runs past the query; it may start before the window
-                if (tq < s && key0 + 7 >= lsq) {
-                    uint4 x;
-                    __builtin_memcpy(&x, wrow + (key0 - lsq), 16);
-                    w[hf] = mask_below(x, lsq - key0);
-                }
-            } else {
-                unsigned d[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int key = key0 + e;
-                    unsigned x = 0;
-                    if (tq < s && key >= lsq && key <= tq) x = wrow[key - lsq];
-                    d[e >> 1] |= x << (16 * (e & 1));
-                }
-                w[hf] = make_uint4(d[0], d[1], d[2], d[3]);
-            }
-        }
-    };
-    uint4 sv[2], sk[2];
-
-    // ---- sweep 1: O^T = V^T P^T, then D = dO . O ----
-    f32x4 ot[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int st = 0; st < NS; st++) { wv[st][0] = make_uint4(0, 0, 0, 0); wv[st][1] = make_uint4(0, 0, 0, 0); }
-    load_pairs(vm, base + KS * st_lo, sv);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
-        const int buf = st & 1;
-        fetch_weights(st, wv[st]);
-        commit_transposed(Tt[buf], sv);
-        __syncthreads();
-        if (st + 1 < NS) load_pairs(vm, base + KS * (st + 1), sv);
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++)
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) ot[dt] = mfma32(ld_op(Tt[buf], 16 * dt, hf), wv[st][hf], ot[dt]);
-    }
-    // O^T tile dt holds dims 16 dt + 4 g + i of query r
-    float dsum = 0.f;
-    if (tq < s) {
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            const f32x4 x = *reinterpret_cast<const f32x4 *>(d_out + (row0 + tq) * total + hoff + 16 * dt + 4 * g);
-#pragma unroll
-            for (int i = 0; i < 4; i++) dsum = fmaf(x[i], ot[dt][i], dsum);
-        }
-    }
-    dsum += __shfl_xor(dsum, 16, 64);
-    dsum += __shfl_xor(dsum, 32, 64);
-    if (g == 0 && tq < s) dvec[(size_t)(b * H + h) * s + tq] = dsum;
-
-    // ---- sweep 2: dW^T tiles recomputed, dS, d_q^T = K^T dS^T ----
-    uint4 doh[2], dol[2];   // dO_t, dims 32 ks + 8 g .. + 7, as hi + lo
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
-        if (tq < s) {
-            const float *p = d_out + (row0 + tq) * total + hoff + 32 * ks + 8 * g;
-            x0 = *reinterpret_cast<const f32x4 *>(p);
-            x1 = *reinterpret_cast<const f32x4 *>(p + 4);
-        }
-        split8(x0, x1, doh[ks], dol[ks]);
-    }
-    f32x4 dq[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) dq[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const float scale = 0.125f;
-    __syncthreads();
-    load_rows(vm, base + KS * st_lo, sv);
-    load_pairs(km, base + KS * st_lo, sk);
-#pragma unroll
-    for (int st = 0; st < NS; st++) {
-        if (st < st_lo) continue;
-        const int buf = st & 1;
-        commit_rows_tiled(Vr[buf], sv);
-        commit_transposed(Tt[buf], sk);
-        __syncthreads();
-        if (st + 1 < NS) { load_rows(vm, base + KS * (st + 1), sv); load_pairs(km, base + KS * (st + 1), sk); }
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            f32x4 ds[2];
-            const unsigned wd[4] = {wv[st][hf].x, wv[st][hf].y, wv[st][hf].z, wv[st][hf].w};
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW^T[key 32 hf + 8 g + 4 c + i][query r]
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++) {
-                    const uint4 a = ld_op(Vr[buf], 16 * (2 * hf + c), ks);
-                    dw = mfma32(a, doh[ks], dw);
-                    dw = mfma32(a, dol[ks], dw);
-                }
-                ds[c][0] = bf_lo(wd[2 * c]) * (dw[0] - dsum) * scale;
-                ds[c][1] = bf_hi(wd[2 * c]) * (dw[1] - dsum) * scale;
-                ds[c][2] = bf_lo(wd[2 * c + 1]) * (dw[2] - dsum) * scale;
-                ds[c][3] = bf_hi(wd[2 * c + 1]) * (dw[3] - dsum) * scale;
-            }
-            uint4 dsh, dsl;
-            split8(ds[0], ds[1], dsh, dsl);
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const uint4 a = ld_op(Tt[buf], 16 * dt, hf);
-                dq[dt] = mfma32(a, dsh, dq[dt]);
-                dq[dt] = mfma32(a, dsl, dq[dt]);
-            }
-        }
-    }
-    if (tq < s) {
-        float *ob = d_q + (row0 + tq) * total + hoff;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = dq[dt];
-    }
-}
-
 // Backward, key pass (one workgroup per 64 keys, one wave per 16 keys): over the up to 575
 // queries t in [j, j + window) that see key j,
 //   d_v[j] += sum_t w[t,j] dO_t,   d_k[j] += sum_t dS[t,j] q_t,   dS recomputed from w, dO.v_j, D_t.
@@ -972,6 +815,158 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
     }
 }
 
+// Query pass of the contract (weights read back from the tensor) in the same blocks and the same single sweep as
+// swa_bwd_q_stats_kernel: A = sum_j (w dW) k_j, B = sum_j w k_j and D = sum_j w dW together, d_q = (A - D B)/sqrt(hd).
+// A lane's four keys of a tile are four consecutive slots of its query's row: one 8-byte load (2-byte aligned),
+// requested a stage ahead; only the stages at the two ends of the window go slot by slot.
+__global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigned short *__restrict__ k,
+                                                                   const unsigned short *__restrict__ v,
+                                                                   const unsigned short *__restrict__ attn_w,
+                                                                   const float *__restrict__ d_out,
+                                                                   float *__restrict__ d_q, float *__restrict__ dvec,
+                                                                   int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Ks[2][KS][LDH], Vs[2][KS][LDH];   // stages [key][dim]
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int qlo = t0 + 32 * wave, qhi = qlo + 31;
+    const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
+    const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
+    const float scale = 0.125f;
+
+    uint4 doh[2][2], dol[2][2];
+    const unsigned short *wrow[2];
+    int lsq[2], tqs[2];
+    float dpart[2] = {0.f, 0.f};
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        tqs[qt] = tq < s ? tq : -1;   // -1: no key passes "key <= tq"
+        lsq[qt] = max(tq + 1 - ws, 0);
+        wrow[qt] = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
+            if (tq < s) {
+                const size_t o = (row0 + tq) * total + hoff + 32 * ks + 8 * g;
+                x0 = *reinterpret_cast<const f32x4 *>(d_out + o);
+                x1 = *reinterpret_cast<const f32x4 *>(d_out + o + 4);
+            }
+            split8(x0, x1, doh[qt][ks], dol[qt][ks]);
+        }
+    }
+    f32x4 aq[2][4], bq[2][4];
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) { aq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; bq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+    // weights of a stage for this lane: wreg[kt][qt] = keys k0 + 16 kt + 4 g .. + 3 of query qt, zero outside the window
+    uint2 wreg[4][2];
+    auto fetch_weights = [&](int k0) {
+        const bool skip = k0 > qhi || k0 + KS - 1 < qlo + 1 - ws;
+        const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                const int key0 = k0 + 16 * kt + 4 * g;
+                wreg[kt][qt] = make_uint2(0u, 0u);
+                if (skip) continue;
+                if (full || (key0 >= lsq[qt] && key0 + 3 <= tqs[qt])) {
+                    __builtin_memcpy(&wreg[kt][qt], wrow[qt] + (key0 - lsq[qt]), 8);
+                } else {
+                    unsigned d[2] = {0u, 0u};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int key = key0 + e;
+                        unsigned x = 0;
+                        if (key >= lsq[qt] && key <= tqs[qt]) x = wrow[qt][key - lsq[qt]];
+                        d[e >> 1] |= x << (16 * (e & 1));
+                    }
+                    wreg[kt][qt] = make_uint2(d[0], d[1]);
+                }
+            }
+    };
+
+    uint4 kreg[2], vreg[2];
+    load_rows(km, KS * st_lo, kreg);
+    load_rows(vm, KS * st_lo, vreg);
+    fetch_weights(KS * st_lo);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, k0 = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = kreg[c];
+            *reinterpret_cast<uint4 *>(&Vs[buf][chunk >> 3][8 * (chunk & 7)]) = vreg[c];
+        }
+        uint2 wcur[4][2];
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) wcur[kt][qt] = wreg[kt][qt];
+        __syncthreads();
+        if (st < st_hi) {
+            load_rows(km, k0 + KS, kreg);
+            load_rows(vm, k0 + KS, vreg);
+            fetch_weights(k0 + KS);
+        }
+        if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            uint4 xh[2], xl[2], wb[2];
+#pragma unroll
+            for (int qt = 0; qt < 2; qt++) {
+                f32x4 x[2];
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const int kt = 2 * hf + c;
+                    const uint4 av0 = ld_op(Vs[buf], 16 * kt, 0), av1 = ld_op(Vs[buf], 16 * kt, 1);
+                    f32x4 dw = mfma32(av0, doh[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                    dw = mfma32(av0, dol[qt][0], dw);
+                    dw = mfma32(av1, doh[qt][1], dw);
+                    dw = mfma32(av1, dol[qt][1], dw);
+                    const uint2 wp = wcur[kt][qt];
+                    x[c][0] = bf_lo(wp.x) * dw[0];
+                    x[c][1] = bf_hi(wp.x) * dw[1];
+                    x[c][2] = bf_lo(wp.y) * dw[2];
+                    x[c][3] = bf_hi(wp.y) * dw[3];
+                    dpart[qt] += (x[c][0] + x[c][1]) + (x[c][2] + x[c][3]);
+                }
+                split8(x[0], x[1], xh[qt], xl[qt]);
+                wb[qt] = make_uint4(wcur[2 * hf][qt].x, wcur[2 * hf][qt].y, wcur[2 * hf + 1][qt].x, wcur[2 * hf + 1][qt].y);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 a = ld_tr2<LDH>(Ks[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++) {
+                    aq[qt][dt] = mfma32(a, xh[qt], aq[qt][dt]);
+                    aq[qt][dt] = mfma32(a, xl[qt], aq[qt][dt]);
+                    bq[qt][dt] = mfma32(a, wb[qt], bq[qt][dt]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++) {
+        const int tq = qlo + 16 * qt + r;
+        float dsum = dpart[qt];
+        dsum += __shfl_xor(dsum, 16, 64);
+        dsum += __shfl_xor(dsum, 32, 64);
+        if (tq < s) {
+            if (g == 0) dvec[(size_t)(b * H + h) * s + tq] = dsum;
+            float *ob = d_q + (row0 + tq) * total + hoff;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+                *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
+        }
+    }
+}
+
 // Key pass on statistics, in query blocks (one workgroup per 128 keys, one wave per 32): over the stages of 64
 // queries that see the block's keys, a wave forms S = Q K^T for its two key tiles (rows = queries, column = the
 // lane's key), the weights from the queries' statistics, dW = dO V^T, dS = w (dW - D_t) / sqrt(hd), and
@@ -1171,10 +1166,10 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
     }
     const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
     {
-        KernelTimer kt("swa_bwd_q_mfma_kernel");
-        hipLaunchKernelGGL(swa_bwd_q_mfma_kernel, grid, dim3(256), 0, stream(), k, v, attn_weights, d_attn_out, d_q, dvec,
-                           seq_len, num_heads, window);
-        check_launch("swa_bwd_q_mfma_kernel");
+        KernelTimer kt("swa_bwd_q_blocked_kernel");
+        hipLaunchKernelGGL(swa_bwd_q_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0,
+                           stream(), k, v, attn_weights, d_attn_out, d_q, dvec, seq_len, num_heads, window);
+        check_launch("swa_bwd_q_blocked_kernel");
     }
     KernelTimer kt("swa_bwd_k_mfma_kernel");
     hipLaunchKernelGGL(swa_bwd_k_mfma_kernel, grid, dim3(256), 0, stream(), q, v, attn_weights, d_attn_out, dvec, d_k,
