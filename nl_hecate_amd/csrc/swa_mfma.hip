@@ -8,21 +8,17 @@
 // elements per lane: lane (r = l % 16, g = l / 16) supplies row r, contraction
 // elements 8 g .. 8 g + 7 of a 32-wide step.
 //
-// Key order.  A 16x16 result tile leaves four rows 4 g + i in a lane.  Where such
-// tiles become an operand again with the keys as contraction index (the weights in
-// O^T = V^T P^T, dS in d_q^T = K^T dS^T), two tiles (c = 0, 1) of a 32-key half hf
-// give the lane its 8 elements; row 4 g + i of tile (hf, c) therefore stands for key
-// 32 hf + 8 g + 4 c + i of the stage, so that those 8 elements are 8 CONSECUTIVE
-// keys: the matching operand is a plain 16-byte LDS read, and in the weight array
-// they are 16 consecutive bytes of the query's slot row (a 2-byte aligned 16-byte
-// access).  A tile's rows come from an LDS matrix whose rows are stored in that
-// order (stage_pos).
-//
-// That order serves the two backward kernels of the contract, which read the stored weights 16 bytes at a time.
-// The forward of the contract (swa_fwd_blocked_kernel) and the pair that keeps two statistics per query instead
-// of the weight tensor (swa_*_stats_kernel) work in blocks of 64 keys with a running maximum, stage every row
-// block as it arrives and read transposed operands through ds_read_b64_tr_b16; they share only the helpers with
-// the two kernels above them.
+// Every kernel works in blocks: one workgroup per 128 queries (keys in the key passes), one wave per 32, stages
+// of 64 keys (queries) whose rows are staged in LDS exactly as they arrive.  A 16x16 result tile leaves rows
+// 4 g + i in a lane; where two such tiles become an operand again with their rows as contraction index (the
+// weights in O^T = V^T w^T, dS in d_q^T = K^T dS^T, ..), the matching operand is read from the row-major stage
+// through ds_read_b64_tr_b16 with group g taking rows 32 hf + 4 g .. + 3 and 32 hf + 16 + 4 g .. + 3 — the rows
+// the two tiles left in that group's lanes — so no stage is ever written transposed or in a permuted order.
+// No kernel holds more than one stage of scores: the forward keeps a running maximum (two sweeps where the
+// contract wants the normalised weights stored), the query passes accumulate A = sum (w dW) k, B = sum w k and
+// D = sum w dW in one sweep and finish with d_q = (A - D B) / sqrt(hd).
+//   contract (weights stored / read back):  swa_fwd_blocked_kernel, swa_bwd_q_blocked_kernel, swa_bwd_k_blocked_kernel
+//   two statistics per query instead:       swa_fwd_stats_kernel,   swa_bwd_q_stats_kernel,   swa_bwd_k_stats_kernel
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -39,10 +35,7 @@ typedef __bf16 bh2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int HD = 64;        // head size
-constexpr int QB = 64;        // queries per workgroup
 constexpr int KS = 64;        // keys per LDS stage
-constexpr int NS = 9;         // stages: 576 keys
-constexpr int NT = 36;        // 16-key tiles
 constexpr int LDH = 72;       // LDS row stride in bf16 elements (144 B: 16-byte rows, conflict-free operand reads)
 
 __device__ __forceinline__ f32x4 mfma32(uint4 a, uint4 b, f32x4 c) {
@@ -66,21 +59,6 @@ __device__ __forceinline__ void split8(f32x4 a, f32x4 b, uint4 &hi, uint4 &lo) {
     split2(b[0], b[1], hi.z, lo.z);
     split2(b[2], b[3], hi.w, lo.w);
 }
-// position of a stage's key 32 a + 8 g + 4 c + i in tile order: 16 (2 a + c) + 4 g + i
-__device__ __forceinline__ int stage_pos(int key) {
-    return (key & 0x23) | ((key & 0x18) >> 1) | ((key & 0x04) << 2);
-}
-// key (relative to the stage) of element i of lane group g in tile kt
-__device__ __forceinline__ int tile_key(int kt, int g, int i) { return 32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i; }
-// clears the elements below cut of 8 packed bf16
-__device__ __forceinline__ uint4 mask_below(uint4 x, int cut) {
-    x.x &= (cut > 0 ? 0u : 0xffffu) | (cut > 1 ? 0u : 0xffff0000u);
-    x.y &= (cut > 2 ? 0u : 0xffffu) | (cut > 3 ? 0u : 0xffff0000u);
-    x.z &= (cut > 4 ? 0u : 0xffffu) | (cut > 5 ? 0u : 0xffff0000u);
-    x.w &= (cut > 6 ? 0u : 0xffffu) | (cut > 7 ? 0u : 0xffff0000u);
-    return x;
-}
-
 // Workgroup -> (block of the sequence, head * batch) with all blocks of one head on one XCD.
 // Workgroups go to the 8 XCDs round robin in linear order, and each XCD has its own L2; blocks
 // of one head share K and V rows, so they are given linear ids that are equal modulo 8.
@@ -97,9 +75,8 @@ __device__ __forceinline__ BlockCoord xcd_block_coord(int H) {
     return BlockCoord{x, bh % H, bh / H};
 }
 
-// Cooperative loads of one stage (64 rows of 64 bf16 = 512 chunks of 16 B, two per thread of a
-// 256-thread block).  rows: chunk = (row, 8 dims), consecutive lanes along a row.  pairs: the thread
-// takes 8 dims of two neighbouring rows, for a transposed tile written as 32-bit row pairs.
+// Cooperative load of one stage (64 rows of 64 bf16 = 512 chunks of 16 B, two per thread of a
+// 256-thread block): chunk = (row, 8 dims), consecutive lanes along a row.
 struct StageSrc { const unsigned short *p; size_t row0; int total, hoff, s; };
 __device__ __forceinline__ void load_rows(const StageSrc &m, int first, uint4 (&regs)[2]) {
     const int tid = threadIdx.x;
@@ -111,215 +88,10 @@ __device__ __forceinline__ void load_rows(const StageSrc &m, int first, uint4 (&
             regs[c] = *reinterpret_cast<const uint4 *>(m.p + (m.row0 + row) * m.total + m.hoff + 8 * (chunk & 7));
     }
 }
-__device__ __forceinline__ void load_pairs(const StageSrc &m, int first, uint4 (&regs)[2]) {
-    const int tid = threadIdx.x, kp = tid & 31, d0 = 8 * (tid >> 5);
-#pragma unroll
-    for (int c = 0; c < 2; c++) {
-        const int row = first + 2 * kp + c;
-        regs[c] = make_uint4(0, 0, 0, 0);
-        if (row >= 0 && row < m.s) regs[c] = *reinterpret_cast<const uint4 *>(m.p + (m.row0 + row) * m.total + m.hoff + d0);
-    }
-}
-// rows in tile order: row -> T[stage_pos(row)][dim]
-__device__ __forceinline__ void commit_rows_tiled(unsigned short (*T)[LDH], const uint4 (&regs)[2]) {
-    const int tid = threadIdx.x;
-#pragma unroll
-    for (int c = 0; c < 2; c++) {
-        const int chunk = tid + 256 * c;
-        *reinterpret_cast<uint4 *>(&T[stage_pos(chunk >> 3)][8 * (chunk & 7)]) = regs[c];
-    }
-}
-// transposed: T[dim][row], rows in natural order (bank = row pair: no conflicts)
-__device__ __forceinline__ void commit_transposed(unsigned short (*T)[LDH], const uint4 (&regs)[2]) {
-    const int tid = threadIdx.x, col = 2 * (tid & 31), d0 = 8 * (tid >> 5);
-    const unsigned e[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
-    const unsigned o[4] = {regs[1].x, regs[1].y, regs[1].z, regs[1].w};
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        *reinterpret_cast<unsigned *>(&T[d0 + 2 * j][col]) = (e[j] & 0xffffu) | (o[j] << 16);
-        *reinterpret_cast<unsigned *>(&T[d0 + 2 * j + 1][col]) = (e[j] >> 16) | (o[j] & 0xffff0000u);
-    }
-}
 // operand of a 32-wide step: row r of the tile at row0, contraction elements 32 ks + 8 g .. + 7
 __device__ __forceinline__ uint4 ld_op(unsigned short (*T)[LDH], int row0, int ks) {
     const int l = threadIdx.x & 63;
     return *reinterpret_cast<const uint4 *>(&T[row0 + (l & 15)][32 * ks + 8 * (l >> 4)]);
-}
-
-// Backward, key pass (one workgroup per 64 keys, one wave per 16 keys): over the up to 575
-// queries t in [j, j + window) that see key j,
-//   d_v[j] += sum_t w[t,j] dO_t,   d_k[j] += sum_t dS[t,j] q_t,   dS recomputed from w, dO.v_j, D_t.
-// Two tiles of dS / w in accumulator layout (rows = queries, column = the lane's key) are the A
-// operand of the products with Q^T / dO^T, which are staged transposed in LDS; the rows of the
-// dO stage are stored in tile order (stage_pos) so that those 8 rows are 8 consecutive queries.
-__global__ __launch_bounds__(256) void swa_bwd_k_mfma_kernel(const unsigned short *__restrict__ q,
-                                                             const unsigned short *__restrict__ v,
-                                                             const unsigned short *__restrict__ attn_w,
-                                                             const float *__restrict__ d_out,
-                                                             const float *__restrict__ dvec,
-                                                             float *__restrict__ d_k, float *__restrict__ d_v,
-                                                             int s, int H, int ws) {
-    __shared__ __align__(16) unsigned short Dh[KS][LDH], Dl[KS][LDH];      // dO hi / lo, [stage_pos(query)][dim]
-    __shared__ __align__(16) unsigned short DhT[HD][LDH], DlT[HD][LDH];    // transposed, [dim][query]
-    __shared__ __align__(16) unsigned short QT[HD][LDH];                   // Q^T, [dim][query]
-    __shared__ __align__(16) unsigned short Pt[KS][LDH];                   // weights, [query][key of the block]
-    __shared__ float Dv[KS];
-    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-    const BlockCoord bc = xcd_block_coord(H);
-    const int j0 = bc.x * QB, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
-    const size_t row0 = (size_t)b * s;
-    const int kj = j0 + 16 * wave + r;   // this lane's key (B-operand / accumulator column)
-    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
-    const float *dvb = dvec + (size_t)(b * H + h) * s;
-    const StageSrc qm{q, row0, total, hoff, s};
-
-    uint4 vf[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        vf[ks] = make_uint4(0, 0, 0, 0);
-        if (kj < s) vf[ks] = *reinterpret_cast<const uint4 *>(v + (row0 + kj) * total + hoff + 32 * ks + 8 * g);
-    }
-    f32x4 dk[4], dv[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) { dk[i] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-    const float scale = 0.125f;
-    const int t_last = min(s - 1, j0 + QB - 1 + ws - 1);
-
-    // global -> register fetch of one stage (64 queries), issued one stage ahead of its use
-    f32x4 gdo[4];
-    uint4 gq[2];
-    unsigned short gw[16];
-    uint4 gwv[2];
-    float gd = 0.f;
-    // dO: query pair (2 rows) x 4 dims per load; pairs so that the transposed tiles are written as
-    // 32-bit words without bank conflicts
-    const int dpair = r + 16 * (wave & 1), dd0 = 4 * g + 16 * (wave >> 1);   // query pair, first dim (+32 for the second half)
-    auto fetch_stage = [&](int st) {
-        const int qs0 = j0 + KS * st;
-#pragma unroll
-        for (int cc = 0; cc < 2; cc++)
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int t = qs0 + 2 * dpair + c;
-                gdo[2 * cc + c] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (t < s) gdo[2 * cc + c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dd0 + 32 * cc);
-            }
-        load_pairs(qm, qs0, gq);
-        // weights of the block's 64 keys for the stage's 64 queries: row t, slots j - ls(t).
-        // Past the first stage every query lies after all keys of the block, so a group of 8 keys
-        // never runs past the query's row: one 16-byte load (2-byte aligned) per group, the keys
-        // before the window masked.  The first stage is read slot by slot.
-        if (st == 0) {
-#pragma unroll
-            for (int c = 0; c < 16; c++) {
-                const int t = qs0 + 4 * c + wave, key = j0 + l;
-                const int slot = key - max(t + 1 - ws, 0);
-                gw[c] = 0;
-                if (t < s && key <= t && slot >= 0 && slot < ws) gw[c] = awb[(size_t)t * ws + slot];
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int chunk = tid + 256 * c, t = qs0 + (chunk >> 3), key0 = j0 + 8 * (chunk & 7);
-                const int ls = max(t + 1 - ws, 0);
-                gwv[c] = make_uint4(0, 0, 0, 0);
-                if (t < s && key0 + 7 >= ls) {
-                    uint4 x;
-                    __builtin_memcpy(&x, awb + (size_t)t * ws + (key0 - ls), 16);
-                    gwv[c] = mask_below(x, ls - key0);
-                }
-            }
-        }
-        gd = (tid < KS && qs0 + tid < s) ? dvb[qs0 + tid] : 0.f;
-    };
-    fetch_stage(0);
-    for (int st = 0; st < NS; st++) {
-        const int qs0 = j0 + KS * st;
-        if (qs0 > t_last) break;
-        __syncthreads();   // previous stage's readers are done
-#pragma unroll
-        for (int cc = 0; cc < 2; cc++) {
-            unsigned hi[2][2], lo[2][2];
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const f32x4 x = gdo[2 * cc + c];
-                split2(x[0], x[1], hi[c][0], lo[c][0]);
-                split2(x[2], x[3], hi[c][1], lo[c][1]);
-                const int row = stage_pos(2 * dpair + c);
-                *reinterpret_cast<uint2 *>(&Dh[row][dd0 + 32 * cc]) = make_uint2(hi[c][0], hi[c][1]);
-                *reinterpret_cast<uint2 *>(&Dl[row][dd0 + 32 * cc]) = make_uint2(lo[c][0], lo[c][1]);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const unsigned h0 = hi[0][j >> 1], h1 = hi[1][j >> 1], l0 = lo[0][j >> 1], l1 = lo[1][j >> 1];
-                *reinterpret_cast<unsigned *>(&DhT[dd0 + 32 * cc + j][2 * dpair]) =
-                    (j & 1) ? ((h0 >> 16) | (h1 & 0xffff0000u)) : ((h0 & 0xffffu) | (h1 << 16));
-                *reinterpret_cast<unsigned *>(&DlT[dd0 + 32 * cc + j][2 * dpair]) =
-                    (j & 1) ? ((l0 >> 16) | (l1 & 0xffff0000u)) : ((l0 & 0xffffu) | (l1 << 16));
-            }
-        }
-        commit_transposed(QT, gq);
-        if (st == 0) {
-#pragma unroll
-            for (int c = 0; c < 16; c++) Pt[4 * c + wave][l] = gw[c];
-        } else {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int chunk = tid + 256 * c;
-                *reinterpret_cast<uint4 *>(&Pt[chunk >> 3][8 * (chunk & 7)]) = gwv[c];
-            }
-        }
-        if (tid < KS) Dv[tid] = gd;
-        __syncthreads();
-        if (qs0 + KS <= t_last) fetch_stage(st + 1);
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            f32x4 ds[2];
-            unsigned pw[2][2];
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                f32x4 dw = f32x4{0.f, 0.f, 0.f, 0.f};   // dW[query 32 hf + 8 g + 4 c + i][key r of this wave]
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++) {
-                    dw = mfma32(ld_op(Dh, 16 * (2 * hf + c), ks), vf[ks], dw);
-                    dw = mfma32(ld_op(Dl, 16 * (2 * hf + c), ks), vf[ks], dw);
-                }
-                unsigned short p4[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int qi = 32 * hf + 8 * g + 4 * c + i;
-                    p4[i] = Pt[qi][16 * wave + r];
-                    ds[c][i] = __uint_as_float((unsigned)p4[i] << 16) * (dw[i] - Dv[qi]) * scale;
-                }
-                pw[c][0] = (unsigned)p4[0] | ((unsigned)p4[1] << 16);
-                pw[c][1] = (unsigned)p4[2] | ((unsigned)p4[3] << 16);
-            }
-            const uint4 pa = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
-            uint4 dsh, dsl;
-            split8(ds[0], ds[1], dsh, dsl);
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const uint4 bh = ld_op(DhT, 16 * dt, hf), bl = ld_op(DlT, 16 * dt, hf), bq = ld_op(QT, 16 * dt, hf);
-                dv[dt] = mfma32(pa, bh, dv[dt]);
-                dv[dt] = mfma32(pa, bl, dv[dt]);
-                dk[dt] = mfma32(dsh, bq, dk[dt]);
-                dk[dt] = mfma32(dsl, bq, dk[dt]);
-            }
-        }
-    }
-    // accumulate: rows = keys 16 wave + 4g + i, column = dim 16 dt + r
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int key = j0 + 16 * wave + 4 * g + i;
-        if (key >= s) continue;
-        float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            pk[16 * dt + r] += dk[dt][i];
-            pv[16 * dt + r] += dv[dt][i];
-        }
-    }
 }
 
 // Forward that keeps statistics instead of weights, in blocks of keys with a running maximum (no score
@@ -1123,6 +895,160 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
     }
 }
 
+// Key pass of the contract in query blocks, like swa_bwd_k_stats_kernel, with the weights read back from the tensor:
+// the stage's 64 query rows x the block's 128 keys are 256 contiguous bytes per query where the window covers them;
+// they are staged in LDS as [query][key] and a lane takes its two tiles (rows = queries, column = its key) with one
+// transposing read, which is both the B operand of d_v^T += dO^T w and the w of dS = w (dW - D_t) / sqrt(hd).
+constexpr int LDW = 144;   // row stride of the weight stage (288 B: the transposing reads of a group fall on 32 banks)
+
+__global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigned short *__restrict__ q,
+                                                                   const unsigned short *__restrict__ v,
+                                                                   const unsigned short *__restrict__ attn_w,
+                                                                   const float *__restrict__ d_out,
+                                                                   const float *__restrict__ dvec,
+                                                                   float *__restrict__ d_k, float *__restrict__ d_v,
+                                                                   int s, int H, int ws) {
+    __shared__ __align__(16) unsigned short Qs[2][KS][LDH], Dh[2][KS][LDH], Dl[2][KS][LDH];   // [query][dim]
+    __shared__ __align__(16) unsigned short Wt[KS][LDW];                                       // [query][key of the block]
+    __shared__ __align__(16) float Dd[2][KS];
+    const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+    const BlockCoord bc = xcd_block_coord(H);
+    const int j0 = bc.x * FQ, h = bc.h, b = bc.b;
+    const int total = H * HD, hoff = h * HD;
+    const size_t row0 = (size_t)b * s;
+    const int jlo = j0 + 32 * wave, jhi = jlo + 31;
+    const int st_lo = j0 / KS, st_hi = min(s - 1, j0 + FQ - 1 + ws - 1) / KS;
+    const float *dvb = dvec + (size_t)(b * H + h) * s;
+    const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
+    const StageSrc qm{q, row0, total, hoff, s};
+    const float scale = 0.125f;
+
+    uint4 vf[2][2];
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const int key = jlo + 16 * jt + r;
+            vf[jt][ks] = make_uint4(0, 0, 0, 0);
+            if (key < s) vf[jt][ks] = *reinterpret_cast<const uint4 *>(v + (row0 + key) * total + hoff + 32 * ks + 8 * g);
+        }
+    f32x4 dk[2][4], dv[2][4];
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) { dk[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+    uint4 qreg[2], wreg[4];
+    f32x4 dreg[4];
+    float ddreg = 0.f;
+    const int drow = tid >> 2, dcol = 16 * (tid & 3);
+    auto fetch_stage = [&](int t_lo) {
+        load_rows(qm, t_lo, qreg);
+        const int t = t_lo + drow;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            dreg[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (t < s) dreg[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dcol + 4 * c);
+        }
+        ddreg = (tid < KS && t_lo + tid < s) ? dvb[t_lo + tid] : 0.f;
+        // weights of query t for keys j0 + 32 (tid % 4) .. + 31: four pieces of 8 keys
+        const int lsq = max(t + 1 - ws, 0), thi = t < s ? t : -1;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int key0 = j0 + 32 * (tid & 3) + 8 * c;
+            wreg[c] = make_uint4(0, 0, 0, 0);
+            if (key0 >= lsq && key0 + 7 <= thi) {
+                __builtin_memcpy(&wreg[c], awb + (size_t)t * ws + (key0 - lsq), 16);
+            } else if (key0 + 7 >= lsq && key0 <= thi) {
+                unsigned d[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int key = key0 + e;
+                    unsigned x = 0;
+                    if (key >= lsq && key <= thi) x = awb[(size_t)t * ws + (key - lsq)];
+                    d[e >> 1] |= x << (16 * (e & 1));
+                }
+                wreg[c] = make_uint4(d[0], d[1], d[2], d[3]);
+            }
+        }
+    };
+    fetch_stage(KS * st_lo);
+    for (int st = st_lo; st <= st_hi; st++) {
+        const int buf = (st - st_lo) & 1, t_lo = KS * st;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int chunk = tid + 256 * c;
+            *reinterpret_cast<uint4 *>(&Qs[buf][chunk >> 3][8 * (chunk & 7)]) = qreg[c];
+            uint4 hi, lo;
+            split8(dreg[2 * c], dreg[2 * c + 1], hi, lo);
+            *reinterpret_cast<uint4 *>(&Dh[buf][drow][dcol + 8 * c]) = hi;
+            *reinterpret_cast<uint4 *>(&Dl[buf][drow][dcol + 8 * c]) = lo;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) *reinterpret_cast<uint4 *>(&Wt[drow][32 * (tid & 3) + 8 * c]) = wreg[c];
+        if (tid < KS) Dd[buf][tid] = ddreg;
+        __syncthreads();
+        if (st < st_hi) fetch_stage(t_lo + KS);
+        if (!(t_lo + KS - 1 < jlo || t_lo > jhi + ws - 1)) {   // a query of this stage sees a key of this wave
+#pragma unroll
+            for (int hq = 0; hq < 2; hq++) {
+                const int ra = 32 * hq + 4 * g, rb = ra + 16;
+                uint4 wpk[2], dsh[2], dsl[2];
+                f32x4 ds[2][2];
+#pragma unroll
+                for (int jt = 0; jt < 2; jt++) wpk[jt] = ld_tr2<LDW>(Wt, ra, rb, 32 * wave + 16 * jt);
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const int qt = 2 * hq + c;
+                    const uint4 ah0 = ld_op(Dh[buf], 16 * qt, 0), ah1 = ld_op(Dh[buf], 16 * qt, 1);
+                    const uint4 al0 = ld_op(Dl[buf], 16 * qt, 0), al1 = ld_op(Dl[buf], 16 * qt, 1);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&Dd[buf][16 * qt + 4 * g]);
+#pragma unroll
+                    for (int jt = 0; jt < 2; jt++) {
+                        f32x4 dw = mfma32(ah0, vf[jt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                        dw = mfma32(al0, vf[jt][0], dw);
+                        dw = mfma32(ah1, vf[jt][1], dw);
+                        dw = mfma32(al1, vf[jt][1], dw);
+                        const unsigned w01 = c ? wpk[jt].z : wpk[jt].x, w23 = c ? wpk[jt].w : wpk[jt].y;
+                        ds[jt][c][0] = bf_lo(w01) * (dw[0] - d4[0]) * scale;
+                        ds[jt][c][1] = bf_hi(w01) * (dw[1] - d4[1]) * scale;
+                        ds[jt][c][2] = bf_lo(w23) * (dw[2] - d4[2]) * scale;
+                        ds[jt][c][3] = bf_hi(w23) * (dw[3] - d4[3]) * scale;
+                    }
+                }
+#pragma unroll
+                for (int jt = 0; jt < 2; jt++) split8(ds[jt][0], ds[jt][1], dsh[jt], dsl[jt]);
+#pragma unroll
+                for (int dt = 0; dt < 4; dt++) {
+                    const uint4 aq = ld_tr2<LDH>(Qs[buf], ra, rb, 16 * dt);    // Q^T [dim][query]
+                    const uint4 ah = ld_tr2<LDH>(Dh[buf], ra, rb, 16 * dt);    // dO^T hi / lo
+                    const uint4 al = ld_tr2<LDH>(Dl[buf], ra, rb, 16 * dt);
+#pragma unroll
+                    for (int jt = 0; jt < 2; jt++) {
+                        dk[jt][dt] = mfma32(aq, dsh[jt], dk[jt][dt]);
+                        dk[jt][dt] = mfma32(aq, dsl[jt], dk[jt][dt]);
+                        dv[jt][dt] = mfma32(ah, wpk[jt], dv[jt][dt]);
+                        dv[jt][dt] = mfma32(al, wpk[jt], dv[jt][dt]);
+                    }
+                }
+            }
+        }
+        __syncthreads();   // the weight stage has one buffer: every wave is done with it before the next one lands
+    }
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+        const int key = jlo + 16 * jt + r;
+        if (key >= s) continue;
+        float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            f32x4 *ck = reinterpret_cast<f32x4 *>(pk + 16 * dt + 4 * g), *cv = reinterpret_cast<f32x4 *>(pv + 16 * dt + 4 * g);
+            *ck = *ck + dk[jt][dt];
+            *cv = *cv + dv[jt][dt];
+        }
+    }
+}
+
 }  // namespace
 
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
@@ -1164,17 +1090,16 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
         check_launch("swa_bwd_k_stats_kernel");
         return true;
     }
-    const dim3 grid((seq_len + QB - 1) / QB, num_heads, batch);
     {
         KernelTimer kt("swa_bwd_q_blocked_kernel");
         hipLaunchKernelGGL(swa_bwd_q_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0,
                            stream(), k, v, attn_weights, d_attn_out, d_q, dvec, seq_len, num_heads, window);
         check_launch("swa_bwd_q_blocked_kernel");
     }
-    KernelTimer kt("swa_bwd_k_mfma_kernel");
-    hipLaunchKernelGGL(swa_bwd_k_mfma_kernel, grid, dim3(256), 0, stream(), q, v, attn_weights, d_attn_out, dvec, d_k,
-                       d_v, seq_len, num_heads, window);
-    check_launch("swa_bwd_k_mfma_kernel");
+    KernelTimer kt("swa_bwd_k_blocked_kernel");
+    hipLaunchKernelGGL(swa_bwd_k_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+                       v, attn_weights, d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
+    check_launch("swa_bwd_k_blocked_kernel");
     return true;
 }
 
