@@ -58,6 +58,11 @@ int nlh_selftest_lane_ops(void);
  * cl, bl, rl, keep, eta, theta, then a_L, beta_L, h_L.  0 on success.  For tests. */
 int nlh_selftest_chunk_coef(const float *alpha, const float *theta, const float *eta, int L, float *tj,
                             float *jt, float *vecs);
+/* The same chunk through the helpers of the coefficient pre-passes (scans for the vectors, per-lane column walk for
+ * the table): table [64][64] = c[t][j], table_scaled = -theta_j c[t][j] (both zero outside j <= t < L);
+ * vecs [5][64] = a, beta, h of G(0..t) and cl, bl of G(t+1..63).  0 on success.  For tests. */
+int nlh_selftest_chunk_coef_prepass(const float *alpha, const float *theta, const float *eta, int L, float *table,
+                                    float *table_scaled, float *vecs);
 
 /* ── Titans LMM, exact per-token rule ───────────────────────────────────────
  * Per token: e = clip(M k - v); S = eta S - theta e k^T; M = (1-alpha) M + S;

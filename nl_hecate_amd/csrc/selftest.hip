@@ -157,3 +157,36 @@ extern "C" int nlh_selftest_chunk_coef(const float *alpha, const float *theta, c
     hipLaunchKernelGGL(chunk_coef_kernel, dim3(1), dim3(64), 0, stream(), alpha, theta, eta, L, tj, jt, vecs);
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
+
+namespace nlh {
+// The helpers of the coefficient pre-passes on one chunk: table[t][j] = theta-free c[t][j] and, with scale = -theta_j,
+// the forward's W[t][j]; vecs [5][64] = a, beta, h, cl, bl of token (lane).
+__global__ void chunk_coef_prepass_kernel(const float *alpha, const float *theta, const float *eta, int L,
+                                          float *table, float *table_scaled, float *vecs) {
+    constexpr int LD = 68;
+    __shared__ __align__(16) float stage[65 * LD];
+    __shared__ float gk[128], ge[128];
+    const int l = threadIdx.x;
+    const bool in = l < L;
+    const float keep = in ? 1.f - alpha[l] : 1.f, et = in ? eta[l] : 0.f, nth = in ? -theta[l] : 0.f;
+    const ChunkVectors cv = coef_vectors(keep, et, in);
+    vecs[0 * 64 + l] = cv.a;
+    vecs[1 * 64 + l] = cv.beta;
+    vecs[2 * 64 + l] = cv.h;
+    vecs[3 * 64 + l] = cv.cl;
+    vecs[4 * 64 + l] = cv.bl;
+    coef_table_columns<LD, false>(stage, gk, ge, keep, et, 1.f, L);
+    for (int t = 0; t < 64; t++) table[t * 64 + l] = stage[t * LD + l];
+    coef_table_columns<LD, true>(stage, gk, ge, keep, et, nth, L);
+    for (int t = 0; t < 64; t++) table_scaled[t * 64 + l] = stage[t * LD + l];
+}
+}  // namespace nlh
+
+extern "C" int nlh_selftest_chunk_coef_prepass(const float *alpha, const float *theta, const float *eta, int L,
+                                               float *table, float *table_scaled, float *vecs) {
+    using namespace nlh;
+    if (L < 1 || L > 64) return -1;
+    hipLaunchKernelGGL(chunk_coef_prepass_kernel, dim3(1), dim3(64), 0, stream(), alpha, theta, eta, L, table,
+                       table_scaled, vecs);
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}

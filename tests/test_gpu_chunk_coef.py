@@ -74,3 +74,38 @@ def test_generated_coefficients_match_the_recurrences(kind, L):
     np.testing.assert_allclose(vecs[5][:L], r[L - 1, :L], err_msg="rl", **tol)
     np.testing.assert_allclose(vecs[8], z(th), err_msg="theta", **tol)
     np.testing.assert_allclose(vecs[9][:3], [a[L - 1], beta[L - 1], h[L - 1]], err_msg="a_L beta_L h_L", **tol)
+
+
+@pytest.mark.parametrize("kind,L", CASES)
+def test_prepass_helpers_match_the_recurrences(kind, L):
+    """coef_vectors and coef_table_columns (what cw_coef_kernel / cw_coef_bwd_kernel are made of) on one chunk."""
+    rs = np.random.default_rng(L * 11 + len(kind))
+    sig = lambda x: 1 / (1 + np.exp(-x))
+    al, th, et = (sig(rs.standard_normal(64)).astype(np.float32) for _ in range(3))
+    if kind == "const":
+        al[:], th[:], et[:] = 0.05, 0.01, 0.9
+    if kind == "saturated":
+        for t in (0, 15, 16, 31, 40, 41, 42, 63):
+            al[t] = 1.0
+        for t in (3, 16, 47, 48, 49):
+            et[t] = 0.0
+        al[20:24] = 0.0
+        et[5:9] = 1.0
+        th[10] = 0.0
+    if kind == "delta":
+        et[:] = 0.0
+    table, scaled, vecs = zeros(64, 64), zeros(64, 64), zeros(5, 64)
+    assert lib.nlh_selftest_chunk_coef_prepass(dev(al).data_ptr(), dev(th).data_ptr(), dev(et).data_ptr(), L,
+                                               table.data_ptr(), scaled.data_ptr(), vecs.data_ptr()) == 0
+    torch.cuda.synchronize()
+    table, scaled, vecs = host(table), host(scaled), host(vecs)
+    c, bb, r, a, beta, h = host_coefficients(al, th, et, L)
+    tol = dict(rtol=2e-5, atol=1e-30)
+    np.testing.assert_allclose(table, c, err_msg="c", **tol)
+    np.testing.assert_allclose(scaled, -th.astype(np.float64)[None, :] * c, err_msg="-theta c", **tol)
+    pad = lambda x: np.concatenate([x[:L], np.full(64 - L, x[L - 1])])
+    np.testing.assert_allclose(vecs[0], pad(a), err_msg="a", **tol)
+    np.testing.assert_allclose(vecs[1], pad(beta), err_msg="beta", **tol)
+    np.testing.assert_allclose(vecs[2], pad(h), err_msg="h", **tol)
+    np.testing.assert_allclose(vecs[3][:L], c[L - 1, :L], err_msg="cl", **tol)
+    np.testing.assert_allclose(vecs[4][:L], bb[L - 1, :L], err_msg="bl", **tol)
