@@ -58,6 +58,32 @@ __device__ __forceinline__ void gstore(float *dst, const float (&src)[CP]) {
         for (int i = 0; i < CP; i += 2) *reinterpret_cast<float2 *>(dst + i) = make_float2(src[i], src[i + 1]);
     }
 }
+// The forward's ownership of a row's columns: lane cq of the row's four takes the 16-byte pieces at columns
+// 4 cq + 16 i (CP a multiple of 4; the CP consecutive columns cq * CP .. for d = 8).  A store instruction of a
+// wave then writes 64 contiguous bytes per row instead of four 16-byte pieces 64 bytes apart; the forward with
+// the whole trajectory as its output is bound by its stores.
+template <int CP>
+__device__ __forceinline__ void row_load(float (&dst)[CP], const float *row, int cq) {
+    if constexpr (CP % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < CP; i += 4) {
+            const float4 t = *reinterpret_cast<const float4 *>(row + 4 * i + 4 * cq);
+            dst[i] = t.x; dst[i + 1] = t.y; dst[i + 2] = t.z; dst[i + 3] = t.w;
+        }
+    } else {
+        gload<CP>(dst, row + cq * CP);
+    }
+}
+template <int CP>
+__device__ __forceinline__ void row_store(float *row, int cq, const float (&src)[CP]) {
+    if constexpr (CP % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < CP; i += 4)
+            *reinterpret_cast<float4 *>(row + 4 * i + 4 * cq) = make_float4(src[i], src[i + 1], src[i + 2], src[i + 3]);
+    } else {
+        gstore<CP>(row + cq * CP, src);
+    }
+}
 template <int CP>
 __device__ __forceinline__ void clear(float (&x)[CP]) {
 #pragma unroll
@@ -159,11 +185,11 @@ __global__ __launch_bounds__(heb_threads(D)) void hebbian_fwd_kernel(HebFwdArgs 
     const size_t tok0 = (size_t)b * a.input_stride + t_off;
     const float *kb = a.k + tok0 * D, *qb = a.q + tok0 * D, *vb = a.v + tok0 * D;
     const float *ab = a.alpha + tok0;
-    float *ms = a.m_states + ((size_t)b * a.states_per_chain + t_off) * D * D + r * D + c0;
+    float *ms = a.m_states + ((size_t)b * a.states_per_chain + t_off) * D * D + r * D;   // this lane's row
     float *yb = a.y + ((size_t)b * a.seq_len + t_off) * D;
     float M[CP];
-    gload<CP>(M, a.m_initial + (a.chunks ? (size_t)blockIdx.x * D * D : (size_t)b * a.m_stride) + r * D + c0);
-    if (valid) gstore<CP>(ms, M);
+    row_load<CP>(M, a.m_initial + (a.chunks ? (size_t)blockIdx.x * D * D : (size_t)b * a.m_stride) + r * D, cq);
+    if (valid) row_store<CP>(ms, cq, M);
     if (len == 0) return;
     int ck = 1;
     const int last = len - 1, ntile = (len + T - 1) / T;
@@ -179,15 +205,15 @@ __global__ __launch_bounds__(heb_threads(D)) void hebbian_fwd_kernel(HebFwdArgs 
             const int t = g * T + j;
             if (t > last) break;
             float kc[CP], qc[CP];
-            lds_vec<CP>(kc, &tile[buf][j][0][c0]);
-            lds_vec<CP>(qc, &tile[buf][j][1][c0]);
+            row_load<CP>(kc, &tile[buf][j][0][0], cq);
+            row_load<CP>(qc, &tile[buf][j][1][0], cq);
             const float v_r = tile[buf][j][2][r], ret = 1.0f - tal[buf][j];
 #pragma unroll
             for (int i = 0; i < CP; i++) M[i] = ret * M[i] + v_r * kc[i];
             if (STORE == HEB_TRAJ) {
-                if (valid && !(inner_chunk && t == last)) gstore<CP>(ms + (size_t)(t + 1) * D * D, M);
+                if (valid && !(inner_chunk && t == last)) row_store<CP>(ms + (size_t)(t + 1) * D * D, cq, M);
             } else if (((t + 1) % a.ckpt == 0) || (t + 1 == a.seq_len)) {
-                if (valid) gstore<CP>(ms + (size_t)ck * D * D, M);
+                if (valid) row_store<CP>(ms + (size_t)ck * D * D, cq, M);
                 ck++;
             }
             const float y_r = quad_allreduce(dotn<CP>(M, qc));
