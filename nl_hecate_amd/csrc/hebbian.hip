@@ -175,7 +175,7 @@ __global__ __launch_bounds__(heb_threads(D)) void hebbian_fwd_kernel(HebFwdArgs 
     constexpr int CP = D / 4, T = 8;
     __shared__ __align__(16) float tile[2][T][3][D];   // k, q, v of a tile's tokens
     __shared__ float tal[2][T];
-    const int tid = threadIdx.x, cq = tid & 3, c0 = cq * CP;
+    const int tid = threadIdx.x, cq = tid & 3;
     const int b = a.chunks ? blockIdx.x / a.chunks : blockIdx.x, chunk = a.chunks ? blockIdx.x % a.chunks : 0;
     const int t_off = chunk * kHC, len = a.chunks ? min(kHC, a.seq_len - t_off) : a.seq_len;
     const bool inner_chunk = a.chunks && chunk + 1 < a.chunks;   // its last state is the next chunk's first store
