@@ -457,13 +457,16 @@ __global__ __launch_bounds__(256) void heb_chunk_seed_kernel(HebBwdArgs a, float
     const size_t tok = (size_t)b * a.seq_len + t0;
     heb_stage_rows(sDY, a.d_y + tok * 64, L, tid);
     heb_stage_rows(sQ, a.q + tok * 64, L, tid);
-    if (tid == 0) {
-        float p = 1.f;
-        sa[0] = 1.f;
-        for (int t = 0; t < kHC; t++) {
-            if (t < L) p *= 1.f - a.alpha[tok + t];
-            sa[t + 1] = p;   // A(t + 1); constant behind the chunk's last token
+    if (tid < 64) {
+        // A(t + 1) = prod_{r <= t} (1 - alpha_r), constant behind the chunk's last token: a scan over the first wave
+        float x = tid < L ? 1.f - a.alpha[tok + tid] : 1.f;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float y = __shfl_up(x, o);
+            if (tid >= o) x *= y;
         }
+        sa[tid + 1] = x;
+        if (tid == 0) sa[0] = 1.f;
     }
     __syncthreads();
     f32x4 acc[4];
@@ -687,14 +690,17 @@ __global__ __launch_bounds__(256) void heb_chunk_fwd_seed_kernel(HebFwdArgs a, f
     const size_t tok = (size_t)b * a.input_stride + t0;
     heb_stage_rows(sV, a.v + tok * 64, L, tid);
     heb_stage_rows(sK, a.k + tok * 64, L, tid);
-    if (tid == 0) {
-        // sb[s] = rho(L-1, s) = prod_{s < r <= L-1} (1 - alpha_r); sb[kHC] = A(L)
-        float p = 1.f;
-        for (int t = kHC - 1; t >= 0; t--) {
-            sb[t] = t < L ? p : 0.f;
-            if (t < L) p *= 1.f - a.alpha[tok + t];
+    if (tid < 64) {
+        // sb[s] = rho(L-1, s) = prod_{s < r <= L-1} (1 - alpha_r); sb[kHC] = A(L): a suffix scan over the first wave
+        float x = tid < L ? 1.f - a.alpha[tok + tid] : 1.f;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float y = __shfl_down(x, o);
+            if (tid + o < 64) x *= y;
         }
-        sb[kHC] = p;
+        const float behind = __shfl_down(x, 1);   // prod_{r > s}
+        sb[tid] = tid < L ? (tid == 63 ? 1.f : behind) : 0.f;
+        if (tid == 0) sb[kHC] = x;
     }
     __syncthreads();
     f32x4 acc[4];
