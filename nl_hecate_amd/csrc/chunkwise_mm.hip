@@ -778,14 +778,7 @@ constexpr size_t kOutFwdLds = 6 * MAT * sizeof(float);
 
 // One workgroup per compute unit for the kernels whose LDS footprint allows no more.
 int persistent_grid(int ntask) {
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        check_hip(hipGetDevice(&dev), "hipGetDevice");
-        check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
-        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
+    const int cus = compute_units();
     return ntask < cus ? ntask : cus;
 }
 

@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+
 #include "hebbian_generic.h"
 #include "quad_rows.h"
 #include "rule_common.h"
@@ -415,22 +417,6 @@ void launch_bwd_d(const HebBwdArgs &a, int batch) {
 // the scan, the gradients per chunk; all products on v_mfma_f32_16x16x4_f32 (fp32 in and out).
 constexpr int kHL = 68;   // LDS row stride (= 4 mod 64: the operand reads of a wave fall on 64 banks)
 
-// acc[jt] += A B for the wave's 16-row strip (rows wr ..) and the four 16-column tiles; AT / BT read
-// the operand transposed (A[i][k] = bufA[k][i], B[k][n] = bufB[n][k]).
-template <bool AT, bool BT>
-__device__ __forceinline__ void heb_strip_mma(const float *bufA, const float *bufB, f32x4 (&acc)[4], int wr, int ml,
-                                              int kg) {
-#pragma unroll 4
-    for (int k0 = 0; k0 < kHC; k0 += 4) {
-        const float av = AT ? bufA[(k0 + kg) * kHL + wr + ml] : bufA[(wr + ml) * kHL + k0 + kg];
-#pragma unroll
-        for (int jt = 0; jt < 4; jt++) {
-            const float bv = BT ? bufB[(16 * jt + ml) * kHL + k0 + kg] : bufB[(k0 + kg) * kHL + 16 * jt + ml];
-            acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[jt], 0, 0, 0);
-        }
-    }
-}
-
 __device__ __forceinline__ void heb_clear(f32x4 (&acc)[4]) {
 #pragma unroll
     for (int jt = 0; jt < 4; jt++) acc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -502,29 +488,81 @@ __global__ __launch_bounds__(256) void heb_chunk_scan_kernel(const float *P, con
 }
 
 constexpr int kHebGradLds = (8 * kHC * kHL + 1024) * (int)sizeof(float);
+constexpr int kHebGradThr = 512;   // 8 waves, two per SIMD: one's operand reads and epilogues run under the other's products
 
-// The gradients of one chunk: one workgroup per (chain, chunk), wave w owning token rows 16 w ..
-__global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, const float *Sc, int nch) {
+// acc[jt] += A B for the wave's 16-row strip (rows wr ..) and two 16-column tiles from column cb on; AT / BT read
+// the operand transposed (A[i][k] = bufA[k][i], B[k][n] = bufB[n][k]).
+template <bool AT, bool BT>
+__device__ __forceinline__ void heb_half_mma(const float *bufA, const float *bufB, f32x4 (&acc)[2], int wr, int cb,
+                                             int ml, int kg) {
+#pragma unroll 4
+    for (int k0 = 0; k0 < kHC; k0 += 4) {
+        const float av = AT ? bufA[(k0 + kg) * kHL + wr + ml] : bufA[(wr + ml) * kHL + k0 + kg];
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++) {
+            const int col = cb + 16 * jt + ml;
+            const float bv = BT ? bufB[col * kHL + k0 + kg] : bufB[(k0 + kg) * kHL + col];
+            acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[jt], 0, 0, 0);
+        }
+    }
+}
+__device__ __forceinline__ void heb_clear2(f32x4 (&acc)[2]) {
+    acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+// Wave w owns rows 16 (w / 2) .. of every product and the 32 columns from 32 (w % 2) on; sums over a row's 64
+// columns are left as two halves (one per wave of the pair) and added where they are used.
+__global__ __launch_bounds__(kHebGradThr) void heb_chunk_grads_kernel(HebBwdArgs a, const float *Sc, int nch,
+                                                                      int ntask) {
     extern __shared__ __align__(16) float heb_lds[];
     float *bK = heb_lds, *bV = bK + kHC * kHL, *bQ = bV + kHC * kHL, *bDY = bQ + kHC * kHL, *bM = bDY + kHC * kHL;
     float *bW1 = bM + kHC * kHL, *bW2 = bW1 + kHC * kHL, *bR = bW2 + kHC * kHL;
-    float *rr = bR + kHC * kHL, *aa = rr + 64, *rhoL = aa + 80, *A1 = rhoL + 64, *gs = A1 + 64, *colp = gs + 64;
+    float *rr = bR + kHC * kHL, *aa = rr + 64, *rhoL = aa + 80, *A1 = rhoL + 64, *gs = A1 + 128, *colp = gs + 128;
     float *red = colp + 256;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, wr = 16 * wave, ml = lane & 15, kg = lane >> 4;
-    const int chunk = blockIdx.x % nch, b = blockIdx.x / nch;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ml = lane & 15, kg = lane >> 4;
+    const int strip = wave >> 1, half = wave & 1, wr = 16 * strip, cb = 32 * half;
     const int seg = a.t_end - a.t_start;
+    // A workgroup walks over chunk tasks blockIdx.x, blockIdx.x + gridDim.x, ...; the six input matrices of the next
+    // task (two 16-byte pieces per thread and matrix) are requested into registers as soon as this task's are in
+    // LDS, so only the first task of a workgroup waits for HBM.
+    f32x4 nx[5][2], nm0[2], m0r[2];
+    float nrr = 1.f;
+    auto fetch_task = [&](int task) {
+        const int chunk = task % nch, b = task / nch;
+        const int t0 = a.t_start + chunk * kHC, L = min(kHC, a.t_end - t0);
+        const size_t tok = (size_t)b * a.seq_len + t0;
+        const float *src[5] = {a.k + tok * 64, a.v + tok * 64, a.q + tok * 64, a.d_y + tok * 64,
+                               Sc + (size_t)task * 4096};
+        const float *m0 = a.m_states + ((size_t)b * (seg + 1) + (t0 - a.t_start)) * 4096;
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int e = tid + it * kHebGradThr, row = e >> 4, j = (e & 15) * 4;
+#pragma unroll
+            for (int m = 0; m < 5; m++)
+                nx[m][it] = (m == 4 || row < L) ? *reinterpret_cast<const f32x4 *>(src[m] + (size_t)row * 64 + j)
+                                                : f32x4{0.f, 0.f, 0.f, 0.f};
+            nm0[it] = *reinterpret_cast<const f32x4 *>(m0 + (size_t)row * 64 + j);
+        }
+        if (tid < 64) nrr = tid < L ? 1.f - a.alpha[tok + tid] : 1.f;
+    };
+    if ((int)blockIdx.x < ntask) fetch_task(blockIdx.x);
+    for (int task = blockIdx.x; task < ntask; task += gridDim.x) {
+    const int chunk = task % nch, b = task / nch;
     const int t0 = a.t_start + chunk * kHC, L = min(kHC, a.t_end - t0);
     const size_t tok = (size_t)b * a.seq_len + t0;
-    const float *m0 = a.m_states + ((size_t)b * (seg + 1) + (t0 - a.t_start)) * 4096;
-    const float *sc = Sc + (size_t)blockIdx.x * 4096;
-
-    heb_stage_rows(bK, a.k + tok * 64, L, tid);
-    heb_stage_rows(bV, a.v + tok * 64, L, tid);
-    heb_stage_rows(bQ, a.q + tok * 64, L, tid);
-    heb_stage_rows(bDY, a.d_y + tok * 64, L, tid);
-    heb_stage_rows(bM, sc, kHC, tid);   // S
-    if (tid < 64) rr[tid] = tid < L ? 1.f - a.alpha[tok + tid] : 1.f;
+    {
+        float *dst[5] = {bK, bV, bQ, bDY, bM};   // bM: S first
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int e = tid + it * kHebGradThr, row = e >> 4, j = (e & 15) * 4;
+#pragma unroll
+            for (int m = 0; m < 5; m++) *reinterpret_cast<f32x4 *>(dst[m] + row * kHL + j) = nx[m][it];
+            m0r[it] = nm0[it];
+        }
+        if (tid < 64) rr[tid] = nrr;
+    }
     __syncthreads();
+    if (task + (int)gridDim.x < ntask) fetch_task(task + gridDim.x);
     if (wave == 0) {
         // lane t builds row t of R from its diagonal rightwards; tau runs in lock step over the wave
         const int t = lane;
@@ -545,9 +583,10 @@ __global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, cons
     // <M_0, S>
     {
         float part = 0.f;
-        for (int e = tid; e < 1024; e += 256) {
-            const int row = e >> 4, j = (e & 15) * 4;
-            const f32x4 mv = *reinterpret_cast<const f32x4 *>(m0 + row * 64 + j);
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int e = tid + it * kHebGradThr, row = e >> 4, j = (e & 15) * 4;
+            const f32x4 mv = m0r[it];
             const f32x4 sv = *reinterpret_cast<const f32x4 *>(bM + row * kHL + j);
             part += mv[0] * sv[0] + mv[1] * sv[1] + mv[2] * sv[2] + mv[3] * sv[3];
         }
@@ -555,51 +594,55 @@ __global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, cons
         if (lane == 0) red[wave] = part;
     }
     // products with S: T1 = K S^T (rows of d_v), T2 = V S (rows of d_k), g_s = v_s^T S k_s
-    f32x4 dv[4], dk[4], dq[4];
-    heb_clear(dv); heb_clear(dk); heb_clear(dq);
-    heb_strip_mma<false, true>(bK, bM, dv, wr, ml, kg);
-    heb_strip_mma<false, false>(bV, bM, dk, wr, ml, kg);
+    f32x4 dv[2], dk[2], dq[2];
+    heb_clear2(dv); heb_clear2(dk); heb_clear2(dq);
+    heb_half_mma<false, true>(bK, bM, dv, wr, cb, ml, kg);
+    heb_half_mma<false, false>(bV, bM, dk, wr, cb, ml, kg);
     __syncthreads();   // tables, red and every read of S are done
-    const float m0s = red[0] + red[1] + red[2] + red[3];
+    const float m0s = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
 #pragma unroll
     for (int v = 0; v < 4; v++) {
         const int row = wr + 4 * kg + v;
         float part = 0.f;
 #pragma unroll
-        for (int jt = 0; jt < 4; jt++) part = fmaf(dk[jt][v], bK[row * kHL + 16 * jt + ml], part);
+        for (int jt = 0; jt < 2; jt++) part = fmaf(dk[jt][v], bK[row * kHL + cb + 16 * jt + ml], part);
         part = group_allreduce<16>(part);
-        if (ml == 0) gs[row] = part;
+        if (ml == 0) gs[64 * half + row] = part;
         const float sL = rhoL[row];
 #pragma unroll
-        for (int jt = 0; jt < 4; jt++) { dv[jt][v] *= sL; dk[jt][v] *= sL; }
+        for (int jt = 0; jt < 2; jt++) { dv[jt][v] *= sL; dk[jt][v] *= sL; }
     }
-    heb_stage_rows(bM, m0, kHC, tid);   // M_0
+#pragma unroll
+    for (int it = 0; it < 2; it++) {   // M_0
+        const int e = tid + it * kHebGradThr, row = e >> 4, j = (e & 15) * 4;
+        *reinterpret_cast<f32x4 *>(bM + row * kHL + j) = m0r[it];
+    }
     __syncthreads();
     // T3 = dY M_0: d_q starts as A(t+1) T3, and A1_tau = dy_tau^T M_0 q_tau
-    heb_strip_mma<false, false>(bDY, bM, dq, wr, ml, kg);
+    heb_half_mma<false, false>(bDY, bM, dq, wr, cb, ml, kg);
 #pragma unroll
     for (int v = 0; v < 4; v++) {
         const int row = wr + 4 * kg + v;
         float part = 0.f;
 #pragma unroll
-        for (int jt = 0; jt < 4; jt++) part = fmaf(dq[jt][v], bQ[row * kHL + 16 * jt + ml], part);
+        for (int jt = 0; jt < 2; jt++) part = fmaf(dq[jt][v], bQ[row * kHL + cb + 16 * jt + ml], part);
         part = group_allreduce<16>(part);
-        if (ml == 0) A1[row] = part;
+        if (ml == 0) A1[64 * half + row] = part;
         const float sA = aa[row + 1];
 #pragma unroll
-        for (int jt = 0; jt < 4; jt++) dq[jt][v] *= sA;
+        for (int jt = 0; jt < 2; jt++) dq[jt][v] *= sA;
     }
     // G1 = K Q^T, G2 = V dY^T (token x token); W1 = R o G1, W2 = R o G2, and G1 o G2 for d_alpha
-    f32x4 g1[4], g2[4];
-    heb_clear(g1); heb_clear(g2);
-    heb_strip_mma<false, true>(bK, bQ, g1, wr, ml, kg);
-    heb_strip_mma<false, true>(bV, bDY, g2, wr, ml, kg);
+    f32x4 g1[2], g2[2];
+    heb_clear2(g1); heb_clear2(g2);
+    heb_half_mma<false, true>(bK, bQ, g1, wr, cb, ml, kg);
+    heb_half_mma<false, true>(bV, bDY, g2, wr, cb, ml, kg);
     __syncthreads();   // M_0 has been read
 #pragma unroll
-    for (int jt = 0; jt < 4; jt++) {
+    for (int jt = 0; jt < 2; jt++) {
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const int o = (wr + 4 * kg + v) * kHL + 16 * jt + ml;
+            const int o = (wr + 4 * kg + v) * kHL + cb + 16 * jt + ml;
             const float rv = bR[o];
             bW1[o] = rv * g1[jt][v];
             bW2[o] = rv * g2[jt][v];
@@ -607,30 +650,30 @@ __global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, cons
         }
     }
     __syncthreads();
-    heb_strip_mma<false, false>(bW1, bDY, dv, wr, ml, kg);
-    heb_strip_mma<false, false>(bW2, bQ, dk, wr, ml, kg);
-    heb_strip_mma<true, false>(bW2, bK, dq, wr, ml, kg);
+    heb_half_mma<false, false>(bW1, bDY, dv, wr, cb, ml, kg);
+    heb_half_mma<false, false>(bW2, bQ, dk, wr, cb, ml, kg);
+    heb_half_mma<true, false>(bW2, bK, dq, wr, cb, ml, kg);
     // U[s][t] = sum_{tau >= t} rho(tau, t) (v_s . dy_tau)(k_s . q_tau)
-    f32x4 u[4];
-    heb_clear(u);
-    heb_strip_mma<false, true>(bM, bR, u, wr, ml, kg);
+    f32x4 u[2];
+    heb_clear2(u);
+    heb_half_mma<false, true>(bM, bR, u, wr, cb, ml, kg);
     float *dvo = a.d_v + tok * 64, *dko = a.d_k + tok * 64, *dqo = a.d_q + tok * 64;
 #pragma unroll
     for (int v = 0; v < 4; v++) {
         const int row = wr + 4 * kg + v;
         if (row < L) {
 #pragma unroll
-            for (int jt = 0; jt < 4; jt++) {
-                dvo[(size_t)row * 64 + 16 * jt + ml] = dv[jt][v];
-                dko[(size_t)row * 64 + 16 * jt + ml] = dk[jt][v];
-                dqo[(size_t)row * 64 + 16 * jt + ml] = dq[jt][v];
+            for (int jt = 0; jt < 2; jt++) {
+                dvo[(size_t)row * 64 + cb + 16 * jt + ml] = dv[jt][v];
+                dko[(size_t)row * 64 + cb + 16 * jt + ml] = dk[jt][v];
+                dqo[(size_t)row * 64 + cb + 16 * jt + ml] = dq[jt][v];
             }
         }
     }
-    // sum_{s < t} rho(t - 1, s) U[s][t]: columns of the wave's 16 rows, then over the waves
+    // sum_{s < t} rho(t - 1, s) U[s][t]: columns of the wave's 16 rows, then over the four row strips
 #pragma unroll
-    for (int jt = 0; jt < 4; jt++) {
-        const int t = 16 * jt + ml;
+    for (int jt = 0; jt < 2; jt++) {
+        const int t = cb + 16 * jt + ml;
         float part = 0.f;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
@@ -638,7 +681,7 @@ __global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, cons
             if (srow < t) part = fmaf(bR[srow * kHL + t - 1], u[jt][v], part);
         }
         part = stride_allreduce<16>(part);
-        if (kg == 0) colp[wave * 64 + t] = part;
+        if (kg == 0) colp[strip * 64 + t] = part;
     }
     __syncthreads();
     if (tid < L) {
@@ -646,11 +689,13 @@ __global__ __launch_bounds__(256) void heb_chunk_grads_kernel(HebBwdArgs a, cons
         //                             + sum_{s<t} rho(t-1,s) [U[s][t] + rho_L(t) g_s] )
         const int t = tid;
         float s1 = 0.f, s4 = 0.f;
-        for (int tau = t; tau < L; tau++) s1 = fmaf(bR[t * kHL + tau], A1[tau], s1);
-        for (int s2 = 0; s2 < t; s2++) s4 = fmaf(bR[s2 * kHL + t - 1], gs[s2], s4);
+        for (int tau = t; tau < L; tau++) s1 = fmaf(bR[t * kHL + tau], A1[tau] + A1[64 + tau], s1);
+        for (int s2 = 0; s2 < t; s2++) s4 = fmaf(bR[s2 * kHL + t - 1], gs[s2] + gs[64 + s2], s4);
         const float s3 = colp[t] + colp[64 + t] + colp[128 + t] + colp[192 + t];
         const float x = aa[t] * fmaf(rhoL[t], m0s, s1) + s3 + rhoL[t] * s4;
         a.d_alpha[tok + t] = -x;
+    }
+    __syncthreads();   // the next task's matrices and tables replace this one's
     }
 }
 
@@ -674,7 +719,9 @@ bool launch_bwd_chunks(const HebBwdArgs &a, int batch) {
                                   hipFuncAttributeMaxDynamicSharedMemorySize, kHebGradLds), "dynamic LDS size");
     {
         KernelTimer kt("hebbian_bwd_kernel");
-        hipLaunchKernelGGL(heb_chunk_grads_kernel, dim3((unsigned)chunks), dim3(256), kHebGradLds, stream(), a, S, nch);
+        const unsigned grid = (unsigned)std::min<size_t>(chunks, (size_t)compute_units());   // one workgroup fits a compute unit
+        hipLaunchKernelGGL(heb_chunk_grads_kernel, dim3(grid), dim3(kHebGradThr), kHebGradLds, stream(), a, S, nch,
+                           (int)chunks);
         check_launch("heb_chunk_grads_kernel");
     }
     return true;

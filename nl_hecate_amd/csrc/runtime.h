@@ -44,6 +44,10 @@ struct KernelTimer {
     int slot;
 };
 
+// Compute units of the current device (cached per process; 256 if the query fails): the grid of kernels whose
+// workgroups loop over tasks, one workgroup per compute unit.
+int compute_units();
+
 inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 }  // namespace nlh

@@ -60,6 +60,20 @@ void check_launch(const char *kernel) {
 
 hipStream_t stream() { return g_stream; }
 
+int compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+            prop.multiProcessorCount > 0)
+            cus = prop.multiProcessorCount;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
 float *scratch(int slot, size_t bytes) {
     if (slot < 0 || slot >= kScratchSlots) {
         fail("scratch slot %d out of range", slot);
