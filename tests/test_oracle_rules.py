@@ -345,3 +345,27 @@ def test_chunkwise_matches_numpy_and_finite_differences(C, has_s, clip, mx):
     an = dict(k=g["d_k"], v=g["d_v"], q=g["d_q"], alpha=g["d_alpha"], theta=g["d_theta"],
               eta=g["d_eta"], m0=g["d_m"], s0=g["d_s"])
     _check_grads(fd, an, P.keys())
+
+
+@pytest.mark.parametrize("s,d,C", [(37, 6, 8), (64, 8, 64), (130, 4, 64), (9, 5, 1), (20, 3, 7)])
+@pytest.mark.parametrize("saturate", [False, True])
+def test_exact_rule_matches_its_chunk_parallel_matrix_form(s, d, C, saturate):
+    """The exact Titans rule restated per chunk as one unit lower triangular solve (np_rules.titans_exact_chunk_*):
+    a different algorithm from the oracle's token loops (dispatch.rs:1226-1563), so agreement of the outputs, the
+    boundary states and every gradient in float64 pins both.  saturate: alpha = 1 and eta = 0 at some tokens
+    (no division anywhere, so the gradients stay finite and equal)."""
+    r = np.random.default_rng(1000 + s + d + C)
+    k, v, q, dy = (r.standard_normal((s, d)) * 0.5 for _ in range(4))
+    al, th, et = r.uniform(0.05, 0.4, s), r.uniform(0.05, 0.5, s), r.uniform(0.3, 0.95, s)
+    if saturate:
+        al[s // 3], et[s // 2], al[s - 1], et[0] = 1.0, 0.0, 1.0, 0.0
+    m0, s0 = r.standard_normal((d, d)) * 0.3, r.standard_normal((d, d)) * 0.3
+    y, mb, sb = npr.titans_exact_chunk_forward(k, v, q, al, th, et, m0, s0, C)
+    yo, mo, so = orc.titans_forward(k, v, q, al, th, et, m0, s0)
+    bounds = list(range(0, s, C)) + [s]
+    assert np.abs(y - yo).max() < 1e-12
+    assert np.abs(mb - mo[bounds]).max() < 1e-12 and np.abs(sb - so[bounds]).max() < 1e-12
+    g = npr.titans_exact_chunk_backward(k, v, q, al, th, et, mb, sb, dy, C)
+    go = orc.titans_backward(k, v, q, al, th, et, mo, so, dy)
+    for n in go:
+        assert np.abs(g[n] - go[n]).max() <= 1e-11 * max(1.0, np.abs(go[n]).max()), n
