@@ -142,3 +142,25 @@ def test_exact_rules_full_and_checkpointed():
                 go = rules._oracle_ckpt_grads(x, C, has_s)
                 for n in g:
                     assert_close(f"{n} has_s={has_s}", g[n], go[n])
+
+
+def test_layer_steps_against_the_autograd_reference():
+    """Whole layer steps (levels, gate, attention branch, projections) at drawn configurations against the float64
+    autograd model of tests/torch_mag_reference.py, tolerance and bias scaling as in tests/test_gpu_mag_layer.py."""
+    from tests import test_gpu_mag_layer as layer
+    rnd = random.Random(61)
+    for it in range(14):
+        rule = rnd.choice(["exact", "chunkwise", "chunkwise"])
+        nh = rnd.choice([1, 2, 3])
+        hd = 64 if rule == "chunkwise" else rnd.choice([16, 32, 64])
+        k = rnd.choice([1, 2, 3, 4])
+        periods = ([1, 2, 4, 8] if rnd.random() < 0.5 else [1, 8, 64, 512])[:k]
+        bs, s = rnd.choice([1, 2, 3]), rnd.choice([5, 16, 33, 64, 70, 100, 129])
+        window = rnd.choice([4, 8, 32, 50, 64, 128])   # one key in the window makes d_w_q exactly zero: not drawn
+        chunk = rnd.choice([4, 8, 16, 32, 64]) if rule == "chunkwise" else rnd.choice([4, 8, 16, 64])
+        steps = rnd.choice([1, 1, 2, 3])
+        print(f"layer case={it} bs={bs} s={s} d={nh * hd} nh={nh} k={k} window={window} periods={periods} rule={rule} "
+              f"chunk={chunk} steps={steps}", flush=True)
+        w = layer.run_case(bs=bs, s=s, d=nh * hd, nh=nh, k=k, window=window, periods=periods, rule=rule, chunk=chunk,
+                           seed=100 + it, steps=steps, bias_scale=True)
+        assert max(w.values()) < 2e-2, {n: f"{e:.1e}" for n, e in w.items() if e > 5e-3}
