@@ -389,10 +389,11 @@ def cpu_baseline_mag_layer(bs, s, d, heads, k, window):
                       f"{bs * s} tokens ({t_opt * 1e6:.1f}); glue kernels not counted"}
 
 
-def setup_mag_layer_c5(torch, D, lib):
+def setup_mag_layer_c5(torch, D, lib, precision="bf16x3"):
     from nl_hecate_amd.mag_layer import MagLayer, MagTrainer
     bs, heads, d, s, k, window = 8, 8, 512, 4096, 4, 512
-    layer = MagLayer(d, heads, k, window, [1, 8, 64, 512], rule="chunkwise", chunk=64, seed=0x5EED0007)
+    layer = MagLayer(d, heads, k, window, [1, 8, 64, 512], rule="chunkwise", chunk=64, seed=0x5EED0007,
+                     precision=precision)
     tr = MagTrainer(layer, lr=3e-4, beta1=0.9, beta2=0.95, weight_decay=0.1)
     g = torch.Generator(device="cpu").manual_seed(0x5EED0008)
     x = (torch.randn(bs, s, d, generator=g) / d ** 0.5).cuda()
@@ -575,7 +576,8 @@ def setup_hebbian_c2(torch, D, lib):
 WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
              "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5,
              "swa_stats_c5": lambda torch, D, lib: setup_swa_c5(torch, D, lib, lse=True),
-             "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5, "hebbian_c2": setup_hebbian_c2}
+             "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5, "hebbian_c2": setup_hebbian_c2,
+             "mag_layer_c5_bf16": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16")}
 
 
 def source_hash():

@@ -870,6 +870,63 @@ void nlh_swa_backward_dispatch(const float *q, const float *k, const float *v, c
                                const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len,
                                int num_heads, int head_dim, int window_size);
 
+/* ── The level step of a CMS layer (no single counterpart symbol in core/src/cuda_ffi.rs: the reference
+ * composes it on the host from cublasSgemm and the glue kernels) ─────────────────────────────────────
+ * gpu_memory_forward (core/src/gpu_forward.rs:1197-1382) for `levels` Titans levels over the same tokens:
+ * k, v, q = x W^T per level, k and q L2-normalised over the model width, the three gates
+ * (sigmoid / softplus / sigmoid of [k | v] . w + b), head split.  One launch computes every projection on the
+ * bf16 matrix cores (x and the weights rounded once to bf16, fp32 accumulation) and writes the rule kernels'
+ * operands directly.  n = bs * seq_len tokens, d = heads * head_dim in {256, 512}, head_dim = 64.
+ *   x [n, d]; w_extra [n_extra * d, d]: plain projections of x (the attention branch's q, k, v) whose results
+ *   leave as bf16 [n, d] in extra_out[0 .. n_extra); w_levels [levels * 3 * d, d]: rows k, v, q of every level;
+ *   gate_params: host array of 6 * levels device pointers (w_alpha [2d], b_alpha [1], w_theta, b_theta, w_eta,
+ *   b_eta per level).  Outputs: x_bf16 [n, d] (x rounded to bf16, the backward's operand; may be null);
+ *   k/v/q_heads bf16 [levels * bs * heads, seq_len, head_dim] (chain = (level, batch element, head));
+ *   alpha/theta/eta_heads [levels * bs * heads, seq_len]; k_norms, q_norms, alpha, theta, eta [levels, n]. */
+void level_project_forward_bf16_rocm(const float *x, const float *w_extra, int n_extra, uint16_t *const *extra_out,
+                                     const float *w_levels, const float *const *gate_params, uint16_t *x_bf16,
+                                     uint16_t *k_heads, uint16_t *v_heads, uint16_t *q_heads, float *alpha_heads,
+                                     float *theta_heads, float *eta_heads, float *k_norms, float *q_norms, float *alpha,
+                                     float *theta, float *eta, int bs, int seq_len, int heads, int head_dim, int levels,
+                                     float eps);
+/* The projections above, then the chunkwise Titans rule on all levels' chains at once
+ * (titans_chunkwise_forward_bf16_tokens_rocm) from the carried context memories m_context, s_context
+ * [levels * bs * heads, head_dim^2], which receive the final states (copy_final_m_batch, gpu_forward.rs:2824).
+ * m/s_chunk_states [levels * bs * heads, num_chunks + 1, head_dim^2]; y_tokens [levels, bs, seq_len, d]. */
+void titans_levels_forward_bf16_rocm(const float *x, const float *w_extra, int n_extra, uint16_t *const *extra_out,
+                                     const float *w_levels, const float *const *gate_params, float *m_context,
+                                     float *s_context, uint16_t *x_bf16, uint16_t *k_heads, uint16_t *v_heads,
+                                     uint16_t *q_heads, float *alpha_heads, float *theta_heads, float *eta_heads,
+                                     float *k_norms, float *q_norms, float *alpha, float *theta, float *eta,
+                                     float *m_chunk_states, float *s_chunk_states, float *y_tokens, int bs, int seq_len,
+                                     int heads, int head_dim, int levels, int chunk_size, float eps);
+/* gpu_memory_backward + accumulate_projection_grads (core/src/gpu_backward.rs:459-640, 2047-2115) for the same
+ * stack: rule backward from ONE upstream gradient d_y_tokens [bs, seq_len, d] that every level reads, head sums
+ * and activation derivatives of the gates, backward of the two normalisations, then d_x [n, d] (overwritten) =
+ * sum over all projections of g W, and d_w_extra [n_extra * d, d], d_w_levels [levels * 3 * d, d] (overwritten)
+ * = g^T x, as bf16 GEMMs with fp32 accumulation; d_extra: host array of n_extra device pointers, the fp32
+ * gradients [n, d] of the plain projections' outputs; d_gate_params: host array of 6 * levels device pointers
+ * (overwritten).  As on the reference's GPU path nothing flows from the gates into k and v.
+ * d_m_initial, d_s_initial [head_dim^2] are accumulated (+=, summed over all chains). */
+void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_extra, int n_extra, const float *const *d_extra,
+                                      const float *w_levels, const uint16_t *k_heads, const uint16_t *v_heads,
+                                      const uint16_t *q_heads, const float *alpha_heads, const float *theta_heads,
+                                      const float *eta_heads, const float *k_norms, const float *q_norms, const float *alpha,
+                                      const float *theta, const float *eta, const float *m_chunk_states,
+                                      const float *s_chunk_states, const float *d_y_tokens, float *d_x, float *d_w_extra,
+                                      float *d_w_levels, float *const *d_gate_params, float *d_m_initial, float *d_s_initial,
+                                      int bs, int seq_len, int heads, int head_dim, int levels, int chunk_size, float eps);
+/* cms_combine_gate_bf16_rocm with gated leaving as plain bf16 [n] (the output projection's operand). */
+void cms_combine_gate_bf16x1_rocm(const float *const *y_levels, int k, const uint16_t *attn_out, float *gate,
+                                  uint16_t *gated_bf16, long long n);
+/* out [n, d_out] = a W^T and its backward d_a [n, d_in] = g W, d_w [d_out, d_in] = g^T a (either may be null)
+ * for a bf16 activation a [n, d_in], fp32 weights W [d_out, d_in] and an fp32 upstream gradient g [n, d_out],
+ * both rounded once to bf16; fp32 accumulation (the cublasSgemm call sites of the output projection,
+ * gpu_forward.rs:1066-1071, gpu_backward.rs:212-260). */
+void linear_forward_bf16_rocm(const uint16_t *a_bf16, const float *w, float *out, int n, int d_in, int d_out);
+void linear_backward_bf16_rocm(const float *d_out_f32, const uint16_t *a_bf16, const float *w, float *d_a, float *d_w, int n,
+                               int d_in, int d_out);
+
 /* ── Opaque VJP blocks of the Wengert tape ───────────────────────────────────────────────────────
  * core/src/tape.rs:141-150 OpaqueBackwardFn(d_outputs, saved, d_inputs) for the OpaqueKey values
  * below (numbered in the order of the enum at tape.rs:100-134), with the saved-buffer layouts of the

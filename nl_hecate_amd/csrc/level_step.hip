@@ -1,0 +1,764 @@
+// The level step of a CMS layer behind the C ABI: what the reference's caller of the rule kernels does
+// per level around them (gpu_memory_forward, core/src/gpu_forward.rs:1197-1382: projections, row L2 norm
+// of k and q at model width, the three gate projections, head split; gpu_memory_backward and
+// accumulate_projection_grads, core/src/gpu_backward.rs:459-640, 2047-2115), for a stack of Titans levels
+// on the chunkwise rule with bf16 tokens.
+//
+// Forward: ONE kernel computes every projection of x (the attention branch's plain ones and k, v, q of
+// every level) on the bf16 matrix cores and finishes them in registers: a workgroup keeps its 128 tokens
+// of x as bf16 in LDS for the whole kernel, each of its eight waves owns 64 output columns and streams
+// the weights of those columns from L2 in the order the matrix instruction wants them (packed once per
+// call), so a weight element is read by exactly one wave of the workgroup and never touches LDS.  The
+// epilogue of a level's k / v / q takes the row norms and the gate dot products from the accumulators
+// (four consecutive columns of one token per lane), normalises, rounds once to bf16 and writes the
+// head-major operands of the rule kernels: no fp32 projection output exists.
+// Backward: the rule's head-major gradients go through one streaming pass (head merge, backward of the
+// two normalisations, gate projections' weight sums) into ONE bf16 operand G [tokens, all projections],
+// and d_x = G W, d_W = G^T x are two library GEMMs with fp32 accumulation.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <rocblas/rocblas.h>
+#include <stdint.h>
+
+#include "../../include/nl_hecate_ffi.h"
+#include "bf16_tiles.h"
+#include "lane_ops.h"
+#include "runtime.h"
+
+namespace nlh {
+namespace {
+
+constexpr int PT = 128;       // tokens per workgroup of the projection kernel
+constexpr int kPThr = 512;    // 8 waves
+constexpr int kMaxLevels = 8;
+constexpr int kMaxExtra = 4;
+constexpr int kSThr = 256;    // streaming kernels
+
+__device__ __forceinline__ float sigmoid_(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplus_(float x) { return x > 20.0f ? x : logf(1.0f + expf(x)); }
+__device__ __forceinline__ float dotv(const f32x4 &a, const float4 &b) { return a[0] * b.x + a[1] * b.y + a[2] * b.z + a[3] * b.w; }
+__device__ __forceinline__ float sum_rows(float x) {   // over the four 16-lane rows of a wave, to every lane
+    x = swapadd16(x, x);
+    return swapadd32(x, x);
+}
+__device__ __forceinline__ void fma4(float4 &acc, float s, const float4 &x) {
+    acc.x = fmaf(s, x.x, acc.x); acc.y = fmaf(s, x.y, acc.y); acc.z = fmaf(s, x.z, acc.z); acc.w = fmaf(s, x.w, acc.w);
+}
+__device__ __forceinline__ float4 bf4_to_f4(const bf16x4 &h) {
+    return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+}
+__device__ __forceinline__ bf16x4 f4_to_bf4(const float4 &x) {
+    return bf16x4{(__bf16)x.x, (__bf16)x.y, (__bf16)x.z, (__bf16)x.w};
+}
+
+struct GateParams { const float *w_alpha, *b_alpha, *w_theta, *b_theta, *w_eta, *b_eta; };
+
+struct ProjArgs {
+    const float *x;            // [n, D]
+    u16 *x_bf16;               // [n, D]: x rounded to bf16 (the backward's GEMM operand); may be null
+    const u16 *wfrag;          // packed weights, projection p at p * D * D (wfrag_pack_kernel)
+    u16 *extra_out[kMaxExtra]; // plain projections, bf16 [n, D] each
+    GateParams lv[kMaxLevels];
+    u16 *kh, *vh, *qh;         // [levels * bs * nh, s, hd]
+    float *ah, *th, *eh;       // [levels * bs * nh, s]
+    float *k_norms, *q_norms, *alpha, *theta, *eta;   // [levels, n]
+    long long n;
+    int bs, s, nh, hd, n_extra, levels;
+    float eps;
+};
+
+// Packs P matrices W_p [D, D] (row = output column, contraction index contiguous) into the order in which
+// the projection kernel's waves read them: [p][column block of 64][k step of 32][tile of 16 columns][lane][8],
+// lane l holding column 16 * tile + l % 16, contraction indices 32 * step + 8 * (l / 16) .. + 8: one 16-byte
+// load per lane and tile, 4 KB contiguous per wave and step.
+__global__ void wfrag_pack_kernel(const float *__restrict__ W, u16 *__restrict__ out, int P, int D) {
+    const long long total = (long long)P * D * D / 8;
+    const int KS = D / 32, CB = D / 64;
+    for (long long o = (long long)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (long long)gridDim.x * blockDim.x) {
+        const int lane = (int)(o & 63), ct = (int)((o >> 6) & 3);
+        long long r = o >> 8;
+        const int ks = (int)(r % KS);
+        r /= KS;
+        const int cb = (int)(r % CB);
+        const long long p = r / CB;
+        const int row = 64 * cb + 16 * ct + (lane & 15), k0 = 32 * ks + 8 * (lane >> 4);
+        const float *src = W + (p * D + row) * D + k0;
+        const float4 a = *reinterpret_cast<const float4 *>(src), b = *reinterpret_cast<const float4 *>(src + 4);
+        const bf16x8 v = {(__bf16)a.x, (__bf16)a.y, (__bf16)a.z, (__bf16)a.w, (__bf16)b.x, (__bf16)b.y, (__bf16)b.z, (__bf16)b.w};
+        *reinterpret_cast<bf16x8 *>(out + o * 8) = v;
+    }
+}
+
+// acc[tt][ct][r] = sum_k W[col][k] x[token][k] with col = 16 ct + 4 (lane / 16) + r of the wave's 64 columns and
+// token = 16 tt + lane % 16 of the workgroup's 128: the weights as the A operand straight from global memory
+// (requested three steps ahead), x as the B operand from LDS.
+template <int D>
+__device__ __forceinline__ void project_block(const u16 *Xs, const u16 *wf, f32x4 (&acc)[PT / 16][4]) {
+    constexpr int XS = D + 8, KS = D / 32, AHEAD = 3;
+    const int lane = threadIdx.x & 63;
+    const bf16x8 *wp = reinterpret_cast<const bf16x8 *>(wf) + lane;
+    const u16 *xb = Xs + (lane & 15) * XS + 8 * (lane >> 4);
+#pragma unroll
+    for (int tt = 0; tt < PT / 16; tt++)
+#pragma unroll
+        for (int ct = 0; ct < 4; ct++) acc[tt][ct] = zero4();
+    static_assert(KS % (AHEAD + 1) == 0, "the k loop is unrolled by the depth of the weight ring");
+    bf16x8 w[AHEAD + 1][4];
+#pragma unroll
+    for (int p = 0; p < AHEAD; p++)
+#pragma unroll
+        for (int ct = 0; ct < 4; ct++) w[p][ct] = wp[(p * 4 + ct) * 64];
+    // a rolled loop over groups of four steps: the ring slots are compile-time indices inside a group, and the
+    // compiler cannot pull the loads of later groups up (a fully unrolled loop spilled hundreds of registers)
+#pragma unroll 1
+    for (int ks0 = 0; ks0 < KS; ks0 += AHEAD + 1) {
+#pragma unroll
+        for (int j = 0; j <= AHEAD; j++) {
+            const int ks = ks0 + j;
+            const int nx = ks + AHEAD < KS ? ks + AHEAD : KS - 1;   // past the end: a harmless repeat of the last step
+#pragma unroll
+            for (int ct = 0; ct < 4; ct++) w[(j + AHEAD) % (AHEAD + 1)][ct] = wp[(nx * 4 + ct) * 64];
+            // the requests stay where they are written: left to itself the scheduler sinks each load to its first use
+            // (three steps later) and the wave then waits a full memory latency per step
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < PT / 16; tt++) {
+                const bf16x8 b = *reinterpret_cast<const bf16x8 *>(xb + 16 * tt * XS + 32 * ks);
+#pragma unroll
+                for (int ct = 0; ct < 4; ct++) acc[tt][ct] = mfma32(w[j][ct], b, acc[tt][ct]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
+    constexpr int XS = D + 8, CB = D / 64, D4 = D / 4;
+    extern __shared__ __align__(16) unsigned char smem[];
+    u16 *Xs = reinterpret_cast<u16 *>(smem);                                   // [PT][XS]
+    float *red = reinterpret_cast<float *>(smem + (size_t)PT * XS * 2);         // [8][PT][4]
+    float *tot = red + 8 * PT * 4;                                              // [PT][4]
+    int *rowoff = reinterpret_cast<int *>(tot + PT * 4);                        // [PT]: b * nh * s + t of the token
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    const long long tok0 = (long long)blockIdx.x * PT, n = a.n;
+    const bool wave_on = wave < CB;
+
+    // x tile: fp32 -> bf16, into LDS (and out as the backward's operand)
+    for (int i0 = 0; i0 < PT * D4; i0 += kPThr * 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = i0 + j * kPThr + tid, row = e / D4, c4 = e % D4;
+            v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e < PT * D4 && tok0 + row < n) v[j] = *reinterpret_cast<const float4 *>(a.x + (tok0 + row) * D + 4 * c4);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = i0 + j * kPThr + tid, row = e / D4, c4 = e % D4;
+            if (e >= PT * D4) continue;
+            const bf16x4 h = f4_to_bf4(v[j]);
+            *reinterpret_cast<bf16x4 *>(Xs + row * XS + 4 * c4) = h;
+            if (a.x_bf16 && tok0 + row < n) *reinterpret_cast<bf16x4 *>(a.x_bf16 + (tok0 + row) * D + 4 * c4) = h;
+        }
+    }
+    if (tid < PT) {
+        const unsigned tok = (unsigned)(tok0 + tid), b = tok / (unsigned)a.s;
+        rowoff[tid] = (int)(b * (unsigned)(a.nh * a.s) + (tok - b * (unsigned)a.s));
+    }
+    __syncthreads();
+
+    f32x4 acc[PT / 16][4];
+    const size_t wave_frag = (size_t)wave * 64 * D;
+    const int colw = 64 * wave + 4 * g;   // the lane's first column in tile 0
+
+    // plain projections: rounded once, token-major
+    if (wave_on)
+        for (int e = 0; e < a.n_extra; e++) {
+            project_block<D>(Xs, a.wfrag + (size_t)e * D * D + wave_frag, acc);
+            u16 *out = a.extra_out[e];
+#pragma unroll
+            for (int tt = 0; tt < PT / 16; tt++) {
+                const long long tok = tok0 + 16 * tt + l16;
+                if (tok >= n) continue;
+#pragma unroll
+                for (int ct = 0; ct < 4; ct++) bf16_store(out + tok * D + colw + 16 * ct, 0, acc[tt][ct]);
+            }
+        }
+
+    for (int lvl = 0; lvl < a.levels; lvl++) {
+        const GateParams gp = a.lv[lvl];
+        const size_t pbase = (size_t)(a.n_extra + 3 * lvl) * D * D;
+        const size_t chain0 = (size_t)lvl * a.bs * a.nh;
+#pragma unroll 1
+        for (int p = 0; p < 3; p++) {   // k, v, q
+            if (wave_on) {
+                project_block<D>(Xs, a.wfrag + pbase + (size_t)p * D * D + wave_frag, acc);
+                float4 wa[4], wt[4], we[4];
+                if (p < 2) {
+#pragma unroll
+                    for (int ct = 0; ct < 4; ct++) {
+                        const int c = p * D + colw + 16 * ct;
+                        wa[ct] = *reinterpret_cast<const float4 *>(gp.w_alpha + c);
+                        wt[ct] = *reinterpret_cast<const float4 *>(gp.w_theta + c);
+                        we[ct] = *reinterpret_cast<const float4 *>(gp.w_eta + c);
+                    }
+                }
+#pragma unroll
+                for (int tt = 0; tt < PT / 16; tt++) {
+                    float ss = 0.f, da = 0.f, dt = 0.f, de = 0.f;
+#pragma unroll
+                    for (int ct = 0; ct < 4; ct++) {
+                        const f32x4 v = acc[tt][ct];
+                        if (p != 1) ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+                        if (p < 2) { da += dotv(v, wa[ct]); dt += dotv(v, wt[ct]); de += dotv(v, we[ct]); }
+                    }
+                    if (p != 1) ss = sum_rows(ss);
+                    if (p < 2) { da = sum_rows(da); dt = sum_rows(dt); de = sum_rows(de); }
+                    if (g == 0) *reinterpret_cast<float4 *>(red + (wave * PT + 16 * tt + l16) * 4) = make_float4(ss, da, dt, de);
+                }
+                if (p == 1) {   // v leaves as it is
+#pragma unroll
+                    for (int tt = 0; tt < PT / 16; tt++) {
+                        if (tok0 + 16 * tt + l16 >= n) continue;
+                        u16 *row = a.vh + (chain0 * a.s + rowoff[16 * tt + l16] + (size_t)wave * a.s) * 64 + 4 * g;
+#pragma unroll
+                        for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct]);
+                    }
+                }
+            }
+            __syncthreads();
+            if (tid < PT) {
+                float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+                for (int w = 0; w < CB; w++) {
+                    const float4 r = *reinterpret_cast<const float4 *>(red + (w * PT + tid) * 4);
+                    s.x += r.x; s.y += r.y; s.z += r.z; s.w += r.w;
+                }
+                const long long tok = tok0 + tid;
+                float *tt_ = tot + tid * 4;
+                if (p == 0) {
+                    const float kn = sqrtf(s.x), ki = 1.0f / fmaxf(kn, a.eps);
+                    tt_[0] = ki; tt_[1] = s.y * ki; tt_[2] = s.z * ki; tt_[3] = s.w * ki;
+                    if (tok < n) a.k_norms[lvl * n + tok] = kn;
+                } else if (p == 1) {
+                    const float al = sigmoid_(tt_[1] + s.y + gp.b_alpha[0]), th = softplus_(tt_[2] + s.z + gp.b_theta[0]);
+                    const float et = sigmoid_(tt_[3] + s.w + gp.b_eta[0]);
+                    if (tok < n) {
+                        a.alpha[lvl * n + tok] = al; a.theta[lvl * n + tok] = th; a.eta[lvl * n + tok] = et;
+                        for (int h = 0; h < a.nh; h++) {
+                            const size_t o = chain0 * a.s + rowoff[tid] + (size_t)h * a.s;
+                            a.ah[o] = al; a.th[o] = th; a.eh[o] = et;
+                        }
+                    }
+                } else {
+                    const float qn = sqrtf(s.x);
+                    tt_[0] = 1.0f / fmaxf(qn, a.eps);
+                    if (tok < n) a.q_norms[lvl * n + tok] = qn;
+                }
+            }
+            __syncthreads();
+            if (wave_on && p != 1) {
+                u16 *dst = p == 0 ? a.kh : a.qh;
+#pragma unroll
+                for (int tt = 0; tt < PT / 16; tt++) {
+                    if (tok0 + 16 * tt + l16 >= n) continue;
+                    const float inv = tot[(16 * tt + l16) * 4];
+                    u16 *row = dst + (chain0 * a.s + rowoff[16 * tt + l16] + (size_t)wave * a.s) * 64 + 4 * g;
+#pragma unroll
+                    for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct] * inv);
+                }
+            }
+        }
+    }
+}
+
+// ── backward glue ────────────────────────────────────────────────────────────────────────────────────
+struct GateGradOut { float *w_alpha, *b_alpha, *w_theta, *b_theta, *w_eta, *b_eta; };
+
+struct GradArgs {
+    const float *dkh, *dvh, *dqh, *dah, *dth, *deh;          // [levels * bs * nh, s, hd] and [levels * bs * nh, s]
+    const u16 *kh, *vh, *qh;                                 // the forward's head-major operands (k, q normalised)
+    const float *k_norms, *q_norms, *alpha, *theta, *eta;    // [levels, n]
+    u16 *G;                                                  // [n, g_ld]: level lvl's d_k, d_v, d_q at col0 + 3 lvl d + {0, d, 2d}
+    long long g_ld, col0;
+    float *part;                                             // [levels][gridDim.x][3][2d + 1]
+    int bs, s, nh, hd, levels;
+    float eps;
+};
+
+// One wave per token and level: head sums of the gate gradients and their activations' derivatives, head merge of
+// d_k, d_v, d_q, backward of the two row normalisations (from the normalised bf16 rows the forward wrote and the
+// stored norms); the token-major gradients leave as bf16 columns of G.  The gate projections' weight and bias
+// gradients are summed per wave in registers and leave as one partial row per workgroup.
+template <int NIT>
+__global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
+    extern __shared__ float redg[];   // [3][2d + 1]
+    const int lane = threadIdx.x & 63, wave_l = threadIdx.x >> 6, d = a.nh * a.hd, d4 = d / 4, lvl = blockIdx.y;
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
+    const long long n = (long long)a.bs * a.s;
+    const size_t chain0 = (size_t)lvl * a.bs * a.nh;
+    const float inv_eps = 1.0f / a.eps;
+    float4 acc[3][2][NIT];
+    float accb[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+    for (int gi = 0; gi < 3; gi++)
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int it = 0; it < NIT; it++) acc[gi][h][it] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (long long tok = wave; tok < n; tok += nwaves) {
+        const long long b = tok / a.s, t = tok - b * a.s;
+        float da = 0.f, dt = 0.f, de = 0.f;
+        for (int h = lane; h < a.nh; h += 64) {
+            const size_t o = (chain0 + b * a.nh + h) * a.s + t;
+            da += a.dah[o]; dt += a.dth[o]; de += a.deh[o];
+        }
+        da = wave_allreduce(da); dt = wave_allreduce(dt); de = wave_allreduce(de);
+        {
+            const float al = a.alpha[lvl * n + tok], th = a.theta[lvl * n + tok], e = a.eta[lvl * n + tok];
+            da *= al * (1.0f - al);
+            dt *= 1.0f - expf(-th);
+            de *= e * (1.0f - e);
+        }
+        accb[0] += da; accb[1] += dt; accb[2] += de;
+        const float kn = a.k_norms[lvl * n + tok], qn = a.q_norms[lvl * n + tok];
+        const float ki = 1.0f / fmaxf(kn, a.eps), qi = 1.0f / fmaxf(qn, a.eps);
+        float4 kk[NIT], qq[NIT], gk[NIT], gv[NIT], gq[NIT];
+        float dk_dot = 0.f, dq_dot = 0.f;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int i4 = lane + 64 * it;
+            kk[it] = qq[it] = gk[it] = gv[it] = gq[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (i4 < d4) {
+                const int i = 4 * i4;
+                const size_t o = ((chain0 + b * a.nh + i / a.hd) * a.s + t) * a.hd + i % a.hd;
+                kk[it] = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(a.kh + o));
+                qq[it] = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(a.qh + o));
+                const float4 vv = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(a.vh + o));
+                gk[it] = *reinterpret_cast<const float4 *>(a.dkh + o);
+                gv[it] = *reinterpret_cast<const float4 *>(a.dvh + o);
+                gq[it] = *reinterpret_cast<const float4 *>(a.dqh + o);
+                fma4(acc[0][0][it], da, kk[it]); fma4(acc[0][1][it], da, vv);
+                fma4(acc[1][0][it], dt, kk[it]); fma4(acc[1][1][it], dt, vv);
+                fma4(acc[2][0][it], de, kk[it]); fma4(acc[2][1][it], de, vv);
+            }
+            dk_dot += dot4(gk[it], kk[it]);
+            dq_dot += dot4(gq[it], qq[it]);
+        }
+        dk_dot = wave_allreduce(dk_dot);
+        dq_dot = wave_allreduce(dq_dot);
+        u16 *grow = a.G + tok * a.g_ld + a.col0 + 3LL * lvl * d;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int i4 = lane + 64 * it;
+            if (i4 >= d4) continue;
+            float4 x, c;
+            if (kn >= a.eps) {
+                x.x = (gk[it].x - kk[it].x * dk_dot) * ki; x.y = (gk[it].y - kk[it].y * dk_dot) * ki;
+                x.z = (gk[it].z - kk[it].z * dk_dot) * ki; x.w = (gk[it].w - kk[it].w * dk_dot) * ki;
+            } else {
+                x.x = gk[it].x * inv_eps; x.y = gk[it].y * inv_eps; x.z = gk[it].z * inv_eps; x.w = gk[it].w * inv_eps;
+            }
+            if (qn >= a.eps) {
+                c.x = (gq[it].x - qq[it].x * dq_dot) * qi; c.y = (gq[it].y - qq[it].y * dq_dot) * qi;
+                c.z = (gq[it].z - qq[it].z * dq_dot) * qi; c.w = (gq[it].w - qq[it].w * dq_dot) * qi;
+            } else {
+                c.x = gq[it].x * inv_eps; c.y = gq[it].y * inv_eps; c.z = gq[it].z * inv_eps; c.w = gq[it].w * inv_eps;
+            }
+            *reinterpret_cast<bf16x4 *>(grow + 4 * i4) = f4_to_bf4(x);
+            *reinterpret_cast<bf16x4 *>(grow + d + 4 * i4) = f4_to_bf4(gv[it]);
+            *reinterpret_cast<bf16x4 *>(grow + 2 * d + 4 * i4) = f4_to_bf4(c);
+        }
+    }
+    // the workgroup's partial row: the waves add their sums into LDS one after the other (fixed order)
+    const int stride = 2 * d + 1;
+    for (int w = 0; w < kSThr / 64; w++) {
+        if (wave_l == w) {
+#pragma unroll
+            for (int gi = 0; gi < 3; gi++) {
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+#pragma unroll
+                    for (int it = 0; it < NIT; it++) {
+                        const int i4 = lane + 64 * it;
+                        if (i4 >= d4) continue;
+                        float *r = redg + gi * stride + h * d + 4 * i4;
+                        const float4 v = acc[gi][h][it];
+                        if (w == 0) { r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w; }
+                        else { r[0] += v.x; r[1] += v.y; r[2] += v.z; r[3] += v.w; }
+                    }
+                if (lane == 0) {
+                    if (w == 0) redg[gi * stride + 2 * d] = accb[gi];
+                    else redg[gi * stride + 2 * d] += accb[gi];
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float *pb = a.part + ((size_t)lvl * gridDim.x + blockIdx.x) * 3 * stride;
+    for (int i = threadIdx.x; i < 3 * stride; i += kSThr) pb[i] = redg[i];
+}
+
+struct GateGradOuts { GateGradOut lv[kMaxLevels]; };
+
+// Sums the workgroups' partial rows [levels][nblk][3][2d + 1] in a fixed order: a workgroup per (64 columns, gate,
+// level), 16 thread groups that each take every 16th row, combined in order.
+__global__ __launch_bounds__(1024) void level_gate_partials_kernel(const float *__restrict__ part, int nblk, int twoD,
+                                                                   GateGradOuts out) {
+    __shared__ float red[16][64];
+    const int col = threadIdx.x & 63, seg = threadIdx.x >> 6, gi = blockIdx.y, lvl = blockIdx.z;
+    const int i = blockIdx.x * 64 + col;
+    const size_t stride = (size_t)twoD + 1;
+    const float *p = part + (size_t)lvl * nblk * 3 * stride;
+    float sum = 0.f;
+    if (i <= twoD)
+        for (int b = seg; b < nblk; b += 16) sum += p[((size_t)b * 3 + gi) * stride + i];
+    red[seg][col] = sum;
+    __syncthreads();
+    if (seg != 0 || i > twoD) return;
+#pragma unroll
+    for (int q = 1; q < 16; q++) sum += red[q][col];
+    const GateGradOut o = out.lv[lvl];
+    float *w = gi == 0 ? o.w_alpha : (gi == 1 ? o.w_theta : o.w_eta);
+    float *bias = gi == 0 ? o.b_alpha : (gi == 1 ? o.b_theta : o.b_eta);
+    if (i < twoD) w[i] = sum;
+    else bias[0] = sum;
+}
+
+// fp32 [n, d] sources side by side into bf16 columns of G (row stride ld), source i at column i * d
+struct ColSrcs { const float *p[kMaxExtra]; };
+__global__ void cols_to_bf16_kernel(ColSrcs src, int count, long long n, int d, u16 *__restrict__ G, long long ld) {
+    const int d4 = d / 4;
+    const long long total = n * count * d4;
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long long)gridDim.x * blockDim.x) {
+        const int c4 = (int)(e % d4), si = (int)((e / d4) % count);
+        const long long r = e / ((long long)d4 * count);
+        const float4 x = *reinterpret_cast<const float4 *>(src.p[si] + r * d + 4 * c4);
+        *reinterpret_cast<bf16x4 *>(G + r * ld + (long long)si * d + 4 * c4) = f4_to_bf4(x);
+    }
+}
+
+__global__ void f32_to_bf16_vec_kernel(const float *__restrict__ x, u16 *__restrict__ out, long long n4) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (long long)gridDim.x * blockDim.x)
+        *reinterpret_cast<bf16x4 *>(out + 4 * i) = f4_to_bf4(*reinterpret_cast<const float4 *>(x + 4 * i));
+}
+
+// last slot of every chain's chunk states -> the carried context memories (copy_final_m_batch, gpu_forward.rs:2824)
+__global__ void final_states_kernel(const float *__restrict__ mc, const float *__restrict__ sc, float *__restrict__ m_ctx,
+                                    float *__restrict__ s_ctx, long long chains, int slots, int dd4) {
+    const long long total = chains * dd4;
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long long)gridDim.x * blockDim.x) {
+        const long long c = e / dd4;
+        const int i = (int)(e % dd4);
+        const size_t src = ((size_t)c * slots + slots - 1) * dd4 + i;
+        reinterpret_cast<float4 *>(m_ctx)[e] = reinterpret_cast<const float4 *>(mc)[src];
+        reinterpret_cast<float4 *>(s_ctx)[e] = reinterpret_cast<const float4 *>(sc)[src];
+    }
+}
+
+// gate = sigmoid(scale * sum_l y_l); gated = attn * gate as bf16 (the output projection's operand)
+struct LevelYs { const float *y[kMaxLevels]; };
+__global__ void combine_gate_x1_kernel(LevelYs lv, int k, float scale, const u16 *__restrict__ attn, float *__restrict__ gate,
+                                       u16 *__restrict__ gated, long long n4) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (long long)gridDim.x * blockDim.x) {
+        float4 sum = *reinterpret_cast<const float4 *>(lv.y[0] + 4 * i);
+        for (int l = 1; l < k; l++) {
+            const float4 y = *reinterpret_cast<const float4 *>(lv.y[l] + 4 * i);
+            sum.x += y.x; sum.y += y.y; sum.z += y.z; sum.w += y.w;
+        }
+        const float4 at = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(attn + 4 * i));
+        float4 gt, o;
+        gt.x = sigmoid_(sum.x * scale); gt.y = sigmoid_(sum.y * scale); gt.z = sigmoid_(sum.z * scale); gt.w = sigmoid_(sum.w * scale);
+        o.x = at.x * gt.x; o.y = at.y * gt.y; o.z = at.z * gt.z; o.w = at.w * gt.w;
+        *reinterpret_cast<float4 *>(gate + 4 * i) = gt;
+        *reinterpret_cast<bf16x4 *>(gated + 4 * i) = f4_to_bf4(o);
+    }
+}
+
+inline int stream_blocks(long long items, int cap) {
+    long long b = (items + kSThr - 1) / kSThr;
+    return (int)(b < 1 ? 1 : (b > cap ? cap : b));
+}
+inline bool al16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+rocblas_handle blas() {
+    static rocblas_handle h = nullptr;
+    if (!h && rocblas_create_handle(&h) != rocblas_status_success) {
+        h = nullptr;
+        fail("level step: rocblas_create_handle failed.");
+        return nullptr;
+    }
+    if (rocblas_set_stream(h, stream()) != rocblas_status_success) {
+        fail("level step: rocblas_set_stream failed.");
+        return nullptr;
+    }
+    return h;
+}
+
+// C (m x n, column-major, ldc, fp32) = op(A) op(B) + beta C with bf16 A, B and fp32 accumulation
+bool gemm_bf16(const char *what, rocblas_operation ta, rocblas_operation tb, long long m, long long n, long long k, const u16 *A,
+               long long lda, const u16 *B, long long ldb, float beta, float *C, long long ldc) {
+    rocblas_handle h = blas();
+    if (!h) return false;
+    const float one = 1.0f;
+    KernelTimer kt(what);
+    const rocblas_status st = rocblas_gemm_ex(h, ta, tb, (rocblas_int)m, (rocblas_int)n, (rocblas_int)k, &one, A,
+                                              rocblas_datatype_bf16_r, (rocblas_int)lda, B, rocblas_datatype_bf16_r,
+                                              (rocblas_int)ldb, &beta, C, rocblas_datatype_f32_r, (rocblas_int)ldc, C,
+                                              rocblas_datatype_f32_r, (rocblas_int)ldc, rocblas_datatype_f32_r,
+                                              rocblas_gemm_algo_standard, 0, 0);
+    if (st != rocblas_status_success) {
+        fail("level step: rocblas_gemm_ex (%s) failed with status %d.", what, (int)st);
+        return false;
+    }
+    return true;
+}
+
+void to_bf16(const float *x, u16 *out, long long count) {
+    KernelTimer kt("f32_to_bf16_vec_kernel");
+    hipLaunchKernelGGL(f32_to_bf16_vec_kernel, dim3(stream_blocks(count / 4, 4096)), dim3(kSThr), 0, stream(), x, out, count / 4);
+    check_launch("f32_to_bf16_vec_kernel");
+}
+
+bool step_dims_ok(const char *fn, int bs, int s, int nh, int hd, int levels, int n_extra, int chunk) {
+    const int d = nh * hd;
+    if (bs <= 0 || s <= 0 || nh <= 0 || hd != 64 || levels < 0 || levels > kMaxLevels || n_extra < 0 ||
+        n_extra > kMaxExtra || (levels == 0 && n_extra == 0) || (d != 256 && d != 512) || chunk < 1 || chunk > 64 ||
+        (long long)bs * s > 0x7fffffffLL / (long long)((3 * levels + n_extra) * d)) {
+        fail("%s: needs head_dim = 64 (got %d), heads * head_dim in {256, 512} (got %d), 0 <= levels <= %d (got %d), "
+             "0 <= n_extra <= %d (got %d), 1 <= chunk_size <= 64 (got %d), bs = %d and seq_len = %d positive and "
+             "bs * seq_len * (projections * d) below 2^31.",
+             fn, hd, d, kMaxLevels, levels, kMaxExtra, n_extra, chunk, bs, s);
+        return false;
+    }
+    return true;
+}
+
+}  // namespace
+}  // namespace nlh
+
+using namespace nlh;
+
+extern "C" {
+
+void level_project_forward_bf16_rocm(const float *x, const float *w_extra, int n_extra, uint16_t *const *extra_out,
+                                     const float *w_levels, const float *const *gate_params, uint16_t *x_bf16,
+                                     uint16_t *k_heads, uint16_t *v_heads, uint16_t *q_heads, float *alpha_heads,
+                                     float *theta_heads, float *eta_heads, float *k_norms, float *q_norms, float *alpha,
+                                     float *theta, float *eta, int bs, int seq_len, int heads, int head_dim, int levels,
+                                     float eps) {
+    const ErrorScope es;
+    if (!step_dims_ok("level_project_forward_bf16_rocm", bs, seq_len, heads, head_dim, levels, n_extra, 1)) return;
+    const int d = heads * head_dim, P = n_extra + 3 * levels;
+    const long long n = (long long)bs * seq_len;
+    if (!al16(x) || !al16(w_extra) || !al16(w_levels) || (x_bf16 && !al16(x_bf16)) || !al16(k_heads) || !al16(v_heads) ||
+        !al16(q_heads)) {
+        fail("level_project_forward_bf16_rocm: buffers must be 16-byte aligned.");
+        return;
+    }
+    u16 *wfrag = reinterpret_cast<u16 *>(scratch(24, (size_t)P * d * d * sizeof(u16)));
+    if (es.failed()) return;
+    ProjArgs a{};
+    a.x = x; a.x_bf16 = x_bf16; a.wfrag = wfrag;
+    for (int e = 0; e < n_extra; e++) {
+        if (!al16(extra_out[e])) { fail("level_project_forward_bf16_rocm: output %d is not 16-byte aligned.", e); return; }
+        a.extra_out[e] = extra_out[e];
+    }
+    for (int l = 0; l < levels; l++) {
+        const float *const *g = gate_params + 6 * l;
+        a.lv[l] = GateParams{g[0], g[1], g[2], g[3], g[4], g[5]};
+        if (!al16(g[0]) || !al16(g[2]) || !al16(g[4])) {
+            fail("level_project_forward_bf16_rocm: gate weight vectors of level %d must be 16-byte aligned.", l);
+            return;
+        }
+    }
+    a.kh = k_heads; a.vh = v_heads; a.qh = q_heads; a.ah = alpha_heads; a.th = theta_heads; a.eh = eta_heads;
+    a.k_norms = k_norms; a.q_norms = q_norms; a.alpha = alpha; a.theta = theta; a.eta = eta;
+    a.n = n; a.bs = bs; a.s = seq_len; a.nh = heads; a.hd = head_dim; a.n_extra = n_extra; a.levels = levels; a.eps = eps;
+    {
+        KernelTimer kt("wfrag_pack_kernel");
+        if (n_extra)
+            hipLaunchKernelGGL(wfrag_pack_kernel, dim3(stream_blocks((long long)n_extra * d * d / 8, 2048)), dim3(kSThr), 0,
+                               stream(), w_extra, wfrag, n_extra, d);
+        if (levels)
+            hipLaunchKernelGGL(wfrag_pack_kernel, dim3(stream_blocks(3LL * levels * d * d / 8, 2048)), dim3(kSThr), 0, stream(),
+                               w_levels, wfrag + (size_t)n_extra * d * d, 3 * levels, d);
+        check_launch("wfrag_pack_kernel");
+    }
+    const size_t lds = (size_t)PT * (d + 8) * 2 + (8 * PT * 4 + PT * 4 + PT) * sizeof(float);
+    static bool attr_set = false;
+    if (!attr_set) {
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(level_project_kernel<512>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 520 * 2 + 18944)), "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(level_project_kernel<256>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 264 * 2 + 18944)), "dynamic LDS size");
+        attr_set = true;
+    }
+    if (es.failed()) return;
+    KernelTimer kt("level_project_kernel");
+    const dim3 grid(ceil_div(n, PT));
+    if (d == 512) hipLaunchKernelGGL(level_project_kernel<512>, grid, dim3(kPThr), lds, stream(), a);
+    else hipLaunchKernelGGL(level_project_kernel<256>, grid, dim3(kPThr), lds, stream(), a);
+    check_launch("level_project_kernel");
+}
+
+void titans_levels_forward_bf16_rocm(const float *x, const float *w_extra, int n_extra, uint16_t *const *extra_out,
+                                     const float *w_levels, const float *const *gate_params, float *m_context,
+                                     float *s_context, uint16_t *x_bf16, uint16_t *k_heads, uint16_t *v_heads,
+                                     uint16_t *q_heads, float *alpha_heads, float *theta_heads, float *eta_heads,
+                                     float *k_norms, float *q_norms, float *alpha, float *theta, float *eta,
+                                     float *m_chunk_states, float *s_chunk_states, float *y_tokens, int bs, int seq_len,
+                                     int heads, int head_dim, int levels, int chunk_size, float eps) {
+    const ErrorScope es;
+    if (!step_dims_ok("titans_levels_forward_bf16_rocm", bs, seq_len, heads, head_dim, levels, n_extra, chunk_size)) return;
+    level_project_forward_bf16_rocm(x, w_extra, n_extra, extra_out, w_levels, gate_params, x_bf16, k_heads, v_heads, q_heads,
+                                    alpha_heads, theta_heads, eta_heads, k_norms, q_norms, alpha, theta, eta, bs, seq_len,
+                                    heads, head_dim, levels, eps);
+    if (es.failed() || levels == 0) return;
+    const int chains = levels * bs * heads, nc = (seq_len + chunk_size - 1) / chunk_size;
+    titans_chunkwise_forward_bf16_tokens_rocm(k_heads, v_heads, q_heads, alpha_heads, theta_heads, eta_heads, m_context,
+                                              s_context, m_chunk_states, s_chunk_states, y_tokens, seq_len, head_dim, chains,
+                                              chunk_size, heads, levels);
+    if (es.failed()) return;
+    KernelTimer kt("final_states_kernel");
+    const int dd4 = head_dim * head_dim / 4;
+    hipLaunchKernelGGL(final_states_kernel, dim3(stream_blocks((long long)chains * dd4, 2048)), dim3(kSThr), 0, stream(),
+                       m_chunk_states, s_chunk_states, m_context, s_context, (long long)chains, nc + 1, dd4);
+    check_launch("final_states_kernel");
+}
+
+void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_extra, int n_extra, const float *const *d_extra,
+                                      const float *w_levels, const uint16_t *k_heads, const uint16_t *v_heads,
+                                      const uint16_t *q_heads, const float *alpha_heads, const float *theta_heads,
+                                      const float *eta_heads, const float *k_norms, const float *q_norms, const float *alpha,
+                                      const float *theta, const float *eta, const float *m_chunk_states,
+                                      const float *s_chunk_states, const float *d_y_tokens, float *d_x, float *d_w_extra,
+                                      float *d_w_levels, float *const *d_gate_params, float *d_m_initial, float *d_s_initial,
+                                      int bs, int seq_len, int heads, int head_dim, int levels, int chunk_size, float eps) {
+    const ErrorScope es;
+    if (!step_dims_ok("titans_levels_backward_bf16_rocm", bs, seq_len, heads, head_dim, levels, n_extra, chunk_size)) return;
+    const int d = heads * head_dim, P = n_extra + 3 * levels, chains = levels * bs * heads;
+    const long long n = (long long)bs * seq_len, R = (long long)P * d;
+    if (!al16(x_bf16) || !al16(d_x) || !al16(w_extra) || !al16(w_levels)) {
+        fail("titans_levels_backward_bf16_rocm: buffers must be 16-byte aligned.");
+        return;
+    }
+    const size_t tok_f = (size_t)chains * seq_len * head_dim, gate_f = (size_t)chains * seq_len;
+    float *hg = scratch(25, (3 * tok_f + 3 * gate_f) * sizeof(float));          // d_k, d_v, d_q, d_alpha, d_theta, d_eta (head-major)
+    u16 *G = reinterpret_cast<u16 *>(scratch(26, (size_t)n * R * sizeof(u16)));
+    u16 *wb = reinterpret_cast<u16 *>(scratch(27, (size_t)R * d * sizeof(u16)));
+    const int nblk = stream_blocks(n * 64, 256);
+    const size_t prow = 3 * (2 * (size_t)d + 1);
+    float *part = scratch(28, (size_t)(levels ? levels : 1) * nblk * prow * sizeof(float));
+    if (es.failed()) return;
+    float *dkh = hg, *dvh = hg + tok_f, *dqh = hg + 2 * tok_f, *dah = hg + 3 * tok_f, *dth = dah + gate_f, *deh = dth + gate_f;
+    if (levels) {
+        titans_chunkwise_backward_bf16_tokens_rocm(k_heads, v_heads, q_heads, alpha_heads, theta_heads, eta_heads,
+                                                   m_chunk_states, s_chunk_states, d_y_tokens, dkh, dvh, dqh, dah, dth, deh,
+                                                   d_m_initial, d_s_initial, seq_len, head_dim, chains, chunk_size, heads,
+                                                   levels, 0);
+        if (es.failed()) return;
+        GradArgs ga{};
+        ga.dkh = dkh; ga.dvh = dvh; ga.dqh = dqh; ga.dah = dah; ga.dth = dth; ga.deh = deh;
+        ga.kh = k_heads; ga.vh = v_heads; ga.qh = q_heads;
+        ga.k_norms = k_norms; ga.q_norms = q_norms; ga.alpha = alpha; ga.theta = theta; ga.eta = eta;
+        ga.G = G; ga.g_ld = R; ga.col0 = (long long)n_extra * d; ga.part = part;
+        ga.bs = bs; ga.s = seq_len; ga.nh = heads; ga.hd = head_dim; ga.levels = levels; ga.eps = eps;
+        {
+            KernelTimer kt("level_grads_bf16_kernel");
+            const dim3 grid(nblk, levels);
+            if (d <= 256) hipLaunchKernelGGL(level_grads_bf16_kernel<1>, grid, dim3(kSThr), prow * sizeof(float), stream(), ga);
+            else hipLaunchKernelGGL(level_grads_bf16_kernel<2>, grid, dim3(kSThr), prow * sizeof(float), stream(), ga);
+            check_launch("level_grads_bf16_kernel");
+        }
+        GateGradOuts go{};
+        for (int l = 0; l < levels; l++) {
+            float *const *g = d_gate_params + 6 * l;
+            go.lv[l] = GateGradOut{g[0], g[1], g[2], g[3], g[4], g[5]};
+        }
+        KernelTimer kt("level_gate_partials_kernel");
+        hipLaunchKernelGGL(level_gate_partials_kernel, dim3(ceil_div(2 * d + 1, 64), 3, levels), dim3(1024), 0, stream(), part,
+                           nblk, 2 * d, go);
+        check_launch("level_gate_partials_kernel");
+    }
+    if (n_extra) {
+        ColSrcs cs{};
+        for (int e = 0; e < n_extra; e++) {
+            if (!al16(d_extra[e])) { fail("titans_levels_backward_bf16_rocm: gradient %d is not 16-byte aligned.", e); return; }
+            cs.p[e] = d_extra[e];
+        }
+        KernelTimer kt("cols_to_bf16_kernel");
+        hipLaunchKernelGGL(cols_to_bf16_kernel, dim3(stream_blocks(n * n_extra * (d / 4), 4096)), dim3(kSThr), 0, stream(), cs,
+                           n_extra, n, d, G, R);
+        check_launch("cols_to_bf16_kernel");
+        to_bf16(w_extra, wb, (long long)n_extra * d * d);
+    }
+    if (levels) to_bf16(w_levels, wb + (size_t)n_extra * d * d, 3LL * levels * d * d);
+    if (es.failed()) return;
+    // d_x [n, d] = G [n, R] Wb [R, d];  d_W [R, d] = G^T x  (row-major buffers as column-major operands)
+    if (!gemm_bf16("gemm d_x", rocblas_operation_none, rocblas_operation_none, d, n, R, wb, d, G, R, 0.f, d_x, d)) return;
+    if (n_extra &&
+        !gemm_bf16("gemm d_w", rocblas_operation_none, rocblas_operation_transpose, d, (long long)n_extra * d, n, x_bf16, d, G, R,
+                   0.f, d_w_extra, d))
+        return;
+    if (levels)
+        gemm_bf16("gemm d_w", rocblas_operation_none, rocblas_operation_transpose, d, 3LL * levels * d, n, x_bf16, d,
+                  G + (size_t)n_extra * d, R, 0.f, d_w_levels, d);
+}
+
+void cms_combine_gate_bf16x1_rocm(const float *const *y_levels, int k, const uint16_t *attn_out, float *gate,
+                                  uint16_t *gated_bf16, long long n) {
+    if (k < 1 || k > kMaxLevels) { fail("cms_combine_gate_bf16x1_rocm: k=%d must be in [1, %d].", k, kMaxLevels); return; }
+    if (n <= 0) return;
+    if (n % 4 || (((uintptr_t)attn_out) & 7) || !al16(gate) || (((uintptr_t)gated_bf16) & 7)) {
+        fail("cms_combine_gate_bf16x1_rocm: n=%lld must be a multiple of 4 and the buffers aligned.", n);
+        return;
+    }
+    LevelYs lv{};
+    for (int l = 0; l < k; l++) {
+        if (!al16(y_levels[l])) { fail("cms_combine_gate_bf16x1_rocm: level %d is not 16-byte aligned.", l); return; }
+        lv.y[l] = y_levels[l];
+    }
+    const float scale = k > 2 ? 1.0f / sqrtf((float)k) : 1.0f;
+    KernelTimer kt("combine_gate_x1_kernel");
+    hipLaunchKernelGGL(combine_gate_x1_kernel, dim3(stream_blocks(n / 4, 4096)), dim3(kSThr), 0, stream(), lv, k, scale, attn_out,
+                       gate, gated_bf16, n / 4);
+    check_launch("combine_gate_x1_kernel");
+}
+
+void linear_forward_bf16_rocm(const uint16_t *a_bf16, const float *w, float *out, int n, int d_in, int d_out) {
+    const ErrorScope es;
+    if (n <= 0 || d_in <= 0 || d_out <= 0 || (d_in * (long long)d_out) % 4) {
+        fail("linear_forward_bf16_rocm: invalid dims n=%d d_in=%d d_out=%d (d_in * d_out must be a multiple of 4).", n, d_in, d_out);
+        return;
+    }
+    u16 *wb = reinterpret_cast<u16 *>(scratch(27, (size_t)d_in * d_out * sizeof(u16)));
+    if (es.failed()) return;
+    to_bf16(w, wb, (long long)d_in * d_out);
+    // out [n, d_out] = a [n, d_in] W^T
+    gemm_bf16("gemm linear", rocblas_operation_transpose, rocblas_operation_none, d_out, n, d_in, wb, d_in, a_bf16, d_in, 0.f, out,
+              d_out);
+}
+
+void linear_backward_bf16_rocm(const float *d_out_f32, const uint16_t *a_bf16, const float *w, float *d_a, float *d_w, int n,
+                               int d_in, int d_out) {
+    const ErrorScope es;
+    if (n <= 0 || d_in <= 0 || d_out <= 0 || (d_in * (long long)d_out) % 4 || ((long long)n * d_out) % 4) {
+        fail("linear_backward_bf16_rocm: invalid dims n=%d d_in=%d d_out=%d (products must be multiples of 4).", n, d_in, d_out);
+        return;
+    }
+    u16 *wb = reinterpret_cast<u16 *>(scratch(27, (size_t)d_in * d_out * sizeof(u16)));
+    u16 *gb = reinterpret_cast<u16 *>(scratch(26, (size_t)n * d_out * sizeof(u16)));
+    if (es.failed()) return;
+    to_bf16(w, wb, (long long)d_in * d_out);
+    to_bf16(d_out_f32, gb, (long long)n * d_out);
+    // d_a [n, d_in] = g [n, d_out] W [d_out, d_in];  d_W [d_out, d_in] = g^T a
+    if (d_a && !gemm_bf16("gemm linear d_a", rocblas_operation_none, rocblas_operation_none, d_in, n, d_out, wb, d_in, gb, d_out,
+                          0.f, d_a, d_in))
+        return;
+    if (d_w)
+        gemm_bf16("gemm linear d_w", rocblas_operation_none, rocblas_operation_transpose, d_in, d_out, n, a_bf16, d_in, gb, d_out,
+                  0.f, d_w, d_in);
+}
+
+}  // extern "C"

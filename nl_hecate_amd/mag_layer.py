@@ -90,8 +90,17 @@ class MagLayer:
     """k Titans levels + SWA, MAG sigmoid gating.  `rule`: "exact" (checkpointed exact recurrence,
     fp32) or "chunkwise" (frozen-M0 chunkwise rule in matrix form, bf16 k/v/q)."""
 
-    def __init__(self, d, heads, k, window, periods, rule="exact", chunk=64, params=None, seed=0):
+    def __init__(self, d, heads, k, window, periods, rule="exact", chunk=64, params=None, seed=0,
+                 precision="bf16x3"):
+        """precision: how the dense projections run.  "bf16x3": operands split into hi + lo bf16 pairs, three
+        products per GEMM (agrees with an fp32 GEMM to 5e-6).  "bf16": operands rounded once to bf16, fp32
+        accumulation, and the level step (projections, normalisation, gates, head split, rule, and the whole
+        backward down to d_x and the weight gradients) is ONE call into the library per direction
+        (titans_levels_{forward,backward}_bf16_rocm): no GEMM is issued from this module.  Needs the chunkwise
+        rule at head size 64, d in {256, 512}, chunk <= 64, window <= 512; other layers keep "bf16x3"."""
         assert d % heads == 0
+        assert precision in ("bf16x3", "bf16")
+        self.precision = precision
         self.d, self.nh, self.hd, self.k, self.window = d, heads, d // heads, k, window
         self.rule, self.chunk = rule, chunk
         self.p = params if params is not None else init_params(d, k, seed)
@@ -408,6 +417,8 @@ class MagLayer:
         pulse = self.conductor.pulse()
         active = [bool(a) for a in pulse.active_levels]
         na = active.index(False) if False in active else self.k
+        if self._single_bf16_ok(active, na):
+            return self._forward_bf16(x, pulse, active, na)
         stacked = (self.rule == "chunkwise" and self.stack_levels and self.split_gemm and self.fused_glue
                    and na >= 2 and not any(active[na:]) and hd == 64 and self.chunk <= 64 and d <= 1024)
         ops = self._split_operands(x2, 3 * d * (1 + na) if stacked else 0) if self.split_gemm else None
@@ -446,6 +457,94 @@ class MagLayer:
         cache = dict(x=x, q=q, k=k, v=v, aw=aw, attn=attn, gate=gate, gated=gated, levels=caches, pulse=pulse,
                      ys=ys, ops=ops, stack=stack)
         return out, cache
+
+    # ── the layer with single-bf16 projections: every heavy step is one call into the library ─────────────
+    def _single_bf16_ok(self, active, na):
+        return (self.precision == "bf16" and self.rule == "chunkwise" and self.hd == 64 and self.d in (256, 512)
+                and self.chunk <= 64 and self.window <= 512 and not any(active[na:]))
+
+    def _gate_ptrs(self, levels):
+        return (ctypes.c_void_p * (6 * len(levels)))(*[t.data_ptr() for l in levels for t in
+                                                       (l.w_alpha, l.b_alpha, l.w_theta, l.b_theta, l.w_eta, l.b_eta)])
+
+    def _forward_bf16(self, x, pulse, active, na):
+        bs, s, d = x.shape
+        nh, hd, C, k = self.nh, self.hd, self.chunk, self.k
+        B, n = bs * nh, bs * s
+        self.ensure_state(bs)
+        bf = torch.bfloat16
+        q, kk, v = (_new(bs, s, d, dtype=bf) for _ in range(3))
+        xb = _new(n, d, dtype=bf)
+        kh, vh, qh = (_new(max(na, 1) * B, s, hd, dtype=bf) for _ in range(3))
+        ah, th, eh = (_new(max(na, 1) * B, s) for _ in range(3))
+        k_norms, q_norms, alpha, theta, eta = (_new(max(na, 1), n) for _ in range(5))
+        nc = (s + C - 1) // C
+        mc, sc = _new(max(na, 1) * B, nc + 1, hd * hd), _new(max(na, 1) * B, nc + 1, hd * hd)
+        y_all = _new(max(na, 1), bs, s, d)
+        extra = (ctypes.c_void_p * 3)(q.data_ptr(), kk.data_ptr(), v.data_ptr())
+        lib.titans_levels_forward_bf16_rocm(
+            x.data_ptr(), self._pack.data_ptr(), 3, extra, self._pack[3 * d:].data_ptr(), self._gate_ptrs(self.p.levels[:na]),
+            self._m_all.data_ptr(), self._s_all.data_ptr(), xb.data_ptr(), kh.data_ptr(), vh.data_ptr(), qh.data_ptr(),
+            ah.data_ptr(), th.data_ptr(), eh.data_ptr(), k_norms.data_ptr(), q_norms.data_ptr(), alpha.data_ptr(),
+            theta.data_ptr(), eta.data_ptr(), mc.data_ptr(), sc.data_ptr(), y_all.data_ptr(), bs, s, nh, hd, na, C, 1e-8)
+        attn = _new(bs, s, d, dtype=bf)
+        aw = _new(bs, nh, s, 2)
+        D.call("swa_forward_lse_bf16_rocm", q, kk, v, attn, aw, s, nh, hd, self.window, bs)
+        ys, frozen = [y_all[lv] for lv in range(na)], []
+        for lv in range(na, k):
+            # frozen level (gpu_memory_read_only, gpu_forward.rs:2906-2950): y = M_h q with the raw projection q
+            q_raw, y = _new(n, d), _new(bs, s, d)
+            lib.linear_forward_bf16_rocm(xb.data_ptr(), self.p.levels[lv].w_q.data_ptr(), q_raw.data_ptr(), n, d, d)
+            m_shared = self.m_state[lv][:nh].contiguous()
+            D.call("memory_read_only_f32_rocm", q_raw, m_shared, y, n, nh, hd)
+            ys.append(y)
+            frozen.append(m_shared)
+        gate, gated = _new(bs, s, d), _new(n, d, dtype=bf)
+        ptrs = (ctypes.c_void_p * k)(*[y.data_ptr() for y in ys])
+        lib.cms_combine_gate_bf16x1_rocm(ptrs, k, attn.data_ptr(), gate.data_ptr(), gated.data_ptr(), n * d)
+        out = _new(bs, s, d)
+        lib.linear_forward_bf16_rocm(gated.data_ptr(), self.p.w_o.data_ptr(), out.data_ptr(), n, d, d)
+        cache = dict(bf16=True, x=x, xb=xb, q=q, k=kk, v=v, aw=aw, attn=attn, gate=gate, gated=gated, pulse=pulse, ys=ys, na=na,
+                     kh=kh, vh=vh, qh=qh, ah=ah, th=th, eh=eh, k_norms=k_norms, q_norms=q_norms, alpha=alpha, theta=theta,
+                     eta=eta, mc=mc, sc=sc, frozen=frozen)
+        return out, cache
+
+    def _backward_bf16(self, c, d_out, grads):
+        x = c["x"]
+        bs, s, d = x.shape
+        nh, hd, k, na = self.nh, self.hd, self.k, c["na"]
+        n = bs * s
+        d_gated = _new(n, d)
+        lib.linear_backward_bf16_rocm(d_out.data_ptr(), c["gated"].data_ptr(), self.p.w_o.data_ptr(), d_gated.data_ptr(),
+                                      grads.w_o.data_ptr(), n, d, d)
+        d_attn, d_ycomb = _new(bs, s, d), _new(bs, s, d)
+        lib.cms_gate_backward_bf16_rocm(d_gated.data_ptr(), c["attn"].data_ptr(), c["gate"].data_ptr(), k,
+                                        d_attn.data_ptr(), d_ycomb.data_ptr(), n * d)
+        dq = _new(bs, s, d)
+        dkv = _zeros(2, bs, s, d)
+        D.call("swa_backward_lse_bf16_rocm", c["q"], c["k"], c["v"], c["aw"], d_attn, dq, dkv[0], dkv[1], s, nh, hd,
+               self.window, bs)
+        d_x = _new(bs, s, d)
+        seeds = _zeros(2, hd, hd)
+        d_extra = (ctypes.c_void_p * 3)(dq.data_ptr(), dkv[0].data_ptr(), dkv[1].data_ptr())
+        gl = grads.levels[:na]
+        gate_out = (ctypes.c_void_p * (6 * na))(*[t.data_ptr() for g in gl for t in
+                                                  (g.w_alpha, g.b_alpha, g.w_theta, g.b_theta, g.w_eta, g.b_eta)])
+        lib.titans_levels_backward_bf16_rocm(
+            c["xb"].data_ptr(), self._pack.data_ptr(), 3, d_extra, self._pack[3 * d:].data_ptr(), c["kh"].data_ptr(),
+            c["vh"].data_ptr(), c["qh"].data_ptr(), c["ah"].data_ptr(), c["th"].data_ptr(), c["eh"].data_ptr(),
+            c["k_norms"].data_ptr(), c["q_norms"].data_ptr(), c["alpha"].data_ptr(), c["theta"].data_ptr(),
+            c["eta"].data_ptr(), c["mc"].data_ptr(), c["sc"].data_ptr(), d_ycomb.data_ptr(), d_x.data_ptr(),
+            grads.pack.data_ptr(), grads.pack[3 * d:].data_ptr(), gate_out, seeds[0].data_ptr(), seeds[1].data_ptr(),
+            bs, s, nh, hd, na, self.chunk, 1e-8)
+        for i, lv in enumerate(range(na, k)):
+            # read-only level: only the q path carries gradient
+            dq_l, dx_l = _new(n, d), _new(n, d)
+            D.call("memory_read_only_backward_f32_rocm", d_ycomb, c["frozen"][i], dq_l, n, nh, hd)
+            lib.linear_backward_bf16_rocm(dq_l.data_ptr(), c["xb"].data_ptr(), self.p.levels[lv].w_q.data_ptr(),
+                                          dx_l.data_ptr(), grads.levels[lv].w_q.data_ptr(), n, d, d)
+            d_x.view(n, d).add_(dx_l)
+        return d_x
 
     # ── decode: one token with a KV cache ────────────────────────────────────
     def decode_reset(self, max_len):
@@ -491,6 +590,8 @@ class MagLayer:
             grads = self.new_grads()
         else:
             grads.flat.zero_()
+        if cache.get("bf16"):
+            return self._backward_bf16(cache, d_out, grads), grads
         ops, stack = cache["ops"], cache["stack"]
         if cache["gated"].dtype == torch.bfloat16:
             # d_gated = d_out W_o and d_W_o = d_out^T gated from one packing (H | L | H) of d_out
