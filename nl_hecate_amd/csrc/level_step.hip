@@ -51,19 +51,19 @@ __device__ __forceinline__ bf16x4 f4_to_bf4(const float4 &x) {
     return bf16x4{(__bf16)x.x, (__bf16)x.y, (__bf16)x.z, (__bf16)x.w};
 }
 
-struct GateParams { const float *w_alpha, *b_alpha, *w_theta, *b_theta, *w_eta, *b_eta; };
 
 struct ProjArgs {
     const float *x;            // [n, D]
     u16 *x_bf16;               // [n, D]: x rounded to bf16 (the backward's GEMM operand); may be null
     const u16 *wfrag;          // packed weights, projection p at p * D * D (wfrag_pack_kernel)
+    const u16 *ufrag;          // folded gate vectors of every level, [levels][D / 32][64][8] (gate_fold_kernel)
     u16 *extra_out[kMaxExtra]; // plain projections, bf16 [n, D] each
-    GateParams lv[kMaxLevels];
+    const float *bias[kMaxLevels][3];   // b_alpha, b_theta, b_eta
     u16 *kh, *vh, *qh;         // [levels * bs * nh, s, hd]
     float *ah, *th, *eh;       // [levels * bs * nh, s]
     float *k_norms, *q_norms, *alpha, *theta, *eta;   // [levels, n]
     long long n;
-    int bs, s, nh, hd, n_extra, levels;
+    int bs, s, nh, n_extra, levels;
     float eps;
 };
 
@@ -89,12 +89,62 @@ __global__ void wfrag_pack_kernel(const float *__restrict__ W, u16 *__restrict__
     }
 }
 
+// The gate projections see k and v, which are projections of x themselves: [k | v] . w = x . (Wk^T w[:D] + Wv^T w[D:])
+// up to the normalisation of k, a scalar per token.  This kernel folds the three gate vectors of a level through
+// the level's (bf16-rounded, as the projection kernel multiplies them) Wk and Wv into six D-vectors u_q,
+// q = (alpha, theta, eta) x (k part, v part), so that the projection kernel gets all six dot products of a token
+// from ONE extra tile of 16 output columns instead of 6 D multiply-adds per token and phase in its epilogue.
+// Each u is stored as a hi + lo pair of bf16 (the sums keep fp32 accuracy), as the A operand of that tile:
+// row 2 q' = hi, row 2 q' + 1 = lo with q' = (k.alpha, k.theta, k.eta, v.alpha, v.theta, v.eta), rows 12..15 zero;
+// element (row r, contraction index j) at [j / 32][lane = 16 ((j % 32) / 8) + r][j % 8].
+struct FoldArgs { const float *w[kMaxLevels][3]; };
+constexpr int kFoldSlices = 16;   // the sum over the D columns is cut into slices that run as separate workgroups
+// part [levels][kFoldSlices][6][D]: slice sl's share of u_q[j]
+__global__ __launch_bounds__(64) void gate_fold_partial_kernel(const float *__restrict__ w_levels, FoldArgs g,
+                                                               float *__restrict__ part, int D) {
+    const int lvl = blockIdx.y, sl = blockIdx.z, j = blockIdx.x * 64 + threadIdx.x;
+    const int per = D / kFoldSlices, c0 = sl * per;
+    if (j >= D) return;
+    const float *Wk = w_levels + (size_t)lvl * 3 * D * D, *Wv = Wk + (size_t)D * D;
+    float u[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+    for (int c = c0; c < c0 + per; c++) {
+        const float wk = (float)(__bf16)Wk[(size_t)c * D + j], wv = (float)(__bf16)Wv[(size_t)c * D + j];
+#pragma unroll
+        for (int q = 0; q < 3; q++) {
+            u[q] = fmaf(wk, g.w[lvl][q][c], u[q]);
+            u[3 + q] = fmaf(wv, g.w[lvl][q][D + c], u[3 + q]);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 6; q++) part[(((size_t)lvl * kFoldSlices + sl) * 6 + q) * D + j] = u[q];
+}
+__global__ __launch_bounds__(64) void gate_fold_finish_kernel(const float *__restrict__ part, u16 *__restrict__ ufrag, int D) {
+    const int lvl = blockIdx.y, j = blockIdx.x * 64 + threadIdx.x;
+    if (j >= D) return;
+    u16 *base = ufrag + ((size_t)lvl * (D / 32) + j / 32) * 512 + (size_t)16 * ((j % 32) / 8) * 8 + j % 8;
+    __bf16 *out = reinterpret_cast<__bf16 *>(base);
+#pragma unroll
+    for (int q = 0; q < 6; q++) {
+        float u = 0.f;
+        for (int sl = 0; sl < kFoldSlices; sl++) u += part[(((size_t)lvl * kFoldSlices + sl) * 6 + q) * D + j];
+        const __bf16 hi = (__bf16)u;
+        out[(2 * q) * 8] = hi;
+        out[(2 * q + 1) * 8] = (__bf16)(u - (float)hi);
+    }
+#pragma unroll
+    for (int r = 12; r < 16; r++) out[r * 8] = (__bf16)0.f;
+}
+
 // acc[tt][ct][r] = sum_k W[col][k] x[token][k] with col = 16 ct + 4 (lane / 16) + r of the wave's 64 columns and
 // token = 16 tt + lane % 16 of the workgroup's 128: the weights as the A operand straight from global memory
-// (requested three steps ahead), x as the B operand from LDS.
+// (a ring of four steps, requested three steps ahead), x as the B operand from LDS (two token tiles per unit of
+// eight products, the next unit's pair requested before this unit's products are issued).  Fully unrolled, with
+// the order of requests and products pinned: left to itself the scheduler sinks every load to its first use and
+// the wave then waits a full memory latency per step.
 template <int D>
 __device__ __forceinline__ void project_block(const u16 *Xs, const u16 *wf, f32x4 (&acc)[PT / 16][4]) {
-    constexpr int XS = D + 8, KS = D / 32, AHEAD = 3;
+    constexpr int XS = D + 8, KS = D / 32, RING = 4, UNITS = KS * (PT / 32);
     const int lane = threadIdx.x & 63;
     const bf16x8 *wp = reinterpret_cast<const bf16x8 *>(wf) + lane;
     const u16 *xb = Xs + (lane & 15) * XS + 8 * (lane >> 4);
@@ -102,44 +152,45 @@ __device__ __forceinline__ void project_block(const u16 *Xs, const u16 *wf, f32x
     for (int tt = 0; tt < PT / 16; tt++)
 #pragma unroll
         for (int ct = 0; ct < 4; ct++) acc[tt][ct] = zero4();
-    static_assert(KS % (AHEAD + 1) == 0, "the k loop is unrolled by the depth of the weight ring");
-    bf16x8 w[AHEAD + 1][4];
+    bf16x8 w[RING][4], b[2][2];
 #pragma unroll
-    for (int p = 0; p < AHEAD; p++)
+    for (int p = 0; p < RING - 1 && p < KS; p++)
 #pragma unroll
         for (int ct = 0; ct < 4; ct++) w[p][ct] = wp[(p * 4 + ct) * 64];
-    // a rolled loop over groups of four steps: the ring slots are compile-time indices inside a group, and the
-    // compiler cannot pull the loads of later groups up (a fully unrolled loop spilled hundreds of registers)
-#pragma unroll 1
-    for (int ks0 = 0; ks0 < KS; ks0 += AHEAD + 1) {
+    b[0][0] = *reinterpret_cast<const bf16x8 *>(xb);
+    b[0][1] = *reinterpret_cast<const bf16x8 *>(xb + 16 * XS);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j <= AHEAD; j++) {
-            const int ks = ks0 + j;
-            const int nx = ks + AHEAD < KS ? ks + AHEAD : KS - 1;   // past the end: a harmless repeat of the last step
+    for (int u = 0; u < UNITS; u++) {
+        const int ks = u / (PT / 32), pr = u % (PT / 32);
+        if (pr == 0 && ks + RING - 1 < KS) {
 #pragma unroll
-            for (int ct = 0; ct < 4; ct++) w[(j + AHEAD) % (AHEAD + 1)][ct] = wp[(nx * 4 + ct) * 64];
-            // the requests stay where they are written: left to itself the scheduler sinks each load to its first use
-            // (three steps later) and the wave then waits a full memory latency per step
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int tt = 0; tt < PT / 16; tt++) {
-                const bf16x8 b = *reinterpret_cast<const bf16x8 *>(xb + 16 * tt * XS + 32 * ks);
-#pragma unroll
-                for (int ct = 0; ct < 4; ct++) acc[tt][ct] = mfma32(w[j][ct], b, acc[tt][ct]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+            for (int ct = 0; ct < 4; ct++) w[(ks + RING - 1) % RING][ct] = wp[((ks + RING - 1) * 4 + ct) * 64];
         }
+        if (u + 1 < UNITS) {
+            const int nks = (u + 1) / (PT / 32), npr = (u + 1) % (PT / 32);
+            b[(u + 1) & 1][0] = *reinterpret_cast<const bf16x8 *>(xb + 32 * npr * XS + 32 * nks);
+            b[(u + 1) & 1][1] = *reinterpret_cast<const bf16x8 *>(xb + (32 * npr + 16) * XS + 32 * nks);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int ct = 0; ct < 4; ct++) acc[2 * pr + h][ct] = mfma32(w[ks % RING][ct], b[u & 1][h], acc[2 * pr + h][ct]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
+__device__ __forceinline__ float gate_act(int q, float pre) { return q == 1 ? softplus_(pre) : sigmoid_(pre); }
+
 template <int D>
 __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
-    constexpr int XS = D + 8, CB = D / 64, D4 = D / 4;
+    constexpr int XS = D + 8, CB = D / 64, D4 = D / 4, KS = D / 32;
     extern __shared__ __align__(16) unsigned char smem[];
     u16 *Xs = reinterpret_cast<u16 *>(smem);                                   // [PT][XS]
-    float *red = reinterpret_cast<float *>(smem + (size_t)PT * XS * 2);         // [8][PT][4]
-    float *tot = red + 8 * PT * 4;                                              // [PT][4]
-    int *rowoff = reinterpret_cast<int *>(tot + PT * 4);                        // [PT]: b * nh * s + t of the token
+    float *red = reinterpret_cast<float *>(smem + (size_t)PT * XS * 2);         // [2][8][PT]: per-wave sums of squares
+    float *gdot = red + 2 * 8 * PT;                                             // [2][PT][8]: x . u_q (6 used)
+    float *tot = gdot + 2 * PT * 8;                                             // [PT]: 1 / max(|k|, eps)
+    int *rowoff = reinterpret_cast<int *>(tot + PT);                            // [PT]: b * nh * s + t of the token
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     const long long tok0 = (long long)blockIdx.x * PT, n = a.n;
     const bool wave_on = wave < CB;
@@ -187,37 +238,24 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
         }
 
     for (int lvl = 0; lvl < a.levels; lvl++) {
-        const GateParams gp = a.lv[lvl];
         const size_t pbase = (size_t)(a.n_extra + 3 * lvl) * D * D;
         const size_t chain0 = (size_t)lvl * a.bs * a.nh;
+        float *gd = gdot + (lvl & 1) * PT * 8;
+        {   // the six gate dot products of the wave's 16 tokens (token tile `wave`): one tile of 16 columns
+            const bf16x8 *up = reinterpret_cast<const bf16x8 *>(a.ufrag) + (size_t)lvl * KS * 64 + lane;
+            const u16 *xb = Xs + (16 * wave + l16) * XS + 8 * g;
+            f32x4 ga = zero4();
+#pragma unroll 4
+            for (int ks = 0; ks < KS; ks++)
+                ga = mfma32(up[ks * 64], *reinterpret_cast<const bf16x8 *>(xb + 32 * ks), ga);
+            // lane group g holds rows 4g .. 4g + 3 = (hi, lo) of quantities 2g and 2g + 1
+            if (g < 3) *reinterpret_cast<float2 *>(gd + (16 * wave + l16) * 8 + 2 * g) = make_float2(ga[0] + ga[1], ga[2] + ga[3]);
+        }
 #pragma unroll 1
         for (int p = 0; p < 3; p++) {   // k, v, q
-            if (wave_on) {
-                project_block<D>(Xs, a.wfrag + pbase + (size_t)p * D * D + wave_frag, acc);
-                float4 wa[4], wt[4], we[4];
-                if (p < 2) {
-#pragma unroll
-                    for (int ct = 0; ct < 4; ct++) {
-                        const int c = p * D + colw + 16 * ct;
-                        wa[ct] = *reinterpret_cast<const float4 *>(gp.w_alpha + c);
-                        wt[ct] = *reinterpret_cast<const float4 *>(gp.w_theta + c);
-                        we[ct] = *reinterpret_cast<const float4 *>(gp.w_eta + c);
-                    }
-                }
-#pragma unroll
-                for (int tt = 0; tt < PT / 16; tt++) {
-                    float ss = 0.f, da = 0.f, dt = 0.f, de = 0.f;
-#pragma unroll
-                    for (int ct = 0; ct < 4; ct++) {
-                        const f32x4 v = acc[tt][ct];
-                        if (p != 1) ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
-                        if (p < 2) { da += dotv(v, wa[ct]); dt += dotv(v, wt[ct]); de += dotv(v, we[ct]); }
-                    }
-                    if (p != 1) ss = sum_rows(ss);
-                    if (p < 2) { da = sum_rows(da); dt = sum_rows(dt); de = sum_rows(de); }
-                    if (g == 0) *reinterpret_cast<float4 *>(red + (wave * PT + 16 * tt + l16) * 4) = make_float4(ss, da, dt, de);
-                }
-                if (p == 1) {   // v leaves as it is
+            if (wave_on) project_block<D>(Xs, a.wfrag + pbase + (size_t)p * D * D + wave_frag, acc);
+            if (p == 1) {   // v leaves as it is
+                if (wave_on) {
 #pragma unroll
                     for (int tt = 0; tt < PT / 16; tt++) {
                         if (tok0 + 16 * tt + l16 >= n) continue;
@@ -226,46 +264,60 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
                         for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct]);
                     }
                 }
+                continue;
             }
-            __syncthreads();
-            if (tid < PT) {
-                float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-                for (int w = 0; w < CB; w++) {
-                    const float4 r = *reinterpret_cast<const float4 *>(red + (w * PT + tid) * 4);
-                    s.x += r.x; s.y += r.y; s.z += r.z; s.w += r.w;
-                }
-                const long long tok = tok0 + tid;
-                float *tt_ = tot + tid * 4;
-                if (p == 0) {
-                    const float kn = sqrtf(s.x), ki = 1.0f / fmaxf(kn, a.eps);
-                    tt_[0] = ki; tt_[1] = s.y * ki; tt_[2] = s.z * ki; tt_[3] = s.w * ki;
-                    if (tok < n) a.k_norms[lvl * n + tok] = kn;
-                } else if (p == 1) {
-                    const float al = sigmoid_(tt_[1] + s.y + gp.b_alpha[0]), th = softplus_(tt_[2] + s.z + gp.b_theta[0]);
-                    const float et = sigmoid_(tt_[3] + s.w + gp.b_eta[0]);
-                    if (tok < n) {
-                        a.alpha[lvl * n + tok] = al; a.theta[lvl * n + tok] = th; a.eta[lvl * n + tok] = et;
-                        for (int h = 0; h < a.nh; h++) {
-                            const size_t o = chain0 * a.s + rowoff[tid] + (size_t)h * a.s;
-                            a.ah[o] = al; a.th[o] = th; a.eh[o] = et;
-                        }
+            // k, q: the row norm over all D columns = over the eight waves
+            float *rd = red + (p >> 1) * 8 * PT;
+            if (wave_on) {
+#pragma unroll
+                for (int tt = 0; tt < PT / 16; tt++) {
+                    float ss = 0.f;
+#pragma unroll
+                    for (int ct = 0; ct < 4; ct++) {
+                        const f32x4 v = acc[tt][ct];
+                        ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
                     }
-                } else {
-                    const float qn = sqrtf(s.x);
-                    tt_[0] = 1.0f / fmaxf(qn, a.eps);
-                    if (tok < n) a.q_norms[lvl * n + tok] = qn;
+                    ss = sum_rows(ss);
+                    if (g == 0) rd[wave * PT + 16 * tt + l16] = ss;
                 }
             }
             __syncthreads();
-            if (wave_on && p != 1) {
+            float inv[PT / 16];
+#pragma unroll
+            for (int tt = 0; tt < PT / 16; tt++) {
+                // lane group g adds the partial sums of waves 2g and 2g + 1, the four groups are then summed
+                float ss = (2 * g < CB ? rd[2 * g * PT + 16 * tt + l16] : 0.f) + (2 * g + 1 < CB ? rd[(2 * g + 1) * PT + 16 * tt + l16] : 0.f);
+                ss = sum_rows(ss);
+                const float nrm = sqrtf(ss);
+                inv[tt] = 1.0f / fmaxf(nrm, a.eps);
+                if (wave == 0 && g == 0) {
+                    const long long tok = tok0 + 16 * tt + l16;
+                    if (p == 0) tot[16 * tt + l16] = inv[tt];
+                    if (tok < n) (p == 0 ? a.k_norms : a.q_norms)[lvl * n + tok] = nrm;
+                }
+            }
+            if (wave_on) {
                 u16 *dst = p == 0 ? a.kh : a.qh;
 #pragma unroll
                 for (int tt = 0; tt < PT / 16; tt++) {
                     if (tok0 + 16 * tt + l16 >= n) continue;
-                    const float inv = tot[(16 * tt + l16) * 4];
                     u16 *row = dst + (chain0 * a.s + rowoff[16 * tt + l16] + (size_t)wave * a.s) * 64 + 4 * g;
 #pragma unroll
-                    for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct] * inv);
+                    for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct] * inv[tt]);
+                }
+            }
+            if (p == 2 && tid < 3 * PT) {
+                // the gates: one (token, gate) per thread; the q phase's barrier lies between wave 0's write of the
+                // k norms' inverses, every wave's write of the gate dot products, and this read
+                const int token = tid & (PT - 1), q = tid >> 7;   // PT = 128
+                const long long tok = tok0 + token;
+                const float pre = gd[token * 8 + q] * tot[token] + gd[token * 8 + 3 + q] + a.bias[lvl][q][0];
+                const float val = gate_act(q, pre);
+                if (tok < n) {
+                    float *tm = q == 0 ? a.alpha : (q == 1 ? a.theta : a.eta), *hm = q == 0 ? a.ah : (q == 1 ? a.th : a.eh);
+                    tm[lvl * n + tok] = val;
+                    hm += chain0 * a.s + rowoff[token];
+                    for (int h = 0; h < a.nh; h++) hm[(size_t)h * a.s] = val;
                 }
             }
         }
@@ -514,6 +566,52 @@ bool gemm_bf16(const char *what, rocblas_operation ta, rocblas_operation tb, lon
     return true;
 }
 
+// sum of `parts` buffers of count floats, in order
+__global__ void sum_parts_kernel(const float *__restrict__ part, float *__restrict__ out, long long count4, int parts) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count4; i += (long long)gridDim.x * blockDim.x) {
+        float4 s = reinterpret_cast<const float4 *>(part)[i];
+        for (int p = 1; p < parts; p++) {
+            const float4 v = reinterpret_cast<const float4 *>(part)[p * count4 + i];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        reinterpret_cast<float4 *>(out)[i] = s;
+    }
+}
+
+// Weight gradient C [rows, m] (row-major) = G^T a over `tokens` tokens, a [tokens, m] (lda), G [tokens, rows] (ldb).
+// A small output leaves most of the chip idle in one GEMM over all tokens: the tokens are then cut into slabs that
+// run as one batched GEMM into partial outputs, added in a fixed order.
+bool gemm_weight_grad(const char *what, long long m, long long rows, long long tokens, const u16 *a, long long lda, const u16 *G,
+                      long long ldb, float *C) {
+    const long long tiles = ((m + 127) / 128) * ((rows + 127) / 128);
+    int parts = 1;
+    while (parts < 16 && tiles * parts < 384 && tokens % (2 * parts) == 0 && tokens / (2 * parts) >= 1024) parts *= 2;
+    if (parts == 1 || (m * rows) % 4)
+        return gemm_bf16(what, rocblas_operation_none, rocblas_operation_transpose, m, rows, tokens, a, lda, G, ldb, 0.f, C, m);
+    const ErrorScope es;
+    float *part = scratch(30, (size_t)parts * m * rows * sizeof(float));
+    rocblas_handle h = blas();
+    if (es.failed() || !h) return false;
+    const float one = 1.0f, zero = 0.0f;
+    const long long kp = tokens / parts;
+    {
+        KernelTimer kt(what);
+        const rocblas_status st = rocblas_gemm_strided_batched_ex(
+            h, rocblas_operation_none, rocblas_operation_transpose, (rocblas_int)m, (rocblas_int)rows, (rocblas_int)kp, &one, a,
+            rocblas_datatype_bf16_r, (rocblas_int)lda, kp * lda, G, rocblas_datatype_bf16_r, (rocblas_int)ldb, kp * ldb, &zero, part,
+            rocblas_datatype_f32_r, (rocblas_int)m, m * rows, part, rocblas_datatype_f32_r, (rocblas_int)m, m * rows, parts,
+            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+        if (st != rocblas_status_success) {
+            fail("level step: rocblas_gemm_strided_batched_ex (%s) failed with status %d.", what, (int)st);
+            return false;
+        }
+    }
+    KernelTimer kt("sum_parts_kernel");
+    hipLaunchKernelGGL(sum_parts_kernel, dim3(stream_blocks(m * rows / 4, 1024)), dim3(kSThr), 0, stream(), part, C, m * rows / 4, parts);
+    check_launch("sum_parts_kernel");
+    return true;
+}
+
 void to_bf16(const float *x, u16 *out, long long count) {
     KernelTimer kt("f32_to_bf16_vec_kernel");
     hipLaunchKernelGGL(f32_to_bf16_vec_kernel, dim3(stream_blocks(count / 4, 4096)), dim3(kSThr), 0, stream(), x, out, count / 4);
@@ -556,25 +654,28 @@ void level_project_forward_bf16_rocm(const float *x, const float *w_extra, int n
         fail("level_project_forward_bf16_rocm: buffers must be 16-byte aligned.");
         return;
     }
-    u16 *wfrag = reinterpret_cast<u16 *>(scratch(24, (size_t)P * d * d * sizeof(u16)));
+    u16 *wfrag = reinterpret_cast<u16 *>(scratch(24, ((size_t)P * d * d + (size_t)levels * d * 16) * sizeof(u16)));
+    if (es.failed()) return;
+    u16 *ufrag = wfrag + (size_t)P * d * d;
+    float *fold_part = scratch(29, (size_t)(levels ? levels : 1) * kFoldSlices * 6 * d * sizeof(float));
     if (es.failed()) return;
     ProjArgs a{};
-    a.x = x; a.x_bf16 = x_bf16; a.wfrag = wfrag;
+    FoldArgs fa{};
+    a.x = x; a.x_bf16 = x_bf16; a.wfrag = wfrag; a.ufrag = ufrag;
     for (int e = 0; e < n_extra; e++) {
         if (!al16(extra_out[e])) { fail("level_project_forward_bf16_rocm: output %d is not 16-byte aligned.", e); return; }
         a.extra_out[e] = extra_out[e];
     }
     for (int l = 0; l < levels; l++) {
         const float *const *g = gate_params + 6 * l;
-        a.lv[l] = GateParams{g[0], g[1], g[2], g[3], g[4], g[5]};
-        if (!al16(g[0]) || !al16(g[2]) || !al16(g[4])) {
-            fail("level_project_forward_bf16_rocm: gate weight vectors of level %d must be 16-byte aligned.", l);
-            return;
+        for (int q = 0; q < 3; q++) {
+            fa.w[l][q] = g[2 * q];
+            a.bias[l][q] = g[2 * q + 1];
         }
     }
     a.kh = k_heads; a.vh = v_heads; a.qh = q_heads; a.ah = alpha_heads; a.th = theta_heads; a.eh = eta_heads;
     a.k_norms = k_norms; a.q_norms = q_norms; a.alpha = alpha; a.theta = theta; a.eta = eta;
-    a.n = n; a.bs = bs; a.s = seq_len; a.nh = heads; a.hd = head_dim; a.n_extra = n_extra; a.levels = levels; a.eps = eps;
+    a.n = n; a.bs = bs; a.s = seq_len; a.nh = heads; a.n_extra = n_extra; a.levels = levels; a.eps = eps;
     {
         KernelTimer kt("wfrag_pack_kernel");
         if (n_extra)
@@ -585,13 +686,20 @@ void level_project_forward_bf16_rocm(const float *x, const float *w_extra, int n
                                w_levels, wfrag + (size_t)n_extra * d * d, 3 * levels, d);
         check_launch("wfrag_pack_kernel");
     }
-    const size_t lds = (size_t)PT * (d + 8) * 2 + (8 * PT * 4 + PT * 4 + PT) * sizeof(float);
+    if (levels) {
+        KernelTimer kt("gate_fold_kernel");
+        hipLaunchKernelGGL(gate_fold_partial_kernel, dim3(ceil_div(d, 64), levels, kFoldSlices), dim3(64), 0, stream(), w_levels,
+                           fa, fold_part, d);
+        hipLaunchKernelGGL(gate_fold_finish_kernel, dim3(ceil_div(d, 64), levels), dim3(64), 0, stream(), fold_part, ufrag, d);
+        check_launch("gate_fold_kernel");
+    }
+    const size_t lds = (size_t)PT * (d + 8) * 2 + (2 * 8 * PT + 2 * PT * 8 + PT + PT) * sizeof(float);
     static bool attr_set = false;
     if (!attr_set) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(level_project_kernel<512>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 520 * 2 + 18944)), "dynamic LDS size");
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 520 * 2 + 17408)), "dynamic LDS size");
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(level_project_kernel<256>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 264 * 2 + 18944)), "dynamic LDS size");
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 264 * 2 + 17408)), "dynamic LDS size");
         attr_set = true;
     }
     if (es.failed()) return;
@@ -697,13 +805,13 @@ void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_ext
     if (es.failed()) return;
     // d_x [n, d] = G [n, R] Wb [R, d];  d_W [R, d] = G^T x  (row-major buffers as column-major operands)
     if (!gemm_bf16("gemm d_x", rocblas_operation_none, rocblas_operation_none, d, n, R, wb, d, G, R, 0.f, d_x, d)) return;
-    if (n_extra &&
-        !gemm_bf16("gemm d_w", rocblas_operation_none, rocblas_operation_transpose, d, (long long)n_extra * d, n, x_bf16, d, G, R,
-                   0.f, d_w_extra, d))
+    // the weight gradients: one product when the two outputs are one buffer (a layer's packed gradients)
+    if (n_extra && levels && d_w_levels == d_w_extra + (size_t)n_extra * d * d) {
+        gemm_weight_grad("gemm d_w", d, R, n, x_bf16, d, G, R, d_w_extra);
         return;
-    if (levels)
-        gemm_bf16("gemm d_w", rocblas_operation_none, rocblas_operation_transpose, d, 3LL * levels * d, n, x_bf16, d,
-                  G + (size_t)n_extra * d, R, 0.f, d_w_levels, d);
+    }
+    if (n_extra && !gemm_weight_grad("gemm d_w", d, (long long)n_extra * d, n, x_bf16, d, G, R, d_w_extra)) return;
+    if (levels) gemm_weight_grad("gemm d_w", d, 3LL * levels * d, n, x_bf16, d, G + (size_t)n_extra * d, R, d_w_levels);
 }
 
 void cms_combine_gate_bf16x1_rocm(const float *const *y_levels, int k, const uint16_t *attn_out, float *gate,
@@ -756,9 +864,7 @@ void linear_backward_bf16_rocm(const float *d_out_f32, const uint16_t *a_bf16, c
     if (d_a && !gemm_bf16("gemm linear d_a", rocblas_operation_none, rocblas_operation_none, d_in, n, d_out, wb, d_in, gb, d_out,
                           0.f, d_a, d_in))
         return;
-    if (d_w)
-        gemm_bf16("gemm linear d_w", rocblas_operation_none, rocblas_operation_transpose, d_in, d_out, n, a_bf16, d_in, gb, d_out,
-                  0.f, d_w, d_in);
+    if (d_w) gemm_weight_grad("gemm linear d_w", d_in, d_out, n, a_bf16, d_in, gb, d_out, d_w);
 }
 
 }  // extern "C"
