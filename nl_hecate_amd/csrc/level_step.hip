@@ -180,6 +180,36 @@ __device__ __forceinline__ void project_block(const u16 *Xs, const u16 *wf, f32x
     }
 }
 
+// The wave's 16 x 64 tile of one token tile leaves through a small LDS buffer so that a store instruction writes
+// whole rows: a lane holds four consecutive columns of ONE token in each of its four column tiles (8-byte pieces,
+// 32 bytes apart per store instruction as they sit); parked as [8 tokens][64 columns] and read back with lane l
+// taking the 16-byte piece l % 8 of token l / 8, one instruction stores eight complete 128-byte rows.  A compute
+// unit's store path moved the 8-byte pieces at about half the rate.  tb: the wave's own [8][72] bf16; row_ptr(R):
+// where the wave's 64 columns of token R (0 .. 15 of this tile) go, or null past the end.
+__device__ __forceinline__ void lanes_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+template <class RowPtr>
+__device__ __forceinline__ void store_tile_rows(const f32x4 (&t)[4], float scale, u16 *tb, RowPtr row_ptr) {
+    const int lane = threadIdx.x & 63, l16 = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        if ((l16 >> 3) == h) {
+#pragma unroll
+            for (int ct = 0; ct < 4; ct++) bf16_store(tb, (l16 & 7) * 72 + 16 * ct + 4 * g, t[ct] * scale);
+        }
+        // lanes exchange data here: to the compiler a lane that skipped the writes above has nothing to wait for and
+        // its read may run before the other lanes' writes (it did); the wave barrier keeps the order for all lanes
+        lanes_sync();
+        const bf16x8 r = *reinterpret_cast<const bf16x8 *>(tb + (lane >> 3) * 72 + (lane & 7) * 8);
+        lanes_sync();
+        u16 *dst = row_ptr(8 * h + (lane >> 3));
+        if (dst) *reinterpret_cast<bf16x8 *>(dst + (lane & 7) * 8) = r;
+    }
+}
+
 __device__ __forceinline__ float gate_act(int q, float pre) { return q == 1 ? softplus_(pre) : sigmoid_(pre); }
 
 template <int D>
@@ -191,6 +221,7 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
     float *gdot = red + 2 * 8 * PT;                                             // [2][PT][8]: x . u_q (6 used)
     float *tot = gdot + 2 * PT * 8;                                             // [PT]: 1 / max(|k|, eps)
     int *rowoff = reinterpret_cast<int *>(tot + PT);                            // [PT]: b * nh * s + t of the token
+    u16 *tb = reinterpret_cast<u16 *>(rowoff + PT) + (threadIdx.x >> 6) * 8 * 72;  // per wave: [8][72], see store_tile_rows
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, g = lane >> 4;
     const long long tok0 = (long long)blockIdx.x * PT, n = a.n;
     const bool wave_on = wave < CB;
@@ -229,12 +260,11 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
             project_block<D>(Xs, a.wfrag + (size_t)e * D * D + wave_frag, acc);
             u16 *out = a.extra_out[e];
 #pragma unroll
-            for (int tt = 0; tt < PT / 16; tt++) {
-                const long long tok = tok0 + 16 * tt + l16;
-                if (tok >= n) continue;
-#pragma unroll
-                for (int ct = 0; ct < 4; ct++) bf16_store(out + tok * D + colw + 16 * ct, 0, acc[tt][ct]);
-            }
+            for (int tt = 0; tt < PT / 16; tt++)
+                store_tile_rows(acc[tt], 1.0f, tb, [&](int r) -> u16 * {
+                    const long long tok = tok0 + 16 * tt + r;
+                    return tok < n ? out + tok * D + 64 * wave : nullptr;
+                });
         }
 
     for (int lvl = 0; lvl < a.levels; lvl++) {
@@ -257,54 +287,71 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
             if (p == 1) {   // v leaves as it is
                 if (wave_on) {
 #pragma unroll
-                    for (int tt = 0; tt < PT / 16; tt++) {
-                        if (tok0 + 16 * tt + l16 >= n) continue;
-                        u16 *row = a.vh + (chain0 * a.s + rowoff[16 * tt + l16] + (size_t)wave * a.s) * 64 + 4 * g;
-#pragma unroll
-                        for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct]);
-                    }
+                    for (int tt = 0; tt < PT / 16; tt++)
+                        store_tile_rows(acc[tt], 1.0f, tb, [&](int r) -> u16 * {
+                            return tok0 + 16 * tt + r < n ? a.vh + (chain0 * a.s + rowoff[16 * tt + r] + (size_t)wave * a.s) * 64 : nullptr;
+                        });
                 }
                 continue;
             }
-            // k, q: the row norm over all D columns = over the eight waves
+            // k, q: the row norm over all D columns = over the eight waves.  Across the four 16-lane rows of a wave
+            // the eight token tiles' sums are reduce-scattered (6 exchanges): row r ends up with the totals of tiles
+            // 2 (r & 1) + (r >> 1) and 4 + 2 (r & 1) + (r >> 1), which it parks as red[token][wave]; behind the barrier
+            // every lane reads the eight waves' sums of its own eight tokens as two 16-byte pieces each.
             float *rd = red + (p >> 1) * 8 * PT;
             if (wave_on) {
+                float ss[PT / 16];
 #pragma unroll
                 for (int tt = 0; tt < PT / 16; tt++) {
-                    float ss = 0.f;
+                    ss[tt] = 0.f;
 #pragma unroll
                     for (int ct = 0; ct < 4; ct++) {
                         const f32x4 v = acc[tt][ct];
-                        ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+                        ss[tt] += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
                     }
-                    ss = sum_rows(ss);
-                    if (g == 0) rd[wave * PT + 16 * tt + l16] = ss;
                 }
+                swap32x4(ss[0], ss[1], ss[2], ss[3], ss[4], ss[5], ss[6], ss[7]);
+                float h0 = ss[0] + ss[1], h1 = ss[2] + ss[3], h2 = ss[4] + ss[5], h3 = ss[6] + ss[7];
+                swap16x2(h0, h1, h2, h3);
+                const int t0 = 2 * (g & 1) + (g >> 1);
+                rd[(16 * t0 + l16) * 8 + wave] = h0 + h1;
+                rd[(16 * (4 + t0) + l16) * 8 + wave] = h2 + h3;
             }
             __syncthreads();
             float inv[PT / 16];
+            {
+                float4 pa[PT / 16], pb[PT / 16];
 #pragma unroll
-            for (int tt = 0; tt < PT / 16; tt++) {
-                // lane group g adds the partial sums of waves 2g and 2g + 1, the four groups are then summed
-                float ss = (2 * g < CB ? rd[2 * g * PT + 16 * tt + l16] : 0.f) + (2 * g + 1 < CB ? rd[(2 * g + 1) * PT + 16 * tt + l16] : 0.f);
-                ss = sum_rows(ss);
-                const float nrm = sqrtf(ss);
-                inv[tt] = 1.0f / fmaxf(nrm, a.eps);
-                if (wave == 0 && g == 0) {
-                    const long long tok = tok0 + 16 * tt + l16;
-                    if (p == 0) tot[16 * tt + l16] = inv[tt];
-                    if (tok < n) (p == 0 ? a.k_norms : a.q_norms)[lvl * n + tok] = nrm;
+                for (int tt = 0; tt < PT / 16; tt++) {
+                    pa[tt] = *reinterpret_cast<const float4 *>(rd + (16 * tt + l16) * 8);
+                    pb[tt] = *reinterpret_cast<const float4 *>(rd + (16 * tt + l16) * 8 + 4);
+                }
+#pragma unroll
+                for (int tt = 0; tt < PT / 16; tt++) {
+                    float ssum = pa[tt].x;   // waves that own no columns (D < 512) never wrote their slot
+                    if (CB > 1) ssum += pa[tt].y;
+                    if (CB > 2) ssum += pa[tt].z;
+                    if (CB > 3) ssum += pa[tt].w;
+                    if (CB > 4) ssum += pb[tt].x;
+                    if (CB > 5) ssum += pb[tt].y;
+                    if (CB > 6) ssum += pb[tt].z;
+                    if (CB > 7) ssum += pb[tt].w;
+                    const float nrm = sqrtf(ssum);
+                    inv[tt] = 1.0f / fmaxf(nrm, a.eps);
+                    if (wave == 0 && g == 0) {
+                        const long long tok = tok0 + 16 * tt + l16;
+                        if (p == 0) tot[16 * tt + l16] = inv[tt];
+                        if (tok < n) (p == 0 ? a.k_norms : a.q_norms)[lvl * n + tok] = nrm;
+                    }
                 }
             }
             if (wave_on) {
                 u16 *dst = p == 0 ? a.kh : a.qh;
 #pragma unroll
-                for (int tt = 0; tt < PT / 16; tt++) {
-                    if (tok0 + 16 * tt + l16 >= n) continue;
-                    u16 *row = dst + (chain0 * a.s + rowoff[16 * tt + l16] + (size_t)wave * a.s) * 64 + 4 * g;
-#pragma unroll
-                    for (int ct = 0; ct < 4; ct++) bf16_store(row + 16 * ct, 0, acc[tt][ct] * inv[tt]);
-                }
+                for (int tt = 0; tt < PT / 16; tt++)
+                    store_tile_rows(acc[tt], inv[tt], tb, [&](int r) -> u16 * {
+                        return tok0 + 16 * tt + r < n ? dst + (chain0 * a.s + rowoff[16 * tt + r] + (size_t)wave * a.s) * 64 : nullptr;
+                    });
             }
             if (p == 2 && tid < 3 * PT) {
                 // the gates: one (token, gate) per thread; the q phase's barrier lies between wave 0's write of the
@@ -693,13 +740,13 @@ void level_project_forward_bf16_rocm(const float *x, const float *w_extra, int n
         hipLaunchKernelGGL(gate_fold_finish_kernel, dim3(ceil_div(d, 64), levels), dim3(64), 0, stream(), fold_part, ufrag, d);
         check_launch("gate_fold_kernel");
     }
-    const size_t lds = (size_t)PT * (d + 8) * 2 + (2 * 8 * PT + 2 * PT * 8 + PT + PT) * sizeof(float);
+    const size_t lds = (size_t)PT * (d + 8) * 2 + (2 * 8 * PT + 2 * PT * 8 + PT + PT) * sizeof(float) + 8 * 8 * 72 * 2;
     static bool attr_set = false;
     if (!attr_set) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(level_project_kernel<512>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 520 * 2 + 17408)), "dynamic LDS size");
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 520 * 2 + 17408 + 9216)), "dynamic LDS size");
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(level_project_kernel<256>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 264 * 2 + 17408)), "dynamic LDS size");
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)PT * 264 * 2 + 17408 + 9216)), "dynamic LDS size");
         attr_set = true;
     }
     if (es.failed()) return;
