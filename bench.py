@@ -224,27 +224,38 @@ def setup_titans_exact_c2(torch, D, lib):
         cpu=lambda: cpu_baseline(x, heads))
 
 
-def setup_titans_chunkwise_c3(torch, D, lib):
+def setup_titans_chunkwise_c3(torch, D, lib, mode="bf16"):
+    """mode: "bf16" (the bf16 pair), "bf16_mnorm" (the same through the entry points that take the reference's
+    error_clip / m_norm_max, with m_norm_max = 100 as cli/configs/gear1_d1024_gpu1.json ships it), "f32_mnorm"
+    (float tokens through the reference-named symbols titans_chunkwise_*_f32_cuda with m_norm_max = 100)."""
     bs, heads, d, s, C = 16, 8, 64, 4096, 64
     B = bs * heads
     x = make_inputs(B, s, d, 0x5EED0003)
     for n in ("k", "v", "q"):
         x[n] = x[n].to(torch.bfloat16)
+        if mode == "f32_mnorm":
+            x[n] = x[n].to(torch.float32)
     dv = {n: t.cuda() for n, t in x.items()}
+    mnorm = 100.0
     nc = s // C
     z = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device="cuda")
     mc, sc, y = z(B, nc + 1, d, d), z(B, nc + 1, d, d), z(B, s, d)
     g = dict(dk=z(B, s, d), dv=z(B, s, d), dq=z(B, s, d), da=z(B, s), dt=z(B, s), de=z(B, s),
              dm=z(d, d), ds=z(d, d))
 
+    tail = () if mode == "bf16" else (0.0, mnorm)
+    f_name, b_name = {"bf16": ("titans_chunkwise_forward_bf16_rocm", "titans_chunkwise_backward_bf16_rocm"),
+                      "bf16_mnorm": ("titans_chunkwise_forward_bf16_guarded_rocm", "titans_chunkwise_backward_bf16_guarded_rocm"),
+                      "f32_mnorm": ("titans_chunkwise_forward_f32_cuda", "titans_chunkwise_backward_f32_cuda")}[mode]
+
     def fwd():
-        D.call("titans_chunkwise_forward_bf16_rocm", dv["k"], dv["v"], dv["q"], dv["alpha"], dv["theta"],
-               dv["eta"], dv["m0"], dv["s0"], mc, sc, y, s, d, B, C)
+        D.call(f_name, dv["k"], dv["v"], dv["q"], dv["alpha"], dv["theta"],
+               dv["eta"], dv["m0"], dv["s0"], mc, sc, y, s, d, B, C, *tail)
 
     def bwd():
-        D.call("titans_chunkwise_backward_bf16_rocm", dv["k"], dv["v"], dv["q"], dv["alpha"], dv["theta"],
+        D.call(b_name, dv["k"], dv["v"], dv["q"], dv["alpha"], dv["theta"],
                dv["eta"], mc, sc, dv["dy"], g["dk"], g["dv"], g["dq"], g["da"], g["dt"], g["de"],
-               g["dm"], g["ds"], s, d, B, C)
+               g["dm"], g["ds"], s, d, B, C, *tail)
 
     def chain(b):
         from oracle import pyoracle as orc
@@ -252,8 +263,14 @@ def setup_titans_chunkwise_c3(torch, D, lib):
         y, mco, sco = orc.chunkwise_forward(*a, x["m0"][b].numpy(), x["s0"][b].numpy(), C, True)
         orc.chunkwise_backward(*a, mco, sco, x["dy"][b].numpy(), C, True)
 
+    what = {"bf16": "bf16 k/v/q with fp32 accumulate and fp32 M/S, fwd+bwd",
+            "bf16_mnorm": "bf16 k/v/q with fp32 accumulate and fp32 M/S, fwd+bwd, through the entry points that take the "
+                          "reference's couplings, m_norm_max = 100 (never reached: the matrix form serves the call behind a "
+                          "device-side test, one stream synchronisation per direction)",
+            "f32_mnorm": "float k/v/q through the reference-named symbols titans_chunkwise_{forward,backward}_f32_cuda with "
+                         "m_norm_max = 100 (never reached: the fp32 matrix form serves the call behind a device-side test)"}[mode]
     return dict(
-        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16",
+        fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s, bound="hbm", dtype="bf16" if mode != "f32_mnorm" else "f32",
         flop_fwd=FLOP_CW_FWD, flop_bwd=FLOP_CW_BWD, bytes_fwd=BYTES_CW_FWD, bytes_bwd=BYTES_CW_BWD,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
         # each kernel's OWN compulsory bytes per head-token (what it must read and write given its role in
@@ -268,7 +285,7 @@ def setup_titans_chunkwise_c3(torch, D, lib):
         kernel_names={"forward": "chunkwise_forward_bf16", "backward": "chunkwise_backward_bf16"},
         cpu_all=lambda: cpu_all_cores(chain, B, s, heads, "chunkwise forward + backward"),
         config={"workload": "BASELINE configs[2]: Titans LMM chunkwise training, chunk 64, 8 heads x 64 (d=512), "
-                            "batch 16, seq 4096, bf16 k/v/q with fp32 accumulate and fp32 M/S, fwd+bwd",
+                            "batch 16, seq 4096, " + what,
                 "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "chunk_size": C},
         cpu=lambda: cpu_baseline_chunkwise(x, C))
 
@@ -423,7 +440,11 @@ def setup_mag_layer_c5(torch, D, lib, precision="bf16x3"):
                             "rule, chunk 64, bf16 k/v/q) with MAG sigmoid gating over sliding-window attention "
                             "(window 512, bf16, fp32 softmax), 8 heads x 64 (d=512), batch 8, seq 4096, x ~ N(0,1/d), "
                             "Xavier weights; forward + backward (replayed from a HIP graph) + AdamW (lr 3e-4, betas "
-                            "0.9/0.95, wd 0.1); the dense projections are library GEMMs",
+                            "0.9/0.95, wd 0.1); " + (
+                                "projections: x and the weights rounded once to bf16, fp32 accumulation (own MFMA kernel with "
+                                "the norm / gate / head-split epilogue forward, library GEMMs backward), every step a call "
+                                "into the C ABI" if precision == "bf16" else
+                                "projections: hi + lo bf16 splits, three products per GEMM (fp32-grade), library GEMMs"),
                 "batch": bs, "heads": heads, "d_model": d, "seq_len": s, "levels": k, "window": window},
         cpu=lambda: cpu_baseline_mag_layer(bs, s, d, heads, k, window))
 
@@ -576,17 +597,41 @@ def setup_hebbian_c2(torch, D, lib):
 WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
              "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5,
              "swa_stats_c5": lambda torch, D, lib: setup_swa_c5(torch, D, lib, lse=True),
-             "adamw_c5": setup_adamw_c5, "mag_layer_c5": setup_mag_layer_c5, "hebbian_c2": setup_hebbian_c2,
-             "mag_layer_c5_bf16": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16")}
+             "adamw_c5": setup_adamw_c5, "hebbian_c2": setup_hebbian_c2,
+             "mag_layer_c5": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16"),
+             "mag_layer_c5_bf16x3": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16x3"),
+             "hbm_copy": None, "mfma_peak": None,
+             "titans_chunkwise_c3_mnorm": lambda torch, D, lib: setup_titans_chunkwise_c3(torch, D, lib, mode="bf16_mnorm"),
+             "titans_chunkwise_c3_f32_mnorm": lambda torch, D, lib: setup_titans_chunkwise_c3(torch, D, lib, mode="f32_mnorm")}
 
 
-def source_hash():
-    """sha256 over the kernel sources and the C ABI header: what a traffic profile belongs to."""
+# The kernel sources each workload's launches come from: a traffic profile is stamped with a hash of THESE files
+# (and the headers they include), so an edit elsewhere in the library does not make it look stale, and an edit
+# here does until the profile is measured again.
+_CW_BF16 = ["chunkwise_chain.hip", "chunkwise_adjoint.hip", "chunkwise_grads.hip", "chunkwise_gates.hip", "chunkwise_mm.hip"]
+_SWA = ["swa_mfma.hip", "swa.hip"]
+WORKLOAD_SOURCES = {
+    "titans_chunkwise_c3": _CW_BF16,
+    "titans_chunkwise_c3_mnorm": _CW_BF16 + ["chunkwise_guard.hip"],
+    "titans_chunkwise_c3_f32_mnorm": ["chunkwise_mm.hip", "chunkwise_gates.hip", "chunkwise_guard.hip", "memory_rules.hip"],
+    "titans_exact_c2": ["memory_rules.hip", "memory_rules_fused.hip"],
+    "hope_selfref_c4": ["selfref.hip"],
+    "swa_c5": _SWA, "swa_stats_c5": _SWA,
+    "adamw_c5": ["optim.hip", "cms.hip"],
+    "hebbian_c2": ["hebbian.hip"],
+    "mag_layer_c5": _CW_BF16 + _SWA + ["level_step.hip", "layer_glue.hip", "cms.hip", "optim.hip"],
+    "mag_layer_c5_bf16x3": _CW_BF16 + _SWA + ["layer_glue.hip", "cms.hip", "optim.hip", "elementwise.hip"],
+    "hbm_copy": ["roof_probes.hip"], "mfma_peak": ["roof_probes.hip"],
+}
+
+
+def source_hash(workload):
+    """sha256 over the kernel sources of a workload, every header of the library and the C ABI header."""
     import glob
     import hashlib
     h = hashlib.sha256()
-    files = sorted(glob.glob(os.path.join(ROOT, "nl_hecate_amd", "csrc", "*.hip")) +
-                   glob.glob(os.path.join(ROOT, "nl_hecate_amd", "csrc", "*.h")) +
+    csrc = os.path.join(ROOT, "nl_hecate_amd", "csrc")
+    files = sorted([os.path.join(csrc, f) for f in WORKLOAD_SOURCES[workload]] + glob.glob(os.path.join(csrc, "*.h")) +
                    [os.path.join(ROOT, "include", "nl_hecate_ffi.h")])
     for f in files:
         h.update(os.path.basename(f).encode())
@@ -695,7 +740,8 @@ def write_profile(workload, raw):
     out_txt = os.path.join(ROOT, "profiles", workload + "_kernels_and_hbm_traffic.txt")
     with open(out_txt, "w") as f:
         f.write("\n".join(lines) + "\n")
-    side = {"workload": workload, "git_head": git_head(), "source_sha256": source_hash(),
+    side = {"workload": workload, "git_head": git_head(), "source_sha256": source_hash(workload),
+            "sources": WORKLOAD_SOURCES[workload],
             "calibration": {"fetch_factor": ff, "write_factor": fw,
                             "note": "counter KiB per dispatch x factor = KiB moved; factors from a map kernel of known size"},
             "kernels": kernels}
@@ -703,6 +749,47 @@ def write_profile(workload, raw):
         json.dump(side, f, indent=1, sort_keys=True)
         f.write("\n")
     print(open(out_txt).read())
+
+
+def run_probe(which, torch, lib, steps, warmup):
+    """What the box sustains, from kernels of the simplest shape (csrc/roof_probes.hip): streaming copies at 1 : 1 and
+    3 : 2 read : write, and the matrix cores' issue peak for the two instructions the library uses."""
+    res = {"metric": "sustained rate of the probe kernels", "n_gpus": 1, "steps": steps, "warmup": warmup,
+           "data": "synthetic", "higher_is_better": True, "config": {"workload": which}, "probes": []}
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        lib.nlh_timer_start()
+        for _ in range(steps):
+            fn()
+        return lib.nlh_timer_stop_ms() / steps
+
+    if which == "hbm_copy":
+        n = 64 << 20   # floats per stream: 256 MiB, far beyond the 256 MB Infinity Cache once several streams are in play
+        for reads, writes in ((1, 1), (3, 2)):
+            a = torch.randn(reads * n, dtype=torch.float32, device="cuda")
+            b = torch.empty(writes * n, dtype=torch.float32, device="cuda")
+            ms = timed(lambda: lib.nlh_probe_stream_rocm(a.data_ptr(), b.data_ptr(), n, reads, writes))
+            gbs = 4 * n * (reads + writes) / (ms * 1e-3) / 1e9
+            res["probes"].append({"name": f"stream {reads} read : {writes} write", "bytes": 4 * n * (reads + writes), "ms": ms,
+                                  "achieved": gbs, "unit": "GB/s", "peak": PEAK_HBM_GBS, "frac": gbs / PEAK_HBM_GBS})
+            del a, b
+        res.update(value=res["probes"][0]["achieved"], unit="GB/s", dtype="f32")
+    else:
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        out = torch.empty(cus * 8 * 256, dtype=torch.float32, device="cuda")
+        for kind, name, flop, per_iter, peak in ((0, "v_mfma_f32_16x16x32_bf16", 16384, 8, PEAK_BF16_TFLOPS),
+                                                 (2, "v_mfma_f32_32x32x16_bf16", 32768, 4, PEAK_BF16_TFLOPS),
+                                                 (1, "v_mfma_f32_16x16x4_f32", 2048, 8, PEAK_FP32_TFLOPS)):
+            for wps in (1, 2, 4):
+                iters = 20000
+                ms = timed(lambda: lib.nlh_probe_mfma_rocm(kind, iters, wps, out.data_ptr()))
+                tf = flop * per_iter * iters * cus * 4 * wps / (ms * 1e-3) / 1e12
+                res["probes"].append({"name": name, "waves_per_simd": wps, "ms": ms, "achieved": tf, "unit": "TFLOP/s",
+                                      "peak": peak, "frac": tf / peak})
+        res.update(value=max(p["achieved"] for p in res["probes"]), unit="TFLOP/s", dtype="bf16")
+    return res
 
 
 def main():
@@ -743,6 +830,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration_kernel": "map_kernel (sigmoid_cuda)", "launches": 5,
                           "read_bytes_per_launch": 4 * n, "written_bytes_per_launch": 4 * n}))
+        return
+
+    if args.workload in ("hbm_copy", "mfma_peak"):
+        print(json.dumps(run_probe(args.workload, torch, lib, args.steps, args.warmup)))
         return
 
     w = WORKLOADS[args.workload](torch, D, lib)
@@ -799,7 +890,7 @@ def main():
         return work_per_ht * head_tokens / (max(ms, 1e-9) * 1e-3) / scale
 
     side = profile_sidecar(args.workload)
-    stale = None if side is None else side.get("source_sha256") != source_hash()
+    stale = None if side is None else side.get("source_sha256") != source_hash(args.workload)
     side_k = {} if side is None else side["kernels"]
 
     def kernel_traffic(nm):   # bytes per launch from the sidecar: the profile's kernel whose name starts with nm

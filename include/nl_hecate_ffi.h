@@ -547,6 +547,24 @@ void titans_chunkwise_backward_bf16_rocm(const uint16_t *k_mem, const uint16_t *
                                          float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                                          float *d_s_initial, int seq_len, int d, int batch_size,
                                          int chunk_size);
+/* The bf16 pair above under the reference's production arguments (core/kernels/titans_chunkwise_forward.cu:89-176
+ * with error_clip / m_norm_max as the json files under cli/configs ship them): the matrix form runs first and is kept when a
+ * device-side test on its chunk-start states shows that neither the clip nor the projection can fire anywhere in
+ * the call (then they are the identity and the results are the reference's); otherwise the sequential kernels,
+ * which apply both per token, redo the call on the widened tokens.  One 4-byte copy to the host and a
+ * synchronisation of the launch stream per call; while that stream is being captured the sequential kernels run.
+ * The reference-named fp32 symbols {titans,delta}_chunkwise_{forward,backward}_f32_cuda do the same. */
+void titans_chunkwise_forward_bf16_guarded_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                                const float *alpha, const float *theta, const float *eta,
+                                                const float *m_initial, const float *s_initial, float *m_chunk_states,
+                                                float *s_chunk_states, float *y, int seq_len, int d, int batch_size,
+                                                int chunk_size, float error_clip, float m_norm_max);
+void titans_chunkwise_backward_bf16_guarded_rocm(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                                 const float *alpha, const float *theta, const float *eta,
+                                                 const float *m_chunk_states, const float *s_chunk_states, const float *d_y,
+                                                 float *d_k_mem, float *d_v_mem, float *d_q_mem, float *d_alpha, float *d_theta,
+                                                 float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d,
+                                                 int batch_size, int chunk_size, float error_clip, float m_norm_max);
 /* The same pair for a layer that keeps its tensors token-major (no counterpart in the reference, whose
  * gpu_memory_forward / gpu_memory_backward transpose between the layouts, core/src/gpu_forward.rs:1197 ff.):
  * chain c = (level, batch element, head), batch_size = levels * bs * heads; y_tokens [levels, bs, seq_len, heads*d]
@@ -926,6 +944,14 @@ void cms_combine_gate_bf16x1_rocm(const float *const *y_levels, int k, const uin
 void linear_forward_bf16_rocm(const uint16_t *a_bf16, const float *w, float *out, int n, int d_in, int d_out);
 void linear_backward_bf16_rocm(const float *d_out_f32, const uint16_t *a_bf16, const float *w, float *d_a, float *d_w, int n,
                                int d_in, int d_out);
+
+/* ── What the box sustains (no counterpart in the reference) ─────────────────────────────────────────
+ * Probe kernels behind `bench.py --workload hbm_copy / mfma_peak`: a streaming kernel that reads `reads` and
+ * writes `writes` streams of n floats (16-byte accesses; in [reads, n], out [writes, n]), and the matrix cores'
+ * issue peak for kind 0 = v_mfma_f32_16x16x32_bf16, 1 = v_mfma_f32_16x16x4_f32, 2 = v_mfma_f32_32x32x16_bf16 (out: compute units *
+ * waves_per_simd * 256 floats; returns matrix instructions per wave, or < 0). */
+int nlh_probe_stream_rocm(const float *in, float *out, long long n, int reads, int writes);
+int nlh_probe_mfma_rocm(int kind, int iters, int waves_per_simd, float *out);
 
 /* ── Opaque VJP blocks of the Wengert tape ───────────────────────────────────────────────────────
  * core/src/tape.rs:141-150 OpaqueBackwardFn(d_outputs, saved, d_inputs) for the OpaqueKey values

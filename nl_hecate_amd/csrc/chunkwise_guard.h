@@ -1,0 +1,21 @@
+// Device-side test of whether the error clip or the Frobenius projection of the reference's chunkwise kernels
+// can fire for a call, given the chunk-start states (chunkwise_guard.hip).  Costs one chunk-parallel kernel, a
+// 4-byte copy to the host and a synchronisation of the launch stream (the reference's chunkwise wrappers
+// synchronise the device themselves); not available while the launch stream is being captured.
+#pragma once
+#include <stdint.h>
+
+namespace nlh {
+
+bool guard_possible();   // false while the launch stream is being captured into a graph, or while force_sequential is set
+extern bool force_sequential;   // set around a call that has already run the test and lost
+// true: a coupling may fire somewhere (or the test could not run): use the sequential kernels.  s_states null:
+// the Delta rule (no momentum).  m_states / s_states [batch, num_chunks + 1, 64 * 64]; head size 64, chunk <= 64.
+bool couplings_may_fire(const float *k, const float *v, const float *alpha, const float *theta, const float *eta,
+                        const float *m_states, const float *s_states, int seq_len, int batch, int chunk_size,
+                        float error_clip, float m_norm_max);
+bool couplings_may_fire_bf16(const uint16_t *k, const uint16_t *v, const float *alpha, const float *theta, const float *eta,
+                             const float *m_states, const float *s_states, int seq_len, int batch, int chunk_size,
+                             float error_clip, float m_norm_max);
+
+}  // namespace nlh

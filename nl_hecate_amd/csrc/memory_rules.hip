@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "../../include/nl_hecate_ffi.h"
+#include "chunkwise_guard.h"
 #include "rule_args.h"
 #include "rule_common.h"
 
@@ -559,6 +560,11 @@ bool coupled_needed(float error_clip, float m_norm_max) {
 // (both break the linearity it rests on).  Everything else takes the sequential kernels.
 bool matrix_form_applies(int d, int chunk_size, float error_clip, float m_norm_max) {
     return d == 64 && chunk_size >= 1 && chunk_size <= 64 && !coupled_needed(error_clip, m_norm_max);
+}
+// With a clip or a projection in the arguments (every shipped configuration of the reference has one) the matrix
+// form still applies whenever neither can fire, which a device-side test decides (chunkwise_guard.h).
+bool guarded_matrix_form(int d, int chunk_size, float error_clip, float m_norm_max) {
+    return d == 64 && chunk_size >= 1 && chunk_size <= 64 && coupled_needed(error_clip, m_norm_max) && guard_possible();
 }
 
 // rows of a chain that one workgroup owns, for a given D and RPL
@@ -1120,6 +1126,15 @@ void titans_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, c
                                              m_chunk_states, s_chunk_states, y, seq_len, d, batch_size, chunk_size);
         return;
     }
+    if (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max)) {
+        // the matrix form first: its chunk-start states are what the test needs; kept when no coupling can fire
+        const ErrorScope es;
+        titans_chunkwise_forward_mm_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial,
+                                             m_chunk_states, s_chunk_states, y, seq_len, d, batch_size, chunk_size);
+        if (!es.failed() && !couplings_may_fire(k_mem, v_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, seq_len,
+                                                batch_size, chunk_size, error_clip, m_norm_max))
+            return;
+    }
     FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial,
               m_chunk_states, s_chunk_states, y, seq_len, seq_len, chunk_size, 1, (long long)d * d,
               (long long)n_ckpt_count(seq_len, chunk_size) * d * d, error_clip, m_norm_max};
@@ -1140,6 +1155,14 @@ void delta_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, co
                                             seq_len, d, batch_size, chunk_size);
         return;
     }
+    if (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max)) {
+        const ErrorScope es;
+        delta_chunkwise_forward_mm_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, m_initial, m_chunk_states, y,
+                                            seq_len, d, batch_size, chunk_size);
+        if (!es.failed() && !couplings_may_fire(k_mem, v_mem, alpha, theta, nullptr, m_chunk_states, nullptr, seq_len,
+                                                batch_size, chunk_size, error_clip, m_norm_max))
+            return;
+    }
     FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial, nullptr,
               m_chunk_states, nullptr, y, seq_len, seq_len, chunk_size, 1, (long long)d * d,
               (long long)n_ckpt_count(seq_len, chunk_size) * d * d, error_clip, m_norm_max};
@@ -1156,7 +1179,11 @@ void titans_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, 
                                         float *d_m_initial, float *d_s_initial,
                                         int seq_len, int d, int batch_size, int chunk_size,
                                         float error_clip, float m_norm_max) {
-    if (seq_len > 0 && batch_size > 0 && matrix_form_applies(d, chunk_size, error_clip, m_norm_max)) {
+    if (seq_len > 0 && batch_size > 0 &&
+        (matrix_form_applies(d, chunk_size, error_clip, m_norm_max) ||
+         (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max) &&
+          !couplings_may_fire(k_mem, v_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, seq_len, batch_size, chunk_size,
+                              error_clip, m_norm_max)))) {
         titans_chunkwise_backward_mm_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_chunk_states, s_chunk_states,
                                               d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, d_m_initial,
                                               d_s_initial, seq_len, d, batch_size, chunk_size);
@@ -1175,7 +1202,11 @@ void delta_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, c
                                        float *d_alpha, float *d_theta, float *d_m_initial,
                                        int seq_len, int d, int batch_size, int chunk_size,
                                        float error_clip, float m_norm_max) {
-    if (seq_len > 0 && batch_size > 0 && matrix_form_applies(d, chunk_size, error_clip, m_norm_max)) {
+    if (seq_len > 0 && batch_size > 0 &&
+        (matrix_form_applies(d, chunk_size, error_clip, m_norm_max) ||
+         (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max) &&
+          !couplings_may_fire(k_mem, v_mem, alpha, theta, nullptr, m_chunk_states, nullptr, seq_len, batch_size, chunk_size,
+                              error_clip, m_norm_max)))) {
         delta_chunkwise_backward_mm_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, m_chunk_states, d_y, d_k_mem, d_v_mem,
                                              d_q_mem, d_alpha, d_theta, d_m_initial, seq_len, d, batch_size,
                                              chunk_size);
