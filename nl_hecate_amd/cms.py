@@ -175,14 +175,27 @@ class ContextState:
             lib.nlh_context_state_reset(_ptr_array(bufs), n, len(bufs))
 
     def seed_self_ref(self, level_inits):
-        """:194-207: level_inits[l] = dict with m_k_init, m_v_init, m_q_init, m_eta_init, m_alpha_init
-        ([d, d] tensors, or absent for static projections) and m_mem_init (or absent)."""
+        """:193-206: level_inits[l] = dict with m_k_init, m_v_init, m_q_init, m_eta_init, m_alpha_init
+        ([d, d] tensors, or absent for static projections) and m_mem_init (or absent).  Per level, as there: the five
+        projection memories are seeded when m_k_init is given (a level without a self-referential block is skipped,
+        later levels are still visited); m_mem_init, when its size matches, is copied into memory[l] whether or not
+        the projections are static (every chain of the level starts from it), and into slot 5 of the level's
+        self-referential block, which is the copy the HOPE kernels read."""
         for lv, init in enumerate(level_inits):
-            if lv >= len(self.self_ref) or self.self_ref[lv] is None:
+            if lv >= len(self.self_ref):
                 break
             mems = self.self_ref[lv]
-            chains, six, d, _ = mems.shape
-            assert six == 6
             get = lambda n: init[n].data_ptr() if init.get(n) is not None else None
-            lib.nlh_context_state_seed_self_ref(mems.data_ptr(), get("m_k_init"), get("m_v_init"), get("m_q_init"),
-                                                get("m_eta_init"), get("m_alpha_init"), get("m_mem_init"), chains, d)
+            mm = init.get("m_mem_init")
+            if mems is not None and init.get("m_k_init") is not None:
+                chains, six, d, _ = mems.shape
+                assert six == 6
+                lib.nlh_context_state_seed_self_ref(mems.data_ptr(), get("m_k_init"), get("m_v_init"), get("m_q_init"),
+                                                    get("m_eta_init"), get("m_alpha_init"), get("m_mem_init"), chains, d)
+            elif mems is not None and mm is not None:
+                chains, six, d, _ = mems.shape
+                lib.nlh_context_state_seed_self_ref(mems.data_ptr(), None, None, None, None, None, mm.data_ptr(), chains, d)
+            if mm is not None and lv < len(self.memory) and self.memory[lv] is not None:
+                mem = self.memory[lv]
+                if mem.numel() % mm.numel() == 0 and mem.numel() >= mm.numel():
+                    mem.view(-1, mm.numel()).copy_(mm.reshape(1, -1).expand(mem.numel() // mm.numel(), -1))

@@ -24,7 +24,7 @@ from . import dispatch as D
 from .cms import ContextState, Pulse
 from .ffi import lib
 from .memory_level import LevelConfig, LevelGrads, gpu_memory_backward, gpu_memory_forward
-from .serving import GpuMAGParams, _memory_read_only
+from .serving import GpuMAGParams, frozen_level_output
 from .tnt import ParallelConfig, gpu_tnt_backward, gpu_tnt_forward
 
 LN_EPS = 1e-5
@@ -139,9 +139,8 @@ def gpu_cms_forward(params: GpuMAGParams, cfg: ModelConfig, input_ids, target_id
             else:
                 y, mc = gpu_memory_forward(params.levels[level], lcfg, mem_input, context.memory[level], s, d, bs)
         else:
-            if lcfg.memory_rule in ("moneta", "yaad") or lcfg.is_mlp_mem:
-                raise ValueError(f"a frozen {lcfg.memory_rule} level with an MLP memory has no read-only path")
-            y, mc = _memory_read_only(params.levels[level], mem_input, context.memory[level], n, nh, hd), None
+            # the matrix read; zeros for MONETA / YAAD, an error for the two-layer Titans memory (gpu_forward.rs:1008-1024)
+            y, mc = frozen_level_output(lcfg, params.levels[level], mem_input, context.memory[level], n, nh, hd, level), None
         ys.append(y)
         caches.append(mc)
     c["memory_caches"], c["y_per_level"] = caches, ys

@@ -68,20 +68,21 @@ struct ProjArgs {
 };
 
 // Packs P matrices W_p [D, D] (row = output column, contraction index contiguous) into the order in which
-// the projection kernel's waves read them: [p][column block of 64][k step of 32][tile of 16 columns][lane][8],
-// lane l holding column 16 * tile + l % 16, contraction indices 32 * step + 8 * (l / 16) .. + 8: one 16-byte
-// load per lane and tile, 4 KB contiguous per wave and step.
+// the projection kernel's waves read them, as A operands of v_mfma_f32_32x32x16_bf16:
+// [p][column block of 64][k step of 16][tile of 32 columns][lane][8], lane l holding column 32 * tile + l % 32,
+// contraction indices 16 * step + 8 * (l / 32) .. + 8: one 16-byte load per lane and tile, 2 KB contiguous per
+// wave and step.
 __global__ void wfrag_pack_kernel(const float *__restrict__ W, u16 *__restrict__ out, int P, int D) {
     const long long total = (long long)P * D * D / 8;
-    const int KS = D / 32, CB = D / 64;
+    const int KS = D / 16, CB = D / 64;
     for (long long o = (long long)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (long long)gridDim.x * blockDim.x) {
-        const int lane = (int)(o & 63), ct = (int)((o >> 6) & 3);
-        long long r = o >> 8;
+        const int lane = (int)(o & 63), c32 = (int)((o >> 6) & 1);
+        long long r = o >> 7;
         const int ks = (int)(r % KS);
         r /= KS;
         const int cb = (int)(r % CB);
         const long long p = r / CB;
-        const int row = 64 * cb + 16 * ct + (lane & 15), k0 = 32 * ks + 8 * (lane >> 4);
+        const int row = 64 * cb + 32 * c32 + (lane & 31), k0 = 16 * ks + 8 * (lane >> 5);
         const float *src = W + (p * D + row) * D + k0;
         const float4 a = *reinterpret_cast<const float4 *>(src), b = *reinterpret_cast<const float4 *>(src + 4);
         const bf16x8 v = {(__bf16)a.x, (__bf16)a.y, (__bf16)a.z, (__bf16)a.w, (__bf16)b.x, (__bf16)b.y, (__bf16)b.z, (__bf16)b.w};
@@ -136,69 +137,82 @@ __global__ __launch_bounds__(64) void gate_fold_finish_kernel(const float *__res
     for (int r = 12; r < 16; r++) out[r * 8] = (__bf16)0.f;
 }
 
-// acc[tt][ct][r] = sum_k W[col][k] x[token][k] with col = 16 ct + 4 (lane / 16) + r of the wave's 64 columns and
-// token = 16 tt + lane % 16 of the workgroup's 128: the weights as the A operand straight from global memory
-// (a ring of four steps, requested three steps ahead), x as the B operand from LDS (two token tiles per unit of
-// eight products, the next unit's pair requested before this unit's products are issued).  Fully unrolled, with
-// the order of requests and products pinned: left to itself the scheduler sinks every load to its first use and
-// the wave then waits a full memory latency per step.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int T32 = PT / 32;   // token tiles of 32 per workgroup
+
+// acc[t32][c32][i] = sum_k W[col][k] x[token][k] with token = 32 t32 + lane % 32 of the workgroup's 128 and
+// col = 32 c32 + 8 (i / 4) + 4 (lane / 32) + i % 4 of the wave's 64 columns, on v_mfma_f32_32x32x16_bf16 (measured
+// on this part: 98 % of the data-sheet rate, where the 16 x 16 x 32 shape issues at 54 %).  The weights are the A
+// operand straight from global memory (a ring of four 32-wide steps, requested three steps ahead), x the B operand
+// from LDS (two token tiles per unit of four products, the next unit's pair requested before this unit's products
+// are issued).  Fully unrolled, with the order of requests and products pinned: left to itself the scheduler sinks
+// every load to its first use and the wave then waits a full memory latency per step.
 template <int D>
-__device__ __forceinline__ void project_block(const u16 *Xs, const u16 *wf, f32x4 (&acc)[PT / 16][4]) {
-    constexpr int XS = D + 8, KS = D / 32, RING = 4, UNITS = KS * (PT / 32);
+__device__ __forceinline__ void project_block(const u16 *Xs, const u16 *wf, f32x16 (&acc)[T32][2]) {
+    constexpr int XS = D + 8, KS = D / 32, RING = 4, UPK = 2 * (T32 / 2), UNITS = KS * UPK;   // units per 32-wide step
     const int lane = threadIdx.x & 63;
-    const bf16x8 *wp = reinterpret_cast<const bf16x8 *>(wf) + lane;
-    const u16 *xb = Xs + (lane & 15) * XS + 8 * (lane >> 4);
+    const bf16x8 *wp = reinterpret_cast<const bf16x8 *>(wf) + lane;   // step ks: [2 k halves][2 column tiles][64 lanes]
+    const u16 *xb = Xs + (lane & 31) * XS + 8 * (lane >> 5);
 #pragma unroll
-    for (int tt = 0; tt < PT / 16; tt++)
+    for (int t = 0; t < T32; t++)
 #pragma unroll
-        for (int ct = 0; ct < 4; ct++) acc[tt][ct] = zero4();
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[t][c][i] = 0.f;
     bf16x8 w[RING][4], b[2][2];
 #pragma unroll
     for (int p = 0; p < RING - 1 && p < KS; p++)
 #pragma unroll
-        for (int ct = 0; ct < 4; ct++) w[p][ct] = wp[(p * 4 + ct) * 64];
+        for (int f = 0; f < 4; f++) w[p][f] = wp[(p * 4 + f) * 64];
     b[0][0] = *reinterpret_cast<const bf16x8 *>(xb);
-    b[0][1] = *reinterpret_cast<const bf16x8 *>(xb + 16 * XS);
+    b[0][1] = *reinterpret_cast<const bf16x8 *>(xb + 32 * XS);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < UNITS; u++) {
-        const int ks = u / (PT / 32), pr = u % (PT / 32);
-        if (pr == 0 && ks + RING - 1 < KS) {
+        // unit u: k half kh of step ks, token tiles 2 pr and 2 pr + 1
+        const int ks = u / UPK, kh = (u % UPK) / (T32 / 2), pr = u % (T32 / 2);
+        if (u % UPK == 0 && ks + RING - 1 < KS) {
 #pragma unroll
-            for (int ct = 0; ct < 4; ct++) w[(ks + RING - 1) % RING][ct] = wp[((ks + RING - 1) * 4 + ct) * 64];
+            for (int f = 0; f < 4; f++) w[(ks + RING - 1) % RING][f] = wp[((ks + RING - 1) * 4 + f) * 64];
         }
         if (u + 1 < UNITS) {
-            const int nks = (u + 1) / (PT / 32), npr = (u + 1) % (PT / 32);
-            b[(u + 1) & 1][0] = *reinterpret_cast<const bf16x8 *>(xb + 32 * npr * XS + 32 * nks);
-            b[(u + 1) & 1][1] = *reinterpret_cast<const bf16x8 *>(xb + (32 * npr + 16) * XS + 32 * nks);
+            const int nks = (u + 1) / UPK, nkh = ((u + 1) % UPK) / (T32 / 2), npr = (u + 1) % (T32 / 2);
+            b[(u + 1) & 1][0] = *reinterpret_cast<const bf16x8 *>(xb + 64 * npr * XS + 32 * nks + 16 * nkh);
+            b[(u + 1) & 1][1] = *reinterpret_cast<const bf16x8 *>(xb + (64 * npr + 32) * XS + 32 * nks + 16 * nkh);
         }
 #pragma unroll
         for (int h = 0; h < 2; h++)
 #pragma unroll
-            for (int ct = 0; ct < 4; ct++) acc[2 * pr + h][ct] = mfma32(w[ks % RING][ct], b[u & 1][h], acc[2 * pr + h][ct]);
+            for (int c = 0; c < 2; c++)
+                acc[2 * pr + h][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w[ks % RING][2 * kh + c], b[u & 1][h], acc[2 * pr + h][c], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
 
-// The wave's 16 x 64 tile of one token tile leaves through a small LDS buffer so that a store instruction writes
-// whole rows: a lane holds four consecutive columns of ONE token in each of its four column tiles (8-byte pieces,
-// 32 bytes apart per store instruction as they sit); parked as [8 tokens][64 columns] and read back with lane l
-// taking the 16-byte piece l % 8 of token l / 8, one instruction stores eight complete 128-byte rows.  A compute
-// unit's store path moved the 8-byte pieces at about half the rate.  tb: the wave's own [8][72] bf16; row_ptr(R):
-// where the wave's 64 columns of token R (0 .. 15 of this tile) go, or null past the end.
+// The wave's 32 x 64 tile of one token tile leaves through a small LDS buffer so that a store instruction writes
+// whole rows: a lane holds, of ONE token, eight 4-column pieces (8 bytes each, 16 bytes apart); parked eight tokens
+// at a time as [8 tokens][64 columns] and read back with lane l taking the 16-byte piece l % 8 of token l / 8, one
+// instruction stores eight complete 128-byte rows.  A compute unit's store path moved the 8-byte pieces at about
+// half the rate.  tb: the wave's own [8][72] bf16; row_ptr(R): where the wave's 64 columns of token R (0 .. 31 of
+// this tile) go, or null past the end.
 __device__ __forceinline__ void lanes_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 template <class RowPtr>
-__device__ __forceinline__ void store_tile_rows(const f32x4 (&t)[4], float scale, u16 *tb, RowPtr row_ptr) {
-    const int lane = threadIdx.x & 63, l16 = lane & 15, g = lane >> 4;
+__device__ __forceinline__ void store_tile_rows(const f32x16 (&t)[2], float scale, u16 *tb, RowPtr row_ptr) {
+    const int lane = threadIdx.x & 63, l32 = lane & 31, hf = lane >> 5;
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-        if ((l16 >> 3) == h) {
+    for (int h = 0; h < 4; h++) {
+        if ((l32 >> 3) == h) {
 #pragma unroll
-            for (int ct = 0; ct < 4; ct++) bf16_store(tb, (l16 & 7) * 72 + 16 * ct + 4 * g, t[ct] * scale);
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const f32x4 v = {t[c][4 * j] * scale, t[c][4 * j + 1] * scale, t[c][4 * j + 2] * scale, t[c][4 * j + 3] * scale};
+                    bf16_store(tb, (l32 & 7) * 72 + 32 * c + 8 * j + 4 * hf, v);
+                }
         }
         // lanes exchange data here: to the compiler a lane that skipped the writes above has nothing to wait for and
         // its read may run before the other lanes' writes (it did); the wave barrier keeps the order for all lanes
@@ -250,9 +264,9 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
     }
     __syncthreads();
 
-    f32x4 acc[PT / 16][4];
+    f32x16 acc[T32][2];
     const size_t wave_frag = (size_t)wave * 64 * D;
-    const int colw = 64 * wave + 4 * g;   // the lane's first column in tile 0
+    const int l32 = lane & 31, hf = lane >> 5;
 
     // plain projections: rounded once, token-major
     if (wave_on)
@@ -260,9 +274,9 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
             project_block<D>(Xs, a.wfrag + (size_t)e * D * D + wave_frag, acc);
             u16 *out = a.extra_out[e];
 #pragma unroll
-            for (int tt = 0; tt < PT / 16; tt++)
+            for (int tt = 0; tt < T32; tt++)
                 store_tile_rows(acc[tt], 1.0f, tb, [&](int r) -> u16 * {
-                    const long long tok = tok0 + 16 * tt + r;
+                    const long long tok = tok0 + 32 * tt + r;
                     return tok < n ? out + tok * D + 64 * wave : nullptr;
                 });
         }
@@ -287,47 +301,42 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
             if (p == 1) {   // v leaves as it is
                 if (wave_on) {
 #pragma unroll
-                    for (int tt = 0; tt < PT / 16; tt++)
+                    for (int tt = 0; tt < T32; tt++)
                         store_tile_rows(acc[tt], 1.0f, tb, [&](int r) -> u16 * {
-                            return tok0 + 16 * tt + r < n ? a.vh + (chain0 * a.s + rowoff[16 * tt + r] + (size_t)wave * a.s) * 64 : nullptr;
+                            return tok0 + 32 * tt + r < n ? a.vh + (chain0 * a.s + rowoff[32 * tt + r] + (size_t)wave * a.s) * 64 : nullptr;
                         });
                 }
                 continue;
             }
-            // k, q: the row norm over all D columns = over the eight waves.  Across the four 16-lane rows of a wave
-            // the eight token tiles' sums are reduce-scattered (6 exchanges): row r ends up with the totals of tiles
-            // 2 (r & 1) + (r >> 1) and 4 + 2 (r & 1) + (r >> 1), which it parks as red[token][wave]; behind the barrier
-            // every lane reads the eight waves' sums of its own eight tokens as two 16-byte pieces each.
+            // k, q: the row norm over all D columns = over the eight waves.  The two half-waves hold different columns
+            // of the same 32 tokens: one exchange per pair of token tiles leaves tile t32's totals in half t32 % 2, which
+            // parks them as red[token][wave]; behind the barrier every lane reads the eight waves' sums of its own four
+            // tokens as two 16-byte pieces each.
             float *rd = red + (p >> 1) * 8 * PT;
             if (wave_on) {
-                float ss[PT / 16];
+                float ss[T32];
 #pragma unroll
-                for (int tt = 0; tt < PT / 16; tt++) {
+                for (int tt = 0; tt < T32; tt++) {
                     ss[tt] = 0.f;
 #pragma unroll
-                    for (int ct = 0; ct < 4; ct++) {
-                        const f32x4 v = acc[tt][ct];
-                        ss[tt] += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
-                    }
+                    for (int c = 0; c < 2; c++)
+#pragma unroll
+                        for (int i = 0; i < 16; i++) ss[tt] += acc[tt][c][i] * acc[tt][c][i];
                 }
-                swap32x4(ss[0], ss[1], ss[2], ss[3], ss[4], ss[5], ss[6], ss[7]);
-                float h0 = ss[0] + ss[1], h1 = ss[2] + ss[3], h2 = ss[4] + ss[5], h3 = ss[6] + ss[7];
-                swap16x2(h0, h1, h2, h3);
-                const int t0 = 2 * (g & 1) + (g >> 1);
-                rd[(16 * t0 + l16) * 8 + wave] = h0 + h1;
-                rd[(16 * (4 + t0) + l16) * 8 + wave] = h2 + h3;
+                rd[(32 * hf + l32) * 8 + wave] = swapadd32(ss[0], ss[1]);          // lower half: tile 0, upper half: tile 1
+                rd[(32 * (2 + hf) + l32) * 8 + wave] = swapadd32(ss[2], ss[3]);
             }
             __syncthreads();
-            float inv[PT / 16];
+            float inv[T32];
             {
-                float4 pa[PT / 16], pb[PT / 16];
+                float4 pa[T32], pb[T32];
 #pragma unroll
-                for (int tt = 0; tt < PT / 16; tt++) {
-                    pa[tt] = *reinterpret_cast<const float4 *>(rd + (16 * tt + l16) * 8);
-                    pb[tt] = *reinterpret_cast<const float4 *>(rd + (16 * tt + l16) * 8 + 4);
+                for (int tt = 0; tt < T32; tt++) {
+                    pa[tt] = *reinterpret_cast<const float4 *>(rd + (32 * tt + l32) * 8);
+                    pb[tt] = *reinterpret_cast<const float4 *>(rd + (32 * tt + l32) * 8 + 4);
                 }
 #pragma unroll
-                for (int tt = 0; tt < PT / 16; tt++) {
+                for (int tt = 0; tt < T32; tt++) {
                     float ssum = pa[tt].x;   // waves that own no columns (D < 512) never wrote their slot
                     if (CB > 1) ssum += pa[tt].y;
                     if (CB > 2) ssum += pa[tt].z;
@@ -338,9 +347,9 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
                     if (CB > 7) ssum += pb[tt].w;
                     const float nrm = sqrtf(ssum);
                     inv[tt] = 1.0f / fmaxf(nrm, a.eps);
-                    if (wave == 0 && g == 0) {
-                        const long long tok = tok0 + 16 * tt + l16;
-                        if (p == 0) tot[16 * tt + l16] = inv[tt];
+                    if (wave == 0 && hf == 0) {
+                        const long long tok = tok0 + 32 * tt + l32;
+                        if (p == 0) tot[32 * tt + l32] = inv[tt];
                         if (tok < n) (p == 0 ? a.k_norms : a.q_norms)[lvl * n + tok] = nrm;
                     }
                 }
@@ -348,9 +357,9 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
             if (wave_on) {
                 u16 *dst = p == 0 ? a.kh : a.qh;
 #pragma unroll
-                for (int tt = 0; tt < PT / 16; tt++)
+                for (int tt = 0; tt < T32; tt++)
                     store_tile_rows(acc[tt], inv[tt], tb, [&](int r) -> u16 * {
-                        return tok0 + 16 * tt + r < n ? dst + (chain0 * a.s + rowoff[16 * tt + r] + (size_t)wave * a.s) * 64 : nullptr;
+                        return tok0 + 32 * tt + r < n ? dst + (chain0 * a.s + rowoff[32 * tt + r] + (size_t)wave * a.s) * 64 : nullptr;
                     });
             }
             if (p == 2 && tid < 3 * PT) {

@@ -1011,7 +1011,11 @@ void titans_backward_noalloc_f32_rocm(const float *k_mem, const float *v_mem, co
     const size_t dd = (size_t)d * d;
     const bool coupled = error_clip > 0.f;
     const size_t state_floats = 2 * (size_t)batch_size * dd;
-    const size_t need = state_floats + bwd_partial_floats(d, batch_size, seq_len, bwd_rpl(d, batch_size, coupled, true));
+    // partial sums only where launch_bwd splits a chain over workgroups: with a clip at d = 128 it takes the general
+    // kernel (one workgroup per chain), which needs none
+    const int rpl = bwd_rpl(d, batch_size, coupled, true);
+    const bool split = !(coupled && ceil_div(d, rows_per_wg(d, rpl)) != 1);
+    const size_t need = state_floats + (split ? bwd_partial_floats(d, batch_size, seq_len, rpl) : 0);
     if (need > kNoAllocFloats) {
         fail("%s: batch_size=%d, d=%d, seq_len=%d need %zu floats of work space; the fixed buffer holds %zu "
              "(use titans_backward_f32_cuda).", fn, batch_size, d, seq_len, need, kNoAllocFloats);

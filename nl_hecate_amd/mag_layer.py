@@ -732,25 +732,7 @@ class MagTrainer:
         graphs = self.__dict__.setdefault("_graphs", GraphCache(lib.nlh_workspace_generation))
         entry = graphs.get(key)
         if entry is None:
-            xs, ds = x.clone(), d_out.clone()
-            # Warm-up on a side stream sizes every scratch buffer (nothing may allocate while a graph
-            # is captured); it advances the context memories, which are put back afterwards.
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                lib.nlh_set_stream(ctypes.c_void_p(side.cuda_stream))
-                layer.ensure_state(x.shape[0])
-                saved = [(m.clone(), z.clone()) for m, z in zip(layer.m_state, layer.s_state)]
-                self._forward_backward(xs, ds)
-                for (m, z), m0, z0 in zip(saved, layer.m_state, layer.s_state):
-                    m0.copy_(m); z0.copy_(z)
-            torch.cuda.current_stream().wait_stream(side)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                lib.nlh_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-                out = self._forward_backward(xs, ds)
-            lib.nlh_set_stream(None)
-            entry = (graph, xs, ds, out)
+            entry = self._capture(x, d_out)
             graphs.put(key, entry)
         graph, xs, ds, out = entry
         xs.copy_(x)
@@ -759,6 +741,38 @@ class MagTrainer:
         self._optimizer_and_error_buffers(pulse)
         layer.conductor.advance()
         return out
+
+    def _capture(self, x, d_out):
+        """Warm-up on a side stream, then the capture.  Whatever happens in between (a recorded scratch error, an
+        allocation failure), the library's launch stream goes back to the null stream and the context memories that
+        the warm-up advanced are put back: a failed capture must not leave every later call of the process launching
+        on a dead or capturing stream."""
+        layer = self.layer
+        xs, ds = x.clone(), d_out.clone()
+        layer.ensure_state(x.shape[0])
+        saved = [(m.clone(), z.clone()) for m, z in zip(layer.m_state, layer.s_state)]
+        restored = False
+        try:
+            # the warm-up sizes every scratch buffer (nothing may allocate while a graph is captured)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                lib.nlh_set_stream(ctypes.c_void_p(side.cuda_stream))
+                self._forward_backward(xs, ds)
+                for (m, z), m0, z0 in zip(saved, layer.m_state, layer.s_state):
+                    m0.copy_(m); z0.copy_(z)
+                restored = True
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                lib.nlh_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+                out = self._forward_backward(xs, ds)
+            return (graph, xs, ds, out)
+        finally:
+            lib.nlh_set_stream(None)
+            if not restored:
+                for (m, z), m0, z0 in zip(saved, layer.m_state, layer.s_state):
+                    m0.copy_(m); z0.copy_(z)
 
     def step(self, x, d_out_fn):
         """One training step; d_out_fn(out) gives the upstream gradient.  Returns out."""

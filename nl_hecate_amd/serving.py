@@ -55,6 +55,7 @@ class ServeConfig:
     levels: List[LevelConfig]       # one per CMS level (cfg.k = len(levels))
     n_persistent: int = 0
     decode_tokens: int = 2048       # prefill sizes the cache for the prompt plus this many decode tokens
+    residual: bool = False          # the reference's cached-generation path refuses residual = true (:3175, :3392)
 
     @property
     def k(self):
@@ -140,6 +141,18 @@ def _memory_read_only(lp, embedded, memory, n, nh, hd):
     return y
 
 
+def frozen_level_output(lcfg, lp, embedded, memory, n, nh, hd, level):
+    """What a frozen level contributes (gpu_forward.rs:1008-1024, 3255-3265, 3449-3459): the read y = M_h q for a
+    matrix memory; zeros for MONETA / YAAD, whose context memory is the flat [W1 | W2] block that the matrix read
+    cannot interpret (frozen_mlp_fallback, :45-57); an error for the two-layer Titans memory
+    (panic_if_frozen_titans_mlp, :32-39)."""
+    if lcfg.is_mlp_mem:
+        raise RuntimeError(f"Frozen TitansLMM MLP level unsupported (level {level}): read-only MLP kernel not implemented")
+    if lcfg.memory_rule in ("moneta", "yaad"):
+        return _zeros(n, nh * hd)
+    return _memory_read_only(lp, embedded, memory, n, nh, hd)
+
+
 def _levels(params, cfg, embedded, pulse, context, s):
     ys = []
     for level in range(cfg.k):
@@ -147,8 +160,8 @@ def _levels(params, cfg, embedded, pulse, context, s):
             y, _cache = gpu_memory_forward(params.levels[level], cfg.levels[level], embedded, context.memory[level], s,
                                            cfg.d_model, 1)
         else:
-            y = _memory_read_only(params.levels[level], embedded, context.memory[level], s, cfg.num_heads,
-                                  cfg.head_dim)
+            y = frozen_level_output(cfg.levels[level], params.levels[level], embedded, context.memory[level], s,
+                                    cfg.num_heads, cfg.head_dim, level)
         ys.append(y)
     return ys
 
@@ -164,6 +177,7 @@ def gpu_prefill_forward(params: GpuMAGParams, cfg: ServeConfig, input_ids, pulse
     """-> (logits of the last prompt position [vocab] on the host, GpuKVCache holding the prompt)."""
     s, d, nh, hd = cfg.seq_len, cfg.d_model, cfg.num_heads, cfg.head_dim
     assert d == nh * hd
+    assert not cfg.residual, "gpu_prefill_forward: residual=true is not served by the cached-generation path"
     assert len(input_ids) >= s
     ids = torch.tensor([int(t) for t in input_ids[:s]], dtype=torch.int32).cuda()
     embedded = _new(s, d)
@@ -193,6 +207,7 @@ def gpu_single_token_forward(params: GpuMAGParams, cfg: ServeConfig, token_id, p
                              kv_cache: GpuKVCache, ws: DecodeWorkspace):
     """One decode step -> logits [vocab] on the host."""
     d, v, nh, hd = cfg.d_model, cfg.vocab_size, cfg.num_heads, cfg.head_dim
+    assert not cfg.residual, "gpu_single_token_forward: residual=true is not served by the cached-generation path"
     if not 0 <= token_id < v:
         raise ValueError(f"token_id {token_id} >= vocab_size {v}")
     if kv_cache.len == 0:

@@ -113,6 +113,10 @@ def forward(p, cfg, input_ids, target_ids, active, memories, quantize=True, gate
             else:
                 y, lc, m = ML.level_forward(p["levels"][lv], lcfg, mem_in.reshape(bs, s, d), memories[lv], gl)
                 y = y.reshape(n, d)
+        elif getattr(lcfg, "memory_layers", 1) == 2 and lcfg.memory_rule == "titans":
+            raise RuntimeError(f"Frozen TitansLMM MLP level unsupported (level {lv})")   # gpu_forward.rs:32-39
+        elif lcfg.memory_rule in ("moneta", "yaad"):   # frozen_mlp_fallback (gpu_forward.rs:45-57, 1010-1012): zeros
+            y, lc, m = np.zeros((n, d), dt), None, memories[lv]
         else:   # gpu_memory_read_only: y = M_h q_h with the projection q as it comes, batch slot 0's memories
             qr = (mem_in @ p["levels"][lv]["w_q"].T).reshape(n, nh, hd)
             y = np.einsum("hij,nhj->nhi", memories[lv][:nh], qr).reshape(n, d)

@@ -31,7 +31,14 @@ def _levels(p, cfg, emb, active, memories):
             ys.append(y[0].astype(f32))
             new.append(carried.astype(f32))
         else:
-            ys.append(_read_only(p["levels"][lv], emb, memories[lv], cfg.num_heads, cfg.head_dim))
+            # frozen (gpu_forward.rs:3255-3265): the matrix read; zeros for MONETA / YAAD (frozen_mlp_fallback, :45-57);
+            # refused for the two-layer Titans memory (panic_if_frozen_titans_mlp, :32-39)
+            if getattr(lcfg, "memory_layers", 1) == 2 and lcfg.memory_rule == "titans":
+                raise RuntimeError(f"Frozen TitansLMM MLP level unsupported (level {lv})")
+            if lcfg.memory_rule in ("moneta", "yaad"):
+                ys.append(np.zeros((emb.shape[0], cfg.num_heads * cfg.head_dim), f32))
+            else:
+                ys.append(_read_only(p["levels"][lv], emb, memories[lv], cfg.num_heads, cfg.head_dim))
             new.append(memories[lv])
     return ys, new
 

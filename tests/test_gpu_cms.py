@@ -173,10 +173,26 @@ def test_context_state_reset_and_seed_self_ref():
     cs.seed_self_ref([dict(m_mem_init=new_mem)])
     torch.cuda.synchronize()
     assert torch.equal(sr[0][:, :5], keep[:, :5]) and all(torch.equal(sr[0][b, 5], new_mem) for b in range(chains))
+    # m_mem_init also lands in the level's carried memory, every chain (conductor.rs:202-204)
+    assert all(torch.equal(mem[0][b], new_mem) for b in range(chains))
     cs.reset()
     torch.cuda.synchronize()
     assert not any(t.any() for t in mem + mom) and not sr[0].any()
     assert ptrs == [t.data_ptr() for t in mem + mom + [sr[0]]], "reset is in place"
+    # a level without a self-referential block does not stop the walk: [None, adaptive]
+    mem2 = [dev(rnd(chains, d, d)) for _ in range(2)]
+    sr2 = [None, dev(rnd(chains, 6, d, d))]
+    cs2 = ContextState(mem2, None, sr2)
+    keep0 = mem2[0].clone()
+    cs2.seed_self_ref([dict(), inits[0]])
+    torch.cuda.synchronize()
+    assert all(torch.equal(sr2[1][b, 0], inits[0]["m_k_init"]) for b in range(chains)), "level 1 is seeded past a static level 0"
+    assert torch.equal(mem2[0], keep0)
+    # a static-projection level (no block at all) that carries a learned m_mem_init gets its memory seeded
+    cs3 = ContextState([dev(rnd(chains, d, d))], None, [None])
+    cs3.seed_self_ref([dict(m_mem_init=new_mem)])
+    torch.cuda.synchronize()
+    assert all(torch.equal(cs3.memory[0][b], new_mem) for b in range(chains))
 
 
 def test_frozen_read_backward_kernel():

@@ -238,3 +238,35 @@ def test_decode_steps_reproduce_the_full_sequence_forward(frozen_second):
     for lv in range(2):
         m_err = (dec.m_state[lv] - full.m_state[lv]).abs().max().item()
         assert m_err <= 1e-4 * max(full.m_state[lv].abs().max().item(), 1e-6), (lv, m_err)
+
+
+def test_failed_capture_restores_the_launch_stream_and_the_context_memories():
+    """A warm-up that raises must not leave the library launching on the side stream, nor the context memories
+    advanced: the next (eager) step then equals the step of a trainer that never tried to capture."""
+    from nl_hecate_amd.mag_layer import MagLayer, MagTrainer
+    bs, s, d, heads, k = 1, 64, 128, 2, 2
+    mk = lambda: MagLayer(d, heads, k, 32, [1, 2], rule="chunkwise", chunk=32, seed=13)
+    broken, plain = MagTrainer(mk()), MagTrainer(mk())
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(bs, s, d, generator=g) / d ** 0.5).cuda()
+    d_out = torch.randn(bs, s, d, generator=g).cuda()
+    real = broken._forward_backward
+
+    def fails_after_the_forward(xs, ds):
+        real(xs, ds)            # advances the context memories, as a warm-up does
+        raise RuntimeError("scratch error during the warm-up")
+    broken._forward_backward = fails_after_the_forward
+    broken.layer.ensure_state(bs)
+    before = [m.clone() for m in broken.layer.m_state]
+    with pytest.raises(RuntimeError, match="warm-up"):
+        broken.step_graphed(x, d_out)
+    torch.cuda.synchronize()
+    for a, b in zip(broken.layer.m_state, before):
+        assert torch.equal(a, b), "the warm-up's memory updates were put back"
+    broken._forward_backward = real
+    out_b = broken.step(x, lambda o: d_out).clone()
+    out_p = plain.step(x, lambda o: d_out).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(out_b, out_p)
+    for a, b in zip(broken.layer.p.tensors(), plain.layer.p.tensors()):
+        assert torch.equal(a, b)

@@ -122,3 +122,39 @@ def test_decode_needs_a_prefilled_cache():
     with pytest.raises(RuntimeError):
         SG.gpu_single_token_forward(gpu_params(p), cfg, 1, Pulse(0, [True]), ContextState([dev(np.zeros((2, 64), f32))]),
                                     SG.GpuKVCache(8, d, 1), SG.DecodeWorkspace(d, v))
+
+
+def test_frozen_mlp_memory_levels_follow_the_reference():
+    """gpu_forward.rs:32-57, 3255-3265: a frozen MONETA / YAAD level contributes zeros (its context memory is the flat
+    [W1 | W2] block, which the matrix read must not interpret); a frozen two-layer Titans memory is refused."""
+    nh, hd, window, s, extra, v, k = 2, 8, 6, 9, 3, 19, 2
+    d = nh * hd
+    p = model(d, v, k, 77)
+    r = np.random.default_rng(9)
+    ids = r.integers(0, v, s + extra)
+    active = [True, False]
+    for frozen_rule in ("moneta", "yaad"):
+        lcfgs = [LevelConfig("delta", nh, hd), LevelConfig(frozen_rule, nh, hd, d_hidden=12)]
+        ocfg = types.SimpleNamespace(d_model=d, num_heads=nh, head_dim=hd, window_size=window, n_persistent=0, levels=lcfgs)
+        cfg = SG.ServeConfig(d, v, nh, hd, window, s, lcfgs, decode_tokens=extra)
+        mem0 = [(0.2 * r.standard_normal((nh, hd, hd))).astype(f32), r.standard_normal(2 * 12 * d).astype(f32)]
+        ctx = ContextState([dev(mem0[0].reshape(nh, hd * hd)), dev(mem0[1])])
+        gp = gpu_params(p)
+        logits, kv = SG.gpu_prefill_forward(gp, cfg, ids, Pulse(0, active), ctx)
+        want, mem, kc, vc = SV.forward_all(p, ocfg, ids[:s], active, mem0)
+        scale = np.abs(want).max()
+        assert np.abs(logits - want[s - 1]).max() <= 2e-2 * scale
+        ws = SG.DecodeWorkspace(d, v)
+        for i in range(extra):
+            step = SG.gpu_single_token_forward(gp, cfg, int(ids[s + i]), Pulse(0, active), ctx, kv, ws)
+            ref, mem, kc, vc = SV.single_token(p, ocfg, int(ids[s + i]), active, mem, kc, vc)
+            assert np.abs(step - ref).max() <= 2e-2 * scale, i
+        assert np.array_equal(host(ctx.memory[1]), mem0[1]), "a frozen level's memory is not touched"
+    lcfgs = [LevelConfig("delta", nh, hd), LevelConfig("titans", nh, hd, memory_layers=2)]
+    cfg = SG.ServeConfig(d, v, nh, hd, window, s, lcfgs, decode_tokens=extra)
+    ctx = ContextState([dev(np.zeros((nh, hd * hd), f32)), dev(np.zeros(8, f32))])
+    with pytest.raises(RuntimeError, match="Frozen TitansLMM MLP"):
+        SG.gpu_prefill_forward(gpu_params(p), cfg, ids, Pulse(0, active), ctx)
+    with pytest.raises(AssertionError, match="residual"):
+        SG.gpu_prefill_forward(gpu_params(p), SG.ServeConfig(d, v, nh, hd, window, s, lcfgs[:1], residual=True), ids,
+                               Pulse(0, [True]), ctx)

@@ -40,3 +40,24 @@ def test_decode_steps_equal_the_whole_sequence(k, active, n_persistent):
         assert np.allclose(step, want[s + i], rtol=2e-2, atol=2e-3 * np.abs(want).max()), i
     for a, b in zip(mem, mem_all):
         assert np.allclose(a, b, rtol=1e-4, atol=1e-6)
+
+
+def test_frozen_mlp_memory_levels_contribute_zeros_or_are_refused():
+    """gpu_forward.rs:32-57: a frozen MONETA / YAAD level adds nothing (the model answers as if the level were not
+    there, up to the 1 / sqrt(k) scaling that only k > 2 applies); a frozen two-layer Titans memory is an error."""
+    nh, hd, v, s, window = 2, 4, 11, 7, 4
+    d = nh * hd
+    p = model(d, v, 2, 51)
+    r = np.random.default_rng(3)
+    ids = r.integers(0, v, s)
+    mem0 = [(0.2 * r.standard_normal((nh, hd, hd))).astype(f32), r.standard_normal(64).astype(f32)]
+    mk = lambda levels: types.SimpleNamespace(d_model=d, num_heads=nh, head_dim=hd, window_size=window, n_persistent=0,
+                                               levels=levels)
+    moneta = types.SimpleNamespace(memory_rule="moneta", memory_layers=1)
+    with_frozen, _, _, _ = SV.forward_all(p, mk([cfg_of("delta", nh, hd), moneta]), ids, [True, False], mem0)
+    p1 = dict(p, levels=p["levels"][:1])
+    alone, _, _, _ = SV.forward_all(p1, mk([cfg_of("delta", nh, hd)]), ids, [True], mem0[:1])
+    assert np.array_equal(with_frozen, alone)
+    mlp = types.SimpleNamespace(memory_rule="titans", memory_layers=2)
+    with pytest.raises(RuntimeError):
+        SV.forward_all(p, mk([cfg_of("delta", nh, hd), mlp]), ids, [True, False], mem0)

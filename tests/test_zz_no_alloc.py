@@ -56,6 +56,38 @@ def test_noalloc_backward_matches_the_allocating_entry_point_on_two_calls_in_a_r
 
 
 @pytest.mark.gpu
+def test_noalloc_backward_allocates_nothing():
+    """The property the entry point exists for: with the library's scratch arena released, a call neither grows the
+    arena (its generation stays) nor takes device memory (the free byte count stays), for a chain kept in one
+    workgroup, for a chain split over four (partial sums in the fixed array) and for the clipped d = 128 case that the
+    general kernel serves."""
+    from nl_hecate_amd.ffi import lib
+    cases = [(6, 50, 64, 0.0), (2, 24, 128, 0.0), (2, 12, 128, 1.0)]
+    bufs = []
+    for B, s, d, clip in cases:
+        x = rule_inputs(B, s, d, 950 + d, m0_scale=0.3)
+        _, ms, ss = orc.titans_forward_batch(x["k"], x["v"], x["q"], x["alpha"], x["theta"], x["eta"], x["m0"], x["s0"],
+                                             error_clip=clip)
+        g = [zeros(B, s, d), zeros(B, s, d), zeros(B, s, d), zeros(B, s), zeros(B, s), zeros(B, s), zeros(d, d), zeros(d, d)]
+        bufs.append(([dev(x[n]) for n in ("k", "v", "q", "alpha", "theta", "eta")] + [dev(ms), dev(ss), dev(x["dy"])] + g,
+                     (s, d, B, clip)))
+    # once beforehand: the array's address is looked up once per device, and the runtime loads a kernel's code (and
+    # sizes its own launch resources) on first use, which is not this library's doing
+    for args, dims in bufs:
+        D.call("titans_backward_noalloc_f32_rocm", *args, *dims)
+    torch.cuda.synchronize()
+    lib.nlh_release_workspace()
+    gen, free = lib.nlh_workspace_generation(), torch.cuda.mem_get_info()[0]
+    for args, dims in bufs:
+        D.call("titans_backward_noalloc_f32_rocm", *args, *dims)
+    torch.cuda.synchronize()
+    assert lib.nlh_workspace_generation() == gen, "the scratch arena grew"
+    assert torch.cuda.mem_get_info()[0] == free, "device memory was taken"
+    # the clipped d = 128 case is within the size limit where the unclipped one of the same shape counts partial sums
+    assert torch.isfinite(bufs[2][0][9]).all()
+
+
+@pytest.mark.gpu
 def test_noalloc_backward_accumulates_into_the_initial_state_gradients():
     """d_m_initial / d_s_initial are += targets, as in titans_backward_f32_cuda."""
     x = rule_inputs(3, 20, 16, 906, m0_scale=0.3)
