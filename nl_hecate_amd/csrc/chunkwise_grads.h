@@ -30,12 +30,28 @@ bool chunkwise_adjoint_bf16(const uint16_t *k, const uint16_t *q, const float *d
                             float *ds_first, int seq_len, int batch, int chunk_size, bool has_s,
                             const HeadRows *dy_rows = nullptr);
 
+// d_k, d_v, d_q as bf16 in token-major slabs instead of fp32 head-major tensors: chain c = (level, batch element,
+// head) writes its 64 columns of token t at slab + rows.offset(c) + t * rows.row_stride
+struct GradOut16 {
+    uint16_t *gk, *gv, *gq;
+    HeadRows rows;
+};
+
 bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *d_y,
                           const float *m_states, const float *s_states, const uint16_t *dm_snap,
                           const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid,
-                          const HeadRows *dy_rows = nullptr);
+                          const HeadRows *dy_rows = nullptr, const GradOut16 *out16 = nullptr);
+
+// titans_chunkwise_backward_bf16_tokens_rocm with d_k, d_v, d_q leaving as bf16 token-major slabs (the level step's
+// GEMM operand): same arguments otherwise
+void titans_chunkwise_backward_bf16_tokens_g16(const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem,
+                                               const float *alpha, const float *theta, const float *eta,
+                                               const float *m_chunk_states, const float *s_chunk_states,
+                                               const float *d_y_tokens, const GradOut16 &out, float *d_alpha, float *d_theta,
+                                               float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d,
+                                               int batch_size, int chunk_size, int heads, int levels, int d_y_per_level);
 
 // also runs the first stage of the batch sum of the initial-state gradients: tmp [nsum][ceil(batch / per)][64*64]
 // receives the sums of `per` consecutive chains of dm_first (and ds_first when nsum = 2), [batch][chain_stride]

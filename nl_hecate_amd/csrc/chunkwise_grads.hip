@@ -114,14 +114,14 @@ __device__ __forceinline__ f32x4 bf4_to_f32(const uint2 b) {
 }
 __device__ __forceinline__ f32x4 bf4_to_f32(const u16 *p) { return bf4_to_f32(*reinterpret_cast<const uint2 *>(p)); }
 
-template <bool HAS_S>
+template <bool HAS_S, bool G16>
 __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q, const float *__restrict__ d_y,
     const float *__restrict__ tab_b, const float *__restrict__ vecs,
     const float *__restrict__ m_states, const float *__restrict__ s_states, const u16 *__restrict__ dm_snap,
     const u16 *__restrict__ ds_snap, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
-    int C, int nc, int ntask, HeadRows dyr) {
+    int C, int nc, int ntask, HeadRows dyr, GradOut16 go) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     // Every input is staged once, in the order it arrives (rows = tokens or state rows); a product that contracts
     // over the row index reads its operand through ld_op_tr.
@@ -198,6 +198,13 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     for (int task = task_lo; task < task_hi; task++) {
         const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
         const size_t tok = (size_t)chain * s + t0;
+        // where four consecutive columns `col` of token t0 + tl of a gradient go: the fp32 head-major tensor, or (G16) a
+        // bf16 token-major slab in which chain = (level, batch element, head) addresses its own columns
+        const size_t g_off = G16 ? go.rows.offset(chain) + (size_t)t0 * go.rows.row_stride : 0;
+        auto put = [&](float *f32base, u16 *g16base, int tl, int col, f32x4 val) {
+            if constexpr (G16) bf16_store(g16base + g_off + (size_t)tl * go.rows.row_stride + col, 0, val);
+            else *reinterpret_cast<f32x4 *>(f32base + (tok + tl) * HD + col) = val;
+        };
         // ── load and stage everything ──
         {
             if (st_t >= L) { nK = make_uint4(0, 0, 0, 0); nQ = nK; nV = nK; }
@@ -433,7 +440,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
                     bf16_store(dEr, j * LDB + bm + 16 * rt + 4 * g, -dk[rt][ct]);
-                    if (j < L) *reinterpret_cast<f32x4 *>(d_v + (tok + j) * HD + bm + 16 * rt + 4 * g) = dk[rt][ct];
+                    if (j < L) put(d_v, go.gv, j, bm + 16 * rt + 4 * g, dk[rt][ct]);
                 }
             }
         } else {
@@ -456,7 +463,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 if (t < L) {
 #pragma unroll
                     for (int rt = 0; rt < 2; rt++)
-                        *reinterpret_cast<f32x4 *>(d_q + (tok + t) * HD + bm + 16 * rt + 4 * g) = keep[rt][ct];
+                        put(d_q, go.gq, t, bm + 16 * rt + 4 * g, keep[rt][ct]);
                 }
             }
             auto state_term = [&](const u16 *Ar, int which, int voff) {   // dte += cvec[voff + j] . (Ar^T E^T); g sums
@@ -535,8 +542,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 if (j < L) {
 #pragma unroll
                     for (int rt = 0; rt < 2; rt++)
-                        *reinterpret_cast<f32x4 *>(d_k + (tok + j) * HD + bm + 16 * rt + 4 * g) =
-                            em[rt][ct] - thj * dte[rt][ct];
+                        put(d_k, go.gk, j, bm + 16 * rt + 4 * g, em[rt][ct] - thj * dte[rt][ct]);
                 }
             }
         } else if (tid < L) {
@@ -578,28 +584,30 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           const float *m_states, const float *s_states, const uint16_t *dm_snap,
                           const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_b, const float *vecs,
-                          int seq_len, int batch, int chunk_size, bool has_s, int grid, const HeadRows *dy_rows) {
+                          int seq_len, int batch, int chunk_size, bool has_s, int grid, const HeadRows *dy_rows,
+                          const GradOut16 *out16) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     const HeadRows dyr = dy_rows ? *dy_rows : head_major_rows(seq_len, HD);
     static bool attr_set = false;
     if (!attr_set) {
-        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_grads_bf16_kernel<true>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
-        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_grads_bf16_kernel<false>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
+        const void *fns[4] = {reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, false>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, false>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, true>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, true>)};
+        for (const void *f : fns) check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
         attr_set = true;
     }
     if (es.failed()) return true;
+    const GradOut16 go = out16 ? *out16 : GradOut16{};
     KernelTimer kt("cw_grads_bf16_kernel");
-    if (has_s)
-        hipLaunchKernelGGL(cw_grads_bf16_kernel<true>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
-                           tab_b, vecs, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec,
-                           xs, scal, seq_len, chunk_size, nc, ntask, dyr);
-    else
-        hipLaunchKernelGGL(cw_grads_bf16_kernel<false>, dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y,
-                           tab_b, vecs, m_states, nullptr, dm_snap, nullptr, d_k, d_v, d_q, d_theta, pvec,
-                           xs, scal, seq_len, chunk_size, nc, ntask, dyr);
+#define NLH_CWG(HS, G) \
+    hipLaunchKernelGGL((cw_grads_bf16_kernel<HS, G>), dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y, tab_b, vecs, \
+                       m_states, HS ? s_states : nullptr, dm_snap, HS ? ds_snap : nullptr, d_k, d_v, d_q, d_theta, pvec, xs, scal, \
+                       seq_len, chunk_size, nc, ntask, dyr, go)
+    if (has_s) { if (out16) NLH_CWG(true, true); else NLH_CWG(true, false); }
+    else { if (out16) NLH_CWG(false, true); else NLH_CWG(false, false); }
+#undef NLH_CWG
     check_launch("cw_grads_bf16_kernel");
     return true;
 }

@@ -843,9 +843,10 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                  const float *eta, const float *m_states, const float *s_states, const float *d_y, float *d_k,
                  float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                  float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s,
-                 const HeadRows *dy_rows = nullptr) {
+                 const HeadRows *dy_rows = nullptr, const GradOut16 *out16 = nullptr) {
     const ErrorScope es;
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
+    if (out16 && sizeof(TIn) != 2) { fail("%s: bf16 gradient slabs are served for bf16 tokens only.", fn); return; }
     if (dy_rows && sizeof(TIn) != 2) { fail("%s: token-major d_y is served for bf16 tokens only.", fn); return; }
     const int nc = ceil_div(seq_len, chunk_size);
     Scratch sc{nullptr, nullptr};
@@ -880,7 +881,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                                reinterpret_cast<float *>(ds_snap + n_snap), seq_len, batch, chunk_size, has_s, dy_rows);
         chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec, xs,
                              scal, tab_b, vecs, seq_len, batch, chunk_size, has_s,
-                             persistent_grid(batch * nc), dy_rows);
+                             persistent_grid(batch * nc), dy_rows, out16);
     } else {
         hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
                            stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc,
@@ -1001,6 +1002,20 @@ extern "C" void titans_chunkwise_backward_bf16_tokens_rocm(
     backward_mm<uint16_t>(fn, k_mem, v_mem, q_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, d_y_tokens,
                           d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d,
                           batch_size, chunk_size, true, &dyr);
+}
+
+void nlh::titans_chunkwise_backward_bf16_tokens_g16(
+    const uint16_t *k_mem, const uint16_t *v_mem, const uint16_t *q_mem, const float *alpha, const float *theta,
+    const float *eta, const float *m_chunk_states, const float *s_chunk_states, const float *d_y_tokens,
+    const GradOut16 &out, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len,
+    int d, int batch_size, int chunk_size, int heads, int levels, int d_y_per_level) {
+    const char *fn = "titans_chunkwise_backward_bf16_tokens_g16";
+    if (seq_len <= 0 || batch_size <= 0) return;
+    if (!token_rows_ok(fn, d, batch_size, chunk_size, heads, levels)) return;
+    const HeadRows dyr = token_major_rows(seq_len, HD, heads, batch_size / levels, d_y_per_level != 0);
+    backward_mm<uint16_t>(fn, k_mem, v_mem, q_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, d_y_tokens,
+                          nullptr, nullptr, nullptr, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d,
+                          batch_size, chunk_size, true, &dyr, &out);
 }
 
 extern "C" void titans_chunkwise_backward_mm_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,

@@ -22,6 +22,7 @@
 
 #include "../../include/nl_hecate_ffi.h"
 #include "bf16_tiles.h"
+#include "chunkwise_grads.h"
 #include "lane_ops.h"
 #include "runtime.h"
 
@@ -384,98 +385,95 @@ __global__ __launch_bounds__(kPThr) void level_project_kernel(ProjArgs a) {
 struct GateGradOut { float *w_alpha, *b_alpha, *w_theta, *b_theta, *w_eta, *b_eta; };
 
 struct GradArgs {
-    const float *dkh, *dvh, *dqh, *dah, *dth, *deh;          // [levels * bs * nh, s, hd] and [levels * bs * nh, s]
+    const float *dah, *dth, *deh;                            // the rule's gate gradients, [levels * bs * nh, s]
     const u16 *kh, *vh, *qh;                                 // the forward's head-major operands (k, q normalised)
     const float *k_norms, *q_norms, *alpha, *theta, *eta;    // [levels, n]
     u16 *G;                                                  // [n, g_ld]: level lvl's d_k, d_v, d_q at col0 + 3 lvl d + {0, d, 2d}
     long long g_ld, col0;
     float *part;                                             // [levels][gridDim.x][3][2d + 1]
-    int bs, s, nh, hd, levels;
+    int bs, s, nh, levels;
     float eps;
 };
 
-// One wave per token and level: head sums of the gate gradients and their activations' derivatives, head merge of
-// d_k, d_v, d_q, backward of the two row normalisations (from the normalised bf16 rows the forward wrote and the
-// stored norms); the token-major gradients leave as bf16 columns of G.  The gate projections' weight and bias
-// gradients are summed per wave in registers and leave as one partial row per workgroup.
-template <int NIT>
+// What is left between the rule's backward and the GEMMs once the rule writes d_k, d_v, d_q as bf16 columns of G
+// itself (token-major, every head in its own 64 columns): one wave per token and level reads the token's d_k and d_q
+// rows, takes them through the backward of the two row normalisations in place (from the normalised bf16 rows the
+// forward wrote and the stored norms; d_v needs nothing), sums the gate gradients over the heads, applies the gate
+// activations' derivatives, and accumulates the gate projections' weight and bias gradients per wave in registers
+// (one partial row per workgroup, summed afterwards in a fixed order).  A lane owns 8 consecutive columns.
 __global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
     extern __shared__ float redg[];   // [3][2d + 1]
-    const int lane = threadIdx.x & 63, wave_l = threadIdx.x >> 6, d = a.nh * a.hd, d4 = d / 4, lvl = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave_l = threadIdx.x >> 6, d = a.nh * 64, lvl = blockIdx.y, c0 = 8 * lane;
+    const bool on = c0 < d;
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
     const long long n = (long long)a.bs * a.s;
     const size_t chain0 = (size_t)lvl * a.bs * a.nh;
     const float inv_eps = 1.0f / a.eps;
-    float4 acc[3][2][NIT];
+    float acc[3][2][8];
     float accb[3] = {0.f, 0.f, 0.f};
 #pragma unroll
     for (int gi = 0; gi < 3; gi++)
 #pragma unroll
         for (int h = 0; h < 2; h++)
 #pragma unroll
-            for (int it = 0; it < NIT; it++) acc[gi][h][it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int e = 0; e < 8; e++) acc[gi][h][e] = 0.f;
+    auto widen = [](const bf16x8 &v, float (&f)[8]) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) f[e] = (float)v[e];
+    };
     for (long long tok = wave; tok < n; tok += nwaves) {
         const long long b = tok / a.s, t = tok - b * a.s;
-        float da = 0.f, dt = 0.f, de = 0.f;
+        float dg[3] = {0.f, 0.f, 0.f};
         for (int h = lane; h < a.nh; h += 64) {
             const size_t o = (chain0 + b * a.nh + h) * a.s + t;
-            da += a.dah[o]; dt += a.dth[o]; de += a.deh[o];
+            dg[0] += a.dah[o]; dg[1] += a.dth[o]; dg[2] += a.deh[o];
         }
-        da = wave_allreduce(da); dt = wave_allreduce(dt); de = wave_allreduce(de);
+#pragma unroll
+        for (int gi = 0; gi < 3; gi++) dg[gi] = wave_allreduce(dg[gi]);
         {
             const float al = a.alpha[lvl * n + tok], th = a.theta[lvl * n + tok], e = a.eta[lvl * n + tok];
-            da *= al * (1.0f - al);
-            dt *= 1.0f - expf(-th);
-            de *= e * (1.0f - e);
+            dg[0] *= al * (1.0f - al);
+            dg[1] *= 1.0f - expf(-th);
+            dg[2] *= e * (1.0f - e);
         }
-        accb[0] += da; accb[1] += dt; accb[2] += de;
+#pragma unroll
+        for (int gi = 0; gi < 3; gi++) accb[gi] += dg[gi];
         const float kn = a.k_norms[lvl * n + tok], qn = a.q_norms[lvl * n + tok];
         const float ki = 1.0f / fmaxf(kn, a.eps), qi = 1.0f / fmaxf(qn, a.eps);
-        float4 kk[NIT], qq[NIT], gk[NIT], gv[NIT], gq[NIT];
+        u16 *grow = a.G + tok * a.g_ld + a.col0 + 3LL * lvl * d + c0;
+        float gk[8], gq[8], kk[8], qq[8], vv[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) gk[e] = gq[e] = kk[e] = qq[e] = vv[e] = 0.f;
+        if (on) {
+            const size_t o = ((chain0 + b * a.nh + c0 / 64) * a.s + t) * 64 + c0 % 64;
+            widen(*reinterpret_cast<const bf16x8 *>(grow), gk);
+            widen(*reinterpret_cast<const bf16x8 *>(grow + 2 * d), gq);
+            widen(*reinterpret_cast<const bf16x8 *>(a.kh + o), kk);
+            widen(*reinterpret_cast<const bf16x8 *>(a.qh + o), qq);
+            widen(*reinterpret_cast<const bf16x8 *>(a.vh + o), vv);
+        }
         float dk_dot = 0.f, dq_dot = 0.f;
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            const int i4 = lane + 64 * it;
-            kk[it] = qq[it] = gk[it] = gv[it] = gq[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (i4 < d4) {
-                const int i = 4 * i4;
-                const size_t o = ((chain0 + b * a.nh + i / a.hd) * a.s + t) * a.hd + i % a.hd;
-                kk[it] = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(a.kh + o));
-                qq[it] = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(a.qh + o));
-                const float4 vv = bf4_to_f4(*reinterpret_cast<const bf16x4 *>(a.vh + o));
-                gk[it] = *reinterpret_cast<const float4 *>(a.dkh + o);
-                gv[it] = *reinterpret_cast<const float4 *>(a.dvh + o);
-                gq[it] = *reinterpret_cast<const float4 *>(a.dqh + o);
-                fma4(acc[0][0][it], da, kk[it]); fma4(acc[0][1][it], da, vv);
-                fma4(acc[1][0][it], dt, kk[it]); fma4(acc[1][1][it], dt, vv);
-                fma4(acc[2][0][it], de, kk[it]); fma4(acc[2][1][it], de, vv);
+        for (int e = 0; e < 8; e++) {
+            dk_dot += gk[e] * kk[e];
+            dq_dot += gq[e] * qq[e];
+#pragma unroll
+            for (int gi = 0; gi < 3; gi++) {
+                acc[gi][0][e] = fmaf(dg[gi], kk[e], acc[gi][0][e]);
+                acc[gi][1][e] = fmaf(dg[gi], vv[e], acc[gi][1][e]);
             }
-            dk_dot += dot4(gk[it], kk[it]);
-            dq_dot += dot4(gq[it], qq[it]);
         }
         dk_dot = wave_allreduce(dk_dot);
         dq_dot = wave_allreduce(dq_dot);
-        u16 *grow = a.G + tok * a.g_ld + a.col0 + 3LL * lvl * d;
+        if (on) {
+            bf16x8 ok, oq;
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            const int i4 = lane + 64 * it;
-            if (i4 >= d4) continue;
-            float4 x, c;
-            if (kn >= a.eps) {
-                x.x = (gk[it].x - kk[it].x * dk_dot) * ki; x.y = (gk[it].y - kk[it].y * dk_dot) * ki;
-                x.z = (gk[it].z - kk[it].z * dk_dot) * ki; x.w = (gk[it].w - kk[it].w * dk_dot) * ki;
-            } else {
-                x.x = gk[it].x * inv_eps; x.y = gk[it].y * inv_eps; x.z = gk[it].z * inv_eps; x.w = gk[it].w * inv_eps;
+            for (int e = 0; e < 8; e++) {
+                ok[e] = (__bf16)(kn >= a.eps ? (gk[e] - kk[e] * dk_dot) * ki : gk[e] * inv_eps);
+                oq[e] = (__bf16)(qn >= a.eps ? (gq[e] - qq[e] * dq_dot) * qi : gq[e] * inv_eps);
             }
-            if (qn >= a.eps) {
-                c.x = (gq[it].x - qq[it].x * dq_dot) * qi; c.y = (gq[it].y - qq[it].y * dq_dot) * qi;
-                c.z = (gq[it].z - qq[it].z * dq_dot) * qi; c.w = (gq[it].w - qq[it].w * dq_dot) * qi;
-            } else {
-                c.x = gq[it].x * inv_eps; c.y = gq[it].y * inv_eps; c.z = gq[it].z * inv_eps; c.w = gq[it].w * inv_eps;
-            }
-            *reinterpret_cast<bf16x4 *>(grow + 4 * i4) = f4_to_bf4(x);
-            *reinterpret_cast<bf16x4 *>(grow + d + 4 * i4) = f4_to_bf4(gv[it]);
-            *reinterpret_cast<bf16x4 *>(grow + 2 * d + 4 * i4) = f4_to_bf4(c);
+            *reinterpret_cast<bf16x8 *>(grow) = ok;
+            *reinterpret_cast<bf16x8 *>(grow + 2 * d) = oq;
         }
     }
     // the workgroup's partial row: the waves add their sums into LDS one after the other (fixed order)
@@ -484,17 +482,16 @@ __global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
         if (wave_l == w) {
 #pragma unroll
             for (int gi = 0; gi < 3; gi++) {
+                if (on) {
 #pragma unroll
-                for (int h = 0; h < 2; h++)
+                    for (int h = 0; h < 2; h++)
 #pragma unroll
-                    for (int it = 0; it < NIT; it++) {
-                        const int i4 = lane + 64 * it;
-                        if (i4 >= d4) continue;
-                        float *r = redg + gi * stride + h * d + 4 * i4;
-                        const float4 v = acc[gi][h][it];
-                        if (w == 0) { r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w; }
-                        else { r[0] += v.x; r[1] += v.y; r[2] += v.z; r[3] += v.w; }
-                    }
+                        for (int e = 0; e < 8; e++) {
+                            float *r = redg + gi * stride + h * d + c0 + e;
+                            if (w == 0) *r = acc[gi][h][e];
+                            else *r += acc[gi][h][e];
+                        }
+                }
                 if (lane == 0) {
                     if (w == 0) redg[gi * stride + 2 * d] = accb[gi];
                     else redg[gi * stride + 2 * d] += accb[gi];
@@ -807,32 +804,36 @@ void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_ext
         fail("titans_levels_backward_bf16_rocm: buffers must be 16-byte aligned.");
         return;
     }
-    const size_t tok_f = (size_t)chains * seq_len * head_dim, gate_f = (size_t)chains * seq_len;
-    float *hg = scratch(25, (3 * tok_f + 3 * gate_f) * sizeof(float));          // d_k, d_v, d_q, d_alpha, d_theta, d_eta (head-major)
+    const size_t gate_f = (size_t)chains * seq_len;
+    float *hg = scratch(25, (3 * gate_f + 4) * sizeof(float));                  // d_alpha, d_theta, d_eta per chain and token
     u16 *G = reinterpret_cast<u16 *>(scratch(26, (size_t)n * R * sizeof(u16)));
     u16 *wb = reinterpret_cast<u16 *>(scratch(27, (size_t)R * d * sizeof(u16)));
     const int nblk = stream_blocks(n * 64, 256);
     const size_t prow = 3 * (2 * (size_t)d + 1);
     float *part = scratch(28, (size_t)(levels ? levels : 1) * nblk * prow * sizeof(float));
     if (es.failed()) return;
-    float *dkh = hg, *dvh = hg + tok_f, *dqh = hg + 2 * tok_f, *dah = hg + 3 * tok_f, *dth = dah + gate_f, *deh = dth + gate_f;
+    float *dah = hg, *dth = dah + gate_f, *deh = dth + gate_f;
     if (levels) {
-        titans_chunkwise_backward_bf16_tokens_rocm(k_heads, v_heads, q_heads, alpha_heads, theta_heads, eta_heads,
-                                                   m_chunk_states, s_chunk_states, d_y_tokens, dkh, dvh, dqh, dah, dth, deh,
-                                                   d_m_initial, d_s_initial, seq_len, head_dim, chains, chunk_size, heads,
-                                                   levels, 0);
+        // the rule writes d_k, d_v, d_q straight into the level's columns of G: chain (level, batch element, head) owns
+        // columns col0 + 3 level d + {0, d, 2d} + 64 head .. + 64 of the rows of its batch element
+        GradOut16 out{};
+        out.gk = G + (size_t)n_extra * d;
+        out.gv = out.gk + d;
+        out.gq = out.gk + 2 * d;
+        out.rows = HeadRows{3LL * d, (long long)seq_len * R, 64, R, bs * heads, heads};
+        titans_chunkwise_backward_bf16_tokens_g16(k_heads, v_heads, q_heads, alpha_heads, theta_heads, eta_heads,
+                                                  m_chunk_states, s_chunk_states, d_y_tokens, out, dah, dth, deh, d_m_initial,
+                                                  d_s_initial, seq_len, head_dim, chains, chunk_size, heads, levels, 0);
         if (es.failed()) return;
         GradArgs ga{};
-        ga.dkh = dkh; ga.dvh = dvh; ga.dqh = dqh; ga.dah = dah; ga.dth = dth; ga.deh = deh;
+        ga.dah = dah; ga.dth = dth; ga.deh = deh;
         ga.kh = k_heads; ga.vh = v_heads; ga.qh = q_heads;
         ga.k_norms = k_norms; ga.q_norms = q_norms; ga.alpha = alpha; ga.theta = theta; ga.eta = eta;
         ga.G = G; ga.g_ld = R; ga.col0 = (long long)n_extra * d; ga.part = part;
-        ga.bs = bs; ga.s = seq_len; ga.nh = heads; ga.hd = head_dim; ga.levels = levels; ga.eps = eps;
+        ga.bs = bs; ga.s = seq_len; ga.nh = heads; ga.levels = levels; ga.eps = eps;
         {
             KernelTimer kt("level_grads_bf16_kernel");
-            const dim3 grid(nblk, levels);
-            if (d <= 256) hipLaunchKernelGGL(level_grads_bf16_kernel<1>, grid, dim3(kSThr), prow * sizeof(float), stream(), ga);
-            else hipLaunchKernelGGL(level_grads_bf16_kernel<2>, grid, dim3(kSThr), prow * sizeof(float), stream(), ga);
+            hipLaunchKernelGGL(level_grads_bf16_kernel, dim3(nblk, levels), dim3(kSThr), prow * sizeof(float), stream(), ga);
             check_launch("level_grads_bf16_kernel");
         }
         GateGradOuts go{};
