@@ -200,3 +200,26 @@ def test_config4_layer_against_autograd_at_k4_periods_up_to_512():
                  seed=0xC6, bias_scale=True)
     print({n: f"{e:.1e}" for n, e in w.items()}, flush=True)
     assert max(w.values()) < 2e-2, w
+
+
+def test_config4_layer_behind_the_c_abi_at_full_sequence_length_against_autograd():
+    """The same layer on the path that issues every projection through the library (precision "bf16": x and the weights
+    rounded once to bf16, fp32 accumulation; titans_levels_{forward,backward}_bf16_rocm) on one sequence of the
+    configuration's full 4096 tokens (64 chunks per chain, every level's period inside the sequence) against the float64
+    autograd restatement: output, d_x and every parameter gradient at the bf16 bar."""
+    import nl_hecate_amd.mag_layer as ML
+    from tests.test_gpu_mag_layer import run_case
+    orig = ML.MagLayer.__init__
+
+    def init_bf16(self, *a, **kw):
+        kw["precision"] = "bf16"
+        orig(self, *a, **kw)
+    ML.MagLayer.__init__ = init_bf16
+    try:
+        print("configs[4]: layer behind the C ABI, 1 x 4096 tokens, k = 4", flush=True)
+        w = run_case(bs=1, s=4096, d=512, nh=8, k=4, window=512, periods=[1, 8, 64, 512], rule="chunkwise", chunk=64,
+                     seed=0xC7, bias_scale=True)
+    finally:
+        ML.MagLayer.__init__ = orig
+    print({n: f"{e:.1e}" for n, e in w.items()}, flush=True)
+    assert max(w.values()) < 2e-2, w
