@@ -709,7 +709,7 @@ def write_profile(workload, raw):
             f.write("\n".join(lines) + "\n")
         with open(os.path.join(ROOT, "profiles", workload + ".json"), "w") as f:
             json.dump({"workload": workload, "git_head": git_head(), "source_sha256": source_hash(workload),
-                       "sources": WORKLOAD_SOURCES[workload], "step_traffic_bytes": int(step_bytes), "probes": res["probes"]}, f, indent=1, sort_keys=True)
+                       "sources": WORKLOAD_SOURCES[workload], "probes": res["probes"]}, f, indent=1, sort_keys=True)
             f.write("\n")
         print("\n".join(lines))
         return
