@@ -628,17 +628,28 @@ WORKLOAD_SOURCES = {
 }
 
 
+def workload_files(workload):
+    """The kernel sources of a workload and the library headers they include, directly or through one another
+    (the C ABI header is left out: a new declaration changes no kernel)."""
+    import re
+    csrc = os.path.join(ROOT, "nl_hecate_amd", "csrc")
+    todo, seen = list(WORKLOAD_SOURCES[workload]), []
+    while todo:
+        f = todo.pop()
+        if f in seen or not os.path.exists(os.path.join(csrc, f)):
+            continue
+        seen.append(f)
+        todo += re.findall(r'#include "([A-Za-z0-9_]+\.h)"', open(os.path.join(csrc, f)).read())
+    return sorted(seen)
+
+
 def source_hash(workload):
-    """sha256 over the kernel sources of a workload, every header of the library and the C ABI header."""
-    import glob
+    """sha256 over the kernel sources of a workload and the headers they include."""
     import hashlib
     h = hashlib.sha256()
-    csrc = os.path.join(ROOT, "nl_hecate_amd", "csrc")
-    files = sorted([os.path.join(csrc, f) for f in WORKLOAD_SOURCES[workload]] + glob.glob(os.path.join(csrc, "*.h")) +
-                   [os.path.join(ROOT, "include", "nl_hecate_ffi.h")])
-    for f in files:
-        h.update(os.path.basename(f).encode())
-        h.update(open(f, "rb").read())
+    for f in workload_files(workload):
+        h.update(f.encode())
+        h.update(open(os.path.join(ROOT, "nl_hecate_amd", "csrc", f), "rb").read())
     return h.hexdigest()
 
 
@@ -695,7 +706,8 @@ def write_profile(workload, raw):
         lines = [f"{workload}: what the probe kernels (csrc/roof_probes.hip) sustain on one MI355X (rocprofv3, ROCm 7.2)", "",
                  f"commands (from /tmp, TMPDIR=/tmp): {cmd} > <out>/bench_{workload}.json; rocprofv3 --kernel-trace --stats "
                  f"--output-format csv -d <out>/trace_{workload} -o t -- {cmd}", "",
-                 f"sources: git {git_head()}, sha256 of csrc/roof_probes.hip, csrc/*.h and the C header {source_hash(workload)[:16]}", "",
+                 f"sources: git {git_head()}, sha256 of {', '.join('csrc/' + f for f in workload_files(workload))} "
+                 f"{source_hash(workload)[:16]}", "",
                  f"{'probe':44s} {'ms':>9s} {'achieved':>10s} {'unit':>8s} {'of data-sheet peak':>19s}"]
         res = json.load(open(os.path.join(raw, f"bench_{workload}.json")))
         for pr in res["probes"]:
@@ -709,7 +721,7 @@ def write_profile(workload, raw):
             f.write("\n".join(lines) + "\n")
         with open(os.path.join(ROOT, "profiles", workload + ".json"), "w") as f:
             json.dump({"workload": workload, "git_head": git_head(), "source_sha256": source_hash(workload),
-                       "sources": WORKLOAD_SOURCES[workload], "probes": res["probes"]}, f, indent=1, sort_keys=True)
+                       "sources": workload_files(workload), "probes": res["probes"]}, f, indent=1, sort_keys=True)
             f.write("\n")
         print("\n".join(lines))
         return
@@ -729,8 +741,8 @@ def write_profile(workload, raw):
              f"  rocprofv3 --pmc WRITE_SIZE --output-format csv -d <out>/pmc_WRITE_SIZE_{workload} -o p -- {cmd} --steps 2 --warmup 1 --no-cpu-baseline",
              "  rocprofv3 --pmc FETCH_SIZE (then WRITE_SIZE) --output-format csv -d <out>/pmc_<counter>_calib -o p -- python3 bench.py --calibrate-copy"
              "   (plain map kernel: 262144 KiB read, 262144 KiB written per launch)", "",
-             f"sources: git {git_head()}, sha256 of {', '.join('csrc/' + f for f in WORKLOAD_SOURCES[workload])}, csrc/*.h and the "
-             f"C header {source_hash(workload)[:16]}", "",
+             f"sources: git {git_head()}, sha256 of {', '.join('csrc/' + f for f in workload_files(workload))} "
+             f"{source_hash(workload)[:16]}", "",
              "kernel trace (warm-up + timed steps + the per-entry-point and per-kernel timing launches of bench.py)",
              f"{'kernel':62s} {'calls':>6s} {'total_us':>11s} {'avg_us':>10s} {'pct':>6s}"]
     kernels = {}
@@ -781,7 +793,7 @@ def write_profile(workload, raw):
     with open(out_txt, "w") as f:
         f.write("\n".join(lines) + "\n")
     side = {"workload": workload, "git_head": git_head(), "source_sha256": source_hash(workload),
-            "sources": WORKLOAD_SOURCES[workload], "step_traffic_bytes": int(step_bytes),
+            "sources": workload_files(workload), "step_traffic_bytes": int(step_bytes),
             "calibration": {"fetch_factor": ff, "write_factor": fw,
                             "note": "counter KiB per dispatch x factor = KiB moved; factors from a map kernel of known size"},
             "kernels": kernels}

@@ -18,113 +18,99 @@
 #include "../../include/nl_hecate_ffi.h"
 #include "chunkwise_guard.h"
 #include "lane_ops.h"
+#include "mm_tiles.h"
 #include "runtime.h"
 
 namespace nlh {
 namespace {
 
-constexpr int GD = 64;        // head size of the matrix form
-constexpr int GS = 68;        // LDS row stride (16-byte rows)
+using namespace mmt;
+
 constexpr float kSlack = 1.0f + 1e-4f;   // covers the rounding of the fp32 sums below
 
-__device__ __forceinline__ float tok1(const float *p, size_t i) { return p[i]; }
-__device__ __forceinline__ float tok1(const uint16_t *p, size_t i) { return __uint_as_float(((unsigned)p[i]) << 16); }
-// four consecutive tokens' elements as floats
-__device__ __forceinline__ float4 tok4(const float *p, size_t i) { return *reinterpret_cast<const float4 *>(p + i); }
-__device__ __forceinline__ float4 tok4(const uint16_t *p, size_t i) {
-    const uint2 u = *reinterpret_cast<const uint2 *>(p + i);
-    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
-                       __uint_as_float(u.y & 0xffff0000u));
+__device__ __forceinline__ float lane_value(float x, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
 }
 
+// One workgroup (8 waves) per chunk; four workgroups share a compute unit, so one's loads overlap another's
+// product (a persistent variant with the next chunk's tiles requested a chunk ahead needs twice the registers,
+// halves the workgroups per compute unit and is slower).  E = K M0^T - V on the fp32 matrix cores, a 16 x 32
+// strip per wave; the sums of squares of the states come from the registers the tiles were loaded into; wave 0
+// then runs the scalar recurrence with lane t holding token t's numbers.
 template <typename TOK, bool HAS_S>
-__global__ __launch_bounds__(256) void cw_guard_kernel(const TOK *__restrict__ k, const TOK *__restrict__ v,
-                                                       const float *__restrict__ alpha, const float *__restrict__ theta,
-                                                       const float *__restrict__ eta, const float *__restrict__ m_states,
-                                                       const float *__restrict__ s_states, int seq_len, int C, int nc,
-                                                       float clip, float mmax, int *__restrict__ flag) {
-    __shared__ __align__(16) float M0[GD * GS], Ks[GD * GS];
-    __shared__ float en[GD], kn[GD], gate[3][GD], red[2][4];
+__global__ __launch_bounds__(kThr) void cw_guard_kernel(const TOK *__restrict__ k, const TOK *__restrict__ v,
+                                                        const float *__restrict__ alpha, const float *__restrict__ theta,
+                                                        const float *__restrict__ eta, const float *__restrict__ m_states,
+                                                        const float *__restrict__ s_states, int seq_len, int C, int nc,
+                                                        float clip, float mmax, int *__restrict__ flag) {
+    __shared__ float Ks[MAT], Ms[MAT];
+    __shared__ float en2[2][CW], kn2[CW], red[2][8];
     const int tid = threadIdx.x, chunk = blockIdx.x % nc, chain = blockIdx.x / nc;
     const int t0 = chunk * C, L = min(C, seq_len - t0);
-    const float *m0 = m_states + ((size_t)chain * (nc + 1) + chunk) * GD * GD;
-    const float *s0 = HAS_S ? s_states + ((size_t)chain * (nc + 1) + chunk) * GD * GD : nullptr;
-    float msq = 0.f, ssq = 0.f;
-    for (int e = tid; e < GD * GD / 4; e += 256) {
-        const float4 x = reinterpret_cast<const float4 *>(m0)[e];
-        *reinterpret_cast<float4 *>(M0 + (e / 16) * GS + (e % 16) * 4) = x;
-        msq += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
-        if (HAS_S) {
-            const float4 y = reinterpret_cast<const float4 *>(s0)[e];
-            ssq += y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
-        }
+    const size_t st0 = ((size_t)chain * (nc + 1) + chunk) * HD * HD;
+    const size_t tok = (size_t)chain * seq_len + t0;
+    const int w = tid >> 6, m0 = 16 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1;
+    Tile<TOK> tk;
+    Tile<float> tm, ts;
+    fetch(tk, k + tok * HD, L);
+    fetch(tm, m_states + st0, 64);
+    if (HAS_S) fetch(ts, s_states + st0, 64);
+    // -V at this wave's accumulator positions
+    Strip e = zero_strip();
+    for_c(e, [&](int r, int c, float &x) { x = m0 + r < L ? -to_f32(v[(tok + m0 + r) * HD + n0 + c]) : 0.f; });
+    float al = 0.f, th = 0.f, et = 0.f;
+    if (w == 0 && tid < L) {
+        al = alpha[tok + tid];
+        th = theta[tok + tid];
+        if (HAS_S) et = eta[tok + tid];
     }
-    const size_t tok0 = ((size_t)chain * seq_len + t0) * GD;
-    for (int e = tid; e < GD * GD / 4; e += 256) {
-        const int t = e / 16, j = (e % 16) * 4;
-        float4 kx = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (t < L) kx = tok4(k, tok0 + 4 * (size_t)e);
-        *reinterpret_cast<float4 *>(Ks + t * GS + j) = kx;
-    }
-    if (tid < GD) {
-        const size_t g = (size_t)chain * seq_len + t0 + tid;
-        gate[0][tid] = tid < L ? alpha[g] : 0.f;
-        gate[1][tid] = tid < L ? theta[g] : 0.f;
-        gate[2][tid] = (HAS_S && tid < L) ? eta[g] : 0.f;
-    }
-    // -V: every thread its own 16 elements (consecutive lanes on consecutive columns), requested before the barrier
-    float e[4][4];
+    commit(Ks, tk);
+    commit(Ms, tm);
     {
-        const int ti = tid >> 4, ii = tid & 15;
+        float msq = 0.f, ssq = 0.f;
 #pragma unroll
-        for (int a = 0; a < 4; a++)
-#pragma unroll
-            for (int b = 0; b < 4; b++)
-                e[a][b] = 4 * ti + a < L ? -tok1(v, tok0 + (size_t)(4 * ti + a) * GD + ii + 16 * b) : 0.f;
-    }
-    msq = wave_allreduce(msq);
-    ssq = wave_allreduce(ssq);
-    if ((tid & 63) == 0) { red[0][tid >> 6] = msq; red[1][tid >> 6] = ssq; }
-    __syncthreads();
-    {   // E = K M0^T - V in 4 x 4 register blocks: thread (ti, ii) owns tokens 4 ti .. + 3 and rows ii, ii + 16, ii + 32,
-        // ii + 48 of M0 (consecutive lanes on consecutive rows: conflict-free 16-byte reads at row stride 68)
-        const int ti = tid >> 4, ii = tid & 15;
-        float ksq[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-        for (int j4 = 0; j4 < GD / 4; j4++) {
-            float4 kx[4], mx[4];
-#pragma unroll
-            for (int a = 0; a < 4; a++) kx[a] = *reinterpret_cast<const float4 *>(Ks + (4 * ti + a) * GS + 4 * j4);
-#pragma unroll
-            for (int b = 0; b < 4; b++) mx[b] = *reinterpret_cast<const float4 *>(M0 + (ii + 16 * b) * GS + 4 * j4);
-#pragma unroll
-            for (int a = 0; a < 4; a++) {
-                if ((j4 & 15) == ii) ksq[a] += kx[a].x * kx[a].x + kx[a].y * kx[a].y + kx[a].z * kx[a].z + kx[a].w * kx[a].w;
-#pragma unroll
-                for (int b = 0; b < 4; b++)
-                    e[a][b] += kx[a].x * mx[b].x + kx[a].y * mx[b].y + kx[a].z * mx[b].z + kx[a].w * mx[b].w;
-            }
+        for (int it = 0; it < 2; it++) {
+            msq += tm.x[it].x * tm.x[it].x + tm.x[it].y * tm.x[it].y + tm.x[it].z * tm.x[it].z + tm.x[it].w * tm.x[it].w;
+            if (HAS_S) ssq += ts.x[it].x * ts.x[it].x + ts.x[it].y * ts.x[it].y + ts.x[it].z * ts.x[it].z + ts.x[it].w * ts.x[it].w;
         }
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-            float esq = e[a][0] * e[a][0] + e[a][1] * e[a][1] + e[a][2] * e[a][2] + e[a][3] * e[a][3];
-            esq = group_allreduce<16>(esq);
-            const float kq = group_allreduce<16>(ksq[a]);
-            if (ii == 0) { en[4 * ti + a] = sqrtf(esq) * kSlack; kn[4 * ti + a] = sqrtf(kq) * kSlack; }
-        }
+        msq = wave_allreduce(msq);
+        ssq = wave_allreduce(ssq);
+        if ((tid & 63) == 0) { red[0][w] = msq; red[1][w] = ssq; }
     }
     __syncthreads();
-    if (tid == 0) {
-        float nM = sqrtf(red[0][0] + red[0][1] + red[0][2] + red[0][3]) * kSlack;
-        float nS = HAS_S ? sqrtf(red[1][0] + red[1][1] + red[1][2] + red[1][3]) * kSlack : 0.f;
+    if (w == 1) {   // |k_t|^2 of row (lane) (rows beyond L were staged as zeros)
+        const int t = tid & 63;
+        float x = 0.f;
+#pragma unroll 16
+        for (int c = 0; c < HD; c++) x = fmaf(Ks[t * LDM + c], Ks[t * LDM + c], x);
+        kn2[t] = x;
+    }
+    mma(e, [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+    for_c(e, [&](int, int, float &x) { x *= x; });
+    strip_row_sums(e);
+    if (row_writer()) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) en2[nh][m0 + row_of(i)] = e.t[0][i];
+    }
+    __syncthreads();
+    if (w == 0) {
+        const float en = sqrtf(en2[0][tid] + en2[1][tid]) * kSlack, kn = sqrtf(kn2[tid]) * kSlack;
+        const float drive = th * en * kn, keep = 1.0f - al;
+        float nM = 0.f, nS = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { nM += red[0][i]; nS += red[1][i]; }
+        nM = sqrtf(nM) * kSlack;
+        nS = HAS_S ? sqrtf(nS) * kSlack : 0.f;
         const bool clip_on = clip > 0.f, proj_on = mmax > 0.f && mmax < 1e30f;
-        bool bad = false;
-        for (int t = 0; t < L; t++) {
-            if (clip_on && en[t] > clip) bad = true;
-            nS = (HAS_S ? gate[2][t] * nS : 0.f) + gate[1][t] * en[t] * kn[t];
-            nM = (1.0f - gate[0][t]) * nM + nS;
-            if (proj_on && nM * kSlack > mmax) bad = true;
+        bool bad = clip_on && tid < L && en > clip;
+        float worst = 0.f;
+#pragma unroll 8
+        for (int t = 0; t < CW; t++) {   // tokens beyond L carry keep = 1, eta = 0, no drive: they only repeat nM
+            nS = (HAS_S ? lane_value(et, t) * nS : 0.f) + lane_value(drive, t);
+            nM = lane_value(keep, t) * nM + nS;
+            worst = t < L ? fmaxf(worst, nM) : worst;
         }
+        if (proj_on && worst * kSlack > mmax) bad = true;
         if (bad) *flag = 1;
     }
 }
@@ -157,10 +143,10 @@ static bool couplings_may_fire_t(const TOK *k, const TOK *v, const float *alpha,
         hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(1), 0, stream(), flag);
         const dim3 grid((unsigned)batch * nc);
         if (s_states)
-            hipLaunchKernelGGL((cw_guard_kernel<TOK, true>), grid, dim3(256), 0, stream(), k, v, alpha, theta, eta, m_states,
+            hipLaunchKernelGGL((cw_guard_kernel<TOK, true>), grid, dim3(kThr), 0, stream(), k, v, alpha, theta, eta, m_states,
                                s_states, seq_len, chunk_size, nc, error_clip, m_norm_max, flag);
         else
-            hipLaunchKernelGGL((cw_guard_kernel<TOK, false>), grid, dim3(256), 0, stream(), k, v, alpha, theta, eta, m_states,
+            hipLaunchKernelGGL((cw_guard_kernel<TOK, false>), grid, dim3(kThr), 0, stream(), k, v, alpha, theta, eta, m_states,
                                s_states, seq_len, chunk_size, nc, error_clip, m_norm_max, flag);
         check_launch("cw_guard_kernel");
     }

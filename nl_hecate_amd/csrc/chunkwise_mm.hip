@@ -31,119 +31,14 @@
 #include "../../include/nl_hecate_ffi.h"
 #include "chunkwise_chain.h"
 #include "chunkwise_grads.h"
+#include "mm_tiles.h"
 #include "rule_common.h"
 #include "runtime.h"
 
 namespace nlh {
 namespace {
 
-using f32x4 = __attribute__((ext_vector_type(4))) float;
-
-constexpr int CW = 64;          // tokens per chunk tile
-constexpr int HD = 64;          // head size
-constexpr int LDM = 65;         // LDS row stride in floats (odd: conflict-free rows and columns)
-constexpr int MAT = 64 * LDM;   // floats per 64x64 LDS matrix
-constexpr int kThr = 512;       // 8 waves (two per SIMD), one 16x32 output strip each
-
-__device__ __forceinline__ float to_f32(float x) { return x; }
-__device__ __forceinline__ float to_f32(uint16_t u) { return __uint_as_float((uint32_t)u << 16); }
-
-// Staging of a row-major [nrows <= 64][64] global tile into LDS in two halves, so that the
-// loads of every tile of a phase are in flight together: fetch() issues the global loads
-// into registers (rows >= nrows read as zero), commit() converts and stores to LDS.
-template <class T> struct Tile;
-template <> struct Tile<float> { float4 x[2]; };
-template <> struct Tile<uint16_t> { uint2 x[2]; };
-
-template <class T>
-__device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows) {
-#pragma unroll
-    for (int it = 0; it < 2; it++) {
-        const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
-        if constexpr (sizeof(T) == 4)
-            r.x[it] = rr < nrows ? *reinterpret_cast<const float4 *>(src + rr * 64 + cc) : make_float4(0, 0, 0, 0);
-        else
-            r.x[it] = rr < nrows ? *reinterpret_cast<const uint2 *>(src + rr * 64 + cc) : make_uint2(0, 0);
-    }
-}
-template <class T>
-__device__ __forceinline__ void commit(float *dst, const Tile<T> &r) {
-#pragma unroll
-    for (int it = 0; it < 2; it++) {
-        const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
-        float *p = dst + rr * LDM + cc;
-        if constexpr (sizeof(T) == 4) {
-            p[0] = r.x[it].x; p[1] = r.x[it].y; p[2] = r.x[it].z; p[3] = r.x[it].w;
-        } else {
-            p[0] = __uint_as_float(r.x[it].x << 16); p[1] = __uint_as_float(r.x[it].x & 0xffff0000u);
-            p[2] = __uint_as_float(r.x[it].y << 16); p[3] = __uint_as_float(r.x[it].y & 0xffff0000u);
-        }
-    }
-}
-template <class T>
-__device__ __forceinline__ void stage(float *dst, const T *src, int nrows) {
-    Tile<T> r;
-    fetch(r, src, nrows);
-    commit(dst, r);
-}
-
-// Output strip of one wave: 16 rows x 32 columns = two 16x16 accumulator tiles side by side.
-// With 8 waves a 64x64 product is 8 strips; two waves share a SIMD, so one wave's LDS reads,
-// epilogue arithmetic and stores overlap the other's matrix-core work.
-struct Strip { f32x4 t[2]; };
-__device__ __forceinline__ Strip zero_strip() {
-    Strip z;
-#pragma unroll
-    for (int i = 0; i < 4; i++) { z.t[0][i] = 0.f; z.t[1][i] = 0.f; }
-    return z;
-}
-// acc += sum_{k<64} a(m,k) b(k,n), m in [0,16), n in [0,32).
-// Operand layout of v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][l/16] and B[l/16][l%16].
-// Sixteen k-steps in four groups; the operands of group g+1 are read while group g runs.
-template <class FA, class FB>
-__device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
-    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4;
-    float av[2][4], b0[2][4], b1[2][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) { av[0][i] = a(r, 4 * i + kq); b0[0][i] = b(4 * i + kq, r); b1[0][i] = b(4 * i + kq, 16 + r); }
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-        if (g < 3) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int kk = 16 * (g + 1) + 4 * i + kq;
-                av[(g + 1) & 1][i] = a(r, kk); b0[(g + 1) & 1][i] = b(kk, r); b1[(g + 1) & 1][i] = b(kk, 16 + r);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g & 1][i], b0[g & 1][i], acc.t[0], 0, 0, 0);
-            acc.t[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g & 1][i], b1[g & 1][i], acc.t[1], 0, 0, 0);
-        }
-    }
-}
-// Element i of tile tl of lane l is C[4*(l/16) + i][16*tl + l%16] of the strip.
-template <class F>
-__device__ __forceinline__ void for_c(Strip &acc, F f) {
-    const int l = threadIdx.x & 63;
-#pragma unroll
-    for (int tl = 0; tl < 2; tl++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float x = acc.t[tl][i];
-            f(4 * (l >> 4) + i, 16 * tl + (l & 15), x);
-            acc.t[tl][i] = x;
-        }
-}
-// Row sums of a strip: afterwards t[0][i] of every lane holds the sum over the 32 columns of
-// strip row 4*(l/16) + i.
-__device__ __forceinline__ void strip_row_sums(Strip &x) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) x.t[0][i] = group_allreduce<16>(x.t[0][i] + x.t[1][i]);
-}
-// lanes that publish the row sums (one per 16-lane group), and the strip rows they hold
-__device__ __forceinline__ bool row_writer() { return (threadIdx.x & 15) == 0; }
-__device__ __forceinline__ int row_of(int i) { return 4 * ((threadIdx.x & 63) >> 4) + i; }
+using namespace mmt;
 
 // Gate coefficients of one chunk (L <= 64 tokens), all in LDS.
 struct Coef {

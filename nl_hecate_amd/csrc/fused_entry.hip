@@ -4,8 +4,8 @@
 //       clamp alpha / theta, then run the recurrence over the full trajectory.
 //   error_subtract_clip_f32_cuda         (core/kernels/error_subtract_clip.cu): pred -= v per
 //       row, then L2-clip each row.
-// The recurrence dominates; normalisation and gates are streaming kernels launched ahead of it
-// on the same stream.
+// The recurrence dominates; normalisation, gates and clamps are one streaming pass (fused_prep_kernel, a wave
+// per token) launched ahead of it on the same stream: two launches per call.
 #include <hip/hip_runtime.h>
 
 #include "../../include/nl_hecate_ffi.h"
@@ -38,6 +38,64 @@ __global__ void error_subtract_clip_kernel(float *__restrict__ pred, const float
     }
 }
 
+__device__ __forceinline__ float sigmoid_(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplus_(float x) { return x > 20.0f ? x : logf(1.0f + expf(x)); }
+
+// What l2_normalize_rows x 2, gate_compute x 2 or 3 and clamp x 2 do, in one pass: one wave per token, the
+// sums over the same lane pattern as those kernels.
+template <bool HAS_ETA>
+__global__ void fused_prep_kernel(float *__restrict__ k, const float *__restrict__ v, float *__restrict__ q,
+                                  const float *__restrict__ w_alpha, const float *__restrict__ b_alpha,
+                                  const float *__restrict__ w_theta, const float *__restrict__ b_theta,
+                                  const float *__restrict__ w_eta, const float *__restrict__ b_eta, float alpha_floor,
+                                  float alpha_ceil, float theta_floor, float theta_ceil, float *__restrict__ alpha,
+                                  float *__restrict__ theta, float *__restrict__ eta, float *__restrict__ k_norms,
+                                  float *__restrict__ q_norms, int rows, int d) {
+    const int lane = threadIdx.x & 63;
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, nwaves = (gridDim.x * blockDim.x) >> 6;
+    const float ba = b_alpha[0], bt = b_theta[0], be = HAS_ETA ? b_eta[0] : 0.f;
+    for (int r = wave; r < rows; r += nwaves) {
+        float *kr = k + (size_t)r * d, *qr = q + (size_t)r * d;
+        const float *vr = v + (size_t)r * d;
+        float sk = 0.f, sq = 0.f;
+        for (int j = lane; j < d; j += 64) { const float a = kr[j], b = qr[j]; sk += a * a; sq += b * b; }
+        const float kn = sqrtf(wave_allreduce(sk)), qn = sqrtf(wave_allreduce(sq));
+        const float ki = 1.0f / fmaxf(kn, 1e-8f), qi = 1.0f / fmaxf(qn, 1e-8f);
+        float ga = 0.f, gt = 0.f, ge = 0.f;
+        for (int j = lane; j < d; j += 64) {
+            const float a = kr[j] * ki, b = vr[j];
+            kr[j] = a;
+            qr[j] *= qi;
+            ga += a * w_alpha[j] + b * w_alpha[d + j];
+            gt += a * w_theta[j] + b * w_theta[d + j];
+            if (HAS_ETA) ge += a * w_eta[j] + b * w_eta[d + j];
+        }
+        ga = wave_allreduce(ga) + ba;
+        gt = wave_allreduce(gt) + bt;
+        if (HAS_ETA) ge = wave_allreduce(ge) + be;
+        if (lane == 0) {
+            k_norms[r] = kn;
+            q_norms[r] = qn;
+            alpha[r] = fmaxf(alpha_floor, fminf(alpha_ceil, sigmoid_(ga)));
+            theta[r] = fmaxf(theta_floor, fminf(theta_ceil, softplus_(gt)));
+            if (HAS_ETA) eta[r] = sigmoid_(ge);
+        }
+    }
+}
+
+template <bool HAS_ETA>
+void fused_prep(float *k, const float *v, float *q, const float *w_alpha, const float *b_alpha, const float *w_theta,
+                const float *b_theta, const float *w_eta, const float *b_eta, float alpha_floor, float alpha_ceil,
+                float theta_floor, float theta_ceil, float *alpha, float *theta, float *eta, float *k_norms, float *q_norms,
+                int rows, int d) {
+    const long long threads = (long long)rows * 64;
+    const int blocks = (int)((threads + 255) / 256 > 65535 * 16 ? 65535 * 16 : (threads + 255) / 256);
+    hipLaunchKernelGGL(fused_prep_kernel<HAS_ETA>, dim3(blocks), dim3(256), 0, stream(), k, v, q, w_alpha, b_alpha, w_theta,
+                       b_theta, w_eta, b_eta, alpha_floor, alpha_ceil, theta_floor, theta_ceil, alpha, theta, eta, k_norms,
+                       q_norms, rows, d);
+    check_launch("fused_prep_kernel");
+}
+
 }  // namespace
 }  // namespace nlh
 
@@ -68,13 +126,8 @@ extern "C" void titans_fused_forward_f32_cuda(float *k_mem, const float *v_mem, 
         return;
     }
     const int rows = batch_size * seq_len;
-    l2_normalize_rows_f32_cuda(k_mem, k_norms_out, rows, d, 1e-8f);
-    l2_normalize_rows_f32_cuda(q_mem, q_norms_out, rows, d, 1e-8f);
-    gate_compute_cuda(k_mem, v_mem, w_alpha, b_alpha_ptr, alpha_out, rows, d, 0);
-    clamp_f32_cuda(alpha_out, rows, alpha_floor, alpha_ceil);
-    gate_compute_cuda(k_mem, v_mem, w_theta, b_theta_ptr, theta_out, rows, d, 1);
-    clamp_f32_cuda(theta_out, rows, theta_floor, theta_ceil);
-    gate_compute_cuda(k_mem, v_mem, w_eta, b_eta_ptr, eta_out, rows, d, 0);
+    fused_prep<true>(k_mem, v_mem, q_mem, w_alpha, b_alpha_ptr, w_theta, b_theta_ptr, w_eta, b_eta_ptr, alpha_floor, alpha_ceil,
+                     theta_floor, theta_ceil, alpha_out, theta_out, eta_out, k_norms_out, q_norms_out, rows, d);
     if (es.failed()) return;
     titans_forward_f32_cuda(k_mem, v_mem, q_mem, alpha_out, theta_out, eta_out, m_initial, s_initial, m_states,
                             s_states, y, seq_len, d, batch_size, seq_len, d * d, error_clip, m_norm_max);
@@ -92,12 +145,8 @@ extern "C" void dgd_fused_forward_f32_cuda(float *k_mem, const float *v_mem, flo
         return;
     }
     const int rows = batch_size * seq_len;
-    l2_normalize_rows_f32_cuda(k_mem, k_norms_out, rows, d, 1e-8f);
-    l2_normalize_rows_f32_cuda(q_mem, q_norms_out, rows, d, 1e-8f);
-    gate_compute_cuda(k_mem, v_mem, w_alpha, b_alpha_ptr, alpha_out, rows, d, 0);
-    clamp_f32_cuda(alpha_out, rows, alpha_floor, alpha_ceil);
-    gate_compute_cuda(k_mem, v_mem, w_theta, b_theta_ptr, theta_out, rows, d, 1);
-    clamp_f32_cuda(theta_out, rows, theta_floor, theta_ceil);
+    fused_prep<false>(k_mem, v_mem, q_mem, w_alpha, b_alpha_ptr, w_theta, b_theta_ptr, nullptr, nullptr, alpha_floor, alpha_ceil,
+                      theta_floor, theta_ceil, alpha_out, theta_out, nullptr, k_norms_out, q_norms_out, rows, d);
     if (es.failed()) return;
     dgd_forward_f32_cuda(k_mem, v_mem, q_mem, alpha_out, theta_out, m_initial, m_states, y, seq_len, d, batch_size,
                          seq_len, d * d, error_clip);
