@@ -184,7 +184,9 @@ def cpu_baseline_hope(mems, x, dy, C, budget_s=12.0):
                       f"forward + backward, {el:.1f} s"}
 
 
-def setup_titans_exact_c2(torch, D, lib):
+def setup_titans_exact_c2(torch, D, lib, m_norm_max=None):
+    """m_norm_max: None = no bound (the largest float, as BASELINE configs[1] states it); a number = the bound the
+    reference's shipped configurations pass (cli/configs/gear1_d1024_gpu1.json:14 has 100)."""
     bs, heads, d, s, C = 8, 8, 64, 2048, 64
     B = bs * heads
     x = make_inputs(B, s, d, 0x5EED0002)
@@ -194,7 +196,7 @@ def setup_titans_exact_c2(torch, D, lib):
     mc, sc, y = z(B, n_ck, d, d), z(B, n_ck, d, d), z(B, s, d)
     g = dict(dk=z(B, s, d), dv=z(B, s, d), dq=z(B, s, d), da=z(B, s), dt=z(B, s), de=z(B, s),
              dm=z(d, d), ds=z(d, d))
-    F32_MAX = float(np.finfo(np.float32).max)
+    F32_MAX = float(np.finfo(np.float32).max) if m_norm_max is None else float(m_norm_max)
 
     def fwd():
         D.call("titans_forward_ckpt_batched_f32_rocm", dv["k"], dv["v"], dv["q"], dv["alpha"],
@@ -219,7 +221,8 @@ def setup_titans_exact_c2(torch, D, lib):
         kernel_names={"forward": "forward_ckpt", "backward": "backward_ckpt_fused"},
         cpu_all=lambda: cpu_all_cores(chain, B, s, heads, "full-trajectory forward + backward"),
         config={"workload": "BASELINE configs[1]: Titans LMM exact recurrence, 8 heads x 64 (d=512), "
-                            "batch 8, seq 2048, fp32 state, checkpoints every 64 tokens, fwd+bwd",
+                            "batch 8, seq 2048, fp32 state, checkpoints every 64 tokens, fwd+bwd" +
+                            ("" if m_norm_max is None else f", m_norm_max = {m_norm_max:g} (never reached)"),
                 "batch": bs, "heads": heads, "head_dim": d, "seq_len": s, "checkpoint_interval": C},
         cpu=lambda: cpu_baseline(x, heads))
 
@@ -605,7 +608,8 @@ WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2"
              "mag_layer_c5_bf16x3": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16x3"),
              "hbm_copy": None, "mfma_peak": None,
              "titans_chunkwise_c3_mnorm": lambda torch, D, lib: setup_titans_chunkwise_c3(torch, D, lib, mode="bf16_mnorm"),
-             "titans_chunkwise_c3_f32_mnorm": lambda torch, D, lib: setup_titans_chunkwise_c3(torch, D, lib, mode="f32_mnorm")}
+             "titans_chunkwise_c3_f32_mnorm": lambda torch, D, lib: setup_titans_chunkwise_c3(torch, D, lib, mode="f32_mnorm"),
+             "titans_exact_c2_mnorm": lambda torch, D, lib: setup_titans_exact_c2(torch, D, lib, m_norm_max=100.0)}
 
 
 # The kernel sources each workload's launches come from: a traffic profile is stamped with a hash of THESE files
@@ -618,6 +622,7 @@ WORKLOAD_SOURCES = {
     "titans_chunkwise_c3_mnorm": _CW_BF16 + ["chunkwise_guard.hip"],
     "titans_chunkwise_c3_f32_mnorm": ["chunkwise_mm.hip", "chunkwise_gates.hip", "chunkwise_guard.hip", "memory_rules.hip"],
     "titans_exact_c2": ["memory_rules.hip", "memory_rules_fused.hip"],
+    "titans_exact_c2_mnorm": ["memory_rules.hip", "memory_rules_fused.hip"],
     "hope_selfref_c4": ["selfref.hip"],
     "swa_c5": _SWA, "swa_stats_c5": _SWA,
     "adamw_c5": ["optim.hip", "cms.hip"],

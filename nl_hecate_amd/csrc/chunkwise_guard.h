@@ -18,4 +18,9 @@ bool couplings_may_fire_bf16(const uint16_t *k, const uint16_t *v, const float *
                              const float *m_states, const float *s_states, int seq_len, int batch, int chunk_size,
                              float error_clip, float m_norm_max);
 
+// For the exact rules and the sequential frozen-M0 kernels: msq_part [batch, parts] holds, per workgroup of a chain,
+// an upper bound of max_t of the sum of squares of its rows of M_t.  true: the bound (plus rounding slack) reaches
+// m_norm_max^2 for some chain, or the test could not run.  Same cost as above.
+bool norm_bound_exceeded(const float *msq_part, int batch, int parts, float m_norm_max);
+
 }  // namespace nlh

@@ -156,6 +156,34 @@ static bool couplings_may_fire_t(const TOK *k, const TOK *v, const float *alpha,
     return es.failed() || *g_host_flag != 0;
 }
 
+namespace {
+__global__ void norm_bound_kernel(const float *__restrict__ msq_part, int batch, int parts, float limit_sq, int *flag) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= batch) return;
+    float tot = 0.f;
+    for (int p = 0; p < parts; p++) tot += msq_part[b * parts + p];
+    if (!(tot * (1.0f + 1e-3f) <= limit_sq)) *flag = 1;   // also raised by a NaN
+}
+}  // namespace
+
+bool norm_bound_exceeded(const float *msq_part, int batch, int parts, float m_norm_max) {
+    const ErrorScope es;
+    int *flag = reinterpret_cast<int *>(scratch(31, 256));
+    if (!g_host_flag) check_hip(hipHostMalloc(reinterpret_cast<void **>(&g_host_flag), 256, hipHostMallocDefault), "hipHostMalloc");
+    if (es.failed() || !g_host_flag) return true;
+    {
+        KernelTimer kt("norm_bound_kernel");
+        hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(1), 0, stream(), flag);
+        hipLaunchKernelGGL(norm_bound_kernel, dim3((batch + 255) / 256), dim3(256), 0, stream(), msq_part, batch, parts,
+                           m_norm_max * m_norm_max, flag);
+        check_launch("norm_bound_kernel");
+    }
+    *g_host_flag = 1;
+    check_hip(hipMemcpyAsync(g_host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, stream()), "guard flag copy");
+    check_hip(hipStreamSynchronize(stream()), "guard flag sync");
+    return es.failed() || *g_host_flag != 0;
+}
+
 bool couplings_may_fire(const float *k, const float *v, const float *alpha, const float *theta, const float *eta,
                         const float *m_states, const float *s_states, int seq_len, int batch, int chunk_size,
                         float error_clip, float m_norm_max) {

@@ -34,6 +34,7 @@ constexpr int kPThr = 512;    // 8 waves
 constexpr int kMaxLevels = 8;
 constexpr int kMaxExtra = 4;
 constexpr int kSThr = 256;    // streaming kernels
+constexpr int kGThr = 768;    // the backward glue pass: 12 waves (three per SIMD at its 140 registers) share one partial row
 
 __device__ __forceinline__ float sigmoid_(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float softplus_(float x) { return x > 20.0f ? x : logf(1.0f + expf(x)); }
@@ -401,7 +402,7 @@ struct GradArgs {
 // forward wrote and the stored norms; d_v needs nothing), sums the gate gradients over the heads, applies the gate
 // activations' derivatives, and accumulates the gate projections' weight and bias gradients per wave in registers
 // (one partial row per workgroup, summed afterwards in a fixed order).  A lane owns 8 consecutive columns.
-__global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
+__global__ __launch_bounds__(kGThr) void level_grads_bf16_kernel(GradArgs a) {
     extern __shared__ float redg[];   // [3][2d + 1]
     const int lane = threadIdx.x & 63, wave_l = threadIdx.x >> 6, d = a.nh * 64, lvl = blockIdx.y, c0 = 8 * lane;
     const bool on = c0 < d;
@@ -421,37 +422,42 @@ __global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; e++) f[e] = (float)v[e];
     };
-    for (long long tok = wave; tok < n; tok += nwaves) {
+    // a wave owns a run of consecutive tokens: their gate gradients share cache lines (4 bytes per token and chain)
+    const long long per = (n + nwaves - 1) / nwaves, tok_hi = min(n, (wave + 1) * per);
+    for (long long tok = wave * per; tok < tok_hi; tok++) {
         const long long b = tok / a.s, t = tok - b * a.s;
+        // every load of the token first: one memory round trip per token and wave
+        u16 *grow = a.G + tok * a.g_ld + a.col0 + 3LL * lvl * d + c0;
+        bf16x8 rgk{}, rgq{}, rk{}, rq{}, rv{};
+        if (on) {
+            const size_t o = ((chain0 + b * a.nh + c0 / 64) * a.s + t) * 64 + c0 % 64;
+            rgk = *reinterpret_cast<const bf16x8 *>(grow);
+            rgq = *reinterpret_cast<const bf16x8 *>(grow + 2 * d);
+            rk = *reinterpret_cast<const bf16x8 *>(a.kh + o);
+            rq = *reinterpret_cast<const bf16x8 *>(a.qh + o);
+            rv = *reinterpret_cast<const bf16x8 *>(a.vh + o);
+        }
         float dg[3] = {0.f, 0.f, 0.f};
         for (int h = lane; h < a.nh; h += 64) {
             const size_t o = (chain0 + b * a.nh + h) * a.s + t;
             dg[0] += a.dah[o]; dg[1] += a.dth[o]; dg[2] += a.deh[o];
         }
+        const float al = a.alpha[lvl * n + tok], th = a.theta[lvl * n + tok], et = a.eta[lvl * n + tok];
+        const float kn = a.k_norms[lvl * n + tok], qn = a.q_norms[lvl * n + tok];
 #pragma unroll
         for (int gi = 0; gi < 3; gi++) dg[gi] = wave_allreduce(dg[gi]);
-        {
-            const float al = a.alpha[lvl * n + tok], th = a.theta[lvl * n + tok], e = a.eta[lvl * n + tok];
-            dg[0] *= al * (1.0f - al);
-            dg[1] *= 1.0f - expf(-th);
-            dg[2] *= e * (1.0f - e);
-        }
+        dg[0] *= al * (1.0f - al);
+        dg[1] *= 1.0f - expf(-th);
+        dg[2] *= et * (1.0f - et);
 #pragma unroll
         for (int gi = 0; gi < 3; gi++) accb[gi] += dg[gi];
-        const float kn = a.k_norms[lvl * n + tok], qn = a.q_norms[lvl * n + tok];
         const float ki = 1.0f / fmaxf(kn, a.eps), qi = 1.0f / fmaxf(qn, a.eps);
-        u16 *grow = a.G + tok * a.g_ld + a.col0 + 3LL * lvl * d + c0;
         float gk[8], gq[8], kk[8], qq[8], vv[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) gk[e] = gq[e] = kk[e] = qq[e] = vv[e] = 0.f;
-        if (on) {
-            const size_t o = ((chain0 + b * a.nh + c0 / 64) * a.s + t) * 64 + c0 % 64;
-            widen(*reinterpret_cast<const bf16x8 *>(grow), gk);
-            widen(*reinterpret_cast<const bf16x8 *>(grow + 2 * d), gq);
-            widen(*reinterpret_cast<const bf16x8 *>(a.kh + o), kk);
-            widen(*reinterpret_cast<const bf16x8 *>(a.qh + o), qq);
-            widen(*reinterpret_cast<const bf16x8 *>(a.vh + o), vv);
-        }
+        widen(rgk, gk);
+        widen(rgq, gq);
+        widen(rk, kk);
+        widen(rq, qq);
+        widen(rv, vv);
         float dk_dot = 0.f, dq_dot = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -478,7 +484,7 @@ __global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
     }
     // the workgroup's partial row: the waves add their sums into LDS one after the other (fixed order)
     const int stride = 2 * d + 1;
-    for (int w = 0; w < kSThr / 64; w++) {
+    for (int w = 0; w < kGThr / 64; w++) {
         if (wave_l == w) {
 #pragma unroll
             for (int gi = 0; gi < 3; gi++) {
@@ -501,7 +507,7 @@ __global__ __launch_bounds__(kSThr) void level_grads_bf16_kernel(GradArgs a) {
         __syncthreads();
     }
     float *pb = a.part + ((size_t)lvl * gridDim.x + blockIdx.x) * 3 * stride;
-    for (int i = threadIdx.x; i < 3 * stride; i += kSThr) pb[i] = redg[i];
+    for (int i = threadIdx.x; i < 3 * stride; i += kGThr) pb[i] = redg[i];
 }
 
 struct GateGradOuts { GateGradOut lv[kMaxLevels]; };
@@ -808,7 +814,7 @@ void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_ext
     float *hg = scratch(25, (3 * gate_f + 4) * sizeof(float));                  // d_alpha, d_theta, d_eta per chain and token
     u16 *G = reinterpret_cast<u16 *>(scratch(26, (size_t)n * R * sizeof(u16)));
     u16 *wb = reinterpret_cast<u16 *>(scratch(27, (size_t)R * d * sizeof(u16)));
-    const int nblk = stream_blocks(n * 64, 256);
+    const int nblk = (int)std::min<long long>(compute_units(), (n * 64 + kGThr - 1) / kGThr);
     const size_t prow = 3 * (2 * (size_t)d + 1);
     float *part = scratch(28, (size_t)(levels ? levels : 1) * nblk * prow * sizeof(float));
     if (es.failed()) return;
@@ -833,7 +839,7 @@ void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_ext
         ga.bs = bs; ga.s = seq_len; ga.nh = heads; ga.levels = levels; ga.eps = eps;
         {
             KernelTimer kt("level_grads_bf16_kernel");
-            hipLaunchKernelGGL(level_grads_bf16_kernel, dim3(nblk, levels), dim3(kSThr), prow * sizeof(float), stream(), ga);
+            hipLaunchKernelGGL(level_grads_bf16_kernel, dim3(nblk, levels), dim3(kGThr), prow * sizeof(float), stream(), ga);
             check_launch("level_grads_bf16_kernel");
         }
         GateGradOuts go{};

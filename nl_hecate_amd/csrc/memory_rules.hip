@@ -41,8 +41,11 @@ static __global__ void zero_fill_kernel(float *__restrict__ p, size_t n) {
 // FROZEN: the frozen-M0 chunkwise rule (core/kernels/titans_chunkwise_forward.cu):
 // errors of a chunk are taken against the chunk-start M; ckpt_interval is the
 // chunk size and the stored checkpoints are the chunk-boundary states.
-template <int D, int RPL, bool HAS_S, int STORE, bool COUPLED, bool FROZEN>
+// MODE: 0 rows split over workgroups, 1 COUPLED (clip / projection: a chain in one workgroup), 2 as 0 and keeps the
+// bound of max_t |M_t|_F^2 that FwdArgs::msq_part describes.
+template <int D, int RPL, bool HAS_S, int STORE, int MODE, bool FROZEN>
 __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
+    constexpr bool COUPLED = MODE == 1, TRACK = MODE == 2;
     constexpr int LPR = D / 4;          // lanes per row
     constexpr int RG = 64 / LPR;        // row groups per wave
     constexpr int ROWS_WG = kWaves * RG * RPL;
@@ -101,6 +104,7 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
     const int ntiles = (seq_len + TB - 1) / TB;
     const bool clip_on = COUPLED && a.error_clip > 0.f;
     const bool mn_on = COUPLED && mnorm_active(a.m_norm_max);
+    float nmax = 0.f;
 
     TileRegs<D, TB> rk, rq, rv;
     GateRegs<TB> rg;
@@ -187,6 +191,12 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
                         for (int r = 0; r < RPL; r++) M[r] = f4_scale(sc, M[r]);
                     }
                 }
+                if (TRACK) {
+                    float sq_sum = 0.f;
+#pragma unroll
+                    for (int r = 0; r < RPL; r++) sq_sum += dot4(M[r], M[r]);
+                    nmax = fmaxf(nmax, sq_sum);
+                }
                 if (STORE == STORE_TRAJ) {
 #pragma unroll
                     for (int r = 0; r < RPL; r++)
@@ -231,6 +241,10 @@ __global__ __launch_bounds__(kThreads) void rule_fwd_kernel(FwdArgs a) {
     }
     __syncthreads();
     if (ntiles > 0) flush_y(ntiles - 1);
+    if (TRACK) {
+        const float tot = block_allreduce(nmax, sred[0], tid);
+        if (tid == 0) a.msq_part[chain * a.parts + part] = tot;
+    }
 }
 
 // ───────────────────────────── backward ────────────────────────────────────
@@ -585,9 +599,11 @@ static void launch_fwd_c(const FwdArgs &a, int batch, bool coupled) {
     dim3 grid(batch * a.parts), block(kThreads);
     KernelTimer kt("rule_fwd_kernel");
     if (coupled)
-        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, true, FROZEN>), grid, block, 0, stream(), a);
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, 1, FROZEN>), grid, block, 0, stream(), a);
+    else if (a.msq_part)
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, 2, FROZEN>), grid, block, 0, stream(), a);
     else
-        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, false, FROZEN>), grid, block, 0, stream(), a);
+        hipLaunchKernelGGL((rule_fwd_kernel<D, RPL, HAS_S, STORE, 0, FROZEN>), grid, block, 0, stream(), a);
     check_launch("rule_fwd_kernel");
 }
 
@@ -596,10 +612,9 @@ static bool tiled_size(int d) { return d == 8 || d == 16 || d == 32 || d == 64 |
 
 // Always launches (returns true) for d >= 1: head sizes without a tiled kernel, and clip / projection
 // where the tiled layout would split a chain over workgroups (d = 128), take the general kernels.
-template <bool HAS_S, int STORE, bool FROZEN = false>
-static bool launch_fwd(FwdArgs a, int d, int batch) {
+template <bool HAS_S, int STORE, bool FROZEN>
+static bool launch_fwd_as(FwdArgs a, int d, int batch, bool coupled) {
     if (d < 1) return false;
-    const bool coupled = coupled_needed(a.error_clip, a.m_norm_max);
     const int rpl = tiled_size(d) ? pick_rpl(d, batch, coupled) : 1;
     a.parts = tiled_size(d) ? ceil_div(d, rows_per_wg(d, rpl)) : 1;
     if (!tiled_size(d) || (coupled && a.parts != 1)) {
@@ -619,6 +634,27 @@ static bool launch_fwd(FwdArgs a, int d, int batch) {
         case 128: launch_fwd_c<128, 4, HAS_S, STORE, FROZEN>(a, batch, false); return true;
         default: return false;
     }
+}
+
+// The Frobenius projection couples the rows of a chain only at the tokens where it fires.  With a bound and no
+// error clip, the uncoupled kernels run first and keep an upper bound of max_t |M_t|_F^2 per workgroup; when the
+// bound stays below m_norm_max^2 no projection could have fired and their results are the coupled kernels' (one
+// 4-byte read-back and a stream synchronisation decide); otherwise the coupled kernels run and overwrite everything.
+template <bool HAS_S, int STORE, bool FROZEN = false>
+static bool launch_fwd(FwdArgs a, int d, int batch) {
+    const bool coupled = coupled_needed(a.error_clip, a.m_norm_max);
+    if (coupled && a.error_clip <= 0.f && tiled_size(d) && guard_possible()) {
+        const ErrorScope es;
+        FwdArgs u = a;
+        const int rpl = pick_rpl(d, batch, false), parts = ceil_div(d, rows_per_wg(d, rpl));
+        u.msq_part = scratch(23, (size_t)batch * parts * sizeof(float));
+        if (es.failed()) return true;
+        launch_fwd_as<HAS_S, STORE, FROZEN>(u, d, batch, false);
+        if (es.failed()) return true;
+        if (!norm_bound_exceeded(u.msq_part, batch, parts, a.m_norm_max)) return true;
+    }
+    a.msq_part = nullptr;
+    return launch_fwd_as<HAS_S, STORE, FROZEN>(a, d, batch, coupled);
 }
 
 template <int D, int RPL, bool HAS_S, bool FROZEN>
@@ -809,9 +845,13 @@ static void backward_ckpt_any(bool has_s, bool frozen, bool allow_fused,
                               float error_clip, float m_norm_max, const char *fn) {
     if (!check_dims(fn, seq_len, d, batch) || batch == 0 || seq_len == 0) return;
     if (C <= 0) { fail("%s: interval/chunk size %d must be > 0.", fn, C); return; }
-    if (allow_fused && !coupled_needed(error_clip, m_norm_max) &&
+    // no clip: the fused kernel replays without the projection; with a bound it checks afterwards that none could
+    // have fired (see launch_fwd) and otherwise leaves the call to the replay schedule below
+    const bool bound = coupled_needed(0.f, m_norm_max);
+    if (allow_fused && error_clip <= 0.f && (!bound || guard_possible()) &&
         backward_ckpt_fused(has_s, frozen, k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v,
-                            d_q, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d, batch, C))
+                            d_q, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d, batch, C,
+                            bound ? m_norm_max : 0.f))
         return;
 #define NLH_REPLAY(HS, FZ)                                                                         \
     backward_ckpt_replay<HS, FZ>(k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v, d_q,  \

@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "../../include/nl_hecate_ffi.h"
+#include "chunkwise_guard.h"
 #include "rule_common.h"
 
 namespace nlh {
@@ -41,11 +42,13 @@ struct FusedArgs {
     float *ws_dq, *ws_dk, *ws_gate;   // partial sums when parts > 1
     float *d_m_out, *d_s_out;         // [B, dd]
     int seq_len, C, n_ckpt, parts, batch;
+    float *msq_part;   // may be null: [batch * parts] upper bounds of max_t sum(M_t^2) over the replayed states (FwdArgs)
 };
 
 // FROZEN: frozen-M0 chunkwise rule, segment = chunk
 // (core/kernels/titans_chunkwise_backward.cu:118-358).
-template <int D, bool HAS_S, bool FROZEN>
+// TRACK: keep the bound of max_t |M_t|_F^2 over the replayed states (FusedArgs::msq_part)
+template <int D, bool HAS_S, bool FROZEN, bool TRACK>
 __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
     constexpr int LPR = D / 4;
     constexpr int RG = 64 / LPR;
@@ -88,6 +91,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
     float4 dM = f4_zero(), dS = f4_zero();
     float4 M = f4_zero(), S = f4_zero();
     float4 M0f = f4_zero(), dM0 = f4_zero();  // FROZEN: chunk-start M and its gradient
+    float nmax = 0.f;
 
     // ── work items: (segment, phase, block) in processing order ──
     const int nseg = (seq_len + C - 1) / C;
@@ -206,6 +210,7 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
                 } else {
                     M = f4_axpby(1.f - al, M, -te, kk);
                 }
+                if (TRACK) nmax = fmaxf(nmax, dot4(M, M));
             }
         };
         auto level2 = [&](auto full_c) {
@@ -333,13 +338,20 @@ __global__ __launch_bounds__(kThreads) void rule_bwd_fused_kernel(FusedArgs a) {
         *reinterpret_cast<float4 *>(a.d_m_out + (size_t)chain * DD + roff) = dM;
         if (HAS_S) *reinterpret_cast<float4 *>(a.d_s_out + (size_t)chain * DD + roff) = dS;
     }
+    if (TRACK) {
+        __syncthreads();   // the flush above was the last reader of the staging buffers
+        const float tot = block_allreduce(nmax, tg[0], tid);
+        if (tid == 0) a.msq_part[chain * a.parts + part] = tot;
+    }
 }
 
 template <int D, bool HAS_S, bool FROZEN>
 static void launch_fused_d(const FusedArgs &a) {
     KernelTimer kt("rule_bwd_fused_kernel");
-    hipLaunchKernelGGL((rule_bwd_fused_kernel<D, HAS_S, FROZEN>), dim3(a.batch * a.parts),
-                       dim3(kThreads), 0, stream(), a);
+    if (a.msq_part)
+        hipLaunchKernelGGL((rule_bwd_fused_kernel<D, HAS_S, FROZEN, true>), dim3(a.batch * a.parts), dim3(kThreads), 0, stream(), a);
+    else
+        hipLaunchKernelGGL((rule_bwd_fused_kernel<D, HAS_S, FROZEN, false>), dim3(a.batch * a.parts), dim3(kThreads), 0, stream(), a);
     check_launch("rule_bwd_fused_kernel");
 }
 
@@ -350,7 +362,7 @@ static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q
                                   float *d_k, float *d_v, float *d_q,
                                   float *d_alpha, float *d_theta, float *d_eta,
                                   float *d_m_initial, float *d_s_initial,
-                                  int seq_len, int d, int batch, int C) {
+                                  int seq_len, int d, int batch, int C, float m_norm_guard) {
     const ErrorScope es;
     if (C > C_MAX) return false;
     if (d != 8 && d != 16 && d != 32 && d != 64 && d != 128) return false;
@@ -358,7 +370,8 @@ static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q
     const int rows_wg = kWaves * (64 / (d / 4));
     FusedArgs a{k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v, d_q, d_alpha, d_theta, d_eta,
                 nullptr, nullptr, nullptr, nullptr, nullptr,
-                seq_len, C, n_ckpt_count(seq_len, C), ceil_div(d, rows_wg), batch};
+                seq_len, C, n_ckpt_count(seq_len, C), ceil_div(d, rows_wg), batch, nullptr};
+    if (m_norm_guard > 0.f) a.msq_part = scratch(23, (size_t)batch * a.parts * sizeof(float));
     a.d_m_out = scratch(0, (size_t)batch * dd * sizeof(float));
     if (HAS_S) a.d_s_out = scratch(1, (size_t)batch * dd * sizeof(float));
     if (a.parts > 1) {
@@ -378,6 +391,8 @@ static bool backward_ckpt_fused_t(const float *k, const float *v, const float *q
     if (a.parts > 1)
         finalize_parts(a.ws_dq, a.ws_dk, a.ws_gate, d_q, d_k, d_alpha, d_theta,
                        HAS_S ? d_eta : nullptr, a.parts, batch, seq_len, d, 0, seq_len);
+    if (es.failed()) return true;
+    if (a.msq_part && norm_bound_exceeded(a.msq_part, batch, a.parts, m_norm_guard)) return false;
     accumulate_over_batch2(a.d_m_out, d_m_initial, HAS_S ? a.d_s_out : nullptr, d_s_initial, batch, (int)dd);
     return true;
 }
@@ -388,11 +403,11 @@ bool backward_ckpt_fused(bool has_s, bool frozen, const float *k, const float *v
                          float *d_k, float *d_v, float *d_q,
                          float *d_alpha, float *d_theta, float *d_eta,
                          float *d_m_initial, float *d_s_initial,
-                         int seq_len, int d, int batch, int C) {
+                         int seq_len, int d, int batch, int C, float m_norm_guard) {
 #define NLH_FUSED(HS, FZ)                                                                        \
     return backward_ckpt_fused_t<HS, FZ>(k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k,  \
                                          d_v, d_q, d_alpha, d_theta, d_eta, d_m_initial,        \
-                                         d_s_initial, seq_len, d, batch, C)
+                                         d_s_initial, seq_len, d, batch, C, m_norm_guard)
     if (has_s) { if (frozen) NLH_FUSED(true, true); else NLH_FUSED(true, false); }
     if (frozen) NLH_FUSED(false, true);
     NLH_FUSED(false, false);

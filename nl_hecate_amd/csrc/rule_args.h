@@ -12,6 +12,9 @@ struct FwdArgs {
     long long m_stride;      // elements between chains in m_initial / s_initial
     long long state_stride;  // elements between chains in m_out / s_out
     float error_clip, m_norm_max;
+    // uncoupled kernels only, may be null: [batch * parts] upper bounds of max_t sum(M_t^2) over the workgroup's rows
+    // (every lane keeps the largest sum of squares its own elements reached; the lanes' maxima are added up)
+    float *msq_part;
 };
 
 enum { STORE_NONE = 0, STORE_TRAJ = 1, STORE_CKPT = 2 };

@@ -67,13 +67,14 @@ void finalize_parts(const float *ws_dq, const float *ws_dk, const float *ws_gate
 
 // Checkpointed / chunkwise backward over all segments in one call.
 // has_s: Titans (momentum) vs Delta; frozen: frozen-M0 chunkwise rule.
-// The fused form returns false when it does not cover (d, C).
+// The fused form returns false when it does not cover (d, C), and, given a bound (m_norm_guard > 0), when the
+// replayed states may have reached it (nothing has been added to d_m_initial / d_s_initial then).
 bool backward_ckpt_fused(bool has_s, bool frozen, const float *k, const float *v, const float *q,
                          const float *alpha, const float *theta, const float *eta,
                          const float *m_ckpt, const float *s_ckpt, const float *d_y,
                          float *d_k, float *d_v, float *d_q,
                          float *d_alpha, float *d_theta, float *d_eta,
                          float *d_m_initial, float *d_s_initial,
-                         int seq_len, int d, int batch, int C);
+                         int seq_len, int d, int batch, int C, float m_norm_guard = 0.f);
 
 }  // namespace nlh

@@ -1,0 +1,167 @@
+"""The exact rules and the sequential frozen-M0 kernels under a finite m_norm_max (the reference's shipped
+configurations pass 100: cli/configs/gear1_d1024_gpu1.json:14; core/kernels/m_norm_project.cuh).  The projection
+couples the rows of a chain only where it fires, so the row-split kernels run first and keep an upper bound of
+max_t |M_t|_F^2; the coupled kernels (a chain in one workgroup, a reduction per token) run only when that bound
+reaches the limit.  Every case is checked against the oracle's token loops WITH the projection, and the kernel
+timers say which kernels ran."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from nl_hecate_amd import dispatch as D
+from nl_hecate_amd.ffi import lib
+from oracle import pyoracle as orc
+from tests.gpu_util import assert_close, dev, host, rule_inputs, zeros
+
+pytestmark = pytest.mark.gpu
+F32_MAX = float(np.finfo(np.float32).max)
+
+
+def kernels_run(fn):
+    lib.nlh_kernel_timer_enable(1)
+    buf = ctypes.create_string_buffer(8192)
+    lib.nlh_kernel_timer_report(buf, len(buf))
+    fn()
+    torch.cuda.synchronize()
+    assert lib.nlh_kernel_timer_report(buf, len(buf)) >= 0
+    lib.nlh_kernel_timer_enable(0)
+    return {item.rsplit(":", 2)[0] for item in buf.value.decode().split(";") if item}
+
+
+def worst_norm(x):
+    """largest |M_t|_F over the exact trajectory without the projection"""
+    worst = 0.0
+    for b in range(x["k"].shape[0]):
+        M, S = x["m0"][b].astype(np.float64), x["s0"][b].astype(np.float64)
+        for t in range(x["k"].shape[1]):
+            e = M @ x["k"][b, t] - x["v"][b, t]
+            S = x["eta"][b, t] * S - x["theta"][b, t] * np.outer(e, x["k"][b, t])
+            M = (1 - x["alpha"][b, t]) * M + S
+            worst = max(worst, float(np.linalg.norm(M)))
+    return worst
+
+
+def run_ckpt_pair(x, C, mmax):
+    B, s, d = x["k"].shape
+    n_ck = orc.checkpoint_count(s, C)
+    t = {n: dev(a) for n, a in x.items()}
+    mc, sc, y = zeros(B, n_ck, d * d), zeros(B, n_ck, d * d), zeros(B, s, d)
+    ran_f = kernels_run(lambda: D.call("titans_forward_ckpt_batched_f32_rocm", t["k"], t["v"], t["q"], t["alpha"], t["theta"],
+                                       t["eta"], t["m0"], t["s0"], mc, sc, y, s, d, B, C, 0.0, mmax))
+    g = {n: zeros(B, s, d) for n in ("d_k", "d_v", "d_q")}
+    g.update({n: zeros(B, s) for n in ("d_alpha", "d_theta", "d_eta")})
+    dm, ds = zeros(d, d), zeros(d, d)
+    ran_b = kernels_run(lambda: D.call("titans_backward_ckpt_f32_rocm", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"],
+                                       mc, sc, t["dy"], g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"],
+                                       dm, ds, s, d, B, C, 0.0, mmax))
+    return host(y), host(mc), {n: host(a) for n, a in g.items()}, host(dm), host(ds), ran_f, ran_b
+
+
+def check_ckpt_pair(x, C, mmax, got, tol=1e-4):
+    y, mc, g, dm, ds = got[:5]
+    B = x["k"].shape[0]
+    ys, mcs, gs = [], [], []
+    for b in range(B):
+        yo, mco, sco = orc.forward_ckpt(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], x["m0"][b],
+                                        x["s0"][b], C, m_norm_max=mmax)
+        gs.append(orc.backward_ckpt(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], mco, sco,
+                                    x["dy"][b], C, m_norm_max=mmax))
+        ys.append(yo); mcs.append(mco)
+    assert_close("y", y, np.stack(ys), tol)
+    assert_close("m_ckpt", mc.reshape(np.stack(mcs).shape), np.stack(mcs), tol)
+    for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta", "d_eta"):
+        assert_close(n, g[n], np.stack([gi[n] for gi in gs]), tol)
+    assert_close("d_m_initial", dm, sum(gi["d_m"] for gi in gs), tol)
+    assert_close("d_s_initial", ds, sum(gi["d_s"] for gi in gs), tol)
+
+
+@pytest.mark.parametrize("B,s,d,C", [(6, 200, 64, 64), (3, 96, 32, 32), (130, 70, 64, 16)])
+def test_bound_never_reached_keeps_the_row_split_kernels(B, s, d, C):
+    x = rule_inputs(B, s, d, seed=61, m0_scale=0.02)
+    assert worst_norm({n: a[:4] for n, a in x.items()}) < 50.0
+    got = run_ckpt_pair(x, C, 100.0)
+    check_ckpt_pair(x, C, 100.0, got)
+    ran_f, ran_b = got[5], got[6]
+    assert "norm_bound_kernel" in ran_f, ran_f
+    assert "rule_bwd_fused_kernel" in ran_b and "norm_bound_kernel" in ran_b, ran_b
+    assert not any(n.startswith("rule_bwd_traj") or n == "rule_fwd_kernel" for n in ran_b), ran_b   # no replay schedule
+
+
+def test_bound_that_is_reached_takes_the_coupled_kernels_and_adds_the_initial_state_gradients_once():
+    B, s, d, C = 5, 160, 64, 64
+    x = rule_inputs(B, s, d, seed=67, m0_scale=0.02)
+    mmax = 0.6 * worst_norm(x)
+    free = [orc.forward_ckpt(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], x["m0"][b], x["s0"][b],
+                             C)[0] for b in range(B)]
+    proj = [orc.forward_ckpt(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], x["m0"][b], x["s0"][b],
+                             C, m_norm_max=mmax)[0] for b in range(B)]
+    assert np.abs(np.stack(free) - np.stack(proj)).max() > 1e-3, "the projection must change the result for this case to mean anything"
+    got = run_ckpt_pair(x, C, mmax)
+    check_ckpt_pair(x, C, mmax, got)
+    assert "norm_bound_kernel" in got[5] and "norm_bound_kernel" in got[6]
+
+
+def test_bound_between_the_true_maximum_and_the_estimate_is_still_exact():
+    """The estimate adds up every lane's own maximum over time, which can exceed the largest norm of any one token:
+    a bound just above the trajectory may cost the coupled kernels, never a wrong result."""
+    B, s, d, C = 3, 128, 64, 64
+    x = rule_inputs(B, s, d, seed=71, m0_scale=0.02)
+    mmax = 1.02 * worst_norm(x)
+    got = run_ckpt_pair(x, C, mmax)
+    check_ckpt_pair(x, C, mmax, got)
+
+
+@pytest.mark.parametrize("scale", [None, 0.6])
+def test_full_trajectory_forward(scale):
+    B, s, d = 4, 90, 64
+    x = rule_inputs(B, s, d, seed=73, m0_scale=0.02)
+    mmax = 100.0 if scale is None else scale * worst_norm(x)
+    t = {n: dev(a) for n, a in x.items()}
+    ms, ss, y = zeros(B, s + 1, d * d), zeros(B, s + 1, d * d), zeros(B, s, d)
+    ran = kernels_run(lambda: D.call("titans_forward_f32_cuda", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"], t["m0"],
+                                     t["s0"], ms, ss, y, s, d, B, s, d * d, 0.0, mmax))
+    assert "norm_bound_kernel" in ran, ran
+    for b in range(B):
+        yo, mo, so = orc.titans_forward(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], x["m0"][b],
+                                        x["s0"][b], m_norm_max=mmax)
+        assert_close("y", host(y)[b], yo, 1e-4)
+        assert_close("m_states", host(ms)[b].reshape(mo.shape), mo, 1e-4)
+        assert_close("s_states", host(ss)[b].reshape(so.shape), so, 1e-4)
+
+
+@pytest.mark.parametrize("scale", [None, 0.6])
+def test_sequential_frozen_kernels_at_head_size_32(scale):
+    """d = 32 has no matrix form: the chunkwise symbols run the sequential frozen-M0 kernels, row-split when the bound
+    allows it."""
+    B, s, d, C = 6, 100, 32, 16
+    x = rule_inputs(B, s, d, seed=79, m0_scale=0.02)
+    nc = (s + C - 1) // C
+    worst = 0.0
+    for b in range(B):
+        _, mco, _ = orc.chunkwise_forward(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], x["m0"][b],
+                                          x["s0"][b], C)
+        worst = max(worst, max(float(np.linalg.norm(m)) for m in mco))
+    mmax = 100.0 if scale is None else scale * worst
+    t = {n: dev(a) for n, a in x.items()}
+    mc, sc, y = zeros(B, nc + 1, d * d), zeros(B, nc + 1, d * d), zeros(B, s, d)
+    ran_f = kernels_run(lambda: D.call("titans_chunkwise_forward_f32_cuda", t["k"], t["v"], t["q"], t["alpha"], t["theta"],
+                                       t["eta"], t["m0"], t["s0"], mc, sc, y, s, d, B, C, 0.0, mmax))
+    g = {n: zeros(B, s, d) for n in ("d_k", "d_v", "d_q")}
+    g.update({n: zeros(B, s) for n in ("d_alpha", "d_theta", "d_eta")})
+    dm, ds = zeros(d, d), zeros(d, d)
+    D.call("titans_chunkwise_backward_f32_cuda", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"], mc, sc, t["dy"],
+           g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], dm, ds, s, d, B, C, 0.0, mmax)
+    assert "norm_bound_kernel" in ran_f, ran_f
+    gos = []
+    for b in range(B):
+        yo, mco, sco = orc.chunkwise_forward(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b],
+                                             x["m0"][b], x["s0"][b], C, m_norm_max=mmax)
+        assert_close("y", host(y)[b], yo, 1e-4)
+        assert_close("m_chunk_states", host(mc)[b].reshape(mco.shape), mco, 1e-4)
+        gos.append(orc.chunkwise_backward(x["k"][b], x["v"][b], x["q"][b], x["alpha"][b], x["theta"][b], x["eta"][b], mco, sco,
+                                          x["dy"][b], C, m_norm_max=mmax))
+    for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta", "d_eta"):
+        assert_close(n, host(g[n]), np.stack([gi[n] for gi in gos]), 1e-4)
+    assert_close("d_m_initial", host(dm), sum(gi["d_m"] for gi in gos), 1e-4)
