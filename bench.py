@@ -317,8 +317,8 @@ def cpu_baseline_swa(q, k, v, d_out, window, heads, budget_s=12.0):
                       f"filled, so this overstates the CPU rate), forward + backward, {el:.1f} s"}
 
 
-def setup_swa_c5(torch, D, lib, lse=False):
-    bs, heads, hd, s, window = 8, 8, 64, 4096, 512
+def setup_swa_c5(torch, D, lib, lse=False, heads=8, hd=64):
+    bs, s, window = 8, 4096, 512
     td = heads * hd
     g = torch.Generator(device="cpu").manual_seed(0x5EED0005)
     q, k, v = (torch.randn(bs, s, td, generator=g).to(torch.bfloat16) for _ in range(3))
@@ -347,11 +347,11 @@ def setup_swa_c5(torch, D, lib, lse=False):
     wbytes = 8 if lse else 1024
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=bs * heads * s, bound="hbm", dtype="bf16",
-        flop_fwd=FLOP_SWA_FWD, flop_bwd=FLOP_SWA_BWD + (FLOP_SWA_FWD if lse else 0),
-        bytes_fwd=BYTES_SWA_FWD - 1024 + wbytes, bytes_bwd=BYTES_SWA_BWD - 1024 + wbytes,
+        flop_fwd=4 * window * hd, flop_bwd=10 * window * hd + (4 * window * hd if lse else 0),
+        bytes_fwd=4 * 2 * hd + wbytes, bytes_bwd=3 * 2 * hd + wbytes + 4 * 4 * hd,
         matrix="bf16_matrix", matrix_peak=PEAK_BF16_TFLOPS,
         kernel_names={"forward": "swa_forward", "backward": "swa_backward"},
-        config={"workload": "BASELINE configs[4], attention branch: sliding-window attention, window 512, 8 heads x 64, "
+        config={"workload": f"BASELINE configs[4], attention branch: sliding-window attention, window 512, {heads} heads x {hd}, "
                             "bf16 storage with fp32 softmax, batch 8, seq 4096, fwd+bwd"
                             + (", per-query softmax statistics kept instead of the weight tensor" if lse else ""),
                 "batch": bs, "heads": heads, "head_dim": hd, "seq_len": s, "window": window},
@@ -603,6 +603,8 @@ def setup_hebbian_c2(torch, D, lib):
 WORKLOADS = {"titans_chunkwise_c3": setup_titans_chunkwise_c3, "titans_exact_c2": setup_titans_exact_c2,
              "hope_selfref_c4": setup_hope_selfref_c4, "swa_c5": setup_swa_c5,
              "swa_stats_c5": lambda torch, D, lib: setup_swa_c5(torch, D, lib, lse=True),
+             "swa_c5_hd32": lambda torch, D, lib: setup_swa_c5(torch, D, lib, heads=16, hd=32),
+             "swa_stats_c5_hd32": lambda torch, D, lib: setup_swa_c5(torch, D, lib, lse=True, heads=16, hd=32),
              "adamw_c5": setup_adamw_c5, "hebbian_c2": setup_hebbian_c2,
              "mag_layer_c5": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16"),
              "mag_layer_c5_bf16x3": lambda torch, D, lib: setup_mag_layer_c5(torch, D, lib, precision="bf16x3"),
@@ -624,7 +626,7 @@ WORKLOAD_SOURCES = {
     "titans_exact_c2": ["memory_rules.hip", "memory_rules_fused.hip"],
     "titans_exact_c2_mnorm": ["memory_rules.hip", "memory_rules_fused.hip"],
     "hope_selfref_c4": ["selfref.hip"],
-    "swa_c5": _SWA, "swa_stats_c5": _SWA,
+    "swa_c5": _SWA, "swa_stats_c5": _SWA, "swa_c5_hd32": _SWA, "swa_stats_c5_hd32": _SWA,
     "adamw_c5": ["optim.hip", "cms.hip"],
     "hebbian_c2": ["hebbian.hip"],
     "mag_layer_c5": _CW_BF16 + _SWA + ["level_step.hip", "layer_glue.hip", "cms.hip", "optim.hip"],

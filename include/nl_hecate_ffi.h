@@ -379,7 +379,7 @@ void swa_backward_f32_cuda(const uint16_t *q, const uint16_t *k, const uint16_t 
  * stored): the same attention with the weight tensor left out.  The forward stores per query only
  * stats [batch, heads, seq, 2] fp32 = (max_j score * log2(e) / sqrt(hd), 1 / sum_j exp(...)); the backward rebuilds
  * each weight from q . k and those two numbers, rounded to bf16 as the stored tensor would hold it.
- * head_dim 64, window_size <= 512, no persistent prefix; other shapes are an error.  out, d_q, d_k, d_v as in
+ * head_dim 64 or 32, window_size <= 512, no persistent prefix; other shapes are an error.  out, d_q, d_k, d_v as in
  * the pair above (d_k, d_v accumulated). */
 void swa_forward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, float *stats,
                                int seq_len, int num_heads, int head_dim, int window_size, int batch_size);

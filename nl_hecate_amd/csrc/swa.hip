@@ -373,7 +373,7 @@ void swa_forward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint1
     if (!swa_check("swa_forward_lse_bf16_rocm", seq_len, num_heads, head_dim, window_size, batch_size, 0)) return;
     if (!stats) return fail("swa_forward_lse_bf16_rocm: stats is null");
     if (!swa_forward_mfma(q, k, v, out, nullptr, seq_len, num_heads, head_dim, window_size, batch_size, 0, stats))
-        fail("swa_forward_lse_bf16_rocm: needs head_dim 64 and window_size <= 512");
+        fail("swa_forward_lse_bf16_rocm: needs head_dim 64 or 32 and window_size <= 512");
 }
 
 void swa_backward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, const float *stats,
@@ -384,7 +384,7 @@ void swa_backward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint
     if (!stats) return fail("swa_backward_lse_bf16_rocm: stats is null");
     if (!swa_backward_mfma(q, k, v, nullptr, d_attn_out, d_q, d_k, d_v, seq_len, num_heads, head_dim, window_size,
                            batch_size, 0, stats))
-        fail("swa_backward_lse_bf16_rocm: needs head_dim 64 and window_size <= 512");
+        fail("swa_backward_lse_bf16_rocm: needs head_dim 64 or 32 and window_size <= 512");
 }
 
 void swa_single_token_cuda(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,

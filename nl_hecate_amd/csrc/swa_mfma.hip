@@ -1,5 +1,5 @@
-// Sliding-window attention on the bf16 matrix cores for head size 64, no
-// persistent prefix, window <= 512 (the production shape).  Contract and mask
+// Sliding-window attention on the bf16 matrix cores for head sizes 64 and 32, no
+// persistent prefix, window <= 512 (the production shapes).  Contract and mask
 // are those of core/kernels/swa_forward.cu / swa_backward.cu; other shapes stay
 // on the wave-per-query kernels of swa.hip.
 //
@@ -34,7 +34,8 @@ typedef __bf16 bh8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bh2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int HD = 64;        // head size
+// The kernels are templates on the head size HDV (64 or 32): NKS = HDV / 32 contraction steps over the dims, NDT = HDV / 16
+// output tiles of dims; the LDS stages keep 64-wide rows either way.
 constexpr int KS = 64;        // keys per LDS stage
 constexpr int LDH = 72;       // LDS row stride in bf16 elements (144 B: 16-byte rows, conflict-free operand reads)
 
@@ -78,13 +79,14 @@ __device__ __forceinline__ BlockCoord xcd_block_coord(int H) {
 // Cooperative load of one stage (64 rows of 64 bf16 = 512 chunks of 16 B, two per thread of a
 // 256-thread block): chunk = (row, 8 dims), consecutive lanes along a row.
 struct StageSrc { const unsigned short *p; size_t row0; int total, hoff, s; };
+template <int HDV>
 __device__ __forceinline__ void load_rows(const StageSrc &m, int first, uint4 (&regs)[2]) {
     const int tid = threadIdx.x;
 #pragma unroll
     for (int c = 0; c < 2; c++) {
         const int chunk = tid + 256 * c, row = first + (chunk >> 3);
         regs[c] = make_uint4(0, 0, 0, 0);
-        if (row >= 0 && row < m.s)
+        if (row >= 0 && row < m.s && 8 * (chunk & 7) < HDV)
             regs[c] = *reinterpret_cast<const uint4 *>(m.p + (m.row0 + row) * m.total + m.hoff + 8 * (chunk & 7));
     }
 }
@@ -116,6 +118,7 @@ __device__ __forceinline__ uint4 ld_tr2(const unsigned short (*T)[LD], int row_a
     return make_uint4(ua.x, ua.y, ub.x, ub.y);
 }
 
+template <int HDV>
 __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned short *__restrict__ q,
                                                             const unsigned short *__restrict__ k,
                                                             const unsigned short *__restrict__ v,
@@ -126,7 +129,9 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
+    constexpr int NKS = HDV / 32, NDT = HDV / 16;
+    constexpr float kInvSqrt = HDV == 64 ? 0.125f : 0.17677669529663687f;   // 1 / sqrt(head size)
+    const int total = H * HDV, hoff = h * HDV;
     const size_t row0 = (size_t)b * s;
     const int qlo = t0 + 32 * wave, qhi = qlo + 31;           // this wave's queries
     const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
 #pragma unroll
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             const int tq = qlo + 16 * qt + r;
             qf[qt][ks] = make_uint4(0, 0, 0, 0);
             if (tq < s) qf[qt][ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
@@ -145,13 +150,13 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
 #pragma unroll
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int dt = 0; dt < NDT; dt++) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     float mrun[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};   // running maximum (exp2 units), this lane's share of the sum
-    const float c2 = 0.125f * 1.44269504088896340736f;   // log2(e) / sqrt(64)
+    const float c2 = kInvSqrt * 1.44269504088896340736f;   // log2(e) / sqrt(head size)
 
     uint4 kreg[2], vreg[2];
-    load_rows(km, KS * st_lo, kreg);
-    load_rows(vm, KS * st_lo, vreg);
+    load_rows<HDV>(km, KS * st_lo, kreg);
+    load_rows<HDV>(vm, KS * st_lo, vreg);
     for (int st = st_lo; st <= st_hi; st++) {
         const int buf = (st - st_lo) & 1, k0 = KS * st;
 #pragma unroll
@@ -162,8 +167,8 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
         }
         __syncthreads();   // also: every wave is done with the stage before the previous one, whose buffer comes next
         if (st < st_hi) {
-            load_rows(km, k0 + KS, kreg);
-            load_rows(vm, k0 + KS, vreg);
+            load_rows<HDV>(km, k0 + KS, kreg);
+            load_rows<HDV>(vm, k0 + KS, vreg);
         }
         if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;   // no key of this stage is seen by this wave's queries
         f32x4 sc[4][2];
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
 #pragma unroll
             for (int qt = 0; qt < 2; qt++) {
                 sc[kt][qt] = mfma32(a0, qf[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
-                sc[kt][qt] = mfma32(a1, qf[qt][1], sc[kt][qt]);
+                if constexpr (NKS == 2) sc[kt][qt] = mfma32(a1, qf[qt][1], sc[kt][qt]);
             }
         }
         const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;   // wave-uniform: nothing to mask
@@ -213,7 +218,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
                 }
             lsum[qt] = fmaf(lsum[qt], alpha, part);
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) o[qt][dt] = o[qt][dt] * alpha;
+            for (int dt = 0; dt < NDT; dt++) o[qt][dt] = o[qt][dt] * alpha;
         }
 #pragma unroll
         for (int hf = 0; hf < 2; hf++) {
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
                 pb[qt] = make_uint4(pack2(p0[0], p0[1]), pack2(p0[2], p0[3]), pack2(p1[0], p1[1]), pack2(p1[2], p1[3]));
             }
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
+            for (int dt = 0; dt < NDT; dt++) {
                 const uint4 av = ld_tr2<LDV>(Vs[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
 #pragma unroll
                 for (int qt = 0; qt < 2; qt++) o[qt][dt] = mfma32(av, pb[qt], o[qt][dt]);
@@ -242,7 +247,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
             if (g == 0) stats[(size_t)(b * H + h) * s + tq] = make_float2(mrun[qt] == -INFINITY ? 0.f : mrun[qt], inv);
             unsigned short *ob = out + (row0 + tq) * total + hoff;
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+            for (int dt = 0; dt < NDT; dt++)
                 *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) =
                     make_uint2(pack2(o[qt][dt][0] * inv, o[qt][dt][1] * inv), pack2(o[qt][dt][2] * inv, o[qt][dt][3] * inv));
         }
@@ -254,6 +259,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_stats_kernel(const unsigned sh
 // w = bf16(exp2(s c - m) / sum) to their slot rows (four consecutive slots per lane and tile: 8-byte stores at
 // 2-byte alignment) and O^T += V^T w^T.  Slots behind an early query's own key (t < window - 1) are zeroed at
 // the end.
+template <int HDV>
 __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned short *__restrict__ q,
                                                               const unsigned short *__restrict__ k,
                                                               const unsigned short *__restrict__ v,
@@ -265,18 +271,20 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
+    constexpr int NKS = HDV / 32, NDT = HDV / 16;
+    constexpr float kInvSqrt = HDV == 64 ? 0.125f : 0.17677669529663687f;   // 1 / sqrt(head size)
+    const int total = H * HDV, hoff = h * HDV;
     const size_t row0 = (size_t)b * s;
     const int qlo = t0 + 32 * wave, qhi = qlo + 31;
     const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
     const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
-    const float c2 = 0.125f * 1.44269504088896340736f;
+    const float c2 = kInvSqrt * 1.44269504088896340736f;
 
     uint4 qf[2][2];
 #pragma unroll
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             const int tq = qlo + 16 * qt + r;
             qf[qt][ks] = make_uint4(0, 0, 0, 0);
             if (tq < s) qf[qt][ks] = *reinterpret_cast<const uint4 *>(q + (row0 + tq) * total + hoff + 32 * ks + 8 * g);
@@ -289,7 +297,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
 #pragma unroll
             for (int qt = 0; qt < 2; qt++) {
                 sc[kt][qt] = mfma32(a0, qf[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
-                sc[kt][qt] = mfma32(a1, qf[qt][1], sc[kt][qt]);
+                if constexpr (NKS == 2) sc[kt][qt] = mfma32(a1, qf[qt][1], sc[kt][qt]);
             }
         }
         const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;
@@ -310,7 +318,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
     // ---- sweep 1: running maximum and sum ----
     float mrun[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
     uint4 kreg[2], vreg[2];
-    load_rows(km, KS * st_lo, kreg);
+    load_rows<HDV>(km, KS * st_lo, kreg);
     for (int st = st_lo; st <= st_hi; st++) {
         const int buf = (st - st_lo) & 1, k0 = KS * st;
 #pragma unroll
@@ -319,7 +327,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
             *reinterpret_cast<uint4 *>(&Ks[buf][chunk >> 3][8 * (chunk & 7)]) = kreg[c];
         }
         __syncthreads();
-        if (st < st_hi) load_rows(km, k0 + KS, kreg);
+        if (st < st_hi) load_rows<HDV>(km, k0 + KS, kreg);
         if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
         f32x4 sc[4][2];
         scores(buf, k0, sc);
@@ -359,7 +367,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
 #pragma unroll
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int dt = 0; dt < NDT; dt++) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     unsigned short *wrow[2];
     int lsq[2];
 #pragma unroll
@@ -369,8 +377,8 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
         wrow[qt] = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
     }
     __syncthreads();   // every wave is done with the buffers of sweep 1
-    load_rows(km, KS * st_lo, kreg);
-    load_rows(vm, KS * st_lo, vreg);
+    load_rows<HDV>(km, KS * st_lo, kreg);
+    load_rows<HDV>(vm, KS * st_lo, vreg);
     for (int st = st_lo; st <= st_hi; st++) {
         const int buf = (st - st_lo) & 1, k0 = KS * st;
 #pragma unroll
@@ -381,8 +389,8 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
         }
         __syncthreads();
         if (st < st_hi) {
-            load_rows(km, k0 + KS, kreg);
-            load_rows(vm, k0 + KS, vreg);
+            load_rows<HDV>(km, k0 + KS, kreg);
+            load_rows<HDV>(vm, k0 + KS, vreg);
         }
         if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
         f32x4 sc[4][2];
@@ -419,7 +427,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
                 pb[qt] = make_uint4(wp[0][0], wp[0][1], wp[1][0], wp[1][1]);
             }
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
+            for (int dt = 0; dt < NDT; dt++) {
                 const uint4 av = ld_tr2<LDV>(Vs[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
 #pragma unroll
                 for (int qt = 0; qt < 2; qt++) o[qt][dt] = mfma32(av, pb[qt], o[qt][dt]);
@@ -441,7 +449,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
         if (tq < s) {
             unsigned short *ob = out + (row0 + tq) * total + hoff;
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+            for (int dt = 0; dt < NDT; dt++)
                 *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) =
                     make_uint2(pack2(o[qt][dt][0], o[qt][dt][1]), pack2(o[qt][dt][2], o[qt][dt][3]));
         }
@@ -457,6 +465,7 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
 // Per stage a wave forms S^T = K Q^T, the weights w = bf16(exp2(s c - m) / sum) as the weight tensor would hold
 // them, dW^T = V dO^T; dO and w dW enter as hi + lo pairs, w is exact in bf16.  K^T is read from the K rows
 // through ds_read_b64_tr_b16 in the key order that the score tiles leave in the lanes.  D goes to dvec.
+template <int HDV>
 __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned short *__restrict__ q,
                                                                  const unsigned short *__restrict__ k,
                                                                  const unsigned short *__restrict__ v,
@@ -468,12 +477,14 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
+    constexpr int NKS = HDV / 32, NDT = HDV / 16;
+    constexpr float kInvSqrt = HDV == 64 ? 0.125f : 0.17677669529663687f;   // 1 / sqrt(head size)
+    const int total = H * HDV, hoff = h * HDV;
     const size_t row0 = (size_t)b * s;
     const int qlo = t0 + 32 * wave, qhi = qlo + 31;
     const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
     const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
-    const float c2 = 0.125f * 1.44269504088896340736f, scale = 0.125f;
+    const float c2 = kInvSqrt * 1.44269504088896340736f, scale = kInvSqrt;
 
     uint4 qf[2][2], doh[2][2], dol[2][2];
     float mc[2], inv[2], dpart[2] = {0.f, 0.f};
@@ -482,7 +493,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
         const int tq = qlo + 16 * qt + r;
         mc[qt] = 0.f; inv[qt] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             qf[qt][ks] = make_uint4(0, 0, 0, 0);
             f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
             if (tq < s) {
@@ -503,11 +514,11 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
 #pragma unroll
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) { aq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; bq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        for (int dt = 0; dt < NDT; dt++) { aq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; bq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
     uint4 kreg[2], vreg[2];
-    load_rows(km, KS * st_lo, kreg);
-    load_rows(vm, KS * st_lo, vreg);
+    load_rows<HDV>(km, KS * st_lo, kreg);
+    load_rows<HDV>(vm, KS * st_lo, vreg);
     for (int st = st_lo; st <= st_hi; st++) {
         const int buf = (st - st_lo) & 1, k0 = KS * st;
 #pragma unroll
@@ -518,8 +529,8 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
         }
         __syncthreads();
         if (st < st_hi) {
-            load_rows(km, k0 + KS, kreg);
-            load_rows(vm, k0 + KS, vreg);
+            load_rows<HDV>(km, k0 + KS, kreg);
+            load_rows<HDV>(vm, k0 + KS, vreg);
         }
         if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
         const bool full = k0 + KS - 1 <= qlo && k0 >= qhi + 1 - ws && qhi < s;
@@ -536,11 +547,11 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
                     const uint4 ak0 = ld_op(Ks[buf], 16 * kt, 0), ak1 = ld_op(Ks[buf], 16 * kt, 1);
                     const uint4 av0 = ld_op(Vs[buf], 16 * kt, 0), av1 = ld_op(Vs[buf], 16 * kt, 1);
                     f32x4 sc = mfma32(ak0, qf[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
-                    sc = mfma32(ak1, qf[qt][1], sc);
+                    if constexpr (NKS == 2) sc = mfma32(ak1, qf[qt][1], sc);
                     f32x4 dw = mfma32(av0, doh[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
                     dw = mfma32(av0, dol[qt][0], dw);
-                    dw = mfma32(av1, doh[qt][1], dw);
-                    dw = mfma32(av1, dol[qt][1], dw);
+                    if constexpr (NKS == 2) dw = mfma32(av1, doh[qt][1], dw);
+                    if constexpr (NKS == 2) dw = mfma32(av1, dol[qt][1], dw);
                     f32x4 w;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -560,7 +571,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
                 wb[qt] = make_uint4(wp[0][0], wp[0][1], wp[1][0], wp[1][1]);
             }
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
+            for (int dt = 0; dt < NDT; dt++) {
                 const uint4 a = ld_tr2<LDH>(Ks[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
 #pragma unroll
                 for (int qt = 0; qt < 2; qt++) {
@@ -581,7 +592,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
             if (g == 0) dvec[(size_t)(b * H + h) * s + tq] = dsum;
             float *ob = d_q + (row0 + tq) * total + hoff;
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+            for (int dt = 0; dt < NDT; dt++)
                 *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
         }
     }
@@ -591,6 +602,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
 // swa_bwd_q_stats_kernel: A = sum_j (w dW) k_j, B = sum_j w k_j and D = sum_j w dW together, d_q = (A - D B)/sqrt(hd).
 // A lane's four keys of a tile are four consecutive slots of its query's row: one 8-byte load (2-byte aligned),
 // requested a stage ahead; only the stages at the two ends of the window go slot by slot.
+template <int HDV>
 __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigned short *__restrict__ k,
                                                                    const unsigned short *__restrict__ v,
                                                                    const unsigned short *__restrict__ attn_w,
@@ -601,12 +613,14 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int t0 = bc.x * FQ, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
+    constexpr int NKS = HDV / 32, NDT = HDV / 16;
+    constexpr float kInvSqrt = HDV == 64 ? 0.125f : 0.17677669529663687f;   // 1 / sqrt(head size)
+    const int total = H * HDV, hoff = h * HDV;
     const size_t row0 = (size_t)b * s;
     const int qlo = t0 + 32 * wave, qhi = qlo + 31;
     const int st_lo = max(t0 + 1 - ws, 0) / KS, st_hi = min(t0 + FQ - 1, s - 1) / KS;
     const StageSrc km{k, row0, total, hoff, s}, vm{v, row0, total, hoff, s};
-    const float scale = 0.125f;
+    const float scale = kInvSqrt;
 
     uint4 doh[2][2], dol[2][2];
     const unsigned short *wrow[2];
@@ -619,7 +633,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
         lsq[qt] = max(tq + 1 - ws, 0);
         wrow[qt] = attn_w + ((size_t)(b * H + h) * s + min(tq, s - 1)) * ws;
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             f32x4 x0 = f32x4{0.f, 0.f, 0.f, 0.f}, x1 = x0;
             if (tq < s) {
                 const size_t o = (row0 + tq) * total + hoff + 32 * ks + 8 * g;
@@ -633,7 +647,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
 #pragma unroll
     for (int qt = 0; qt < 2; qt++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) { aq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; bq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        for (int dt = 0; dt < NDT; dt++) { aq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; bq[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
     // weights of a stage for this lane: wreg[kt][qt] = keys k0 + 16 kt + 4 g .. + 3 of query qt, zero outside the window
     uint2 wreg[4][2];
@@ -664,8 +678,8 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
     };
 
     uint4 kreg[2], vreg[2];
-    load_rows(km, KS * st_lo, kreg);
-    load_rows(vm, KS * st_lo, vreg);
+    load_rows<HDV>(km, KS * st_lo, kreg);
+    load_rows<HDV>(vm, KS * st_lo, vreg);
     fetch_weights(KS * st_lo);
     for (int st = st_lo; st <= st_hi; st++) {
         const int buf = (st - st_lo) & 1, k0 = KS * st;
@@ -682,8 +696,8 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
             for (int qt = 0; qt < 2; qt++) wcur[kt][qt] = wreg[kt][qt];
         __syncthreads();
         if (st < st_hi) {
-            load_rows(km, k0 + KS, kreg);
-            load_rows(vm, k0 + KS, vreg);
+            load_rows<HDV>(km, k0 + KS, kreg);
+            load_rows<HDV>(vm, k0 + KS, vreg);
             fetch_weights(k0 + KS);
         }
         if (k0 > qhi || k0 + KS - 1 < qlo + 1 - ws) continue;
@@ -699,8 +713,8 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
                     const uint4 av0 = ld_op(Vs[buf], 16 * kt, 0), av1 = ld_op(Vs[buf], 16 * kt, 1);
                     f32x4 dw = mfma32(av0, doh[qt][0], f32x4{0.f, 0.f, 0.f, 0.f});
                     dw = mfma32(av0, dol[qt][0], dw);
-                    dw = mfma32(av1, doh[qt][1], dw);
-                    dw = mfma32(av1, dol[qt][1], dw);
+                    if constexpr (NKS == 2) dw = mfma32(av1, doh[qt][1], dw);
+                    if constexpr (NKS == 2) dw = mfma32(av1, dol[qt][1], dw);
                     const uint2 wp = wcur[kt][qt];
                     x[c][0] = bf_lo(wp.x) * dw[0];
                     x[c][1] = bf_hi(wp.x) * dw[1];
@@ -712,7 +726,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
                 wb[qt] = make_uint4(wcur[2 * hf][qt].x, wcur[2 * hf][qt].y, wcur[2 * hf + 1][qt].x, wcur[2 * hf + 1][qt].y);
             }
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
+            for (int dt = 0; dt < NDT; dt++) {
                 const uint4 a = ld_tr2<LDH>(Ks[buf], 32 * hf + 4 * g, 32 * hf + 16 + 4 * g, 16 * dt);
 #pragma unroll
                 for (int qt = 0; qt < 2; qt++) {
@@ -733,7 +747,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
             if (g == 0) dvec[(size_t)(b * H + h) * s + tq] = dsum;
             float *ob = d_q + (row0 + tq) * total + hoff;
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+            for (int dt = 0; dt < NDT; dt++)
                 *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
         }
     }
@@ -745,6 +759,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
 // accumulates d_v^T += dO^T w and d_k^T += Q^T dS.  The Q and dO rows of a stage are staged as they arrive (dO as
 // hi + lo); the products that contract over queries read them through ds_read_b64_tr_b16 in the query order
 // that the score tiles leave in the lanes.  K and V of the wave's keys sit in registers.
+template <int HDV>
 __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned short *__restrict__ q,
                                                                  const unsigned short *__restrict__ k,
                                                                  const unsigned short *__restrict__ v,
@@ -758,20 +773,22 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int j0 = bc.x * FQ, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
+    constexpr int NKS = HDV / 32, NDT = HDV / 16;
+    constexpr float kInvSqrt = HDV == 64 ? 0.125f : 0.17677669529663687f;   // 1 / sqrt(head size)
+    const int total = H * HDV, hoff = h * HDV;
     const size_t row0 = (size_t)b * s;
     const int jlo = j0 + 32 * wave, jhi = jlo + 31;            // this wave's keys
     const int st_lo = j0 / KS, st_hi = min(s - 1, j0 + FQ - 1 + ws - 1) / KS;
     const float *dvb = dvec + (size_t)(b * H + h) * s;
     const float2 *stb = stats + (size_t)(b * H + h) * s;
     const StageSrc qm{q, row0, total, hoff, s};
-    const float c2 = 0.125f * 1.44269504088896340736f, scale = 0.125f;
+    const float c2 = kInvSqrt * 1.44269504088896340736f, scale = kInvSqrt;
 
     uint4 kf[2][2], vf[2][2];   // B operands: key jlo + 16 jt + r, dims 32 ks + 8 g ..
 #pragma unroll
     for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             const int key = jlo + 16 * jt + r;
             kf[jt][ks] = make_uint4(0, 0, 0, 0);
             vf[jt][ks] = make_uint4(0, 0, 0, 0);
@@ -785,7 +802,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
 #pragma unroll
     for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) { dk[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        for (int dt = 0; dt < NDT; dt++) { dk[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
     // one stage ahead in registers: Q rows (two 16-byte pieces per thread), dO rows (thread = quarter row)
     uint4 qreg[2];
@@ -794,12 +811,12 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
     float ddreg = 0.f;
     const int drow = tid >> 2, dcol = 16 * (tid & 3);
     auto fetch_stage = [&](int t_lo) {
-        load_rows(qm, t_lo, qreg);
+        load_rows<HDV>(qm, t_lo, qreg);
         const int t = t_lo + drow;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             dreg[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (t < s) dreg[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dcol + 4 * c);
+            if (t < s && dcol < HDV) dreg[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dcol + 4 * c);
         }
         streg = make_float2(0.f, 0.f);
         ddreg = 0.f;
@@ -839,11 +856,11 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
 #pragma unroll
                 for (int jt = 0; jt < 2; jt++) {
                     f32x4 sc = mfma32(aq0, kf[jt][0], f32x4{0.f, 0.f, 0.f, 0.f});
-                    sc = mfma32(aq1, kf[jt][1], sc);
+                    if constexpr (NKS == 2) sc = mfma32(aq1, kf[jt][1], sc);
                     f32x4 dw = mfma32(ah0, vf[jt][0], f32x4{0.f, 0.f, 0.f, 0.f});
                     dw = mfma32(al0, vf[jt][0], dw);
-                    dw = mfma32(ah1, vf[jt][1], dw);
-                    dw = mfma32(al1, vf[jt][1], dw);
+                    if constexpr (NKS == 2) dw = mfma32(ah1, vf[jt][1], dw);
+                    if constexpr (NKS == 2) dw = mfma32(al1, vf[jt][1], dw);
                     f32x4 w;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -865,7 +882,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
                 split8(ds[jt][0], ds[jt][1], dsh[jt], dsl[jt]);
             }
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
+            for (int dt = 0; dt < NDT; dt++) {
                 const int ra = 32 * hq + 4 * g, rb = ra + 16;
                 const uint4 aq = ld_tr2<LDH>(Qs[buf], ra, rb, 16 * dt);    // Q^T [dim][query]
                 const uint4 ah = ld_tr2<LDH>(Dh[buf], ra, rb, 16 * dt);    // dO^T hi / lo
@@ -887,7 +904,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
         if (key >= s) continue;
         float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
+        for (int dt = 0; dt < NDT; dt++) {
             f32x4 *ck = reinterpret_cast<f32x4 *>(pk + 16 * dt + 4 * g), *cv = reinterpret_cast<f32x4 *>(pv + 16 * dt + 4 * g);
             *ck = *ck + dk[jt][dt];
             *cv = *cv + dv[jt][dt];
@@ -901,6 +918,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
 // transposing read, which is both the B operand of d_v^T += dO^T w and the w of dS = w (dW - D_t) / sqrt(hd).
 constexpr int LDW = 144;   // row stride of the weight stage (288 B: the transposing reads of a group fall on 32 banks)
 
+template <int HDV>
 __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigned short *__restrict__ q,
                                                                    const unsigned short *__restrict__ v,
                                                                    const unsigned short *__restrict__ attn_w,
@@ -914,20 +932,22 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigne
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
     const int j0 = bc.x * FQ, h = bc.h, b = bc.b;
-    const int total = H * HD, hoff = h * HD;
+    constexpr int NKS = HDV / 32, NDT = HDV / 16;
+    constexpr float kInvSqrt = HDV == 64 ? 0.125f : 0.17677669529663687f;   // 1 / sqrt(head size)
+    const int total = H * HDV, hoff = h * HDV;
     const size_t row0 = (size_t)b * s;
     const int jlo = j0 + 32 * wave, jhi = jlo + 31;
     const int st_lo = j0 / KS, st_hi = min(s - 1, j0 + FQ - 1 + ws - 1) / KS;
     const float *dvb = dvec + (size_t)(b * H + h) * s;
     const unsigned short *awb = attn_w + ((size_t)(b * H + h) * s) * ws;
     const StageSrc qm{q, row0, total, hoff, s};
-    const float scale = 0.125f;
+    const float scale = kInvSqrt;
 
     uint4 vf[2][2];
 #pragma unroll
     for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             const int key = jlo + 16 * jt + r;
             vf[jt][ks] = make_uint4(0, 0, 0, 0);
             if (key < s) vf[jt][ks] = *reinterpret_cast<const uint4 *>(v + (row0 + key) * total + hoff + 32 * ks + 8 * g);
@@ -936,19 +956,19 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigne
 #pragma unroll
     for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) { dk[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        for (int dt = 0; dt < NDT; dt++) { dk[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; dv[jt][dt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
     uint4 qreg[2], wreg[4];
     f32x4 dreg[4];
     float ddreg = 0.f;
     const int drow = tid >> 2, dcol = 16 * (tid & 3);
     auto fetch_stage = [&](int t_lo) {
-        load_rows(qm, t_lo, qreg);
+        load_rows<HDV>(qm, t_lo, qreg);
         const int t = t_lo + drow;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             dreg[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (t < s) dreg[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dcol + 4 * c);
+            if (t < s && dcol < HDV) dreg[c] = *reinterpret_cast<const f32x4 *>(d_out + (row0 + t) * total + hoff + dcol + 4 * c);
         }
         ddreg = (tid < KS && t_lo + tid < s) ? dvb[t_lo + tid] : 0.f;
         // weights of query t for keys j0 + 32 (tid % 4) .. + 31: four pieces of 8 keys
@@ -1007,8 +1027,8 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigne
                     for (int jt = 0; jt < 2; jt++) {
                         f32x4 dw = mfma32(ah0, vf[jt][0], f32x4{0.f, 0.f, 0.f, 0.f});
                         dw = mfma32(al0, vf[jt][0], dw);
-                        dw = mfma32(ah1, vf[jt][1], dw);
-                        dw = mfma32(al1, vf[jt][1], dw);
+                        if constexpr (NKS == 2) dw = mfma32(ah1, vf[jt][1], dw);
+                        if constexpr (NKS == 2) dw = mfma32(al1, vf[jt][1], dw);
                         const unsigned w01 = c ? wpk[jt].z : wpk[jt].x, w23 = c ? wpk[jt].w : wpk[jt].y;
                         ds[jt][c][0] = bf_lo(w01) * (dw[0] - d4[0]) * scale;
                         ds[jt][c][1] = bf_hi(w01) * (dw[1] - d4[1]) * scale;
@@ -1019,7 +1039,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigne
 #pragma unroll
                 for (int jt = 0; jt < 2; jt++) split8(ds[jt][0], ds[jt][1], dsh[jt], dsl[jt]);
 #pragma unroll
-                for (int dt = 0; dt < 4; dt++) {
+                for (int dt = 0; dt < NDT; dt++) {
                     const uint4 aq = ld_tr2<LDH>(Qs[buf], ra, rb, 16 * dt);    // Q^T [dim][query]
                     const uint4 ah = ld_tr2<LDH>(Dh[buf], ra, rb, 16 * dt);    // dO^T hi / lo
                     const uint4 al = ld_tr2<LDH>(Dl[buf], ra, rb, 16 * dt);
@@ -1041,7 +1061,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigne
         if (key >= s) continue;
         float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
+        for (int dt = 0; dt < NDT; dt++) {
             f32x4 *ck = reinterpret_cast<f32x4 *>(pk + 16 * dt + 4 * g), *cv = reinterpret_cast<f32x4 *>(pv + 16 * dt + 4 * g);
             *ck = *ck + dk[jt][dt];
             *cv = *cv + dv[jt][dt];
@@ -1053,16 +1073,20 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_blocked_kernel(const unsigne
 
 bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, uint16_t *out, uint16_t *attn_weights,
                       int seq_len, int num_heads, int head_dim, int window, int batch, int n_persistent, float *stats) {
-    if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
+    if ((head_dim != 64 && head_dim != 32) || n_persistent != 0 || window > 512 || window < 1) return false;
     if (stats) {
         KernelTimer kt("swa_fwd_stats_kernel");
-        hipLaunchKernelGGL(swa_fwd_stats_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+        if (head_dim == 64) hipLaunchKernelGGL(swa_fwd_stats_kernel<64>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+                           k, v, out, reinterpret_cast<float2 *>(stats), seq_len, num_heads, window);
+        else hipLaunchKernelGGL(swa_fwd_stats_kernel<32>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
                            k, v, out, reinterpret_cast<float2 *>(stats), seq_len, num_heads, window);
         check_launch("swa_fwd_stats_kernel");
         return true;
     }
     KernelTimer kt("swa_fwd_blocked_kernel");
-    hipLaunchKernelGGL(swa_fwd_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+    if (head_dim == 64) hipLaunchKernelGGL(swa_fwd_blocked_kernel<64>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+                       k, v, out, attn_weights, seq_len, num_heads, window);
+    else hipLaunchKernelGGL(swa_fwd_blocked_kernel<32>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
                        k, v, out, attn_weights, seq_len, num_heads, window);
     check_launch("swa_fwd_blocked_kernel");
     return true;
@@ -1072,7 +1096,7 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
                        const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
                        int head_dim, int window, int batch, int n_persistent, const float *stats) {
     const ErrorScope es;
-    if (head_dim != HD || n_persistent != 0 || window > 512 || window < 1) return false;
+    if ((head_dim != 64 && head_dim != 32) || n_persistent != 0 || window > 512 || window < 1) return false;
     float *dvec = scratch(1, (size_t)batch * num_heads * seq_len * sizeof(float));
     if (es.failed()) return true;
     if (stats) {
@@ -1080,24 +1104,32 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
         const dim3 grid((seq_len + FQ - 1) / FQ, num_heads, batch);
         {
             KernelTimer kt("swa_bwd_q_stats_kernel");
-            hipLaunchKernelGGL(swa_bwd_q_stats_kernel, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, dvec,
+            if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_q_stats_kernel<64>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, dvec,
+                               seq_len, num_heads, window);
+            else hipLaunchKernelGGL(swa_bwd_q_stats_kernel<32>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, dvec,
                                seq_len, num_heads, window);
             check_launch("swa_bwd_q_stats_kernel");
         }
         KernelTimer kt("swa_bwd_k_stats_kernel");
-        hipLaunchKernelGGL(swa_bwd_k_stats_kernel, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec, d_k, d_v,
+        if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_k_stats_kernel<64>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec, d_k, d_v,
+                           seq_len, num_heads, window);
+        else hipLaunchKernelGGL(swa_bwd_k_stats_kernel<32>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec, d_k, d_v,
                            seq_len, num_heads, window);
         check_launch("swa_bwd_k_stats_kernel");
         return true;
     }
     {
         KernelTimer kt("swa_bwd_q_blocked_kernel");
-        hipLaunchKernelGGL(swa_bwd_q_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0,
+        if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_q_blocked_kernel<64>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0,
+                           stream(), k, v, attn_weights, d_attn_out, d_q, dvec, seq_len, num_heads, window);
+        else hipLaunchKernelGGL(swa_bwd_q_blocked_kernel<32>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0,
                            stream(), k, v, attn_weights, d_attn_out, d_q, dvec, seq_len, num_heads, window);
         check_launch("swa_bwd_q_blocked_kernel");
     }
     KernelTimer kt("swa_bwd_k_blocked_kernel");
-    hipLaunchKernelGGL(swa_bwd_k_blocked_kernel, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+    if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_k_blocked_kernel<64>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
+                       v, attn_weights, d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
+    else hipLaunchKernelGGL(swa_bwd_k_blocked_kernel<32>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0, stream(), q,
                        v, attn_weights, d_attn_out, dvec, d_k, d_v, seq_len, num_heads, window);
     check_launch("swa_bwd_k_blocked_kernel");
     return true;

@@ -45,7 +45,9 @@ def gpu_backward(q, k, v, aw, go, ws, H, npers):
 @pytest.mark.parametrize("B,s,H,hd,ws,npers", [(2, 40, 2, 64, 16, 0), (1, 70, 3, 32, 64, 0),
                                                (2, 33, 2, 64, 8, 5), (1, 20, 1, 8, 32, 0),
                                                (1, 600, 2, 64, 512, 0), (1, 50, 2, 24, 7, 3),
-                                               (2, 200, 2, 64, 101, 0), (1, 1100, 1, 64, 300, 0)])
+                                               (2, 200, 2, 64, 101, 0), (1, 1100, 1, 64, 300, 0),
+                                               (2, 600, 4, 32, 512, 0), (1, 200, 2, 32, 101, 0), (3, 130, 2, 32, 64, 0),
+                                               (1, 1100, 1, 32, 300, 0), (1, 2, 1, 32, 2, 0)])
 def test_swa_forward_backward_parity(B, s, H, hd, ws, npers):
     q, k, v, go = _case(B, s, H, hd, 100 + s + ws)
     out, aw = gpu_forward(q, k, v, ws, H, npers)
@@ -95,13 +97,13 @@ def test_swa_backward_accumulates_dk_dv_and_overwrites_dq():
     assert_close("d_v", host(dv) - 2.0, ov, 1e-4)
 
 
+@pytest.mark.parametrize("hd", [64, 32])
 @pytest.mark.parametrize("B,s,H,ws", [(2, 40, 2, 16), (1, 600, 2, 512), (2, 200, 2, 101), (1, 1100, 1, 300),
                                       (1, 2, 1, 2), (8, 130, 2, 64), (1, 64, 1, 64), (1, 65, 3, 2)])
-def test_swa_without_weight_tensor(B, s, H, ws):
+def test_swa_without_weight_tensor(B, s, H, ws, hd):
     """The pair that keeps per-query softmax statistics instead of the weight tensor: output against the
     weight-storing forward and the oracle, statistics against the oracle's scores, gradients against the weight-storing
     backward (same rounding of the weights: fp32 round-off) and the oracle (bf16 tolerance)."""
-    hd = 64
     q, k, v, go = _case(B, s, H, hd, 300 + s + ws)
     out_w, aw = gpu_forward(q, k, v, ws, H, 0)
     out = torch.zeros(B, s, H * hd, dtype=torch.uint16, device="cuda")
@@ -118,7 +120,7 @@ def test_swa_without_weight_tensor(B, s, H, ws):
     st = host(stats)
     for b in range(B):
         for h in range(H):
-            sc = qf[b, :, h] @ kf[b, :, h].T / 8.0
+            sc = qf[b, :, h] @ kf[b, :, h].T / np.sqrt(hd)
             for t in range(0, s, max(1, s // 37)):
                 row = sc[t, max(t + 1 - ws, 0):t + 1]
                 assert abs(st[b, h, t, 0] - row.max() * np.log2(np.e)) < 1e-3 * max(1.0, abs(row.max()))
@@ -146,16 +148,16 @@ def test_swa_without_weight_tensor(B, s, H, ws):
 
 def test_swa_without_weight_tensor_rejects_other_shapes():
     from nl_hecate_amd.ffi import lib
-    z = torch.zeros(1, 8, 32, dtype=torch.uint16, device="cuda")
+    z = torch.zeros(1, 8, 16, dtype=torch.uint16, device="cuda")
     st = torch.zeros(1, 1, 8, 2, device="cuda")
     lib.nlh_set_error_mode(1)
     try:
         lib.nlh_clear_error()
-        D.call("swa_forward_lse_bf16_rocm", z, z, z, z, st, 8, 1, 32, 4, 1)
+        D.call("swa_forward_lse_bf16_rocm", z, z, z, z, st, 8, 1, 16, 4, 1)
         assert b"head_dim 64" in lib.nlh_last_error()
         lib.nlh_clear_error()
-        g = torch.zeros(1, 8, 32, device="cuda")
-        D.call("swa_backward_lse_bf16_rocm", z, z, z, st, g, g, g, g, 8, 1, 32, 4, 1)
+        g = torch.zeros(1, 8, 16, device="cuda")
+        D.call("swa_backward_lse_bf16_rocm", z, z, z, st, g, g, g, g, 8, 1, 16, 4, 1)
         assert b"head_dim 64" in lib.nlh_last_error()
     finally:
         lib.nlh_clear_error()
