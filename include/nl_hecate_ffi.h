@@ -386,6 +386,12 @@ void swa_forward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint1
 void swa_backward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, const float *stats,
                                 const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len,
                                 int num_heads, int head_dim, int window_size, int batch_size);
+/* The same backward with the three gradients written (not accumulated) as bf16 into columns of a wider row-major
+ * matrix: g_q, g_k, g_v point at the first row's columns, ld is the row stride in elements.  No counterpart in the
+ * reference: for a caller whose next step is a bf16 GEMM over those columns (the level step's projection gradients). */
+void swa_backward_lse_bf16_cols_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, const float *stats,
+                                     const float *d_attn_out, uint16_t *g_q, uint16_t *g_k, uint16_t *g_v, long long ld,
+                                     int seq_len, int num_heads, int head_dim, int window_size, int batch_size);
 
 /* ── AdamW and gradient clipping; return hipError_t as unsigned, 0 = success ─ */
 /* core/src/cuda_ffi.rs:674 */
@@ -923,8 +929,9 @@ void titans_levels_forward_bf16_rocm(const float *x, const float *w_extra, int n
  * and activation derivatives of the gates, backward of the two normalisations, then d_x [n, d] (overwritten) =
  * sum over all projections of g W, and d_w_extra [n_extra * d, d], d_w_levels [levels * 3 * d, d] (overwritten)
  * = g^T x, as bf16 GEMMs with fp32 accumulation; d_extra: host array of n_extra device pointers, the fp32
- * gradients [n, d] of the plain projections' outputs; d_gate_params: host array of 6 * levels device pointers
- * (overwritten).  As on the reference's GPU path nothing flows from the gates into k and v.
+ * gradients [n, d] of the plain projections' outputs, or n_extra null pointers when the caller has already
+ * written them as bf16 into columns e * d .. of the operand that level_grad_operand_rocm returns; d_gate_params:
+ * host array of 6 * levels device pointers (overwritten).  As on the reference's GPU path nothing flows from the gates into k and v.
  * d_m_initial, d_s_initial [head_dim^2] are accumulated (+=, summed over all chains). */
 void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_extra, int n_extra, const float *const *d_extra,
                                       const float *w_levels, const uint16_t *k_heads, const uint16_t *v_heads,
@@ -934,6 +941,11 @@ void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_ext
                                       const float *s_chunk_states, const float *d_y_tokens, float *d_x, float *d_w_extra,
                                       float *d_w_levels, float *const *d_gate_params, float *d_m_initial, float *d_s_initial,
                                       int bs, int seq_len, int heads, int head_dim, int levels, int chunk_size, float eps);
+/* The bf16 operand g [bs * seq_len, (n_extra + 3 * levels) * d] of the backward's two GEMMs, in the library's
+ * scratch (stable until a larger call or nlh_release_workspace): projection e's output gradient belongs in columns
+ * e * d .. e * d + d - 1.  A producer that can write bf16 with a row stride (swa_backward_lse_bf16_cols_rocm) fills
+ * them in place and passes null pointers as d_extra.  *ld receives the row stride in elements.  Null on bad shapes. */
+uint16_t *level_grad_operand_rocm(int bs, int seq_len, int heads, int head_dim, int levels, int n_extra, long long *ld);
 /* cms_combine_gate_bf16_rocm with gated leaving as plain bf16 [n] (the output projection's operand). */
 void cms_combine_gate_bf16x1_rocm(const float *const *y_levels, int k, const uint16_t *attn_out, float *gate,
                                   uint16_t *gated_bf16, long long n);

@@ -794,6 +794,14 @@ void titans_levels_forward_bf16_rocm(const float *x, const float *w_extra, int n
     check_launch("final_states_kernel");
 }
 
+uint16_t *level_grad_operand_rocm(int bs, int seq_len, int heads, int head_dim, int levels, int n_extra, long long *ld) {
+    const ErrorScope es;
+    if (!step_dims_ok("level_grad_operand_rocm", bs, seq_len, heads, head_dim, levels, n_extra, 1)) return nullptr;
+    const long long n = (long long)bs * seq_len, R = (long long)(n_extra + 3 * levels) * heads * head_dim;
+    if (ld) *ld = R;
+    return reinterpret_cast<uint16_t *>(scratch(26, (size_t)n * R * sizeof(u16)));
+}
+
 void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_extra, int n_extra, const float *const *d_extra,
                                       const float *w_levels, const uint16_t *k_heads, const uint16_t *v_heads,
                                       const uint16_t *q_heads, const float *alpha_heads, const float *theta_heads,
@@ -853,15 +861,23 @@ void titans_levels_backward_bf16_rocm(const uint16_t *x_bf16, const float *w_ext
         check_launch("level_gate_partials_kernel");
     }
     if (n_extra) {
-        ColSrcs cs{};
-        for (int e = 0; e < n_extra; e++) {
-            if (!al16(d_extra[e])) { fail("titans_levels_backward_bf16_rocm: gradient %d is not 16-byte aligned.", e); return; }
-            cs.p[e] = d_extra[e];
+        int given = 0;
+        for (int e = 0; e < n_extra; e++) given += d_extra[e] != nullptr;
+        if (given != 0 && given != n_extra) {
+            fail("titans_levels_backward_bf16_rocm: d_extra must hold %d pointers or none (gradients already in the operand).", n_extra);
+            return;
         }
-        KernelTimer kt("cols_to_bf16_kernel");
-        hipLaunchKernelGGL(cols_to_bf16_kernel, dim3(stream_blocks(n * n_extra * (d / 4), 4096)), dim3(kSThr), 0, stream(), cs,
-                           n_extra, n, d, G, R);
-        check_launch("cols_to_bf16_kernel");
+        if (given) {
+            ColSrcs cs{};
+            for (int e = 0; e < n_extra; e++) {
+                if (!al16(d_extra[e])) { fail("titans_levels_backward_bf16_rocm: gradient %d is not 16-byte aligned.", e); return; }
+                cs.p[e] = d_extra[e];
+            }
+            KernelTimer kt("cols_to_bf16_kernel");
+            hipLaunchKernelGGL(cols_to_bf16_kernel, dim3(stream_blocks(n * n_extra * (d / 4), 4096)), dim3(kSThr), 0, stream(), cs,
+                               n_extra, n, d, G, R);
+            check_launch("cols_to_bf16_kernel");
+        }
         to_bf16(w_extra, wb, (long long)n_extra * d * d);
     }
     if (levels) to_bf16(w_levels, wb + (size_t)n_extra * d * d, 3LL * levels * d * d);

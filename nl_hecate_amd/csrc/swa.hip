@@ -387,6 +387,21 @@ void swa_backward_lse_bf16_rocm(const uint16_t *q, const uint16_t *k, const uint
         fail("swa_backward_lse_bf16_rocm: needs head_dim 64 or 32 and window_size <= 512");
 }
 
+void swa_backward_lse_bf16_cols_rocm(const uint16_t *q, const uint16_t *k, const uint16_t *v, const float *stats,
+                                     const float *d_attn_out, uint16_t *g_q, uint16_t *g_k, uint16_t *g_v, long long ld,
+                                     int seq_len, int num_heads, int head_dim, int window_size, int batch_size) {
+    const ErrorScope es;
+    const char *fn = "swa_backward_lse_bf16_cols_rocm";
+    if (!swa_check(fn, seq_len, num_heads, head_dim, window_size, batch_size, 0)) return;
+    if (!stats || !g_q || !g_k || !g_v) return fail("%s: a pointer is null", fn);
+    if (ld < (long long)num_heads * head_dim || ld % 4 || (((uintptr_t)g_q | (uintptr_t)g_k | (uintptr_t)g_v) & 7))
+        return fail("%s: ld=%lld must be a multiple of 4 and at least heads * head_dim, the columns 8-byte aligned", fn, ld);
+    const SwaGradCols cols{g_q, g_k, g_v, ld};
+    if (!swa_backward_mfma(q, k, v, nullptr, d_attn_out, nullptr, nullptr, nullptr, seq_len, num_heads, head_dim, window_size,
+                           batch_size, 0, stats, &cols))
+        fail("%s: needs head_dim 64 or 32 and window_size <= 512", fn);
+}
+
 void swa_single_token_cuda(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
                            int cache_len, int num_heads, int head_dim, int window_size, int n_persistent) {
     const char *fn = "swa_single_token_cuda";

@@ -79,6 +79,9 @@ __device__ __forceinline__ BlockCoord xcd_block_coord(int H) {
 // Cooperative load of one stage (64 rows of 64 bf16 = 512 chunks of 16 B, two per thread of a
 // 256-thread block): chunk = (row, 8 dims), consecutive lanes along a row.
 struct StageSrc { const unsigned short *p; size_t row0; int total, hoff, s; };
+// OUT16 instantiations of the backward passes: the gradients leave as bf16 into columns of a wider row-major matrix
+// (row stride ld elements, the head's dims at the same column offset as in q, k, v), written, not accumulated.
+struct Out16 { unsigned short *q, *k, *v; long long ld; };
 template <int HDV>
 __device__ __forceinline__ void load_rows(const StageSrc &m, int first, uint4 (&regs)[2]) {
     const int tid = threadIdx.x;
@@ -465,14 +468,14 @@ __global__ __launch_bounds__(256, 3) void swa_fwd_blocked_kernel(const unsigned 
 // Per stage a wave forms S^T = K Q^T, the weights w = bf16(exp2(s c - m) / sum) as the weight tensor would hold
 // them, dW^T = V dO^T; dO and w dW enter as hi + lo pairs, w is exact in bf16.  K^T is read from the K rows
 // through ds_read_b64_tr_b16 in the key order that the score tiles leave in the lanes.  D goes to dvec.
-template <int HDV>
+template <int HDV, bool OUT16>
 __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned short *__restrict__ q,
                                                                  const unsigned short *__restrict__ k,
                                                                  const unsigned short *__restrict__ v,
                                                                  const float2 *__restrict__ stats,
                                                                  const float *__restrict__ d_out,
                                                                  float *__restrict__ d_q, float *__restrict__ dvec,
-                                                                 int s, int H, int ws) {
+                                                                 int s, int H, int ws, Out16 o16) {
     __shared__ __align__(16) unsigned short Ks[2][KS][LDH], Vs[2][KS][LDH];   // stages [key][dim]
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
     const BlockCoord bc = xcd_block_coord(H);
@@ -590,10 +593,19 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_stats_kernel(const unsigned 
         dsum += __shfl_xor(dsum, 32, 64);
         if (tq < s) {
             if (g == 0) dvec[(size_t)(b * H + h) * s + tq] = dsum;
-            float *ob = d_q + (row0 + tq) * total + hoff;
+            if (OUT16) {
+                unsigned short *ob = o16.q + (row0 + tq) * o16.ld + hoff;
 #pragma unroll
-            for (int dt = 0; dt < NDT; dt++)
-                *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
+                for (int dt = 0; dt < NDT; dt++) {
+                    const f32x4 x = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
+                    *reinterpret_cast<uint2 *>(ob + 16 * dt + 4 * g) = make_uint2(pack2(x[0], x[1]), pack2(x[2], x[3]));
+                }
+            } else {
+                float *ob = d_q + (row0 + tq) * total + hoff;
+#pragma unroll
+                for (int dt = 0; dt < NDT; dt++)
+                    *reinterpret_cast<f32x4 *>(ob + 16 * dt + 4 * g) = (aq[qt][dt] - dsum * bq[qt][dt]) * scale;
+            }
         }
     }
 }
@@ -759,7 +771,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_q_blocked_kernel(const unsigne
 // accumulates d_v^T += dO^T w and d_k^T += Q^T dS.  The Q and dO rows of a stage are staged as they arrive (dO as
 // hi + lo); the products that contract over queries read them through ds_read_b64_tr_b16 in the query order
 // that the score tiles leave in the lanes.  K and V of the wave's keys sit in registers.
-template <int HDV>
+template <int HDV, bool OUT16>
 __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned short *__restrict__ q,
                                                                  const unsigned short *__restrict__ k,
                                                                  const unsigned short *__restrict__ v,
@@ -767,7 +779,7 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
                                                                  const float *__restrict__ d_out,
                                                                  const float *__restrict__ dvec,
                                                                  float *__restrict__ d_k, float *__restrict__ d_v,
-                                                                 int s, int H, int ws) {
+                                                                 int s, int H, int ws, Out16 o16) {
     __shared__ __align__(16) unsigned short Qs[2][KS][LDH], Dh[2][KS][LDH], Dl[2][KS][LDH];   // [query][dim]
     __shared__ __align__(16) float Mc[2][KS], Iv[2][KS], Dd[2][KS];   // the stage's queries: maximum, 1 / sum, D
     const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
@@ -902,6 +914,16 @@ __global__ __launch_bounds__(256, 2) void swa_bwd_k_stats_kernel(const unsigned 
     for (int jt = 0; jt < 2; jt++) {
         const int key = jlo + 16 * jt + r;
         if (key >= s) continue;
+        if (OUT16) {
+            unsigned short *pk = o16.k + (row0 + key) * o16.ld + hoff, *pv = o16.v + (row0 + key) * o16.ld + hoff;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++) {
+                const f32x4 a = dk[jt][dt], c = dv[jt][dt];
+                *reinterpret_cast<uint2 *>(pk + 16 * dt + 4 * g) = make_uint2(pack2(a[0], a[1]), pack2(a[2], a[3]));
+                *reinterpret_cast<uint2 *>(pv + 16 * dt + 4 * g) = make_uint2(pack2(c[0], c[1]), pack2(c[2], c[3]));
+            }
+            continue;
+        }
         float *pk = d_k + (row0 + key) * total + hoff, *pv = d_v + (row0 + key) * total + hoff;
 #pragma unroll
         for (int dt = 0; dt < NDT; dt++) {
@@ -1094,7 +1116,7 @@ bool swa_forward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, u
 
 bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, const uint16_t *attn_weights,
                        const float *d_attn_out, float *d_q, float *d_k, float *d_v, int seq_len, int num_heads,
-                       int head_dim, int window, int batch, int n_persistent, const float *stats) {
+                       int head_dim, int window, int batch, int n_persistent, const float *stats, const SwaGradCols *cols) {
     const ErrorScope es;
     if ((head_dim != 64 && head_dim != 32) || n_persistent != 0 || window > 512 || window < 1) return false;
     float *dvec = scratch(1, (size_t)batch * num_heads * seq_len * sizeof(float));
@@ -1102,22 +1124,26 @@ bool swa_backward_mfma(const uint16_t *q, const uint16_t *k, const uint16_t *v, 
     if (stats) {
         const float2 *st2 = reinterpret_cast<const float2 *>(stats);
         const dim3 grid((seq_len + FQ - 1) / FQ, num_heads, batch);
-        {
-            KernelTimer kt("swa_bwd_q_stats_kernel");
-            if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_q_stats_kernel<64>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, dvec,
-                               seq_len, num_heads, window);
-            else hipLaunchKernelGGL(swa_bwd_q_stats_kernel<32>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, dvec,
-                               seq_len, num_heads, window);
-            check_launch("swa_bwd_q_stats_kernel");
-        }
-        KernelTimer kt("swa_bwd_k_stats_kernel");
-        if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_k_stats_kernel<64>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec, d_k, d_v,
-                           seq_len, num_heads, window);
-        else hipLaunchKernelGGL(swa_bwd_k_stats_kernel<32>, grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec, d_k, d_v,
-                           seq_len, num_heads, window);
-        check_launch("swa_bwd_k_stats_kernel");
+        const Out16 o16 = cols ? Out16{cols->q, cols->k, cols->v, cols->ld} : Out16{nullptr, nullptr, nullptr, 0};
+#define NLH_SWA_BWD_STATS(HDV, O16)                                                                                       \
+    {                                                                                                                     \
+        {                                                                                                                 \
+            KernelTimer kt("swa_bwd_q_stats_kernel");                                                                     \
+            hipLaunchKernelGGL((swa_bwd_q_stats_kernel<HDV, O16>), grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, d_q, \
+                               dvec, seq_len, num_heads, window, o16);                                                    \
+            check_launch("swa_bwd_q_stats_kernel");                                                                       \
+        }                                                                                                                 \
+        KernelTimer kt("swa_bwd_k_stats_kernel");                                                                         \
+        hipLaunchKernelGGL((swa_bwd_k_stats_kernel<HDV, O16>), grid, dim3(256), 0, stream(), q, k, v, st2, d_attn_out, dvec,   \
+                           d_k, d_v, seq_len, num_heads, window, o16);                                                    \
+        check_launch("swa_bwd_k_stats_kernel");                                                                           \
+    }
+        if (head_dim == 64) { if (cols) NLH_SWA_BWD_STATS(64, true) else NLH_SWA_BWD_STATS(64, false) }
+        else { if (cols) NLH_SWA_BWD_STATS(32, true) else NLH_SWA_BWD_STATS(32, false) }
+#undef NLH_SWA_BWD_STATS
         return true;
     }
+    if (cols) return false;   // bf16 column output exists for the statistics pair only
     {
         KernelTimer kt("swa_bwd_q_blocked_kernel");
         if (head_dim == 64) hipLaunchKernelGGL(swa_bwd_q_blocked_kernel<64>, dim3((seq_len + FQ - 1) / FQ, num_heads, batch), dim3(256), 0,

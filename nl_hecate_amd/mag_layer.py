@@ -520,13 +520,17 @@ class MagLayer:
         d_attn, d_ycomb = _new(bs, s, d), _new(bs, s, d)
         lib.cms_gate_backward_bf16_rocm(d_gated.data_ptr(), c["attn"].data_ptr(), c["gate"].data_ptr(), k,
                                         d_attn.data_ptr(), d_ycomb.data_ptr(), n * d)
-        dq = _new(bs, s, d)
-        dkv = _zeros(2, bs, s, d)
-        D.call("swa_backward_lse_bf16_rocm", c["q"], c["k"], c["v"], c["aw"], d_attn, dq, dkv[0], dkv[1], s, nh, hd,
-               self.window, bs)
+        # the attention gradients go straight into their columns of the level step's bf16 GEMM operand
+        ld = ctypes.c_longlong(0)
+        g_op = lib.level_grad_operand_rocm(bs, s, nh, hd, na, 3, ctypes.byref(ld))
+        if not g_op:
+            raise RuntimeError("level_grad_operand_rocm failed")
+        lib.swa_backward_lse_bf16_cols_rocm(c["q"].data_ptr(), c["k"].data_ptr(), c["v"].data_ptr(), c["aw"].data_ptr(),
+                                            d_attn.data_ptr(), g_op, g_op + 2 * d, g_op + 4 * d, ld.value, s, nh, hd,
+                                            self.window, bs)
         d_x = _new(bs, s, d)
         seeds = _zeros(2, hd, hd)
-        d_extra = (ctypes.c_void_p * 3)(dq.data_ptr(), dkv[0].data_ptr(), dkv[1].data_ptr())
+        d_extra = (ctypes.c_void_p * 3)(None, None, None)
         gl = grads.levels[:na]
         gate_out = (ctypes.c_void_p * (6 * na))(*[t.data_ptr() for g in gl for t in
                                                   (g.w_alpha, g.b_alpha, g.w_theta, g.b_theta, g.w_eta, g.b_eta)])

@@ -146,6 +146,36 @@ def test_swa_without_weight_tensor(B, s, H, ws, hd):
     assert np.array_equal(host(dk), 2 * k1) and np.array_equal(host(dv), 2 * v1)
 
 
+@pytest.mark.parametrize("B,s,H,hd,ws", [(2, 200, 2, 64, 101), (1, 130, 4, 32, 64), (1, 600, 2, 64, 512)])
+def test_swa_backward_into_bf16_columns(B, s, H, hd, ws):
+    """The statistics backward that writes its gradients as bf16 into columns of a wider matrix: the same numbers as the
+    fp32 outputs rounded to bf16, bit for bit (the sums are the same, the rounding happens at the store); columns
+    between and around the three blocks are left alone."""
+    from nl_hecate_amd.ffi import lib
+    q, k, v, go = _case(B, s, H, hd, 900 + s + ws)
+    td = H * hd
+    out = torch.zeros(B, s, td, dtype=torch.uint16, device="cuda")
+    stats = torch.zeros(B, H, s, 2, device="cuda")
+    D.call("swa_forward_lse_bf16_rocm", _u16(q), _u16(k), _u16(v), out, stats, s, H, hd, ws, B)
+    dq, dk, dv = zeros(B, s, td), zeros(B, s, td), zeros(B, s, td)
+    god = dev(go)
+    D.call("swa_backward_lse_bf16_rocm", _u16(q), _u16(k), _u16(v), stats, god, dq, dk, dv, s, H, hd, ws, B)
+    ld = 3 * td + 24
+    G = _u16(np.full((B * s, ld), 0x7fc1, dtype=np.uint16))   # a NaN pattern: untouched columns keep it
+    qd, kd, vd = _u16(q), _u16(k), _u16(v)
+    base = G.data_ptr()
+    lib.swa_backward_lse_bf16_cols_rocm(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), stats.data_ptr(), god.data_ptr(),
+                                        base + 2 * 8, base + 2 * (8 + td), base + 2 * (16 + 2 * td), ld, s, H, hd, ws, B)
+    torch.cuda.synchronize()
+    Gh = G.cpu().numpy()
+    want = lambda t: t.reshape(B * s, td).to(torch.bfloat16).view(torch.uint16).cpu().numpy()
+    assert np.array_equal(Gh[:, 8:8 + td], want(dq))
+    assert np.array_equal(Gh[:, 8 + td:8 + 2 * td], want(dk))
+    assert np.array_equal(Gh[:, 16 + 2 * td:16 + 3 * td], want(dv))
+    for lo, hi in ((0, 8), (8 + 2 * td, 16 + 2 * td), (16 + 3 * td, ld)):
+        assert np.all(Gh[:, lo:hi] == 0x7fc1)
+
+
 def test_swa_without_weight_tensor_rejects_other_shapes():
     from nl_hecate_amd.ffi import lib
     z = torch.zeros(1, 8, 16, dtype=torch.uint16, device="cuda")
