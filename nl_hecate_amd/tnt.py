@@ -158,10 +158,14 @@ def gpu_tnt_forward(level_params, cfg: LevelConfig, embedded, context_m, s, d, b
 
 
 def gpu_tnt_backward(level_params, cfg: LevelConfig, cache: TntCache, d_y, embedded, level_grads: LevelGrads, s, d,
-                     batch_size):
+                     batch_size, per_head_memory_gradient=False):
     """d_y, embedded [s, d].  Adds the gate gradients of every retained shard into level_grads (zero them first),
     writes the projection gradients, returns d_embedded [s, d].  Shards whose inner caches were dropped pass
-    the global memory's gradient on and contribute nothing else."""
+    the global memory's gradient on and contribute nothing else.
+    per_head_memory_gradient=False is the reference's behaviour (the local chains' initial-memory gradients, summed
+    over all chains by the rule's backward, land on head 0: see the module text); True sends every chain's gradient
+    to its own head's global memory (the rule's segment backward over the whole chain returns it per chain), which
+    is the gradient of the forward for any number of heads."""
     lp, c, g = level_params, cache, level_grads
     if batch_size != 1:
         raise ValueError("TNT backward currently supports batch_size=1 only")
@@ -216,7 +220,16 @@ def gpu_tnt_backward(level_params, cfg: LevelConfig, cache: TntCache, d_y, embed
                 s_bw = _new(kb, cl + 1, dd)
                 rc = D.call("broadcast_fill_f32_cuda", s_bw, inner.s_states, dd, cl + 1, kb)
                 assert rc == 0, f"broadcast_fill S failed (rc={rc})"
-        if titans:
+        if per_head_memory_gradient:   # the segment form over the whole chain: d_m_out is per chain
+            seed = _zeros(kb, dd)
+            if titans:
+                D.titans_backward_dd_segment(inner.k_mem, inner.v_mem, inner.q_mem, inner.alpha, inner.theta, inner.eta,
+                                             m_bw, s_bw, d_y_b, seed, seed, dk, dv, dq, da, dth, de, d_m_initial,
+                                             _zeros(kb, dd), 0, cl, hd, kb, cl, clip)
+            else:
+                D.delta_backward_dd_segment(inner.k_mem, inner.v_mem, inner.q_mem, inner.alpha, inner.theta, m_bw, d_y_b,
+                                            seed, dk, dv, dq, da, dth, d_m_initial, 0, cl, hd, kb, cl, clip)
+        elif titans:
             D.titans_backward_dd(inner.k_mem, inner.v_mem, inner.q_mem, inner.alpha, inner.theta, inner.eta, m_bw, s_bw,
                                  d_y_b, dk, dv, dq, da, dth, de, d_m_initial, _zeros(kb, dd), cl, hd, kb, clip)
         else:

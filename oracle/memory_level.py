@@ -348,10 +348,11 @@ def tnt_forward(p, cfg, x, m0, cg, cl, gates=None):
     return y_full, shards, m_glob
 
 
-def tnt_backward(p, cfg, shards, d_y, x, cl, first_retained=0):
+def tnt_backward(p, cfg, shards, d_y, x, cl, first_retained=0, per_head_memory_gradient=False):
     """-> (grads, d_x).  The rule's backward returns the gradient of the initial memory summed over the chains of
     a call; as in the reference (gpu_backward.rs:1408-1418) the whole sum is added to head 0's global memory
-    gradient — the gradient itself for one head."""
+    gradient — the gradient itself for one head.  per_head_memory_gradient: every chain's gradient goes to its own
+    head's global memory instead, which is the gradient of the forward for any number of heads."""
     s, d = x.shape
     nh, hd = cfg.num_heads, cfg.head_dim
     dt = x.dtype
@@ -376,6 +377,7 @@ def tnt_backward(p, cfg, shards, d_y, x, cl, first_retained=0):
         dk, dv, dq = (np.zeros((nh, padded, hd), dt) for _ in range(3))
         da, dth, de = (np.zeros((nh, padded), dt) for _ in range(3))
         d_m_sum = np.zeros((hd, hd), dt)
+        d_m_head = np.zeros((nh, hd, hd), dt)
         for h in range(nh):
             for b in range(n_batch):
                 sl = slice(b * cl, (b + 1) * cl)
@@ -395,8 +397,12 @@ def tnt_backward(p, cfg, shards, d_y, x, cl, first_retained=0):
                 dk[h, sl], dv[h, sl], dq[h, sl] = gi["d_k"], gi["d_v"], gi["d_q"]
                 da[h, sl], dth[h, sl] = gi["d_alpha"], gi["d_theta"]
                 d_m_sum += gi["d_m"]
+                d_m_head[h] += gi["d_m"]
         if not cfg.proxy:
-            d_m_old[0] += d_m_sum
+            if per_head_memory_gradient:
+                d_m_old += d_m_head
+            else:
+                d_m_old[0] += d_m_sum
         ca, ct = _clamped(cfg)
         if ca:
             da = np.where((c["ah"] <= cfg.alpha_floor) | (c["ah"] >= cfg.alpha_ceil), 0.0, da)

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def run(cfg, s, cg, cl, seed, max_retained=None):
+def run(cfg, s, cg, cl, seed, max_retained=None, per_head=False):
     nh, hd = cfg.num_heads, cfg.head_dim
     d = nh * hd
     r = np.random.default_rng(seed)
@@ -27,12 +27,12 @@ def run(cfg, s, cg, cl, seed, max_retained=None):
     y_o, shards, m_fin = ML.tnt_forward(p, cfg, x, m0, cg, cl)
     n_shards = len(shards)
     first = 0 if max_retained is None else max(0, n_shards - max(1, max_retained))
-    g_o, dx_o = ML.tnt_backward(p, cfg, shards, dy, x, cl, first_retained=first)
+    g_o, dx_o = ML.tnt_backward(p, cfg, shards, dy, x, cl, first_retained=first, per_head_memory_gradient=per_head)
     lp = MemoryLevelParams(*[dev(p[n]) for n in NAMES])
     ctx, emb = dev(m0.reshape(nh, hd * hd)), dev(x)
     y, cache = TN.gpu_tnt_forward(lp, cfg, emb, ctx, s, d, 1, TN.ParallelConfig(cg, cl), max_retained)
     grads = GL.LevelGrads.zeros(d)
-    d_emb = TN.gpu_tnt_backward(lp, cfg, cache, dev(dy), emb, grads, s, d, 1)
+    d_emb = TN.gpu_tnt_backward(lp, cfg, cache, dev(dy), emb, grads, s, d, 1, per_head_memory_gradient=per_head)
     torch.cuda.synchronize()
     assert cache.total_shards == n_shards and cache.first_retained_shard == first
     assert len(cache.shard_inner_caches) == n_shards - first and len(cache.k_summaries) == n_shards
@@ -61,6 +61,15 @@ def test_forward_and_backward_match_the_composition(rule, nh, hd, s, cg, cl):
     inner = cache.shard_inner_caches[0]
     assert inner.kind == ("Titans" if rule == "titans" else "Delta") and not inner.proxy
     assert inner.m_states.shape == (nh * -(-min(cg, s) // cl), cl + 1, hd * hd)
+
+
+@pytest.mark.parametrize("rule", ["delta", "titans"])
+@pytest.mark.parametrize("nh,hd,s,cg,cl", [(2, 8, 22, 8, 3), (3, 8, 20, 5, 5)])
+def test_per_head_attribution_of_the_initial_memory_gradients(rule, nh, hd, s, cg, cl):
+    """The option that sends every local chain's initial-memory gradient to its own head (the gradient of the forward
+    for several heads: central differences of the float64 composition confirm it, tests/test_oracle_memory_level.py);
+    the default above is the reference's attribution to head 0."""
+    run(GL.LevelConfig(rule, nh, hd), s, cg, cl, 500 + s + hd, per_head=True)
 
 
 @pytest.mark.parametrize("rule", ["delta", "titans"])

@@ -163,12 +163,14 @@ def test_carried_memory_is_clamped():
     assert abs(np.sqrt((carried[0] ** 2).sum()) - 0.5) < 1e-12
 
 
-@pytest.mark.parametrize("rule", ["delta", "titans"])
-def test_tnt_backward_is_the_gradient_of_the_forward(rule):
-    """TNT level (shards of local chunks around a global memory), one head, float64: central differences of
+@pytest.mark.parametrize("rule,nh", [("delta", 1), ("titans", 1), ("delta", 3), ("titans", 2)])
+def test_tnt_backward_is_the_gradient_of_the_forward(rule, nh):
+    """TNT level (shards of local chunks around a global memory), float64: central differences of
     L = sum(y * dY) + sum(M_final * dM) are not needed — the reference's backward starts from a zero gradient of the
-    final global memory, so L = sum(y * dY).  Ragged last shard and a padded last local chunk included."""
-    nh, hd, s, cg, cl = 1, 4, 11, 4, 3        # shards of 4, 4, 3 tokens; local chunks of 3 (+ padding)
+    final global memory, so L = sum(y * dY).  Ragged last shard and a padded last local chunk included.
+    One head: the reference's attribution of the local chains' initial-memory gradients (all onto head 0) is the
+    gradient.  Several heads: it is not; the per-head attribution is, and that is what is checked there."""
+    hd, s, cg, cl = 4, 11, 4, 3        # shards of 4, 4, 3 tokens; local chunks of 3 (+ padding)
     d = nh * hd
     cfg = cfg_of(rule, nh, hd)
     r = np.random.default_rng(21)
@@ -178,7 +180,10 @@ def test_tnt_backward_is_the_gradient_of_the_forward(rule):
     dy = r.standard_normal((s, d))
     y, shards, m_fin = ML.tnt_forward(p, cfg, x, m0, cg, cl)
     assert len(shards) == 3 and shards[0]["padded"] == 6 and shards[2]["padded"] == 3
-    grads, d_x = ML.tnt_backward(p, cfg, shards, dy, x, cl)
+    grads, d_x = ML.tnt_backward(p, cfg, shards, dy, x, cl, per_head_memory_gradient=nh > 1)
+    if nh > 1:   # the reference's attribution differs from the gradient once there is a second head
+        ref_grads, _ = ML.tnt_backward(p, cfg, shards, dy, x, cl)
+        assert np.abs(ref_grads["w_k"] - grads["w_k"]).max() > 1e-6
     gates = [(c["alpha"], c["theta"], c["eta"]) for c in shards]
     eps = 1e-6
 
