@@ -128,7 +128,9 @@ __global__ __launch_bounds__(64 * kGateWaves) void cw_gates_sweep_kernel(
     float rho = 1.f, cc = 1.f, bb = 1.f, accA = 0.f, accE = 0.f;
     // row s seen from column 0: what it reads at t < s belongs to earlier rows and is weighted by zero
     const float *Ur = U + tri_row(lane) - lane, *Vr = V + tri_row(lane) - lane;
-#pragma unroll
+    // unrolled by 8 only: fully unrolled, the lane reads of both sweeps (four scalars per step) overflowed the scalar
+    // register file and were spilled
+#pragma unroll 8
     for (int t = 0; t < GW; t++) {
         const float kp = bcast(keep_l, t);
         const bool after = t > lane && t < L, on = t >= lane;   // tokens beyond a short chunk change no weight
