@@ -25,6 +25,7 @@
 #include "bf16_tiles.h"
 #include "chunk_coef.h"
 #include "chunkwise_chain.h"
+#include "lane_ops.h"
 #include "runtime.h"
 
 namespace nlh {
@@ -107,12 +108,13 @@ __global__ __launch_bounds__(64) void cw_coef_kernel(const float *__restrict__ a
 // for K, Q and W).  Waves 0..3 (group X): E, then Y^T, one 16-token strip each.  Waves 4..7
 // (group Y): one 32x32 block of W.P each, then one 16-column strip of the transposed state
 // update; they hold the fp32 master state.
-template <bool HAS_S>
+// TRACK: also leaves the per-token error norms and the chunk-start state norms of ChainTracks behind.
+template <bool HAS_S, bool TRACK>
 __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q,
     const float *__restrict__ table, const float *__restrict__ vecs, const float *__restrict__ m_initial,
     const float *__restrict__ s_initial, float *__restrict__ m_states, float *__restrict__ s_states,
-    float *__restrict__ y, int s, int C, int nc, int batch, HeadRows yr) {
+    float *__restrict__ y, int s, int C, int nc, int batch, HeadRows yr, ChainTracks tr) {
     constexpr int HMAT = 32 * LDB;   // a 32-row matrix
     extern __shared__ __align__(16) unsigned char smem_raw[];
     u16 *Kr = reinterpret_cast<u16 *>(smem_raw);   // K [t][c]
@@ -250,6 +252,20 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
         u16 *Qc = (c & 1) ? Qr1 : Qr0, *Kc = (c & 1) ? Kt1 : Kt0;
         u16 *Qn = (c & 1) ? Qr0 : Qr1, *Kn = (c & 1) ? Kt0 : Kt1;
         fetch(min(c + 1, nc - 1));
+        if (TRACK && !grpX) {   // sums of squares of this wave's part of the chunk-start states
+            float msq = 0.f, ssq = 0.f;
+#pragma unroll
+            for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    msq = fmaf(Mm[ct][e], Mm[ct][e], msq);
+                    if (HAS_S) ssq = fmaf(Sm[ct][e], Sm[ct][e], ssq);
+                }
+            msq = wave_allreduce(msq);
+            ssq = wave_allreduce(ssq);
+            if (l == 0)
+                *reinterpret_cast<float2 *>(tr.nrm + ((((size_t)chain * nc + c) * 2 + half) * 4 + bi) * 2) = make_float2(msq, ssq);
+        }
         // ── first half: E^T, (E.wM)^T, (E.wS)^T (group X) and W.P (group Y) ──
         if (grpX) {
             // E[t][i]: rows t = 16 bi .., columns i = 16 ct ..
@@ -257,6 +273,7 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
             const bf16x8 aV = ld_op(Kn, 16 * bi, 0);
             const f32x4 wm = *reinterpret_cast<const f32x4 *>(cvec + 2 * CW + 16 * bi + 4 * g);
             const f32x4 wsv = *reinterpret_cast<const f32x4 *>(cvec + 3 * CW + 16 * bi + 4 * g);
+            f32x4 esq = zero4();
 #pragma unroll
             for (int ct = 0; ct < 2; ct++) {
                 f32x4 e = zero4();
@@ -266,10 +283,17 @@ __global__ __launch_bounds__(kChainThr) void cw_chain_fwd_kernel(
                     e = mfma32(aK[ks], ld_op(Ml, 16 * ct, ks), e);
                 }
                 e = mfma32(aV, negI[ct], e);
+                if (TRACK) esq += e * e;
                 const int off = (16 * ct + r16) * LDB + 16 * bi + 4 * g;   // [i][t .. t+3]
                 split_store(Eh, El, off, e);
                 split_store(EMh, EMl, off, e * wm);
                 if (HAS_S) split_store(ESh, ESl, off, e * wsv);
+            }
+            if (TRACK) {   // a lane holds tokens 16 bi + 4 g .. + 3 of rows 16 ct + l % 16: sum over the 16 lanes of the group
+#pragma unroll
+                for (int e = 0; e < 4; e++) esq[e] = group_allreduce<16>(esq[e]);
+                if (r16 == 0)
+                    *reinterpret_cast<f32x4 *>(tr.e2 + (((size_t)chain * 2 + half) * nc + c) * CW + 16 * bi + 4 * g) = esq;
             }
         } else {
             bf16x8 aK[2][2];
@@ -374,14 +398,18 @@ constexpr size_t kChainFwdLds = (7 * BMAT + 10 * 32 * LDB) * sizeof(u16) + (4 * 
 template <bool HAS_S>
 void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, const float *alpha, const float *theta,
                     const float *eta, const float *m_initial, const float *s_initial, float *m_states,
-                    float *s_states, float *y, int seq_len, int batch, int chunk_size, const HeadRows &yr) {
+                    float *s_states, float *y, int seq_len, int batch, int chunk_size, const HeadRows &yr,
+                    const ChainTracks *tracks) {
     const ErrorScope es;
     const int nc = ceil_div(seq_len, chunk_size), nchunks = batch * nc;
     float *table = scratch(3, (size_t)nchunks * kTableFloats * sizeof(float));
     float *vecs = scratch(4, (size_t)nchunks * kVecFloats * sizeof(float));
     static bool attr_set = false;
     if (!attr_set) {
-        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_chain_fwd_kernel<HAS_S>),
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_chain_fwd_kernel<HAS_S, false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kChainFwdLds),
+                  "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_chain_fwd_kernel<HAS_S, true>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kChainFwdLds),
                   "dynamic LDS size");
         attr_set = true;
@@ -395,8 +423,14 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
     check_launch("cw_coef_kernel");
     {
         KernelTimer kt("cw_chain_fwd_kernel");
-        hipLaunchKernelGGL(cw_chain_fwd_kernel<HAS_S>, dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k, v, q,
-                           table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch, yr);
+        if (tracks)
+            hipLaunchKernelGGL((cw_chain_fwd_kernel<HAS_S, true>), dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k,
+                               v, q, table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch,
+                               yr, *tracks);
+        else
+            hipLaunchKernelGGL((cw_chain_fwd_kernel<HAS_S, false>), dim3(2 * batch), dim3(kChainThr), kChainFwdLds, stream(), k,
+                               v, q, table, vecs, m_initial, s_initial, m_states, s_states, y, seq_len, chunk_size, nc, batch,
+                               yr, ChainTracks{nullptr, nullptr});
     }
     check_launch(fn);
 }
@@ -406,15 +440,16 @@ void launch_forward(const char *fn, const u16 *k, const u16 *v, const u16 *q, co
 bool chunkwise_chain_forward_bf16(const char *fn, const uint16_t *k, const uint16_t *v, const uint16_t *q,
                                   const float *alpha, const float *theta, const float *eta, const float *m_initial,
                                   const float *s_initial, float *m_states, float *s_states, float *y, int seq_len,
-                                  int d, int batch, int chunk_size, bool has_s, const HeadRows *y_rows) {
+                                  int d, int batch, int chunk_size, bool has_s, const HeadRows *y_rows,
+                                  const ChainTracks *tracks) {
     if (d != HD || chunk_size < 1 || chunk_size > CW || seq_len <= 0 || batch <= 0) return false;
     const HeadRows yr = y_rows ? *y_rows : head_major_rows(seq_len, HD);
     if (has_s)
         launch_forward<true>(fn, k, v, q, alpha, theta, eta, m_initial, s_initial, m_states, s_states, y, seq_len,
-                             batch, chunk_size, yr);
+                             batch, chunk_size, yr, tracks);
     else
         launch_forward<false>(fn, k, v, q, alpha, theta, nullptr, m_initial, nullptr, m_states, nullptr, y, seq_len,
-                              batch, chunk_size, yr);
+                              batch, chunk_size, yr, tracks);
     return true;
 }
 

@@ -16,6 +16,7 @@
 #include <stdint.h>
 
 #include "../../include/nl_hecate_ffi.h"
+#include "chunkwise_chain.h"
 #include "chunkwise_guard.h"
 #include "lane_ops.h"
 #include "mm_tiles.h"
@@ -115,6 +116,59 @@ __global__ __launch_bounds__(kThr) void cw_guard_kernel(const TOK *__restrict__ 
     }
 }
 
+// The same test from what the bf16 forward chain kernel leaves behind (ChainTracks): per token the squared error
+// norm of each half of the memory rows, per chunk eight partial sums of squares of the chunk-start states.  One wave
+// per chunk, lane = token; reads k once for |k_t|.  The errors there were formed against a hi + lo bf16 copy of M0
+// (16 mantissa bits): |e_t| is raised by 2^-15 |M0|_F |k_t| to cover it.
+template <bool HAS_S>
+__global__ __launch_bounds__(256) void cw_guard_tracks_kernel(const uint16_t *__restrict__ k, const float *__restrict__ alpha,
+                                                              const float *__restrict__ theta, const float *__restrict__ eta,
+                                                              const float *__restrict__ e2, const float *__restrict__ nrm,
+                                                              int seq_len, int C, int nc, int nchunks, float clip, float mmax,
+                                                              int *__restrict__ flag) {
+    const int lane = threadIdx.x & 63, task = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (task >= nchunks) return;   // waves are independent: no barrier below
+    const int chain = task / nc, c = task % nc, t0 = c * C, L = min(C, seq_len - t0);
+    const bool in = lane < L;
+    const size_t tok = (size_t)chain * seq_len + t0 + lane;
+    float ksq = 0.f, esq = 0.f, al = 0.f, th = 0.f, et = 0.f;
+    if (in) {
+        const uint4 *row = reinterpret_cast<const uint4 *>(k + tok * HD);
+#pragma unroll
+        for (int i = 0; i < HD / 8; i++) {
+            const uint4 x = row[i];
+            const unsigned w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float lo = __uint_as_float(w[j] << 16), hi = __uint_as_float(w[j] & 0xffff0000u);
+                ksq = fmaf(lo, lo, fmaf(hi, hi, ksq));
+            }
+        }
+        esq = e2[(((size_t)chain * 2 + 0) * nc + c) * CW + lane] + e2[(((size_t)chain * 2 + 1) * nc + c) * CW + lane];
+        al = alpha[tok];
+        th = theta[tok];
+        if (HAS_S) et = eta[tok];
+    }
+    float2 part = make_float2(0.f, 0.f);
+    if (lane < 8) part = reinterpret_cast<const float2 *>(nrm)[((size_t)chain * nc + c) * 8 + lane];
+    float nM = sqrtf(wave_allreduce(part.x)) * kSlack;
+    float nS = HAS_S ? sqrtf(wave_allreduce(part.y)) * kSlack : 0.f;
+    const float kn = sqrtf(ksq) * kSlack;
+    const float en = sqrtf(esq) * kSlack + 3.0517578125e-5f * nM * kn;
+    const float drive = th * en * kn, keep = 1.0f - al;
+    const bool clip_on = clip > 0.f, proj_on = mmax > 0.f && mmax < 1e30f;
+    bool bad = clip_on && in && en > clip;
+    float worst = 0.f;
+#pragma unroll 8
+    for (int t = 0; t < CW; t++) {   // tokens beyond L carry keep = 1, eta = 0, no drive
+        nS = (HAS_S ? lane_value(et, t) * nS : 0.f) + lane_value(drive, t);
+        nM = lane_value(keep, t) * nM + nS;
+        worst = t < L ? fmaxf(worst, nM) : worst;
+    }
+    if (proj_on && worst * kSlack > mmax) bad = true;
+    if (bad) *flag = 1;
+}
+
 __global__ void guard_clear_kernel(int *flag) { *flag = 0; }
 
 int *g_host_flag = nullptr;
@@ -184,6 +238,32 @@ bool norm_bound_exceeded(const float *msq_part, int batch, int parts, float m_no
     return es.failed() || *g_host_flag != 0;
 }
 
+bool couplings_may_fire_tracked(const uint16_t *k, const float *alpha, const float *theta, const float *eta,
+                                const ChainTracks &tr, bool has_s, int seq_len, int batch, int chunk_size, float error_clip,
+                                float m_norm_max) {
+    const ErrorScope es;
+    int *flag = reinterpret_cast<int *>(scratch(31, 256));
+    if (!g_host_flag) check_hip(hipHostMalloc(reinterpret_cast<void **>(&g_host_flag), 256, hipHostMallocDefault), "hipHostMalloc");
+    if (es.failed() || !g_host_flag) return true;
+    const int nc = (seq_len + chunk_size - 1) / chunk_size, nchunks = batch * nc;
+    {
+        KernelTimer kt("cw_guard_tracks_kernel");
+        hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(1), 0, stream(), flag);
+        const dim3 grid((unsigned)((nchunks + 3) / 4));
+        if (has_s)
+            hipLaunchKernelGGL(cw_guard_tracks_kernel<true>, grid, dim3(256), 0, stream(), k, alpha, theta, eta, tr.e2, tr.nrm,
+                               seq_len, chunk_size, nc, nchunks, error_clip, m_norm_max, flag);
+        else
+            hipLaunchKernelGGL(cw_guard_tracks_kernel<false>, grid, dim3(256), 0, stream(), k, alpha, theta, eta, tr.e2, tr.nrm,
+                               seq_len, chunk_size, nc, nchunks, error_clip, m_norm_max, flag);
+        check_launch("cw_guard_tracks_kernel");
+    }
+    *g_host_flag = 1;
+    check_hip(hipMemcpyAsync(g_host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, stream()), "guard flag copy");
+    check_hip(hipStreamSynchronize(stream()), "guard flag sync");
+    return es.failed() || *g_host_flag != 0;
+}
+
 bool couplings_may_fire(const float *k, const float *v, const float *alpha, const float *theta, const float *eta,
                         const float *m_states, const float *s_states, int seq_len, int batch, int chunk_size,
                         float error_clip, float m_norm_max) {
@@ -225,7 +305,22 @@ void titans_chunkwise_forward_bf16_guarded_rocm(const uint16_t *k_mem, const uin
     const ErrorScope es;
     if (seq_len <= 0 || batch_size <= 0) return;
     const bool mm = d == 64 && chunk_size >= 1 && chunk_size <= 64;
-    if (mm && (!coupled(error_clip, m_norm_max) || guard_possible())) {
+    if (mm && coupled(error_clip, m_norm_max) && guard_possible()) {
+        // the chain kernel leaves the error and state norms behind as it goes: the test is then a scalar recurrence
+        const int nc = (seq_len + chunk_size - 1) / chunk_size;
+        const size_t e2_floats = (size_t)batch_size * 2 * nc * 64, nrm_floats = (size_t)batch_size * nc * 16;
+        float *buf = scratch(12, (e2_floats + nrm_floats) * sizeof(float));
+        if (es.failed()) return;
+        const ChainTracks tr{buf, buf + e2_floats};
+        if (chunkwise_chain_forward_bf16("titans_chunkwise_forward_bf16_guarded_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
+                                         m_initial, s_initial, m_chunk_states, s_chunk_states, y, seq_len, d, batch_size,
+                                         chunk_size, true, nullptr, &tr)) {
+            if (es.failed()) return;
+            if (!couplings_may_fire_tracked(k_mem, alpha, theta, eta, tr, true, seq_len, batch_size, chunk_size, error_clip,
+                                            m_norm_max))
+                return;
+        }
+    } else if (mm && (!coupled(error_clip, m_norm_max) || guard_possible())) {
         titans_chunkwise_forward_bf16_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial, m_chunk_states,
                                            s_chunk_states, y, seq_len, d, batch_size, chunk_size);
         if (es.failed()) return;
