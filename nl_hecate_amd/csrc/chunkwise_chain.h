@@ -21,4 +21,20 @@ bool chunkwise_chain_forward_bf16(const char *fn, const uint16_t *k, const uint1
                                   int d, int batch, int chunk_size, bool has_s, const HeadRows *y_rows = nullptr,
                                   const ChainTracks *tracks = nullptr);
 
+// The float-token matrix form (chunkwise_mm.hip) with the same side outputs; eta / s_initial / s_states null without
+// momentum.
+void chunkwise_forward_mm_f32_tracked(const char *fn, const float *k, const float *v, const float *q, const float *alpha,
+                                      const float *theta, const float *eta, const float *m_initial, const float *s_initial,
+                                      float *m_states, float *s_states, float *y, int seq_len, int d, int batch,
+                                      int chunk_size, bool has_s, const ChainTracks &tracks);
+
+// The float-token matrix-form backward whose gradient pass leaves the same side outputs and which ends with the test
+// of the couplings on them, before anything is added to d_m_initial / d_s_initial.  false: a coupling may have
+// fired; the caller runs the sequential kernels, which overwrite every other output.
+bool chunkwise_backward_mm_f32_guarded(const char *fn, const float *k, const float *v, const float *q, const float *alpha,
+                                       const float *theta, const float *eta, const float *m_states, const float *s_states,
+                                       const float *d_y, float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta,
+                                       float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d, int batch,
+                                       int chunk_size, bool has_s, float error_clip, float m_norm_max);
+
 }  // namespace nlh

@@ -29,6 +29,14 @@ using namespace mmt;
 
 constexpr float kSlack = 1.0f + 1e-4f;   // covers the rounding of the fp32 sums below
 
+// four consecutive elements of a token row as floats
+__device__ __forceinline__ float4 tok4(const float *p, size_t i) { return *reinterpret_cast<const float4 *>(p + i); }
+__device__ __forceinline__ float4 tok4(const uint16_t *p, size_t i) {
+    const uint2 u = *reinterpret_cast<const uint2 *>(p + i);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                       __uint_as_float(u.y & 0xffff0000u));
+}
+
 __device__ __forceinline__ float lane_value(float x, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
 }
@@ -120,12 +128,12 @@ __global__ __launch_bounds__(kThr) void cw_guard_kernel(const TOK *__restrict__ 
 // norm of each half of the memory rows, per chunk eight partial sums of squares of the chunk-start states.  One wave
 // per chunk, lane = token; reads k once for |k_t|.  The errors there were formed against a hi + lo bf16 copy of M0
 // (16 mantissa bits): |e_t| is raised by 2^-15 |M0|_F |k_t| to cover it.
-template <bool HAS_S>
-__global__ __launch_bounds__(256) void cw_guard_tracks_kernel(const uint16_t *__restrict__ k, const float *__restrict__ alpha,
+template <typename TOK, bool HAS_S>
+__global__ __launch_bounds__(256) void cw_guard_tracks_kernel(const TOK *__restrict__ k, const float *__restrict__ alpha,
                                                               const float *__restrict__ theta, const float *__restrict__ eta,
                                                               const float *__restrict__ e2, const float *__restrict__ nrm,
                                                               int seq_len, int C, int nc, int nchunks, float clip, float mmax,
-                                                              int *__restrict__ flag) {
+                                                              float split_slack, int *__restrict__ flag) {
     const int lane = threadIdx.x & 63, task = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (task >= nchunks) return;   // waves are independent: no barrier below
     const int chain = task / nc, c = task % nc, t0 = c * C, L = min(C, seq_len - t0);
@@ -133,16 +141,10 @@ __global__ __launch_bounds__(256) void cw_guard_tracks_kernel(const uint16_t *__
     const size_t tok = (size_t)chain * seq_len + t0 + lane;
     float ksq = 0.f, esq = 0.f, al = 0.f, th = 0.f, et = 0.f;
     if (in) {
-        const uint4 *row = reinterpret_cast<const uint4 *>(k + tok * HD);
 #pragma unroll
-        for (int i = 0; i < HD / 8; i++) {
-            const uint4 x = row[i];
-            const unsigned w[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float lo = __uint_as_float(w[j] << 16), hi = __uint_as_float(w[j] & 0xffff0000u);
-                ksq = fmaf(lo, lo, fmaf(hi, hi, ksq));
-            }
+        for (int i = 0; i < HD / 4; i++) {
+            const float4 x = tok4(k, tok * HD + 4 * i);
+            ksq += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
         }
         esq = e2[(((size_t)chain * 2 + 0) * nc + c) * CW + lane] + e2[(((size_t)chain * 2 + 1) * nc + c) * CW + lane];
         al = alpha[tok];
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(256) void cw_guard_tracks_kernel(const uint16_t *__
     float nM = sqrtf(wave_allreduce(part.x)) * kSlack;
     float nS = HAS_S ? sqrtf(wave_allreduce(part.y)) * kSlack : 0.f;
     const float kn = sqrtf(ksq) * kSlack;
-    const float en = sqrtf(esq) * kSlack + 3.0517578125e-5f * nM * kn;
+    const float en = sqrtf(esq) * kSlack + split_slack * nM * kn;
     const float drive = th * en * kn, keep = 1.0f - al;
     const bool clip_on = clip > 0.f, proj_on = mmax > 0.f && mmax < 1e30f;
     bool bad = clip_on && in && en > clip;
@@ -176,6 +178,7 @@ int *g_host_flag = nullptr;
 }  // namespace
 
 bool force_sequential = false;
+bool last_test_fired = false;
 
 bool guard_possible() {
     if (force_sequential) return false;
@@ -207,7 +210,8 @@ static bool couplings_may_fire_t(const TOK *k, const TOK *v, const float *alpha,
     *g_host_flag = 1;
     check_hip(hipMemcpyAsync(g_host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, stream()), "guard flag copy");
     check_hip(hipStreamSynchronize(stream()), "guard flag sync");
-    return es.failed() || *g_host_flag != 0;
+    last_test_fired = es.failed() || *g_host_flag != 0;
+    return last_test_fired;
 }
 
 namespace {
@@ -235,12 +239,14 @@ bool norm_bound_exceeded(const float *msq_part, int batch, int parts, float m_no
     *g_host_flag = 1;
     check_hip(hipMemcpyAsync(g_host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, stream()), "guard flag copy");
     check_hip(hipStreamSynchronize(stream()), "guard flag sync");
-    return es.failed() || *g_host_flag != 0;
+    last_test_fired = es.failed() || *g_host_flag != 0;
+    return last_test_fired;
 }
 
-bool couplings_may_fire_tracked(const uint16_t *k, const float *alpha, const float *theta, const float *eta,
-                                const ChainTracks &tr, bool has_s, int seq_len, int batch, int chunk_size, float error_clip,
-                                float m_norm_max) {
+template <typename TOK>
+static bool tracked_test(const TOK *k, const float *alpha, const float *theta, const float *eta, const ChainTracks &tr,
+                         bool has_s, int seq_len, int batch, int chunk_size, float error_clip, float m_norm_max,
+                         float split_slack) {
     const ErrorScope es;
     int *flag = reinterpret_cast<int *>(scratch(31, 256));
     if (!g_host_flag) check_hip(hipHostMalloc(reinterpret_cast<void **>(&g_host_flag), 256, hipHostMallocDefault), "hipHostMalloc");
@@ -251,17 +257,37 @@ bool couplings_may_fire_tracked(const uint16_t *k, const float *alpha, const flo
         hipLaunchKernelGGL(guard_clear_kernel, dim3(1), dim3(1), 0, stream(), flag);
         const dim3 grid((unsigned)((nchunks + 3) / 4));
         if (has_s)
-            hipLaunchKernelGGL(cw_guard_tracks_kernel<true>, grid, dim3(256), 0, stream(), k, alpha, theta, eta, tr.e2, tr.nrm,
-                               seq_len, chunk_size, nc, nchunks, error_clip, m_norm_max, flag);
+            hipLaunchKernelGGL((cw_guard_tracks_kernel<TOK, true>), grid, dim3(256), 0, stream(), k, alpha, theta, eta, tr.e2,
+                               tr.nrm, seq_len, chunk_size, nc, nchunks, error_clip, m_norm_max, split_slack, flag);
         else
-            hipLaunchKernelGGL(cw_guard_tracks_kernel<false>, grid, dim3(256), 0, stream(), k, alpha, theta, eta, tr.e2, tr.nrm,
-                               seq_len, chunk_size, nc, nchunks, error_clip, m_norm_max, flag);
+            hipLaunchKernelGGL((cw_guard_tracks_kernel<TOK, false>), grid, dim3(256), 0, stream(), k, alpha, theta, eta, tr.e2,
+                               tr.nrm, seq_len, chunk_size, nc, nchunks, error_clip, m_norm_max, split_slack, flag);
         check_launch("cw_guard_tracks_kernel");
     }
     *g_host_flag = 1;
     check_hip(hipMemcpyAsync(g_host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, stream()), "guard flag copy");
     check_hip(hipStreamSynchronize(stream()), "guard flag sync");
-    return es.failed() || *g_host_flag != 0;
+    last_test_fired = es.failed() || *g_host_flag != 0;
+    return last_test_fired;
+}
+
+ChainTracks chain_tracks(int seq_len, int batch, int chunk_size) {
+    const int nc = (seq_len + chunk_size - 1) / chunk_size;
+    const size_t e2_floats = (size_t)batch * 2 * nc * 64, nrm_floats = (size_t)batch * nc * 16;
+    float *buf = scratch(12, (e2_floats + nrm_floats) * sizeof(float));
+    return ChainTracks{buf, buf ? buf + e2_floats : nullptr};
+}
+
+// bf16 tokens: the errors were formed against a hi + lo bf16 copy of M0, hence the 2^-15 |M0|_F |k_t| on top
+bool couplings_may_fire_tracked(const uint16_t *k, const float *alpha, const float *theta, const float *eta,
+                                const ChainTracks &tr, bool has_s, int seq_len, int batch, int chunk_size, float error_clip,
+                                float m_norm_max) {
+    return tracked_test(k, alpha, theta, eta, tr, has_s, seq_len, batch, chunk_size, error_clip, m_norm_max, 3.0517578125e-5f);
+}
+bool couplings_may_fire_tracked(const float *k, const float *alpha, const float *theta, const float *eta,
+                                const ChainTracks &tr, bool has_s, int seq_len, int batch, int chunk_size, float error_clip,
+                                float m_norm_max) {
+    return tracked_test(k, alpha, theta, eta, tr, has_s, seq_len, batch, chunk_size, error_clip, m_norm_max, 0.f);
 }
 
 bool couplings_may_fire(const float *k, const float *v, const float *alpha, const float *theta, const float *eta,
@@ -307,11 +333,8 @@ void titans_chunkwise_forward_bf16_guarded_rocm(const uint16_t *k_mem, const uin
     const bool mm = d == 64 && chunk_size >= 1 && chunk_size <= 64;
     if (mm && coupled(error_clip, m_norm_max) && guard_possible()) {
         // the chain kernel leaves the error and state norms behind as it goes: the test is then a scalar recurrence
-        const int nc = (seq_len + chunk_size - 1) / chunk_size;
-        const size_t e2_floats = (size_t)batch_size * 2 * nc * 64, nrm_floats = (size_t)batch_size * nc * 16;
-        float *buf = scratch(12, (e2_floats + nrm_floats) * sizeof(float));
+        const ChainTracks tr = chain_tracks(seq_len, batch_size, chunk_size);
         if (es.failed()) return;
-        const ChainTracks tr{buf, buf + e2_floats};
         if (chunkwise_chain_forward_bf16("titans_chunkwise_forward_bf16_guarded_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
                                          m_initial, s_initial, m_chunk_states, s_chunk_states, y, seq_len, d, batch_size,
                                          chunk_size, true, nullptr, &tr)) {

@@ -31,6 +31,7 @@
 #include "../../include/nl_hecate_ffi.h"
 #include "chunkwise_chain.h"
 #include "chunkwise_grads.h"
+#include "chunkwise_guard.h"
 #include "mm_tiles.h"
 #include "rule_common.h"
 #include "runtime.h"
@@ -276,7 +277,9 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
 }
 
 // ── pass 3 (forward): outputs of one chunk ──────────────────────────────────
-template <class TIn>
+// TRACK: also leaves the ChainTracks of chunkwise_chain.h behind (per-token squared error norms per half of the
+// memory rows, eight partial sums of squares of the chunk-start states per chunk).
+template <class TIn, bool TRACK>
 __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict__ k, const TIn *__restrict__ v,
                                                           const TIn *__restrict__ q,
                                                           const float *__restrict__ alpha,
@@ -285,7 +288,7 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
                                                           const float *__restrict__ m_states,
                                                           const float *__restrict__ s_states,
                                                           float *__restrict__ y, int s, int C, int nc, int has_s,
-                                                          int ntask) {
+                                                          int ntask, ChainTracks tr) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Es = Qs + MAT, *Ms = Es + MAT, *Ss = Ms + MAT, *Cc = Ss + MAT;
     __shared__ Coef cf;
@@ -319,6 +322,18 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
     commit(Es, tv);
     commit(Ms, tm);
     if (has_s) commit(Ss, ts);
+    if (TRACK) {   // this wave's share of the sums of squares of the chunk-start states, from the staged registers
+        float msq = 0.f, ssq = 0.f;
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            msq += tm.x[it].x * tm.x[it].x + tm.x[it].y * tm.x[it].y + tm.x[it].z * tm.x[it].z + tm.x[it].w * tm.x[it].w;
+            if (has_s) ssq += ts.x[it].x * ts.x[it].x + ts.x[it].y * ts.x[it].y + ts.x[it].z * ts.x[it].z + ts.x[it].w * ts.x[it].w;
+        }
+        msq = wave_allreduce(msq);
+        ssq = wave_allreduce(ssq);
+        if ((threadIdx.x & 63) == 0)
+            *reinterpret_cast<float2 *>(tr.nrm + (((size_t)chain * nc + ci) * 8 + w) * 2) = make_float2(msq, ssq);
+    }
     __syncthreads();
     if (task + 1 < task_hi) fetch_task(task + 1);
     {
@@ -329,8 +344,17 @@ __global__ __launch_bounds__(kThr) void cw_out_fwd_kernel(const TIn *__restrict_
         // P[t][j] = sum_k Q[t][k] K[j][k];  Pw = W.P over the coefficient matrix, W[t][j] = -theta_j c[t][j]
         mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; },
             [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-        for_c(e, [&](int r, int c, float &x) { float *d = Es + (m0 + r) * LDM + n0 + c; *d = x - *d; });
+        for_c(e, [&](int r, int c, float &x) { float *d = Es + (m0 + r) * LDM + n0 + c; x -= *d; *d = x; });
         for_c(p, [&](int r, int c, float &x) { float *d = Cc + (m0 + r) * LDM + n0 + c; *d = -cf.th[n0 + c] * *d * x; });
+        if (TRACK) {   // squared error norm of the strip's 16 tokens over its 32 memory rows
+            for_c(e, [&](int, int, float &x) { x *= x; });
+            strip_row_sums(e);
+            if (row_writer()) {
+                float *eo = tr.e2 + (((size_t)chain * 2 + nh) * nc + ci) * CW + m0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) eo[row_of(i)] = e.t[0][i];
+            }
+        }
     }
     __syncthreads();
     const float *Pw = Cc;
@@ -477,14 +501,14 @@ __global__ __launch_bounds__(256) void cw_state_dots_kernel(const float *__restr
 
 // ── backward, main per-chunk pass: dQ, dK, dV, dtheta; exports for the gate pass ──
 //   pvec [chain][token][4] = p0, ps, -theta g1, -theta g2   xs [chain][chunk][j][t] = -theta_j (dy_t.e_j)(q_t.k_j)
-template <class TIn>
+template <class TIn, bool TRACK>
 __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     const TIn *__restrict__ k, const TIn *__restrict__ v, const TIn *__restrict__ q, const float *__restrict__ d_y,
     const float *__restrict__ alpha, const float *__restrict__ theta, const float *__restrict__ eta,
     const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
     const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, int s, int C, int nc,
-    int has_s, int ntask) {
+    int has_s, int ntask, ChainTracks tr) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Es = Ds + MAT, *Ms = Es + MAT, *B5 = Ms + MAT,
           *B6 = B5 + MAT, *B7 = B6 + MAT, *B8 = B7 + MAT;
@@ -524,6 +548,18 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     commit(Ds, td);
     commit(Ms, tm);
     if (has_s) commit(Ss, ts);
+    if (TRACK) {   // as in cw_out_fwd_kernel: the chunk-start states' sums of squares, then the error norms below
+        float msq = 0.f, ssq = 0.f;
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            msq += tm.x[it].x * tm.x[it].x + tm.x[it].y * tm.x[it].y + tm.x[it].z * tm.x[it].z + tm.x[it].w * tm.x[it].w;
+            if (has_s) ssq += ts.x[it].x * ts.x[it].x + ts.x[it].y * ts.x[it].y + ts.x[it].z * ts.x[it].z + ts.x[it].w * ts.x[it].w;
+        }
+        msq = wave_allreduce(msq);
+        ssq = wave_allreduce(ssq);
+        if ((threadIdx.x & 63) == 0)
+            *reinterpret_cast<float2 *>(tr.nrm + (((size_t)chain * nc + ci) * 8 + w) * 2) = make_float2(msq, ssq);
+    }
     __syncthreads();
     auto publish = [&](int which, Strip &x) {   // row sums of x -> part[which][column half][row]
         strip_row_sums(x);
@@ -544,7 +580,16 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
         if (has_s)
             mma(ys, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; },
                 [&](int kk, int n) { return Ss[kk * LDM + n0 + n]; });
-        for_c(e, [&](int r, int c, float &x) { float *d = Es + (m0 + r) * LDM + n0 + c; *d = x - *d; });
+        for_c(e, [&](int r, int c, float &x) { float *d = Es + (m0 + r) * LDM + n0 + c; x -= *d; *d = x; });
+        if (TRACK) {
+            for_c(e, [&](int, int, float &x) { x *= x; });
+            strip_row_sums(e);
+            if (row_writer()) {
+                float *eo = tr.e2 + (((size_t)chain * 2 + nh) * nc + ci) * CW + m0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) eo[row_of(i)] = e.t[0][i];
+            }
+        }
 #pragma unroll
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
@@ -700,7 +745,7 @@ bool check_mm_args(const char *fn, int seq_len, int d, int batch, int chunk_size
 template <class TIn>
 void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const float *alpha, const float *theta,
                 const float *eta, const float *m_initial, const float *s_initial, float *m_states, float *s_states,
-                float *y, int seq_len, int d, int batch, int chunk_size, bool has_s) {
+                float *y, int seq_len, int d, int batch, int chunk_size, bool has_s, const ChainTracks *tracks = nullptr) {
     const ErrorScope es;
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
     const int nc = ceil_div(seq_len, chunk_size);
@@ -709,9 +754,13 @@ void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const 
     static bool attr_set = false;
     if (!attr_set) {
         const size_t lds = kOutFwdLds;
-        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<float>),
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<float, false>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "dynamic LDS size");
-        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<uint16_t>),
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<float, true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<uint16_t, false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "dynamic LDS size");
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(cw_out_fwd_kernel<uint16_t, true>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "dynamic LDS size");
         attr_set = true;
     }
@@ -721,9 +770,14 @@ void forward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const 
     hipLaunchKernelGGL((cw_scan_kernel<true>), dim3(batch * 2), dim3(kThr), 0, stream(), m_initial, s_initial,
                        sc.loc, sc.locs, m_states, has_s ? s_states : nullptr, nc, (int)has_s);
     check_launch("cw_scan_kernel");
-    hipLaunchKernelGGL((cw_out_fwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kOutFwdLds,
-                       stream(), k, v, q, alpha, theta, eta, m_states, s_states, y, seq_len, chunk_size, nc,
-                       (int)has_s, batch * nc);
+    if (tracks)
+        hipLaunchKernelGGL((cw_out_fwd_kernel<TIn, true>), dim3(persistent_grid(batch * nc)), dim3(kThr), kOutFwdLds,
+                           stream(), k, v, q, alpha, theta, eta, m_states, s_states, y, seq_len, chunk_size, nc,
+                           (int)has_s, batch * nc, *tracks);
+    else
+        hipLaunchKernelGGL((cw_out_fwd_kernel<TIn, false>), dim3(persistent_grid(batch * nc)), dim3(kThr), kOutFwdLds,
+                           stream(), k, v, q, alpha, theta, eta, m_states, s_states, y, seq_len, chunk_size, nc,
+                           (int)has_s, batch * nc, ChainTracks{nullptr, nullptr});
     check_launch("cw_out_fwd_kernel");
 }
 
@@ -733,16 +787,23 @@ void set_lds(K kernel, size_t bytes) {
                                   (int)bytes), "dynamic LDS size");
 }
 
+// guard (float tokens only): the gradient pass also leaves the ChainTracks behind, and the call ends with the test of
+// the reference's couplings on them BEFORE anything is added to d_m_initial / d_s_initial; false: a coupling may have
+// fired, the caller runs the sequential kernels, which overwrite every other output.
+struct BackwardGuard { float error_clip, m_norm_max; };
 template <class TIn>
-void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const float *alpha, const float *theta,
+bool backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const float *alpha, const float *theta,
                  const float *eta, const float *m_states, const float *s_states, const float *d_y, float *d_k,
                  float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                  float *d_s_initial, int seq_len, int d, int batch, int chunk_size, bool has_s,
-                 const HeadRows *dy_rows = nullptr, const GradOut16 *out16 = nullptr) {
+                 const HeadRows *dy_rows = nullptr, const GradOut16 *out16 = nullptr, const BackwardGuard *guard = nullptr) {
     const ErrorScope es;
-    if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return;
-    if (out16 && sizeof(TIn) != 2) { fail("%s: bf16 gradient slabs are served for bf16 tokens only.", fn); return; }
-    if (dy_rows && sizeof(TIn) != 2) { fail("%s: token-major d_y is served for bf16 tokens only.", fn); return; }
+    if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return true;
+    if (out16 && sizeof(TIn) != 2) { fail("%s: bf16 gradient slabs are served for bf16 tokens only.", fn); return true; }
+    if (dy_rows && sizeof(TIn) != 2) { fail("%s: token-major d_y is served for bf16 tokens only.", fn); return true; }
+    if (guard && sizeof(TIn) != 4) { fail("%s: the in-pass test is served for float tokens only.", fn); return true; }
+    ChainTracks tracks{nullptr, nullptr};
+    if (guard) tracks = chain_tracks(seq_len, batch, chunk_size);
     const int nc = ceil_div(seq_len, chunk_size);
     Scratch sc{nullptr, nullptr};
     if constexpr (sizeof(TIn) == 4) sc = local_scratch(batch, nc);
@@ -755,13 +816,14 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     float *xs = scratch(7, (size_t)batch * nc * CW * CW * sizeof(float));
     float *pvec = scratch(8, (size_t)batch * seq_len * 4 * sizeof(float));
     float *scal = scratch(9, (size_t)batch * nc * 4 * sizeof(float));
-    if (es.failed()) return;
+    if (es.failed()) return true;
     static bool attr_set = false;
     if (!attr_set) {
         set_lds(cw_local_bwd_kernel<float>, kLocalBwdLds);
         set_lds(cw_local_bwd_kernel<uint16_t>, kLocalBwdLds);
-        set_lds(cw_grads_bwd_kernel<float>, kGradsBwdLds);
-        set_lds(cw_grads_bwd_kernel<uint16_t>, kGradsBwdLds);
+        set_lds(cw_grads_bwd_kernel<float, false>, kGradsBwdLds);
+        set_lds(cw_grads_bwd_kernel<float, true>, kGradsBwdLds);
+        set_lds(cw_grads_bwd_kernel<uint16_t, false>, kGradsBwdLds);
         attr_set = true;
     }
     if constexpr (sizeof(TIn) == 2) {
@@ -769,7 +831,7 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         const size_t nchunks = (size_t)batch * nc;
         float *tab_b = scratch(13, nchunks * chunkwise_grads_table_floats() * sizeof(float));
         float *vecs = scratch(14, nchunks * chunkwise_grads_vec_floats() * sizeof(float));
-        if (es.failed()) return;
+        if (es.failed()) return true;
         chunkwise_backward_coefficients(alpha, theta, eta, tab_b, vecs, seq_len, batch, chunk_size, has_s);
         uint16_t *dm_snap = reinterpret_cast<uint16_t *>(dm_states), *ds_snap = reinterpret_cast<uint16_t *>(ds_states);
         chunkwise_adjoint_bf16(k, q, d_y, tab_b, vecs, dm_snap, ds_snap, reinterpret_cast<float *>(dm_snap + n_snap),
@@ -789,9 +851,16 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                            dm_states, ds_states, scal, nc, (int)has_s);
         check_launch("cw_state_dots_kernel");
         KernelTimer kt("cw_grads_bwd_kernel");
-        hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn>), dim3(batch * nc), dim3(kThr), kGradsBwdLds,
-                           stream(), k, v, q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k,
-                           d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc);
+        if (guard)
+            hipLaunchKernelGGL((cw_grads_bwd_kernel<float, true>), dim3(batch * nc), dim3(kThr), kGradsBwdLds, stream(),
+                               reinterpret_cast<const float *>(k), reinterpret_cast<const float *>(v),
+                               reinterpret_cast<const float *>(q), d_y, alpha, theta, eta, m_states, s_states, dm_states,
+                               ds_states, d_k, d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc,
+                               tracks);
+        else
+            hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn, false>), dim3(batch * nc), dim3(kThr), kGradsBwdLds, stream(), k, v,
+                               q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta,
+                               pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc, ChainTracks{nullptr, nullptr});
         check_launch("cw_grads_bwd_kernel");
     }
     const bool packed = sizeof(TIn) == 2;   // where the gradient of the initial state sits (see above)
@@ -803,17 +872,40 @@ void backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     const int per = 8, rows = ceil_div(batch, per);
     const int nsum = has_s && d_s_initial ? 2 : 1;
     float *tmp = scratch(10, (size_t)nsum * rows * HD * HD * sizeof(float));
-    if (es.failed()) return;
+    if (es.failed()) return true;
     // d_alpha, d_eta, and in the same launch the first stage of the deterministic sum of d_m_initial, d_s_initial
     chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s, dm_first,
                              ds_first, chain_stride, per, nsum, tmp);
+    if (guard && couplings_may_fire_tracked(reinterpret_cast<const float *>(k), alpha, theta, eta, tracks, has_s, seq_len, batch,
+                                            chunk_size, guard->error_clip, guard->m_norm_max))
+        return false;
     KernelTimer kt("cw_add_rows_kernel");
     hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256, 1, nsum), dim3(256), 0, stream(), tmp, d_m_initial,
                        d_s_initial, rows);
     check_launch("cw_add_rows_kernel");
+    return true;
 }
 
 }  // namespace
+
+void chunkwise_forward_mm_f32_tracked(const char *fn, const float *k, const float *v, const float *q, const float *alpha,
+                                      const float *theta, const float *eta, const float *m_initial, const float *s_initial,
+                                      float *m_states, float *s_states, float *y, int seq_len, int d, int batch,
+                                      int chunk_size, bool has_s, const ChainTracks &tracks) {
+    forward_mm<float>(fn, k, v, q, alpha, theta, eta, m_initial, s_initial, m_states, s_states, y, seq_len, d, batch,
+                      chunk_size, has_s, &tracks);
+}
+
+bool chunkwise_backward_mm_f32_guarded(const char *fn, const float *k, const float *v, const float *q, const float *alpha,
+                                       const float *theta, const float *eta, const float *m_states, const float *s_states,
+                                       const float *d_y, float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta,
+                                       float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d, int batch,
+                                       int chunk_size, bool has_s, float error_clip, float m_norm_max) {
+    const BackwardGuard g{error_clip, m_norm_max};
+    return backward_mm<float>(fn, k, v, q, alpha, theta, eta, m_states, s_states, d_y, d_k, d_v, d_q, d_alpha, d_theta, d_eta,
+                              d_m_initial, d_s_initial, seq_len, d, batch, chunk_size, has_s, nullptr, nullptr, &g);
+}
+
 }  // namespace nlh
 
 using namespace nlh;

@@ -1173,10 +1173,12 @@ void titans_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, c
     if (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max)) {
         // the matrix form first: its chunk-start states are what the test needs; kept when no coupling can fire
         const ErrorScope es;
-        titans_chunkwise_forward_mm_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial,
-                                             m_chunk_states, s_chunk_states, y, seq_len, d, batch_size, chunk_size);
-        if (!es.failed() && !couplings_may_fire(k_mem, v_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, seq_len,
-                                                batch_size, chunk_size, error_clip, m_norm_max))
+        const ChainTracks tr = chain_tracks(seq_len, batch_size, chunk_size);
+        if (es.failed()) return;
+        chunkwise_forward_mm_f32_tracked(fn, k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial, m_chunk_states,
+                                         s_chunk_states, y, seq_len, d, batch_size, chunk_size, true, tr);
+        if (!es.failed() && !couplings_may_fire_tracked(k_mem, alpha, theta, eta, tr, true, seq_len, batch_size, chunk_size,
+                                                        error_clip, m_norm_max))
             return;
     }
     FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, eta, m_initial, s_initial,
@@ -1201,10 +1203,12 @@ void delta_chunkwise_forward_f32_cuda(const float *k_mem, const float *v_mem, co
     }
     if (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max)) {
         const ErrorScope es;
-        delta_chunkwise_forward_mm_f32_rocm(k_mem, v_mem, q_mem, alpha, theta, m_initial, m_chunk_states, y,
-                                            seq_len, d, batch_size, chunk_size);
-        if (!es.failed() && !couplings_may_fire(k_mem, v_mem, alpha, theta, nullptr, m_chunk_states, nullptr, seq_len,
-                                                batch_size, chunk_size, error_clip, m_norm_max))
+        const ChainTracks tr = chain_tracks(seq_len, batch_size, chunk_size);
+        if (es.failed()) return;
+        chunkwise_forward_mm_f32_tracked(fn, k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial, nullptr, m_chunk_states,
+                                         nullptr, y, seq_len, d, batch_size, chunk_size, false, tr);
+        if (!es.failed() && !couplings_may_fire_tracked(k_mem, alpha, theta, nullptr, tr, false, seq_len, batch_size,
+                                                        chunk_size, error_clip, m_norm_max))
             return;
     }
     FwdArgs a{k_mem, v_mem, q_mem, alpha, theta, nullptr, m_initial, nullptr,
@@ -1223,7 +1227,14 @@ void titans_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, 
                                         float *d_m_initial, float *d_s_initial,
                                         int seq_len, int d, int batch_size, int chunk_size,
                                         float error_clip, float m_norm_max) {
-    if (seq_len > 0 && batch_size > 0 &&
+    if (seq_len > 0 && batch_size > 0 && guarded_matrix_form(d, chunk_size, error_clip, m_norm_max) && !last_test_fired) {
+        // the matrix form with the test inside: its gradient pass forms the errors anyway
+        if (chunkwise_backward_mm_f32_guarded("titans_chunkwise_backward_f32_cuda", k_mem, v_mem, q_mem, alpha, theta, eta,
+                                              m_chunk_states, s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta,
+                                              d_eta, d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, true,
+                                              error_clip, m_norm_max))
+            return;
+    } else if (seq_len > 0 && batch_size > 0 &&
         (matrix_form_applies(d, chunk_size, error_clip, m_norm_max) ||
          (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max) &&
           !couplings_may_fire(k_mem, v_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, seq_len, batch_size, chunk_size,
@@ -1246,7 +1257,13 @@ void delta_chunkwise_backward_f32_cuda(const float *k_mem, const float *v_mem, c
                                        float *d_alpha, float *d_theta, float *d_m_initial,
                                        int seq_len, int d, int batch_size, int chunk_size,
                                        float error_clip, float m_norm_max) {
-    if (seq_len > 0 && batch_size > 0 &&
+    if (seq_len > 0 && batch_size > 0 && guarded_matrix_form(d, chunk_size, error_clip, m_norm_max) && !last_test_fired) {
+        if (chunkwise_backward_mm_f32_guarded("delta_chunkwise_backward_f32_cuda", k_mem, v_mem, q_mem, alpha, theta, nullptr,
+                                              m_chunk_states, nullptr, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta,
+                                              nullptr, d_m_initial, nullptr, seq_len, d, batch_size, chunk_size, false,
+                                              error_clip, m_norm_max))
+            return;
+    } else if (seq_len > 0 && batch_size > 0 &&
         (matrix_form_applies(d, chunk_size, error_clip, m_norm_max) ||
          (guarded_matrix_form(d, chunk_size, error_clip, m_norm_max) &&
           !couplings_may_fire(k_mem, v_mem, alpha, theta, nullptr, m_chunk_states, nullptr, seq_len, batch_size, chunk_size,

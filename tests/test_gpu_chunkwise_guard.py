@@ -100,8 +100,8 @@ def test_production_bound_that_never_fires_keeps_the_matrix_form():
     got = run_f32(x, C, 0.0, 100.0)
     check(x, C, 0.0, 100.0, got)
     ran_f, ran_b = got[5], got[6]
-    assert "cw_guard_kernel" in ran_f and "rule_fwd_kernel" not in ran_f, ran_f
-    assert "cw_guard_kernel" in ran_b and not any(n.startswith("rule_bwd") for n in ran_b), ran_b
+    assert "cw_guard_tracks_kernel" in ran_f and "rule_fwd_kernel" not in ran_f, ran_f   # the forward tests from its own side outputs
+    assert "cw_guard_tracks_kernel" in ran_b and not any(n.startswith("rule_bwd") for n in ran_b), ran_b   # test inside the pass
     # and with a clip far above every error, as the reference's sfl5 configuration ships one
     got = run_f32(x, C, 4.0 * worst_e, 100.0)
     check(x, C, 4.0 * worst_e, 100.0, got)
@@ -129,6 +129,33 @@ def test_clip_that_fires_takes_the_sequential_kernels():
     got = run_f32(x, C, clip, F32_MAX)
     check(x, C, clip, F32_MAX, got)
     assert "rule_fwd_kernel" in got[5], got[5]
+
+
+def test_backward_alone_after_a_forward_whose_test_fired_and_after_one_whose_test_did_not():
+    """The backward picks the order of its work from how the last test came out (stand-alone test first after one that
+    fired, test inside the matrix-form pass otherwise); either order gives the reference's numbers, also when the hint
+    is wrong for the call: a backward with a bound that fires right after a forward with one that does not, and the
+    other way round.  d_m_initial is added to exactly once either way."""
+    B, s, d, C = 4, 192, 64, 64
+    x = rule_inputs(B, s, d, seed=53, m0_scale=0.02)
+    worst, _ = max_state_norm(x, C)
+    t = {n: dev(a) for n, a in x.items()}
+    nc = (s + C - 1) // C
+    for fwd_bound, bwd_bound in ((100.0, 0.6 * worst), (0.6 * worst, 100.0)):
+        mc, sc, y = zeros(B, nc + 1, d * d), zeros(B, nc + 1, d * d), zeros(B, s, d)
+        D.call("titans_chunkwise_forward_f32_cuda", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"], t["m0"], t["s0"],
+               mc, sc, y, s, d, B, C, 0.0, fwd_bound)
+        # states of the trajectory the backward's own bound describes
+        yo, mco, sco, go = oracle_pair(x, C, 0.0, bwd_bound)
+        g = {n: zeros(B, s, d) for n in ("d_k", "d_v", "d_q")}
+        g.update({n: zeros(B, s) for n in ("d_alpha", "d_theta", "d_eta")})
+        dm, ds = zeros(d, d), zeros(d, d)
+        D.call("titans_chunkwise_backward_f32_cuda", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"],
+               dev(mco.reshape(B, nc + 1, d * d)), dev(sco.reshape(B, nc + 1, d * d)), t["dy"], g["d_k"], g["d_v"], g["d_q"],
+               g["d_alpha"], g["d_theta"], g["d_eta"], dm, ds, s, d, B, C, 0.0, bwd_bound)
+        for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta", "d_eta"):
+            assert_close(n, host(g[n]), np.stack([gi[n] for gi in go]), 1e-4)
+        assert_close("d_m_initial", host(dm), sum(gi["d_m"] for gi in go), 1e-4)
 
 
 def test_bound_just_above_the_trajectory_is_still_exact():
