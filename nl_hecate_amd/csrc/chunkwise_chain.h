@@ -37,4 +37,11 @@ bool chunkwise_backward_mm_f32_guarded(const char *fn, const float *k, const flo
                                        float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d, int batch,
                                        int chunk_size, bool has_s, float error_clip, float m_norm_max);
 
+// the same for bf16 tokens (the chain-resident kernels' backward)
+bool chunkwise_backward_bf16_guarded(const char *fn, const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *alpha,
+                                     const float *theta, const float *eta, const float *m_states, const float *s_states,
+                                     const float *d_y, float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta,
+                                     float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d, int batch,
+                                     int chunk_size, bool has_s, float error_clip, float m_norm_max);
+
 }  // namespace nlh

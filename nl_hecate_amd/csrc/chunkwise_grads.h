@@ -15,6 +15,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "chunkwise_chain.h"
 #include "head_rows.h"
 
 namespace nlh {
@@ -42,7 +43,8 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid,
-                          const HeadRows *dy_rows = nullptr, const GradOut16 *out16 = nullptr);
+                          const HeadRows *dy_rows = nullptr, const GradOut16 *out16 = nullptr,
+                          const ChainTracks *tracks = nullptr);   // tracks: also leave the side outputs of chunkwise_chain.h
 
 // titans_chunkwise_backward_bf16_tokens_rocm with d_k, d_v, d_q leaving as bf16 token-major slabs (the level step's
 // GEMM operand): same arguments otherwise

@@ -32,6 +32,7 @@
 
 #include "bf16_tiles.h"
 #include "chunk_coef.h"
+#include "chunkwise_chain.h"
 #include "chunkwise_grads.h"
 #include "runtime.h"
 
@@ -114,14 +115,15 @@ __device__ __forceinline__ f32x4 bf4_to_f32(const uint2 b) {
 }
 __device__ __forceinline__ f32x4 bf4_to_f32(const u16 *p) { return bf4_to_f32(*reinterpret_cast<const uint2 *>(p)); }
 
-template <bool HAS_S, bool G16>
+// TRACK: also leaves the ChainTracks of chunkwise_chain.h behind (what a test of the reference's couplings needs).
+template <bool HAS_S, bool G16, bool TRACK>
 __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
     const u16 *__restrict__ k, const u16 *__restrict__ v, const u16 *__restrict__ q, const float *__restrict__ d_y,
     const float *__restrict__ tab_b, const float *__restrict__ vecs,
     const float *__restrict__ m_states, const float *__restrict__ s_states, const u16 *__restrict__ dm_snap,
     const u16 *__restrict__ ds_snap, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
     float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s,
-    int C, int nc, int ntask, HeadRows dyr, GradOut16 go) {
+    int C, int nc, int ntask, HeadRows dyr, GradOut16 go, ChainTracks tr) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     // Every input is staged once, in the order it arrives (rows = tokens or state rows); a product that contracts
     // over the row index reads its operand through ld_op_tr.
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
             *reinterpret_cast<uint4 *>(Kr + st_t * LDB + st_cb * 8) = nK;
             *reinterpret_cast<uint4 *>(Qr + st_t * LDB + st_cb * 8) = nQ;
             *reinterpret_cast<uint4 *>(Vr + st_t * LDB + st_cb * 8) = nV;
-            float d0 = 0.f, d1 = 0.f, d2 = 0.f;
+            float d0 = 0.f, d1 = 0.f, d2 = 0.f, msq = 0.f, ssq = 0.f;
 #pragma unroll
             for (int it = 0; it < 2; it++) {
                 const int c4 = (fg0 + 8 * it) * 4, off = ft * LDB + c4;
@@ -230,10 +232,19 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
                 for (int i = 0; i < 4; i++) {
                     d0 = fmaf(nM0[it][i], fdM[i], d0);
                     if (HAS_S) { d1 = fmaf(nS0[it][i], fdM[i], d1); d2 = fmaf(nS0[it][i], fdS[i], d2); }
+                    if (TRACK) {
+                        msq = fmaf(nM0[it][i], nM0[it][i], msq);
+                        if (HAS_S) ssq = fmaf(nS0[it][i], nS0[it][i], ssq);
+                    }
                 }
             }
             d0 = sum_wave(d0); d1 = sum_wave(d1); d2 = sum_wave(d2);
             if (l == 0) { dots[w] = d0; dots[8 + w] = d1; dots[16 + w] = d2; }
+            if (TRACK) {
+                msq = sum_wave(msq);
+                ssq = sum_wave(ssq);
+                if (l == 0) *reinterpret_cast<float2 *>(tr.nrm + (((size_t)chain * nc + ci) * 8 + w) * 2) = make_float2(msq, ssq);
+            }
             if (tid < 5 * CW) cvec[tid] = nvec;
             if (grpA) {   // c[t .. t+3][j] of this wave's block
 #pragma unroll
@@ -285,10 +296,19 @@ __global__ __launch_bounds__(kTileThr) void cw_grads_bf16_kernel(
 #pragma unroll
             for (int ct = 0; ct < 2; ct++) {
                 const bf16x8 bv = ld_op(Vr, bn + 16 * ct, bm >> 5);
+                float esq = 0.f;
 #pragma unroll
                 for (int rt = 0; rt < 2; rt++) {
                     e[rt][ct] = mfma32(negI[rt], bv, e[rt][ct]);
                     bf16_store(Er, (bn + 16 * ct + r16) * LDB + bm + 16 * rt + 4 * g, e[rt][ct]);   // E[t][i .. i+3]
+                    if (TRACK) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) esq = fmaf(e[rt][ct][r], e[rt][ct][r], esq);
+                    }
+                }
+                if (TRACK) {   // token bn + 16 ct + l % 16, this wave's 32 memory rows (half bm / 32)
+                    esq = sum_groups(esq);
+                    if (g == 0) tr.e2[(((size_t)chain * 2 + (bm >> 5)) * nc + ci) * CW + bn + 16 * ct + r16] = esq;
                 }
             }
         } else {
@@ -585,28 +605,33 @@ bool chunkwise_grads_bf16(const uint16_t *k, const uint16_t *v, const uint16_t *
                           const uint16_t *ds_snap, float *d_k, float *d_v, float *d_q, float *d_theta, float *pvec,
                           float *xs, float *scal, const float *tab_b, const float *vecs,
                           int seq_len, int batch, int chunk_size, bool has_s, int grid, const HeadRows *dy_rows,
-                          const GradOut16 *out16) {
+                          const GradOut16 *out16, const ChainTracks *tracks) {
     const ErrorScope es;
+    if (tracks && out16) { fail("chunkwise_grads_bf16: the in-pass test is not served together with bf16 gradient slabs."); return true; }
     const int nc = ceil_div(seq_len, chunk_size), ntask = batch * nc;
     const HeadRows dyr = dy_rows ? *dy_rows : head_major_rows(seq_len, HD);
     static bool attr_set = false;
     if (!attr_set) {
-        const void *fns[4] = {reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, false>),
-                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, false>),
-                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, true>),
-                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, true>)};
+        const void *fns[6] = {reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, false, false>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, false, false>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, true, false>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, true, false>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<true, false, true>),
+                              reinterpret_cast<const void *>(cw_grads_bf16_kernel<false, false, true>)};
         for (const void *f : fns) check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGradsLds), "dynamic LDS size");
         attr_set = true;
     }
     if (es.failed()) return true;
     const GradOut16 go = out16 ? *out16 : GradOut16{};
     KernelTimer kt("cw_grads_bf16_kernel");
-#define NLH_CWG(HS, G) \
-    hipLaunchKernelGGL((cw_grads_bf16_kernel<HS, G>), dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y, tab_b, vecs, \
+    const ChainTracks tr = tracks ? *tracks : ChainTracks{nullptr, nullptr};
+#define NLH_CWG(HS, G, T) \
+    hipLaunchKernelGGL((cw_grads_bf16_kernel<HS, G, T>), dim3(grid), dim3(kTileThr), kGradsLds, stream(), k, v, q, d_y, tab_b, vecs, \
                        m_states, HS ? s_states : nullptr, dm_snap, HS ? ds_snap : nullptr, d_k, d_v, d_q, d_theta, pvec, xs, scal, \
-                       seq_len, chunk_size, nc, ntask, dyr, go)
-    if (has_s) { if (out16) NLH_CWG(true, true); else NLH_CWG(true, false); }
-    else { if (out16) NLH_CWG(false, true); else NLH_CWG(false, false); }
+                       seq_len, chunk_size, nc, ntask, dyr, go, tr)
+    if (tracks) { if (has_s) NLH_CWG(true, false, true); else NLH_CWG(false, false, true); }
+    else if (has_s) { if (out16) NLH_CWG(true, true, false); else NLH_CWG(true, false, false); }
+    else { if (out16) NLH_CWG(false, true, false); else NLH_CWG(false, false, false); }
 #undef NLH_CWG
     check_launch("cw_grads_bf16_kernel");
     return true;

@@ -370,7 +370,15 @@ void titans_chunkwise_backward_bf16_guarded_rocm(const uint16_t *k_mem, const ui
     const ErrorScope es;
     if (seq_len <= 0 || batch_size <= 0) return;
     const bool mm = d == 64 && chunk_size >= 1 && chunk_size <= 64;
-    if (mm && (!coupled(error_clip, m_norm_max) ||
+    if (mm && coupled(error_clip, m_norm_max) && guard_possible() && !last_test_fired) {
+        // the test inside the matrix-form pass (its gradient kernel forms the errors anyway); see memory_rules.hip for
+        // why the order of work follows the last test
+        if (chunkwise_backward_bf16_guarded("titans_chunkwise_backward_bf16_guarded_rocm", k_mem, v_mem, q_mem, alpha, theta, eta,
+                                            m_chunk_states, s_chunk_states, d_y, d_k_mem, d_v_mem, d_q_mem, d_alpha, d_theta,
+                                            d_eta, d_m_initial, d_s_initial, seq_len, d, batch_size, chunk_size, true, error_clip,
+                                            m_norm_max))
+            return;
+    } else if (mm && (!coupled(error_clip, m_norm_max) ||
                (guard_possible() && !couplings_may_fire_bf16(k_mem, v_mem, alpha, theta, eta, m_chunk_states, s_chunk_states,
                                                              seq_len, batch_size, chunk_size, error_clip, m_norm_max)))) {
         titans_chunkwise_backward_bf16_rocm(k_mem, v_mem, q_mem, alpha, theta, eta, m_chunk_states, s_chunk_states, d_y, d_k_mem,

@@ -787,7 +787,7 @@ void set_lds(K kernel, size_t bytes) {
                                   (int)bytes), "dynamic LDS size");
 }
 
-// guard (float tokens only): the gradient pass also leaves the ChainTracks behind, and the call ends with the test of
+// guard: the gradient pass also leaves the ChainTracks behind, and the call ends with the test of
 // the reference's couplings on them BEFORE anything is added to d_m_initial / d_s_initial; false: a coupling may have
 // fired, the caller runs the sequential kernels, which overwrite every other output.
 struct BackwardGuard { float error_clip, m_norm_max; };
@@ -801,7 +801,7 @@ bool backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     if (!check_mm_args(fn, seq_len, d, batch, chunk_size)) return true;
     if (out16 && sizeof(TIn) != 2) { fail("%s: bf16 gradient slabs are served for bf16 tokens only.", fn); return true; }
     if (dy_rows && sizeof(TIn) != 2) { fail("%s: token-major d_y is served for bf16 tokens only.", fn); return true; }
-    if (guard && sizeof(TIn) != 4) { fail("%s: the in-pass test is served for float tokens only.", fn); return true; }
+    if (guard && (out16 || dy_rows)) { fail("%s: the in-pass test is served for head-major fp32 gradients only.", fn); return true; }
     ChainTracks tracks{nullptr, nullptr};
     if (guard) tracks = chain_tracks(seq_len, batch, chunk_size);
     const int nc = ceil_div(seq_len, chunk_size);
@@ -838,7 +838,7 @@ bool backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
                                reinterpret_cast<float *>(ds_snap + n_snap), seq_len, batch, chunk_size, has_s, dy_rows);
         chunkwise_grads_bf16(k, v, q, d_y, m_states, s_states, dm_snap, ds_snap, d_k, d_v, d_q, d_theta, pvec, xs,
                              scal, tab_b, vecs, seq_len, batch, chunk_size, has_s,
-                             persistent_grid(batch * nc), dy_rows, out16);
+                             persistent_grid(batch * nc), dy_rows, out16, guard ? &tracks : nullptr);
     } else {
         hipLaunchKernelGGL((cw_local_bwd_kernel<TIn>), dim3(persistent_grid(batch * nc)), dim3(kThr), kLocalBwdLds,
                            stream(), k, q, d_y, alpha, theta, eta, sc.loc, sc.locs, seq_len, chunk_size, nc,
@@ -876,8 +876,8 @@ bool backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
     // d_alpha, d_eta, and in the same launch the first stage of the deterministic sum of d_m_initial, d_s_initial
     chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, chunk_size, has_s, dm_first,
                              ds_first, chain_stride, per, nsum, tmp);
-    if (guard && couplings_may_fire_tracked(reinterpret_cast<const float *>(k), alpha, theta, eta, tracks, has_s, seq_len, batch,
-                                            chunk_size, guard->error_clip, guard->m_norm_max))
+    if (guard && couplings_may_fire_tracked(k, alpha, theta, eta, tracks, has_s, seq_len, batch, chunk_size, guard->error_clip,
+                                            guard->m_norm_max))
         return false;
     KernelTimer kt("cw_add_rows_kernel");
     hipLaunchKernelGGL(cw_add_rows_kernel, dim3(HD * HD / 256, 1, nsum), dim3(256), 0, stream(), tmp, d_m_initial,
@@ -894,6 +894,16 @@ void chunkwise_forward_mm_f32_tracked(const char *fn, const float *k, const floa
                                       int chunk_size, bool has_s, const ChainTracks &tracks) {
     forward_mm<float>(fn, k, v, q, alpha, theta, eta, m_initial, s_initial, m_states, s_states, y, seq_len, d, batch,
                       chunk_size, has_s, &tracks);
+}
+
+bool chunkwise_backward_bf16_guarded(const char *fn, const uint16_t *k, const uint16_t *v, const uint16_t *q, const float *alpha,
+                                     const float *theta, const float *eta, const float *m_states, const float *s_states,
+                                     const float *d_y, float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta,
+                                     float *d_eta, float *d_m_initial, float *d_s_initial, int seq_len, int d, int batch,
+                                     int chunk_size, bool has_s, float error_clip, float m_norm_max) {
+    const BackwardGuard g{error_clip, m_norm_max};
+    return backward_mm<uint16_t>(fn, k, v, q, alpha, theta, eta, m_states, s_states, d_y, d_k, d_v, d_q, d_alpha, d_theta, d_eta,
+                                 d_m_initial, d_s_initial, seq_len, d, batch, chunk_size, has_s, nullptr, nullptr, &g);
 }
 
 bool chunkwise_backward_mm_f32_guarded(const char *fn, const float *k, const float *v, const float *q, const float *alpha,

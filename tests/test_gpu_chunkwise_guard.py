@@ -158,6 +158,40 @@ def test_backward_alone_after_a_forward_whose_test_fired_and_after_one_whose_tes
         assert_close("d_m_initial", host(dm), sum(gi["d_m"] for gi in go), 1e-4)
 
 
+def test_bf16_backward_alone_with_the_hint_wrong_either_way():
+    """The same for the bf16 symbols: the matrix-form gradient pass leaves the error and state norms behind and is
+    discarded when the test on them fires."""
+    B, s, d, C = 4, 192, 64, 64
+    x = rule_inputs(B, s, d, seed=59, m0_scale=0.02)
+    for n in ("k", "v", "q"):
+        x[n] = torch.from_numpy(x[n]).to(torch.bfloat16).to(torch.float32).numpy()
+    worst, _ = max_state_norm(x, C)
+    t = {n: dev(a) for n, a in x.items()}
+    kb, vb, qb = (t[n].to(torch.bfloat16) for n in ("k", "v", "q"))
+    nc = (s + C - 1) // C
+    for fwd_bound, bwd_bound in ((100.0, 0.6 * worst), (0.6 * worst, 100.0)):
+        mc, sc, y = zeros(B, nc + 1, d * d), zeros(B, nc + 1, d * d), zeros(B, s, d)
+        D.call("titans_chunkwise_forward_bf16_guarded_rocm", kb, vb, qb, t["alpha"], t["theta"], t["eta"], t["m0"], t["s0"],
+               mc, sc, y, s, d, B, C, 0.0, fwd_bound)
+        yo, mco, sco, go = oracle_pair(x, C, 0.0, bwd_bound)
+        g = {n: zeros(B, s, d) for n in ("d_k", "d_v", "d_q")}
+        g.update({n: zeros(B, s) for n in ("d_alpha", "d_theta", "d_eta")})
+        dm, ds = zeros(d, d), zeros(d, d)
+        ran = kernels_run(lambda: D.call("titans_chunkwise_backward_bf16_guarded_rocm", kb, vb, qb, t["alpha"], t["theta"],
+                                         t["eta"], dev(mco.reshape(B, nc + 1, d * d)), dev(sco.reshape(B, nc + 1, d * d)),
+                                         t["dy"], g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], dm, ds,
+                                         s, d, B, C, 0.0, bwd_bound))
+        fires = bwd_bound < worst
+        tol = 1e-4 if fires else 1e-2
+        for n in ("d_k", "d_v", "d_q", "d_alpha", "d_theta", "d_eta"):
+            assert_close(n, host(g[n]), np.stack([gi[n] for gi in go]), tol)
+        assert_close("d_m_initial", host(dm), sum(gi["d_m"] for gi in go), tol)
+        if fires:   # hint said "did not fire": the pass with the test inside ran first and was discarded
+            assert "cw_grads_bf16_kernel" in ran and "cw_guard_tracks_kernel" in ran, ran
+        else:       # hint said "fired": the stand-alone test ran first and cleared the matrix form
+            assert "cw_guard_kernel" in ran and "cw_grads_bf16_kernel" in ran, ran
+
+
 def test_bound_just_above_the_trajectory_is_still_exact():
     """A bound the triangle-inequality test cannot clear (between the true maximum and the test's estimate) costs the
     sequential kernels but never a wrong result."""
