@@ -1,0 +1,656 @@
+// Backward of the exact Titans / Delta rule from checkpoints every C <= 64 tokens, in chunk-parallel matrix form on
+// the fp32 matrix cores (v_mfma_f32_16x16x4_f32), head size 64.
+//
+// Semantics are those of core/kernels/titans_backward.cu:66-341 run segment by segment from the checkpoints of
+// core/kernels/titans_forward.cu (the schedule of core/src/gpu_backward.rs:1770-1962) with error_clip and the
+// M-norm projection off: every error is taken against the CURRENT memory, u_t = M_(t-1) k_t - v_t.
+//
+// The rule is linear in (M, S).  Inside a chunk that starts at the checkpoint (M0, S0), with the coefficients of
+// the frozen-M0 form (mm_coef.h: a, beta, h, c, bb; W[t][j] = -theta_j c[t][j], wM = W[L-1], wS_j = -theta_j
+// bb[j][L-1]) and am, bm = a, beta shifted by one token (am_0 = 1, bm_0 = 0), the errors of a chunk obey a unit
+// lower triangular system
+//   (I - Lam) U = R,   Lam[t][j] = W[t-1][j] (k_j . k_t)  (j < t),   R = am.(K M0^T) + bm.(K S0^T) - V
+// and everything else is the frozen rule with its errors replaced by U plus the terms through T = (I - Lam)^-1:
+//   dU = (W.P)^T dY + wM.(K dMo^T) + wS.(K dSo^T)     dR = T^T dU      (P = Q K^T; dMo, dSo: adjoints at chunk end)
+//   dV = -dR     dQ = a.(dY M0) + beta.(dY S0) + (W.tril(dY U^T)) K
+//   dK = (W.tril(dY U^T))^T Q + wM.(U dMo) + wS.(U dSo) + am.(dR M0) + bm.(dR S0) + (dG + dG^T) K,
+//        dG[t][j] = W[t-1][j] strict_tril(dR U^T)[t][j]
+//   adjoints at chunk start:  dM' = a_L dMo + (a.dY)^T Q + (am.dR)^T K,   dS' = beta_L dMo + h_L dSo + (beta.dY)^T Q + (bm.dR)^T K
+// The last line is affine in (dMo, dSo) with matrices that depend on the chunk only, so the reverse scan over the
+// chunks of a chain multiplies by four 64x64 matrices per step and the rest is chunk-parallel:
+//   1. ex_local_kernel   per chunk: T (blocked inverse: 16x16 diagonal blocks by substitution, then
+//                        (I + N)(I + N^2) D with N = D Lam_off, N^4 = 0), U, dU_loc = (W.P)^T dY, the four matrices
+//                        Phi = (w.K)^T T (m.K) and the two additive terms of the scan
+//   2. ex_scan_kernel    per (chain, 16-row block): the adjoints at every chunk boundary
+//   3. ex_grads_kernel   per chunk: dQ, dK, dV, dtheta and the hand-off of the gate pass
+//   4. cw_gates_sweep_kernel (chunkwise_gates.hip): dalpha, deta.  The inner products <M_s, J_t> it sweeps obey the
+//      rule's own recurrence with J_t = dy_t q_t^T + dR_(t+1) k_(t+1)^T, i.e. per-token terms
+//      xs[s][t] = -theta_s [ (dy_t.u_s)(q_t.k_s) + (dR_(t+1).u_s)(k_(t+1).k_s) ].
+// The algebra is written out and checked against the reference's token loops in float64 in tests/np_rules.py
+// (titans_exact_chunk_backward).
+//
+// Under a finite m_norm_max / error clip the pass also leaves the ChainTracks of chunkwise_chain.h behind (|u_t|^2 per
+// token, sums of squares of the checkpoints); the caller tests on them whether a coupling could have fired.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "chunkwise_chain.h"
+#include "chunkwise_grads.h"
+#include "chunkwise_guard.h"
+#include "exact_mm.h"
+#include "mm_coef.h"
+#include "mm_tiles.h"
+#include "rule_common.h"
+#include "runtime.h"
+
+namespace nlh {
+namespace {
+
+using namespace mmt;
+
+#define NLH_STRIP_ORIGIN() \
+    const int w = threadIdx.x >> 6, m0 = 16 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1; \
+    (void)nh
+
+// per chunk, for the scan: Phi_MM, Phi_SM, Phi_MS, Phi_SS (source state, destination state), C_M, C_S
+constexpr size_t kExLocMats = 6;
+constexpr size_t kDD = (size_t)HD * HD;
+
+struct ChunkVecs { float wM[CW], wS[CW], am[CW], bm[CW]; };
+__device__ __forceinline__ void chunk_vectors(ChunkVecs &cv, const Coef &cf, int L) {
+    const int j = threadIdx.x;
+    if (j < CW) {
+        cv.wM[j] = -cf.th[j] * cf.cl[j];
+        cv.wS[j] = -cf.th[j] * cf.bl[j];
+        cv.am[j] = j == 0 ? 1.f : (j < L ? cf.a[j - 1] : 0.f);
+        cv.bm[j] = (j == 0 || j >= L) ? 0.f : cf.beta[j - 1];
+    }
+}
+
+// sum of squares of a staged tile's registers over the wave
+__device__ __forceinline__ float tile_dot(const Tile<float> &a, const Tile<float> &b) {
+    float x = 0.f;
+#pragma unroll
+    for (int it = 0; it < 2; it++)
+        x += a.x[it].x * b.x[it].x + a.x[it].y * b.x[it].y + a.x[it].z * b.x[it].z + a.x[it].w * b.x[it].w;
+    return x;
+}
+
+// ── pass 1: chunk-local matrices ────────────────────────────────────────────
+template <bool TRACK>
+__global__ __launch_bounds__(kThr) void ex_local_kernel(
+    const float *__restrict__ k, const float *__restrict__ v, const float *__restrict__ q, const float *__restrict__ d_y,
+    const float *__restrict__ alpha, const float *__restrict__ theta, const float *__restrict__ eta,
+    const float *__restrict__ m_ckpt, const float *__restrict__ s_ckpt, float *__restrict__ loc, float *__restrict__ locs,
+    float *__restrict__ Tg, float *__restrict__ Ug, float *__restrict__ dUg, int s, int C, int nc, int nck, int has_s,
+    ChainTracks tr) {
+    extern __shared__ float smem[];
+    float *Ks = smem, *Vs = Ks + MAT, *Qs = Vs + MAT, *Ds = Qs + MAT, *Ms = Ds + MAT, *Ss = Ms + MAT, *Cc = Ss + MAT,
+          *B8 = Cc + MAT, *B9 = B8 + MAT;
+    __shared__ Coef cf;
+    __shared__ ChunkVecs cv;
+    NLH_STRIP_ORIGIN();
+    const int l = threadIdx.x & 63;
+    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0, task = (size_t)chain * nc + ci;
+    {
+        Tile<float> tk, tv, tq, td, tm, ts;
+        fetch(tk, k + tok * HD, L);
+        fetch(tv, v + tok * HD, L);
+        fetch(tq, q + tok * HD, L);
+        fetch(td, d_y + tok * HD, L);
+        fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
+        if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
+        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        load_gates(cf, gt);
+        coefficients(cf, gt, L, Cc, nullptr, nullptr);
+        commit(Ks, tk);
+        commit(Vs, tv);
+        commit(Qs, tq);
+        commit(Ds, td);
+        commit(Ms, tm);
+        if (has_s) commit(Ss, ts);
+        if (TRACK) {
+            float msq = wave_allreduce(tile_dot(tm, tm)), ssq = has_s ? wave_allreduce(tile_dot(ts, ts)) : 0.f;
+            if (l == 0) *reinterpret_cast<float2 *>(tr.nrm + (task * 8 + w) * 2) = make_float2(msq, ssq);
+        }
+    }
+    __syncthreads();
+    chunk_vectors(cv, cf, L);
+    if (threadIdx.x == 0) {
+        float *sc = locs + task * 4;
+        sc[0] = cf.a[L - 1]; sc[1] = cf.beta[L - 1]; sc[2] = cf.h[L - 1]; sc[3] = 0.f;
+    }
+    {
+        Strip g = zero_strip(), km = zero_strip(), ks = zero_strip(), p = zero_strip();
+        auto aK = [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; };
+        mma(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        mma(km, aK, [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+        if (has_s) mma(ks, aK, [&](int kk, int n) { return Ss[(n0 + n) * LDM + kk]; });
+        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        __syncthreads();   // the vectors are there
+        Strip e2 = zero_strip();
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                // R in place over V (own strip)
+                float *d = Vs + row * LDM + col;
+                *d = cv.am[row] * km.t[tl][i] + cv.bm[row] * ks.t[tl][i] - *d;
+                const float nth = -cf.th[col];
+                B8[row * LDM + col] = (col < row) ? nth * Cc[(row - 1) * LDM + col] * g.t[tl][i] : 0.f;   // Lam
+                B9[row * LDM + col] = nth * Cc[row * LDM + col] * p.t[tl][i];                            // W.P
+            }
+        (void)e2;
+    }
+    __syncthreads();
+    Strip dul = zero_strip();
+    mma(dul, [&](int m, int kk) { return B9[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
+    if (w < 4 && l < 16) {
+        // D_b = (I - Lam_bb)^-1 by substitution: lane c holds column c of block b = w
+        const float *A = B8 + (16 * w) * LDM + 16 * w;
+        float x[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float acc = r == l ? 1.f : 0.f;
+#pragma unroll
+            for (int j = 0; j < r; j++) acc = fmaf(A[r * LDM + j], x[j], acc);
+            x[r] = acc;
+        }
+        float *Dd = Ms + (16 * w) * LDM + 16 * w + l;
+#pragma unroll
+        for (int r = 0; r < 16; r++) Dd[r * LDM] = x[r];
+    }
+    __syncthreads();
+    {   // N = D Lam_off -> Ss; dU_loc -> B9 and out
+        const int ib = w >> 1;
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++) {
+            const int jb = 2 * (w & 1) + tl;
+            f32x4 nacc = {0.f, 0.f, 0.f, 0.f};
+            if (jb < ib)
+                mma_tile16(nacc, [&](int m, int kk) { return Ms[(m0 + m) * LDM + kk]; },
+                           [&](int kk, int n) { return B8[kk * LDM + 16 * jb + n]; }, 16 * ib);
+#pragma unroll
+            for (int i = 0; i < 4; i++) Ss[(m0 + row_of(i)) * LDM + 16 * jb + (l & 15)] = nacc[i];
+        }
+        float *go = dUg + task * kDD;
+        for_c(dul, [&](int r, int c, float &x) {
+            B9[(m0 + r) * LDM + n0 + c] = x;
+            go[(m0 + r) * HD + n0 + c] = x;
+        });
+    }
+    __syncthreads();
+    {   // N^2 -> B8
+        Strip n2 = zero_strip();
+        mma(n2, [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ss[kk * LDM + n0 + n]; });
+        for_c(n2, [&](int r, int c, float &x) { B8[(m0 + r) * LDM + n0 + c] = x; });
+    }
+    __syncthreads();
+    {   // X = (I + N)(I + N^2) -> Cc
+        Strip x3 = zero_strip();
+        mma(x3, [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return B8[kk * LDM + n0 + n]; });
+        for_c(x3, [&](int r, int c, float &x) {
+            const int row = m0 + r, col = n0 + c;
+            Cc[row * LDM + col] = x + Ss[row * LDM + col] + B8[row * LDM + col] + (row == col ? 1.f : 0.f);
+        });
+    }
+    __syncthreads();
+    {   // T = X D -> Ss and out
+        float *go = Tg + task * kDD;
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++) {
+            const int jb = 2 * (w & 1) + tl;
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            mma_tile16(t, [&](int m, int kk) { return Cc[(m0 + m) * LDM + kk]; },
+                       [&](int kk, int n) { return Ms[kk * LDM + 16 * jb + n]; }, 16 * jb);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = 16 * jb + (l & 15);
+                Ss[row * LDM + col] = t[i];
+                go[row * HD + col] = t[i];
+            }
+        }
+    }
+    __syncthreads();
+    {   // U = T R -> out;  Z1 = T (am.K) -> B8,  Z2 = T (bm.K) -> Ms
+        Strip u = zero_strip(), z1 = zero_strip(), z2 = zero_strip();
+        auto aT = [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; };
+        mma(u, aT, [&](int kk, int n) { return Vs[kk * LDM + n0 + n]; });
+        mma(z1, aT, [&](int kk, int n) { return cv.am[kk] * Ks[kk * LDM + n0 + n]; });
+        if (has_s) mma(z2, aT, [&](int kk, int n) { return cv.bm[kk] * Ks[kk * LDM + n0 + n]; });
+        float *go = Ug + task * kDD;
+        for_c(u, [&](int r, int c, float &x) { go[(m0 + r) * HD + n0 + c] = x; });
+        for_c(z1, [&](int r, int c, float &x) { B8[(m0 + r) * LDM + n0 + c] = x; });
+        if (has_s) for_c(z2, [&](int r, int c, float &x) { Ms[(m0 + r) * LDM + n0 + c] = x; });
+        if (TRACK) {   // squared error norm of the strip's 16 tokens over its 32 memory rows
+            for_c(u, [&](int, int, float &x) { x *= x; });
+            strip_row_sums(u);
+            if (row_writer()) {
+                float *eo = tr.e2 + (((size_t)chain * 2 + nh) * nc + ci) * CW + m0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) eo[row_of(i)] = u.t[0][i];
+            }
+        }
+    }
+    __syncthreads();
+    float *out = loc + task * kExLocMats * kDD;
+    auto store = [&](int which, Strip &x) {
+        for_c(x, [&](int r, int c, float &y) { out[(size_t)which * kDD + (m0 + r) * HD + n0 + c] = y; });
+    };
+    auto bZ1 = [&](int kk, int n) { return B8[kk * LDM + n0 + n]; };
+    auto bZ2 = [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; };
+    auto aWM = [&](int m, int kk) { return cv.wM[kk] * Ks[kk * LDM + m0 + m]; };
+    auto aWS = [&](int m, int kk) { return cv.wS[kk] * Ks[kk * LDM + m0 + m]; };
+    auto bQ = [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; };
+    auto aDU = [&](int m, int kk) { return B9[kk * LDM + m0 + m]; };
+    {
+        Strip x = zero_strip();
+        mma(x, aWM, bZ1);
+        store(0, x);
+    }
+    {
+        Strip x = zero_strip();
+        mma(x, [&](int m, int kk) { return cf.a[kk] * Ds[kk * LDM + m0 + m]; }, bQ);
+        mma(x, aDU, bZ1);
+        store(4, x);
+    }
+    if (has_s) {
+        {
+            Strip x = zero_strip();
+            mma(x, aWS, bZ1);
+            store(1, x);
+        }
+        {
+            Strip x = zero_strip();
+            mma(x, aWM, bZ2);
+            store(2, x);
+        }
+        {
+            Strip x = zero_strip();
+            mma(x, aWS, bZ2);
+            store(3, x);
+        }
+        {
+            Strip x = zero_strip();
+            mma(x, [&](int m, int kk) { return cf.beta[kk] * Ds[kk * LDM + m0 + m]; }, bQ);
+            mma(x, aDU, bZ2);
+            store(5, x);
+        }
+    }
+}
+constexpr size_t kExLocalLds = 9 * MAT * sizeof(float);
+
+// ── pass 2: reverse scan over the chunks of a chain, one workgroup per 16-row block ──
+//   X1' = a_L X1 + X1 Phi_MM + X2 Phi_SM + C_M,   X2' = beta_L X1 + h_L X2 + X1 Phi_MS + X2 Phi_SS + C_S
+// ends [chain][nc + 1][64*64]: slot c = adjoint of the state at the start of chunk c (slot nc = 0, slot 0 = the
+// gradient of the initial state, also written to first [chain][64*64]).
+// Wave w: destination w / 4, source (w / 2) % 2, column half w % 2; the two sources of a destination meet in LDS.
+__global__ __launch_bounds__(kThr) void ex_scan_kernel(const float *__restrict__ loc, const float *__restrict__ locs,
+                                                       float *__restrict__ em, float *__restrict__ es_,
+                                                       float *__restrict__ first_m, float *__restrict__ first_s, int nc,
+                                                       int has_s) {
+    extern __shared__ float smem[];
+    float *F = smem;                       // four 64x64 matrices
+    float *X1 = F + 4 * MAT, *X2 = X1 + 16 * LDM, *part = X2 + 16 * LDM;   // part [4][16*33]
+    const int chain = blockIdx.x >> 2, r0 = 16 * (blockIdx.x & 3);
+    const int w = threadIdx.x >> 6, dst = w >> 2, src = (w >> 1) & 1, n0 = 32 * (w & 1), pidx = dst * 2 + (w & 1);
+    float *emp = em + (size_t)chain * (nc + 1) * kDD, *esp = has_s ? es_ + (size_t)chain * (nc + 1) * kDD : nullptr;
+    for (int e = threadIdx.x; e < 16 * 64; e += kThr) {
+        const int rr = e >> 6, cc = e & 63;
+        X1[rr * LDM + cc] = 0.f;
+        X2[rr * LDM + cc] = 0.f;
+        emp[(size_t)nc * kDD + (r0 + rr) * HD + cc] = 0.f;
+        if (esp) esp[(size_t)nc * kDD + (r0 + rr) * HD + cc] = 0.f;
+    }
+    Tile<float> tf[4];
+    Strip cnext = zero_strip(), cadd;
+    float aLn = 0.f, bLn = 0.f, hLn = 0.f, aL, bL, hL;
+    const bool live = has_s || (dst == 0 && src == 0);   // the Delta rule has one state and one matrix
+    auto prefetch = [&](int ci) {
+        const float *lc = loc + ((size_t)chain * nc + ci) * kExLocMats * kDD;
+        const float *sc = locs + ((size_t)chain * nc + ci) * 4;
+        fetch(tf[0], lc, 64);
+        if (has_s) {
+            fetch(tf[1], lc + kDD, 64);
+            fetch(tf[2], lc + 2 * kDD, 64);
+            fetch(tf[3], lc + 3 * kDD, 64);
+        }
+        aLn = sc[0]; bLn = sc[1]; hLn = sc[2];
+        if (src == 0 && live) {
+            const float *Cm = lc + (4 + dst) * kDD;
+            for_c(cnext, [&](int r, int c, float &x) { x = Cm[(r0 + r) * HD + n0 + c]; });
+        }
+    };
+    prefetch(nc - 1);
+    for (int ci = nc - 1; ci >= 0; ci--) {
+        __syncthreads();   // the previous step's readers of F and writers of X1 / X2 are done
+        commit(F, tf[0]);
+        if (has_s) {
+            commit(F + MAT, tf[1]);
+            commit(F + 2 * MAT, tf[2]);
+            commit(F + 3 * MAT, tf[3]);
+        }
+        aL = aLn; bL = bLn; hL = hLn; cadd = cnext;
+        __syncthreads();
+        if (ci > 0) prefetch(ci - 1);
+        Strip acc = zero_strip(), out = zero_strip();
+        if (live) {
+            const float *Xs = src ? X2 : X1;
+            const float *Fm = F + (dst * 2 + src) * MAT;
+            mma(acc, [&](int m, int kk) { return Xs[m * LDM + kk]; }, [&](int kk, int n) { return Fm[kk * LDM + n0 + n]; });
+            if (src) {
+                for_c(acc, [&](int r, int c, float &x) { part[pidx * 16 * 33 + r * 33 + c] = x; });
+            } else {
+                for_c(out, [&](int r, int c, float &x) {
+                    const float x1 = X1[r * LDM + n0 + c];
+                    x = dst ? bL * x1 + hL * X2[r * LDM + n0 + c] : aL * x1;
+                });
+#pragma unroll
+                for (int i = 0; i < 4; i++) { out.t[0][i] += acc.t[0][i] + cadd.t[0][i]; out.t[1][i] += acc.t[1][i] + cadd.t[1][i]; }
+            }
+        }
+        __syncthreads();   // every read of the old X1 / X2 is done; the partial products are in LDS
+        if (live && !src) {
+            float *Xd = dst ? X2 : X1;
+            float *gd = dst ? esp : emp;
+            float *gf = (ci == 0) ? (dst ? first_s : first_m) : nullptr;
+            for_c(out, [&](int r, int c, float &x) {
+                if (has_s) x += part[pidx * 16 * 33 + r * 33 + c];
+                Xd[r * LDM + n0 + c] = x;
+                gd[(size_t)ci * kDD + (r0 + r) * HD + n0 + c] = x;
+                if (gf) gf[(size_t)chain * kDD + (r0 + r) * HD + n0 + c] = x;
+            });
+        }
+    }
+}
+constexpr size_t kExScanLds = (4 * MAT + 2 * 16 * LDM + 4 * 16 * 33) * sizeof(float);
+
+// ── pass 3: gradients of one chunk ──────────────────────────────────────────
+//   pvec [chain][token][4] = <M0, J_t>, <S0, J_t>, -theta_t u_t^T dMo k_t, -theta_t u_t^T dSo k_t
+//   xs [chain][chunk][s][t] as above     scal [chunk][4] = <M0, dMo>, <S0, dMo>, <S0, dSo>
+__global__ __launch_bounds__(kThr) void ex_grads_kernel(
+    const float *__restrict__ k, const float *__restrict__ q, const float *__restrict__ d_y, const float *__restrict__ alpha,
+    const float *__restrict__ theta, const float *__restrict__ eta, const float *__restrict__ m_ckpt,
+    const float *__restrict__ s_ckpt, const float *__restrict__ Tg, const float *__restrict__ Ug,
+    const float *__restrict__ dUg, const float *__restrict__ em, const float *__restrict__ es_, float *__restrict__ d_k,
+    float *__restrict__ d_v, float *__restrict__ d_q, float *__restrict__ d_theta, float *__restrict__ pvec,
+    float *__restrict__ xs, float *__restrict__ scal, int s, int C, int nc, int nck, int has_s) {
+    extern __shared__ float smem[];
+    float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Ts = Ds + MAT, *Us = Ts + MAT, *A1 = Us + MAT, *A2 = A1 + MAT,
+          *Cc = A2 + MAT, *B9 = Cc + MAT;
+    __shared__ Coef cf;
+    __shared__ ChunkVecs cv;
+    __shared__ float part[6][2][CW];   // row sums per column half: p0, ps, g1, g2, dam, dbm
+    __shared__ float part_th[4][CW];   // column sums of dW.c per 16-row block
+    __shared__ float dots[3][8];
+    NLH_STRIP_ORIGIN();
+    const int l = threadIdx.x & 63;
+    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0, task = (size_t)chain * nc + ci;
+    const size_t end = ((size_t)chain * (nc + 1) + ci + 1) * kDD;
+    Tile<float> tm, ts;
+    {
+        Tile<float> tk, tq, td, tt, tu, tdm, tds;
+        fetch(tk, k + tok * HD, L);
+        fetch(tq, q + tok * HD, L);
+        fetch(td, d_y + tok * HD, L);
+        fetch(tt, Tg + task * kDD, 64);
+        fetch(tu, Ug + task * kDD, 64);
+        fetch(tdm, em + end, 64);
+        if (has_s) fetch(tds, es_ + end, 64);
+        fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
+        if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
+        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        load_gates(cf, gt);
+        coefficients(cf, gt, L, Cc, nullptr, nullptr);
+        commit(Ks, tk);
+        commit(Qs, tq);
+        commit(Ds, td);
+        commit(Ts, tt);
+        commit(Us, tu);
+        commit(A1, tdm);
+        if (has_s) commit(A2, tds);
+        const float x0 = wave_allreduce(tile_dot(tm, tdm));
+        const float x1 = has_s ? wave_allreduce(tile_dot(ts, tdm)) : 0.f;
+        const float x2 = has_s ? wave_allreduce(tile_dot(ts, tds)) : 0.f;
+        if (l == 0) { dots[0][w] = x0; dots[1][w] = x1; dots[2][w] = x2; }
+    }
+    __syncthreads();
+    chunk_vectors(cv, cf, L);
+    if (threadIdx.x < 3) {
+        const float *p = dots[threadIdx.x];
+        scal[task * 4 + threadIdx.x] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+    }
+    auto publish = [&](int which, Strip &x) {   // row sums of x -> part[which][column half][row]
+        strip_row_sums(x);
+        if (row_writer()) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) part[which][nh][m0 + row_of(i)] = x.t[0][i];
+        }
+    };
+    auto aK = [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; };
+    auto aU = [&](int m, int kk) { return Us[(m0 + m) * LDM + kk]; };
+    Strip udm = zero_strip(), uds = zero_strip();
+    {
+        Strip kdm = zero_strip(), kds = zero_strip();
+        mma(kdm, aK, [&](int kk, int n) { return A1[(n0 + n) * LDM + kk]; });
+        mma(udm, aU, [&](int kk, int n) { return A1[kk * LDM + n0 + n]; });
+        if (has_s) {
+            mma(kds, aK, [&](int kk, int n) { return A2[(n0 + n) * LDM + kk]; });
+            mma(uds, aU, [&](int kk, int n) { return A2[kk * LDM + n0 + n]; });
+        }
+        __syncthreads();   // the vectors are there
+        const float *gi = dUg + task * kDD;
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                B9[row * LDM + col] = gi[row * HD + col] + cv.wM[row] * kdm.t[tl][i] + cv.wS[row] * kds.t[tl][i];   // dU
+            }
+    }
+    __syncthreads();   // dU complete; dMo, dSo no longer needed
+    Strip p = zero_strip(), g = zero_strip();
+    {
+        Strip dr = zero_strip();
+        mma(dr, [&](int m, int kk) { return Ts[kk * LDM + m0 + m]; }, [&](int kk, int n) { return B9[kk * LDM + n0 + n]; });
+        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        mma(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        for_c(dr, [&](int r, int c, float &x) {
+            if (m0 + r < L) d_v[(tok + m0 + r) * HD + n0 + c] = -x;
+        });
+        __syncthreads();   // T no longer needed
+        for_c(dr, [&](int r, int c, float &x) { Ts[(m0 + r) * LDM + n0 + c] = x; });   // dR
+    }
+    __syncthreads();
+    const float *dRs = Ts;
+    Strip dwa;
+    {
+        Strip dlam = zero_strip(), dyu = zero_strip();
+        auto bU = [&](int kk, int n) { return Us[(n0 + n) * LDM + kk]; };
+        mma(dlam, [&](int m, int kk) { return dRs[(m0 + m) * LDM + kk]; }, bU);
+        mma(dyu, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; }, bU);
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const float nth = -cf.th[col];
+                const float c0 = Cc[row * LDM + col], c1 = row > 0 ? Cc[(row - 1) * LDM + col] : 0.f;
+                const float lam = (col < row && row < L) ? dlam.t[tl][i] : 0.f;
+                const float yu = (col <= row && row < L) ? dyu.t[tl][i] : 0.f;
+                B9[row * LDM + col] = nth * c0 * yu;            // dP = W . tril(dY U^T)
+                A2[row * LDM + col] = lam * g.t[tl][i];         // dLam . G, read one row down below
+                const float dg = nth * c1 * lam;                // dG, stored symmetrised
+                if (col < row) { A1[row * LDM + col] = dg; A1[col * LDM + row] = dg; }
+                if (col == row) A1[row * LDM + col] = 0.f;
+                dwa.t[tl][i] = yu * p.t[tl][i];
+            }
+    }
+    __syncthreads();
+    {
+        float *xo = xs + task * CW * CW;
+        float cs[2] = {0.f, 0.f};
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const float dw = dwa.t[tl][i] + (row + 1 < CW ? A2[(row + 1) * LDM + col] : 0.f);
+                xo[col * CW + row] = -cf.th[col] * dw;          // [s][t]
+                cs[tl] = fmaf(dw, Cc[row * LDM + col], cs[tl]);
+            }
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++) {
+            float x = xor_add<16>(cs[tl]);
+            x = xor_add<32>(x);
+            if (l < 16) part_th[w >> 1][n0 + 16 * tl + l] = x;
+        }
+    }
+    __syncthreads();   // c and U no longer needed
+    commit(Us, tm);
+    if (has_s) commit(Cc, ts);
+    __syncthreads();
+    const float *M0s = Us, *S0s = Cc, *dPs = B9, *dGs = A1;
+    {
+        Strip dym = zero_strip(), dys = zero_strip(), dq = zero_strip(), r0 = zero_strip(), r1 = zero_strip();
+        auto aD = [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; };
+        mma(dym, aD, [&](int kk, int n) { return M0s[kk * LDM + n0 + n]; });
+        if (has_s) mma(dys, aD, [&](int kk, int n) { return S0s[kk * LDM + n0 + n]; });
+        mma(dq, [&](int m, int kk) { return dPs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const float qv = Qs[row * LDM + col];
+                r0.t[tl][i] = dym.t[tl][i] * qv;
+                r1.t[tl][i] = dys.t[tl][i] * qv;
+                if (row < L)
+                    d_q[(tok + row) * HD + col] = cf.a[row] * dym.t[tl][i] + cf.beta[row] * dys.t[tl][i] + dq.t[tl][i];
+            }
+        publish(0, r0);
+        publish(1, r1);
+    }
+    {
+        Strip dk = zero_strip(), drm = zero_strip(), drs = zero_strip(), r2 = zero_strip(), r3 = zero_strip(),
+              r4 = zero_strip(), r5 = zero_strip();
+        auto aR = [&](int m, int kk) { return dRs[(m0 + m) * LDM + kk]; };
+        mma(dk, [&](int m, int kk) { return dPs[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+        mma(dk, [&](int m, int kk) { return dGs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
+        mma(drm, aR, [&](int kk, int n) { return M0s[kk * LDM + n0 + n]; });
+        if (has_s) mma(drs, aR, [&](int kk, int n) { return S0s[kk * LDM + n0 + n]; });
+#pragma unroll
+        for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const float kv = Ks[row * LDM + col];
+                r2.t[tl][i] = udm.t[tl][i] * kv;
+                r3.t[tl][i] = uds.t[tl][i] * kv;
+                r4.t[tl][i] = drm.t[tl][i] * kv;
+                r5.t[tl][i] = drs.t[tl][i] * kv;
+                if (row < L)
+                    d_k[(tok + row) * HD + col] = dk.t[tl][i] + cv.wM[row] * udm.t[tl][i] + cv.wS[row] * uds.t[tl][i] +
+                                                  cv.am[row] * drm.t[tl][i] + cv.bm[row] * drs.t[tl][i];
+            }
+        publish(2, r2);
+        publish(3, r3);
+        publish(4, r4);
+        publish(5, r5);
+    }
+    __syncthreads();
+    if (threadIdx.x < L) {
+        const int t = threadIdx.x;
+        auto sum = [&](int which, int row) { return part[which][0][row] + part[which][1][row]; };
+        const float g1 = sum(2, t), g2 = sum(3, t);
+        const float dam = t + 1 < CW ? sum(4, t + 1) : 0.f, dbm = t + 1 < CW ? sum(5, t + 1) : 0.f;
+        d_theta[tok + t] = -(((part_th[0][t] + part_th[1][t]) + (part_th[2][t] + part_th[3][t])) + cf.cl[t] * g1 + cf.bl[t] * g2);
+        float *pv = pvec + (tok + t) * 4;
+        pv[0] = sum(0, t) + dam;
+        pv[1] = sum(1, t) + dbm;
+        pv[2] = -cf.th[t] * g1;
+        pv[3] = -cf.th[t] * g2;
+    }
+}
+constexpr size_t kExGradsLds = 9 * MAT * sizeof(float);
+
+template <class K>
+void set_lds(K kernel, size_t bytes) {
+    check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)bytes), "dynamic LDS size");
+}
+
+}  // namespace
+
+bool exact_backward_mm_applies(int d, int C) { return d == HD && C >= 1 && C <= CW; }
+
+bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *v, const float *q, const float *alpha,
+                       const float *theta, const float *eta, const float *m_ckpt, const float *s_ckpt, const float *d_y,
+                       float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
+                       float *d_s_initial, int seq_len, int batch, int C, float error_clip, float m_norm_guard) {
+    const ErrorScope es;
+    const int nc = ceil_div(seq_len, C), nck = n_ckpt_count(seq_len, C);
+    const size_t nchunks = (size_t)batch * nc;
+    const bool guard = error_clip > 0.f || m_norm_guard > 0.f;
+    ChainTracks tracks{nullptr, nullptr};
+    if (guard) tracks = chain_tracks(seq_len, batch, C);
+    float *loc = scratch(32, nchunks * kExLocMats * kDD * sizeof(float));
+    float *Tg = scratch(33, nchunks * kDD * sizeof(float));
+    float *Ug = scratch(34, nchunks * kDD * sizeof(float));
+    float *dUg = scratch(35, nchunks * kDD * sizeof(float));
+    float *locs = scratch(4, nchunks * 4 * sizeof(float));
+    float *em = scratch(5, (size_t)batch * (nc + 1) * kDD * sizeof(float));
+    float *esn = has_s ? scratch(6, (size_t)batch * (nc + 1) * kDD * sizeof(float)) : nullptr;
+    float *xs = scratch(7, nchunks * CW * CW * sizeof(float));
+    float *pvec = scratch(8, (size_t)batch * seq_len * 4 * sizeof(float));
+    float *scal = scratch(9, nchunks * 4 * sizeof(float));
+    const int per = 8, rows = ceil_div(batch, per), nsum = has_s ? 2 : 1;
+    float *tmp = scratch(10, (size_t)nsum * rows * kDD * sizeof(float));
+    float *first = scratch(36, (size_t)2 * batch * kDD * sizeof(float));
+    if (es.failed()) return true;
+    float *first_m = first, *first_s = first + (size_t)batch * kDD;
+    static bool attr_set = false;
+    if (!attr_set) {
+        set_lds(ex_local_kernel<false>, kExLocalLds);
+        set_lds(ex_local_kernel<true>, kExLocalLds);
+        set_lds(ex_scan_kernel, kExScanLds);
+        set_lds(ex_grads_kernel, kExGradsLds);
+        attr_set = true;
+    }
+    if (es.failed()) return true;
+    {
+        KernelTimer kt("ex_local_kernel");
+        if (guard)
+            hipLaunchKernelGGL(ex_local_kernel<true>, dim3((unsigned)nchunks), dim3(kThr), kExLocalLds, stream(), k, v, q, d_y,
+                               alpha, theta, eta, m_ckpt, s_ckpt, loc, locs, Tg, Ug, dUg, seq_len, C, nc, nck, (int)has_s, tracks);
+        else
+            hipLaunchKernelGGL(ex_local_kernel<false>, dim3((unsigned)nchunks), dim3(kThr), kExLocalLds, stream(), k, v, q, d_y,
+                               alpha, theta, eta, m_ckpt, s_ckpt, loc, locs, Tg, Ug, dUg, seq_len, C, nc, nck, (int)has_s, tracks);
+        check_launch("ex_local_kernel");
+    }
+    {
+        KernelTimer kt("ex_scan_kernel");
+        hipLaunchKernelGGL(ex_scan_kernel, dim3((unsigned)batch * 4), dim3(kThr), kExScanLds, stream(), loc, locs, em, esn,
+                           first_m, first_s, nc, (int)has_s);
+        check_launch("ex_scan_kernel");
+    }
+    {
+        KernelTimer kt("ex_grads_kernel");
+        hipLaunchKernelGGL(ex_grads_kernel, dim3((unsigned)nchunks), dim3(kThr), kExGradsLds, stream(), k, q, d_y, alpha, theta,
+                           eta, m_ckpt, s_ckpt, Tg, Ug, dUg, em, esn, d_k, d_v, d_q, d_theta, pvec, xs, scal, seq_len, C, nc, nck,
+                           (int)has_s);
+        check_launch("ex_grads_kernel");
+    }
+    chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, C, has_s, first_m, first_s, kDD, per,
+                             nsum, tmp);
+    if (es.failed()) return true;
+    if (guard && couplings_may_fire_tracked(k, alpha, theta, eta, tracks, has_s, seq_len, batch, C, error_clip, m_norm_guard))
+        return false;
+    accumulate_over_batch2(tmp, d_m_initial, has_s ? tmp + (size_t)rows * kDD : nullptr, d_s_initial, rows, (int)kDD);
+    return true;
+}
+
+}  // namespace nlh

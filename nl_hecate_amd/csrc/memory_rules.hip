@@ -28,6 +28,7 @@
 #include "../../include/nl_hecate_ffi.h"
 #include "chunkwise_guard.h"
 #include "rule_args.h"
+#include "exact_mm.h"
 #include "rule_common.h"
 
 namespace nlh {
@@ -834,6 +835,7 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
 
 // One-call checkpointed / chunkwise backward: fused on-chip replay when it
 // covers the case, the replay-through-memory schedule otherwise.
+constexpr int kExactMmMinInterval = 32;
 static void backward_ckpt_any(bool has_s, bool frozen, bool allow_fused,
                               const float *k, const float *v, const float *q,
                               const float *alpha, const float *theta, const float *eta,
@@ -848,6 +850,29 @@ static void backward_ckpt_any(bool has_s, bool frozen, bool allow_fused,
     // no clip: the fused kernel replays without the projection; with a bound it checks afterwards that none could
     // have fired (see launch_fwd) and otherwise leaves the call to the replay schedule below
     const bool bound = coupled_needed(0.f, m_norm_max);
+    // chunk-parallel matrix form: checkpoint intervals long enough that a 64-token tile is mostly tokens.  Under a
+    // clip or a bound it tests afterwards that neither could have fired.  A caller whose couplings do fire should not
+    // pay for a pass that is thrown away every step: after a test that fired, the next calls (1, 2, 4 .. 64 of them,
+    // doubling while the tests keep firing) go to the sequential kernels directly, and so does a call under a bound
+    // right after any other test of a bound that fired.
+    const bool coupled = bound || error_clip > 0.f;
+    static int skip_left = 0, skip_len = 0;
+    bool try_mm = allow_fused && !frozen && exact_backward_mm_applies(d, C) && C >= kExactMmMinInterval;
+    if (try_mm && coupled) {
+        if (!guard_possible()) try_mm = false;
+        else if (skip_left > 0) { skip_left--; try_mm = false; }
+        else if (error_clip <= 0.f && last_test_fired) try_mm = false;
+    }
+    if (try_mm) {
+        if (exact_backward_mm(fn, has_s, k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v, d_q, d_alpha, d_theta,
+                              d_eta, d_m_initial, d_s_initial, seq_len, batch, C, error_clip, bound ? m_norm_max : 0.f)) {
+            if (coupled) skip_len = 0;
+            return;
+        }
+        skip_len = skip_len ? (skip_len < 64 ? 2 * skip_len : 64) : 1;
+        skip_left = skip_len;
+        allow_fused = false;   // the test fired: the fused kernel's own test would fire too
+    }
     if (allow_fused && error_clip <= 0.f && (!bound || guard_possible()) &&
         backward_ckpt_fused(has_s, frozen, k, v, q, alpha, theta, eta, m_ckpt, s_ckpt, d_y, d_k, d_v,
                             d_q, d_alpha, d_theta, d_eta, d_m_initial, d_s_initial, seq_len, d, batch, C,

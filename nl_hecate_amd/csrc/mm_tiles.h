@@ -96,6 +96,17 @@ __device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
         }
     }
 }
+// One 16x16 tile, contraction over the 16 indices k0 .. k0 + 15 only (block-diagonal operands):
+// acc += sum_{k0 <= k < k0+16} a(m,k) b(k,n), m, n in [0,16).
+template <class FA, class FB>
+__device__ __forceinline__ void mma_tile16(f32x4 &acc, FA a, FB b, int k0) {
+    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4;
+    float av[4], bv[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { av[i] = a(r, k0 + 4 * i + kq); bv[i] = b(k0 + 4 * i + kq, r); }
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[i], acc, 0, 0, 0);
+}
 // Element i of tile tl of lane l is C[4*(l/16) + i][16*tl + l%16] of the strip.
 template <class F>
 __device__ __forceinline__ void for_c(Strip &acc, F f) {

@@ -33,7 +33,7 @@ hipStream_t stream();   // launch stream (the null stream unless nlh_set_stream 
 // a HIP graph captured earlier still holds the old address and must be dropped, not replayed.
 // While the launch stream is being captured a slot cannot grow: the call fails instead.
 float *scratch(int slot, size_t bytes);
-constexpr int kScratchSlots = 32;
+constexpr int kScratchSlots = 40;
 
 // Optional per-kernel timing: while enabled (nlh_kernel_timer_enable), a
 // KernelTimer around a launch records an event pair on the launch stream;
