@@ -51,6 +51,10 @@ float nlh_timer_stop_ms(void);
 int nlh_kernel_timer_enable(int on);
 float nlh_kernel_timer_read_ms(int *launches, char *name, int name_len);
 int nlh_kernel_timer_report(char *buf, int buf_len);
+/* Which form the checkpointed backward of the exact rules takes where several apply (see
+ * titans_backward_ckpt_f32_rocm): 0 = by the cost model (default), 1 = the matrix form wherever it applies,
+ * 2 = never the matrix form.  Returns the previous setting.  No counterpart in the reference; for tests and tuning. */
+int nlh_exact_backward_form(int mode);
 /* Runs the cross-lane primitives on known data; returns 0 when all agree. */
 int nlh_selftest_lane_ops(void);
 /* Gate coefficients of one chunk (L <= 64 device-resident gates each) from the in-kernel generator:
@@ -287,9 +291,14 @@ void delta_backward_ckpt_replay_f32_rocm(const float *k_mem, const float *v_mem,
                                          float *d_alpha, float *d_theta, float *d_m_initial,
                                          int seq_len, int d, int batch_size, int checkpoint_interval,
                                          float error_clip, float m_norm_max);
-/* Fused form: the replayed trajectory stays in LDS and registers (two-level
- * recomputation inside one kernel); takes the `_replay_` schedule instead when
- * clip / projection is active or checkpoint_interval > 64. */
+/* One call over all segments (the loop of core/src/gpu_backward.rs:1770-1962 inside the library).  Three forms, chosen
+ * per call: (1) head size 64, checkpoint_interval <= 64: the rule in chunk-parallel matrix form on the fp32 matrix
+ * cores (a triangular solve per segment, an adjoint scan over the segments, gradients per segment), taken where a cost
+ * model says it beats (2) at the call's shape (long intervals, or few chains); (2) the fused form: the replayed
+ * trajectory stays in LDS and registers (two-level recomputation inside one kernel), checkpoint_interval <= 64;
+ * (3) the `_replay_` schedule.  With a finite m_norm_max (1) and (2) end with a device-side test that the bound
+ * could not have been reached and leave the call to (3) when it could; with an error clip (1) does the same and
+ * (2) is not used. */
 void titans_backward_ckpt_f32_rocm(const float *k_mem, const float *v_mem, const float *q_mem,
                                    const float *alpha, const float *theta, const float *eta,
                                    const float *m_ckpt, const float *s_ckpt, const float *d_y,

@@ -5,6 +5,7 @@
 namespace nlh {
 
 bool exact_backward_mm_applies(int d, int C);
+bool exact_backward_mm_pays(int seq_len, int batch, int C);   // faster than the fused sequential kernel at this shape
 // error_clip / m_norm_guard > 0: the pass also leaves the error and state norms behind and ends with the test of
 // whether a coupling could have fired, BEFORE anything is added to d_m_initial / d_s_initial; false: one may have,
 // the caller runs the kernels that apply the couplings, which overwrite every other output.  s_ckpt, eta, d_eta,

@@ -48,8 +48,10 @@ namespace {
 
 using namespace mmt;
 
+// Waves w and w + 4 share a SIMD.  Products with the lower triangular T (or its transpose) cost a 16-row block
+// ib + 1 (or 4 - ib) quarter products, so the row blocks are dealt out as (0, 3) and (1, 2) per SIMD.
 #define NLH_STRIP_ORIGIN() \
-    const int w = threadIdx.x >> 6, m0 = 16 * (w >> 1), n0 = 32 * (w & 1), nh = w & 1; \
+    const int w = threadIdx.x >> 6, ib = w < 4 ? w >> 1 : 3 - ((w - 4) >> 1), m0 = 16 * ib, n0 = 32 * (w & 1), nh = w & 1; \
     (void)nh
 
 // per chunk, for the scan: Phi_MM, Phi_SM, Phi_MS, Phi_SS (source state, destination state), C_M, C_S
@@ -94,6 +96,8 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
     const size_t tok = (size_t)chain * s + t0, task = (size_t)chain * nc + ci;
     {
+        // the gates first: the coefficient loops wait for them only and run while the tiles are in flight
+        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
         Tile<float> tk, tv, tq, td, tm, ts;
         fetch(tk, k + tok * HD, L);
         fetch(tv, v + tok * HD, L);
@@ -101,7 +105,6 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         fetch(td, d_y + tok * HD, L);
         fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
         if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
-        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
         load_gates(cf, gt);
         coefficients(cf, gt, L, Cc, nullptr, nullptr);
         commit(Ks, tk);
@@ -129,7 +132,6 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         if (has_s) mma(ks, aK, [&](int kk, int n) { return Ss[(n0 + n) * LDM + kk]; });
         mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
         __syncthreads();   // the vectors are there
-        Strip e2 = zero_strip();
 #pragma unroll
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
@@ -142,7 +144,6 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
                 B8[row * LDM + col] = (col < row) ? nth * Cc[(row - 1) * LDM + col] * g.t[tl][i] : 0.f;   // Lam
                 B9[row * LDM + col] = nth * Cc[row * LDM + col] * p.t[tl][i];                            // W.P
             }
-        (void)e2;
     }
     __syncthreads();
     Strip dul = zero_strip();
@@ -164,7 +165,6 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     }
     __syncthreads();
     {   // N = D Lam_off -> Ss; dU_loc -> B9 and out
-        const int ib = w >> 1;
 #pragma unroll
         for (int tl = 0; tl < 2; tl++) {
             const int jb = 2 * (w & 1) + tl;
@@ -182,19 +182,29 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         });
     }
     __syncthreads();
-    {   // N^2 -> B8
-        Strip n2 = zero_strip();
-        mma(n2, [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ss[kk * LDM + n0 + n]; });
-        for_c(n2, [&](int r, int c, float &x) { B8[(m0 + r) * LDM + n0 + c] = x; });
+    auto aN = [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; };
+    // N is strictly block lower triangular (blocks of 16): its powers need only the block products that can be non-zero
+#pragma unroll
+    for (int tl = 0; tl < 2; tl++) {   // N^2 -> B8
+        const int jb = 2 * (w & 1) + tl;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int kb = jb + 1; kb < ib; kb++)
+            mma_tile16(acc, aN, [&](int kk, int n) { return Ss[kk * LDM + 16 * jb + n]; }, 16 * kb);
+#pragma unroll
+        for (int i = 0; i < 4; i++) B8[(m0 + row_of(i)) * LDM + 16 * jb + (l & 15)] = acc[i];
     }
     __syncthreads();
-    {   // X = (I + N)(I + N^2) -> Cc
-        Strip x3 = zero_strip();
-        mma(x3, [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return B8[kk * LDM + n0 + n]; });
-        for_c(x3, [&](int r, int c, float &x) {
-            const int row = m0 + r, col = n0 + c;
-            Cc[row * LDM + col] = x + Ss[row * LDM + col] + B8[row * LDM + col] + (row == col ? 1.f : 0.f);
-        });
+#pragma unroll
+    for (int tl = 0; tl < 2; tl++) {   // X = (I + N)(I + N^2) = I + N + N^2 + N N^2 -> Cc
+        const int jb = 2 * (w & 1) + tl;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int kb = jb + 2; kb < ib; kb++)
+            mma_tile16(acc, aN, [&](int kk, int n) { return B8[kk * LDM + 16 * jb + n]; }, 16 * kb);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = m0 + row_of(i), col = 16 * jb + (l & 15);
+            Cc[row * LDM + col] = acc[i] + Ss[row * LDM + col] + B8[row * LDM + col] + (row == col ? 1.f : 0.f);
+        }
     }
     __syncthreads();
     {   // T = X D -> Ss and out
@@ -217,9 +227,11 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     {   // U = T R -> out;  Z1 = T (am.K) -> B8,  Z2 = T (bm.K) -> Ms
         Strip u = zero_strip(), z1 = zero_strip(), z2 = zero_strip();
         auto aT = [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; };
-        mma(u, aT, [&](int kk, int n) { return Vs[kk * LDM + n0 + n]; });
-        mma(z1, aT, [&](int kk, int n) { return cv.am[kk] * Ks[kk * LDM + n0 + n]; });
-        if (has_s) mma(z2, aT, [&](int kk, int n) { return cv.bm[kk] * Ks[kk * LDM + n0 + n]; });
+        // T is lower triangular: row block ib contracts over the first ib + 1 blocks of 16 (taken in pairs)
+        const int pe = (ib >> 1) + 1;
+        mma_range(u, aT, [&](int kk, int n) { return Vs[kk * LDM + n0 + n]; }, 0, pe);
+        mma_range(z1, aT, [&](int kk, int n) { return cv.am[kk] * Ks[kk * LDM + n0 + n]; }, 0, pe);
+        if (has_s) mma_range(z2, aT, [&](int kk, int n) { return cv.bm[kk] * Ks[kk * LDM + n0 + n]; }, 0, pe);
         float *go = Ug + task * kDD;
         for_c(u, [&](int r, int c, float &x) { go[(m0 + r) * HD + n0 + c] = x; });
         for_c(z1, [&](int r, int c, float &x) { B8[(m0 + r) * LDM + n0 + c] = x; });
@@ -294,7 +306,11 @@ __global__ __launch_bounds__(kThr) void ex_scan_kernel(const float *__restrict__
     extern __shared__ float smem[];
     float *F = smem;                       // four 64x64 matrices
     float *X1 = F + 4 * MAT, *X2 = X1 + 16 * LDM, *part = X2 + 16 * LDM;   // part [4][16*33]
-    const int chain = blockIdx.x >> 2, r0 = 16 * (blockIdx.x & 3);
+    // the four row blocks of a chain sit 8 workgroups apart: consecutive workgroups go to consecutive XCDs, so the
+    // four share one XCD's L2 for the chunk matrices they all read
+    const int chain0 = (blockIdx.x & 7) + 8 * (blockIdx.x >> 5), rb0 = (blockIdx.x >> 3) & 3;
+    const bool whole = (int)(blockIdx.x | 31) < (int)gridDim.x;   // a full group of 32 workgroups
+    const int chain = whole ? chain0 : blockIdx.x >> 2, r0 = 16 * (whole ? rb0 : blockIdx.x & 3);
     const int w = threadIdx.x >> 6, dst = w >> 2, src = (w >> 1) & 1, n0 = 32 * (w & 1), pidx = dst * 2 + (w & 1);
     float *emp = em + (size_t)chain * (nc + 1) * kDD, *esp = has_s ? es_ + (size_t)chain * (nc + 1) * kDD : nullptr;
     for (int e = threadIdx.x; e < 16 * 64; e += kThr) {
@@ -392,6 +408,7 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
     const size_t end = ((size_t)chain * (nc + 1) + ci + 1) * kDD;
     Tile<float> tm, ts;
     {
+        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);   // first: see ex_local_kernel
         Tile<float> tk, tq, td, tt, tu, tdm, tds;
         fetch(tk, k + tok * HD, L);
         fetch(tq, q + tok * HD, L);
@@ -402,7 +419,6 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
         if (has_s) fetch(tds, es_ + end, 64);
         fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
         if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
-        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
         load_gates(cf, gt);
         coefficients(cf, gt, L, Cc, nullptr, nullptr);
         commit(Ks, tk);
@@ -455,7 +471,9 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
     Strip p = zero_strip(), g = zero_strip();
     {
         Strip dr = zero_strip();
-        mma(dr, [&](int m, int kk) { return Ts[kk * LDM + m0 + m]; }, [&](int kk, int n) { return B9[kk * LDM + n0 + n]; });
+        // T^T is upper triangular: row block ib contracts over the blocks ib .. 3 of 16 (taken in pairs)
+        mma_range(dr, [&](int m, int kk) { return Ts[kk * LDM + m0 + m]; }, [&](int kk, int n) { return B9[kk * LDM + n0 + n]; },
+                  ib >> 1, 2);
         mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
         mma(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
         for_c(dr, [&](int r, int c, float &x) {
@@ -506,7 +524,7 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
         for (int tl = 0; tl < 2; tl++) {
             float x = xor_add<16>(cs[tl]);
             x = xor_add<32>(x);
-            if (l < 16) part_th[w >> 1][n0 + 16 * tl + l] = x;
+            if (l < 16) part_th[ib][n0 + 16 * tl + l] = x;
         }
     }
     __syncthreads();   // c and U no longer needed
@@ -586,6 +604,16 @@ void set_lds(K kernel, size_t bytes) {
 }  // namespace
 
 bool exact_backward_mm_applies(int d, int C) { return d == HD && C >= 1 && C <= CW; }
+
+// Cost model from measurements on one MI355X: a chunk costs the two chunk-parallel kernels about 72 us of a compute
+// unit whatever its length, a scan step 4 us; the fused sequential kernel walks a chain's tokens at 0.6 us each on a
+// quarter of a compute unit's worth of workgroups (four per chain).
+bool exact_backward_mm_pays(int seq_len, int batch, int C) {
+    const int nc = ceil_div(seq_len, C), cus = compute_units();
+    const double t_mm = (double)ceil_div(batch * nc, cus) * 72.0 + nc * 4.0;
+    const double t_seq = (double)seq_len * 0.6 * ceil_div(batch * 4, cus);
+    return t_mm < t_seq;
+}
 
 bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *v, const float *q, const float *alpha,
                        const float *theta, const float *eta, const float *m_ckpt, const float *s_ckpt, const float *d_y,

@@ -835,7 +835,7 @@ static void backward_ckpt_replay(const float *k, const float *v, const float *q,
 
 // One-call checkpointed / chunkwise backward: fused on-chip replay when it
 // covers the case, the replay-through-memory schedule otherwise.
-constexpr int kExactMmMinInterval = 32;
+static int g_exact_form = 0;   // nlh_exact_backward_form
 static void backward_ckpt_any(bool has_s, bool frozen, bool allow_fused,
                               const float *k, const float *v, const float *q,
                               const float *alpha, const float *theta, const float *eta,
@@ -850,14 +850,15 @@ static void backward_ckpt_any(bool has_s, bool frozen, bool allow_fused,
     // no clip: the fused kernel replays without the projection; with a bound it checks afterwards that none could
     // have fired (see launch_fwd) and otherwise leaves the call to the replay schedule below
     const bool bound = coupled_needed(0.f, m_norm_max);
-    // chunk-parallel matrix form: checkpoint intervals long enough that a 64-token tile is mostly tokens.  Under a
-    // clip or a bound it tests afterwards that neither could have fired.  A caller whose couplings do fire should not
-    // pay for a pass that is thrown away every step: after a test that fired, the next calls (1, 2, 4 .. 64 of them,
-    // doubling while the tests keep firing) go to the sequential kernels directly, and so does a call under a bound
-    // right after any other test of a bound that fired.
+    // chunk-parallel matrix form where it is the faster one (long checkpoint intervals, or too few chains to fill the
+    // chip with one sequential walk each).  Under a clip or a bound it tests afterwards that neither could have fired.
+    // A caller whose couplings do fire should not pay for a pass that is thrown away every step: after a test that
+    // fired, the next calls (1, 2, 4 .. 64 of them, doubling while the tests keep firing) go to the sequential kernels
+    // directly, and so does a call under a bound right after any other test of a bound that fired.
     const bool coupled = bound || error_clip > 0.f;
     static int skip_left = 0, skip_len = 0;
-    bool try_mm = allow_fused && !frozen && exact_backward_mm_applies(d, C) && C >= kExactMmMinInterval;
+    bool try_mm = allow_fused && !frozen && exact_backward_mm_applies(d, C) && g_exact_form != 2 &&
+                  (g_exact_form == 1 || exact_backward_mm_pays(seq_len, batch, C));
     if (try_mm && coupled) {
         if (!guard_possible()) try_mm = false;
         else if (skip_left > 0) { skip_left--; try_mm = false; }
@@ -893,6 +894,12 @@ using namespace nlh;
 
 // ───────────────────────────── C ABI ───────────────────────────────────────
 extern "C" {
+
+int nlh_exact_backward_form(int mode) {
+    const int prev = g_exact_form;
+    if (mode >= 0 && mode <= 2) g_exact_form = mode;
+    return prev;
+}
 
 void titans_forward_f32_cuda(const float *k_mem, const float *v_mem, const float *q_mem,
                              const float *alpha, const float *theta, const float *eta,

@@ -72,20 +72,24 @@ __device__ __forceinline__ Strip zero_strip() {
     return z;
 }
 // acc += sum_{k<64} a(m,k) b(k,n), m in [0,16), n in [0,32).
-// Operand layout of v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][l/16] and B[l/16][l%16].
+// Operand layout of v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][j] and B[j][l%16] with j = l/16 of the step's four
+// contraction indices.  Which four indices a step takes is free (a sum), so lane group l/16 walks through its own
+// block of 16 indices: with the odd row stride LDM an operand element X[row][col] sits in bank (row + col) % banks, and
+// the lanes of one read then differ by l%16 + 16 (l/16), i.e. fall on different banks whichever way the matrix is
+// read (the assignment 4 i + l/16 put up to four lanes on a bank).
 // Sixteen k-steps in four groups; the operands of group g+1 are read while group g runs.
 template <class FA, class FB>
 __device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
-    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4;
+    const int l = threadIdx.x & 63, r = l & 15, kb = 16 * (l >> 4);
     float av[2][4], b0[2][4], b1[2][4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) { av[0][i] = a(r, 4 * i + kq); b0[0][i] = b(4 * i + kq, r); b1[0][i] = b(4 * i + kq, 16 + r); }
+    for (int i = 0; i < 4; i++) { av[0][i] = a(r, kb + i); b0[0][i] = b(kb + i, r); b1[0][i] = b(kb + i, 16 + r); }
 #pragma unroll
     for (int g = 0; g < 4; g++) {
         if (g < 3) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int kk = 16 * (g + 1) + 4 * i + kq;
+                const int kk = kb + 4 * (g + 1) + i;
                 av[(g + 1) & 1][i] = a(r, kk); b0[(g + 1) & 1][i] = b(kk, r); b1[(g + 1) & 1][i] = b(kk, 16 + r);
             }
         }
@@ -93,6 +97,29 @@ __device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
         for (int i = 0; i < 4; i++) {
             acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g & 1][i], b0[g & 1][i], acc.t[0], 0, 0, 0);
             acc.t[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g & 1][i], b1[g & 1][i], acc.t[1], 0, 0, 0);
+        }
+    }
+}
+// The same over the contraction indices 32 p0 .. 32 p1 - 1 only (wave-uniform bounds): triangular operands.  Lane
+// group j = l/16 takes the indices 32 p + 16 (j % 2) + 8 (j / 2) + 0..7 of a block of 32: the two groups of a
+// half-wave stay 16 banks apart.
+template <class FA, class FB>
+__device__ __forceinline__ void mma_range(Strip &acc, FA a, FB b, int p0, int p1) {
+    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4, kb = 16 * (kq & 1) + 8 * (kq >> 1);
+    for (int p = p0; p < p1; p++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float av[4], b0[4], b1[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int kk = 32 * p + kb + 4 * h + i;
+                av[i] = a(r, kk); b0[i] = b(kk, r); b1[i] = b(kk, 16 + r);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                acc.t[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], b0[i], acc.t[0], 0, 0, 0);
+                acc.t[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], b1[i], acc.t[1], 0, 0, 0);
+            }
         }
     }
 }

@@ -67,6 +67,14 @@ def check(got, gs, tol=1e-4):
 F32_MAX = float(np.finfo(np.float32).max)
 
 
+@pytest.fixture(autouse=True)
+def matrix_form_wherever_it_applies():
+    """The library picks the form by a cost model (short test sequences would go to the sequential kernel)."""
+    prev = lib.nlh_exact_backward_form(1)
+    yield
+    lib.nlh_exact_backward_form(prev)
+
+
 @pytest.mark.parametrize("B,s,C", [(3, 128, 64), (5, 200, 64), (2, 64, 64), (4, 100, 32), (1, 330, 48), (7, 65, 64), (2, 40, 64)])
 def test_titans_against_the_token_loops(B, s, C):
     x = rule_inputs(B, s, 64, seed=101 + s, m0_scale=0.02)
@@ -169,3 +177,19 @@ def test_error_clip_that_never_fires_and_one_that_does():
     got4 = gpu_backward(x, cks, C, F32_MAX, clip=2.0 * werr)
     check(got4, gs)
     assert "ex_grads_kernel" in got4[3], got4[3]
+
+
+def test_cost_model_picks_the_form():
+    """Default setting: one long chain goes to the matrix form (the sequential kernel would leave the chip idle),
+    many 8-token chains stay on the sequential kernel; both match the token loops."""
+    lib.nlh_exact_backward_form(0)
+    x = rule_inputs(1, 1024, 64, seed=149, m0_scale=0.02)
+    cks, gs = oracle_pair(x, 64)
+    got = gpu_backward(x, cks, 64, F32_MAX)
+    check(got, gs)
+    assert "ex_grads_kernel" in got[3], got[3]
+    x = rule_inputs(300, 8, 64, seed=151, m0_scale=0.02)
+    cks, gs = oracle_pair(x, 8)
+    got = gpu_backward(x, cks, 8, F32_MAX)
+    check(got, gs)
+    assert "ex_grads_kernel" not in got[3] and "rule_bwd_fused_kernel" in got[3], got[3]

@@ -85,8 +85,8 @@ def test_bound_never_reached_keeps_the_row_split_kernels(B, s, d, C):
     check_ckpt_pair(x, C, 100.0, got)
     ran_f, ran_b = got[5], got[6]
     assert "norm_bound_kernel" in ran_f, ran_f
-    if d == 64 and C >= 32:   # the chunk-parallel matrix form and its test on the error norms
-        assert "ex_grads_kernel" in ran_b and "cw_guard_tracks_kernel" in ran_b, ran_b
+    if "ex_grads_kernel" in ran_b:   # the cost model took the chunk-parallel matrix form: its test is on the error norms
+        assert d == 64 and "cw_guard_tracks_kernel" in ran_b, ran_b
     else:
         assert "rule_bwd_fused_kernel" in ran_b and "norm_bound_kernel" in ran_b, ran_b
     assert not any(n.startswith("rule_bwd_traj") or n == "rule_fwd_kernel" for n in ran_b), ran_b   # no replay schedule
