@@ -54,6 +54,13 @@ PEAK_BF16_TFLOPS = 2500.0
 D_HEAD = 64
 FLOP_FWD = 9 * D_HEAD * D_HEAD
 FLOP_BWD = 30 * D_HEAD * D_HEAD
+# The checkpointed backward in chunk-parallel matrix form executes more than the token loop's 30 d^2: per 64-token
+# chunk, in 64^3 products (2 * 64^3 flop each, block-sparse ones counted by the blocks they issue): chunk-local pass
+# 15.6 (Gram and state products 4, (W.P)^T dY 1, blocked inverse 0.35, T R and T (m.K) 2.25, scan matrices 4, additive
+# terms 4), gradient pass 15.75, adjoint scan 4.
+EXACT_MM_PRODUCTS = {"ex_local_kernel": 15.6, "ex_grads_kernel": 15.75, "ex_scan_kernel": 4.0}
+FLOP_EXACT_MM = {k: v * 2 * 64 ** 3 / 64 for k, v in EXACT_MM_PRODUCTS.items()}   # per head-token
+FLOP_BWD_MM = sum(FLOP_EXACT_MM.values())
 BYTES_FWD = 1548
 BYTES_BWD = 2328
 
@@ -215,10 +222,13 @@ def setup_titans_exact_c2(torch, D, lib, m_norm_max=None):
 
     return dict(
         fwd=fwd, bwd=bwd, tokens=bs * s, head_tokens=B * s,
-        flop_fwd=FLOP_FWD, flop_bwd=FLOP_BWD, bytes_fwd=BYTES_FWD, bytes_bwd=BYTES_BWD,
-        # own algorithmic flops per head-token of the instrumented kernels
-        kernel_work={"rule_fwd_kernel": FLOP_FWD, "rule_bwd_fused_kernel": FLOP_BWD},
-        kernel_names={"forward": "forward_ckpt", "backward": "backward_ckpt_fused"},
+        # the backward runs in chunk-parallel matrix form (csrc/exact_mm.hip): roofline.frac is priced on the flops its
+        # kernels execute, the figure on the token loop's count sits beside it (on_reference_flops)
+        flop_fwd=FLOP_FWD, flop_bwd=FLOP_BWD_MM, flop_ref_fwd=FLOP_FWD, flop_ref_bwd=FLOP_BWD,
+        bytes_fwd=BYTES_FWD, bytes_bwd=BYTES_BWD,
+        # flops per head-token that each instrumented kernel executes
+        kernel_work=dict(FLOP_EXACT_MM, rule_fwd_kernel=FLOP_FWD, rule_bwd_fused_kernel=FLOP_BWD),
+        kernel_names={"forward": "forward_ckpt", "backward": "backward_ckpt_matrix_form"},
         cpu_all=lambda: cpu_all_cores(chain, B, s, heads, "full-trajectory forward + backward"),
         config={"workload": "BASELINE configs[1]: Titans LMM exact recurrence, 8 heads x 64 (d=512), "
                             "batch 8, seq 2048, fp32 state, checkpoints every 64 tokens, fwd+bwd" +
@@ -623,8 +633,8 @@ WORKLOAD_SOURCES = {
     "titans_chunkwise_c3": _CW_BF16,
     "titans_chunkwise_c3_mnorm": _CW_BF16 + ["chunkwise_guard.hip"],
     "titans_chunkwise_c3_f32_mnorm": ["chunkwise_mm.hip", "chunkwise_gates.hip", "chunkwise_guard.hip", "memory_rules.hip"],
-    "titans_exact_c2": ["memory_rules.hip", "memory_rules_fused.hip"],
-    "titans_exact_c2_mnorm": ["memory_rules.hip", "memory_rules_fused.hip"],
+    "titans_exact_c2": ["memory_rules.hip", "exact_mm.hip", "chunkwise_gates.hip"],
+    "titans_exact_c2_mnorm": ["memory_rules.hip", "exact_mm.hip", "chunkwise_gates.hip", "chunkwise_guard.hip"],
     "hope_selfref_c4": ["selfref.hip"],
     "swa_c5": _SWA, "swa_stats_c5": _SWA, "swa_c5_hd32": _SWA, "swa_stats_c5_hd32": _SWA,
     "adamw_c5": ["optim.hip", "cms.hip"],

@@ -251,6 +251,16 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     auto store = [&](int which, Strip &x) {
         for_c(x, [&](int r, int c, float &y) { out[(size_t)which * kDD + (m0 + r) * HD + n0 + c] = y; });
     };
+    // The four scan matrices leave in the order in which the scan's waves take them as the second operand of their
+    // product: lane 16 (k / 16) + n % 16 of the wave for column half n / 32 takes, as its 16-byte piece j = (k % 16) / 2,
+    // the elements (k, n), (k, n + 16), (k + 1, n), (k + 1, n + 16) with k even, n % 32 < 16.  Pieces are stored
+    // [column half][j][lane], so a load instruction of the scan reads 1 KB of consecutive memory.  A lane of this strip
+    // holds two pieces.
+    auto store_operand = [&](int which, const Strip &x) {
+        float *o = out + (size_t)which * kDD + (size_t)(((nh * 8 + 2 * (l >> 4)) * 64 + 16 * ib + (l & 15)) * 4);
+        *reinterpret_cast<float4 *>(o) = make_float4(x.t[0][0], x.t[1][0], x.t[0][1], x.t[1][1]);
+        *reinterpret_cast<float4 *>(o + 64 * 4) = make_float4(x.t[0][2], x.t[1][2], x.t[0][3], x.t[1][3]);
+    };
     auto bZ1 = [&](int kk, int n) { return B8[kk * LDM + n0 + n]; };
     auto bZ2 = [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; };
     auto aWM = [&](int m, int kk) { return cv.wM[kk] * Ks[kk * LDM + m0 + m]; };
@@ -260,7 +270,7 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     {
         Strip x = zero_strip();
         mma(x, aWM, bZ1);
-        store(0, x);
+        store_operand(0, x);
     }
     {
         Strip x = zero_strip();
@@ -272,17 +282,17 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         {
             Strip x = zero_strip();
             mma(x, aWS, bZ1);
-            store(1, x);
+            store_operand(1, x);
         }
         {
             Strip x = zero_strip();
             mma(x, aWM, bZ2);
-            store(2, x);
+            store_operand(2, x);
         }
         {
             Strip x = zero_strip();
             mma(x, aWS, bZ2);
-            store(3, x);
+            store_operand(3, x);
         }
         {
             Strip x = zero_strip();
@@ -298,90 +308,103 @@ constexpr size_t kExLocalLds = 9 * MAT * sizeof(float);
 //   X1' = a_L X1 + X1 Phi_MM + X2 Phi_SM + C_M,   X2' = beta_L X1 + h_L X2 + X1 Phi_MS + X2 Phi_SS + C_S
 // ends [chain][nc + 1][64*64]: slot c = adjoint of the state at the start of chunk c (slot nc = 0, slot 0 = the
 // gradient of the initial state, also written to first [chain][64*64]).
-// Wave w: destination w / 4, source (w / 2) % 2, column half w % 2; the two sources of a destination meet in LDS.
+// Wave w: destination w / 4, source (w / 2) % 2, column half w % 2: one 16 x 64 x 32 product per step.  The two
+// source waves of a destination strip then finish one 16 x 16 tile of it each (they swap the other tile through
+// LDS), so every wave runs the same instructions: per step 12 loads, then 4 stores.  That matters: the memory
+// counter of this hardware counts loads and stores together and in order, and the wait for the next step's operands
+// at the top of a step can only leave this step's stores in flight if their number is the same on every path
+// (with the stores under a branch the wait was for all of them: 4 of a step's 9 thousand cycles).
+// Without momentum (the Delta rule) there is one state and one matrix: the two source waves split its contraction.
+template <bool HAS_S>
 __global__ __launch_bounds__(kThr) void ex_scan_kernel(const float *__restrict__ loc, const float *__restrict__ locs,
                                                        float *__restrict__ em, float *__restrict__ es_,
-                                                       float *__restrict__ first_m, float *__restrict__ first_s, int nc,
-                                                       int has_s) {
-    extern __shared__ float smem[];
-    float *F = smem;                       // four 64x64 matrices
-    float *X1 = F + 4 * MAT, *X2 = X1 + 16 * LDM, *part = X2 + 16 * LDM;   // part [4][16*33]
+                                                       float *__restrict__ first_m, float *__restrict__ first_s, int nc) {
+    __shared__ float X1[16 * LDM], X2[16 * LDM], part[8 * 256];
     // the four row blocks of a chain sit 8 workgroups apart: consecutive workgroups go to consecutive XCDs, so the
     // four share one XCD's L2 for the chunk matrices they all read
     const int chain0 = (blockIdx.x & 7) + 8 * (blockIdx.x >> 5), rb0 = (blockIdx.x >> 3) & 3;
     const bool whole = (int)(blockIdx.x | 31) < (int)gridDim.x;   // a full group of 32 workgroups
     const int chain = whole ? chain0 : blockIdx.x >> 2, r0 = 16 * (whole ? rb0 : blockIdx.x & 3);
-    const int w = threadIdx.x >> 6, dst = w >> 2, src = (w >> 1) & 1, n0 = 32 * (w & 1), pidx = dst * 2 + (w & 1);
-    float *emp = em + (size_t)chain * (nc + 1) * kDD, *esp = has_s ? es_ + (size_t)chain * (nc + 1) * kDD : nullptr;
+    const int l = threadIdx.x & 63, w = threadIdx.x >> 6, dst = w >> 2, src = (w >> 1) & 1, half = w & 1;
+    const int col = 32 * half + 16 * src + (l & 15), rw = 4 * (l >> 4);   // the tile this wave finishes: rows rw + i
+    float *emp = em + (size_t)chain * (nc + 1) * kDD, *esp = HAS_S ? es_ + (size_t)chain * (nc + 1) * kDD : nullptr;
     for (int e = threadIdx.x; e < 16 * 64; e += kThr) {
         const int rr = e >> 6, cc = e & 63;
         X1[rr * LDM + cc] = 0.f;
         X2[rr * LDM + cc] = 0.f;
         emp[(size_t)nc * kDD + (r0 + rr) * HD + cc] = 0.f;
-        if (esp) esp[(size_t)nc * kDD + (r0 + rr) * HD + cc] = 0.f;
+        if (HAS_S) esp[(size_t)nc * kDD + (r0 + rr) * HD + cc] = 0.f;
     }
-    Tile<float> tf[4];
-    Strip cnext = zero_strip(), cadd;
-    float aLn = 0.f, bLn = 0.f, hLn = 0.f, aL, bL, hL;
-    const bool live = has_s || (dst == 0 && src == 0);   // the Delta rule has one state and one matrix
+    const bool active = HAS_S || dst == 0;   // wave-uniform; the idle waves of the Delta rule only keep the barriers
+    constexpr int NB = HAS_S ? 8 : 4;   // 16-byte pieces of the operand per lane and step
+    // The wave's second operand (a 64 x 32 piece of one chunk matrix) comes straight from memory in the lane order
+    // of the product (ex_local_kernel writes it that way), requested a step ahead.
+    float4 bn[NB], bc[NB];
+    f32x4 cn = {0.f, 0.f, 0.f, 0.f}, out = {0.f, 0.f, 0.f, 0.f};
+    float scn = 0.f;   // lanes 4 j + 0, 1, 2: a_L, beta_L, h_L of the next step
     auto prefetch = [&](int ci) {
         const float *lc = loc + ((size_t)chain * nc + ci) * kExLocMats * kDD;
         const float *sc = locs + ((size_t)chain * nc + ci) * 4;
-        fetch(tf[0], lc, 64);
-        if (has_s) {
-            fetch(tf[1], lc + kDD, 64);
-            fetch(tf[2], lc + 2 * kDD, 64);
-            fetch(tf[3], lc + 3 * kDD, 64);
-        }
-        aLn = sc[0]; bLn = sc[1]; hLn = sc[2];
-        if (src == 0 && live) {
-            const float *Cm = lc + (4 + dst) * kDD;
-            for_c(cnext, [&](int r, int c, float &x) { x = Cm[(r0 + r) * HD + n0 + c]; });
-        }
-    };
-    prefetch(nc - 1);
-    for (int ci = nc - 1; ci >= 0; ci--) {
-        __syncthreads();   // the previous step's readers of F and writers of X1 / X2 are done
-        commit(F, tf[0]);
-        if (has_s) {
-            commit(F + MAT, tf[1]);
-            commit(F + 2 * MAT, tf[2]);
-            commit(F + 3 * MAT, tf[3]);
-        }
-        aL = aLn; bL = bLn; hL = hLn; cadd = cnext;
-        __syncthreads();
-        if (ci > 0) prefetch(ci - 1);
-        Strip acc = zero_strip(), out = zero_strip();
-        if (live) {
-            const float *Xs = src ? X2 : X1;
-            const float *Fm = F + (dst * 2 + src) * MAT;
-            mma(acc, [&](int m, int kk) { return Xs[m * LDM + kk]; }, [&](int kk, int n) { return Fm[kk * LDM + n0 + n]; });
-            if (src) {
-                for_c(acc, [&](int r, int c, float &x) { part[pidx * 16 * 33 + r * 33 + c] = x; });
-            } else {
-                for_c(out, [&](int r, int c, float &x) {
-                    const float x1 = X1[r * LDM + n0 + c];
-                    x = dst ? bL * x1 + hL * X2[r * LDM + n0 + c] : aL * x1;
-                });
+        const float4 *bp = reinterpret_cast<const float4 *>(lc + (size_t)(HAS_S ? dst * 2 + src : 0) * kDD) +
+                           (half * 8 + (HAS_S ? 0 : 4 * src)) * 64 + l;
 #pragma unroll
-                for (int i = 0; i < 4; i++) { out.t[0][i] += acc.t[0][i] + cadd.t[0][i]; out.t[1][i] += acc.t[1][i] + cadd.t[1][i]; }
+        for (int j = 0; j < NB; j++) bn[j] = bp[j * 64];
+        // a vector load (lane-dependent address) on purpose: a scalar load would join the LDS reads under one counter
+        // that only knows "all done", and the first product of the step would wait for it to come back from memory
+        scn = sc[l & 3];
+        const float *Cm = lc + (4 + dst) * kDD + (r0 + rw) * HD + col;
+#pragma unroll
+        for (int i = 0; i < 4; i++) cn[i] = Cm[i * HD];
+    };
+    if (active) prefetch(nc - 1);
+    __syncthreads();
+    float *Xd = dst ? X2 : X1;
+    float *gd = (dst ? esp : emp) + (size_t)(r0 + rw) * HD + col;
+    const float *Xs = ((HAS_S && src) ? X2 : X1) + (l & 15) * LDM + 16 * (l >> 4) + (HAS_S ? 0 : 8 * src);
+    for (int ci = nc - 1; ci >= 0; ci--) {
+        if (active) {
+#pragma unroll
+            for (int j = 0; j < NB; j++) bc[j] = bn[j];
+            const float aL = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, scn), 0)),
+                        bL = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, scn), 1)),
+                        hL = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, scn), 2));
+            const f32x4 ca = cn;
+            if (ci > 0) prefetch(ci - 1);
+            f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int j = 0; j < NB; j++) {   // contraction indices 16 (l / 16) + 2 j, + 1 (+ 8 for the second Delta wave)
+                const float a0 = Xs[2 * j], a1 = Xs[2 * j + 1];
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, bc[j].x, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, bc[j].y, acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, bc[j].z, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, bc[j].w, acc[1], 0, 0, 0);
+            }
+            // the tile the partner wave (w ^ 2) finishes goes to LDS; this wave keeps tile `src`
+            const f32x4 mine = src ? acc[1] : acc[0], theirs = src ? acc[0] : acc[1];
+#pragma unroll
+            for (int i = 0; i < 4; i++) part[w * 256 + i * 64 + l] = theirs[i];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float x1 = X1[(rw + i) * LDM + col];
+                out[i] = mine[i] + ca[i] + (dst ? bL * x1 + hL * X2[(rw + i) * LDM + col] : aL * x1);
             }
         }
-        __syncthreads();   // every read of the old X1 / X2 is done; the partial products are in LDS
-        if (live && !src) {
-            float *Xd = dst ? X2 : X1;
-            float *gd = dst ? esp : emp;
-            float *gf = (ci == 0) ? (dst ? first_s : first_m) : nullptr;
-            for_c(out, [&](int r, int c, float &x) {
-                if (has_s) x += part[pidx * 16 * 33 + r * 33 + c];
-                Xd[r * LDM + n0 + c] = x;
-                gd[(size_t)ci * kDD + (r0 + r) * HD + n0 + c] = x;
-                if (gf) gf[(size_t)chain * kDD + (r0 + r) * HD + n0 + c] = x;
-            });
+        __syncthreads();   // every read of the old X1 / X2 is done; the partners' tiles are in LDS
+        if (active) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                out[i] += part[(w ^ 2) * 256 + i * 64 + l];
+                Xd[(rw + i) * LDM + col] = out[i];
+                gd[(size_t)ci * kDD + i * HD] = out[i];
+            }
         }
+        __syncthreads();   // the new X1 / X2 are complete
     }
+    if (!active) return;
+    float *gf = (dst ? first_s : first_m) + (size_t)chain * kDD + (size_t)(r0 + rw) * HD + col;
+#pragma unroll
+    for (int i = 0; i < 4; i++) gf[i * HD] = out[i];
 }
-constexpr size_t kExScanLds = (4 * MAT + 2 * 16 * LDM + 4 * 16 * 33) * sizeof(float);
 
 // ── pass 3: gradients of one chunk ──────────────────────────────────────────
 //   pvec [chain][token][4] = <M0, J_t>, <S0, J_t>, -theta_t u_t^T dMo k_t, -theta_t u_t^T dSo k_t
@@ -644,7 +667,6 @@ bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *
     if (!attr_set) {
         set_lds(ex_local_kernel<false>, kExLocalLds);
         set_lds(ex_local_kernel<true>, kExLocalLds);
-        set_lds(ex_scan_kernel, kExScanLds);
         set_lds(ex_grads_kernel, kExGradsLds);
         attr_set = true;
     }
@@ -661,8 +683,12 @@ bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *
     }
     {
         KernelTimer kt("ex_scan_kernel");
-        hipLaunchKernelGGL(ex_scan_kernel, dim3((unsigned)batch * 4), dim3(kThr), kExScanLds, stream(), loc, locs, em, esn,
-                           first_m, first_s, nc, (int)has_s);
+        if (has_s)
+            hipLaunchKernelGGL(ex_scan_kernel<true>, dim3((unsigned)batch * 4), dim3(kThr), 0, stream(), loc, locs, em, esn,
+                               first_m, first_s, nc);
+        else
+            hipLaunchKernelGGL(ex_scan_kernel<false>, dim3((unsigned)batch * 4), dim3(kThr), 0, stream(), loc, locs, em, esn,
+                               first_m, first_s, nc);
         check_launch("ex_scan_kernel");
     }
     {
