@@ -136,14 +136,16 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
     // scalars) are fetched into registers while step runs, so a step costs no HBM round trip.
     Tile<float> ta, tb;
     Strip cnext = zero_strip(), cadd;
-    float s1n = 0.f, s2n = 0.f, s1, s2;
+    float scn = 0.f, s1, s2;   // lanes 4 j + 1, 2 of scn: the two scalars of the next step
     auto prefetch = [&](int step) {
         const int ci = FWD ? step : nc - 1 - step;
         const float *lc = loc + ((size_t)chain * nc + ci) * kLocMats * HD * HD;
         const float *sc = locs + ((size_t)chain * nc + ci) * 4;
         fetch(ta, lc, 64);
         fetch(tb, lc + HD * HD, 64);
-        s1n = sc[1]; s2n = sc[2];
+        // a vector load (lane-dependent address) on purpose: a scalar load would share a counter with the LDS reads of
+        // the step's product, which would then wait for it to come back from memory
+        scn = sc[threadIdx.x & 3];
         const float *Cm = lc + (FWD ? 2 + which : (which ? 3 : 2)) * HD * HD;
         for_c(cnext, [&](int r, int c, float &x) { x = Cm[(r0 + m0 + r) * HD + n0 + c]; });
     };
@@ -153,7 +155,9 @@ __global__ __launch_bounds__(kThr) void cw_scan_kernel(const float *__restrict__
         __syncthreads();  // previous step's readers of Ta/Tb and writers of X1/X2 are done
         commit(Ta, ta);
         commit(Tb, tb);
-        s1 = s1n; s2 = s2n; cadd = cnext;
+        s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, scn), 1));
+        s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, scn), 2));
+        cadd = cnext;
         __syncthreads();
         if (step + 1 < nc) prefetch(step + 1);
         Strip acc = zero_strip(), out = zero_strip();
