@@ -50,9 +50,12 @@ using namespace mmt;
 
 // Waves w and w + 4 share a SIMD.  Products with the lower triangular T (or its transpose) cost a 16-row block
 // ib + 1 (or 4 - ib) quarter products, so the row blocks are dealt out as (0, 3) and (1, 2) per SIMD.
-#define NLH_STRIP_ORIGIN() \
-    const int w = threadIdx.x >> 6, ib = w < 4 ? w >> 1 : 3 - ((w - 4) >> 1), m0 = 16 * ib, n0 = 32 * (w & 1), nh = w & 1; \
+#define NLH_STRIP_ORIGIN_OF(w) \
+    const int ib = w < 4 ? w >> 1 : 3 - ((w - 4) >> 1), m0 = 16 * ib, n0 = 32 * (w & 1), nh = w & 1; \
     (void)nh
+#define NLH_STRIP_ORIGIN() \
+    const int w = threadIdx.x >> 6; \
+    NLH_STRIP_ORIGIN_OF(w)
 
 // per chunk, for the scan: Phi_MM, Phi_SM, Phi_MS, Phi_SS (source state, destination state), C_M, C_S
 constexpr size_t kExLocMats = 6;
@@ -85,34 +88,54 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     const float *__restrict__ alpha, const float *__restrict__ theta, const float *__restrict__ eta,
     const float *__restrict__ m_ckpt, const float *__restrict__ s_ckpt, float *__restrict__ loc, float *__restrict__ locs,
     float *__restrict__ Tg, float *__restrict__ Ug, float *__restrict__ dUg, int s, int C, int nc, int nck, int has_s,
-    ChainTracks tr) {
+    int ntask, ChainTracks tr) {
     extern __shared__ float smem[];
     float *Ks = smem, *Vs = Ks + MAT, *Qs = Vs + MAT, *Ds = Qs + MAT, *Ms = Ds + MAT, *Ss = Ms + MAT, *Cc = Ss + MAT,
           *B8 = Cc + MAT, *B9 = B8 + MAT;
     __shared__ Coef cf;
     __shared__ ChunkVecs cv;
-    NLH_STRIP_ORIGIN();
-    const int l = threadIdx.x & 63;
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0, task = (size_t)chain * nc + ci;
+    // Persistent over a contiguous range of chunks.  A workgroup fills the compute unit's LDS, so nothing else would
+    // hide its loads: the next chunk's tiles are requested at the start of this chunk's last phase (the longest one,
+    // ten products back to back) and land in LDS at the top of the next round.
+    Tile<float> tk, tv, tq, td, tm, ts;
+    Gates gt;
+    auto fetch_task = [&](int task, int tid) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        fetch(tk, k + tok * HD, L, tid);
+        fetch(tv, v + tok * HD, L, tid);
+        fetch(tq, q + tok * HD, L, tid);
+        fetch(td, d_y + tok * HD, L, tid);
+        fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64, tid);
+        if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64, tid);
+    };
+    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per, task_hi = min(ntask, task_lo + per);
+    if (task_lo < task_hi) fetch_task(task_lo, threadIdx.x);
+    for (int itask = task_lo; itask < task_hi; itask++) {
+    // thread and wave index through opaque copies, once per chunk (see mm_tiles.h)
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int l = tid & 63;
+    int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    asm volatile("" : "+s"(w));
+    NLH_STRIP_ORIGIN_OF(w);
+    auto MMA = [&](Strip &acc, auto fa, auto fb) { mma(acc, fa, fb, l); };
+    auto MMAR = [&](Strip &acc, auto fa, auto fb, int p0, int p1) { mma_range(acc, fa, fb, p0, p1, l); };
+    auto MMAT = [&](f32x4 &acc, auto fa, auto fb, int k0) { mma_tile16(acc, fa, fb, k0, l); };
+    auto FORC = [&](Strip &acc, auto f) { for_c(acc, f, l); };
+    const int chain = itask / nc, ci = itask % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t task = (size_t)itask;
+    (void)t0;
     {
-        // the gates first: the coefficient loops wait for them only and run while the tiles are in flight
-        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
-        Tile<float> tk, tv, tq, td, tm, ts;
-        fetch(tk, k + tok * HD, L);
-        fetch(tv, v + tok * HD, L);
-        fetch(tq, q + tok * HD, L);
-        fetch(td, d_y + tok * HD, L);
-        fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
-        if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
         load_gates(cf, gt);
         coefficients(cf, gt, L, Cc, nullptr, nullptr);
-        commit(Ks, tk);
-        commit(Vs, tv);
-        commit(Qs, tq);
-        commit(Ds, td);
-        commit(Ms, tm);
-        if (has_s) commit(Ss, ts);
+        commit(Ks, tk, tid);
+        commit(Vs, tv, tid);
+        commit(Qs, tq, tid);
+        commit(Ds, td, tid);
+        commit(Ms, tm, tid);
+        if (has_s) commit(Ss, ts, tid);
         if (TRACK) {
             float msq = wave_allreduce(tile_dot(tm, tm)), ssq = has_s ? wave_allreduce(tile_dot(ts, ts)) : 0.f;
             if (l == 0) *reinterpret_cast<float2 *>(tr.nrm + (task * 8 + w) * 2) = make_float2(msq, ssq);
@@ -127,16 +150,16 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     {
         Strip g = zero_strip(), km = zero_strip(), ks = zero_strip(), p = zero_strip();
         auto aK = [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; };
-        mma(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-        mma(km, aK, [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
-        if (has_s) mma(ks, aK, [&](int kk, int n) { return Ss[(n0 + n) * LDM + kk]; });
-        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        MMA(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+        MMA(km, aK, [&](int kk, int n) { return Ms[(n0 + n) * LDM + kk]; });
+        if (has_s) MMA(ks, aK, [&](int kk, int n) { return Ss[(n0 + n) * LDM + kk]; });
+        MMA(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
         __syncthreads();   // the vectors are there
 #pragma unroll
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
                 // R in place over V (own strip)
                 float *d = Vs + row * LDM + col;
                 *d = cv.am[row] * km.t[tl][i] + cv.bm[row] * ks.t[tl][i] - *d;
@@ -147,7 +170,7 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
     }
     __syncthreads();
     Strip dul = zero_strip();
-    mma(dul, [&](int m, int kk) { return B9[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
+    MMA(dul, [&](int m, int kk) { return B9[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Ds[kk * LDM + n0 + n]; });
     if (w < 4 && l < 16) {
         // D_b = (I - Lam_bb)^-1 by substitution: lane c holds column c of block b = w
         const float *A = B8 + (16 * w) * LDM + 16 * w;
@@ -170,13 +193,13 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
             const int jb = 2 * (w & 1) + tl;
             f32x4 nacc = {0.f, 0.f, 0.f, 0.f};
             if (jb < ib)
-                mma_tile16(nacc, [&](int m, int kk) { return Ms[(m0 + m) * LDM + kk]; },
+                MMAT(nacc, [&](int m, int kk) { return Ms[(m0 + m) * LDM + kk]; },
                            [&](int kk, int n) { return B8[kk * LDM + 16 * jb + n]; }, 16 * ib);
 #pragma unroll
-            for (int i = 0; i < 4; i++) Ss[(m0 + row_of(i)) * LDM + 16 * jb + (l & 15)] = nacc[i];
+            for (int i = 0; i < 4; i++) Ss[(m0 + row_of(i, l)) * LDM + 16 * jb + (l & 15)] = nacc[i];
         }
         float *go = dUg + task * kDD;
-        for_c(dul, [&](int r, int c, float &x) {
+        FORC(dul, [&](int r, int c, float &x) {
             B9[(m0 + r) * LDM + n0 + c] = x;
             go[(m0 + r) * HD + n0 + c] = x;
         });
@@ -189,9 +212,9 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         const int jb = 2 * (w & 1) + tl;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int kb = jb + 1; kb < ib; kb++)
-            mma_tile16(acc, aN, [&](int kk, int n) { return Ss[kk * LDM + 16 * jb + n]; }, 16 * kb);
+            MMAT(acc, aN, [&](int kk, int n) { return Ss[kk * LDM + 16 * jb + n]; }, 16 * kb);
 #pragma unroll
-        for (int i = 0; i < 4; i++) B8[(m0 + row_of(i)) * LDM + 16 * jb + (l & 15)] = acc[i];
+        for (int i = 0; i < 4; i++) B8[(m0 + row_of(i, l)) * LDM + 16 * jb + (l & 15)] = acc[i];
     }
     __syncthreads();
 #pragma unroll
@@ -199,10 +222,10 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         const int jb = 2 * (w & 1) + tl;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int kb = jb + 2; kb < ib; kb++)
-            mma_tile16(acc, aN, [&](int kk, int n) { return B8[kk * LDM + 16 * jb + n]; }, 16 * kb);
+            MMAT(acc, aN, [&](int kk, int n) { return B8[kk * LDM + 16 * jb + n]; }, 16 * kb);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int row = m0 + row_of(i), col = 16 * jb + (l & 15);
+            const int row = m0 + row_of(i, l), col = 16 * jb + (l & 15);
             Cc[row * LDM + col] = acc[i] + Ss[row * LDM + col] + B8[row * LDM + col] + (row == col ? 1.f : 0.f);
         }
     }
@@ -213,11 +236,11 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         for (int tl = 0; tl < 2; tl++) {
             const int jb = 2 * (w & 1) + tl;
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
-            mma_tile16(t, [&](int m, int kk) { return Cc[(m0 + m) * LDM + kk]; },
+            MMAT(t, [&](int m, int kk) { return Cc[(m0 + m) * LDM + kk]; },
                        [&](int kk, int n) { return Ms[kk * LDM + 16 * jb + n]; }, 16 * jb);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = 16 * jb + (l & 15);
+                const int row = m0 + row_of(i, l), col = 16 * jb + (l & 15);
                 Ss[row * LDM + col] = t[i];
                 go[row * HD + col] = t[i];
             }
@@ -229,27 +252,28 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         auto aT = [&](int m, int kk) { return Ss[(m0 + m) * LDM + kk]; };
         // T is lower triangular: row block ib contracts over the first ib + 1 blocks of 16 (taken in pairs)
         const int pe = (ib >> 1) + 1;
-        mma_range(u, aT, [&](int kk, int n) { return Vs[kk * LDM + n0 + n]; }, 0, pe);
-        mma_range(z1, aT, [&](int kk, int n) { return cv.am[kk] * Ks[kk * LDM + n0 + n]; }, 0, pe);
-        if (has_s) mma_range(z2, aT, [&](int kk, int n) { return cv.bm[kk] * Ks[kk * LDM + n0 + n]; }, 0, pe);
+        MMAR(u, aT, [&](int kk, int n) { return Vs[kk * LDM + n0 + n]; }, 0, pe);
+        MMAR(z1, aT, [&](int kk, int n) { return cv.am[kk] * Ks[kk * LDM + n0 + n]; }, 0, pe);
+        if (has_s) MMAR(z2, aT, [&](int kk, int n) { return cv.bm[kk] * Ks[kk * LDM + n0 + n]; }, 0, pe);
         float *go = Ug + task * kDD;
-        for_c(u, [&](int r, int c, float &x) { go[(m0 + r) * HD + n0 + c] = x; });
-        for_c(z1, [&](int r, int c, float &x) { B8[(m0 + r) * LDM + n0 + c] = x; });
-        if (has_s) for_c(z2, [&](int r, int c, float &x) { Ms[(m0 + r) * LDM + n0 + c] = x; });
+        FORC(u, [&](int r, int c, float &x) { go[(m0 + r) * HD + n0 + c] = x; });
+        FORC(z1, [&](int r, int c, float &x) { B8[(m0 + r) * LDM + n0 + c] = x; });
+        if (has_s) FORC(z2, [&](int r, int c, float &x) { Ms[(m0 + r) * LDM + n0 + c] = x; });
         if (TRACK) {   // squared error norm of the strip's 16 tokens over its 32 memory rows
-            for_c(u, [&](int, int, float &x) { x *= x; });
+            FORC(u, [&](int, int, float &x) { x *= x; });
             strip_row_sums(u);
-            if (row_writer()) {
+            if (row_writer(l)) {
                 float *eo = tr.e2 + (((size_t)chain * 2 + nh) * nc + ci) * CW + m0;
 #pragma unroll
-                for (int i = 0; i < 4; i++) eo[row_of(i)] = u.t[0][i];
+                for (int i = 0; i < 4; i++) eo[row_of(i, l)] = u.t[0][i];
             }
         }
     }
     __syncthreads();
+    if (itask + 1 < task_hi) fetch_task(itask + 1, tid);
     float *out = loc + task * kExLocMats * kDD;
     auto store = [&](int which, Strip &x) {
-        for_c(x, [&](int r, int c, float &y) { out[(size_t)which * kDD + (m0 + r) * HD + n0 + c] = y; });
+        FORC(x, [&](int r, int c, float &y) { out[(size_t)which * kDD + (m0 + r) * HD + n0 + c] = y; });
     };
     // The four scan matrices leave in the order in which the scan's waves take them as the second operand of their
     // product: lane 16 (k / 16) + n % 16 of the wave for column half n / 32 takes, as its 16-byte piece j = (k % 16) / 2,
@@ -261,45 +285,23 @@ __global__ __launch_bounds__(kThr) void ex_local_kernel(
         *reinterpret_cast<float4 *>(o) = make_float4(x.t[0][0], x.t[1][0], x.t[0][1], x.t[1][1]);
         *reinterpret_cast<float4 *>(o + 64 * 4) = make_float4(x.t[0][2], x.t[1][2], x.t[0][3], x.t[1][3]);
     };
-    auto bZ1 = [&](int kk, int n) { return B8[kk * LDM + n0 + n]; };
-    auto bZ2 = [&](int kk, int n) { return Ms[kk * LDM + n0 + n]; };
-    auto aWM = [&](int m, int kk) { return cv.wM[kk] * Ks[kk * LDM + m0 + m]; };
-    auto aWS = [&](int m, int kk) { return cv.wS[kk] * Ks[kk * LDM + m0 + m]; };
-    auto bQ = [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; };
-    auto aDU = [&](int m, int kk) { return B9[kk * LDM + m0 + m]; };
-    {
+    // one product at a time (no unrolling over the outputs): the next chunk's tiles are in registers during this phase
+#pragma unroll 1
+    for (int o = 0; o < (has_s ? 4 : 1); o++) {   // Phi_MM, Phi_SM, Phi_MS, Phi_SS = (w.K)^T Z
+        const float *wv = (o & 1) ? cv.wS : cv.wM, *Z = (o & 2) ? Ms : B8;
         Strip x = zero_strip();
-        mma(x, aWM, bZ1);
-        store_operand(0, x);
+        MMA(x, [&](int m, int kk) { return wv[kk] * Ks[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Z[kk * LDM + n0 + n]; });
+        store_operand(o, x);
     }
-    {
+#pragma unroll 1
+    for (int o = 0; o < (has_s ? 2 : 1); o++) {   // C_M = (a.dY)^T Q + dU_loc^T Z1,  C_S = (beta.dY)^T Q + dU_loc^T Z2
+        const float *vec = o ? cf.beta : cf.a, *Z = o ? Ms : B8;
         Strip x = zero_strip();
-        mma(x, [&](int m, int kk) { return cf.a[kk] * Ds[kk * LDM + m0 + m]; }, bQ);
-        mma(x, aDU, bZ1);
-        store(4, x);
+        MMA(x, [&](int m, int kk) { return vec[kk] * Ds[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+        MMA(x, [&](int m, int kk) { return B9[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Z[kk * LDM + n0 + n]; });
+        store(4 + o, x);
     }
-    if (has_s) {
-        {
-            Strip x = zero_strip();
-            mma(x, aWS, bZ1);
-            store_operand(1, x);
-        }
-        {
-            Strip x = zero_strip();
-            mma(x, aWM, bZ2);
-            store_operand(2, x);
-        }
-        {
-            Strip x = zero_strip();
-            mma(x, aWS, bZ2);
-            store_operand(3, x);
-        }
-        {
-            Strip x = zero_strip();
-            mma(x, [&](int m, int kk) { return cf.beta[kk] * Ds[kk * LDM + m0 + m]; }, bQ);
-            mma(x, aDU, bZ2);
-            store(5, x);
-        }
+    __syncthreads();   // LDS is rewritten by the next chunk
     }
 }
 constexpr size_t kExLocalLds = 9 * MAT * sizeof(float);
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
     const float *__restrict__ s_ckpt, const float *__restrict__ Tg, const float *__restrict__ Ug,
     const float *__restrict__ dUg, const float *__restrict__ em, const float *__restrict__ es_, float *__restrict__ d_k,
     float *__restrict__ d_v, float *__restrict__ d_q, float *__restrict__ d_theta, float *__restrict__ pvec,
-    float *__restrict__ xs, float *__restrict__ scal, int s, int C, int nc, int nck, int has_s) {
+    float *__restrict__ xs, float *__restrict__ scal, int s, int C, int nc, int nck, int has_s, int ntask) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Ts = Ds + MAT, *Us = Ts + MAT, *A1 = Us + MAT, *A2 = A1 + MAT,
           *Cc = A2 + MAT, *B9 = Cc + MAT;
@@ -424,86 +426,108 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
     __shared__ float part[6][2][CW];   // row sums per column half: p0, ps, g1, g2, dam, dbm
     __shared__ float part_th[4][CW];   // column sums of dW.c per 16-row block
     __shared__ float dots[3][8];
-    NLH_STRIP_ORIGIN();
-    const int l = threadIdx.x & 63;
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc, t0 = ci * C, L = min(C, s - t0);
-    const size_t tok = (size_t)chain * s + t0, task = (size_t)chain * nc + ci;
-    const size_t end = ((size_t)chain * (nc + 1) + ci + 1) * kDD;
-    Tile<float> tm, ts;
+    // Persistent over a contiguous range of chunks, as ex_local_kernel: the next chunk's nine tiles are requested at the
+    // start of this chunk's last phase.
+    Tile<float> tk, tq, td, tt, tu, tdm, tds, tm, ts;
+    Gates gt;
+    // K, Q, dY of the next chunk are requested during this chunk's last phase (more does not fit next to its
+    // accumulators); the other six tiles at the top of the chunk, behind two products that need K and Q only
+    auto fetch_a = [&](int task, int tid) {
+        const int chain = task / nc, ci = task % nc, t0 = ci * C, L = min(C, s - t0);
+        const size_t tok = (size_t)chain * s + t0;
+        gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);
+        fetch(tk, k + tok * HD, L, tid);
+        fetch(tq, q + tok * HD, L, tid);
+        fetch(td, d_y + tok * HD, L, tid);
+    };
+    auto fetch_b = [&](int task, int tid) {
+        const int chain = task / nc, ci = task % nc;
+        const size_t end = ((size_t)chain * (nc + 1) + ci + 1) * kDD;
+        fetch(tt, Tg + (size_t)task * kDD, 64, tid);
+        fetch(tu, Ug + (size_t)task * kDD, 64, tid);
+        fetch(tdm, em + end, 64, tid);
+        if (has_s) fetch(tds, es_ + end, 64, tid);
+        fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64, tid);
+        if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64, tid);
+    };
+    const int per = (ntask + (int)gridDim.x - 1) / (int)gridDim.x, task_lo = blockIdx.x * per, task_hi = min(ntask, task_lo + per);
+    if (task_lo < task_hi) fetch_a(task_lo, threadIdx.x);
+    for (int itask = task_lo; itask < task_hi; itask++) {
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int l = tid & 63;
+    int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    asm volatile("" : "+s"(w));
+    NLH_STRIP_ORIGIN_OF(w);
+    auto MMA = [&](Strip &acc, auto fa, auto fb) { mma(acc, fa, fb, l); };
+    auto MMAR = [&](Strip &acc, auto fa, auto fb, int p0, int p1) { mma_range(acc, fa, fb, p0, p1, l); };
+    auto FORC = [&](Strip &acc, auto f) { for_c(acc, f, l); };
+    const int chain = itask / nc, ci = itask % nc, t0 = ci * C, L = min(C, s - t0);
+    const size_t tok = (size_t)chain * s + t0, task = (size_t)itask;
+    fetch_b(itask, tid);
+    load_gates(cf, gt);
+    coefficients(cf, gt, L, Cc, nullptr, nullptr);
+    commit(Ks, tk, tid);
+    commit(Qs, tq, tid);
+    commit(Ds, td, tid);
+    __syncthreads();
+    chunk_vectors(cv, cf, L);
+    auto aK = [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; };
+    Strip p = zero_strip(), g = zero_strip();   // Q K^T and K K^T while the other tiles are in flight
+    MMA(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
+    MMA(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
     {
-        const Gates gt = fetch_gates(alpha + tok, theta + tok, eta + tok, L, has_s != 0);   // first: see ex_local_kernel
-        Tile<float> tk, tq, td, tt, tu, tdm, tds;
-        fetch(tk, k + tok * HD, L);
-        fetch(tq, q + tok * HD, L);
-        fetch(td, d_y + tok * HD, L);
-        fetch(tt, Tg + task * kDD, 64);
-        fetch(tu, Ug + task * kDD, 64);
-        fetch(tdm, em + end, 64);
-        if (has_s) fetch(tds, es_ + end, 64);
-        fetch(tm, m_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
-        if (has_s) fetch(ts, s_ckpt + ((size_t)chain * nck + ci) * kDD, 64);
-        load_gates(cf, gt);
-        coefficients(cf, gt, L, Cc, nullptr, nullptr);
-        commit(Ks, tk);
-        commit(Qs, tq);
-        commit(Ds, td);
-        commit(Ts, tt);
-        commit(Us, tu);
-        commit(A1, tdm);
-        if (has_s) commit(A2, tds);
+        commit(Ts, tt, tid);
+        commit(Us, tu, tid);
+        commit(A1, tdm, tid);
+        if (has_s) commit(A2, tds, tid);
         const float x0 = wave_allreduce(tile_dot(tm, tdm));
         const float x1 = has_s ? wave_allreduce(tile_dot(ts, tdm)) : 0.f;
         const float x2 = has_s ? wave_allreduce(tile_dot(ts, tds)) : 0.f;
         if (l == 0) { dots[0][w] = x0; dots[1][w] = x1; dots[2][w] = x2; }
     }
     __syncthreads();
-    chunk_vectors(cv, cf, L);
-    if (threadIdx.x < 3) {
-        const float *p = dots[threadIdx.x];
-        scal[task * 4 + threadIdx.x] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+    if (tid < 3) {
+        const float *pp = dots[tid];
+        scal[task * 4 + tid] = ((pp[0] + pp[1]) + (pp[2] + pp[3])) + ((pp[4] + pp[5]) + (pp[6] + pp[7]));
     }
     auto publish = [&](int which, Strip &x) {   // row sums of x -> part[which][column half][row]
         strip_row_sums(x);
-        if (row_writer()) {
+        if (row_writer(l)) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) part[which][nh][m0 + row_of(i)] = x.t[0][i];
+            for (int i = 0; i < 4; i++) part[which][nh][m0 + row_of(i, l)] = x.t[0][i];
         }
     };
-    auto aK = [&](int m, int kk) { return Ks[(m0 + m) * LDM + kk]; };
     auto aU = [&](int m, int kk) { return Us[(m0 + m) * LDM + kk]; };
     Strip udm = zero_strip(), uds = zero_strip();
     {
         Strip kdm = zero_strip(), kds = zero_strip();
-        mma(kdm, aK, [&](int kk, int n) { return A1[(n0 + n) * LDM + kk]; });
-        mma(udm, aU, [&](int kk, int n) { return A1[kk * LDM + n0 + n]; });
+        MMA(kdm, aK, [&](int kk, int n) { return A1[(n0 + n) * LDM + kk]; });
+        MMA(udm, aU, [&](int kk, int n) { return A1[kk * LDM + n0 + n]; });
         if (has_s) {
-            mma(kds, aK, [&](int kk, int n) { return A2[(n0 + n) * LDM + kk]; });
-            mma(uds, aU, [&](int kk, int n) { return A2[kk * LDM + n0 + n]; });
+            MMA(kds, aK, [&](int kk, int n) { return A2[(n0 + n) * LDM + kk]; });
+            MMA(uds, aU, [&](int kk, int n) { return A2[kk * LDM + n0 + n]; });
         }
-        __syncthreads();   // the vectors are there
         const float *gi = dUg + task * kDD;
 #pragma unroll
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
                 B9[row * LDM + col] = gi[row * HD + col] + cv.wM[row] * kdm.t[tl][i] + cv.wS[row] * kds.t[tl][i];   // dU
             }
     }
     __syncthreads();   // dU complete; dMo, dSo no longer needed
-    Strip p = zero_strip(), g = zero_strip();
     {
         Strip dr = zero_strip();
         // T^T is upper triangular: row block ib contracts over the blocks ib .. 3 of 16 (taken in pairs)
-        mma_range(dr, [&](int m, int kk) { return Ts[kk * LDM + m0 + m]; }, [&](int kk, int n) { return B9[kk * LDM + n0 + n]; },
-                  ib >> 1, 2);
-        mma(p, [&](int m, int kk) { return Qs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-        mma(g, aK, [&](int kk, int n) { return Ks[(n0 + n) * LDM + kk]; });
-        for_c(dr, [&](int r, int c, float &x) {
+        MMAR(dr, [&](int m, int kk) { return Ts[kk * LDM + m0 + m]; }, [&](int kk, int n) { return B9[kk * LDM + n0 + n]; },
+             ib >> 1, 2);
+        FORC(dr, [&](int r, int c, float &x) {
             if (m0 + r < L) d_v[(tok + m0 + r) * HD + n0 + c] = -x;
         });
         __syncthreads();   // T no longer needed
-        for_c(dr, [&](int r, int c, float &x) { Ts[(m0 + r) * LDM + n0 + c] = x; });   // dR
+        FORC(dr, [&](int r, int c, float &x) { Ts[(m0 + r) * LDM + n0 + c] = x; });   // dR
     }
     __syncthreads();
     const float *dRs = Ts;
@@ -511,13 +535,13 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
     {
         Strip dlam = zero_strip(), dyu = zero_strip();
         auto bU = [&](int kk, int n) { return Us[(n0 + n) * LDM + kk]; };
-        mma(dlam, [&](int m, int kk) { return dRs[(m0 + m) * LDM + kk]; }, bU);
-        mma(dyu, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; }, bU);
+        MMA(dlam, [&](int m, int kk) { return dRs[(m0 + m) * LDM + kk]; }, bU);
+        MMA(dyu, [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; }, bU);
 #pragma unroll
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
                 const float nth = -cf.th[col];
                 const float c0 = Cc[row * LDM + col], c1 = row > 0 ? Cc[(row - 1) * LDM + col] : 0.f;
                 const float lam = (col < row && row < L) ? dlam.t[tl][i] : 0.f;
@@ -538,7 +562,7 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
                 const float dw = dwa.t[tl][i] + (row + 1 < CW ? A2[(row + 1) * LDM + col] : 0.f);
                 xo[col * CW + row] = -cf.th[col] * dw;          // [s][t]
                 cs[tl] = fmaf(dw, Cc[row * LDM + col], cs[tl]);
@@ -551,21 +575,22 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
         }
     }
     __syncthreads();   // c and U no longer needed
-    commit(Us, tm);
-    if (has_s) commit(Cc, ts);
+    commit(Us, tm, tid);
+    if (has_s) commit(Cc, ts, tid);
     __syncthreads();
+    if (itask + 1 < task_hi) fetch_a(itask + 1, tid);
     const float *M0s = Us, *S0s = Cc, *dPs = B9, *dGs = A1;
     {
         Strip dym = zero_strip(), dys = zero_strip(), dq = zero_strip(), r0 = zero_strip(), r1 = zero_strip();
         auto aD = [&](int m, int kk) { return Ds[(m0 + m) * LDM + kk]; };
-        mma(dym, aD, [&](int kk, int n) { return M0s[kk * LDM + n0 + n]; });
-        if (has_s) mma(dys, aD, [&](int kk, int n) { return S0s[kk * LDM + n0 + n]; });
-        mma(dq, [&](int m, int kk) { return dPs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
+        MMA(dym, aD, [&](int kk, int n) { return M0s[kk * LDM + n0 + n]; });
+        if (has_s) MMA(dys, aD, [&](int kk, int n) { return S0s[kk * LDM + n0 + n]; });
+        MMA(dq, [&](int m, int kk) { return dPs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
 #pragma unroll
         for (int tl = 0; tl < 2; tl++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
+                const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
                 const float qv = Qs[row * LDM + col];
                 r0.t[tl][i] = dym.t[tl][i] * qv;
                 r1.t[tl][i] = dys.t[tl][i] * qv;
@@ -575,36 +600,48 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
         publish(0, r0);
         publish(1, r1);
     }
-    {
-        Strip dk = zero_strip(), drm = zero_strip(), drs = zero_strip(), r2 = zero_strip(), r3 = zero_strip(),
-              r4 = zero_strip(), r5 = zero_strip();
-        auto aR = [&](int m, int kk) { return dRs[(m0 + m) * LDM + kk]; };
-        mma(dk, [&](int m, int kk) { return dPs[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
-        mma(dk, [&](int m, int kk) { return dGs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
-        mma(drm, aR, [&](int kk, int n) { return M0s[kk * LDM + n0 + n]; });
-        if (has_s) mma(drs, aR, [&](int kk, int n) { return S0s[kk * LDM + n0 + n]; });
+    {   // d_k in two halves: fewer accumulators alive at once
+        Strip dk = zero_strip();
+        {
+            Strip r2 = zero_strip(), r3 = zero_strip();
+            MMA(dk, [&](int m, int kk) { return dPs[kk * LDM + m0 + m]; }, [&](int kk, int n) { return Qs[kk * LDM + n0 + n]; });
+            MMA(dk, [&](int m, int kk) { return dGs[(m0 + m) * LDM + kk]; }, [&](int kk, int n) { return Ks[kk * LDM + n0 + n]; });
 #pragma unroll
-        for (int tl = 0; tl < 2; tl++)
+            for (int tl = 0; tl < 2; tl++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int row = m0 + row_of(i), col = n0 + 16 * tl + (l & 15);
-                const float kv = Ks[row * LDM + col];
-                r2.t[tl][i] = udm.t[tl][i] * kv;
-                r3.t[tl][i] = uds.t[tl][i] * kv;
-                r4.t[tl][i] = drm.t[tl][i] * kv;
-                r5.t[tl][i] = drs.t[tl][i] * kv;
-                if (row < L)
-                    d_k[(tok + row) * HD + col] = dk.t[tl][i] + cv.wM[row] * udm.t[tl][i] + cv.wS[row] * uds.t[tl][i] +
-                                                  cv.am[row] * drm.t[tl][i] + cv.bm[row] * drs.t[tl][i];
-            }
-        publish(2, r2);
-        publish(3, r3);
-        publish(4, r4);
-        publish(5, r5);
+                for (int i = 0; i < 4; i++) {
+                    const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
+                    const float kv = Ks[row * LDM + col];
+                    r2.t[tl][i] = udm.t[tl][i] * kv;
+                    r3.t[tl][i] = uds.t[tl][i] * kv;
+                    dk.t[tl][i] += cv.wM[row] * udm.t[tl][i] + cv.wS[row] * uds.t[tl][i];
+                }
+            publish(2, r2);
+            publish(3, r3);
+        }
+        {
+            Strip drm = zero_strip(), drs = zero_strip(), r4 = zero_strip(), r5 = zero_strip();
+            auto aR = [&](int m, int kk) { return dRs[(m0 + m) * LDM + kk]; };
+            MMA(drm, aR, [&](int kk, int n) { return M0s[kk * LDM + n0 + n]; });
+            if (has_s) MMA(drs, aR, [&](int kk, int n) { return S0s[kk * LDM + n0 + n]; });
+#pragma unroll
+            for (int tl = 0; tl < 2; tl++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int row = m0 + row_of(i, l), col = n0 + 16 * tl + (l & 15);
+                    const float kv = Ks[row * LDM + col];
+                    r4.t[tl][i] = drm.t[tl][i] * kv;
+                    r5.t[tl][i] = drs.t[tl][i] * kv;
+                    if (row < L)
+                        d_k[(tok + row) * HD + col] = dk.t[tl][i] + cv.am[row] * drm.t[tl][i] + cv.bm[row] * drs.t[tl][i];
+                }
+            publish(4, r4);
+            publish(5, r5);
+        }
     }
     __syncthreads();
-    if (threadIdx.x < L) {
-        const int t = threadIdx.x;
+    if (tid < L) {
+        const int t = tid;
         auto sum = [&](int which, int row) { return part[which][0][row] + part[which][1][row]; };
         const float g1 = sum(2, t), g2 = sum(3, t);
         const float dam = t + 1 < CW ? sum(4, t + 1) : 0.f, dbm = t + 1 < CW ? sum(5, t + 1) : 0.f;
@@ -614,6 +651,8 @@ __global__ __launch_bounds__(kThr) void ex_grads_kernel(
         pv[1] = sum(1, t) + dbm;
         pv[2] = -cf.th[t] * g1;
         pv[3] = -cf.th[t] * g2;
+    }
+    __syncthreads();   // LDS is rewritten by the next chunk
     }
 }
 constexpr size_t kExGradsLds = 9 * MAT * sizeof(float);
@@ -671,14 +710,15 @@ bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *
         attr_set = true;
     }
     if (es.failed()) return true;
+    const int cus = compute_units(), pgrid = nchunks < (size_t)cus ? (int)nchunks : cus;   // one workgroup per compute unit (LDS)
     {
         KernelTimer kt("ex_local_kernel");
         if (guard)
-            hipLaunchKernelGGL(ex_local_kernel<true>, dim3((unsigned)nchunks), dim3(kThr), kExLocalLds, stream(), k, v, q, d_y,
-                               alpha, theta, eta, m_ckpt, s_ckpt, loc, locs, Tg, Ug, dUg, seq_len, C, nc, nck, (int)has_s, tracks);
+            hipLaunchKernelGGL(ex_local_kernel<true>, dim3((unsigned)pgrid), dim3(kThr), kExLocalLds, stream(), k, v, q, d_y,
+                               alpha, theta, eta, m_ckpt, s_ckpt, loc, locs, Tg, Ug, dUg, seq_len, C, nc, nck, (int)has_s, (int)nchunks, tracks);
         else
-            hipLaunchKernelGGL(ex_local_kernel<false>, dim3((unsigned)nchunks), dim3(kThr), kExLocalLds, stream(), k, v, q, d_y,
-                               alpha, theta, eta, m_ckpt, s_ckpt, loc, locs, Tg, Ug, dUg, seq_len, C, nc, nck, (int)has_s, tracks);
+            hipLaunchKernelGGL(ex_local_kernel<false>, dim3((unsigned)pgrid), dim3(kThr), kExLocalLds, stream(), k, v, q, d_y,
+                               alpha, theta, eta, m_ckpt, s_ckpt, loc, locs, Tg, Ug, dUg, seq_len, C, nc, nck, (int)has_s, (int)nchunks, tracks);
         check_launch("ex_local_kernel");
     }
     {
@@ -693,9 +733,9 @@ bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *
     }
     {
         KernelTimer kt("ex_grads_kernel");
-        hipLaunchKernelGGL(ex_grads_kernel, dim3((unsigned)nchunks), dim3(kThr), kExGradsLds, stream(), k, q, d_y, alpha, theta,
+        hipLaunchKernelGGL(ex_grads_kernel, dim3((unsigned)pgrid), dim3(kThr), kExGradsLds, stream(), k, q, d_y, alpha, theta,
                            eta, m_ckpt, s_ckpt, Tg, Ug, dUg, em, esn, d_k, d_v, d_q, d_theta, pvec, xs, scal, seq_len, C, nc, nck,
-                           (int)has_s);
+                           (int)has_s, (int)nchunks);
         check_launch("ex_grads_kernel");
     }
     chunkwise_gate_gradients(alpha, eta, pvec, xs, scal, d_alpha, d_eta, seq_len, batch, C, has_s, first_m, first_s, kDD, per,

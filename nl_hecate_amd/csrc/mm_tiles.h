@@ -29,11 +29,14 @@ template <class T> struct Tile;
 template <> struct Tile<float> { float4 x[2]; };
 template <> struct Tile<uint16_t> { uint2 x[2]; };
 
+// The helpers below take the thread (or lane) index as an optional last argument.  A kernel that loops over tasks
+// passes a copy that is opaque to the compiler per task: otherwise every LDS address of every phase is loop-invariant,
+// gets hoisted out of the loop and lives in a register for its whole length.
 template <class T>
-__device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows) {
+__device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows, int tid = threadIdx.x) {
 #pragma unroll
     for (int it = 0; it < 2; it++) {
-        const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
+        const int e = (it * kThr + tid) * 4, rr = e >> 6, cc = e & 63;
         if constexpr (sizeof(T) == 4)
             r.x[it] = rr < nrows ? *reinterpret_cast<const float4 *>(src + rr * 64 + cc) : make_float4(0, 0, 0, 0);
         else
@@ -41,10 +44,10 @@ __device__ __forceinline__ void fetch(Tile<T> &r, const T *src, int nrows) {
     }
 }
 template <class T>
-__device__ __forceinline__ void commit(float *dst, const Tile<T> &r) {
+__device__ __forceinline__ void commit(float *dst, const Tile<T> &r, int tid = threadIdx.x) {
 #pragma unroll
     for (int it = 0; it < 2; it++) {
-        const int e = (it * kThr + threadIdx.x) * 4, rr = e >> 6, cc = e & 63;
+        const int e = (it * kThr + tid) * 4, rr = e >> 6, cc = e & 63;
         float *p = dst + rr * LDM + cc;
         if constexpr (sizeof(T) == 4) {
             p[0] = r.x[it].x; p[1] = r.x[it].y; p[2] = r.x[it].z; p[3] = r.x[it].w;
@@ -79,8 +82,8 @@ __device__ __forceinline__ Strip zero_strip() {
 // read (the assignment 4 i + l/16 put up to four lanes on a bank).
 // Sixteen k-steps in four groups; the operands of group g+1 are read while group g runs.
 template <class FA, class FB>
-__device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
-    const int l = threadIdx.x & 63, r = l & 15, kb = 16 * (l >> 4);
+__device__ __forceinline__ void mma(Strip &acc, FA a, FB b, int l = threadIdx.x & 63) {
+    const int r = l & 15, kb = 16 * (l >> 4);
     float av[2][4], b0[2][4], b1[2][4];
 #pragma unroll
     for (int i = 0; i < 4; i++) { av[0][i] = a(r, kb + i); b0[0][i] = b(kb + i, r); b1[0][i] = b(kb + i, 16 + r); }
@@ -104,8 +107,8 @@ __device__ __forceinline__ void mma(Strip &acc, FA a, FB b) {
 // group j = l/16 takes the indices 32 p + 16 (j % 2) + 8 (j / 2) + 0..7 of a block of 32: the two groups of a
 // half-wave stay 16 banks apart.
 template <class FA, class FB>
-__device__ __forceinline__ void mma_range(Strip &acc, FA a, FB b, int p0, int p1) {
-    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4, kb = 16 * (kq & 1) + 8 * (kq >> 1);
+__device__ __forceinline__ void mma_range(Strip &acc, FA a, FB b, int p0, int p1, int l = threadIdx.x & 63) {
+    const int r = l & 15, kq = l >> 4, kb = 16 * (kq & 1) + 8 * (kq >> 1);
     for (int p = p0; p < p1; p++) {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -126,8 +129,8 @@ __device__ __forceinline__ void mma_range(Strip &acc, FA a, FB b, int p0, int p1
 // One 16x16 tile, contraction over the 16 indices k0 .. k0 + 15 only (block-diagonal operands):
 // acc += sum_{k0 <= k < k0+16} a(m,k) b(k,n), m, n in [0,16).
 template <class FA, class FB>
-__device__ __forceinline__ void mma_tile16(f32x4 &acc, FA a, FB b, int k0) {
-    const int l = threadIdx.x & 63, r = l & 15, kq = l >> 4;
+__device__ __forceinline__ void mma_tile16(f32x4 &acc, FA a, FB b, int k0, int l = threadIdx.x & 63) {
+    const int r = l & 15, kq = l >> 4;
     float av[4], bv[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) { av[i] = a(r, k0 + 4 * i + kq); bv[i] = b(k0 + 4 * i + kq, r); }
@@ -136,8 +139,7 @@ __device__ __forceinline__ void mma_tile16(f32x4 &acc, FA a, FB b, int k0) {
 }
 // Element i of tile tl of lane l is C[4*(l/16) + i][16*tl + l%16] of the strip.
 template <class F>
-__device__ __forceinline__ void for_c(Strip &acc, F f) {
-    const int l = threadIdx.x & 63;
+__device__ __forceinline__ void for_c(Strip &acc, F f, int l = threadIdx.x & 63) {
 #pragma unroll
     for (int tl = 0; tl < 2; tl++)
 #pragma unroll
@@ -154,8 +156,8 @@ __device__ __forceinline__ void strip_row_sums(Strip &x) {
     for (int i = 0; i < 4; i++) x.t[0][i] = group_allreduce<16>(x.t[0][i] + x.t[1][i]);
 }
 // lanes that publish the row sums (one per 16-lane group), and the strip rows they hold
-__device__ __forceinline__ bool row_writer() { return (threadIdx.x & 15) == 0; }
-__device__ __forceinline__ int row_of(int i) { return 4 * ((threadIdx.x & 63) >> 4) + i; }
+__device__ __forceinline__ bool row_writer(int l = threadIdx.x & 63) { return (l & 15) == 0; }
+__device__ __forceinline__ int row_of(int i, int l = threadIdx.x & 63) { return 4 * (l >> 4) + i; }
 
 }  // namespace mmt
 }  // namespace nlh
