@@ -739,12 +739,25 @@ class MagTrainer:
             entry = self._capture(x, d_out)
             graphs.put(key, entry)
         graph, xs, ds, out = entry
-        xs.copy_(x)
-        ds.copy_(d_out)
+        # the graph reads its inputs at fixed addresses; a caller that already writes its batch there
+        # (graph_inputs) spares the two copies
+        if x.data_ptr() != xs.data_ptr():
+            xs.copy_(x)
+        if d_out.data_ptr() != ds.data_ptr():
+            ds.copy_(d_out)
         graph.replay()
         self._optimizer_and_error_buffers(pulse)
         layer.conductor.advance()
         return out
+
+    def graph_inputs(self, shape):
+        """The input and upstream-gradient buffers that the captured step for the current pulse pattern and this
+        input shape reads (None before its first step_graphed): a producer that fills them in place and passes
+        them to step_graphed avoids a copy of each per step."""
+        pulse = self.layer.conductor.pulse()
+        graphs = self.__dict__.get("_graphs")
+        entry = None if graphs is None else graphs.get((tuple(bool(a) for a in pulse.active_levels), tuple(shape)))
+        return None if entry is None else (entry[1], entry[2])
 
     def _capture(self, x, d_out):
         """Warm-up on a side stream, then the capture.  Whatever happens in between (a recorded scratch error, an
