@@ -20,6 +20,7 @@ import pytest
 import torch
 
 from nl_hecate_amd import dispatch as D
+from nl_hecate_amd.ffi import lib
 from nl_hecate_amd import selfref as SR
 from oracle import pyoracle as orc
 from tests.gpu_util import assert_close, dev, host, rule_inputs, zeros
@@ -55,6 +56,14 @@ def test_config1_exact_titans_full_size_against_the_oracle():
            dx["m0"], dx["s0"], mc, sc, y, s, d, B, C, 0.0, F32_MAX)
     D.call("titans_backward_ckpt_f32_rocm", dx["k"], dx["v"], dx["q"], dx["alpha"], dx["theta"], dx["eta"], mc, sc,
            dx["dy"], *g.values(), s, d, B, C, 0.0, F32_MAX)
+    # the library's choice at this shape is the chunk-parallel matrix form; the fused sequential kernel once more
+    g2 = {n_: torch.zeros_like(t) for n_, t in g.items()}
+    prev = lib.nlh_exact_backward_form(2)
+    try:
+        D.call("titans_backward_ckpt_f32_rocm", dx["k"], dx["v"], dx["q"], dx["alpha"], dx["theta"], dx["eta"], mc, sc,
+               dx["dy"], *g2.values(), s, d, B, C, 0.0, F32_MAX)
+    finally:
+        lib.nlh_exact_backward_form(prev)
     torch.cuda.synchronize()
 
     def chain(b):
@@ -69,6 +78,10 @@ def test_config1_exact_titans_full_size_against_the_oracle():
         assert_close(n_, host(g[n_]), np.stack([w[3][n_] for w in want]))
     for n_ in ("d_m", "d_s"):   # summed over the batch
         assert_close(n_, host(g[n_]), np.sum([w[3][n_].astype(np.float64) for w in want], axis=0))
+    for n_ in ("d_k", "d_v", "d_q", "d_alpha", "d_theta", "d_eta"):
+        assert_close(n_ + " (fused kernel)", host(g2[n_]), np.stack([w[3][n_] for w in want]))
+    for n_ in ("d_m", "d_s"):
+        assert_close(n_ + " (fused kernel)", host(g2[n_]), np.sum([w[3][n_].astype(np.float64) for w in want], axis=0))
 
 
 def test_config2_chunkwise_bf16_full_size_against_the_oracle():
