@@ -667,12 +667,12 @@ void set_lds(K kernel, size_t bytes) {
 
 bool exact_backward_mm_applies(int d, int C) { return d == HD && C >= 1 && C <= CW; }
 
-// Cost model from measurements on one MI355X: a chunk costs the two chunk-parallel kernels about 72 us of a compute
-// unit whatever its length, a scan step 4 us; the fused sequential kernel walks a chain's tokens at 0.6 us each on a
+// Cost model from measurements on one MI355X: a chunk costs the two chunk-parallel kernels about 65 us of a compute
+// unit whatever its length, a scan step 2.7 us; the fused sequential kernel walks a chain's tokens at 0.6 us each on a
 // quarter of a compute unit's worth of workgroups (four per chain).
 bool exact_backward_mm_pays(int seq_len, int batch, int C) {
     const int nc = ceil_div(seq_len, C), cus = compute_units();
-    const double t_mm = (double)ceil_div(batch * nc, cus) * 72.0 + nc * 4.0;
+    const double t_mm = (double)ceil_div(batch * nc, cus) * 65.0 + nc * 2.7;
     const double t_seq = (double)seq_len * 0.6 * ceil_div(batch * 4, cus);
     return t_mm < t_seq;
 }
