@@ -387,51 +387,23 @@ __global__ __launch_bounds__(kThr) void cw_local_bwd_kernel(const TIn *__restric
 }
 constexpr size_t kLocalBwdLds = 5 * MAT * sizeof(float);
 
-// <M0, dMo>, <S0, dMo>, <S0, dSo> per chunk (dMo, dSo: adjoints of the chunk's end state)
-__global__ __launch_bounds__(256) void cw_state_dots_kernel(const float *__restrict__ m_states,
-                                                            const float *__restrict__ s_states,
-                                                            const float *__restrict__ dm_states,
-                                                            const float *__restrict__ ds_states,
-                                                            float *__restrict__ scal, int nc, int has_s) {
-    __shared__ float slot[3][4];
-    const int chain = blockIdx.x / nc, ci = blockIdx.x % nc;
-    const size_t o0 = ((size_t)chain * (nc + 1) + ci) * HD * HD, o1 = o0 + HD * HD;
-    float x0 = 0.f, x1 = 0.f, x2 = 0.f;
-    for (int e = threadIdx.x; e < HD * HD; e += 256) {
-        const float m = m_states[o0 + e], dm = dm_states[o1 + e];
-        x0 = fmaf(m, dm, x0);
-        if (has_s) {
-            const float sv = s_states[o0 + e];
-            x1 = fmaf(sv, dm, x1);
-            x2 = fmaf(sv, ds_states[o1 + e], x2);
-        }
-    }
-    x0 = wave_allreduce(x0); x1 = wave_allreduce(x1); x2 = wave_allreduce(x2);
-    if ((threadIdx.x & 63) == 0) {
-        slot[0][threadIdx.x >> 6] = x0; slot[1][threadIdx.x >> 6] = x1; slot[2][threadIdx.x >> 6] = x2;
-    }
-    __syncthreads();
-    if (threadIdx.x < 3) {
-        const float *p = slot[threadIdx.x];
-        scal[((size_t)chain * nc + ci) * 4 + threadIdx.x] = p[0] + p[1] + p[2] + p[3];
-    }
-}
-
 // ── backward, main per-chunk pass: dQ, dK, dV, dtheta; exports for the gate pass ──
 //   pvec [chain][token][4] = p0, ps, -theta g1, -theta g2   xs [chain][chunk][j][t] = -theta_j (dy_t.e_j)(q_t.k_j)
+//   scal [chunk][4] = <M0, dMo>, <S0, dMo>, <S0, dSo> (dMo, dSo: adjoints of the chunk's end state)
 template <class TIn, bool TRACK>
 __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     const TIn *__restrict__ k, const TIn *__restrict__ v, const TIn *__restrict__ q, const float *__restrict__ d_y,
     const float *__restrict__ alpha, const float *__restrict__ theta, const float *__restrict__ eta,
     const float *__restrict__ m_states, const float *__restrict__ s_states, const float *__restrict__ dm_states,
     const float *__restrict__ ds_states, float *__restrict__ d_k, float *__restrict__ d_v, float *__restrict__ d_q,
-    float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, int s, int C, int nc,
-    int has_s, int ntask, ChainTracks tr) {
+    float *__restrict__ d_theta, float *__restrict__ pvec, float *__restrict__ xs, float *__restrict__ scal, int s, int C,
+    int nc, int has_s, int ntask, ChainTracks tr) {
     extern __shared__ float smem[];
     float *Ks = smem, *Qs = Ks + MAT, *Ds = Qs + MAT, *Es = Ds + MAT, *Ms = Es + MAT, *B5 = Ms + MAT,
           *B6 = B5 + MAT, *B7 = B6 + MAT, *B8 = B7 + MAT;
     __shared__ Coef cf;
     __shared__ float part[5][2][CW];   // p0, ps, dtheta, g1, g2: one partial per column half
+    __shared__ float dots[3][8];       // partial <M0, dMo>, <S0, dMo>, <S0, dSo> per wave (the gate pass's scalars)
     float *Ss = B5, *Cc = B6;
     NLH_STRIP_ORIGIN();
     Tile<TIn> tk, tq, tv;
@@ -551,7 +523,17 @@ __global__ __launch_bounds__(kThr) void cw_grads_bwd_kernel(
     float *dMs = B6, *dSs = B8;
     commit(dMs, tdm);
     if (has_s) commit(dSs, tds);
+    {   // from the staged registers; M0 is still in LDS (this thread's own eight elements), S0 is not
+        const float x0 = wave_allreduce(tile_dot_lds(Ms, tdm));
+        const float x1 = has_s ? wave_allreduce(tile_dot(ts, tdm)) : 0.f;
+        const float x2 = has_s ? wave_allreduce(tile_dot(ts, tds)) : 0.f;
+        if ((threadIdx.x & 63) == 0) { dots[0][w] = x0; dots[1][w] = x1; dots[2][w] = x2; }
+    }
     __syncthreads();
+    if (threadIdx.x < 3) {
+        const float *pp = dots[threadIdx.x];
+        scal[((size_t)chain * nc + ci) * 4 + threadIdx.x] = ((pp[0] + pp[1]) + (pp[2] + pp[3])) + ((pp[4] + pp[5]) + (pp[6] + pp[7]));
+    }
     {
         // Dk[j][i] = sum_t CP[t][j] dY[t][i] + cl_j (K dMo^T)[j][i] + bl_j (K dSo^T)[j][i]
         Strip dk = zero_strip(), t1 = zero_strip(), t2 = zero_strip(), rt = zero_strip();
@@ -765,20 +747,17 @@ bool backward_mm(const char *fn, const TIn *k, const TIn *v, const TIn *q, const
         hipLaunchKernelGGL((cw_scan_kernel<false>), dim3(batch * 2), dim3(kThr), 0, stream(), nullptr, nullptr,
                            sc.loc, sc.locs, dm_states, ds_states, nc, (int)has_s);
         check_launch("cw_scan_kernel");
-        hipLaunchKernelGGL(cw_state_dots_kernel, dim3(batch * nc), dim3(256), 0, stream(), m_states, s_states,
-                           dm_states, ds_states, scal, nc, (int)has_s);
-        check_launch("cw_state_dots_kernel");
         KernelTimer kt("cw_grads_bwd_kernel");
         if (guard)
             hipLaunchKernelGGL((cw_grads_bwd_kernel<float, true>), dim3(batch * nc), dim3(kThr), kGradsBwdLds, stream(),
                                reinterpret_cast<const float *>(k), reinterpret_cast<const float *>(v),
                                reinterpret_cast<const float *>(q), d_y, alpha, theta, eta, m_states, s_states, dm_states,
-                               ds_states, d_k, d_v, d_q, d_theta, pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc,
+                               ds_states, d_k, d_v, d_q, d_theta, pvec, xs, scal, seq_len, chunk_size, nc, (int)has_s, batch * nc,
                                tracks);
         else
             hipLaunchKernelGGL((cw_grads_bwd_kernel<TIn, false>), dim3(batch * nc), dim3(kThr), kGradsBwdLds, stream(), k, v,
                                q, d_y, alpha, theta, eta, m_states, s_states, dm_states, ds_states, d_k, d_v, d_q, d_theta,
-                               pvec, xs, seq_len, chunk_size, nc, (int)has_s, batch * nc, ChainTracks{nullptr, nullptr});
+                               pvec, xs, scal, seq_len, chunk_size, nc, (int)has_s, batch * nc, ChainTracks{nullptr, nullptr});
         check_launch("cw_grads_bwd_kernel");
     }
     const bool packed = sizeof(TIn) == 2;   // where the gradient of the initial state sits (see above)

@@ -72,15 +72,6 @@ __device__ __forceinline__ void chunk_vectors(ChunkVecs &cv, const Coef &cf, int
     }
 }
 
-// sum of squares of a staged tile's registers over the wave
-__device__ __forceinline__ float tile_dot(const Tile<float> &a, const Tile<float> &b) {
-    float x = 0.f;
-#pragma unroll
-    for (int it = 0; it < 2; it++)
-        x += a.x[it].x * b.x[it].x + a.x[it].y * b.x[it].y + a.x[it].z * b.x[it].z + a.x[it].w * b.x[it].w;
-    return x;
-}
-
 // ── pass 1: chunk-local matrices ────────────────────────────────────────────
 template <bool TRACK>
 __global__ __launch_bounds__(kThr) void ex_local_kernel(

@@ -64,6 +64,27 @@ __device__ __forceinline__ void stage(float *dst, const T *src, int nrows) {
     commit(dst, r);
 }
 
+// dot product of two staged tiles' registers (this thread's eight elements of each)
+__device__ __forceinline__ float tile_dot(const Tile<float> &a, const Tile<float> &b) {
+    float x = 0.f;
+#pragma unroll
+    for (int it = 0; it < 2; it++)
+        x += a.x[it].x * b.x[it].x + a.x[it].y * b.x[it].y + a.x[it].z * b.x[it].z + a.x[it].w * b.x[it].w;
+    return x;
+}
+
+// the same against a tile that this thread committed to LDS earlier (its own eight elements: no barrier needed)
+__device__ __forceinline__ float tile_dot_lds(const float *src, const Tile<float> &b, int tid = threadIdx.x) {
+    float x = 0.f;
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+        const int e = (it * kThr + tid) * 4, rr = e >> 6, cc = e & 63;
+        const float *p = src + rr * LDM + cc;
+        x += p[0] * b.x[it].x + p[1] * b.x[it].y + p[2] * b.x[it].z + p[3] * b.x[it].w;
+    }
+    return x;
+}
+
 // Output strip of one wave: 16 rows x 32 columns = two 16x16 accumulator tiles side by side.
 // With 8 waves a 64x64 product is 8 strips; two waves share a SIMD, so one wave's LDS reads,
 // epilogue arithmetic and stores overlap the other's matrix-core work.
