@@ -84,6 +84,39 @@ def test_titans_against_the_token_loops(B, s, C):
     assert {"ex_local_kernel", "ex_scan_kernel", "ex_grads_kernel"} <= got[3], got[3]
 
 
+@pytest.mark.parametrize("B,s,C", [(2, 1, 64), (3, 5, 64), (2, 129, 1), (3, 64, 7), (1, 97, 16), (9, 63, 63), (2, 130, 33)])
+def test_edge_shapes(B, s, C):
+    """One-token sequences and chunks, intervals that divide nothing, a last chunk of one token."""
+    x = rule_inputs(B, s, 64, seed=211 + 7 * s + C, m0_scale=0.02)
+    cks, gs = oracle_pair(x, C)
+    got = gpu_backward(x, cks, C, F32_MAX, poison=True)
+    check(got, gs)
+    assert "ex_grads_kernel" in got[3], got[3]
+
+
+def test_twice_the_upstream_gradient_gives_twice_the_gradients_at_full_size():
+    """BASELINE configs[1] at full size (64 chains x 2048 tokens, checkpoints every 64): the backward is linear in d_y
+    (the values themselves are checked against the oracle in test_gpu_fullsize_values.py)."""
+    B, s, d, C = 64, 2048, 64, 64
+    x = rule_inputs(B, s, d, seed=223, m0_scale=0.02)
+    t = {n: dev(a) for n, a in x.items()}
+    n_ck = orc.checkpoint_count(s, C)
+    mc, sc, y = zeros(B, n_ck, d * d), zeros(B, n_ck, d * d), zeros(B, s, d)
+    D.call("titans_forward_ckpt_batched_f32_rocm", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"], t["m0"], t["s0"],
+           mc, sc, y, s, d, B, C, 0.0, F32_MAX)
+    outs = []
+    for scale in (1.0, 2.0):
+        g = {n: zeros(B, s, d) for n in ("d_k", "d_v", "d_q")}
+        g.update({n: zeros(B, s) for n in ("d_alpha", "d_theta", "d_eta")})
+        dm, ds = zeros(d, d), zeros(d, d)
+        D.call("titans_backward_ckpt_f32_rocm", t["k"], t["v"], t["q"], t["alpha"], t["theta"], t["eta"], mc, sc,
+               t["dy"] * scale, g["d_k"], g["d_v"], g["d_q"], g["d_alpha"], g["d_theta"], g["d_eta"], dm, ds, s, d, B, C, 0.0,
+               F32_MAX)
+        outs.append({**g, "d_m": dm, "d_s": ds})
+    for n in outs[0]:
+        assert_close(n, host(outs[1][n]), 2.0 * host(outs[0][n]), 1e-5)
+
+
 def test_saturated_gates():
     """theta = 0, alpha in {0, 1}, eta in {0, 1} on some tokens: nothing divides by a gate."""
     B, s, C = 3, 160, 64
