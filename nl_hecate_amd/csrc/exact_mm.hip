@@ -673,6 +673,11 @@ bool exact_backward_mm(const char *fn, bool has_s, const float *k, const float *
                        float *d_k, float *d_v, float *d_q, float *d_alpha, float *d_theta, float *d_eta, float *d_m_initial,
                        float *d_s_initial, int seq_len, int batch, int C, float error_clip, float m_norm_guard) {
     const ErrorScope es;
+    if (seq_len <= 0 || batch <= 0 || !exact_backward_mm_applies(HD, C)) {
+        fail("%s: the matrix form needs seq_len=%d and batch=%d positive and a checkpoint interval %d in [1, %d].", fn, seq_len, batch,
+             C, CW);
+        return true;
+    }
     const int nc = ceil_div(seq_len, C), nck = n_ckpt_count(seq_len, C);
     const size_t nchunks = (size_t)batch * nc;
     const bool guard = error_clip > 0.f || m_norm_guard > 0.f;
